@@ -1,0 +1,266 @@
+/*
+ * kmoe.h — C ABI of libkmoe.so: the MI355X (gfx950) quantized fused-MoE path.
+ *
+ * Every entry point takes raw DEVICE pointers plus explicit sizes, enqueues
+ * hand-written HIP kernels on the given stream and returns at once:
+ *   - returns KMOE_OK (0) or a negative KMOE_ERR_* code; never throws;
+ *   - never allocates or frees device memory, never synchronises the stream
+ *     (scratch comes in through `workspace` arguments sized by the
+ *     *_workspace_bytes functions), so calls can be captured into a HIP graph;
+ *   - kmoe_last_error() gives the text of the calling thread's last failure.
+ * A `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *
+ * Each function cites the reference interface (baidu/vLLM-Kunlun, paths under
+ * vllm_kunlun/) whose closed-source kernel it stands in for.
+ *
+ * Conventions shared by all functions
+ *   M tokens, H hidden, E experts, K experts per token, I intermediate size,
+ *   P = M*K routed (token, slot) pairs, flat pair index j = m*K + k.
+ *   "sorted row" r in [0,P): position of a pair after the stable sort by
+ *   expert id; rows of expert e are [lod[e], lod[e+1]).
+ *   bf16 tensors are uint16_t bit patterns; rounding is round-to-nearest-even.
+ *   int8 quantisation carries the row ABSMAX ("max"), not a scale: the value
+ *   represented by q is q * max / 127 (reference: quantization/kernels/
+ *   scale_mm.py:43-50, compressed_tensors_moe.py:116-120).
+ */
+#ifndef KMOE_H
+#define KMOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KMOE_OK 0
+#define KMOE_ERR_NULL (-1)        /* a required pointer is NULL            */
+#define KMOE_ERR_SHAPE (-2)       /* a size is out of range / inconsistent */
+#define KMOE_ERR_UNSUPPORTED (-3) /* valid request this build cannot serve */
+#define KMOE_ERR_WORKSPACE (-4)   /* workspace missing or too small        */
+#define KMOE_ERR_LAUNCH (-5)      /* the HIP runtime refused a launch      */
+
+typedef void* kmoe_stream_t;
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char* kmoe_last_error(void);
+/* Library version string, e.g. "kmoe 0.1 gfx950". */
+const char* kmoe_version(void);
+
+/* ------------------------------------------------------------------ routing */
+
+/*
+ * Softmax top-K routing. Replaces kunlun_ops.moe_softmax_topk (renorm=0;
+ * ops/_custom_ops.py:781-790, called ops/_kunlun_ops.py:666-668) and
+ * kunlun_ops.moe_softmax_topk_norm (renorm=1; ops/_custom_ops.py:1084-1094,
+ * called quantization/compressed_tensors/compressed_tensors_moe.py:152-159).
+ *   logits [M,E] f32 -> topk_w [M,K] f32, topk_ids [M,K] i32.
+ * ids: the K largest logits per row, descending, ties -> lower expert id.
+ * w = softmax(logits)[ids]; with renorm, divided by their sum over K.
+ * Limits: 1 <= K <= min(E,64), E <= 1024.
+ */
+int kmoe_softmax_topk(const float* logits, int M, int E, int K, int renorm,
+                      float* topk_w, int32_t* topk_ids, kmoe_stream_t stream);
+
+/*
+ * DeepSeek-V3 "noaux_tc" routing. Replaces kunlun_ops.moe_sigmoid_group_topk_norm
+ * (ops/_custom_ops.py:1351-1371, called compressed_tensors_moe.py:160-170 and
+ * ops/_kunlun_ops.py:421-431; prototype csrc/xops.h:153-160).
+ *   s = sigmoid(logits); c = s + bias (bias may be NULL = 0);
+ *   group score = sum of the 2 largest c in the group; keep the topk_group
+ *   best groups (ties -> lower group); take the K largest c among their
+ *   experts (ties -> lower id); w = s[ids] / (sum_k s[ids] + 1e-20) * scale.
+ * n_group <= 1 disables the group stage. Limits as above, n_group <= 64,
+ * E % n_group == 0, E / n_group >= 2, K <= topk_group * E / n_group.
+ */
+int kmoe_sigmoid_group_topk_norm(const float* logits, const float* bias, int M,
+                                 int E, int K, int n_group, int topk_group,
+                                 float scale, float* topk_w, int32_t* topk_ids,
+                                 kmoe_stream_t stream);
+
+/* -------------------------------------------------------------------- align */
+
+/*
+ * Per-block histogram of expert ids. Replaces kunlun_ops.gen_block_statistic
+ * (ops/_custom_ops.py:1123-1125, called compressed_tensors_moe.py:186).
+ * Block b of n_blocks counts the pairs j in [b*ceil(P/n_blocks), ...).
+ *   topk_ids [P] i32 -> block_statistic [n_blocks,E] i32 (overwritten).
+ */
+int kmoe_block_statistic(const int32_t* topk_ids, int P, int E, int n_blocks,
+                         int32_t* block_statistic, kmoe_stream_t stream);
+
+/* Scratch bytes kmoe_align needs for P pairs and E experts. */
+size_t kmoe_align_workspace_bytes(int P, int E);
+
+/*
+ * Stable counting sort of the routed pairs by expert. Replaces the index part
+ * of kunlun_ops.moe_pre_sorted (ops/_custom_ops.py:1144-1163, called
+ * compressed_tensors_moe.py:188-196) and xspeedgate_ops.moe_pre_small
+ * (compressed_tensors_moe.py:199-207).
+ *   topk_ids [P] i32 (all in [0,E)) ->
+ *   moe_index [P]   : sorted row of pair j              (reference: moe_index)
+ *   sorted_src [P]  : pair j that sits in sorted row r   (inverse; may be NULL)
+ *   expert_m [E]    : rows per expert                    (may be NULL)
+ *   lod [E+1]       : exclusive prefix sum of expert_m   (sorted_tokens_num_lod)
+ * Limits: E <= 1024, P <= 2^24.
+ */
+int kmoe_align(const int32_t* topk_ids, int P, int E, int32_t* moe_index,
+               int32_t* sorted_src, int32_t* expert_m, int32_t* lod,
+               void* workspace, size_t workspace_bytes, kmoe_stream_t stream);
+
+/*
+ * Gather of activation rows into sorted order: the data part of
+ * kunlun_ops.moe_pre_sorted (output moe_expand, compressed_tensors_moe.py:173-196).
+ *   dst[r, :] = src[sorted_src[r] / K, :]   for r in [0,P); 16-bit elements,
+ *   H % 8 == 0, rows 16-byte aligned.
+ */
+int kmoe_gather_rows(const uint16_t* src, int64_t ld_src,
+                     const int32_t* sorted_src, int P, int K, int H,
+                     uint16_t* dst, int64_t ld_dst, kmoe_stream_t stream);
+
+/* ------------------------------------------------------ activation quantise */
+
+/*
+ * Per-row dynamic symmetric int8. Replaces kunlun_ops.quant2d
+ * (ops/_custom_ops.py:1912-1924, called compressed_tensors_moe.py:224,253; and
+ * through _C.scaled_int8_quant, ops/_custom_ops.py:1633-1657).
+ *   x [R,C] bf16 -> q [R,C] i8, row_max [R] f32 (absmax of the row);
+ *   q = clamp(rne(x * (127 / row_max)), -127, 127); an all-zero row gives q=0, max=0.
+ * Limits: C % 8 == 0, C <= 16384, ld_x % 8 == 0, ld_q % 8 == 0.
+ */
+int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q,
+                       int64_t ld_q, float* row_max, kmoe_stream_t stream);
+
+/*
+ * Per-row, per-128-column-group dynamic fp8-e4m3fn (OCP). No counterpart in the
+ * reference (its fp8 ops are empty stubs, ops/_custom_ops.py:44-89); follows
+ * the DeepSeek-V3 block-scaled recipe.
+ *   x [R,C] bf16 -> q [R,C] e4m3fn bytes, scale [R, C/128] f32;
+ *   scale = absmax/448 (absmax 0 -> scale 0, q 0); q = e4m3fn_rne_sat(x / scale).
+ * Limits: C % 128 == 0.
+ */
+int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, int C,
+                            uint8_t* q, int64_t ld_q, float* scale,
+                            kmoe_stream_t stream);
+
+/* ------------------------------------------------------------- grouped GEMM */
+
+#define KMOE_ACT_NONE 0
+#define KMOE_ACT_SWIGLU 1 /* out[r,i] = silu(y[r,i]) * y[r,i+n/2], i < n/2 */
+
+typedef struct kmoe_gemm_i8_args {
+  const int8_t* a;        /* [a_rows, k] quantised activations, row stride lda  */
+  int64_t lda;
+  const float* a_max;     /* [a_rows] absmax of each activation row             */
+  const int32_t* row_src; /* NULL: sorted row r reads a[r]. Else it reads
+                             a[row_src[r] / src_div] (gather through the sort)  */
+  int32_t src_div;        /* >= 1                                               */
+  const int8_t* w;        /* [E, n, k] weights, k contiguous                    */
+  const float* w_max;     /* [E, n] absmax of each output channel               */
+  const int32_t* lod;     /* [E+1] row offsets per expert (device)              */
+  int32_t E, n, k;
+  int32_t rows;           /* capacity = lod[E] upper bound (P)                  */
+  uint16_t* y;            /* bf16 [rows, n] (act none) or [rows, n/2] (SwiGLU)  */
+  int64_t ldy;
+  int32_t* acc_out;       /* NULL, or int32 [rows, n]: raw accumulators         */
+  int32_t act;            /* KMOE_ACT_*                                         */
+  int32_t variant;        /* 0 = choose from shape; >0 force a kernel variant   */
+} kmoe_gemm_i8_args;
+
+/*
+ * W8A8 grouped GEMM. Replaces kunlun_ops.moe_fc in its int8 form
+ * (ops/_custom_ops.py:1204-1244, called compressed_tensors_moe.py:226-238 and
+ * 263-275; prototype csrc/xops.h:230-239) and, with E=1, the dense
+ * kunlun_ops.matmul with x_pc_max/w_pc_max (ops/_custom_ops.py:1811-1845,
+ * called quantization/kernels/scale_mm.py:83-90).
+ * For each expert e and sorted row r in [lod[e], lod[e+1]):
+ *   acc[r,c] = sum_k a[src(r),k] * w[e,c,k]                      (int32, exact)
+ *   y[r,c]   = bf16( float(acc) * (a_max[src(r)]/127) * (w_max[e,c]/127) )
+ * With KMOE_ACT_SWIGLU the bf16 y is never stored: the kernel stores
+ *   bf16( silu(float(y[r,i])) * float(y[r,i+n/2]) ),  silu(t) = t/(1+exp(-t)).
+ * Limits: k % 16 == 0, n % 16 == 0 (SwiGLU: n % 32 == 0), 16-byte aligned rows.
+ */
+int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* args, kmoe_stream_t stream);
+
+/*
+ * SiLU-and-mul on a stored gate_up result. Replaces kunlun_ops.swiglu
+ * (ops/_custom_ops.py:699-706, called compressed_tensors_moe.py:240-243).
+ *   y [R,2I] bf16 -> out [R,I] bf16 = bf16( silu(y[:, :I]) * y[:, I:] ).
+ */
+int kmoe_silu_and_mul(const uint16_t* y, int64_t ld_y, int R, int I,
+                      uint16_t* out, int64_t ld_out, kmoe_stream_t stream);
+
+/*
+ * Un-permute + weighted top-K sum. Replaces kunlun_ops.moe_post
+ * (ops/_custom_ops.py:1316-1324, called compressed_tensors_moe.py:278-290).
+ *   out[m,h] = bf16( sum_k topk_w[m,k] * dq[m,k] * float(x[moe_index[m*K+k], h]) )
+ * f32 accumulation, k ascending; dequant_scale (dq) may be NULL (= 1).
+ * Optional caller epilogue (models/deepseek_v2.py:288-296), applied when
+ * out_scale != 1 or addend != NULL:
+ *   out = bf16( float(bf16(float(out) * out_scale)) + float(addend[m,h]) ).
+ */
+int kmoe_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_index,
+                 const float* topk_w, const float* dequant_scale, int M, int K,
+                 int H, float out_scale, const uint16_t* addend,
+                 int64_t ld_addend, uint16_t* out, int64_t ld_out,
+                 kmoe_stream_t stream);
+
+/* ------------------------------------------------------------ fused forward */
+
+#define KMOE_SCORE_SOFTMAX 0
+#define KMOE_SCORE_SIGMOID 1
+
+typedef struct kmoe_w8a8_args {
+  /* shape */
+  int32_t M, H, E, K, I;
+  /* routing */
+  int32_t scoring;       /* KMOE_SCORE_*                                        */
+  int32_t renormalize;   /* softmax only: divide the K weights by their sum     */
+  int32_t n_group, topk_group; /* sigmoid only; n_group <= 1: no group stage    */
+  float routed_scale;    /* sigmoid only: multiplies the routing weights        */
+  const float* logits;   /* [M,E] f32                                           */
+  const float* bias;     /* [E] f32 correction bias or NULL                     */
+  /* activations and routed expert weights */
+  const uint16_t* x;     /* [M,H] bf16                                          */
+  const int8_t* w13;     /* [E,2I,H]                                            */
+  const float* w13_max;  /* [E,2I]                                              */
+  const int8_t* w2;      /* [E,H,I]                                             */
+  const float* w2_max;   /* [E,H]                                               */
+  /* optional dense shared expert (I_shared = 0: none) */
+  int32_t I_shared;
+  const int8_t* ws13;    /* [2*I_shared,H]                                      */
+  const float* ws13_max; /* [2*I_shared]                                        */
+  const int8_t* ws2;     /* [H,I_shared]                                        */
+  const float* ws2_max;  /* [H]                                                 */
+  /* caller epilogue: out = routed*out_scale (+ shared) */
+  float out_scale;
+  uint16_t* out;         /* [M,H] bf16                                          */
+} kmoe_w8a8_args;
+
+/* Byte offsets of the intermediates kmoe_forward_w8a8 keeps in its workspace. */
+typedef struct kmoe_w8a8_layout {
+  size_t total_bytes;
+  size_t topk_w, topk_ids, moe_index, sorted_src, expert_m, lod, align_ws;
+  size_t xq, xmax, act, actq, actmax, down;
+  size_t sh_lod, sh_act, sh_actq, sh_actmax, sh_out;
+} kmoe_w8a8_layout;
+
+/* Workspace layout (and total size) for a shape; only the shape fields of args are read. */
+int kmoe_w8a8_workspace_layout(const kmoe_w8a8_args* args, kmoe_w8a8_layout* layout);
+
+/*
+ * The whole layer: routing -> align -> per-token int8 quant -> gate_up GEMM with
+ * fused SiLU-mul -> per-row int8 quant -> down GEMM -> weighted combine
+ * (+ shared expert, + caller epilogue). Replaces
+ * KunlunCompressedTensorsW8A8Int8MoEMethod.apply_monolithic
+ * (compressed_tensors_moe.py:122-291) and, for the shared expert,
+ * KunlunScaledMMLinearKernel.apply_weights (quantization/kernels/scale_mm.py:52-90).
+ * Results are bit-identical to running the stage functions above one by one.
+ */
+int kmoe_forward_w8a8(const kmoe_w8a8_args* args, void* workspace,
+                      size_t workspace_bytes, kmoe_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KMOE_H */

@@ -1,0 +1,219 @@
+"""ctypes/numpy front end of oracle/libmoe_oracle.so — TEST INFRASTRUCTURE.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg import
+this. Every function takes and returns numpy arrays (bf16 as uint16 bit
+patterns) and forwards to the C restatement in moe_oracle.c, whose header
+states what it follows in the reference and what pins it.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libmoe_oracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (seconds)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.run(["make", "-C", _HERE] + (["-B"] if force else []), check=True,
+                       stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.orc_exp.restype = C.c_float
+        _lib.orc_exp.argtypes = [C.c_float]
+        _lib.orc_sigmoid.restype = C.c_float
+        _lib.orc_sigmoid.argtypes = [C.c_float]
+        _lib.orc_silu.restype = C.c_float
+        _lib.orc_silu.argtypes = [C.c_float]
+        _lib.orc_f32_to_e4m3fn.restype = C.c_uint8
+        _lib.orc_f32_to_e4m3fn.argtypes = [C.c_float]
+        _lib.orc_e4m3fn_to_f32.restype = C.c_float
+        _lib.orc_e4m3fn_to_f32.argtypes = [C.c_uint8]
+    return _lib
+
+
+def _p(a):
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"], "oracle arrays must be contiguous"
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _c(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+# -- bf16 helpers (bit patterns in uint16) -----------------------------------
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = u + 0x7FFF + ((u >> 16) & 1)
+    return (u >> 16).astype(np.uint16)
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+# -- scalar functions ---------------------------------------------------------
+def exp(x: np.ndarray) -> np.ndarray:
+    f = lib().orc_exp
+    return np.array([f(float(v)) for v in np.asarray(x, dtype=np.float32).ravel()], dtype=np.float32).reshape(np.shape(x))
+
+
+def sigmoid(x: np.ndarray) -> np.ndarray:
+    f = lib().orc_sigmoid
+    return np.array([f(float(v)) for v in np.asarray(x, dtype=np.float32).ravel()], dtype=np.float32).reshape(np.shape(x))
+
+
+def silu(x: np.ndarray) -> np.ndarray:
+    f = lib().orc_silu
+    return np.array([f(float(v)) for v in np.asarray(x, dtype=np.float32).ravel()], dtype=np.float32).reshape(np.shape(x))
+
+
+# -- stages -------------------------------------------------------------------
+def softmax_topk(logits, K, renorm):
+    logits = _c(logits, np.float32)
+    M, E = logits.shape
+    w = np.empty((M, K), np.float32)
+    ids = np.empty((M, K), np.int32)
+    lib().orc_softmax_topk(_p(logits), M, E, K, int(bool(renorm)), _p(w), _p(ids))
+    return w, ids
+
+
+def sigmoid_group_topk_norm(logits, bias, K, n_group, topk_group, scale):
+    logits = _c(logits, np.float32)
+    bias = None if bias is None else _c(bias, np.float32)
+    M, E = logits.shape
+    w = np.empty((M, K), np.float32)
+    ids = np.empty((M, K), np.int32)
+    lib().orc_sigmoid_group_topk_norm(_p(logits), _p(bias), M, E, K, int(n_group or 1), int(topk_group or 1),
+                                      C.c_float(scale), _p(w), _p(ids))
+    return w, ids
+
+
+def align(ids, E):
+    ids = _c(ids, np.int32).ravel()
+    P = ids.size
+    moe_index = np.empty(P, np.int32)
+    sorted_src = np.full(P, -1, np.int32)
+    expert_m = np.empty(E, np.int32)
+    lod = np.empty(E + 1, np.int32)
+    lib().orc_align(_p(ids), P, E, _p(moe_index), _p(sorted_src), _p(expert_m), _p(lod))
+    return moe_index, sorted_src, expert_m, lod
+
+
+def block_statistic(ids, E, n_blocks):
+    ids = _c(ids, np.int32).ravel()
+    out = np.empty((n_blocks, E), np.int32)
+    lib().orc_block_statistic(_p(ids), ids.size, E, n_blocks, _p(out))
+    return out
+
+
+def quant_i8_rows(x_bits):
+    x_bits = _c(x_bits, np.uint16)
+    R, Cc = x_bits.shape
+    q = np.empty((R, Cc), np.int8)
+    mx = np.empty(R, np.float32)
+    lib().orc_quant_i8_rows(_p(x_bits), C.c_int64(Cc), R, Cc, _p(q), C.c_int64(Cc), _p(mx))
+    return q, mx
+
+
+def quant_fp8_group128(x_bits):
+    x_bits = _c(x_bits, np.uint16)
+    R, Cc = x_bits.shape
+    q = np.empty((R, Cc), np.uint8)
+    s = np.empty((R, Cc // 128), np.float32)
+    lib().orc_quant_fp8_group128(_p(x_bits), C.c_int64(Cc), R, Cc, _p(q), C.c_int64(Cc), _p(s))
+    return q, s
+
+
+def grouped_gemm_i8(a, a_max, w, w_max, lod, act=0, row_src=None, src_div=1, want_acc=False, want_y=True):
+    a = _c(a, np.int8)
+    a_max = _c(a_max, np.float32).ravel()
+    w = _c(w, np.int8)
+    w_max = _c(w_max, np.float32).reshape(w.shape[0], w.shape[1])
+    lod = _c(lod, np.int32)
+    E, n, k = w.shape
+    rows = int(lod[-1])
+    row_src = None if row_src is None else _c(row_src, np.int32)
+    n_out = n // 2 if act else n
+    y = np.zeros((rows, n_out), np.uint16) if want_y else None
+    acc = np.zeros((rows, n), np.int32) if want_acc else None
+    lib().orc_grouped_gemm_i8(_p(a), C.c_int64(a.shape[1]), _p(a_max), _p(row_src), int(src_div), _p(w), _p(w_max),
+                              _p(lod), E, n, k, _p(y), C.c_int64(n_out), _p(acc), int(act))
+    return y, acc
+
+
+def silu_and_mul(y_bits):
+    y_bits = _c(y_bits, np.uint16)
+    R, two_i = y_bits.shape
+    out = np.empty((R, two_i // 2), np.uint16)
+    lib().orc_silu_and_mul(_p(y_bits), C.c_int64(two_i), R, two_i // 2, _p(out), C.c_int64(two_i // 2))
+    return out
+
+
+def combine(x_bits, moe_index, topk_w, dq=None, out_scale=1.0, addend=None):
+    x_bits = _c(x_bits, np.uint16)
+    topk_w = _c(topk_w, np.float32)
+    M, K = topk_w.shape
+    H = x_bits.shape[1]
+    moe_index = _c(moe_index, np.int32).reshape(M, K)
+    dq = None if dq is None else _c(dq, np.float32)
+    addend = None if addend is None else _c(addend, np.uint16)
+    out = np.empty((M, H), np.uint16)
+    lib().orc_combine(_p(x_bits), C.c_int64(H), _p(moe_index), _p(topk_w), _p(dq), M, K, H, C.c_float(out_scale),
+                      _p(addend), C.c_int64(H), _p(out), C.c_int64(H))
+    return out
+
+
+def forward_w8a8(x_bits, logits, w13, w13_max, w2, w2_max, K, scoring="softmax", renormalize=True, n_group=1,
+                 topk_group=1, routed_scale=1.0, bias=None, shared=None, out_scale=1.0, intermediates=False):
+    """Whole layer. `shared` = (ws13, ws13_max, ws2, ws2_max) or None.
+    Returns out bits [M,H], plus a dict of intermediates when asked."""
+    x_bits = _c(x_bits, np.uint16)
+    logits = _c(logits, np.float32)
+    w13 = _c(w13, np.int8)
+    w2 = _c(w2, np.int8)
+    E, two_i, H = w13.shape
+    I = two_i // 2
+    M = x_bits.shape[0]
+    P = M * K
+    w13_max = _c(w13_max, np.float32).reshape(E, two_i)
+    w2_max = _c(w2_max, np.float32).reshape(E, H)
+    bias = None if bias is None else _c(bias, np.float32)
+    if shared is not None:
+        ws13, ws13_max, ws2, ws2_max = shared
+        ws13 = _c(ws13, np.int8)
+        ws2 = _c(ws2, np.int8)
+        ws13_max = _c(ws13_max, np.float32).ravel()
+        ws2_max = _c(ws2_max, np.float32).ravel()
+        Is = ws13.shape[0] // 2
+    else:
+        ws13 = ws13_max = ws2 = ws2_max = None
+        Is = 0
+    out = np.empty((M, H), np.uint16)
+    inter = {}
+    if intermediates:
+        inter = dict(topk_w=np.empty((M, K), np.float32), topk_ids=np.empty((M, K), np.int32),
+                     moe_index=np.empty(P, np.int32), lod=np.empty(E + 1, np.int32),
+                     actq=np.empty((P, I), np.int8), actmax=np.empty(P, np.float32),
+                     down=np.empty((P, H), np.uint16))
+    g = inter.get
+    lib().orc_forward_w8a8(M, H, E, K, I, 0 if scoring == "softmax" else 1, int(bool(renormalize)), int(n_group or 1),
+                           int(topk_group or 1), C.c_float(routed_scale), _p(logits), _p(bias), _p(x_bits), _p(w13),
+                           _p(w13_max), _p(w2), _p(w2_max), Is, _p(ws13), _p(ws13_max), _p(ws2), _p(ws2_max),
+                           C.c_float(out_scale), _p(out), _p(g("topk_w")), _p(g("topk_ids")), _p(g("moe_index")),
+                           _p(g("lod")), _p(g("actq")), _p(g("actmax")), _p(g("down")))
+    return (out, inter) if intermediates else out

@@ -1,0 +1,433 @@
+/*
+ * moe_oracle.c — TEST INFRASTRUCTURE, not product code.
+ *
+ * A plain-C CPU restatement of the quantized fused-MoE computation that
+ * baidu/vLLM-Kunlun drives through closed kernels, stage by stage in the order
+ * of KunlunCompressedTensorsW8A8Int8MoEMethod.apply_monolithic
+ * (vllm_kunlun/quantization/compressed_tensors/compressed_tensors_moe.py:122-291).
+ * Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may load
+ * it; the product library never does.
+ *
+ * The reference's arithmetic lives in binary wheels (kunlun_ops 0.1.58,
+ * xspeedgate_ops 1.1.0; docs/source/installation.md:131-137) that are not in
+ * the reference tree, and the reference holds no test or golden vector for this
+ * path: PARITY WITH THOSE KERNELS IS UNPINNED. What this file computes is fixed
+ * by the call sites (shapes, dtypes, stage order, max-not-scale convention) and
+ * by the mathematics; tests/test_oracle_*.py pin every function against closed
+ * forms, exact integer arithmetic, brute force and independent torch /
+ * transformers restatements.
+ *
+ * Where the reference leaves a bit-level choice open, this file fixes it once:
+ *   - rounding is round-half-to-even everywhere (rintf under the default mode);
+ *   - top-k order: score descending, ties to the lower expert id;
+ *   - exp() is the fixed fma sequence orc_exp() below (< 2 ulp from libm), so a
+ *     device kernel performing the same sequence yields the same bits;
+ *   - the softmax row sum adds 64 interleaved partial sums (element e goes to
+ *     partial e % 64, in ascending e) with a balanced binary tree;
+ *   - dequant is ((float)acc * (a_max/127)) * (w_max/127), left to right;
+ *   - no operation is contracted into an fma unless written as fmaf.
+ * Build with -ffp-contract=off.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------ scalar pieces */
+
+static inline float bf16_to_f32(uint16_t h) {
+  union { uint32_t u; float f; } v;
+  v.u = (uint32_t)h << 16;
+  return v.f;
+}
+
+static inline uint16_t f32_to_bf16(float f) {
+  union { uint32_t u; float f; } v;
+  v.f = f;
+  uint32_t u = v.u;
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+ORC_API float orc_exp(float x) {
+  x = fminf(fmaxf(x, -86.0f), 86.0f);
+  const float n = rintf(x * 0x1.715476p+0f);
+  float r = fmaf(n, -0x1.62e4p-1f, x);
+  r = fmaf(n, -0x1.7f7d1cp-20f, r);
+  float p = 0x1.a01a02p-13f;
+  p = fmaf(p, r, 0x1.6c16c2p-10f);
+  p = fmaf(p, r, 0x1.111112p-7f);
+  p = fmaf(p, r, 0x1.555556p-5f);
+  p = fmaf(p, r, 0x1.555556p-3f);
+  p = fmaf(p, r, 0.5f);
+  p = fmaf(p, r, 1.0f);
+  p = fmaf(p, r, 1.0f);
+  return ldexpf(p, (int)n);
+}
+
+ORC_API float orc_sigmoid(float x) { return 1.0f / (1.0f + orc_exp(-x)); }
+ORC_API float orc_silu(float x) { return x / (1.0f + orc_exp(-x)); }
+
+/* K best of score[0..E) among eligible entries: score descending, ties to the
+ * lower index. O(E*K) selection; out_ids in selection order. */
+static void select_topk(const float* score, const uint8_t* eligible, int E, int K, int32_t* out_ids) {
+  uint8_t* taken = (uint8_t*)calloc((size_t)E, 1);
+  for (int k = 0; k < K; ++k) {
+    int best = -1;
+    for (int e = 0; e < E; ++e) {
+      if (taken[e] || (eligible && !eligible[e])) continue;
+      if (best < 0 || score[e] > score[best]) best = e;
+    }
+    out_ids[k] = best;
+    if (best >= 0) taken[best] = 1;
+  }
+  free(taken);
+}
+
+/* ------------------------------------------------------------------ routing */
+
+/* softmax -> top-K (-> renorm). Follows the call at compressed_tensors_moe.py:151-159
+ * (logits already f32, normalised weights, int32 ids) and ops/_kunlun_ops.py:666-671. */
+ORC_API void orc_softmax_topk(const float* logits, int M, int E, int K, int renorm, float* topk_w,
+                              int32_t* topk_ids) {
+  float* ex = (float*)malloc(sizeof(float) * (size_t)E);
+  for (int m = 0; m < M; ++m) {
+    const float* row = logits + (size_t)m * E;
+    float mx = row[0];
+    for (int e = 1; e < E; ++e) mx = fmaxf(mx, row[e]);
+    float part[64];
+    for (int l = 0; l < 64; ++l) part[l] = 0.0f;
+    for (int e = 0; e < E; ++e) {
+      ex[e] = orc_exp(row[e] - mx);
+      part[e & 63] = part[e & 63] + ex[e];
+    }
+    for (int off = 32; off > 0; off >>= 1)
+      for (int l = 0; l < off; ++l) part[l] = part[l] + part[l + off];
+    const float total = part[0];
+    int32_t* ids = topk_ids + (size_t)m * K;
+    float* w = topk_w + (size_t)m * K;
+    select_topk(row, NULL, E, K, ids); /* softmax is monotone: choose on the logits */
+    for (int k = 0; k < K; ++k) w[k] = ex[ids[k]] / total;
+    if (renorm) {
+      float denom = 0.0f;
+      for (int k = 0; k < K; ++k) denom = denom + w[k];
+      for (int k = 0; k < K; ++k) w[k] = w[k] / denom;
+    }
+  }
+  free(ex);
+}
+
+/* DeepSeek-V3 grouped top-k with correction bias. Follows the call at
+ * compressed_tensors_moe.py:160-170 (args x, bias, n_group, topk_group, scale). */
+ORC_API void orc_sigmoid_group_topk_norm(const float* logits, const float* bias, int M, int E, int K, int n_group,
+                                         int topk_group, float scale, float* topk_w, int32_t* topk_ids) {
+  float* s = (float*)malloc(sizeof(float) * (size_t)E);
+  float* c = (float*)malloc(sizeof(float) * (size_t)E);
+  uint8_t* ok = (uint8_t*)malloc((size_t)E);
+  if (n_group < 1) n_group = 1;
+  float* gscore = (float*)malloc(sizeof(float) * (size_t)n_group);
+  int32_t* gsel = (int32_t*)malloc(sizeof(int32_t) * (size_t)n_group);
+  const int gsize = E / n_group;
+  for (int m = 0; m < M; ++m) {
+    const float* row = logits + (size_t)m * E;
+    for (int e = 0; e < E; ++e) {
+      s[e] = orc_sigmoid(row[e]);
+      c[e] = bias ? s[e] + bias[e] : s[e];
+      ok[e] = 1;
+    }
+    if (n_group > 1) {
+      for (int g = 0; g < n_group; ++g) {
+        float t1 = -INFINITY, t2 = -INFINITY;
+        for (int i = 0; i < gsize; ++i) {
+          const float x = c[g * gsize + i];
+          if (x > t1) {
+            t2 = t1;
+            t1 = x;
+          } else if (x > t2) {
+            t2 = x;
+          }
+        }
+        gscore[g] = t1 + t2;
+      }
+      select_topk(gscore, NULL, n_group, topk_group, gsel);
+      memset(ok, 0, (size_t)E);
+      for (int t = 0; t < topk_group; ++t)
+        for (int i = 0; i < gsize; ++i) ok[gsel[t] * gsize + i] = 1;
+    }
+    int32_t* ids = topk_ids + (size_t)m * K;
+    float* w = topk_w + (size_t)m * K;
+    select_topk(c, ok, E, K, ids);
+    float denom = 0.0f;
+    for (int k = 0; k < K; ++k) denom = denom + s[ids[k]];
+    denom = denom + 1e-20f;
+    for (int k = 0; k < K; ++k) w[k] = (s[ids[k]] / denom) * scale;
+  }
+  free(s);
+  free(c);
+  free(ok);
+  free(gscore);
+  free(gsel);
+}
+
+/* -------------------------------------------------------------------- align */
+
+/* Stable counting sort by expert (moe_pre_sorted / moe_pre_small index outputs,
+ * compressed_tensors_moe.py:172-207). ids outside [0,E) get moe_index -1. */
+ORC_API void orc_align(const int32_t* ids, int P, int E, int32_t* moe_index, int32_t* sorted_src,
+                       int32_t* expert_m, int32_t* lod) {
+  int32_t* cnt = (int32_t*)calloc((size_t)E, sizeof(int32_t));
+  for (int j = 0; j < P; ++j)
+    if (ids[j] >= 0 && ids[j] < E) cnt[ids[j]]++;
+  lod[0] = 0;
+  for (int e = 0; e < E; ++e) lod[e + 1] = lod[e] + cnt[e];
+  if (expert_m) memcpy(expert_m, cnt, sizeof(int32_t) * (size_t)E);
+  memset(cnt, 0, sizeof(int32_t) * (size_t)E);
+  for (int j = 0; j < P; ++j) {
+    const int e = ids[j];
+    if (e < 0 || e >= E) {
+      moe_index[j] = -1;
+      continue;
+    }
+    const int pos = lod[e] + cnt[e]++;
+    moe_index[j] = pos;
+    if (sorted_src) sorted_src[pos] = j;
+  }
+  free(cnt);
+}
+
+/* gen_block_statistic (compressed_tensors_moe.py:186): per-block histograms. */
+ORC_API void orc_block_statistic(const int32_t* ids, int P, int E, int n_blocks, int32_t* out) {
+  int per = (P + n_blocks - 1) / n_blocks;
+  if (per < 1) per = 1;
+  memset(out, 0, sizeof(int32_t) * (size_t)n_blocks * (size_t)E);
+  for (int j = 0; j < P; ++j)
+    if (ids[j] >= 0 && ids[j] < E) out[(size_t)(j / per) * E + ids[j]]++;
+}
+
+/* ------------------------------------------------------------------- quant */
+
+/* quant2d (compressed_tensors_moe.py:224,253): per-row absmax int8; `max` out. */
+ORC_API void orc_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q,
+                               float* row_max) {
+#pragma omp parallel for schedule(static)
+  for (int r = 0; r < R; ++r) {
+    const uint16_t* xr = x + (size_t)r * ld_x;
+    float amax = 0.0f;
+    for (int c = 0; c < C; ++c) amax = fmaxf(amax, fabsf(bf16_to_f32(xr[c])));
+    const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+    for (int c = 0; c < C; ++c) {
+      float f = rintf(bf16_to_f32(xr[c]) * inv);
+      f = fminf(fmaxf(f, -127.0f), 127.0f);
+      q[(size_t)r * ld_q + c] = (int8_t)(int)f;
+    }
+    row_max[r] = amax;
+  }
+}
+
+/* OCP e4m3fn encoding by exhaustive nearest-value search (ties to even code). */
+static float e4m3fn_value(int code) { /* code in [0,127), positive */
+  const int ex = code >> 3, man = code & 7;
+  return ex == 0 ? ldexpf((float)man, -9) : ldexpf(1.0f + (float)man / 8.0f, ex - 7);
+}
+
+ORC_API uint8_t orc_f32_to_e4m3fn(float f) {
+  const uint8_t sign = signbit(f) ? 0x80 : 0;
+  const float a = fabsf(f);
+  if (!(a < 448.0f)) return (uint8_t)(sign | 0x7e);
+  int best = 0;
+  double bestd = fabs((double)a - 0.0);
+  for (int code = 1; code <= 0x7e; ++code) {
+    const double d = fabs((double)a - (double)e4m3fn_value(code));
+    if (d < bestd || (d == bestd && (code & 1) == 0 && (best & 1) == 1)) {
+      best = code;
+      bestd = d;
+    }
+  }
+  return (uint8_t)(sign | best);
+}
+
+ORC_API float orc_e4m3fn_to_f32(uint8_t b) {
+  const float v = e4m3fn_value(b & 0x7f);
+  return (b & 0x80) ? -v : v;
+}
+
+/* Per-row, per-128-column fp8 quantisation (no reference counterpart; DeepSeek-V3 recipe). */
+ORC_API void orc_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, int C, uint8_t* q, int64_t ld_q,
+                                    float* scale) {
+  const int G = C / 128;
+#pragma omp parallel for schedule(static)
+  for (int r = 0; r < R; ++r) {
+    for (int g = 0; g < G; ++g) {
+      const uint16_t* xr = x + (size_t)r * ld_x + g * 128;
+      float amax = 0.0f;
+      for (int c = 0; c < 128; ++c) amax = fmaxf(amax, fabsf(bf16_to_f32(xr[c])));
+      const float s = amax / 448.0f;
+      for (int c = 0; c < 128; ++c)
+        q[(size_t)r * ld_q + g * 128 + c] = orc_f32_to_e4m3fn(s > 0.0f ? bf16_to_f32(xr[c]) / s : 0.0f);
+      scale[(size_t)r * G + g] = s;
+    }
+  }
+}
+
+/* -------------------------------------------------------------- grouped GEMM */
+
+__attribute__((target_clones("arch=skylake-avx512", "avx2", "default"))) static int32_t dot_i8(const int8_t* a,
+                                                                                    const int8_t* b, int k) {
+  int32_t acc = 0;
+  for (int i = 0; i < k; ++i) acc += (int32_t)a[i] * (int32_t)b[i];
+  return acc;
+}
+
+/* moe_fc in its int8 form (compressed_tensors_moe.py:226-238, 263-275): rows
+ * [lod[e], lod[e+1]) times weight[e]^T, exact int32, dequant by the two maxes.
+ * act = 1 fuses silu_and_mul (ops/_custom_ops.py:699-706; gate = first half). */
+ORC_API void orc_grouped_gemm_i8(const int8_t* a, int64_t lda, const float* a_max, const int32_t* row_src,
+                                 int src_div, const int8_t* w, const float* w_max, const int32_t* lod, int E,
+                                 int n, int k, uint16_t* y, int64_t ldy, int32_t* acc_out, int act) {
+  for (int e = 0; e < E; ++e) {
+    const int r0 = lod[e], r1 = lod[e + 1];
+    const int8_t* we = w + (size_t)e * n * k;
+    const float* wm = w_max + (size_t)e * n;
+#pragma omp parallel for schedule(static)
+    for (int r = r0; r < r1; ++r) {
+      const int sr = row_src ? row_src[r] / src_div : r;
+      const int8_t* ar = a + (size_t)sr * lda;
+      const float sa = a_max[sr] / 127.0f;
+      const int half = n / 2;
+      if (act == 0) {
+        for (int c = 0; c < n; ++c) {
+          const int32_t acc = dot_i8(ar, we + (size_t)c * k, k);
+          if (acc_out) acc_out[(size_t)r * n + c] = acc;
+          if (y) y[(size_t)r * ldy + c] = f32_to_bf16(((float)acc * sa) * (wm[c] / 127.0f));
+        }
+      } else {
+        for (int c = 0; c < half; ++c) {
+          const int32_t ag = dot_i8(ar, we + (size_t)c * k, k);
+          const int32_t au = dot_i8(ar, we + (size_t)(half + c) * k, k);
+          if (acc_out) {
+            acc_out[(size_t)r * n + c] = ag;
+            acc_out[(size_t)r * n + half + c] = au;
+          }
+          const uint16_t yg = f32_to_bf16(((float)ag * sa) * (wm[c] / 127.0f));
+          const uint16_t yu = f32_to_bf16(((float)au * sa) * (wm[half + c] / 127.0f));
+          if (y) y[(size_t)r * ldy + c] = f32_to_bf16(orc_silu(bf16_to_f32(yg)) * bf16_to_f32(yu));
+        }
+      }
+    }
+  }
+}
+
+/* silu_and_mul on a stored gate_up tensor (compressed_tensors_moe.py:240-243). */
+ORC_API void orc_silu_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, uint16_t* out, int64_t ld_out) {
+  for (int r = 0; r < R; ++r)
+    for (int i = 0; i < I; ++i)
+      out[(size_t)r * ld_out + i] = f32_to_bf16(orc_silu(bf16_to_f32(y[(size_t)r * ld_y + i])) *
+                                                 bf16_to_f32(y[(size_t)r * ld_y + I + i]));
+}
+
+/* moe_post (compressed_tensors_moe.py:278-290): weighted top-K sum, f32
+ * weights, f32 accumulate over ascending k, one bf16 rounding; then the caller
+ * epilogue of models/deepseek_v2.py:288-296 when requested. */
+ORC_API void orc_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_index, const float* topk_w,
+                         const float* dq, int M, int K, int H, float out_scale, const uint16_t* addend,
+                         int64_t ld_addend, uint16_t* out, int64_t ld_out) {
+  const int epilogue = (out_scale != 1.0f) || addend;
+#pragma omp parallel for schedule(static)
+  for (int m = 0; m < M; ++m) {
+    for (int h = 0; h < H; ++h) {
+      float acc = 0.0f;
+      for (int k = 0; k < K; ++k) {
+        const size_t j = (size_t)m * K + k;
+        const int r = moe_index[j];
+        if (r < 0) continue;
+        const float wt = dq ? topk_w[j] * dq[j] : topk_w[j];
+        acc = fmaf(wt, bf16_to_f32(x[(size_t)r * ld_x + h]), acc);
+      }
+      uint16_t o = f32_to_bf16(acc);
+      if (epilogue) {
+        o = f32_to_bf16(bf16_to_f32(o) * out_scale);
+        if (addend) o = f32_to_bf16(bf16_to_f32(o) + bf16_to_f32(addend[(size_t)m * ld_addend + h]));
+      }
+      out[(size_t)m * ld_out + h] = o;
+    }
+  }
+}
+
+/* ------------------------------------------------------------ whole layer */
+
+/* apply_monolithic restated: the eight stages of compressed_tensors_moe.py:151-291
+ * (+ shared expert per quantization/kernels/scale_mm.py:52-90 and the caller
+ * epilogue models/deepseek_v2.py:288-296). Optional outputs expose the
+ * intermediates the parity tests compare bit for bit. scoring: 0 softmax, 1 sigmoid. */
+ORC_API void orc_forward_w8a8(int M, int H, int E, int K, int I, int scoring, int renorm, int n_group,
+                              int topk_group, float routed_scale, const float* logits, const float* bias,
+                              const uint16_t* x, const int8_t* w13, const float* w13_max, const int8_t* w2,
+                              const float* w2_max, int I_shared, const int8_t* ws13, const float* ws13_max,
+                              const int8_t* ws2, const float* ws2_max, float out_scale, uint16_t* out,
+                              /* optional intermediates (NULL to skip) */
+                              float* o_topk_w, int32_t* o_topk_ids, int32_t* o_moe_index, int32_t* o_lod,
+                              int8_t* o_actq, float* o_actmax, uint16_t* o_down) {
+  const int P = M * K;
+  float* topk_w = (float*)malloc(sizeof(float) * (size_t)(P ? P : 1));
+  int32_t* topk_ids = (int32_t*)malloc(sizeof(int32_t) * (size_t)(P ? P : 1));
+  int32_t* moe_index = (int32_t*)malloc(sizeof(int32_t) * (size_t)(P ? P : 1));
+  int32_t* sorted_src = (int32_t*)malloc(sizeof(int32_t) * (size_t)(P ? P : 1));
+  int32_t* lod = (int32_t*)malloc(sizeof(int32_t) * (size_t)(E + 1));
+  int8_t* xq = (int8_t*)malloc((size_t)M * H + 1);
+  float* xmax = (float*)malloc(sizeof(float) * (size_t)(M ? M : 1));
+  uint16_t* act = (uint16_t*)malloc(sizeof(uint16_t) * ((size_t)P * I + 1));
+  int8_t* actq = (int8_t*)malloc((size_t)P * I + 1);
+  float* actmax = (float*)malloc(sizeof(float) * (size_t)(P ? P : 1));
+  uint16_t* down = (uint16_t*)malloc(sizeof(uint16_t) * ((size_t)P * H + 1));
+
+  if (scoring == 0)
+    orc_softmax_topk(logits, M, E, K, renorm, topk_w, topk_ids);
+  else
+    orc_sigmoid_group_topk_norm(logits, bias, M, E, K, n_group, topk_group, routed_scale, topk_w, topk_ids);
+  orc_align(topk_ids, P, E, moe_index, sorted_src, NULL, lod);
+  /* quant2d of the expanded rows == quant of each token row once */
+  orc_quant_i8_rows(x, H, M, H, xq, H, xmax);
+  orc_grouped_gemm_i8(xq, H, xmax, sorted_src, K, w13, w13_max, lod, E, 2 * I, H, act, I, NULL, 1);
+  orc_quant_i8_rows(act, I, P, I, actq, I, actmax);
+  orc_grouped_gemm_i8(actq, I, actmax, NULL, 1, w2, w2_max, lod, E, H, I, down, H, NULL, 0);
+
+  uint16_t* sh_out = NULL;
+  if (I_shared > 0) {
+    const int Is = I_shared;
+    const int32_t dlod[2] = {0, M};
+    uint16_t* sact = (uint16_t*)malloc(sizeof(uint16_t) * ((size_t)M * Is + 1));
+    int8_t* sq = (int8_t*)malloc((size_t)M * Is + 1);
+    float* smax = (float*)malloc(sizeof(float) * (size_t)(M ? M : 1));
+    sh_out = (uint16_t*)malloc(sizeof(uint16_t) * ((size_t)M * H + 1));
+    orc_grouped_gemm_i8(xq, H, xmax, NULL, 1, ws13, ws13_max, dlod, 1, 2 * Is, H, sact, Is, NULL, 1);
+    orc_quant_i8_rows(sact, Is, M, Is, sq, Is, smax);
+    orc_grouped_gemm_i8(sq, Is, smax, NULL, 1, ws2, ws2_max, dlod, 1, H, Is, sh_out, H, NULL, 0);
+    free(sact);
+    free(sq);
+    free(smax);
+  }
+  orc_combine(down, H, moe_index, topk_w, NULL, M, K, H, out_scale, sh_out, H, out, H);
+
+  if (o_topk_w) memcpy(o_topk_w, topk_w, sizeof(float) * (size_t)P);
+  if (o_topk_ids) memcpy(o_topk_ids, topk_ids, sizeof(int32_t) * (size_t)P);
+  if (o_moe_index) memcpy(o_moe_index, moe_index, sizeof(int32_t) * (size_t)P);
+  if (o_lod) memcpy(o_lod, lod, sizeof(int32_t) * (size_t)(E + 1));
+  if (o_actq) memcpy(o_actq, actq, (size_t)P * I);
+  if (o_actmax) memcpy(o_actmax, actmax, sizeof(float) * (size_t)P);
+  if (o_down) memcpy(o_down, down, sizeof(uint16_t) * (size_t)P * H);
+  free(topk_w);
+  free(topk_ids);
+  free(moe_index);
+  free(sorted_src);
+  free(lod);
+  free(xq);
+  free(xmax);
+  free(act);
+  free(actq);
+  free(actmax);
+  free(down);
+  free(sh_out);
+}

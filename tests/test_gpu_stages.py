@@ -1,0 +1,304 @@
+"""GPU parity, stage by stage: every kernel is called through the C ABI (ctypes on
+libkmoe.so) and compared with the C oracle on the same seeded inputs.
+
+Bars: routing ids, sort maps, int8 codes, int32 accumulators — bit-exact.
+bf16/f32 stage outputs — bit-exact too, because oracle and kernels perform the
+same fixed float sequences; the looser north-star tolerance (rel-L2 <= 1e-2) is
+asserted against the independently written torch oracle in test_gpu_layer.py.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import bits, from_bits
+
+pytestmark = pytest.mark.gpu
+
+from oracle import c_oracle as co  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def L():
+    from vllm_kunlun_amd import _lib
+    return _lib
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.view(dtype)
+    return t.cuda()
+
+
+def sync():
+    torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------ routing
+@pytest.mark.parametrize("M,E,K", [(32, 8, 2), (64, 128, 8), (1000, 128, 8), (7, 60, 6), (33, 384, 8), (5, 1024, 64),
+                                   (1, 1, 1), (3, 65, 65 // 2)])
+@pytest.mark.parametrize("renorm", [0, 1])
+def test_softmax_topk(L, M, E, K, renorm):
+    rng = np.random.default_rng(M * 1000 + E + K)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    logits[0, : min(E, 4)] = 0.5  # exact ties: lower id must win
+    w_ref, ids_ref = co.softmax_topk(logits, K, renorm)
+    d_logits = dev(logits)
+    w = torch.empty(M, K, dtype=torch.float32, device="cuda")
+    ids = torch.empty(M, K, dtype=torch.int32, device="cuda")
+    L.check(L.lib.kmoe_softmax_topk(L.ptr(d_logits), M, E, K, renorm, L.ptr(w), L.ptr(ids), L.stream()))
+    sync()
+    assert np.array_equal(ids.cpu().numpy(), ids_ref)
+    assert np.array_equal(w.cpu().numpy().view(np.uint32), w_ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("M,E,K,ng,tg", [(128, 256, 8, 8, 4), (64, 384, 8, 1, 1), (17, 64, 6, 4, 2),
+                                         (9, 16, 4, 8, 2), (300, 256, 8, 8, 4), (4, 1024, 8, 16, 4)])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_sigmoid_group_topk(L, M, E, K, ng, tg, with_bias):
+    rng = np.random.default_rng(M + E + K + ng)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    bias = (rng.standard_normal(E) * 0.01).astype(np.float32) if with_bias else None
+    w_ref, ids_ref = co.sigmoid_group_topk_norm(logits, bias, K, ng, tg, 2.5)
+    w = torch.empty(M, K, dtype=torch.float32, device="cuda")
+    ids = torch.empty(M, K, dtype=torch.int32, device="cuda")
+    d_logits = dev(logits)
+    d_bias = None if bias is None else dev(bias)
+    L.check(L.lib.kmoe_sigmoid_group_topk_norm(L.ptr(d_logits), L.ptr(d_bias), M, E, K, ng, tg, 2.5, L.ptr(w),
+                                               L.ptr(ids), L.stream()))
+    sync()
+    assert np.array_equal(ids.cpu().numpy(), ids_ref)
+    assert np.array_equal(w.cpu().numpy().view(np.uint32), w_ref.view(np.uint32))
+
+
+# -------------------------------------------------------------------- align
+def _run_align(L, ids_np, E):
+    P = ids_np.size
+    d_ids = dev(ids_np.astype(np.int32))
+    moe_index = torch.full((P,), -7, dtype=torch.int32, device="cuda")
+    sorted_src = torch.full((P,), -7, dtype=torch.int32, device="cuda")
+    expert_m = torch.empty(E, dtype=torch.int32, device="cuda")
+    lod = torch.empty(E + 1, dtype=torch.int32, device="cuda")
+    nbytes = L.lib.kmoe_align_workspace_bytes(P, E)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    L.check(L.lib.kmoe_align(L.ptr(d_ids), P, E, L.ptr(moe_index), L.ptr(sorted_src), L.ptr(expert_m), L.ptr(lod),
+                             L.ptr(ws), nbytes, L.stream()))
+    sync()
+    return moe_index.cpu().numpy(), sorted_src.cpu().numpy(), expert_m.cpu().numpy(), lod.cpu().numpy()
+
+
+@pytest.mark.parametrize("P,E,kind", [(0, 8, "uniform"), (1, 8, "uniform"), (64, 8, "uniform"), (512, 128, "uniform"),
+                                      (1024, 256, "uniform"), (1000, 384, "skew"), (8192, 128, "skew"),
+                                      (8193, 128, "uniform"), (65536, 128, "skew"), (32768, 256, "uniform"),
+                                      (40000, 1024, "onehot"), (5000, 33, "holes")])
+def test_align(L, P, E, kind):
+    rng = np.random.default_rng(P + E)
+    if kind == "uniform":
+        ids = rng.integers(0, E, P)
+    elif kind == "skew":
+        p = np.ones(E)
+        p[:: max(1, E // 8)] += 20.0
+        ids = rng.choice(E, P, p=p / p.sum())
+    elif kind == "onehot":
+        ids = np.full(P, E - 1)
+    else:  # experts that nobody picks
+        ids = rng.integers(0, E // 3, P) * 3
+    mi_ref, src_ref, em_ref, lod_ref = co.align(ids, E)
+    mi, src, em, lod = _run_align(L, ids, E)
+    assert np.array_equal(lod, lod_ref)
+    assert np.array_equal(em, em_ref)
+    assert np.array_equal(mi, mi_ref)
+    assert np.array_equal(src, src_ref)
+
+
+def test_align_skips_out_of_range_ids(L):
+    ids = np.array([3, -1, 2, 99, 3, 0, 2, 3], dtype=np.int32)
+    mi_ref, src_ref, em_ref, lod_ref = co.align(ids, 4)
+    mi, src, em, lod = _run_align(L, ids, 4)
+    assert np.array_equal(mi, mi_ref) and np.array_equal(lod, lod_ref) and np.array_equal(em, em_ref)
+    assert np.array_equal(src[: lod[-1]], src_ref[: lod_ref[-1]])
+
+
+@pytest.mark.parametrize("P,E,B", [(512, 128, 12), (65536, 128, 12), (7, 8, 12)])
+def test_block_statistic(L, P, E, B):
+    ids = np.random.default_rng(P).integers(0, E, P).astype(np.int32)
+    out = torch.empty(B, E, dtype=torch.int32, device="cuda")
+    L.check(L.lib.kmoe_block_statistic(L.ptr(dev(ids)), P, E, B, L.ptr(out), L.stream()))
+    sync()
+    got = out.cpu().numpy()
+    assert np.array_equal(got, co.block_statistic(ids, E, B))
+    assert np.array_equal(got.sum(0), np.bincount(ids, minlength=E))
+
+
+def test_gather_rows(L):
+    M, K, H, E = 37, 4, 256, 16
+    x = torch.randn(M, H).bfloat16().cuda()
+    ids = np.random.default_rng(0).integers(0, E, M * K).astype(np.int32)
+    _, src, _, _ = co.align(ids, E)
+    out = torch.empty(M * K, H, dtype=torch.bfloat16, device="cuda")
+    L.check(L.lib.kmoe_gather_rows(L.ptr(x), H, L.ptr(dev(src)), M * K, K, H, L.ptr(out), H, L.stream()))
+    sync()
+    assert torch.equal(out.cpu(), x.cpu()[torch.from_numpy(src // K).long()])
+
+
+# -------------------------------------------------------------------- quant
+@pytest.mark.parametrize("R,Cc", [(1, 8), (5, 256), (64, 2048), (100, 768), (33, 7168), (3, 16384), (7, 1000),
+                                  (512, 2048)])
+def test_quant_i8_rows(L, R, Cc):
+    torch.manual_seed(R + Cc)
+    x = (torch.randn(R, Cc) * torch.rand(R, 1) * 4).bfloat16()
+    x[0] = 0  # all-zero row
+    if R > 2:
+        x[1, :] = 0.5  # constant row: every element is the max
+        x[2, Cc // 2] = 300.0
+    q_ref, mx_ref = co.quant_i8_rows(bits(x))
+    dx = x.cuda()
+    q = torch.empty(R, Cc, dtype=torch.int8, device="cuda")
+    mx = torch.empty(R, dtype=torch.float32, device="cuda")
+    L.check(L.lib.kmoe_quant_i8_rows(L.ptr(dx), Cc, R, Cc, L.ptr(q), Cc, L.ptr(mx), L.stream()))
+    sync()
+    assert np.array_equal(mx.cpu().numpy().view(np.uint32), mx_ref.view(np.uint32))
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+
+
+@pytest.mark.parametrize("R,Cc", [(1, 128), (17, 2048), (64, 7168), (5, 384)])
+def test_quant_fp8_group128(L, R, Cc):
+    torch.manual_seed(R + Cc)
+    x = (torch.randn(R, Cc) * torch.rand(R, 1) * 4).bfloat16()
+    x[0, :128] = 0
+    x[0, 130] = 2.0 ** -12
+    q_ref, s_ref = co.quant_fp8_group128(bits(x))
+    dx = x.cuda()
+    q = torch.empty(R, Cc, dtype=torch.uint8, device="cuda")
+    s = torch.empty(R, Cc // 128, dtype=torch.float32, device="cuda")
+    L.check(L.lib.kmoe_quant_fp8_group128(L.ptr(dx), Cc, R, Cc, L.ptr(q), Cc, L.ptr(s), L.stream()))
+    sync()
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), s_ref.view(np.uint32))
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+
+
+# --------------------------------------------------------------- grouped GEMM
+def _gemm_case(L, E, n, k, counts, act, variant, gather, seed=0):
+    """Runs one grouped GEMM on device and returns (y, acc, y_ref, acc_ref)."""
+    rng = np.random.default_rng(seed)
+    counts = np.asarray(counts, dtype=np.int32)
+    assert counts.size == E
+    lod = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(lod[-1])
+    w = rng.integers(-127, 128, (E, n, k), dtype=np.int8)
+    w_max = (rng.random((E, n)) * 0.1 + 0.01).astype(np.float32)
+    if gather:
+        src_div = 4
+        a_rows = max(1, (rows + src_div - 1) // src_div)
+        row_src = rng.permutation(a_rows * src_div)[:rows].astype(np.int32)
+    else:
+        src_div, a_rows, row_src = 1, max(rows, 1), None
+    a = rng.integers(-127, 128, (a_rows, k), dtype=np.int8)
+    a_max = (rng.random(a_rows) * 4 + 0.1).astype(np.float32)
+    y_ref, acc_ref = co.grouped_gemm_i8(a, a_max, w, w_max, lod, act=act, row_src=row_src, src_div=src_div,
+                                        want_acc=True)
+    n_out = n // 2 if act else n
+    d = dict(a=dev(a), a_max=dev(a_max), w=dev(w), w_max=dev(w_max), lod=dev(lod),
+             row_src=None if row_src is None else dev(row_src))
+    y = torch.zeros(max(rows, 1), n_out, dtype=torch.bfloat16, device="cuda")
+    acc = torch.zeros(max(rows, 1), n, dtype=torch.int32, device="cuda")
+    args = L.GemmI8Args()
+    args.a, args.lda, args.a_max = d["a"].data_ptr(), k, d["a_max"].data_ptr()
+    args.row_src = 0 if row_src is None else d["row_src"].data_ptr()
+    args.src_div = src_div
+    args.w, args.w_max, args.lod = d["w"].data_ptr(), d["w_max"].data_ptr(), d["lod"].data_ptr()
+    args.E, args.n, args.k, args.rows = E, n, k, rows
+    args.y, args.ldy, args.acc_out = y.data_ptr(), n_out, acc.data_ptr()
+    args.act, args.variant = act, variant
+    L.check(L.lib.kmoe_grouped_gemm_i8(args, L.stream()))
+    sync()
+    return bits(y)[:rows], acc.cpu().numpy()[:rows], y_ref, acc_ref
+
+
+GEMM_CASES = [
+    # E, n, k, counts
+    (1, 64, 256, [16]),
+    (4, 64, 256, [3, 0, 17, 1]),
+    (8, 128, 512, [4, 4, 0, 9, 33, 1, 0, 2]),
+    (3, 96, 768, [5, 40, 7]),          # n not a multiple of the workgroup's channel span
+    (2, 256, 2048, [130, 129]),
+    (5, 1536, 64, [1, 2, 3, 4, 5]),    # k shorter than one 256-byte chunk
+    (2, 64, 272, [20, 3]),             # k = 256 + 16: ragged last chunk
+    (16, 192, 384, [0] * 15 + [300]),  # everything on one expert
+]
+
+
+@pytest.mark.parametrize("E,n,k,counts", GEMM_CASES)
+@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("act", [0, 1])
+@pytest.mark.parametrize("gather", [False, True])
+def test_grouped_gemm_i8(L, E, n, k, counts, variant, act, gather):
+    if act and n % 32:
+        pytest.skip("SwiGLU needs n % 32 == 0")
+    y, acc, y_ref, acc_ref = _gemm_case(L, E, n, k, counts, act, variant, gather, seed=E * n + k)
+    assert np.array_equal(acc, acc_ref), "int32 accumulators differ"
+    assert np.array_equal(y, y_ref), "bf16 outputs differ"
+
+
+def test_grouped_gemm_i8_extreme_values(L):
+    """All operands at +-127: the largest accumulators the path can produce."""
+    E, n, k, rows = 1, 32, 7168, 16
+    a = np.full((rows, k), 127, np.int8)
+    a[1::2] = -127
+    w = np.full((E, n, k), 127, np.int8)
+    w[:, 1::2] = -127
+    lod = np.array([0, rows], np.int32)
+    y_ref, acc_ref = co.grouped_gemm_i8(a, np.ones(rows, np.float32), w, np.ones((E, n), np.float32), lod,
+                                        want_acc=True)
+    assert abs(int(acc_ref[0, 0])) == 127 * 127 * k
+    d = dict(a=dev(a), a_max=torch.ones(rows, device="cuda"), w=dev(w), w_max=torch.ones(E, n, device="cuda"),
+             lod=dev(lod))
+    y = torch.zeros(rows, n, dtype=torch.bfloat16, device="cuda")
+    acc = torch.zeros(rows, n, dtype=torch.int32, device="cuda")
+    args = L.GemmI8Args()
+    args.a, args.lda, args.a_max = d["a"].data_ptr(), k, d["a_max"].data_ptr()
+    args.src_div = 1
+    args.w, args.w_max, args.lod = d["w"].data_ptr(), d["w_max"].data_ptr(), d["lod"].data_ptr()
+    args.E, args.n, args.k, args.rows = E, n, k, rows
+    args.y, args.ldy, args.acc_out = y.data_ptr(), n, acc.data_ptr()
+    L.check(L.lib.kmoe_grouped_gemm_i8(args, L.stream()))
+    sync()
+    assert np.array_equal(acc.cpu().numpy(), acc_ref)
+    assert np.array_equal(bits(y), y_ref)
+
+
+# -------------------------------------------------------------- elementwise
+@pytest.mark.parametrize("R,I", [(1, 8), (33, 768), (512, 2048)])
+def test_silu_and_mul(L, R, I):
+    torch.manual_seed(R)
+    y = (torch.randn(R, 2 * I) * 3).bfloat16()
+    y[0, :4] = torch.tensor([0.0, -100.0, 100.0, -0.0]).bfloat16()
+    ref = co.silu_and_mul(bits(y))
+    out = torch.empty(R, I, dtype=torch.bfloat16, device="cuda")
+    dy = y.cuda()
+    L.check(L.lib.kmoe_silu_and_mul(L.ptr(dy), 2 * I, R, I, L.ptr(out), I, L.stream()))
+    sync()
+    assert np.array_equal(bits(out), ref)
+
+
+@pytest.mark.parametrize("M,K,H", [(1, 1, 8), (64, 8, 2048), (33, 6, 7168), (128, 8, 512)])
+@pytest.mark.parametrize("epilogue", [False, True])
+def test_combine(L, M, K, H, epilogue):
+    torch.manual_seed(M + K)
+    P = M * K
+    x = torch.randn(P, H).bfloat16()
+    w = torch.rand(M, K)
+    dq = torch.rand(M, K) + 0.5
+    perm = torch.randperm(P).int()
+    addend = torch.randn(M, H).bfloat16() if epilogue else None
+    scale = 2.5 if epilogue else 1.0
+    ref = co.combine(bits(x), perm.numpy(), w.numpy(), dq.numpy(), scale, None if addend is None else bits(addend))
+    out = torch.empty(M, H, dtype=torch.bfloat16, device="cuda")
+    d = [t.cuda() for t in (x, perm, w, dq)]
+    dadd = None if addend is None else addend.cuda()
+    L.check(L.lib.kmoe_combine(L.ptr(d[0]), H, L.ptr(d[1]), L.ptr(d[2]), L.ptr(d[3]), M, K, H, scale, L.ptr(dadd), H,
+                               L.ptr(out), H, L.stream()))
+    sync()
+    assert np.array_equal(bits(out), ref)

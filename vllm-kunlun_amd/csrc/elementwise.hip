@@ -1,0 +1,275 @@
+// Bandwidth-bound stages: per-row int8 quantisation, per-group fp8 quantisation,
+// SiLU-and-mul, and the weighted top-K combine. All move 16 bytes per lane.
+#include "kmoe_common.h"
+
+namespace kmoe {
+namespace {
+
+union Pack8 {  // 8 bf16
+  uint4 v;
+  uint16_t h[8];
+};
+
+// ---------------------------------------------------------------- int8 rows
+// TPR threads cooperate on one row; each keeps NV vectors of 8 values in
+// registers, so the row is read from memory once.
+template <int TPR, int NV>
+__global__ __launch_bounds__(256) void quant_i8_rows_kernel(const uint16_t* __restrict__ x, int64_t ld_x, int R,
+                                                           int C, int8_t* __restrict__ q, int64_t ld_q,
+                                                           float* __restrict__ row_max) {
+  constexpr int kRowsPerBlock = 256 / TPR;
+  __shared__ float red[256 / kWave];
+  const int sub = threadIdx.x / TPR;
+  const int t = threadIdx.x % TPR;
+  const int r = blockIdx.x * kRowsPerBlock + sub;
+  const bool live = r < R;
+  const int nvec = C / 8;
+  Pack8 val[NV];
+  float amax = 0.0f;
+  if (live) {
+    const uint4* src = reinterpret_cast<const uint4*>(x + static_cast<size_t>(r) * ld_x);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = t + i * TPR;
+      if (v < nvec) {
+        val[i].v = src[v];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(bf16_to_f32(val[i].h[j])));
+      }
+    }
+  }
+  amax = wave_max(amax);
+  if (TPR > kWave) {  // one row per block: combine the waves
+    if (lane_id() == 0) red[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = red[0];
+#pragma unroll
+    for (int w = 1; w < TPR / kWave; ++w) amax = fmaxf(amax, red[w]);
+  }
+  if (!live) return;
+  const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+  uint2* dst = reinterpret_cast<uint2*>(q + static_cast<size_t>(r) * ld_q);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = t + i * TPR;
+    if (v < nvec) {
+      uint32_t w[2] = {0, 0};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float f = __builtin_rintf(bf16_to_f32(val[i].h[j]) * inv);
+        f = fminf(fmaxf(f, -127.0f), 127.0f);
+        const int qi = static_cast<int>(f);
+        w[j >> 2] |= static_cast<uint32_t>(qi & 0xff) << (8 * (j & 3));
+      }
+      dst[v] = make_uint2(w[0], w[1]);
+    }
+  }
+  if (t == 0) row_max[r] = amax;
+}
+
+// ------------------------------------------------------------- fp8 group128
+// OCP e4m3fn encode of a finite float, round-to-nearest-even, saturating at 448.
+__device__ inline uint8_t f32_to_e4m3fn(float f) {
+  union { float f; uint32_t u; } v;
+  v.f = f;
+  const uint32_t sign = (v.u >> 24) & 0x80u;
+  float a = fabsf(f);
+  if (!(a < 448.0f)) return static_cast<uint8_t>(sign | 0x7eu);  // saturate (and NaN -> max)
+  if (a < 0x1p-10f) return static_cast<uint8_t>(sign);           // below half the smallest subnormal
+  // Quantise to the grid: 3 mantissa bits for normals (>= 2^-6), step 2^-9 for subnormals.
+  int ex;
+  (void)__builtin_frexpf(a, &ex);  // a = m * 2^ex, m in [0.5,1)
+  int e = ex - 1;                  // a in [2^e, 2^(e+1))
+  if (e < -6) e = -6;
+  const float step = __builtin_ldexpf(1.0f, e - 3);
+  const float qv = __builtin_rintf(a / step) * step;  // exact: step is a power of two
+  v.f = qv;
+  const int fe = static_cast<int>((v.u >> 23) & 0xff) - 127;
+  uint32_t bits;
+  if (qv < 0x1p-6f) {
+    bits = static_cast<uint32_t>(qv * 512.0f);  // subnormal: mantissa count of 2^-9
+  } else {
+    bits = (static_cast<uint32_t>(fe + 7) << 3) | ((v.u >> 20) & 0x7u);
+  }
+  return static_cast<uint8_t>(sign | bits);
+}
+
+// 16 lanes x 8 values = one 128-column group; 4 groups per wave.
+__global__ __launch_bounds__(256) void quant_fp8_group128_kernel(const uint16_t* __restrict__ x, int64_t ld_x,
+                                                                int R, int C, uint8_t* __restrict__ q,
+                                                                int64_t ld_q, float* __restrict__ scale) {
+  const int groups_per_row = C / 128;
+  const long long total = static_cast<long long>(R) * groups_per_row;
+  const long long gid = static_cast<long long>(blockIdx.x) * 16 + (threadIdx.x >> 4);
+  const int t = threadIdx.x & 15;
+  const bool live = gid < total;
+  const int r = live ? static_cast<int>(gid / groups_per_row) : 0;
+  const int g = live ? static_cast<int>(gid % groups_per_row) : 0;
+  Pack8 val;
+  val.v = make_uint4(0, 0, 0, 0);
+  if (live) val.v = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(r) * ld_x + g * 128 + t * 8);
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(bf16_to_f32(val.h[j])));
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, kWave));
+  if (!live) return;
+  const float s = amax / 448.0f;
+  uint32_t w[2] = {0, 0};
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float f = s > 0.0f ? bf16_to_f32(val.h[j]) / s : 0.0f;
+    w[j >> 2] |= static_cast<uint32_t>(f32_to_e4m3fn(f)) << (8 * (j & 3));
+  }
+  *reinterpret_cast<uint2*>(q + static_cast<size_t>(r) * ld_q + g * 128 + t * 8) = make_uint2(w[0], w[1]);
+  if (t == 0) scale[static_cast<size_t>(r) * groups_per_row + g] = s;
+}
+
+// ------------------------------------------------------------ silu-and-mul
+__global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __restrict__ y, int64_t ld_y, int R,
+                                                          int I, uint16_t* __restrict__ out, int64_t ld_out) {
+  const int vec_per_row = I / 8;
+  const long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= static_cast<long long>(R) * vec_per_row) return;
+  const int r = static_cast<int>(idx / vec_per_row);
+  const int c = static_cast<int>(idx % vec_per_row) * 8;
+  Pack8 g, u, o;
+  g.v = *reinterpret_cast<const uint4*>(y + static_cast<size_t>(r) * ld_y + c);
+  u.v = *reinterpret_cast<const uint4*>(y + static_cast<size_t>(r) * ld_y + I + c);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) o.h[j] = f32_to_bf16(silu_fixed(bf16_to_f32(g.h[j])) * bf16_to_f32(u.h[j]));
+  *reinterpret_cast<uint4*>(out + static_cast<size_t>(r) * ld_out + c) = o.v;
+}
+
+// ----------------------------------------------------------------- combine
+constexpr int kMaxTopK = 64;
+
+__global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict__ x, int64_t ld_x,
+                                                     const int32_t* __restrict__ moe_index,
+                                                     const float* __restrict__ topk_w,
+                                                     const float* __restrict__ dq, int K, int H, float out_scale,
+                                                     int epilogue, const uint16_t* __restrict__ addend,
+                                                     int64_t ld_addend, uint16_t* __restrict__ out,
+                                                     int64_t ld_out) {
+  __shared__ int rows[kMaxTopK];
+  __shared__ float wts[kMaxTopK];
+  const int m = blockIdx.x;
+  if (threadIdx.x < K) {
+    const size_t j = static_cast<size_t>(m) * K + threadIdx.x;
+    rows[threadIdx.x] = moe_index[j];
+    wts[threadIdx.x] = dq ? topk_w[j] * dq[j] : topk_w[j];
+  }
+  __syncthreads();
+  for (int c = threadIdx.x * 8; c < H; c += blockDim.x * 8) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int k = 0; k < K; ++k) {
+      const int r = rows[k];
+      if (r < 0) continue;  // pair without a sorted row contributes nothing
+      Pack8 p;
+      p.v = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(r) * ld_x + c);
+      const float w = wts[k];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(w, bf16_to_f32(p.h[j]), acc[j]);
+    }
+    Pack8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o.h[j] = f32_to_bf16(acc[j]);
+    if (epilogue) {
+      Pack8 a;
+      a.v = make_uint4(0, 0, 0, 0);
+      if (addend) a.v = *reinterpret_cast<const uint4*>(addend + static_cast<size_t>(m) * ld_addend + c);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint16_t scaled = f32_to_bf16(bf16_to_f32(o.h[j]) * out_scale);
+        o.h[j] = addend ? f32_to_bf16(bf16_to_f32(scaled) + bf16_to_f32(a.h[j])) : scaled;
+      }
+    }
+    *reinterpret_cast<uint4*>(out + static_cast<size_t>(m) * ld_out + c) = o.v;
+  }
+}
+
+__global__ void fill_dense_lod_kernel(int32_t* lod2, int rows) {
+  if (threadIdx.x == 0) lod2[0] = 0;
+  if (threadIdx.x == 1) lod2[1] = rows;
+}
+
+}  // namespace
+
+int fill_dense_lod(int32_t* lod2, int rows, hipStream_t stream) {
+  hipLaunchKernelGGL(fill_dense_lod_kernel, dim3(1), dim3(64), 0, stream, lod2, rows);
+  return check_launch("fill_dense_lod");
+}
+
+}  // namespace kmoe
+
+using namespace kmoe;
+
+extern "C" int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q,
+                                  float* row_max, kmoe_stream_t stream) {
+  KMOE_REQUIRE(x && q && row_max, KMOE_ERR_NULL, "quant_i8_rows: NULL pointer");
+  KMOE_REQUIRE(R >= 0 && C >= 8 && C % 8 == 0 && C <= 16384, KMOE_ERR_SHAPE,
+               "quant_i8_rows: R=%d C=%d (need C %% 8 == 0, 8 <= C <= 16384)", R, C);
+  KMOE_REQUIRE(ld_x % 8 == 0 && ld_q % 8 == 0 && ld_x >= C && ld_q >= C, KMOE_ERR_SHAPE,
+               "quant_i8_rows: row strides %lld/%lld must be multiples of 8 and >= C", (long long)ld_x,
+               (long long)ld_q);
+  if (R == 0) return KMOE_OK;
+  hipStream_t s = as_stream(stream);
+  if (C <= 64 * 8 * 2) {
+    hipLaunchKernelGGL((quant_i8_rows_kernel<64, 2>), dim3(ceil_div(R, 4)), dim3(256), 0, s, x, ld_x, R, C, q, ld_q,
+                       row_max);
+  } else if (C <= 64 * 8 * 4) {
+    hipLaunchKernelGGL((quant_i8_rows_kernel<64, 4>), dim3(ceil_div(R, 4)), dim3(256), 0, s, x, ld_x, R, C, q, ld_q,
+                       row_max);
+  } else if (C <= 256 * 8 * 4) {
+    hipLaunchKernelGGL((quant_i8_rows_kernel<256, 4>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max);
+  } else {
+    hipLaunchKernelGGL((quant_i8_rows_kernel<256, 8>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max);
+  }
+  return check_launch("kmoe_quant_i8_rows");
+}
+
+extern "C" int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, int C, uint8_t* q, int64_t ld_q,
+                                       float* scale, kmoe_stream_t stream) {
+  KMOE_REQUIRE(x && q && scale, KMOE_ERR_NULL, "quant_fp8_group128: NULL pointer");
+  KMOE_REQUIRE(R >= 0 && C >= 128 && C % 128 == 0, KMOE_ERR_SHAPE, "quant_fp8_group128: R=%d C=%d (need C %% 128 == 0)",
+               R, C);
+  KMOE_REQUIRE(ld_x % 8 == 0 && ld_q % 8 == 0 && ld_x >= C && ld_q >= C, KMOE_ERR_SHAPE,
+               "quant_fp8_group128: row strides %lld/%lld must be multiples of 8 and >= C", (long long)ld_x,
+               (long long)ld_q);
+  if (R == 0) return KMOE_OK;
+  const long long groups = static_cast<long long>(R) * (C / 128);
+  hipLaunchKernelGGL(quant_fp8_group128_kernel, dim3(static_cast<unsigned>((groups + 15) / 16)), dim3(256), 0,
+                     as_stream(stream), x, ld_x, R, C, q, ld_q, scale);
+  return check_launch("kmoe_quant_fp8_group128");
+}
+
+extern "C" int kmoe_silu_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, uint16_t* out, int64_t ld_out,
+                                 kmoe_stream_t stream) {
+  KMOE_REQUIRE(y && out, KMOE_ERR_NULL, "silu_and_mul: NULL pointer");
+  KMOE_REQUIRE(R >= 0 && I >= 8 && I % 8 == 0, KMOE_ERR_SHAPE, "silu_and_mul: R=%d I=%d (need I %% 8 == 0)", R, I);
+  KMOE_REQUIRE(ld_y % 8 == 0 && ld_out % 8 == 0 && ld_y >= 2 * I && ld_out >= I, KMOE_ERR_SHAPE,
+               "silu_and_mul: row strides %lld/%lld", (long long)ld_y, (long long)ld_out);
+  if (R == 0) return KMOE_OK;
+  const long long n = static_cast<long long>(R) * (I / 8);
+  hipLaunchKernelGGL(silu_and_mul_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0,
+                     as_stream(stream), y, ld_y, R, I, out, ld_out);
+  return check_launch("kmoe_silu_and_mul");
+}
+
+extern "C" int kmoe_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_index, const float* topk_w,
+                            const float* dequant_scale, int M, int K, int H, float out_scale,
+                            const uint16_t* addend, int64_t ld_addend, uint16_t* out, int64_t ld_out,
+                            kmoe_stream_t stream) {
+  KMOE_REQUIRE(x && moe_index && topk_w && out, KMOE_ERR_NULL, "combine: NULL pointer");
+  KMOE_REQUIRE(M >= 0 && K >= 1 && K <= kMaxTopK && H >= 8 && H % 8 == 0, KMOE_ERR_SHAPE,
+               "combine: M=%d K=%d H=%d (need 1 <= K <= 64, H %% 8 == 0)", M, K, H);
+  KMOE_REQUIRE(ld_x % 8 == 0 && ld_out % 8 == 0 && ld_x >= H && ld_out >= H, KMOE_ERR_SHAPE,
+               "combine: row strides %lld/%lld", (long long)ld_x, (long long)ld_out);
+  KMOE_REQUIRE(!addend || (ld_addend % 8 == 0 && ld_addend >= H), KMOE_ERR_SHAPE, "combine: addend stride %lld",
+               (long long)ld_addend);
+  if (M == 0) return KMOE_OK;
+  const int epilogue = (out_scale != 1.0f || addend) ? 1 : 0;
+  hipLaunchKernelGGL(combine_kernel, dim3(M), dim3(256), 0, as_stream(stream), x, ld_x, moe_index, topk_w,
+                     dequant_scale, K, H, out_scale, epilogue, addend, ld_addend, out, ld_out);
+  return check_launch("kmoe_combine");
+}

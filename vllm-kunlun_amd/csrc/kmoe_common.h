@@ -1,0 +1,109 @@
+// Shared device/host helpers for libkmoe (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kmoe.h"
+
+namespace kmoe {
+
+constexpr int kWave = 64;
+
+// ---- error plumbing (host) -------------------------------------------------
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+// Writes {0, rows} to lod2: the row offsets of a dense (single-expert) GEMM.
+int fill_dense_lod(int32_t* lod2, int rows, hipStream_t stream);
+
+#define KMOE_REQUIRE(cond, code, ...) \
+  do {                                \
+    if (!(cond)) return ::kmoe::fail((code), __VA_ARGS__); \
+  } while (0)
+
+// ---- bf16 <-> f32, bit-exact round-to-nearest-even --------------------------
+__host__ __device__ inline float bf16_to_f32(uint16_t h) {
+  union { uint32_t u; float f; } v;
+  v.u = static_cast<uint32_t>(h) << 16;
+  return v.f;
+}
+
+__host__ __device__ inline uint16_t f32_to_bf16(float f) {
+  union { uint32_t u; float f; } v;
+  v.f = f;
+  uint32_t u = v.u;
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<uint16_t>(u >> 16);
+}
+
+// ---- fixed-sequence transcendental -----------------------------------------
+// exp(x) as one fixed sequence of IEEE single operations (mul, round-to-even,
+// fma, exact power-of-two scaling), so that a CPU restatement performing the
+// same sequence gives the same bits. Argument clamped to [-86, 86] so neither
+// the result nor 1/(1+result) leaves the normal range. Error < 2 ulp.
+__device__ inline float exp_fixed(float x) {
+  x = fminf(fmaxf(x, -86.0f), 86.0f);
+  const float n = __builtin_rintf(x * 0x1.715476p+0f);            // x * log2(e)
+  float r = __builtin_fmaf(n, -0x1.62e4p-1f, x);                  // - n * ln2_hi
+  r = __builtin_fmaf(n, -0x1.7f7d1cp-20f, r);                     // - n * ln2_lo
+  float p = 0x1.a01a02p-13f;                                      // 1/5040
+  p = __builtin_fmaf(p, r, 0x1.6c16c2p-10f);                      // 1/720
+  p = __builtin_fmaf(p, r, 0x1.111112p-7f);                       // 1/120
+  p = __builtin_fmaf(p, r, 0x1.555556p-5f);                       // 1/24
+  p = __builtin_fmaf(p, r, 0x1.555556p-3f);                       // 1/6
+  p = __builtin_fmaf(p, r, 0.5f);
+  p = __builtin_fmaf(p, r, 1.0f);
+  p = __builtin_fmaf(p, r, 1.0f);
+  return __builtin_ldexpf(p, static_cast<int>(n));
+}
+
+__device__ inline float sigmoid_fixed(float x) { return 1.0f / (1.0f + exp_fixed(-x)); }
+__device__ inline float silu_fixed(float x) { return x / (1.0f + exp_fixed(-x)); }
+
+// ---- wave64 helpers ---------------------------------------------------------
+__device__ inline int lane_id() { return static_cast<int>(threadIdx.x) & (kWave - 1); }
+
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Butterfly sum: every lane ends with the same bits (each step adds the same
+// two numbers on both sides). Equivalent to the balanced binary tree
+// t[l] = t[l] + t[l + off], off = 32,16,...,1, over the 64 lane values.
+__device__ inline float wave_sum_tree(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = v + __shfl_xor(v, off, kWave);
+  return v;
+}
+
+__device__ inline int wave_sum_int(int v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+// (value, index) argmax with ties to the lower index; all lanes get the winner.
+__device__ inline void wave_argmax(float& v, int& idx) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(v, off, kWave);
+    const int oi = __shfl_xor(idx, off, kWave);
+    if (ov > v || (ov == v && oi < idx)) {
+      v = ov;
+      idx = oi;
+    }
+  }
+}
+
+__device__ inline uint64_t lanemask_lt() {
+  return (static_cast<uint64_t>(1) << lane_id()) - 1;
+}
+
+inline hipStream_t as_stream(kmoe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace kmoe

@@ -1,0 +1,342 @@
+"""torch.ops surface of the MoE path, backed by libkmoe.so.
+
+Same operator names, argument names/order and out-parameter style as the
+reference's shims in vllm_kunlun/ops/_custom_ops.py (each op cites its line
+there); the body of every op is one call through the C ABI on the current HIP
+stream. Nothing here computes with torch.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch.library import custom_op
+
+from .. import _lib as L
+
+_BF16 = torch.bfloat16
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _act_bits(t: torch.Tensor, what: str) -> torch.Tensor:
+    if t.dtype != _BF16:
+        raise NotImplementedError(f"{what}: activations must be bfloat16, got {t.dtype}")
+    return t
+
+
+# --------------------------------------------------------------------- routing
+@custom_op("_C::moe_softmax_topk", mutates_args=("normed_score", "topk_index"))
+def moe_softmax_topk(x: torch.Tensor, normed_score: torch.Tensor, topk_index: torch.Tensor,
+                     block_statistic: Optional[torch.Tensor], axis: int = -1, turn: bool = True) -> None:
+    """softmax + top-K without renormalisation (reference: ops/_custom_ops.py:781-790)."""
+    L.require_device(x, normed_score, topk_index)
+    L.require_contig(x, normed_score, topk_index)
+    _need(x.dtype == torch.float32 and normed_score.dtype == torch.float32 and topk_index.dtype == torch.int32,
+          "moe_softmax_topk: x/normed_score must be float32 and topk_index int32")
+    M, E = x.shape
+    _need(tuple(normed_score.shape) == tuple(topk_index.shape) and normed_score.shape[0] == M,
+          "moe_softmax_topk: output shapes must be [M, K]")
+    L.check(L.lib.kmoe_softmax_topk(L.ptr(x), M, E, normed_score.shape[1], 0, L.ptr(normed_score),
+                                    L.ptr(topk_index), L.stream()))
+
+
+@custom_op("_C::moe_softmax_topk_norm", mutates_args=("normed_score", "topk_index"))
+def moe_softmax_topk_norm(x: torch.Tensor, normed_score: torch.Tensor, topk_index: torch.Tensor,
+                          block_statistic: Optional[torch.Tensor], stable: bool = True) -> None:
+    """softmax + top-K + renormalise (reference: ops/_custom_ops.py:1084-1094).
+    `stable` is accepted for signature parity; ties always go to the lower expert id."""
+    L.require_device(x, normed_score, topk_index)
+    L.require_contig(x, normed_score, topk_index)
+    _need(x.dtype == torch.float32 and normed_score.dtype == torch.float32 and topk_index.dtype == torch.int32,
+          "moe_softmax_topk_norm: x/normed_score must be float32 and topk_index int32")
+    M, E = x.shape
+    _need(tuple(normed_score.shape) == tuple(topk_index.shape) and normed_score.shape[0] == M,
+          "moe_softmax_topk_norm: output shapes must be [M, K]")
+    L.check(L.lib.kmoe_softmax_topk(L.ptr(x), M, E, normed_score.shape[1], 1, L.ptr(normed_score),
+                                    L.ptr(topk_index), L.stream()))
+
+
+@custom_op("_C::moe_sigmoid_group_topk_norm", mutates_args=("topk_index", "norm_score", "block_static"))
+def moe_sigmoid_group_topk_norm(x: torch.Tensor, topk_index: torch.Tensor, norm_score: torch.Tensor,
+                                block_static: Optional[torch.Tensor], bias: Optional[torch.Tensor], scale: float,
+                                n_group: Optional[int], topk_group: Optional[int]) -> None:
+    """DeepSeek-V3 grouped top-K with correction bias (reference: ops/_custom_ops.py:1351-1371).
+    When block_static [B, E] is given it also receives the per-block histogram of the chosen ids."""
+    L.require_device(x, topk_index, norm_score, bias, block_static)
+    L.require_contig(x, topk_index, norm_score, bias, block_static)
+    _need(x.dtype == torch.float32 and norm_score.dtype == torch.float32 and topk_index.dtype == torch.int32,
+          "moe_sigmoid_group_topk_norm: x/norm_score must be float32 and topk_index int32")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == x.shape[1]),
+          "moe_sigmoid_group_topk_norm: bias must be float32 [E]")
+    M, E = x.shape
+    K = topk_index.shape[1]
+    L.check(L.lib.kmoe_sigmoid_group_topk_norm(L.ptr(x), L.ptr(bias), M, E, K, int(n_group or 1), int(topk_group or 1),
+                                               float(scale), L.ptr(norm_score), L.ptr(topk_index), L.stream()))
+    if block_static is not None and block_static.numel() > 0:
+        _need(block_static.dtype == torch.int32 and block_static.dim() == 2 and block_static.shape[1] == E,
+              "moe_sigmoid_group_topk_norm: block_static must be int32 [B, E]")
+        L.check(L.lib.kmoe_block_statistic(L.ptr(topk_index), M * K, E, block_static.shape[0], L.ptr(block_static),
+                                           L.stream()))
+
+
+@custom_op("_moe_C::topk_softmax", mutates_args=("topk_weights", "topk_ids", "token_expert_indices"))
+def topk_softmax(topk_weights: torch.Tensor, topk_ids: torch.Tensor, token_expert_indices: torch.Tensor,
+                 gating_output: torch.Tensor, renormalize: bool = False,
+                 e_score_correction_bias: Optional[torch.Tensor] = None) -> None:
+    """Upstream's non-monolithic routing op; an empty stub in the reference
+    (ops/_custom_ops.py:8-17, prototype csrc/xops.h:162-166), real here."""
+    if e_score_correction_bias is not None:
+        raise NotImplementedError("topk_softmax: correction bias belongs to moe_sigmoid_group_topk_norm")
+    L.require_device(topk_weights, topk_ids, gating_output)
+    L.require_contig(topk_weights, topk_ids, gating_output)
+    _need(gating_output.dtype == torch.float32 and topk_weights.dtype == torch.float32
+          and topk_ids.dtype == torch.int32, "topk_softmax: float32 scores/weights and int32 ids expected")
+    M, E = gating_output.shape
+    K = topk_ids.shape[1]
+    L.check(L.lib.kmoe_softmax_topk(L.ptr(gating_output), M, E, K, int(renormalize), L.ptr(topk_weights),
+                                    L.ptr(topk_ids), L.stream()))
+    if token_expert_indices.numel() == M * K:  # upstream convention: k * M + m
+        idx = torch.arange(K, device=topk_ids.device, dtype=torch.int32)[None, :] * M + \
+            torch.arange(M, device=topk_ids.device, dtype=torch.int32)[:, None]
+        token_expert_indices.copy_(idx)
+
+
+# ----------------------------------------------------------------------- align
+@custom_op("_C::gen_block_statistic", mutates_args=("block_statistic",))
+def gen_block_statistic(topk_ids: torch.Tensor, block_statistic: torch.Tensor) -> None:
+    """Per-block expert histogram [B, E] (reference: ops/_custom_ops.py:1123-1125)."""
+    L.require_device(topk_ids, block_statistic)
+    L.require_contig(topk_ids, block_statistic)
+    _need(topk_ids.dtype == torch.int32 and block_statistic.dtype == torch.int32 and block_statistic.dim() == 2,
+          "gen_block_statistic: int32 ids and int32 [B, E] histogram expected")
+    B, E = block_statistic.shape
+    L.check(L.lib.kmoe_block_statistic(L.ptr(topk_ids), topk_ids.numel(), E, B, L.ptr(block_statistic), L.stream()))
+
+
+def _align(topk_index: torch.Tensor, E: int, moe_index: torch.Tensor, sorted_src: torch.Tensor,
+           expert_m: Optional[torch.Tensor], lod: torch.Tensor) -> None:
+    P = topk_index.numel()
+    ws_bytes = L.lib.kmoe_align_workspace_bytes(P, E)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=topk_index.device)
+    L.check(L.lib.kmoe_align(L.ptr(topk_index), P, E, L.ptr(moe_index), L.ptr(sorted_src), L.ptr(expert_m),
+                             L.ptr(lod), L.ptr(ws), ws_bytes, L.stream()))
+
+
+@custom_op("_C::moe_pre_sorted", mutates_args=("moe_expand", "moe_index", "expert_m", "sorted_tokens_num_lod"))
+def moe_pre_sorted(x: torch.Tensor, topk_index: torch.Tensor, block_statistic: Optional[torch.Tensor],
+                   moe_expand: torch.Tensor, moe_index: torch.Tensor, expert_m: torch.Tensor,
+                   sorted_tokens_num_lod: torch.Tensor, index_have_neg: bool = False) -> None:
+    """Stable sort of routed pairs by expert + gather of their activation rows
+    (reference: ops/_custom_ops.py:1144-1163). block_statistic is not needed: the
+    histograms are rebuilt in LDS."""
+    L.require_device(x, topk_index, moe_expand, moe_index, expert_m, sorted_tokens_num_lod)
+    L.require_contig(x, topk_index, moe_expand, moe_index, expert_m, sorted_tokens_num_lod)
+    _need(topk_index.dtype == torch.int32 and moe_index.dtype == torch.int32 and expert_m.dtype == torch.int32
+          and sorted_tokens_num_lod.dtype == torch.int32, "moe_pre_sorted: index tensors must be int32")
+    _need(x.element_size() == 2 and moe_expand.dtype == x.dtype, "moe_pre_sorted: x/moe_expand must be 16-bit and alike")
+    M, H = x.shape
+    K = topk_index.shape[1]
+    E = expert_m.numel()
+    P = M * K
+    _need(moe_index.numel() == P and sorted_tokens_num_lod.numel() == E + 1 and moe_expand.numel() == P * H,
+          "moe_pre_sorted: output shapes do not match M, K, E, H")
+    sorted_src = torch.empty(P, dtype=torch.int32, device=x.device)
+    _align(topk_index, E, moe_index, sorted_src, expert_m, sorted_tokens_num_lod)
+    L.check(L.lib.kmoe_gather_rows(L.ptr(x), H, L.ptr(sorted_src), P, K, H, L.ptr(moe_expand), H, L.stream()))
+
+
+@custom_op("xspeedgate_ops::moe_pre_small", mutates_args=())
+def moe_pre_small(topk_ids: torch.Tensor, global_num_experts: int, index_have_neg: bool, sort_mode: bool,
+                  x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Small-P variant of moe_pre_sorted that allocates its outputs
+    (reference call: compressed_tensors_moe.py:199-207). Returns
+    (sorted_tokens_idx [P], sorted_tokens_num_lod [E+1], moe_expand [P, H])."""
+    L.require_device(topk_ids, x)
+    L.require_contig(topk_ids, x)
+    M, H = x.shape
+    P = topk_ids.numel()
+    E = int(global_num_experts)
+    dev = x.device
+    moe_index = torch.empty(P, dtype=torch.int32, device=dev)
+    sorted_src = torch.empty(P, dtype=torch.int32, device=dev)
+    lod = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    moe_expand = torch.empty(P, H, dtype=x.dtype, device=dev)
+    _align(topk_ids, E, moe_index, sorted_src, None, lod)
+    L.check(L.lib.kmoe_gather_rows(L.ptr(x), H, L.ptr(sorted_src), P, topk_ids.shape[1], H, L.ptr(moe_expand), H,
+                                   L.stream()))
+    return moe_index, lod, moe_expand
+
+
+# ----------------------------------------------------------------------- quant
+@custom_op("_C::quant2d", mutates_args=("x_q", "max"))
+def quant2d(x: torch.Tensor, x_q: torch.Tensor, max: torch.Tensor, force_sdnn: bool = False) -> None:
+    """Per-row dynamic int8; `max` receives the row ABSMAX (reference: ops/_custom_ops.py:1912-1924)."""
+    L.require_device(x, x_q, max)
+    L.require_contig(x, x_q, max)
+    _act_bits(x, "quant2d")
+    _need(x_q.dtype == torch.int8 and max.dtype == torch.float32, "quant2d: x_q must be int8 and max float32")
+    C = x.shape[-1]
+    R = x.numel() // C
+    _need(x_q.numel() == x.numel() and max.numel() == R, "quant2d: x_q/max shapes do not match x")
+    L.check(L.lib.kmoe_quant_i8_rows(L.ptr(x), C, R, C, L.ptr(x_q), C, L.ptr(max), L.stream()))
+
+
+@custom_op("_C::scaled_int8_quant", mutates_args=())
+def scaled_int8_quant(x: torch.Tensor, scale: Optional[torch.Tensor], azp: Optional[torch.Tensor] = None,
+                      symmetric: bool = True) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, bool]:
+    """Dynamic per-token symmetric int8 (reference: ops/_custom_ops.py:1633-1657).
+    The returned `scale` holds the row MAX, as in the reference. The third
+    result stands for azp=None and is an empty tensor (operator schemas cannot
+    return None). Static and asymmetric modes are not on this path."""
+    if scale is not None or not symmetric:
+        raise NotImplementedError("scaled_int8_quant: only dynamic symmetric quantisation is implemented")
+    xc = x.contiguous()
+    x_q = torch.empty_like(xc, dtype=torch.int8)
+    mx = torch.empty((xc.numel() // xc.shape[-1], 1), device=x.device, dtype=torch.float32)
+    quant2d(xc, x_q, mx, True)
+    return x_q, mx, torch.empty(0, dtype=torch.int32, device=x.device), False
+
+
+# ------------------------------------------------------------------------ GEMM
+def _gemm_i8(a, a_max, w, w_max, lod, y2d, ldy, act, rows, row_src=None, src_div=1, acc_out=None, variant=0):
+    E, n, k = w.shape
+    args = L.GemmI8Args()
+    args.a = a.data_ptr()
+    args.lda = a.stride(0)
+    args.a_max = a_max.data_ptr()
+    args.row_src = 0 if row_src is None else row_src.data_ptr()
+    args.src_div = src_div
+    args.w = w.data_ptr()
+    args.w_max = w_max.data_ptr()
+    args.lod = lod.data_ptr()
+    args.E, args.n, args.k, args.rows = E, n, k, rows
+    args.y = y2d.data_ptr()
+    args.ldy = ldy
+    args.acc_out = 0 if acc_out is None else acc_out.data_ptr()
+    args.act = act
+    args.variant = variant
+    L.check(L.lib.kmoe_grouped_gemm_i8(args, L.stream()))
+
+
+@custom_op("_C::moe_fc", mutates_args=("y",))
+def moe_fc(x: torch.Tensor, weight: torch.Tensor, sorted_tokens_num_lod: torch.Tensor,
+           sorted_tokens_idx: torch.Tensor, moe_topk: int, y: torch.Tensor, act: Optional[str] = None,
+           x_perchannel_max: Optional[torch.Tensor] = None, w_perchannel_max: Optional[torch.Tensor] = None,
+           topk_ids: Optional[torch.Tensor] = None, topk_w: Optional[torch.Tensor] = None,
+           bias: Optional[torch.Tensor] = None, tgemm_type: Optional[str] = None,
+           tweight_type: Optional[str] = None, scale_n: Optional[int] = 0, scale_k: Optional[int] = 0,
+           use_pack_int4: Optional[bool] = False, sort_mode: Optional[bool] = True) -> None:
+    """Grouped GEMM over sorted rows (reference: ops/_custom_ops.py:1204-1244).
+    x [P, k] holds the rows in sorted order; rows [lod[e], lod[e+1]) meet weight[e] [n, k].
+    int8 x/weight with x_perchannel_max [P,1] and w_perchannel_max [E,n,1] give the
+    W8A8 path; act="SWISH_GLU" writes silu(gate)*up into the first n/2 columns of y."""
+    L.require_device(x, weight, sorted_tokens_num_lod, y, x_perchannel_max, w_perchannel_max)
+    L.require_contig(x, weight, sorted_tokens_num_lod, y, x_perchannel_max, w_perchannel_max)
+    if bias is not None or topk_w is not None or use_pack_int4 or scale_n or scale_k:
+        raise NotImplementedError("moe_fc: bias / topk_w / int4 / block-scale arguments are not on this path")
+    _need(act in (None, "SWISH_GLU"), f"moe_fc: act={act!r} unknown")
+    _act_bits(y, "moe_fc")
+    E, n, k = weight.shape
+    rows = x.numel() // k
+    _need(x.shape[-1] == k and y.numel() == rows * n and sorted_tokens_num_lod.numel() == E + 1,
+          "moe_fc: x/y/lod shapes do not match weight")
+    if x.dtype == torch.int8:
+        _need(weight.dtype == torch.int8 and x_perchannel_max is not None and w_perchannel_max is not None,
+              "moe_fc: int8 x needs int8 weight and both per-channel max tensors")
+        _need(x_perchannel_max.numel() == rows and w_perchannel_max.numel() == E * n,
+              "moe_fc: per-channel max shapes must be [P,1] and [E,n,1]")
+        _gemm_i8(x.view(rows, k), x_perchannel_max, weight, w_perchannel_max, sorted_tokens_num_lod,
+                 y, n, L.KMOE_ACT_SWIGLU if act else L.KMOE_ACT_NONE, rows)
+    else:
+        raise NotImplementedError(f"moe_fc: x dtype {x.dtype} is not implemented yet")
+
+
+@custom_op("_C::matmul", mutates_args=())
+def matmul(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, x_trans: bool = False, w_trans: bool = True,
+           alpha: float = 1.0, beta: float = 0.0, bias: Optional[torch.Tensor] = None,
+           x_max: Optional[torch.Tensor] = None, w_max: Optional[torch.Tensor] = None,
+           x_pc_max: Optional[torch.Tensor] = None, w_pc_max: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Dense W8A8 linear: x int8 [M,k] with per-row max, w int8 [n,k] with per-channel
+    max -> out [M,n] (reference: ops/_custom_ops.py:1811-1845; caller
+    quantization/kernels/scale_mm.py:83-90). One-expert case of the grouped GEMM."""
+    if x.dtype != torch.int8 or w.dtype != torch.int8 or x_pc_max is None or w_pc_max is None:
+        raise NotImplementedError("matmul: only the int8 path with x_pc_max / w_pc_max is implemented")
+    if x_trans or not w_trans or alpha != 1.0 or beta != 0.0 or bias is not None:
+        raise NotImplementedError("matmul: x_trans / w_trans=False / alpha / beta / bias are not on this path")
+    if out_dtype != _BF16:
+        raise NotImplementedError(f"matmul: out_dtype {out_dtype} is not implemented")
+    L.require_device(x, w, x_pc_max, w_pc_max)
+    xc, wc = x.contiguous(), w.contiguous()
+    M, k = xc.shape
+    n = wc.shape[0]
+    out = torch.empty((M, n), dtype=out_dtype, device=x.device)
+    lod = torch.tensor([0, M], dtype=torch.int32).to(x.device, non_blocking=True)
+    _gemm_i8(xc, x_pc_max.contiguous(), wc.view(1, n, k), w_pc_max.contiguous(), lod, out, n, L.KMOE_ACT_NONE, M)
+    return out
+
+
+# ---------------------------------------------------------------- elementwise
+@custom_op("_C::silu_and_mul", mutates_args=("out",))
+def silu_and_mul(out: torch.Tensor, x: torch.Tensor, axis: int = -1, turn: bool = True) -> None:
+    """out = silu(x[..., :d]) * x[..., d:] (reference: ops/_custom_ops.py:699-706)."""
+    L.require_device(out, x)
+    L.require_contig(out, x)
+    _act_bits(x, "silu_and_mul")
+    _need(out.dtype == x.dtype, "silu_and_mul: out and x must share a dtype")
+    two_i = x.shape[-1]
+    R = x.numel() // two_i
+    _need(two_i % 2 == 0 and out.numel() == R * (two_i // 2), "silu_and_mul: out must be [..., d] for x [..., 2d]")
+    L.check(L.lib.kmoe_silu_and_mul(L.ptr(x), two_i, R, two_i // 2, L.ptr(out), two_i // 2, L.stream()))
+
+
+@custom_op("_C::moe_post", mutates_args=("y",))
+def moe_post(x: torch.Tensor, moe_index: torch.Tensor, normed_scale: torch.Tensor, dequant_scale: torch.Tensor,
+             y: torch.Tensor) -> None:
+    """y[m] = sum_k normed_scale[m,k] * dequant_scale[m,k] * x[moe_index[m,k]]
+    (reference: ops/_custom_ops.py:1316-1324)."""
+    L.require_device(x, moe_index, normed_scale, dequant_scale, y)
+    L.require_contig(x, moe_index, normed_scale, dequant_scale, y)
+    _act_bits(x, "moe_post")
+    _need(y.dtype == x.dtype and moe_index.dtype == torch.int32 and normed_scale.dtype == torch.float32
+          and dequant_scale.dtype == torch.float32, "moe_post: dtypes must be (x, int32, float32, float32, x)")
+    M, H = y.shape
+    K = moe_index.numel() // M
+    _need(x.numel() == M * K * H and normed_scale.numel() == M * K and dequant_scale.numel() == M * K,
+          "moe_post: shapes must be x [M,K,H], index/scales [M,K], y [M,H]")
+    L.check(L.lib.kmoe_combine(L.ptr(x), H, L.ptr(moe_index), L.ptr(normed_scale), L.ptr(dequant_scale), M, K, H,
+                               1.0, None, 0, L.ptr(y), H, L.stream()))
+
+
+# Fake (meta) implementations so the ops can be traced, as the reference registers for each op.
+def _none(*args, **kwargs):
+    return None
+
+
+for _op in (moe_softmax_topk, moe_softmax_topk_norm, moe_sigmoid_group_topk_norm, topk_softmax, gen_block_statistic,
+            moe_pre_sorted, quant2d, moe_fc, silu_and_mul, moe_post):
+    _op.register_fake(_none)
+
+
+@moe_pre_small.register_fake
+def _fake_moe_pre_small(topk_ids, global_num_experts, index_have_neg, sort_mode, x):
+    P = topk_ids.numel()
+    return (torch.empty(P, dtype=torch.int32, device=x.device),
+            torch.empty(global_num_experts + 1, dtype=torch.int32, device=x.device),
+            torch.empty(P, x.shape[1], dtype=x.dtype, device=x.device))
+
+
+@scaled_int8_quant.register_fake
+def _fake_scaled_int8_quant(x, scale, azp=None, symmetric=True):
+    return (torch.empty_like(x, dtype=torch.int8),
+            torch.empty((x.numel() // x.shape[-1], 1), device=x.device, dtype=torch.float32),
+            torch.empty(0, dtype=torch.int32, device=x.device), False)
+
+
+@matmul.register_fake
+def _fake_matmul(x, w, out_dtype, x_trans=False, w_trans=True, alpha=1.0, beta=0.0, bias=None, x_max=None,
+                 w_max=None, x_pc_max=None, w_pc_max=None):
+    return torch.empty((x.shape[0], w.shape[0] if w_trans else w.shape[1]), dtype=out_dtype, device=x.device)

@@ -1,0 +1,235 @@
+"""W8A8-int8 fused-MoE method: the plugin-level entry of the path.
+
+Mirrors the interface of the reference's
+vllm_kunlun/quantization/compressed_tensors/compressed_tensors_moe.py
+(KunlunCompressedTensorsMoEMethod.get_moe_method :43-108,
+KunlunCompressedTensorsW8A8Int8MoEMethod :111-291): `is_monolithic`,
+`process_weights_after_loading(layer)` and
+`apply_monolithic(layer, x, router_logits, ...)`, same argument meaning, same
+exceptions. Where the reference launches nine closed kernels and allocates every
+intermediate per call, `apply_monolithic` here makes ONE call into libkmoe
+(kmoe_forward_w8a8) on a cached workspace.
+"""
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+
+from ... import _lib as L
+from ...ops import _custom_ops  # noqa: F401  (torch.ops._C.* used by the staged path)
+
+WNA16_SUPPORTED_BITS = (4, 8)
+
+
+class _Workspace:
+    """Per-device scratch buffer that only grows (plays the role of vLLM's
+    current_workspace_manager(), reference: ops/_kunlun_ops.py:528-531)."""
+
+    def __init__(self):
+        self._buf = {}
+
+    def get(self, nbytes: int, device: torch.device) -> torch.Tensor:
+        key = (device.type, device.index)
+        buf = self._buf.get(key)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            self._buf[key] = buf
+        return buf
+
+
+_WORKSPACE = _Workspace()
+
+
+def _scheme_is_dynamic_token_w8a8(weight_quant, input_quant) -> bool:
+    """compressed-tensors "int-quantized" W8A8: 8-bit symmetric channel/tensor
+    weights, 8-bit symmetric dynamic per-token activations."""
+    if weight_quant is None or input_quant is None:
+        return False
+    g = lambda o, k, d=None: o.get(k, d) if isinstance(o, dict) else getattr(o, k, d)  # noqa: E731
+    return (g(weight_quant, "num_bits") == 8 and g(input_quant, "num_bits") == 8
+            and str(g(weight_quant, "strategy")).split(".")[-1].lower() in ("channel", "tensor")
+            and str(g(input_quant, "strategy")).split(".")[-1].lower() == "token"
+            and bool(g(weight_quant, "symmetric", True)) and bool(g(input_quant, "symmetric", True))
+            and bool(g(input_quant, "dynamic", False)) and not bool(g(weight_quant, "dynamic", False)))
+
+
+def _scheme_is_wna16(weight_quant, input_quant) -> bool:
+    if weight_quant is None or input_quant is not None:
+        return False
+    g = lambda o, k, d=None: o.get(k, d) if isinstance(o, dict) else getattr(o, k, d)  # noqa: E731
+    return str(g(weight_quant, "strategy")).split(".")[-1].lower() in ("channel", "group")
+
+
+class KunlunCompressedTensorsMoEMethod:
+    """Scheme dispatcher (reference: compressed_tensors_moe.py:42-108)."""
+
+    @staticmethod
+    def get_moe_method(quant_config, layer: torch.nn.Module, layer_name: str):
+        if hasattr(quant_config, "_add_fused_moe_to_target_scheme_map"):
+            quant_config._add_fused_moe_to_target_scheme_map()
+        unfused = [layer_name + p for p in (".0.gate_proj", ".0.up_proj", ".0.down_proj")]
+        schemes = [quant_config.get_scheme_dict(layer, name) for name in unfused]
+        scheme = schemes.pop()
+        if not all(s == scheme for s in schemes):
+            raise ValueError("All MoE projections need to have same quantization scheme but found multiple")
+        if scheme is None:  # ignored layer
+            from ...ops.fused_moe.layer import KunlunUnquantizedFusedMoEMethod
+            return KunlunUnquantizedFusedMoEMethod(layer.moe_config)
+        weight_quant = scheme.get("weights")
+        input_quant = scheme.get("input_activations")
+        if _scheme_is_wna16(weight_quant, input_quant):
+            raise NotImplementedError("W4A16/W8A16 weight-only MoE is outside the W8A8 path of this build")
+        if _scheme_is_dynamic_token_w8a8(weight_quant, input_quant):
+            return KunlunCompressedTensorsW8A8Int8MoEMethod(weight_quant, input_quant, layer.moe_config)
+        raise RuntimeError(f"Unsupported FusedMoe scheme: {weight_quant}, {input_quant}")
+
+
+class KunlunCompressedTensorsW8A8Int8MoEMethod:
+    """Dynamic-per-token W8A8 int8 MoE (reference: compressed_tensors_moe.py:111-291)."""
+
+    def __init__(self, weight_quant=None, input_quant=None, moe=None):
+        self.weight_quant = weight_quant
+        self.input_quant = input_quant
+        self.moe = moe
+
+    @property
+    def is_monolithic(self) -> bool:
+        return True
+
+    def create_weights(self, layer: torch.nn.Module, num_experts: int, hidden_size: int,
+                       intermediate_size_per_partition: int, params_dtype: torch.dtype = torch.bfloat16,
+                       device=None, **_) -> None:
+        """Parameters as upstream's W8A8 int8 MoE method creates them: int8 weights
+        and one f32 SCALE per output channel (shapes per compressed_tensors_moe.py:135-137,212,258)."""
+        E, H, I = num_experts, hidden_size, intermediate_size_per_partition
+        mk = lambda *s, dt: torch.nn.Parameter(torch.zeros(*s, dtype=dt, device=device), requires_grad=False)  # noqa
+        layer.w13_weight = mk(E, 2 * I, H, dt=torch.int8)
+        layer.w2_weight = mk(E, H, I, dt=torch.int8)
+        layer.w13_weight_scale = mk(E, 2 * I, 1, dt=torch.float32)
+        layer.w2_weight_scale = mk(E, H, 1, dt=torch.float32)
+
+    def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
+        """scale -> absmax: the kernels dequantise with max/127 (reference: :116-120)."""
+        with torch.no_grad():
+            layer.w13_weight_scale.mul_(127.0)
+            layer.w2_weight_scale.mul_(127.0)
+
+    # -- routing parameters: kwargs win; a kwarg left at its default falls back to the layer
+    @staticmethod
+    def _routing(layer, topk_group, num_expert_group, scoring_func, routed_scaling_factor, bias):
+        if scoring_func == "softmax" and getattr(layer, "scoring_func", "softmax") != "softmax":
+            scoring_func = layer.scoring_func
+        if topk_group is None:
+            topk_group = getattr(layer, "topk_group", None)
+        if num_expert_group is None:
+            num_expert_group = getattr(layer, "num_expert_group", None)
+        if bias is None:
+            bias = getattr(layer, "e_score_correction_bias", None)
+        if routed_scaling_factor == 1.0:
+            routed_scaling_factor = float(getattr(layer, "routed_scaling_factor", 1.0) or 1.0)
+        if scoring_func not in ("softmax", "sigmoid"):
+            raise ValueError(f"Unsupported scoring_func: {scoring_func}")
+        return topk_group, num_expert_group, scoring_func, routed_scaling_factor, bias
+
+    def apply_monolithic(
+        self,
+        layer: torch.nn.Module,
+        x: torch.Tensor,
+        router_logits: torch.Tensor,
+        topk_group: Optional[int] = None,
+        num_expert_group: Optional[int] = None,
+        global_num_experts: int = -1,
+        scoring_func: str = "softmax",
+        routed_scaling_factor: float = 1.0,
+        e_score_correction_bias: Optional[torch.Tensor] = None,
+        shared_expert=None,
+        out_scale: float = 1.0,
+    ) -> Union[torch.Tensor, tuple]:
+        """x [M,H] bf16, router_logits [M,E] -> [M,H] bf16 (reference: :122-291).
+        `shared_expert` (w13, w13_max, w2, w2_max of a dense W8A8 MLP) and
+        `out_scale` fold the caller's epilogue (models/deepseek_v2.py:288-296) into the call."""
+        topk_group, num_expert_group, scoring_func, routed_scaling_factor, bias = self._routing(
+            layer, topk_group, num_expert_group, scoring_func, routed_scaling_factor, e_score_correction_bias)
+        L.require_device(x, router_logits, layer.w13_weight, layer.w2_weight)
+        if x.dtype != torch.bfloat16:
+            raise NotImplementedError(f"apply_monolithic: activations must be bfloat16, got {x.dtype}")
+        E, two_i, H = layer.w13_weight.shape
+        M = x.shape[0]
+        x = x.contiguous()
+        logits = router_logits.float().contiguous()
+        out = torch.empty((M, H), dtype=x.dtype, device=x.device)
+
+        a = L.W8A8Args()
+        a.M, a.H, a.E, a.K, a.I = M, H, E, self.moe.experts_per_token, two_i // 2
+        a.scoring = L.KMOE_SCORE_SOFTMAX if scoring_func == "softmax" else L.KMOE_SCORE_SIGMOID
+        a.renormalize = 1  # the reference always routes with the *_norm kernels
+        a.n_group = int(num_expert_group or 1)
+        a.topk_group = int(topk_group or 1)
+        a.routed_scale = float(routed_scaling_factor)
+        a.logits = logits.data_ptr()
+        a.bias = 0 if bias is None else bias.data_ptr()
+        a.x = x.data_ptr()
+        a.w13, a.w13_max = layer.w13_weight.data_ptr(), layer.w13_weight_scale.data_ptr()
+        a.w2, a.w2_max = layer.w2_weight.data_ptr(), layer.w2_weight_scale.data_ptr()
+        if shared_expert is not None:
+            ws13, ws13_max, ws2, ws2_max = shared_expert
+            a.I_shared = ws13.shape[0] // 2
+            a.ws13, a.ws13_max, a.ws2, a.ws2_max = (ws13.data_ptr(), ws13_max.data_ptr(), ws2.data_ptr(),
+                                                    ws2_max.data_ptr())
+        a.out_scale = float(out_scale)
+        a.out = out.data_ptr()
+        lay = L.W8A8Layout()
+        L.check(L.lib.kmoe_w8a8_workspace_layout(a, lay))
+        ws = _WORKSPACE.get(lay.total_bytes, x.device)
+        L.check(L.lib.kmoe_forward_w8a8(a, L.ptr(ws), ws.numel(), L.stream()))
+        self.last_layout, self.last_workspace = lay, ws  # lets tests read the intermediates
+        return out
+
+    def apply_staged(self, layer, x, router_logits, topk_group=None, num_expert_group=None, global_num_experts=-1,
+                     scoring_func="softmax", routed_scaling_factor=1.0, e_score_correction_bias=None):
+        """The same layer through the operator-level surface, one torch.ops._C.* call
+        per stage in the reference's order (compressed_tensors_moe.py:139-291).
+        Bit-identical to apply_monolithic; kept for callers that drive the ops themselves."""
+        topk_group, num_expert_group, scoring_func, routed_scaling_factor, bias = self._routing(
+            layer, topk_group, num_expert_group, scoring_func, routed_scaling_factor, e_score_correction_bias)
+        ops = torch.ops._C
+        E, two_i, H = layer.w13_weight.shape
+        M, K, dev = x.shape[0], self.moe.experts_per_token, x.device
+        normed_score = torch.empty(M, K, dtype=torch.float32, device=dev)
+        topk_ids = torch.empty(M, K, dtype=torch.int32, device=dev)
+        block_statistic = torch.zeros(12, E, dtype=torch.int32, device=dev)
+        logits = router_logits.float()
+        if scoring_func == "softmax":
+            ops.moe_softmax_topk_norm(logits, normed_score, topk_ids, None, True)
+        else:
+            ops.moe_sigmoid_group_topk_norm(logits, topk_ids, normed_score, block_statistic, bias,
+                                            routed_scaling_factor, num_expert_group, topk_group)
+        if M * K > 768:
+            moe_expand = torch.empty(M * K, H, dtype=x.dtype, device=dev)
+            expert_m = torch.zeros(E, dtype=torch.int32, device=dev)
+            lod = torch.zeros(E + 1, dtype=torch.int32, device=dev)
+            sorted_tokens_idx = torch.zeros(M * K, dtype=torch.int32, device=dev)
+            ops.gen_block_statistic(topk_ids, block_statistic)
+            ops.moe_pre_sorted(x, topk_ids, block_statistic, moe_expand, sorted_tokens_idx, expert_m, lod)
+        else:
+            sorted_tokens_idx, lod, moe_expand = torch.ops.xspeedgate_ops.moe_pre_small(topk_ids, E, False, True, x)
+        y = torch.empty(M, K, two_i, dtype=x.dtype, device=dev)
+        x_q = torch.empty(M * K, H, dtype=torch.int8, device=dev)
+        x_scale = torch.empty(M * K, 1, dtype=torch.float32, device=dev)
+        ops.quant2d(moe_expand, x_q, x_scale, True)
+        ops.moe_fc(x_q, layer.w13_weight, lod, sorted_tokens_idx, K, y, None, x_scale, layer.w13_weight_scale,
+                   topk_ids)
+        out1 = torch.empty(M, K, two_i // 2, dtype=x.dtype, device=dev)
+        ops.silu_and_mul(out1, y)
+        out1 = out1.reshape(-1, two_i // 2)
+        x_q = torch.empty(out1.shape, dtype=torch.int8, device=dev)
+        x_scale = torch.empty(out1.shape[0], 1, dtype=torch.float32, device=dev)
+        ops.quant2d(out1, x_q, x_scale, True)
+        out = torch.empty(M, K, H, dtype=x.dtype, device=dev)
+        ops.moe_fc(x_q, layer.w2_weight, lod, sorted_tokens_idx, K, out, None, x_scale, layer.w2_weight_scale,
+                   topk_ids)
+        dequant_scale = torch.ones(M, K, dtype=torch.float32, device=dev)
+        output = torch.empty(M, H, dtype=x.dtype, device=dev)
+        ops.moe_post(out, sorted_tokens_idx.view(M, K), normed_score, dequant_scale, output)
+        return output

@@ -1,0 +1,119 @@
+"""Seeded synthetic MoE layers of the benchmark shapes.
+
+Weights ~ N(0, 0.02) quantised per output channel to int8 (scale = absmax/127),
+activations ~ N(0, 1) bf16, router logits ~ N(0, 1) f32, correction bias
+~ N(0, 0.01). Everything is generated on the target device from one seeded
+generator, expert by expert, so the 11 GB DeepSeek-V3-shape layer never needs a
+float copy of itself; tests copy back to the host whatever their checker needs.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, replace
+from typing import Optional
+
+import torch
+
+from .ops.fused_moe.layer import FusedMoE
+from .quantization.compressed_tensors.compressed_tensors_moe import KunlunCompressedTensorsW8A8Int8MoEMethod
+
+
+@dataclass(frozen=True)
+class MoEShape:
+    name: str
+    M: int            # tokens
+    H: int            # hidden
+    E: int            # routed experts
+    K: int            # experts per token
+    I: int            # moe intermediate
+    scoring: str = "softmax"
+    n_group: int = 1
+    topk_group: int = 1
+    routed_scale: float = 1.0
+    I_shared: int = 0  # intermediate of the dense shared expert (0: none)
+    hot_experts: int = 0   # add +hot_bias to the logits of this many fixed experts
+    hot_bias: float = 0.0
+    quant: str = "int8"    # "none" (bf16 weights), "int8", "fp8"
+
+    @property
+    def P(self) -> int:
+        return self.M * self.K
+
+
+# The benchmark configurations (tokens are the decode / prefill batch of each).
+SHAPES = {
+    "tiny-bf16": MoEShape("tiny-bf16", 32, 512, 8, 2, 256, quant="none"),
+    "qwen3-decode": MoEShape("qwen3-decode", 64, 2048, 128, 8, 768),
+    "qwen3-prefill": MoEShape("qwen3-prefill", 8192, 2048, 128, 8, 768),
+    "qwen3-prefill-skew": MoEShape("qwen3-prefill-skew", 8192, 2048, 128, 8, 768, hot_experts=8, hot_bias=2.0),
+    "dsv3-decode": MoEShape("dsv3-decode", 128, 7168, 256, 8, 2048, "sigmoid", 8, 4, 2.5, 2048),
+    "dsv3-prefill": MoEShape("dsv3-prefill", 4096, 7168, 256, 8, 2048, "sigmoid", 8, 4, 2.5, 2048),
+    "kimi-decode": MoEShape("kimi-decode", 128, 7168, 384, 8, 2048, "sigmoid", 1, 1, 2.5, 2048),
+    "kimi-prefill": MoEShape("kimi-prefill", 4096, 7168, 384, 8, 2048, "sigmoid", 1, 1, 2.5, 2048),
+}
+
+
+def scaled(shape: MoEShape, **kw) -> MoEShape:
+    """A copy of a shape with some fields replaced (reduced sizes for CPU-checkable tests)."""
+    return replace(shape, **kw)
+
+
+def _quant_rows_int8(w: torch.Tensor):
+    mx = w.abs().amax(dim=-1, keepdim=True).clamp_min(1e-12)
+    q = torch.round(w * (127.0 / mx)).clamp_(-127, 127).to(torch.int8)
+    return q, mx / 127.0
+
+
+@dataclass
+class SynthLayer:
+    shape: MoEShape
+    layer: FusedMoE
+    x: torch.Tensor                 # [M,H] bf16
+    logits: torch.Tensor            # [M,E] f32
+    bias: Optional[torch.Tensor]    # [E] f32 (sigmoid routing)
+    shared: Optional[tuple]         # (ws13 i8 [2Is,H], ws13_max f32 [2Is], ws2 i8 [H,Is], ws2_max f32 [H])
+
+    def apply_kwargs(self) -> dict:
+        s = self.shape
+        kw = dict(scoring_func=s.scoring)
+        if s.scoring == "sigmoid":
+            kw.update(num_expert_group=s.n_group, topk_group=s.topk_group, routed_scaling_factor=s.routed_scale,
+                      e_score_correction_bias=self.bias)
+        if self.shared is not None:
+            kw["shared_expert"] = self.shared
+        return kw
+
+
+def make_w8a8_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
+    """Builds a FusedMoE with the W8A8 method, fills it with quantised random
+    weights and runs process_weights_after_loading (scales become maxes)."""
+    dev = torch.device(device)
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    s = shape
+    method = KunlunCompressedTensorsW8A8Int8MoEMethod()
+    bias = None
+    if s.scoring == "sigmoid":
+        bias = torch.randn(s.E, generator=g, device=dev, dtype=torch.float32) * 0.01
+    layer = FusedMoE(num_experts=s.E, top_k=s.K, hidden_size=s.H, intermediate_size=s.I,
+                     renormalize=True, use_grouped_topk=s.n_group > 1, num_expert_group=s.n_group,
+                     topk_group=s.topk_group, scoring_func=s.scoring, e_score_correction_bias=bias,
+                     quant_method=method, device=dev)
+    for e in range(s.E):
+        q, sc = _quant_rows_int8(torch.randn(2 * s.I, s.H, generator=g, device=dev) * 0.02)
+        layer.w13_weight.data[e].copy_(q)
+        layer.w13_weight_scale.data[e].copy_(sc)
+        q, sc = _quant_rows_int8(torch.randn(s.H, s.I, generator=g, device=dev) * 0.02)
+        layer.w2_weight.data[e].copy_(q)
+        layer.w2_weight_scale.data[e].copy_(sc)
+    method.process_weights_after_loading(layer)
+    shared = None
+    if s.I_shared:
+        q13, s13 = _quant_rows_int8(torch.randn(2 * s.I_shared, s.H, generator=g, device=dev) * 0.02)
+        q2, s2 = _quant_rows_int8(torch.randn(s.H, s.I_shared, generator=g, device=dev) * 0.02)
+        shared = (q13, (s13 * 127.0).reshape(-1).contiguous(), q2, (s2 * 127.0).reshape(-1).contiguous())
+    x = torch.randn(s.M, s.H, generator=g, device=dev).to(torch.bfloat16)
+    logits = torch.randn(s.M, s.E, generator=g, device=dev, dtype=torch.float32)
+    if s.hot_experts:
+        hot = torch.arange(s.hot_experts, device=dev) * (s.E // s.hot_experts)
+        logits[:, hot] += s.hot_bias
+    return SynthLayer(s, layer, x, logits, bias, shared)

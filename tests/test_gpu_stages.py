@@ -168,7 +168,8 @@ def test_quant_fp8_group128(L, R, Cc):
     torch.manual_seed(R + Cc)
     x = (torch.randn(R, Cc) * torch.rand(R, 1) * 4).bfloat16()
     x[0, :128] = 0
-    x[0, 130] = 2.0 ** -12
+    if Cc > 128:
+        x[0, 130] = 2.0 ** -12
     q_ref, s_ref = co.quant_fp8_group128(bits(x))
     dx = x.cuda()
     q = torch.empty(R, Cc, dtype=torch.uint8, device="cuda")

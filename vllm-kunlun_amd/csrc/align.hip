@@ -221,7 +221,7 @@ extern "C" size_t kmoe_align_workspace_bytes(int P, int E) {
 extern "C" int kmoe_align(const int32_t* topk_ids, int P, int E, int32_t* moe_index, int32_t* sorted_src,
                           int32_t* expert_m, int32_t* lod, void* workspace, size_t workspace_bytes,
                           kmoe_stream_t stream) {
-  KMOE_REQUIRE(topk_ids && moe_index && lod, KMOE_ERR_NULL, "align: NULL pointer");
+  KMOE_REQUIRE(lod && (P == 0 || (topk_ids && moe_index)), KMOE_ERR_NULL, "align: NULL pointer");
   KMOE_REQUIRE(E >= 1 && E <= kMaxE, KMOE_ERR_SHAPE, "align: E=%d outside [1,%d]", E, kMaxE);
   KMOE_REQUIRE(P >= 0 && P <= (1 << 24), KMOE_ERR_SHAPE, "align: P=%d outside [0,2^24]", P);
   hipStream_t s = as_stream(stream);

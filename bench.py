@@ -1,0 +1,226 @@
+#!/usr/bin/env python3
+"""MoE-layer throughput of the W8A8 fused-MoE path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one call of the whole layer (routing -> align -> int8 quant -> gate_up
+GEMM + SiLU-mul -> int8 quant -> down GEMM -> combine, plus the shared expert
+where the shape has one) over one batch of synthetic tokens that already sits
+in HBM. Prints ONE JSON line: tokens/s, the roofline of the dominant kernel
+(HIP events recorded around it inside the timed calls) and the CPU baseline
+(the torch-CPU restatement of the reference's expert loop, timed on this host).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "vllm-kunlun_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+INT8_PEAK_TOPS = 5000.0    # MI355X dense int8 MFMA
+
+WORKLOAD_LABEL = {
+    "qwen3-decode": "Qwen3-MoE-30B-A3B-shape MoE layer, W8A8 int8, decode, 64 tokens",
+    "qwen3-prefill": "Qwen3-MoE-30B-A3B-shape MoE layer, W8A8 int8, prefill, 8192 tokens",
+    "qwen3-prefill-skew": "Qwen3-MoE-30B-A3B-shape MoE layer, W8A8 int8, prefill, 8192 tokens, +2.0 logit bias on 8 experts",
+    "dsv3-decode": "DeepSeek-V3-shape MoE layer (+1 shared expert), W8A8 int8, decode, 128 tokens",
+    "dsv3-prefill": "DeepSeek-V3-shape MoE layer (+1 shared expert), W8A8 int8, prefill, 4096 tokens",
+}
+
+
+class HipEvents:
+    """hipEvent_t handles made through the HIP runtime torch already loaded."""
+
+    def __init__(self, n):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.hip.hipEventDestroy.argtypes = [C.c_void_p]
+        self.handles = (C.c_void_p * n)()
+        for i in range(n):
+            ev = C.c_void_p()
+            rc = self.hip.hipEventCreate(C.byref(ev))
+            assert rc == 0, f"hipEventCreate failed: {rc}"
+            self.handles[i] = ev
+
+    def elapsed_ms(self, i, j):
+        self.hip.hipEventSynchronize(self.handles[j])
+        ms = C.c_float()
+        rc = self.hip.hipEventElapsedTime(C.byref(ms), self.handles[i], self.handles[j])
+        assert rc == 0, f"hipEventElapsedTime failed: {rc}"
+        return ms.value
+
+    def close(self):
+        for h in self.handles:
+            self.hip.hipEventDestroy(h)
+
+
+def algorithmic_work(shape, n_active):
+    """Bytes that must cross HBM and int8 operations that must run, per layer call
+    and for each GEMM launch, from the shape and the number of experts hit."""
+    M, H, E, K, I, Is, P = shape.M, shape.H, shape.E, shape.K, shape.I, shape.I_shared, shape.P
+    g1_bytes = n_active * (2 * I * H + 2 * I * 4) + M * H + M * 4 + P * 4 + P * I * 2
+    g2_bytes = n_active * (H * I + H * 4) + P * I + P * 4 + P * H * 2
+    shared_bytes = (3 * Is * H + (2 * Is + H) * 4) if Is else 0
+    layer_bytes = (n_active * (3 * I * H + (2 * I + H) * 4) + shared_bytes + 2 * M * H * 2 + M * E * 4)
+    g1_ops = 2 * P * 2 * I * H
+    g2_ops = 2 * P * H * I
+    layer_ops = g1_ops + g2_ops + 2 * M * 3 * Is * H
+    return dict(g1_bytes=g1_bytes, g2_bytes=g2_bytes, layer_bytes=layer_bytes, g1_ops=g1_ops, g2_ops=g2_ops,
+                layer_ops=layer_ops)
+
+
+def cpu_baseline(sl, budget_s=20.0):
+    """The reference's torch expert loop (oracle/torch_moe.py) on the host cores."""
+    import torch
+    from oracle import torch_moe as tm
+    s = sl.shape
+    lay = sl.layer
+    host = lambda t: None if t is None else t.detach().cpu()  # noqa: E731
+    args = (host(sl.x), host(sl.logits), host(lay.w13_weight), host(lay.w13_weight_scale), host(lay.w2_weight),
+            host(lay.w2_weight_scale), s.K, s.scoring, True, s.n_group, s.topk_group, s.routed_scale, host(sl.bias),
+            None if sl.shared is None else tuple(host(t) for t in sl.shared))
+    t0 = time.perf_counter()
+    tm.w8a8_moe(*args)  # warm-up
+    first = time.perf_counter() - t0
+    runs = max(1, min(3, int(budget_s / max(first, 1e-3))))
+    times = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        tm.w8a8_moe(*args)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {"value": s.M / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{runs} full layer call(s) of the same workload ({s.M} tokens) after 1 warm-up, median; "
+                      f"torch-CPU restatement of the reference expert loop; host has {os.cpu_count()} cpus"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="qwen3-decode", choices=sorted(WORKLOAD_LABEL))
+    ap.add_argument("--launch", default="graph", choices=["graph", "eager"],
+                    help="replay the layer from a captured HIP graph (as a serving engine does) or launch it eagerly")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=0)
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build measures ONE GPU; the layer does not span GPUs (run with --gpus 1)")
+
+    import torch
+    from vllm_kunlun_amd import _lib as L
+    from vllm_kunlun_amd import synth
+
+    torch.cuda.set_device(0)
+    shape = synth.SHAPES[a.workload]
+    sl = synth.make_w8a8_layer(shape, "cuda:0", seed=a.seed)
+    method = sl.layer.quant_method
+    kw = sl.apply_kwargs()
+    x, logits = sl.x.contiguous(), sl.logits.contiguous()
+    out = torch.empty_like(x)
+    plan_kw = dict(topk_group=kw.get("topk_group"), num_expert_group=kw.get("num_expert_group"),
+                   scoring_func=kw.get("scoring_func", "softmax"),
+                   routed_scaling_factor=kw.get("routed_scaling_factor", 1.0),
+                   e_score_correction_bias=kw.get("e_score_correction_bias"), shared_expert=kw.get("shared_expert"))
+    plan = method.make_plan(sl.layer, x, logits, out, **plan_kw)
+
+    # The layer, its inputs and the workspace were produced on the default stream;
+    # finish that work before a second stream touches (recycled) memory.
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        for _ in range(3):
+            plan()
+        stream.synchronize()
+        graph = None
+        if a.launch == "graph":
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                plan()
+        step = graph.replay if graph is not None else plan
+
+        for _ in range(a.warmup):
+            step()
+        stream.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            step()
+        stream.synchronize()
+        wall = time.perf_counter() - t0
+        ms_per_step = wall * 1e3 / a.steps
+
+        # the same calls again with HIP events around each stage (eager: events are
+        # not captured), for the per-kernel durations of the roofline
+        ev = HipEvents(2 * len(L.STAGES))
+        plan_ev = method.make_plan(sl.layer, x, logits, out, stage_events=ev.handles, **plan_kw)
+        stage_ms = {s: 0.0 for s in L.STAGES}
+        for it in range(a.warmup + a.steps):
+            plan_ev()
+            if it >= a.warmup:
+                for i, s in enumerate(L.STAGES):
+                    stage_ms[s] += ev.elapsed_ms(2 * i, 2 * i + 1)
+        stage_ms = {s: v / a.steps for s, v in stage_ms.items()}
+        stream.synchronize()
+        ev.close()
+
+    lod = plan.view("lod", shape.E + 1, torch.int32).cpu()
+    n_active = int(((lod[1:] - lod[:-1]) > 0).sum())
+    work = algorithmic_work(shape, n_active)
+    intensity = work["layer_ops"] / work["layer_bytes"]
+    hbm_bound = intensity < INT8_PEAK_TOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+    g1_s = stage_ms["gemm1"] * 1e-3
+    if hbm_bound:
+        achieved = work["g1_bytes"] / g1_s / 1e9
+        roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": achieved / HBM_PEAK_GBS, "traffic": None}
+    else:
+        achieved = work["g1_ops"] / g1_s / 1e12
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s",
+                    "frac": achieved / INT8_PEAK_TOPS, "traffic": None}
+    roofline.update(kernel="gemm_i8_kernel (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
+                    algorithmic_bytes=work["g1_bytes"], algorithmic_ops=work["g1_ops"])
+
+    t_s = ms_per_step * 1e-3
+    result = {
+        "metric": "MoE-layer tokens/s at 1 GPU",
+        "value": shape.M / t_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": WORKLOAD_LABEL[a.workload], "name": a.workload, "tokens": shape.M, "hidden": shape.H,
+                   "experts": shape.E, "top_k": shape.K, "moe_intermediate": shape.I,
+                   "shared_intermediate": shape.I_shared, "routing": shape.scoring, "experts_hit": n_active,
+                   "launch": "hipgraph replay" if graph is not None else "eager", "seed": a.seed},
+        "roofline": roofline,
+        "layer": {"hbm_gbs": work["layer_bytes"] / t_s / 1e9, "hbm_frac": work["layer_bytes"] / t_s / 1e9 / HBM_PEAK_GBS,
+                  "int8_tops": work["layer_ops"] / t_s / 1e12,
+                  "mfma_frac": work["layer_ops"] / t_s / 1e12 / INT8_PEAK_TOPS,
+                  "algorithmic_bytes": work["layer_bytes"], "algorithmic_ops": work["layer_ops"],
+                  "stage_ms": stage_ms},
+    }
+    if not a.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(sl)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

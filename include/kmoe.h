@@ -235,7 +235,21 @@ typedef struct kmoe_w8a8_args {
   /* caller epilogue: out = routed*out_scale (+ shared) */
   float out_scale;
   uint16_t* out;         /* [M,H] bf16                                          */
+  /* optional profiling: NULL, or 2*KMOE_N_STAGES hipEvent_t handles; entry 2s is
+     recorded on the stream before stage s and entry 2s+1 after it (NULL entries
+     are skipped). Leave NULL under graph capture.                             */
+  void* const* stage_events;
 } kmoe_w8a8_args;
+
+#define KMOE_STAGE_ROUTING 0
+#define KMOE_STAGE_ALIGN 1
+#define KMOE_STAGE_QUANT1 2
+#define KMOE_STAGE_GEMM1 3 /* gate_up + SiLU-mul */
+#define KMOE_STAGE_QUANT2 4
+#define KMOE_STAGE_GEMM2 5 /* down */
+#define KMOE_STAGE_SHARED 6
+#define KMOE_STAGE_COMBINE 7
+#define KMOE_N_STAGES 8
 
 /* Byte offsets of the intermediates kmoe_forward_w8a8 keeps in its workspace. */
 typedef struct kmoe_w8a8_layout {

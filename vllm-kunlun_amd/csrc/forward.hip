@@ -108,8 +108,14 @@ extern "C" int kmoe_forward_w8a8(const kmoe_w8a8_args* a, void* workspace, size_
   float* xmax = static_cast<float*>(at(L.xmax));
   const int M = a->M, H = a->H, E = a->E, K = a->K, I = a->I, P = M * K;
   int rc;
+  auto mark = [&](int stage, int end) {
+    if (!a->stage_events) return;
+    void* ev = a->stage_events[2 * stage + end];
+    if (ev) (void)hipEventRecord(static_cast<hipEvent_t>(ev), as_stream(stream));
+  };
 
   // 1. routing
+  mark(KMOE_STAGE_ROUTING, 0);
   if (a->scoring == KMOE_SCORE_SOFTMAX) {
     rc = kmoe_softmax_topk(a->logits, M, E, K, a->renormalize, topk_w, topk_ids, stream);
   } else {
@@ -117,13 +123,19 @@ extern "C" int kmoe_forward_w8a8(const kmoe_w8a8_args* a, void* workspace, size_
                                       topk_ids, stream);
   }
   if (rc) return rc;
+  mark(KMOE_STAGE_ROUTING, 1);
   // 2. stable sort of the routed pairs by expert
+  mark(KMOE_STAGE_ALIGN, 0);
   rc = kmoe_align(topk_ids, P, E, moe_index, sorted_src, static_cast<int32_t*>(at(L.expert_m)), lod, at(L.align_ws),
                   kmoe_align_workspace_bytes(P, E), stream);
   if (rc) return rc;
+  mark(KMOE_STAGE_ALIGN, 1);
+  mark(KMOE_STAGE_QUANT1, 0);
   // 3. one int8 row per TOKEN (the reference quantises the K-times expanded copy; same values)
   rc = kmoe_quant_i8_rows(a->x, H, M, H, xq, H, xmax, stream);
   if (rc) return rc;
+  mark(KMOE_STAGE_QUANT1, 1);
+  mark(KMOE_STAGE_GEMM1, 0);
   // 4. gate_up GEMM with dequant + SiLU-mul epilogue; rows gathered through the sort
   kmoe_gemm_i8_args g1 = {};
   g1.a = xq;
@@ -143,10 +155,14 @@ extern "C" int kmoe_forward_w8a8(const kmoe_w8a8_args* a, void* workspace, size_
   g1.act = KMOE_ACT_SWIGLU;
   rc = kmoe_grouped_gemm_i8(&g1, stream);
   if (rc) return rc;
+  mark(KMOE_STAGE_GEMM1, 1);
+  mark(KMOE_STAGE_QUANT2, 0);
   // 5. requantise the activation rows
   rc = kmoe_quant_i8_rows(static_cast<uint16_t*>(at(L.act)), I, P, I, static_cast<int8_t*>(at(L.actq)), I,
                           static_cast<float*>(at(L.actmax)), stream);
   if (rc) return rc;
+  mark(KMOE_STAGE_QUANT2, 1);
+  mark(KMOE_STAGE_GEMM2, 0);
   // 6. down GEMM
   kmoe_gemm_i8_args g2 = {};
   g2.a = static_cast<int8_t*>(at(L.actq));
@@ -164,8 +180,10 @@ extern "C" int kmoe_forward_w8a8(const kmoe_w8a8_args* a, void* workspace, size_
   g2.act = KMOE_ACT_NONE;
   rc = kmoe_grouped_gemm_i8(&g2, stream);
   if (rc) return rc;
+  mark(KMOE_STAGE_GEMM2, 1);
 
   // 7. dense shared expert on all M rows: one "expert" whose lod is [0, M]
+  mark(KMOE_STAGE_SHARED, 0);
   const uint16_t* shared_out = nullptr;
   if (a->I_shared > 0) {
     const int Is = a->I_shared;
@@ -210,7 +228,11 @@ extern "C" int kmoe_forward_w8a8(const kmoe_w8a8_args* a, void* workspace, size_
     if (rc) return rc;
     shared_out = static_cast<uint16_t*>(at(L.sh_out));
   }
+  mark(KMOE_STAGE_SHARED, 1);
   // 8. weighted combine (+ caller epilogue)
-  return kmoe_combine(static_cast<uint16_t*>(at(L.down)), H, moe_index, topk_w, nullptr, M, K, H, a->out_scale,
+  mark(KMOE_STAGE_COMBINE, 0);
+  rc = kmoe_combine(static_cast<uint16_t*>(at(L.down)), H, moe_index, topk_w, nullptr, M, K, H, a->out_scale,
                       shared_out, H, a->out, H, stream);
+  mark(KMOE_STAGE_COMBINE, 1);
+  return rc;
 }

@@ -18,6 +18,7 @@ KMOE_ACT_NONE = 0
 KMOE_ACT_SWIGLU = 1
 KMOE_SCORE_SOFTMAX = 0
 KMOE_SCORE_SIGMOID = 1
+STAGES = ("routing", "align", "quant1", "gemm1", "quant2", "gemm2", "shared", "combine")
 
 _ERR_KIND = {-1: ValueError, -2: ValueError, -3: NotImplementedError, -4: RuntimeError, -5: RuntimeError}
 
@@ -40,6 +41,7 @@ class W8A8Args(C.Structure):
         ("x", C.c_void_p), ("w13", C.c_void_p), ("w13_max", C.c_void_p), ("w2", C.c_void_p), ("w2_max", C.c_void_p),
         ("I_shared", C.c_int32), ("ws13", C.c_void_p), ("ws13_max", C.c_void_p), ("ws2", C.c_void_p),
         ("ws2_max", C.c_void_p), ("out_scale", C.c_float), ("out", C.c_void_p),
+        ("stage_events", C.POINTER(C.c_void_p)),
     ]
 
 

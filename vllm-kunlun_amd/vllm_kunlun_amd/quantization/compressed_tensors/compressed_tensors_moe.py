@@ -61,6 +61,23 @@ def _scheme_is_wna16(weight_quant, input_quant) -> bool:
     return str(g(weight_quant, "strategy")).split(".")[-1].lower() in ("channel", "group")
 
 
+class W8A8Plan:
+    """A filled kmoe_w8a8_args block plus its workspace; calling it enqueues the layer
+    on the current stream."""
+
+    def __init__(self, args, layout, workspace, keepalive):
+        self.args, self.layout, self.workspace, self._keep = args, layout, workspace, keepalive
+
+    def __call__(self) -> None:
+        L.check(L.lib.kmoe_forward_w8a8(self.args, L.ptr(self.workspace), self.workspace.numel(), L.stream()))
+
+    def view(self, name: str, count: int, dtype: torch.dtype) -> torch.Tensor:
+        """An intermediate of the last call, e.g. view("topk_ids", M*K, torch.int32)."""
+        off = getattr(self.layout, name)
+        nbytes = count * torch.empty(0, dtype=dtype).element_size()
+        return self.workspace[off: off + nbytes].view(dtype)
+
+
 class KunlunCompressedTensorsMoEMethod:
     """Scheme dispatcher (reference: compressed_tensors_moe.py:42-108)."""
 
@@ -149,17 +166,34 @@ class KunlunCompressedTensorsW8A8Int8MoEMethod:
         """x [M,H] bf16, router_logits [M,E] -> [M,H] bf16 (reference: :122-291).
         `shared_expert` (w13, w13_max, w2, w2_max of a dense W8A8 MLP) and
         `out_scale` fold the caller's epilogue (models/deepseek_v2.py:288-296) into the call."""
-        topk_group, num_expert_group, scoring_func, routed_scaling_factor, bias = self._routing(
-            layer, topk_group, num_expert_group, scoring_func, routed_scaling_factor, e_score_correction_bias)
-        L.require_device(x, router_logits, layer.w13_weight, layer.w2_weight)
         if x.dtype != torch.bfloat16:
             raise NotImplementedError(f"apply_monolithic: activations must be bfloat16, got {x.dtype}")
-        E, two_i, H = layer.w13_weight.shape
-        M = x.shape[0]
         x = x.contiguous()
         logits = router_logits.float().contiguous()
-        out = torch.empty((M, H), dtype=x.dtype, device=x.device)
+        out = torch.empty((x.shape[0], layer.w2_weight.shape[1]), dtype=x.dtype, device=x.device)
+        plan = self.make_plan(layer, x, logits, out, topk_group, num_expert_group, scoring_func,
+                              routed_scaling_factor, e_score_correction_bias, shared_expert, out_scale)
+        plan()
+        self.last_layout, self.last_workspace = plan.layout, plan.workspace  # lets tests read the intermediates
+        return out
 
+    def make_plan(self, layer, x, logits, out, topk_group=None, num_expert_group=None, scoring_func="softmax",
+                  routed_scaling_factor=1.0, e_score_correction_bias=None, shared_expert=None, out_scale=1.0,
+                  stage_events=None) -> "W8A8Plan":
+        """Argument block for repeated calls on fixed buffers (x bf16 [M,H], logits f32
+        [M,E], out bf16 [M,H], all contiguous): what a serving loop or a HIP-graph
+        capture replays without touching Python-side allocation."""
+        topk_group, num_expert_group, scoring_func, routed_scaling_factor, bias = self._routing(
+            layer, topk_group, num_expert_group, scoring_func, routed_scaling_factor, e_score_correction_bias)
+        L.require_device(x, logits, out, layer.w13_weight, layer.w2_weight, bias)
+        L.require_contig(x, logits, out, layer.w13_weight, layer.w2_weight, layer.w13_weight_scale,
+                         layer.w2_weight_scale, bias)
+        if x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or logits.dtype != torch.float32:
+            raise ValueError("make_plan: x/out must be bfloat16 and logits float32")
+        E, two_i, H = layer.w13_weight.shape
+        M = x.shape[0]
+        if tuple(x.shape) != (M, H) or tuple(out.shape) != (M, H) or tuple(logits.shape) != (M, E):
+            raise ValueError("make_plan: x/out must be [M,H] and logits [M,E]")
         a = L.W8A8Args()
         a.M, a.H, a.E, a.K, a.I = M, H, E, self.moe.experts_per_token, two_i // 2
         a.scoring = L.KMOE_SCORE_SOFTMAX if scoring_func == "softmax" else L.KMOE_SCORE_SIGMOID
@@ -172,19 +206,24 @@ class KunlunCompressedTensorsW8A8Int8MoEMethod:
         a.x = x.data_ptr()
         a.w13, a.w13_max = layer.w13_weight.data_ptr(), layer.w13_weight_scale.data_ptr()
         a.w2, a.w2_max = layer.w2_weight.data_ptr(), layer.w2_weight_scale.data_ptr()
+        keep = [x, logits, out, bias, layer]
         if shared_expert is not None:
             ws13, ws13_max, ws2, ws2_max = shared_expert
+            L.require_device(ws13, ws13_max, ws2, ws2_max)
+            L.require_contig(ws13, ws13_max, ws2, ws2_max)
             a.I_shared = ws13.shape[0] // 2
             a.ws13, a.ws13_max, a.ws2, a.ws2_max = (ws13.data_ptr(), ws13_max.data_ptr(), ws2.data_ptr(),
                                                     ws2_max.data_ptr())
+            keep.append(shared_expert)
         a.out_scale = float(out_scale)
         a.out = out.data_ptr()
+        if stage_events is not None:
+            a.stage_events = stage_events
+            keep.append(stage_events)
         lay = L.W8A8Layout()
         L.check(L.lib.kmoe_w8a8_workspace_layout(a, lay))
         ws = _WORKSPACE.get(lay.total_bytes, x.device)
-        L.check(L.lib.kmoe_forward_w8a8(a, L.ptr(ws), ws.numel(), L.stream()))
-        self.last_layout, self.last_workspace = lay, ws  # lets tests read the intermediates
-        return out
+        return W8A8Plan(a, lay, ws, keep)
 
     def apply_staged(self, layer, x, router_logits, topk_group=None, num_expert_group=None, global_num_experts=-1,
                      scoring_func="softmax", routed_scaling_factor=1.0, e_score_correction_bias=None):

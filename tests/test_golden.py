@@ -1,0 +1,100 @@
+"""Golden fixtures (tests/golden/*.npz, written by tests/golden/make_golden.py).
+CPU: the oracle still reproduces them. GPU: the kernels reproduce them through the
+C ABI without needing the oracle at all."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import bits, from_bits, rel_l2
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def load(name):
+    return dict(np.load(os.path.join(GOLD, name), allow_pickle=False))
+
+
+def test_oracle_reproduces_routing_fixture():
+    from oracle import c_oracle as co
+    g = load("routing.npz")
+    w, ids = co.softmax_topk(g["logits"], 4, True)
+    assert np.array_equal(ids, g["softmax_ids"]) and np.array_equal(w, g["softmax_w"])
+    assert list(ids[0]) == [0, 1, 2, 3]  # the tied logits of row 0 resolve to the lowest ids
+    w, ids = co.sigmoid_group_topk_norm(g["logits"], g["bias"], 4, 4, 2, 2.5)
+    assert np.array_equal(ids, g["sigmoid_ids"]) and np.array_equal(w, g["sigmoid_w"])
+
+
+def test_oracle_reproduces_layer_fixture():
+    from oracle import c_oracle as co
+    g = load("w8a8_tiny_layer.npz")
+    out, inter = co.forward_w8a8(g["x"], g["logits"], g["w13"], g["w13_max"], g["w2"], g["w2_max"], int(g["K"]),
+                                 shared=(g["ws13"], g["ws13_max"], g["ws2"], g["ws2_max"]),
+                                 out_scale=float(g["out_scale"]), intermediates=True)
+    assert np.array_equal(out, g["out"])
+    for k in ("topk_ids", "moe_index", "lod", "actq", "down"):
+        assert np.array_equal(inter[k], g[k]), k
+
+
+def test_oracle_reproduces_fp8_fixture():
+    from oracle import c_oracle as co
+    g = load("fp8_group_quant.npz")
+    q, s = co.quant_fp8_group128(g["x"])
+    assert np.array_equal(q, g["q"]) and np.array_equal(s, g["scale"])
+    assert g["q"][0, 1] == 0x7E and g["q"][0, 2] == 0xFE and g["scale"][0, 0] == 1.0
+
+
+@pytest.mark.gpu
+def test_gpu_routing_matches_fixture():
+    from vllm_kunlun_amd import _lib as L
+    g = load("routing.npz")
+    logits = torch.from_numpy(g["logits"]).cuda()
+    bias = torch.from_numpy(g["bias"]).cuda()
+    w = torch.empty(16, 4, device="cuda")
+    ids = torch.empty(16, 4, dtype=torch.int32, device="cuda")
+    L.check(L.lib.kmoe_softmax_topk(L.ptr(logits), 16, 32, 4, 1, L.ptr(w), L.ptr(ids), L.stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(ids.cpu().numpy(), g["softmax_ids"]) and np.array_equal(w.cpu().numpy(), g["softmax_w"])
+    L.check(L.lib.kmoe_sigmoid_group_topk_norm(L.ptr(logits), L.ptr(bias), 16, 32, 4, 4, 2, 2.5, L.ptr(w), L.ptr(ids),
+                                               L.stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(ids.cpu().numpy(), g["sigmoid_ids"]) and np.array_equal(w.cpu().numpy(), g["sigmoid_w"])
+
+
+@pytest.mark.gpu
+def test_gpu_layer_matches_fixture():
+    from vllm_kunlun_amd.ops.fused_moe.layer import FusedMoE
+    from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors_moe import (
+        KunlunCompressedTensorsW8A8Int8MoEMethod)
+    g = load("w8a8_tiny_layer.npz")
+    E, two_i, H = g["w13"].shape
+    K = int(g["K"])
+    method = KunlunCompressedTensorsW8A8Int8MoEMethod()
+    layer = FusedMoE(num_experts=E, top_k=K, hidden_size=H, intermediate_size=two_i // 2, quant_method=method,
+                     device="cuda")
+    layer.w13_weight.data.copy_(torch.from_numpy(g["w13"]))
+    layer.w2_weight.data.copy_(torch.from_numpy(g["w2"]))
+    layer.w13_weight_scale.data.copy_(torch.from_numpy(g["w13_max"] / 127.0))
+    layer.w2_weight_scale.data.copy_(torch.from_numpy(g["w2_max"] / 127.0))
+    method.process_weights_after_loading(layer)
+    # x/127*127 need not round-trip: install the fixture's maxes exactly
+    layer.w13_weight_scale.data.copy_(torch.from_numpy(g["w13_max"]))
+    layer.w2_weight_scale.data.copy_(torch.from_numpy(g["w2_max"]))
+    shared = tuple(torch.from_numpy(g[k]).cuda() for k in ("ws13", "ws13_max", "ws2", "ws2_max"))
+    out = method.apply_monolithic(layer, from_bits(g["x"]).cuda(), torch.from_numpy(g["logits"]).cuda(),
+                                  shared_expert=shared, out_scale=float(g["out_scale"]))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(out), g["out"])
+
+
+@pytest.mark.gpu
+def test_gpu_fp8_quant_matches_fixture():
+    from vllm_kunlun_amd import _lib as L
+    g = load("fp8_group_quant.npz")
+    x = from_bits(g["x"]).cuda()
+    q = torch.empty(3, 128, dtype=torch.uint8, device="cuda")
+    s = torch.empty(3, 1, dtype=torch.float32, device="cuda")
+    L.check(L.lib.kmoe_quant_fp8_group128(L.ptr(x), 128, 3, 128, L.ptr(q), 128, L.ptr(s), L.stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy(), g["q"]) and np.array_equal(s.cpu().numpy(), g["scale"])

@@ -1,0 +1,445 @@
+"""Pins the C oracle (oracle/moe_oracle.c) WITHOUT the reference: the reference
+holds no test, fixture or golden vector for the MoE path and its arithmetic sits
+in closed wheels, so each oracle function is tied down by what the mathematics
+fixes — closed forms, exact integer arithmetic, brute force on tiny inputs,
+invariants — and by independently written code: torch ops, the torch oracle, and
+the DeepSeek-V3 / Qwen3-MoE router and expert modules of the `transformers`
+library installed in the image. Each check is chosen so that a plausible slip
+(dropped term, wrong sign or index, transposed operand, wrong tie-break) fails it.
+"""
+import itertools
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from conftest import bits, from_bits, rel_l2
+from oracle import c_oracle as co
+from oracle import torch_moe as tm
+
+
+# ------------------------------------------------------------------ scalars
+def test_exp_matches_libm_within_2ulp_and_is_monotone():
+    xs = np.concatenate([np.linspace(-86, 86, 40001), np.linspace(-1, 1, 20001), [0.0, -0.0, 1e-30, -1e-30]])
+    xs = xs.astype(np.float32)
+    got = co.exp(xs).astype(np.float64)
+    ref = np.exp(xs.astype(np.float64))
+    ulp = np.spacing(ref.astype(np.float32)).astype(np.float64)
+    assert np.max(np.abs(got - ref) / ulp) < 2.0
+    order = np.argsort(xs, kind="stable")
+    assert np.all(np.diff(got[order]) >= 0)
+    assert co.exp(np.float32(0.0)) == 1.0
+
+
+def test_exp_clamps_outside_range():
+    assert co.exp(np.float32(-1000.0)) == co.exp(np.float32(-86.0)) > 0
+    assert co.exp(np.float32(1000.0)) == co.exp(np.float32(86.0)) < np.inf
+
+
+def test_sigmoid_and_silu_closed_forms():
+    xs = np.linspace(-30, 30, 6001).astype(np.float32)
+    s = co.sigmoid(xs).astype(np.float64)
+    assert np.max(np.abs(s - 1 / (1 + np.exp(-xs.astype(np.float64))))) < 2e-7
+    # symmetry sigma(x) + sigma(-x) = 1 and silu(x) - silu(-x) = x
+    assert np.max(np.abs(s + co.sigmoid(-xs) - 1)) < 3e-7
+    si = co.silu(xs).astype(np.float64)
+    assert np.max(np.abs(si - co.silu(-xs) - xs)) < 4e-6
+    assert co.silu(np.float32(0.0)) == 0.0
+    assert abs(co.silu(np.float32(40.0)) - 40.0) < 1e-5 and abs(co.silu(np.float32(-40.0))) < 1e-10
+    ref = F.silu(torch.from_numpy(xs).double()).numpy()
+    assert np.max(np.abs(si - ref)) < 4e-6
+
+
+# ------------------------------------------------------------------ routing
+def _brute_topk(score, K, eligible=None):
+    idx = [e for e in range(len(score)) if eligible is None or eligible[e]]
+    idx.sort(key=lambda e: (-float(score[e]), e))
+    return idx[:K]
+
+
+@pytest.mark.parametrize("renorm", [False, True])
+def test_softmax_topk_brute_force_and_closed_form(renorm):
+    rng = np.random.default_rng(0)
+    for E, K in [(4, 1), (8, 2), (16, 5), (70, 8), (130, 8)]:
+        logits = rng.standard_normal((64, E)).astype(np.float32)
+        logits[0, :3] = 1.25  # ties
+        logits[1] = 0.0       # all tied: ids must be 0..K-1
+        w, ids = co.softmax_topk(logits, K, renorm)
+        p = torch.softmax(torch.from_numpy(logits).double(), -1).numpy()
+        for m in range(logits.shape[0]):
+            want = _brute_topk(logits[m], K)
+            assert list(ids[m]) == want
+            pw = p[m, want]
+            if renorm:
+                pw = pw / pw.sum()
+            assert np.allclose(w[m], pw, rtol=2e-6, atol=1e-9)
+        if renorm:
+            assert np.allclose(w.sum(-1), 1.0, atol=1e-6)
+        assert list(ids[1]) == list(range(K))
+
+
+def test_softmax_topk_agrees_with_torch_and_transformers_router():
+    from transformers.models.qwen3_moe.configuration_qwen3_moe import Qwen3MoeConfig
+    from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeTopKRouter
+    E, K, M = 128, 8, 512
+    torch.manual_seed(1)
+    logits = torch.randn(M, E)
+    w, ids = co.softmax_topk(logits.numpy(), K, True)
+    tw, tids = tm.softmax_topk(logits, K, True)
+    assert np.array_equal(ids, tids.numpy())  # no exact ties in random normal data
+    assert np.allclose(w, tw.numpy(), rtol=2e-6)
+    cfg = Qwen3MoeConfig(hidden_size=E, num_experts=E, num_experts_per_tok=K, norm_topk_prob=True,
+                         num_hidden_layers=1, vocab_size=8, intermediate_size=8, moe_intermediate_size=8)
+    router = Qwen3MoeTopKRouter(cfg)
+    with torch.no_grad():
+        router.weight.copy_(torch.eye(E))  # logits = hidden_states
+        _, rw, rids = router(logits)
+    assert np.array_equal(ids, rids.numpy())
+    assert np.allclose(w, rw.numpy(), rtol=2e-6)
+
+
+def test_sigmoid_group_topk_brute_force():
+    rng = np.random.default_rng(3)
+    for E, K, ng, tg in [(8, 2, 4, 2), (16, 4, 4, 2), (16, 3, 1, 1), (12, 4, 3, 2), (16, 8, 8, 4)]:
+        logits = rng.standard_normal((40, E)).astype(np.float32)
+        bias = (rng.standard_normal(E) * 0.3).astype(np.float32)
+        w, ids = co.sigmoid_group_topk_norm(logits, bias, K, ng, tg, 2.5)
+        s = co.sigmoid(logits)
+        c = (s + bias).astype(np.float32)
+        gsz = E // ng
+        for m in range(logits.shape[0]):
+            if ng > 1:
+                gscore = [np.float32(sum(sorted(c[m, g * gsz:(g + 1) * gsz], reverse=True)[:2])) for g in range(ng)]
+                groups = _brute_topk(gscore, tg)
+                elig = [e // gsz in groups for e in range(E)]
+            else:
+                elig = None
+            want = _brute_topk(c[m], K, elig)
+            assert list(ids[m]) == want
+            sw = s[m, want].astype(np.float64)
+            assert np.allclose(w[m], sw / sw.sum() * 2.5, rtol=3e-6)
+            if ng > 1:
+                assert len({e // gsz for e in ids[m]}) <= tg
+        assert np.allclose(w.sum(-1), 2.5, rtol=1e-5)
+
+
+def test_sigmoid_group_topk_special_case_reduces_to_plain_sigmoid_topk():
+    rng = np.random.default_rng(4)
+    logits = rng.standard_normal((50, 32)).astype(np.float32)
+    w, ids = co.sigmoid_group_topk_norm(logits, None, 6, 1, 1, 1.0)
+    for m in range(50):
+        assert list(ids[m]) == _brute_topk(logits[m], 6)  # sigmoid is monotone, bias 0
+    w0, ids0 = co.sigmoid_group_topk_norm(logits, np.zeros(32, np.float32), 6, 1, 1, 1.0)
+    assert np.array_equal(ids, ids0) and np.array_equal(w, w0)
+
+
+def test_sigmoid_group_topk_agrees_with_transformers_deepseek_v3_router():
+    from transformers.models.deepseek_v3.configuration_deepseek_v3 import DeepseekV3Config
+    from transformers.models.deepseek_v3.modeling_deepseek_v3 import DeepseekV3TopkRouter
+    E, K, ng, tg, M = 256, 8, 8, 4, 256
+    cfg = DeepseekV3Config(hidden_size=E, n_routed_experts=E, num_experts_per_tok=K, n_group=ng, topk_group=tg,
+                           routed_scaling_factor=2.5, norm_topk_prob=True, num_hidden_layers=1, intermediate_size=8,
+                           moe_intermediate_size=8, vocab_size=8)
+    router = DeepseekV3TopkRouter(cfg)
+    torch.manual_seed(5)
+    logits = torch.randn(M, E)
+    bias = torch.randn(E) * 0.01
+    with torch.no_grad():
+        router.weight.copy_(torch.eye(E))
+        router.e_score_correction_bias.copy_(bias)
+        _, rw, rids = router(logits)
+    w, ids = co.sigmoid_group_topk_norm(logits.numpy(), bias.numpy(), K, ng, tg, 2.5)
+    # the library returns the K experts unsorted: compare as sets, weights by expert
+    for m in range(M):
+        mine = dict(zip(ids[m].tolist(), w[m].tolist()))
+        theirs = dict(zip(rids[m].tolist(), rw[m].tolist()))
+        assert set(mine) == set(theirs)
+        for e in mine:
+            assert math.isclose(mine[e], theirs[e], rel_tol=3e-6)
+    tw, tids = tm.sigmoid_group_topk_norm(logits, bias, K, ng, tg, 2.5)
+    assert np.array_equal(np.sort(ids, -1), np.sort(tids.numpy(), -1))
+
+
+# -------------------------------------------------------------------- align
+@pytest.mark.parametrize("P,E", [(0, 4), (1, 4), (100, 7), (4096, 128), (5000, 1024)])
+def test_align_closed_form(P, E):
+    rng = np.random.default_rng(P + E)
+    ids = rng.integers(0, E, P).astype(np.int32)
+    moe_index, sorted_src, expert_m, lod = co.align(ids, E)
+    order = np.argsort(ids, kind="stable")
+    assert np.array_equal(sorted_src, order)
+    assert np.array_equal(expert_m, np.bincount(ids, minlength=E))
+    assert np.array_equal(lod, np.concatenate([[0], np.cumsum(expert_m)]))
+    inv = np.empty(P, np.int64)
+    inv[order] = np.arange(P)
+    assert np.array_equal(moe_index, inv)
+    t_mi, t_src, t_em, t_lod = tm.align(torch.from_numpy(ids), E)
+    assert np.array_equal(moe_index, t_mi.numpy()) and np.array_equal(lod, t_lod.numpy())
+
+
+def test_align_properties_hypothesis():
+    from hypothesis import given, settings
+    from hypothesis import strategies as st
+
+    @settings(max_examples=60, deadline=None)
+    @given(st.integers(1, 40).flatmap(lambda E: st.tuples(st.just(E), st.lists(st.integers(0, E - 1), max_size=300))))
+    def prop(args):
+        E, lst = args
+        ids = np.array(lst, dtype=np.int32)
+        P = ids.size
+        moe_index, sorted_src, expert_m, lod = co.align(ids, E)
+        assert lod[0] == 0 and lod[E] == P and np.all(np.diff(lod) == expert_m)
+        assert sorted(moe_index.tolist()) == list(range(P))          # a permutation
+        assert np.all(np.diff(ids[sorted_src]) >= 0) if P else True    # experts non-decreasing
+        for e in range(E):                                             # stable inside an expert
+            seg = sorted_src[lod[e]:lod[e + 1]]
+            assert np.all(np.diff(seg) > 0) and np.all(ids[seg] == e)
+        assert np.array_equal(sorted_src[moe_index], np.arange(P))
+
+    prop()
+
+
+def test_block_statistic_sums_to_histogram():
+    ids = np.random.default_rng(0).integers(0, 50, 1234).astype(np.int32)
+    bs = co.block_statistic(ids, 50, 12)
+    assert np.array_equal(bs.sum(0), np.bincount(ids, minlength=50))
+    per = -(-1234 // 12)
+    assert np.array_equal(bs[3], np.bincount(ids[3 * per:4 * per], minlength=50))
+
+
+# -------------------------------------------------------------------- quant
+def test_quant_i8_rows_closed_form_and_invariants():
+    torch.manual_seed(0)
+    x = (torch.randn(64, 1000) * 3).bfloat16()
+    x[0] = 0
+    x[1] = -2.0
+    q, mx = co.quant_i8_rows(bits(x))
+    xf = x.float().numpy()
+    assert np.array_equal(mx, np.abs(xf).max(-1))
+    assert np.all(q[0] == 0) and mx[0] == 0
+    assert np.all(q[1] == -127)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        inv = np.where(mx > 0, np.float32(127.0) / mx, np.float32(0))[:, None].astype(np.float32)
+    want = np.clip(np.rint(xf * inv), -127, 127).astype(np.int8)  # np.rint = half-to-even
+    assert np.array_equal(q, want)
+    assert np.abs(q).max() <= 127
+    am = np.abs(xf).argmax(-1)
+    assert np.all(np.abs(q[np.arange(64), am])[mx > 0] == 127)       # the max element maps to +-127
+    err = np.abs(xf - q.astype(np.float32) * mx[:, None] / 127)
+    assert np.all(err <= mx[:, None] / 254 * 1.0001 + 1e-12)         # half a step
+    tq, tmx = tm.quant_i8_rows(x)
+    # torch evaluates 127/max with its own vectorised division: codes may differ by one
+    # at exact .5 boundaries, nowhere else
+    dq = np.abs(q.astype(np.int32) - tq.numpy().astype(np.int32))
+    assert dq.max() <= 1 and (dq != 0).mean() < 1e-3 and np.array_equal(mx, tmx.numpy().ravel())
+
+
+def test_quant_i8_rounds_half_to_even():
+    # max = 127 makes the scale exactly 1: values k + 0.5 must go to the even neighbour
+    vals = torch.tensor([[127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5]]).bfloat16()
+    q, mx = co.quant_i8_rows(bits(vals))
+    assert mx[0] == 127.0
+    assert q[0].tolist() == [127, 0, 2, 2, 0, -2, -2, 4]
+
+
+def test_e4m3fn_encoder_matches_torch_cast():
+    # every representable value round-trips; random values match torch's RNE cast
+    codes = np.arange(0, 0x7F, dtype=np.uint8)
+    vals = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    for c, v in zip(codes, vals):
+        assert co.lib().orc_f32_to_e4m3fn(float(v)) == c
+        assert co.lib().orc_e4m3fn_to_f32(int(c)) == v
+    rng = np.random.default_rng(0)
+    xs = np.concatenate([rng.standard_normal(4000) * 100, rng.standard_normal(4000) * 0.01,
+                         (vals[:-1] + vals[1:]) / 2, [448.0, 449.0, 1e9, -1e9, 2.0 ** -10, 2.0 ** -9 * 1.5]])
+    xs = xs.astype(np.float32)
+    want = torch.from_numpy(xs).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = np.array([co.lib().orc_f32_to_e4m3fn(float(v)) for v in xs], dtype=np.uint8)
+    nz = (want & 0x7F) != 0  # torch keeps the sign of values that round to zero; so do we
+    assert np.array_equal(got[nz], want[nz])
+    assert np.all((got[~nz] & 0x7F) == 0)
+
+
+def test_quant_fp8_group128_closed_form():
+    torch.manual_seed(1)
+    x = (torch.randn(9, 384) * 5).bfloat16()
+    x[0, :128] = 0
+    q, s = co.quant_fp8_group128(bits(x))
+    tq, ts = tm.quant_fp8_group128(x)
+    assert np.array_equal(s, ts.numpy())
+    assert np.array_equal(s, np.abs(x.float().numpy().reshape(9, 3, 128)).max(-1) / np.float32(448.0))
+    a, b = q, tq.view(torch.uint8).numpy()
+    nz = (b & 0x7F) != 0
+    assert np.array_equal(a[nz], b[nz]) and np.all((a[~nz] & 0x7F) == 0)
+    assert np.all(q[0, :128] == 0) and s[0, 0] == 0
+
+
+# --------------------------------------------------------------- grouped GEMM
+def test_grouped_gemm_accumulators_are_exact_integers():
+    rng = np.random.default_rng(0)
+    E, n, k = 5, 48, 320
+    counts = np.array([3, 0, 11, 1, 6])
+    lod = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(lod[-1])
+    a = rng.integers(-127, 128, (rows, k), dtype=np.int8)
+    w = rng.integers(-127, 128, (E, n, k), dtype=np.int8)
+    a_max = (rng.random(rows) + 0.5).astype(np.float32)
+    w_max = (rng.random((E, n)) + 0.5).astype(np.float32)
+    y, acc = co.grouped_gemm_i8(a, a_max, w, w_max, lod, want_acc=True)
+    for e in range(E):
+        r0, r1 = lod[e], lod[e + 1]
+        want = a[r0:r1].astype(np.int64) @ w[e].astype(np.int64).T          # textbook, int64
+        assert np.array_equal(acc[r0:r1], want)
+        assert np.array_equal(acc[r0:r1], tm._int8_mm(torch.from_numpy(a[r0:r1]), torch.from_numpy(w[e])).numpy())
+        deq = (want.astype(np.float32) * (a_max[r0:r1, None] / np.float32(127))) * (w_max[e][None] / np.float32(127))
+        assert np.array_equal(y[r0:r1], co.f32_to_bf16_bits(deq))            # one fixed f32 order, bf16 RNE
+    # transposing the weight operand, or using the wrong expert's block, must fail the check above:
+    assert not np.array_equal(acc[lod[2]:lod[3]], a[lod[2]:lod[3]].astype(np.int64) @ w[0].astype(np.int64).T)
+
+
+def test_grouped_gemm_row_gather_and_swiglu():
+    rng = np.random.default_rng(1)
+    E, n, k, K = 3, 64, 128, 2
+    tokens = 10
+    a = rng.integers(-127, 128, (tokens, k), dtype=np.int8)
+    a_max = (rng.random(tokens) + 0.5).astype(np.float32)
+    w = rng.integers(-127, 128, (E, n, k), dtype=np.int8)
+    w_max = (rng.random((E, n)) * 0.05 + 0.01).astype(np.float32)
+    ids = rng.integers(0, E, tokens * K).astype(np.int32)
+    _, src, _, lod = co.align(ids, E)
+    y_gather, _ = co.grouped_gemm_i8(a, a_max, w, w_max, lod, row_src=src, src_div=K)
+    y_expanded, _ = co.grouped_gemm_i8(a[src // K], a_max[src // K], w, w_max, lod)
+    assert np.array_equal(y_gather, y_expanded)           # gather == the reference's expanded copy
+    fused, _ = co.grouped_gemm_i8(a, a_max, w, w_max, lod, act=1, row_src=src, src_div=K)
+    assert np.array_equal(fused, co.silu_and_mul(y_gather))  # fused act == act on the stored bf16 tensor
+
+
+def test_bf16_round_trip_helpers():
+    x = torch.randn(1000).float()
+    assert np.array_equal(co.f32_to_bf16_bits(x.numpy()), bits(x.bfloat16()))
+    assert np.array_equal(co.bf16_bits_to_f32(bits(x.bfloat16())), x.bfloat16().float().numpy())
+
+
+def test_silu_and_mul_against_torch():
+    torch.manual_seed(2)
+    y = (torch.randn(33, 96) * 3).bfloat16()
+    got = from_bits(co.silu_and_mul(bits(y))).float()
+    want = tm.silu_and_mul(y).float()
+    assert (got - want).abs().max() <= 2 ** -7 * want.abs().max()   # at most 1 bf16 ulp apart
+    assert (got == want).float().mean() > 0.98
+    # gate is the FIRST half: swapping halves must change the result
+    swapped = from_bits(co.silu_and_mul(bits(torch.cat([y[:, 48:], y[:, :48]], 1)))).float()
+    assert not torch.equal(swapped, got)
+
+
+def test_combine_closed_form():
+    torch.manual_seed(3)
+    M, K, H = 20, 4, 64
+    x = torch.randn(M * K, H).bfloat16()
+    w = torch.rand(M, K)
+    perm = torch.randperm(M * K).int()
+    got = from_bits(co.combine(bits(x), perm.numpy(), w.numpy())).double()
+    want = (x.double()[perm.long()].view(M, K, H) * w.double().unsqueeze(-1)).sum(1)
+    assert (got - want).abs().max() <= 2 ** -8 * want.abs().max() + 1e-6
+    # equal weights: permuting the K slots of a token only changes f32 summation order
+    w1 = torch.full((M, K), 0.25)
+    a = from_bits(co.combine(bits(x), perm.numpy(), w1.numpy())).float()
+    b = from_bits(co.combine(bits(x), perm.view(M, K).flip(1).contiguous().numpy(), w1.numpy())).float()
+    assert (a - b).abs().max() <= 2 ** -7 * a.abs().max()
+    # caller epilogue: bf16(out*scale) + addend
+    add = torch.randn(M, H).bfloat16()
+    e = from_bits(co.combine(bits(x), perm.numpy(), w.numpy(), None, 2.5, bits(add)))
+    base = from_bits(co.combine(bits(x), perm.numpy(), w.numpy()))
+    assert torch.equal(e, (base * 2.5) + add)
+
+
+# ------------------------------------------------------------- whole layer
+def _layer_inputs(M, H, E, K, I, seed, shared_I=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, H, generator=g).bfloat16()
+    logits = torch.randn(M, E, generator=g)
+    w13, s13 = tm.quantize_weight_per_channel(torch.randn(E, 2 * I, H, generator=g) * 0.02)
+    w2, s2 = tm.quantize_weight_per_channel(torch.randn(E, H, I, generator=g) * 0.02)
+    shared = None
+    if shared_I:
+        a, sa = tm.quantize_weight_per_channel(torch.randn(2 * shared_I, H, generator=g) * 0.02)
+        b, sb = tm.quantize_weight_per_channel(torch.randn(H, shared_I, generator=g) * 0.02)
+        shared = (a, (sa * 127).reshape(-1), b, (sb * 127).reshape(-1))
+    return x, logits, w13, s13 * 127, w2, s2 * 127, shared
+
+
+def test_layer_c_oracle_vs_torch_expert_loop():
+    """Two independently written restatements of the reference layer agree within the
+    north-star tolerance; routing ids agree exactly."""
+    M, H, E, K, I = 96, 256, 16, 4, 128
+    x, logits, w13, m13, w2, m2, shared = _layer_inputs(M, H, E, K, I, 0, shared_I=64)
+    bias = torch.randn(E) * 0.01
+    for kw in (dict(scoring="softmax"), dict(scoring="sigmoid", n_group=4, topk_group=2, routed_scale=2.5, bias=bias)):
+        ref = tm.w8a8_moe(x, logits, w13, m13, w2, m2, K, shared=shared, out_scale=1.0,
+                          **{k: v for k, v in kw.items()})
+        np_kw = dict(kw)
+        if "bias" in np_kw:
+            np_kw["bias"] = bias.numpy()
+        out, inter = co.forward_w8a8(bits(x), logits.numpy(), w13.numpy(), m13.numpy(), w2.numpy(), m2.numpy(), K,
+                                     shared=tuple(t.numpy() for t in shared), intermediates=True, **np_kw)
+        assert rel_l2(from_bits(out), ref) <= 1e-2
+        tw, tids = tm.route(logits, K, kw["scoring"], True, kw.get("n_group", 1), kw.get("topk_group", 1),
+                            kw.get("routed_scale", 1.0), kw.get("bias"))
+        assert np.array_equal(np.sort(inter["topk_ids"], -1), np.sort(tids.numpy(), -1))
+
+
+def test_layer_against_transformers_deepseek_experts_on_dequantised_weights():
+    """Independent end-to-end anchor: the library's float expert loop on the
+    DEQUANTISED weights; the W8A8 layer may differ only by quantisation noise."""
+    from transformers.models.deepseek_v3.configuration_deepseek_v3 import DeepseekV3Config
+    from transformers.models.deepseek_v3.modeling_deepseek_v3 import DeepseekV3Experts
+    M, H, E, K, I = 64, 256, 8, 2, 128
+    x, logits, w13, m13, w2, m2, _ = _layer_inputs(M, H, E, K, I, 7)
+    cfg = DeepseekV3Config(hidden_size=H, n_routed_experts=E, num_local_experts=E, moe_intermediate_size=I,
+                           num_experts_per_tok=K, num_hidden_layers=1, intermediate_size=8, vocab_size=8)
+    experts = DeepseekV3Experts(cfg)
+    with torch.no_grad():
+        experts.gate_up_proj.copy_(w13.float() * (m13 / 127))
+        experts.down_proj.copy_(w2.float() * (m2 / 127))
+        w, ids = co.softmax_topk(logits.numpy(), K, True)
+        ref = experts(x.float(), torch.from_numpy(ids).long(), torch.from_numpy(w))
+    out = co.forward_w8a8(bits(x), logits.numpy(), w13.numpy(), m13.numpy(), w2.numpy(), m2.numpy(), K)
+    assert rel_l2(from_bits(out), ref) <= 3e-2   # int8 activation quantisation noise only
+    # a swapped gate/up or a transposed down projection is far outside this band
+    with torch.no_grad():
+        experts.gate_up_proj.copy_(torch.cat([experts.gate_up_proj[:, I:], experts.gate_up_proj[:, :I]], 1))
+        bad = experts(x.float(), torch.from_numpy(ids).long(), torch.from_numpy(w))
+    assert rel_l2(from_bits(out), bad) > 0.3
+
+
+def test_process_weights_scale_times_127_is_the_max_convention():
+    """scale -> max: dequantising with max/127 must reproduce scale (reference:
+    compressed_tensors_moe.py:116-120, scale_mm.py:43-50)."""
+    w = torch.randn(3, 16, 32) * 0.02
+    q, s = tm.quantize_weight_per_channel(w)
+    mx = s * 127.0
+    assert torch.allclose(mx, w.abs().amax(-1, keepdim=True), rtol=1e-6)
+    assert (q.float() * (mx / 127.0) - w).abs().max() <= (s.max() / 2) * 1.001
+
+
+def test_bf16_expert_loop_matches_float_math():
+    """The unquantized torch loop (config 1: 32 tokens, hidden 512, 8 experts, top-2, I=256)."""
+    g = torch.Generator().manual_seed(0)
+    M, H, E, K, I = 32, 512, 8, 2, 256
+    x = torch.randn(M, H, generator=g).bfloat16()
+    logits = torch.randn(M, E, generator=g)
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * 0.02).bfloat16()
+    w2 = (torch.randn(E, H, I, generator=g) * 0.02).bfloat16()
+    out = tm.bf16_moe(x, logits, w13, w2, K, True)
+    p = torch.softmax(logits.double(), -1)
+    tw, ti = p.topk(K, -1)
+    tw = tw / tw.sum(-1, keepdim=True)
+    ref = torch.zeros(M, H, dtype=torch.double)
+    for m in range(M):
+        for k in range(K):
+            e = ti[m, k]
+            h = x[m].double() @ w13[e].double().T
+            ref[m] += tw[m, k] * ((F.silu(h[:I]) * h[I:]) @ w2[e].double().T)
+    assert rel_l2(out, ref) <= 1e-2

@@ -187,7 +187,7 @@ def main():
         achieved = work["g1_ops"] / g1_s / 1e12
         roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s",
                     "frac": achieved / INT8_PEAK_TOPS, "traffic": None}
-    roofline.update(kernel="gemm_i8_kernel (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
+    roofline.update(kernel="grouped_gemm_kernel (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
                     algorithmic_bytes=work["g1_bytes"], algorithmic_ops=work["g1_ops"])
 
     t_s = ms_per_step * 1e-3

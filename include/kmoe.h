@@ -182,6 +182,55 @@ typedef struct kmoe_gemm_i8_args {
  */
 int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* args, kmoe_stream_t stream);
 
+typedef struct kmoe_gemm_bf16_args {
+  const uint16_t* a;      /* [a_rows, k] bf16 activations, row stride lda (elements) */
+  int64_t lda;
+  const int32_t* row_src; /* as in kmoe_gemm_i8_args                                  */
+  int32_t src_div;
+  const uint16_t* w;      /* [E, n, k] bf16 weights, k contiguous                     */
+  const int32_t* lod;     /* [E+1]                                                    */
+  int32_t E, n, k, rows;
+  uint16_t* y;            /* bf16 [rows, n] or [rows, n/2] with SwiGLU                */
+  int64_t ldy;
+  int32_t act;
+  int32_t variant;
+} kmoe_gemm_bf16_args;
+
+/*
+ * Unquantized grouped GEMM: kunlun_ops.moe_fc with bf16 x and weight
+ * (ops/_kunlun_ops.py:578-585, 595-603, 615-622; act="SWISH_GLU" at :595-603).
+ *   y[r,c] = bf16( sum_k float(a[src(r),k]) * float(w[e,c,k]) ), f32 accumulation
+ *   on MFMA (summation order is the hardware's; compare within tolerance).
+ * Limits: k % 8 == 0, n % 16 == 0 (SwiGLU: n % 32 == 0).
+ */
+int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* args, kmoe_stream_t stream);
+
+typedef struct kmoe_gemm_fp8_args {
+  const uint8_t* a;       /* [a_rows, k] e4m3fn activations, row stride lda           */
+  int64_t lda;
+  const float* a_scale;   /* [a_rows, k/128] per-row, per-128-column scales           */
+  const int32_t* row_src;
+  int32_t src_div;
+  const uint8_t* w;       /* [E, n, k] e4m3fn weights                                 */
+  const float* w_scale;   /* [E, n/128, k/128] one scale per 128x128 block            */
+  const int32_t* lod;
+  int32_t E, n, k, rows;
+  uint16_t* y;
+  int64_t ldy;
+  int32_t act;
+  int32_t variant;
+} kmoe_gemm_fp8_args;
+
+/*
+ * fp8-e4m3fn block-scaled grouped GEMM (DeepSeek-V3 recipe). The reference has no
+ * fp8 MoE (platforms/kunlun.py:350-364 rejects fp8; moe_fc only exposes the
+ * scale_n/scale_k arguments, ops/_custom_ops.py:1218-1221).
+ *   y[r,c] = bf16( sum_kb [ sum_{k in kb} a[src(r),k]*w[e,c,k] ] * a_scale[src(r),kb] * w_scale[e,c/128,kb] )
+ * with kb the 128-wide K blocks, f32 accumulation.
+ * Limits: k % 128 == 0, n % 128 == 0 (SwiGLU: n % 256 == 0).
+ */
+int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* args, kmoe_stream_t stream);
+
 /*
  * SiLU-and-mul on a stored gate_up result. Replaces kunlun_ops.swiglu
  * (ops/_custom_ops.py:699-706, called compressed_tensors_moe.py:240-243).
@@ -210,9 +259,14 @@ int kmoe_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_index,
 #define KMOE_SCORE_SOFTMAX 0
 #define KMOE_SCORE_SIGMOID 1
 
-typedef struct kmoe_w8a8_args {
+#define KMOE_FMT_INT8 0      /* int8 weights + per-channel max, per-token int8 activations   */
+#define KMOE_FMT_FP8_BLOCK 1 /* e4m3fn weights + 128x128 block scales, 1x128 activation scales */
+#define KMOE_FMT_BF16 2      /* bf16 weights, no quantisation                                 */
+
+typedef struct kmoe_moe_args {
   /* shape */
   int32_t M, H, E, K, I;
+  int32_t format;        /* KMOE_FMT_*                                           */
   /* routing */
   int32_t scoring;       /* KMOE_SCORE_*                                        */
   int32_t renormalize;   /* softmax only: divide the K weights by their sum     */
@@ -222,16 +276,16 @@ typedef struct kmoe_w8a8_args {
   const float* bias;     /* [E] f32 correction bias or NULL                     */
   /* activations and routed expert weights */
   const uint16_t* x;     /* [M,H] bf16                                          */
-  const int8_t* w13;     /* [E,2I,H]                                            */
-  const float* w13_max;  /* [E,2I]                                              */
-  const int8_t* w2;      /* [E,H,I]                                             */
-  const float* w2_max;   /* [E,H]                                               */
-  /* optional dense shared expert (I_shared = 0: none) */
+  const void* w13;       /* [E,2I,H] int8 / e4m3fn / bf16                       */
+  const float* w13_max;  /* INT8: [E,2I] absmax. FP8: [E,2I/128,H/128] scales. BF16: NULL */
+  const void* w2;        /* [E,H,I]                                             */
+  const float* w2_max;   /* INT8: [E,H]. FP8: [E,H/128,I/128]. BF16: NULL       */
+  /* optional dense shared expert in the same format (I_shared = 0: none) */
   int32_t I_shared;
-  const int8_t* ws13;    /* [2*I_shared,H]                                      */
-  const float* ws13_max; /* [2*I_shared]                                        */
-  const int8_t* ws2;     /* [H,I_shared]                                        */
-  const float* ws2_max;  /* [H]                                                 */
+  const void* ws13;      /* [2*I_shared,H]                                      */
+  const float* ws13_max; /* INT8: [2*I_shared]. FP8: [2*I_shared/128,H/128]     */
+  const void* ws2;       /* [H,I_shared]                                        */
+  const float* ws2_max;  /* INT8: [H]. FP8: [H/128,I_shared/128]                */
   /* caller epilogue: out = routed*out_scale (+ shared) */
   float out_scale;
   uint16_t* out;         /* [M,H] bf16                                          */
@@ -239,7 +293,7 @@ typedef struct kmoe_w8a8_args {
      recorded on the stream before stage s and entry 2s+1 after it (NULL entries
      are skipped). Leave NULL under graph capture.                             */
   void* const* stage_events;
-} kmoe_w8a8_args;
+} kmoe_moe_args;
 
 #define KMOE_STAGE_ROUTING 0
 #define KMOE_STAGE_ALIGN 1
@@ -251,28 +305,32 @@ typedef struct kmoe_w8a8_args {
 #define KMOE_STAGE_COMBINE 7
 #define KMOE_N_STAGES 8
 
-/* Byte offsets of the intermediates kmoe_forward_w8a8 keeps in its workspace. */
-typedef struct kmoe_w8a8_layout {
+/* Byte offsets of the intermediates kmoe_moe_forward keeps in its workspace.
+ * xq/actq hold int8 or e4m3fn codes; xmax/actmax hold row maxes (INT8) or
+ * per-128-column scales (FP8); all four are unused for BF16. */
+typedef struct kmoe_moe_layout {
   size_t total_bytes;
   size_t topk_w, topk_ids, moe_index, sorted_src, expert_m, lod, align_ws;
   size_t xq, xmax, act, actq, actmax, down;
   size_t sh_lod, sh_act, sh_actq, sh_actmax, sh_out;
-} kmoe_w8a8_layout;
+} kmoe_moe_layout;
 
-/* Workspace layout (and total size) for a shape; only the shape fields of args are read. */
-int kmoe_w8a8_workspace_layout(const kmoe_w8a8_args* args, kmoe_w8a8_layout* layout);
+/* Workspace layout (and total size) for a shape; only the shape and format fields of args are read. */
+int kmoe_moe_workspace_layout(const kmoe_moe_args* args, kmoe_moe_layout* layout);
 
 /*
- * The whole layer: routing -> align -> per-token int8 quant -> gate_up GEMM with
- * fused SiLU-mul -> per-row int8 quant -> down GEMM -> weighted combine
- * (+ shared expert, + caller epilogue). Replaces
+ * The whole layer: routing -> align -> activation quant -> gate_up GEMM with
+ * fused SiLU-mul -> activation quant -> down GEMM -> weighted combine
+ * (+ shared expert, + caller epilogue). Replaces, for KMOE_FMT_INT8,
  * KunlunCompressedTensorsW8A8Int8MoEMethod.apply_monolithic
- * (compressed_tensors_moe.py:122-291) and, for the shared expert,
- * KunlunScaledMMLinearKernel.apply_weights (quantization/kernels/scale_mm.py:52-90).
- * Results are bit-identical to running the stage functions above one by one.
+ * (compressed_tensors_moe.py:122-291) with the shared expert of
+ * KunlunScaledMMLinearKernel.apply_weights (quantization/kernels/scale_mm.py:52-90);
+ * for KMOE_FMT_BF16, KunlunOps.fused_moe (ops/_kunlun_ops.py:377-637). KMOE_FMT_FP8_BLOCK
+ * has no counterpart in the reference. Results are bit-identical to running the
+ * stage functions above one by one.
  */
-int kmoe_forward_w8a8(const kmoe_w8a8_args* args, void* workspace,
-                      size_t workspace_bytes, kmoe_stream_t stream);
+int kmoe_moe_forward(const kmoe_moe_args* args, void* workspace,
+                     size_t workspace_bytes, kmoe_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -217,3 +217,71 @@ def forward_w8a8(x_bits, logits, w13, w13_max, w2, w2_max, K, scoring="softmax",
                            C.c_float(out_scale), _p(out), _p(g("topk_w")), _p(g("topk_ids")), _p(g("moe_index")),
                            _p(g("lod")), _p(g("actq")), _p(g("actmax")), _p(g("down")))
     return (out, inter) if intermediates else out
+
+
+def grouped_gemm_bf16(a_bits, w_bits, lod, act=0, row_src=None, src_div=1):
+    a_bits = _c(a_bits, np.uint16)
+    w_bits = _c(w_bits, np.uint16)
+    lod = _c(lod, np.int32)
+    E, n, k = w_bits.shape
+    rows = int(lod[-1])
+    row_src = None if row_src is None else _c(row_src, np.int32)
+    n_out = n // 2 if act else n
+    y = np.zeros((rows, n_out), np.uint16)
+    lib().orc_grouped_gemm_bf16(_p(a_bits), C.c_int64(a_bits.shape[1]), _p(row_src), int(src_div), _p(w_bits),
+                                _p(lod), E, n, k, _p(y), C.c_int64(n_out), int(act))
+    return y
+
+
+def grouped_gemm_fp8(a, a_scale, w, w_scale, lod, act=0, row_src=None, src_div=1):
+    a = _c(a, np.uint8)
+    w = _c(w, np.uint8)
+    a_scale = _c(a_scale, np.float32)
+    w_scale = _c(w_scale, np.float32)
+    lod = _c(lod, np.int32)
+    E, n, k = w.shape
+    rows = int(lod[-1])
+    row_src = None if row_src is None else _c(row_src, np.int32)
+    n_out = n // 2 if act else n
+    y = np.zeros((rows, n_out), np.uint16)
+    lib().orc_grouped_gemm_fp8(_p(a), C.c_int64(a.shape[1]), _p(a_scale), _p(row_src), int(src_div), _p(w),
+                               _p(w_scale), _p(lod), E, n, k, _p(y), C.c_int64(n_out), int(act))
+    return y
+
+
+def _route(logits, K, scoring, renormalize, n_group, topk_group, routed_scale, bias):
+    if scoring == "softmax":
+        return softmax_topk(logits, K, renormalize)
+    return sigmoid_group_topk_norm(logits, bias, K, n_group, topk_group, routed_scale)
+
+
+def forward_bf16(x_bits, logits, w13_bits, w2_bits, K, scoring="softmax", renormalize=True, n_group=1, topk_group=1,
+                 routed_scale=1.0, bias=None):
+    """Unquantized layer in the stage order of KunlunOps.fused_moe (ops/_kunlun_ops.py:412-637)."""
+    E = w13_bits.shape[0]
+    w, ids = _route(logits, K, scoring, renormalize, n_group, topk_group, routed_scale, bias)
+    moe_index, src, _, lod = align(ids, E)
+    act = grouped_gemm_bf16(x_bits, w13_bits, lod, act=1, row_src=src, src_div=K)
+    down = grouped_gemm_bf16(act, w2_bits, lod)
+    return combine(down, moe_index, w)
+
+
+def forward_fp8(x_bits, logits, w13, w13_scale, w2, w2_scale, K, scoring="softmax", renormalize=True, n_group=1,
+                topk_group=1, routed_scale=1.0, bias=None, shared=None, out_scale=1.0):
+    """fp8 block-scaled layer: same stage order as the int8 layer with the fp8 quantiser and GEMM."""
+    E = w13.shape[0]
+    M = x_bits.shape[0]
+    w, ids = _route(logits, K, scoring, renormalize, n_group, topk_group, routed_scale, bias)
+    moe_index, src, _, lod = align(ids, E)
+    xq, xs = quant_fp8_group128(x_bits)
+    act = grouped_gemm_fp8(xq, xs, w13, w13_scale, lod, act=1, row_src=src, src_div=K)
+    aq, as_ = quant_fp8_group128(act)
+    down = grouped_gemm_fp8(aq, as_, w2, w2_scale, lod)
+    sh = None
+    if shared is not None:
+        ws13, ws13_scale, ws2, ws2_scale = shared
+        dlod = np.array([0, M], np.int32)
+        sact = grouped_gemm_fp8(xq, xs, ws13[None], ws13_scale[None], dlod, act=1)
+        sq, ss = quant_fp8_group128(sact)
+        sh = grouped_gemm_fp8(sq, ss, ws2[None], ws2_scale[None], dlod)
+    return combine(down, moe_index, w, None, out_scale, sh)

@@ -320,6 +320,82 @@ ORC_API void orc_grouped_gemm_i8(const int8_t* a, int64_t lda, const float* a_ma
   }
 }
 
+/* moe_fc with bf16 x and weight (ops/_kunlun_ops.py:578-585, 595-603, 615-622):
+ * f32 accumulation in ascending k, one bf16 rounding. A device MFMA sums in its
+ * own order, so comparisons with this function are within tolerance, not exact. */
+ORC_API void orc_grouped_gemm_bf16(const uint16_t* a, int64_t lda, const int32_t* row_src, int src_div,
+                                   const uint16_t* w, const int32_t* lod, int E, int n, int k, uint16_t* y,
+                                   int64_t ldy, int act) {
+  for (int e = 0; e < E; ++e) {
+    const int r0 = lod[e], r1 = lod[e + 1];
+    const uint16_t* we = w + (size_t)e * n * k;
+#pragma omp parallel for schedule(static)
+    for (int r = r0; r < r1; ++r) {
+      const int sr = row_src ? row_src[r] / src_div : r;
+      const uint16_t* ar = a + (size_t)sr * lda;
+      const int half = n / 2;
+      const int nout = act ? half : n;
+      for (int c = 0; c < nout; ++c) {
+        float g = 0.0f, u = 0.0f;
+        const uint16_t* wg = we + (size_t)c * k;
+        for (int i = 0; i < k; ++i) g += bf16_to_f32(ar[i]) * bf16_to_f32(wg[i]);
+        if (act) {
+          const uint16_t* wu = we + (size_t)(half + c) * k;
+          for (int i = 0; i < k; ++i) u += bf16_to_f32(ar[i]) * bf16_to_f32(wu[i]);
+          y[(size_t)r * ldy + c] =
+              f32_to_bf16(orc_silu(bf16_to_f32(f32_to_bf16(g))) * bf16_to_f32(f32_to_bf16(u)));
+        } else {
+          y[(size_t)r * ldy + c] = f32_to_bf16(g);
+        }
+      }
+    }
+  }
+}
+
+/* fp8-e4m3fn block-scaled grouped GEMM (no reference counterpart; DeepSeek-V3 recipe):
+ * per 128-wide K block the exact f32 sum of code products, times the activation
+ * scale of (row, block) and the weight scale of (channel/128, block); blocks added in
+ * ascending order; one bf16 rounding. Device MFMA order differs: tolerance, not exact. */
+ORC_API void orc_grouped_gemm_fp8(const uint8_t* a, int64_t lda, const float* a_scale, const int32_t* row_src,
+                                  int src_div, const uint8_t* w, const float* w_scale, const int32_t* lod, int E,
+                                  int n, int k, uint16_t* y, int64_t ldy, int act) {
+  float lut[256];
+  for (int i = 0; i < 256; ++i) lut[i] = orc_e4m3fn_to_f32((uint8_t)i);
+  const int kb_n = k / 128, nb_n = n / 128;
+  for (int e = 0; e < E; ++e) {
+    const int r0 = lod[e], r1 = lod[e + 1];
+    const uint8_t* we = w + (size_t)e * n * k;
+    const float* ws = w_scale + (size_t)e * nb_n * kb_n;
+#pragma omp parallel for schedule(static)
+    for (int r = r0; r < r1; ++r) {
+      const int sr = row_src ? row_src[r] / src_div : r;
+      const uint8_t* ar = a + (size_t)sr * lda;
+      const float* as = a_scale + (size_t)sr * kb_n;
+      const int half = n / 2;
+      const int nout = act ? half : n;
+      for (int c = 0; c < nout; ++c) {
+        float tot[2] = {0.0f, 0.0f};
+        for (int part = 0; part < (act ? 2 : 1); ++part) {
+          const int cc = part ? half + c : c;
+          const uint8_t* wr = we + (size_t)cc * k;
+          float t = 0.0f;
+          for (int kb = 0; kb < kb_n; ++kb) {
+            float s = 0.0f;
+            for (int i = 0; i < 128; ++i) s += lut[ar[kb * 128 + i]] * lut[wr[kb * 128 + i]];
+            t = fmaf(s, as[kb] * ws[(size_t)(cc / 128) * kb_n + kb], t);
+          }
+          tot[part] = t;
+        }
+        if (act)
+          y[(size_t)r * ldy + c] =
+              f32_to_bf16(orc_silu(bf16_to_f32(f32_to_bf16(tot[0]))) * bf16_to_f32(f32_to_bf16(tot[1])));
+        else
+          y[(size_t)r * ldy + c] = f32_to_bf16(tot[0]);
+      }
+    }
+  }
+}
+
 /* silu_and_mul on a stored gate_up tensor (compressed_tensors_moe.py:240-243). */
 ORC_API void orc_silu_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, uint16_t* out, int64_t ld_out) {
   for (int r = 0; r < R; ++r)

@@ -24,7 +24,7 @@ def _declared_functions():
 
 def test_header_declares_functions():
     names = _declared_functions()
-    assert "kmoe_forward_w8a8" in names and "kmoe_grouped_gemm_i8" in names and len(names) >= 15
+    assert "kmoe_moe_forward" in names and "kmoe_grouped_gemm_i8" in names and len(names) >= 15
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -37,9 +37,9 @@ def test_library_exports_every_declared_symbol(L):
 def test_struct_layouts_match_the_header(L):
     # sizes implied by the C declarations (LP64): guards the ctypes mirrors against drift
     assert C.sizeof(L.GemmI8Args) == 8 + 8 + 8 + 8 + 8 + 8 + 8 + 8 + 16 + 8 + 8 + 8 + 8
-    assert C.sizeof(L.W8A8Layout) == 19 * 8
-    a = L.W8A8Args()
-    assert L.W8A8Args.M.offset == 0 and L.W8A8Args.logits.offset == 40 and C.sizeof(a) % 8 == 0
+    assert C.sizeof(L.MoELayout) == 19 * 8
+    a = L.MoEArgs()
+    assert L.MoEArgs.M.offset == 0 and L.MoEArgs.logits.offset == 48 and C.sizeof(a) % 8 == 0
 
 
 def test_null_and_shape_errors_are_status_codes(L):
@@ -79,24 +79,24 @@ def test_gemm_argument_validation(L):
 
 
 def test_forward_validation_and_workspace_layout(L):
-    a = L.W8A8Args()
-    lay = L.W8A8Layout()
+    a = L.MoEArgs()
+    lay = L.MoELayout()
     a.M, a.H, a.E, a.K, a.I = 64, 2048, 128, 8, 768
-    assert L.lib.kmoe_w8a8_workspace_layout(a, lay) == 0
+    assert L.lib.kmoe_moe_workspace_layout(a, lay) == 0
     P = 64 * 8
     assert lay.total_bytes >= P * 2048 * 2 + P * 768 * 3 + 64 * 2048
-    offs = [getattr(lay, n) for n, _ in L.W8A8Layout._fields_[1:]]
+    offs = [getattr(lay, n) for n, _ in L.MoELayout._fields_[1:]]
     assert offs == sorted(offs) and all(o % 256 == 0 for o in offs)
     a.K = 200
-    assert L.lib.kmoe_w8a8_workspace_layout(a, lay) == -2
+    assert L.lib.kmoe_moe_workspace_layout(a, lay) == -2
     a.K = 8
-    assert L.lib.kmoe_forward_w8a8(a, None, 0, None) == -1        # tensor pointers missing
+    assert L.lib.kmoe_moe_forward(a, None, 0, None) == -1        # tensor pointers missing
     for f in ("logits", "x", "w13", "w13_max", "w2", "w2_max", "out"):
         setattr(a, f, 0x1000)
-    assert L.lib.kmoe_forward_w8a8(a, None, 0, None) == -4        # no workspace
-    assert L.lib.kmoe_forward_w8a8(a, C.c_void_p(0x10000), 16, None) == -4
+    assert L.lib.kmoe_moe_forward(a, None, 0, None) == -4        # no workspace
+    assert L.lib.kmoe_moe_forward(a, C.c_void_p(0x10000), 16, None) == -4
     a.scoring = 9
-    assert L.lib.kmoe_forward_w8a8(a, C.c_void_p(0x10000), 1 << 40, None) == -3
+    assert L.lib.kmoe_moe_forward(a, C.c_void_p(0x10000), 1 << 40, None) == -3
 
 
 def test_python_errors_follow_the_reference_convention(L):

@@ -1,5 +1,5 @@
 """GPU parity of the whole W8A8 layer through the plugin surface
-(FusedMoE -> quant_method.apply_monolithic -> kmoe_forward_w8a8 in libkmoe.so).
+(FusedMoE -> quant_method.apply_monolithic -> kmoe_moe_forward in libkmoe.so).
 
 Checked against (1) the C oracle, bit for bit, including the intermediates the
 north star names (routing ids, sorted token map, second-GEMM int8 inputs), and

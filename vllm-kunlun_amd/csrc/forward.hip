@@ -1,5 +1,5 @@
-// Host side of libkmoe: error state, and the fused W8A8 layer call that strings
-// the stage kernels together on one stream out of one caller-owned workspace.
+// Host side of libkmoe: error state, and the fused layer call that strings the
+// stage kernels together on one stream out of one caller-owned workspace.
 #include <cstdarg>
 #include <cstdio>
 
@@ -28,30 +28,143 @@ int check_launch(const char* what) {
 using namespace kmoe;
 
 extern "C" const char* kmoe_last_error(void) { return g_error; }
-extern "C" const char* kmoe_version(void) { return "kmoe 0.1 gfx950"; }
+extern "C" const char* kmoe_version(void) { return "kmoe 0.2 gfx950"; }
 
 namespace {
 
-int check_shape(const kmoe_w8a8_args* a) {
-  KMOE_REQUIRE(a, KMOE_ERR_NULL, "forward_w8a8: args is NULL");
+int check_shape(const kmoe_moe_args* a) {
+  KMOE_REQUIRE(a, KMOE_ERR_NULL, "moe_forward: args is NULL");
   KMOE_REQUIRE(a->M >= 0 && a->H >= 16 && a->E >= 1 && a->K >= 1 && a->I >= 16, KMOE_ERR_SHAPE,
-               "forward_w8a8: M=%d H=%d E=%d K=%d I=%d", a->M, a->H, a->E, a->K, a->I);
-  KMOE_REQUIRE(a->H % 16 == 0 && a->I % 16 == 0, KMOE_ERR_SHAPE, "forward_w8a8: H=%d and I=%d must be multiples of 16",
-               a->H, a->I);
-  KMOE_REQUIRE(a->K <= a->E && a->K <= 64 && a->E <= 1024, KMOE_ERR_SHAPE, "forward_w8a8: K=%d E=%d out of range", a->K,
+               "moe_forward: M=%d H=%d E=%d K=%d I=%d", a->M, a->H, a->E, a->K, a->I);
+  KMOE_REQUIRE(a->format == KMOE_FMT_INT8 || a->format == KMOE_FMT_FP8_BLOCK || a->format == KMOE_FMT_BF16,
+               KMOE_ERR_UNSUPPORTED, "moe_forward: format=%d unknown", a->format);
+  const int mult = a->format == KMOE_FMT_FP8_BLOCK ? 128 : 16;
+  KMOE_REQUIRE(a->H % mult == 0 && a->I % mult == 0, KMOE_ERR_SHAPE,
+               "moe_forward: H=%d and I=%d must be multiples of %d", a->H, a->I, mult);
+  KMOE_REQUIRE(a->K <= a->E && a->K <= 64 && a->E <= 1024, KMOE_ERR_SHAPE, "moe_forward: K=%d E=%d out of range", a->K,
                a->E);
-  KMOE_REQUIRE(a->I_shared >= 0 && a->I_shared % 16 == 0, KMOE_ERR_SHAPE,
-               "forward_w8a8: I_shared=%d must be a non-negative multiple of 16", a->I_shared);
-  KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "forward_w8a8: M*K too large");
+  KMOE_REQUIRE(a->I_shared >= 0 && a->I_shared % mult == 0, KMOE_ERR_SHAPE,
+               "moe_forward: I_shared=%d must be a non-negative multiple of %d", a->I_shared, mult);
+  KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "moe_forward: M*K too large");
+  return KMOE_OK;
+}
+
+// One expert-MLP pass (gate_up + SiLU-mul, requantise, down) over `rows` rows in
+// the layer's format. `x_rows` is what the first GEMM reads: quantised codes, or
+// the bf16 activations themselves for KMOE_FMT_BF16.
+struct MlpPass {
+  int format;
+  const void* x_rows;      // [*, H]
+  const float* x_aux;      // row maxes / group scales (NULL for bf16)
+  const int32_t* row_src;  // gather for the first GEMM (NULL: identity)
+  int src_div;
+  const void *w13, *w2;
+  const float *w13_aux, *w2_aux;
+  const int32_t* lod;
+  int E, H, I, rows;
+  uint16_t* act;   // [rows, I] bf16
+  void* actq;      // [rows, I] codes
+  float* act_aux;  // [rows] or [rows, I/128]
+  uint16_t* out;   // [rows, H] bf16
+};
+
+int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
+  const int n = first ? 2 * m.I : m.H;
+  const int k = first ? m.H : m.I;
+  const void* a = first ? m.x_rows : (m.format == KMOE_FMT_BF16 ? static_cast<const void*>(m.act) : m.actq);
+  const float* a_aux = first ? m.x_aux : m.act_aux;
+  const void* w = first ? m.w13 : m.w2;
+  const float* w_aux = first ? m.w13_aux : m.w2_aux;
+  uint16_t* y = first ? m.act : m.out;
+  const int64_t ldy = first ? m.I : m.H;
+  const int act = first ? KMOE_ACT_SWIGLU : KMOE_ACT_NONE;
+  const int32_t* row_src = first ? m.row_src : nullptr;
+  const int src_div = first ? m.src_div : 1;
+  if (m.format == KMOE_FMT_INT8) {
+    kmoe_gemm_i8_args g = {};
+    g.a = static_cast<const int8_t*>(a);
+    g.lda = k;
+    g.a_max = a_aux;
+    g.row_src = row_src;
+    g.src_div = src_div;
+    g.w = static_cast<const int8_t*>(w);
+    g.w_max = w_aux;
+    g.lod = m.lod;
+    g.E = m.E;
+    g.n = n;
+    g.k = k;
+    g.rows = m.rows;
+    g.y = y;
+    g.ldy = ldy;
+    g.act = act;
+    return kmoe_grouped_gemm_i8(&g, stream);
+  }
+  if (m.format == KMOE_FMT_FP8_BLOCK) {
+    kmoe_gemm_fp8_args g = {};
+    g.a = static_cast<const uint8_t*>(a);
+    g.lda = k;
+    g.a_scale = a_aux;
+    g.row_src = row_src;
+    g.src_div = src_div;
+    g.w = static_cast<const uint8_t*>(w);
+    g.w_scale = w_aux;
+    g.lod = m.lod;
+    g.E = m.E;
+    g.n = n;
+    g.k = k;
+    g.rows = m.rows;
+    g.y = y;
+    g.ldy = ldy;
+    g.act = act;
+    return kmoe_grouped_gemm_fp8_block(&g, stream);
+  }
+  kmoe_gemm_bf16_args g = {};
+  g.a = static_cast<const uint16_t*>(a);
+  g.lda = k;
+  g.row_src = row_src;
+  g.src_div = src_div;
+  g.w = static_cast<const uint16_t*>(w);
+  g.lod = m.lod;
+  g.E = m.E;
+  g.n = n;
+  g.k = k;
+  g.rows = m.rows;
+  g.y = y;
+  g.ldy = ldy;
+  g.act = act;
+  return kmoe_grouped_gemm_bf16(&g, stream);
+}
+
+template <class Mark>
+int run_mlp(const MlpPass& m, kmoe_stream_t stream, Mark&& mark) {
+  int rc;
+  mark(KMOE_STAGE_GEMM1, 0);
+  rc = run_gemm(m, true, stream);
+  if (rc) return rc;
+  mark(KMOE_STAGE_GEMM1, 1);
+  mark(KMOE_STAGE_QUANT2, 0);
+  if (m.format == KMOE_FMT_INT8) {
+    rc = kmoe_quant_i8_rows(m.act, m.I, m.rows, m.I, static_cast<int8_t*>(m.actq), m.I, m.act_aux, stream);
+  } else if (m.format == KMOE_FMT_FP8_BLOCK) {
+    rc = kmoe_quant_fp8_group128(m.act, m.I, m.rows, m.I, static_cast<uint8_t*>(m.actq), m.I, m.act_aux, stream);
+  }
+  if (rc) return rc;
+  mark(KMOE_STAGE_QUANT2, 1);
+  mark(KMOE_STAGE_GEMM2, 0);
+  rc = run_gemm(m, false, stream);
+  if (rc) return rc;
+  mark(KMOE_STAGE_GEMM2, 1);
   return KMOE_OK;
 }
 
 }  // namespace
 
-extern "C" int kmoe_w8a8_workspace_layout(const kmoe_w8a8_args* a, kmoe_w8a8_layout* L) {
+extern "C" int kmoe_moe_workspace_layout(const kmoe_moe_args* a, kmoe_moe_layout* L) {
   if (int rc = check_shape(a)) return rc;
-  KMOE_REQUIRE(L, KMOE_ERR_NULL, "w8a8_workspace_layout: layout is NULL");
+  KMOE_REQUIRE(L, KMOE_ERR_NULL, "moe_workspace_layout: layout is NULL");
   const size_t M = a->M, H = a->H, E = a->E, K = a->K, I = a->I, P = M * K, Is = a->I_shared;
+  const bool quant = a->format != KMOE_FMT_BF16;
+  const bool fp8 = a->format == KMOE_FMT_FP8_BLOCK;
   size_t off = 0;
   auto take = [&](size_t bytes) {
     const size_t at = off;
@@ -65,37 +178,38 @@ extern "C" int kmoe_w8a8_workspace_layout(const kmoe_w8a8_args* a, kmoe_w8a8_lay
   L->expert_m = take(E * 4);
   L->lod = take((E + 1) * 4);
   L->align_ws = take(kmoe_align_workspace_bytes(static_cast<int>(P), a->E));
-  L->xq = take(M * H);
-  L->xmax = take(M * 4);
+  L->xq = take(quant ? M * H : 0);
+  L->xmax = take(quant ? M * 4 * (fp8 ? H / 128 : 1) : 0);
   L->act = take(P * I * 2);
-  L->actq = take(P * I);
-  L->actmax = take(P * 4);
+  L->actq = take(quant ? P * I : 0);
+  L->actmax = take(quant ? P * 4 * (fp8 ? I / 128 : 1) : 0);
   L->down = take(P * H * 2);
   L->sh_lod = take(2 * 4);
   L->sh_act = take(M * Is * 2);
-  L->sh_actq = take(M * Is);
-  L->sh_actmax = take(M * 4);
+  L->sh_actq = take(quant ? M * Is : 0);
+  L->sh_actmax = take(quant ? M * 4 * (fp8 ? Is / 128 : 1) : 0);
   L->sh_out = take(Is ? M * H * 2 : 0);
   L->total_bytes = off;
   return KMOE_OK;
 }
 
-extern "C" int kmoe_forward_w8a8(const kmoe_w8a8_args* a, void* workspace, size_t workspace_bytes,
-                                 kmoe_stream_t stream) {
-  kmoe_w8a8_layout L;
-  if (int rc = kmoe_w8a8_workspace_layout(a, &L)) return rc;
+extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t workspace_bytes,
+                                kmoe_stream_t stream) {
+  kmoe_moe_layout L;
+  if (int rc = kmoe_moe_workspace_layout(a, &L)) return rc;
   if (a->M == 0) return KMOE_OK;
-  KMOE_REQUIRE(a->logits && a->x && a->w13 && a->w13_max && a->w2 && a->w2_max && a->out, KMOE_ERR_NULL,
-               "forward_w8a8: NULL tensor pointer");
-  KMOE_REQUIRE(a->I_shared == 0 || (a->ws13 && a->ws13_max && a->ws2 && a->ws2_max), KMOE_ERR_NULL,
-               "forward_w8a8: shared expert pointers are NULL");
+  const bool quant = a->format != KMOE_FMT_BF16;
+  KMOE_REQUIRE(a->logits && a->x && a->w13 && a->w2 && a->out, KMOE_ERR_NULL, "moe_forward: NULL tensor pointer");
+  KMOE_REQUIRE(!quant || (a->w13_max && a->w2_max), KMOE_ERR_NULL, "moe_forward: weight max/scale pointers are NULL");
+  KMOE_REQUIRE(a->I_shared == 0 || (a->ws13 && a->ws2 && (!quant || (a->ws13_max && a->ws2_max))), KMOE_ERR_NULL,
+               "moe_forward: shared expert pointers are NULL");
   KMOE_REQUIRE(a->scoring == KMOE_SCORE_SOFTMAX || a->scoring == KMOE_SCORE_SIGMOID, KMOE_ERR_UNSUPPORTED,
-               "forward_w8a8: scoring=%d unknown", a->scoring);
-  KMOE_REQUIRE(workspace, KMOE_ERR_WORKSPACE, "forward_w8a8: workspace is NULL (need %zu bytes)", L.total_bytes);
-  KMOE_REQUIRE(workspace_bytes >= L.total_bytes, KMOE_ERR_WORKSPACE, "forward_w8a8: workspace %zu < %zu bytes",
+               "moe_forward: scoring=%d unknown", a->scoring);
+  KMOE_REQUIRE(workspace, KMOE_ERR_WORKSPACE, "moe_forward: workspace is NULL (need %zu bytes)", L.total_bytes);
+  KMOE_REQUIRE(workspace_bytes >= L.total_bytes, KMOE_ERR_WORKSPACE, "moe_forward: workspace %zu < %zu bytes",
                workspace_bytes, L.total_bytes);
   KMOE_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, KMOE_ERR_WORKSPACE,
-               "forward_w8a8: workspace must be 256-byte aligned");
+               "moe_forward: workspace must be 256-byte aligned");
 
   char* ws = static_cast<char*>(workspace);
   auto at = [&](size_t off) { return static_cast<void*>(ws + off); };
@@ -104,10 +218,8 @@ extern "C" int kmoe_forward_w8a8(const kmoe_w8a8_args* a, void* workspace, size_
   int32_t* moe_index = static_cast<int32_t*>(at(L.moe_index));
   int32_t* sorted_src = static_cast<int32_t*>(at(L.sorted_src));
   int32_t* lod = static_cast<int32_t*>(at(L.lod));
-  int8_t* xq = static_cast<int8_t*>(at(L.xq));
-  float* xmax = static_cast<float*>(at(L.xmax));
   const int M = a->M, H = a->H, E = a->E, K = a->K, I = a->I, P = M * K;
-  int rc;
+  int rc = KMOE_OK;
   auto mark = [&](int stage, int end) {
     if (!a->stage_events) return;
     void* ev = a->stage_events[2 * stage + end];
@@ -130,109 +242,74 @@ extern "C" int kmoe_forward_w8a8(const kmoe_w8a8_args* a, void* workspace, size_
                   kmoe_align_workspace_bytes(P, E), stream);
   if (rc) return rc;
   mark(KMOE_STAGE_ALIGN, 1);
+  // 3. quantise each TOKEN row once (the reference quantises the K-times expanded copy; same values)
   mark(KMOE_STAGE_QUANT1, 0);
-  // 3. one int8 row per TOKEN (the reference quantises the K-times expanded copy; same values)
-  rc = kmoe_quant_i8_rows(a->x, H, M, H, xq, H, xmax, stream);
+  const void* x_rows = a->x;
+  if (a->format == KMOE_FMT_INT8) {
+    rc = kmoe_quant_i8_rows(a->x, H, M, H, static_cast<int8_t*>(at(L.xq)), H, static_cast<float*>(at(L.xmax)), stream);
+    x_rows = at(L.xq);
+  } else if (a->format == KMOE_FMT_FP8_BLOCK) {
+    rc = kmoe_quant_fp8_group128(a->x, H, M, H, static_cast<uint8_t*>(at(L.xq)), H, static_cast<float*>(at(L.xmax)),
+                                 stream);
+    x_rows = at(L.xq);
+  }
   if (rc) return rc;
   mark(KMOE_STAGE_QUANT1, 1);
-  mark(KMOE_STAGE_GEMM1, 0);
-  // 4. gate_up GEMM with dequant + SiLU-mul epilogue; rows gathered through the sort
-  kmoe_gemm_i8_args g1 = {};
-  g1.a = xq;
-  g1.lda = H;
-  g1.a_max = xmax;
-  g1.row_src = sorted_src;
-  g1.src_div = K;
-  g1.w = a->w13;
-  g1.w_max = a->w13_max;
-  g1.lod = lod;
-  g1.E = E;
-  g1.n = 2 * I;
-  g1.k = H;
-  g1.rows = P;
-  g1.y = static_cast<uint16_t*>(at(L.act));
-  g1.ldy = I;
-  g1.act = KMOE_ACT_SWIGLU;
-  rc = kmoe_grouped_gemm_i8(&g1, stream);
-  if (rc) return rc;
-  mark(KMOE_STAGE_GEMM1, 1);
-  mark(KMOE_STAGE_QUANT2, 0);
-  // 5. requantise the activation rows
-  rc = kmoe_quant_i8_rows(static_cast<uint16_t*>(at(L.act)), I, P, I, static_cast<int8_t*>(at(L.actq)), I,
-                          static_cast<float*>(at(L.actmax)), stream);
-  if (rc) return rc;
-  mark(KMOE_STAGE_QUANT2, 1);
-  mark(KMOE_STAGE_GEMM2, 0);
-  // 6. down GEMM
-  kmoe_gemm_i8_args g2 = {};
-  g2.a = static_cast<int8_t*>(at(L.actq));
-  g2.lda = I;
-  g2.a_max = static_cast<float*>(at(L.actmax));
-  g2.w = a->w2;
-  g2.w_max = a->w2_max;
-  g2.lod = lod;
-  g2.E = E;
-  g2.n = H;
-  g2.k = I;
-  g2.rows = P;
-  g2.y = static_cast<uint16_t*>(at(L.down));
-  g2.ldy = H;
-  g2.act = KMOE_ACT_NONE;
-  rc = kmoe_grouped_gemm_i8(&g2, stream);
-  if (rc) return rc;
-  mark(KMOE_STAGE_GEMM2, 1);
 
-  // 7. dense shared expert on all M rows: one "expert" whose lod is [0, M]
+  // 4-6. routed experts: gate_up GEMM (+SiLU-mul, rows gathered through the sort), requantise, down GEMM
+  MlpPass routed = {};
+  routed.format = a->format;
+  routed.x_rows = x_rows;
+  routed.x_aux = quant ? static_cast<const float*>(at(L.xmax)) : nullptr;
+  routed.row_src = sorted_src;
+  routed.src_div = K;
+  routed.w13 = a->w13;
+  routed.w2 = a->w2;
+  routed.w13_aux = a->w13_max;
+  routed.w2_aux = a->w2_max;
+  routed.lod = lod;
+  routed.E = E;
+  routed.H = H;
+  routed.I = I;
+  routed.rows = P;
+  routed.act = static_cast<uint16_t*>(at(L.act));
+  routed.actq = at(L.actq);
+  routed.act_aux = static_cast<float*>(at(L.actmax));
+  routed.out = static_cast<uint16_t*>(at(L.down));
+  rc = run_mlp(routed, stream, mark);
+  if (rc) return rc;
+
+  // 7. dense shared expert on all M rows: the grouped GEMM with a single expert whose lod is {0, M}
   mark(KMOE_STAGE_SHARED, 0);
   const uint16_t* shared_out = nullptr;
   if (a->I_shared > 0) {
-    const int Is = a->I_shared;
-    // the dense call is the grouped GEMM with a single expert whose lod is {0, M}
     int32_t* dense_lod = static_cast<int32_t*>(at(L.sh_lod));
     rc = fill_dense_lod(dense_lod, M, as_stream(stream));
     if (rc) return rc;
-    kmoe_gemm_i8_args s1 = {};
-    s1.a = xq;
-    s1.lda = H;
-    s1.a_max = xmax;
-    s1.w = a->ws13;
-    s1.w_max = a->ws13_max;
-    s1.lod = dense_lod;
-    s1.E = 1;
-    s1.n = 2 * Is;
-    s1.k = H;
-    s1.rows = M;
-    s1.y = static_cast<uint16_t*>(at(L.sh_act));
-    s1.ldy = Is;
-    s1.act = KMOE_ACT_SWIGLU;
-    rc = kmoe_grouped_gemm_i8(&s1, stream);
+    MlpPass sh = routed;
+    sh.row_src = nullptr;
+    sh.src_div = 1;
+    sh.w13 = a->ws13;
+    sh.w2 = a->ws2;
+    sh.w13_aux = a->ws13_max;
+    sh.w2_aux = a->ws2_max;
+    sh.lod = dense_lod;
+    sh.E = 1;
+    sh.I = a->I_shared;
+    sh.rows = M;
+    sh.act = static_cast<uint16_t*>(at(L.sh_act));
+    sh.actq = at(L.sh_actq);
+    sh.act_aux = static_cast<float*>(at(L.sh_actmax));
+    sh.out = static_cast<uint16_t*>(at(L.sh_out));
+    rc = run_mlp(sh, stream, [](int, int) {});
     if (rc) return rc;
-    rc = kmoe_quant_i8_rows(static_cast<uint16_t*>(at(L.sh_act)), Is, M, Is, static_cast<int8_t*>(at(L.sh_actq)), Is,
-                            static_cast<float*>(at(L.sh_actmax)), stream);
-    if (rc) return rc;
-    kmoe_gemm_i8_args s2 = {};
-    s2.a = static_cast<int8_t*>(at(L.sh_actq));
-    s2.lda = Is;
-    s2.a_max = static_cast<float*>(at(L.sh_actmax));
-    s2.w = a->ws2;
-    s2.w_max = a->ws2_max;
-    s2.lod = dense_lod;
-    s2.E = 1;
-    s2.n = H;
-    s2.k = Is;
-    s2.rows = M;
-    s2.y = static_cast<uint16_t*>(at(L.sh_out));
-    s2.ldy = H;
-    s2.act = KMOE_ACT_NONE;
-    rc = kmoe_grouped_gemm_i8(&s2, stream);
-    if (rc) return rc;
-    shared_out = static_cast<uint16_t*>(at(L.sh_out));
+    shared_out = sh.out;
   }
   mark(KMOE_STAGE_SHARED, 1);
   // 8. weighted combine (+ caller epilogue)
   mark(KMOE_STAGE_COMBINE, 0);
   rc = kmoe_combine(static_cast<uint16_t*>(at(L.down)), H, moe_index, topk_w, nullptr, M, K, H, a->out_scale,
-                      shared_out, H, a->out, H, stream);
+                    shared_out, H, a->out, H, stream);
   mark(KMOE_STAGE_COMBINE, 1);
   return rc;
 }

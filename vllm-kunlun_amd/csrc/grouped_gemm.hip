@@ -1,0 +1,455 @@
+// Grouped GEMM over expert-sorted rows on gfx950 MFMA: int8 (W8A8), bf16
+// (unquantized) and fp8-e4m3 with 128x128 / 1x128 block scales.
+//
+// Roles: the WEIGHT fragment is the first MFMA operand (16 output channels x K
+// bytes), the ACTIVATION fragment the second (K bytes x 16 sorted rows). A lane
+// therefore ends up with 4 consecutive output channels of one row: channel
+// 4*(lane/16)+q, row lane%16 — what the dequant / SiLU-mul epilogue (gate and up
+// fragments of the same channels sit in the same lane) and an 8-byte store want.
+//
+// Data movement per workgroup:
+//   weights     global -> registers, one 256-byte K chunk per channel row
+//               prefetched ahead of the MFMAs that consume it; every wave owns
+//               its own output channels, so weights never pass through LDS;
+//   activations global (gathered through the sort) -> LDS, double-buffered per
+//               K chunk, shared by all waves of the workgroup.
+// K is handled in BYTES: a chunk is 256 bytes of a row; MFMA step j consumes
+// bytes [j*4*LB, (j+1)*4*LB) of the chunk, lane group g = lane/16 holding bytes
+// [g*LB, (g+1)*LB) of the step (LB = 16 for int8/bf16, 32 for fp8).
+#include "kmoe_common.h"
+
+namespace kmoe {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+constexpr int kKC = 256;          // bytes of K per chunk and row
+constexpr int kPitch = kKC + 16;  // LDS row pitch: 16 rows of a b128 read fall in 16 different bank groups
+
+enum class Kind { I8, BF16, FP8 };
+
+template <Kind K> struct Traits;
+template <> struct Traits<Kind::I8> {
+  using acc_t = v4i;
+  static constexpr int LB = 16;   // bytes per lane and MFMA step
+  __device__ static acc_t zero() { return (v4i){0, 0, 0, 0}; }
+};
+template <> struct Traits<Kind::BF16> {
+  using acc_t = v4f;
+  static constexpr int LB = 16;
+  __device__ static acc_t zero() { return (v4f){0.f, 0.f, 0.f, 0.f}; }
+};
+template <> struct Traits<Kind::FP8> {
+  using acc_t = v4f;
+  static constexpr int LB = 32;
+  __device__ static acc_t zero() { return (v4f){0.f, 0.f, 0.f, 0.f}; }
+};
+
+struct GemmParams {
+  const int8_t* a;         // activations, rows of kbytes bytes
+  int64_t lda;             // row stride in BYTES
+  const float* a_max;      // I8: [a_rows] absmax; FP8: [a_rows, k/128] scales; BF16: unused
+  const int32_t* row_src;
+  int32_t src_div;
+  const int8_t* w;         // [E, n, kbytes]
+  const float* w_max;      // I8: [E, n] absmax; FP8: [E, n/128, k/128] scales; BF16: unused
+  const int32_t* lod;
+  int32_t E, n, kbytes;
+  uint16_t* y;
+  int64_t ldy;             // in elements
+  int32_t* acc_out;        // I8 only
+};
+
+__device__ inline int wave_incl_scan(int v) {
+  const int lane = lane_id();
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int o = __shfl_up(v, off, kWave);
+    if (lane >= off) v += o;
+  }
+  return v;
+}
+
+// Finds the expert and first row of m-tile number `t` when every expert's rows
+// are cut into tiles of TM. Returns false when t is past the last tile.
+template <int TM>
+__device__ inline bool locate_tile(const int32_t* __restrict__ lod, int E, int t, int& e_out, int& row0_out) {
+  const int lane = lane_id();
+  const int epl = (E + kWave - 1) / kWave;
+  const int e_begin = lane * epl;
+  int local = 0;
+  for (int i = 0; i < epl; ++i) {
+    const int e = e_begin + i;
+    if (e < E) local += (lod[e + 1] - lod[e] + TM - 1) / TM;
+  }
+  const int incl = wave_incl_scan(local);
+  const int total = __shfl(incl, kWave - 1, kWave);
+  if (t >= total) return false;
+  int excl = incl - local;
+  int found_e = -1, found_row = 0;
+  if (t >= excl && t < incl) {
+    for (int i = 0; i < epl; ++i) {
+      const int e = e_begin + i;
+      if (e >= E) break;
+      const int lo = lod[e];
+      const int tiles = (lod[e + 1] - lo + TM - 1) / TM;
+      if (t < excl + tiles) {
+        found_e = e;
+        found_row = lo + (t - excl) * TM;
+        break;
+      }
+      excl += tiles;
+    }
+  }
+  const uint64_t who = __ballot(found_e >= 0);
+  const int src_lane = __builtin_ctzll(who);
+  e_out = __shfl(found_e, src_lane, kWave);
+  row0_out = __shfl(found_row, src_lane, kWave);
+  return true;
+}
+
+// MF: 16-row fragments per workgroup tile; NF: 16-channel fragments per wave
+// (SWIGLU: NF/2 gate + NF/2 up fragments of the same channels); LOCATE: the
+// m-tile comes from blockIdx.y through locate_tile (balanced over skewed
+// experts) instead of blockIdx.y being the expert.
+template <Kind KIND, int MF, int NF, int WAVES, bool SWIGLU, bool LOCATE>
+__global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmParams p) {
+  using T = Traits<KIND>;
+  using acc_t = typename T::acc_t;
+  constexpr int LB = T::LB;
+  constexpr int kJ = kKC / (4 * LB);  // MFMA steps per chunk
+  constexpr int kV = LB / 16;         // 16-byte vectors per lane and step
+  constexpr int TM = 16 * MF;
+  constexpr int THREADS = WAVES * kWave;
+  constexpr int NFH = SWIGLU ? NF / 2 : NF;
+  constexpr int NA = (TM * (kKC / 16) + THREADS - 1) / THREADS;  // activation vectors per thread per chunk
+  static_assert(!SWIGLU || NF % 2 == 0, "SwiGLU pairs gate and up fragments");
+
+  __shared__ __attribute__((aligned(16))) int8_t lds_a[2][TM * kPitch];
+
+  const int lane = lane_id();
+  const int wave = threadIdx.x >> 6;
+  const int li = lane & 15;
+  const int lg = lane >> 4;
+
+  int e, row_begin, row_end;
+  if (LOCATE) {
+    if (!locate_tile<TM>(p.lod, p.E, blockIdx.y, e, row_begin)) return;
+    row_end = min(p.lod[e + 1], row_begin + TM);
+  } else {
+    e = blockIdx.y;
+    row_begin = p.lod[e];
+    row_end = p.lod[e + 1];
+    if (row_begin >= row_end) return;
+  }
+
+  const int n_half = SWIGLU ? p.n / 2 : p.n;
+  const int col_base = (blockIdx.x * WAVES + wave) * NFH * 16;
+
+  const int8_t* wp[NF];
+  bool wok[NF];
+  int col[NF];
+#pragma unroll
+  for (int f = 0; f < NF; ++f) {
+    const int fh = SWIGLU ? f % NFH : f;
+    const int c = col_base + fh * 16;
+    wok[f] = c < n_half;
+    col[f] = (SWIGLU && f >= NFH) ? n_half + c : c;
+    wp[f] = p.w + (static_cast<size_t>(e) * p.n + (wok[f] ? col[f] + li : 0)) * p.kbytes + lg * LB;
+  }
+  const int nchunks = (p.kbytes + kKC - 1) / kKC;
+  const int kblocks = p.kbytes / 128;  // FP8: scale blocks along K
+
+  for (int row0 = row_begin; row0 < row_end; row0 += TM) {
+    const int8_t* ap[NA];
+    int a_lds[NA];
+    int a_kv[NA];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      const int v = threadIdx.x + i * THREADS;
+      const int r = v >> 4;
+      const int kv = v & 15;
+      a_kv[i] = kv * 16;
+      a_lds[i] = (v < TM * 16) ? r * kPitch + kv * 16 : -1;
+      ap[i] = nullptr;
+      if (v < TM * 16 && row0 + r < row_end) {
+        const int sr = p.row_src ? p.row_src[row0 + r] / p.src_div : row0 + r;
+        ap[i] = p.a + static_cast<size_t>(sr) * p.lda + kv * 16;
+      }
+    }
+    // source row of this lane's output rows (for scales / maxes)
+    int srow[MF];
+#pragma unroll
+    for (int mf = 0; mf < MF; ++mf) {
+      const int r = row0 + mf * 16 + li;
+      srow[mf] = r < row_end ? (p.row_src ? p.row_src[r] / p.src_div : r) : -1;
+    }
+
+    acc_t acc[MF][NF];
+#pragma unroll
+    for (int mf = 0; mf < MF; ++mf)
+#pragma unroll
+      for (int f = 0; f < NF; ++f) acc[mf][f] = T::zero();
+
+    v4i wbuf[2][NF][kJ][kV];
+    v4i areg[NA];
+
+    auto load_w = [&](v4i(&dst)[NF][kJ][kV], int chunk) {
+      const int kc = chunk * kKC;
+#pragma unroll
+      for (int f = 0; f < NF; ++f)
+#pragma unroll
+        for (int j = 0; j < kJ; ++j)
+#pragma unroll
+          for (int v = 0; v < kV; ++v) {
+            const int off = kc + j * 4 * LB + v * 16;  // + lg*LB is folded into wp
+            dst[f][j][v] = (wok[f] && off + lg * LB < p.kbytes) ? *reinterpret_cast<const v4i*>(wp[f] + off)
+                                                                 : (v4i){0, 0, 0, 0};
+          }
+    };
+    auto load_a = [&](int chunk) {
+      const int kc = chunk * kKC;
+#pragma unroll
+      for (int i = 0; i < NA; ++i)
+        areg[i] = (ap[i] && kc + a_kv[i] < p.kbytes) ? *reinterpret_cast<const v4i*>(ap[i] + kc) : (v4i){0, 0, 0, 0};
+    };
+    auto store_a = [&](int buf) {
+#pragma unroll
+      for (int i = 0; i < NA; ++i)
+        if (a_lds[i] >= 0) *reinterpret_cast<v4i*>(&lds_a[buf][a_lds[i]]) = areg[i];
+    };
+    auto compute = [&](const v4i(&wcur)[NF][kJ][kV], int buf, int chunk) {
+#pragma unroll
+      for (int j = 0; j < kJ; ++j) {
+        v4i af[MF][kV];
+#pragma unroll
+        for (int mf = 0; mf < MF; ++mf)
+#pragma unroll
+          for (int v = 0; v < kV; ++v)
+            af[mf][v] = *reinterpret_cast<const v4i*>(
+                &lds_a[buf][(mf * 16 + li) * kPitch + j * 4 * LB + lg * LB + v * 16]);
+        if constexpr (KIND == Kind::I8) {
+#pragma unroll
+          for (int mf = 0; mf < MF; ++mf)
+#pragma unroll
+            for (int f = 0; f < NF; ++f)
+              acc[mf][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wcur[f][j][0], af[mf][0], acc[mf][f], 0, 0, 0);
+        } else if constexpr (KIND == Kind::BF16) {
+#pragma unroll
+          for (int mf = 0; mf < MF; ++mf)
+#pragma unroll
+            for (int f = 0; f < NF; ++f)
+              acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wcur[f][j][0]),
+                                                                   __builtin_bit_cast(v8bf, af[mf][0]), acc[mf][f], 0,
+                                                                   0, 0);
+        } else {
+          // one MFMA = one 128-wide scale block: scale the block's partial sum, then add
+          const int kb = chunk * kJ + j;
+          if (kb < kblocks) {
+            float sa[MF];
+#pragma unroll
+            for (int mf = 0; mf < MF; ++mf)
+              sa[mf] = srow[mf] >= 0 ? p.a_max[static_cast<size_t>(srow[mf]) * kblocks + kb] : 0.0f;
+#pragma unroll
+            for (int f = 0; f < NF; ++f) {
+              const float sw =
+                  wok[f] ? p.w_max[(static_cast<size_t>(e) * (p.n / 128) + col[f] / 128) * kblocks + kb] : 0.0f;
+              v8i wv;
+              wv.lo = wcur[f][j][0];
+              wv.hi = wcur[f][j][1];
+#pragma unroll
+              for (int mf = 0; mf < MF; ++mf) {
+                v8i av;
+                av.lo = af[mf][0];
+                av.hi = af[mf][1];
+                const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    wv, av, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+                const float s = sa[mf] * sw;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) acc[mf][f][q] = __builtin_fmaf(blk[q], s, acc[mf][f][q]);
+              }
+            }
+          }
+        }
+      }
+    };
+    auto stage = [&](int chunk, const v4i(&wcur)[NF][kJ][kV], v4i(&wnext)[NF][kJ][kV], int buf) {
+      const bool more = chunk + 1 < nchunks;
+      if (more) {
+        load_w(wnext, chunk + 1);
+        load_a(chunk + 1);
+      }
+      compute(wcur, buf, chunk);
+      if (more) store_a(buf ^ 1);
+      __syncthreads();
+    };
+
+    load_w(wbuf[0], 0);
+    load_a(0);
+    store_a(0);
+    __syncthreads();
+    for (int c = 0; c < nchunks; c += 2) {
+      stage(c, wbuf[0], wbuf[1], 0);
+      if (c + 1 < nchunks) stage(c + 1, wbuf[1], wbuf[0], 1);
+    }
+
+    // ---- epilogue: dequantise, optional SiLU-mul, store ----
+#pragma unroll
+    for (int mf = 0; mf < MF; ++mf) {
+      const int r = row0 + mf * 16 + li;
+      if (r >= row_end) continue;
+      float sa = 1.0f;
+      if constexpr (KIND == Kind::I8) sa = p.a_max[srow[mf]] / 127.0f;
+#pragma unroll
+      for (int f = 0; f < NFH; ++f) {
+        if (!wok[f]) continue;
+        const int c0 = col[f] + lg * 4;
+        uint16_t yv[4];
+        auto finish = [&](const acc_t& a, int cc, uint16_t(&out)[4]) {
+          if constexpr (KIND == Kind::I8) {
+            const float4 wm = *reinterpret_cast<const float4*>(p.w_max + static_cast<size_t>(e) * p.n + cc);
+            const float sw[4] = {wm.x / 127.0f, wm.y / 127.0f, wm.z / 127.0f, wm.w / 127.0f};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) out[q] = f32_to_bf16((static_cast<float>(a[q]) * sa) * sw[q]);
+            if (p.acc_out) *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + cc) = a;
+          } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) out[q] = f32_to_bf16(a[q]);
+          }
+        };
+        finish(acc[mf][f], c0, yv);
+        if (SWIGLU) {
+          uint16_t uv[4];
+          finish(acc[mf][f + NFH], col[f + NFH] + lg * 4, uv);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) yv[q] = f32_to_bf16(silu_fixed(bf16_to_f32(yv[q])) * bf16_to_f32(uv[q]));
+        }
+        const uint2 packed = make_uint2(yv[0] | (static_cast<uint32_t>(yv[1]) << 16),
+                                        yv[2] | (static_cast<uint32_t>(yv[3]) << 16));
+        *reinterpret_cast<uint2*>(p.y + static_cast<size_t>(r) * p.ldy + c0) = packed;
+      }
+    }
+  }
+}
+
+template <Kind KIND, int MF, int NF, int WAVES, bool SWIGLU, bool LOCATE>
+int launch(const GemmParams& p, int rows, hipStream_t s, const char* what) {
+  constexpr int TM = 16 * MF;
+  constexpr int NFH = SWIGLU ? NF / 2 : NF;
+  const int n_half = SWIGLU ? p.n / 2 : p.n;
+  const int grid_x = ceil_div(n_half, WAVES * NFH * 16);
+  const int grid_y = LOCATE ? rows / TM + min(p.E, rows) : p.E;
+  if (grid_y == 0) return KMOE_OK;
+  hipLaunchKernelGGL((grouped_gemm_kernel<KIND, MF, NF, WAVES, SWIGLU, LOCATE>), dim3(grid_x, grid_y),
+                     dim3(WAVES * kWave), 0, s, p);
+  return check_launch(what);
+}
+
+template <Kind KIND>
+int dispatch(const GemmParams& p, int rows, bool swiglu, int variant, hipStream_t s, const char* what) {
+  if (variant == 0) {
+    // rows per expert if the routing were uniform; decides streaming vs tiled
+    const int avg = ceil_div(rows, p.E);
+    variant = avg <= 16 ? 1 : (avg <= 48 ? 2 : 3);
+  }
+  switch (variant) {
+    case 1:  // weight streaming: 16-row tiles, one expert per workgroup row
+      return swiglu ? launch<KIND, 1, 2, 4, true, false>(p, rows, s, what)
+                    : launch<KIND, 1, 1, 4, false, false>(p, rows, s, what);
+    case 2:  // 32-row tiles
+      return swiglu ? launch<KIND, 2, 2, 4, true, false>(p, rows, s, what)
+                    : launch<KIND, 2, 2, 4, false, false>(p, rows, s, what);
+    case 3:  // 128-row tiles, work list balanced over experts
+      return swiglu ? launch<KIND, 8, 4, 4, true, true>(p, rows, s, what)
+                    : launch<KIND, 8, 4, 4, false, true>(p, rows, s, what);
+    default:
+      return fail(KMOE_ERR_UNSUPPORTED, "%s: variant=%d unknown", what, variant);
+  }
+}
+
+bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+}  // namespace
+}  // namespace kmoe
+
+using namespace kmoe;
+
+extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t stream) {
+  KMOE_REQUIRE(a, KMOE_ERR_NULL, "grouped_gemm_i8: args is NULL");
+  KMOE_REQUIRE(a->a && a->a_max && a->w && a->w_max && a->lod && a->y, KMOE_ERR_NULL,
+               "grouped_gemm_i8: NULL tensor pointer");
+  KMOE_REQUIRE(a->E >= 1 && a->n >= 16 && a->k >= 16 && a->rows >= 0, KMOE_ERR_SHAPE,
+               "grouped_gemm_i8: E=%d n=%d k=%d rows=%d", a->E, a->n, a->k, a->rows);
+  KMOE_REQUIRE(a->k % 16 == 0, KMOE_ERR_SHAPE, "grouped_gemm_i8: k=%d must be a multiple of 16", a->k);
+  const bool swiglu = a->act == KMOE_ACT_SWIGLU;
+  KMOE_REQUIRE(a->act == KMOE_ACT_NONE || swiglu, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: act=%d unknown", a->act);
+  KMOE_REQUIRE(a->n % (swiglu ? 32 : 16) == 0, KMOE_ERR_SHAPE, "grouped_gemm_i8: n=%d must be a multiple of %d",
+               a->n, swiglu ? 32 : 16);
+  KMOE_REQUIRE(a->lda % 16 == 0 && a->lda >= a->k, KMOE_ERR_SHAPE,
+               "grouped_gemm_i8: lda=%lld must be a multiple of 16 and >= k", (long long)a->lda);
+  const int n_out = swiglu ? a->n / 2 : a->n;
+  KMOE_REQUIRE(a->ldy % 4 == 0 && a->ldy >= n_out, KMOE_ERR_SHAPE,
+               "grouped_gemm_i8: ldy=%lld must be a multiple of 4 and >= %d", (long long)a->ldy, n_out);
+  KMOE_REQUIRE(aligned(a->a, 16) && aligned(a->w, 16) && aligned(a->y, 8) && aligned(a->w_max, 16) &&
+                   aligned(a->acc_out, 16),
+               KMOE_ERR_SHAPE, "grouped_gemm_i8: misaligned tensor pointer");
+  KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_i8: src_div=%d < 1", a->src_div);
+  if (a->rows == 0) return KMOE_OK;
+  GemmParams p{a->a, a->lda, a->a_max, a->row_src, a->src_div, a->w,  a->w_max,
+               a->lod, a->E,  a->n,     a->k,       a->y,       a->ldy, a->acc_out};
+  return dispatch<Kind::I8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_i8");
+}
+
+extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_t stream) {
+  KMOE_REQUIRE(a, KMOE_ERR_NULL, "grouped_gemm_bf16: args is NULL");
+  KMOE_REQUIRE(a->a && a->w && a->lod && a->y, KMOE_ERR_NULL, "grouped_gemm_bf16: NULL tensor pointer");
+  KMOE_REQUIRE(a->E >= 1 && a->n >= 16 && a->k >= 8 && a->rows >= 0, KMOE_ERR_SHAPE,
+               "grouped_gemm_bf16: E=%d n=%d k=%d rows=%d", a->E, a->n, a->k, a->rows);
+  KMOE_REQUIRE(a->k % 8 == 0, KMOE_ERR_SHAPE, "grouped_gemm_bf16: k=%d must be a multiple of 8", a->k);
+  const bool swiglu = a->act == KMOE_ACT_SWIGLU;
+  KMOE_REQUIRE(a->act == KMOE_ACT_NONE || swiglu, KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: act=%d unknown", a->act);
+  KMOE_REQUIRE(a->n % (swiglu ? 32 : 16) == 0, KMOE_ERR_SHAPE, "grouped_gemm_bf16: n=%d must be a multiple of %d",
+               a->n, swiglu ? 32 : 16);
+  KMOE_REQUIRE(a->lda % 8 == 0 && a->lda >= a->k, KMOE_ERR_SHAPE,
+               "grouped_gemm_bf16: lda=%lld must be a multiple of 8 and >= k", (long long)a->lda);
+  const int n_out = swiglu ? a->n / 2 : a->n;
+  KMOE_REQUIRE(a->ldy % 4 == 0 && a->ldy >= n_out, KMOE_ERR_SHAPE,
+               "grouped_gemm_bf16: ldy=%lld must be a multiple of 4 and >= %d", (long long)a->ldy, n_out);
+  KMOE_REQUIRE(aligned(a->a, 16) && aligned(a->w, 16) && aligned(a->y, 8), KMOE_ERR_SHAPE,
+               "grouped_gemm_bf16: misaligned tensor pointer");
+  KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_bf16: src_div=%d < 1", a->src_div);
+  if (a->rows == 0) return KMOE_OK;
+  GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
+               reinterpret_cast<const int8_t*>(a->w), nullptr,    a->lod,  a->E,       a->n,
+               a->k * 2,                              a->y,       a->ldy,  nullptr};
+  return dispatch<Kind::BF16>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_bf16");
+}
+
+extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_stream_t stream) {
+  KMOE_REQUIRE(a, KMOE_ERR_NULL, "grouped_gemm_fp8_block: args is NULL");
+  KMOE_REQUIRE(a->a && a->a_scale && a->w && a->w_scale && a->lod && a->y, KMOE_ERR_NULL,
+               "grouped_gemm_fp8_block: NULL tensor pointer");
+  KMOE_REQUIRE(a->E >= 1 && a->n >= 128 && a->k >= 128 && a->rows >= 0, KMOE_ERR_SHAPE,
+               "grouped_gemm_fp8_block: E=%d n=%d k=%d rows=%d", a->E, a->n, a->k, a->rows);
+  const bool swiglu = a->act == KMOE_ACT_SWIGLU;
+  KMOE_REQUIRE(a->act == KMOE_ACT_NONE || swiglu, KMOE_ERR_UNSUPPORTED, "grouped_gemm_fp8_block: act=%d unknown",
+               a->act);
+  KMOE_REQUIRE(a->k % 128 == 0 && a->n % (swiglu ? 256 : 128) == 0, KMOE_ERR_SHAPE,
+               "grouped_gemm_fp8_block: k=%d and n=%d must be multiples of 128 (n of 256 with SwiGLU)", a->k, a->n);
+  KMOE_REQUIRE(a->lda % 16 == 0 && a->lda >= a->k, KMOE_ERR_SHAPE,
+               "grouped_gemm_fp8_block: lda=%lld must be a multiple of 16 and >= k", (long long)a->lda);
+  const int n_out = swiglu ? a->n / 2 : a->n;
+  KMOE_REQUIRE(a->ldy % 4 == 0 && a->ldy >= n_out, KMOE_ERR_SHAPE,
+               "grouped_gemm_fp8_block: ldy=%lld must be a multiple of 4 and >= %d", (long long)a->ldy, n_out);
+  KMOE_REQUIRE(aligned(a->a, 16) && aligned(a->w, 16) && aligned(a->y, 8), KMOE_ERR_SHAPE,
+               "grouped_gemm_fp8_block: misaligned tensor pointer");
+  KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_fp8_block: src_div=%d < 1", a->src_div);
+  if (a->rows == 0) return KMOE_OK;
+  GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,
+               reinterpret_cast<const int8_t*>(a->w), a->w_scale, a->lod,  a->E,       a->n,
+               a->k,                                  a->y,       a->ldy,  nullptr};
+  return dispatch<Kind::FP8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_fp8_block");
+}

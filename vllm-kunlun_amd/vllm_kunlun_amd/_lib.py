@@ -18,6 +18,9 @@ KMOE_ACT_NONE = 0
 KMOE_ACT_SWIGLU = 1
 KMOE_SCORE_SOFTMAX = 0
 KMOE_SCORE_SIGMOID = 1
+KMOE_FMT_INT8 = 0
+KMOE_FMT_FP8_BLOCK = 1
+KMOE_FMT_BF16 = 2
 STAGES = ("routing", "align", "quant1", "gemm1", "quant2", "gemm2", "shared", "combine")
 
 _ERR_KIND = {-1: ValueError, -2: ValueError, -3: NotImplementedError, -4: RuntimeError, -5: RuntimeError}
@@ -33,10 +36,28 @@ class GemmI8Args(C.Structure):
     ]
 
 
-class W8A8Args(C.Structure):
+class GemmBf16Args(C.Structure):
+    _fields_ = [
+        ("a", C.c_void_p), ("lda", C.c_int64), ("row_src", C.c_void_p), ("src_div", C.c_int32),
+        ("w", C.c_void_p), ("lod", C.c_void_p),
+        ("E", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("rows", C.c_int32),
+        ("y", C.c_void_p), ("ldy", C.c_int64), ("act", C.c_int32), ("variant", C.c_int32),
+    ]
+
+
+class GemmFp8Args(C.Structure):
+    _fields_ = [
+        ("a", C.c_void_p), ("lda", C.c_int64), ("a_scale", C.c_void_p), ("row_src", C.c_void_p),
+        ("src_div", C.c_int32), ("w", C.c_void_p), ("w_scale", C.c_void_p), ("lod", C.c_void_p),
+        ("E", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("rows", C.c_int32),
+        ("y", C.c_void_p), ("ldy", C.c_int64), ("act", C.c_int32), ("variant", C.c_int32),
+    ]
+
+
+class MoEArgs(C.Structure):
     _fields_ = [
         ("M", C.c_int32), ("H", C.c_int32), ("E", C.c_int32), ("K", C.c_int32), ("I", C.c_int32),
-        ("scoring", C.c_int32), ("renormalize", C.c_int32), ("n_group", C.c_int32), ("topk_group", C.c_int32),
+        ("format", C.c_int32), ("scoring", C.c_int32), ("renormalize", C.c_int32), ("n_group", C.c_int32), ("topk_group", C.c_int32),
         ("routed_scale", C.c_float), ("logits", C.c_void_p), ("bias", C.c_void_p),
         ("x", C.c_void_p), ("w13", C.c_void_p), ("w13_max", C.c_void_p), ("w2", C.c_void_p), ("w2_max", C.c_void_p),
         ("I_shared", C.c_int32), ("ws13", C.c_void_p), ("ws13_max", C.c_void_p), ("ws2", C.c_void_p),
@@ -45,7 +66,7 @@ class W8A8Args(C.Structure):
     ]
 
 
-class W8A8Layout(C.Structure):
+class MoELayout(C.Structure):
     _fields_ = [(n, C.c_size_t) for n in (
         "total_bytes", "topk_w", "topk_ids", "moe_index", "sorted_src", "expert_m", "lod", "align_ws",
         "xq", "xmax", "act", "actq", "actmax", "down", "sh_lod", "sh_act", "sh_actq", "sh_actmax", "sh_out")]
@@ -72,8 +93,10 @@ def _load() -> C.CDLL:
         "kmoe_grouped_gemm_i8": (i32, [C.POINTER(GemmI8Args), vp]),
         "kmoe_silu_and_mul": (i32, [vp, i64, i32, i32, vp, i64, vp]),
         "kmoe_combine": (i32, [vp, i64, vp, vp, vp, i32, i32, i32, f32, vp, i64, vp, i64, vp]),
-        "kmoe_w8a8_workspace_layout": (i32, [C.POINTER(W8A8Args), C.POINTER(W8A8Layout)]),
-        "kmoe_forward_w8a8": (i32, [C.POINTER(W8A8Args), vp, sz, vp]),
+        "kmoe_grouped_gemm_bf16": (i32, [C.POINTER(GemmBf16Args), vp]),
+        "kmoe_grouped_gemm_fp8_block": (i32, [C.POINTER(GemmFp8Args), vp]),
+        "kmoe_moe_workspace_layout": (i32, [C.POINTER(MoEArgs), C.POINTER(MoELayout)]),
+        "kmoe_moe_forward": (i32, [C.POINTER(MoEArgs), vp, sz, vp]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)
@@ -86,7 +109,8 @@ lib = _load()
 EXPORTS = (
     "kmoe_last_error", "kmoe_version", "kmoe_softmax_topk", "kmoe_sigmoid_group_topk_norm", "kmoe_block_statistic",
     "kmoe_align_workspace_bytes", "kmoe_align", "kmoe_gather_rows", "kmoe_quant_i8_rows", "kmoe_quant_fp8_group128",
-    "kmoe_grouped_gemm_i8", "kmoe_silu_and_mul", "kmoe_combine", "kmoe_w8a8_workspace_layout", "kmoe_forward_w8a8",
+    "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
+    "kmoe_moe_workspace_layout", "kmoe_moe_forward",
 )
 
 

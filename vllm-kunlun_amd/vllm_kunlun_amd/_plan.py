@@ -1,0 +1,109 @@
+"""Argument blocks for kmoe_moe_forward: one filled `kmoe_moe_args` + its workspace.
+
+A plan binds fixed device buffers (x, logits, out, weights); calling it enqueues
+the whole layer on the current HIP stream without allocating or synchronising,
+so a serving loop — or a HIP-graph capture — can replay it.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib as L
+
+
+class _Workspace:
+    """Per-device scratch buffer that only grows (plays the role of vLLM's
+    current_workspace_manager(), reference: vllm_kunlun/ops/_kunlun_ops.py:528-531)."""
+
+    def __init__(self):
+        self._buf = {}
+
+    def get(self, nbytes: int, device: torch.device) -> torch.Tensor:
+        key = (device.type, device.index)
+        buf = self._buf.get(key)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            self._buf[key] = buf
+        return buf
+
+
+WORKSPACE = _Workspace()
+
+
+class MoEPlan:
+    def __init__(self, args, layout, workspace, keepalive):
+        self.args, self.layout, self.workspace, self._keep = args, layout, workspace, keepalive
+
+    def __call__(self) -> None:
+        L.check(L.lib.kmoe_moe_forward(self.args, L.ptr(self.workspace), self.workspace.numel(), L.stream()))
+
+    def view(self, name: str, count: int, dtype: torch.dtype) -> torch.Tensor:
+        """An intermediate of the last call, e.g. view("topk_ids", M*K, torch.int32)."""
+        off = getattr(self.layout, name)
+        nbytes = count * torch.empty(0, dtype=dtype).element_size()
+        return self.workspace[off: off + nbytes].view(dtype)
+
+
+_WEIGHT_DTYPE = {L.KMOE_FMT_INT8: (torch.int8,), L.KMOE_FMT_FP8_BLOCK: (torch.float8_e4m3fn, torch.uint8),
+                 L.KMOE_FMT_BF16: (torch.bfloat16,)}
+
+
+def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Tensor, top_k: int,
+                  w13: torch.Tensor, w2: torch.Tensor, w13_aux: Optional[torch.Tensor], w2_aux: Optional[torch.Tensor],
+                  scoring_func: str = "softmax", renormalize: bool = True, num_expert_group: Optional[int] = None,
+                  topk_group: Optional[int] = None, routed_scaling_factor: float = 1.0,
+                  e_score_correction_bias: Optional[torch.Tensor] = None, shared_expert=None, out_scale: float = 1.0,
+                  stage_events=None) -> MoEPlan:
+    """x bf16 [M,H], logits f32 [M,E], out bf16 [M,H]; w13 [E,2I,H], w2 [E,H,I] in the
+    format's dtype; w13_aux/w2_aux: per-channel maxes (int8) or block scales (fp8), None for bf16.
+    shared_expert: (ws13 [2Is,H], ws13_aux, ws2 [H,Is], ws2_aux) in the same format."""
+    if scoring_func not in ("softmax", "sigmoid"):
+        raise ValueError(f"Unsupported scoring_func: {scoring_func}")
+    tensors = [x, logits, out, w13, w2, w13_aux, w2_aux, e_score_correction_bias]
+    L.require_device(*tensors)
+    L.require_contig(*tensors)
+    if x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or logits.dtype != torch.float32:
+        raise ValueError("moe plan: x/out must be bfloat16 and logits float32")
+    if w13.dtype not in _WEIGHT_DTYPE[fmt] or w2.dtype != w13.dtype:
+        raise ValueError(f"moe plan: weight dtype {w13.dtype} does not fit the layer format")
+    E, two_i, H = w13.shape
+    M = x.shape[0]
+    if tuple(x.shape) != (M, H) or tuple(out.shape) != (M, H) or tuple(logits.shape) != (M, E):
+        raise ValueError("moe plan: x/out must be [M,H] and logits [M,E]")
+    if tuple(w2.shape) != (E, H, two_i // 2):
+        raise ValueError("moe plan: w2 must be [E,H,I] for w13 [E,2I,H]")
+    a = L.MoEArgs()
+    a.M, a.H, a.E, a.K, a.I = M, H, E, int(top_k), two_i // 2
+    a.format = fmt
+    a.scoring = L.KMOE_SCORE_SOFTMAX if scoring_func == "softmax" else L.KMOE_SCORE_SIGMOID
+    a.renormalize = int(bool(renormalize))
+    a.n_group = int(num_expert_group or 1)
+    a.topk_group = int(topk_group or 1)
+    a.routed_scale = float(routed_scaling_factor)
+    a.logits = logits.data_ptr()
+    a.bias = 0 if e_score_correction_bias is None else e_score_correction_bias.data_ptr()
+    a.x = x.data_ptr()
+    a.w13, a.w2 = w13.data_ptr(), w2.data_ptr()
+    a.w13_max = 0 if w13_aux is None else w13_aux.data_ptr()
+    a.w2_max = 0 if w2_aux is None else w2_aux.data_ptr()
+    keep = list(tensors)
+    if shared_expert is not None:
+        ws13, ws13_aux, ws2, ws2_aux = shared_expert
+        L.require_device(ws13, ws13_aux, ws2, ws2_aux)
+        L.require_contig(ws13, ws13_aux, ws2, ws2_aux)
+        a.I_shared = ws13.shape[0] // 2
+        a.ws13, a.ws2 = ws13.data_ptr(), ws2.data_ptr()
+        a.ws13_max = 0 if ws13_aux is None else ws13_aux.data_ptr()
+        a.ws2_max = 0 if ws2_aux is None else ws2_aux.data_ptr()
+        keep.append(shared_expert)
+    a.out_scale = float(out_scale)
+    a.out = out.data_ptr()
+    if stage_events is not None:
+        a.stage_events = stage_events
+        keep.append(stage_events)
+    lay = L.MoELayout()
+    L.check(L.lib.kmoe_moe_workspace_layout(a, lay))
+    ws = WORKSPACE.get(lay.total_bytes, x.device)
+    return MoEPlan(a, lay, ws, keep)

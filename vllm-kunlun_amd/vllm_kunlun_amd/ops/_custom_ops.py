@@ -251,8 +251,17 @@ def moe_fc(x: torch.Tensor, weight: torch.Tensor, sorted_tokens_num_lod: torch.T
               "moe_fc: per-channel max shapes must be [P,1] and [E,n,1]")
         _gemm_i8(x.view(rows, k), x_perchannel_max, weight, w_perchannel_max, sorted_tokens_num_lod,
                  y, n, L.KMOE_ACT_SWIGLU if act else L.KMOE_ACT_NONE, rows)
+    elif x.dtype == _BF16:
+        _need(weight.dtype == _BF16, "moe_fc: bf16 x needs a bf16 weight")
+        g = L.GemmBf16Args()
+        g.a, g.lda, g.src_div = x.data_ptr(), k, 1
+        g.w, g.lod = weight.data_ptr(), sorted_tokens_num_lod.data_ptr()
+        g.E, g.n, g.k, g.rows = E, n, k, rows
+        g.y, g.ldy = y.data_ptr(), n
+        g.act = L.KMOE_ACT_SWIGLU if act else L.KMOE_ACT_NONE
+        L.check(L.lib.kmoe_grouped_gemm_bf16(g, L.stream()))
     else:
-        raise NotImplementedError(f"moe_fc: x dtype {x.dtype} is not implemented yet")
+        raise NotImplementedError(f"moe_fc: x dtype {x.dtype} is outside this build's path (int8 or bfloat16)")
 
 
 @custom_op("_C::matmul", mutates_args=())

@@ -1,0 +1,83 @@
+"""`KunlunOps`: the static façade the reference's MoE methods call, MoE part only.
+
+Mirrors `KunlunOps.fused_moe` and `KunlunOps.fused_moe_ep` of
+vllm_kunlun/ops/_kunlun_ops.py (:377-637 and :639-696): same argument lists, same
+return value ([M,H] in the activation dtype). Both run the unquantized (bf16)
+layer as one call into libkmoe (kmoe_moe_forward, KMOE_FMT_BF16); the reference's
+device pipeline and its torch expert loop compute the same function.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import _lib as L
+from .._plan import make_moe_plan
+
+
+class KunlunOps:
+    @staticmethod
+    def fused_moe(
+        hidden_states: torch.Tensor,
+        w1: torch.Tensor,
+        w2: torch.Tensor,
+        router_logits: torch.Tensor,
+        ep_rank: int,
+        moe_top_k: int,
+        renormalize: bool,
+        inplace: bool = False,
+        use_grouped_topk: bool = False,
+        num_expert_group: Optional[int] = None,
+        topk_group: Optional[int] = None,
+        w1_bias: Optional[torch.Tensor] = None,
+        w2_bias: Optional[torch.Tensor] = None,
+        scoring_func: str = "softmax",
+        e_score_correction_bias: Optional[torch.Tensor] = None,
+    ) -> torch.Tensor:
+        """bf16 fused MoE (reference: ops/_kunlun_ops.py:377-637). As there, routing is
+        chosen by `scoring_func` alone and always normalises (`renormalize`,
+        `use_grouped_topk` and `inplace` are accepted and ignored, :385-389 vs :413-431);
+        the sigmoid path uses scale 1.0 (:428)."""
+        if w1_bias is not None or w2_bias is not None:
+            raise NotImplementedError("fused_moe: the expert-bias (gpt-oss) branch is outside this build's path")
+        if hidden_states.dtype != torch.bfloat16:
+            raise NotImplementedError(f"fused_moe: activations must be bfloat16, got {hidden_states.dtype}")
+        x = hidden_states.contiguous()
+        logits = router_logits.to(torch.float).contiguous()
+        out = torch.empty_like(x)
+        plan = make_moe_plan(L.KMOE_FMT_BF16, x, logits, out, moe_top_k, w1, w2, None, None, scoring_func, True,
+                             num_expert_group, topk_group, 1.0, e_score_correction_bias)
+        plan()
+        return out
+
+    @staticmethod
+    def fused_moe_ep(
+        hidden_states: torch.Tensor,
+        w13_weight: torch.Tensor,
+        w2_weight: torch.Tensor,
+        router_logits: torch.Tensor,
+        ep_rank: int,
+        top_k: int,
+        renormalize: bool,
+        inplace: bool = False,
+        use_grouped_topk: bool = False,
+        num_expert_group: Optional[int] = None,
+        topk_group: Optional[int] = None,
+        w1_bias: Optional[torch.Tensor] = None,
+        w2_bias: Optional[torch.Tensor] = None,
+    ) -> torch.Tensor:
+        """The expert-parallel entry (reference: ops/_kunlun_ops.py:639-696): softmax
+        routing, `renormalize` honoured (:670-671). One GPU holds every expert here, so
+        ep_rank must be 0 and the local experts are the global ones."""
+        if ep_rank != 0:
+            raise NotImplementedError("fused_moe_ep: this build runs all experts on one GPU (ep_rank must be 0)")
+        if hidden_states.dtype != torch.bfloat16:
+            raise NotImplementedError(f"fused_moe_ep: activations must be bfloat16, got {hidden_states.dtype}")
+        x = hidden_states.contiguous()
+        logits = router_logits.to(torch.float).contiguous()
+        out = torch.empty_like(x)
+        plan = make_moe_plan(L.KMOE_FMT_BF16, x, logits, out, top_k, w13_weight, w2_weight, None, None, "softmax",
+                             bool(renormalize))
+        plan()
+        return out

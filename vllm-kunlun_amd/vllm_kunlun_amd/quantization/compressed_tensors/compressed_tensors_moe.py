@@ -1,4 +1,4 @@
-"""W8A8-int8 fused-MoE method: the plugin-level entry of the path.
+"""Quantized fused-MoE methods: the plugin-level entry of the path.
 
 Mirrors the interface of the reference's
 vllm_kunlun/quantization/compressed_tensors/compressed_tensors_moe.py
@@ -8,7 +8,7 @@ KunlunCompressedTensorsW8A8Int8MoEMethod :111-291): `is_monolithic`,
 `apply_monolithic(layer, x, router_logits, ...)`, same argument meaning, same
 exceptions. Where the reference launches nine closed kernels and allocates every
 intermediate per call, `apply_monolithic` here makes ONE call into libkmoe
-(kmoe_forward_w8a8) on a cached workspace.
+(kmoe_moe_forward) on a cached workspace.
 """
 from __future__ import annotations
 
@@ -17,28 +17,19 @@ from typing import Optional, Union
 import torch
 
 from ... import _lib as L
+from ..._plan import MoEPlan, make_moe_plan
 from ...ops import _custom_ops  # noqa: F401  (torch.ops._C.* used by the staged path)
 
 WNA16_SUPPORTED_BITS = (4, 8)
+W8A8Plan = MoEPlan  # the plan type returned by make_plan
 
 
-class _Workspace:
-    """Per-device scratch buffer that only grows (plays the role of vLLM's
-    current_workspace_manager(), reference: ops/_kunlun_ops.py:528-531)."""
-
-    def __init__(self):
-        self._buf = {}
-
-    def get(self, nbytes: int, device: torch.device) -> torch.Tensor:
-        key = (device.type, device.index)
-        buf = self._buf.get(key)
-        if buf is None or buf.numel() < nbytes:
-            buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
-            self._buf[key] = buf
-        return buf
+def _get(o, k, d=None):
+    return o.get(k, d) if isinstance(o, dict) else getattr(o, k, d)
 
 
-_WORKSPACE = _Workspace()
+def _strategy(o) -> str:
+    return str(_get(o, "strategy")).split(".")[-1].lower()
 
 
 def _scheme_is_dynamic_token_w8a8(weight_quant, input_quant) -> bool:
@@ -46,36 +37,28 @@ def _scheme_is_dynamic_token_w8a8(weight_quant, input_quant) -> bool:
     weights, 8-bit symmetric dynamic per-token activations."""
     if weight_quant is None or input_quant is None:
         return False
-    g = lambda o, k, d=None: o.get(k, d) if isinstance(o, dict) else getattr(o, k, d)  # noqa: E731
-    return (g(weight_quant, "num_bits") == 8 and g(input_quant, "num_bits") == 8
-            and str(g(weight_quant, "strategy")).split(".")[-1].lower() in ("channel", "tensor")
-            and str(g(input_quant, "strategy")).split(".")[-1].lower() == "token"
-            and bool(g(weight_quant, "symmetric", True)) and bool(g(input_quant, "symmetric", True))
-            and bool(g(input_quant, "dynamic", False)) and not bool(g(weight_quant, "dynamic", False)))
+    return (_get(weight_quant, "num_bits") == 8 and _get(input_quant, "num_bits") == 8
+            and str(_get(weight_quant, "type", "int")).split(".")[-1].lower() == "int"
+            and _strategy(weight_quant) in ("channel", "tensor") and _strategy(input_quant) == "token"
+            and bool(_get(weight_quant, "symmetric", True)) and bool(_get(input_quant, "symmetric", True))
+            and bool(_get(input_quant, "dynamic", False)) and not bool(_get(weight_quant, "dynamic", False)))
+
+
+def _scheme_is_fp8_block(weight_quant, input_quant) -> bool:
+    """8-bit float weights in 128x128 blocks, dynamic per-token-group(128) float activations."""
+    if weight_quant is None or input_quant is None:
+        return False
+    return (_get(weight_quant, "num_bits") == 8 and _get(input_quant, "num_bits") == 8
+            and str(_get(weight_quant, "type", "int")).split(".")[-1].lower() == "float"
+            and _strategy(weight_quant) == "block" and list(_get(weight_quant, "block_structure", [])) == [128, 128]
+            and _strategy(input_quant) == "group" and _get(input_quant, "group_size") == 128
+            and bool(_get(input_quant, "dynamic", False)))
 
 
 def _scheme_is_wna16(weight_quant, input_quant) -> bool:
     if weight_quant is None or input_quant is not None:
         return False
-    g = lambda o, k, d=None: o.get(k, d) if isinstance(o, dict) else getattr(o, k, d)  # noqa: E731
-    return str(g(weight_quant, "strategy")).split(".")[-1].lower() in ("channel", "group")
-
-
-class W8A8Plan:
-    """A filled kmoe_w8a8_args block plus its workspace; calling it enqueues the layer
-    on the current stream."""
-
-    def __init__(self, args, layout, workspace, keepalive):
-        self.args, self.layout, self.workspace, self._keep = args, layout, workspace, keepalive
-
-    def __call__(self) -> None:
-        L.check(L.lib.kmoe_forward_w8a8(self.args, L.ptr(self.workspace), self.workspace.numel(), L.stream()))
-
-    def view(self, name: str, count: int, dtype: torch.dtype) -> torch.Tensor:
-        """An intermediate of the last call, e.g. view("topk_ids", M*K, torch.int32)."""
-        off = getattr(self.layout, name)
-        nbytes = count * torch.empty(0, dtype=dtype).element_size()
-        return self.workspace[off: off + nbytes].view(dtype)
+    return _strategy(weight_quant) in ("channel", "group")
 
 
 class KunlunCompressedTensorsMoEMethod:
@@ -99,11 +82,15 @@ class KunlunCompressedTensorsMoEMethod:
             raise NotImplementedError("W4A16/W8A16 weight-only MoE is outside the W8A8 path of this build")
         if _scheme_is_dynamic_token_w8a8(weight_quant, input_quant):
             return KunlunCompressedTensorsW8A8Int8MoEMethod(weight_quant, input_quant, layer.moe_config)
+        if _scheme_is_fp8_block(weight_quant, input_quant):
+            return KunlunCompressedTensorsW8A8Fp8MoEMethod(weight_quant, input_quant, layer.moe_config)
         raise RuntimeError(f"Unsupported FusedMoe scheme: {weight_quant}, {input_quant}")
 
 
-class KunlunCompressedTensorsW8A8Int8MoEMethod:
-    """Dynamic-per-token W8A8 int8 MoE (reference: compressed_tensors_moe.py:111-291)."""
+class _MonolithicQuantMoE:
+    """What the int8 and fp8 methods share: routing-argument resolution and the plan."""
+
+    FORMAT = None
 
     def __init__(self, weight_quant=None, input_quant=None, moe=None):
         self.weight_quant = weight_quant
@@ -114,25 +101,7 @@ class KunlunCompressedTensorsW8A8Int8MoEMethod:
     def is_monolithic(self) -> bool:
         return True
 
-    def create_weights(self, layer: torch.nn.Module, num_experts: int, hidden_size: int,
-                       intermediate_size_per_partition: int, params_dtype: torch.dtype = torch.bfloat16,
-                       device=None, **_) -> None:
-        """Parameters as upstream's W8A8 int8 MoE method creates them: int8 weights
-        and one f32 SCALE per output channel (shapes per compressed_tensors_moe.py:135-137,212,258)."""
-        E, H, I = num_experts, hidden_size, intermediate_size_per_partition
-        mk = lambda *s, dt: torch.nn.Parameter(torch.zeros(*s, dtype=dt, device=device), requires_grad=False)  # noqa
-        layer.w13_weight = mk(E, 2 * I, H, dt=torch.int8)
-        layer.w2_weight = mk(E, H, I, dt=torch.int8)
-        layer.w13_weight_scale = mk(E, 2 * I, 1, dt=torch.float32)
-        layer.w2_weight_scale = mk(E, H, 1, dt=torch.float32)
-
-    def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
-        """scale -> absmax: the kernels dequantise with max/127 (reference: :116-120)."""
-        with torch.no_grad():
-            layer.w13_weight_scale.mul_(127.0)
-            layer.w2_weight_scale.mul_(127.0)
-
-    # -- routing parameters: kwargs win; a kwarg left at its default falls back to the layer
+    # routing parameters: kwargs win; a kwarg left at its default falls back to the layer
     @staticmethod
     def _routing(layer, topk_group, num_expert_group, scoring_func, routed_scaling_factor, bias):
         if scoring_func == "softmax" and getattr(layer, "scoring_func", "softmax") != "softmax":
@@ -164,7 +133,7 @@ class KunlunCompressedTensorsW8A8Int8MoEMethod:
         out_scale: float = 1.0,
     ) -> Union[torch.Tensor, tuple]:
         """x [M,H] bf16, router_logits [M,E] -> [M,H] bf16 (reference: :122-291).
-        `shared_expert` (w13, w13_max, w2, w2_max of a dense W8A8 MLP) and
+        `shared_expert` (w13, w13_max, w2, w2_max of a dense MLP in the layer's format) and
         `out_scale` fold the caller's epilogue (models/deepseek_v2.py:288-296) into the call."""
         if x.dtype != torch.bfloat16:
             raise NotImplementedError(f"apply_monolithic: activations must be bfloat16, got {x.dtype}")
@@ -179,51 +148,41 @@ class KunlunCompressedTensorsW8A8Int8MoEMethod:
 
     def make_plan(self, layer, x, logits, out, topk_group=None, num_expert_group=None, scoring_func="softmax",
                   routed_scaling_factor=1.0, e_score_correction_bias=None, shared_expert=None, out_scale=1.0,
-                  stage_events=None) -> "W8A8Plan":
+                  stage_events=None) -> MoEPlan:
         """Argument block for repeated calls on fixed buffers (x bf16 [M,H], logits f32
         [M,E], out bf16 [M,H], all contiguous): what a serving loop or a HIP-graph
         capture replays without touching Python-side allocation."""
         topk_group, num_expert_group, scoring_func, routed_scaling_factor, bias = self._routing(
             layer, topk_group, num_expert_group, scoring_func, routed_scaling_factor, e_score_correction_bias)
-        L.require_device(x, logits, out, layer.w13_weight, layer.w2_weight, bias)
-        L.require_contig(x, logits, out, layer.w13_weight, layer.w2_weight, layer.w13_weight_scale,
-                         layer.w2_weight_scale, bias)
-        if x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or logits.dtype != torch.float32:
-            raise ValueError("make_plan: x/out must be bfloat16 and logits float32")
-        E, two_i, H = layer.w13_weight.shape
-        M = x.shape[0]
-        if tuple(x.shape) != (M, H) or tuple(out.shape) != (M, H) or tuple(logits.shape) != (M, E):
-            raise ValueError("make_plan: x/out must be [M,H] and logits [M,E]")
-        a = L.W8A8Args()
-        a.M, a.H, a.E, a.K, a.I = M, H, E, self.moe.experts_per_token, two_i // 2
-        a.scoring = L.KMOE_SCORE_SOFTMAX if scoring_func == "softmax" else L.KMOE_SCORE_SIGMOID
-        a.renormalize = 1  # the reference always routes with the *_norm kernels
-        a.n_group = int(num_expert_group or 1)
-        a.topk_group = int(topk_group or 1)
-        a.routed_scale = float(routed_scaling_factor)
-        a.logits = logits.data_ptr()
-        a.bias = 0 if bias is None else bias.data_ptr()
-        a.x = x.data_ptr()
-        a.w13, a.w13_max = layer.w13_weight.data_ptr(), layer.w13_weight_scale.data_ptr()
-        a.w2, a.w2_max = layer.w2_weight.data_ptr(), layer.w2_weight_scale.data_ptr()
-        keep = [x, logits, out, bias, layer]
-        if shared_expert is not None:
-            ws13, ws13_max, ws2, ws2_max = shared_expert
-            L.require_device(ws13, ws13_max, ws2, ws2_max)
-            L.require_contig(ws13, ws13_max, ws2, ws2_max)
-            a.I_shared = ws13.shape[0] // 2
-            a.ws13, a.ws13_max, a.ws2, a.ws2_max = (ws13.data_ptr(), ws13_max.data_ptr(), ws2.data_ptr(),
-                                                    ws2_max.data_ptr())
-            keep.append(shared_expert)
-        a.out_scale = float(out_scale)
-        a.out = out.data_ptr()
-        if stage_events is not None:
-            a.stage_events = stage_events
-            keep.append(stage_events)
-        lay = L.W8A8Layout()
-        L.check(L.lib.kmoe_w8a8_workspace_layout(a, lay))
-        ws = _WORKSPACE.get(lay.total_bytes, x.device)
-        return W8A8Plan(a, lay, ws, keep)
+        return make_moe_plan(self.FORMAT, x, logits, out, self.moe.experts_per_token, layer.w13_weight,
+                             layer.w2_weight, layer.w13_weight_scale, layer.w2_weight_scale, scoring_func,
+                             True,  # the reference always routes with the *_norm kernels
+                             num_expert_group, topk_group, routed_scaling_factor, bias, shared_expert, out_scale,
+                             stage_events)
+
+
+class KunlunCompressedTensorsW8A8Int8MoEMethod(_MonolithicQuantMoE):
+    """Dynamic-per-token W8A8 int8 MoE (reference: compressed_tensors_moe.py:111-291)."""
+
+    FORMAT = L.KMOE_FMT_INT8
+
+    def create_weights(self, layer: torch.nn.Module, num_experts: int, hidden_size: int,
+                       intermediate_size_per_partition: int, params_dtype: torch.dtype = torch.bfloat16,
+                       device=None, **_) -> None:
+        """Parameters as upstream's W8A8 int8 MoE method creates them: int8 weights
+        and one f32 SCALE per output channel (shapes per compressed_tensors_moe.py:135-137,212,258)."""
+        E, H, I = num_experts, hidden_size, intermediate_size_per_partition
+        mk = lambda *s, dt: torch.nn.Parameter(torch.zeros(*s, dtype=dt, device=device), requires_grad=False)  # noqa
+        layer.w13_weight = mk(E, 2 * I, H, dt=torch.int8)
+        layer.w2_weight = mk(E, H, I, dt=torch.int8)
+        layer.w13_weight_scale = mk(E, 2 * I, 1, dt=torch.float32)
+        layer.w2_weight_scale = mk(E, H, 1, dt=torch.float32)
+
+    def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
+        """scale -> absmax: the kernels dequantise with max/127 (reference: :116-120)."""
+        with torch.no_grad():
+            layer.w13_weight_scale.mul_(127.0)
+            layer.w2_weight_scale.mul_(127.0)
 
     def apply_staged(self, layer, x, router_logits, topk_group=None, num_expert_group=None, global_num_experts=-1,
                      scoring_func="softmax", routed_scaling_factor=1.0, e_score_correction_bias=None):
@@ -272,3 +231,26 @@ class KunlunCompressedTensorsW8A8Int8MoEMethod:
         output = torch.empty(M, H, dtype=x.dtype, device=dev)
         ops.moe_post(out, sorted_tokens_idx.view(M, K), normed_score, dequant_scale, output)
         return output
+
+
+class KunlunCompressedTensorsW8A8Fp8MoEMethod(_MonolithicQuantMoE):
+    """fp8-e4m3fn weights with 128x128 block scales, dynamic per-token-group(128) fp8
+    activations (DeepSeek-V3 recipe). No counterpart in the reference, whose platform
+    rejects fp8 (platforms/kunlun.py:350-364); same monolithic interface as the int8 method."""
+
+    FORMAT = L.KMOE_FMT_FP8_BLOCK
+
+    def create_weights(self, layer: torch.nn.Module, num_experts: int, hidden_size: int,
+                       intermediate_size_per_partition: int, params_dtype: torch.dtype = torch.bfloat16,
+                       device=None, **_) -> None:
+        E, H, I = num_experts, hidden_size, intermediate_size_per_partition
+        if H % 128 or I % 128:
+            raise ValueError("fp8 block-scaled MoE needs hidden and intermediate sizes that are multiples of 128")
+        mk = lambda *s, dt: torch.nn.Parameter(torch.zeros(*s, dtype=dt, device=device), requires_grad=False)  # noqa
+        layer.w13_weight = mk(E, 2 * I, H, dt=torch.float8_e4m3fn)
+        layer.w2_weight = mk(E, H, I, dt=torch.float8_e4m3fn)
+        layer.w13_weight_scale = mk(E, 2 * I // 128, H // 128, dt=torch.float32)
+        layer.w2_weight_scale = mk(E, H // 128, I // 128, dt=torch.float32)
+
+    def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
+        """Block scales are used as they are (dequant = code * scale); nothing to convert."""

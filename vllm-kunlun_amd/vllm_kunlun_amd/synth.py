@@ -83,6 +83,78 @@ class SynthLayer:
         return kw
 
 
+def _quant_block_fp8(w: torch.Tensor):
+    """[n,k] float -> e4m3fn codes + one f32 scale per 128x128 block (absmax/448)."""
+    n, k = w.shape
+    wb = w.reshape(n // 128, 128, k // 128, 128)
+    s = wb.abs().amax(dim=(1, 3), keepdim=True).clamp_min(1e-12) / 448.0
+    q = (wb / s).clamp_(-448.0, 448.0).to(torch.float8_e4m3fn).reshape(n, k)
+    return q, s.reshape(n // 128, k // 128)
+
+
+def _routing_inputs(s: MoEShape, g, dev):
+    bias = None
+    if s.scoring == "sigmoid":
+        bias = torch.randn(s.E, generator=g, device=dev, dtype=torch.float32) * 0.01
+    return bias
+
+
+def _activations(s: MoEShape, g, dev):
+    x = torch.randn(s.M, s.H, generator=g, device=dev).to(torch.bfloat16)
+    logits = torch.randn(s.M, s.E, generator=g, device=dev, dtype=torch.float32)
+    if s.hot_experts:
+        hot = torch.arange(s.hot_experts, device=dev) * (s.E // s.hot_experts)
+        logits[:, hot] += s.hot_bias
+    return x, logits
+
+
+def make_fp8_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
+    """FusedMoE with the fp8 block-scaled method and random weights quantised per 128x128 block."""
+    from .quantization.compressed_tensors.compressed_tensors_moe import KunlunCompressedTensorsW8A8Fp8MoEMethod
+    dev = torch.device(device)
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    s = shape
+    method = KunlunCompressedTensorsW8A8Fp8MoEMethod()
+    bias = _routing_inputs(s, g, dev)
+    layer = FusedMoE(num_experts=s.E, top_k=s.K, hidden_size=s.H, intermediate_size=s.I, renormalize=True,
+                     use_grouped_topk=s.n_group > 1, num_expert_group=s.n_group, topk_group=s.topk_group,
+                     scoring_func=s.scoring, e_score_correction_bias=bias, quant_method=method, device=dev)
+    for e in range(s.E):
+        q, sc = _quant_block_fp8(torch.randn(2 * s.I, s.H, generator=g, device=dev) * 0.02)
+        layer.w13_weight.data[e].copy_(q)
+        layer.w13_weight_scale.data[e].copy_(sc)
+        q, sc = _quant_block_fp8(torch.randn(s.H, s.I, generator=g, device=dev) * 0.02)
+        layer.w2_weight.data[e].copy_(q)
+        layer.w2_weight_scale.data[e].copy_(sc)
+    method.process_weights_after_loading(layer)
+    shared = None
+    if s.I_shared:
+        q13, s13 = _quant_block_fp8(torch.randn(2 * s.I_shared, s.H, generator=g, device=dev) * 0.02)
+        q2, s2 = _quant_block_fp8(torch.randn(s.H, s.I_shared, generator=g, device=dev) * 0.02)
+        shared = (q13, s13.contiguous(), q2, s2.contiguous())
+    x, logits = _activations(s, g, dev)
+    return SynthLayer(s, layer, x, logits, bias, shared)
+
+
+def make_bf16_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
+    """FusedMoE with the unquantized method and bf16 weights ~ N(0, 0.02)."""
+    dev = torch.device(device)
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    s = shape
+    bias = _routing_inputs(s, g, dev)
+    layer = FusedMoE(num_experts=s.E, top_k=s.K, hidden_size=s.H, intermediate_size=s.I, renormalize=True,
+                     use_grouped_topk=s.n_group > 1, num_expert_group=s.n_group, topk_group=s.topk_group,
+                     scoring_func=s.scoring, e_score_correction_bias=bias, device=dev)
+    for e in range(s.E):
+        layer.w13_weight.data[e].copy_(torch.randn(2 * s.I, s.H, generator=g, device=dev) * 0.02)
+        layer.w2_weight.data[e].copy_(torch.randn(s.H, s.I, generator=g, device=dev) * 0.02)
+    layer.quant_method.process_weights_after_loading(layer)
+    x, logits = _activations(s, g, dev)
+    return SynthLayer(s, layer, x, logits, bias, None)
+
+
 def make_w8a8_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
     """Builds a FusedMoE with the W8A8 method, fills it with quantised random
     weights and runs process_weights_after_loading (scales become maxes)."""

@@ -82,11 +82,10 @@ def cpu_baseline(sl, budget_s=20.0):
     import torch
     from oracle import torch_moe as tm
     s = sl.shape
-    lay = sl.layer
     host = lambda t: None if t is None else t.detach().cpu()  # noqa: E731
-    args = (host(sl.x), host(sl.logits), host(lay.w13_weight), host(lay.w13_weight_scale), host(lay.w2_weight),
-            host(lay.w2_weight_scale), s.K, s.scoring, True, s.n_group, s.topk_group, s.routed_scale, host(sl.bias),
-            None if sl.shared is None else tuple(host(t) for t in sl.shared))
+    w13, w13_max, w2, w2_max, shared = sl.host_weights()  # row-major copies of the (tiled) device weights
+    args = (host(sl.x), host(sl.logits), w13, w13_max, w2, w2_max, s.K, s.scoring, True, s.n_group, s.topk_group,
+            s.routed_scale, host(sl.bias), shared)
     t0 = time.perf_counter()
     tm.w8a8_moe(*args)  # warm-up
     first = time.perf_counter() - t0

@@ -132,6 +132,14 @@ int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q,
                        int64_t ld_q, float* row_max, kmoe_stream_t stream);
 
 /*
+ * Same quantisation, codes written "chunk-major": q is [C/16][R][16], i.e. code
+ * (r, c) sits at ((c/16)*R + r)*16 + c%16 — the activation layout of the
+ * weight-streaming GEMM (KMOE_A_CHUNKED). Limits as above, and C % 16 == 0.
+ */
+int kmoe_quant_i8_rows_chunked(const uint16_t* x, int64_t ld_x, int R, int C,
+                               int8_t* q, float* row_max, kmoe_stream_t stream);
+
+/*
  * Per-row, per-128-column-group dynamic fp8-e4m3fn (OCP). No counterpart in the
  * reference (its fp8 ops are empty stubs, ops/_custom_ops.py:44-89); follows
  * the DeepSeek-V3 block-scaled recipe.
@@ -165,7 +173,27 @@ typedef struct kmoe_gemm_i8_args {
   int32_t* acc_out;       /* NULL, or int32 [rows, n]: raw accumulators         */
   int32_t act;            /* KMOE_ACT_*                                         */
   int32_t variant;        /* 0 = choose from shape; >0 force a kernel variant   */
+  int32_t w_layout;       /* KMOE_W_ROWMAJOR, or KMOE_W_TILED (kmoe_tile_weights_i8) */
+  int32_t a_layout;       /* KMOE_A_ROWMAJOR, or KMOE_A_CHUNKED: a is [k/16][a_rows][16]
+                             (kmoe_quant_i8_rows_chunked); needs w_layout TILED   */
+  int32_t a_rows;         /* rows of the chunked activation array               */
 } kmoe_gemm_i8_args;
+
+#define KMOE_W_ROWMAJOR 0
+#define KMOE_W_TILED 1
+#define KMOE_A_ROWMAJOR 0
+#define KMOE_A_CHUNKED 1
+
+/*
+ * Re-arranges int8 weights [E,n,k] (k contiguous) into MFMA-ready 1 KB blocks
+ * [E][n/16][k/64][4][16][16]: block byte 256*g + 16*c + t holds channel 16*nb + c,
+ * k = 64*kb + 16*g + t. Done once after loading (the reference's hook for load-time
+ * work is process_weights_after_loading, compressed_tensors_moe.py:116-120); the
+ * values and every result are unchanged, only the streaming pattern is.
+ * dst must not alias src. Limits: n % 16 == 0, k % 64 == 0.
+ */
+int kmoe_tile_weights_i8(const int8_t* src, int8_t* dst, int E, int n, int k,
+                         kmoe_stream_t stream);
 
 /*
  * W8A8 grouped GEMM. Replaces kunlun_ops.moe_fc in its int8 form
@@ -293,6 +321,8 @@ typedef struct kmoe_moe_args {
      recorded on the stream before stage s and entry 2s+1 after it (NULL entries
      are skipped). Leave NULL under graph capture.                             */
   void* const* stage_events;
+  int32_t w_layout;      /* INT8 only: KMOE_W_TILED if w13, w2 (and ws13, ws2) went
+                            through kmoe_tile_weights_i8; else KMOE_W_ROWMAJOR  */
 } kmoe_moe_args;
 
 #define KMOE_STAGE_ROUTING 0
@@ -313,6 +343,8 @@ typedef struct kmoe_moe_layout {
   size_t topk_w, topk_ids, moe_index, sorted_src, expert_m, lod, align_ws;
   size_t xq, xmax, act, actq, actmax, down;
   size_t sh_lod, sh_act, sh_actq, sh_actmax, sh_out;
+  size_t codes_chunked; /* 1: xq/actq/sh_actq are chunk-major [C/16][rows][16] (the
+                           weight-streaming decode path), 0: row-major [rows][C] */
 } kmoe_moe_layout;
 
 /* Workspace layout (and total size) for a shape; only the shape and format fields of args are read. */

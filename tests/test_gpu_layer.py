@@ -26,13 +26,12 @@ def _host(t):
 
 def _oracle_inputs(sl):
     """Host copies of a SynthLayer's tensors in the oracle's formats."""
-    lay = sl.layer
-    shared = None
-    if sl.shared is not None:
-        shared = tuple(_host(t).numpy() for t in sl.shared)
-    return dict(x_bits=bits(sl.x), logits=_host(sl.logits).numpy(), w13=_host(lay.w13_weight).numpy(),
-                w13_max=_host(lay.w13_weight_scale).numpy(), w2=_host(lay.w2_weight).numpy(),
-                w2_max=_host(lay.w2_weight_scale).numpy(), K=sl.shape.K, scoring=sl.shape.scoring,
+    w13, w13_max, w2, w2_max, shared = sl.host_weights()
+    if shared is not None:
+        shared = tuple(t.numpy() for t in shared)
+    return dict(x_bits=bits(sl.x), logits=_host(sl.logits).numpy(), w13=w13.numpy(),
+                w13_max=w13_max.numpy(), w2=w2.numpy(),
+                w2_max=w2_max.numpy(), K=sl.shape.K, scoring=sl.shape.scoring,
                 n_group=sl.shape.n_group, topk_group=sl.shape.topk_group, routed_scale=sl.shape.routed_scale,
                 bias=None if sl.bias is None else _host(sl.bias).numpy(), shared=shared)
 
@@ -72,7 +71,10 @@ def test_layer_matches_oracles(name, base, over):
     ids = _view(ws, lay.topk_ids, P, torch.int32).cpu().numpy().reshape(shape.M, shape.K)
     moe_index = _view(ws, lay.moe_index, P, torch.int32).cpu().numpy()
     lod = _view(ws, lay.lod, E + 1, torch.int32).cpu().numpy()
-    actq = _view(ws, lay.actq, P * I, torch.int8).cpu().numpy().reshape(P, I)
+    actq = _view(ws, lay.actq, P * I, torch.int8).cpu().numpy()
+    if lay.codes_chunked:  # [I/16][P][16] -> [P][I]
+        actq = actq.reshape(I // 16, P, 16).transpose(1, 0, 2)
+    actq = np.ascontiguousarray(actq).reshape(P, I)
     topk_w = _view(ws, lay.topk_w, P, torch.float32).cpu().numpy().reshape(shape.M, shape.K)
     assert np.array_equal(ids, inter["topk_ids"]), "routing ids"
     assert np.array_equal(moe_index, inter["moe_index"]), "sorted token map"
@@ -82,10 +84,8 @@ def test_layer_matches_oracles(name, base, over):
     assert np.array_equal(bits(out), ref_bits), "bf16 output vs C oracle"
 
     # the reference's torch expert loop, written independently of the C oracle
-    lay_ = sl.layer
-    shared = None if sl.shared is None else tuple(_host(t) for t in sl.shared)
-    ref_t = tm.w8a8_moe(_host(sl.x), _host(sl.logits), _host(lay_.w13_weight), _host(lay_.w13_weight_scale),
-                        _host(lay_.w2_weight), _host(lay_.w2_weight_scale), shape.K, shape.scoring, True,
+    w13, w13_max, w2, w2_max, shared = sl.host_weights()
+    ref_t = tm.w8a8_moe(_host(sl.x), _host(sl.logits), w13, w13_max, w2, w2_max, shape.K, shape.scoring, True,
                         shape.n_group, shape.topk_group, shape.routed_scale, _host(sl.bias), shared, out_scale)
     assert rel_l2(out, ref_t) <= REL_L2_BF16
 
@@ -108,6 +108,30 @@ def test_staged_ops_equal_fused():
     staged = m.apply_staged(sl.layer, sl.x, sl.logits, **kw)
     torch.cuda.synchronize()
     assert torch.equal(fused, staged)
+
+
+def test_tiled_and_rowmajor_weights_give_the_same_bits():
+    """process_weights_after_loading tiles the int8 weights in place on the GPU; a layer
+    kept row-major (tile_weights=False) must produce identical outputs, in the streaming
+    regime (few rows per expert) and in the tiled-GEMM regime (many rows per expert)."""
+    from vllm_kunlun_amd import _plan, synth
+    from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors_moe import (
+        KunlunCompressedTensorsW8A8Int8MoEMethod)
+    for over in (dict(M=48, H=512, E=16, K=4, I=256), dict(M=900, H=256, E=8, K=2, I=128)):
+        shape = synth.scaled(synth.SHAPES["dsv3-decode"], n_group=4, topk_group=2, I_shared=128, **over)
+        tiled = synth.make_w8a8_layer(shape, "cuda", seed=9)
+        assert _plan.is_tiled(tiled.layer.w13_weight) and _plan.is_tiled(tiled.shared[0])
+        KunlunCompressedTensorsW8A8Int8MoEMethod.tile_weights = False
+        try:
+            plain = synth.make_w8a8_layer(shape, "cuda", seed=9)
+        finally:
+            del KunlunCompressedTensorsW8A8Int8MoEMethod.tile_weights
+        assert not _plan.is_tiled(plain.layer.w13_weight)
+        a = tiled.layer.quant_method.apply_monolithic(tiled.layer, tiled.x, tiled.logits, **tiled.apply_kwargs())
+        assert tiled.layer.quant_method.last_layout.codes_chunked == (1 if over["M"] == 48 else 0)
+        b = plain.layer.quant_method.apply_monolithic(plain.layer, plain.x, plain.logits, **plain.apply_kwargs())
+        torch.cuda.synchronize()
+        assert torch.equal(a, b)
 
 
 def test_layer_forward_via_module_call():

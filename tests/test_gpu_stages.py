@@ -303,3 +303,105 @@ def test_combine(L, M, K, H, epilogue):
                                L.ptr(out), H, L.stream()))
     sync()
     assert np.array_equal(bits(out), ref)
+
+
+# ------------------------------------------- tiled weights / chunked activations
+def _tile_ref(w):
+    """numpy restatement of the 1 KB block layout: [E][n/16][k/64][g(4)][c(16)][16]."""
+    E, n, k = w.shape
+    return np.ascontiguousarray(w.reshape(E, n // 16, 16, k // 64, 4, 16).transpose(0, 1, 3, 4, 2, 5))
+
+
+@pytest.mark.parametrize("E,n,k", [(1, 16, 64), (3, 48, 192), (2, 1536, 2048)])
+def test_tile_weights(L, E, n, k):
+    w = np.random.default_rng(E + n).integers(-128, 128, (E, n, k), dtype=np.int8)
+    src = dev(w)
+    dst = torch.empty_like(src)
+    L.check(L.lib.kmoe_tile_weights_i8(L.ptr(src), L.ptr(dst), E, n, k, L.stream()))
+    sync()
+    assert np.array_equal(dst.cpu().numpy().reshape(-1), _tile_ref(w).reshape(-1))
+    assert L.lib.kmoe_tile_weights_i8(L.ptr(src), L.ptr(src), E, n, k, L.stream()) == -2  # in place is refused
+
+
+@pytest.mark.parametrize("R,Cc", [(1, 16), (64, 2048), (100, 768), (33, 7168), (512, 2048)])
+def test_quant_i8_rows_chunked(L, R, Cc):
+    torch.manual_seed(R + Cc)
+    x = (torch.randn(R, Cc) * 3).bfloat16()
+    x[0] = 0
+    q_ref, mx_ref = co.quant_i8_rows(bits(x))
+    dx = x.cuda()
+    q = torch.empty(Cc // 16, R, 16, dtype=torch.int8, device="cuda")
+    mx = torch.empty(R, dtype=torch.float32, device="cuda")
+    L.check(L.lib.kmoe_quant_i8_rows_chunked(L.ptr(dx), Cc, R, Cc, L.ptr(q), L.ptr(mx), L.stream()))
+    sync()
+    assert np.array_equal(mx.cpu().numpy(), mx_ref)
+    assert np.array_equal(q.cpu().numpy().transpose(1, 0, 2).reshape(R, Cc), q_ref)
+
+
+def _gemm_layout_case(L, E, n, k, counts, act, variant, gather, chunked, seed=0):
+    rng = np.random.default_rng(seed)
+    counts = np.asarray(counts, dtype=np.int32)
+    lod = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(lod[-1])
+    w = rng.integers(-127, 128, (E, n, k), dtype=np.int8)
+    w_max = (rng.random((E, n)) * 0.1 + 0.01).astype(np.float32)
+    if gather:
+        src_div = 4
+        a_rows = max(1, (rows + src_div - 1) // src_div)
+        row_src = rng.permutation(a_rows * src_div)[:rows].astype(np.int32)
+    else:
+        src_div, a_rows, row_src = 1, max(rows, 1), None
+    a = rng.integers(-127, 128, (a_rows, k), dtype=np.int8)
+    a_max = (rng.random(a_rows) * 4 + 0.1).astype(np.float32)
+    y_ref, acc_ref = co.grouped_gemm_i8(a, a_max, w, w_max, lod, act=act, row_src=row_src, src_div=src_div,
+                                        want_acc=True)
+    n_out = n // 2 if act else n
+    a_dev = dev(np.ascontiguousarray(a.reshape(a_rows, k // 16, 16).transpose(1, 0, 2))) if chunked else dev(a)
+    d = dict(a=a_dev, a_max=dev(a_max), w=dev(_tile_ref(w)), w_max=dev(w_max), lod=dev(lod),
+             row_src=None if row_src is None else dev(row_src))
+    y = torch.zeros(max(rows, 1), n_out, dtype=torch.bfloat16, device="cuda")
+    acc = torch.zeros(max(rows, 1), n, dtype=torch.int32, device="cuda")
+    args = L.GemmI8Args()
+    args.a, args.lda, args.a_max = d["a"].data_ptr(), k, d["a_max"].data_ptr()
+    args.row_src = 0 if row_src is None else d["row_src"].data_ptr()
+    args.src_div = src_div
+    args.w, args.w_max, args.lod = d["w"].data_ptr(), d["w_max"].data_ptr(), d["lod"].data_ptr()
+    args.E, args.n, args.k, args.rows = E, n, k, rows
+    args.y, args.ldy, args.acc_out = y.data_ptr(), n_out, acc.data_ptr()
+    args.act, args.variant = act, variant
+    args.w_layout = L.KMOE_W_TILED
+    args.a_layout = L.KMOE_A_CHUNKED if chunked else L.KMOE_A_ROWMAJOR
+    args.a_rows = a_rows
+    L.check(L.lib.kmoe_grouped_gemm_i8(args, L.stream()))
+    sync()
+    assert np.array_equal(acc.cpu().numpy()[:rows], acc_ref), "int32 accumulators differ"
+    assert np.array_equal(bits(y)[:rows], y_ref), "bf16 outputs differ"
+
+
+TILED_CASES = [
+    (1, 64, 256, [16]),
+    (4, 64, 256, [3, 0, 17, 1]),
+    (8, 128, 512, [4, 4, 0, 9, 33, 1, 0, 2]),
+    (3, 96, 768, [5, 40, 7]),
+    (2, 256, 2048, [130, 129]),
+    (5, 1536, 64, [1, 2, 3, 4, 5]),
+    (2, 32, 320, [20, 3]),
+    (16, 192, 384, [0] * 15 + [300]),
+]
+
+
+@pytest.mark.parametrize("E,n,k,counts", TILED_CASES)
+@pytest.mark.parametrize("variant", [1, 2, 4, 8])
+@pytest.mark.parametrize("act", [0, 1])
+@pytest.mark.parametrize("gather", [False, True])
+def test_stream_gemm_i8(L, E, n, k, counts, variant, act, gather):
+    """Weight-streaming kernel: tiled weights x chunk-major activations."""
+    _gemm_layout_case(L, E, n, k, counts, act, variant, gather, chunked=True, seed=E * n + k)
+
+
+@pytest.mark.parametrize("E,n,k,counts", TILED_CASES)
+@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("act", [0, 1])
+def test_lds_gemm_i8_with_tiled_weights(L, E, n, k, counts, variant, act):
+    """LDS-tiled kernel reading tiled weights and row-major activations."""
+    _gemm_layout_case(L, E, n, k, counts, act, variant, True, chunked=False, seed=E * n + k + 7)

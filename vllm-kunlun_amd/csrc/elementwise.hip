@@ -16,7 +16,7 @@ union Pack8 {  // 8 bf16
 template <int TPR, int NV>
 __global__ __launch_bounds__(256) void quant_i8_rows_kernel(const uint16_t* __restrict__ x, int64_t ld_x, int R,
                                                            int C, int8_t* __restrict__ q, int64_t ld_q,
-                                                           float* __restrict__ row_max) {
+                                                           float* __restrict__ row_max, int chunked) {
   constexpr int kRowsPerBlock = 256 / TPR;
   __shared__ float red[256 / kWave];
   const int sub = threadIdx.x / TPR;
@@ -48,7 +48,9 @@ __global__ __launch_bounds__(256) void quant_i8_rows_kernel(const uint16_t* __re
   }
   if (!live) return;
   const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
-  uint2* dst = reinterpret_cast<uint2*>(q + static_cast<size_t>(r) * ld_q);
+  // row-major: vector v of the row; chunk-major [C/16][R][16]: vector v is half v%2 of chunk v/2
+  uint2* dst = reinterpret_cast<uint2*>(q + static_cast<size_t>(r) * (chunked ? 16 : ld_q));
+  const size_t vstride = chunked ? static_cast<size_t>(R) : 0;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int v = t + i * TPR;
@@ -61,7 +63,7 @@ __global__ __launch_bounds__(256) void quant_i8_rows_kernel(const uint16_t* __re
         const int qi = static_cast<int>(f);
         w[j >> 2] |= static_cast<uint32_t>(qi & 0xff) << (8 * (j & 3));
       }
-      dst[v] = make_uint2(w[0], w[1]);
+      dst[chunked ? (v >> 1) * vstride * 2 + (v & 1) : v] = make_uint2(w[0], w[1]);
     }
   }
   if (t == 0) row_max[r] = amax;
@@ -204,6 +206,26 @@ int fill_dense_lod(int32_t* lod2, int rows, hipStream_t stream) {
 
 using namespace kmoe;
 
+namespace {
+int quant_i8_launch(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q, float* row_max,
+                    int chunked, hipStream_t s, const char* what) {
+  if (C <= 64 * 8 * 2) {
+    hipLaunchKernelGGL((quant_i8_rows_kernel<64, 2>), dim3(ceil_div(R, 4)), dim3(256), 0, s, x, ld_x, R, C, q, ld_q,
+                       row_max, chunked);
+  } else if (C <= 64 * 8 * 4) {
+    hipLaunchKernelGGL((quant_i8_rows_kernel<64, 4>), dim3(ceil_div(R, 4)), dim3(256), 0, s, x, ld_x, R, C, q, ld_q,
+                       row_max, chunked);
+  } else if (C <= 256 * 8 * 4) {
+    hipLaunchKernelGGL((quant_i8_rows_kernel<256, 4>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max,
+                       chunked);
+  } else {
+    hipLaunchKernelGGL((quant_i8_rows_kernel<256, 8>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max,
+                       chunked);
+  }
+  return check_launch(what);
+}
+}  // namespace
+
 extern "C" int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q,
                                   float* row_max, kmoe_stream_t stream) {
   KMOE_REQUIRE(x && q && row_max, KMOE_ERR_NULL, "quant_i8_rows: NULL pointer");
@@ -213,19 +235,18 @@ extern "C" int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C,
                "quant_i8_rows: row strides %lld/%lld must be multiples of 8 and >= C", (long long)ld_x,
                (long long)ld_q);
   if (R == 0) return KMOE_OK;
-  hipStream_t s = as_stream(stream);
-  if (C <= 64 * 8 * 2) {
-    hipLaunchKernelGGL((quant_i8_rows_kernel<64, 2>), dim3(ceil_div(R, 4)), dim3(256), 0, s, x, ld_x, R, C, q, ld_q,
-                       row_max);
-  } else if (C <= 64 * 8 * 4) {
-    hipLaunchKernelGGL((quant_i8_rows_kernel<64, 4>), dim3(ceil_div(R, 4)), dim3(256), 0, s, x, ld_x, R, C, q, ld_q,
-                       row_max);
-  } else if (C <= 256 * 8 * 4) {
-    hipLaunchKernelGGL((quant_i8_rows_kernel<256, 4>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max);
-  } else {
-    hipLaunchKernelGGL((quant_i8_rows_kernel<256, 8>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max);
-  }
-  return check_launch("kmoe_quant_i8_rows");
+  return quant_i8_launch(x, ld_x, R, C, q, ld_q, row_max, 0, as_stream(stream), "kmoe_quant_i8_rows");
+}
+
+extern "C" int kmoe_quant_i8_rows_chunked(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, float* row_max,
+                                          kmoe_stream_t stream) {
+  KMOE_REQUIRE(x && q && row_max, KMOE_ERR_NULL, "quant_i8_rows_chunked: NULL pointer");
+  KMOE_REQUIRE(R >= 0 && C >= 16 && C % 16 == 0 && C <= 16384, KMOE_ERR_SHAPE,
+               "quant_i8_rows_chunked: R=%d C=%d (need C %% 16 == 0, 16 <= C <= 16384)", R, C);
+  KMOE_REQUIRE(ld_x % 8 == 0 && ld_x >= C, KMOE_ERR_SHAPE,
+               "quant_i8_rows_chunked: row stride %lld must be a multiple of 8 and >= C", (long long)ld_x);
+  if (R == 0) return KMOE_OK;
+  return quant_i8_launch(x, ld_x, R, C, q, 0, row_max, 1, as_stream(stream), "kmoe_quant_i8_rows_chunked");
 }
 
 extern "C" int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, int C, uint8_t* q, int64_t ld_q,

@@ -46,7 +46,18 @@ int check_shape(const kmoe_moe_args* a) {
   KMOE_REQUIRE(a->I_shared >= 0 && a->I_shared % mult == 0, KMOE_ERR_SHAPE,
                "moe_forward: I_shared=%d must be a non-negative multiple of %d", a->I_shared, mult);
   KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "moe_forward: M*K too large");
+  KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR ||
+                   (a->w_layout == KMOE_W_TILED && a->format == KMOE_FMT_INT8 && a->H % 64 == 0 && a->I % 64 == 0 &&
+                    a->I_shared % 64 == 0),
+               KMOE_ERR_SHAPE, "moe_forward: w_layout=%d needs int8 weights and H, I multiples of 64", a->w_layout);
   return KMOE_OK;
+}
+
+// Few rows per expert: every weight byte is used once, so stream tiled weights
+// against chunk-major codes; otherwise the LDS-tiled GEMM on row-major codes.
+bool use_stream_path(const kmoe_moe_args* a) {
+  const long long P = static_cast<long long>(a->M) * a->K;
+  return a->format == KMOE_FMT_INT8 && a->w_layout == KMOE_W_TILED && (P + a->E - 1) / a->E <= 64 && a->M <= 1024;
 }
 
 // One expert-MLP pass (gate_up + SiLU-mul, requantise, down) over `rows` rows in
@@ -66,6 +77,9 @@ struct MlpPass {
   void* actq;      // [rows, I] codes
   float* act_aux;  // [rows] or [rows, I/128]
   uint16_t* out;   // [rows, H] bf16
+  int w_layout;    // INT8: KMOE_W_*
+  bool stream;     // INT8 + tiled weights: chunk-major codes and the weight-streaming GEMM
+  int x_count;     // rows of x_rows (chunk-major addressing)
 };
 
 int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
@@ -97,6 +111,11 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.y = y;
     g.ldy = ldy;
     g.act = act;
+    g.w_layout = m.w_layout;
+    if (m.stream) {
+      g.a_layout = KMOE_A_CHUNKED;
+      g.a_rows = first ? m.x_count : m.rows;
+    }
     return kmoe_grouped_gemm_i8(&g, stream);
   }
   if (m.format == KMOE_FMT_FP8_BLOCK) {
@@ -144,7 +163,8 @@ int run_mlp(const MlpPass& m, kmoe_stream_t stream, Mark&& mark) {
   mark(KMOE_STAGE_GEMM1, 1);
   mark(KMOE_STAGE_QUANT2, 0);
   if (m.format == KMOE_FMT_INT8) {
-    rc = kmoe_quant_i8_rows(m.act, m.I, m.rows, m.I, static_cast<int8_t*>(m.actq), m.I, m.act_aux, stream);
+    rc = m.stream ? kmoe_quant_i8_rows_chunked(m.act, m.I, m.rows, m.I, static_cast<int8_t*>(m.actq), m.act_aux, stream)
+                  : kmoe_quant_i8_rows(m.act, m.I, m.rows, m.I, static_cast<int8_t*>(m.actq), m.I, m.act_aux, stream);
   } else if (m.format == KMOE_FMT_FP8_BLOCK) {
     rc = kmoe_quant_fp8_group128(m.act, m.I, m.rows, m.I, static_cast<uint8_t*>(m.actq), m.I, m.act_aux, stream);
   }
@@ -190,6 +210,7 @@ extern "C" int kmoe_moe_workspace_layout(const kmoe_moe_args* a, kmoe_moe_layout
   L->sh_actmax = take(quant ? M * 4 * (fp8 ? Is / 128 : 1) : 0);
   L->sh_out = take(Is ? M * H * 2 : 0);
   L->total_bytes = off;
+  L->codes_chunked = use_stream_path(a) ? 1 : 0;
   return KMOE_OK;
 }
 
@@ -245,8 +266,12 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   // 3. quantise each TOKEN row once (the reference quantises the K-times expanded copy; same values)
   mark(KMOE_STAGE_QUANT1, 0);
   const void* x_rows = a->x;
+  const bool stream_mode = use_stream_path(a);
   if (a->format == KMOE_FMT_INT8) {
-    rc = kmoe_quant_i8_rows(a->x, H, M, H, static_cast<int8_t*>(at(L.xq)), H, static_cast<float*>(at(L.xmax)), stream);
+    rc = stream_mode ? kmoe_quant_i8_rows_chunked(a->x, H, M, H, static_cast<int8_t*>(at(L.xq)),
+                                                  static_cast<float*>(at(L.xmax)), stream)
+                     : kmoe_quant_i8_rows(a->x, H, M, H, static_cast<int8_t*>(at(L.xq)), H,
+                                          static_cast<float*>(at(L.xmax)), stream);
     x_rows = at(L.xq);
   } else if (a->format == KMOE_FMT_FP8_BLOCK) {
     rc = kmoe_quant_fp8_group128(a->x, H, M, H, static_cast<uint8_t*>(at(L.xq)), H, static_cast<float*>(at(L.xmax)),
@@ -276,6 +301,9 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   routed.actq = at(L.actq);
   routed.act_aux = static_cast<float*>(at(L.actmax));
   routed.out = static_cast<uint16_t*>(at(L.down));
+  routed.w_layout = a->w_layout;
+  routed.stream = stream_mode;
+  routed.x_count = M;
   rc = run_mlp(routed, stream, mark);
   if (rc) return rc;
 

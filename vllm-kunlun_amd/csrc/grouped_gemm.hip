@@ -61,6 +61,7 @@ struct GemmParams {
   uint16_t* y;
   int64_t ldy;             // in elements
   int32_t* acc_out;        // I8 only
+  int32_t w_tiled;         // weights in 64*LB-byte MFMA blocks [E][n/16][kbytes/(4*LB)] instead of row-major
 };
 
 __device__ inline int wave_incl_scan(int v) {
@@ -158,8 +159,14 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
     const int c = col_base + fh * 16;
     wok[f] = c < n_half;
     col[f] = (SWIGLU && f >= NFH) ? n_half + c : c;
-    wp[f] = p.w + (static_cast<size_t>(e) * p.n + (wok[f] ? col[f] + li : 0)) * p.kbytes + lg * LB;
+    if (p.w_tiled) {  // block (fragment, step): 64*LB consecutive bytes, lane l at l*LB
+      const size_t frag = static_cast<size_t>(e) * (p.n / 16) + (wok[f] ? col[f] / 16 : 0);
+      wp[f] = p.w + frag * (p.kbytes / (4 * LB)) * (64 * LB) + lane * LB;
+    } else {
+      wp[f] = p.w + (static_cast<size_t>(e) * p.n + (wok[f] ? col[f] + li : 0)) * p.kbytes + lg * LB;
+    }
   }
+  const int w_step = p.w_tiled ? 64 * LB : 4 * LB;  // bytes between consecutive MFMA steps of a fragment
   const int nchunks = (p.kbytes + kKC - 1) / kKC;
   const int kblocks = p.kbytes / 128;  // FP8: scale blocks along K
 
@@ -205,9 +212,10 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
         for (int j = 0; j < kJ; ++j)
 #pragma unroll
           for (int v = 0; v < kV; ++v) {
-            const int off = kc + j * 4 * LB + v * 16;  // + lg*LB is folded into wp
-            dst[f][j][v] = (wok[f] && off + lg * LB < p.kbytes) ? *reinterpret_cast<const v4i*>(wp[f] + off)
-                                                                 : (v4i){0, 0, 0, 0};
+            const int koff = kc + j * 4 * LB + v * 16;  // k position (+ lg*LB, folded into wp)
+            const size_t off = static_cast<size_t>(chunk * kJ + j) * w_step + v * 16;
+            dst[f][j][v] = (wok[f] && koff + lg * LB < p.kbytes) ? *reinterpret_cast<const v4i*>(wp[f] + off)
+                                                                  : (v4i){0, 0, 0, 0};
           }
     };
     auto load_a = [&](int chunk) {
@@ -388,7 +396,7 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
   KMOE_REQUIRE(a->act == KMOE_ACT_NONE || swiglu, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: act=%d unknown", a->act);
   KMOE_REQUIRE(a->n % (swiglu ? 32 : 16) == 0, KMOE_ERR_SHAPE, "grouped_gemm_i8: n=%d must be a multiple of %d",
                a->n, swiglu ? 32 : 16);
-  KMOE_REQUIRE(a->lda % 16 == 0 && a->lda >= a->k, KMOE_ERR_SHAPE,
+  KMOE_REQUIRE(a->a_layout == KMOE_A_CHUNKED || (a->lda % 16 == 0 && a->lda >= a->k), KMOE_ERR_SHAPE,
                "grouped_gemm_i8: lda=%lld must be a multiple of 16 and >= k", (long long)a->lda);
   const int n_out = swiglu ? a->n / 2 : a->n;
   KMOE_REQUIRE(a->ldy % 4 == 0 && a->ldy >= n_out, KMOE_ERR_SHAPE,
@@ -397,9 +405,20 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
                    aligned(a->acc_out, 16),
                KMOE_ERR_SHAPE, "grouped_gemm_i8: misaligned tensor pointer");
   KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_i8: src_div=%d < 1", a->src_div);
+  KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR || (a->w_layout == KMOE_W_TILED && a->k % 64 == 0), KMOE_ERR_SHAPE,
+               "grouped_gemm_i8: w_layout=%d (tiled weights need k %% 64 == 0, k=%d)", a->w_layout, a->k);
+  if (a->a_layout == KMOE_A_CHUNKED) {
+    KMOE_REQUIRE(a->w_layout == KMOE_W_TILED, KMOE_ERR_UNSUPPORTED,
+                 "grouped_gemm_i8: chunked activations need tiled weights");
+    KMOE_REQUIRE(a->a_rows >= 1, KMOE_ERR_SHAPE, "grouped_gemm_i8: a_rows=%d < 1", a->a_rows);
+    if (a->rows == 0) return KMOE_OK;
+    return stream_gemm_i8(a, as_stream(stream));
+  }
+  KMOE_REQUIRE(a->a_layout == KMOE_A_ROWMAJOR, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: a_layout=%d unknown",
+               a->a_layout);
   if (a->rows == 0) return KMOE_OK;
-  GemmParams p{a->a, a->lda, a->a_max, a->row_src, a->src_div, a->w,  a->w_max,
-               a->lod, a->E,  a->n,     a->k,       a->y,       a->ldy, a->acc_out};
+  GemmParams p{a->a,   a->lda, a->a_max, a->row_src, a->src_div, a->w,   a->w_max,
+               a->lod, a->E,   a->n,     a->k,       a->y,       a->ldy, a->acc_out, a->w_layout == KMOE_W_TILED};
   return dispatch<Kind::I8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_i8");
 }
 
@@ -424,7 +443,7 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
   if (a->rows == 0) return KMOE_OK;
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), nullptr,    a->lod,  a->E,       a->n,
-               a->k * 2,                              a->y,       a->ldy,  nullptr};
+               a->k * 2,                              a->y,       a->ldy,  nullptr, 0};
   return dispatch<Kind::BF16>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_bf16");
 }
 
@@ -450,6 +469,6 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
   if (a->rows == 0) return KMOE_OK;
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), a->w_scale, a->lod,  a->E,       a->n,
-               a->k,                                  a->y,       a->ldy,  nullptr};
+               a->k,                                  a->y,       a->ldy,  nullptr, 0};
   return dispatch<Kind::FP8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_fp8_block");
 }

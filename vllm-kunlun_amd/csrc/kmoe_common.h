@@ -14,6 +14,8 @@ int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
 // Writes {0, rows} to lod2: the row offsets of a dense (single-expert) GEMM.
 int fill_dense_lod(int32_t* lod2, int rows, hipStream_t stream);
+// Weight-streaming int8 GEMM (tiled weights, chunk-major activations); arguments already validated.
+int stream_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);
 
 #define KMOE_REQUIRE(cond, code, ...) \
   do {                                \

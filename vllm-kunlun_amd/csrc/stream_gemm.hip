@@ -1,0 +1,215 @@
+// Weight-streaming W8A8 grouped GEMM for the decode regime (a handful of rows
+// per expert): HBM-bound, every weight byte is read once, MFMA is ~5% busy.
+//
+// Both operands arrive already arranged for v_mfma_i32_16x16x64_i8, so a wave
+// needs no LDS, no barrier and no address arithmetic beyond a stride:
+//   weights  "tiled": [E][n/16][k/64] blocks of 1 KB; inside a block byte
+//            256*g + 16*c + t is channel c (of 16), k = 16*g + t (g = 0..3) —
+//            i.e. exactly what lane 16*g + c feeds the MFMA. A wave reads 1 KB
+//            of consecutive bytes per MFMA step and the next step's block follows
+//            directly: one long sequential stream per 16 output channels.
+//   activations "chunk-major": [k/16][rows][16 B]; lane (g, r) reads 16 bytes of
+//            row r at chunk 4*step + g. Rows of an expert are consecutive (down
+//            GEMM) or a gather inside a slab of a few KB (gate_up GEMM), so these
+//            reads hit the same few cache lines for every wave of the expert.
+// Each wave owns NF channel fragments and keeps D MFMA steps of loads in flight.
+#include "kmoe_common.h"
+
+namespace kmoe {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+struct StreamParams {
+  const int8_t* a;  // chunk-major [k/16][a_rows][16]
+  int32_t a_rows;
+  const float* a_max;
+  const int32_t* row_src;
+  int32_t src_div;
+  const int8_t* w;  // tiled
+  const float* w_max;
+  const int32_t* lod;
+  int32_t E, n, k;
+  uint16_t* y;
+  int64_t ldy;
+  int32_t* acc_out;
+};
+
+constexpr int kWaves = 4;
+
+template <int MF, int NF, bool SWIGLU, int D>
+__global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const StreamParams p) {
+  constexpr int NFH = SWIGLU ? NF / 2 : NF;
+  constexpr int TM = 16 * MF;
+  const int lane = lane_id();
+  const int wave = threadIdx.x >> 6;
+  const int li = lane & 15;
+  const int lg = lane >> 4;
+
+  const int e = blockIdx.y;
+  const int row_begin = p.lod[e];
+  const int row_end = p.lod[e + 1];
+  if (row_begin >= row_end) return;
+
+  const int n_half = SWIGLU ? p.n / 2 : p.n;
+  const int ksteps = p.k / 64;
+  const int col_base = (blockIdx.x * kWaves + wave) * NFH * 16;
+  if (col_base >= n_half) return;  // whole wave has nothing to do (no barriers in this kernel)
+
+  const int8_t* wp[NF];
+  bool wok[NF];
+  int col[NF];
+#pragma unroll
+  for (int f = 0; f < NF; ++f) {
+    const int fh = SWIGLU ? f % NFH : f;
+    const int c = col_base + fh * 16;
+    wok[f] = c < n_half;
+    col[f] = (SWIGLU && f >= NFH) ? n_half + c : c;
+    const size_t frag = static_cast<size_t>(e) * (p.n / 16) + (wok[f] ? col[f] / 16 : 0);
+    wp[f] = p.w + frag * ksteps * 1024 + lane * 16;
+  }
+  const size_t a_step = static_cast<size_t>(4) * p.a_rows * 16;  // bytes between MFMA steps
+
+  for (int row0 = row_begin; row0 < row_end; row0 += TM) {
+    const int8_t* ap[MF];
+    int srow[MF];
+#pragma unroll
+    for (int mf = 0; mf < MF; ++mf) {
+      const int r = row0 + mf * 16 + li;
+      srow[mf] = r < row_end ? (p.row_src ? p.row_src[r] / p.src_div : r) : -1;
+      // rows past the end read row 0: valid memory, results never stored
+      ap[mf] = p.a + (static_cast<size_t>(lg) * p.a_rows + (srow[mf] >= 0 ? srow[mf] : 0)) * 16;
+    }
+
+    v4i acc[MF][NF];
+#pragma unroll
+    for (int mf = 0; mf < MF; ++mf)
+#pragma unroll
+      for (int f = 0; f < NF; ++f) acc[mf][f] = (v4i){0, 0, 0, 0};
+
+    v4i wreg[D][NF];
+    v4i areg[D][MF];
+    auto load_step = [&](int slot, int kb) {
+#pragma unroll
+      for (int f = 0; f < NF; ++f)
+        wreg[slot][f] = wok[f] ? *reinterpret_cast<const v4i*>(wp[f] + static_cast<size_t>(kb) * 1024)
+                               : (v4i){0, 0, 0, 0};
+#pragma unroll
+      for (int mf = 0; mf < MF; ++mf) areg[slot][mf] = *reinterpret_cast<const v4i*>(ap[mf] + kb * a_step);
+    };
+
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+      if (d < ksteps) load_step(d, d);
+
+    for (int kb0 = 0; kb0 < ksteps; kb0 += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        const int kb = kb0 + d;
+        if (kb < ksteps) {
+#pragma unroll
+          for (int mf = 0; mf < MF; ++mf)
+#pragma unroll
+            for (int f = 0; f < NF; ++f)
+              acc[mf][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wreg[d][f], areg[d][mf], acc[mf][f], 0, 0, 0);
+          if (kb + D < ksteps) load_step(d, kb + D);
+        }
+      }
+    }
+
+#pragma unroll
+    for (int mf = 0; mf < MF; ++mf) {
+      const int r = row0 + mf * 16 + li;
+      if (r >= row_end) continue;
+      const float sa = p.a_max[srow[mf]] / 127.0f;
+#pragma unroll
+      for (int f = 0; f < NFH; ++f) {
+        if (!wok[f]) continue;
+        const int c0 = col[f] + lg * 4;
+        uint16_t yv[4];
+        auto finish = [&](const v4i& a, int cc, uint16_t(&out)[4]) {
+          const float4 wm = *reinterpret_cast<const float4*>(p.w_max + static_cast<size_t>(e) * p.n + cc);
+          const float sw[4] = {wm.x / 127.0f, wm.y / 127.0f, wm.z / 127.0f, wm.w / 127.0f};
+#pragma unroll
+          for (int q = 0; q < 4; ++q) out[q] = f32_to_bf16((static_cast<float>(a[q]) * sa) * sw[q]);
+          if (p.acc_out) *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + cc) = a;
+        };
+        finish(acc[mf][f], c0, yv);
+        if (SWIGLU) {
+          uint16_t uv[4];
+          finish(acc[mf][f + NFH], col[f + NFH] + lg * 4, uv);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) yv[q] = f32_to_bf16(silu_fixed(bf16_to_f32(yv[q])) * bf16_to_f32(uv[q]));
+        }
+        const uint2 packed = make_uint2(yv[0] | (static_cast<uint32_t>(yv[1]) << 16),
+                                        yv[2] | (static_cast<uint32_t>(yv[3]) << 16));
+        *reinterpret_cast<uint2*>(p.y + static_cast<size_t>(r) * p.ldy + c0) = packed;
+      }
+    }
+  }
+}
+
+template <int MF, int NF, bool SWIGLU, int D>
+int launch_stream(const StreamParams& p, hipStream_t s) {
+  constexpr int NFH = SWIGLU ? NF / 2 : NF;
+  const int n_half = SWIGLU ? p.n / 2 : p.n;
+  const dim3 grid(ceil_div(n_half, kWaves * NFH * 16), p.E);
+  hipLaunchKernelGGL((stream_gemm_i8_kernel<MF, NF, SWIGLU, D>), grid, dim3(kWaves * kWave), 0, s, p);
+  return check_launch("kmoe_grouped_gemm_i8 (stream)");
+}
+
+// [E][n][k] row-major -> tiled blocks; one thread moves 16 bytes.
+__global__ void tile_weights_kernel(const int8_t* __restrict__ src, int8_t* __restrict__ dst, int n, int k,
+                                    long long total_vec) {
+  const long long v = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (v >= total_vec) return;
+  const int ksteps = k / 64;
+  const int lane = static_cast<int>(v & 63);
+  const long long blk = v >> 6;  // (e * n/16 + nb) * ksteps + kb
+  const int kb = static_cast<int>(blk % ksteps);
+  const long long frag = blk / ksteps;  // e * n/16 + nb
+  const long long row = frag * 16 + (lane & 15);
+  const int kk = kb * 64 + (lane >> 4) * 16;
+  *reinterpret_cast<uint4*>(dst + v * 16) = *reinterpret_cast<const uint4*>(src + row * k + kk);
+}
+
+}  // namespace
+
+int stream_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
+  StreamParams p{a->a, a->a_rows, a->a_max, a->row_src, a->src_div, a->w, a->w_max,
+                 a->lod, a->E,     a->n,     a->k,       a->y,       a->ldy, a->acc_out};
+  const bool swiglu = a->act == KMOE_ACT_SWIGLU;
+  // m-fragments per pass from the rows an expert gets under uniform routing
+  int mf = a->variant;
+  if (mf == 0) {
+    const int avg = ceil_div(a->rows, a->E);
+    mf = avg <= 16 ? 1 : (avg <= 32 ? 2 : (avg <= 64 ? 4 : 8));
+  }
+  switch (mf) {
+    case 1:
+      return swiglu ? launch_stream<1, 2, true, 4>(p, s) : launch_stream<1, 2, false, 4>(p, s);
+    case 2:
+      return swiglu ? launch_stream<2, 2, true, 4>(p, s) : launch_stream<2, 2, false, 4>(p, s);
+    case 4:
+      return swiglu ? launch_stream<4, 2, true, 4>(p, s) : launch_stream<4, 2, false, 4>(p, s);
+    case 8:
+      return swiglu ? launch_stream<8, 2, true, 2>(p, s) : launch_stream<8, 2, false, 2>(p, s);
+    default:
+      return fail(KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8 (stream): variant=%d must be 0, 1, 2, 4 or 8", a->variant);
+  }
+}
+
+}  // namespace kmoe
+
+using namespace kmoe;
+
+extern "C" int kmoe_tile_weights_i8(const int8_t* src, int8_t* dst, int E, int n, int k, kmoe_stream_t stream) {
+  KMOE_REQUIRE(src && dst, KMOE_ERR_NULL, "tile_weights_i8: NULL pointer");
+  KMOE_REQUIRE(src != dst, KMOE_ERR_SHAPE, "tile_weights_i8: src and dst must differ (not an in-place transform)");
+  KMOE_REQUIRE(E >= 1 && n >= 16 && n % 16 == 0 && k >= 64 && k % 64 == 0, KMOE_ERR_SHAPE,
+               "tile_weights_i8: E=%d n=%d k=%d (need n %% 16 == 0, k %% 64 == 0)", E, n, k);
+  const long long total_vec = static_cast<long long>(E) * n * k / 16;
+  hipLaunchKernelGGL(tile_weights_kernel, dim3(static_cast<unsigned>((total_vec + 255) / 256)), dim3(256), 0,
+                     as_stream(stream), src, dst, n, k, total_vec);
+  return check_launch("kmoe_tile_weights_i8");
+}

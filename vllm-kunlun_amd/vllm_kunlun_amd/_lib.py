@@ -21,6 +21,8 @@ KMOE_SCORE_SIGMOID = 1
 KMOE_FMT_INT8 = 0
 KMOE_FMT_FP8_BLOCK = 1
 KMOE_FMT_BF16 = 2
+KMOE_W_ROWMAJOR, KMOE_W_TILED = 0, 1
+KMOE_A_ROWMAJOR, KMOE_A_CHUNKED = 0, 1
 STAGES = ("routing", "align", "quant1", "gemm1", "quant2", "gemm2", "shared", "combine")
 
 _ERR_KIND = {-1: ValueError, -2: ValueError, -3: NotImplementedError, -4: RuntimeError, -5: RuntimeError}
@@ -32,7 +34,7 @@ class GemmI8Args(C.Structure):
         ("src_div", C.c_int32), ("w", C.c_void_p), ("w_max", C.c_void_p), ("lod", C.c_void_p),
         ("E", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("rows", C.c_int32),
         ("y", C.c_void_p), ("ldy", C.c_int64), ("acc_out", C.c_void_p), ("act", C.c_int32),
-        ("variant", C.c_int32),
+        ("variant", C.c_int32), ("w_layout", C.c_int32), ("a_layout", C.c_int32), ("a_rows", C.c_int32),
     ]
 
 
@@ -62,14 +64,15 @@ class MoEArgs(C.Structure):
         ("x", C.c_void_p), ("w13", C.c_void_p), ("w13_max", C.c_void_p), ("w2", C.c_void_p), ("w2_max", C.c_void_p),
         ("I_shared", C.c_int32), ("ws13", C.c_void_p), ("ws13_max", C.c_void_p), ("ws2", C.c_void_p),
         ("ws2_max", C.c_void_p), ("out_scale", C.c_float), ("out", C.c_void_p),
-        ("stage_events", C.POINTER(C.c_void_p)),
+        ("stage_events", C.POINTER(C.c_void_p)), ("w_layout", C.c_int32),
     ]
 
 
 class MoELayout(C.Structure):
     _fields_ = [(n, C.c_size_t) for n in (
         "total_bytes", "topk_w", "topk_ids", "moe_index", "sorted_src", "expert_m", "lod", "align_ws",
-        "xq", "xmax", "act", "actq", "actmax", "down", "sh_lod", "sh_act", "sh_actq", "sh_actmax", "sh_out")]
+        "xq", "xmax", "act", "actq", "actmax", "down", "sh_lod", "sh_act", "sh_actq", "sh_actmax", "sh_out",
+        "codes_chunked")]
 
 
 def _load() -> C.CDLL:
@@ -89,6 +92,8 @@ def _load() -> C.CDLL:
         "kmoe_align": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, sz, vp]),
         "kmoe_gather_rows": (i32, [vp, i64, vp, i32, i32, i32, vp, i64, vp]),
         "kmoe_quant_i8_rows": (i32, [vp, i64, i32, i32, vp, i64, vp, vp]),
+        "kmoe_quant_i8_rows_chunked": (i32, [vp, i64, i32, i32, vp, vp, vp]),
+        "kmoe_tile_weights_i8": (i32, [vp, vp, i32, i32, i32, vp]),
         "kmoe_quant_fp8_group128": (i32, [vp, i64, i32, i32, vp, i64, vp, vp]),
         "kmoe_grouped_gemm_i8": (i32, [C.POINTER(GemmI8Args), vp]),
         "kmoe_silu_and_mul": (i32, [vp, i64, i32, i32, vp, i64, vp]),
@@ -108,7 +113,7 @@ def _load() -> C.CDLL:
 lib = _load()
 EXPORTS = (
     "kmoe_last_error", "kmoe_version", "kmoe_softmax_topk", "kmoe_sigmoid_group_topk_norm", "kmoe_block_statistic",
-    "kmoe_align_workspace_bytes", "kmoe_align", "kmoe_gather_rows", "kmoe_quant_i8_rows", "kmoe_quant_fp8_group128",
+    "kmoe_align_workspace_bytes", "kmoe_align", "kmoe_gather_rows", "kmoe_quant_i8_rows", "kmoe_quant_i8_rows_chunked", "kmoe_tile_weights_i8", "kmoe_quant_fp8_group128",
     "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
     "kmoe_moe_workspace_layout", "kmoe_moe_forward",
 )

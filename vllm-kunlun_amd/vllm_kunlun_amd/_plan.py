@@ -46,6 +46,42 @@ class MoEPlan:
         return self.workspace[off: off + nbytes].view(dtype)
 
 
+def is_tiled(w: torch.Tensor) -> bool:
+    """True if tile_int8_weights_ re-arranged this tensor. The mark lives on the tensor
+    (or Parameter) OBJECT: views and copies made afterwards do not carry it."""
+    return bool(getattr(w, "_kmoe_tiled", False))
+
+
+def tile_int8_weights_(w: torch.Tensor) -> bool:
+    """Re-arranges int8 weights [..., n, k] IN PLACE into the MFMA-ready 1 KB blocks of
+    kmoe_tile_weights_i8 (one expert at a time through a scratch copy) and marks the
+    object. Returns False and leaves the tensor alone when the shape does not allow it
+    (n % 16, k % 64)."""
+    data = w.data
+    n, k = data.shape[-2], data.shape[-1]
+    if data.dtype != torch.int8 or not data.is_cuda or not data.is_contiguous() or n % 16 or k % 64:
+        return False
+    if is_tiled(w):
+        return True
+    flat = data.view(-1, n, k)
+    tmp = torch.empty_like(flat[0])
+    for e in range(flat.shape[0]):
+        L.check(L.lib.kmoe_tile_weights_i8(L.ptr(flat[e]), L.ptr(tmp), 1, n, k, L.stream()))
+        flat[e].copy_(tmp)
+    w._kmoe_tiled = True
+    return True
+
+
+def rowmajor_int8_weights(w: torch.Tensor) -> torch.Tensor:
+    """A row-major [..., n, k] COPY of int8 weights, undoing tile_int8_weights_ if it was applied."""
+    if not is_tiled(w):
+        return w.data.clone()
+    n, k = w.shape[-2], w.shape[-1]
+    lead = w.shape[:-2]
+    t = w.data.reshape(-1, n // 16, k // 64, 4, 16, 16).permute(0, 1, 4, 2, 3, 5)
+    return t.reshape(*lead, n, k).contiguous()
+
+
 _WEIGHT_DTYPE = {L.KMOE_FMT_INT8: (torch.int8,), L.KMOE_FMT_FP8_BLOCK: (torch.float8_e4m3fn, torch.uint8),
                  L.KMOE_FMT_BF16: (torch.bfloat16,)}
 
@@ -55,7 +91,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
                   scoring_func: str = "softmax", renormalize: bool = True, num_expert_group: Optional[int] = None,
                   topk_group: Optional[int] = None, routed_scaling_factor: float = 1.0,
                   e_score_correction_bias: Optional[torch.Tensor] = None, shared_expert=None, out_scale: float = 1.0,
-                  stage_events=None) -> MoEPlan:
+                  stage_events=None, w_layout: Optional[int] = None) -> MoEPlan:
     """x bf16 [M,H], logits f32 [M,E], out bf16 [M,H]; w13 [E,2I,H], w2 [E,H,I] in the
     format's dtype; w13_aux/w2_aux: per-channel maxes (int8) or block scales (fp8), None for bf16.
     shared_expert: (ws13 [2Is,H], ws13_aux, ws2 [H,Is], ws2_aux) in the same format."""
@@ -100,6 +136,12 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
         keep.append(shared_expert)
     a.out_scale = float(out_scale)
     a.out = out.data_ptr()
+    if w_layout is None:  # tiled only if every int8 weight of the call has been tiled
+        ws_all = [w13, w2] + ([shared_expert[0], shared_expert[2]] if shared_expert is not None else [])
+        w_layout = L.KMOE_W_TILED if fmt == L.KMOE_FMT_INT8 and all(is_tiled(t) for t in ws_all) else L.KMOE_W_ROWMAJOR
+        if w_layout == L.KMOE_W_ROWMAJOR and any(is_tiled(t) for t in ws_all):
+            raise ValueError("moe plan: routed and shared expert weights must be either all tiled or all row-major")
+    a.w_layout = int(w_layout)
     if stage_events is not None:
         a.stage_events = stage_events
         keep.append(stage_events)

@@ -203,6 +203,7 @@ def scaled_int8_quant(x: torch.Tensor, scale: Optional[torch.Tensor], azp: Optio
 
 # ------------------------------------------------------------------------ GEMM
 def _gemm_i8(a, a_max, w, w_max, lod, y2d, ldy, act, rows, row_src=None, src_div=1, acc_out=None, variant=0):
+    from .._plan import is_tiled
     E, n, k = w.shape
     args = L.GemmI8Args()
     args.a = a.data_ptr()
@@ -219,6 +220,7 @@ def _gemm_i8(a, a_max, w, w_max, lod, y2d, ldy, act, rows, row_src=None, src_div
     args.acc_out = 0 if acc_out is None else acc_out.data_ptr()
     args.act = act
     args.variant = variant
+    args.w_layout = L.KMOE_W_TILED if is_tiled(w) else L.KMOE_W_ROWMAJOR
     L.check(L.lib.kmoe_grouped_gemm_i8(args, L.stream()))
 
 

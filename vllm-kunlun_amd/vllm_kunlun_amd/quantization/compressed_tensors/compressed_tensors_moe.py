@@ -17,7 +17,7 @@ from typing import Optional, Union
 import torch
 
 from ... import _lib as L
-from ..._plan import MoEPlan, make_moe_plan
+from ..._plan import MoEPlan, make_moe_plan, tile_int8_weights_
 from ...ops import _custom_ops  # noqa: F401  (torch.ops._C.* used by the staged path)
 
 WNA16_SUPPORTED_BITS = (4, 8)
@@ -179,10 +179,17 @@ class KunlunCompressedTensorsW8A8Int8MoEMethod(_MonolithicQuantMoE):
         layer.w2_weight_scale = mk(E, H, 1, dt=torch.float32)
 
     def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
-        """scale -> absmax: the kernels dequantise with max/127 (reference: :116-120)."""
+        """scale -> absmax: the kernels dequantise with max/127 (reference: :116-120).
+        On the GPU the int8 weights are also re-arranged in place into MFMA-ready blocks
+        (same values, same results; see kmoe_tile_weights_i8) when both shapes allow it."""
         with torch.no_grad():
             layer.w13_weight_scale.mul_(127.0)
             layer.w2_weight_scale.mul_(127.0)
+            w13, w2 = layer.w13_weight, layer.w2_weight
+            if (getattr(self, "tile_weights", True) and w13.is_cuda and w13.shape[-1] % 64 == 0
+                    and w2.shape[-1] % 64 == 0 and w13.shape[-2] % 16 == 0 and w2.shape[-2] % 16 == 0):
+                tile_int8_weights_(w13)
+                tile_int8_weights_(w2)
 
     def apply_staged(self, layer, x, router_logits, topk_group=None, num_expert_group=None, global_num_experts=-1,
                      scoring_func="softmax", routed_scaling_factor=1.0, e_score_correction_bias=None):

@@ -72,6 +72,23 @@ class SynthLayer:
     bias: Optional[torch.Tensor]    # [E] f32 (sigmoid routing)
     shared: Optional[tuple]         # (ws13 i8 [2Is,H], ws13_max f32 [2Is], ws2 i8 [H,Is], ws2_max f32 [H])
 
+    def host_weights(self):
+        """(w13, w13_aux, w2, w2_aux, shared) as host tensors in the reference's row-major
+        layout (int8 weights are un-tiled), for a CPU checker."""
+        from ._plan import rowmajor_int8_weights
+        lay = self.layer
+
+        def rm(t):
+            return (rowmajor_int8_weights(t) if t.dtype == torch.int8 else t).detach().cpu()
+
+        aux = lambda name: getattr(lay, name).detach().cpu() if hasattr(lay, name) else None  # noqa: E731
+        shared = None
+        if self.shared is not None:
+            shared = (rm(self.shared[0]), self.shared[1].detach().cpu(), rm(self.shared[2]),
+                      self.shared[3].detach().cpu())
+        return (rm(lay.w13_weight), aux("w13_weight_scale"), rm(lay.w2_weight), aux("w2_weight_scale"),
+                shared)
+
     def apply_kwargs(self) -> dict:
         s = self.shape
         kw = dict(scoring_func=s.scoring)
@@ -183,6 +200,10 @@ def make_w8a8_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer
         q13, s13 = _quant_rows_int8(torch.randn(2 * s.I_shared, s.H, generator=g, device=dev) * 0.02)
         q2, s2 = _quant_rows_int8(torch.randn(s.H, s.I_shared, generator=g, device=dev) * 0.02)
         shared = (q13, (s13 * 127.0).reshape(-1).contiguous(), q2, (s2 * 127.0).reshape(-1).contiguous())
+        from ._plan import is_tiled, tile_int8_weights_
+        if is_tiled(layer.w13_weight):  # the shared expert goes through the same load-time step
+            tile_int8_weights_(q13)
+            tile_int8_weights_(q2)
     x = torch.randn(s.M, s.H, generator=g, device=dev).to(torch.bfloat16)
     logits = torch.randn(s.M, s.E, generator=g, device=dev, dtype=torch.float32)
     if s.hot_experts:

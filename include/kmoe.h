@@ -177,6 +177,13 @@ typedef struct kmoe_gemm_i8_args {
   int32_t a_layout;       /* KMOE_A_ROWMAJOR, or KMOE_A_CHUNKED: a is [k/16][a_rows][16]
                              (kmoe_quant_i8_rows_chunked); needs w_layout TILED   */
   int32_t a_rows;         /* rows of the chunked activation array               */
+  /* Optional "tail expert": one more expert (e.g. a dense shared expert run in the
+     same launch) whose weights live outside w. Its rows are [tail_row0, tail_row0 +
+     tail_rows) — host values, not in lod — and row r of it reads activation row
+     tail_src0 + r - tail_row0 (row_src is not consulted). NULL w_tail: none.      */
+  const int8_t* w_tail;   /* [n, k], same layout as w                           */
+  const float* w_max_tail; /* [n]                                                */
+  int32_t tail_row0, tail_rows, tail_src0;
 } kmoe_gemm_i8_args;
 
 #define KMOE_W_ROWMAJOR 0
@@ -336,6 +343,9 @@ typedef struct kmoe_moe_args {
 #define KMOE_N_STAGES 8
 
 /* Byte offsets of the intermediates kmoe_moe_forward keeps in its workspace.
+ * An int8 shared expert as wide as the routed experts (I_shared == I) is run as
+ * one more expert of the routed launches: its rows are [P, P+M) of act / actq /
+ * actmax / down, and the sh_* slots stay empty.
  * xq/actq hold int8 or e4m3fn codes; xmax/actmax hold row maxes (INT8) or
  * per-128-column scales (FP8); all four are unused for BF16. */
 typedef struct kmoe_moe_layout {

@@ -36,7 +36,7 @@ def test_library_exports_every_declared_symbol(L):
 
 def test_struct_layouts_match_the_header(L):
     # sizes implied by the C declarations (LP64): guards the ctypes mirrors against drift
-    assert C.sizeof(L.GemmI8Args) == 8 * 8 + 16 + 8 * 3 + 8 + 16  # 8 ptr/int64, 4 int32, y/ldy/acc_out, act+variant, 3 int32 + pad
+    assert C.sizeof(L.GemmI8Args) == 8 * 8 + 16 + 8 * 3 + 8 + 16 + 16 + 16  # 8 ptr/int64, 4 int32, y/ldy/acc_out, act+variant, 3 int32 + pad
     assert C.sizeof(L.MoELayout) == 20 * 8
     a = L.MoEArgs()
     assert L.MoEArgs.M.offset == 0 and L.MoEArgs.logits.offset == 48 and C.sizeof(a) % 8 == 0

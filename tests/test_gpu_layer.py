@@ -50,6 +50,12 @@ SMALL = [
                                                    I_shared=256)),
     ("sigmoid-flat-shared", "kimi-decode", dict(M=16, H=256, E=48, K=8, I=64, I_shared=128)),
     ("single-token", "qwen3-decode", dict(M=1, H=256, E=8, K=2, I=64)),
+    ("shared-same-width-stream", "dsv3-decode", dict(M=40, H=512, E=32, K=4, I=128, n_group=4, topk_group=2,
+                                                     I_shared=128)),
+    ("shared-same-width-tiled-gemm", "dsv3-decode", dict(M=700, H=256, E=8, K=2, I=128, n_group=2, topk_group=1,
+                                                         I_shared=128)),
+    ("shared-same-width-rowmajor", "dsv3-decode", dict(M=50, H=272, E=8, K=2, I=80, n_group=2, topk_group=1,
+                                                       I_shared=80)),
 ]
 
 
@@ -71,10 +77,11 @@ def test_layer_matches_oracles(name, base, over):
     ids = _view(ws, lay.topk_ids, P, torch.int32).cpu().numpy().reshape(shape.M, shape.K)
     moe_index = _view(ws, lay.moe_index, P, torch.int32).cpu().numpy()
     lod = _view(ws, lay.lod, E + 1, torch.int32).cpu().numpy()
-    actq = _view(ws, lay.actq, P * I, torch.int8).cpu().numpy()
-    if lay.codes_chunked:  # [I/16][P][16] -> [P][I]
-        actq = actq.reshape(I // 16, P, 16).transpose(1, 0, 2)
-    actq = np.ascontiguousarray(actq).reshape(P, I)
+    R = P + (shape.M if shape.I_shared == I else 0)  # an equal-width shared expert adds rows [P, P+M)
+    actq = _view(ws, lay.actq, R * I, torch.int8).cpu().numpy()
+    if lay.codes_chunked:  # [I/16][R][16] -> [R][I]
+        actq = actq.reshape(I // 16, R, 16).transpose(1, 0, 2)
+    actq = np.ascontiguousarray(actq).reshape(R, I)[:P]
     topk_w = _view(ws, lay.topk_w, P, torch.float32).cpu().numpy().reshape(shape.M, shape.K)
     assert np.array_equal(ids, inter["topk_ids"]), "routing ids"
     assert np.array_equal(moe_index, inter["moe_index"]), "sorted token map"

@@ -60,6 +60,13 @@ bool use_stream_path(const kmoe_moe_args* a) {
   return a->format == KMOE_FMT_INT8 && a->w_layout == KMOE_W_TILED && (P + a->E - 1) / a->E <= 64 && a->M <= 1024;
 }
 
+// A shared expert of the routed experts' width runs inside the routed GEMM launches
+// as one more ("tail") expert over rows [P, P+M): no extra launches, and its few
+// workgroups overlap the routed experts' instead of leaving most CUs idle.
+bool fold_shared(const kmoe_moe_args* a) {
+  return a->format == KMOE_FMT_INT8 && a->I_shared > 0 && a->I_shared == a->I;
+}
+
 // One expert-MLP pass (gate_up + SiLU-mul, requantise, down) over `rows` rows in
 // the layer's format. `x_rows` is what the first GEMM reads: quantised codes, or
 // the bf16 activations themselves for KMOE_FMT_BF16.
@@ -80,6 +87,10 @@ struct MlpPass {
   int w_layout;    // INT8: KMOE_W_*
   bool stream;     // INT8 + tiled weights: chunk-major codes and the weight-streaming GEMM
   int x_count;     // rows of x_rows (chunk-major addressing)
+  // INT8 tail expert (folded shared expert): rows [rows, rows + tail_rows) of act/actq/out
+  const void *w13_tail, *w2_tail;
+  const float *w13_aux_tail, *w2_aux_tail;
+  int tail_rows;
 };
 
 int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
@@ -114,7 +125,14 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.w_layout = m.w_layout;
     if (m.stream) {
       g.a_layout = KMOE_A_CHUNKED;
-      g.a_rows = first ? m.x_count : m.rows;
+      g.a_rows = first ? m.x_count : m.rows + m.tail_rows;
+    }
+    if (m.tail_rows > 0) {
+      g.w_tail = static_cast<const int8_t*>(first ? m.w13_tail : m.w2_tail);
+      g.w_max_tail = first ? m.w13_aux_tail : m.w2_aux_tail;
+      g.tail_row0 = m.rows;
+      g.tail_rows = m.tail_rows;
+      g.tail_src0 = first ? 0 : m.rows;  // gate_up reads token rows, down reads its own act rows
     }
     return kmoe_grouped_gemm_i8(&g, stream);
   }
@@ -163,8 +181,9 @@ int run_mlp(const MlpPass& m, kmoe_stream_t stream, Mark&& mark) {
   mark(KMOE_STAGE_GEMM1, 1);
   mark(KMOE_STAGE_QUANT2, 0);
   if (m.format == KMOE_FMT_INT8) {
-    rc = m.stream ? kmoe_quant_i8_rows_chunked(m.act, m.I, m.rows, m.I, static_cast<int8_t*>(m.actq), m.act_aux, stream)
-                  : kmoe_quant_i8_rows(m.act, m.I, m.rows, m.I, static_cast<int8_t*>(m.actq), m.I, m.act_aux, stream);
+    const int qrows = m.rows + m.tail_rows;
+    rc = m.stream ? kmoe_quant_i8_rows_chunked(m.act, m.I, qrows, m.I, static_cast<int8_t*>(m.actq), m.act_aux, stream)
+                  : kmoe_quant_i8_rows(m.act, m.I, qrows, m.I, static_cast<int8_t*>(m.actq), m.I, m.act_aux, stream);
   } else if (m.format == KMOE_FMT_FP8_BLOCK) {
     rc = kmoe_quant_fp8_group128(m.act, m.I, m.rows, m.I, static_cast<uint8_t*>(m.actq), m.I, m.act_aux, stream);
   }
@@ -185,6 +204,9 @@ extern "C" int kmoe_moe_workspace_layout(const kmoe_moe_args* a, kmoe_moe_layout
   const size_t M = a->M, H = a->H, E = a->E, K = a->K, I = a->I, P = M * K, Is = a->I_shared;
   const bool quant = a->format != KMOE_FMT_BF16;
   const bool fp8 = a->format == KMOE_FMT_FP8_BLOCK;
+  const bool fold = fold_shared(a);
+  const size_t R = P + (fold ? M : 0);  // rows of the routed intermediates (+ folded shared expert rows)
+  const size_t Ms = fold ? 0 : (Is ? M : 0);  // rows of the separate shared-expert intermediates
   size_t off = 0;
   auto take = [&](size_t bytes) {
     const size_t at = off;
@@ -200,15 +222,15 @@ extern "C" int kmoe_moe_workspace_layout(const kmoe_moe_args* a, kmoe_moe_layout
   L->align_ws = take(kmoe_align_workspace_bytes(static_cast<int>(P), a->E));
   L->xq = take(quant ? M * H : 0);
   L->xmax = take(quant ? M * 4 * (fp8 ? H / 128 : 1) : 0);
-  L->act = take(P * I * 2);
-  L->actq = take(quant ? P * I : 0);
-  L->actmax = take(quant ? P * 4 * (fp8 ? I / 128 : 1) : 0);
-  L->down = take(P * H * 2);
+  L->act = take(R * I * 2);
+  L->actq = take(quant ? R * I : 0);
+  L->actmax = take(quant ? R * 4 * (fp8 ? I / 128 : 1) : 0);
+  L->down = take(R * H * 2);
   L->sh_lod = take(2 * 4);
-  L->sh_act = take(M * Is * 2);
-  L->sh_actq = take(quant ? M * Is : 0);
-  L->sh_actmax = take(quant ? M * 4 * (fp8 ? Is / 128 : 1) : 0);
-  L->sh_out = take(Is ? M * H * 2 : 0);
+  L->sh_act = take(Ms * Is * 2);
+  L->sh_actq = take(quant ? Ms * Is : 0);
+  L->sh_actmax = take(quant ? Ms * 4 * (fp8 ? Is / 128 : 1) : 0);
+  L->sh_out = take(Ms * H * 2);
   L->total_bytes = off;
   L->codes_chunked = use_stream_path(a) ? 1 : 0;
   return KMOE_OK;
@@ -304,17 +326,26 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   routed.w_layout = a->w_layout;
   routed.stream = stream_mode;
   routed.x_count = M;
+  const bool fold = fold_shared(a);
+  if (fold) {
+    routed.w13_tail = a->ws13;
+    routed.w2_tail = a->ws2;
+    routed.w13_aux_tail = a->ws13_max;
+    routed.w2_aux_tail = a->ws2_max;
+    routed.tail_rows = M;
+  }
   rc = run_mlp(routed, stream, mark);
   if (rc) return rc;
 
   // 7. dense shared expert on all M rows: the grouped GEMM with a single expert whose lod is {0, M}
   mark(KMOE_STAGE_SHARED, 0);
-  const uint16_t* shared_out = nullptr;
-  if (a->I_shared > 0) {
+  const uint16_t* shared_out = fold ? routed.out + static_cast<size_t>(P) * H : nullptr;
+  if (a->I_shared > 0 && !fold) {
     int32_t* dense_lod = static_cast<int32_t*>(at(L.sh_lod));
     rc = fill_dense_lod(dense_lod, M, as_stream(stream));
     if (rc) return rc;
     MlpPass sh = routed;
+    sh.tail_rows = 0;
     sh.row_src = nullptr;
     sh.src_div = 1;
     sh.w13 = a->ws13;

@@ -62,7 +62,16 @@ struct GemmParams {
   int64_t ldy;             // in elements
   int32_t* acc_out;        // I8 only
   int32_t w_tiled;         // weights in 64*LB-byte MFMA blocks [E][n/16][kbytes/(4*LB)] instead of row-major
+  const int8_t* w_tail;    // optional extra expert (index E): rows [tail_row0, tail_row0 + tail_rows), identity source
+  const float* w_max_tail;
+  int32_t tail_row0, tail_rows, tail_src0;
 };
+
+// Rows of expert e, with the tail expert (e == E) taken from the host-side range.
+__device__ inline int rows_begin(const GemmParams& p, int e) { return e < p.E ? p.lod[e] : p.tail_row0; }
+__device__ inline int rows_end(const GemmParams& p, int e) {
+  return e < p.E ? p.lod[e + 1] : p.tail_row0 + p.tail_rows;
+}
 
 __device__ inline int wave_incl_scan(int v) {
   const int lane = lane_id();
@@ -75,16 +84,17 @@ __device__ inline int wave_incl_scan(int v) {
 }
 
 // Finds the expert and first row of m-tile number `t` when every expert's rows
-// are cut into tiles of TM. Returns false when t is past the last tile.
+// (the tail expert included) are cut into tiles of TM. Returns false when t is past the last tile.
 template <int TM>
-__device__ inline bool locate_tile(const int32_t* __restrict__ lod, int E, int t, int& e_out, int& row0_out) {
+__device__ inline bool locate_tile(const GemmParams& p, int t, int& e_out, int& row0_out) {
   const int lane = lane_id();
+  const int E = p.E + (p.w_tail ? 1 : 0);
   const int epl = (E + kWave - 1) / kWave;
   const int e_begin = lane * epl;
   int local = 0;
   for (int i = 0; i < epl; ++i) {
     const int e = e_begin + i;
-    if (e < E) local += (lod[e + 1] - lod[e] + TM - 1) / TM;
+    if (e < E) local += (rows_end(p, e) - rows_begin(p, e) + TM - 1) / TM;
   }
   const int incl = wave_incl_scan(local);
   const int total = __shfl(incl, kWave - 1, kWave);
@@ -95,8 +105,8 @@ __device__ inline bool locate_tile(const int32_t* __restrict__ lod, int E, int t
     for (int i = 0; i < epl; ++i) {
       const int e = e_begin + i;
       if (e >= E) break;
-      const int lo = lod[e];
-      const int tiles = (lod[e + 1] - lo + TM - 1) / TM;
+      const int lo = rows_begin(p, e);
+      const int tiles = (rows_end(p, e) - lo + TM - 1) / TM;
       if (t < excl + tiles) {
         found_e = e;
         found_row = lo + (t - excl) * TM;
@@ -138,14 +148,17 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
 
   int e, row_begin, row_end;
   if (LOCATE) {
-    if (!locate_tile<TM>(p.lod, p.E, blockIdx.y, e, row_begin)) return;
-    row_end = min(p.lod[e + 1], row_begin + TM);
+    if (!locate_tile<TM>(p, blockIdx.y, e, row_begin)) return;
+    row_end = min(rows_end(p, e), row_begin + TM);
   } else {
     e = blockIdx.y;
-    row_begin = p.lod[e];
-    row_end = p.lod[e + 1];
+    row_begin = rows_begin(p, e);
+    row_end = rows_end(p, e);
     if (row_begin >= row_end) return;
   }
+  const bool tail = e >= p.E;
+  const int8_t* w_base = tail ? p.w_tail : p.w + static_cast<size_t>(e) * p.n * p.kbytes;
+  const float* w_aux = tail ? p.w_max_tail : p.w_max;  // I8: + e*n below; FP8: indexed with e
 
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int col_base = (blockIdx.x * WAVES + wave) * NFH * 16;
@@ -160,10 +173,10 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
     wok[f] = c < n_half;
     col[f] = (SWIGLU && f >= NFH) ? n_half + c : c;
     if (p.w_tiled) {  // block (fragment, step): 64*LB consecutive bytes, lane l at l*LB
-      const size_t frag = static_cast<size_t>(e) * (p.n / 16) + (wok[f] ? col[f] / 16 : 0);
-      wp[f] = p.w + frag * (p.kbytes / (4 * LB)) * (64 * LB) + lane * LB;
+      const size_t frag = wok[f] ? col[f] / 16 : 0;
+      wp[f] = w_base + frag * (p.kbytes / (4 * LB)) * (64 * LB) + lane * LB;
     } else {
-      wp[f] = p.w + (static_cast<size_t>(e) * p.n + (wok[f] ? col[f] + li : 0)) * p.kbytes + lg * LB;
+      wp[f] = w_base + static_cast<size_t>(wok[f] ? col[f] + li : 0) * p.kbytes + lg * LB;
     }
   }
   const int w_step = p.w_tiled ? 64 * LB : 4 * LB;  // bytes between consecutive MFMA steps of a fragment
@@ -183,7 +196,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
       a_lds[i] = (v < TM * 16) ? r * kPitch + kv * 16 : -1;
       ap[i] = nullptr;
       if (v < TM * 16 && row0 + r < row_end) {
-        const int sr = p.row_src ? p.row_src[row0 + r] / p.src_div : row0 + r;
+        const int sr = tail ? p.tail_src0 + row0 + r - p.tail_row0 : (p.row_src ? p.row_src[row0 + r] / p.src_div : row0 + r);
         ap[i] = p.a + static_cast<size_t>(sr) * p.lda + kv * 16;
       }
     }
@@ -192,7 +205,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
 #pragma unroll
     for (int mf = 0; mf < MF; ++mf) {
       const int r = row0 + mf * 16 + li;
-      srow[mf] = r < row_end ? (p.row_src ? p.row_src[r] / p.src_div : r) : -1;
+      srow[mf] = r < row_end ? (tail ? p.tail_src0 + r - p.tail_row0 : (p.row_src ? p.row_src[r] / p.src_div : r)) : -1;
     }
 
     acc_t acc[MF][NF];
@@ -318,7 +331,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
         uint16_t yv[4];
         auto finish = [&](const acc_t& a, int cc, uint16_t(&out)[4]) {
           if constexpr (KIND == Kind::I8) {
-            const float4 wm = *reinterpret_cast<const float4*>(p.w_max + static_cast<size_t>(e) * p.n + cc);
+            const float4 wm = *reinterpret_cast<const float4*>(w_aux + (tail ? 0 : static_cast<size_t>(e) * p.n) + cc);
             const float sw[4] = {wm.x / 127.0f, wm.y / 127.0f, wm.z / 127.0f, wm.w / 127.0f};
 #pragma unroll
             for (int q = 0; q < 4; ++q) out[q] = f32_to_bf16((static_cast<float>(a[q]) * sa) * sw[q]);
@@ -349,7 +362,8 @@ int launch(const GemmParams& p, int rows, hipStream_t s, const char* what) {
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int grid_x = ceil_div(n_half, WAVES * NFH * 16);
-  const int grid_y = LOCATE ? rows / TM + min(p.E, rows) : p.E;
+  const int n_exp = p.E + (p.w_tail ? 1 : 0);
+  const int grid_y = LOCATE ? (rows + p.tail_rows) / TM + min(n_exp, rows + p.tail_rows) : n_exp;
   if (grid_y == 0) return KMOE_OK;
   hipLaunchKernelGGL((grouped_gemm_kernel<KIND, MF, NF, WAVES, SWIGLU, LOCATE>), dim3(grid_x, grid_y),
                      dim3(WAVES * kWave), 0, s, p);
@@ -405,20 +419,25 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
                    aligned(a->acc_out, 16),
                KMOE_ERR_SHAPE, "grouped_gemm_i8: misaligned tensor pointer");
   KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_i8: src_div=%d < 1", a->src_div);
+  KMOE_REQUIRE(!a->w_tail || (a->w_max_tail && a->tail_rows >= 0 && a->tail_row0 >= 0 && aligned(a->w_tail, 16) &&
+                              aligned(a->w_max_tail, 16)),
+               KMOE_ERR_SHAPE, "grouped_gemm_i8: bad tail expert (w_max_tail, tail_row0=%d, tail_rows=%d)",
+               a->tail_row0, a->tail_rows);
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR || (a->w_layout == KMOE_W_TILED && a->k % 64 == 0), KMOE_ERR_SHAPE,
                "grouped_gemm_i8: w_layout=%d (tiled weights need k %% 64 == 0, k=%d)", a->w_layout, a->k);
   if (a->a_layout == KMOE_A_CHUNKED) {
     KMOE_REQUIRE(a->w_layout == KMOE_W_TILED, KMOE_ERR_UNSUPPORTED,
                  "grouped_gemm_i8: chunked activations need tiled weights");
     KMOE_REQUIRE(a->a_rows >= 1, KMOE_ERR_SHAPE, "grouped_gemm_i8: a_rows=%d < 1", a->a_rows);
-    if (a->rows == 0) return KMOE_OK;
+    if (a->rows == 0 && !(a->w_tail && a->tail_rows > 0)) return KMOE_OK;
     return stream_gemm_i8(a, as_stream(stream));
   }
   KMOE_REQUIRE(a->a_layout == KMOE_A_ROWMAJOR, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: a_layout=%d unknown",
                a->a_layout);
-  if (a->rows == 0) return KMOE_OK;
+  if (a->rows == 0 && !(a->w_tail && a->tail_rows > 0)) return KMOE_OK;
   GemmParams p{a->a,   a->lda, a->a_max, a->row_src, a->src_div, a->w,   a->w_max,
-               a->lod, a->E,   a->n,     a->k,       a->y,       a->ldy, a->acc_out, a->w_layout == KMOE_W_TILED};
+               a->lod, a->E,   a->n,     a->k,       a->y,       a->ldy, a->acc_out, a->w_layout == KMOE_W_TILED,
+               a->w_tail, a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0};
   return dispatch<Kind::I8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_i8");
 }
 
@@ -443,7 +462,7 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
   if (a->rows == 0) return KMOE_OK;
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), nullptr,    a->lod,  a->E,       a->n,
-               a->k * 2,                              a->y,       a->ldy,  nullptr, 0};
+               a->k * 2,                              a->y,       a->ldy,  nullptr, 0, nullptr, nullptr, 0, 0, 0};
   return dispatch<Kind::BF16>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_bf16");
 }
 
@@ -469,6 +488,6 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
   if (a->rows == 0) return KMOE_OK;
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), a->w_scale, a->lod,  a->E,       a->n,
-               a->k,                                  a->y,       a->ldy,  nullptr, 0};
+               a->k,                                  a->y,       a->ldy,  nullptr, 0, nullptr, nullptr, 0, 0, 0};
   return dispatch<Kind::FP8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_fp8_block");
 }

@@ -33,6 +33,9 @@ struct StreamParams {
   uint16_t* y;
   int64_t ldy;
   int32_t* acc_out;
+  const int8_t* w_tail;
+  const float* w_max_tail;
+  int32_t tail_row0, tail_rows, tail_src0;
 };
 
 constexpr int kWaves = 4;
@@ -46,10 +49,20 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
   const int li = lane & 15;
   const int lg = lane >> 4;
 
-  const int e = blockIdx.y;
-  const int row_begin = p.lod[e];
-  const int row_end = p.lod[e + 1];
+  // blockIdx.y < E: routed expert, all its rows. Beyond: one 16*MF-row slice of the tail expert.
+  const bool tail = static_cast<int>(blockIdx.y) >= p.E;
+  const int e = tail ? p.E : blockIdx.y;
+  int row_begin, row_end;
+  if (tail) {
+    row_begin = p.tail_row0 + (static_cast<int>(blockIdx.y) - p.E) * TM;
+    row_end = min(p.tail_row0 + p.tail_rows, row_begin + TM);
+  } else {
+    row_begin = p.lod[e];
+    row_end = p.lod[e + 1];
+  }
   if (row_begin >= row_end) return;
+  const int8_t* w_base = tail ? p.w_tail : p.w + static_cast<size_t>(e) * p.n * p.k;
+  const float* w_max = tail ? p.w_max_tail : p.w_max + static_cast<size_t>(e) * p.n;
 
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int ksteps = p.k / 64;
@@ -65,8 +78,8 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
     const int c = col_base + fh * 16;
     wok[f] = c < n_half;
     col[f] = (SWIGLU && f >= NFH) ? n_half + c : c;
-    const size_t frag = static_cast<size_t>(e) * (p.n / 16) + (wok[f] ? col[f] / 16 : 0);
-    wp[f] = p.w + frag * ksteps * 1024 + lane * 16;
+    const size_t frag = wok[f] ? col[f] / 16 : 0;
+    wp[f] = w_base + frag * ksteps * 1024 + lane * 16;
   }
   const size_t a_step = static_cast<size_t>(4) * p.a_rows * 16;  // bytes between MFMA steps
 
@@ -76,7 +89,7 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
 #pragma unroll
     for (int mf = 0; mf < MF; ++mf) {
       const int r = row0 + mf * 16 + li;
-      srow[mf] = r < row_end ? (p.row_src ? p.row_src[r] / p.src_div : r) : -1;
+      srow[mf] = r < row_end ? (tail ? p.tail_src0 + r - p.tail_row0 : (p.row_src ? p.row_src[r] / p.src_div : r)) : -1;
       // rows past the end read row 0: valid memory, results never stored
       ap[mf] = p.a + (static_cast<size_t>(lg) * p.a_rows + (srow[mf] >= 0 ? srow[mf] : 0)) * 16;
     }
@@ -128,7 +141,7 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
         const int c0 = col[f] + lg * 4;
         uint16_t yv[4];
         auto finish = [&](const v4i& a, int cc, uint16_t(&out)[4]) {
-          const float4 wm = *reinterpret_cast<const float4*>(p.w_max + static_cast<size_t>(e) * p.n + cc);
+          const float4 wm = *reinterpret_cast<const float4*>(w_max + cc);
           const float sw[4] = {wm.x / 127.0f, wm.y / 127.0f, wm.z / 127.0f, wm.w / 127.0f};
 #pragma unroll
           for (int q = 0; q < 4; ++q) out[q] = f32_to_bf16((static_cast<float>(a[q]) * sa) * sw[q]);
@@ -153,7 +166,7 @@ template <int MF, int NF, bool SWIGLU, int D>
 int launch_stream(const StreamParams& p, hipStream_t s) {
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
-  const dim3 grid(ceil_div(n_half, kWaves * NFH * 16), p.E);
+  const dim3 grid(ceil_div(n_half, kWaves * NFH * 16), p.E + (p.w_tail ? ceil_div(p.tail_rows, 16 * MF) : 0));
   hipLaunchKernelGGL((stream_gemm_i8_kernel<MF, NF, SWIGLU, D>), grid, dim3(kWaves * kWave), 0, s, p);
   return check_launch("kmoe_grouped_gemm_i8 (stream)");
 }
@@ -177,7 +190,8 @@ __global__ void tile_weights_kernel(const int8_t* __restrict__ src, int8_t* __re
 
 int stream_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   StreamParams p{a->a, a->a_rows, a->a_max, a->row_src, a->src_div, a->w, a->w_max,
-                 a->lod, a->E,     a->n,     a->k,       a->y,       a->ldy, a->acc_out};
+                 a->lod, a->E,     a->n,     a->k,       a->y,       a->ldy, a->acc_out,
+                 a->w_tail, a->w_max_tail, a->tail_row0, a->tail_rows, a->tail_src0};
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
   // m-fragments per pass from the rows an expert gets under uniform routing
   int mf = a->variant;

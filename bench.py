@@ -69,9 +69,12 @@ def algorithmic_work(shape, n_active):
     g1_bytes = n_active * (2 * I * H + 2 * I * 4) + M * H + M * 4 + P * 4 + P * I * 2
     g2_bytes = n_active * (H * I + H * 4) + P * I + P * 4 + P * H * 2
     shared_bytes = (3 * Is * H + (2 * Is + H) * 4) if Is else 0
+    if Is == I:  # the shared expert runs inside the two routed GEMM launches
+        g1_bytes += 2 * Is * H + 2 * Is * 4 + M * Is * 2
+        g2_bytes += H * Is + H * 4 + M * Is + M * H * 2
     layer_bytes = (n_active * (3 * I * H + (2 * I + H) * 4) + shared_bytes + 2 * M * H * 2 + M * E * 4)
-    g1_ops = 2 * P * 2 * I * H
-    g2_ops = 2 * P * H * I
+    g1_ops = 2 * (P + (M if Is == I else 0)) * 2 * I * H
+    g2_ops = 2 * (P + (M if Is == I else 0)) * H * I
     layer_ops = g1_ops + g2_ops + 2 * M * 3 * Is * H
     return dict(g1_bytes=g1_bytes, g2_bytes=g2_bytes, layer_bytes=layer_bytes, g1_ops=g1_ops, g2_ops=g2_ops,
                 layer_ops=layer_ops)

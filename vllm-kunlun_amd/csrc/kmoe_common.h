@@ -99,6 +99,41 @@ __device__ inline void wave_argmax(float& v, int& idx) {
   }
 }
 
+// ---- wave-wide arg-max on packed keys, over DPP (no LDS crossbar) ------------
+// A float maps to an unsigned int with the same order (-0 counts as +0); the key
+// is (ordered value << 32) | ~index, so the largest key is the largest value
+// and, among equal values, the lowest index. Key 0 means "no candidate".
+__device__ inline uint32_t ordered_bits(float v) {
+  union { float f; uint32_t u; } b;
+  b.f = v + 0.0f;
+  return (b.u & 0x80000000u) ? ~b.u : (b.u | 0x80000000u);
+}
+__device__ inline uint64_t arg_key(float v, int idx) {
+  return (static_cast<uint64_t>(ordered_bits(v)) << 32) | static_cast<uint32_t>(~static_cast<uint32_t>(idx));
+}
+__device__ inline int arg_key_index(uint64_t key) { return static_cast<int>(~static_cast<uint32_t>(key)); }
+
+template <int CTRL, int ROW_MASK>
+__device__ inline uint64_t dpp_max_step(uint64_t k) {
+  const uint32_t lo = static_cast<uint32_t>(k), hi = static_cast<uint32_t>(k >> 32);
+  const uint32_t olo = __builtin_amdgcn_update_dpp(lo, lo, CTRL, ROW_MASK, 0xf, false);
+  const uint32_t ohi = __builtin_amdgcn_update_dpp(hi, hi, CTRL, ROW_MASK, 0xf, false);
+  const uint64_t o = (static_cast<uint64_t>(ohi) << 32) | olo;
+  return o > k ? o : k;
+}
+// Max of a 64-bit key over the 64 lanes; every lane gets the result.
+__device__ inline uint64_t wave_max_u64(uint64_t k) {
+  k = dpp_max_step<0xB1, 0xf>(k);   // quad_perm [1,0,3,2]
+  k = dpp_max_step<0x4E, 0xf>(k);   // quad_perm [2,3,0,1]
+  k = dpp_max_step<0x141, 0xf>(k);  // row_half_mirror
+  k = dpp_max_step<0x140, 0xf>(k);  // row_mirror: every lane of a 16-lane row holds the row max
+  k = dpp_max_step<0x142, 0xa>(k);  // row_bcast15 into rows 1 and 3
+  k = dpp_max_step<0x143, 0xc>(k);  // row_bcast31 into rows 2 and 3: lane 63 holds the wave max
+  const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(k), 63);
+  const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(k >> 32), 63);
+  return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
 __device__ inline uint64_t lanemask_lt() {
   return (static_cast<uint64_t>(1) << lane_id()) - 1;
 }

@@ -9,26 +9,24 @@ constexpr int kMaxSlots = 16;  // E <= 1024
 constexpr int kWavesPerBlock = 4;
 
 // Picks the K best (score desc, expert id asc) entries of the row held as
-// score[s] (expert lane + 64*s); lanes k < K return the k-th winner.
+// score[s] (expert lane + 64*s); lane k < K returns the k-th winner in my_id.
 template <int SLOTS>
 __device__ inline void select_topk(const float (&score)[SLOTS], const bool (&eligible)[SLOTS], int K,
                                    int lane, int& my_id) {
-  unsigned taken = 0;
+  uint64_t key[SLOTS];
+#pragma unroll
+  for (int s = 0; s < SLOTS; ++s) key[s] = eligible[s] ? arg_key(score[s], lane + kWave * s) : 0;
   my_id = -1;
   for (int k = 0; k < K; ++k) {
-    float best = -__builtin_inff();
-    int best_id = 0x7fffffff;
+    uint64_t best = 0;
 #pragma unroll
-    for (int s = 0; s < SLOTS; ++s) {
-      const bool ok = eligible[s] && !((taken >> s) & 1u);
-      if (ok && (best_id == 0x7fffffff || score[s] > best)) {  // ascending id inside a lane
-        best = score[s];
-        best_id = lane + kWave * s;
-      }
-    }
-    wave_argmax(best, best_id);
-    if ((best_id & (kWave - 1)) == lane) taken |= 1u << (best_id >> 6);
-    if (lane == k) my_id = best_id;
+    for (int s = 0; s < SLOTS; ++s) best = key[s] > best ? key[s] : best;
+    best = wave_max_u64(best);
+    const int id = arg_key_index(best);
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s)
+      if (id == lane + kWave * s) key[s] = 0;  // taken
+    if (lane == k) my_id = id;
   }
 }
 
@@ -139,13 +137,11 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void sigmoid_group_topk_kern
       gscore = t1 + t2;
     }
     uint64_t keep = 0;
-    bool mine_taken = false;
+    uint64_t gkey = lane < n_group ? arg_key(gscore, lane) : 0;
     for (int t = 0; t < topk_group; ++t) {
-      float bv = (lane < n_group && !mine_taken) ? gscore : -__builtin_inff();
-      int bi = (lane < n_group && !mine_taken) ? lane : 0x7fffffff;
-      wave_argmax(bv, bi);
-      if (bi == lane) mine_taken = true;
-      keep |= static_cast<uint64_t>(1) << bi;
+      const int bi = arg_key_index(wave_max_u64(gkey));
+      if (bi == lane) gkey = 0;
+      keep |= static_cast<uint64_t>(1) << (bi & 63);
     }
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s) {

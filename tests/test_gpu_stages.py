@@ -400,8 +400,11 @@ def test_stream_gemm_i8(L, E, n, k, counts, variant, act, gather):
 
 
 @pytest.mark.parametrize("E,n,k,counts", TILED_CASES)
-@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("variant", [1, 2, 3, 5])
 @pytest.mark.parametrize("act", [0, 1])
 def test_lds_gemm_i8_with_tiled_weights(L, E, n, k, counts, variant, act):
-    """LDS-tiled kernel reading tiled weights and row-major activations."""
+    """LDS-staged kernels (variants 1-3: small tiles; 5: the 128x256-tile MFMA-bound kernel) reading
+    tiled weights and row-major activations."""
+    if variant == 5 and k % 128:
+        pytest.skip("the MFMA-bound kernel takes k % 128 == 0")
     _gemm_layout_case(L, E, n, k, counts, act, variant, True, chunked=False, seed=E * n + k + 7)

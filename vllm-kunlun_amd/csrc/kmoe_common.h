@@ -16,6 +16,8 @@ int check_launch(const char* what);
 int fill_dense_lod(int32_t* lod2, int rows, hipStream_t stream);
 // Weight-streaming int8 GEMM (tiled weights, chunk-major activations); arguments already validated.
 int stream_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);
+// MFMA-bound int8 GEMM on 128x512 tiles (tiled weights, row-major activations); arguments already validated.
+int tiled_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);
 
 #define KMOE_REQUIRE(cond, code, ...) \
   do {                                \
@@ -37,6 +39,15 @@ __host__ __device__ inline uint16_t f32_to_bf16(float f) {
   u += 0x7fffu + ((u >> 16) & 1u);
   return static_cast<uint16_t>(u >> 16);
 }
+
+// Device-only: the gfx950 conversion instruction (v_cvt_pk_bf16_f32, round to nearest
+// even) — same bits as f32_to_bf16 for every finite input, one instruction per pair.
+typedef float kmoe_v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 kmoe_v2bf __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t pack2_bf16(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((kmoe_v2f){lo, hi}, kmoe_v2bf));
+}
+__device__ inline uint16_t f32_to_bf16_hw(float f) { return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f)); }
 
 // ---- fixed-sequence transcendental -----------------------------------------
 // exp(x) as one fixed sequence of IEEE single operations (mul, round-to-even,

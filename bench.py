@@ -23,7 +23,6 @@ for _p in (ROOT, os.path.join(ROOT, "vllm-kunlun_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
-INT8_PEAK_TOPS = 5000.0    # MI355X dense int8 MFMA
 
 WORKLOAD_LABEL = {
     "qwen3-decode": "Qwen3-MoE-30B-A3B-shape MoE layer, W8A8 int8, decode, 64 tokens",
@@ -31,7 +30,14 @@ WORKLOAD_LABEL = {
     "qwen3-prefill-skew": "Qwen3-MoE-30B-A3B-shape MoE layer, W8A8 int8, prefill, 8192 tokens, +2.0 logit bias on 8 experts",
     "dsv3-decode": "DeepSeek-V3-shape MoE layer (+1 shared expert), W8A8 int8, decode, 128 tokens",
     "dsv3-prefill": "DeepSeek-V3-shape MoE layer (+1 shared expert), W8A8 int8, prefill, 4096 tokens",
+    "dsv3-fp8-decode": "DeepSeek-V3-shape MoE layer (+1 shared expert), fp8-e4m3 128x128-block weights, decode, 128 tokens",
+    "dsv3-fp8-prefill": "DeepSeek-V3-shape MoE layer (+1 shared expert), fp8-e4m3 128x128-block weights, prefill, 4096 tokens",
+    "kimi-fp8-decode": "Kimi-K2-shape MoE layer (384 experts, +1 shared), fp8-e4m3 128x128-block weights, decode, 128 tokens",
+    "kimi-fp8-prefill": "Kimi-K2-shape MoE layer (384 experts, +1 shared), fp8-e4m3 128x128-block weights, prefill, 4096 tokens",
+    "tiny-bf16": "tiny bf16 MoE layer (32 tokens, hidden 512, 8 experts, top-2, intermediate 256), no quantization",
 }
+PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0, "none": 2500.0}  # MI355X dense MFMA: int8, fp8, bf16
+DTYPE = {"int8": "int8", "fp8": "fp8_e4m3", "none": "bf16"}
 
 
 class HipEvents:
@@ -66,42 +72,72 @@ def algorithmic_work(shape, n_active):
     """Bytes that must cross HBM and int8 operations that must run, per layer call
     and for each GEMM launch, from the shape and the number of experts hit."""
     M, H, E, K, I, Is, P = shape.M, shape.H, shape.E, shape.K, shape.I, shape.I_shared, shape.P
-    g1_bytes = n_active * (2 * I * H + 2 * I * 4) + M * H + M * 4 + P * 4 + P * I * 2
-    g2_bytes = n_active * (H * I + H * 4) + P * I + P * 4 + P * H * 2
-    shared_bytes = (3 * Is * H + (2 * Is + H) * 4) if Is else 0
-    if Is == I:  # the shared expert runs inside the two routed GEMM launches
-        g1_bytes += 2 * Is * H + 2 * Is * 4 + M * Is * 2
-        g2_bytes += H * Is + H * 4 + M * Is + M * H * 2
-    layer_bytes = (n_active * (3 * I * H + (2 * I + H) * 4) + shared_bytes + 2 * M * H * 2 + M * E * 4)
-    g1_ops = 2 * (P + (M if Is == I else 0)) * 2 * I * H
-    g2_ops = 2 * (P + (M if Is == I else 0)) * H * I
+    wb = 2 if shape.quant == "none" else 1  # bytes per weight / activation code
+
+    def w_bytes(n, k):  # one [n,k] weight matrix with its scales
+        return n * k * wb + {"int8": n * 4, "fp8": (n // 128) * (k // 128) * 4, "none": 0}[shape.quant]
+
+    def a_bytes(rows, k):  # quantised activations of `rows` rows with their scales
+        return rows * k * wb + {"int8": rows * 4, "fp8": rows * (k // 128) * 4, "none": 0}[shape.quant]
+
+    g1_bytes = n_active * w_bytes(2 * I, H) + a_bytes(M, H) + P * 4 + P * I * 2
+    g2_bytes = n_active * w_bytes(H, I) + a_bytes(P, I) + P * H * 2
+    shared_bytes = (w_bytes(2 * Is, H) + w_bytes(H, Is)) if Is else 0
+    if Is == I and shape.quant == "int8":  # the shared expert runs inside the two routed GEMM launches
+        g1_bytes += w_bytes(2 * Is, H) + M * Is * 2
+        g2_bytes += w_bytes(H, Is) + a_bytes(M, Is) + M * H * 2
+    layer_bytes = (n_active * (w_bytes(2 * I, H) + w_bytes(H, I)) + shared_bytes + 2 * M * H * 2 + M * E * 4)
+    fold = M if (Is == I and shape.quant == "int8") else 0
+    g1_ops = 2 * (P + fold) * 2 * I * H
+    g2_ops = 2 * (P + fold) * H * I
     layer_ops = g1_ops + g2_ops + 2 * M * 3 * Is * H
     return dict(g1_bytes=g1_bytes, g2_bytes=g2_bytes, layer_bytes=layer_bytes, g1_ops=g1_ops, g2_ops=g2_ops,
                 layer_ops=layer_ops)
 
 
-def cpu_baseline(sl, budget_s=20.0):
+def measured_traffic(workload):
+    """HBM bytes per launch of the gate_up GEMM from the committed counter summary
+    (profiles/<workload>_gemm1_traffic.txt, line 'traffic_bytes_per_launch = N'), or None."""
+    path = os.path.join(ROOT, "profiles", f"{workload}_gemm1_traffic.txt")
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch"):
+                    return float(line.split("=")[1])
+    except OSError:
+        pass
+    return None
+
+
+def cpu_baseline(sl, budget_s=10.0):
     """The reference's torch expert loop (oracle/torch_moe.py) on the host cores."""
     import torch
     from oracle import torch_moe as tm
     s = sl.shape
     host = lambda t: None if t is None else t.detach().cpu()  # noqa: E731
     w13, w13_max, w2, w2_max, shared = sl.host_weights()  # row-major copies of the (tiled) device weights
-    args = (host(sl.x), host(sl.logits), w13, w13_max, w2, w2_max, s.K, s.scoring, True, s.n_group, s.topk_group,
-            s.routed_scale, host(sl.bias), shared)
+    if s.quant == "int8":
+        fn, what = tm.w8a8_moe, "torch-CPU restatement of the reference expert loop"
+        args = (host(sl.x), host(sl.logits), w13, w13_max, w2, w2_max, s.K, s.scoring, True, s.n_group, s.topk_group,
+                s.routed_scale, host(sl.bias), shared)
+    elif s.quant == "none":
+        fn, what = tm.bf16_moe, "torch-CPU restatement of the reference expert loop"
+        args = (host(sl.x), host(sl.logits), w13, w2, s.K, True)
+    else:
+        return None  # no CPU restatement of the fp8 layer is timed (the reference has no fp8 MoE path)
     t0 = time.perf_counter()
-    tm.w8a8_moe(*args)  # warm-up
+    fn(*args)  # warm-up
     first = time.perf_counter() - t0
-    runs = max(1, min(3, int(budget_s / max(first, 1e-3))))
+    runs = max(1, min(200, int(budget_s / max(first, 1e-3))))  # about budget_s seconds of CPU work
     times = []
     for _ in range(runs):
         t0 = time.perf_counter()
-        tm.w8a8_moe(*args)
+        fn(*args)
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
     return {"value": s.M / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"{runs} full layer call(s) of the same workload ({s.M} tokens) after 1 warm-up, median; "
-                      f"torch-CPU restatement of the reference expert loop; host has {os.cpu_count()} cpus"}
+                      f"{what}; host has {os.cpu_count()} cpus"}
 
 
 def main():
@@ -114,6 +150,9 @@ def main():
                     help="replay the layer from a captured HIP graph (as a serving engine does) or launch it eagerly")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (a kernel of known HBM traffic) before the "
+                         "timed region: the yardstick for FETCH_SIZE / WRITE_SIZE counter runs")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures ONE GPU; the layer does not span GPUs (run with --gpus 1)")
@@ -124,16 +163,21 @@ def main():
 
     torch.cuda.set_device(0)
     shape = synth.SHAPES[a.workload]
-    sl = synth.make_w8a8_layer(shape, "cuda:0", seed=a.seed)
-    method = sl.layer.quant_method
-    kw = sl.apply_kwargs()
+    from vllm_kunlun_amd._plan import make_moe_plan
+    sl = synth.make_layer(shape, "cuda:0", seed=a.seed)
+    lay = sl.layer
     x, logits = sl.x.contiguous(), sl.logits.contiguous()
     out = torch.empty_like(x)
-    plan_kw = dict(topk_group=kw.get("topk_group"), num_expert_group=kw.get("num_expert_group"),
-                   scoring_func=kw.get("scoring_func", "softmax"),
-                   routed_scaling_factor=kw.get("routed_scaling_factor", 1.0),
-                   e_score_correction_bias=kw.get("e_score_correction_bias"), shared_expert=kw.get("shared_expert"))
-    plan = method.make_plan(sl.layer, x, logits, out, **plan_kw)
+    fmt = {"int8": L.KMOE_FMT_INT8, "fp8": L.KMOE_FMT_FP8_BLOCK, "none": L.KMOE_FMT_BF16}[shape.quant]
+
+    def make_plan(stage_events=None):
+        # the argument block the plugin methods build (apply_monolithic / KunlunOps.fused_moe)
+        return make_moe_plan(fmt, x, logits, out, shape.K, lay.w13_weight, lay.w2_weight,
+                             getattr(lay, "w13_weight_scale", None), getattr(lay, "w2_weight_scale", None),
+                             shape.scoring, True, shape.n_group, shape.topk_group, shape.routed_scale, sl.bias,
+                             sl.shared, 1.0, stage_events)
+
+    plan = make_plan()
 
     # The layer, its inputs and the workspace were produced on the default stream;
     # finish that work before a second stream touches (recycled) memory.
@@ -141,6 +185,9 @@ def main():
     stream = torch.cuda.Stream()
     stream.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(stream):
+        if a.copy_probe:
+            src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0")
+            torch.empty_like(src).copy_(src)
         for _ in range(3):
             plan()
         stream.synchronize()
@@ -164,7 +211,7 @@ def main():
         # the same calls again with HIP events around each stage (eager: events are
         # not captured), for the per-kernel durations of the roofline
         ev = HipEvents(2 * len(L.STAGES))
-        plan_ev = method.make_plan(sl.layer, x, logits, out, stage_events=ev.handles, **plan_kw)
+        plan_ev = make_plan(ev.handles)
         stage_ms = {s: 0.0 for s in L.STAGES}
         for it in range(a.warmup + a.steps):
             plan_ev()
@@ -179,17 +226,20 @@ def main():
     n_active = int(((lod[1:] - lod[:-1]) > 0).sum())
     work = algorithmic_work(shape, n_active)
     intensity = work["layer_ops"] / work["layer_bytes"]
-    hbm_bound = intensity < INT8_PEAK_TOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+    peak_tops = PEAK_TOPS[shape.quant]
+    hbm_bound = intensity < peak_tops * 1e12 / (HBM_PEAK_GBS * 1e9)
     g1_s = stage_ms["gemm1"] * 1e-3
     if hbm_bound:
         achieved = work["g1_bytes"] / g1_s / 1e9
         roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": achieved / HBM_PEAK_GBS, "traffic": None}
+                    "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(a.workload)}
     else:
         achieved = work["g1_ops"] / g1_s / 1e12
-        roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s",
-                    "frac": achieved / INT8_PEAK_TOPS, "traffic": None}
-    roofline.update(kernel="grouped_gemm_kernel (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": peak_tops, "unit": "TFLOP/s",
+                    "frac": achieved / peak_tops, "traffic": measured_traffic(a.workload)}
+    g1_kernel = ("grouped_gemm_kernel" if shape.quant != "int8" else
+                 "stream_gemm_i8_kernel" if plan.layout.codes_chunked else "tiled_gemm_i8_kernel")
+    roofline.update(kernel=g1_kernel + " (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
                     algorithmic_bytes=work["g1_bytes"], algorithmic_ops=work["g1_ops"])
 
     t_s = ms_per_step * 1e-3
@@ -204,7 +254,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8",
+        "dtype": DTYPE[shape.quant],
         "data": "synthetic",
         "config": {"workload": WORKLOAD_LABEL[a.workload], "name": a.workload, "tokens": shape.M, "hidden": shape.H,
                    "experts": shape.E, "top_k": shape.K, "moe_intermediate": shape.I,
@@ -212,8 +262,8 @@ def main():
                    "launch": "hipgraph replay" if graph is not None else "eager", "seed": a.seed},
         "roofline": roofline,
         "layer": {"hbm_gbs": work["layer_bytes"] / t_s / 1e9, "hbm_frac": work["layer_bytes"] / t_s / 1e9 / HBM_PEAK_GBS,
-                  "int8_tops": work["layer_ops"] / t_s / 1e12,
-                  "mfma_frac": work["layer_ops"] / t_s / 1e12 / INT8_PEAK_TOPS,
+                  "tops": work["layer_ops"] / t_s / 1e12,
+                  "mfma_frac": work["layer_ops"] / t_s / 1e12 / peak_tops,
                   "algorithmic_bytes": work["layer_bytes"], "algorithmic_ops": work["layer_ops"],
                   "stage_ms": stage_ms},
     }

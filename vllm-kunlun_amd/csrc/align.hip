@@ -12,120 +12,131 @@
 namespace kmoe {
 namespace {
 
-constexpr int kThreads = 1024;
+constexpr int kThreads = 1024;            // workgroup size of the multi-workgroup kernels
 constexpr int kWaves = kThreads / kWave;  // 16
 constexpr int kMaxE = 1024;
 constexpr int kSingleMaxP = 8192;         // one workgroup handles up to this many pairs
 constexpr int kChunk = 2048;              // pairs per workgroup in the multi-workgroup path
 
+__device__ inline int key_bits(int E) { return 32 - __builtin_clz(max(E - 1, 1)); }
+
 // Rank of this lane among the lower lanes holding the same key, and the number
-// of lanes holding it. Lanes with key < 0 are idle.
-__device__ inline void wave_match_rank(int key, int& rank, int& count) {
-  rank = 0;
-  count = 0;
-  bool done = key < 0;
-  uint64_t pending = __ballot(!done);
-  while (pending) {
-    const int leader = __builtin_ctzll(pending);
-    const int lk = __shfl(key, leader, kWave);
-    const uint64_t same = __ballot(!done && key == lk);
-    if (!done && key == lk) {
-      rank = __builtin_popcountll(same & lanemask_lt());
-      count = __builtin_popcountll(same);
-      done = true;
-    }
-    pending &= ~same;
+// of lanes holding it. Lanes with key < 0 are idle. One ballot per key bit: the
+// lanes whose key agrees with mine on every bit are the lanes with my key.
+__device__ inline void wave_match_rank(int key, int bits, int& rank, int& count) {
+  const bool live = key >= 0;
+  uint64_t same = __ballot(live);
+  for (int b = 0; b < bits; ++b) {
+    const bool bit = (key >> b) & 1;
+    const uint64_t set = __ballot(live && bit);
+    same &= bit ? set : ~set;
   }
+  rank = live ? __builtin_popcountll(same & lanemask_lt()) : 0;
+  count = live ? __builtin_popcountll(same) : 0;
 }
 
-// Scatter phase for one chunk. `base[e]` (LDS) holds the sorted row at which
-// this chunk's first pair of expert e lands. `wcnt` is LDS scratch [kWaves][E].
-__device__ inline void scatter_chunk(const int32_t* __restrict__ ids, int begin, int end, int E,
-                                     int steps, int* base, int* wcnt, int32_t* __restrict__ moe_index,
-                                     int32_t* __restrict__ sorted_src) {
+__device__ inline int load_key(const int32_t* __restrict__ ids, int j, int end, int E) {
+  if (j >= end) return -1;
+  const int e = ids[j];
+  return static_cast<unsigned>(e) < static_cast<unsigned>(E) ? e : -1;  // ids outside [0,E): no sorted row
+}
+
+// Counting phase for one chunk: wave w owns pairs [begin + w*64*steps, +64*steps).
+// Leaves in wcnt[w][e] the number of expert-e pairs of this chunk in waves < w and
+// returns to thread e < E the chunk's total for expert e (0 to the other threads).
+// `wcnt` is LDS scratch [waves][E].
+__device__ inline int count_chunk(const int32_t* __restrict__ ids, int begin, int end, int E, int steps,
+                                  int* wcnt) {
+  const int waves = blockDim.x >> 6;
   const int wave = threadIdx.x >> 6;
   const int lane = lane_id();
+  const int bits = key_bits(E);
   const int wbegin = begin + wave * kWave * steps;
-  for (int i = threadIdx.x; i < kWaves * E; i += kThreads) wcnt[i] = 0;
-  __syncthreads();
-  // per-wave histogram of the wave's slice
-  for (int s = 0; s < steps; ++s) {
-    const int j = wbegin + s * kWave + lane;
-    if (j < end) {
-      const int e = ids[j];
-      if (static_cast<unsigned>(e) < static_cast<unsigned>(E)) atomicAdd(&wcnt[wave * E + e], 1);
-    }
-  }
-  __syncthreads();
-  // exclusive prefix over waves for each expert, offset by the chunk base
-  for (int e = threadIdx.x; e < E; e += kThreads) {
-    int run = base[e];
-    for (int w = 0; w < kWaves; ++w) {
-      const int c = wcnt[w * E + e];
-      wcnt[w * E + e] = run;
-      run += c;
-    }
-  }
+  for (int i = threadIdx.x; i < waves * E; i += blockDim.x) wcnt[i] = 0;
   __syncthreads();
   int* mine = wcnt + wave * E;
   for (int s = 0; s < steps; ++s) {
-    const int j = wbegin + s * kWave + lane;
-    int key = j < end ? ids[j] : -1;
-    if (key >= E) key = -1;  // ids outside [0,E) are skipped: no sorted row
+    const int key = load_key(ids, wbegin + s * kWave + lane, end, E);
     int rank, count;
-    wave_match_rank(key, rank, count);
+    wave_match_rank(key, bits, rank, count);
+    if (key >= 0 && rank == 0) mine[key] += count;  // one lane per distinct expert; a wave's LDS ops stay in order
+  }
+  __syncthreads();
+  int total = 0;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {  // at most one trip: blockDim.x >= E
+    for (int w = 0; w < waves; ++w) {
+      const int c = wcnt[w * E + e];
+      wcnt[w * E + e] = total;
+      total += c;
+    }
+  }
+  return total;
+}
+
+// Scatter phase: pair j of expert e lands at base[e] + wcnt[wave][e] + (rank among the
+// wave's earlier pairs of e). Call after count_chunk and a barrier that publishes base.
+__device__ inline void scatter_chunk(const int32_t* __restrict__ ids, int begin, int end, int E, int steps,
+                                     const int* base, int* wcnt, int32_t* __restrict__ moe_index,
+                                     int32_t* __restrict__ sorted_src) {
+  const int wave = threadIdx.x >> 6;
+  const int lane = lane_id();
+  const int bits = key_bits(E);
+  const int wbegin = begin + wave * kWave * steps;
+  int* mine = wcnt + wave * E;
+  for (int s = 0; s < steps; ++s) {
+    const int j = wbegin + s * kWave + lane;
+    const int key = load_key(ids, j, end, E);
+    int rank, count;
+    wave_match_rank(key, bits, rank, count);
     if (j < end && key < 0) moe_index[j] = -1;
     if (key >= 0) {
-      const int pos = mine[key] + rank;
+      const int pos = base[key] + mine[key] + rank;
       moe_index[j] = pos;
       if (sorted_src) sorted_src[pos] = j;
     }
     __builtin_amdgcn_wave_barrier();
-    if (key >= 0 && rank == 0) mine[key] += count;  // one lane per distinct expert
+    if (key >= 0 && rank == 0) mine[key] += count;
     __builtin_amdgcn_wave_barrier();
   }
 }
 
-// Exclusive scan of cnt[0..E) by one workgroup; writes lod[0..E] and expert_m.
-// `scan` is LDS scratch of kThreads ints. Leaves lod values also in out_base[e].
-__device__ inline void scan_experts(int my_count /* thread e < E */, int E, int* scan, int* out_base,
+// Exclusive scan of cnt[0..E) by one workgroup (blockDim.x >= E): a shuffle scan
+// inside each wave, then the wave totals through LDS. Writes lod[0..E] and
+// expert_m, and leaves lod[e] also in out_base[e]. `wtot` is LDS scratch of 16 ints.
+__device__ inline void scan_experts(int my_count /* thread e < E */, int E, int* wtot, int* out_base,
                                     int32_t* __restrict__ lod, int32_t* __restrict__ expert_m) {
   const int t = threadIdx.x;
-  scan[t] = t < E ? my_count : 0;
-  __syncthreads();
-  for (int off = 1; off < kThreads; off <<= 1) {  // Hillis-Steele inclusive scan
-    const int v = t >= off ? scan[t - off] : 0;
-    __syncthreads();
-    scan[t] += v;
-    __syncthreads();
+  const int lane = lane_id();
+  int incl = t < E ? my_count : 0;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int o = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += o;
   }
+  if (lane == kWave - 1) wtot[t >> 6] = incl;
+  __syncthreads();
+  int before = 0;
+  for (int w = 0; w < (t >> 6); ++w) before += wtot[w];
   if (t < E) {
-    const int excl = scan[t] - my_count;
+    const int excl = before + incl - my_count;
     out_base[t] = excl;
     lod[t] = excl;
     if (expert_m) expert_m[t] = my_count;
-    if (t == E - 1) lod[E] = scan[t];
+    if (t == E - 1) lod[E] = before + incl;
   }
   __syncthreads();
 }
 
+// Single-workgroup path (P <= kSingleMaxP); blockDim.x is 256 or 1024, >= E.
 __global__ __launch_bounds__(kThreads) void align_single_kernel(
     const int32_t* __restrict__ ids, int P, int E, int steps, int32_t* __restrict__ moe_index,
     int32_t* __restrict__ sorted_src, int32_t* __restrict__ expert_m, int32_t* __restrict__ lod) {
   extern __shared__ int lds[];
-  int* scan = lds;               // [kThreads]
-  int* base = scan + kThreads;   // [E]
-  int* wcnt = base + E;          // [kWaves][E]
-  for (int e = threadIdx.x; e < E; e += kThreads) base[e] = 0;
-  __syncthreads();
-  for (int j = threadIdx.x; j < P; j += kThreads) {
-    const int e = ids[j];
-    if (static_cast<unsigned>(e) < static_cast<unsigned>(E)) atomicAdd(&base[e], 1);
-  }
-  __syncthreads();
-  const int mine = threadIdx.x < E ? base[threadIdx.x] : 0;
-  __syncthreads();
-  scan_experts(mine, E, scan, base, lod, expert_m);
+  int* wtot = lds;          // [16]
+  int* base = wtot + 16;    // [E]
+  int* wcnt = base + E;     // [waves][E]
+  const int mine = count_chunk(ids, 0, P, E, steps, wcnt);
+  scan_experts(mine, E, wtot, base, lod, expert_m);
   scatter_chunk(ids, 0, P, E, steps, base, wcnt, moe_index, sorted_src);
 }
 
@@ -150,7 +161,7 @@ __global__ __launch_bounds__(kThreads) void align_hist_kernel(const int32_t* __r
 __global__ __launch_bounds__(kThreads) void align_scan_kernel(int E, int n_chunks, int32_t* __restrict__ hist,
                                                              int32_t* __restrict__ expert_m,
                                                              int32_t* __restrict__ lod) {
-  __shared__ int scan[kThreads];
+  __shared__ int scan[16];
   __shared__ int base[kMaxE];
   const int e = threadIdx.x;
   int total = 0;
@@ -177,9 +188,10 @@ __global__ __launch_bounds__(kThreads) void align_scatter_kernel(const int32_t* 
   int* base = lds;       // [E]
   int* wcnt = base + E;  // [kWaves][E]
   for (int e = threadIdx.x; e < E; e += kThreads) base[e] = hist[static_cast<size_t>(blockIdx.x) * E + e];
-  __syncthreads();
   const int begin = blockIdx.x * kChunk;
   const int end = min(P, begin + kChunk);
+  count_chunk(ids, begin, end, E, kChunk / kThreads, wcnt);
+  __syncthreads();
   scatter_chunk(ids, begin, end, E, kChunk / kThreads, base, wcnt, moe_index, sorted_src);
 }
 
@@ -226,9 +238,10 @@ extern "C" int kmoe_align(const int32_t* topk_ids, int P, int E, int32_t* moe_in
   KMOE_REQUIRE(P >= 0 && P <= (1 << 24), KMOE_ERR_SHAPE, "align: P=%d outside [0,2^24]", P);
   hipStream_t s = as_stream(stream);
   if (P <= kSingleMaxP) {
-    const int steps = max(1, ceil_div(P, kThreads));
-    const size_t lds = sizeof(int) * (kThreads + E + static_cast<size_t>(kWaves) * E);
-    hipLaunchKernelGGL(align_single_kernel, dim3(1), dim3(kThreads), lds, s, topk_ids, P, E, steps, moe_index,
+    const int threads = (E <= 256 && P <= 1024) ? 256 : kThreads;  // few waves: cheap barriers for decode sizes
+    const int steps = max(1, ceil_div(P, threads));
+    const size_t lds = sizeof(int) * (16 + E + static_cast<size_t>(threads / kWave) * E);
+    hipLaunchKernelGGL(align_single_kernel, dim3(1), dim3(threads), lds, s, topk_ids, P, E, steps, moe_index,
                        sorted_src, expert_m, lod);
     return check_launch("kmoe_align");
   }

@@ -50,6 +50,15 @@ SHAPES = {
     "kimi-decode": MoEShape("kimi-decode", 128, 7168, 384, 8, 2048, "sigmoid", 1, 1, 2.5, 2048),
     "kimi-prefill": MoEShape("kimi-prefill", 4096, 7168, 384, 8, 2048, "sigmoid", 1, 1, 2.5, 2048),
 }
+# the same layers with fp8-e4m3 block-scaled weights (128x128 blocks) and per-token-group activations
+for _n in ("dsv3-decode", "dsv3-prefill", "kimi-decode", "kimi-prefill"):
+    _f = _n.replace("-", "-fp8-")
+    SHAPES[_f] = replace(SHAPES[_n], name=_f, quant="fp8")
+
+
+def make_layer(shape: MoEShape, device="cuda", seed: int = 0) -> "SynthLayer":
+    """The synthetic layer of a shape in the format the shape names."""
+    return {"int8": make_w8a8_layer, "fp8": make_fp8_layer, "none": make_bf16_layer}[shape.quant](shape, device, seed)
 
 
 def scaled(shape: MoEShape, **kw) -> MoEShape:

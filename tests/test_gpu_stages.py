@@ -399,12 +399,25 @@ def test_stream_gemm_i8(L, E, n, k, counts, variant, act, gather):
     _gemm_layout_case(L, E, n, k, counts, act, variant, gather, chunked=True, seed=E * n + k)
 
 
-@pytest.mark.parametrize("E,n,k,counts", TILED_CASES)
-@pytest.mark.parametrize("variant", [1, 2, 3, 5])
+# more K lengths (1..7 chunks of 128: every remainder of both ring periods) and a case with more
+# work items than persistent workgroups (every workgroup walks several tiles, ragged experts)
+PERSISTENT_CASES = TILED_CASES + [
+    (2, 64, 128, [5, 131]),
+    (2, 96, 640, [140, 3]),
+    (3, 64, 896, [1, 260, 17]),
+    (64, 2048, 256, [((37 * i) % 290) for i in range(64)]),
+]
+
+
+@pytest.mark.parametrize("E,n,k,counts", PERSISTENT_CASES)
+@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 7])
 @pytest.mark.parametrize("act", [0, 1])
 def test_lds_gemm_i8_with_tiled_weights(L, E, n, k, counts, variant, act):
-    """LDS-staged kernels (variants 1-3: small tiles; 5: the 128x256-tile MFMA-bound kernel) reading
-    tiled weights and row-major activations."""
-    if variant == 5 and k % 128:
-        pytest.skip("the MFMA-bound kernel takes k % 128 == 0")
+    """LDS-staged kernels reading tiled weights and row-major activations. Variants 1-3: small
+    tiles; 5-7: the persistent 128-row-tile kernel (6: 256-channel tiles, 7: 128-channel tiles
+    with the deep weight ring, 5: the default of the two)."""
+    if variant >= 5 and k % 128:
+        pytest.skip("the persistent kernel takes k % 128 == 0")
+    if variant < 5 and E == 64:
+        pytest.skip("large case: persistent kernel only")
     _gemm_layout_case(L, E, n, k, counts, act, variant, True, chunked=False, seed=E * n + k + 7)

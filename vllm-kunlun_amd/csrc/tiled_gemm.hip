@@ -11,13 +11,19 @@
 //                every A fragment read from LDS feeds 4 MFMAs.
 //   weights:     straight from L2 into registers, 1 KB of consecutive bytes per
 //                fragment and MFMA step (tiled layout), through a ring of 4 step
-//                buffers loaded 3 MFMA steps (~1 us) ahead of use; every B fragment
+//                buffers loaded 3 MFMA steps ahead of use; every B fragment
 //                feeds 8 MFMAs. No weight byte goes through LDS.
-// Per CU and clock that is 64 B of LDS reads and 32 B of L2 reads against 8192
-// int8 operations.
-// Tiles are found from lod by a wave scan (no host-side work list, so routing skew
-// is balanced inside one launch), and workgroup ids are re-mapped so that the
-// tiles sharing an expert's weights run on the same XCD (one L2).
+// Workgroups are persistent: each walks a strided list of tiles. The tile after
+// the current one is located (from an LDS copy of lod) and its gather indices are
+// fetched while the current tile computes; its first activation chunk and weight
+// steps are requested BEFORE the current tile's epilogue, which hides their
+// latency. Per-row and per-channel scales of a tile wait in LDS, so the epilogue
+// touches global memory only to store. Output tiles are transposed through a
+// per-wave LDS patch so every store instruction writes whole 64/128-byte row
+// segments. Tile ids are mapped so that the tiles sharing an expert's weights run
+// at the same time on the same XCD (one L2).
+#include <type_traits>
+
 #include "kmoe_common.h"
 
 namespace kmoe {
@@ -35,14 +41,15 @@ __device__ inline v4i buffer_load16(__amdgpu_buffer_rsrc_t r, uint32_t lane_off,
   return (v4i)__builtin_amdgcn_raw_buffer_load_b128(r, lane_off, wave_off, 0);
 }
 
-constexpr int kMF = 8, kNF = 4, kWavesT = 4;
+constexpr int kMF = 8, kWavesT = 4;
 constexpr int kTM = 16 * kMF;              // 128 rows
 constexpr int kThreads = kWavesT * kWave;  // 256
 constexpr int kChunk = 128;                // bytes of K per row and chunk (2 MFMA steps)
 constexpr int kSteps = kChunk / 64;
 constexpr int kPitchT = kChunk + 32;       // 160 B: measured conflict-free for the b128 fragment reads (144 is not)
-constexpr int kGroupTiles = 4;              // consecutive m-tiles kept on one XCD
+constexpr int kGroupTiles = 4;             // consecutive m-tiles kept on one XCD
 constexpr int kNA = kTM * (kChunk / 16) / kThreads;  // 16-byte activation vectors per thread and chunk (= 4)
+constexpr int kMaxExperts = 1024 + 1;      // routed experts + the tail expert
 
 struct TiledParams {
   const int8_t* a;
@@ -60,139 +67,118 @@ struct TiledParams {
   const int8_t* w_tail;
   const float* w_max_tail;
   int32_t tail_row0, tail_rows, tail_src0;
-  int32_t n_blocks;   // channel blocks per tile
-  int32_t max_tiles;  // upper bound of m-tiles (grid = n_blocks * max_tiles, rounded up to 8)
+  int32_t n_blocks;  // channel blocks per tile
+  int32_t max_items; // upper bound of work items (n_blocks * bound of m-tiles): caps the grid
 };
 
-__device__ inline int t_rows_begin(const TiledParams& p, int e) { return e < p.E ? p.lod[e] : p.tail_row0; }
-__device__ inline int t_rows_end(const TiledParams& p, int e) {
-  return e < p.E ? p.lod[e + 1] : p.tail_row0 + p.tail_rows;
-}
+struct Tile {
+  int it;    // position in this workgroup's list
+  int e;     // expert (E = the tail expert)
+  int row0;  // first sorted row
+  int nb;    // channel block
+  bool valid;
+};
 
-__device__ inline int t_incl_scan(int v) {
-  const int lane = lane_id();
-#pragma unroll
-  for (int off = 1; off < kWave; off <<= 1) {
-    const int o = __shfl_up(v, off, kWave);
-    if (lane >= off) v += o;
-  }
-  return v;
-}
-
-__device__ inline bool t_locate(const TiledParams& p, int t, int& e_out, int& row0_out) {
-  const int lane = lane_id();
-  const int E = p.E + (p.w_tail ? 1 : 0);
-  const int epl = (E + kWave - 1) / kWave;
-  const int e_begin = lane * epl;
-  int local = 0;
-  for (int i = 0; i < epl; ++i) {
-    const int e = e_begin + i;
-    if (e < E) local += (t_rows_end(p, e) - t_rows_begin(p, e) + kTM - 1) / kTM;
-  }
-  const int incl = t_incl_scan(local);
-  const int total = __shfl(incl, kWave - 1, kWave);
-  if (t >= total) return false;
-  int excl = incl - local;
-  int found_e = -1, found_row = 0;
-  if (t >= excl && t < incl) {
-    for (int i = 0; i < epl; ++i) {
-      const int e = e_begin + i;
-      if (e >= E) break;
-      const int lo = t_rows_begin(p, e);
-      const int tiles = (t_rows_end(p, e) - lo + kTM - 1) / kTM;
-      if (t < excl + tiles) {
-        found_e = e;
-        found_row = lo + (t - excl) * kTM;
-        break;
-      }
-      excl += tiles;
-    }
-  }
-  const uint64_t who = __ballot(found_e >= 0);
-  const int src_lane = __builtin_ctzll(who);
-  e_out = __shfl(found_e, src_lane, kWave);
-  row0_out = __shfl(found_row, src_lane, kWave);
-  return true;
-}
-
-template <bool SWIGLU>
-__global__ __launch_bounds__(kThreads, 2) void tiled_gemm_i8_kernel(const TiledParams p) {
+// NF: 16-channel fragments per wave (4: 256-channel tiles, 2: 128-channel tiles);
+// R: weight ring slots (R - 1 MFMA steps of weights in flight per wave), 4 or 8;
+// WGS: workgroups per CU the register budget is cut for.
+// <4,4,2> is the shape in use; <2,8,3> trades operand reuse for more waves and more bytes
+// in flight (a tuning variant).
+template <bool SWIGLU, int NF, int R, int WGS>
+__global__ __launch_bounds__(kThreads, WGS) void tiled_gemm_i8_kernel(const TiledParams p) {
+  static_assert(R == 4 || R == 8, "the chunk buffer parity is static only for R/2 even");
+  constexpr int kNF = NF;
   constexpr int NFH = SWIGLU ? kNF / 2 : kNF;
+  constexpr int kOutBytes = NFH * 16 * 2;   // bytes of one output row owned by a wave: 32 .. 128
+  constexpr int kPatchPitch = kOutBytes + 16;  // bytes per row of a wave's output patch (16 rows)
   __shared__ __attribute__((aligned(16))) int8_t lds_a[2][kTM * kPitchT];
+  __shared__ __attribute__((aligned(16))) int8_t patch[kWavesT][16 * kPatchPitch];
+  __shared__ __attribute__((aligned(16))) float sw_lds[2][kWavesT * NF * 16];  // per tile parity: channel scales (w_max / 127)
+  __shared__ float sa_lds[2][kTM];                                              // per tile parity: row scales (a_max / 127)
+  extern __shared__ int dyn_lds[];
+  const int n_exp = p.E + (p.w_tail ? 1 : 0);
+  int* row_lo = dyn_lds;               // [E + 1]: lod
+  int* tile_lo = dyn_lds + p.E + 1;    // [n_exp + 1]: first m-tile of each expert, then the total
 
   const int lane = lane_id();
   const int wave = threadIdx.x >> 6;
   const int li = lane & 15;
   const int lg = lane >> 4;
-
-  // Workgroups are dealt round-robin to the 8 XCDs. Re-map ids so that a run of
-  // kGroupTiles consecutive tiles (about one expert: same weights) lands on ONE XCD
-  // and its L2, while successive runs still rotate over the XCDs (the empty tiles at
-  // the end of the list are then spread over all of them).
-  const int run = p.n_blocks * kGroupTiles;  // workgroups per run; gridDim.x is a multiple of 8 * run
-  const int xcd = blockIdx.x & 7;
-  const int j = blockIdx.x >> 3;             // index among this XCD's workgroups
-  const int lid = ((j / run) * 8 + xcd) * run + j % run;
-  const int tile = lid / p.n_blocks;
-  const int nb = lid - tile * p.n_blocks;
-  if (tile >= p.max_tiles) return;
-
-  int e, row0;
-  if (!t_locate(p, tile, e, row0)) return;
-  e = __builtin_amdgcn_readfirstlane(e);  // wave-uniform by construction; tell the compiler
-  row0 = __builtin_amdgcn_readfirstlane(row0);
-  const bool tail = e >= p.E;
-  const int row_end = min(t_rows_end(p, e), row0 + kTM);
-  const int8_t* w_base = tail ? p.w_tail : p.w + static_cast<size_t>(e) * p.n * p.k;
-  const float* w_max = tail ? p.w_max_tail : p.w_max + static_cast<size_t>(e) * p.n;
-
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int ksteps = p.k / 64;
   const int nchunks = ksteps / kSteps;  // the host only sends k % 128 == 0 here
-  const int col_base = (nb * kWavesT + wave) * NFH * 16;
+  const int last_step = ksteps - 1, last_chunk = nchunks - 1;
+  auto rows_begin = [&](int e) { return e < p.E ? row_lo[e] : p.tail_row0; };
+  auto rows_end = [&](int e) { return e < p.E ? row_lo[e + 1] : p.tail_row0 + p.tail_rows; };
 
-  // Weight fragment offsets (bytes from w_base) of this lane. Fragments past the last
-  // channel read fragment 0 instead (valid memory): their results are never stored.
-  bool wok[kNF];
-  int col[kNF];
-  uint32_t woff[kNF];
+  // ---- once per workgroup: rows and m-tiles of every expert into LDS ----
+  for (int e = threadIdx.x; e <= p.E; e += kThreads) row_lo[e] = p.lod[e];
+  __syncthreads();
+  if (wave == 0) {
+    int carry = 0;
+    for (int base = 0; base < n_exp; base += kWave) {
+      const int e = base + lane;
+      const int mine = e < n_exp ? (rows_end(e) - rows_begin(e) + kTM - 1) / kTM : 0;
+      int incl = mine;
 #pragma unroll
-  for (int f = 0; f < kNF; ++f) {
-    const int fh = SWIGLU ? f % NFH : f;
-    const int c = col_base + fh * 16;
-    wok[f] = c < n_half;
-    col[f] = (SWIGLU && f >= NFH) ? n_half + c : c;
-    woff[f] = static_cast<uint32_t>(wok[f] ? col[f] / 16 : 0) * ksteps * 1024u + lane * 16u;
+      for (int off = 1; off < kWave; off <<= 1) {
+        const int o = __shfl_up(incl, off, kWave);
+        if (lane >= off) incl += o;
+      }
+      if (e < n_exp) tile_lo[e] = carry + incl - mine;
+      carry += __shfl(incl, kWave - 1, kWave);
+    }
+    if (lane == 0) tile_lo[n_exp] = carry;
   }
+  __syncthreads();
+  const int total_tiles = tile_lo[n_exp];
 
-  // Activation slots of this thread in the LDS tile. Rows past the tile's end read
-  // the tile's first row (valid memory); their results are never stored.
+  // Work items = (m-tile, channel block) pairs, n_items of them, all non-empty; workgroup b
+  // takes items b, b + gridDim.x, ... so every workgroup gets the same count (+-1). Item ids
+  // are dealt to the 8 XCDs in runs: a run of kGroupTiles consecutive m-tiles (about one
+  // expert: same weights) with all their channel blocks is taken by workgroups of ONE XCD at
+  // about the same time, and successive runs rotate over the XCDs. The ids past the last
+  // whole round of 8 runs keep their natural order.
+  const int run = p.n_blocks * kGroupTiles;
+  const int n_items = total_tiles * p.n_blocks;
+  const int n_remapped = n_items / (8 * run) * (8 * run);
+  const int xcd = blockIdx.x & 7;
+  auto find_tile = [&](int it) -> Tile {
+    Tile t{it, 0, 0, 0, false};
+    const int q = blockIdx.x + it * gridDim.x;  // gridDim.x is a multiple of 8: the XCD stays
+    if (q >= n_items) return t;
+    const int j = q >> 3;
+    const int lid = q < n_remapped ? ((j / run) * 8 + xcd) * run + j % run : q;
+    const int m_tile = lid / p.n_blocks;
+    int found = -1;
+    for (int e = lane; e < n_exp; e += kWave)
+      if (tile_lo[e] <= m_tile && m_tile < tile_lo[e + 1]) found = e;
+    const uint64_t who = __ballot(found >= 0);  // exactly one lane
+    t.e = __builtin_amdgcn_readfirstlane(__shfl(found, __builtin_ctzll(who), kWave));
+    t.row0 = __builtin_amdgcn_readfirstlane(rows_begin(t.e) + (m_tile - tile_lo[t.e]) * kTM);
+    t.nb = lid - m_tile * p.n_blocks;
+    t.valid = true;
+    return t;
+  };
+
+  // ---- per-tile state of the loads ----
+  __amdgpu_buffer_rsrc_t w_rsrc;
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(p.a);
+  uint32_t woff[kNF];
   uint32_t aoff[kNA];
   int a_lds[kNA];
 #pragma unroll
   for (int i = 0; i < kNA; ++i) {
     const int v = threadIdx.x + i * kThreads;
-    const int r = v >> 3;  // 8 vectors of 16 B per row and chunk
-    const int kv = v & 7;
-    a_lds[i] = r * kPitchT + kv * 16;
-    const int rr = row0 + r < row_end ? row0 + r : row0;
-    const int sr = tail ? p.tail_src0 + rr - p.tail_row0 : (p.row_src ? p.row_src[rr] / p.src_div : rr);
-    aoff[i] = static_cast<uint32_t>(sr) * static_cast<uint32_t>(p.lda) + kv * 16;  // < 4 GiB: host-checked
+    a_lds[i] = (v >> 3) * kPitchT + (v & 7) * 16;  // row v/8, 16-byte vector v%8 of the chunk
   }
-  const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(w_base), a_rsrc = make_rsrc(p.a);
-
-  v4i acc[kMF][kNF];
-#pragma unroll
-  for (int mf = 0; mf < kMF; ++mf)
-#pragma unroll
-    for (int f = 0; f < kNF; ++f) acc[mf][f] = (v4i){0, 0, 0, 0};
-
-  v4i wring[4][kNF];  // weight fragments of MFMA step s live in slot s % 4
+  v4i wring[R][kNF];  // weight fragments of MFMA step s live in slot s % R
   v4i areg[kNA];
+  v4i acc[kMF][kNF];
 
-  // Every load below is unconditional (indices clamped to the last valid step / chunk),
-  // so the loop body is one basic block the scheduler can interleave freely.
-  const int last_step = ksteps - 1, last_chunk = nchunks - 1;
+  // Every load is unconditional (indices clamped to the last valid step / chunk, rows past a
+  // tile's end read its first row, fragments past the last channel read fragment 0): the
+  // results of those are never stored, and the loop body stays one basic block.
   auto load_w = [&](v4i(&dst)[kNF], int kb) {
     const uint32_t off = static_cast<uint32_t>(min(kb, last_step)) * 1024u;
 #pragma unroll
@@ -217,95 +203,208 @@ __global__ __launch_bounds__(kThreads, 2) void tiled_gemm_i8_kernel(const TiledP
         acc[mf][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wcur[f], af, acc[mf][f], 0, 0, 0);
     }
   };
+  // Gather index of sorted row r of tile t (rows past the expert's end: the tile's first row),
+  // and the source row (row of p.a / p.a_max) it names.
+  auto fetch_src = [&](const Tile& t, int r) -> int {
+    const int rr = r < rows_end(t.e) ? r : t.row0;
+    return (t.e < p.E && p.row_src) ? p.row_src[rr] : rr;
+  };
+  auto src_row = [&](const Tile& t, int fetched) -> int {
+    return t.e >= p.E ? p.tail_src0 + fetched - p.tail_row0 : (p.row_src ? fetched / p.src_div : fetched);
+  };
+  auto col_of = [&](const Tile& t, int f, bool& ok) -> int {
+    const int fh = SWIGLU ? f % NFH : f;
+    const int c = (t.nb * kWavesT + wave) * NFH * 16 + fh * 16;
+    ok = c < n_half;
+    return (SWIGLU && f >= NFH) ? n_half + c : c;
+  };
 
-  load_a(0);
-  load_w(wring[0], 0);
-  load_w(wring[1], 1);
-  load_w(wring[2], 2);
-  store_a(0);
-  __syncthreads();
-  int c = 0;
-  for (; c + 1 < nchunks; c += 2) {  // two chunks = four MFMA steps per iteration; k % 128 == 0
-    // The fences pin the issue order: loads leave at the START of the MFMA run that
-    // hides them, and each wait sits just before the first use (the counters retire in
-    // issue order, so a wait lets the later loads stay in flight).
-    const int s0 = c * kSteps;
-    load_a(c + 1);
-    load_w(wring[3], s0 + 3);
-    __builtin_amdgcn_sched_barrier(0);
-    compute(wring[0], 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    load_w(wring[0], s0 + 4);
-    __builtin_amdgcn_sched_barrier(0);
-    compute(wring[1], 0, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    store_a(1);
-    __syncthreads();
-    load_a(c + 2);
-    load_w(wring[1], s0 + 5);
-    __builtin_amdgcn_sched_barrier(0);
-    compute(wring[2], 1, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    load_w(wring[2], s0 + 6);
-    __builtin_amdgcn_sched_barrier(0);
-    compute(wring[3], 1, 1);
-    __builtin_amdgcn_sched_barrier(0);
+  Tile cur = find_tile(0);
+  if (!cur.valid) return;  // the whole workgroup leaves together
+  int rs[kNA];             // gather indices of this thread's activation rows
+#pragma unroll
+  for (int i = 0; i < kNA; ++i) rs[i] = fetch_src(cur, cur.row0 + ((threadIdx.x + i * kThreads) >> 3));
+  float sw_reg = 0.0f, sa_reg = 0.0f;  // this thread's share of the tile's scales, on their way to LDS
+
+  // Points the loaders at tile t and requests its first chunk, first three weight steps and scales.
+  auto start_tile = [&](const Tile& t) {
+    const int8_t* w_base = t.e >= p.E ? p.w_tail : p.w + static_cast<size_t>(t.e) * p.n * p.k;
+    const float* w_max = t.e >= p.E ? p.w_max_tail : p.w_max + static_cast<size_t>(t.e) * p.n;
+    w_rsrc = make_rsrc(w_base);
+#pragma unroll
+    for (int f = 0; f < kNF; ++f) {
+      bool ok;
+      const int c = col_of(t, f, ok);
+      woff[f] = static_cast<uint32_t>(ok ? c / 16 : 0) * ksteps * 1024u + lane * 16u;
+    }
+#pragma unroll
+    for (int i = 0; i < kNA; ++i)
+      aoff[i] = static_cast<uint32_t>(src_row(t, rs[i])) * static_cast<uint32_t>(p.lda) +
+                ((threadIdx.x + i * kThreads) & 7) * 16;  // < 4 GiB: host-checked
+    load_a(0);
+#pragma unroll
+    for (int i = 0; i < R - 1; ++i) load_w(wring[i], i);
+    if ((lane >> 4) < kNF) {  // thread (wave, f = lane / 16, c = lane % 16): scale of channel c of fragment f of this wave
+      bool ok;
+      const int c = col_of(t, lane >> 4, ok);
+      sw_reg = ok ? w_max[c + (lane & 15)] : 0.0f;
+    }
+    if (threadIdx.x < kTM)  // thread r: scale of tile row r
+      sa_reg = p.a_max[src_row(t, fetch_src(t, t.row0 + threadIdx.x))];
+  };
+  start_tile(cur);
+
+  for (int parity = 0;; parity ^= 1) {
+    // the tile after this one: found now, its gather indices travel during the MFMA loop
+    const Tile nxt = find_tile(cur.it + 1);
+    int rs_next[kNA];
+#pragma unroll
+    for (int i = 0; i < kNA; ++i)
+      rs_next[i] = nxt.valid ? fetch_src(nxt, nxt.row0 + ((threadIdx.x + i * kThreads) >> 3)) : 0;
+
+    if ((lane >> 4) < kNF) sw_lds[parity][wave * kNF * 16 + lane] = sw_reg / 127.0f;
+    if (threadIdx.x < kTM) sa_lds[parity][threadIdx.x] = sa_reg / 127.0f;
     store_a(0);
+#pragma unroll
+    for (int mf = 0; mf < kMF; ++mf)
+#pragma unroll
+      for (int f = 0; f < kNF; ++f) acc[mf][f] = (v4i){0, 0, 0, 0};
     __syncthreads();
-  }
-  if (c < nchunks) {  // odd number of chunks: the last one sits in buffer 0, slots 0 and 1
-    compute(wring[0], 0, 0);
-    compute(wring[1], 0, 1);
-  }
 
-  // ---- epilogue: dequantise, optional SiLU-mul, store ----
-  // per-channel scales once per fragment (not per row fragment): the 4 channels of this lane
-  float sw[kNF][4];
+    // One chunk (two MFMA steps) of the pipeline; h = position of the chunk in the ring
+    // period, c0 = first chunk of the period. The fences pin the issue order: loads leave at
+    // the START of the MFMA run that hides them, and each wait sits just before the first use
+    // (the counters retire in issue order, so a wait lets the later loads stay in flight).
+    auto chunk_step = [&](int c0, auto h_tag) {
+      constexpr int h = decltype(h_tag)::value;
+      constexpr int buf = h & 1;
+      const int s0 = (c0 + h) * kSteps;
+      load_a(c0 + h + 1);
+      load_w(wring[(2 * h + R - 1) % R], s0 + R - 1);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(wring[(2 * h) % R], buf, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      load_w(wring[(2 * h) % R], s0 + R);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(wring[(2 * h + 1) % R], buf, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      store_a(buf ^ 1);
+      __syncthreads();
+    };
+    int c = 0;
+    for (; c + R / 2 <= nchunks; c += R / 2) {  // one ring period = R MFMA steps per iteration
+      chunk_step(c, std::integral_constant<int, 0>{});
+      chunk_step(c, std::integral_constant<int, 1>{});
+      if constexpr (R == 8) {
+        chunk_step(c, std::integral_constant<int, 2>{});
+        chunk_step(c, std::integral_constant<int, 3>{});
+      }
+    }
+    // the chunks left over (fewer than a period): same steps, loads past the end are clamped
+    if (c < nchunks) chunk_step(c, std::integral_constant<int, 0>{});
+    if constexpr (R == 8) {
+      if (c + 1 < nchunks) chunk_step(c, std::integral_constant<int, 1>{});
+      if (c + 2 < nchunks) chunk_step(c, std::integral_constant<int, 2>{});
+    }
+
+    // ---- switch: request the next tile's first loads, then finish this tile ----
+    const Tile done = cur;
+    if (nxt.valid) {
 #pragma unroll
-  for (int f = 0; f < kNF; ++f) {
-    const float4 wm = wok[f] ? *reinterpret_cast<const float4*>(w_max + col[f] + lg * 4) : make_float4(0, 0, 0, 0);
-    sw[f][0] = wm.x / 127.0f;
-    sw[f][1] = wm.y / 127.0f;
-    sw[f][2] = wm.z / 127.0f;
-    sw[f][3] = wm.w / 127.0f;
-  }
+      for (int i = 0; i < kNA; ++i) rs[i] = rs_next[i];
+      cur = nxt;
+      start_tile(cur);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- epilogue of `done`: dequantise, optional SiLU-mul, transpose through LDS, store ----
+    const int row_end = min(rows_end(done.e), done.row0 + kTM);
+    bool wok[kNF];
+    int col[kNF];
+    float sw[kNF][4];
 #pragma unroll
-  for (int mf = 0; mf < kMF; ++mf) {
-    const int r = row0 + mf * 16 + li;
-    if (r >= row_end) continue;
-    const int sr = tail ? p.tail_src0 + r - p.tail_row0 : (p.row_src ? p.row_src[r] / p.src_div : r);
-    const float sa = p.a_max[sr] / 127.0f;
+    for (int f = 0; f < kNF; ++f) {
+      col[f] = col_of(done, f, wok[f]);
+      const float4 s4 = *reinterpret_cast<const float4*>(&sw_lds[parity][(wave * kNF + f) * 16 + lg * 4]);
+      sw[f][0] = s4.x;
+      sw[f][1] = s4.y;
+      sw[f][2] = s4.z;
+      sw[f][3] = s4.w;
+    }
+    int8_t* my_patch = patch[wave];
+    // reader side of the patch: lane -> (row, 16-byte vector), consecutive lanes cover a row
+    constexpr int kVecPerRow = kOutBytes / 16;        // 2, 4 or 8
+    constexpr int kRowsPerRead = kWave / kVecPerRow;  // 32 (half the lanes idle), 16 or 8
+    constexpr int kReads = kRowsPerRead >= 16 ? 1 : 16 / kRowsPerRead;
+    const int rd_row = lane / kVecPerRow, rd_vec = lane % kVecPerRow;
+    const int out_col0 = (done.nb * kWavesT + wave) * NFH * 16;  // first output channel of this wave
 #pragma unroll
-    for (int f = 0; f < NFH; ++f) {
-      if (!wok[f]) continue;
-      const int c0 = col[f] + lg * 4;
-      float yv[4];
+    for (int mf = 0; mf < kMF; ++mf) {
+      const float sa = sa_lds[parity][mf * 16 + li];
+      const int r = done.row0 + mf * 16 + li;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) yv[q] = (static_cast<float>(acc[mf][f][q]) * sa) * sw[f][q];
-      if (p.acc_out) *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + c0) = acc[mf][f];
-      if (SWIGLU) {
-        const int fu = f + NFH;
-        if (p.acc_out)
-          *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[fu] + lg * 4) = acc[mf][fu];
+      for (int f = 0; f < NFH; ++f) {
+        float yv[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const float g = bf16_to_f32(f32_to_bf16_hw(yv[q]));  // gate and up are bf16 values first
-          const float u = bf16_to_f32(f32_to_bf16_hw((static_cast<float>(acc[mf][fu][q]) * sa) * sw[fu][q]));
-          yv[q] = silu_fixed(g) * u;
+        for (int q = 0; q < 4; ++q) yv[q] = (static_cast<float>(acc[mf][f][q]) * sa) * sw[f][q];
+        if (SWIGLU) {
+          const int fu = f + NFH;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float g = bf16_to_f32(f32_to_bf16_hw(yv[q]));  // gate and up are bf16 values first
+            const float u = bf16_to_f32(f32_to_bf16_hw((static_cast<float>(acc[mf][fu][q]) * sa) * sw[fu][q]));
+            yv[q] = silu_fixed(g) * u;
+          }
+        }
+        *reinterpret_cast<uint2*>(&my_patch[li * kPatchPitch + f * 32 + lg * 8]) =
+            make_uint2(pack2_bf16(yv[0], yv[1]), pack2_bf16(yv[2], yv[3]));
+        if (p.acc_out && r < row_end && wok[f]) {
+          *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[f] + lg * 4) = acc[mf][f];
+          if (SWIGLU)
+            *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[f + NFH] + lg * 4) =
+                acc[mf][f + NFH];
         }
       }
-      *reinterpret_cast<uint2*>(p.y + static_cast<size_t>(r) * p.ldy + c0) =
-          make_uint2(pack2_bf16(yv[0], yv[1]), pack2_bf16(yv[2], yv[3]));
+      __builtin_amdgcn_wave_barrier();  // a wave's LDS operations execute in order: the reads see the writes
+#pragma unroll
+      for (int h = 0; h < kReads; ++h) {
+        const int pr = h * kRowsPerRead + rd_row;
+        const v4i v = *reinterpret_cast<const v4i*>(&my_patch[(pr & 15) * kPatchPitch + rd_vec * 16]);
+        const int orow = done.row0 + mf * 16 + pr;
+        const int ocol = out_col0 + rd_vec * 8;
+        if (pr < 16 && orow < row_end && ocol < n_half)  // n_half % 16 == 0: a vector of 8 channels is all in or all out
+          *reinterpret_cast<v4i*>(p.y + static_cast<size_t>(orow) * p.ldy + ocol) = v;
+      }
+      __builtin_amdgcn_wave_barrier();
     }
+    if (!nxt.valid) break;
   }
+}
+
+template <bool SWIGLU, int NF, int R, int WGS>
+int launch_tiled(const kmoe_gemm_i8_args* a, hipStream_t s, int n_cu) {
+  const int n_half = SWIGLU ? a->n / 2 : a->n;
+  const int nfh = SWIGLU ? NF / 2 : NF;
+  const int tail_rows = a->w_tail ? a->tail_rows : 0;
+  const int n_exp = a->E + (a->w_tail ? 1 : 0);
+  const int n_blocks = ceil_div(n_half, kWavesT * nfh * 16);
+  const int max_tiles = (a->rows + tail_rows) / kTM + min(n_exp, a->rows + tail_rows);
+  const int max_items = n_blocks * max_tiles;
+  TiledParams p{a->a,      a->lda,        a->a_max,      a->row_src, a->src_div,   a->w,         a->w_max, a->lod,
+                a->E,      a->n,          a->k,          a->y,       a->ldy,       a->acc_out,   a->w_tail,
+                a->w_max_tail, a->tail_row0, tail_rows,  a->tail_src0, n_blocks, max_items};
+  // persistent workgroups: WGS per CU
+  const int grid = min(ceil_div(max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8);
+  const size_t dyn = sizeof(int) * (static_cast<size_t>(a->E) + 1 + n_exp + 1);
+  hipLaunchKernelGGL((tiled_gemm_i8_kernel<SWIGLU, NF, R, WGS>), dim3(grid), dim3(kThreads), dyn, s, p);
+  return check_launch("kmoe_grouped_gemm_i8 (tiled)");
 }
 
 }  // namespace
 
+// variants 5, 6: 256-channel tiles, 4-slot weight ring; 7: 128-channel tiles, 8-slot ring, 3 workgroups per CU
 int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
-  const int n_half = swiglu ? a->n / 2 : a->n;
-  const int nfh = swiglu ? kNF / 2 : kNF;
   const int tail_rows = a->w_tail ? a->tail_rows : 0;
   const int n_exp = a->E + (a->w_tail ? 1 : 0);
   // 32-bit buffer offsets: one expert's weights and every source row of the activations
@@ -313,18 +412,24 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
                "grouped_gemm_i8 (tiled): n*k = %lld needs 32-bit offsets", static_cast<long long>(a->n) * a->k);
   KMOE_REQUIRE((static_cast<int64_t>(a->rows) + a->tail_src0 + tail_rows + 1) * a->lda < (1ll << 32), KMOE_ERR_SHAPE,
                "grouped_gemm_i8 (tiled): activations span more than 4 GiB");
-  TiledParams p{a->a,      a->lda,        a->a_max,      a->row_src, a->src_div,   a->w,         a->w_max, a->lod,
-                a->E,      a->n,          a->k,          a->y,       a->ldy,       a->acc_out,   a->w_tail,
-                a->w_max_tail, a->tail_row0, tail_rows,  a->tail_src0,
-                ceil_div(n_half, kWavesT * nfh * 16),
-                (a->rows + tail_rows) / kTM + min(n_exp, a->rows + tail_rows)};
-  const int grid = ceil_div(p.n_blocks * p.max_tiles, 8 * p.n_blocks * kGroupTiles) * 8 * p.n_blocks * kGroupTiles;
-  if (swiglu) {
-    hipLaunchKernelGGL((tiled_gemm_i8_kernel<true>), dim3(grid), dim3(kThreads), 0, s, p);
-  } else {
-    hipLaunchKernelGGL((tiled_gemm_i8_kernel<false>), dim3(grid), dim3(kThreads), 0, s, p);
+  KMOE_REQUIRE(n_exp <= kMaxExperts, KMOE_ERR_SHAPE, "grouped_gemm_i8 (tiled): E=%d > %d", a->E, kMaxExperts - 1);
+  KMOE_REQUIRE(a->ldy % 8 == 0 && reinterpret_cast<uintptr_t>(a->y) % 16 == 0, KMOE_ERR_SHAPE,
+               "grouped_gemm_i8 (tiled): y must be 16-byte aligned with ldy %% 8 == 0 (ldy=%lld)",
+               static_cast<long long>(a->ldy));
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+      return fail(KMOE_ERR_LAUNCH, "grouped_gemm_i8 (tiled): cannot query the device");
+    n_cu = prop.multiProcessorCount;
   }
-  return check_launch("kmoe_grouped_gemm_i8 (tiled)");
+  // The 128-channel / deep-ring shape is a tuning variant only: measured slower than the
+  // 256-channel shape also when an expert has ~128 rows (DeepSeek-V3 prefill at 4096 tokens),
+  // where HBM traffic, not bytes in flight, is the limit (twice the workgroups re-read A).
+  if (a->variant == 7)
+    return swiglu ? launch_tiled<true, 2, 8, 3>(a, s, n_cu) : launch_tiled<false, 2, 8, 3>(a, s, n_cu);
+  return swiglu ? launch_tiled<true, 4, 4, 2>(a, s, n_cu) : launch_tiled<false, 4, 4, 2>(a, s, n_cu);
 }
 
 }  // namespace kmoe

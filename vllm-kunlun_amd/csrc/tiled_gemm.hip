@@ -41,14 +41,12 @@ __device__ inline v4i buffer_load16(__amdgpu_buffer_rsrc_t r, uint32_t lane_off,
   return (v4i)__builtin_amdgcn_raw_buffer_load_b128(r, lane_off, wave_off, 0);
 }
 
-constexpr int kMF = 8, kWavesT = 4;
-constexpr int kTM = 16 * kMF;              // 128 rows
-constexpr int kThreads = kWavesT * kWave;  // 256
+constexpr int kMF = 8, kWavesT = 4;        // a wave: 8 row fragments (128 rows); 4 waves side by side along the channels
 constexpr int kChunk = 128;                // bytes of K per row and chunk (2 MFMA steps)
 constexpr int kSteps = kChunk / 64;
 constexpr int kPitchT = kChunk + 32;       // 160 B: measured conflict-free for the b128 fragment reads (144 is not)
 constexpr int kGroupTiles = 4;             // consecutive m-tiles kept on one XCD
-constexpr int kNA = kTM * (kChunk / 16) / kThreads;  // 16-byte activation vectors per thread and chunk (= 4)
+constexpr int kNA = 16 * kMF * (kChunk / 16) / (kWavesT * kWave);  // 16-byte activation vectors per thread and chunk (= 4)
 constexpr int kMaxExperts = 1024 + 1;      // routed experts + the tail expert
 
 struct TiledParams {
@@ -84,15 +82,20 @@ struct Tile {
 // WGS: workgroups per CU the register budget is cut for.
 // <4,4,2> is the shape in use; <2,8,3> trades operand reuse for more waves and more bytes
 // in flight (a tuning variant).
-template <bool SWIGLU, int NF, int R, int WGS>
-__global__ __launch_bounds__(kThreads, WGS) void tiled_gemm_i8_kernel(const TiledParams p) {
+// WM: rows of waves. 1: 128-row tiles, 4 waves; 2: 256-row tiles, 8 waves, where the two waves
+// that share channels read the same weight bytes within one barrier interval (an expert with
+// up to 256 rows then streams its weights from HBM once).
+template <bool SWIGLU, int NF, int R, int WGS, int WM>
+__global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kernel(const TiledParams p) {
+  constexpr int kTM = WM * 16 * kMF;             // rows of a tile
+  constexpr int kThreads = WM * kWavesT * kWave;
   static_assert(R == 4 || R == 8, "the chunk buffer parity is static only for R/2 even");
   constexpr int kNF = NF;
   constexpr int NFH = SWIGLU ? kNF / 2 : kNF;
   constexpr int kOutBytes = NFH * 16 * 2;   // bytes of one output row owned by a wave: 32 .. 128
   constexpr int kPatchPitch = kOutBytes + 16;  // bytes per row of a wave's output patch (16 rows)
   __shared__ __attribute__((aligned(16))) int8_t lds_a[2][kTM * kPitchT];
-  __shared__ __attribute__((aligned(16))) int8_t patch[kWavesT][16 * kPatchPitch];
+  __shared__ __attribute__((aligned(16))) int8_t patch[WM * kWavesT][16 * kPatchPitch];
   __shared__ __attribute__((aligned(16))) float sw_lds[2][kWavesT * NF * 16];  // per tile parity: channel scales (w_max / 127)
   __shared__ float sa_lds[2][kTM];                                              // per tile parity: row scales (a_max / 127)
   extern __shared__ int dyn_lds[];
@@ -101,7 +104,9 @@ __global__ __launch_bounds__(kThreads, WGS) void tiled_gemm_i8_kernel(const Tile
   int* tile_lo = dyn_lds + p.E + 1;    // [n_exp + 1]: first m-tile of each expert, then the total
 
   const int lane = lane_id();
-  const int wave = threadIdx.x >> 6;
+  const int wave_id = threadIdx.x >> 6;
+  const int wave = WM == 1 ? wave_id : wave_id % kWavesT;  // position along the channels
+  const int wave_m = WM == 1 ? 0 : wave_id / kWavesT;      // position along the rows
   const int li = lane & 15;
   const int lg = lane >> 4;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
@@ -114,7 +119,7 @@ __global__ __launch_bounds__(kThreads, WGS) void tiled_gemm_i8_kernel(const Tile
   // ---- once per workgroup: rows and m-tiles of every expert into LDS ----
   for (int e = threadIdx.x; e <= p.E; e += kThreads) row_lo[e] = p.lod[e];
   __syncthreads();
-  if (wave == 0) {
+  if (wave_id == 0) {
     int carry = 0;
     for (int base = 0; base < n_exp; base += kWave) {
       const int e = base + lane;
@@ -197,7 +202,7 @@ __global__ __launch_bounds__(kThreads, WGS) void tiled_gemm_i8_kernel(const Tile
   auto compute = [&](const v4i(&wcur)[kNF], int buf, int j) {
 #pragma unroll
     for (int mf = 0; mf < kMF; ++mf) {
-      const v4i af = *reinterpret_cast<const v4i*>(&lds_a[buf][(mf * 16 + li) * kPitchT + j * 64 + lg * 16]);
+      const v4i af = *reinterpret_cast<const v4i*>(&lds_a[buf][(wave_m * 16 * kMF + mf * 16 + li) * kPitchT + j * 64 + lg * 16]);
 #pragma unroll
       for (int f = 0; f < kNF; ++f)
         acc[mf][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wcur[f], af, acc[mf][f], 0, 0, 0);
@@ -244,7 +249,7 @@ __global__ __launch_bounds__(kThreads, WGS) void tiled_gemm_i8_kernel(const Tile
     load_a(0);
 #pragma unroll
     for (int i = 0; i < R - 1; ++i) load_w(wring[i], i);
-    if ((lane >> 4) < kNF) {  // thread (wave, f = lane / 16, c = lane % 16): scale of channel c of fragment f of this wave
+    if (wave_m == 0 && (lane >> 4) < kNF) {  // thread (wave, f = lane / 16, c = lane % 16): scale of channel c of fragment f of this wave
       bool ok;
       const int c = col_of(t, lane >> 4, ok);
       sw_reg = ok ? w_max[c + (lane & 15)] : 0.0f;
@@ -262,7 +267,7 @@ __global__ __launch_bounds__(kThreads, WGS) void tiled_gemm_i8_kernel(const Tile
     for (int i = 0; i < kNA; ++i)
       rs_next[i] = nxt.valid ? fetch_src(nxt, nxt.row0 + ((threadIdx.x + i * kThreads) >> 3)) : 0;
 
-    if ((lane >> 4) < kNF) sw_lds[parity][wave * kNF * 16 + lane] = sw_reg / 127.0f;
+    if (wave_m == 0 && (lane >> 4) < kNF) sw_lds[parity][wave * kNF * 16 + lane] = sw_reg / 127.0f;
     if (threadIdx.x < kTM) sa_lds[parity][threadIdx.x] = sa_reg / 127.0f;
     store_a(0);
 #pragma unroll
@@ -331,7 +336,7 @@ __global__ __launch_bounds__(kThreads, WGS) void tiled_gemm_i8_kernel(const Tile
       sw[f][2] = s4.z;
       sw[f][3] = s4.w;
     }
-    int8_t* my_patch = patch[wave];
+    int8_t* my_patch = patch[wave_id];
     // reader side of the patch: lane -> (row, 16-byte vector), consecutive lanes cover a row
     constexpr int kVecPerRow = kOutBytes / 16;        // 2, 4 or 8
     constexpr int kRowsPerRead = kWave / kVecPerRow;  // 32 (half the lanes idle), 16 or 8
@@ -340,8 +345,8 @@ __global__ __launch_bounds__(kThreads, WGS) void tiled_gemm_i8_kernel(const Tile
     const int out_col0 = (done.nb * kWavesT + wave) * NFH * 16;  // first output channel of this wave
 #pragma unroll
     for (int mf = 0; mf < kMF; ++mf) {
-      const float sa = sa_lds[parity][mf * 16 + li];
-      const int r = done.row0 + mf * 16 + li;
+      const float sa = sa_lds[parity][wave_m * 16 * kMF + mf * 16 + li];
+      const int r = done.row0 + wave_m * 16 * kMF + mf * 16 + li;
 #pragma unroll
       for (int f = 0; f < NFH; ++f) {
         float yv[4];
@@ -370,7 +375,7 @@ __global__ __launch_bounds__(kThreads, WGS) void tiled_gemm_i8_kernel(const Tile
       for (int h = 0; h < kReads; ++h) {
         const int pr = h * kRowsPerRead + rd_row;
         const v4i v = *reinterpret_cast<const v4i*>(&my_patch[(pr & 15) * kPatchPitch + rd_vec * 16]);
-        const int orow = done.row0 + mf * 16 + pr;
+        const int orow = done.row0 + wave_m * 16 * kMF + mf * 16 + pr;
         const int ocol = out_col0 + rd_vec * 8;
         if (pr < 16 && orow < row_end && ocol < n_half)  // n_half % 16 == 0: a vector of 8 channels is all in or all out
           *reinterpret_cast<v4i*>(p.y + static_cast<size_t>(orow) * p.ldy + ocol) = v;
@@ -381,8 +386,9 @@ __global__ __launch_bounds__(kThreads, WGS) void tiled_gemm_i8_kernel(const Tile
   }
 }
 
-template <bool SWIGLU, int NF, int R, int WGS>
+template <bool SWIGLU, int NF, int R, int WGS, int WM>
 int launch_tiled(const kmoe_gemm_i8_args* a, hipStream_t s, int n_cu) {
+  constexpr int kTM = WM * 16 * kMF;
   const int n_half = SWIGLU ? a->n / 2 : a->n;
   const int nfh = SWIGLU ? NF / 2 : NF;
   const int tail_rows = a->w_tail ? a->tail_rows : 0;
@@ -396,13 +402,14 @@ int launch_tiled(const kmoe_gemm_i8_args* a, hipStream_t s, int n_cu) {
   // persistent workgroups: WGS per CU
   const int grid = min(ceil_div(max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8);
   const size_t dyn = sizeof(int) * (static_cast<size_t>(a->E) + 1 + n_exp + 1);
-  hipLaunchKernelGGL((tiled_gemm_i8_kernel<SWIGLU, NF, R, WGS>), dim3(grid), dim3(kThreads), dyn, s, p);
+  hipLaunchKernelGGL((tiled_gemm_i8_kernel<SWIGLU, NF, R, WGS, WM>), dim3(grid), dim3(WM * kWavesT * kWave), dyn, s, p);
   return check_launch("kmoe_grouped_gemm_i8 (tiled)");
 }
 
 }  // namespace
 
-// variants 5, 6: 256-channel tiles, 4-slot weight ring; 7: 128-channel tiles, 8-slot ring, 3 workgroups per CU
+// variants 5, 6: 128x256 tiles, 4-slot weight ring, 2 workgroups per CU (the shape in use);
+// 7: 128x128 tiles, 8-slot ring, 3 workgroups per CU; 8: 256x256 tiles, 8 waves, 1 workgroup per CU
 int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
   const int tail_rows = a->w_tail ? a->tail_rows : 0;
@@ -428,8 +435,13 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   // 256-channel shape also when an expert has ~128 rows (DeepSeek-V3 prefill at 4096 tokens),
   // where HBM traffic, not bytes in flight, is the limit (twice the workgroups re-read A).
   if (a->variant == 7)
-    return swiglu ? launch_tiled<true, 2, 8, 3>(a, s, n_cu) : launch_tiled<false, 2, 8, 3>(a, s, n_cu);
-  return swiglu ? launch_tiled<true, 4, 4, 2>(a, s, n_cu) : launch_tiled<false, 4, 4, 2>(a, s, n_cu);
+    return swiglu ? launch_tiled<true, 2, 8, 3, 1>(a, s, n_cu) : launch_tiled<false, 2, 8, 3, 1>(a, s, n_cu);
+  // 256-row tiles bring DeepSeek-V3 prefill (128-256 rows per expert) down to its algorithmic HBM
+  // traffic (measured 1.01x against 1.5x), but with one workgroup per CU too few bytes are in
+  // flight: 3.4 TB/s against 5.6 TB/s, slower overall. Kept as a tuning variant.
+  if (a->variant == 8)
+    return swiglu ? launch_tiled<true, 4, 4, 1, 2>(a, s, n_cu) : launch_tiled<false, 4, 4, 1, 2>(a, s, n_cu);
+  return swiglu ? launch_tiled<true, 4, 4, 2, 1>(a, s, n_cu) : launch_tiled<false, 4, 4, 2, 1>(a, s, n_cu);
 }
 
 }  // namespace kmoe

@@ -254,6 +254,9 @@ typedef struct kmoe_gemm_fp8_args {
   int64_t ldy;
   int32_t act;
   int32_t variant;
+  int32_t w_layout;       /* KMOE_W_ROWMAJOR, or KMOE_W_TILED: the bytes of w re-arranged
+                             by kmoe_tile_weights_i8 (which moves bytes whatever they
+                             encode); needs k % 128 == 0, always true here          */
 } kmoe_gemm_fp8_args;
 
 /*

@@ -77,10 +77,29 @@ FP8_CASES = [
 ]
 
 
+FP8_TILED_CASES = FP8_CASES + [
+    (2, 256, 640, [140, 3]),                                      # odd number of 128-byte chunks
+    (20, 1024, 256, [((53 * i) % 300) for i in range(20)]),       # several tiles per workgroup walk
+]
+
+
+@pytest.mark.parametrize("E,n,k,counts", FP8_TILED_CASES)
+@pytest.mark.parametrize("variant", [1, 2, 3, 5])
+@pytest.mark.parametrize("act", [0, 1])
+def test_grouped_gemm_fp8_block_tiled_weights(L, E, n, k, counts, variant, act):
+    """The same product with the weight bytes re-arranged by kmoe_tile_weights_i8: the LDS-staged
+    kernels (1-3) and the persistent 128-row-tile kernel (5)."""
+    _fp8_case(L, E, n, k, counts, variant, act, tiled=True)
+
+
 @pytest.mark.parametrize("E,n,k,counts", FP8_CASES)
 @pytest.mark.parametrize("variant", [1, 2, 3])
 @pytest.mark.parametrize("act", [0, 1])
 def test_grouped_gemm_fp8_block(L, E, n, k, counts, variant, act):
+    _fp8_case(L, E, n, k, counts, variant, act, tiled=False)
+
+
+def _fp8_case(L, E, n, k, counts, variant, act, tiled):
     if act and n % 256:
         pytest.skip("SwiGLU needs n % 256 == 0 for block scales")
     torch.manual_seed(E * n + k + 1)
@@ -95,6 +114,11 @@ def test_grouped_gemm_fp8_block(L, E, n, k, counts, variant, act):
     da, ds, dw, dws, dl = a8.cuda(), xs.contiguous().cuda(), w8.cuda(), ws.contiguous().cuda(), torch.from_numpy(lod).cuda()
     y = torch.zeros(rows, n_out, dtype=torch.bfloat16, device="cuda")
     g = L.GemmFp8Args()
+    if tiled:
+        dt = torch.empty_like(dw)
+        L.check(L.lib.kmoe_tile_weights_i8(dw.data_ptr(), dt.data_ptr(), E, n, k, L.stream()))
+        dw = dt
+        g.w_layout = L.KMOE_W_TILED
     g.a, g.lda, g.a_scale, g.src_div = da.data_ptr(), k, ds.data_ptr(), 1
     g.w, g.w_scale, g.lod = dw.data_ptr(), dws.data_ptr(), dl.data_ptr()
     g.E, g.n, g.k, g.rows = E, n, k, rows
@@ -185,13 +209,13 @@ def test_fp8_layer(name, base, over):
     m = sl.layer.quant_method
     out = m.apply_monolithic(sl.layer, sl.x, sl.logits, **sl.apply_kwargs())
     torch.cuda.synchronize()
-    lay = sl.layer
     u8 = lambda t: _host(t).view(torch.uint8).numpy()  # noqa: E731
+    w13, w13_s, w2, w2_s, sh = sl.host_weights()  # row-major copies of the (tiled) device weights
     shared = None
-    if sl.shared is not None:
-        shared = (u8(sl.shared[0]), _host(sl.shared[1]).numpy(), u8(sl.shared[2]), _host(sl.shared[3]).numpy())
-    ref = co.forward_fp8(bits(sl.x), _host(sl.logits).numpy(), u8(lay.w13_weight), _host(lay.w13_weight_scale).numpy(),
-                         u8(lay.w2_weight), _host(lay.w2_weight_scale).numpy(), shape.K, shape.scoring, True,
+    if sh is not None:
+        shared = (u8(sh[0]), sh[1].numpy(), u8(sh[2]), sh[3].numpy())
+    ref = co.forward_fp8(bits(sl.x), _host(sl.logits).numpy(), u8(w13), w13_s.numpy(),
+                         u8(w2), w2_s.numpy(), shape.K, shape.scoring, True,
                          shape.n_group, shape.topk_group, shape.routed_scale,
                          None if sl.bias is None else _host(sl.bias).numpy(), shared)
     assert rel_l2(out, from_bits(ref)) <= REL_L2_FP8

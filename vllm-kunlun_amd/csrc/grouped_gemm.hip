@@ -61,7 +61,9 @@ struct GemmParams {
   uint16_t* y;
   int64_t ldy;             // in elements
   int32_t* acc_out;        // I8 only
-  int32_t w_tiled;         // weights in 64*LB-byte MFMA blocks [E][n/16][kbytes/(4*LB)] instead of row-major
+  int32_t w_tiled;         // weights in 1 KB MFMA blocks [E][n/16][kbytes/64] (kmoe_tile_weights_i8) instead of row-major.
+                           // FP8: an MFMA step takes two consecutive blocks, i.e. lane (g, c) holds k = 16g..16g+15 and
+                           // 64+16g..64+16g+15 of the step; the activation fragment takes the same two halves
   const int8_t* w_tail;    // optional extra expert (index E): rows [tail_row0, tail_row0 + tail_rows), identity source
   const float* w_max_tail;
   int32_t tail_row0, tail_rows, tail_src0;
@@ -172,14 +174,17 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
     const int c = col_base + fh * 16;
     wok[f] = c < n_half;
     col[f] = (SWIGLU && f >= NFH) ? n_half + c : c;
-    if (p.w_tiled) {  // block (fragment, step): 64*LB consecutive bytes, lane l at l*LB
+    if (p.w_tiled) {  // 1 KB block (fragment, 64 bytes of K): lane l at l*16
       const size_t frag = wok[f] ? col[f] / 16 : 0;
-      wp[f] = w_base + frag * (p.kbytes / (4 * LB)) * (64 * LB) + lane * LB;
+      wp[f] = w_base + frag * (p.kbytes / 64) * 1024 + lane * 16;
     } else {
       wp[f] = w_base + static_cast<size_t>(wok[f] ? col[f] + li : 0) * p.kbytes + lg * LB;
     }
   }
   const int w_step = p.w_tiled ? 64 * LB : 4 * LB;  // bytes between consecutive MFMA steps of a fragment
+  const int w_vec = p.w_tiled ? 1024 : 16;           // bytes between the 16-byte halves of a lane's operand (FP8)
+  const int a_lane = p.w_tiled ? 16 : LB;            // activation fragment: byte offset of lane group lg ...
+  const int a_vec = p.w_tiled ? 64 : 16;             // ... and of its second half (FP8)
   const int nchunks = (p.kbytes + kKC - 1) / kKC;
   const int kblocks = p.kbytes / 128;  // FP8: scale blocks along K
 
@@ -226,7 +231,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
 #pragma unroll
           for (int v = 0; v < kV; ++v) {
             const int koff = kc + j * 4 * LB + v * 16;  // k position (+ lg*LB, folded into wp)
-            const size_t off = static_cast<size_t>(chunk * kJ + j) * w_step + v * 16;
+            const size_t off = static_cast<size_t>(chunk * kJ + j) * w_step + v * w_vec;
             dst[f][j][v] = (wok[f] && koff + lg * LB < p.kbytes) ? *reinterpret_cast<const v4i*>(wp[f] + off)
                                                                   : (v4i){0, 0, 0, 0};
           }
@@ -251,7 +256,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
 #pragma unroll
           for (int v = 0; v < kV; ++v)
             af[mf][v] = *reinterpret_cast<const v4i*>(
-                &lds_a[buf][(mf * 16 + li) * kPitch + j * 4 * LB + lg * LB + v * 16]);
+                &lds_a[buf][(mf * 16 + li) * kPitch + j * 4 * LB + lg * a_lane + v * a_vec]);
         if constexpr (KIND == Kind::I8) {
 #pragma unroll
           for (int mf = 0; mf < MF; ++mf)
@@ -491,8 +496,16 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
                "grouped_gemm_fp8_block: misaligned tensor pointer");
   KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_fp8_block: src_div=%d < 1", a->src_div);
   if (a->rows == 0) return KMOE_OK;
+  KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR || a->w_layout == KMOE_W_TILED, KMOE_ERR_UNSUPPORTED,
+               "grouped_gemm_fp8_block: w_layout=%d unknown", a->w_layout);
+  // many rows per expert and tiled weights: the persistent 128-row-tile kernel (variant 5 forces it)
+  if (a->w_layout == KMOE_W_TILED && a->k <= 8192 && a->ldy % 8 == 0 &&
+      (a->variant == 5 || (a->variant == 0 && ceil_div(a->rows, a->E) > 48)))
+    return tiled_gemm_fp8(a, as_stream(stream));
+  KMOE_REQUIRE(a->variant != 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_fp8_block: variant 5 needs tiled weights, k <= 8192");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), a->w_scale, a->lod,  a->E,       a->n,
-               a->k,                                  a->y,       a->ldy,  nullptr, 0, nullptr, nullptr, 0, 0, 0};
+               a->k,                                  a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,
+               nullptr, nullptr, 0, 0, 0};
   return dispatch<Kind::FP8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_fp8_block");
 }

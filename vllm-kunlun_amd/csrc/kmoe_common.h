@@ -16,8 +16,10 @@ int check_launch(const char* what);
 int fill_dense_lod(int32_t* lod2, int rows, hipStream_t stream);
 // Weight-streaming int8 GEMM (tiled weights, chunk-major activations); arguments already validated.
 int stream_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);
-// MFMA-bound int8 GEMM on 128x512 tiles (tiled weights, row-major activations); arguments already validated.
+// Persistent 128-row-tile GEMMs for many rows per expert (tiled weights, row-major activations);
+// arguments already validated.
 int tiled_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);
+int tiled_gemm_fp8(const kmoe_gemm_fp8_args* args, hipStream_t stream);
 
 #define KMOE_REQUIRE(cond, code, ...) \
   do {                                \

@@ -30,7 +30,16 @@ namespace kmoe {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+// Operand format. F8: e4m3fn codes with block scales (one f32 per 128x128 weight block and
+// per activation row and 128 of K); one v_mfma_scale_f32_16x16x128_f8f6f4 covers a whole
+// 128-byte chunk (the two 1 KB weight blocks of a chunk are its two K halves, and the
+// activation fragment takes the same two halves), its partial sum is scaled and added in f32.
+enum class TKind { I8, F8 };
+constexpr int kMaxKBlocks = 64;  // F8: K <= 8192
 
 // Raw buffer descriptor over [base, base + 4 GiB): loads take a 32-bit per-lane offset
 // plus a scalar offset, so no 64-bit address arithmetic sits in the MFMA loop.
@@ -52,11 +61,11 @@ constexpr int kMaxExperts = 1024 + 1;      // routed experts + the tail expert
 struct TiledParams {
   const int8_t* a;
   int64_t lda;
-  const float* a_max;
+  const float* a_max;   // I8: [a_rows] absmax. F8: [a_rows, k/128] scales
   const int32_t* row_src;
   int32_t src_div;
   const int8_t* w;  // tiled
-  const float* w_max;
+  const float* w_max;   // I8: [E, n] absmax. F8: [E, n/128, k/128] scales
   const int32_t* lod;
   int32_t E, n, k;
   uint16_t* y;
@@ -85,8 +94,10 @@ struct Tile {
 // WM: rows of waves. 1: 128-row tiles, 4 waves; 2: 256-row tiles, 8 waves, where the two waves
 // that share channels read the same weight bytes within one barrier interval (an expert with
 // up to 256 rows then streams its weights from HBM once).
-template <bool SWIGLU, int NF, int R, int WGS, int WM>
-__global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kernel(const TiledParams p) {
+template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM>
+__global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(const TiledParams p) {
+  constexpr bool F8 = KIND == TKind::F8;
+  using acc_t = std::conditional_t<F8, v4f, v4i>;
   constexpr int kTM = WM * 16 * kMF;             // rows of a tile
   constexpr int kThreads = WM * kWavesT * kWave;
   static_assert(R == 4 || R == 8, "the chunk buffer parity is static only for R/2 even");
@@ -96,8 +107,13 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kerne
   constexpr int kPatchPitch = kOutBytes + 16;  // bytes per row of a wave's output patch (16 rows)
   __shared__ __attribute__((aligned(16))) int8_t lds_a[2][kTM * kPitchT];
   __shared__ __attribute__((aligned(16))) int8_t patch[WM * kWavesT][16 * kPatchPitch];
-  __shared__ __attribute__((aligned(16))) float sw_lds[2][kWavesT * NF * 16];  // per tile parity: channel scales (w_max / 127)
-  __shared__ float sa_lds[2][kTM];                                              // per tile parity: row scales (a_max / 127)
+  // I8, per tile parity: channel scales (w_max / 127) and row scales (a_max / 127)
+  __shared__ __attribute__((aligned(16))) float sw_lds[F8 ? 1 : 2][F8 ? 4 : kWavesT * NF * 16];
+  __shared__ float sa_lds[F8 ? 1 : 2][F8 ? 4 : kTM];
+  // F8: weight block scales of the tile [parity][wave][fragment][k block], and the row scales
+  // of the chunk in each activation buffer
+  __shared__ float wsc_lds[F8 ? 2 : 1][F8 ? kWavesT * NF * kMaxKBlocks : 4];
+  __shared__ float asc_lds[F8 ? 2 : 1][F8 ? kThreads : 4];  // every thread stores (rows repeat): no branch in the loop
   extern __shared__ int dyn_lds[];
   const int n_exp = p.E + (p.w_tail ? 1 : 0);
   int* row_lo = dyn_lds;               // [E + 1]: lod
@@ -179,7 +195,10 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kerne
   }
   v4i wring[R][kNF];  // weight fragments of MFMA step s live in slot s % R
   v4i areg[kNA];
-  v4i acc[kMF][kNF];
+  acc_t acc[kMF][kNF];
+  const int kblocks = p.k / 128;  // F8: scale blocks along K (= chunks)
+  int my_srow = 0;                // F8: source row of tile row threadIdx.x % kTM
+  float asc_reg = 0.0f;           // F8: that row's scale of the chunk in flight
 
   // Every load is unconditional (indices clamped to the last valid step / chunk, rows past a
   // tile's end read its first row, fragments past the last channel read fragment 0): the
@@ -193,10 +212,12 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kerne
     const uint32_t kc = static_cast<uint32_t>(min(chunk, last_chunk)) * kChunk;
 #pragma unroll
     for (int i = 0; i < kNA; ++i) areg[i] = buffer_load16(a_rsrc, aoff[i], kc);
+    if constexpr (F8) asc_reg = p.a_max[static_cast<size_t>(my_srow) * kblocks + min(chunk, last_chunk)];
   };
   auto store_a = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < kNA; ++i) *reinterpret_cast<v4i*>(&lds_a[buf][a_lds[i]]) = areg[i];
+    if constexpr (F8) asc_lds[buf][threadIdx.x] = asc_reg;
   };
   // one MFMA step: 8 A fragments from LDS, each against the 4 weight fragments of the slot
   auto compute = [&](const v4i(&wcur)[kNF], int buf, int j) {
@@ -206,6 +227,34 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kerne
 #pragma unroll
       for (int f = 0; f < kNF; ++f)
         acc[mf][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wcur[f], af, acc[mf][f], 0, 0, 0);
+    }
+  };
+  // F8, one whole chunk: the two ring slots of the chunk are the K halves of one MFMA
+  auto compute_f8 = [&](const v4i(&w_lo)[kNF], const v4i(&w_hi)[kNF], int buf, int chunk, int parity) {
+    float swc[kNF];
+#pragma unroll
+    for (int f = 0; f < kNF; ++f) swc[f] = wsc_lds[parity][(wave * kNF + f) * kMaxKBlocks + chunk];
+#pragma unroll
+    for (int mf = 0; mf < kMF; ++mf) {
+      const int row = wave_m * 16 * kMF + mf * 16 + li;
+      v8i av;
+      av.lo = *reinterpret_cast<const v4i*>(&lds_a[buf][row * kPitchT + lg * 16]);
+      av.hi = *reinterpret_cast<const v4i*>(&lds_a[buf][row * kPitchT + 64 + lg * 16]);
+      const float sa = asc_lds[buf][row];
+#pragma unroll
+      for (int f = 0; f < kNF; ++f) {
+        v8i wv;
+        wv.lo = w_lo[f];
+        wv.hi = w_hi[f];
+        const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, av, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0,
+                                                                         0x7f7f7f7f, 0, 0x7f7f7f7f);
+        const float sc = sa * swc[f];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[mf][f][q] = __builtin_fmaf(blk[q], sc, acc[mf][f][q]);
+      }
+      // keep the partial sums of one row fragment at a time in registers: without the fence the
+      // scheduler issues all 32 MFMAs first and spills their 128 results
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
   // Gather index of sorted row r of tile t (rows past the expert's end: the tile's first row),
@@ -230,11 +279,12 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kerne
 #pragma unroll
   for (int i = 0; i < kNA; ++i) rs[i] = fetch_src(cur, cur.row0 + ((threadIdx.x + i * kThreads) >> 3));
   float sw_reg = 0.0f, sa_reg = 0.0f;  // this thread's share of the tile's scales, on their way to LDS
+  float wsc_reg[kMaxKBlocks / 16];     // F8: weight block scales k = c, c + 16, ... of fragment lane / 16
 
   // Points the loaders at tile t and requests its first chunk, first three weight steps and scales.
   auto start_tile = [&](const Tile& t) {
     const int8_t* w_base = t.e >= p.E ? p.w_tail : p.w + static_cast<size_t>(t.e) * p.n * p.k;
-    const float* w_max = t.e >= p.E ? p.w_max_tail : p.w_max + static_cast<size_t>(t.e) * p.n;
+    [[maybe_unused]] const float* w_max = t.e >= p.E ? p.w_max_tail : p.w_max + static_cast<size_t>(t.e) * p.n;
     w_rsrc = make_rsrc(w_base);
 #pragma unroll
     for (int f = 0; f < kNF; ++f) {
@@ -246,16 +296,31 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kerne
     for (int i = 0; i < kNA; ++i)
       aoff[i] = static_cast<uint32_t>(src_row(t, rs[i])) * static_cast<uint32_t>(p.lda) +
                 ((threadIdx.x + i * kThreads) & 7) * 16;  // < 4 GiB: host-checked
+    if constexpr (F8) my_srow = src_row(t, fetch_src(t, t.row0 + threadIdx.x % kTM));
     load_a(0);
 #pragma unroll
     for (int i = 0; i < R - 1; ++i) load_w(wring[i], i);
-    if (wave_m == 0 && (lane >> 4) < kNF) {  // thread (wave, f = lane / 16, c = lane % 16): scale of channel c of fragment f of this wave
-      bool ok;
-      const int c = col_of(t, lane >> 4, ok);
-      sw_reg = ok ? w_max[c + (lane & 15)] : 0.0f;
+    if constexpr (F8) {
+      if (wave_m == 0 && (lane >> 4) < kNF) {  // thread (wave, f = lane / 16, c = lane % 16): block scales c, c + 16, ...
+        bool ok;
+        const int c = col_of(t, lane >> 4, ok);
+        const float* ws = (t.e >= p.E ? p.w_max_tail : p.w_max + static_cast<size_t>(t.e) * (p.n / 128) * kblocks) +
+                          static_cast<size_t>(ok ? c / 128 : 0) * kblocks;
+#pragma unroll
+        for (int i = 0; i < kMaxKBlocks / 16; ++i) {
+          const int kb = (lane & 15) + 16 * i;
+          wsc_reg[i] = kb < kblocks ? ws[kb] : 0.0f;
+        }
+      }
+    } else {
+      if (wave_m == 0 && (lane >> 4) < kNF) {  // thread (wave, f = lane / 16, c = lane % 16): scale of channel c of fragment f of this wave
+        bool ok;
+        const int c = col_of(t, lane >> 4, ok);
+        sw_reg = ok ? w_max[c + (lane & 15)] : 0.0f;
+      }
+      if (threadIdx.x < kTM)  // thread r: scale of tile row r
+        sa_reg = p.a_max[src_row(t, fetch_src(t, t.row0 + threadIdx.x))];
     }
-    if (threadIdx.x < kTM)  // thread r: scale of tile row r
-      sa_reg = p.a_max[src_row(t, fetch_src(t, t.row0 + threadIdx.x))];
   };
   start_tile(cur);
 
@@ -267,13 +332,24 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kerne
     for (int i = 0; i < kNA; ++i)
       rs_next[i] = nxt.valid ? fetch_src(nxt, nxt.row0 + ((threadIdx.x + i * kThreads) >> 3)) : 0;
 
-    if (wave_m == 0 && (lane >> 4) < kNF) sw_lds[parity][wave * kNF * 16 + lane] = sw_reg / 127.0f;
-    if (threadIdx.x < kTM) sa_lds[parity][threadIdx.x] = sa_reg / 127.0f;
+    if constexpr (F8) {
+      if (wave_m == 0 && (lane >> 4) < kNF) {
+#pragma unroll
+        for (int i = 0; i < kMaxKBlocks / 16; ++i)
+          wsc_lds[parity][(wave * kNF + (lane >> 4)) * kMaxKBlocks + (lane & 15) + 16 * i] = wsc_reg[i];
+      }
+    } else {
+      if (wave_m == 0 && (lane >> 4) < kNF) sw_lds[parity][wave * kNF * 16 + lane] = sw_reg / 127.0f;
+      if (threadIdx.x < kTM) sa_lds[parity][threadIdx.x] = sa_reg / 127.0f;
+    }
     store_a(0);
 #pragma unroll
     for (int mf = 0; mf < kMF; ++mf)
 #pragma unroll
-      for (int f = 0; f < kNF; ++f) acc[mf][f] = (v4i){0, 0, 0, 0};
+      for (int f = 0; f < kNF; ++f) {
+        if constexpr (F8) acc[mf][f] = (v4f){0.f, 0.f, 0.f, 0.f};
+        else acc[mf][f] = (v4i){0, 0, 0, 0};
+      }
     __syncthreads();
 
     // One chunk (two MFMA steps) of the pipeline; h = position of the chunk in the ring
@@ -287,11 +363,17 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kerne
       load_a(c0 + h + 1);
       load_w(wring[(2 * h + R - 1) % R], s0 + R - 1);
       __builtin_amdgcn_sched_barrier(0);
-      compute(wring[(2 * h) % R], buf, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      load_w(wring[(2 * h) % R], s0 + R);
-      __builtin_amdgcn_sched_barrier(0);
-      compute(wring[(2 * h + 1) % R], buf, 1);
+      if constexpr (F8) {
+        compute_f8(wring[(2 * h) % R], wring[(2 * h + 1) % R], buf, c0 + h, parity);
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(wring[(2 * h) % R], s0 + R);
+      } else {
+        compute(wring[(2 * h) % R], buf, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(wring[(2 * h) % R], s0 + R);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(wring[(2 * h + 1) % R], buf, 1);
+      }
       __builtin_amdgcn_sched_barrier(0);
       store_a(buf ^ 1);
       __syncthreads();
@@ -330,11 +412,13 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kerne
 #pragma unroll
     for (int f = 0; f < kNF; ++f) {
       col[f] = col_of(done, f, wok[f]);
-      const float4 s4 = *reinterpret_cast<const float4*>(&sw_lds[parity][(wave * kNF + f) * 16 + lg * 4]);
-      sw[f][0] = s4.x;
-      sw[f][1] = s4.y;
-      sw[f][2] = s4.z;
-      sw[f][3] = s4.w;
+      if constexpr (!F8) {
+        const float4 s4 = *reinterpret_cast<const float4*>(&sw_lds[parity][(wave * kNF + f) * 16 + lg * 4]);
+        sw[f][0] = s4.x;
+        sw[f][1] = s4.y;
+        sw[f][2] = s4.z;
+        sw[f][3] = s4.w;
+      }
     }
     int8_t* my_patch = patch[wave_id];
     // reader side of the patch: lane -> (row, 16-byte vector), consecutive lanes cover a row
@@ -345,29 +429,38 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kerne
     const int out_col0 = (done.nb * kWavesT + wave) * NFH * 16;  // first output channel of this wave
 #pragma unroll
     for (int mf = 0; mf < kMF; ++mf) {
-      const float sa = sa_lds[parity][wave_m * 16 * kMF + mf * 16 + li];
+      float sa = 1.0f;
+      if constexpr (!F8) sa = sa_lds[parity][wave_m * 16 * kMF + mf * 16 + li];
       const int r = done.row0 + wave_m * 16 * kMF + mf * 16 + li;
 #pragma unroll
       for (int f = 0; f < NFH; ++f) {
         float yv[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) yv[q] = (static_cast<float>(acc[mf][f][q]) * sa) * sw[f][q];
+        for (int q = 0; q < 4; ++q) {
+          if constexpr (F8) yv[q] = acc[mf][f][q];
+          else yv[q] = (static_cast<float>(acc[mf][f][q]) * sa) * sw[f][q];
+        }
         if (SWIGLU) {
           const int fu = f + NFH;
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             const float g = bf16_to_f32(f32_to_bf16_hw(yv[q]));  // gate and up are bf16 values first
-            const float u = bf16_to_f32(f32_to_bf16_hw((static_cast<float>(acc[mf][fu][q]) * sa) * sw[fu][q]));
+            float uf;
+            if constexpr (F8) uf = acc[mf][fu][q];
+            else uf = (static_cast<float>(acc[mf][fu][q]) * sa) * sw[fu][q];
+            const float u = bf16_to_f32(f32_to_bf16_hw(uf));
             yv[q] = silu_fixed(g) * u;
           }
         }
         *reinterpret_cast<uint2*>(&my_patch[li * kPatchPitch + f * 32 + lg * 8]) =
             make_uint2(pack2_bf16(yv[0], yv[1]), pack2_bf16(yv[2], yv[3]));
-        if (p.acc_out && r < row_end && wok[f]) {
-          *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[f] + lg * 4) = acc[mf][f];
-          if (SWIGLU)
-            *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[f + NFH] + lg * 4) =
-                acc[mf][f + NFH];
+        if constexpr (!F8) {
+          if (p.acc_out && r < row_end && wok[f]) {
+            *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[f] + lg * 4) = acc[mf][f];
+            if (SWIGLU)
+              *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[f + NFH] + lg * 4) =
+                  acc[mf][f + NFH];
+          }
         }
       }
       __builtin_amdgcn_wave_barrier();  // a wave's LDS operations execute in order: the reads see the writes
@@ -386,24 +479,44 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_i8_kerne
   }
 }
 
-template <bool SWIGLU, int NF, int R, int WGS, int WM>
-int launch_tiled(const kmoe_gemm_i8_args* a, hipStream_t s, int n_cu) {
+template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM>
+int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* what) {
   constexpr int kTM = WM * 16 * kMF;
-  const int n_half = SWIGLU ? a->n / 2 : a->n;
+  const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int nfh = SWIGLU ? NF / 2 : NF;
-  const int tail_rows = a->w_tail ? a->tail_rows : 0;
-  const int n_exp = a->E + (a->w_tail ? 1 : 0);
-  const int n_blocks = ceil_div(n_half, kWavesT * nfh * 16);
-  const int max_tiles = (a->rows + tail_rows) / kTM + min(n_exp, a->rows + tail_rows);
-  const int max_items = n_blocks * max_tiles;
-  TiledParams p{a->a,      a->lda,        a->a_max,      a->row_src, a->src_div,   a->w,         a->w_max, a->lod,
-                a->E,      a->n,          a->k,          a->y,       a->ldy,       a->acc_out,   a->w_tail,
-                a->w_max_tail, a->tail_row0, tail_rows,  a->tail_src0, n_blocks, max_items};
+  const int n_exp = p.E + (p.w_tail ? 1 : 0);
+  p.n_blocks = ceil_div(n_half, kWavesT * nfh * 16);
+  const int max_tiles = (rows + p.tail_rows) / kTM + min(n_exp, rows + p.tail_rows);
+  p.max_items = p.n_blocks * max_tiles;
   // persistent workgroups: WGS per CU
-  const int grid = min(ceil_div(max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8);
-  const size_t dyn = sizeof(int) * (static_cast<size_t>(a->E) + 1 + n_exp + 1);
-  hipLaunchKernelGGL((tiled_gemm_i8_kernel<SWIGLU, NF, R, WGS, WM>), dim3(grid), dim3(WM * kWavesT * kWave), dyn, s, p);
-  return check_launch("kmoe_grouped_gemm_i8 (tiled)");
+  const int grid = min(ceil_div(p.max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8);
+  const size_t dyn = sizeof(int) * (static_cast<size_t>(p.E) + 1 + n_exp + 1);
+  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM>), dim3(grid), dim3(WM * kWavesT * kWave), dyn, s,
+                     p);
+  return check_launch(what);
+}
+
+// Checks shared by both formats; fills n_cu.
+int tiled_common(const TiledParams& p, int rows, int* n_cu_out, const char* what) {
+  const int n_exp = p.E + (p.w_tail ? 1 : 0);
+  // 32-bit buffer offsets: one expert's weights and every source row of the activations
+  KMOE_REQUIRE(static_cast<int64_t>(p.n) * p.k < (1ll << 32), KMOE_ERR_SHAPE, "%s: n*k = %lld needs 32-bit offsets", what,
+               static_cast<long long>(p.n) * p.k);
+  KMOE_REQUIRE((static_cast<int64_t>(rows) + p.tail_src0 + p.tail_rows + 1) * p.lda < (1ll << 32), KMOE_ERR_SHAPE,
+               "%s: activations span more than 4 GiB", what);
+  KMOE_REQUIRE(n_exp <= kMaxExperts, KMOE_ERR_SHAPE, "%s: E=%d > %d", what, p.E, kMaxExperts - 1);
+  KMOE_REQUIRE(p.ldy % 8 == 0 && reinterpret_cast<uintptr_t>(p.y) % 16 == 0, KMOE_ERR_SHAPE,
+               "%s: y must be 16-byte aligned with ldy %% 8 == 0 (ldy=%lld)", what, static_cast<long long>(p.ldy));
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+      return fail(KMOE_ERR_LAUNCH, "%s: cannot query the device", what);
+    n_cu = prop.multiProcessorCount;
+  }
+  *n_cu_out = n_cu;
+  return KMOE_OK;
 }
 
 }  // namespace
@@ -411,37 +524,44 @@ int launch_tiled(const kmoe_gemm_i8_args* a, hipStream_t s, int n_cu) {
 // variants 5, 6: 128x256 tiles, 4-slot weight ring, 2 workgroups per CU (the shape in use);
 // 7: 128x128 tiles, 8-slot ring, 3 workgroups per CU; 8: 256x256 tiles, 8 waves, 1 workgroup per CU
 int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
+  const char* what = "kmoe_grouped_gemm_i8 (tiled)";
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
-  const int tail_rows = a->w_tail ? a->tail_rows : 0;
-  const int n_exp = a->E + (a->w_tail ? 1 : 0);
-  // 32-bit buffer offsets: one expert's weights and every source row of the activations
-  KMOE_REQUIRE(static_cast<int64_t>(a->n) * a->k < (1ll << 32), KMOE_ERR_SHAPE,
-               "grouped_gemm_i8 (tiled): n*k = %lld needs 32-bit offsets", static_cast<long long>(a->n) * a->k);
-  KMOE_REQUIRE((static_cast<int64_t>(a->rows) + a->tail_src0 + tail_rows + 1) * a->lda < (1ll << 32), KMOE_ERR_SHAPE,
-               "grouped_gemm_i8 (tiled): activations span more than 4 GiB");
-  KMOE_REQUIRE(n_exp <= kMaxExperts, KMOE_ERR_SHAPE, "grouped_gemm_i8 (tiled): E=%d > %d", a->E, kMaxExperts - 1);
-  KMOE_REQUIRE(a->ldy % 8 == 0 && reinterpret_cast<uintptr_t>(a->y) % 16 == 0, KMOE_ERR_SHAPE,
-               "grouped_gemm_i8 (tiled): y must be 16-byte aligned with ldy %% 8 == 0 (ldy=%lld)",
-               static_cast<long long>(a->ldy));
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-      return fail(KMOE_ERR_LAUNCH, "grouped_gemm_i8 (tiled): cannot query the device");
-    n_cu = prop.multiProcessorCount;
-  }
+  TiledParams p{a->a,      a->lda,        a->a_max,      a->row_src, a->src_div,   a->w,         a->w_max, a->lod,
+                a->E,      a->n,          a->k,          a->y,       a->ldy,       a->acc_out,   a->w_tail,
+                a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0, 0, 0};
+  int n_cu = 0;
+  if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
+  constexpr TKind K = TKind::I8;
   // The 128-channel / deep-ring shape is a tuning variant only: measured slower than the
   // 256-channel shape also when an expert has ~128 rows (DeepSeek-V3 prefill at 4096 tokens),
   // where HBM traffic, not bytes in flight, is the limit (twice the workgroups re-read A).
   if (a->variant == 7)
-    return swiglu ? launch_tiled<true, 2, 8, 3, 1>(a, s, n_cu) : launch_tiled<false, 2, 8, 3, 1>(a, s, n_cu);
+    return swiglu ? launch_tiled<K, true, 2, 8, 3, 1>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 2, 8, 3, 1>(p, a->rows, s, n_cu, what);
   // 256-row tiles bring DeepSeek-V3 prefill (128-256 rows per expert) down to its algorithmic HBM
   // traffic (measured 1.01x against 1.5x), but with one workgroup per CU too few bytes are in
   // flight: 3.4 TB/s against 5.6 TB/s, slower overall. Kept as a tuning variant.
   if (a->variant == 8)
-    return swiglu ? launch_tiled<true, 4, 4, 1, 2>(a, s, n_cu) : launch_tiled<false, 4, 4, 1, 2>(a, s, n_cu);
-  return swiglu ? launch_tiled<true, 4, 4, 2, 1>(a, s, n_cu) : launch_tiled<false, 4, 4, 2, 1>(a, s, n_cu);
+    return swiglu ? launch_tiled<K, true, 4, 4, 1, 2>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 4, 4, 1, 2>(p, a->rows, s, n_cu, what);
+  return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)
+                : launch_tiled<K, false, 4, 4, 2, 1>(p, a->rows, s, n_cu, what);
+}
+
+// fp8 block-scaled operands on the same tiles (weights tiled with kmoe_tile_weights_i8: the
+// re-arrangement moves bytes and does not care what they encode).
+int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
+  const char* what = "kmoe_grouped_gemm_fp8_block (tiled)";
+  const bool swiglu = a->act == KMOE_ACT_SWIGLU;
+  KMOE_REQUIRE(a->k / 128 <= kMaxKBlocks, KMOE_ERR_UNSUPPORTED, "%s: k=%d > %d", what, a->k, 128 * kMaxKBlocks);
+  TiledParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,
+                reinterpret_cast<const int8_t*>(a->w), a->w_scale, a->lod, a->E, a->n, a->k, a->y, a->ldy, nullptr,
+                nullptr, nullptr, 0, 0, 0, 0, 0};
+  int n_cu = 0;
+  if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
+  constexpr TKind K = TKind::F8;
+  return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)
+                : launch_tiled<K, false, 4, 4, 2, 1>(p, a->rows, s, n_cu, what);
 }
 
 }  // namespace kmoe

@@ -52,18 +52,21 @@ def is_tiled(w: torch.Tensor) -> bool:
     return bool(getattr(w, "_kmoe_tiled", False))
 
 
+_ONE_BYTE = (torch.int8, torch.uint8, torch.float8_e4m3fn)
+
+
 def tile_int8_weights_(w: torch.Tensor) -> bool:
-    """Re-arranges int8 weights [..., n, k] IN PLACE into the MFMA-ready 1 KB blocks of
-    kmoe_tile_weights_i8 (one expert at a time through a scratch copy) and marks the
-    object. Returns False and leaves the tensor alone when the shape does not allow it
-    (n % 16, k % 64)."""
+    """Re-arranges one-byte weights (int8, or e4m3 codes) [..., n, k] IN PLACE into the
+    MFMA-ready 1 KB blocks of kmoe_tile_weights_i8 (one expert at a time through a scratch
+    copy) and marks the object. Returns False and leaves the tensor alone when the shape
+    does not allow it (n % 16, k % 64)."""
     data = w.data
     n, k = data.shape[-2], data.shape[-1]
-    if data.dtype != torch.int8 or not data.is_cuda or not data.is_contiguous() or n % 16 or k % 64:
+    if data.dtype not in _ONE_BYTE or not data.is_cuda or not data.is_contiguous() or n % 16 or k % 64:
         return False
     if is_tiled(w):
         return True
-    flat = data.view(-1, n, k)
+    flat = data.view(torch.int8).view(-1, n, k)
     tmp = torch.empty_like(flat[0])
     for e in range(flat.shape[0]):
         L.check(L.lib.kmoe_tile_weights_i8(L.ptr(flat[e]), L.ptr(tmp), 1, n, k, L.stream()))
@@ -78,8 +81,8 @@ def rowmajor_int8_weights(w: torch.Tensor) -> torch.Tensor:
         return w.data.clone()
     n, k = w.shape[-2], w.shape[-1]
     lead = w.shape[:-2]
-    t = w.data.reshape(-1, n // 16, k // 64, 4, 16, 16).permute(0, 1, 4, 2, 3, 5)
-    return t.reshape(*lead, n, k).contiguous()
+    t = w.data.view(torch.int8).reshape(-1, n // 16, k // 64, 4, 16, 16).permute(0, 1, 4, 2, 3, 5)
+    return t.reshape(*lead, n, k).contiguous().view(w.dtype)
 
 
 _WEIGHT_DTYPE = {L.KMOE_FMT_INT8: (torch.int8,), L.KMOE_FMT_FP8_BLOCK: (torch.float8_e4m3fn, torch.uint8),
@@ -138,7 +141,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     a.out = out.data_ptr()
     if w_layout is None:  # tiled only if every int8 weight of the call has been tiled
         ws_all = [w13, w2] + ([shared_expert[0], shared_expert[2]] if shared_expert is not None else [])
-        w_layout = L.KMOE_W_TILED if fmt == L.KMOE_FMT_INT8 and all(is_tiled(t) for t in ws_all) else L.KMOE_W_ROWMAJOR
+        w_layout = L.KMOE_W_TILED if fmt != L.KMOE_FMT_BF16 and all(is_tiled(t) for t in ws_all) else L.KMOE_W_ROWMAJOR
         if w_layout == L.KMOE_W_ROWMAJOR and any(is_tiled(t) for t in ws_all):
             raise ValueError("moe plan: routed and shared expert weights must be either all tiled or all row-major")
     a.w_layout = int(w_layout)

@@ -260,4 +260,10 @@ class KunlunCompressedTensorsW8A8Fp8MoEMethod(_MonolithicQuantMoE):
         layer.w2_weight_scale = mk(E, H // 128, I // 128, dt=torch.float32)
 
     def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
-        """Block scales are used as they are (dequant = code * scale); nothing to convert."""
+        """Block scales are used as they are (dequant = code * scale). On the GPU the e4m3 codes
+        are re-arranged in place into the same MFMA-ready 1 KB blocks as int8 weights."""
+        w13, w2 = layer.w13_weight, layer.w2_weight
+        if getattr(self, "tile_weights", True) and w13.is_cuda:
+            with torch.no_grad():
+                tile_int8_weights_(w13)
+                tile_int8_weights_(w2)

@@ -88,7 +88,7 @@ class SynthLayer:
         lay = self.layer
 
         def rm(t):
-            return (rowmajor_int8_weights(t) if t.dtype == torch.int8 else t).detach().cpu()
+            return (rowmajor_int8_weights(t) if t.element_size() == 1 else t).detach().cpu()
 
         aux = lambda name: getattr(lay, name).detach().cpu() if hasattr(lay, name) else None  # noqa: E731
         shared = None
@@ -159,6 +159,10 @@ def make_fp8_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
         q13, s13 = _quant_block_fp8(torch.randn(2 * s.I_shared, s.H, generator=g, device=dev) * 0.02)
         q2, s2 = _quant_block_fp8(torch.randn(s.H, s.I_shared, generator=g, device=dev) * 0.02)
         shared = (q13, s13.contiguous(), q2, s2.contiguous())
+        from ._plan import is_tiled, tile_int8_weights_
+        if is_tiled(layer.w13_weight):
+            tile_int8_weights_(q13)
+            tile_int8_weights_(q2)
     x, logits = _activations(s, g, dev)
     return SynthLayer(s, layer, x, logits, bias, shared)
 

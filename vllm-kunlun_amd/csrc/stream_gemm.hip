@@ -227,8 +227,10 @@ int stream_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   // m-fragments per pass from the rows an expert gets under uniform routing
   int mf = a->variant;
   if (mf == 0) {
+    // An expert with more rows than one pass holds streams its weights again: leave headroom
+    // over the mean for the spread of a random routing (about +-2 sigma at these sizes).
     const int avg = ceil_div(a->rows, a->E);
-    mf = avg <= 16 ? 1 : (avg <= 32 ? 2 : (avg <= 64 ? 4 : 8));
+    mf = avg <= 10 ? 1 : (avg <= 22 ? 2 : (avg <= 48 ? 4 : 8));
   }
   switch (mf) {
     // tuning variants of the 16-row kernel: 1xy = prefetch depth x, K split y

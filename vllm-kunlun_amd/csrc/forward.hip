@@ -270,9 +270,21 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
     if (ev) (void)hipEventRecord(static_cast<hipEvent_t>(ev), as_stream(stream));
   };
 
-  // 1. routing
+  // 1. routing; on the int8 decode path together with step 3 (independent work, one launch)
+  const bool stream_mode = use_stream_path(a);
+  bool quant_done = false;
   mark(KMOE_STAGE_ROUTING, 0);
-  if (a->scoring == KMOE_SCORE_SOFTMAX) {
+  if (a->format == KMOE_FMT_INT8 && M <= 1024) {
+    rc = fused_route_quant_i8(a->logits, a->bias, M, E, K, a->scoring == KMOE_SCORE_SIGMOID, a->renormalize, a->n_group,
+                              a->topk_group, a->routed_scale, topk_w, topk_ids, a->x, H, static_cast<int8_t*>(at(L.xq)),
+                              static_cast<float*>(at(L.xmax)), stream_mode ? 1 : 0, as_stream(stream));
+    if (rc < 0) return rc;
+    quant_done = rc == KMOE_OK;
+    rc = KMOE_OK;
+  }
+  if (quant_done) {
+    // both done
+  } else if (a->scoring == KMOE_SCORE_SOFTMAX) {
     rc = kmoe_softmax_topk(a->logits, M, E, K, a->renormalize, topk_w, topk_ids, stream);
   } else {
     rc = kmoe_sigmoid_group_topk_norm(a->logits, a->bias, M, E, K, a->n_group, a->topk_group, a->routed_scale, topk_w,
@@ -289,8 +301,9 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   // 3. quantise each TOKEN row once (the reference quantises the K-times expanded copy; same values)
   mark(KMOE_STAGE_QUANT1, 0);
   const void* x_rows = a->x;
-  const bool stream_mode = use_stream_path(a);
-  if (a->format == KMOE_FMT_INT8) {
+  if (quant_done) {
+    x_rows = at(L.xq);
+  } else if (a->format == KMOE_FMT_INT8) {
     rc = stream_mode ? kmoe_quant_i8_rows_chunked(a->x, H, M, H, static_cast<int8_t*>(at(L.xq)),
                                                   static_cast<float*>(at(L.xmax)), stream)
                      : kmoe_quant_i8_rows(a->x, H, M, H, static_cast<int8_t*>(at(L.xq)), H,

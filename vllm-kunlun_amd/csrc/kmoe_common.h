@@ -20,6 +20,11 @@ int stream_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);
 // arguments already validated.
 int tiled_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);
 int tiled_gemm_fp8(const kmoe_gemm_fp8_args* args, hipStream_t stream);
+// Routing + per-token int8 quantisation of x [M,H] in one launch. Returns 1 (nothing launched)
+// when the arguments are outside its instantiations: the caller then uses the two entry points.
+int fused_route_quant_i8(const float* logits, const float* bias, int M, int E, int K, int sigmoid, int renorm,
+                         int n_group, int topk_group, float scale, float* topk_w, int32_t* topk_ids,
+                         const uint16_t* x, int H, int8_t* xq, float* xmax, int chunked, hipStream_t stream);
 
 #define KMOE_REQUIRE(cond, code, ...) \
   do {                                \

@@ -150,6 +150,9 @@ def main():
                     help="replay the layer from a captured HIP graph (as a serving engine does) or launch it eagerly")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--router", action="store_true",
+                    help="hand the layer the bf16 gate weight [E,H] instead of router logits: the router GEMM "
+                         "then runs inside each step (reported in config; not the default workload)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one bitwise_not over 256 MiB (a kernel of known HBM traffic and a name nothing "
                          "else here has) before the timed region: the yardstick for FETCH_SIZE / WRITE_SIZE runs")
@@ -170,12 +173,18 @@ def main():
     out = torch.empty_like(x)
     fmt = {"int8": L.KMOE_FMT_INT8, "fp8": L.KMOE_FMT_FP8_BLOCK, "none": L.KMOE_FMT_BF16}[shape.quant]
 
+    w_gate = None
+    if a.router:
+        gen = torch.Generator(device="cuda:0")
+        gen.manual_seed(a.seed + 1)
+        w_gate = (torch.randn(shape.E, shape.H, generator=gen, device="cuda:0") * shape.H ** -0.5).bfloat16()  # logits ~ N(0,1)
+
     def make_plan(stage_events=None):
         # the argument block the plugin methods build (apply_monolithic / KunlunOps.fused_moe)
-        return make_moe_plan(fmt, x, logits, out, shape.K, lay.w13_weight, lay.w2_weight,
+        return make_moe_plan(fmt, x, None if a.router else logits, out, shape.K, lay.w13_weight, lay.w2_weight,
                              getattr(lay, "w13_weight_scale", None), getattr(lay, "w2_weight_scale", None),
                              shape.scoring, True, shape.n_group, shape.topk_group, shape.routed_scale, sl.bias,
-                             sl.shared, 1.0, stage_events)
+                             sl.shared, 1.0, stage_events, router_weight=w_gate)
 
     plan = make_plan()
 
@@ -259,7 +268,8 @@ def main():
         "config": {"workload": WORKLOAD_LABEL[a.workload], "name": a.workload, "tokens": shape.M, "hidden": shape.H,
                    "experts": shape.E, "top_k": shape.K, "moe_intermediate": shape.I,
                    "shared_intermediate": shape.I_shared, "routing": shape.scoring, "experts_hit": n_active,
-                   "launch": "hipgraph replay" if graph is not None else "eager", "seed": a.seed},
+                   "launch": "hipgraph replay" if graph is not None else "eager", "seed": a.seed,
+                   "router_gemm_inside": bool(a.router)},
         "roofline": roofline,
         "layer": {"hbm_gbs": work["layer_bytes"] / t_s / 1e9, "hbm_frac": work["layer_bytes"] / t_s / 1e9 / HBM_PEAK_GBS,
                   "tops": work["layer_ops"] / t_s / 1e12,

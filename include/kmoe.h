@@ -292,6 +292,22 @@ int kmoe_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_index,
                  int64_t ld_addend, uint16_t* out, int64_t ld_out,
                  kmoe_stream_t stream);
 
+/* ---------------------------------------------------------------- router GEMM */
+
+/*
+ * Router logits: logits[M,E] (f32) = x[M,H] (bf16) . w_gate[E,H]^T (bf16), accumulated in
+ * f32. Replaces the gate projection in front of the layer: GateLinear.forward /
+ * ops.router_gemm_bf16_fp32 (ops/fused_moe/router/gate_linear.py:91-116), called as
+ * `router_logits, _ = self.gate(hidden_states)` (models/deepseek_v2.py:178-184, 275).
+ * K is split over workgroups for small M; the partial planes (in `workspace`,
+ * kmoe_router_gemm_workspace_bytes) are added in a fixed order, so the result does not
+ * depend on scheduling. Limits: H % 32 == 0, E <= 1024, 16-byte aligned tensors.
+ */
+size_t kmoe_router_gemm_workspace_bytes(int M, int H, int E);
+int kmoe_router_gemm_bf16(const uint16_t* x, int64_t ld_x, const uint16_t* w_gate,
+                          int M, int H, int E, float* logits, int64_t ld_logits,
+                          void* workspace, size_t workspace_bytes, kmoe_stream_t stream);
+
 /* ------------------------------------------------------------ fused forward */
 
 #define KMOE_SCORE_SOFTMAX 0
@@ -310,7 +326,9 @@ typedef struct kmoe_moe_args {
   int32_t renormalize;   /* softmax only: divide the K weights by their sum     */
   int32_t n_group, topk_group; /* sigmoid only; n_group <= 1: no group stage    */
   float routed_scale;    /* sigmoid only: multiplies the routing weights        */
-  const float* logits;   /* [M,E] f32                                           */
+  const float* logits;   /* [M,E] f32, or NULL with w_gate set: the layer then computes
+                            them itself (kmoe_router_gemm_bf16 without the reduction
+                            pass: the routing kernel adds the partial planes)     */
   const float* bias;     /* [E] f32 correction bias or NULL                     */
   /* activations and routed expert weights */
   const uint16_t* x;     /* [M,H] bf16                                          */
@@ -331,8 +349,9 @@ typedef struct kmoe_moe_args {
      recorded on the stream before stage s and entry 2s+1 after it (NULL entries
      are skipped). Leave NULL under graph capture.                             */
   void* const* stage_events;
-  int32_t w_layout;      /* INT8 only: KMOE_W_TILED if w13, w2 (and ws13, ws2) went
+  int32_t w_layout;      /* INT8, FP8: KMOE_W_TILED if w13, w2 (and ws13, ws2) went
                             through kmoe_tile_weights_i8; else KMOE_W_ROWMAJOR  */
+  const uint16_t* w_gate; /* NULL, or [E,H] bf16 router weight (used when logits is NULL) */
 } kmoe_moe_args;
 
 #define KMOE_STAGE_ROUTING 0
@@ -358,6 +377,8 @@ typedef struct kmoe_moe_layout {
   size_t sh_lod, sh_act, sh_actq, sh_actmax, sh_out;
   size_t codes_chunked; /* 1: xq/actq/sh_actq are chunk-major [C/16][rows][16] (the
                            weight-streaming decode path), 0: row-major [rows][C] */
+  size_t logit_planes;  /* partial router logits [planes][M][E] f32 (w_gate given)   */
+  size_t n_logit_planes;
 } kmoe_moe_layout;
 
 /* Workspace layout (and total size) for a shape; only the shape and format fields of args are read. */

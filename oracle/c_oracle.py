@@ -219,6 +219,18 @@ def forward_w8a8(x_bits, logits, w13, w13_max, w2, w2_max, K, scoring="softmax",
     return (out, inter) if intermediates else out
 
 
+def router_gemm(x_bits, w_bits):
+    """(logits f32 [M,E], abs_sum f32 [M,E]): x bf16 bits [M,H], w bf16 bits [E,H]."""
+    x_bits = _c(x_bits, np.uint16)
+    w_bits = _c(w_bits, np.uint16)
+    M, H = x_bits.shape
+    E = w_bits.shape[0]
+    logits = np.zeros((M, E), np.float32)
+    abs_sum = np.zeros((M, E), np.float32)
+    lib().orc_router_gemm(_p(x_bits), C.c_int64(H), _p(w_bits), M, H, E, _p(logits), _p(abs_sum))
+    return logits, abs_sum
+
+
 def grouped_gemm_bf16(a_bits, w_bits, lod, act=0, row_src=None, src_div=1):
     a_bits = _c(a_bits, np.uint16)
     w_bits = _c(w_bits, np.uint16)

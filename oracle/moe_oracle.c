@@ -320,6 +320,30 @@ ORC_API void orc_grouped_gemm_i8(const int8_t* a, int64_t lda, const float* a_ma
   }
 }
 
+/* Router logits in front of the layer: `router_logits, _ = self.gate(hidden_states)`
+ * (models/deepseek_v2.py:178-184, 275), the bf16 x bf16 -> fp32 product of
+ * ops/fused_moe/router/gate_linear.py:105-108. logits[m,e] = sum_k x[m,k] * w[e,k], every
+ * product exact in double and the sum kept in double, rounded to f32 once: the value every
+ * f32 summation order approximates. Comparisons with a device result are within the bound
+ * (H * 2^-24) * sum_k |x[m,k] * w[e,k]|, which `abs_sum` (optional) returns. Parity unpinned
+ * against the reference's closed/absent kernels; pinned against torch's f64 matmul. */
+ORC_API void orc_router_gemm(const uint16_t* x, int64_t ld_x, const uint16_t* w, int M, int H, int E, float* logits,
+                             float* abs_sum) {
+#pragma omp parallel for schedule(static)
+  for (int m = 0; m < M; ++m) {
+    for (int e = 0; e < E; ++e) {
+      double s = 0.0, sa = 0.0;
+      for (int k = 0; k < H; ++k) {
+        const double p = (double)bf16_to_f32(x[(size_t)m * ld_x + k]) * (double)bf16_to_f32(w[(size_t)e * H + k]);
+        s += p;
+        sa += p < 0 ? -p : p;
+      }
+      logits[(size_t)m * E + e] = (float)s;
+      if (abs_sum) abs_sum[(size_t)m * E + e] = (float)sa;
+    }
+  }
+}
+
 /* moe_fc with bf16 x and weight (ops/_kunlun_ops.py:578-585, 595-603, 615-622):
  * f32 accumulation in ascending k, one bf16 rounding. A device MFMA sums in its
  * own order, so comparisons with this function are within tolerance, not exact. */

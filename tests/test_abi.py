@@ -37,7 +37,9 @@ def test_library_exports_every_declared_symbol(L):
 def test_struct_layouts_match_the_header(L):
     # sizes implied by the C declarations (LP64): guards the ctypes mirrors against drift
     assert C.sizeof(L.GemmI8Args) == 8 * 8 + 16 + 8 * 3 + 8 + 16 + 16 + 16  # 8 ptr/int64, 4 int32, y/ldy/acc_out, act+variant, 3 int32 + pad
-    assert C.sizeof(L.MoELayout) == 20 * 8
+    assert C.sizeof(L.MoELayout) == 22 * 8
+    assert C.sizeof(L.GemmFp8Args) == 8 * 8 + 16 + 16 + 16  # 8 ptr/int64, 4 int32, y/ldy, act+variant+w_layout+pad
+    assert L.MoEArgs.w_gate.offset == C.sizeof(L.MoEArgs) - 8
     a = L.MoEArgs()
     assert L.MoEArgs.M.offset == 0 and L.MoEArgs.logits.offset == 48 and C.sizeof(a) % 8 == 0
 
@@ -85,7 +87,7 @@ def test_forward_validation_and_workspace_layout(L):
     assert L.lib.kmoe_moe_workspace_layout(a, lay) == 0
     P = 64 * 8
     assert lay.total_bytes >= P * 2048 * 2 + P * 768 * 3 + 64 * 2048
-    offs = [getattr(lay, n) for n, _ in L.MoELayout._fields_[1:-1]]
+    offs = [getattr(lay, n) for n, _ in L.MoELayout._fields_[1:-3]] + [lay.logit_planes]
     assert offs == sorted(offs) and all(o % 256 == 0 for o in offs)
     a.K = 200
     assert L.lib.kmoe_moe_workspace_layout(a, lay) == -2

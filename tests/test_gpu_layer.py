@@ -159,3 +159,50 @@ def test_empty_batch():
     sl = synth.make_w8a8_layer(synth.scaled(synth.SHAPES["qwen3-decode"], M=4, H=256, E=8, K=2, I=64), "cuda")
     out = sl.layer.quant_method.apply_monolithic(sl.layer, sl.x[:0], sl.logits[:0])
     assert out.shape == (0, 256)
+
+
+ROUTER_CASES = [(1, 64, 8), (7, 256, 130), (64, 2048, 128), (128, 7168, 256), (300, 512, 384), (1100, 1024, 64)]
+
+
+@pytest.mark.parametrize("M,H,E", ROUTER_CASES)
+def test_router_gemm(M, H, E):
+    """kmoe_router_gemm_bf16 through torch.ops._C.router_gemm_bf16_fp32 against the exact-sum oracle,
+    within the f32 summation bound, and bit-identical from run to run (fixed plane order)."""
+    import vllm_kunlun_amd  # noqa: F401
+    torch.manual_seed(M + H + E)
+    x = torch.randn(M, H).bfloat16()
+    w = (torch.randn(E, H) * 0.05).bfloat16()
+    ref, abs_sum = co.router_gemm(bits(x), bits(w))
+    xd, wd = x.cuda(), w.cuda()
+    got = torch.ops._C.router_gemm_bf16_fp32(xd, wd)
+    again = torch.ops._C.router_gemm_bf16_fp32(xd, wd)
+    torch.cuda.synchronize()
+    assert torch.equal(got, again)
+    err = np.abs(got.cpu().numpy() - ref)
+    assert np.all(err <= H * 2.0 ** -24 * abs_sum + 1e-30), float(err.max())
+
+
+@pytest.mark.parametrize("base,over", [("qwen3-decode", dict(M=40, H=256, E=64, K=4, I=128)),
+                                       ("dsv3-decode", dict(M=48, H=512, E=32, K=4, I=256, n_group=4, topk_group=2,
+                                                            I_shared=256)),
+                                       ("qwen3-prefill", dict(M=1500, H=256, E=16, K=2, I=128))],
+                         ids=["softmax", "sigmoid-shared", "many-tokens"])
+def test_layer_with_the_router_inside(base, over):
+    """apply_monolithic(router_logits=None, router_weight=W): the same bits as computing the logits
+    with the stand-alone router GEMM and handing them in (the routing kernel adds the split-K planes
+    in the order the reduction kernel does)."""
+    from vllm_kunlun_amd import synth
+    from vllm_kunlun_amd.ops.fused_moe.router import GateLinear
+    shape = synth.scaled(synth.SHAPES[base], **over)
+    sl = synth.make_w8a8_layer(shape, "cuda", seed=3)
+    gate = GateLinear(shape.H, shape.E, device="cuda")
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    gate.weight.data.copy_((torch.randn(shape.E, shape.H, generator=g, device="cuda") * 0.05).bfloat16())
+    logits, _ = gate(sl.x)
+    m = sl.layer.quant_method
+    kw = sl.apply_kwargs()
+    ref = m.apply_monolithic(sl.layer, sl.x, logits, **kw)
+    got = m.apply_monolithic(sl.layer, sl.x, None, router_weight=gate.weight, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(got, ref)

@@ -443,3 +443,16 @@ def test_bf16_expert_loop_matches_float_math():
             h = x[m].double() @ w13[e].double().T
             ref[m] += tw[m, k] * ((F.silu(h[:I]) * h[I:]) @ w2[e].double().T)
     assert rel_l2(out, ref) <= 1e-2
+
+
+def test_router_gemm_against_f64_matmul():
+    """logits = x . w^T: exact products, double sum, one rounding; a transposed operand, a wrong
+    stride or a dropped k would show against torch's f64 matmul; abs_sum is sum |x*w|."""
+    torch.manual_seed(11)
+    for M, H, E in ((1, 32, 1), (5, 96, 7), (33, 256, 130)):
+        x = torch.randn(M, H).bfloat16()
+        w = (torch.randn(E, H) * 0.05).bfloat16()
+        got, abs_sum = co.router_gemm(bits(x), bits(w))
+        ref = x.double() @ w.double().T
+        assert np.array_equal(got, ref.float().numpy())
+        assert np.allclose(abs_sum, (x.double().abs() @ w.double().abs().T).numpy(), rtol=1e-6)

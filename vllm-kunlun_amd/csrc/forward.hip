@@ -232,6 +232,10 @@ extern "C" int kmoe_moe_workspace_layout(const kmoe_moe_args* a, kmoe_moe_layout
   L->sh_actq = take(quant ? Ms * Is : 0);
   L->sh_actmax = take(quant ? Ms * 4 * (fp8 ? Is / 128 : 1) : 0);
   L->sh_out = take(Ms * H * 2);
+  int ks = 0, mf = 0;
+  if (a->w_gate && a->H % 32 == 0) router_plan(a->M, a->H, a->E, &ks, &mf);
+  L->n_logit_planes = ks;
+  L->logit_planes = take(ks ? static_cast<size_t>(ks) * M * E * 4 : 0);
   L->total_bytes = off;
   L->codes_chunked = use_stream_path(a) ? 1 : 0;
   return KMOE_OK;
@@ -243,7 +247,11 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   if (int rc = kmoe_moe_workspace_layout(a, &L)) return rc;
   if (a->M == 0) return KMOE_OK;
   const bool quant = a->format != KMOE_FMT_BF16;
-  KMOE_REQUIRE(a->logits && a->x && a->w13 && a->w2 && a->out, KMOE_ERR_NULL, "moe_forward: NULL tensor pointer");
+  KMOE_REQUIRE((a->logits || a->w_gate) && a->x && a->w13 && a->w2 && a->out, KMOE_ERR_NULL,
+               "moe_forward: NULL tensor pointer");
+  KMOE_REQUIRE(a->logits || (a->H % 32 == 0 && (reinterpret_cast<uintptr_t>(a->w_gate) & 15) == 0 &&
+                             (reinterpret_cast<uintptr_t>(a->x) & 15) == 0),
+               KMOE_ERR_SHAPE, "moe_forward: the router GEMM needs H %% 32 == 0 and 16-byte aligned x, w_gate");
   KMOE_REQUIRE(!quant || (a->w13_max && a->w2_max), KMOE_ERR_NULL, "moe_forward: weight max/scale pointers are NULL");
   KMOE_REQUIRE(a->I_shared == 0 || (a->ws13 && a->ws2 && (!quant || (a->ws13_max && a->ws2_max))), KMOE_ERR_NULL,
                "moe_forward: shared expert pointers are NULL");
@@ -270,24 +278,42 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
     if (ev) (void)hipEventRecord(static_cast<hipEvent_t>(ev), as_stream(stream));
   };
 
-  // 1. routing; on the int8 decode path together with step 3 (independent work, one launch)
+  // 0. router logits if the caller handed over the gate weight instead: split-K partial planes,
+  //    which the routing kernel adds up as it loads them (timed as part of the routing stage)
   const bool stream_mode = use_stream_path(a);
   bool quant_done = false;
   mark(KMOE_STAGE_ROUTING, 0);
+  const float* logits = a->logits;
+  int planes = 1;
+  size_t plane_stride = 0;
+  if (!logits) {
+    int mf = 0;
+    router_plan(M, H, E, &planes, &mf);
+    float* buf = static_cast<float*>(at(L.logit_planes));
+    plane_stride = static_cast<size_t>(M) * E;
+    rc = router_gemm_planes(a->x, H, a->w_gate, M, H, E, buf, plane_stride, E, planes, mf, as_stream(stream));
+    if (rc) return rc;
+    logits = buf;
+  }
+  // 1. routing; on the int8 decode path together with step 3 (independent work, one launch)
   if (a->format == KMOE_FMT_INT8 && M <= 1024) {
-    rc = fused_route_quant_i8(a->logits, a->bias, M, E, K, a->scoring == KMOE_SCORE_SIGMOID, a->renormalize, a->n_group,
+    rc = fused_route_quant_i8(logits, planes, plane_stride, a->bias, M, E, K, a->scoring == KMOE_SCORE_SIGMOID, a->renormalize, a->n_group,
                               a->topk_group, a->routed_scale, topk_w, topk_ids, a->x, H, static_cast<int8_t*>(at(L.xq)),
                               static_cast<float*>(at(L.xmax)), stream_mode ? 1 : 0, as_stream(stream));
     if (rc < 0) return rc;
     quant_done = rc == KMOE_OK;
     rc = KMOE_OK;
   }
+  if (!quant_done && planes > 1) {  // the stand-alone routing kernels take finished logits: add the planes into plane 0
+    rc = router_reduce(logits, plane_stride, planes, M, E, static_cast<float*>(at(L.logit_planes)), E, as_stream(stream));
+    if (rc) return rc;
+  }
   if (quant_done) {
     // both done
   } else if (a->scoring == KMOE_SCORE_SOFTMAX) {
-    rc = kmoe_softmax_topk(a->logits, M, E, K, a->renormalize, topk_w, topk_ids, stream);
+    rc = kmoe_softmax_topk(logits, M, E, K, a->renormalize, topk_w, topk_ids, stream);
   } else {
-    rc = kmoe_sigmoid_group_topk_norm(a->logits, a->bias, M, E, K, a->n_group, a->topk_group, a->routed_scale, topk_w,
+    rc = kmoe_sigmoid_group_topk_norm(logits, a->bias, M, E, K, a->n_group, a->topk_group, a->routed_scale, topk_w,
                                       topk_ids, stream);
   }
   if (rc) return rc;

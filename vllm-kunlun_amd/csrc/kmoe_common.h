@@ -22,9 +22,18 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);
 int tiled_gemm_fp8(const kmoe_gemm_fp8_args* args, hipStream_t stream);
 // Routing + per-token int8 quantisation of x [M,H] in one launch. Returns 1 (nothing launched)
 // when the arguments are outside its instantiations: the caller then uses the two entry points.
-int fused_route_quant_i8(const float* logits, const float* bias, int M, int E, int K, int sigmoid, int renorm,
+int fused_route_quant_i8(const float* logits, int planes, size_t plane_stride, const float* bias, int M, int E, int K, int sigmoid, int renorm,
                          int n_group, int topk_group, float scale, float* topk_w, int32_t* topk_ids,
                          const uint16_t* x, int H, int8_t* xq, float* xmax, int chunked, hipStream_t stream);
+
+// Router GEMM pieces for the fused layer: the split (ks planes, mf*16 tokens per wave) chosen for
+// a shape, and the launch that leaves the partial planes [ks][M][E] (ks == 1: the logits).
+void router_plan(int M, int H, int E, int* ks_out, int* mf_out);
+int router_gemm_planes(const uint16_t* x, int64_t ld_x, const uint16_t* w, int M, int H, int E, float* planes,
+                       size_t plane_stride, int64_t ld_out, int ks, int mf, hipStream_t stream);
+// out[m,e] = planes[0][m,e] + planes[1][m,e] + ... (that order); out may be plane 0 itself.
+int router_reduce(const float* planes, size_t plane_stride, int n_planes, int M, int E, float* out, int64_t ld_out,
+                  hipStream_t stream);
 
 #define KMOE_REQUIRE(cond, code, ...) \
   do {                                \

@@ -10,7 +10,9 @@ namespace kmoe {
 namespace {
 
 struct RouteArgs {
-  const float* logits;
+  const float* logits;  // [planes][M][E]; the logit is the sum over planes, plane 0 first
+  int planes;
+  size_t plane_stride;
   const float* bias;
   int M, E, K, renorm, n_group, topk_group;
   float scale;
@@ -32,10 +34,10 @@ __global__ __launch_bounds__(256) void route_quant_kernel(const RouteArgs r, con
   extern __shared__ float choice_lds[];  // sigmoid routing: [kWavesPerBlock][E]
   if (static_cast<int>(blockIdx.x) < routing_blocks) {
     if (SIGMOID)
-      sigmoid_group_topk_body<SLOTS>(r.logits, r.bias, r.M, r.E, r.K, r.n_group, r.topk_group, r.scale, r.topk_w,
+      sigmoid_group_topk_body<SLOTS>(r.logits, r.planes, r.plane_stride, r.bias, r.M, r.E, r.K, r.n_group, r.topk_group, r.scale, r.topk_w,
                                      r.topk_ids, choice_lds, blockIdx.x);
     else
-      softmax_topk_body<SLOTS>(r.logits, r.M, r.E, r.K, r.renorm, r.topk_w, r.topk_ids, blockIdx.x);
+      softmax_topk_body<SLOTS>(r.logits, r.planes, r.plane_stride, r.M, r.E, r.K, r.renorm, r.topk_w, r.topk_ids, blockIdx.x);
   } else {
     quant_i8_rows_body<TPR, NV>(q.x, q.ld_x, q.R, q.C, q.q, q.ld_q, q.row_max, q.chunked,
                                 static_cast<int>(blockIdx.x) - routing_blocks);
@@ -64,7 +66,7 @@ void launch_q(const RouteArgs& r, const QuantArgs& q, hipStream_t s) {
 // Returns KMOE_OK after a launch, a negative code on a launch error, or 1 when the
 // arguments are outside what the fused kernel is instantiated for (nothing launched:
 // the caller runs the two stand-alone entry points, which also report bad arguments).
-int fused_route_quant_i8(const float* logits, const float* bias, int M, int E, int K, int sigmoid, int renorm,
+int fused_route_quant_i8(const float* logits, int planes, size_t plane_stride, const float* bias, int M, int E, int K, int sigmoid, int renorm,
                          int n_group, int topk_group, float scale, float* topk_w, int32_t* topk_ids,
                          const uint16_t* x, int H, int8_t* xq, float* xmax, int chunked, hipStream_t s) {
   if (M <= 0 || E < 1 || E > 512 || K < 1 || K > E || K > kWave) return 1;
@@ -78,7 +80,7 @@ int fused_route_quant_i8(const float* logits, const float* bias, int M, int E, i
       return 1;
     }
   }
-  const RouteArgs r{logits, bias, M, E, K, renorm, n_group, topk_group, scale, topk_w, topk_ids};
+  const RouteArgs r{logits, planes, plane_stride, bias, M, E, K, renorm, n_group, topk_group, scale, topk_w, topk_ids};
   const QuantArgs q{x, H, M, H, xq, chunked ? 0 : H, xmax, chunked};
   const int slots = ceil_div(E, kWave);
   if (sigmoid) {

@@ -9,7 +9,7 @@ template <int SLOTS>
 __global__ __launch_bounds__(kWavesPerBlock* kWave) void softmax_topk_kernel(
     const float* __restrict__ logits, int M, int E, int K, int renorm, float* __restrict__ topk_w,
     int32_t* __restrict__ topk_ids) {
-  softmax_topk_body<SLOTS>(logits, M, E, K, renorm, topk_w, topk_ids, blockIdx.x);
+  softmax_topk_body<SLOTS>(logits, 1, 0, M, E, K, renorm, topk_w, topk_ids, blockIdx.x);
 }
 
 template <int SLOTS>
@@ -18,7 +18,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void sigmoid_group_topk_kern
     int n_group, int topk_group, float scale, float* __restrict__ topk_w,
     int32_t* __restrict__ topk_ids) {
   extern __shared__ float choice_lds[];  // [kWavesPerBlock][E]
-  sigmoid_group_topk_body<SLOTS>(logits, bias, M, E, K, n_group, topk_group, scale, topk_w, topk_ids, choice_lds,
+  sigmoid_group_topk_body<SLOTS>(logits, 1, 0, bias, M, E, K, n_group, topk_group, scale, topk_w, topk_ids, choice_lds,
                                  blockIdx.x);
 }
 

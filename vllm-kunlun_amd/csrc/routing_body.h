@@ -31,11 +31,27 @@ __device__ inline void select_topk(const float (&score)[SLOTS], const bool (&eli
   }
 }
 
+// Logit of (token row, expert e): the sum, plane 0 first, of `planes` partial planes that lie
+// `plane_stride` floats apart (what a split-K router GEMM leaves); planes == 1: the logit itself.
+__device__ inline float load_logit(const float* __restrict__ row, int e, int planes, size_t plane_stride) {
+  float v = row[e];
+  if (planes > 1) {  // at most 8 planes: request them all, then add in plane order
+    float t[7];
+#pragma unroll
+    for (int p = 1; p < 8; ++p) t[p - 1] = p < planes ? row[e + p * plane_stride] : 0.0f;
+#pragma unroll
+    for (int p = 1; p < 8; ++p)
+      if (p < planes) v = v + t[p - 1];
+  }
+  return v;
+}
+
 // One wave per token: workgroup `block` of kWavesPerBlock waves serves tokens
 // block * kWavesPerBlock + wave.
 template <int SLOTS>
-__device__ inline void softmax_topk_body(const float* __restrict__ logits, int M, int E, int K, int renorm,
-                                         float* __restrict__ topk_w, int32_t* __restrict__ topk_ids, int block) {
+__device__ inline void softmax_topk_body(const float* __restrict__ logits, int planes, size_t plane_stride, int M,
+                                         int E, int K, int renorm, float* __restrict__ topk_w,
+                                         int32_t* __restrict__ topk_ids, int block) {
   const int lane = lane_id();
   const int m = block * kWavesPerBlock + (threadIdx.x >> 6);
   if (m >= M) return;
@@ -48,7 +64,7 @@ __device__ inline void softmax_topk_body(const float* __restrict__ logits, int M
   for (int s = 0; s < SLOTS; ++s) {
     const int e = lane + kWave * s;
     ok[s] = e < E;
-    v[s] = ok[s] ? row[e] : -__builtin_inff();
+    v[s] = ok[s] ? load_logit(row, e, planes, plane_stride) : -__builtin_inff();
     mx = fmaxf(mx, v[s]);
   }
   mx = wave_max(mx);
@@ -91,8 +107,9 @@ __device__ inline void softmax_topk_body(const float* __restrict__ logits, int M
 
 // choice_lds: [kWavesPerBlock][E] floats of (dynamic) LDS.
 template <int SLOTS>
-__device__ inline void sigmoid_group_topk_body(const float* __restrict__ logits, const float* __restrict__ bias, int M,
-                                               int E, int K, int n_group, int topk_group, float scale,
+__device__ inline void sigmoid_group_topk_body(const float* __restrict__ logits, int planes, size_t plane_stride,
+                                               const float* __restrict__ bias, int M, int E, int K, int n_group,
+                                               int topk_group, float scale,
                                                float* __restrict__ topk_w, int32_t* __restrict__ topk_ids,
                                                float* choice_lds, int block) {
   const int lane = lane_id();
@@ -112,7 +129,7 @@ __device__ inline void sigmoid_group_topk_body(const float* __restrict__ logits,
     sg[s] = 0.0f;
     c[s] = -__builtin_inff();
     if (ok[s]) {
-      sg[s] = sigmoid_fixed(row[e]);
+      sg[s] = sigmoid_fixed(load_logit(row, e, planes, plane_stride));
       c[s] = bias ? sg[s] + bias[e] : sg[s];
       choice[e] = c[s];
     }

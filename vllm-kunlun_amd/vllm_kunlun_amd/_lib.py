@@ -67,7 +67,7 @@ class MoEArgs(C.Structure):
         ("x", C.c_void_p), ("w13", C.c_void_p), ("w13_max", C.c_void_p), ("w2", C.c_void_p), ("w2_max", C.c_void_p),
         ("I_shared", C.c_int32), ("ws13", C.c_void_p), ("ws13_max", C.c_void_p), ("ws2", C.c_void_p),
         ("ws2_max", C.c_void_p), ("out_scale", C.c_float), ("out", C.c_void_p),
-        ("stage_events", C.POINTER(C.c_void_p)), ("w_layout", C.c_int32),
+        ("stage_events", C.POINTER(C.c_void_p)), ("w_layout", C.c_int32), ("w_gate", C.c_void_p),
     ]
 
 
@@ -75,7 +75,7 @@ class MoELayout(C.Structure):
     _fields_ = [(n, C.c_size_t) for n in (
         "total_bytes", "topk_w", "topk_ids", "moe_index", "sorted_src", "expert_m", "lod", "align_ws",
         "xq", "xmax", "act", "actq", "actmax", "down", "sh_lod", "sh_act", "sh_actq", "sh_actmax", "sh_out",
-        "codes_chunked")]
+        "codes_chunked", "logit_planes", "n_logit_planes")]
 
 
 def _load() -> C.CDLL:
@@ -97,6 +97,8 @@ def _load() -> C.CDLL:
         "kmoe_quant_i8_rows": (i32, [vp, i64, i32, i32, vp, i64, vp, vp]),
         "kmoe_quant_i8_rows_chunked": (i32, [vp, i64, i32, i32, vp, vp, vp]),
         "kmoe_tile_weights_i8": (i32, [vp, vp, i32, i32, i32, vp]),
+        "kmoe_router_gemm_workspace_bytes": (sz, [i32, i32, i32]),
+        "kmoe_router_gemm_bf16": (i32, [vp, i64, vp, i32, i32, i32, vp, i64, vp, sz, vp]),
         "kmoe_quant_fp8_group128": (i32, [vp, i64, i32, i32, vp, i64, vp, vp]),
         "kmoe_grouped_gemm_i8": (i32, [C.POINTER(GemmI8Args), vp]),
         "kmoe_silu_and_mul": (i32, [vp, i64, i32, i32, vp, i64, vp]),
@@ -118,7 +120,7 @@ EXPORTS = (
     "kmoe_last_error", "kmoe_version", "kmoe_softmax_topk", "kmoe_sigmoid_group_topk_norm", "kmoe_block_statistic",
     "kmoe_align_workspace_bytes", "kmoe_align", "kmoe_gather_rows", "kmoe_quant_i8_rows", "kmoe_quant_i8_rows_chunked", "kmoe_tile_weights_i8", "kmoe_quant_fp8_group128",
     "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
-    "kmoe_moe_workspace_layout", "kmoe_moe_forward",
+    "kmoe_moe_workspace_layout", "kmoe_moe_forward", "kmoe_router_gemm_workspace_bytes", "kmoe_router_gemm_bf16",
 )
 
 

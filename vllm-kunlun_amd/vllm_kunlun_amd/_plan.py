@@ -94,23 +94,30 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
                   scoring_func: str = "softmax", renormalize: bool = True, num_expert_group: Optional[int] = None,
                   topk_group: Optional[int] = None, routed_scaling_factor: float = 1.0,
                   e_score_correction_bias: Optional[torch.Tensor] = None, shared_expert=None, out_scale: float = 1.0,
-                  stage_events=None, w_layout: Optional[int] = None) -> MoEPlan:
+                  stage_events=None, w_layout: Optional[int] = None,
+                  router_weight: Optional[torch.Tensor] = None) -> MoEPlan:
     """x bf16 [M,H], logits f32 [M,E], out bf16 [M,H]; w13 [E,2I,H], w2 [E,H,I] in the
     format's dtype; w13_aux/w2_aux: per-channel maxes (int8) or block scales (fp8), None for bf16.
-    shared_expert: (ws13 [2Is,H], ws13_aux, ws2 [H,Is], ws2_aux) in the same format."""
+    shared_expert: (ws13 [2Is,H], ws13_aux, ws2 [H,Is], ws2_aux) in the same format.
+    logits may be None when router_weight (bf16 [E,H], the gate projection) is given: the
+    layer then computes the router logits itself."""
     if scoring_func not in ("softmax", "sigmoid"):
         raise ValueError(f"Unsupported scoring_func: {scoring_func}")
-    tensors = [x, logits, out, w13, w2, w13_aux, w2_aux, e_score_correction_bias]
+    if logits is None and router_weight is None:
+        raise ValueError("moe plan: either router logits or the router weight is needed")
+    tensors = [x, logits, out, w13, w2, w13_aux, w2_aux, e_score_correction_bias, router_weight]
     L.require_device(*tensors)
     L.require_contig(*tensors)
-    if x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or logits.dtype != torch.float32:
+    if x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or (logits is not None and logits.dtype != torch.float32):
         raise ValueError("moe plan: x/out must be bfloat16 and logits float32")
     if w13.dtype not in _WEIGHT_DTYPE[fmt] or w2.dtype != w13.dtype:
         raise ValueError(f"moe plan: weight dtype {w13.dtype} does not fit the layer format")
     E, two_i, H = w13.shape
     M = x.shape[0]
-    if tuple(x.shape) != (M, H) or tuple(out.shape) != (M, H) or tuple(logits.shape) != (M, E):
+    if tuple(x.shape) != (M, H) or tuple(out.shape) != (M, H) or (logits is not None and tuple(logits.shape) != (M, E)):
         raise ValueError("moe plan: x/out must be [M,H] and logits [M,E]")
+    if logits is None and (router_weight.dtype != torch.bfloat16 or tuple(router_weight.shape) != (E, H)):
+        raise ValueError("moe plan: router_weight must be bfloat16 [E,H]")
     if tuple(w2.shape) != (E, H, two_i // 2):
         raise ValueError("moe plan: w2 must be [E,H,I] for w13 [E,2I,H]")
     a = L.MoEArgs()
@@ -121,7 +128,8 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     a.n_group = int(num_expert_group or 1)
     a.topk_group = int(topk_group or 1)
     a.routed_scale = float(routed_scaling_factor)
-    a.logits = logits.data_ptr()
+    a.logits = 0 if logits is None else logits.data_ptr()
+    a.w_gate = 0 if logits is not None or router_weight is None else router_weight.data_ptr()
     a.bias = 0 if e_score_correction_bias is None else e_score_correction_bias.data_ptr()
     a.x = x.data_ptr()
     a.w13, a.w2 = w13.data_ptr(), w2.data_ptr()

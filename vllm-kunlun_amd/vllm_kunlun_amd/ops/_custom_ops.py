@@ -323,6 +323,29 @@ def moe_post(x: torch.Tensor, moe_index: torch.Tensor, normed_scale: torch.Tenso
 
 
 # Fake (meta) implementations so the ops can be traced, as the reference registers for each op.
+@custom_op("_C::router_gemm_bf16_fp32", mutates_args=())
+def router_gemm_bf16_fp32(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """bf16 [M,H] x bf16 [E,H]^T -> f32 [M,E] router logits (reference: ops.router_gemm_bf16_fp32,
+    ops/fused_moe/router/gate_linear.py:105-108)."""
+    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "router_gemm_bf16_fp32: bf16 inputs only")
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "router_gemm_bf16_fp32: shapes")
+    L.require_device(x, weight)
+    x, weight = x.contiguous(), weight.contiguous()
+    M, H = x.shape
+    E = weight.shape[0]
+    out = torch.empty((M, E), dtype=torch.float32, device=x.device)
+    nbytes = L.lib.kmoe_router_gemm_workspace_bytes(M, H, E)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    L.check(L.lib.kmoe_router_gemm_bf16(L.ptr(x), H, L.ptr(weight), M, H, E, L.ptr(out), E, L.ptr(ws), nbytes,
+                                        L.stream()))
+    return out
+
+
+@router_gemm_bf16_fp32.register_fake
+def _fake_router_gemm(x, weight):
+    return x.new_empty((x.shape[0], weight.shape[0]), dtype=torch.float32)
+
+
 def _none(*args, **kwargs):
     return None
 

@@ -131,24 +131,28 @@ class _MonolithicQuantMoE:
         e_score_correction_bias: Optional[torch.Tensor] = None,
         shared_expert=None,
         out_scale: float = 1.0,
+        router_weight: Optional[torch.Tensor] = None,
     ) -> Union[torch.Tensor, tuple]:
         """x [M,H] bf16, router_logits [M,E] -> [M,H] bf16 (reference: :122-291).
         `shared_expert` (w13, w13_max, w2, w2_max of a dense MLP in the layer's format) and
-        `out_scale` fold the caller's epilogue (models/deepseek_v2.py:288-296) into the call."""
+        `out_scale` fold the caller's epilogue (models/deepseek_v2.py:288-296) into the call;
+        with `router_logits=None` and `router_weight` (the bf16 [E,H] weight of the gate,
+        models/deepseek_v2.py:178-184) the gate projection of :275 runs inside the call too."""
         if x.dtype != torch.bfloat16:
             raise NotImplementedError(f"apply_monolithic: activations must be bfloat16, got {x.dtype}")
         x = x.contiguous()
-        logits = router_logits.float().contiguous()
+        logits = None if router_logits is None else router_logits.float().contiguous()
         out = torch.empty((x.shape[0], layer.w2_weight.shape[1]), dtype=x.dtype, device=x.device)
         plan = self.make_plan(layer, x, logits, out, topk_group, num_expert_group, scoring_func,
-                              routed_scaling_factor, e_score_correction_bias, shared_expert, out_scale)
+                              routed_scaling_factor, e_score_correction_bias, shared_expert, out_scale,
+                              router_weight=router_weight)
         plan()
         self.last_layout, self.last_workspace = plan.layout, plan.workspace  # lets tests read the intermediates
         return out
 
     def make_plan(self, layer, x, logits, out, topk_group=None, num_expert_group=None, scoring_func="softmax",
                   routed_scaling_factor=1.0, e_score_correction_bias=None, shared_expert=None, out_scale=1.0,
-                  stage_events=None) -> MoEPlan:
+                  stage_events=None, router_weight=None) -> MoEPlan:
         """Argument block for repeated calls on fixed buffers (x bf16 [M,H], logits f32
         [M,E], out bf16 [M,H], all contiguous): what a serving loop or a HIP-graph
         capture replays without touching Python-side allocation."""
@@ -158,7 +162,7 @@ class _MonolithicQuantMoE:
                              layer.w2_weight, layer.w13_weight_scale, layer.w2_weight_scale, scoring_func,
                              True,  # the reference always routes with the *_norm kernels
                              num_expert_group, topk_group, routed_scaling_factor, bias, shared_expert, out_scale,
-                             stage_events)
+                             stage_events, router_weight=router_weight)
 
 
 class KunlunCompressedTensorsW8A8Int8MoEMethod(_MonolithicQuantMoE):

@@ -94,6 +94,82 @@ class FusedMoE(torch.nn.Module):
             raise RuntimeError("only monolithic MoE methods are served by this build")
         return self.quant_method.apply_monolithic(self, hidden_states, router_logits)
 
+    # ---- checkpoint -> parameters (reference use: models/deepseek_v2.py:1285-1384) ----
+    @classmethod
+    def make_expert_params_mapping(cls, ckpt_gate_proj_name: str, ckpt_down_proj_name: str,
+                                   ckpt_up_proj_name: str, num_experts: int,
+                                   num_redundant_experts: int = 0) -> list[tuple[str, str, int, str]]:
+        """(param_name, weight_name, expert_id, shard_id) for every expert projection, as the
+        model's load_weights expects (models/deepseek_v2.py:1296-1302): a checkpoint tensor
+        whose name contains `weight_name` ("experts.7.up_proj.") belongs to the stacked
+        parameter named by replacing that piece with `param_name` ("experts.w13_"), at
+        expert 7, shard w3. Redundant experts (expert-parallel load balancing) are not
+        served on one GPU."""
+        if num_redundant_experts:
+            raise NotImplementedError("redundant experts belong to expert parallelism, which this build does not span")
+        out = []
+        for e in range(num_experts):
+            for shard_id, proj in (("w1", ckpt_gate_proj_name), ("w2", ckpt_down_proj_name), ("w3", ckpt_up_proj_name)):
+                param = "experts.w13_" if shard_id in ("w1", "w3") else "experts.w2_"
+                out.append((param, f"experts.{e}.{proj}.", e, shard_id))
+        return out
+
+    def weight_loader(self, param: torch.nn.Parameter, loaded_weight: torch.Tensor, weight_name: str,
+                      shard_id: str, expert_id: int, return_success: bool = False):
+        """Copies one projection (or its scales) of one expert into the stacked parameter:
+        w1 -> rows [0, n/2) of w13 (gate), w3 -> rows [n/2, n) (up), w2 -> all of w2. Row
+        counts follow the parameter, so weights [2I,H], per-channel scales [2I,1] and block
+        scales [2I/128, H/128] all load through here. Must run BEFORE
+        process_weights_after_loading (which re-tiles the codes in place)."""
+        if shard_id not in ("w1", "w2", "w3"):
+            raise ValueError(f"shard_id must be w1, w2 or w3, got {shard_id}")
+        if getattr(param, "_kmoe_tiled", False):
+            raise RuntimeError("weight_loader: this parameter was already re-tiled by process_weights_after_loading")
+        if not 0 <= expert_id < param.shape[0]:
+            return False if return_success else None
+        dst = param.data[expert_id]
+        if shard_id != "w2":
+            half = dst.shape[0] // 2
+            dst = dst[:half] if shard_id == "w1" else dst[half:]
+        src = loaded_weight
+        if src.dim() == dst.dim() - 1:  # per-channel scales stored as [n]
+            src = src.unsqueeze(-1)
+        if tuple(src.shape) != tuple(dst.shape):
+            raise ValueError(f"{weight_name}: checkpoint tensor {tuple(loaded_weight.shape)} does not fit "
+                             f"{tuple(dst.shape)} (expert {expert_id}, shard {shard_id})")
+        if src.dtype != dst.dtype and src.element_size() == 1 and dst.element_size() == 1:
+            src = src.view(dst.dtype)  # e4m3 codes stored as uint8
+        dst.copy_(src)
+        return True if return_success else None
+
+    def load_weights(self, weights, ckpt_gate_proj_name: str = "gate_proj", ckpt_down_proj_name: str = "down_proj",
+                     ckpt_up_proj_name: str = "up_proj") -> set:
+        """Loads every tensor of `weights` (an iterable of (name, tensor), e.g. from safetensors)
+        that names an expert projection of this layer: "...experts.<e>.<proj>.weight",
+        ".weight_scale". Returns the names consumed; other names are left to the caller."""
+        mapping = self.make_expert_params_mapping(ckpt_gate_proj_name, ckpt_down_proj_name, ckpt_up_proj_name,
+                                                  self.global_num_experts)
+        by_piece = {weight_name: (param_name, e, shard) for param_name, weight_name, e, shard in mapping}
+        params = dict(self.named_parameters())
+        loaded = set()
+        for name, tensor in weights:
+            i = name.find("experts.")
+            if i < 0:
+                continue
+            parts = name[i:].split(".")  # experts, <e>, <proj>, <suffix...>
+            if len(parts) < 4 or not parts[1].isdigit():
+                continue
+            piece = ".".join(parts[:3]) + "."
+            if piece not in by_piece:
+                continue
+            param_name, e, shard = by_piece[piece]
+            target = param_name.split(".", 1)[1] + ".".join(parts[3:])  # "w13_" + "weight_scale"
+            if target not in params:
+                continue
+            self.weight_loader(params[target], tensor, name, shard_id=shard, expert_id=e)
+            loaded.add(name)
+        return loaded
+
 
 class SharedFusedMoE(FusedMoE):
     """FusedMoE plus a dense shared expert evaluated on the same input; returns

@@ -34,6 +34,8 @@ WORKLOAD_LABEL = {
     "dsv3-fp8-prefill": "DeepSeek-V3-shape MoE layer (+1 shared expert), fp8-e4m3 128x128-block weights, prefill, 4096 tokens",
     "kimi-fp8-decode": "Kimi-K2-shape MoE layer (384 experts, +1 shared), fp8-e4m3 128x128-block weights, decode, 128 tokens",
     "kimi-fp8-prefill": "Kimi-K2-shape MoE layer (384 experts, +1 shared), fp8-e4m3 128x128-block weights, prefill, 4096 tokens",
+    "qwen3-bf16-decode": "Qwen3-MoE-30B-A3B-shape MoE layer, bf16 weights (no quantization), decode, 64 tokens",
+    "qwen3-bf16-prefill": "Qwen3-MoE-30B-A3B-shape MoE layer, bf16 weights (no quantization), prefill, 8192 tokens",
     "tiny-bf16": "tiny bf16 MoE layer (32 tokens, hidden 512, 8 experts, top-2, intermediate 256), no quantization",
 }
 PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0, "none": 2500.0}  # MI355X dense MFMA: int8, fp8, bf16
@@ -246,8 +248,9 @@ def main():
         achieved = work["g1_ops"] / g1_s / 1e12
         roofline = {"bound": "mfma", "achieved": achieved, "peak": peak_tops, "unit": "TFLOP/s",
                     "frac": achieved / peak_tops, "traffic": measured_traffic(a.workload)}
-    g1_kernel = ("grouped_gemm_kernel" if shape.quant != "int8" else
-                 "stream_gemm_i8_kernel" if plan.layout.codes_chunked else "tiled_gemm_i8_kernel")
+    many_rows = shape.P > 48 * shape.E  # the launchers' switch to the persistent 128-row-tile kernel
+    g1_kernel = ("stream_gemm_i8_kernel" if plan.layout.codes_chunked else
+                 "tiled_gemm_kernel" if many_rows and plan.args.w_layout == L.KMOE_W_TILED else "grouped_gemm_kernel")
     roofline.update(kernel=g1_kernel + " (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
                     algorithmic_bytes=work["g1_bytes"], algorithmic_ops=work["g1_ops"])
 

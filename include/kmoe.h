@@ -229,6 +229,8 @@ typedef struct kmoe_gemm_bf16_args {
   int64_t ldy;
   int32_t act;
   int32_t variant;
+  int32_t w_layout;       /* KMOE_W_ROWMAJOR, or KMOE_W_TILED: the BYTES of w ([E, n, 2k])
+                             re-arranged by kmoe_tile_weights_i8(E, n, 2k); needs k % 32 == 0 */
 } kmoe_gemm_bf16_args;
 
 /*

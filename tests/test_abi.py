@@ -38,6 +38,7 @@ def test_struct_layouts_match_the_header(L):
     # sizes implied by the C declarations (LP64): guards the ctypes mirrors against drift
     assert C.sizeof(L.GemmI8Args) == 8 * 8 + 16 + 8 * 3 + 8 + 16 + 16 + 16  # 8 ptr/int64, 4 int32, y/ldy/acc_out, act+variant, 3 int32 + pad
     assert C.sizeof(L.MoELayout) == 22 * 8
+    assert C.sizeof(L.GemmBf16Args) == 6 * 8 + 16 + 16 + 16  # 6 ptr/int64 (src_div padded), 4 int32, y/ldy, act+variant+w_layout+pad
     assert C.sizeof(L.GemmFp8Args) == 8 * 8 + 16 + 16 + 16  # 8 ptr/int64, 4 int32, y/ldy, act+variant+w_layout+pad
     assert L.MoEArgs.w_gate.offset == C.sizeof(L.MoEArgs) - 8
     a = L.MoEArgs()

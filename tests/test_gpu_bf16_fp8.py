@@ -40,10 +40,33 @@ CASES = [
 ]
 
 
+BF16_TILED_CASES = [
+    (1, 64, 128, [16]),
+    (4, 64, 256, [3, 0, 17, 1]),
+    (2, 256, 1024, [130, 129]),
+    (3, 96, 320, [5, 140, 7]),                                    # 5 chunks of 128 bytes
+    (8, 128, 64, [4, 4, 0, 9, 33, 1, 0, 2]),
+    (20, 1024, 128, [((53 * i) % 300) for i in range(20)]),       # several tiles per workgroup walk
+]
+
+
+@pytest.mark.parametrize("E,n,k,counts", BF16_TILED_CASES)
+@pytest.mark.parametrize("variant", [1, 2, 3, 5])
+@pytest.mark.parametrize("act", [0, 1])
+def test_grouped_gemm_bf16_tiled_weights(L, E, n, k, counts, variant, act):
+    """bf16 weights re-arranged (as bytes) by kmoe_tile_weights_i8: the LDS-staged kernels (1-3) and
+    the persistent 128-row-tile kernel (5)."""
+    _bf16_case(L, E, n, k, counts, variant, act, tiled=True)
+
+
 @pytest.mark.parametrize("E,n,k,counts", CASES)
 @pytest.mark.parametrize("variant", [1, 2, 3])
 @pytest.mark.parametrize("act", [0, 1])
 def test_grouped_gemm_bf16(L, E, n, k, counts, variant, act):
+    _bf16_case(L, E, n, k, counts, variant, act, tiled=False)
+
+
+def _bf16_case(L, E, n, k, counts, variant, act, tiled):
     torch.manual_seed(E * n + k)
     lod = _lod(counts)
     rows = int(lod[-1])
@@ -54,6 +77,11 @@ def test_grouped_gemm_bf16(L, E, n, k, counts, variant, act):
     da, dw, dl = a.cuda(), w.cuda(), torch.from_numpy(lod).cuda()
     y = torch.zeros(rows, n_out, dtype=torch.bfloat16, device="cuda")
     g = L.GemmBf16Args()
+    if tiled:
+        dt = torch.empty_like(dw)
+        L.check(L.lib.kmoe_tile_weights_i8(dw.data_ptr(), dt.data_ptr(), E, n, 2 * k, L.stream()))
+        dw = dt
+        g.w_layout = L.KMOE_W_TILED
     g.a, g.lda, g.src_div = da.data_ptr(), k, 1
     g.w, g.lod = dw.data_ptr(), dl.data_ptr()
     g.E, g.n, g.k, g.rows = E, n, k, rows
@@ -148,13 +176,13 @@ def test_bf16_layer_config1_and_variants():
         sl = synth.make_bf16_layer(shape, "cuda", seed=5)
         out = sl.layer(sl.x, sl.logits)
         torch.cuda.synchronize()
-        lay = sl.layer
-        ref = co.forward_bf16(bits(sl.x), _host(sl.logits).numpy(), bits(lay.w13_weight), bits(lay.w2_weight), shape.K,
+        w13, _, w2, _, _ = sl.host_weights()  # row-major copies of the (tiled) device weights
+        ref = co.forward_bf16(bits(sl.x), _host(sl.logits).numpy(), bits(w13), bits(w2), shape.K,
                               shape.scoring, True, shape.n_group, shape.topk_group, 1.0,
                               None if sl.bias is None else _host(sl.bias).numpy())
         assert rel_l2(out, from_bits(ref)) <= REL_L2_BF16
         if shape.scoring == "softmax":  # the reference's own torch loop (fused_moe_ep)
-            ref_t = tm.bf16_moe(_host(sl.x), _host(sl.logits), _host(lay.w13_weight), _host(lay.w2_weight), shape.K,
+            ref_t = tm.bf16_moe(_host(sl.x), _host(sl.logits), w13, w2, shape.K,
                                 True)
             assert rel_l2(out, ref_t) <= REL_L2_BF16
 

@@ -47,9 +47,8 @@ int check_shape(const kmoe_moe_args* a) {
                "moe_forward: I_shared=%d must be a non-negative multiple of %d", a->I_shared, mult);
   KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "moe_forward: M*K too large");
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR ||
-                   (a->w_layout == KMOE_W_TILED && a->format != KMOE_FMT_BF16 && a->H % 64 == 0 && a->I % 64 == 0 &&
-                    a->I_shared % 64 == 0),
-               KMOE_ERR_SHAPE, "moe_forward: w_layout=%d needs int8 or fp8 weights and H, I multiples of 64", a->w_layout);
+                   (a->w_layout == KMOE_W_TILED && a->H % 64 == 0 && a->I % 64 == 0 && a->I_shared % 64 == 0),
+               KMOE_ERR_SHAPE, "moe_forward: w_layout=%d needs H, I multiples of 64", a->w_layout);
   return KMOE_OK;
 }
 
@@ -84,7 +83,7 @@ struct MlpPass {
   void* actq;      // [rows, I] codes
   float* act_aux;  // [rows] or [rows, I/128]
   uint16_t* out;   // [rows, H] bf16
-  int w_layout;    // INT8, FP8: KMOE_W_*
+  int w_layout;    // KMOE_W_*
   bool stream;     // INT8 + tiled weights: chunk-major codes and the weight-streaming GEMM
   int x_count;     // rows of x_rows (chunk-major addressing)
   // INT8 tail expert (folded shared expert): rows [rows, rows + tail_rows) of act/actq/out
@@ -170,6 +169,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
   g.y = y;
   g.ldy = ldy;
   g.act = act;
+  g.w_layout = m.w_layout;
   return kmoe_grouped_gemm_bf16(&g, stream);
 }
 

@@ -470,9 +470,17 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
                "grouped_gemm_bf16: misaligned tensor pointer");
   KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_bf16: src_div=%d < 1", a->src_div);
   if (a->rows == 0) return KMOE_OK;
+  KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR || (a->w_layout == KMOE_W_TILED && a->k % 32 == 0), KMOE_ERR_SHAPE,
+               "grouped_gemm_bf16: w_layout=%d (tiled weights need k %% 32 == 0, k=%d)", a->w_layout, a->k);
+  // many rows per expert and tiled weights: the persistent 128-row-tile kernel (variant 5 forces it)
+  if (a->w_layout == KMOE_W_TILED && a->k % 64 == 0 && a->ldy % 8 == 0 &&
+      (a->variant == 5 || (a->variant == 0 && ceil_div(a->rows, a->E) > 48)))
+    return tiled_gemm_bf16(a, as_stream(stream));
+  KMOE_REQUIRE(a->variant != 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variant 5 needs tiled weights, k %% 64 == 0");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), nullptr,    a->lod,  a->E,       a->n,
-               a->k * 2,                              a->y,       a->ldy,  nullptr, 0, nullptr, nullptr, 0, 0, 0};
+               a->k * 2,                              a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,
+               nullptr, nullptr, 0, 0, 0};
   return dispatch<Kind::BF16>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_bf16");
 }
 

@@ -20,6 +20,7 @@ int stream_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);
 // arguments already validated.
 int tiled_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);
 int tiled_gemm_fp8(const kmoe_gemm_fp8_args* args, hipStream_t stream);
+int tiled_gemm_bf16(const kmoe_gemm_bf16_args* args, hipStream_t stream);
 // Routing + per-token int8 quantisation of x [M,H] in one launch. Returns 1 (nothing launched)
 // when the arguments are outside its instantiations: the caller then uses the two entry points.
 int fused_route_quant_i8(const float* logits, int planes, size_t plane_stride, const float* bias, int M, int E, int K, int sigmoid, int renorm,

@@ -32,13 +32,16 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 // Operand format. F8: e4m3fn codes with block scales (one f32 per 128x128 weight block and
 // per activation row and 128 of K); one v_mfma_scale_f32_16x16x128_f8f6f4 covers a whole
 // 128-byte chunk (the two 1 KB weight blocks of a chunk are its two K halves, and the
 // activation fragment takes the same two halves), its partial sum is scaled and added in f32.
-enum class TKind { I8, F8 };
+// BF16: unscaled bf16 operands on v_mfma_f32_16x16x32_bf16; sizes along K are in BYTES here (a
+// 1 KB weight block holds 16 channels x 32 values, a 128-byte chunk two MFMA steps).
+enum class TKind { I8, F8, BF16 };
 constexpr int kMaxKBlocks = 64;  // F8: K <= 8192
 
 // Raw buffer descriptor over [base, base + 4 GiB): loads take a 32-bit per-lane offset
@@ -97,7 +100,9 @@ struct Tile {
 template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM>
 __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(const TiledParams p) {
   constexpr bool F8 = KIND == TKind::F8;
-  using acc_t = std::conditional_t<F8, v4f, v4i>;
+  constexpr bool I8 = KIND == TKind::I8;
+  constexpr bool BF = KIND == TKind::BF16;
+  using acc_t = std::conditional_t<I8, v4i, v4f>;
   constexpr int kTM = WM * 16 * kMF;             // rows of a tile
   constexpr int kThreads = WM * kWavesT * kWave;
   static_assert(R == 4 || R == 8, "the chunk buffer parity is static only for R/2 even");
@@ -108,8 +113,8 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   __shared__ __attribute__((aligned(16))) int8_t lds_a[2][kTM * kPitchT];
   __shared__ __attribute__((aligned(16))) int8_t patch[WM * kWavesT][16 * kPatchPitch];
   // I8, per tile parity: channel scales (w_max / 127) and row scales (a_max / 127)
-  __shared__ __attribute__((aligned(16))) float sw_lds[F8 ? 1 : 2][F8 ? 4 : kWavesT * NF * 16];
-  __shared__ float sa_lds[F8 ? 1 : 2][F8 ? 4 : kTM];
+  __shared__ __attribute__((aligned(16))) float sw_lds[I8 ? 2 : 1][I8 ? kWavesT * NF * 16 : 4];
+  __shared__ float sa_lds[I8 ? 2 : 1][I8 ? kTM : 4];
   // F8: weight block scales of the tile [parity][wave][fragment][k block], and the row scales
   // of the chunk in each activation buffer
   __shared__ float wsc_lds[F8 ? 2 : 1][F8 ? kWavesT * NF * kMaxKBlocks : 4];
@@ -225,8 +230,13 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     for (int mf = 0; mf < kMF; ++mf) {
       const v4i af = *reinterpret_cast<const v4i*>(&lds_a[buf][(wave_m * 16 * kMF + mf * 16 + li) * kPitchT + j * 64 + lg * 16]);
 #pragma unroll
-      for (int f = 0; f < kNF; ++f)
-        acc[mf][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wcur[f], af, acc[mf][f], 0, 0, 0);
+      for (int f = 0; f < kNF; ++f) {
+        if constexpr (BF)
+          acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wcur[f]),
+                                                               __builtin_bit_cast(v8bf, af), acc[mf][f], 0, 0, 0);
+        else if constexpr (I8)
+          acc[mf][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wcur[f], af, acc[mf][f], 0, 0, 0);
+      }
     }
   };
   // F8, one whole chunk: the two ring slots of the chunk are the K halves of one MFMA
@@ -312,7 +322,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
           wsc_reg[i] = kb < kblocks ? ws[kb] : 0.0f;
         }
       }
-    } else {
+    } else if constexpr (I8) {
       if (wave_m == 0 && (lane >> 4) < kNF) {  // thread (wave, f = lane / 16, c = lane % 16): scale of channel c of fragment f of this wave
         bool ok;
         const int c = col_of(t, lane >> 4, ok);
@@ -338,7 +348,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         for (int i = 0; i < kMaxKBlocks / 16; ++i)
           wsc_lds[parity][(wave * kNF + (lane >> 4)) * kMaxKBlocks + (lane & 15) + 16 * i] = wsc_reg[i];
       }
-    } else {
+    } else if constexpr (I8) {
       if (wave_m == 0 && (lane >> 4) < kNF) sw_lds[parity][wave * kNF * 16 + lane] = sw_reg / 127.0f;
       if (threadIdx.x < kTM) sa_lds[parity][threadIdx.x] = sa_reg / 127.0f;
     }
@@ -347,7 +357,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     for (int mf = 0; mf < kMF; ++mf)
 #pragma unroll
       for (int f = 0; f < kNF; ++f) {
-        if constexpr (F8) acc[mf][f] = (v4f){0.f, 0.f, 0.f, 0.f};
+        if constexpr (!I8) acc[mf][f] = (v4f){0.f, 0.f, 0.f, 0.f};
         else acc[mf][f] = (v4i){0, 0, 0, 0};
       }
     __syncthreads();
@@ -412,7 +422,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
 #pragma unroll
     for (int f = 0; f < kNF; ++f) {
       col[f] = col_of(done, f, wok[f]);
-      if constexpr (!F8) {
+      if constexpr (I8) {
         const float4 s4 = *reinterpret_cast<const float4*>(&sw_lds[parity][(wave * kNF + f) * 16 + lg * 4]);
         sw[f][0] = s4.x;
         sw[f][1] = s4.y;
@@ -430,14 +440,14 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
 #pragma unroll
     for (int mf = 0; mf < kMF; ++mf) {
       float sa = 1.0f;
-      if constexpr (!F8) sa = sa_lds[parity][wave_m * 16 * kMF + mf * 16 + li];
+      if constexpr (I8) sa = sa_lds[parity][wave_m * 16 * kMF + mf * 16 + li];
       const int r = done.row0 + wave_m * 16 * kMF + mf * 16 + li;
 #pragma unroll
       for (int f = 0; f < NFH; ++f) {
         float yv[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          if constexpr (F8) yv[q] = acc[mf][f][q];
+          if constexpr (!I8) yv[q] = acc[mf][f][q];
           else yv[q] = (static_cast<float>(acc[mf][f][q]) * sa) * sw[f][q];
         }
         if (SWIGLU) {
@@ -446,7 +456,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
           for (int q = 0; q < 4; ++q) {
             const float g = bf16_to_f32(f32_to_bf16_hw(yv[q]));  // gate and up are bf16 values first
             float uf;
-            if constexpr (F8) uf = acc[mf][fu][q];
+            if constexpr (!I8) uf = acc[mf][fu][q];
             else uf = (static_cast<float>(acc[mf][fu][q]) * sa) * sw[fu][q];
             const float u = bf16_to_f32(f32_to_bf16_hw(uf));
             yv[q] = silu_fixed(g) * u;
@@ -454,7 +464,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         }
         *reinterpret_cast<uint2*>(&my_patch[li * kPatchPitch + f * 32 + lg * 8]) =
             make_uint2(pack2_bf16(yv[0], yv[1]), pack2_bf16(yv[2], yv[3]));
-        if constexpr (!F8) {
+        if constexpr (I8) {
           if (p.acc_out && r < row_end && wok[f]) {
             *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[f] + lg * 4) = acc[mf][f];
             if (SWIGLU)
@@ -560,6 +570,21 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
   int n_cu = 0;
   if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
   constexpr TKind K = TKind::F8;
+  return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)
+                : launch_tiled<K, false, 4, 4, 2, 1>(p, a->rows, s, n_cu, what);
+}
+
+// bf16 operands: the same tiles on the byte view of the tensors ([E, n, 2k] bytes, tiled with
+// kmoe_tile_weights_i8; activations [rows, 2k] bytes).
+int tiled_gemm_bf16(const kmoe_gemm_bf16_args* a, hipStream_t s) {
+  const char* what = "kmoe_grouped_gemm_bf16 (tiled)";
+  const bool swiglu = a->act == KMOE_ACT_SWIGLU;
+  TiledParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
+                reinterpret_cast<const int8_t*>(a->w), nullptr, a->lod, a->E, a->n, a->k * 2, a->y, a->ldy, nullptr,
+                nullptr, nullptr, 0, 0, 0, 0, 0};
+  int n_cu = 0;
+  if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
+  constexpr TKind K = TKind::BF16;
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)
                 : launch_tiled<K, false, 4, 4, 2, 1>(p, a->rows, s, n_cu, what);
 }

@@ -52,17 +52,20 @@ def is_tiled(w: torch.Tensor) -> bool:
     return bool(getattr(w, "_kmoe_tiled", False))
 
 
-_ONE_BYTE = (torch.int8, torch.uint8, torch.float8_e4m3fn)
+_TILEABLE = (torch.int8, torch.uint8, torch.float8_e4m3fn, torch.bfloat16)
 
 
 def tile_int8_weights_(w: torch.Tensor) -> bool:
-    """Re-arranges one-byte weights (int8, or e4m3 codes) [..., n, k] IN PLACE into the
-    MFMA-ready 1 KB blocks of kmoe_tile_weights_i8 (one expert at a time through a scratch
-    copy) and marks the object. Returns False and leaves the tensor alone when the shape
-    does not allow it (n % 16, k % 64)."""
+    """Re-arranges weights [..., n, k] (int8, e4m3 codes, or bf16 — the kernel moves BYTES: a
+    1 KB block is 16 channels x 64 bytes of K) IN PLACE into the MFMA-ready blocks of
+    kmoe_tile_weights_i8 (one expert at a time through a scratch copy) and marks the object.
+    Returns False and leaves the tensor alone when the shape does not allow it (n % 16,
+    64 bytes of K)."""
     data = w.data
-    n, k = data.shape[-2], data.shape[-1]
-    if data.dtype not in _ONE_BYTE or not data.is_cuda or not data.is_contiguous() or n % 16 or k % 64:
+    if data.dtype not in _TILEABLE or not data.is_cuda or not data.is_contiguous():
+        return False
+    n, k = data.shape[-2], data.shape[-1] * data.element_size()  # k in bytes
+    if n % 16 or k % 64:
         return False
     if is_tiled(w):
         return True
@@ -79,7 +82,7 @@ def rowmajor_int8_weights(w: torch.Tensor) -> torch.Tensor:
     """A row-major [..., n, k] COPY of int8 weights, undoing tile_int8_weights_ if it was applied."""
     if not is_tiled(w):
         return w.data.clone()
-    n, k = w.shape[-2], w.shape[-1]
+    n, k = w.shape[-2], w.shape[-1] * w.element_size()  # k in bytes
     lead = w.shape[:-2]
     t = w.data.view(torch.int8).reshape(-1, n // 16, k // 64, 4, 16, 16).permute(0, 1, 4, 2, 3, 5)
     return t.reshape(*lead, n, k).contiguous().view(w.dtype)
@@ -149,7 +152,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     a.out = out.data_ptr()
     if w_layout is None:  # tiled only if every int8 weight of the call has been tiled
         ws_all = [w13, w2] + ([shared_expert[0], shared_expert[2]] if shared_expert is not None else [])
-        w_layout = L.KMOE_W_TILED if fmt != L.KMOE_FMT_BF16 and all(is_tiled(t) for t in ws_all) else L.KMOE_W_ROWMAJOR
+        w_layout = L.KMOE_W_TILED if all(is_tiled(t) for t in ws_all) else L.KMOE_W_ROWMAJOR
         if w_layout == L.KMOE_W_ROWMAJOR and any(is_tiled(t) for t in ws_all):
             raise ValueError("moe plan: routed and shared expert weights must be either all tiled or all row-major")
     a.w_layout = int(w_layout)

@@ -56,6 +56,12 @@ for _n in ("dsv3-decode", "dsv3-prefill", "kimi-decode", "kimi-prefill"):
     SHAPES[_f] = replace(SHAPES[_n], name=_f, quant="fp8")
 
 
+# the Qwen3 layers unquantized (bf16 weights): what KunlunOps.fused_moe serves
+for _n in ("qwen3-decode", "qwen3-prefill"):
+    _f = _n.replace("-", "-bf16-")
+    SHAPES[_f] = replace(SHAPES[_n], name=_f, quant="none")
+
+
 def make_layer(shape: MoEShape, device="cuda", seed: int = 0) -> "SynthLayer":
     """The synthetic layer of a shape in the format the shape names."""
     return {"int8": make_w8a8_layer, "fp8": make_fp8_layer, "none": make_bf16_layer}[shape.quant](shape, device, seed)
@@ -88,7 +94,7 @@ class SynthLayer:
         lay = self.layer
 
         def rm(t):
-            return (rowmajor_int8_weights(t) if t.element_size() == 1 else t).detach().cpu()
+            return rowmajor_int8_weights(t).detach().cpu()
 
         aux = lambda name: getattr(lay, name).detach().cpu() if hasattr(lay, name) else None  # noqa: E731
         shared = None

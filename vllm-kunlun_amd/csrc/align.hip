@@ -165,17 +165,30 @@ __global__ __launch_bounds__(kThreads) void align_scan_kernel(int E, int n_chunk
   __shared__ int base[kMaxE];
   const int e = threadIdx.x;
   int total = 0;
+  constexpr int kBatch = 8;  // loads of a batch are independent: one memory round trip per 8 chunks, not per chunk
   if (e < E) {
-    for (int c = 0; c < n_chunks; ++c) {
-      const int v = hist[static_cast<size_t>(c) * E + e];
-      hist[static_cast<size_t>(c) * E + e] = total;
-      total += v;
+    for (int c0 = 0; c0 < n_chunks; c0 += kBatch) {
+      int v[kBatch];
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) v[i] = c0 + i < n_chunks ? hist[static_cast<size_t>(c0 + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) {
+        if (c0 + i < n_chunks) hist[static_cast<size_t>(c0 + i) * E + e] = total;
+        total += v[i];
+      }
     }
   }
   scan_experts(total, E, scan, base, lod, expert_m);
   if (e < E) {
     const int b = base[e];
-    for (int c = 0; c < n_chunks; ++c) hist[static_cast<size_t>(c) * E + e] += b;
+    for (int c0 = 0; c0 < n_chunks; c0 += kBatch) {
+      int v[kBatch];
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) v[i] = c0 + i < n_chunks ? hist[static_cast<size_t>(c0 + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i)
+        if (c0 + i < n_chunks) hist[static_cast<size_t>(c0 + i) * E + e] = v[i] + b;
+    }
   }
 }
 

@@ -155,6 +155,8 @@ int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, int C,
 
 #define KMOE_ACT_NONE 0
 #define KMOE_ACT_SWIGLU 1 /* out[r,i] = silu(y[r,i]) * y[r,i+n/2], i < n/2 */
+#define KMOE_ACT_SWIGLUOAI 2 /* bf16 only: out[r,i] = (u+1) * g * sigmoid(alpha*g), g = min(y[r,2i], limit),
+                                u = clamp(y[r,2i+1], -limit, limit), i < n/2 (gate/up interleaved) */
 
 typedef struct kmoe_gemm_i8_args {
   const int8_t* a;        /* [a_rows, k] quantised activations, row stride lda  */
@@ -231,6 +233,10 @@ typedef struct kmoe_gemm_bf16_args {
   int32_t variant;
   int32_t w_layout;       /* KMOE_W_ROWMAJOR, or KMOE_W_TILED: the BYTES of w ([E, n, 2k])
                              re-arranged by kmoe_tile_weights_i8(E, n, 2k); needs k % 32 == 0 */
+  /* the expert-bias branch of KunlunOps.fused_moe (ops/_kunlun_ops.py:433-468): */
+  const uint16_t* bias;   /* NULL, or [E, n] bf16: y = bf16(bf16(gemm) + bias), before the activation;
+                             with KMOE_ACT_NONE or KMOE_ACT_SWIGLUOAI                  */
+  float act_alpha, act_limit; /* KMOE_ACT_SWIGLUOAI (the reference uses 1.702 and 7.0)    */
 } kmoe_gemm_bf16_args;
 
 /*
@@ -270,6 +276,15 @@ typedef struct kmoe_gemm_fp8_args {
  * Limits: k % 128 == 0, n % 128 == 0 (SwiGLU: n % 256 == 0).
  */
 int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* args, kmoe_stream_t stream);
+
+/*
+ * The gpt-oss activation on a stored, interleaved gate_up result. Replaces
+ * torch.ops._C.swigluoai_and_mul (ops/_custom_ops.py:728-742).
+ *   y [R,2I] bf16 -> out [R,I] bf16, out[r,i] = (u+1) * g * sigmoid(alpha*g),
+ *   g = min(y[r,2i], limit), u = clamp(y[r,2i+1], -limit, limit).
+ */
+int kmoe_swigluoai_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, float alpha,
+                           float limit, uint16_t* out, int64_t ld_out, kmoe_stream_t stream);
 
 /*
  * SiLU-and-mul on a stored gate_up result. Replaces kunlun_ops.swiglu
@@ -354,6 +369,12 @@ typedef struct kmoe_moe_args {
   int32_t w_layout;      /* INT8, FP8: KMOE_W_TILED if w13, w2 (and ws13, ws2) went
                             through kmoe_tile_weights_i8; else KMOE_W_ROWMAJOR  */
   const uint16_t* w_gate; /* NULL, or [E,H] bf16 router weight (used when logits is NULL) */
+  /* BF16 only, the expert-bias branch (ops/_kunlun_ops.py:433-468): */
+  const uint16_t* w13_bias; /* NULL, or [E,2I] bf16                                   */
+  const uint16_t* w2_bias;  /* NULL, or [E,H] bf16                                    */
+  int32_t activation;    /* KMOE_ACT_SWIGLU (0 means the same) or KMOE_ACT_SWIGLUOAI: w13
+                            then holds gate and up rows interleaved               */
+  float act_alpha, act_limit;
 } kmoe_moe_args;
 
 #define KMOE_STAGE_ROUTING 0

@@ -267,14 +267,46 @@ def _route(logits, K, scoring, renormalize, n_group, topk_group, routed_scale, b
     return sigmoid_group_topk_norm(logits, bias, K, n_group, topk_group, routed_scale)
 
 
+def swigluoai_and_mul(y_bits, alpha=1.702, limit=7.0):
+    y_bits = _c(y_bits, np.uint16)
+    R, two_i = y_bits.shape
+    out = np.zeros((R, two_i // 2), np.uint16)
+    lib().orc_swigluoai_and_mul(_p(y_bits), C.c_int64(two_i), R, two_i // 2, C.c_float(alpha), C.c_float(limit), _p(out),
+                                C.c_int64(two_i // 2))
+    return out
+
+
+def grouped_gemm_bf16_bias(a_bits, w_bits, bias_bits, lod, act=0, row_src=None, src_div=1, alpha=1.702, limit=7.0):
+    """The expert-bias branch: act 0 (none) or 2 (gpt-oss activation over interleaved columns)."""
+    a_bits = _c(a_bits, np.uint16)
+    w_bits = _c(w_bits, np.uint16)
+    bias_bits = None if bias_bits is None else _c(bias_bits, np.uint16)
+    lod = _c(lod, np.int32)
+    E, n, k = w_bits.shape
+    rows = int(lod[-1])
+    row_src = None if row_src is None else _c(row_src, np.int32)
+    n_out = n // 2 if act == 2 else n
+    y = np.zeros((rows, n_out), np.uint16)
+    lib().orc_grouped_gemm_bf16_bias(_p(a_bits), C.c_int64(a_bits.shape[1]), _p(row_src), int(src_div), _p(w_bits),
+                                     _p(bias_bits), _p(lod), E, n, k, _p(y), C.c_int64(n_out), int(act),
+                                     C.c_float(alpha), C.c_float(limit))
+    return y
+
+
 def forward_bf16(x_bits, logits, w13_bits, w2_bits, K, scoring="softmax", renormalize=True, n_group=1, topk_group=1,
-                 routed_scale=1.0, bias=None):
-    """Unquantized layer in the stage order of KunlunOps.fused_moe (ops/_kunlun_ops.py:412-637)."""
+                 routed_scale=1.0, bias=None, w13_bias=None, w2_bias=None, alpha=1.702, limit=7.0):
+    """Unquantized layer in the stage order of KunlunOps.fused_moe (ops/_kunlun_ops.py:412-637); with
+    expert biases, its gpt-oss branch (:433-468): interleaved gate/up, swigluoai."""
     E = w13_bits.shape[0]
     w, ids = _route(logits, K, scoring, renormalize, n_group, topk_group, routed_scale, bias)
     moe_index, src, _, lod = align(ids, E)
-    act = grouped_gemm_bf16(x_bits, w13_bits, lod, act=1, row_src=src, src_div=K)
-    down = grouped_gemm_bf16(act, w2_bits, lod)
+    if w13_bias is not None or w2_bias is not None:
+        act = grouped_gemm_bf16_bias(x_bits, w13_bits, w13_bias, lod, act=2, row_src=src, src_div=K, alpha=alpha,
+                                     limit=limit)
+        down = grouped_gemm_bf16_bias(act, w2_bits, w2_bias, lod)
+    else:
+        act = grouped_gemm_bf16(x_bits, w13_bits, lod, act=1, row_src=src, src_div=K)
+        down = grouped_gemm_bf16(act, w2_bits, lod)
     return combine(down, moe_index, w)
 
 

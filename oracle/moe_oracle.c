@@ -376,6 +376,55 @@ ORC_API void orc_grouped_gemm_bf16(const uint16_t* a, int64_t lda, const int32_t
   }
 }
 
+/* gpt-oss activation (swigluoai_and_mul, ops/_custom_ops.py:728-742): gate and up interleaved,
+ * g = min(gate, limit), u = clamp(up, -limit, limit), out = (u + 1) * g * sigmoid(alpha * g), computed
+ * in f32 from the bf16 inputs and rounded once (the reference rounds after each torch op; the
+ * difference is inside the bf16 tolerance). */
+static inline uint16_t swigluoai_bits(uint16_t gate, uint16_t up, float alpha, float limit) {
+  const float g = fminf(bf16_to_f32(gate), limit);
+  const float u = fminf(fmaxf(bf16_to_f32(up), -limit), limit);
+  const float glu = g * orc_sigmoid(g * alpha);
+  return f32_to_bf16((u + 1.0f) * glu);
+}
+
+ORC_API void orc_swigluoai_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, float alpha, float limit,
+                                   uint16_t* out, int64_t ld_out) {
+  for (int r = 0; r < R; ++r)
+    for (int i = 0; i < I; ++i)
+      out[(size_t)r * ld_out + i] = swigluoai_bits(y[(size_t)r * ld_y + 2 * i], y[(size_t)r * ld_y + 2 * i + 1], alpha, limit);
+}
+
+/* The expert-bias branch of KunlunOps.fused_moe (ops/_kunlun_ops.py:433-468) as a grouped GEMM:
+ * y = bf16(bf16(a . w^T) + bias[e]) (`gemm + bias` on bf16 tensors rounds twice), then, with
+ * act == 2, the gpt-oss activation over interleaved columns (n/2 outputs). bias may be NULL. */
+ORC_API void orc_grouped_gemm_bf16_bias(const uint16_t* a, int64_t lda, const int32_t* row_src, int src_div,
+                                        const uint16_t* w, const uint16_t* bias, const int32_t* lod, int E, int n,
+                                        int k, uint16_t* y, int64_t ldy, int act, float alpha, float limit) {
+  for (int e = 0; e < E; ++e) {
+    const int r0 = lod[e], r1 = lod[e + 1];
+    const uint16_t* we = w + (size_t)e * n * k;
+#pragma omp parallel for schedule(static)
+    for (int r = r0; r < r1; ++r) {
+      const int sr = row_src ? row_src[r] / src_div : r;
+      const uint16_t* ar = a + (size_t)sr * lda;
+      uint16_t prev = 0;
+      for (int c = 0; c < n; ++c) {
+        float s = 0.0f;
+        const uint16_t* wc = we + (size_t)c * k;
+        for (int i = 0; i < k; ++i) s += bf16_to_f32(ar[i]) * bf16_to_f32(wc[i]);
+        uint16_t v = f32_to_bf16(s);
+        if (bias) v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(bias[(size_t)e * n + c]));
+        if (act == 2) {
+          if (c & 1) y[(size_t)r * ldy + c / 2] = swigluoai_bits(prev, v, alpha, limit);
+          prev = v;
+        } else {
+          y[(size_t)r * ldy + c] = v;
+        }
+      }
+    }
+  }
+}
+
 /* fp8-e4m3fn block-scaled grouped GEMM (no reference counterpart; DeepSeek-V3 recipe):
  * per 128-wide K block the exact f32 sum of code products, times the activation
  * scale of (row, block) and the weight scale of (channel/128, block); blocks added in

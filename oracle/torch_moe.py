@@ -167,6 +167,40 @@ def bf16_moe(x, logits, w13, w2, K, renormalize=True):
     return (out.view(M, K, H) * w.unsqueeze(2)).sum(dim=1).to(x.dtype)
 
 
+def swigluoai_and_mul(x: torch.Tensor, alpha: float = 1.702, limit: float = 7.0) -> torch.Tensor:
+    """torch.ops._C.swigluoai_and_mul as the reference defines it (ops/_custom_ops.py:728-742)."""
+    gate, up = x[..., ::2], x[..., 1::2]
+    gate = gate.clamp(min=None, max=limit)
+    up = up.clamp(min=-limit, max=limit)
+    glu = gate * torch.sigmoid(gate * alpha)
+    return (up + 1) * glu
+
+
+def bf16_moe_bias(x, logits, w13, w2, w13_bias, w2_bias, K, alpha: float = 1.702, limit: float = 7.0):
+    """The expert-bias (gpt-oss) branch of KunlunOps.fused_moe restated line for line in meaning
+    (ops/_kunlun_ops.py:433-468): routing weights cast to the activation dtype, per-expert
+    `x @ w1.T + b1`, swigluoai, `@ w2.T + b2`, weighted sum over K in that dtype."""
+    M, H = x.shape
+    E = w13.shape[0]
+    w, ids = softmax_topk(logits, K, True)
+    w = w.to(x.dtype)
+    out = torch.zeros(M * K, H, dtype=x.dtype)
+    repeat_x = x.repeat_interleave(K, dim=0)
+    flat = ids.reshape(-1)
+    for e in range(E):
+        sel = flat == e
+        if sel.sum():
+            g1 = repeat_x[sel] @ w13[e].T
+            if w13_bias is not None:
+                g1 = g1 + w13_bias[e]
+            up_gate = swigluoai_and_mul(g1, alpha, limit)
+            g2 = up_gate @ w2[e].T
+            if w2_bias is not None:
+                g2 = g2 + w2_bias[e]
+            out[sel] = g2
+    return (out.view(M, K, H) * w.unsqueeze(2)).sum(dim=1).to(x.dtype)
+
+
 # -------------------------------------------------------------- fp8 (c5)
 FP8_MAX = 448.0
 

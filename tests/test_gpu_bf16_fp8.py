@@ -166,7 +166,7 @@ def _host(t):
 
 
 def test_bf16_layer_config1_and_variants():
-    """BASELINE config 1 (32 tokens, hidden 512, 8 experts, top-2 softmax, I=256, bf16)
+    """The small unquantized configuration (32 tokens, hidden 512, 8 experts, top-2 softmax, I=256, bf16)
     through FusedMoE -> KunlunUnquantizedFusedMoEMethod.apply_monolithic -> KunlunOps.fused_moe."""
     from vllm_kunlun_amd import synth
     for shape in (synth.SHAPES["tiny-bf16"],
@@ -254,3 +254,68 @@ def test_fp8_layer(name, base, over):
                       co.sigmoid_group_topk_norm(_host(sl.logits).numpy(), _host(sl.bias).numpy(), shape.K,
                                                  shape.n_group, shape.topk_group, shape.routed_scale))
     assert np.array_equal(ids.reshape(shape.M, shape.K), ids_ref)
+
+
+@pytest.mark.parametrize("E,n,k,counts", [(1, 64, 128, [16]), (4, 128, 256, [3, 0, 17, 40]), (3, 96, 776, [5, 40, 7])])
+@pytest.mark.parametrize("act", [0, 2])
+@pytest.mark.parametrize("tiled", [False, True])
+def test_grouped_gemm_bf16_bias_and_swigluoai(L, E, n, k, counts, act, tiled):
+    """The expert-bias branch of the bf16 GEMM: y = bf16(bf16(a.w^T) + bias), act 2 = gpt-oss activation."""
+    if tiled and (2 * k) % 64:
+        pytest.skip("tiled weights need 64 bytes of K")
+    torch.manual_seed(E + n + k + act)
+    lod = _lod(counts)
+    rows = int(lod[-1])
+    a = torch.randn(rows, k).bfloat16()
+    w = (torch.randn(E, n, k) * 0.05).bfloat16()
+    b = (torch.randn(E, n) * 0.3).bfloat16()
+    ref = co.grouped_gemm_bf16_bias(bits(a), bits(w), bits(b), lod, act=act)
+    n_out = n // 2 if act else n
+    da, dw, db, dl = a.cuda(), w.cuda(), b.cuda(), torch.from_numpy(lod).cuda()
+    y = torch.zeros(rows, n_out, dtype=torch.bfloat16, device="cuda")
+    g = L.GemmBf16Args()
+    if tiled:
+        dt = torch.empty_like(dw)
+        L.check(L.lib.kmoe_tile_weights_i8(dw.data_ptr(), dt.data_ptr(), E, n, 2 * k, L.stream()))
+        dw = dt
+        g.w_layout = L.KMOE_W_TILED
+    g.a, g.lda, g.src_div = da.data_ptr(), k, 1
+    g.w, g.lod, g.bias = dw.data_ptr(), dl.data_ptr(), db.data_ptr()
+    g.E, g.n, g.k, g.rows = E, n, k, rows
+    g.y, g.ldy, g.act, g.act_alpha, g.act_limit = y.data_ptr(), n_out, act, 1.702, 7.0
+    L.check(L.lib.kmoe_grouped_gemm_bf16(g, L.stream()))
+    torch.cuda.synchronize()
+    assert rel_l2(y, from_bits(ref)) <= 3e-3
+    g.act = 1  # SwiGLU with a bias is not a path of the reference
+    with pytest.raises(NotImplementedError):
+        L.check(L.lib.kmoe_grouped_gemm_bf16(g, L.stream()))
+
+
+def test_swigluoai_op_is_the_oracle_sequence():
+    import vllm_kunlun_amd  # noqa: F401
+    torch.manual_seed(2)
+    y = (torch.randn(37, 64) * 4).bfloat16()
+    got = torch.ops._C.swigluoai_and_mul(y.cuda())
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(got), co.swigluoai_and_mul(bits(y)))
+
+
+def test_fused_moe_expert_bias_branch():
+    """KunlunOps.fused_moe(..., w1_bias, w2_bias): the gpt-oss branch (ops/_kunlun_ops.py:433-468) against the
+    C oracle and the reference's torch loop restated."""
+    from vllm_kunlun_amd.ops._kunlun_ops import KunlunOps
+    torch.manual_seed(4)
+    M, H, E, K, I = 70, 128, 8, 4, 64
+    x = torch.randn(M, H).bfloat16()
+    logits = torch.randn(M, E)
+    w13 = (torch.randn(E, 2 * I, H) * 0.1).bfloat16()
+    w2 = (torch.randn(E, H, I) * 0.1).bfloat16()
+    b13 = (torch.randn(E, 2 * I) * 0.2).bfloat16()
+    b2 = (torch.randn(E, H) * 0.2).bfloat16()
+    out = KunlunOps.fused_moe(x.cuda(), w13.cuda(), w2.cuda(), logits.cuda(), 0, K, True, w1_bias=b13.cuda(),
+                              w2_bias=b2.cuda())
+    torch.cuda.synchronize()
+    ref = from_bits(co.forward_bf16(bits(x), logits.numpy(), bits(w13), bits(w2), K, w13_bias=bits(b13),
+                                    w2_bias=bits(b2)))
+    assert rel_l2(out, ref) <= REL_L2_BF16
+    assert rel_l2(out, tm.bf16_moe_bias(x, logits, w13, w2, b13, b2, K)) <= REL_L2_BF16

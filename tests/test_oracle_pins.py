@@ -456,3 +456,43 @@ def test_router_gemm_against_f64_matmul():
         ref = x.double() @ w.double().T
         assert np.array_equal(got, ref.float().numpy())
         assert np.allclose(abs_sum, (x.double().abs() @ w.double().abs().T).numpy(), rtol=1e-6)
+
+
+def test_swigluoai_matches_the_reference_definition_and_its_clamps():
+    """The C oracle's gpt-oss activation against the reference's own torch definition
+    (restated in oracle/torch_moe.py from ops/_custom_ops.py:728-742) evaluated in f32, and the
+    closed forms at the clamps: a dropped `+1`, a swapped gate/up or a missing clamp fails."""
+    torch.manual_seed(3)
+    y = (torch.randn(64, 96) * 4).bfloat16()
+    y[0, :8] = torch.tensor([9.0, 0.5, -3.0, 9.0, 0.0, 2.0, 1.0, -9.0]).bfloat16()
+    got = from_bits(co.swigluoai_and_mul(bits(y))).float()
+    ref = tm.swigluoai_and_mul(y.float())
+    assert rel_l2(got, ref) < 3e-3
+    assert torch.allclose(got, ref, rtol=2 ** -7, atol=1e-6)
+    a, lim = 1.702, 7.0
+    sig = lambda v: 1.0 / (1.0 + math.exp(-v))  # noqa: E731
+    want = [(0.5 + 1) * lim * sig(a * lim),      # gate 9 -> limit
+            (lim + 1) * -3.0 * sig(a * -3.0),    # up 9 -> limit
+            0.0,                                  # gate 0
+            (-lim + 1) * 1.0 * sig(a * 1.0)]      # up -9 -> -limit
+    assert np.allclose(got[0, :4].numpy(), want, rtol=2 ** -7)
+
+
+def test_expert_bias_branch_against_the_reference_loop():
+    """C oracle forward with expert biases vs the reference's gpt-oss torch loop
+    (ops/_kunlun_ops.py:433-468, restated in oracle/torch_moe.py)."""
+    torch.manual_seed(8)
+    M, H, E, K, I = 24, 64, 6, 2, 32
+    x = torch.randn(M, H).bfloat16()
+    logits = torch.randn(M, E)
+    w13 = (torch.randn(E, 2 * I, H) * 0.1).bfloat16()
+    w2 = (torch.randn(E, H, I) * 0.1).bfloat16()
+    b13 = (torch.randn(E, 2 * I) * 0.2).bfloat16()
+    b2 = (torch.randn(E, H) * 0.2).bfloat16()
+    got = from_bits(co.forward_bf16(bits(x), logits.numpy(), bits(w13), bits(w2), K, w13_bias=bits(b13),
+                                    w2_bias=bits(b2)))
+    ref = tm.bf16_moe_bias(x, logits, w13, w2, b13, b2, K)
+    assert rel_l2(got, ref) <= 1e-2
+    no_b2 = from_bits(co.forward_bf16(bits(x), logits.numpy(), bits(w13), bits(w2), K, w13_bias=bits(b13)))
+    assert rel_l2(no_b2, tm.bf16_moe_bias(x, logits, w13, w2, b13, None, K)) <= 1e-2
+    assert rel_l2(no_b2, ref) > 5e-2   # the down bias matters

@@ -138,6 +138,22 @@ __global__ void fill_dense_lod_kernel(int32_t* lod2, int rows) {
   if (threadIdx.x == 1) lod2[1] = rows;
 }
 
+// one thread: 8 interleaved inputs (16 B) -> 4 outputs (8 B)
+__global__ void swigluoai_and_mul_kernel(const uint16_t* __restrict__ y, int64_t ld_y, int R, int I, float alpha,
+                                         float limit, uint16_t* __restrict__ out, int64_t ld_out) {
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int per_row = I / 4;
+  if (i >= static_cast<long long>(R) * per_row) return;
+  const int r = static_cast<int>(i / per_row), v = static_cast<int>(i % per_row);
+  Pack8 in;
+  in.v = *reinterpret_cast<const uint4*>(y + static_cast<size_t>(r) * ld_y + v * 8);
+  uint16_t o[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = swigluoai_bf16(in.h[2 * j], in.h[2 * j + 1], alpha, limit);
+  *reinterpret_cast<uint2*>(out + static_cast<size_t>(r) * ld_out + v * 4) =
+      make_uint2(o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16));
+}
+
 }  // namespace
 
 int fill_dense_lod(int32_t* lod2, int rows, hipStream_t stream) {
@@ -205,6 +221,19 @@ extern "C" int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, i
   hipLaunchKernelGGL(quant_fp8_group128_kernel, dim3(static_cast<unsigned>((groups + 15) / 16)), dim3(256), 0,
                      as_stream(stream), x, ld_x, R, C, q, ld_q, scale);
   return check_launch("kmoe_quant_fp8_group128");
+}
+
+extern "C" int kmoe_swigluoai_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, float alpha, float limit,
+                                      uint16_t* out, int64_t ld_out, kmoe_stream_t stream) {
+  KMOE_REQUIRE(y && out, KMOE_ERR_NULL, "swigluoai_and_mul: NULL pointer");
+  KMOE_REQUIRE(R >= 0 && I >= 4 && I % 4 == 0, KMOE_ERR_SHAPE, "swigluoai_and_mul: R=%d I=%d (need I %% 4 == 0)", R, I);
+  KMOE_REQUIRE(ld_y % 8 == 0 && ld_out % 4 == 0 && ld_y >= 2 * I && ld_out >= I, KMOE_ERR_SHAPE,
+               "swigluoai_and_mul: row strides %lld/%lld", (long long)ld_y, (long long)ld_out);
+  if (R == 0) return KMOE_OK;
+  const long long n = static_cast<long long>(R) * (I / 4);
+  hipLaunchKernelGGL(swigluoai_and_mul_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0,
+                     as_stream(stream), y, ld_y, R, I, alpha, limit, out, ld_out);
+  return check_launch("kmoe_swigluoai_and_mul");
 }
 
 extern "C" int kmoe_silu_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, uint16_t* out, int64_t ld_out,

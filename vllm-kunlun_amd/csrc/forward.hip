@@ -90,6 +90,10 @@ struct MlpPass {
   const void *w13_tail, *w2_tail;
   const float *w13_aux_tail, *w2_aux_tail;
   int tail_rows;
+  // BF16 expert-bias branch
+  const uint16_t *w13_bias, *w2_bias;
+  int oai;  // 1: gate_up rows interleaved, gpt-oss activation
+  float act_alpha, act_limit;
 };
 
 int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
@@ -168,8 +172,11 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
   g.rows = m.rows;
   g.y = y;
   g.ldy = ldy;
-  g.act = act;
+  g.act = first && m.oai ? KMOE_ACT_SWIGLUOAI : act;
   g.w_layout = m.w_layout;
+  g.bias = first ? m.w13_bias : m.w2_bias;
+  g.act_alpha = m.act_alpha;
+  g.act_limit = m.act_limit;
   return kmoe_grouped_gemm_bf16(&g, stream);
 }
 
@@ -257,6 +264,13 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
                "moe_forward: shared expert pointers are NULL");
   KMOE_REQUIRE(a->scoring == KMOE_SCORE_SOFTMAX || a->scoring == KMOE_SCORE_SIGMOID, KMOE_ERR_UNSUPPORTED,
                "moe_forward: scoring=%d unknown", a->scoring);
+  KMOE_REQUIRE(a->activation == 0 || a->activation == KMOE_ACT_SWIGLU ||
+                   (a->activation == KMOE_ACT_SWIGLUOAI && a->format == KMOE_FMT_BF16),
+               KMOE_ERR_UNSUPPORTED, "moe_forward: activation=%d (swigluoai goes with bf16 weights only)", a->activation);
+  KMOE_REQUIRE((!a->w13_bias && !a->w2_bias) || a->format == KMOE_FMT_BF16, KMOE_ERR_UNSUPPORTED,
+               "moe_forward: expert biases go with bf16 weights only");
+  KMOE_REQUIRE(!a->w13_bias || a->activation == KMOE_ACT_SWIGLUOAI, KMOE_ERR_UNSUPPORTED,
+               "moe_forward: a gate_up bias goes with the swigluoai activation");
   KMOE_REQUIRE(workspace, KMOE_ERR_WORKSPACE, "moe_forward: workspace is NULL (need %zu bytes)", L.total_bytes);
   KMOE_REQUIRE(workspace_bytes >= L.total_bytes, KMOE_ERR_WORKSPACE, "moe_forward: workspace %zu < %zu bytes",
                workspace_bytes, L.total_bytes);
@@ -364,6 +378,13 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   routed.act_aux = static_cast<float*>(at(L.actmax));
   routed.out = static_cast<uint16_t*>(at(L.down));
   routed.w_layout = a->w_layout;
+  if (a->format == KMOE_FMT_BF16) {
+    routed.w13_bias = a->w13_bias;
+    routed.w2_bias = a->w2_bias;
+    routed.oai = a->activation == KMOE_ACT_SWIGLUOAI;
+    routed.act_alpha = a->act_alpha;
+    routed.act_limit = a->act_limit;
+  }
   routed.stream = stream_mode;
   routed.x_count = M;
   const bool fold = fold_shared(a);

@@ -67,6 +67,10 @@ struct GemmParams {
   const int8_t* w_tail;    // optional extra expert (index E): rows [tail_row0, tail_row0 + tail_rows), identity source
   const float* w_max_tail;
   int32_t tail_row0, tail_rows, tail_src0;
+  // BF16 only (the expert-bias branch, ops/_kunlun_ops.py:433-468):
+  const uint16_t* bias;    // NULL, or [E, n] bf16 added to the bf16 result (rounded again, as `gemm + bias` in bf16 is)
+  int32_t oai;             // 1: out[r, i] = swigluoai(y[r, 2i], y[r, 2i+1]) (interleaved gate/up), n/2 outputs per row
+  float oai_alpha, oai_limit;
 };
 
 // Rows of expert e, with the tail expert (e == E) taken from the host-side range.
@@ -353,6 +357,22 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
 #pragma unroll
           for (int q = 0; q < 4; ++q) yv[q] = f32_to_bf16(silu_fixed(bf16_to_f32(yv[q])) * bf16_to_f32(uv[q]));
         }
+        if constexpr (KIND == Kind::BF16 && !SWIGLU) {
+          if (p.bias) {
+            const uint2 b4 = *reinterpret_cast<const uint2*>(p.bias + static_cast<size_t>(e) * p.n + c0);
+            const uint16_t bv[4] = {static_cast<uint16_t>(b4.x), static_cast<uint16_t>(b4.x >> 16),
+                                    static_cast<uint16_t>(b4.y), static_cast<uint16_t>(b4.y >> 16)};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) yv[q] = f32_to_bf16(bf16_to_f32(yv[q]) + bf16_to_f32(bv[q]));
+          }
+          if (p.oai) {  // this lane holds (gate, up, gate, up) of output channels c0/2 and c0/2 + 1
+            const uint16_t o0 = swigluoai_bf16(yv[0], yv[1], p.oai_alpha, p.oai_limit);
+            const uint16_t o1 = swigluoai_bf16(yv[2], yv[3], p.oai_alpha, p.oai_limit);
+            *reinterpret_cast<uint32_t*>(p.y + static_cast<size_t>(r) * p.ldy + c0 / 2) =
+                o0 | (static_cast<uint32_t>(o1) << 16);
+            continue;
+          }
+        }
         const uint2 packed = make_uint2(yv[0] | (static_cast<uint32_t>(yv[1]) << 16),
                                         yv[2] | (static_cast<uint32_t>(yv[3]) << 16));
         *reinterpret_cast<uint2*>(p.y + static_cast<size_t>(r) * p.ldy + c0) = packed;
@@ -447,7 +467,7 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
   KMOE_REQUIRE(a->variant < 5 || a->variant > 8, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-8 need tiled weights and k %% 128 == 0");
   GemmParams p{a->a,   a->lda, a->a_max, a->row_src, a->src_div, a->w,   a->w_max,
                a->lod, a->E,   a->n,     a->k,       a->y,       a->ldy, a->acc_out, a->w_layout == KMOE_W_TILED,
-               a->w_tail, a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0};
+               a->w_tail, a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0, nullptr, 0, 0.f, 0.f};
   return dispatch<Kind::I8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_i8");
 }
 
@@ -458,12 +478,16 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
                "grouped_gemm_bf16: E=%d n=%d k=%d rows=%d", a->E, a->n, a->k, a->rows);
   KMOE_REQUIRE(a->k % 8 == 0, KMOE_ERR_SHAPE, "grouped_gemm_bf16: k=%d must be a multiple of 8", a->k);
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
-  KMOE_REQUIRE(a->act == KMOE_ACT_NONE || swiglu, KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: act=%d unknown", a->act);
+  const bool oai = a->act == KMOE_ACT_SWIGLUOAI;
+  KMOE_REQUIRE(a->act == KMOE_ACT_NONE || swiglu || oai, KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: act=%d unknown",
+               a->act);
   KMOE_REQUIRE(a->n % (swiglu ? 32 : 16) == 0, KMOE_ERR_SHAPE, "grouped_gemm_bf16: n=%d must be a multiple of %d",
                a->n, swiglu ? 32 : 16);
+  KMOE_REQUIRE(!a->bias || (!swiglu && aligned(a->bias, 8)), KMOE_ERR_UNSUPPORTED,
+               "grouped_gemm_bf16: a bias goes with act none or swigluoai and must be 8-byte aligned");
   KMOE_REQUIRE(a->lda % 8 == 0 && a->lda >= a->k, KMOE_ERR_SHAPE,
                "grouped_gemm_bf16: lda=%lld must be a multiple of 8 and >= k", (long long)a->lda);
-  const int n_out = swiglu ? a->n / 2 : a->n;
+  const int n_out = (swiglu || oai) ? a->n / 2 : a->n;
   KMOE_REQUIRE(a->ldy % 4 == 0 && a->ldy >= n_out, KMOE_ERR_SHAPE,
                "grouped_gemm_bf16: ldy=%lld must be a multiple of 4 and >= %d", (long long)a->ldy, n_out);
   KMOE_REQUIRE(aligned(a->a, 16) && aligned(a->w, 16) && aligned(a->y, 8), KMOE_ERR_SHAPE,
@@ -473,14 +497,14 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR || (a->w_layout == KMOE_W_TILED && a->k % 32 == 0), KMOE_ERR_SHAPE,
                "grouped_gemm_bf16: w_layout=%d (tiled weights need k %% 32 == 0, k=%d)", a->w_layout, a->k);
   // many rows per expert and tiled weights: the persistent 128-row-tile kernel (variant 5 forces it)
-  if (a->w_layout == KMOE_W_TILED && a->k % 64 == 0 && a->ldy % 8 == 0 &&
+  if (a->w_layout == KMOE_W_TILED && a->k % 64 == 0 && a->ldy % 8 == 0 && !a->bias && !oai &&
       (a->variant == 5 || (a->variant == 0 && ceil_div(a->rows, a->E) > 48)))
     return tiled_gemm_bf16(a, as_stream(stream));
   KMOE_REQUIRE(a->variant != 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variant 5 needs tiled weights, k %% 64 == 0");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), nullptr,    a->lod,  a->E,       a->n,
                a->k * 2,                              a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,
-               nullptr, nullptr, 0, 0, 0};
+               nullptr, nullptr, 0, 0, 0, a->bias, oai ? 1 : 0, a->act_alpha, a->act_limit};
   return dispatch<Kind::BF16>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_bf16");
 }
 
@@ -514,6 +538,6 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), a->w_scale, a->lod,  a->E,       a->n,
                a->k,                                  a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,
-               nullptr, nullptr, 0, 0, 0};
+               nullptr, nullptr, 0, 0, 0, nullptr, 0, 0.f, 0.f};
   return dispatch<Kind::FP8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_fp8_block");
 }

@@ -89,6 +89,15 @@ __device__ inline float exp_fixed(float x) {
 
 __device__ inline float sigmoid_fixed(float x) { return 1.0f / (1.0f + exp_fixed(-x)); }
 __device__ inline float silu_fixed(float x) { return x / (1.0f + exp_fixed(-x)); }
+// gpt-oss activation on a (gate, up) pair of bf16 values, one rounding at the end:
+// g = min(gate, limit), u = clamp(up, -limit, limit), out = (u + 1) * g * sigmoid(alpha * g)
+// (reference: swigluoai_and_mul, ops/_custom_ops.py:728-742).
+__device__ inline uint16_t swigluoai_bf16(uint16_t gate, uint16_t up, float alpha, float limit) {
+  const float g = fminf(bf16_to_f32(gate), limit);
+  const float u = fminf(fmaxf(bf16_to_f32(up), -limit), limit);
+  const float glu = g * sigmoid_fixed(g * alpha);
+  return f32_to_bf16((u + 1.0f) * glu);
+}
 
 // ---- wave64 helpers ---------------------------------------------------------
 __device__ inline int lane_id() { return static_cast<int>(threadIdx.x) & (kWave - 1); }

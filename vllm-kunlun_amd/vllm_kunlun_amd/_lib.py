@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(PROJECT_DIR, "lib", "libkmoe.so")
 
 KMOE_ACT_NONE = 0
 KMOE_ACT_SWIGLU = 1
+KMOE_ACT_SWIGLUOAI = 2
 KMOE_SCORE_SOFTMAX = 0
 KMOE_SCORE_SIGMOID = 1
 KMOE_FMT_INT8 = 0
@@ -46,7 +47,7 @@ class GemmBf16Args(C.Structure):
         ("w", C.c_void_p), ("lod", C.c_void_p),
         ("E", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("rows", C.c_int32),
         ("y", C.c_void_p), ("ldy", C.c_int64), ("act", C.c_int32), ("variant", C.c_int32),
-        ("w_layout", C.c_int32),
+        ("w_layout", C.c_int32), ("bias", C.c_void_p), ("act_alpha", C.c_float), ("act_limit", C.c_float),
     ]
 
 
@@ -69,6 +70,8 @@ class MoEArgs(C.Structure):
         ("I_shared", C.c_int32), ("ws13", C.c_void_p), ("ws13_max", C.c_void_p), ("ws2", C.c_void_p),
         ("ws2_max", C.c_void_p), ("out_scale", C.c_float), ("out", C.c_void_p),
         ("stage_events", C.POINTER(C.c_void_p)), ("w_layout", C.c_int32), ("w_gate", C.c_void_p),
+        ("w13_bias", C.c_void_p), ("w2_bias", C.c_void_p), ("activation", C.c_int32), ("act_alpha", C.c_float),
+        ("act_limit", C.c_float),
     ]
 
 
@@ -98,6 +101,7 @@ def _load() -> C.CDLL:
         "kmoe_quant_i8_rows": (i32, [vp, i64, i32, i32, vp, i64, vp, vp]),
         "kmoe_quant_i8_rows_chunked": (i32, [vp, i64, i32, i32, vp, vp, vp]),
         "kmoe_tile_weights_i8": (i32, [vp, vp, i32, i32, i32, vp]),
+        "kmoe_swigluoai_and_mul": (i32, [vp, i64, i32, i32, f32, f32, vp, i64, vp]),
         "kmoe_router_gemm_workspace_bytes": (sz, [i32, i32, i32]),
         "kmoe_router_gemm_bf16": (i32, [vp, i64, vp, i32, i32, i32, vp, i64, vp, sz, vp]),
         "kmoe_quant_fp8_group128": (i32, [vp, i64, i32, i32, vp, i64, vp, vp]),
@@ -122,6 +126,7 @@ EXPORTS = (
     "kmoe_align_workspace_bytes", "kmoe_align", "kmoe_gather_rows", "kmoe_quant_i8_rows", "kmoe_quant_i8_rows_chunked", "kmoe_tile_weights_i8", "kmoe_quant_fp8_group128",
     "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
     "kmoe_moe_workspace_layout", "kmoe_moe_forward", "kmoe_router_gemm_workspace_bytes", "kmoe_router_gemm_bf16",
+    "kmoe_swigluoai_and_mul",
 )
 
 

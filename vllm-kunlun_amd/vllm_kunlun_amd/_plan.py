@@ -98,12 +98,15 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
                   topk_group: Optional[int] = None, routed_scaling_factor: float = 1.0,
                   e_score_correction_bias: Optional[torch.Tensor] = None, shared_expert=None, out_scale: float = 1.0,
                   stage_events=None, w_layout: Optional[int] = None,
-                  router_weight: Optional[torch.Tensor] = None) -> MoEPlan:
+                  router_weight: Optional[torch.Tensor] = None, w13_bias: Optional[torch.Tensor] = None,
+                  w2_bias: Optional[torch.Tensor] = None, activation: str = "silu", act_alpha: float = 1.702,
+                  act_limit: float = 7.0) -> MoEPlan:
     """x bf16 [M,H], logits f32 [M,E], out bf16 [M,H]; w13 [E,2I,H], w2 [E,H,I] in the
     format's dtype; w13_aux/w2_aux: per-channel maxes (int8) or block scales (fp8), None for bf16.
     shared_expert: (ws13 [2Is,H], ws13_aux, ws2 [H,Is], ws2_aux) in the same format.
     logits may be None when router_weight (bf16 [E,H], the gate projection) is given: the
-    layer then computes the router logits itself."""
+    layer then computes the router logits itself. bf16 only: w13_bias [E,2I] / w2_bias [E,H] (bf16)
+    and activation "swigluoai" (gate and up rows of w13 interleaved) select the expert-bias branch."""
     if scoring_func not in ("softmax", "sigmoid"):
         raise ValueError(f"Unsupported scoring_func: {scoring_func}")
     if logits is None and router_weight is None:
@@ -148,6 +151,21 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
         a.ws13_max = 0 if ws13_aux is None else ws13_aux.data_ptr()
         a.ws2_max = 0 if ws2_aux is None else ws2_aux.data_ptr()
         keep.append(shared_expert)
+    if activation not in ("silu", "swigluoai"):
+        raise ValueError(f"Unsupported activation: {activation}")
+    if (w13_bias is not None or w2_bias is not None or activation == "swigluoai") and fmt != L.KMOE_FMT_BF16:
+        raise NotImplementedError("moe plan: expert biases and swigluoai go with bf16 weights only")
+    for b, cols in ((w13_bias, two_i), (w2_bias, H)):
+        if b is not None:
+            L.require_device(b)
+            L.require_contig(b)
+            if b.dtype != torch.bfloat16 or tuple(b.shape) != (E, cols):
+                raise ValueError(f"moe plan: expert bias must be bfloat16 [{E},{cols}]")
+            keep.append(b)
+    a.w13_bias = 0 if w13_bias is None else w13_bias.data_ptr()
+    a.w2_bias = 0 if w2_bias is None else w2_bias.data_ptr()
+    a.activation = L.KMOE_ACT_SWIGLUOAI if activation == "swigluoai" else L.KMOE_ACT_SWIGLU
+    a.act_alpha, a.act_limit = float(act_alpha), float(act_limit)
     a.out_scale = float(out_scale)
     a.out = out.data_ptr()
     if w_layout is None:  # tiled only if every int8 weight of the call has been tiled

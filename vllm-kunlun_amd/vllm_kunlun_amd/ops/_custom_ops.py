@@ -323,6 +323,27 @@ def moe_post(x: torch.Tensor, moe_index: torch.Tensor, normed_scale: torch.Tenso
 
 
 # Fake (meta) implementations so the ops can be traced, as the reference registers for each op.
+@custom_op("_C::swigluoai_and_mul", mutates_args=())
+def swigluoai_and_mul(x: torch.Tensor, alpha: float = 1.702, limit: float = 7.0, axis: int = -1,
+                      turn: bool = True) -> torch.Tensor:
+    """gate = x[..., ::2], up = x[..., 1::2]; (up.clamp(-limit, limit) + 1) * g * sigmoid(alpha * g) with
+    g = gate.clamp(max=limit) (reference: ops/_custom_ops.py:728-742)."""
+    _need(axis in (-1, x.dim() - 1), "swigluoai_and_mul: only the last axis")
+    bits_in = _act_bits(x, "swigluoai_and_mul")
+    x2 = bits_in.reshape(-1, x.shape[-1])
+    _need(x2.shape[1] % 8 == 0, "swigluoai_and_mul: the last dimension must be a multiple of 8")
+    L.require_device(x2)
+    out = torch.empty((*x.shape[:-1], x.shape[-1] // 2), dtype=x.dtype, device=x.device)
+    L.check(L.lib.kmoe_swigluoai_and_mul(L.ptr(x2), x2.shape[1], x2.shape[0], x2.shape[1] // 2, float(alpha),
+                                         float(limit), L.ptr(out), x2.shape[1] // 2, L.stream()))
+    return out
+
+
+@swigluoai_and_mul.register_fake
+def _fake_swigluoai_and_mul(x, alpha=1.702, limit=7.0, axis=-1, turn=True):
+    return x.new_empty((*x.shape[:-1], x.shape[-1] // 2))
+
+
 @custom_op("_C::router_gemm_bf16_fp32", mutates_args=())
 def router_gemm_bf16_fp32(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """bf16 [M,H] x bf16 [E,H]^T -> f32 [M,E] router logits (reference: ops.router_gemm_bf16_fp32,

@@ -39,15 +39,19 @@ class KunlunOps:
         chosen by `scoring_func` alone and always normalises (`renormalize`,
         `use_grouped_topk` and `inplace` are accepted and ignored, :385-389 vs :413-431);
         the sigmoid path uses scale 1.0 (:428)."""
-        if w1_bias is not None or w2_bias is not None:
-            raise NotImplementedError("fused_moe: the expert-bias (gpt-oss) branch is outside this build's path")
         if hidden_states.dtype != torch.bfloat16:
             raise NotImplementedError(f"fused_moe: activations must be bfloat16, got {hidden_states.dtype}")
         x = hidden_states.contiguous()
         logits = router_logits.to(torch.float).contiguous()
         out = torch.empty_like(x)
+        extra = {}
+        if w1_bias is not None or w2_bias is not None:
+            # the gpt-oss branch (:433-468): per-expert biases, gate/up interleaved, swigluoai_and_mul
+            extra = dict(w13_bias=None if w1_bias is None else w1_bias.to(torch.bfloat16).contiguous(),
+                         w2_bias=None if w2_bias is None else w2_bias.to(torch.bfloat16).contiguous(),
+                         activation="swigluoai")
         plan = make_moe_plan(L.KMOE_FMT_BF16, x, logits, out, moe_top_k, w1, w2, None, None, scoring_func, True,
-                             num_expert_group, topk_group, 1.0, e_score_correction_bias)
+                             num_expert_group, topk_group, 1.0, e_score_correction_bias, **extra)
         plan()
         return out
 

@@ -1,0 +1,119 @@
+"""The benchmark configurations at their FULL sizes. The oracle cannot run thousands of tokens
+through 256 experts in test time, so the large batches are held to what does not depend on
+size: every token's result is independent of the batch it travels in. That gives, bit for bit,
+  * permutation equivariance: shuffling the tokens shuffles the outputs;
+  * batch-size independence: a token gets the same bits in a decode batch (weight-streaming
+    kernels, chunk-major codes, fused prologue) as in a prefill batch (persistent tile kernel);
+  * a spot check: a handful of tokens of the big batch through the C oracle.
+The decode batches are compared with the C oracle in full."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import bits
+
+pytestmark = pytest.mark.gpu
+
+from oracle import c_oracle as co  # noqa: E402
+
+
+def _host(t):
+    return None if t is None else t.detach().cpu()
+
+
+def _oracle(sl, host, x, logits):
+    w13, w13_max, w2, w2_max, shared = host
+    s = sl.shape
+    sh = None if shared is None else tuple(t.numpy() for t in shared)
+    return co.forward_w8a8(bits(x), _host(logits).float().numpy(), w13.numpy(), w13_max.numpy(), w2.numpy(),
+                           w2_max.numpy(), s.K, s.scoring, True, s.n_group, s.topk_group, s.routed_scale,
+                           None if sl.bias is None else _host(sl.bias).numpy(), sh)
+
+
+def _run(sl, x, logits):
+    out = sl.layer.quant_method.apply_monolithic(sl.layer, x, logits, **sl.apply_kwargs())
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.fixture(scope="module")
+def qwen3():
+    from vllm_kunlun_amd import synth
+    sl = synth.make_w8a8_layer(synth.SHAPES["qwen3-prefill"], "cuda", seed=0)  # 8192 tokens; decode = its first 64
+    return sl, sl.host_weights()
+
+
+@pytest.fixture(scope="module")
+def dsv3():
+    from vllm_kunlun_amd import synth
+    sl = synth.make_w8a8_layer(synth.SHAPES["dsv3-prefill"], "cuda", seed=0)   # 4096 tokens; decode = its first 128
+    return sl, sl.host_weights()
+
+
+def _properties(sl, host, n_decode, n_spot, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    x, logits = sl.x, sl.logits
+    M = x.shape[0]
+    full = _run(sl, x, logits)
+    assert bool(torch.isfinite(full.float()).all())
+    # permutation equivariance
+    perm = torch.randperm(M, generator=g, device="cuda")
+    shuffled = _run(sl, x[perm].contiguous(), logits[perm].contiguous())
+    assert torch.equal(shuffled, full[perm]), "a token's output depends on its position in the batch"
+    # the decode batch of the configuration, alone: same bits as inside the prefill batch, and the oracle's bits
+    dec = _run(sl, x[:n_decode].contiguous(), logits[:n_decode].contiguous())
+    assert torch.equal(dec, full[:n_decode]), "decode and prefill kernels disagree"
+    ref = _oracle(sl, host, x[:n_decode], logits[:n_decode])
+    assert np.array_equal(bits(dec), ref), "decode batch vs C oracle"
+    # spot check of the big batch: random tokens through the oracle
+    idx = torch.randperm(M, generator=g, device="cuda")[:n_spot]
+    ref_spot = _oracle(sl, host, x[idx], logits[idx])
+    assert np.array_equal(bits(full[idx]), ref_spot), "prefill batch vs C oracle on a sample of its tokens"
+
+
+def test_qwen3_full_size(qwen3):
+    """Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, intermediate 768; 8192 and 64 tokens."""
+    sl, host = qwen3
+    _properties(sl, host, n_decode=64, n_spot=48, seed=1)
+
+
+def test_qwen3_full_size_skewed_routing(qwen3):
+    """+2.0 on the logits of 8 experts: a few experts get thousands of rows, most a handful."""
+    sl, host = qwen3
+    logits = sl.logits.clone()
+    logits[:, torch.arange(8, device="cuda") * 16] += 2.0
+    full = _run(sl, sl.x, logits)
+    idx = torch.arange(0, sl.x.shape[0], 171, device="cuda")[:48]
+    assert np.array_equal(bits(full[idx]), _oracle(sl, host, sl.x[idx], logits[idx]))
+
+
+def test_dsv3_full_size(dsv3):
+    """DeepSeek-V3 shape: 256 experts + shared, sigmoid grouped top-8, hidden 7168, intermediate 2048;
+    4096 and 128 tokens."""
+    sl, host = dsv3
+    _properties(sl, host, n_decode=128, n_spot=16, seed=2)
+
+
+def test_dsv3_fp8_full_size_sample_against_the_oracle():
+    """The fp8 block-scaled layer at the DeepSeek-V3 shape, 4096 tokens: a sample of its tokens against
+    the C oracle within the fp8 tolerance (MFMA and oracle sum in different orders), routing bit-exact."""
+    from conftest import from_bits, rel_l2
+    from vllm_kunlun_amd import synth
+    shape = synth.SHAPES["dsv3-fp8-prefill"]
+    sl = synth.make_fp8_layer(shape, "cuda", seed=0)
+    m = sl.layer.quant_method
+    full = m.apply_monolithic(sl.layer, sl.x, sl.logits, **sl.apply_kwargs())
+    torch.cuda.synchronize()
+    idx = torch.arange(5, shape.M, 257, device="cuda")[:16]
+    w13, w13_s, w2, w2_s, sh = sl.host_weights()
+    u8 = lambda t: t.view(torch.uint8).numpy()  # noqa: E731
+    shared = (u8(sh[0]), sh[1].numpy(), u8(sh[2]), sh[3].numpy())
+    ref = co.forward_fp8(bits(sl.x[idx]), _host(sl.logits[idx]).numpy(), u8(w13), w13_s.numpy(), u8(w2), w2_s.numpy(),
+                         shape.K, shape.scoring, True, shape.n_group, shape.topk_group, shape.routed_scale,
+                         _host(sl.bias).numpy(), shared)
+    assert rel_l2(full[idx], from_bits(ref)) <= 3e-2
+    ids = m.last_workspace[m.last_layout.topk_ids: m.last_layout.topk_ids + 4 * shape.P].view(torch.int32)
+    ids = ids.view(shape.M, shape.K)[idx].cpu().numpy()
+    _, ids_ref = co.sigmoid_group_topk_norm(_host(sl.logits[idx]).numpy(), _host(sl.bias).numpy(), shape.K,
+                                            shape.n_group, shape.topk_group, shape.routed_scale)
+    assert np.array_equal(ids, ids_ref)

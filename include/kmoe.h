@@ -309,6 +309,20 @@ int kmoe_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_index,
                  int64_t ld_addend, uint16_t* out, int64_t ld_out,
                  kmoe_stream_t stream);
 
+/*
+ * Unpacks 4-bit weights to bf16 once, at load time. Replaces dequant_int4_native
+ * (quantization/kernels/quant_ops.py:71-86), which KunlunCompressedTensorsWNA16MoEMethod.apply
+ * runs on the whole weight tensor in EVERY forward call (compressed_tensors_moe.py:320-327).
+ * packed [rows, k/2] bytes, low nibble = element 2j, high nibble = element 2j+1, unsigned code c
+ * means c - 8; scale [rows, k/group_size] bf16 (group_size == k: one scale per row):
+ *   out[r, j] = bf16( float(c - 8) * float(scale[r, j / group_size]) ).
+ * (The reference tiles its scale tensor along k with Tensor.repeat, which equals this for one
+ * scale per row; for several groups per row this function follows the contiguous groups of the
+ * compressed-tensors format.) Limits: k % 16 == 0, group_size % 2 == 0, k % group_size == 0.
+ */
+int kmoe_dequant_w4_bf16(const uint8_t* packed, const uint16_t* scale, int64_t rows, int k,
+                         int group_size, uint16_t* out, kmoe_stream_t stream);
+
 /* ---------------------------------------------------------------- router GEMM */
 
 /*

@@ -267,6 +267,17 @@ def _route(logits, K, scoring, renormalize, n_group, topk_group, routed_scale, b
     return sigmoid_group_topk_norm(logits, bias, K, n_group, topk_group, routed_scale)
 
 
+def dequant_w4_bf16(packed, scale_bits, group_size):
+    """packed uint8 [..., k/2], scale bf16 bits [..., k/group_size] -> bf16 bits [..., k]."""
+    packed = _c(packed, np.uint8)
+    scale_bits = _c(scale_bits, np.uint16)
+    k = packed.shape[-1] * 2
+    rows = int(np.prod(packed.shape[:-1]))
+    out = np.zeros((*packed.shape[:-1], k), np.uint16)
+    lib().orc_dequant_w4_bf16(_p(packed), _p(scale_bits), C.c_int64(rows), k, int(group_size), _p(out))
+    return out
+
+
 def swigluoai_and_mul(y_bits, alpha=1.702, limit=7.0):
     y_bits = _c(y_bits, np.uint16)
     R, two_i = y_bits.shape

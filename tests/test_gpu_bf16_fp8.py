@@ -319,3 +319,48 @@ def test_fused_moe_expert_bias_branch():
                                     w2_bias=bits(b2)))
     assert rel_l2(out, ref) <= REL_L2_BF16
     assert rel_l2(out, tm.bf16_moe_bias(x, logits, w13, w2, b13, b2, K)) <= REL_L2_BF16
+
+
+@pytest.mark.parametrize("group_size", [None, 32])
+def test_w4a16_method_unpacks_once_and_runs_the_bf16_path(group_size):
+    """KunlunCompressedTensorsWNA16MoEMethod: packed 4-bit weights -> bf16 (kmoe_dequant_w4_bf16, bit-exact
+    vs the oracle) -> tiled -> KunlunOps.fused_moe; output against the C oracle on the unpacked weights."""
+    from vllm_kunlun_amd.ops.fused_moe.layer import FusedMoE
+    from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors import CompressedTensorsConfig
+    from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors_moe import (
+        KunlunCompressedTensorsMoEMethod, KunlunCompressedTensorsWNA16MoEMethod)
+    from vllm_kunlun_amd._plan import rowmajor_int8_weights
+    weights = {"num_bits": 4, "type": "int", "symmetric": True, "dynamic": False,
+               "strategy": "group" if group_size else "channel", "group_size": group_size}
+    cfg = CompressedTensorsConfig.from_config({"quant_method": "compressed-tensors", "format": "pack-quantized",
+                                               "config_groups": {"g": {"targets": ["Linear"], "weights": weights,
+                                                                       "input_activations": None,
+                                                                       "format": "pack-quantized"}}})
+    E, H, I, M, K = 8, 128, 64, 50, 2
+    stub = FusedMoE(num_experts=E, top_k=K, hidden_size=H, intermediate_size=I)
+    method = KunlunCompressedTensorsMoEMethod.get_moe_method(cfg, stub, "m.experts")
+    assert isinstance(method, KunlunCompressedTensorsWNA16MoEMethod)
+    layer = FusedMoE(num_experts=E, top_k=K, hidden_size=H, intermediate_size=I, quant_method=method, device="cuda")
+    g = torch.Generator().manual_seed(9)
+    ckpt = {}
+    for e in range(E):
+        for proj, (n, k) in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
+            ckpt[f"m.experts.{e}.{proj}.weight_packed"] = torch.randint(0, 256, (n, k // 2), generator=g, dtype=torch.uint8)
+            ckpt[f"m.experts.{e}.{proj}.weight_scale"] = (torch.rand(n, k // group_size if group_size else 1,
+                                                                      generator=g) * 0.02 + 0.002).bfloat16()
+    assert len(layer.load_weights(ckpt.items())) == 6 * E
+    packed13, scale13 = layer.w13_weight_packed.data.cpu(), layer.w13_weight_scale.data.cpu()
+    packed2, scale2 = layer.w2_weight_packed.data.cpu(), layer.w2_weight_scale.data.cpu()
+    method.process_weights_after_loading(layer)
+    assert not hasattr(layer, "w13_weight_packed")
+    w13 = rowmajor_int8_weights(layer.w13_weight).cpu()
+    w2 = rowmajor_int8_weights(layer.w2_weight).cpu()
+    assert np.array_equal(bits(w13), co.dequant_w4_bf16(packed13.numpy(), bits(scale13), group_size or H))
+    assert np.array_equal(bits(w2), co.dequant_w4_bf16(packed2.numpy(), bits(scale2), group_size or I))
+    gx = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(M, H, generator=gx, device="cuda").bfloat16()
+    logits = torch.randn(M, E, generator=gx, device="cuda")
+    out = layer(x, logits)
+    torch.cuda.synchronize()
+    ref = co.forward_bf16(bits(x), logits.cpu().numpy(), bits(w13), bits(w2), K)
+    assert rel_l2(out, from_bits(ref)) <= REL_L2_BF16

@@ -68,8 +68,11 @@ def test_method_selection_from_a_checkpoint_config():
     w4 = json.loads(json.dumps(QUANT_CONFIG))
     w4["config_groups"]["group_0"]["input_activations"] = None
     w4["config_groups"]["group_0"]["weights"].update(num_bits=4, strategy="group", group_size=128)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError):   # 4-bit weight-only needs the pack-quantized format (reference :76-93)
         KunlunCompressedTensorsMoEMethod.get_moe_method(CompressedTensorsConfig.from_config(w4), stub, "x.experts")
+    w4["config_groups"]["group_0"]["format"] = "pack-quantized"
+    m4 = KunlunCompressedTensorsMoEMethod.get_moe_method(CompressedTensorsConfig.from_config(w4), stub, "x.experts")
+    assert type(m4).__name__ == "KunlunCompressedTensorsWNA16MoEMethod" and m4.group_size == 128
     with pytest.raises(ValueError):
         CompressedTensorsConfig.from_config({"quant_method": "gptq"})
 

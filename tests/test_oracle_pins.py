@@ -496,3 +496,18 @@ def test_expert_bias_branch_against_the_reference_loop():
     no_b2 = from_bits(co.forward_bf16(bits(x), logits.numpy(), bits(w13), bits(w2), K, w13_bias=bits(b13)))
     assert rel_l2(no_b2, tm.bf16_moe_bias(x, logits, w13, w2, b13, None, K)) <= 1e-2
     assert rel_l2(no_b2, ref) > 5e-2   # the down bias matters
+
+
+def test_dequant_w4_against_the_reference_expression():
+    """Low nibble first, code - 8, times the scale (quantization/kernels/quant_ops.py:71-86, with
+    contiguous groups): checked against that expression written with torch ops."""
+    torch.manual_seed(5)
+    for rows, k, gs in ((3, 32, 32), (4, 64, 16), (2, 256, 128)):
+        packed = torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8)
+        scale = (torch.rand(rows, k // gs) * 0.1 + 0.01).bfloat16()
+        got = from_bits(co.dequant_w4_bf16(packed.numpy(), bits(scale), gs))
+        codes = torch.stack((packed & 0xF, (packed >> 4) & 0xF), dim=-1).reshape(rows, k).float() - 8.0
+        ref = (codes * scale.float().repeat_interleave(gs, dim=1)).bfloat16()
+        assert torch.equal(got, ref)
+    one = co.dequant_w4_bf16(np.array([[0x1F] * 8], np.uint8), bits(torch.tensor([[2.0]]).bfloat16()), 16)
+    assert from_bits(one).tolist()[0][:2] == [14.0, -14.0]   # 0xF - 8 = 7 first (low nibble), 0x1 - 8 = -7 second

@@ -154,6 +154,32 @@ __global__ void swigluoai_and_mul_kernel(const uint16_t* __restrict__ y, int64_t
       make_uint2(o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16));
 }
 
+// one thread: 8 packed bytes -> 16 bf16 values
+__global__ void dequant_w4_kernel(const uint8_t* __restrict__ packed, const uint16_t* __restrict__ scale, long long rows,
+                                  int k, int group_size, uint16_t* __restrict__ out) {
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int per_row = k / 16;
+  if (i >= rows * per_row) return;
+  const long long r = i / per_row;
+  const int j0 = static_cast<int>(i % per_row) * 16;
+  const uint2 in = *reinterpret_cast<const uint2*>(packed + r * (k / 2) + j0 / 2);
+  const uint32_t word[2] = {in.x, in.y};
+  const uint16_t* srow = scale + r * (k / group_size);
+  uint32_t o[8];
+#pragma unroll
+  for (int b = 0; b < 8; ++b) {
+    const uint32_t byte = (word[b >> 2] >> (8 * (b & 3))) & 0xffu;
+    const int j = j0 + 2 * b;  // group_size is even: both nibbles of a byte share a scale
+    const float s = bf16_to_f32(srow[j / group_size]);
+    const uint16_t lo = f32_to_bf16(static_cast<float>(static_cast<int>(byte & 0xf) - 8) * s);
+    const uint16_t hi = f32_to_bf16(static_cast<float>(static_cast<int>(byte >> 4) - 8) * s);
+    o[b] = lo | (static_cast<uint32_t>(hi) << 16);
+  }
+  uint4* dst = reinterpret_cast<uint4*>(out + r * k + j0);
+  dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+  dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+}
+
 }  // namespace
 
 int fill_dense_lod(int32_t* lod2, int rows, hipStream_t stream) {
@@ -221,6 +247,20 @@ extern "C" int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, i
   hipLaunchKernelGGL(quant_fp8_group128_kernel, dim3(static_cast<unsigned>((groups + 15) / 16)), dim3(256), 0,
                      as_stream(stream), x, ld_x, R, C, q, ld_q, scale);
   return check_launch("kmoe_quant_fp8_group128");
+}
+
+extern "C" int kmoe_dequant_w4_bf16(const uint8_t* packed, const uint16_t* scale, int64_t rows, int k, int group_size,
+                                    uint16_t* out, kmoe_stream_t stream) {
+  KMOE_REQUIRE(packed && scale && out, KMOE_ERR_NULL, "dequant_w4_bf16: NULL pointer");
+  KMOE_REQUIRE(rows >= 0 && k >= 16 && k % 16 == 0 && group_size >= 2 && group_size % 2 == 0 && k % group_size == 0,
+               KMOE_ERR_SHAPE, "dequant_w4_bf16: rows=%lld k=%d group_size=%d", (long long)rows, k, group_size);
+  KMOE_REQUIRE((reinterpret_cast<uintptr_t>(packed) & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0,
+               KMOE_ERR_SHAPE, "dequant_w4_bf16: misaligned tensor pointer");
+  if (rows == 0) return KMOE_OK;
+  const long long n = rows * (k / 16);
+  hipLaunchKernelGGL(dequant_w4_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     packed, scale, static_cast<long long>(rows), k, group_size, out);
+  return check_launch("kmoe_dequant_w4_bf16");
 }
 
 extern "C" int kmoe_swigluoai_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, float alpha, float limit,

@@ -102,6 +102,7 @@ def _load() -> C.CDLL:
         "kmoe_quant_i8_rows_chunked": (i32, [vp, i64, i32, i32, vp, vp, vp]),
         "kmoe_tile_weights_i8": (i32, [vp, vp, i32, i32, i32, vp]),
         "kmoe_swigluoai_and_mul": (i32, [vp, i64, i32, i32, f32, f32, vp, i64, vp]),
+        "kmoe_dequant_w4_bf16": (i32, [vp, vp, i64, i32, i32, vp, vp]),
         "kmoe_router_gemm_workspace_bytes": (sz, [i32, i32, i32]),
         "kmoe_router_gemm_bf16": (i32, [vp, i64, vp, i32, i32, i32, vp, i64, vp, sz, vp]),
         "kmoe_quant_fp8_group128": (i32, [vp, i64, i32, i32, vp, i64, vp, vp]),
@@ -126,7 +127,7 @@ EXPORTS = (
     "kmoe_align_workspace_bytes", "kmoe_align", "kmoe_gather_rows", "kmoe_quant_i8_rows", "kmoe_quant_i8_rows_chunked", "kmoe_tile_weights_i8", "kmoe_quant_fp8_group128",
     "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
     "kmoe_moe_workspace_layout", "kmoe_moe_forward", "kmoe_router_gemm_workspace_bytes", "kmoe_router_gemm_bf16",
-    "kmoe_swigluoai_and_mul",
+    "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16",
 )
 
 

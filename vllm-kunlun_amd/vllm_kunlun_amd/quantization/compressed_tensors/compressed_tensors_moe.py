@@ -79,7 +79,11 @@ class KunlunCompressedTensorsMoEMethod:
         weight_quant = scheme.get("weights")
         input_quant = scheme.get("input_activations")
         if _scheme_is_wna16(weight_quant, input_quant):
-            raise NotImplementedError("W4A16/W8A16 weight-only MoE is outside the W8A8 path of this build")
+            fmt = scheme.get("format")
+            if _get(weight_quant, "num_bits") != 4 or fmt not in (None, "pack-quantized"):
+                raise ValueError(f"For Fused MoE layers, only format pack-quantized and 4 bits is supported but got "
+                                 f"format: {fmt} and bits: {_get(weight_quant, 'num_bits')}")
+            return KunlunCompressedTensorsWNA16MoEMethod(weight_quant, input_quant, layer.moe_config)
         if _scheme_is_dynamic_token_w8a8(weight_quant, input_quant):
             return KunlunCompressedTensorsW8A8Int8MoEMethod(weight_quant, input_quant, layer.moe_config)
         if _scheme_is_fp8_block(weight_quant, input_quant):
@@ -271,3 +275,71 @@ class KunlunCompressedTensorsW8A8Fp8MoEMethod(_MonolithicQuantMoE):
             with torch.no_grad():
                 tile_int8_weights_(w13)
                 tile_int8_weights_(w2)
+
+
+class KunlunCompressedTensorsWNA16MoEMethod:
+    """4-bit weight-only MoE (reference: compressed_tensors_moe.py:294-360). The reference
+    unpacks the whole packed weight tensors to fp16 inside EVERY apply() (:320-327) and then
+    calls the unquantized fused_moe; here the unpacking (kmoe_dequant_w4_bf16) runs once in
+    process_weights_after_loading, the bf16 weights are tiled for the MFMA kernels, and the
+    packed tensors are dropped. Packed layout as in dequant_int4_native
+    (quantization/kernels/quant_ops.py:71-86): uint8, two codes per byte, low nibble first,
+    code - 8; scales per contiguous group of `group_size` along k, or one per row."""
+
+    def __init__(self, weight_quant=None, input_quant=None, moe=None):
+        self.weight_quant = weight_quant
+        self.input_quant = input_quant
+        self.moe = moe
+        gs = _get(weight_quant, "group_size") if weight_quant is not None else None
+        self.group_size = int(gs) if (gs and _strategy(weight_quant) == "group") else None  # None: one scale per row
+
+    @property
+    def is_monolithic(self) -> bool:
+        return True
+
+    def create_weights(self, layer: torch.nn.Module, num_experts: int, hidden_size: int,
+                       intermediate_size_per_partition: int, params_dtype: torch.dtype = torch.bfloat16,
+                       device=None, **_) -> None:
+        E, H, I = num_experts, hidden_size, intermediate_size_per_partition
+        if H % 16 or I % 16:
+            raise ValueError("4-bit MoE weights need hidden and intermediate sizes that are multiples of 16")
+        g13 = H // self.group_size if self.group_size else 1
+        g2 = I // self.group_size if self.group_size else 1
+        mk = lambda *s, dt: torch.nn.Parameter(torch.zeros(*s, dtype=dt, device=device), requires_grad=False)  # noqa
+        layer.w13_weight_packed = mk(E, 2 * I, H // 2, dt=torch.uint8)
+        layer.w2_weight_packed = mk(E, H, I // 2, dt=torch.uint8)
+        layer.w13_weight_scale = mk(E, 2 * I, g13, dt=torch.bfloat16)
+        layer.w2_weight_scale = mk(E, H, g2, dt=torch.bfloat16)
+
+    def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
+        with torch.no_grad():
+            for name in ("w13", "w2"):
+                packed = getattr(layer, f"{name}_weight_packed").data.contiguous()
+                scale = getattr(layer, f"{name}_weight_scale").data.to(torch.bfloat16).contiguous()
+                E, n, half_k = packed.shape
+                k = 2 * half_k
+                gs = self.group_size or k
+                if k % gs or scale.shape[-1] != k // gs:
+                    raise ValueError(f"{name}: scales {tuple(scale.shape)} do not fit k={k}, group_size={gs}")
+                L.require_device(packed, scale)
+                w = torch.empty((E, n, k), dtype=torch.bfloat16, device=packed.device)
+                L.check(L.lib.kmoe_dequant_w4_bf16(L.ptr(packed), L.ptr(scale), E * n, k, gs, L.ptr(w), L.stream()))
+                param = torch.nn.Parameter(w, requires_grad=False)
+                setattr(layer, f"{name}_weight", param)
+                delattr(layer, f"{name}_weight_packed")
+            if getattr(self, "tile_weights", True):
+                tile_int8_weights_(layer.w13_weight)
+                tile_int8_weights_(layer.w2_weight)
+
+    def apply_monolithic(self, layer, x: torch.Tensor, router_logits: torch.Tensor, **kwargs):
+        """bf16 activations against the unpacked weights: KunlunOps.fused_moe, as the reference's
+        apply() ends (:343-360)."""
+        from ...ops._kunlun_ops import KunlunOps as ops
+        return ops.fused_moe(x, layer.w13_weight, layer.w2_weight, router_logits, 0, self.moe.experts_per_token,
+                             renormalize=getattr(layer, "renormalize", True), inplace=True,
+                             use_grouped_topk=getattr(layer, "use_grouped_topk", False),
+                             num_expert_group=getattr(layer, "num_expert_group", None),
+                             topk_group=getattr(layer, "topk_group", None),
+                             scoring_func=getattr(layer, "scoring_func", "softmax"),
+                             e_score_correction_bias=getattr(layer, "e_score_correction_bias", None),
+                             w1_bias=getattr(layer, "w13_bias", None), w2_bias=getattr(layer, "w2_bias", None))

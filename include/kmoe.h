@@ -380,8 +380,8 @@ typedef struct kmoe_moe_args {
      recorded on the stream before stage s and entry 2s+1 after it (NULL entries
      are skipped). Leave NULL under graph capture.                             */
   void* const* stage_events;
-  int32_t w_layout;      /* INT8, FP8: KMOE_W_TILED if w13, w2 (and ws13, ws2) went
-                            through kmoe_tile_weights_i8; else KMOE_W_ROWMAJOR  */
+  int32_t w_layout;      /* KMOE_W_TILED if w13, w2 went through kmoe_tile_weights_i8;
+                            else KMOE_W_ROWMAJOR                                   */
   const uint16_t* w_gate; /* NULL, or [E,H] bf16 router weight (used when logits is NULL) */
   /* BF16 only, the expert-bias branch (ops/_kunlun_ops.py:433-468): */
   const uint16_t* w13_bias; /* NULL, or [E,2I] bf16                                   */
@@ -389,6 +389,8 @@ typedef struct kmoe_moe_args {
   int32_t activation;    /* KMOE_ACT_SWIGLU (0 means the same) or KMOE_ACT_SWIGLUOAI: w13
                             then holds gate and up rows interleaved               */
   float act_alpha, act_limit;
+  int32_t ws_layout;     /* layout of ws13, ws2 (KMOE_W_*): a shared expert whose sizes do not allow
+                            tiling (k % 64) stays row-major next to tiled routed experts  */
 } kmoe_moe_args;
 
 #define KMOE_STAGE_ROUTING 0

@@ -40,7 +40,7 @@ def test_struct_layouts_match_the_header(L):
     assert C.sizeof(L.MoELayout) == 22 * 8
     assert C.sizeof(L.GemmBf16Args) == 6 * 8 + 16 + 16 + 16 + 16  # ..., act+variant+w_layout+pad, bias, alpha+limit  # 6 ptr/int64 (src_div padded), 4 int32, y/ldy, act+variant+w_layout+pad
     assert C.sizeof(L.GemmFp8Args) == 8 * 8 + 16 + 16 + 16  # 8 ptr/int64, 4 int32, y/ldy, act+variant+w_layout+pad
-    assert L.MoEArgs.w_gate.offset == C.sizeof(L.MoEArgs) - 8 - 32  # then w13_bias, w2_bias, activation, alpha, limit, pad
+    assert L.MoEArgs.w_gate.offset == C.sizeof(L.MoEArgs) - 8 - 32  # then w13_bias, w2_bias, activation, alpha, limit, ws_layout
     a = L.MoEArgs()
     assert L.MoEArgs.M.offset == 0 and L.MoEArgs.logits.offset == 48 and C.sizeof(a) % 8 == 0
 

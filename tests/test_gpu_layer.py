@@ -56,6 +56,11 @@ SMALL = [
                                                          I_shared=128)),
     ("shared-same-width-rowmajor", "dsv3-decode", dict(M=50, H=272, E=8, K=2, I=80, n_group=2, topk_group=1,
                                                        I_shared=80)),
+    # routed weights tile, the shared expert's down projection (k = 32 bytes) cannot: one layout per group
+    ("tiled-routed-rowmajor-shared", "dsv3-decode", dict(M=2, H=1024, E=130, K=8, I=256, n_group=2, topk_group=2,
+                                                         I_shared=32)),
+    ("tiled-routed-rowmajor-shared-many", "dsv3-decode", dict(M=600, H=256, E=8, K=2, I=128, n_group=2,
+                                                              topk_group=1, I_shared=32)),
 ]
 
 

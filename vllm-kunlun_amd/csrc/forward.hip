@@ -47,8 +47,11 @@ int check_shape(const kmoe_moe_args* a) {
                "moe_forward: I_shared=%d must be a non-negative multiple of %d", a->I_shared, mult);
   KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "moe_forward: M*K too large");
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR ||
-                   (a->w_layout == KMOE_W_TILED && a->H % 64 == 0 && a->I % 64 == 0 && a->I_shared % 64 == 0),
+                   (a->w_layout == KMOE_W_TILED && a->H % 64 == 0 && a->I % 64 == 0),
                KMOE_ERR_SHAPE, "moe_forward: w_layout=%d needs H, I multiples of 64", a->w_layout);
+  KMOE_REQUIRE(a->I_shared == 0 || a->ws_layout == KMOE_W_ROWMAJOR ||
+                   (a->ws_layout == KMOE_W_TILED && a->H % 64 == 0 && a->I_shared % 64 == 0),
+               KMOE_ERR_SHAPE, "moe_forward: ws_layout=%d needs H, I_shared multiples of 64", a->ws_layout);
   return KMOE_OK;
 }
 
@@ -56,14 +59,16 @@ int check_shape(const kmoe_moe_args* a) {
 // against chunk-major codes; otherwise the LDS-tiled GEMM on row-major codes.
 bool use_stream_path(const kmoe_moe_args* a) {
   const long long P = static_cast<long long>(a->M) * a->K;
-  return a->format == KMOE_FMT_INT8 && a->w_layout == KMOE_W_TILED && (P + a->E - 1) / a->E <= 64 && a->M <= 1024;
+  // a row-major shared expert cannot read the chunk-major codes this path quantises x into
+  return a->format == KMOE_FMT_INT8 && a->w_layout == KMOE_W_TILED && (P + a->E - 1) / a->E <= 64 && a->M <= 1024 &&
+         (a->I_shared == 0 || a->ws_layout == KMOE_W_TILED);
 }
 
 // A shared expert of the routed experts' width runs inside the routed GEMM launches
 // as one more ("tail") expert over rows [P, P+M): no extra launches, and its few
 // workgroups overlap the routed experts' instead of leaving most CUs idle.
 bool fold_shared(const kmoe_moe_args* a) {
-  return a->format == KMOE_FMT_INT8 && a->I_shared > 0 && a->I_shared == a->I;
+  return a->format == KMOE_FMT_INT8 && a->I_shared > 0 && a->I_shared == a->I && a->ws_layout == a->w_layout;
 }
 
 // One expert-MLP pass (gate_up + SiLU-mul, requantise, down) over `rows` rows in
@@ -411,6 +416,7 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
     sh.src_div = 1;
     sh.w13 = a->ws13;
     sh.w2 = a->ws2;
+    sh.w_layout = a->ws_layout;
     sh.w13_aux = a->ws13_max;
     sh.w2_aux = a->ws2_max;
     sh.lod = dense_lod;

@@ -78,6 +78,19 @@ def tile_int8_weights_(w: torch.Tensor) -> bool:
     return True
 
 
+def can_tile(w: torch.Tensor) -> bool:
+    d = w.data
+    return (d.dtype in _TILEABLE and d.is_cuda and d.is_contiguous() and d.shape[-2] % 16 == 0
+            and (d.shape[-1] * d.element_size()) % 64 == 0)
+
+
+def tile_pair_(w13: torch.Tensor, w2: torch.Tensor) -> bool:
+    """Tiles the two weights of an MLP, or neither (a launch takes one layout for both)."""
+    if not (can_tile(w13) and can_tile(w2)):
+        return False
+    return tile_int8_weights_(w13) and tile_int8_weights_(w2)
+
+
 def rowmajor_int8_weights(w: torch.Tensor) -> torch.Tensor:
     """A row-major [..., n, k] COPY of int8 weights, undoing tile_int8_weights_ if it was applied."""
     if not is_tiled(w):
@@ -168,11 +181,17 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     a.act_alpha, a.act_limit = float(act_alpha), float(act_limit)
     a.out_scale = float(out_scale)
     a.out = out.data_ptr()
-    if w_layout is None:  # tiled only if every int8 weight of the call has been tiled
-        ws_all = [w13, w2] + ([shared_expert[0], shared_expert[2]] if shared_expert is not None else [])
-        w_layout = L.KMOE_W_TILED if all(is_tiled(t) for t in ws_all) else L.KMOE_W_ROWMAJOR
-        if w_layout == L.KMOE_W_ROWMAJOR and any(is_tiled(t) for t in ws_all):
-            raise ValueError("moe plan: routed and shared expert weights must be either all tiled or all row-major")
+    if w_layout is None:  # per group of weights: tiled if both of its tensors have been tiled
+        w_layout = L.KMOE_W_TILED if is_tiled(w13) and is_tiled(w2) else L.KMOE_W_ROWMAJOR
+        if w_layout == L.KMOE_W_ROWMAJOR and (is_tiled(w13) or is_tiled(w2)):
+            raise ValueError("moe plan: w13 and w2 must be either both tiled or both row-major")
+    ws_layout = L.KMOE_W_ROWMAJOR
+    if shared_expert is not None:
+        ws_tiled = [is_tiled(shared_expert[0]), is_tiled(shared_expert[2])]
+        if any(ws_tiled) and not all(ws_tiled):
+            raise ValueError("moe plan: the shared expert's two weights must be either both tiled or both row-major")
+        ws_layout = L.KMOE_W_TILED if all(ws_tiled) else L.KMOE_W_ROWMAJOR
+    a.ws_layout = int(ws_layout)
     a.w_layout = int(w_layout)
     if stage_events is not None:
         a.stage_events = stage_events

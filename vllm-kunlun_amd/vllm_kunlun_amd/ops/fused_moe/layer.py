@@ -46,12 +46,10 @@ class KunlunUnquantizedFusedMoEMethod:
     def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
         """The reference skips upstream's Triton kernel set-up here; on the GPU this build
         re-arranges the bf16 weights in place into MFMA-ready blocks (same values)."""
-        from ..._plan import tile_int8_weights_
-        w13, w2 = layer.w13_weight, layer.w2_weight
-        if getattr(self, "tile_weights", True) and w13.is_cuda and w13.shape[-1] % 32 == 0 and w2.shape[-1] % 32 == 0:
+        from ..._plan import tile_pair_
+        if getattr(self, "tile_weights", True):
             with torch.no_grad():
-                tile_int8_weights_(w13)
-                tile_int8_weights_(w2)
+                tile_pair_(layer.w13_weight, layer.w2_weight)
 
     def apply_monolithic(self, layer, x: torch.Tensor, router_logits: torch.Tensor):
         from .._kunlun_ops import KunlunOps as ops

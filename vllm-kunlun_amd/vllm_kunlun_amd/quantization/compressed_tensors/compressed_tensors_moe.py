@@ -17,7 +17,7 @@ from typing import Optional, Union
 import torch
 
 from ... import _lib as L
-from ..._plan import MoEPlan, make_moe_plan, tile_int8_weights_
+from ..._plan import MoEPlan, make_moe_plan, tile_pair_
 from ...ops import _custom_ops  # noqa: F401  (torch.ops._C.* used by the staged path)
 
 WNA16_SUPPORTED_BITS = (4, 8)
@@ -193,11 +193,8 @@ class KunlunCompressedTensorsW8A8Int8MoEMethod(_MonolithicQuantMoE):
         with torch.no_grad():
             layer.w13_weight_scale.mul_(127.0)
             layer.w2_weight_scale.mul_(127.0)
-            w13, w2 = layer.w13_weight, layer.w2_weight
-            if (getattr(self, "tile_weights", True) and w13.is_cuda and w13.shape[-1] % 64 == 0
-                    and w2.shape[-1] % 64 == 0 and w13.shape[-2] % 16 == 0 and w2.shape[-2] % 16 == 0):
-                tile_int8_weights_(w13)
-                tile_int8_weights_(w2)
+            if getattr(self, "tile_weights", True):
+                tile_pair_(layer.w13_weight, layer.w2_weight)
 
     def apply_staged(self, layer, x, router_logits, topk_group=None, num_expert_group=None, global_num_experts=-1,
                      scoring_func="softmax", routed_scaling_factor=1.0, e_score_correction_bias=None):
@@ -270,11 +267,9 @@ class KunlunCompressedTensorsW8A8Fp8MoEMethod(_MonolithicQuantMoE):
     def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
         """Block scales are used as they are (dequant = code * scale). On the GPU the e4m3 codes
         are re-arranged in place into the same MFMA-ready 1 KB blocks as int8 weights."""
-        w13, w2 = layer.w13_weight, layer.w2_weight
-        if getattr(self, "tile_weights", True) and w13.is_cuda:
+        if getattr(self, "tile_weights", True):
             with torch.no_grad():
-                tile_int8_weights_(w13)
-                tile_int8_weights_(w2)
+                tile_pair_(layer.w13_weight, layer.w2_weight)
 
 
 class KunlunCompressedTensorsWNA16MoEMethod:
@@ -328,8 +323,7 @@ class KunlunCompressedTensorsWNA16MoEMethod:
                 setattr(layer, f"{name}_weight", param)
                 delattr(layer, f"{name}_weight_packed")
             if getattr(self, "tile_weights", True):
-                tile_int8_weights_(layer.w13_weight)
-                tile_int8_weights_(layer.w2_weight)
+                tile_pair_(layer.w13_weight, layer.w2_weight)
 
     def apply_monolithic(self, layer, x: torch.Tensor, router_logits: torch.Tensor, **kwargs):
         """bf16 activations against the unpacked weights: KunlunOps.fused_moe, as the reference's

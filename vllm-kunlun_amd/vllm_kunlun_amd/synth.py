@@ -165,10 +165,9 @@ def make_fp8_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
         q13, s13 = _quant_block_fp8(torch.randn(2 * s.I_shared, s.H, generator=g, device=dev) * 0.02)
         q2, s2 = _quant_block_fp8(torch.randn(s.H, s.I_shared, generator=g, device=dev) * 0.02)
         shared = (q13, s13.contiguous(), q2, s2.contiguous())
-        from ._plan import is_tiled, tile_int8_weights_
+        from ._plan import is_tiled, tile_pair_
         if is_tiled(layer.w13_weight):
-            tile_int8_weights_(q13)
-            tile_int8_weights_(q2)
+            tile_pair_(q13, q2)
     x, logits = _activations(s, g, dev)
     return SynthLayer(s, layer, x, logits, bias, shared)
 
@@ -219,10 +218,9 @@ def make_w8a8_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer
         q13, s13 = _quant_rows_int8(torch.randn(2 * s.I_shared, s.H, generator=g, device=dev) * 0.02)
         q2, s2 = _quant_rows_int8(torch.randn(s.H, s.I_shared, generator=g, device=dev) * 0.02)
         shared = (q13, (s13 * 127.0).reshape(-1).contiguous(), q2, (s2 * 127.0).reshape(-1).contiguous())
-        from ._plan import is_tiled, tile_int8_weights_
+        from ._plan import is_tiled, tile_pair_
         if is_tiled(layer.w13_weight):  # the shared expert goes through the same load-time step
-            tile_int8_weights_(q13)
-            tile_int8_weights_(q2)
+            tile_pair_(q13, q2)
     x = torch.randn(s.M, s.H, generator=g, device=dev).to(torch.bfloat16)
     logits = torch.randn(s.M, s.E, generator=g, device=dev, dtype=torch.float32)
     if s.hot_experts:

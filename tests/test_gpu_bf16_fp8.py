@@ -171,6 +171,7 @@ def test_bf16_layer_config1_and_variants():
     from vllm_kunlun_amd import synth
     for shape in (synth.SHAPES["tiny-bf16"],
                   synth.scaled(synth.SHAPES["tiny-bf16"], M=300, H=256, E=16, K=4, I=128),
+                  synth.scaled(synth.SHAPES["tiny-bf16"], M=150, H=96, E=16, K=4, I=96),  # 192-byte rows tile
                   synth.scaled(synth.SHAPES["dsv3-decode"], M=40, H=256, E=32, K=4, I=128, n_group=4, topk_group=2,
                                I_shared=0, quant="none")):
         sl = synth.make_bf16_layer(shape, "cuda", seed=5)

@@ -46,12 +46,13 @@ int check_shape(const kmoe_moe_args* a) {
   KMOE_REQUIRE(a->I_shared >= 0 && a->I_shared % mult == 0, KMOE_ERR_SHAPE,
                "moe_forward: I_shared=%d must be a non-negative multiple of %d", a->I_shared, mult);
   KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "moe_forward: M*K too large");
+  const int row64 = a->format == KMOE_FMT_BF16 ? 32 : 64;  // elements in 64 bytes of a weight row
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR ||
-                   (a->w_layout == KMOE_W_TILED && a->H % 64 == 0 && a->I % 64 == 0),
-               KMOE_ERR_SHAPE, "moe_forward: w_layout=%d needs H, I multiples of 64", a->w_layout);
+                   (a->w_layout == KMOE_W_TILED && a->H % row64 == 0 && a->I % row64 == 0),
+               KMOE_ERR_SHAPE, "moe_forward: w_layout=%d needs H, I multiples of %d", a->w_layout, row64);
   KMOE_REQUIRE(a->I_shared == 0 || a->ws_layout == KMOE_W_ROWMAJOR ||
-                   (a->ws_layout == KMOE_W_TILED && a->H % 64 == 0 && a->I_shared % 64 == 0),
-               KMOE_ERR_SHAPE, "moe_forward: ws_layout=%d needs H, I_shared multiples of 64", a->ws_layout);
+                   (a->ws_layout == KMOE_W_TILED && a->H % row64 == 0 && a->I_shared % row64 == 0),
+               KMOE_ERR_SHAPE, "moe_forward: ws_layout=%d needs H, I_shared multiples of %d", a->ws_layout, row64);
   return KMOE_OK;
 }
 

@@ -462,9 +462,9 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
   if (a->rows == 0 && !(a->w_tail && a->tail_rows > 0)) return KMOE_OK;
   // Many rows per expert and tiled weights: the persistent 128-row-tile kernel (variants 5-7 force it)
   if (a->w_layout == KMOE_W_TILED && a->k % 128 == 0 &&
-      ((a->variant >= 5 && a->variant <= 8) || (a->variant == 0 && ceil_div(a->rows, a->E) > 48)))
+      ((a->variant >= 5 && a->variant <= 9) || (a->variant == 0 && ceil_div(a->rows, a->E) > 48)))
     return tiled_gemm_i8(a, as_stream(stream));
-  KMOE_REQUIRE(a->variant < 5 || a->variant > 8, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-8 need tiled weights and k %% 128 == 0");
+  KMOE_REQUIRE(a->variant < 5 || a->variant > 9, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-9 need tiled weights and k %% 128 == 0");
   GemmParams p{a->a,   a->lda, a->a_max, a->row_src, a->src_div, a->w,   a->w_max,
                a->lod, a->E,   a->n,     a->k,       a->y,       a->ldy, a->acc_out, a->w_layout == KMOE_W_TILED,
                a->w_tail, a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0, nullptr, 0, 0.f, 0.f};

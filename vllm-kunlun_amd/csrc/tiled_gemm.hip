@@ -1,27 +1,35 @@
-// MFMA-bound W8A8 grouped GEMM for the prefill regime (hundreds of rows per
-// expert), v_mfma_i32_16x16x64_i8, tiled int8 weights.
+// Grouped GEMM for the prefill regime (hundreds of rows per expert) on MFMA, tiled weights;
+// int8 (v_mfma_i32_16x16x64_i8), fp8 block-scaled and bf16 operands.
 //
 // Workgroup = 4 waves on a 128-row x 256-channel tile; each wave owns 64 channels
 // of all 128 rows: 8 x 4 accumulator fragments = 128 registers. Two workgroups
-// share a CU (2 waves per SIMD): one workgroup's LDS/L2 waits, barriers and its
+// share a CU (2 waves per SIMD): one workgroup's waits, barriers and its
 // VALU-heavy epilogue (dequant, exp, divide) run under the other's MFMAs.
-//   activations: global (rows gathered through the sort) -> registers -> LDS,
-//                128 bytes of K per row and chunk, double-buffered, pitch 160 B
-//                (measured: fragment reads at full LDS rate; pitch 144 costs 60% more);
-//                every A fragment read from LDS feeds 4 MFMAs.
+//   activations: int8 / bf16: asynchronous copies global -> LDS (rows gathered through the
+//                sort), 128 bytes of K per row and chunk, three chunks ahead into a ring of
+//                four chunk buffers, swizzled so that fragment reads are conflict-free without
+//                padding; no register holds them. fp8: through registers into two padded
+//                buffers (pitch 160 B), one chunk ahead, with the row scales of the chunk.
+//                Every A fragment read from LDS feeds 4 MFMAs.
 //   weights:     straight from L2 into registers, 1 KB of consecutive bytes per
 //                fragment and MFMA step (tiled layout), through a ring of 4 step
 //                buffers loaded 3 MFMA steps ahead of use; every B fragment
 //                feeds 8 MFMAs. No weight byte goes through LDS.
 // Workgroups are persistent: each walks a strided list of tiles. The tile after
 // the current one is located (from an LDS copy of lod) and its gather indices are
-// fetched while the current tile computes; its first activation chunk and weight
+// fetched while the current tile computes; its first activation chunks and weight
 // steps are requested BEFORE the current tile's epilogue, which hides their
 // latency. Per-row and per-channel scales of a tile wait in LDS, so the epilogue
 // touches global memory only to store. Output tiles are transposed through a
 // per-wave LDS patch so every store instruction writes whole 64/128-byte row
-// segments. Tile ids are mapped so that the tiles sharing an expert's weights run
-// at the same time on the same XCD (one L2).
+// segments. The tiles that read the same weight bytes run side by side on one XCD
+// (one L2), so an expert's weights leave HBM about once.
+//
+// The compiler drains every asynchronous copy in flight before any LDS access it can see.
+// Inside the pipeline the LDS accesses are therefore inline assembly with their own waits, and
+// the waits on the copies are explicit s_waitcnt vmcnt(N): a wave's loads complete in issue
+// order, so "at most N in flight" means "everything older than the N youngest has landed". Each
+// N below is the number of loads the wave is known to have issued after the copies it needs.
 #include <type_traits>
 
 #include "kmoe_common.h"
@@ -31,6 +39,8 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
@@ -53,12 +63,40 @@ __device__ inline v4i buffer_load16(__amdgpu_buffer_rsrc_t r, uint32_t lane_off,
   return (v4i)__builtin_amdgcn_raw_buffer_load_b128(r, lane_off, wave_off, 0);
 }
 
+// Asynchronous copy global -> LDS, 16 bytes per lane: lane l's bytes land at lds + 16 l (the
+// destination is one contiguous KB per instruction; which global bytes a lane fetches is free).
+// No register holds the data; the wave's VMEM counter covers completion.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+__device__ inline void buffer_load16_to_lds(__amdgpu_buffer_rsrc_t r, lds_ptr_t lds, uint32_t lane_off,
+                                            uint32_t wave_off) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, lds, 16, lane_off, wave_off, 0, 0);
+}
+// LDS reads the compiler does not see: it would otherwise drain every asynchronous copy in
+// flight before each of them. OFF: immediate byte offset. The wait that makes the value usable
+// is lds_wait<N> on the same variable (LDS operations of a wave complete in order).
+template <int OFF>
+__device__ inline v4i lds_read16_raw(uint32_t addr) {
+  v4i v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+  return v;
+}
+template <int N>
+__device__ inline void lds_wait(v4i& v) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(N));
+}
+// s_waitcnt with only the vector-memory counter set: at most N loads of this wave in flight
+template <int N>
+__device__ inline void vmem_wait() {
+  static_assert(N >= 0 && N < 64, "6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+
 constexpr int kMF = 8, kWavesT = 4;        // a wave: 8 row fragments (128 rows); 4 waves side by side along the channels
 constexpr int kChunk = 128;                // bytes of K per row and chunk (2 MFMA steps)
 constexpr int kSteps = kChunk / 64;
 constexpr int kPitchT = kChunk + 32;       // 160 B: measured conflict-free for the b128 fragment reads (144 is not)
-constexpr int kGroupTiles = 4;             // consecutive m-tiles kept on one XCD
 constexpr int kNA = 16 * kMF * (kChunk / 16) / (kWavesT * kWave);  // 16-byte activation vectors per thread and chunk (= 4)
+constexpr int kStagesA = 4;                // chunk buffers of the asynchronous activation path
 constexpr int kMaxExperts = 1024 + 1;      // routed experts + the tail expert
 
 struct TiledParams {
@@ -97,12 +135,24 @@ struct Tile {
 // WM: rows of waves. 1: 128-row tiles, 4 waves; 2: 256-row tiles, 8 waves, where the two waves
 // that share channels read the same weight bytes within one barrier interval (an expert with
 // up to 256 rows then streams its weights from HBM once).
-template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM>
+// M32: 32x32 MFMA shapes (v_mfma_i32_32x32x32_i8, v_mfma_f32_32x32x16_bf16) on the same tiles and
+// the same bytes: a wave's 128 x 64 patch is 4 x 2 accumulator fragments of 16 registers. One
+// wave alone on a SIMD issues these at 89 % of the peak rate (measured), the 16x16 shapes at
+// 58 %; with two waves on the SIMD both reach 91 %. A 32-channel weight fragment of one MFMA
+// (32 bytes of K) is two 16-lane quarters of two neighbouring 1 KB blocks, lanes 32-63 taking
+// the next 16 bytes of K; the activation fragment takes the same bytes of its rows, so the
+// order of K inside a step differs from the 16x16 path while the sums (exact in int32) do not.
+template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false>
 __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(const TiledParams p) {
   constexpr bool F8 = KIND == TKind::F8;
   constexpr bool I8 = KIND == TKind::I8;
   constexpr bool BF = KIND == TKind::BF16;
-  using acc_t = std::conditional_t<I8, v4i, v4f>;
+  static_assert(!(M32 && F8), "the 32x32 shapes are wired for int8 and bf16");
+  using acc_t = std::conditional_t<M32, std::conditional_t<I8, v16i, v16f>, std::conditional_t<I8, v4i, v4f>>;
+  constexpr int kFragRows = M32 ? 32 : 16;       // rows (and channels) of an accumulator fragment
+  constexpr int AM = 16 * kMF / kFragRows;       // accumulator fragments of a wave along the rows
+  constexpr int AN = 16 * NF / kFragRows;        // ... and along the channels
+  constexpr int kAccRegs = M32 ? 16 : 4;
   constexpr int kTM = WM * 16 * kMF;             // rows of a tile
   constexpr int kThreads = WM * kWavesT * kWave;
   static_assert(R == 4 || R == 8, "the chunk buffer parity is static only for R/2 even");
@@ -110,8 +160,14 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   constexpr int NFH = SWIGLU ? kNF / 2 : kNF;
   constexpr int kOutBytes = NFH * 16 * 2;   // bytes of one output row owned by a wave: 32 .. 128
   constexpr int kPatchPitch = kOutBytes + 16;  // bytes per row of a wave's output patch (16 rows)
-  __shared__ __attribute__((aligned(16))) int8_t lds_a[2][kTM * kPitchT];
-  __shared__ __attribute__((aligned(16))) int8_t patch[WM * kWavesT][16 * kPatchPitch];
+  // ADMA: activations go global -> LDS asynchronously, three chunks ahead, into a ring of four
+  // unpadded chunk buffers (row r, 16-byte vector c of a chunk at r * 128 + 16 (c ^ r % 8): eight
+  // consecutive rows of one fragment column fall on eight different bank groups). F8 keeps the
+  // register path (its row scales travel with the data): two padded buffers.
+  constexpr bool ADMA = !F8 && WM == 1;
+  constexpr int kStageBytes = ADMA ? kTM * kChunk : kTM * kPitchT;
+  __shared__ __attribute__((aligned(1024))) int8_t lds_a[ADMA ? kStagesA : 2][kStageBytes];
+  __shared__ __attribute__((aligned(16))) int8_t patch[WM * kWavesT][kFragRows * kPatchPitch];
   // I8, per tile parity: channel scales (w_max / 127) and row scales (a_max / 127)
   __shared__ __attribute__((aligned(16))) float sw_lds[I8 ? 2 : 1][I8 ? kWavesT * NF * 16 : 4];
   __shared__ float sa_lds[I8 ? 2 : 1][I8 ? kTM : 4];
@@ -128,8 +184,8 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   const int wave_id = threadIdx.x >> 6;
   const int wave = WM == 1 ? wave_id : wave_id % kWavesT;  // position along the channels
   const int wave_m = WM == 1 ? 0 : wave_id / kWavesT;      // position along the rows
-  const int li = lane & 15;
-  const int lg = lane >> 4;
+  const int li = lane & (kFragRows - 1);  // row (or channel) of a fragment held by this lane
+  const int lg = lane / kFragRows;        // 16-byte group of K (16x16: 0..3; 32x32: 0..1)
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int ksteps = p.k / 64;
   const int nchunks = ksteps / kSteps;  // the host only sends k % 128 == 0 here
@@ -159,30 +215,30 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   __syncthreads();
   const int total_tiles = tile_lo[n_exp];
 
-  // Work items = (m-tile, channel block) pairs, n_items of them, all non-empty; workgroup b
-  // takes items b, b + gridDim.x, ... so every workgroup gets the same count (+-1). Item ids
-  // are dealt to the 8 XCDs in runs: a run of kGroupTiles consecutive m-tiles (about one
-  // expert: same weights) with all their channel blocks is taken by workgroups of ONE XCD at
-  // about the same time, and successive runs rotate over the XCDs. The ids past the last
-  // whole round of 8 runs keep their natural order.
-  const int run = p.n_blocks * kGroupTiles;
+  // Work items = (m-tile, channel block) pairs, n_items of them, all non-empty, numbered expert
+  // by expert; inside an expert the m-tiles of one channel block are consecutive. The list is
+  // cut into 8 equal segments, one per XCD (workgroup b runs on XCD b % 8), and the workgroups
+  // of an XCD walk their segment side by side: the m-tiles that read the same weight bytes (and
+  // the channel blocks that read the same rows) run at the same time behind ONE L2, so an
+  // expert's weights leave HBM once - except for the experts a segment or a round cuts in two.
   const int n_items = total_tiles * p.n_blocks;
-  const int n_remapped = n_items / (8 * run) * (8 * run);
+  const int seg = (n_items + 7) >> 3;
   const int xcd = blockIdx.x & 7;
+  const int seg_end = min((xcd + 1) * seg, n_items);
   auto find_tile = [&](int it) -> Tile {
     Tile t{it, 0, 0, 0, false};
-    const int q = blockIdx.x + it * gridDim.x;  // gridDim.x is a multiple of 8: the XCD stays
-    if (q >= n_items) return t;
-    const int j = q >> 3;
-    const int lid = q < n_remapped ? ((j / run) * 8 + xcd) * run + j % run : q;
-    const int m_tile = lid / p.n_blocks;
+    const int lid = xcd * seg + (blockIdx.x >> 3) + it * (gridDim.x >> 3);  // gridDim.x is a multiple of 8
+    if (lid >= seg_end) return t;
+    const int m_tile = lid / p.n_blocks;  // tile_lo[e] <= m_tile < tile_lo[e + 1] <=> the item belongs to e
     int found = -1;
     for (int e = lane; e < n_exp; e += kWave)
       if (tile_lo[e] <= m_tile && m_tile < tile_lo[e + 1]) found = e;
     const uint64_t who = __ballot(found >= 0);  // exactly one lane
     t.e = __builtin_amdgcn_readfirstlane(__shfl(found, __builtin_ctzll(who), kWave));
-    t.row0 = __builtin_amdgcn_readfirstlane(rows_begin(t.e) + (m_tile - tile_lo[t.e]) * kTM);
-    t.nb = lid - m_tile * p.n_blocks;
+    const int first = tile_lo[t.e], mt = tile_lo[t.e + 1] - first;
+    const int u = lid - first * p.n_blocks;
+    t.nb = u / mt;
+    t.row0 = __builtin_amdgcn_readfirstlane(rows_begin(t.e) + (u - t.nb * mt) * kTM);
     t.valid = true;
     return t;
   };
@@ -199,8 +255,21 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     a_lds[i] = (v >> 3) * kPitchT + (v & 7) * 16;  // row v/8, 16-byte vector v%8 of the chunk
   }
   v4i wring[R][kNF];  // weight fragments of MFMA step s live in slot s % R
-  v4i areg[kNA];
-  acc_t acc[kMF][kNF];
+  v4i areg[ADMA ? 1 : kNA];
+  // ADMA: copy i of this wave fills rows 32 wave_id + 8 i + lane / 8 of a chunk buffer; the lane
+  // fetches vector (lane % 8) ^ (lane / 8 % 8) of its row, which lands at position lane % 8.
+  const int dma_row = wave_id * 32 + (lane >> 3);
+  const uint32_t dma_vec = static_cast<uint32_t>((lane & 7) ^ ((lane >> 3) & 7));
+  const uint32_t lds_a_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)&lds_a[0][0]));
+  // fragment reads: row li (+ 16 or 32 per fragment: same row % 8), vector v of the chunk at (v ^ li % 8)
+  auto frag_addr = [&](int v) -> uint32_t {
+    return lds_a_base + static_cast<uint32_t>((wave_m * 16 * kMF + li) * kChunk + ((v ^ (li & 7)) << 4));
+  };
+  // 16x16: vector 4 j + lg of step j; 32x32: vector 4 j + 2 t + lg of step j, K part t
+  uint32_t fa[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) fa[q] = M32 ? frag_addr(2 * q + lg) : frag_addr(4 * (q & 1) + lg);
+  acc_t acc[AM][AN];
   const int kblocks = p.k / 128;  // F8: scale blocks along K (= chunks)
   int my_srow = 0;                // F8: source row of tile row threadIdx.x % kTM
   float asc_reg = 0.0f;           // F8: that row's scale of the chunk in flight
@@ -210,25 +279,51 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   // results of those are never stored, and the loop body stays one basic block.
   auto load_w = [&](v4i(&dst)[kNF], int kb) {
     const uint32_t off = static_cast<uint32_t>(min(kb, last_step)) * 1024u;
+    if constexpr (M32) {
 #pragma unroll
-    for (int f = 0; f < kNF; ++f) dst[f] = buffer_load16(w_rsrc, woff[f], off);
+      for (int f = 0; f < kNF; ++f) dst[f] = buffer_load16(w_rsrc, woff[f >> 1], off + (f & 1) * 512u);
+    } else {
+#pragma unroll
+      for (int f = 0; f < kNF; ++f) dst[f] = buffer_load16(w_rsrc, woff[f], off);
+    }
   };
   auto load_a = [&](int chunk) {
-    const uint32_t kc = static_cast<uint32_t>(min(chunk, last_chunk)) * kChunk;
+    if constexpr (!ADMA) {
+      const uint32_t kc = static_cast<uint32_t>(min(chunk, last_chunk)) * kChunk;
 #pragma unroll
-    for (int i = 0; i < kNA; ++i) areg[i] = buffer_load16(a_rsrc, aoff[i], kc);
-    if constexpr (F8) asc_reg = p.a_max[static_cast<size_t>(my_srow) * kblocks + min(chunk, last_chunk)];
+      for (int i = 0; i < kNA; ++i) areg[i] = buffer_load16(a_rsrc, aoff[i], kc);
+      if constexpr (F8) asc_reg = p.a_max[static_cast<size_t>(my_srow) * kblocks + min(chunk, last_chunk)];
+    }
   };
   auto store_a = [&](int buf) {
+    if constexpr (!ADMA) {
 #pragma unroll
-    for (int i = 0; i < kNA; ++i) *reinterpret_cast<v4i*>(&lds_a[buf][a_lds[i]]) = areg[i];
-    if constexpr (F8) asc_lds[buf][threadIdx.x] = asc_reg;
+      for (int i = 0; i < kNA; ++i) *reinterpret_cast<v4i*>(&lds_a[buf][a_lds[i]]) = areg[i];
+      if constexpr (F8) asc_lds[buf][threadIdx.x] = asc_reg;
+    }
+  };
+  // ADMA: requests chunk `chunk` of the tile into ring buffer `stage` (4 copies per wave)
+  auto dma_a = [&](int chunk, int stage) {
+    if constexpr (ADMA) {
+      const uint32_t kc = static_cast<uint32_t>(min(chunk, last_chunk)) * kChunk;
+#pragma unroll
+      for (int i = 0; i < kNA; ++i)
+        buffer_load16_to_lds(a_rsrc, (lds_ptr_t)&lds_a[stage][(wave_id * kNA + i) * 1024], aoff[i], kc);
+    }
   };
   // one MFMA step: 8 A fragments from LDS, each against the 4 weight fragments of the slot
-  auto compute = [&](const v4i(&wcur)[kNF], int buf, int j) {
+  auto mfma_row = [&](const v4i(&wcur)[kNF], const v4i& af, int mf, int t) {
+    if constexpr (M32) {
+      // slot entry 2 g + t: 32-channel fragment g, K bytes [32 t, 32 t + 32) of the step
 #pragma unroll
-    for (int mf = 0; mf < kMF; ++mf) {
-      const v4i af = *reinterpret_cast<const v4i*>(&lds_a[buf][(wave_m * 16 * kMF + mf * 16 + li) * kPitchT + j * 64 + lg * 16]);
+      for (int g = 0; g < AN; ++g) {
+        if constexpr (BF)
+          acc[mf][g] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, wcur[2 * g + t]),
+                                                               __builtin_bit_cast(v8bf, af), acc[mf][g], 0, 0, 0);
+        else if constexpr (I8)
+          acc[mf][g] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wcur[2 * g + t], af, acc[mf][g], 0, 0, 0);
+      }
+    } else {
 #pragma unroll
       for (int f = 0; f < kNF; ++f) {
         if constexpr (BF)
@@ -239,8 +334,42 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
       }
     }
   };
+  // fragment n of a step: (row fragment, K part); 16x16: 8 row fragments; 32x32: 2 K parts x 4
+  constexpr int kFragReads = M32 ? 2 * AM : kMF;
+  auto compute = [&](const v4i(&wcur)[kNF], auto buf_tag, auto j_tag) {
+    constexpr int buf = decltype(buf_tag)::value, j = decltype(j_tag)::value;
+    if constexpr (ADMA) {
+      // two fragments in flight: the read of fragment n + 1 leaves before the MFMAs of fragment n
+      v4i af[2];
+      af[0] = lds_read16_raw<buf * kStageBytes>(fa[M32 ? 2 * j : j]);
+#pragma unroll
+      for (int n = 0; n < kFragReads; ++n) {
+        const int mf = M32 ? n % AM : n, t = M32 ? n / AM : 0;
+        if (n + 1 < kFragReads) {
+          const int mf1 = M32 ? (n + 1) % AM : n + 1, t1 = M32 ? (n + 1) / AM : 0;
+          asm volatile("ds_read_b128 %0, %1 offset:%2"
+                       : "=v"(af[(n + 1) & 1])
+                       : "v"(fa[M32 ? 2 * j + t1 : j]), "i"(buf * kStageBytes + mf1 * kFragRows * kChunk)
+                       : "memory");
+          lds_wait<1>(af[n & 1]);
+        } else {
+          lds_wait<0>(af[n & 1]);
+        }
+        mfma_row(wcur, af[n & 1], mf, t);
+      }
+    } else {
+#pragma unroll
+      for (int n = 0; n < kFragReads; ++n) {
+        const int mf = M32 ? n % AM : n, t = M32 ? n / AM : 0;
+        const v4i af = *reinterpret_cast<const v4i*>(
+            &lds_a[buf][(wave_m * 16 * kMF + mf * kFragRows + li) * kPitchT + j * 64 + (M32 ? t * 32 : 0) + lg * 16]);
+        mfma_row(wcur, af, mf, t);
+      }
+    }
+  };
   // F8, one whole chunk: the two ring slots of the chunk are the K halves of one MFMA
   auto compute_f8 = [&](const v4i(&w_lo)[kNF], const v4i(&w_hi)[kNF], int buf, int chunk, int parity) {
+    if constexpr (!M32) {
     float swc[kNF];
 #pragma unroll
     for (int f = 0; f < kNF; ++f) swc[f] = wsc_lds[parity][(wave * kNF + f) * kMaxKBlocks + chunk];
@@ -266,15 +395,22 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
       // scheduler issues all 32 MFMAs first and spills their 128 results
       __builtin_amdgcn_sched_barrier(0);
     }
+    }
   };
   // Gather index of sorted row r of tile t (rows past the expert's end: the tile's first row),
   // and the source row (row of p.a / p.a_max) it names.
   auto fetch_src = [&](const Tile& t, int r) -> int {
     const int rr = r < rows_end(t.e) ? r : t.row0;
-    return (t.e < p.E && p.row_src) ? p.row_src[rr] : rr;
+    if (!p.row_src) return rr;
+    const int g = p.row_src[t.e < p.E ? rr : 0];  // always one load (the tail expert's rows are not gathered)
+    return t.e < p.E ? g : rr;
   };
+  // gather entries are flat (source row, slot) ids: source row = entry / src_div (a shift for the usual powers of two)
+  const int src_shift = (p.src_div & (p.src_div - 1)) == 0 ? __builtin_ctz(p.src_div) : -1;
   auto src_row = [&](const Tile& t, int fetched) -> int {
-    return t.e >= p.E ? p.tail_src0 + fetched - p.tail_row0 : (p.row_src ? fetched / p.src_div : fetched);
+    if (t.e >= p.E) return p.tail_src0 + fetched - p.tail_row0;
+    if (!p.row_src) return fetched;
+    return src_shift >= 0 ? fetched >> src_shift : fetched / p.src_div;
   };
   auto col_of = [&](const Tile& t, int f, bool& ok) -> int {
     const int fh = SWIGLU ? f % NFH : f;
@@ -283,31 +419,63 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     return (SWIGLU && f >= NFH) ? n_half + c : c;
   };
 
+  // tile row and byte column (within a chunk) of this thread's i-th activation vector
+  auto a_row = [&](int i) -> int { return ADMA ? dma_row + 8 * i : (threadIdx.x + i * kThreads) >> 3; };
+  const uint32_t a_col = ADMA ? dma_vec * 16u : (threadIdx.x & 7) * 16u;  // kThreads % 8 == 0
   Tile cur = find_tile(0);
   if (!cur.valid) return;  // the whole workgroup leaves together
   int rs[kNA];             // gather indices of this thread's activation rows
 #pragma unroll
-  for (int i = 0; i < kNA; ++i) rs[i] = fetch_src(cur, cur.row0 + ((threadIdx.x + i * kThreads) >> 3));
+  for (int i = 0; i < kNA; ++i) rs[i] = fetch_src(cur, cur.row0 + a_row(i));
+  // gather index of the tile row whose scale this thread fetches (I8: row threadIdx.x; F8: threadIdx.x % kTM)
+  const int scale_row = F8 ? threadIdx.x % kTM : min(static_cast<int>(threadIdx.x), kTM - 1);
+  int rs_scale = fetch_src(cur, cur.row0 + scale_row);
   float sw_reg = 0.0f, sa_reg = 0.0f;  // this thread's share of the tile's scales, on their way to LDS
   float wsc_reg[kMaxKBlocks / 16];     // F8: weight block scales k = c, c + 16, ... of fragment lane / 16
 
   // Points the loaders at tile t and requests its first chunk, first three weight steps and scales.
-  auto start_tile = [&](const Tile& t) {
+  auto start_tile = [&](const Tile& t, int t_parity) {
     const int8_t* w_base = t.e >= p.E ? p.w_tail : p.w + static_cast<size_t>(t.e) * p.n * p.k;
     [[maybe_unused]] const float* w_max = t.e >= p.E ? p.w_max_tail : p.w_max + static_cast<size_t>(t.e) * p.n;
     w_rsrc = make_rsrc(w_base);
+    if constexpr (M32) {
+      // lane: channel lane % 32 of the fragment = row lane % 16 of block (lane / 16) % 2; K quarter lane / 32 (+ 2 t)
 #pragma unroll
-    for (int f = 0; f < kNF; ++f) {
-      bool ok;
-      const int c = col_of(t, f, ok);
-      woff[f] = static_cast<uint32_t>(ok ? c / 16 : 0) * ksteps * 1024u + lane * 16u;
+      for (int g = 0; g < AN; ++g) {
+        bool ok;
+        const int c = col_of(t, 2 * g + ((lane >> 4) & 1), ok);
+        woff[g] = static_cast<uint32_t>(ok ? c / 16 : 0) * ksteps * 1024u + (lane >> 5) * 256u + (lane & 15) * 16u;
+      }
+    } else {
+#pragma unroll
+      for (int f = 0; f < kNF; ++f) {
+        bool ok;
+        const int c = col_of(t, f, ok);
+        woff[f] = static_cast<uint32_t>(ok ? c / 16 : 0) * ksteps * 1024u + lane * 16u;
+      }
     }
 #pragma unroll
     for (int i = 0; i < kNA; ++i)
-      aoff[i] = static_cast<uint32_t>(src_row(t, rs[i])) * static_cast<uint32_t>(p.lda) +
-                ((threadIdx.x + i * kThreads) & 7) * 16;  // < 4 GiB: host-checked
-    if constexpr (F8) my_srow = src_row(t, fetch_src(t, t.row0 + threadIdx.x % kTM));
+      aoff[i] = static_cast<uint32_t>(src_row(t, rs[i])) * static_cast<uint32_t>(p.lda) + a_col;  // < 4 GiB: host-checked
+    if constexpr (F8) my_srow = src_row(t, rs_scale);
     load_a(0);
+    dma_a(0, 0);
+    dma_a(1, 1);
+    dma_a(2, 2);
+    if constexpr (I8 && ADMA) {
+      // the tile's absmax values travel the same way, 4 bytes per lane, straight into the slots
+      // their scales will occupy (the loop top divides them by 127 in place)
+      if ((lane >> 4) < kNF) {  // lane = 16 f + c: channel c of fragment f of this wave
+        bool ok;
+        const int c = col_of(t, lane >> 4, ok);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(make_rsrc(w_max), (lds_ptr_t)&sw_lds[t_parity][wave * kNF * 16], 4,
+                                                 static_cast<uint32_t>(ok ? c + (lane & 15) : 0) * 4u, 0, 0, 0);
+      }
+      if (wave_id * kWave < kTM)  // thread r: tile row r
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(make_rsrc(p.a_max), (lds_ptr_t)&sa_lds[t_parity][wave_id * kWave], 4,
+                                                 static_cast<uint32_t>(src_row(t, rs_scale)) * 4u, 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // the weight loads below stay younger than the copies above (see the wait at the loop top)
 #pragma unroll
     for (int i = 0; i < R - 1; ++i) load_w(wring[i], i);
     if constexpr (F8) {
@@ -322,25 +490,29 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
           wsc_reg[i] = kb < kblocks ? ws[kb] : 0.0f;
         }
       }
-    } else if constexpr (I8) {
+    } else if constexpr (I8 && !ADMA) {
       if (wave_m == 0 && (lane >> 4) < kNF) {  // thread (wave, f = lane / 16, c = lane % 16): scale of channel c of fragment f of this wave
         bool ok;
         const int c = col_of(t, lane >> 4, ok);
         sw_reg = ok ? w_max[c + (lane & 15)] : 0.0f;
       }
       if (threadIdx.x < kTM)  // thread r: scale of tile row r
-        sa_reg = p.a_max[src_row(t, fetch_src(t, t.row0 + threadIdx.x))];
+        sa_reg = p.a_max[src_row(t, rs_scale)];
     }
   };
-  start_tile(cur);
+  start_tile(cur, 0);
 
   for (int parity = 0;; parity ^= 1) {
     // the tile after this one: found now, its gather indices travel during the MFMA loop
     const Tile nxt = find_tile(cur.it + 1);
+    // (after the last tile the loads repeat the current one's: always kNA + 1 loads, which the
+    // wait below counts on)
+    const Tile look = nxt.valid ? nxt : cur;
     int rs_next[kNA];
 #pragma unroll
-    for (int i = 0; i < kNA; ++i)
-      rs_next[i] = nxt.valid ? fetch_src(nxt, nxt.row0 + ((threadIdx.x + i * kThreads) >> 3)) : 0;
+    for (int i = 0; i < kNA; ++i) rs_next[i] = fetch_src(look, look.row0 + a_row(i));
+    const int rs_scale_next = fetch_src(look, look.row0 + scale_row);
+    __builtin_amdgcn_sched_barrier(0);
 
     if constexpr (F8) {
       if (wave_m == 0 && (lane >> 4) < kNF) {
@@ -348,18 +520,39 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         for (int i = 0; i < kMaxKBlocks / 16; ++i)
           wsc_lds[parity][(wave * kNF + (lane >> 4)) * kMaxKBlocks + (lane & 15) + 16 * i] = wsc_reg[i];
       }
-    } else if constexpr (I8) {
+    } else if constexpr (I8 && !ADMA) {
       if (wave_m == 0 && (lane >> 4) < kNF) sw_lds[parity][wave * kNF * 16 + lane] = sw_reg / 127.0f;
       if (threadIdx.x < kTM) sa_lds[parity][threadIdx.x] = sa_reg / 127.0f;
     }
     store_a(0);
+    // ADMA: the copies of chunks 0-2 have landed - after them start_tile issued its (R - 1) kNF
+    // weight loads and the lines above kNA + 1 index loads (with a gather), so that many younger
+    // operations may stay in flight (the epilogue's stores among them); the barrier below then
+    // publishes the chunks
+    if constexpr (ADMA) {
+      if (p.row_src) vmem_wait<(R - 1) * kNF + kNA + 1>();
+      else vmem_wait<(R - 1) * kNF>();
+    }
+    if constexpr (I8 && ADMA) {
+      // absmax -> scale in place, each slot by the thread that requested it (LDS instructions
+      // the compiler does not see: no wait for the gather-index loads just issued)
+      auto scale_in_place = [&](const float* slot) {
+        const uint32_t addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)slot));
+        float raw;
+        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(raw) : "v"(addr) : "memory");
+        const float scaled = raw / 127.0f;
+        asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(scaled) : "memory");
+      };
+      if ((lane >> 4) < kNF) scale_in_place(&sw_lds[parity][wave * kNF * 16 + lane]);
+      if (threadIdx.x < kTM) scale_in_place(&sa_lds[parity][threadIdx.x]);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
 #pragma unroll
-    for (int mf = 0; mf < kMF; ++mf)
+    for (int mf = 0; mf < AM; ++mf)
 #pragma unroll
-      for (int f = 0; f < kNF; ++f) {
-        if constexpr (!I8) acc[mf][f] = (v4f){0.f, 0.f, 0.f, 0.f};
-        else acc[mf][f] = (v4i){0, 0, 0, 0};
-      }
+      for (int f = 0; f < AN; ++f)
+#pragma unroll
+        for (int q = 0; q < kAccRegs; ++q) acc[mf][f][q] = 0;
     __syncthreads();
 
     // One chunk (two MFMA steps) of the pipeline; h = position of the chunk in the ring
@@ -368,7 +561,10 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     // (the counters retire in issue order, so a wait lets the later loads stay in flight).
     auto chunk_step = [&](int c0, auto h_tag) {
       constexpr int h = decltype(h_tag)::value;
-      constexpr int buf = h & 1;
+      constexpr int buf = ADMA ? h % kStagesA : h & 1;
+      using buf_t = std::integral_constant<int, buf>;
+      using j0_t = std::integral_constant<int, 0>;
+      using j1_t = std::integral_constant<int, 1>;
       const int s0 = (c0 + h) * kSteps;
       load_a(c0 + h + 1);
       load_w(wring[(2 * h + R - 1) % R], s0 + R - 1);
@@ -378,98 +574,144 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         __builtin_amdgcn_sched_barrier(0);
         load_w(wring[(2 * h) % R], s0 + R);
       } else {
-        compute(wring[(2 * h) % R], buf, 0);
+        compute(wring[(2 * h) % R], buf_t{}, j0_t{});
         __builtin_amdgcn_sched_barrier(0);
         load_w(wring[(2 * h) % R], s0 + R);
+        // the buffer chunk c - 1 was read from is free since the last barrier: chunk c + 3 goes there
+        dma_a(c0 + h + kStagesA - 1, (buf + kStagesA - 1) % kStagesA);
         __builtin_amdgcn_sched_barrier(0);
-        compute(wring[(2 * h + 1) % R], buf, 1);
+        compute(wring[(2 * h + 1) % R], buf_t{}, j1_t{});
       }
       __builtin_amdgcn_sched_barrier(0);
       store_a(buf ^ 1);
-      __syncthreads();
+      // ADMA: the 12 loads above may still be in flight, everything older has landed - among
+      // it this wave's part of chunks c + 1 and c + 2; the barrier publishes them
+      // (a bare barrier: the fence of __syncthreads would drain every load in flight, since the
+      // asynchronous copies count as stores to LDS)
+      if constexpr (ADMA) {
+        vmem_wait<2 * kNF + kNA>();
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      } else {
+        __syncthreads();
+      }
     };
+    constexpr int kPeriod = ADMA ? kStagesA : R / 2;  // chunks after which ring slots and buffers repeat
+    static_assert(kPeriod == 2 || kPeriod == 4, "unrolled by hand below");
     int c = 0;
-    for (; c + R / 2 <= nchunks; c += R / 2) {  // one ring period = R MFMA steps per iteration
+    for (; c + kPeriod <= nchunks; c += kPeriod) {
       chunk_step(c, std::integral_constant<int, 0>{});
       chunk_step(c, std::integral_constant<int, 1>{});
-      if constexpr (R == 8) {
+      if constexpr (kPeriod == 4) {
         chunk_step(c, std::integral_constant<int, 2>{});
         chunk_step(c, std::integral_constant<int, 3>{});
       }
     }
     // the chunks left over (fewer than a period): same steps, loads past the end are clamped
     if (c < nchunks) chunk_step(c, std::integral_constant<int, 0>{});
-    if constexpr (R == 8) {
+    if constexpr (kPeriod == 4) {
       if (c + 1 < nchunks) chunk_step(c, std::integral_constant<int, 1>{});
       if (c + 2 < nchunks) chunk_step(c, std::integral_constant<int, 2>{});
     }
 
-    // ---- switch: request the next tile's first loads, then finish this tile ----
+    // ---- switch: the finished tile's scales leave LDS first (LDS reads the compiler sees wait
+    // for every asynchronous copy in flight, so none may follow start_tile), then the next
+    // tile's first loads are requested, then this tile is finished ----
     const Tile done = cur;
+    // Registers of a lane: row li of the fragment; channel-in-wave fr * kFragRows + 8 (v / 4) + 4 lg + v % 4
+    // for register v of fragment fr (16x16: v < 4).
+    constexpr int ANH = SWIGLU ? AN / 2 : AN;
+    constexpr int kQuads = kAccRegs / 4;
+    float sw[AN][kAccRegs];
+    float sa_r[AM];
+    if constexpr (I8) {
+#pragma unroll
+      for (int fr = 0; fr < AN; ++fr)
+#pragma unroll
+        for (int b = 0; b < kQuads; ++b) {
+          const float4 s4 = *reinterpret_cast<const float4*>(
+              &sw_lds[parity][wave * kNF * 16 + fr * kFragRows + b * 8 + lg * 4]);
+          sw[fr][4 * b + 0] = s4.x;
+          sw[fr][4 * b + 1] = s4.y;
+          sw[fr][4 * b + 2] = s4.z;
+          sw[fr][4 * b + 3] = s4.w;
+        }
+#pragma unroll
+      for (int mf = 0; mf < AM; ++mf) sa_r[mf] = sa_lds[parity][wave_m * 16 * kMF + mf * kFragRows + li];
+    }
+    __builtin_amdgcn_sched_barrier(0);
     if (nxt.valid) {
 #pragma unroll
       for (int i = 0; i < kNA; ++i) rs[i] = rs_next[i];
+      rs_scale = rs_scale_next;
       cur = nxt;
-      start_tile(cur);
+      start_tile(cur, parity ^ 1);
     }
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- epilogue of `done`: dequantise, optional SiLU-mul, transpose through LDS, store ----
     const int row_end = min(rows_end(done.e), done.row0 + kTM);
     bool wok[kNF];
-    int col[kNF];
-    float sw[kNF][4];
+    int col[kNF];  // per 16-channel block of this wave
 #pragma unroll
-    for (int f = 0; f < kNF; ++f) {
-      col[f] = col_of(done, f, wok[f]);
-      if constexpr (I8) {
-        const float4 s4 = *reinterpret_cast<const float4*>(&sw_lds[parity][(wave * kNF + f) * 16 + lg * 4]);
-        sw[f][0] = s4.x;
-        sw[f][1] = s4.y;
-        sw[f][2] = s4.z;
-        sw[f][3] = s4.w;
-      }
-    }
-    int8_t* my_patch = patch[wave_id];
+    for (int f = 0; f < kNF; ++f) col[f] = col_of(done, f, wok[f]);
+    // the patch is written and read with LDS instructions the compiler does not see (same reason)
+    const uint32_t patch_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)&patch[wave_id][0]));
+    const uint32_t patch_wr = patch_base + static_cast<uint32_t>(li * kPatchPitch + lg * 8);
     // reader side of the patch: lane -> (row, 16-byte vector), consecutive lanes cover a row
     constexpr int kVecPerRow = kOutBytes / 16;        // 2, 4 or 8
-    constexpr int kRowsPerRead = kWave / kVecPerRow;  // 32 (half the lanes idle), 16 or 8
-    constexpr int kReads = kRowsPerRead >= 16 ? 1 : 16 / kRowsPerRead;
+    constexpr int kRowsPerRead = kWave / kVecPerRow;  // 32, 16 or 8
+    constexpr int kReads = kRowsPerRead >= kFragRows ? 1 : kFragRows / kRowsPerRead;
     const int rd_row = lane / kVecPerRow, rd_vec = lane % kVecPerRow;
+    const uint32_t patch_rd =
+        patch_base + static_cast<uint32_t>((rd_row & (kFragRows - 1)) * kPatchPitch + rd_vec * 16);
     const int out_col0 = (done.nb * kWavesT + wave) * NFH * 16;  // first output channel of this wave
 #pragma unroll
-    for (int mf = 0; mf < kMF; ++mf) {
+    for (int mf = 0; mf < AM; ++mf) {
       float sa = 1.0f;
-      if constexpr (I8) sa = sa_lds[parity][wave_m * 16 * kMF + mf * 16 + li];
-      const int r = done.row0 + wave_m * 16 * kMF + mf * 16 + li;
+      if constexpr (I8) sa = sa_r[mf];
+      const int r = done.row0 + wave_m * 16 * kMF + mf * kFragRows + li;
 #pragma unroll
-      for (int f = 0; f < NFH; ++f) {
-        float yv[4];
+      for (int fr = 0; fr < ANH; ++fr) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          if constexpr (!I8) yv[q] = acc[mf][f][q];
-          else yv[q] = (static_cast<float>(acc[mf][f][q]) * sa) * sw[f][q];
-        }
-        if (SWIGLU) {
-          const int fu = f + NFH;
+        for (int b = 0; b < kQuads; ++b) {
+          float yv[4];
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const float g = bf16_to_f32(f32_to_bf16_hw(yv[q]));  // gate and up are bf16 values first
-            float uf;
-            if constexpr (!I8) uf = acc[mf][fu][q];
-            else uf = (static_cast<float>(acc[mf][fu][q]) * sa) * sw[fu][q];
-            const float u = bf16_to_f32(f32_to_bf16_hw(uf));
-            yv[q] = silu_fixed(g) * u;
+            if constexpr (!I8) yv[q] = acc[mf][fr][4 * b + q];
+            else yv[q] = (static_cast<float>(acc[mf][fr][4 * b + q]) * sa) * sw[fr][4 * b + q];
           }
-        }
-        *reinterpret_cast<uint2*>(&my_patch[li * kPatchPitch + f * 32 + lg * 8]) =
-            make_uint2(pack2_bf16(yv[0], yv[1]), pack2_bf16(yv[2], yv[3]));
-        if constexpr (I8) {
-          if (p.acc_out && r < row_end && wok[f]) {
-            *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[f] + lg * 4) = acc[mf][f];
-            if (SWIGLU)
-              *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[f + NFH] + lg * 4) =
-                  acc[mf][f + NFH];
+          if (SWIGLU) {
+            const int fu = fr + ANH;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float g = bf16_to_f32(f32_to_bf16_hw(yv[q]));  // gate and up are bf16 values first
+              float uf;
+              if constexpr (!I8) uf = acc[mf][fu][4 * b + q];
+              else uf = (static_cast<float>(acc[mf][fu][4 * b + q]) * sa) * sw[fu][4 * b + q];
+              const float u = bf16_to_f32(f32_to_bf16_hw(uf));
+              yv[q] = silu_fixed(g) * u;
+            }
+          }
+          // channel of yv[0] within the wave's output: fr * kFragRows + b * 8 + lg * 4
+          const uint2 packed = make_uint2(pack2_bf16(yv[0], yv[1]), pack2_bf16(yv[2], yv[3]));
+          asm volatile("ds_write_b64 %0, %1 offset:%2"
+                       :
+                       : "v"(patch_wr), "v"(packed), "i"((fr * kFragRows + b * 8) * 2)
+                       : "memory");
+          if constexpr (I8) {
+            const int f16 = M32 ? 2 * fr + (b >> 1) : fr;
+            const int cofs = M32 ? (b & 1) * 8 + lg * 4 : lg * 4;
+            if (p.acc_out && r < row_end && wok[f16]) {
+              const v4i lo = {acc[mf][fr][4 * b], acc[mf][fr][4 * b + 1], acc[mf][fr][4 * b + 2], acc[mf][fr][4 * b + 3]};
+              *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[f16] + cofs) = lo;
+              if (SWIGLU) {
+                const int fu = fr + ANH;
+                const v4i hi = {acc[mf][fu][4 * b], acc[mf][fu][4 * b + 1], acc[mf][fu][4 * b + 2],
+                                acc[mf][fu][4 * b + 3]};
+                *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + col[f16 + NFH] + cofs) = hi;
+              }
+            }
           }
         }
       }
@@ -477,10 +719,15 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
 #pragma unroll
       for (int h = 0; h < kReads; ++h) {
         const int pr = h * kRowsPerRead + rd_row;
-        const v4i v = *reinterpret_cast<const v4i*>(&my_patch[(pr & 15) * kPatchPitch + rd_vec * 16]);
-        const int orow = done.row0 + wave_m * 16 * kMF + mf * 16 + pr;
+        v4i v;  // a wave's LDS operations execute in order: this read sees the writes above
+        asm volatile("ds_read_b128 %0, %1 offset:%2"
+                     : "=v"(v)
+                     : "v"(patch_rd), "i"(kReads > 1 ? h * kRowsPerRead * kPatchPitch : 0)
+                     : "memory");
+        lds_wait<0>(v);
+        const int orow = done.row0 + wave_m * 16 * kMF + mf * kFragRows + pr;
         const int ocol = out_col0 + rd_vec * 8;
-        if (pr < 16 && orow < row_end && ocol < n_half)  // n_half % 16 == 0: a vector of 8 channels is all in or all out
+        if (pr < kFragRows && orow < row_end && ocol < n_half)  // n_half % 16 == 0: a vector of 8 channels is all in or all out
           *reinterpret_cast<v4i*>(p.y + static_cast<size_t>(orow) * p.ldy + ocol) = v;
       }
       __builtin_amdgcn_wave_barrier();
@@ -489,7 +736,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   }
 }
 
-template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM>
+template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false>
 int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* what) {
   constexpr int kTM = WM * 16 * kMF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
@@ -501,7 +748,7 @@ int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* w
   // persistent workgroups: WGS per CU
   const int grid = min(ceil_div(p.max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8);
   const size_t dyn = sizeof(int) * (static_cast<size_t>(p.E) + 1 + n_exp + 1);
-  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM>), dim3(grid), dim3(WM * kWavesT * kWave), dyn, s,
+  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32>), dim3(grid), dim3(WM * kWavesT * kWave), dyn, s,
                      p);
   return check_launch(what);
 }
@@ -554,6 +801,9 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   if (a->variant == 8)
     return swiglu ? launch_tiled<K, true, 4, 4, 1, 2>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 1, 2>(p, a->rows, s, n_cu, what);
+  if (a->variant == 9)
+    return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what);
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)
                 : launch_tiled<K, false, 4, 4, 2, 1>(p, a->rows, s, n_cu, what);
 }

@@ -164,7 +164,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   // unpadded chunk buffers (row r, 16-byte vector c of a chunk at r * 128 + 16 (c ^ r % 8): eight
   // consecutive rows of one fragment column fall on eight different bank groups). F8 keeps the
   // register path (its row scales travel with the data): two padded buffers.
-  constexpr bool ADMA = !F8 && WM == 1;
+  constexpr bool ADMA = !F8;
   constexpr int kStageBytes = ADMA ? kTM * kChunk : kTM * kPitchT;
   __shared__ __attribute__((aligned(1024))) int8_t lds_a[ADMA ? kStagesA : 2][kStageBytes];
   __shared__ __attribute__((aligned(16))) int8_t patch[WM * kWavesT][kFragRows * kPatchPitch];
@@ -256,9 +256,9 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   }
   v4i wring[R][kNF];  // weight fragments of MFMA step s live in slot s % R
   v4i areg[ADMA ? 1 : kNA];
-  // ADMA: copy i of this wave fills rows 32 wave_id + 8 i + lane / 8 of a chunk buffer; the lane
+  // ADMA: copy i of this wave fills rows 8 (kNA wave_id + i) + lane / 8 of a chunk buffer; the lane
   // fetches vector (lane % 8) ^ (lane / 8 % 8) of its row, which lands at position lane % 8.
-  const int dma_row = wave_id * 32 + (lane >> 3);
+  const int dma_row = wave_id * 8 * kNA + (lane >> 3);
   const uint32_t dma_vec = static_cast<uint32_t>((lane & 7) ^ ((lane >> 3) & 7));
   const uint32_t lds_a_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)&lds_a[0][0]));
   // fragment reads: row li (+ 16 or 32 per fragment: same row % 8), vector v of the chunk at (v ^ li % 8)
@@ -341,7 +341,13 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     if constexpr (ADMA) {
       // two fragments in flight: the read of fragment n + 1 leaves before the MFMAs of fragment n
       v4i af[2];
-      af[0] = lds_read16_raw<buf * kStageBytes>(fa[M32 ? 2 * j : j]);
+      // (the instruction's offset field has 16 bits: with 32 KB buffers the buffer's offset goes into the address)
+      constexpr bool kFarStages = kStagesA * kStageBytes > 65536;
+      constexpr int kImm = kFarStages ? 0 : buf * kStageBytes;
+      uint32_t fa_s[2];
+      fa_s[0] = fa[M32 ? 2 * j : j] + (kFarStages ? buf * kStageBytes : 0);
+      fa_s[1] = M32 ? fa[2 * j + 1] + (kFarStages ? buf * kStageBytes : 0) : fa_s[0];
+      af[0] = lds_read16_raw<kImm>(fa_s[0]);
 #pragma unroll
       for (int n = 0; n < kFragReads; ++n) {
         const int mf = M32 ? n % AM : n, t = M32 ? n / AM : 0;
@@ -349,7 +355,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
           const int mf1 = M32 ? (n + 1) % AM : n + 1, t1 = M32 ? (n + 1) / AM : 0;
           asm volatile("ds_read_b128 %0, %1 offset:%2"
                        : "=v"(af[(n + 1) & 1])
-                       : "v"(fa[M32 ? 2 * j + t1 : j]), "i"(buf * kStageBytes + mf1 * kFragRows * kChunk)
+                       : "v"(fa_s[t1]), "i"(kImm + mf1 * kFragRows * kChunk)
                        : "memory");
           lds_wait<1>(af[n & 1]);
         } else {
@@ -465,7 +471,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     if constexpr (I8 && ADMA) {
       // the tile's absmax values travel the same way, 4 bytes per lane, straight into the slots
       // their scales will occupy (the loop top divides them by 127 in place)
-      if ((lane >> 4) < kNF) {  // lane = 16 f + c: channel c of fragment f of this wave
+      if (wave_m == 0 && (lane >> 4) < kNF) {  // lane = 16 f + c: channel c of fragment f of this wave
         bool ok;
         const int c = col_of(t, lane >> 4, ok);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(make_rsrc(w_max), (lds_ptr_t)&sw_lds[t_parity][wave * kNF * 16], 4,
@@ -543,7 +549,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         const float scaled = raw / 127.0f;
         asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(scaled) : "memory");
       };
-      if ((lane >> 4) < kNF) scale_in_place(&sw_lds[parity][wave * kNF * 16 + lane]);
+      if (wave_m == 0 && (lane >> 4) < kNF) scale_in_place(&sw_lds[parity][wave * kNF * 16 + lane]);
       if (threadIdx.x < kTM) scale_in_place(&sa_lds[parity][threadIdx.x]);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
@@ -796,8 +802,8 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
     return swiglu ? launch_tiled<K, true, 2, 8, 3, 1>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 2, 8, 3, 1>(p, a->rows, s, n_cu, what);
   // 256-row tiles bring DeepSeek-V3 prefill (128-256 rows per expert) down to its algorithmic HBM
-  // traffic (measured 1.01x against 1.5x), but with one workgroup per CU too few bytes are in
-  // flight: 3.4 TB/s against 5.6 TB/s, slower overall. Kept as a tuning variant.
+  // traffic (measured 1.04x against 1.44x), but one workgroup per CU has nothing to run under its
+  // epilogue and tile switch: 3.7 TB/s, 13 % slower overall. Kept as a tuning variant.
   if (a->variant == 8)
     return swiglu ? launch_tiled<K, true, 4, 4, 1, 2>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 1, 2>(p, a->rows, s, n_cu, what);

@@ -406,6 +406,10 @@ PERSISTENT_CASES = TILED_CASES + [
     (2, 96, 640, [140, 3]),
     (3, 64, 896, [1, 260, 17]),
     (64, 2048, 256, [((37 * i) % 290) for i in range(64)]),
+    # 9 and 11 chunks (one and three past the 4-chunk period of the activation ring); hundreds of
+    # experts (several passes of the 64-lane expert search), most of them empty
+    (40, 512, 1152, [((53 * i) % 400) for i in range(40)]),
+    (300, 256, 1408, [(129 if i % 7 == 0 else (i % 3)) for i in range(300)]),
 ]
 
 
@@ -418,6 +422,6 @@ def test_lds_gemm_i8_with_tiled_weights(L, E, n, k, counts, variant, act):
     with the deep weight ring, 8: 256-row tiles with 8 waves, 5: the default)."""
     if variant >= 5 and k % 128:
         pytest.skip("the persistent kernel takes k % 128 == 0")
-    if variant < 5 and E == 64:
+    if variant < 5 and E >= 40:
         pytest.skip("large case: persistent kernel only")
     _gemm_layout_case(L, E, n, k, counts, act, variant, True, chunked=False, seed=E * n + k + 7)

@@ -36,10 +36,12 @@ WORKLOAD_LABEL = {
     "kimi-fp8-prefill": "Kimi-K2-shape MoE layer (384 experts, +1 shared), fp8-e4m3 128x128-block weights, prefill, 4096 tokens",
     "qwen3-bf16-decode": "Qwen3-MoE-30B-A3B-shape MoE layer, bf16 weights (no quantization), decode, 64 tokens",
     "qwen3-bf16-prefill": "Qwen3-MoE-30B-A3B-shape MoE layer, bf16 weights (no quantization), prefill, 8192 tokens",
+    "qwen3-w4a16-decode": "Qwen3-MoE-30B-A3B-shape MoE layer, 4-bit weights (groups of 128) and bf16 activations, "
+                          "decode, 64 tokens",
     "tiny-bf16": "tiny bf16 MoE layer (32 tokens, hidden 512, 8 experts, top-2, intermediate 256), no quantization",
 }
-PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0, "none": 2500.0}  # MI355X dense MFMA: int8, fp8, bf16
-DTYPE = {"int8": "int8", "fp8": "fp8_e4m3", "none": "bf16"}
+PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0, "none": 2500.0, "w4": 2500.0}  # MI355X dense MFMA: int8, fp8, bf16
+DTYPE = {"int8": "int8", "fp8": "fp8_e4m3", "none": "bf16", "w4": "bf16 (4-bit weights)"}
 
 
 class HipEvents:
@@ -74,13 +76,15 @@ def algorithmic_work(shape, n_active):
     """Bytes that must cross HBM and int8 operations that must run, per layer call
     and for each GEMM launch, from the shape and the number of experts hit."""
     M, H, E, K, I, Is, P = shape.M, shape.H, shape.E, shape.K, shape.I, shape.I_shared, shape.P
-    wb = 2 if shape.quant == "none" else 1  # bytes per weight / activation code
+    wb = {"none": 2, "w4": 0.5}.get(shape.quant, 1)  # bytes per weight
+    ab = 2 if shape.quant in ("none", "w4") else 1    # bytes per activation value / code
 
     def w_bytes(n, k):  # one [n,k] weight matrix with its scales
-        return n * k * wb + {"int8": n * 4, "fp8": (n // 128) * (k // 128) * 4, "none": 0}[shape.quant]
+        return int(n * k * wb) + {"int8": n * 4, "fp8": (n // 128) * (k // 128) * 4, "none": 0,
+                                  "w4": n * (k // shape.group_size) * 2}[shape.quant]
 
-    def a_bytes(rows, k):  # quantised activations of `rows` rows with their scales
-        return rows * k * wb + {"int8": rows * 4, "fp8": rows * (k // 128) * 4, "none": 0}[shape.quant]
+    def a_bytes(rows, k):  # (quantised) activations of `rows` rows with their scales
+        return rows * k * ab + {"int8": rows * 4, "fp8": rows * (k // 128) * 4, "none": 0, "w4": 0}[shape.quant]
 
     g1_bytes = n_active * w_bytes(2 * I, H) + a_bytes(M, H) + P * 4 + P * I * 2
     g2_bytes = n_active * w_bytes(H, I) + a_bytes(P, I) + P * H * 2
@@ -126,7 +130,7 @@ def cpu_baseline(sl, budget_s=10.0):
         fn, what = tm.bf16_moe, "torch-CPU restatement of the reference expert loop"
         args = (host(sl.x), host(sl.logits), w13, w2, s.K, True)
     else:
-        return None  # no CPU restatement of the fp8 layer is timed (the reference has no fp8 MoE path)
+        return None  # no CPU restatement of the fp8 / 4-bit layers is timed
     t0 = time.perf_counter()
     fn(*args)  # warm-up
     first = time.perf_counter() - t0
@@ -173,7 +177,9 @@ def main():
     lay = sl.layer
     x, logits = sl.x.contiguous(), sl.logits.contiguous()
     out = torch.empty_like(x)
-    fmt = {"int8": L.KMOE_FMT_INT8, "fp8": L.KMOE_FMT_FP8_BLOCK, "none": L.KMOE_FMT_BF16}[shape.quant]
+    fmt = {"int8": L.KMOE_FMT_INT8, "fp8": L.KMOE_FMT_FP8_BLOCK, "none": L.KMOE_FMT_BF16,
+           "w4": L.KMOE_FMT_W4A16}[shape.quant]
+    w4 = shape.quant == "w4"
 
     w_gate = None
     if a.router:
@@ -183,10 +189,13 @@ def main():
 
     def make_plan(stage_events=None):
         # the argument block the plugin methods build (apply_monolithic / KunlunOps.fused_moe)
-        return make_moe_plan(fmt, x, None if a.router else logits, out, shape.K, lay.w13_weight, lay.w2_weight,
+        return make_moe_plan(fmt, x, None if a.router else logits, out, shape.K,
+                             lay.w13_weight_packed if w4 else lay.w13_weight,
+                             lay.w2_weight_packed if w4 else lay.w2_weight,
                              getattr(lay, "w13_weight_scale", None), getattr(lay, "w2_weight_scale", None),
                              shape.scoring, True, shape.n_group, shape.topk_group, shape.routed_scale, sl.bias,
-                             sl.shared, 1.0, stage_events, router_weight=w_gate)
+                             sl.shared, 1.0, stage_events, router_weight=w_gate,
+                             group_size=shape.group_size if w4 else None)
 
     plan = make_plan()
 
@@ -249,7 +258,7 @@ def main():
         roofline = {"bound": "mfma", "achieved": achieved, "peak": peak_tops, "unit": "TFLOP/s",
                     "frac": achieved / peak_tops, "traffic": measured_traffic(a.workload)}
     many_rows = shape.P > 48 * shape.E  # the launchers' switch to the persistent 128-row-tile kernel
-    g1_kernel = ("stream_gemm_i8_kernel" if plan.layout.codes_chunked else
+    g1_kernel = ("w4_stream_kernel" if w4 else "stream_gemm_i8_kernel" if plan.layout.codes_chunked else
                  "tiled_gemm_kernel" if many_rows and plan.args.w_layout == L.KMOE_W_TILED else "grouped_gemm_kernel")
     roofline.update(kernel=g1_kernel + " (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
                     algorithmic_bytes=work["g1_bytes"], algorithmic_ops=work["g1_ops"])

@@ -277,6 +277,39 @@ typedef struct kmoe_gemm_fp8_args {
  */
 int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* args, kmoe_stream_t stream);
 
+typedef struct kmoe_gemm_w4_args {
+  const uint16_t* a;      /* [a_rows, k] bf16 activations, row stride lda (elements)  */
+  int64_t lda;
+  const int32_t* row_src; /* as in kmoe_gemm_i8_args                                  */
+  int32_t src_div;
+  const uint8_t* w;       /* [E, n, k/2] packed 4-bit codes: two per byte, low nibble first,
+                             code c means c - 8; the bytes re-arranged by
+                             kmoe_tile_weights_i8(E, n, k/2) (w_layout = KMOE_W_TILED)  */
+  const uint16_t* w_scale;/* [E, n, k/group_size] bf16                                */
+  int32_t group_size;     /* values per scale along k: a multiple of 32 that divides k
+                             (k itself: one scale per output channel)                 */
+  const int32_t* lod;     /* [E+1]                                                    */
+  int32_t E, n, k, rows;
+  uint16_t* y;            /* bf16 [rows, n] or [rows, n/2] with SwiGLU                */
+  int64_t ldy;
+  int32_t act;            /* KMOE_ACT_NONE or KMOE_ACT_SWIGLU                         */
+  int32_t variant;        /* 0 = from the shape; 1, 2, 4 = 16-row fragments per pass  */
+  int32_t w_layout;       /* KMOE_W_TILED                                             */
+} kmoe_gemm_w4_args;
+
+/*
+ * 4-bit weight-only grouped GEMM (W4A16). The reference unpacks the packed tensors to
+ * fp16 inside every call (dequant_int4_native, quantization/kernels/quant_ops.py:71-86,
+ * called compressed_tensors_moe.py:320-327) and then runs the unquantized moe_fc; this
+ * entry point reads the packed weights once and unpacks them in registers:
+ *   y[r,c] = bf16( sum_k float(a[src(r),k]) * float(bf16((code[e,c,k] - 8) * scale[e,c,k/group])) )
+ * i.e. the bf16 grouped GEMM on the weights kmoe_dequant_w4_bf16 would produce, with
+ * f32 accumulation on MFMA (compare within tolerance). Made for the decode regime
+ * (an expert with more rows than one pass holds streams its weights again).
+ * Limits: k % 128 == 0, n % 16 == 0 (SwiGLU: n % 32 == 0), tiled weights.
+ */
+int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* args, kmoe_stream_t stream);
+
 /*
  * The gpt-oss activation on a stored, interleaved gate_up result. Replaces
  * torch.ops._C.swigluoai_and_mul (ops/_custom_ops.py:728-742).
@@ -347,6 +380,8 @@ int kmoe_router_gemm_bf16(const uint16_t* x, int64_t ld_x, const uint16_t* w_gat
 #define KMOE_FMT_INT8 0      /* int8 weights + per-channel max, per-token int8 activations   */
 #define KMOE_FMT_FP8_BLOCK 1 /* e4m3fn weights + 128x128 block scales, 1x128 activation scales */
 #define KMOE_FMT_BF16 2      /* bf16 weights, no quantisation                                 */
+#define KMOE_FMT_W4A16 3     /* packed 4-bit weights + bf16 group scales, bf16 activations
+                                (kmoe_grouped_gemm_w4a16); no shared expert, no bias     */
 
 typedef struct kmoe_moe_args {
   /* shape */
@@ -391,6 +426,10 @@ typedef struct kmoe_moe_args {
   float act_alpha, act_limit;
   int32_t ws_layout;     /* layout of ws13, ws2 (KMOE_W_*): a shared expert whose sizes do not allow
                             tiling (k % 64) stays row-major next to tiled routed experts  */
+  /* W4A16 only: w13 / w2 hold the packed codes ([E,2I,H/2], [E,H,I/2] bytes, tiled) */
+  const uint16_t* w13_scale; /* [E,2I,H/group_size] bf16                               */
+  const uint16_t* w2_scale;  /* [E,H,I/group_size] bf16                                */
+  int32_t group_size;    /* a multiple of 32 dividing H and I (one value for both tensors) */
 } kmoe_moe_args;
 
 #define KMOE_STAGE_ROUTING 0

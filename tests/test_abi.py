@@ -40,7 +40,8 @@ def test_struct_layouts_match_the_header(L):
     assert C.sizeof(L.MoELayout) == 22 * 8
     assert C.sizeof(L.GemmBf16Args) == 6 * 8 + 16 + 16 + 16 + 16  # ..., act+variant+w_layout+pad, bias, alpha+limit  # 6 ptr/int64 (src_div padded), 4 int32, y/ldy, act+variant+w_layout+pad
     assert C.sizeof(L.GemmFp8Args) == 8 * 8 + 16 + 16 + 16  # 8 ptr/int64, 4 int32, y/ldy, act+variant+w_layout+pad
-    assert L.MoEArgs.w_gate.offset == C.sizeof(L.MoEArgs) - 8 - 32  # then w13_bias, w2_bias, activation, alpha, limit, ws_layout
+    assert L.MoEArgs.w_gate.offset == C.sizeof(L.MoEArgs) - 8 - 32 - 24  # then w13_bias, w2_bias, activation, alpha, limit, ws_layout; w13_scale, w2_scale, group_size + pad
+    assert C.sizeof(L.GemmW4Args) == 3 * 8 + 8 + 2 * 8 + 8 + 8 + 16 + 16 + 16  # a/lda/row_src, src_div+pad, w/w_scale, group_size+pad, lod, 4 int32, y/ldy, act+variant+w_layout+pad
     a = L.MoEArgs()
     assert L.MoEArgs.M.offset == 0 and L.MoEArgs.logits.offset == 48 and C.sizeof(a) % 8 == 0
 

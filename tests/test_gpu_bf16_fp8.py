@@ -365,3 +365,117 @@ def test_w4a16_method_unpacks_once_and_runs_the_bf16_path(group_size):
     torch.cuda.synchronize()
     ref = co.forward_bf16(bits(x), logits.cpu().numpy(), bits(w13), bits(w2), K)
     assert rel_l2(out, from_bits(ref)) <= REL_L2_BF16
+
+
+W4_CASES = [
+    # E, n, k, rows per expert, group size (None: one scale per row)
+    (1, 64, 128, [16], 128),
+    (4, 64, 256, [3, 0, 17, 1], 32),
+    (3, 96, 384, [5, 40, 7], 128),
+    (8, 256, 1024, [4, 4, 0, 9, 33, 1, 0, 2], 64),
+    (2, 128, 512, [70, 3], None),
+    (16, 1536, 256, [(5 * i) % 11 for i in range(16)], 128),
+]
+
+
+@pytest.mark.parametrize("E,n,k,counts,gs", W4_CASES)
+@pytest.mark.parametrize("variant", [0, 1, 2, 4])
+@pytest.mark.parametrize("act", [0, 1])
+@pytest.mark.parametrize("gather", [False, True])
+def test_grouped_gemm_w4a16(L, E, n, k, counts, gs, variant, act, gather):
+    """Packed 4-bit weights streamed and unpacked in registers against the oracle's route: unpack
+    (orc_dequant_w4_bf16, itself pinned by a brute-force check) then the bf16 grouped GEMM."""
+    g = torch.Generator().manual_seed(E * n + k + (gs or 0))
+    lod = _lod(counts)
+    rows = int(lod[-1])
+    group = gs or k
+    packed = torch.randint(0, 256, (E, n, k // 2), generator=g, dtype=torch.uint8)
+    scale = (torch.rand(E, n, k // group, generator=g) * 0.02 + 0.002).bfloat16()
+    K = 2
+    src_rows = (rows + K - 1) // K if gather else rows
+    a = torch.randn(max(src_rows, 1), k, generator=g).bfloat16()
+    row_src = torch.randperm(src_rows * K, generator=g)[:rows].int() if gather else None
+    w_bits = co.dequant_w4_bf16(packed.numpy(), bits(scale), group)
+    ref = co.grouped_gemm_bf16(bits(a), w_bits, lod, act=act, row_src=None if row_src is None else row_src.numpy(),
+                               src_div=K if gather else 1)
+    n_out = n // 2 if act else n
+    dp = packed.cuda()
+    dt = torch.empty_like(dp)
+    L.check(L.lib.kmoe_tile_weights_i8(dp.data_ptr(), dt.data_ptr(), E, n, k // 2, L.stream()))
+    da, ds, dl = a.cuda(), scale.cuda(), torch.from_numpy(lod).cuda()
+    dsrc = None if row_src is None else row_src.cuda()
+    y = torch.zeros(rows, n_out, dtype=torch.bfloat16, device="cuda")
+    args = L.GemmW4Args()
+    args.a, args.lda, args.src_div = da.data_ptr(), k, K if gather else 1
+    args.row_src = 0 if dsrc is None else dsrc.data_ptr()
+    args.w, args.w_scale, args.group_size, args.lod = dt.data_ptr(), ds.data_ptr(), group, dl.data_ptr()
+    args.E, args.n, args.k, args.rows = E, n, k, rows
+    args.y, args.ldy, args.act, args.variant, args.w_layout = y.data_ptr(), n_out, act, variant, L.KMOE_W_TILED
+    L.check(L.lib.kmoe_grouped_gemm_w4a16(args, L.stream()))
+    torch.cuda.synchronize()
+    assert rel_l2(y, from_bits(ref)) <= 2e-3   # the operands are the same bits: only summation order differs
+    # an independent torch statement of the unpacking and of one expert's product
+    e = int(np.argmax(counts))
+    r0, r1 = int(lod[e]), int(lod[e + 1])
+    codes = torch.stack([packed[e] & 15, packed[e] >> 4], dim=-1).reshape(n, k).float() - 8.0
+    w_e = (codes * scale[e].float().repeat_interleave(group, dim=1)).bfloat16().float()
+    rows_e = a[(row_src[r0:r1] // K).long()] if gather else a[r0:r1]
+    t = rows_e.float() @ w_e.T
+    if act:
+        t = tm.silu_and_mul(t.bfloat16()).float()
+    assert rel_l2(y[r0:r1], t) <= REL_L2_BF16
+
+
+def test_grouped_gemm_w4a16_rejects_what_it_cannot_run(L):
+    args = L.GemmW4Args()
+    t = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    args.a = args.w = args.w_scale = args.lod = args.y = t.data_ptr()
+    args.lda, args.ldy, args.src_div = 128, 64, 1
+    args.E, args.n, args.k, args.rows, args.group_size = 1, 64, 128, 1, 128
+    args.w_layout = L.KMOE_W_ROWMAJOR
+    with pytest.raises(NotImplementedError):
+        L.check(L.lib.kmoe_grouped_gemm_w4a16(args, L.stream()))
+    args.w_layout, args.group_size = L.KMOE_W_TILED, 48
+    with pytest.raises(ValueError):
+        L.check(L.lib.kmoe_grouped_gemm_w4a16(args, L.stream()))
+    args.group_size, args.k = 128, 192
+    with pytest.raises(ValueError):
+        L.check(L.lib.kmoe_grouped_gemm_w4a16(args, L.stream()))
+
+
+@pytest.mark.parametrize("native", ["auto", "only"])
+@pytest.mark.parametrize("group_size,M", [(128, 24), (32, 5), (None, 24), (128, 700)])
+def test_w4a16_layer_on_the_packed_weights(native, group_size, M):
+    """The 4-bit method with shapes the packed-weight kernel takes: decode-sized batches run
+    kmoe_moe_forward with KMOE_FMT_W4A16, large ones the unpacked copy ("auto") or the packed
+    weights again ("only"); both against the C oracle on the unpacked weights."""
+    from vllm_kunlun_amd.ops.fused_moe.layer import FusedMoE
+    from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors_moe import (
+        KunlunCompressedTensorsWNA16MoEMethod)
+    from types import SimpleNamespace
+    E, H, I, K = 16, 256, 256, 4  # H == I: one scale per row is then one group size for both tensors
+    wq = SimpleNamespace(num_bits=4, type="int", symmetric=True, dynamic=False,
+                         strategy="group" if group_size else "channel", group_size=group_size)
+    method = KunlunCompressedTensorsWNA16MoEMethod(wq, None, SimpleNamespace(experts_per_token=K), native=native)
+    layer = FusedMoE(num_experts=E, top_k=K, hidden_size=H, intermediate_size=I, quant_method=method, device="cuda")
+    g = torch.Generator().manual_seed(11)
+    with torch.no_grad():
+        for name, (n, k) in (("w13", (2 * I, H)), ("w2", (H, I))):
+            getattr(layer, f"{name}_weight_packed").data = torch.randint(0, 256, (E, n, k // 2), generator=g,
+                                                                         dtype=torch.uint8).cuda()
+            getattr(layer, f"{name}_weight_scale").data = (torch.rand(E, n, k // (group_size or k), generator=g)
+                                                           * 0.02 + 0.002).bfloat16().cuda()
+    packed13, scale13 = layer.w13_weight_packed.data.cpu(), layer.w13_weight_scale.data.cpu()
+    packed2, scale2 = layer.w2_weight_packed.data.cpu(), layer.w2_weight_scale.data.cpu()
+    method.process_weights_after_loading(layer)
+    assert layer.w4_native and hasattr(layer, "w13_weight_packed")
+    assert hasattr(layer, "w13_weight") == (native == "auto")
+    gx = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(M, H, generator=gx, device="cuda").bfloat16()
+    logits = torch.randn(M, E, generator=gx, device="cuda")
+    out = layer(x, logits)
+    torch.cuda.synchronize()
+    w13 = co.dequant_w4_bf16(packed13.numpy(), bits(scale13), group_size or H)
+    w2 = co.dequant_w4_bf16(packed2.numpy(), bits(scale2), group_size or I)
+    ref = co.forward_bf16(bits(x), logits.cpu().numpy(), w13, w2, K)
+    assert rel_l2(out, from_bits(ref)) <= REL_L2_BF16

@@ -32,13 +32,25 @@ extern "C" const char* kmoe_version(void) { return "kmoe 0.2 gfx950"; }
 
 namespace {
 
+// formats whose GEMMs read the bf16 activations themselves (no activation quantisation)
+bool bf16_activations(int format) { return format == KMOE_FMT_BF16 || format == KMOE_FMT_W4A16; }
+
 int check_shape(const kmoe_moe_args* a) {
   KMOE_REQUIRE(a, KMOE_ERR_NULL, "moe_forward: args is NULL");
   KMOE_REQUIRE(a->M >= 0 && a->H >= 16 && a->E >= 1 && a->K >= 1 && a->I >= 16, KMOE_ERR_SHAPE,
                "moe_forward: M=%d H=%d E=%d K=%d I=%d", a->M, a->H, a->E, a->K, a->I);
-  KMOE_REQUIRE(a->format == KMOE_FMT_INT8 || a->format == KMOE_FMT_FP8_BLOCK || a->format == KMOE_FMT_BF16,
+  KMOE_REQUIRE(a->format == KMOE_FMT_INT8 || a->format == KMOE_FMT_FP8_BLOCK || a->format == KMOE_FMT_BF16 ||
+                   a->format == KMOE_FMT_W4A16,
                KMOE_ERR_UNSUPPORTED, "moe_forward: format=%d unknown", a->format);
-  const int mult = a->format == KMOE_FMT_FP8_BLOCK ? 128 : 16;
+  if (a->format == KMOE_FMT_W4A16) {
+    KMOE_REQUIRE(a->I_shared == 0, KMOE_ERR_UNSUPPORTED, "moe_forward: no shared expert with 4-bit weights");
+    KMOE_REQUIRE(a->w_layout == KMOE_W_TILED, KMOE_ERR_UNSUPPORTED, "moe_forward: 4-bit weights must be tiled");
+    KMOE_REQUIRE(a->group_size >= 32 && a->group_size % 32 == 0 && a->H % a->group_size == 0 &&
+                     a->I % a->group_size == 0,
+                 KMOE_ERR_SHAPE, "moe_forward: group_size=%d must be a multiple of 32 dividing H=%d and I=%d",
+                 a->group_size, a->H, a->I);
+  }
+  const int mult = a->format == KMOE_FMT_FP8_BLOCK || a->format == KMOE_FMT_W4A16 ? 128 : 16;
   KMOE_REQUIRE(a->H % mult == 0 && a->I % mult == 0, KMOE_ERR_SHAPE,
                "moe_forward: H=%d and I=%d must be multiples of %d", a->H, a->I, mult);
   KMOE_REQUIRE(a->K <= a->E && a->K <= 64 && a->E <= 1024, KMOE_ERR_SHAPE, "moe_forward: K=%d E=%d out of range", a->K,
@@ -46,7 +58,8 @@ int check_shape(const kmoe_moe_args* a) {
   KMOE_REQUIRE(a->I_shared >= 0 && a->I_shared % mult == 0, KMOE_ERR_SHAPE,
                "moe_forward: I_shared=%d must be a non-negative multiple of %d", a->I_shared, mult);
   KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "moe_forward: M*K too large");
-  const int row64 = a->format == KMOE_FMT_BF16 ? 32 : 64;  // elements in 64 bytes of a weight row
+  // elements in 64 bytes of a weight row
+  const int row64 = a->format == KMOE_FMT_BF16 ? 32 : (a->format == KMOE_FMT_W4A16 ? 128 : 64);
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR ||
                    (a->w_layout == KMOE_W_TILED && a->H % row64 == 0 && a->I % row64 == 0),
                KMOE_ERR_SHAPE, "moe_forward: w_layout=%d needs H, I multiples of %d", a->w_layout, row64);
@@ -100,12 +113,15 @@ struct MlpPass {
   const uint16_t *w13_bias, *w2_bias;
   int oai;  // 1: gate_up rows interleaved, gpt-oss activation
   float act_alpha, act_limit;
+  // W4A16: group scales of the packed weights
+  const uint16_t *w13_scale, *w2_scale;
+  int group_size;
 };
 
 int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
   const int n = first ? 2 * m.I : m.H;
   const int k = first ? m.H : m.I;
-  const void* a = first ? m.x_rows : (m.format == KMOE_FMT_BF16 ? static_cast<const void*>(m.act) : m.actq);
+  const void* a = first ? m.x_rows : (bf16_activations(m.format) ? static_cast<const void*>(m.act) : m.actq);
   const float* a_aux = first ? m.x_aux : m.act_aux;
   const void* w = first ? m.w13 : m.w2;
   const float* w_aux = first ? m.w13_aux : m.w2_aux;
@@ -165,6 +181,26 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.w_layout = m.w_layout;
     return kmoe_grouped_gemm_fp8_block(&g, stream);
   }
+  if (m.format == KMOE_FMT_W4A16) {
+    kmoe_gemm_w4_args g = {};
+    g.a = static_cast<const uint16_t*>(a);
+    g.lda = k;
+    g.row_src = row_src;
+    g.src_div = src_div;
+    g.w = static_cast<const uint8_t*>(w);
+    g.w_scale = first ? m.w13_scale : m.w2_scale;
+    g.group_size = m.group_size;
+    g.lod = m.lod;
+    g.E = m.E;
+    g.n = n;
+    g.k = k;
+    g.rows = m.rows;
+    g.y = y;
+    g.ldy = ldy;
+    g.act = act;
+    g.w_layout = m.w_layout;
+    return kmoe_grouped_gemm_w4a16(&g, stream);
+  }
   kmoe_gemm_bf16_args g = {};
   g.a = static_cast<const uint16_t*>(a);
   g.lda = k;
@@ -216,7 +252,7 @@ extern "C" int kmoe_moe_workspace_layout(const kmoe_moe_args* a, kmoe_moe_layout
   if (int rc = check_shape(a)) return rc;
   KMOE_REQUIRE(L, KMOE_ERR_NULL, "moe_workspace_layout: layout is NULL");
   const size_t M = a->M, H = a->H, E = a->E, K = a->K, I = a->I, P = M * K, Is = a->I_shared;
-  const bool quant = a->format != KMOE_FMT_BF16;
+  const bool quant = !bf16_activations(a->format);
   const bool fp8 = a->format == KMOE_FMT_FP8_BLOCK;
   const bool fold = fold_shared(a);
   const size_t R = P + (fold ? M : 0);  // rows of the routed intermediates (+ folded shared expert rows)
@@ -259,13 +295,15 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   kmoe_moe_layout L;
   if (int rc = kmoe_moe_workspace_layout(a, &L)) return rc;
   if (a->M == 0) return KMOE_OK;
-  const bool quant = a->format != KMOE_FMT_BF16;
+  const bool quant = !bf16_activations(a->format);
   KMOE_REQUIRE((a->logits || a->w_gate) && a->x && a->w13 && a->w2 && a->out, KMOE_ERR_NULL,
                "moe_forward: NULL tensor pointer");
   KMOE_REQUIRE(a->logits || (a->H % 32 == 0 && (reinterpret_cast<uintptr_t>(a->w_gate) & 15) == 0 &&
                              (reinterpret_cast<uintptr_t>(a->x) & 15) == 0),
                KMOE_ERR_SHAPE, "moe_forward: the router GEMM needs H %% 32 == 0 and 16-byte aligned x, w_gate");
   KMOE_REQUIRE(!quant || (a->w13_max && a->w2_max), KMOE_ERR_NULL, "moe_forward: weight max/scale pointers are NULL");
+  KMOE_REQUIRE(a->format != KMOE_FMT_W4A16 || (a->w13_scale && a->w2_scale), KMOE_ERR_NULL,
+               "moe_forward: group scale pointers are NULL");
   KMOE_REQUIRE(a->I_shared == 0 || (a->ws13 && a->ws2 && (!quant || (a->ws13_max && a->ws2_max))), KMOE_ERR_NULL,
                "moe_forward: shared expert pointers are NULL");
   KMOE_REQUIRE(a->scoring == KMOE_SCORE_SOFTMAX || a->scoring == KMOE_SCORE_SIGMOID, KMOE_ERR_UNSUPPORTED,
@@ -384,6 +422,9 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   routed.act_aux = static_cast<float*>(at(L.actmax));
   routed.out = static_cast<uint16_t*>(at(L.down));
   routed.w_layout = a->w_layout;
+  routed.w13_scale = a->w13_scale;
+  routed.w2_scale = a->w2_scale;
+  routed.group_size = a->group_size;
   if (a->format == KMOE_FMT_BF16) {
     routed.w13_bias = a->w13_bias;
     routed.w2_bias = a->w2_bias;

@@ -363,14 +363,6 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         }
         mfma_row(wcur, af[n & 1], mf, t);
       }
-    } else {
-#pragma unroll
-      for (int n = 0; n < kFragReads; ++n) {
-        const int mf = M32 ? n % AM : n, t = M32 ? n / AM : 0;
-        const v4i af = *reinterpret_cast<const v4i*>(
-            &lds_a[buf][(wave_m * 16 * kMF + mf * kFragRows + li) * kPitchT + j * 64 + (M32 ? t * 32 : 0) + lg * 16]);
-        mfma_row(wcur, af, mf, t);
-      }
     }
   };
   // F8, one whole chunk: the two ring slots of the chunk are the K halves of one MFMA
@@ -436,7 +428,6 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   // gather index of the tile row whose scale this thread fetches (I8: row threadIdx.x; F8: threadIdx.x % kTM)
   const int scale_row = F8 ? threadIdx.x % kTM : min(static_cast<int>(threadIdx.x), kTM - 1);
   int rs_scale = fetch_src(cur, cur.row0 + scale_row);
-  float sw_reg = 0.0f, sa_reg = 0.0f;  // this thread's share of the tile's scales, on their way to LDS
   float wsc_reg[kMaxKBlocks / 16];     // F8: weight block scales k = c, c + 16, ... of fragment lane / 16
 
   // Points the loaders at tile t and requests its first chunk, first three weight steps and scales.
@@ -468,7 +459,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     dma_a(0, 0);
     dma_a(1, 1);
     dma_a(2, 2);
-    if constexpr (I8 && ADMA) {
+    if constexpr (I8) {
       // the tile's absmax values travel the same way, 4 bytes per lane, straight into the slots
       // their scales will occupy (the loop top divides them by 127 in place)
       if (wave_m == 0 && (lane >> 4) < kNF) {  // lane = 16 f + c: channel c of fragment f of this wave
@@ -496,14 +487,6 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
           wsc_reg[i] = kb < kblocks ? ws[kb] : 0.0f;
         }
       }
-    } else if constexpr (I8 && !ADMA) {
-      if (wave_m == 0 && (lane >> 4) < kNF) {  // thread (wave, f = lane / 16, c = lane % 16): scale of channel c of fragment f of this wave
-        bool ok;
-        const int c = col_of(t, lane >> 4, ok);
-        sw_reg = ok ? w_max[c + (lane & 15)] : 0.0f;
-      }
-      if (threadIdx.x < kTM)  // thread r: scale of tile row r
-        sa_reg = p.a_max[src_row(t, rs_scale)];
     }
   };
   start_tile(cur, 0);
@@ -526,9 +509,6 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         for (int i = 0; i < kMaxKBlocks / 16; ++i)
           wsc_lds[parity][(wave * kNF + (lane >> 4)) * kMaxKBlocks + (lane & 15) + 16 * i] = wsc_reg[i];
       }
-    } else if constexpr (I8 && !ADMA) {
-      if (wave_m == 0 && (lane >> 4) < kNF) sw_lds[parity][wave * kNF * 16 + lane] = sw_reg / 127.0f;
-      if (threadIdx.x < kTM) sa_lds[parity][threadIdx.x] = sa_reg / 127.0f;
     }
     store_a(0);
     // ADMA: the copies of chunks 0-2 have landed - after them start_tile issued its (R - 1) kNF
@@ -539,7 +519,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
       if (p.row_src) vmem_wait<(R - 1) * kNF + kNA + 1>();
       else vmem_wait<(R - 1) * kNF>();
     }
-    if constexpr (I8 && ADMA) {
+    if constexpr (I8) {
       // absmax -> scale in place, each slot by the thread that requested it (LDS instructions
       // the compiler does not see: no wait for the gather-index loads just issued)
       auto scale_in_place = [&](const float* slot) {

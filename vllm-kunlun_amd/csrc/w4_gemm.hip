@@ -1,0 +1,241 @@
+// Weight-streaming grouped GEMM on 4-bit weights and bf16 activations (W4A16) for the decode
+// regime: the packed weights are read from HBM once, unpacked in registers and fed to
+// v_mfma_f32_16x16x32_bf16. A quarter of the bytes of the bf16 path; the unpacking (23 VALU
+// instructions per 8 weights) is what bounds the kernel once the bytes are that few.
+//
+//   weights  [E][n][k/2] bytes, two codes per byte, low nibble first, code c means c - 8
+//            (dequant_int4_native, quantization/kernels/quant_ops.py:71-86), re-arranged by
+//            kmoe_tile_weights_i8(E, n, k/2): 1 KB blocks of 16 channels x 128 values. Lane
+//            16 g + c of a wave reads 16 consecutive bytes of a block: the 32 values
+//            k = 128 kb + 32 g + [0, 32) of channel c. Its t-th 4-byte word (8 values) is its
+//            operand of the t-th MFMA of the block; the activation lane (g, row) supplies the
+//            same 8 values of its row. So one MFMA step covers k = 32 g + 8 t + [0, 8) for
+//            g = 0..3 - not a contiguous range, which the sum does not care about.
+//   scales   [E][n][k/group] bf16; a group is a multiple of 32 values, so a lane needs ONE
+//            scale per block: group (128 kb + 32 g) / group_size of its channel.
+//   value    bf16(float(c - 8) * scale), computed as fma(128 + c, scale, -136 scale): both
+//            products and their sum are exact in f32 (8-bit x 8-bit mantissas), so the one
+//            rounding is the bf16 one - the same bits as unpacking first (kmoe_dequant_w4_bf16).
+#include "kmoe_common.h"
+
+namespace kmoe {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+struct W4Params {
+  const uint16_t* a;  // [a_rows, k] bf16
+  int64_t lda;
+  const int32_t* row_src;
+  int32_t src_div;
+  const uint8_t* w;       // tiled packed codes
+  const uint16_t* scale;  // [E, n, k / gs] bf16
+  int32_t gs;
+  const int32_t* lod;
+  int32_t E, n, k;
+  uint16_t* y;
+  int64_t ldy;
+};
+
+constexpr int kWaves = 4;
+
+// 128 + (byte J of v) as a float, in one full-rate instruction: v_perm_b32 puts the byte into
+// mantissa bits 16-23 of 0x43000000 = 128.0f (whose unit in the last place is 2^-16, so
+// bit 16 counts ones). The integer-to-float conversions run at a fraction of that rate.
+template <int J>
+__device__ inline float byte_plus_128(uint32_t v) {
+  // selector bytes, most significant first: byte 3 of the first source, byte J of the second, zero, zero
+  return __builtin_bit_cast(float, __builtin_amdgcn_perm(0x43000000u, v, 0x07000c0cu | (static_cast<uint32_t>(J) << 16)));
+}
+
+// 8 codes of one 4-byte word -> 8 bf16 values, value 2 j in the low half of register j:
+// 3 instructions split the nibbles into bytes, then per value 1 v_perm and 1 fma
+// ((128 + c) s - 136 s: both products have at most 16 significant bits and their sum is
+// (c - 8) s, so nothing rounds before the bf16 rounding), and 1 rounding per pair
+__device__ inline v4i unpack8(uint32_t word, float s, float m136s) {
+  const uint32_t lo = word & 0x0f0f0f0fu;         // codes 0, 2, 4, 6 in bytes 0..3
+  const uint32_t hi = (word >> 4) & 0x0f0f0f0fu;  // codes 1, 3, 5, 7
+  v4i out;
+  out[0] = static_cast<int>(pack2_bf16(__builtin_fmaf(byte_plus_128<0>(lo), s, m136s), __builtin_fmaf(byte_plus_128<0>(hi), s, m136s)));
+  out[1] = static_cast<int>(pack2_bf16(__builtin_fmaf(byte_plus_128<1>(lo), s, m136s), __builtin_fmaf(byte_plus_128<1>(hi), s, m136s)));
+  out[2] = static_cast<int>(pack2_bf16(__builtin_fmaf(byte_plus_128<2>(lo), s, m136s), __builtin_fmaf(byte_plus_128<2>(hi), s, m136s)));
+  out[3] = static_cast<int>(pack2_bf16(__builtin_fmaf(byte_plus_128<3>(lo), s, m136s), __builtin_fmaf(byte_plus_128<3>(hi), s, m136s)));
+  return out;
+}
+
+// MF: 16-row fragments per pass over the weights; NF: 16-channel fragments per wave;
+// D: 128-value blocks of loads in flight per wave.
+template <int MF, int NF, bool SWIGLU, int D>
+__global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params p) {
+  constexpr int NFH = SWIGLU ? NF / 2 : NF;
+  constexpr int TM = 16 * MF;
+  const int lane = lane_id();
+  const int wave = threadIdx.x >> 6;
+  const int li = lane & 15;
+  const int lg = lane >> 4;
+  const int e = blockIdx.y;
+  const int row_begin = p.lod[e], row_end = p.lod[e + 1];
+  if (row_begin >= row_end) return;
+  const int n_half = SWIGLU ? p.n / 2 : p.n;
+  const int col_base = (blockIdx.x * kWaves + wave) * NFH * 16;
+  if (col_base >= n_half) return;
+  const int kblocks = p.k / 128;
+  const int groups = p.k / p.gs;
+  const uint8_t* w_base = p.w + static_cast<size_t>(e) * p.n * (p.k / 2);
+  const uint16_t* s_base = p.scale + static_cast<size_t>(e) * p.n * groups;
+
+  const uint8_t* wp[NF];
+  const uint16_t* sp[NF];
+  bool wok[NF];
+  int col[NF];
+#pragma unroll
+  for (int f = 0; f < NF; ++f) {
+    const int fh = SWIGLU ? f % NFH : f;
+    const int c = col_base + fh * 16;
+    wok[f] = c < n_half;
+    col[f] = (SWIGLU && f >= NFH) ? n_half + c : c;
+    const int ch0 = wok[f] ? col[f] : 0;  // fragments past the last channel read fragment 0: never stored
+    wp[f] = w_base + static_cast<size_t>(ch0 / 16) * kblocks * 1024 + lane * 16;
+    sp[f] = s_base + static_cast<size_t>(ch0 + li) * groups;
+  }
+
+  for (int row0 = row_begin; row0 < row_end; row0 += TM) {
+    const uint16_t* ap[MF];
+#pragma unroll
+    for (int mf = 0; mf < MF; ++mf) {
+      const int r = row0 + mf * 16 + li;
+      const int rr = r < row_end ? r : row_begin;  // rows past the end read a valid row: never stored
+      const int src = p.row_src ? p.row_src[rr] / p.src_div : rr;
+      ap[mf] = p.a + static_cast<size_t>(src) * p.lda + 32 * lg;
+    }
+    v4f acc[MF][NF];
+#pragma unroll
+    for (int mf = 0; mf < MF; ++mf)
+#pragma unroll
+      for (int f = 0; f < NF; ++f) acc[mf][f] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    v4i wreg[D][NF];
+    uint16_t sreg[D][NF];
+    v4i areg[D][MF][4];
+    auto load_block = [&](int slot, int kb) {
+      const int g = (128 * kb + 32 * lg) / p.gs;
+#pragma unroll
+      for (int f = 0; f < NF; ++f) {
+        wreg[slot][f] = *reinterpret_cast<const v4i*>(wp[f] + static_cast<size_t>(kb) * 1024);
+        sreg[slot][f] = sp[f][g];
+      }
+#pragma unroll
+      for (int mf = 0; mf < MF; ++mf)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) areg[slot][mf][t] = *reinterpret_cast<const v4i*>(ap[mf] + 128 * kb + 8 * t);
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+      if (d < kblocks) load_block(d, d);
+
+    for (int kb0 = 0; kb0 < kblocks; kb0 += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        const int kb = kb0 + d;
+        if (kb < kblocks) {
+#pragma unroll
+          for (int f = 0; f < NF; ++f) {
+            const float s = bf16_to_f32(sreg[d][f]);
+            const float m136s = -136.0f * s;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              const v4i wv = unpack8(static_cast<uint32_t>(wreg[d][f][t]), s, m136s);
+#pragma unroll
+              for (int mf = 0; mf < MF; ++mf)
+                acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wv),
+                                                                     __builtin_bit_cast(v8bf, areg[d][mf][t]),
+                                                                     acc[mf][f], 0, 0, 0);
+            }
+          }
+          if (kb + D < kblocks) load_block(d, kb + D);
+        }
+      }
+    }
+
+    // epilogue: as the bf16 grouped GEMM - round to bf16, optional SiLU-mul on the bf16 values
+#pragma unroll
+    for (int mf = 0; mf < MF; ++mf) {
+      const int r = row0 + mf * 16 + li;
+      if (r >= row_end) continue;
+#pragma unroll
+      for (int f = 0; f < NFH; ++f) {
+        if (!wok[f]) continue;
+        const int c0 = col[f] + lg * 4;
+        uint16_t yv[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) yv[q] = f32_to_bf16(acc[mf][f][q]);
+        if (SWIGLU) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            yv[q] = f32_to_bf16(silu_fixed(bf16_to_f32(yv[q])) * bf16_to_f32(f32_to_bf16(acc[mf][f + NFH][q])));
+        }
+        const uint2 packed = make_uint2(yv[0] | (static_cast<uint32_t>(yv[1]) << 16),
+                                        yv[2] | (static_cast<uint32_t>(yv[3]) << 16));
+        *reinterpret_cast<uint2*>(p.y + static_cast<size_t>(r) * p.ldy + c0) = packed;
+      }
+    }
+  }
+}
+
+template <int MF, int NF, bool SWIGLU, int D>
+int launch_w4(const W4Params& p, hipStream_t s) {
+  constexpr int NFH = SWIGLU ? NF / 2 : NF;
+  const int n_half = SWIGLU ? p.n / 2 : p.n;
+  const dim3 grid(ceil_div(n_half, kWaves * NFH * 16), p.E);
+  hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D>), grid, dim3(kWaves * kWave), 0, s, p);
+  return check_launch("kmoe_grouped_gemm_w4a16");
+}
+
+}  // namespace
+}  // namespace kmoe
+
+using namespace kmoe;
+
+extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t stream) {
+  KMOE_REQUIRE(a, KMOE_ERR_NULL, "grouped_gemm_w4a16: NULL args");
+  KMOE_REQUIRE(a->a && a->w && a->w_scale && a->lod && a->y, KMOE_ERR_NULL, "grouped_gemm_w4a16: NULL pointer");
+  KMOE_REQUIRE(a->E >= 1 && a->rows >= 0, KMOE_ERR_SHAPE, "grouped_gemm_w4a16: E=%d rows=%d", a->E, a->rows);
+  const bool swiglu = a->act == KMOE_ACT_SWIGLU;
+  KMOE_REQUIRE(a->act == KMOE_ACT_NONE || swiglu, KMOE_ERR_UNSUPPORTED, "grouped_gemm_w4a16: act=%d", a->act);
+  KMOE_REQUIRE(a->w_layout == KMOE_W_TILED, KMOE_ERR_UNSUPPORTED,
+               "grouped_gemm_w4a16: the packed weights must be tiled (kmoe_tile_weights_i8 on [E, n, k/2] bytes)");
+  KMOE_REQUIRE(a->k >= 128 && a->k % 128 == 0 && a->n >= 16 && a->n % (swiglu ? 32 : 16) == 0, KMOE_ERR_SHAPE,
+               "grouped_gemm_w4a16: n=%d k=%d (need k %% 128 == 0, n %% %d == 0)", a->n, a->k, swiglu ? 32 : 16);
+  KMOE_REQUIRE(a->group_size >= 32 && a->group_size % 32 == 0 && a->k % a->group_size == 0, KMOE_ERR_SHAPE,
+               "grouped_gemm_w4a16: group_size=%d must be a multiple of 32 that divides k=%d", a->group_size, a->k);
+  KMOE_REQUIRE(a->lda >= a->k && a->lda % 8 == 0 && reinterpret_cast<uintptr_t>(a->a) % 16 == 0, KMOE_ERR_SHAPE,
+               "grouped_gemm_w4a16: activations need 16-byte aligned rows (lda=%lld)", static_cast<long long>(a->lda));
+  KMOE_REQUIRE(a->ldy % 4 == 0 && a->ldy >= (swiglu ? a->n / 2 : a->n), KMOE_ERR_SHAPE, "grouped_gemm_w4a16: ldy=%lld",
+               static_cast<long long>(a->ldy));
+  KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_w4a16: src_div=%d", a->src_div);
+  if (a->rows == 0) return KMOE_OK;
+  const W4Params p{a->a, a->lda, a->row_src, a->src_div, a->w, a->w_scale, a->group_size, a->lod,
+                   a->E, a->n,   a->k,       a->y,       a->ldy};
+  hipStream_t s = as_stream(stream);
+  int mf = a->variant;
+  if (mf == 0) {
+    // rows an expert gets under uniform routing, with headroom for the spread: an expert with
+    // more rows than one pass holds streams (and unpacks) its weights again
+    const int avg = ceil_div(a->rows, a->E);
+    mf = avg <= 10 ? 1 : (avg <= 22 ? 2 : 4);
+  }
+  switch (mf) {
+    case 1: return swiglu ? launch_w4<1, 2, true, 3>(p, s) : launch_w4<1, 2, false, 3>(p, s);
+    // tuning variants of the 16-row kernel: 1xy = x fragments per wave, y blocks in flight
+    case 122: return swiglu ? launch_w4<1, 2, true, 2>(p, s) : launch_w4<1, 2, false, 2>(p, s);
+    case 124: return swiglu ? launch_w4<1, 2, true, 4>(p, s) : launch_w4<1, 2, false, 4>(p, s);
+    case 142: return swiglu ? launch_w4<1, 4, true, 2>(p, s) : launch_w4<1, 4, false, 2>(p, s);
+    case 143: return swiglu ? launch_w4<1, 4, true, 3>(p, s) : launch_w4<1, 4, false, 3>(p, s);
+    case 2: return swiglu ? launch_w4<2, 2, true, 2>(p, s) : launch_w4<2, 2, false, 2>(p, s);
+    case 4: return swiglu ? launch_w4<4, 2, true, 2>(p, s) : launch_w4<4, 2, false, 2>(p, s);
+    default:
+      return fail(KMOE_ERR_UNSUPPORTED, "grouped_gemm_w4a16: variant=%d must be 0, 1, 2 or 4 (or a tuning variant)", a->variant);
+  }
+}

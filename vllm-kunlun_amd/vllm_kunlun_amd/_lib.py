@@ -22,6 +22,7 @@ KMOE_SCORE_SIGMOID = 1
 KMOE_FMT_INT8 = 0
 KMOE_FMT_FP8_BLOCK = 1
 KMOE_FMT_BF16 = 2
+KMOE_FMT_W4A16 = 3
 KMOE_W_ROWMAJOR, KMOE_W_TILED = 0, 1
 KMOE_A_ROWMAJOR, KMOE_A_CHUNKED = 0, 1
 STAGES = ("routing", "align", "quant1", "gemm1", "quant2", "gemm2", "shared", "combine")
@@ -51,6 +52,16 @@ class GemmBf16Args(C.Structure):
     ]
 
 
+class GemmW4Args(C.Structure):
+    _fields_ = [
+        ("a", C.c_void_p), ("lda", C.c_int64), ("row_src", C.c_void_p), ("src_div", C.c_int32),
+        ("w", C.c_void_p), ("w_scale", C.c_void_p), ("group_size", C.c_int32), ("lod", C.c_void_p),
+        ("E", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("rows", C.c_int32),
+        ("y", C.c_void_p), ("ldy", C.c_int64), ("act", C.c_int32), ("variant", C.c_int32),
+        ("w_layout", C.c_int32),
+    ]
+
+
 class GemmFp8Args(C.Structure):
     _fields_ = [
         ("a", C.c_void_p), ("lda", C.c_int64), ("a_scale", C.c_void_p), ("row_src", C.c_void_p),
@@ -72,6 +83,7 @@ class MoEArgs(C.Structure):
         ("stage_events", C.POINTER(C.c_void_p)), ("w_layout", C.c_int32), ("w_gate", C.c_void_p),
         ("w13_bias", C.c_void_p), ("w2_bias", C.c_void_p), ("activation", C.c_int32), ("act_alpha", C.c_float),
         ("act_limit", C.c_float), ("ws_layout", C.c_int32),
+        ("w13_scale", C.c_void_p), ("w2_scale", C.c_void_p), ("group_size", C.c_int32),
     ]
 
 
@@ -110,6 +122,7 @@ def _load() -> C.CDLL:
         "kmoe_silu_and_mul": (i32, [vp, i64, i32, i32, vp, i64, vp]),
         "kmoe_combine": (i32, [vp, i64, vp, vp, vp, i32, i32, i32, f32, vp, i64, vp, i64, vp]),
         "kmoe_grouped_gemm_bf16": (i32, [C.POINTER(GemmBf16Args), vp]),
+        "kmoe_grouped_gemm_w4a16": (i32, [C.POINTER(GemmW4Args), vp]),
         "kmoe_grouped_gemm_fp8_block": (i32, [C.POINTER(GemmFp8Args), vp]),
         "kmoe_moe_workspace_layout": (i32, [C.POINTER(MoEArgs), C.POINTER(MoELayout)]),
         "kmoe_moe_forward": (i32, [C.POINTER(MoEArgs), vp, sz, vp]),
@@ -125,7 +138,7 @@ lib = _load()
 EXPORTS = (
     "kmoe_last_error", "kmoe_version", "kmoe_softmax_topk", "kmoe_sigmoid_group_topk_norm", "kmoe_block_statistic",
     "kmoe_align_workspace_bytes", "kmoe_align", "kmoe_gather_rows", "kmoe_quant_i8_rows", "kmoe_quant_i8_rows_chunked", "kmoe_tile_weights_i8", "kmoe_quant_fp8_group128",
-    "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
+    "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_w4a16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
     "kmoe_moe_workspace_layout", "kmoe_moe_forward", "kmoe_router_gemm_workspace_bytes", "kmoe_router_gemm_bf16",
     "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16",
 )

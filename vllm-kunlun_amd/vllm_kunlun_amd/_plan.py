@@ -102,7 +102,7 @@ def rowmajor_int8_weights(w: torch.Tensor) -> torch.Tensor:
 
 
 _WEIGHT_DTYPE = {L.KMOE_FMT_INT8: (torch.int8,), L.KMOE_FMT_FP8_BLOCK: (torch.float8_e4m3fn, torch.uint8),
-                 L.KMOE_FMT_BF16: (torch.bfloat16,)}
+                 L.KMOE_FMT_BF16: (torch.bfloat16,), L.KMOE_FMT_W4A16: (torch.uint8,)}
 
 
 def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Tensor, top_k: int,
@@ -113,13 +113,15 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
                   stage_events=None, w_layout: Optional[int] = None,
                   router_weight: Optional[torch.Tensor] = None, w13_bias: Optional[torch.Tensor] = None,
                   w2_bias: Optional[torch.Tensor] = None, activation: str = "silu", act_alpha: float = 1.702,
-                  act_limit: float = 7.0) -> MoEPlan:
+                  act_limit: float = 7.0, group_size: Optional[int] = None) -> MoEPlan:
     """x bf16 [M,H], logits f32 [M,E], out bf16 [M,H]; w13 [E,2I,H], w2 [E,H,I] in the
     format's dtype; w13_aux/w2_aux: per-channel maxes (int8) or block scales (fp8), None for bf16.
     shared_expert: (ws13 [2Is,H], ws13_aux, ws2 [H,Is], ws2_aux) in the same format.
     logits may be None when router_weight (bf16 [E,H], the gate projection) is given: the
     layer then computes the router logits itself. bf16 only: w13_bias [E,2I] / w2_bias [E,H] (bf16)
-    and activation "swigluoai" (gate and up rows of w13 interleaved) select the expert-bias branch."""
+    and activation "swigluoai" (gate and up rows of w13 interleaved) select the expert-bias branch.
+    KMOE_FMT_W4A16: w13 [E,2I,H/2] and w2 [E,H,I/2] uint8 (two 4-bit codes per byte), tiled;
+    w13_aux/w2_aux their bf16 group scales [E,2I,H/group_size], [E,H,I/group_size]."""
     if scoring_func not in ("softmax", "sigmoid"):
         raise ValueError(f"Unsupported scoring_func: {scoring_func}")
     if logits is None and router_weight is None:
@@ -132,13 +134,26 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     if w13.dtype not in _WEIGHT_DTYPE[fmt] or w2.dtype != w13.dtype:
         raise ValueError(f"moe plan: weight dtype {w13.dtype} does not fit the layer format")
     E, two_i, H = w13.shape
+    w4 = fmt == L.KMOE_FMT_W4A16
+    if w4:
+        H *= 2  # two codes per byte
     M = x.shape[0]
     if tuple(x.shape) != (M, H) or tuple(out.shape) != (M, H) or (logits is not None and tuple(logits.shape) != (M, E)):
         raise ValueError("moe plan: x/out must be [M,H] and logits [M,E]")
     if logits is None and (router_weight.dtype != torch.bfloat16 or tuple(router_weight.shape) != (E, H)):
         raise ValueError("moe plan: router_weight must be bfloat16 [E,H]")
-    if tuple(w2.shape) != (E, H, two_i // 2):
+    if tuple(w2.shape) != (E, H, two_i // (4 if w4 else 2)):
         raise ValueError("moe plan: w2 must be [E,H,I] for w13 [E,2I,H]")
+    if w4:
+        gs = int(group_size or 0)
+        if w13_aux is None or w2_aux is None or w13_aux.dtype != torch.bfloat16 or w2_aux.dtype != torch.bfloat16:
+            raise ValueError("moe plan: 4-bit weights need bfloat16 group scales")
+        if gs < 32 or gs % 32 or H % gs or (two_i // 2) % gs:
+            raise ValueError(f"moe plan: group_size={group_size} must be a multiple of 32 dividing H and I")
+        if tuple(w13_aux.shape) != (E, two_i, H // gs) or tuple(w2_aux.shape) != (E, H, two_i // 2 // gs):
+            raise ValueError("moe plan: group scales must be [E,2I,H/group_size] and [E,H,I/group_size]")
+        if shared_expert is not None:
+            raise NotImplementedError("moe plan: no shared expert with 4-bit weights")
     a = L.MoEArgs()
     a.M, a.H, a.E, a.K, a.I = M, H, E, int(top_k), two_i // 2
     a.format = fmt
@@ -152,8 +167,11 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     a.bias = 0 if e_score_correction_bias is None else e_score_correction_bias.data_ptr()
     a.x = x.data_ptr()
     a.w13, a.w2 = w13.data_ptr(), w2.data_ptr()
-    a.w13_max = 0 if w13_aux is None else w13_aux.data_ptr()
-    a.w2_max = 0 if w2_aux is None else w2_aux.data_ptr()
+    if w4:
+        a.w13_scale, a.w2_scale, a.group_size = w13_aux.data_ptr(), w2_aux.data_ptr(), int(group_size)
+    else:
+        a.w13_max = 0 if w13_aux is None else w13_aux.data_ptr()
+        a.w2_max = 0 if w2_aux is None else w2_aux.data_ptr()
     keep = list(tensors)
     if shared_expert is not None:
         ws13, ws13_aux, ws2, ws2_aux = shared_expert

@@ -275,18 +275,30 @@ class KunlunCompressedTensorsW8A8Fp8MoEMethod(_MonolithicQuantMoE):
 class KunlunCompressedTensorsWNA16MoEMethod:
     """4-bit weight-only MoE (reference: compressed_tensors_moe.py:294-360). The reference
     unpacks the whole packed weight tensors to fp16 inside EVERY apply() (:320-327) and then
-    calls the unquantized fused_moe; here the unpacking (kmoe_dequant_w4_bf16) runs once in
-    process_weights_after_loading, the bf16 weights are tiled for the MFMA kernels, and the
-    packed tensors are dropped. Packed layout as in dequant_int4_native
-    (quantization/kernels/quant_ops.py:71-86): uint8, two codes per byte, low nibble first,
-    code - 8; scales per contiguous group of `group_size` along k, or one per row."""
+    calls the unquantized fused_moe. Here, in process_weights_after_loading:
+      * the packed tensors are tiled in place and kept for kmoe_grouped_gemm_w4a16, which reads
+        them once per call and unpacks in registers: the path for decode-sized batches
+        (`native` = "auto" or "only"; needs hidden and intermediate sizes that are multiples of
+        128 and a group size that is a multiple of 32);
+      * the weights are unpacked ONCE (kmoe_dequant_w4_bf16) to tiled bf16 tensors for batches with
+        many rows per expert (`native` = "auto" or False). "auto" keeps both copies (1.25x the
+        bf16 bytes); "only" keeps the packed one and serves every batch from it.
+    Packed layout as in dequant_int4_native (quantization/kernels/quant_ops.py:71-86): uint8,
+    two codes per byte, low nibble first, code - 8; scales per contiguous group of `group_size`
+    along k, or one per row."""
 
-    def __init__(self, weight_quant=None, input_quant=None, moe=None):
+    # rows per expert up to which the packed weights are streamed (above: the unpacked copy)
+    NATIVE_MAX_ROWS_PER_EXPERT = 48
+
+    def __init__(self, weight_quant=None, input_quant=None, moe=None, native="auto"):
         self.weight_quant = weight_quant
         self.input_quant = input_quant
         self.moe = moe
         gs = _get(weight_quant, "group_size") if weight_quant is not None else None
         self.group_size = int(gs) if (gs and _strategy(weight_quant) == "group") else None  # None: one scale per row
+        if native not in ("auto", "only", False):
+            raise ValueError("native must be 'auto', 'only' or False")
+        self.native = native
 
     @property
     def is_monolithic(self) -> bool:
@@ -306,8 +318,20 @@ class KunlunCompressedTensorsWNA16MoEMethod:
         layer.w13_weight_scale = mk(E, 2 * I, g13, dt=torch.bfloat16)
         layer.w2_weight_scale = mk(E, H, g2, dt=torch.bfloat16)
 
+    def _native_possible(self, layer) -> bool:
+        E, n13, half_h = layer.w13_weight_packed.shape
+        H, I = 2 * half_h, n13 // 2
+        gs13, gs2 = self.group_size or H, self.group_size or I
+        return (layer.w13_weight_packed.is_cuda and H % 128 == 0 and I % 128 == 0 and gs13 == gs2
+                and gs13 % 32 == 0 and H % gs13 == 0 and I % gs13 == 0)
+
     def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
         with torch.no_grad():
+            native = self.native and self._native_possible(layer)
+            if self.native == "only" and not native:
+                raise ValueError("native='only' needs CUDA tensors, H and I multiples of 128 and one group size "
+                                 "(a multiple of 32) for both weight tensors")
+            keep_bf16 = self.native != "only"
             for name in ("w13", "w2"):
                 packed = getattr(layer, f"{name}_weight_packed").data.contiguous()
                 scale = getattr(layer, f"{name}_weight_scale").data.to(torch.bfloat16).contiguous()
@@ -317,19 +341,54 @@ class KunlunCompressedTensorsWNA16MoEMethod:
                 if k % gs or scale.shape[-1] != k // gs:
                     raise ValueError(f"{name}: scales {tuple(scale.shape)} do not fit k={k}, group_size={gs}")
                 L.require_device(packed, scale)
-                w = torch.empty((E, n, k), dtype=torch.bfloat16, device=packed.device)
-                L.check(L.lib.kmoe_dequant_w4_bf16(L.ptr(packed), L.ptr(scale), E * n, k, gs, L.ptr(w), L.stream()))
-                param = torch.nn.Parameter(w, requires_grad=False)
-                setattr(layer, f"{name}_weight", param)
-                delattr(layer, f"{name}_weight_packed")
-            if getattr(self, "tile_weights", True):
+                if keep_bf16:
+                    w = torch.empty((E, n, k), dtype=torch.bfloat16, device=packed.device)
+                    L.check(L.lib.kmoe_dequant_w4_bf16(L.ptr(packed), L.ptr(scale), E * n, k, gs, L.ptr(w), L.stream()))
+                    setattr(layer, f"{name}_weight", torch.nn.Parameter(w, requires_grad=False))
+                if native:
+                    getattr(layer, f"{name}_weight_packed").data = packed
+                    getattr(layer, f"{name}_weight_scale").data = scale
+                else:
+                    delattr(layer, f"{name}_weight_packed")
+            if native:
+                if not tile_pair_(layer.w13_weight_packed, layer.w2_weight_packed):
+                    raise RuntimeError("4-bit weights: tiling the packed tensors failed")
+            layer.w4_native = bool(native)
+            if keep_bf16 and getattr(self, "tile_weights", True):
                 tile_pair_(layer.w13_weight, layer.w2_weight)
 
+    def _routing_kwargs(self, layer):
+        return dict(scoring_func=getattr(layer, "scoring_func", "softmax"),
+                    num_expert_group=getattr(layer, "num_expert_group", None),
+                    topk_group=getattr(layer, "topk_group", None),
+                    e_score_correction_bias=getattr(layer, "e_score_correction_bias", None))
+
     def apply_monolithic(self, layer, x: torch.Tensor, router_logits: torch.Tensor, **kwargs):
-        """bf16 activations against the unpacked weights: KunlunOps.fused_moe, as the reference's
-        apply() ends (:343-360)."""
+        """bf16 activations. Few rows per expert: the packed weights (kmoe_grouped_gemm_w4a16
+        inside kmoe_moe_forward). Otherwise the unpacked weights through KunlunOps.fused_moe, as
+        the reference's apply() ends (:343-360). Routing as in KunlunOps.fused_moe (always
+        normalised, sigmoid scale 1.0)."""
+        top_k = self.moe.experts_per_token
+        E = layer.w13_weight_scale.shape[0] if getattr(layer, "w4_native", False) else layer.w13_weight.shape[0]
+        rows_per_expert = -(-x.shape[0] * top_k // E)
+        has_bias = getattr(layer, "w13_bias", None) is not None or getattr(layer, "w2_bias", None) is not None
+        use_native = getattr(layer, "w4_native", False) and not has_bias and (
+            self.native == "only" or rows_per_expert <= self.NATIVE_MAX_ROWS_PER_EXPERT)
+        if use_native:
+            if x.dtype != torch.bfloat16:
+                raise NotImplementedError(f"4-bit MoE: activations must be bfloat16, got {x.dtype}")
+            xc = x.contiguous()
+            out = torch.empty_like(xc)
+            rk = self._routing_kwargs(layer)
+            gs = self.group_size or 2 * layer.w13_weight_packed.shape[-1]
+            plan = make_moe_plan(L.KMOE_FMT_W4A16, xc, router_logits.to(torch.float).contiguous(), out, top_k,
+                                 layer.w13_weight_packed, layer.w2_weight_packed, layer.w13_weight_scale,
+                                 layer.w2_weight_scale, rk["scoring_func"], True, rk["num_expert_group"],
+                                 rk["topk_group"], 1.0, rk["e_score_correction_bias"], group_size=gs)
+            plan()
+            return out
         from ...ops._kunlun_ops import KunlunOps as ops
-        return ops.fused_moe(x, layer.w13_weight, layer.w2_weight, router_logits, 0, self.moe.experts_per_token,
+        return ops.fused_moe(x, layer.w13_weight, layer.w2_weight, router_logits, 0, top_k,
                              renormalize=getattr(layer, "renormalize", True), inplace=True,
                              use_grouped_topk=getattr(layer, "use_grouped_topk", False),
                              num_expert_group=getattr(layer, "num_expert_group", None),

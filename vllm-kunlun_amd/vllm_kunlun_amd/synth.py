@@ -32,7 +32,8 @@ class MoEShape:
     I_shared: int = 0  # intermediate of the dense shared expert (0: none)
     hot_experts: int = 0   # add +hot_bias to the logits of this many fixed experts
     hot_bias: float = 0.0
-    quant: str = "int8"    # "none" (bf16 weights), "int8", "fp8"
+    quant: str = "int8"    # "none" (bf16 weights), "int8", "fp8", "w4" (4-bit weights, bf16 activations)
+    group_size: int = 128  # "w4": values per weight scale
 
     @property
     def P(self) -> int:
@@ -62,9 +63,14 @@ for _n in ("qwen3-decode", "qwen3-prefill"):
     SHAPES[_f] = replace(SHAPES[_n], name=_f, quant="none")
 
 
+# ... and with 4-bit weights (group scales of 128 values) on the packed-weight decode path
+SHAPES["qwen3-w4a16-decode"] = replace(SHAPES["qwen3-decode"], name="qwen3-w4a16-decode", quant="w4")
+
+
 def make_layer(shape: MoEShape, device="cuda", seed: int = 0) -> "SynthLayer":
     """The synthetic layer of a shape in the format the shape names."""
-    return {"int8": make_w8a8_layer, "fp8": make_fp8_layer, "none": make_bf16_layer}[shape.quant](shape, device, seed)
+    return {"int8": make_w8a8_layer, "fp8": make_fp8_layer, "none": make_bf16_layer,
+            "w4": make_w4_layer}[shape.quant](shape, device, seed)
 
 
 def scaled(shape: MoEShape, **kw) -> MoEShape:
@@ -101,8 +107,9 @@ class SynthLayer:
         if self.shared is not None:
             shared = (rm(self.shared[0]), self.shared[1].detach().cpu(), rm(self.shared[2]),
                       self.shared[3].detach().cpu())
-        return (rm(lay.w13_weight), aux("w13_weight_scale"), rm(lay.w2_weight), aux("w2_weight_scale"),
-                shared)
+        packed = not hasattr(lay, "w13_weight")  # 4-bit layer that kept only its packed weights
+        return (rm(lay.w13_weight_packed if packed else lay.w13_weight), aux("w13_weight_scale"),
+                rm(lay.w2_weight_packed if packed else lay.w2_weight), aux("w2_weight_scale"), shared)
 
     def apply_kwargs(self) -> dict:
         s = self.shape
@@ -186,6 +193,42 @@ def make_bf16_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer
         layer.w13_weight.data[e].copy_(torch.randn(2 * s.I, s.H, generator=g, device=dev) * 0.02)
         layer.w2_weight.data[e].copy_(torch.randn(s.H, s.I, generator=g, device=dev) * 0.02)
     layer.quant_method.process_weights_after_loading(layer)
+    x, logits = _activations(s, g, dev)
+    return SynthLayer(s, layer, x, logits, bias, None)
+
+
+def make_w4_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
+    """FusedMoE with the 4-bit method (packed weights kept, native="only"): weights ~ N(0, 0.02)
+    quantised per group of `group_size` values to codes 0..15 (value = (code - 8) * scale)."""
+    from types import SimpleNamespace
+    from .quantization.compressed_tensors.compressed_tensors_moe import KunlunCompressedTensorsWNA16MoEMethod
+    dev = torch.device(device)
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    s = shape
+    bias = _routing_inputs(s, g, dev)
+    wq = SimpleNamespace(num_bits=4, type="int", symmetric=True, dynamic=False, strategy="group",
+                         group_size=s.group_size)
+    method = KunlunCompressedTensorsWNA16MoEMethod(wq, None, SimpleNamespace(experts_per_token=s.K), native="only")
+    layer = FusedMoE(num_experts=s.E, top_k=s.K, hidden_size=s.H, intermediate_size=s.I, renormalize=True,
+                     use_grouped_topk=s.n_group > 1, num_expert_group=s.n_group, topk_group=s.topk_group,
+                     scoring_func=s.scoring, e_score_correction_bias=bias, quant_method=method, device=dev)
+
+    def quantise(w):  # [n, k] float -> packed uint8 [n, k/2], bf16 scales [n, k/gs]
+        n, k = w.shape
+        grp = w.view(n, k // s.group_size, s.group_size)
+        scale = (grp.abs().amax(-1) / 7.0).clamp_min(1e-8).bfloat16()
+        codes = (torch.round(grp / scale.float().unsqueeze(-1)).clamp(-8, 7) + 8).to(torch.uint8).view(n, k)
+        return codes[:, 0::2] | (codes[:, 1::2] << 4), scale
+
+    for e in range(s.E):
+        p13, s13 = quantise(torch.randn(2 * s.I, s.H, generator=g, device=dev) * 0.02)
+        p2, s2 = quantise(torch.randn(s.H, s.I, generator=g, device=dev) * 0.02)
+        layer.w13_weight_packed.data[e].copy_(p13)
+        layer.w13_weight_scale.data[e].copy_(s13)
+        layer.w2_weight_packed.data[e].copy_(p2)
+        layer.w2_weight_scale.data[e].copy_(s2)
+    method.process_weights_after_loading(layer)
     x, logits = _activations(s, g, dev)
     return SynthLayer(s, layer, x, logits, bias, None)
 

@@ -105,16 +105,25 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
     wts[threadIdx.x] = dq ? topk_w[j] * dq[j] : topk_w[j];
   }
   __syncthreads();
-  for (int c = threadIdx.x * 8; c < H; c += blockDim.x * 8) {
+  // blockIdx.y: which 2048-column slice of the row (wide rows at small M: more workgroups)
+  for (int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8; c < H; c += gridDim.y * blockDim.x * 8) {
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int k = 0; k < K; ++k) {
-      const int r = rows[k];
-      if (r < 0) continue;  // pair without a sorted row contributes nothing
-      Pack8 p;
-      p.v = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(r) * ld_x + c);
-      const float w = wts[k];
+    constexpr int kBatch = 4;  // rows loaded together: one memory round trip per 4 experts, not per expert
+    for (int k0 = 0; k0 < K; k0 += kBatch) {
+      Pack8 p[kBatch];
+      int r[kBatch];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(w, bf16_to_f32(p.h[j]), acc[j]);
+      for (int i = 0; i < kBatch; ++i) {
+        r[i] = k0 + i < K ? rows[k0 + i] : -1;
+        p[i].v = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(max(r[i], 0)) * ld_x + c);
+      }
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) {
+        if (r[i] < 0) continue;  // pair without a sorted row contributes nothing (its load read row 0)
+        const float w = wts[k0 + i];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(w, bf16_to_f32(p[i].h[j]), acc[j]);
+      }
     }
     Pack8 o;
 #pragma unroll
@@ -302,7 +311,7 @@ extern "C" int kmoe_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_
                (long long)ld_addend);
   if (M == 0) return KMOE_OK;
   const int epilogue = (out_scale != 1.0f || addend) ? 1 : 0;
-  hipLaunchKernelGGL(combine_kernel, dim3(M), dim3(256), 0, as_stream(stream), x, ld_x, moe_index, topk_w,
+  hipLaunchKernelGGL(combine_kernel, dim3(M, ceil_div(H, 256 * 8)), dim3(256), 0, as_stream(stream), x, ld_x, moe_index, topk_w,
                      dequant_scale, K, H, out_scale, epilogue, addend, ld_addend, out, ld_out);
   return check_launch("kmoe_combine");
 }

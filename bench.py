@@ -134,7 +134,7 @@ def cpu_baseline(sl, budget_s=10.0):
     t0 = time.perf_counter()
     fn(*args)  # warm-up
     first = time.perf_counter() - t0
-    runs = max(1, min(200, int(budget_s / max(first, 1e-3))))  # about budget_s seconds of CPU work
+    runs = max(1, min(600, int(budget_s / max(first, 1e-3))))  # about budget_s seconds of CPU work
     times = []
     for _ in range(runs):
         t0 = time.perf_counter()

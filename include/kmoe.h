@@ -132,9 +132,11 @@ int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q,
                        int64_t ld_q, float* row_max, kmoe_stream_t stream);
 
 /*
- * Same quantisation, codes written "chunk-major": q is [C/16][R][16], i.e. code
- * (r, c) sits at ((c/16)*R + r)*16 + c%16 — the activation layout of the
- * weight-streaming GEMM (KMOE_A_CHUNKED). Limits as above, and C % 16 == 0.
+ * Same quantisation, codes written "chunk-major": q is [C/64][R][64], i.e. code
+ * (r, c) sits at ((c/64)*R + r)*64 + c%64 — the activation layout of the
+ * weight-streaming GEMM (KMOE_A_CHUNKED): the 64 bytes of a row that one MFMA step
+ * consumes are contiguous, the rows of a step next to each other.
+ * Limits as above, and C % 64 == 0.
  */
 int kmoe_quant_i8_rows_chunked(const uint16_t* x, int64_t ld_x, int R, int C,
                                int8_t* q, float* row_max, kmoe_stream_t stream);
@@ -176,7 +178,7 @@ typedef struct kmoe_gemm_i8_args {
   int32_t act;            /* KMOE_ACT_*                                         */
   int32_t variant;        /* 0 = choose from shape; >0 force a kernel variant   */
   int32_t w_layout;       /* KMOE_W_ROWMAJOR, or KMOE_W_TILED (kmoe_tile_weights_i8) */
-  int32_t a_layout;       /* KMOE_A_ROWMAJOR, or KMOE_A_CHUNKED: a is [k/16][a_rows][16]
+  int32_t a_layout;       /* KMOE_A_ROWMAJOR, or KMOE_A_CHUNKED: a is [k/64][a_rows][64]
                              (kmoe_quant_i8_rows_chunked); needs w_layout TILED   */
   int32_t a_rows;         /* rows of the chunked activation array               */
   /* Optional "tail expert": one more expert (e.g. a dense shared expert run in the
@@ -453,7 +455,7 @@ typedef struct kmoe_moe_layout {
   size_t topk_w, topk_ids, moe_index, sorted_src, expert_m, lod, align_ws;
   size_t xq, xmax, act, actq, actmax, down;
   size_t sh_lod, sh_act, sh_actq, sh_actmax, sh_out;
-  size_t codes_chunked; /* 1: xq/actq/sh_actq are chunk-major [C/16][rows][16] (the
+  size_t codes_chunked; /* 1: xq/actq/sh_actq are chunk-major [C/64][rows][64] (the
                            weight-streaming decode path), 0: row-major [rows][C] */
   size_t logit_planes;  /* partial router logits [planes][M][E] f32 (w_gate given)   */
   size_t n_logit_planes;

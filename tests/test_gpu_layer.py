@@ -84,8 +84,8 @@ def test_layer_matches_oracles(name, base, over):
     lod = _view(ws, lay.lod, E + 1, torch.int32).cpu().numpy()
     R = P + (shape.M if shape.I_shared == I else 0)  # an equal-width shared expert adds rows [P, P+M)
     actq = _view(ws, lay.actq, R * I, torch.int8).cpu().numpy()
-    if lay.codes_chunked:  # [I/16][R][16] -> [R][I]
-        actq = actq.reshape(I // 16, R, 16).transpose(1, 0, 2)
+    if lay.codes_chunked:  # [I/64][R][64] -> [R][I]
+        actq = actq.reshape(I // 64, R, 64).transpose(1, 0, 2)
     actq = np.ascontiguousarray(actq).reshape(R, I)[:P]
     topk_w = _view(ws, lay.topk_w, P, torch.float32).cpu().numpy().reshape(shape.M, shape.K)
     assert np.array_equal(ids, inter["topk_ids"]), "routing ids"

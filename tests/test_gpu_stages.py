@@ -323,14 +323,14 @@ def test_tile_weights(L, E, n, k):
     assert L.lib.kmoe_tile_weights_i8(L.ptr(src), L.ptr(src), E, n, k, L.stream()) == -2  # in place is refused
 
 
-@pytest.mark.parametrize("R,Cc", [(1, 16), (64, 2048), (100, 768), (33, 7168), (512, 2048)])
+@pytest.mark.parametrize("R,Cc", [(1, 64), (64, 2048), (100, 768), (33, 7168), (512, 2048)])
 def test_quant_i8_rows_chunked(L, R, Cc):
     torch.manual_seed(R + Cc)
     x = (torch.randn(R, Cc) * 3).bfloat16()
     x[0] = 0
     q_ref, mx_ref = co.quant_i8_rows(bits(x))
     dx = x.cuda()
-    q = torch.empty(Cc // 16, R, 16, dtype=torch.int8, device="cuda")
+    q = torch.empty(Cc // 64, R, 64, dtype=torch.int8, device="cuda")
     mx = torch.empty(R, dtype=torch.float32, device="cuda")
     L.check(L.lib.kmoe_quant_i8_rows_chunked(L.ptr(dx), Cc, R, Cc, L.ptr(q), L.ptr(mx), L.stream()))
     sync()
@@ -356,7 +356,7 @@ def _gemm_layout_case(L, E, n, k, counts, act, variant, gather, chunked, seed=0)
     y_ref, acc_ref = co.grouped_gemm_i8(a, a_max, w, w_max, lod, act=act, row_src=row_src, src_div=src_div,
                                         want_acc=True)
     n_out = n // 2 if act else n
-    a_dev = dev(np.ascontiguousarray(a.reshape(a_rows, k // 16, 16).transpose(1, 0, 2))) if chunked else dev(a)
+    a_dev = dev(np.ascontiguousarray(a.reshape(a_rows, k // 64, 64).transpose(1, 0, 2))) if chunked else dev(a)
     d = dict(a=a_dev, a_max=dev(a_max), w=dev(_tile_ref(w)), w_max=dev(w_max), lod=dev(lod),
              row_src=None if row_src is None else dev(row_src))
     y = torch.zeros(max(rows, 1), n_out, dtype=torch.bfloat16, device="cuda")

@@ -235,8 +235,8 @@ extern "C" int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C,
 extern "C" int kmoe_quant_i8_rows_chunked(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, float* row_max,
                                           kmoe_stream_t stream) {
   KMOE_REQUIRE(x && q && row_max, KMOE_ERR_NULL, "quant_i8_rows_chunked: NULL pointer");
-  KMOE_REQUIRE(R >= 0 && C >= 16 && C % 16 == 0 && C <= 16384, KMOE_ERR_SHAPE,
-               "quant_i8_rows_chunked: R=%d C=%d (need C %% 16 == 0, 16 <= C <= 16384)", R, C);
+  KMOE_REQUIRE(R >= 0 && C >= 64 && C % 64 == 0 && C <= 16384, KMOE_ERR_SHAPE,
+               "quant_i8_rows_chunked: R=%d C=%d (need C %% 64 == 0, 64 <= C <= 16384)", R, C);
   KMOE_REQUIRE(ld_x % 8 == 0 && ld_x >= C, KMOE_ERR_SHAPE,
                "quant_i8_rows_chunked: row stride %lld must be a multiple of 8 and >= C", (long long)ld_x);
   if (R == 0) return KMOE_OK;

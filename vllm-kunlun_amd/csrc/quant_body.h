@@ -49,8 +49,8 @@ __device__ inline void quant_i8_rows_body(const uint16_t* __restrict__ x, int64_
   }
   if (!live) return;
   const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
-  // row-major: vector v of the row; chunk-major [C/16][R][16]: vector v is half v%2 of chunk v/2
-  uint2* dst = reinterpret_cast<uint2*>(q + static_cast<size_t>(r) * (chunked ? 16 : ld_q));
+  // row-major: vector v of the row; chunk-major [C/64][R][64]: vector v is eighth v%8 of chunk v/8
+  uint2* dst = reinterpret_cast<uint2*>(q + static_cast<size_t>(r) * (chunked ? 64 : ld_q));
   const size_t vstride = chunked ? static_cast<size_t>(R) : 0;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -64,7 +64,7 @@ __device__ inline void quant_i8_rows_body(const uint16_t* __restrict__ x, int64_
         const int qi = static_cast<int>(f);
         w[j >> 2] |= static_cast<uint32_t>(qi & 0xff) << (8 * (j & 3));
       }
-      dst[chunked ? (v >> 1) * vstride * 2 + (v & 1) : v] = make_uint2(w[0], w[1]);
+      dst[chunked ? (v >> 3) * vstride * 8 + (v & 7) : v] = make_uint2(w[0], w[1]);
     }
   }
   if (t == 0) row_max[r] = amax;

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """MoE-layer throughput of the W8A8 fused-MoE path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--tokens M]
 
 A step is one call of the whole layer (routing -> align -> int8 quant -> gate_up
 GEMM + SiLU-mul -> int8 quant -> down GEMM -> combine, plus the shared expert
@@ -14,6 +14,7 @@ import argparse
 import ctypes as C
 import json
 import os
+import re
 import sys
 import time
 
@@ -156,6 +157,8 @@ def main():
                     help="replay the layer from a captured HIP graph (as a serving engine does) or launch it eagerly")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--tokens", type=int, default=0,
+                    help="run the workload's layer at another batch (tokens per call); the config then says so")
     ap.add_argument("--router", action="store_true",
                     help="hand the layer the bf16 gate weight [E,H] instead of router logits: the router GEMM "
                          "then runs inside each step (reported in config; not the default workload)")
@@ -172,6 +175,10 @@ def main():
 
     torch.cuda.set_device(0)
     shape = synth.SHAPES[a.workload]
+    label = WORKLOAD_LABEL[a.workload]
+    if a.tokens and a.tokens != shape.M:
+        shape = synth.scaled(shape, M=a.tokens)
+        label = re.sub(r"(decode|prefill), \d+ tokens", f"{a.tokens} tokens (batch set by --tokens)", label)
     from vllm_kunlun_amd._plan import make_moe_plan
     sl = synth.make_layer(shape, "cuda:0", seed=a.seed)
     lay = sl.layer
@@ -249,15 +256,16 @@ def main():
     peak_tops = PEAK_TOPS[shape.quant]
     hbm_bound = intensity < peak_tops * 1e12 / (HBM_PEAK_GBS * 1e9)
     g1_s = stage_ms["gemm1"] * 1e-3
+    traffic = None if a.tokens else measured_traffic(a.workload)  # the counter summaries are of the named batch
     if hbm_bound:
         achieved = work["g1_bytes"] / g1_s / 1e9
         roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(a.workload)}
+                    "frac": achieved / HBM_PEAK_GBS, "traffic": traffic}
     else:
         achieved = work["g1_ops"] / g1_s / 1e12
         roofline = {"bound": "mfma", "achieved": achieved, "peak": peak_tops, "unit": "TFLOP/s",
-                    "frac": achieved / peak_tops, "traffic": measured_traffic(a.workload)}
-    many_rows = shape.P > 48 * shape.E  # the launchers' switch to the persistent 128-row-tile kernel
+                    "frac": achieved / peak_tops, "traffic": traffic}
+    many_rows = shape.P > 10 * shape.E  # the launchers' switch to the persistent 128-row-tile kernel
     g1_kernel = ("w4_stream_kernel" if w4 else "stream_gemm_i8_kernel" if plan.layout.codes_chunked else
                  "tiled_gemm_kernel" if many_rows and plan.args.w_layout == L.KMOE_W_TILED else "grouped_gemm_kernel")
     roofline.update(kernel=g1_kernel + " (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
@@ -277,7 +285,7 @@ def main():
         "vs_baseline": None,
         "dtype": DTYPE[shape.quant],
         "data": "synthetic",
-        "config": {"workload": WORKLOAD_LABEL[a.workload], "name": a.workload, "tokens": shape.M, "hidden": shape.H,
+        "config": {"workload": label, "name": a.workload, "tokens": shape.M, "hidden": shape.H,
                    "experts": shape.E, "top_k": shape.K, "moe_intermediate": shape.I,
                    "shared_intermediate": shape.I_shared, "routing": shape.scoring, "experts_hit": n_active,
                    "launch": "hipgraph replay" if graph is not None else "eager", "seed": a.seed,

@@ -395,6 +395,11 @@ int launch(const GemmParams& p, int rows, hipStream_t s, const char* what) {
   return check_launch(what);
 }
 
+// Tiled weights: from this many rows per expert (on average) the persistent 128-row-tile kernel wins over
+// the 16/32/64-row kernels of this file although most of its tile is padding: its weight stream is asynchronous
+// and it is bound by the weight bytes either way (measured cross-over: 8 to 16 rows, all three formats).
+constexpr int kTiledMinRows = 10;
+
 template <Kind KIND>
 int dispatch(const GemmParams& p, int rows, bool swiglu, int variant, hipStream_t s, const char* what) {
   if (variant == 0) {
@@ -462,7 +467,7 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
   if (a->rows == 0 && !(a->w_tail && a->tail_rows > 0)) return KMOE_OK;
   // Many rows per expert and tiled weights: the persistent 128-row-tile kernel (variants 5-7 force it)
   if (a->w_layout == KMOE_W_TILED && a->k % 128 == 0 &&
-      ((a->variant >= 5 && a->variant <= 9) || (a->variant == 0 && ceil_div(a->rows, a->E) > 48)))
+      ((a->variant >= 5 && a->variant <= 9) || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
     return tiled_gemm_i8(a, as_stream(stream));
   KMOE_REQUIRE(a->variant < 5 || a->variant > 9, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-9 need tiled weights and k %% 128 == 0");
   GemmParams p{a->a,   a->lda, a->a_max, a->row_src, a->src_div, a->w,   a->w_max,
@@ -498,7 +503,7 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
                "grouped_gemm_bf16: w_layout=%d (tiled weights need k %% 32 == 0, k=%d)", a->w_layout, a->k);
   // many rows per expert and tiled weights: the persistent 128-row-tile kernel (variant 5 forces it)
   if (a->w_layout == KMOE_W_TILED && a->k % 64 == 0 && a->ldy % 8 == 0 && !a->bias && !oai &&
-      (a->variant == 5 || (a->variant == 0 && ceil_div(a->rows, a->E) > 48)))
+      (a->variant == 5 || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
     return tiled_gemm_bf16(a, as_stream(stream));
   KMOE_REQUIRE(a->variant != 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variant 5 needs tiled weights, k %% 64 == 0");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
@@ -532,7 +537,7 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
                "grouped_gemm_fp8_block: w_layout=%d unknown", a->w_layout);
   // many rows per expert and tiled weights: the persistent 128-row-tile kernel (variant 5 forces it)
   if (a->w_layout == KMOE_W_TILED && a->k <= 8192 && a->ldy % 8 == 0 &&
-      (a->variant == 5 || (a->variant == 0 && ceil_div(a->rows, a->E) > 48)))
+      (a->variant == 5 || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
     return tiled_gemm_fp8(a, as_stream(stream));
   KMOE_REQUIRE(a->variant != 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_fp8_block: variant 5 needs tiled weights, k <= 8192");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,

@@ -287,8 +287,10 @@ class KunlunCompressedTensorsWNA16MoEMethod:
     two codes per byte, low nibble first, code - 8; scales per contiguous group of `group_size`
     along k, or one per row."""
 
-    # rows per expert up to which the packed weights are streamed (above: the unpacked copy)
-    NATIVE_MAX_ROWS_PER_EXPERT = 48
+    # rows per expert up to which the packed weights are streamed (above: the unpacked copy). The packed
+    # kernel unpacks every weight once per 16-64 rows, so its time grows with the rows; the tiled bf16 GEMM's
+    # hardly does. Measured cross-over on the Qwen3-30B-A3B shape: 22 rows per expert (about 360 tokens).
+    NATIVE_MAX_ROWS_PER_EXPERT = 20
 
     def __init__(self, weight_quant=None, input_quant=None, moe=None, native="auto"):
         self.weight_quant = weight_quant

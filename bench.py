@@ -147,6 +147,32 @@ def cpu_baseline(sl, budget_s=10.0):
                       f"{what}; host has {os.cpu_count()} cpus"}
 
 
+def vendor_dense_gemm(shape, g1_ops, peak_tops, reps=20):
+    """The vendor library's dense GEMM of the gate_up GEMM's size, as a yardstick only: one
+    [H,2I] weight matrix for all P rows (no experts, no gather, no dequantisation, no SiLU-mul)."""
+    import torch
+    P, H, N = shape.P, shape.H, 2 * shape.I
+    if shape.quant == "int8":
+        x = torch.randint(-127, 128, (P, H), dtype=torch.int8, device="cuda:0")
+        w = torch.randint(-127, 128, (N, H), dtype=torch.int8, device="cuda:0")
+        fn, what = (lambda: torch._int_mm(x, w.t())), "torch._int_mm (int8 x int8 -> int32)"
+    else:
+        x = torch.randn(P, H, device="cuda:0").bfloat16()
+        w = torch.randn(N, H, device="cuda:0").bfloat16()
+        fn, what = (lambda: x @ w.t()), "torch bf16 matmul"
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / reps
+    ops = 2.0 * P * H * N
+    return {"what": f"{what}, [{P},{H}] x [{H},{N}]", "ms": ms, "tops": ops / ms / 1e9,
+            "frac_of_peak": ops / ms / 1e9 / peak_tops}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -162,6 +188,9 @@ def main():
     ap.add_argument("--router", action="store_true",
                     help="hand the layer the bf16 gate weight [E,H] instead of router logits: the router GEMM "
                          "then runs inside each step (reported in config; not the default workload)")
+    ap.add_argument("--yardstick", action="store_true",
+                    help="also time the vendor library's dense GEMM (torch._int_mm / bf16 matmul) with the gate_up "
+                         "GEMM's operation count: [P,H] x [H,2I], one weight matrix, no gather, no epilogue")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one bitwise_not over 256 MiB (a kernel of known HBM traffic and a name nothing "
                          "else here has) before the timed region: the yardstick for FETCH_SIZE / WRITE_SIZE runs")
@@ -297,6 +326,8 @@ def main():
                   "algorithmic_bytes": work["layer_bytes"], "algorithmic_ops": work["layer_ops"],
                   "stage_ms": stage_ms},
     }
+    if a.yardstick and shape.quant in ("int8", "none"):
+        result["vendor_dense_gemm"] = vendor_dense_gemm(shape, work["g1_ops"], peak_tops)
     if not a.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(sl)
     else:

@@ -46,6 +46,12 @@ SMALL = [
     ("softmax-small", "qwen3-decode", dict(M=48, H=512, E=16, K=4, I=256)),
     ("softmax-ragged", "qwen3-decode", dict(M=33, H=768, E=24, K=6, I=160)),
     ("softmax-many-rows", "qwen3-decode", dict(M=700, H=256, E=8, K=2, I=128)),
+    # 24 rows per expert: the last batch on the weight-streaming path; 30: the first ones on the tile kernel,
+    # whose 128-row tiles are then mostly padding
+    ("softmax-stream-limit", "qwen3-decode", dict(M=96, H=512, E=16, K=4, I=256)),
+    ("softmax-mid-rows", "qwen3-decode", dict(M=120, H=512, E=16, K=4, I=256)),
+    ("shared-same-width-mid-rows", "dsv3-decode", dict(M=100, H=256, E=8, K=2, I=128, n_group=2, topk_group=1,
+                                                       I_shared=128)),
     ("sigmoid-grouped-shared", "dsv3-decode", dict(M=40, H=512, E=32, K=4, I=128, n_group=4, topk_group=2,
                                                    I_shared=256)),
     ("sigmoid-flat-shared", "kimi-decode", dict(M=16, H=256, E=48, K=8, I=64, I_shared=128)),

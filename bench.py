@@ -294,7 +294,7 @@ def main():
         achieved = work["g1_ops"] / g1_s / 1e12
         roofline = {"bound": "mfma", "achieved": achieved, "peak": peak_tops, "unit": "TFLOP/s",
                     "frac": achieved / peak_tops, "traffic": traffic}
-    many_rows = shape.P > 10 * shape.E  # the launchers' switch to the persistent 128-row-tile kernel
+    many_rows = shape.P > 10 * shape.E  # the launchers' switch to the persistent tile kernel
     g1_kernel = ("w4_stream_kernel" if w4 else "stream_gemm_i8_kernel" if plan.layout.codes_chunked else
                  "tiled_gemm_kernel" if many_rows and plan.args.w_layout == L.KMOE_W_TILED else "grouped_gemm_kernel")
     roofline.update(kernel=g1_kernel + " (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],

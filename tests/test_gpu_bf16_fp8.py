@@ -51,11 +51,11 @@ BF16_TILED_CASES = [
 
 
 @pytest.mark.parametrize("E,n,k,counts", BF16_TILED_CASES)
-@pytest.mark.parametrize("variant", [1, 2, 3, 5])
+@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 11])
 @pytest.mark.parametrize("act", [0, 1])
 def test_grouped_gemm_bf16_tiled_weights(L, E, n, k, counts, variant, act):
     """bf16 weights re-arranged (as bytes) by kmoe_tile_weights_i8: the LDS-staged kernels (1-3) and
-    the persistent 128-row-tile kernel (5)."""
+    the persistent tile kernel (5: tile height from the rows per expert; 6: 128 rows; 11: 64 rows)."""
     _bf16_case(L, E, n, k, counts, variant, act, tiled=True)
 
 
@@ -112,11 +112,11 @@ FP8_TILED_CASES = FP8_CASES + [
 
 
 @pytest.mark.parametrize("E,n,k,counts", FP8_TILED_CASES)
-@pytest.mark.parametrize("variant", [1, 2, 3, 5])
+@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 11])
 @pytest.mark.parametrize("act", [0, 1])
 def test_grouped_gemm_fp8_block_tiled_weights(L, E, n, k, counts, variant, act):
     """The same product with the weight bytes re-arranged by kmoe_tile_weights_i8: the LDS-staged
-    kernels (1-3) and the persistent 128-row-tile kernel (5)."""
+    kernels (1-3) and the persistent tile kernel (5: tile height by the rows per expert; 6: 128; 11: 64 rows)."""
     _fp8_case(L, E, n, k, counts, variant, act, tiled=True)
 
 

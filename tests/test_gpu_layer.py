@@ -46,12 +46,13 @@ SMALL = [
     ("softmax-small", "qwen3-decode", dict(M=48, H=512, E=16, K=4, I=256)),
     ("softmax-ragged", "qwen3-decode", dict(M=33, H=768, E=24, K=6, I=160)),
     ("softmax-many-rows", "qwen3-decode", dict(M=700, H=256, E=8, K=2, I=128)),
-    # 24 rows per expert: the last batch on the weight-streaming path; 30: the first ones on the tile kernel,
-    # whose 128-row tiles are then mostly padding
-    ("softmax-stream-limit", "qwen3-decode", dict(M=96, H=512, E=16, K=4, I=256)),
-    ("softmax-mid-rows", "qwen3-decode", dict(M=120, H=512, E=16, K=4, I=256)),
-    ("shared-same-width-mid-rows", "dsv3-decode", dict(M=100, H=256, E=8, K=2, I=128, n_group=2, topk_group=1,
-                                                       I_shared=128)),
+    # 10 rows per expert: the last batch on the weight-streaming path; 12 and 30: on the tile kernel (64-row tiles
+    # that are mostly padding); 60: 128-row tiles
+    ("softmax-stream-limit", "qwen3-decode", dict(M=40, H=512, E=16, K=4, I=256)),
+    ("softmax-short-tiles", "qwen3-decode", dict(M=120, H=512, E=16, K=4, I=256)),
+    ("softmax-tall-tiles-few-rows", "qwen3-decode", dict(M=240, H=512, E=16, K=4, I=256)),
+    ("shared-same-width-short-tiles", "dsv3-decode", dict(M=100, H=256, E=8, K=2, I=128, n_group=2, topk_group=1,
+                                                          I_shared=128)),
     ("sigmoid-grouped-shared", "dsv3-decode", dict(M=40, H=512, E=32, K=4, I=128, n_group=4, topk_group=2,
                                                    I_shared=256)),
     ("sigmoid-flat-shared", "kimi-decode", dict(M=16, H=256, E=48, K=8, I=64, I_shared=128)),
@@ -131,11 +132,12 @@ def test_staged_ops_equal_fused():
 def test_tiled_and_rowmajor_weights_give_the_same_bits():
     """process_weights_after_loading tiles the int8 weights in place on the GPU; a layer
     kept row-major (tile_weights=False) must produce identical outputs, in the streaming
-    regime (few rows per expert) and in the tiled-GEMM regime (many rows per expert)."""
+    regime (8 rows per expert) and in the tile kernel's (40 rows: 64-row tiles; 225 rows: 128-row tiles)."""
     from vllm_kunlun_amd import _plan, synth
     from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors_moe import (
         KunlunCompressedTensorsW8A8Int8MoEMethod)
-    for over in (dict(M=48, H=512, E=16, K=4, I=256), dict(M=900, H=256, E=8, K=2, I=128)):
+    for over in (dict(M=32, H=512, E=16, K=4, I=256), dict(M=160, H=512, E=16, K=4, I=256),
+                 dict(M=900, H=256, E=8, K=2, I=128)):
         shape = synth.scaled(synth.SHAPES["dsv3-decode"], n_group=4, topk_group=2, I_shared=128, **over)
         tiled = synth.make_w8a8_layer(shape, "cuda", seed=9)
         assert _plan.is_tiled(tiled.layer.w13_weight) and _plan.is_tiled(tiled.shared[0])
@@ -146,7 +148,7 @@ def test_tiled_and_rowmajor_weights_give_the_same_bits():
             del KunlunCompressedTensorsW8A8Int8MoEMethod.tile_weights
         assert not _plan.is_tiled(plain.layer.w13_weight)
         a = tiled.layer.quant_method.apply_monolithic(tiled.layer, tiled.x, tiled.logits, **tiled.apply_kwargs())
-        assert tiled.layer.quant_method.last_layout.codes_chunked == (1 if over["M"] == 48 else 0)
+        assert tiled.layer.quant_method.last_layout.codes_chunked == (1 if over["M"] == 32 else 0)
         b = plain.layer.quant_method.apply_monolithic(plain.layer, plain.x, plain.logits, **plain.apply_kwargs())
         torch.cuda.synchronize()
         assert torch.equal(a, b)

@@ -69,19 +69,15 @@ int check_shape(const kmoe_moe_args* a) {
   return KMOE_OK;
 }
 
-// Few rows per expert: every weight byte is used once, so stream tiled weights
-// against chunk-major codes; otherwise the LDS-tiled GEMM on row-major codes.
 // The weight-streaming decode path (chunk-major codes, no row tiles) against the persistent tile kernel:
-// the stream kernels' time grows with the rows per expert, the tile kernel's hardly does but it has a floor
-// set by how evenly its work items (an expert's 256-channel blocks) spread over the workgroups. Measured
-// cross-over: about 28 rows per expert at Qwen3's 768 items, about 11 at DeepSeek-V3's 4096.
+// the stream kernels re-read the weights once per 16-64 rows of an expert, so their time grows with the rows
+// per expert; the tile kernel's hardly does. Measured cross-over with 64-row tiles: 10-12 rows per expert on
+// both the Qwen3 and the DeepSeek-V3 shape.
 bool use_stream_path(const kmoe_moe_args* a) {
   const long long P = static_cast<long long>(a->M) * a->K;
-  const long long items = static_cast<long long>(a->E) * ((2 * a->I + 255) / 256);
-  const int max_rows = items >= 2048 ? 10 : 24;
   // a row-major shared expert cannot read the chunk-major codes this path quantises x into
-  return a->format == KMOE_FMT_INT8 && a->w_layout == KMOE_W_TILED && (P + a->E - 1) / a->E <= max_rows &&
-         a->M <= 1024 && (a->I_shared == 0 || a->ws_layout == KMOE_W_TILED);
+  return a->format == KMOE_FMT_INT8 && a->w_layout == KMOE_W_TILED && (P + a->E - 1) / a->E <= 10 && a->M <= 1024 &&
+         (a->I_shared == 0 || a->ws_layout == KMOE_W_TILED);
 }
 
 // A shared expert of the routed experts' width runs inside the routed GEMM launches

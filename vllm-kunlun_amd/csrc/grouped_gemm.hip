@@ -399,6 +399,9 @@ int launch(const GemmParams& p, int rows, hipStream_t s, const char* what) {
 // the 16/32/64-row kernels of this file although most of its tile is padding: its weight stream is asynchronous
 // and it is bound by the weight bytes either way (measured cross-over: 8 to 16 rows, all three formats).
 constexpr int kTiledMinRows = 10;
+// variants of the bf16 and fp8 launchers that force the tile kernel: 5 (tile height from the rows per expert),
+// 6 (128-row tiles), 11 (64-row tiles)
+inline bool tile_variant(int v) { return v == 5 || v == 6 || v == 11; }
 
 template <Kind KIND>
 int dispatch(const GemmParams& p, int rows, bool swiglu, int variant, hipStream_t s, const char* what) {
@@ -465,11 +468,11 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
   KMOE_REQUIRE(a->a_layout == KMOE_A_ROWMAJOR, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: a_layout=%d unknown",
                a->a_layout);
   if (a->rows == 0 && !(a->w_tail && a->tail_rows > 0)) return KMOE_OK;
-  // Many rows per expert and tiled weights: the persistent 128-row-tile kernel (variants 5-7 force it)
+  // Tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5-9, 11 force it)
   if (a->w_layout == KMOE_W_TILED && a->k % 128 == 0 &&
-      ((a->variant >= 5 && a->variant <= 9) || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
+      ((a->variant >= 5 && a->variant <= 9) || a->variant == 11 || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
     return tiled_gemm_i8(a, as_stream(stream));
-  KMOE_REQUIRE(a->variant < 5 || a->variant > 9, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-9 need tiled weights and k %% 128 == 0");
+  KMOE_REQUIRE(a->variant < 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-11 need tiled weights and k %% 128 == 0");
   GemmParams p{a->a,   a->lda, a->a_max, a->row_src, a->src_div, a->w,   a->w_max,
                a->lod, a->E,   a->n,     a->k,       a->y,       a->ldy, a->acc_out, a->w_layout == KMOE_W_TILED,
                a->w_tail, a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0, nullptr, 0, 0.f, 0.f};
@@ -501,11 +504,11 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
   if (a->rows == 0) return KMOE_OK;
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR || (a->w_layout == KMOE_W_TILED && a->k % 32 == 0), KMOE_ERR_SHAPE,
                "grouped_gemm_bf16: w_layout=%d (tiled weights need k %% 32 == 0, k=%d)", a->w_layout, a->k);
-  // many rows per expert and tiled weights: the persistent 128-row-tile kernel (variant 5 forces it)
+  // tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5, 6, 11 force it)
   if (a->w_layout == KMOE_W_TILED && a->k % 64 == 0 && a->ldy % 8 == 0 && !a->bias && !oai &&
-      (a->variant == 5 || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
+      (tile_variant(a->variant) || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
     return tiled_gemm_bf16(a, as_stream(stream));
-  KMOE_REQUIRE(a->variant != 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variant 5 needs tiled weights, k %% 64 == 0");
+  KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variants 5, 6, 11 need tiled weights, k %% 64 == 0");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), nullptr,    a->lod,  a->E,       a->n,
                a->k * 2,                              a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,
@@ -535,11 +538,11 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
   if (a->rows == 0) return KMOE_OK;
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR || a->w_layout == KMOE_W_TILED, KMOE_ERR_UNSUPPORTED,
                "grouped_gemm_fp8_block: w_layout=%d unknown", a->w_layout);
-  // many rows per expert and tiled weights: the persistent 128-row-tile kernel (variant 5 forces it)
+  // tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5, 6, 11 force it)
   if (a->w_layout == KMOE_W_TILED && a->k <= 8192 && a->ldy % 8 == 0 &&
-      (a->variant == 5 || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
+      (tile_variant(a->variant) || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
     return tiled_gemm_fp8(a, as_stream(stream));
-  KMOE_REQUIRE(a->variant != 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_fp8_block: variant 5 needs tiled weights, k <= 8192");
+  KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_fp8_block: variants 5, 6, 11 need tiled weights, k <= 8192");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), a->w_scale, a->lod,  a->E,       a->n,
                a->k,                                  a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,

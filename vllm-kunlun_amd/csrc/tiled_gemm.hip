@@ -91,11 +91,10 @@ __device__ inline void vmem_wait() {
   __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 
-constexpr int kMF = 8, kWavesT = 4;        // a wave: 8 row fragments (128 rows); 4 waves side by side along the channels
+constexpr int kWavesT = 4;                 // 4 waves side by side along the channels
 constexpr int kChunk = 128;                // bytes of K per row and chunk (2 MFMA steps)
 constexpr int kSteps = kChunk / 64;
 constexpr int kPitchT = kChunk + 32;       // 160 B: measured conflict-free for the b128 fragment reads (144 is not)
-constexpr int kNA = 16 * kMF * (kChunk / 16) / (kWavesT * kWave);  // 16-byte activation vectors per thread and chunk (= 4)
 constexpr int kStagesA = 4;                // chunk buffers of the asynchronous activation path
 constexpr int kMaxExperts = 1024 + 1;      // routed experts + the tail expert
 
@@ -142,8 +141,14 @@ struct Tile {
 // (32 bytes of K) is two 16-lane quarters of two neighbouring 1 KB blocks, lanes 32-63 taking
 // the next 16 bytes of K; the activation fragment takes the same bytes of its rows, so the
 // order of K inside a step differs from the 16x16 path while the sums (exact in int32) do not.
-template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false>
+// MF: 16-row fragments of a wave along the rows. 8: 128-row tiles; 4: 64-row tiles for launches whose
+// experts hold a few dozen rows each (half the MFMAs, fragment reads and epilogue per weight byte,
+// and registers for a third workgroup per CU).
+template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8>
 __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(const TiledParams p) {
+  constexpr int kMF = MF;
+  constexpr int kNA = 16 * kMF * (kChunk / 16) / (kWavesT * kWave);  // 16-byte activation vectors per thread and chunk
+  static_assert(kNA >= 1 && (M32 ? MF % 2 == 0 : true), "tile height");
   constexpr bool F8 = KIND == TKind::F8;
   constexpr bool I8 = KIND == TKind::I8;
   constexpr bool BF = KIND == TKind::BF16;
@@ -170,7 +175,8 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   __shared__ __attribute__((aligned(16))) int8_t patch[WM * kWavesT][kFragRows * kPatchPitch];
   // I8, per tile parity: channel scales (w_max / 127) and row scales (a_max / 127)
   __shared__ __attribute__((aligned(16))) float sw_lds[I8 ? 2 : 1][I8 ? kWavesT * NF * 16 : 4];
-  __shared__ float sa_lds[I8 ? 2 : 1][I8 ? kTM : 4];
+  // (a wave's copy of row maxes always writes 64 slots: tiles of fewer rows still get 64)
+  __shared__ float sa_lds[I8 ? 2 : 1][I8 ? (kTM > kWave ? kTM : kWave) : 4];
   // F8: weight block scales of the tile [parity][wave][fragment][k block], and the row scales
   // of the chunk in each activation buffer
   __shared__ float wsc_lds[F8 ? 2 : 1][F8 ? kWavesT * NF * kMaxKBlocks : 4];
@@ -722,9 +728,9 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   }
 }
 
-template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false>
+template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8>
 int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* what) {
-  constexpr int kTM = WM * 16 * kMF;
+  constexpr int kTM = WM * 16 * MF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int nfh = SWIGLU ? NF / 2 : NF;
   const int n_exp = p.E + (p.w_tail ? 1 : 0);
@@ -734,7 +740,7 @@ int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* w
   // persistent workgroups: WGS per CU
   const int grid = min(ceil_div(p.max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8);
   const size_t dyn = sizeof(int) * (static_cast<size_t>(p.E) + 1 + n_exp + 1);
-  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32>), dim3(grid), dim3(WM * kWavesT * kWave), dyn, s,
+  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32, MF>), dim3(grid), dim3(WM * kWavesT * kWave), dyn, s,
                      p);
   return check_launch(what);
 }
@@ -762,10 +768,23 @@ int tiled_common(const TiledParams& p, int rows, int* n_cu_out, const char* what
   return KMOE_OK;
 }
 
+// 64-row tiles (MF = 4) when nearly every expert fits one of them (48 rows per expert on average): the launch
+// is bound by the weight stream, and half the MFMAs, fragment reads and epilogue per weight byte leave more of
+// the CU to it (measured, int8 gate_up / down: Qwen3 shape at 32 rows per expert 101 -> 80 us; DeepSeek-V3 shape
+// at 32 rows 1426 -> 1284 / 770 -> 683 us). At 64 rows per expert half of the experts need a second tile and
+// a second pass over their weights: DeepSeek-V3 gate_up 1434 -> 1585 us, so the switch sits below that.
+// Variant 6 forces 128 rows, 11 forces 64.
+bool short_tiles(int variant, int rows, int n_experts, int max_avg_rows = 48) {
+  if (variant == 11) return true;
+  if (variant == 6) return false;
+  return ceil_div(rows, n_experts) <= max_avg_rows;
+}
+
 }  // namespace
 
-// variants 5, 6: 128x256 tiles, 4-slot weight ring, 2 workgroups per CU (the shape in use);
-// 7: 128x128 tiles, 8-slot ring, 3 workgroups per CU; 8: 256x256 tiles, 8 waves, 1 workgroup per CU
+// variant 5: 128x256 or 64x256 tiles by the rows per expert (6, 11: one of them), 4-slot weight ring, 2 workgroups
+// per CU (the shape in use); 7: 128x128 tiles, 8-slot ring, 3 workgroups per CU; 8: 256x256 tiles, 8 waves,
+// 1 workgroup per CU; 9: 128x256 tiles on the 32x32 MFMA shapes
 int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   const char* what = "kmoe_grouped_gemm_i8 (tiled)";
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
@@ -790,6 +809,9 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   if (a->variant == 9)
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what);
+  if (short_tiles(a->variant, a->rows, a->E))
+    return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)
                 : launch_tiled<K, false, 4, 4, 2, 1>(p, a->rows, s, n_cu, what);
 }
@@ -806,6 +828,9 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
   int n_cu = 0;
   if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
   constexpr TKind K = TKind::F8;
+  if (short_tiles(a->variant, a->rows, a->E))
+    return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)
                 : launch_tiled<K, false, 4, 4, 2, 1>(p, a->rows, s, n_cu, what);
 }
@@ -821,6 +846,9 @@ int tiled_gemm_bf16(const kmoe_gemm_bf16_args* a, hipStream_t s) {
   int n_cu = 0;
   if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
   constexpr TKind K = TKind::BF16;
+  if (short_tiles(a->variant, a->rows, a->E, 40))  // measured: at 48 rows per expert the 128-row tiles are 4 % ahead
+    return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)
                 : launch_tiled<K, false, 4, 4, 2, 1>(p, a->rows, s, n_cu, what);
 }

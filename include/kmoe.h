@@ -176,7 +176,10 @@ typedef struct kmoe_gemm_i8_args {
   int64_t ldy;
   int32_t* acc_out;       /* NULL, or int32 [rows, n]: raw accumulators         */
   int32_t act;            /* KMOE_ACT_*                                         */
-  int32_t variant;        /* 0 = choose from shape; >0 force a kernel variant   */
+  int32_t variant;        /* 0 = choose from the shape. Tuning and tests: 1-3 LDS-staged 16/32/64-row
+                             kernels; with tiled weights 5 = tile kernel (6: 128-row tiles, 11: 64-row
+                             tiles, 7-9: other tile shapes); with chunked activations 1, 2, 4, 8 =
+                             16-row fragments per pass of the streaming kernel      */
   int32_t w_layout;       /* KMOE_W_ROWMAJOR, or KMOE_W_TILED (kmoe_tile_weights_i8) */
   int32_t a_layout;       /* KMOE_A_ROWMAJOR, or KMOE_A_CHUNKED: a is [k/64][a_rows][64]
                              (kmoe_quant_i8_rows_chunked); needs w_layout TILED   */

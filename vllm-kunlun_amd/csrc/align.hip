@@ -15,7 +15,7 @@ namespace {
 constexpr int kThreads = 1024;            // workgroup size of the multi-workgroup kernels
 constexpr int kWaves = kThreads / kWave;  // 16
 constexpr int kMaxE = 1024;
-constexpr int kSingleMaxP = 8192;         // one workgroup handles up to this many pairs
+constexpr int kSingleMaxP = 4096;         // one workgroup handles up to this many pairs
 constexpr int kChunk = 2048;              // pairs per workgroup in the multi-workgroup path
 
 __device__ inline int key_bits(int E) { return 32 - __builtin_clz(max(E - 1, 1)); }
@@ -251,7 +251,7 @@ extern "C" int kmoe_align(const int32_t* topk_ids, int P, int E, int32_t* moe_in
   KMOE_REQUIRE(P >= 0 && P <= (1 << 24), KMOE_ERR_SHAPE, "align: P=%d outside [0,2^24]", P);
   hipStream_t s = as_stream(stream);
   if (P <= kSingleMaxP) {
-    const int threads = (E <= 256 && P <= 1024) ? 256 : kThreads;  // few waves: cheap barriers for decode sizes
+    const int threads = (E <= 256 && P <= 512) ? 256 : kThreads;  // few waves: cheap barriers for decode sizes
     const int steps = max(1, ceil_div(P, threads));
     const size_t lds = sizeof(int) * (16 + E + static_cast<size_t>(threads / kWave) * E);
     hipLaunchKernelGGL(align_single_kernel, dim3(1), dim3(threads), lds, s, topk_ids, P, E, steps, moe_index,

@@ -270,6 +270,12 @@ typedef struct kmoe_gemm_fp8_args {
   int32_t w_layout;       /* KMOE_W_ROWMAJOR, or KMOE_W_TILED: the bytes of w re-arranged
                              by kmoe_tile_weights_i8 (which moves bytes whatever they
                              encode); needs k % 128 == 0, always true here          */
+  /* Optional "tail expert", as in kmoe_gemm_i8_args: one more expert whose weights live
+     outside w (a dense shared expert run in the same launch). Its rows are
+     [tail_row0, tail_row0 + tail_rows) of y and read a rows tail_src0 + i (no gather). */
+  const uint8_t* w_tail;      /* NULL, or [n, k] in w_layout                          */
+  const float* w_scale_tail;  /* [n/128, k/128]                                       */
+  int32_t tail_row0, tail_rows, tail_src0;
 } kmoe_gemm_fp8_args;
 
 /*

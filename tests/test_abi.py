@@ -39,7 +39,7 @@ def test_struct_layouts_match_the_header(L):
     assert C.sizeof(L.GemmI8Args) == 8 * 8 + 16 + 8 * 3 + 8 + 16 + 16 + 16  # 8 ptr/int64, 4 int32, y/ldy/acc_out, act+variant, 3 int32 + pad
     assert C.sizeof(L.MoELayout) == 22 * 8
     assert C.sizeof(L.GemmBf16Args) == 6 * 8 + 16 + 16 + 16 + 16  # ..., act+variant+w_layout+pad, bias, alpha+limit  # 6 ptr/int64 (src_div padded), 4 int32, y/ldy, act+variant+w_layout+pad
-    assert C.sizeof(L.GemmFp8Args) == 8 * 8 + 16 + 16 + 16  # 8 ptr/int64, 4 int32, y/ldy, act+variant+w_layout+pad
+    assert C.sizeof(L.GemmFp8Args) == 8 * 8 + 16 + 16 + 16 + 16 + 16  # ..., act+variant+w_layout+pad, 2 tail ptrs, 3 int32 + pad
     assert L.MoEArgs.w_gate.offset == C.sizeof(L.MoEArgs) - 8 - 32 - 24  # then w13_bias, w2_bias, activation, alpha, limit, ws_layout; w13_scale, w2_scale, group_size + pad
     assert C.sizeof(L.GemmW4Args) == 3 * 8 + 8 + 2 * 8 + 8 + 8 + 16 + 16 + 16  # a/lda/row_src, src_div+pad, w/w_scale, group_size+pad, lod, 4 int32, y/ldy, act+variant+w_layout+pad
     a = L.MoEArgs()

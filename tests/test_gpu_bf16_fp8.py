@@ -223,10 +223,59 @@ def test_moe_fc_op_bf16_swish_glu():
     assert torch.all(y.view(rows, n)[:, n // 2:] == 0)
 
 
+@pytest.mark.parametrize("E,n,k,counts,tail", [(3, 256, 384, [5, 0, 21], 40), (2, 512, 1024, [70, 3], 7),
+                                               (20, 1024, 256, [((53 * i) % 300) for i in range(20)], 300),
+                                               (2, 256, 128, [0, 0], 33)])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 5, 6, 11])
+@pytest.mark.parametrize("act", [0, 1])
+def test_grouped_gemm_fp8_block_tail_expert(L, E, n, k, counts, tail, variant, act):
+    """w_tail / w_scale_tail: one more expert in the same launch, whose `tail` rows follow the routed
+    rows and read activation rows tail_src0 + i (a shared expert folded into the routed GEMM). The
+    oracle runs it as expert E of a weight tensor with E + 1 experts."""
+    torch.manual_seed(E * n + k + tail + act)
+    lod = _lod(counts)
+    rows = int(lod[-1])
+    lod_all = np.concatenate([lod, [rows + tail]]).astype(np.int32)
+    x = (torch.randn(rows + tail, k) * 2).bfloat16()
+    xq, xs = tm.quant_fp8_group128(x)
+    wq, ws = tm.quantize_weight_fp8_block128(torch.randn(E + 1, n, k) * 0.02)
+    a8, w8 = xq.view(torch.uint8), wq.view(torch.uint8)
+    ref = co.grouped_gemm_fp8(a8.numpy(), xs.numpy(), w8.numpy(), ws.numpy(), lod_all, act=act)
+    n_out = n // 2 if act else n
+    da, ds, dws = a8.cuda(), xs.contiguous().cuda(), ws.contiguous().cuda()
+    dl = torch.from_numpy(lod).cuda()
+    dw, dwt = torch.empty(E, n, k, dtype=torch.uint8, device="cuda"), torch.empty(1, n, k, dtype=torch.uint8, device="cuda")
+    L.check(L.lib.kmoe_tile_weights_i8(w8[:E].contiguous().cuda().data_ptr(), dw.data_ptr(), E, n, k, L.stream()))
+    L.check(L.lib.kmoe_tile_weights_i8(w8[E:].contiguous().cuda().data_ptr(), dwt.data_ptr(), 1, n, k, L.stream()))
+    y = torch.zeros(rows + tail, n_out, dtype=torch.bfloat16, device="cuda")
+    g = L.GemmFp8Args()
+    g.w_layout = L.KMOE_W_TILED
+    g.a, g.lda, g.a_scale, g.src_div = da.data_ptr(), k, ds.data_ptr(), 1
+    g.w, g.w_scale, g.lod = dw.data_ptr(), dws[:E].contiguous().data_ptr(), dl.data_ptr()
+    ws_tail = dws[E].contiguous()
+    g.w_tail, g.w_scale_tail = dwt.data_ptr(), ws_tail.data_ptr()
+    g.tail_row0, g.tail_rows, g.tail_src0 = rows, tail, rows
+    g.E, g.n, g.k, g.rows = E, n, k, rows
+    g.y, g.ldy, g.act, g.variant = y.data_ptr(), n_out, act, variant
+    L.check(L.lib.kmoe_grouped_gemm_fp8_block(g, L.stream()))
+    torch.cuda.synchronize()
+    want = from_bits(ref)
+    assert rel_l2(y[:rows], want[:rows]) <= 2e-3 if rows else True
+    assert rel_l2(y[rows:], want[rows:]) <= 2e-3
+
+
 FP8_LAYERS = [
     ("fp8-softmax", "qwen3-decode", dict(M=40, H=256, E=16, K=4, I=128)),
     ("fp8-dsv3-shared", "dsv3-decode", dict(M=48, H=512, E=32, K=4, I=256, n_group=4, topk_group=2, I_shared=128)),
     ("fp8-kimi-many-rows", "kimi-decode", dict(M=400, H=256, E=24, K=8, I=128, I_shared=0)),
+    # a shared expert of the routed experts' width: a pass of its own at 5 rows per expert; inside the routed
+    # launches as one more expert at 30 (64-row tiles) and 175 rows per expert (128-row tiles)
+    ("fp8-shared-same-width-few-rows", "dsv3-decode", dict(M=40, H=512, E=32, K=4, I=128, n_group=4, topk_group=2,
+                                                       I_shared=128)),
+    ("fp8-shared-folded-short-tiles", "dsv3-decode", dict(M=120, H=256, E=8, K=2, I=128, n_group=2, topk_group=1,
+                                                          I_shared=128)),
+    ("fp8-shared-folded-tall-tiles", "dsv3-decode", dict(M=700, H=256, E=8, K=2, I=128, n_group=2, topk_group=1,
+                                                         I_shared=128)),
 ]
 
 

@@ -180,6 +180,34 @@ def test_quant_fp8_group128(L, R, Cc):
     assert np.array_equal(q.cpu().numpy(), q_ref)
 
 
+def test_quant_fp8_every_bf16_value(L):
+    """Every finite bf16 value of magnitude <= 448 (both zeros and the subnormals included), each in
+    a group whose absmax is exactly 448, so that the scale is 1 and the value itself is encoded:
+    the conversion instruction against the oracle's nearest-value search, code by code. A second pass
+    with absmax 3.5 (scale 2^-7) puts the small values onto the e4m3 subnormal grid."""
+    allbits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    vals = (allbits.astype(np.uint32) << 16).view(np.float32)
+    for top in (448.0, 3.5):
+        keep = allbits[np.isfinite(vals) & (np.abs(vals) <= top)]
+        rows = -(-keep.size // 127)
+        x = np.zeros((rows, 128), dtype=np.uint16)
+        x[:, 0] = np.array([top], dtype=np.float32).view(np.uint32)[0] >> 16
+        body = np.zeros(rows * 127, dtype=np.uint16)
+        body[:keep.size] = keep
+        x[:, 1:] = body.reshape(rows, 127)
+        q_ref, s_ref = co.quant_fp8_group128(x)
+        assert np.all(s_ref == np.float32(top) / np.float32(448.0))
+        dx = torch.from_numpy(x.view(np.int16)).cuda()
+        q = torch.empty(rows, 128, dtype=torch.uint8, device="cuda")
+        s = torch.empty(rows, 1, dtype=torch.float32, device="cuda")
+        L.check(L.lib.kmoe_quant_fp8_group128(L.ptr(dx), 128, rows, 128, L.ptr(q), 128, L.ptr(s), L.stream()))
+        sync()
+        assert np.array_equal(s.cpu().numpy().view(np.uint32), s_ref.reshape(rows, 1).view(np.uint32))
+        got = q.cpu().numpy()
+        assert np.array_equal(got, q_ref), np.argwhere(got != q_ref)[:5]
+        assert len(np.unique(got & 0x7f)) >= 120  # nearly every code occurs
+
+
 # --------------------------------------------------------------- grouped GEMM
 def _gemm_case(L, E, n, k, counts, act, variant, gather, seed=0):
     """Runs one grouped GEMM on device and returns (y, acc, y_ref, acc_ref)."""

@@ -83,8 +83,15 @@ bool use_stream_path(const kmoe_moe_args* a) {
 // A shared expert of the routed experts' width runs inside the routed GEMM launches
 // as one more ("tail") expert over rows [P, P+M): no extra launches, and its few
 // workgroups overlap the routed experts' instead of leaving most CUs idle.
+// fp8: only where the routed experts run on the tile kernel (more than 10 rows per expert). With fewer
+// rows the routed launch uses the 16-row LDS-staged kernel, which would stream the tail expert's weights once
+// per 16 token rows (measured at 128 tokens: gate_up +260 us against 57 us for a launch of its own).
 bool fold_shared(const kmoe_moe_args* a) {
-  return a->format == KMOE_FMT_INT8 && a->I_shared > 0 && a->I_shared == a->I && a->ws_layout == a->w_layout;
+  if (a->I_shared <= 0 || a->I_shared != a->I || a->ws_layout != a->w_layout) return false;
+  if (a->format == KMOE_FMT_INT8) return true;
+  const long long P = static_cast<long long>(a->M) * a->K;
+  return a->format == KMOE_FMT_FP8_BLOCK && a->w_layout == KMOE_W_TILED && a->H <= 8192 && a->I <= 8192 &&
+         (P + a->E - 1) / a->E > 10;
 }
 
 // One expert-MLP pass (gate_up + SiLU-mul, requantise, down) over `rows` rows in
@@ -107,7 +114,7 @@ struct MlpPass {
   int w_layout;    // KMOE_W_*
   bool stream;     // INT8 + tiled weights: chunk-major codes and the weight-streaming GEMM
   int x_count;     // rows of x_rows (chunk-major addressing)
-  // INT8 tail expert (folded shared expert): rows [rows, rows + tail_rows) of act/actq/out
+  // INT8, FP8 tail expert (folded shared expert): rows [rows, rows + tail_rows) of act/actq/out
   const void *w13_tail, *w2_tail;
   const float *w13_aux_tail, *w2_aux_tail;
   int tail_rows;
@@ -181,6 +188,13 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.ldy = ldy;
     g.act = act;
     g.w_layout = m.w_layout;
+    if (m.tail_rows > 0) {
+      g.w_tail = static_cast<const uint8_t*>(first ? m.w13_tail : m.w2_tail);
+      g.w_scale_tail = first ? m.w13_aux_tail : m.w2_aux_tail;
+      g.tail_row0 = m.rows;
+      g.tail_rows = m.tail_rows;
+      g.tail_src0 = first ? 0 : m.rows;  // gate_up reads token rows, down reads its own act rows
+    }
     return kmoe_grouped_gemm_fp8_block(&g, stream);
   }
   if (m.format == KMOE_FMT_W4A16) {
@@ -237,7 +251,8 @@ int run_mlp(const MlpPass& m, kmoe_stream_t stream, Mark&& mark) {
     rc = m.stream ? kmoe_quant_i8_rows_chunked(m.act, m.I, qrows, m.I, static_cast<int8_t*>(m.actq), m.act_aux, stream)
                   : kmoe_quant_i8_rows(m.act, m.I, qrows, m.I, static_cast<int8_t*>(m.actq), m.I, m.act_aux, stream);
   } else if (m.format == KMOE_FMT_FP8_BLOCK) {
-    rc = kmoe_quant_fp8_group128(m.act, m.I, m.rows, m.I, static_cast<uint8_t*>(m.actq), m.I, m.act_aux, stream);
+    rc = kmoe_quant_fp8_group128(m.act, m.I, m.rows + m.tail_rows, m.I, static_cast<uint8_t*>(m.actq), m.I, m.act_aux,
+                                 stream);
   }
   if (rc) return rc;
   mark(KMOE_STAGE_QUANT2, 1);

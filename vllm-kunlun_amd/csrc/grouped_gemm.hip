@@ -286,7 +286,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
 #pragma unroll
             for (int f = 0; f < NF; ++f) {
               const float sw =
-                  wok[f] ? p.w_max[(static_cast<size_t>(e) * (p.n / 128) + col[f] / 128) * kblocks + kb] : 0.0f;
+                  wok[f] ? w_aux[((tail ? 0 : static_cast<size_t>(e) * (p.n / 128)) + col[f] / 128) * kblocks + kb] : 0.0f;
               v8i wv;
               wv.lo = wcur[f][j][0];
               wv.hi = wcur[f][j][1];
@@ -535,7 +535,12 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
   KMOE_REQUIRE(aligned(a->a, 16) && aligned(a->w, 16) && aligned(a->y, 8), KMOE_ERR_SHAPE,
                "grouped_gemm_fp8_block: misaligned tensor pointer");
   KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_fp8_block: src_div=%d < 1", a->src_div);
-  if (a->rows == 0) return KMOE_OK;
+  KMOE_REQUIRE(!a->w_tail || (a->w_scale_tail && a->tail_rows >= 0 && a->tail_row0 >= 0 && a->tail_src0 >= 0 &&
+                              aligned(a->w_tail, 16)),
+               KMOE_ERR_SHAPE, "grouped_gemm_fp8_block: bad tail expert (w_scale_tail, tail_row0=%d, tail_rows=%d)",
+               a->tail_row0, a->tail_rows);
+  const int tail_rows = a->w_tail ? a->tail_rows : 0;
+  if (a->rows == 0 && tail_rows == 0) return KMOE_OK;
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR || a->w_layout == KMOE_W_TILED, KMOE_ERR_UNSUPPORTED,
                "grouped_gemm_fp8_block: w_layout=%d unknown", a->w_layout);
   // tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5, 6, 11 force it)
@@ -546,6 +551,7 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), a->w_scale, a->lod,  a->E,       a->n,
                a->k,                                  a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,
-               nullptr, nullptr, 0, 0, 0, nullptr, 0, 0.f, 0.f};
+               reinterpret_cast<const int8_t*>(a->w_tail), a->w_scale_tail, a->tail_row0, tail_rows, a->tail_src0,
+               nullptr, 0, 0.f, 0.f};
   return dispatch<Kind::FP8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_fp8_block");
 }

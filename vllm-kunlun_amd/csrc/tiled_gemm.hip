@@ -773,11 +773,15 @@ int tiled_common(const TiledParams& p, int rows, int* n_cu_out, const char* what
 // the CU to it (measured, int8 gate_up / down: Qwen3 shape at 32 rows per expert 101 -> 80 us; DeepSeek-V3 shape
 // at 32 rows 1426 -> 1284 / 770 -> 683 us). At 64 rows per expert half of the experts need a second tile and
 // a second pass over their weights: DeepSeek-V3 gate_up 1434 -> 1585 us, so the switch sits below that.
+// Also when 128-row tiles would leave most workgroups without an item (a dense GEMM of a few hundred rows: one
+// expert, fp8 [rows,7168] x [4096,7168]: 102 -> 57 us at 128 rows, 105 -> 62 us at 1024, 150 -> 163 us at 4096).
 // Variant 6 forces 128 rows, 11 forces 64.
-bool short_tiles(int variant, int rows, int n_experts, int max_avg_rows = 48) {
+bool short_tiles(int variant, int rows, int n_experts, int n, bool swiglu, int n_cu, int max_avg_rows = 48) {
   if (variant == 11) return true;
   if (variant == 6) return false;
-  return ceil_div(rows, n_experts) <= max_avg_rows;
+  if (ceil_div(rows, n_experts) <= max_avg_rows) return true;
+  const int n_blocks = ceil_div(swiglu ? n / 2 : n, kWavesT * (swiglu ? 2 : 4) * 16);
+  return static_cast<long long>(rows / 128 + n_experts) * n_blocks < 2ll * n_cu;
 }
 
 }  // namespace
@@ -809,7 +813,7 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   if (a->variant == 9)
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what);
-  if (short_tiles(a->variant, a->rows, a->E))
+  if (short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu))
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)
@@ -824,11 +828,14 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
   KMOE_REQUIRE(a->k / 128 <= kMaxKBlocks, KMOE_ERR_UNSUPPORTED, "%s: k=%d > %d", what, a->k, 128 * kMaxKBlocks);
   TiledParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,
                 reinterpret_cast<const int8_t*>(a->w), a->w_scale, a->lod, a->E, a->n, a->k, a->y, a->ldy, nullptr,
-                nullptr, nullptr, 0, 0, 0, 0, 0};
+                reinterpret_cast<const int8_t*>(a->w_tail), a->w_scale_tail, a->tail_row0,
+                a->w_tail ? a->tail_rows : 0, a->tail_src0, 0, 0};
   int n_cu = 0;
   if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
   constexpr TKind K = TKind::F8;
-  if (short_tiles(a->variant, a->rows, a->E))
+  // (64x128 tiles for a dense GEMM of a few rows, twice the work items: 57 -> 42 us on [128,7168] x [4096,7168],
+  // still bound by what one workgroup keeps in flight; not instantiated)
+  if (short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu))
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)
@@ -846,7 +853,7 @@ int tiled_gemm_bf16(const kmoe_gemm_bf16_args* a, hipStream_t s) {
   int n_cu = 0;
   if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
   constexpr TKind K = TKind::BF16;
-  if (short_tiles(a->variant, a->rows, a->E, 40))  // measured: at 48 rows per expert the 128-row tiles are 4 % ahead
+  if (short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu, 40))  // measured: at 48 rows per expert the 128-row tiles are 4 % ahead
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)

@@ -69,6 +69,8 @@ class GemmFp8Args(C.Structure):
         ("E", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("rows", C.c_int32),
         ("y", C.c_void_p), ("ldy", C.c_int64), ("act", C.c_int32), ("variant", C.c_int32),
         ("w_layout", C.c_int32),
+        ("w_tail", C.c_void_p), ("w_scale_tail", C.c_void_p),
+        ("tail_row0", C.c_int32), ("tail_rows", C.c_int32), ("tail_src0", C.c_int32),
     ]
 
 

@@ -1,0 +1,113 @@
+"""The dense W8A8 linear kernel class (reference: quantization/kernels/scale_mm.py:30-90): what
+process_weights_after_loading leaves on the layer (CPU), and apply_weights against the oracle's
+quantise -> int8 GEMM -> rescale on the GPU, bit for bit."""
+import os
+import sys
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (ROOT, os.path.join(ROOT, "vllm-kunlun_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+from conftest import bits, from_bits  # noqa: E402
+from oracle import c_oracle as co  # noqa: E402
+from oracle import torch_moe as tm  # noqa: E402
+
+
+def _layer(n, k, device, seed):
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(n, k, generator=g) * 0.05
+    wq, scale = tm.quantize_weight_per_channel(w)  # int8 [n,k], scale [n,1] as a checkpoint stores it
+    layer = SimpleNamespace(weight=torch.nn.Parameter(wq.to(device), requires_grad=False),
+                            weight_scale=torch.nn.Parameter(scale.clone().to(device), requires_grad=False),
+                            input_scale=None)
+    return layer, wq, (scale * 127.0).reshape(n)  # the absmax the kernels take
+
+
+def test_process_weights_after_loading_on_the_host():
+    from vllm_kunlun_amd.quantization.kernels.scale_mm import (Int8ScaledMMLinearLayerConfig,
+                                                               KunlunScaledMMLinearKernel)
+    layer, wq, w_max = _layer(48, 96, "cpu", 0)
+    scale_before = layer.weight_scale.data.clone()
+    kern = KunlunScaledMMLinearKernel(Int8ScaledMMLinearLayerConfig())
+    kern.process_weights_after_loading(layer)
+    # scale -> absmax: x 127 (scale_mm.py:43-50); one f32 per output channel
+    assert torch.equal(layer.weight_scale.data, scale_before * 127.0)
+    assert layer.weight_scale.shape == (48, 1) and layer.weight_scale.dtype == torch.float32
+    # the base class leaves the weight as the [k, n] transpose view of its [n, k] storage
+    assert layer.weight.shape == (96, 48)
+    assert torch.equal(layer.weight.data.t(), wq)  # not a HIP tensor: stays row-major
+    assert layer.input_scale is None and layer.input_zero_point is None and layer.azp_adj is None
+    # a per-tensor scale becomes one per channel
+    layer2, _, _ = _layer(32, 64, "cpu", 1)
+    layer2.weight_scale = torch.nn.Parameter(torch.tensor([0.25]), requires_grad=False)
+    kern.process_weights_after_loading(layer2)
+    assert torch.equal(layer2.weight_scale.data, torch.full((32, 1), 0.25 * 127.0))
+    # schemes outside the path are refused by name
+    ok, why = KunlunScaledMMLinearKernel.can_implement(Int8ScaledMMLinearLayerConfig(is_static_input_scheme=True))
+    assert not ok and "static" in why
+    ok, why = KunlunScaledMMLinearKernel.can_implement(Int8ScaledMMLinearLayerConfig(input_symmetric=False))
+    assert not ok and "asymmetric" in why
+    with pytest.raises(ValueError):
+        bad, _, _ = _layer(16, 64, "cpu", 2)
+        bad.weight_scale = torch.nn.Parameter(torch.ones(5), requires_grad=False)
+        kern.process_weights_after_loading(bad)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,n,k", [(1, 64, 128), (37, 256, 512), (128, 512, 1024), (700, 256, 256),
+                                   (5, 48, 80)])  # the last one does not tile: row-major weights
+def test_apply_weights_matches_the_oracle(M, n, k):
+    from vllm_kunlun_amd import _plan
+    from vllm_kunlun_amd.quantization.kernels.scale_mm import KunlunScaledMMLinearKernel
+    layer, wq, w_max = _layer(n, k, "cuda", M + n + k)
+    kern = KunlunScaledMMLinearKernel()
+    kern.process_weights_after_loading(layer)
+    assert _plan.is_tiled(layer._kmoe_w_1nk) == (n % 16 == 0 and k % 64 == 0)
+    g = torch.Generator().manual_seed(M)
+    x = (torch.randn(3, M, k, generator=g) * 1.5).bfloat16()  # leading dimensions are flattened
+    out = kern.apply_weights(layer, x.cuda())
+    torch.cuda.synchronize()
+    assert out.shape == (3, M, n) and out.dtype == torch.bfloat16
+    xq, x_max = co.quant_i8_rows(bits(x.reshape(-1, k)))
+    lod = np.array([0, 3 * M], dtype=np.int32)
+    ref, _ = co.grouped_gemm_i8(xq, x_max, wq.numpy()[None], w_max.numpy()[None], lod)
+    assert np.array_equal(bits(out.reshape(-1, n)), ref)
+    with pytest.raises(NotImplementedError):
+        kern.apply_weights(layer, x.cuda(), bias=torch.zeros(n, device="cuda"))
+
+
+@pytest.mark.gpu
+def test_shared_expert_mlp_through_two_linears():
+    """The shared expert as the model code runs it (deepseek_v2.py:280-296 in the reference's tree:
+    gate_up_proj, silu_and_mul, down_proj): the same bits as the dense MLP of the oracle."""
+    import vllm_kunlun_amd  # noqa: F401
+    from vllm_kunlun_amd.quantization.kernels.scale_mm import KunlunScaledMMLinearKernel
+    M, H, I = 96, 512, 256
+    up, w13q, w13_max = _layer(2 * I, H, "cuda", 11)
+    down, w2q, w2_max = _layer(H, I, "cuda", 12)
+    kern = KunlunScaledMMLinearKernel()
+    kern.process_weights_after_loading(up)
+    kern.process_weights_after_loading(down)
+    x = (torch.randn(M, H, generator=torch.Generator().manual_seed(13)) * 1.5).bfloat16()
+    y = kern.apply_weights(up, x.cuda())
+    act = torch.empty(M, I, dtype=torch.bfloat16, device="cuda")
+    torch.ops._C.silu_and_mul(act, y)
+    out = kern.apply_weights(down, act)
+    torch.cuda.synchronize()
+    lod = np.array([0, M], dtype=np.int32)
+    xq, x_max = co.quant_i8_rows(bits(x))
+    y_ref, _ = co.grouped_gemm_i8(xq, x_max, w13q.numpy()[None], w13_max.numpy()[None], lod)
+    a_ref = co.silu_and_mul(y_ref)
+    aq, a_max = co.quant_i8_rows(a_ref)
+    ref, _ = co.grouped_gemm_i8(aq, a_max, w2q.numpy()[None], w2_max.numpy()[None], lod)
+    assert np.array_equal(bits(y), y_ref)
+    assert np.array_equal(bits(out), ref)
+    # and the torch restatement of the reference's two scaled_int8_quant -> matmul steps agrees within bf16 rounding
+    t_ref = tm.w8a8_dense(x, w13q, w13_max.reshape(-1, 1), w2q, w2_max.reshape(-1, 1))
+    assert (out.cpu().float() - t_ref.float()).norm() / t_ref.float().norm() <= 1e-2

@@ -3,7 +3,8 @@ through 256 experts in test time, so the large batches are held to what does not
 size: every token's result is independent of the batch it travels in. That gives, bit for bit,
   * permutation equivariance: shuffling the tokens shuffles the outputs;
   * batch-size independence: a token gets the same bits in a decode batch (weight-streaming
-    kernels, chunk-major codes, fused prologue) as in a prefill batch (persistent tile kernel);
+    kernels, chunk-major codes, fused prologue) as in a prefill batch (persistent tile kernel), and in
+    the batches in between, on either side of every switch of kernel and tile height;
   * a spot check: a handful of tokens of the big batch through the C oracle.
 The decode batches are compared with the C oracle in full."""
 import numpy as np
@@ -50,7 +51,7 @@ def dsv3():
     return sl, sl.host_weights()
 
 
-def _properties(sl, host, n_decode, n_spot, seed):
+def _properties(sl, host, n_decode, n_spot, seed, mids=()):
     g = torch.Generator(device="cuda").manual_seed(seed)
     x, logits = sl.x, sl.logits
     M = x.shape[0]
@@ -65,6 +66,11 @@ def _properties(sl, host, n_decode, n_spot, seed):
     assert torch.equal(dec, full[:n_decode]), "decode and prefill kernels disagree"
     ref = _oracle(sl, host, x[:n_decode], logits[:n_decode])
     assert np.array_equal(bits(dec), ref), "decode batch vs C oracle"
+    # batches in between: the streaming kernels' last sizes, the tile kernel on 64-row tiles, on 128-row
+    # tiles that are mostly padding
+    for m in mids:
+        mid = _run(sl, x[:m].contiguous(), logits[:m].contiguous())
+        assert torch.equal(mid, full[:m]), f"a batch of {m} tokens disagrees with the full batch"
     # spot check of the big batch: random tokens through the oracle
     idx = torch.randperm(M, generator=g, device="cuda")[:n_spot]
     ref_spot = _oracle(sl, host, x[idx], logits[idx])
@@ -74,7 +80,7 @@ def _properties(sl, host, n_decode, n_spot, seed):
 def test_qwen3_full_size(qwen3):
     """Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, intermediate 768; 8192 and 64 tokens."""
     sl, host = qwen3
-    _properties(sl, host, n_decode=64, n_spot=48, seed=1)
+    _properties(sl, host, n_decode=64, n_spot=48, seed=1, mids=(160, 176, 512, 768, 800, 1500))
 
 
 def test_qwen3_full_size_skewed_routing(qwen3):
@@ -91,7 +97,7 @@ def test_dsv3_full_size(dsv3):
     """DeepSeek-V3 shape: 256 experts + shared, sigmoid grouped top-8, hidden 7168, intermediate 2048;
     4096 and 128 tokens."""
     sl, host = dsv3
-    _properties(sl, host, n_decode=128, n_spot=16, seed=2)
+    _properties(sl, host, n_decode=128, n_spot=16, seed=2, mids=(320, 352, 1024, 1536, 1600))
 
 
 def test_dsv3_fp8_full_size_sample_against_the_oracle():

@@ -231,20 +231,45 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   const int seg = (n_items + 7) >> 3;
   const int xcd = blockIdx.x & 7;
   const int seg_end = min((xcd + 1) * seg, n_items);
+  // The items of this workgroup are resolved 64 at a time: lane l of wave 0 finds item it0 + l (a binary
+  // search over tile_lo and two divisions, all lanes at once) and leaves (expert, first row, channel
+  // block) in LDS; the tile loop then reads three words per tile instead of searching.
+  __shared__ int item_e[kWave], item_row0[kWave], item_nb[kWave];
+  auto resolve_items = [&](int it0) {
+    if (wave_id == 0) {
+      const int lid = xcd * seg + (blockIdx.x >> 3) + (it0 + lane) * (gridDim.x >> 3);  // gridDim.x is a multiple of 8
+      int e = -1, row0 = 0, nb = 0;
+      if (lid < seg_end) {
+        const int m_tile = lid / p.n_blocks;
+        // the last e with tile_lo[e] <= m_tile: of a run of equal entries (empty experts) the one that owns the tile
+        int lo = 0, hi = n_exp - 1;
+        while (lo < hi) {
+          const int mid = (lo + hi + 1) >> 1;
+          if (tile_lo[mid] <= m_tile) lo = mid;
+          else hi = mid - 1;
+        }
+        e = lo;
+        const int first = tile_lo[e], mt = tile_lo[e + 1] - first;
+        const int u = lid - first * p.n_blocks;
+        nb = u / mt;
+        row0 = rows_begin(e) + (u - nb * mt) * kTM;
+      }
+      item_e[lane] = e;
+      item_row0[lane] = row0;
+      item_nb[lane] = nb;
+    }
+    __syncthreads();
+  };
+  resolve_items(0);
+  // (called by every wave at the same point of the tile loop: the refill every 64 tiles has a barrier inside)
   auto find_tile = [&](int it) -> Tile {
+    if (it > 0 && (it & (kWave - 1)) == 0) resolve_items(it);
     Tile t{it, 0, 0, 0, false};
-    const int lid = xcd * seg + (blockIdx.x >> 3) + it * (gridDim.x >> 3);  // gridDim.x is a multiple of 8
-    if (lid >= seg_end) return t;
-    const int m_tile = lid / p.n_blocks;  // tile_lo[e] <= m_tile < tile_lo[e + 1] <=> the item belongs to e
-    int found = -1;
-    for (int e = lane; e < n_exp; e += kWave)
-      if (tile_lo[e] <= m_tile && m_tile < tile_lo[e + 1]) found = e;
-    const uint64_t who = __ballot(found >= 0);  // exactly one lane
-    t.e = __builtin_amdgcn_readfirstlane(__shfl(found, __builtin_ctzll(who), kWave));
-    const int first = tile_lo[t.e], mt = tile_lo[t.e + 1] - first;
-    const int u = lid - first * p.n_blocks;
-    t.nb = u / mt;
-    t.row0 = __builtin_amdgcn_readfirstlane(rows_begin(t.e) + (u - t.nb * mt) * kTM);
+    const int slot = it & (kWave - 1);
+    t.e = __builtin_amdgcn_readfirstlane(item_e[slot]);
+    if (t.e < 0) return t;
+    t.row0 = __builtin_amdgcn_readfirstlane(item_row0[slot]);
+    t.nb = __builtin_amdgcn_readfirstlane(item_nb[slot]);
     t.valid = true;
     return t;
   };

@@ -176,8 +176,8 @@ def vendor_dense_gemm(shape, g1_ops, peak_tops, reps=20):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="qwen3-decode", choices=sorted(WORKLOAD_LABEL))
     ap.add_argument("--launch", default="graph", choices=["graph", "eager"],
                     help="replay the layer from a captured HIP graph (as a serving engine does) or launch it eagerly")

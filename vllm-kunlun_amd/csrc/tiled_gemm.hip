@@ -129,7 +129,7 @@ struct Tile {
 // NF: 16-channel fragments per wave (4: 256-channel tiles, 2: 128-channel tiles);
 // R: weight ring slots (R - 1 MFMA steps of weights in flight per wave), 4 or 8;
 // WGS: workgroups per CU the register budget is cut for.
-// <4,4,2> is the shape in use; <2,8,3> trades operand reuse for more waves and more bytes
+// <4,4,2> is the shape in use; <2,8,2> trades operand reuse for narrower tiles and more bytes
 // in flight (a tuning variant).
 // WM: rows of waves. 1: 128-row tiles, 4 waves; 2: 256-row tiles, 8 waves, where the two waves
 // that share channels read the same weight bytes within one barrier interval (an expert with
@@ -812,7 +812,7 @@ bool short_tiles(int variant, int rows, int n_experts, int n, bool swiglu, int n
 }  // namespace
 
 // variant 5: 128x256 or 64x256 tiles by the rows per expert (6, 11: one of them), 4-slot weight ring, 2 workgroups
-// per CU (the shape in use); 7: 128x128 tiles, 8-slot ring, 3 workgroups per CU; 8: 256x256 tiles, 8 waves,
+// per CU (the shape in use); 7: 128x128 tiles, 8-slot ring; 8: 256x256 tiles, 8 waves,
 // 1 workgroup per CU; 9: 128x256 tiles on the 32x32 MFMA shapes
 int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   const char* what = "kmoe_grouped_gemm_i8 (tiled)";
@@ -824,20 +824,20 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
   constexpr TKind K = TKind::I8;
   // The 128-channel / deep-ring shape is a tuning variant only: measured slower than the
-  // 256-channel shape also when an expert has ~128 rows (DeepSeek-V3 prefill at 4096 tokens),
-  // where HBM traffic, not bytes in flight, is the limit (twice the workgroups re-read A).
+  // 256-channel shape (Qwen3 gate_up 321 vs 299 us, DeepSeek-V3 at 4096 tokens 2292 vs 1913 us):
+  // twice the workgroups re-read the activations.
   if (a->variant == 7)
-    return swiglu ? launch_tiled<K, true, 2, 8, 3, 1>(p, a->rows, s, n_cu, what)
-                  : launch_tiled<K, false, 2, 8, 3, 1>(p, a->rows, s, n_cu, what);
+    return swiglu ? launch_tiled<K, true, 2, 8, 2, 1>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 2, 8, 2, 1>(p, a->rows, s, n_cu, what);
   // 256-row tiles bring DeepSeek-V3 prefill (128-256 rows per expert) down to its algorithmic HBM
   // traffic (measured 1.04x against 1.44x), but one workgroup per CU has nothing to run under its
   // epilogue and tile switch: 3.7 TB/s, 13 % slower overall. Kept as a tuning variant.
   if (a->variant == 8)
     return swiglu ? launch_tiled<K, true, 4, 4, 1, 2>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 1, 2>(p, a->rows, s, n_cu, what);
-  if (a->variant == 9)
-    return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what)
-                  : launch_tiled<K, false, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what);
+  // (the 32x32 shapes are instantiated for the gate_up launch only: without SiLU-mul the 16-register
+  // fragments of the plain epilogue do not fit two workgroups per CU)
+  if (a->variant == 9 && swiglu) return launch_tiled<K, true, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what);
   if (short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu))
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);

@@ -179,8 +179,9 @@ def main():
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="qwen3-decode", choices=sorted(WORKLOAD_LABEL))
-    ap.add_argument("--launch", default="graph", choices=["graph", "eager"],
-                    help="replay the layer from a captured HIP graph (as a serving engine does) or launch it eagerly")
+    ap.add_argument("--launch", default="auto", choices=["auto", "graph", "eager"],
+                    help="replay the layer from a captured HIP graph (as a serving engine does), launch it eagerly, "
+                         "or (auto) time K steps each way and report the faster; config.launch says which")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--tokens", type=int, default=0,
@@ -247,22 +248,26 @@ def main():
         for _ in range(3):
             plan()
         stream.synchronize()
-        graph = None
-        if a.launch == "graph":
+        def timed(step):
+            for _ in range(a.warmup):
+                step()
+            stream.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(a.steps):
+                step()
+            stream.synchronize()
+            return (time.perf_counter() - t0) * 1e3 / a.steps
+
+        launch_ms = {}
+        if a.launch in ("auto", "graph"):
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
                 plan()
-        step = graph.replay if graph is not None else plan
-
-        for _ in range(a.warmup):
-            step()
-        stream.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(a.steps):
-            step()
-        stream.synchronize()
-        wall = time.perf_counter() - t0
-        ms_per_step = wall * 1e3 / a.steps
+            launch_ms["hipgraph replay"] = timed(graph.replay)
+        if a.launch in ("auto", "eager"):
+            launch_ms["eager"] = timed(plan)
+        launch_mode = min(launch_ms, key=launch_ms.get)
+        ms_per_step = launch_ms[launch_mode]
 
         # the same calls again with HIP events around each stage (eager: events are
         # not captured), for the per-kernel durations of the roofline
@@ -317,7 +322,7 @@ def main():
         "config": {"workload": label, "name": a.workload, "tokens": shape.M, "hidden": shape.H,
                    "experts": shape.E, "top_k": shape.K, "moe_intermediate": shape.I,
                    "shared_intermediate": shape.I_shared, "routing": shape.scoring, "experts_hit": n_active,
-                   "launch": "hipgraph replay" if graph is not None else "eager", "seed": a.seed,
+                   "launch": launch_mode, "launch_ms_per_step": launch_ms, "seed": a.seed,
                    "router_gemm_inside": bool(a.router)},
         "roofline": roofline,
         "layer": {"hbm_gbs": work["layer_bytes"] / t_s / 1e9, "hbm_frac": work["layer_bytes"] / t_s / 1e9 / HBM_PEAK_GBS,

@@ -31,6 +31,8 @@ WORKLOAD_LABEL = {
     "qwen3-prefill-skew": "Qwen3-MoE-30B-A3B-shape MoE layer, W8A8 int8, prefill, 8192 tokens, +2.0 logit bias on 8 experts",
     "dsv3-decode": "DeepSeek-V3-shape MoE layer (+1 shared expert), W8A8 int8, decode, 128 tokens",
     "dsv3-prefill": "DeepSeek-V3-shape MoE layer (+1 shared expert), W8A8 int8, prefill, 4096 tokens",
+    "kimi-decode": "Kimi-K2-shape MoE layer (384 experts, +1 shared), W8A8 int8, decode, 128 tokens",
+    "kimi-prefill": "Kimi-K2-shape MoE layer (384 experts, +1 shared), W8A8 int8, prefill, 4096 tokens",
     "dsv3-fp8-decode": "DeepSeek-V3-shape MoE layer (+1 shared expert), fp8-e4m3 128x128-block weights, decode, 128 tokens",
     "dsv3-fp8-prefill": "DeepSeek-V3-shape MoE layer (+1 shared expert), fp8-e4m3 128x128-block weights, prefill, 4096 tokens",
     "kimi-fp8-decode": "Kimi-K2-shape MoE layer (384 experts, +1 shared), fp8-e4m3 128x128-block weights, decode, 128 tokens",

@@ -8,9 +8,10 @@ few pieces of that base it relies on (the parameter names and what the base's
 `process_weights_after_loading` leaves behind: the weight as the [k, n] transpose view of its
 [n, k] storage, a per-channel weight scale, no input scale for dynamic quantisation).
 
-Path taken by `apply_weights`: per-token absmax int8 quantisation (`_C::scaled_int8_quant`) and the
-one-expert case of the grouped int8 GEMM on the weights re-arranged at load time into the MFMA
-tiles (`kmoe_grouped_gemm_i8`), the same kernels the fused MoE layer runs its shared expert on.
+Path taken by `apply_weights`: per-token absmax int8 quantisation and the grouped int8 GEMM
+(`kmoe_grouped_gemm_i8`) on the weights re-arranged at load time into the MFMA tiles - for up to 256
+rows as the tail expert of the weight-streaming kernel, beyond as its one-expert case on the tile
+kernel: the same kernels the fused MoE layer runs its shared expert on.
 """
 from __future__ import annotations
 
@@ -112,12 +113,45 @@ class KunlunScaledMMLinearKernel:
         from ...ops import _custom_ops as ops  # registers torch.ops._C.*
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1]).contiguous()
-        M, n = x2.shape[0], w.shape[1]
+        M, n, k = x2.shape[0], w.shape[1], w.shape[2]
         out = torch.empty((M, n), dtype=x.dtype, device=x.device)
-        if M:
+        if M == 0:
+            return out.reshape(*lead, n)
+        if is_tiled(w) and M <= self.STREAM_MAX_ROWS:
+            self._stream_gemm(x2, w, w_s.data.reshape(-1), out)
+        else:
             x_q, x_max, _, _ = torch.ops._C.scaled_int8_quant(x2, None, None, True)
-            key = (x.device, M)
-            if key not in self._lod:
-                self._lod[key] = torch.tensor([0, M], dtype=torch.int32).to(x.device)
-            ops._gemm_i8(x_q, x_max, w, w_s.data.reshape(-1), self._lod[key], out, n, L.KMOE_ACT_NONE, M)
+            ops._gemm_i8(x_q, x_max, w, w_s.data.reshape(-1), self._row_range(x.device, M), out, n, L.KMOE_ACT_NONE, M)
         return out.reshape(*lead, n)
+
+    # Up to this many rows the GEMM runs on the weight-streaming kernel (the one the fused MoE layer
+    # runs decode batches and its folded shared expert on): the dense matrix is handed over as the
+    # launch's "tail expert", whose rows the kernel cuts into slices of 16 or 32 for as many
+    # workgroups - a tile kernel has too few tiles to fill the chip here. Measured on
+    # [M,7168] x [4096,7168]: 16 us against 36 us at 16 rows, 25 against 38 at 128, 31 against 38 at 256;
+    # at 512 rows the tile kernel is ahead (39 against 46 us).
+    STREAM_MAX_ROWS = 256
+
+    def _row_range(self, device, rows):
+        key = (device, rows)
+        if key not in self._lod:
+            self._lod[key] = torch.tensor([0, rows], dtype=torch.int32).to(device)
+        return self._lod[key]
+
+    def _stream_gemm(self, x2, w, w_max, out):
+        M, k = x2.shape
+        n = w.shape[1]
+        x_q = torch.empty((k // 64, M, 64), dtype=torch.int8, device=x2.device)  # chunk-major codes
+        x_max = torch.empty((M,), dtype=torch.float32, device=x2.device)
+        L.check(L.lib.kmoe_quant_i8_rows_chunked(L.ptr(x2), k, M, k, L.ptr(x_q), L.ptr(x_max), L.stream()))
+        g = L.GemmI8Args()
+        g.a, g.lda, g.a_max, g.src_div = x_q.data_ptr(), k, x_max.data_ptr(), 1
+        g.a_layout, g.a_rows = L.KMOE_A_CHUNKED, M
+        # one routed expert without rows (the launch needs an expert list), the matrix as the tail expert
+        g.w, g.w_max, g.lod = w.data_ptr(), w_max.data_ptr(), self._row_range(x2.device, 0).data_ptr()
+        g.E, g.n, g.k, g.rows = 1, n, k, 0
+        g.w_tail, g.w_max_tail = w.data_ptr(), w_max.data_ptr()
+        g.tail_row0, g.tail_rows, g.tail_src0 = 0, M, 0
+        g.y, g.ldy, g.act, g.w_layout = out.data_ptr(), n, L.KMOE_ACT_NONE, L.KMOE_W_TILED
+        g.variant = 1 if M <= 128 else 2  # 16 or 32 rows per slice
+        L.check(L.lib.kmoe_grouped_gemm_i8(g, L.stream()))

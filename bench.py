@@ -191,6 +191,9 @@ def main():
     ap.add_argument("--router", action="store_true",
                     help="hand the layer the bf16 gate weight [E,H] instead of router logits: the router GEMM "
                          "then runs inside each step (reported in config; not the default workload)")
+    ap.add_argument("--dims", default="",
+                    help="other layer dimensions for the workload's format and routing, e.g. "
+                         "H=4096,E=8,K=2,I=14336,I_shared=0 (Mixtral-8x7B); the config then says so")
     ap.add_argument("--yardstick", action="store_true",
                     help="also time the vendor library's dense GEMM (torch._int_mm / bf16 matmul) with the gate_up "
                          "GEMM's operation count: [P,H] x [H,2I], one weight matrix, no gather, no epilogue")
@@ -211,6 +214,17 @@ def main():
     if a.tokens and a.tokens != shape.M:
         shape = synth.scaled(shape, M=a.tokens)
         label = re.sub(r"(decode|prefill), \d+ tokens", f"{a.tokens} tokens (batch set by --tokens)", label)
+    if a.dims:
+        allowed = {"H": int, "E": int, "K": int, "I": int, "I_shared": int, "n_group": int, "topk_group": int,
+                   "scoring": str, "routed_scale": float}
+        over = {}
+        for item in a.dims.split(","):
+            key, _, val = item.partition("=")
+            if key not in allowed:
+                sys.exit(f"bench.py: --dims takes {sorted(allowed)}, not {key!r}")
+            over[key] = allowed[key](val)
+        shape = synth.scaled(shape, **over)
+        label = f"MoE layer with --dims {a.dims} on the format and routing of {a.workload}, {shape.M} tokens"
     from vllm_kunlun_amd._plan import make_moe_plan
     sl = synth.make_layer(shape, "cuda:0", seed=a.seed)
     lay = sl.layer
@@ -292,7 +306,7 @@ def main():
     peak_tops = PEAK_TOPS[shape.quant]
     hbm_bound = intensity < peak_tops * 1e12 / (HBM_PEAK_GBS * 1e9)
     g1_s = stage_ms["gemm1"] * 1e-3
-    traffic = None if a.tokens else measured_traffic(a.workload)  # the counter summaries are of the named batch
+    traffic = None if (a.tokens or a.dims) else measured_traffic(a.workload)  # the counter summaries are of the named workload
     if hbm_bound:
         achieved = work["g1_bytes"] / g1_s / 1e9
         roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",

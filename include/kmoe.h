@@ -126,7 +126,7 @@ int kmoe_gather_rows(const uint16_t* src, int64_t ld_src,
  * through _C.scaled_int8_quant, ops/_custom_ops.py:1633-1657).
  *   x [R,C] bf16 -> q [R,C] i8, row_max [R] f32 (absmax of the row);
  *   q = clamp(rne(x * (127 / row_max)), -127, 127); an all-zero row gives q=0, max=0.
- * Limits: C % 8 == 0, C <= 16384, ld_x % 8 == 0, ld_q % 8 == 0.
+ * Limits: C % 8 == 0, C <= 65536, ld_x % 8 == 0, ld_q % 8 == 0.
  */
 int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q,
                        int64_t ld_q, float* row_max, kmoe_stream_t stream);

@@ -145,7 +145,7 @@ def test_gather_rows(L):
 
 # -------------------------------------------------------------------- quant
 @pytest.mark.parametrize("R,Cc", [(1, 8), (5, 256), (64, 2048), (100, 768), (33, 7168), (3, 16384), (7, 1000),
-                                  (512, 2048)])
+                                  (512, 2048), (5, 20480), (2, 65536)])
 def test_quant_i8_rows(L, R, Cc):
     torch.manual_seed(R + Cc)
     x = (torch.randn(R, Cc) * torch.rand(R, 1) * 4).bfloat16()
@@ -351,7 +351,7 @@ def test_tile_weights(L, E, n, k):
     assert L.lib.kmoe_tile_weights_i8(L.ptr(src), L.ptr(src), E, n, k, L.stream()) == -2  # in place is refused
 
 
-@pytest.mark.parametrize("R,Cc", [(1, 64), (64, 2048), (100, 768), (33, 7168), (512, 2048)])
+@pytest.mark.parametrize("R,Cc", [(1, 64), (64, 2048), (100, 768), (33, 7168), (512, 2048), (5, 20480), (2, 65536)])
 def test_quant_i8_rows_chunked(L, R, Cc):
     torch.manual_seed(R + Cc)
     x = (torch.randn(R, Cc) * 3).bfloat16()

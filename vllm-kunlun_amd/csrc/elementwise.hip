@@ -197,8 +197,14 @@ int quant_i8_launch(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, in
   } else if (C <= 256 * 8 * 4) {
     hipLaunchKernelGGL((quant_i8_rows_kernel<256, 4>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max,
                        chunked);
-  } else {
+  } else if (C <= 256 * 8 * 8) {
     hipLaunchKernelGGL((quant_i8_rows_kernel<256, 8>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max,
+                       chunked);
+  } else if (C <= 256 * 8 * 16) {
+    hipLaunchKernelGGL((quant_i8_rows_kernel<256, 16>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max,
+                       chunked);
+  } else {  // up to 65536 values: 128 registers of row data per thread
+    hipLaunchKernelGGL((quant_i8_rows_kernel<256, 32>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max,
                        chunked);
   }
   return check_launch(what);
@@ -208,8 +214,8 @@ int quant_i8_launch(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, in
 extern "C" int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q,
                                   float* row_max, kmoe_stream_t stream) {
   KMOE_REQUIRE(x && q && row_max, KMOE_ERR_NULL, "quant_i8_rows: NULL pointer");
-  KMOE_REQUIRE(R >= 0 && C >= 8 && C % 8 == 0 && C <= 16384, KMOE_ERR_SHAPE,
-               "quant_i8_rows: R=%d C=%d (need C %% 8 == 0, 8 <= C <= 16384)", R, C);
+  KMOE_REQUIRE(R >= 0 && C >= 8 && C % 8 == 0 && C <= 65536, KMOE_ERR_SHAPE,
+               "quant_i8_rows: R=%d C=%d (need C %% 8 == 0, 8 <= C <= 65536)", R, C);
   KMOE_REQUIRE(ld_x % 8 == 0 && ld_q % 8 == 0 && ld_x >= C && ld_q >= C, KMOE_ERR_SHAPE,
                "quant_i8_rows: row strides %lld/%lld must be multiples of 8 and >= C", (long long)ld_x,
                (long long)ld_q);
@@ -220,8 +226,8 @@ extern "C" int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C,
 extern "C" int kmoe_quant_i8_rows_chunked(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, float* row_max,
                                           kmoe_stream_t stream) {
   KMOE_REQUIRE(x && q && row_max, KMOE_ERR_NULL, "quant_i8_rows_chunked: NULL pointer");
-  KMOE_REQUIRE(R >= 0 && C >= 64 && C % 64 == 0 && C <= 16384, KMOE_ERR_SHAPE,
-               "quant_i8_rows_chunked: R=%d C=%d (need C %% 64 == 0, 64 <= C <= 16384)", R, C);
+  KMOE_REQUIRE(R >= 0 && C >= 64 && C % 64 == 0 && C <= 65536, KMOE_ERR_SHAPE,
+               "quant_i8_rows_chunked: R=%d C=%d (need C %% 64 == 0, 64 <= C <= 65536)", R, C);
   KMOE_REQUIRE(ld_x % 8 == 0 && ld_x >= C, KMOE_ERR_SHAPE,
                "quant_i8_rows_chunked: row stride %lld must be a multiple of 8 and >= C", (long long)ld_x);
   if (R == 0) return KMOE_OK;

@@ -53,6 +53,14 @@ SMALL = [
     ("softmax-tall-tiles-few-rows", "qwen3-decode", dict(M=240, H=512, E=16, K=4, I=256)),
     ("shared-same-width-short-tiles", "dsv3-decode", dict(M=100, H=256, E=8, K=2, I=128, n_group=2, topk_group=1,
                                                           I_shared=128)),
+    # expert counts and groupings of other model families (reduced widths): 160 experts in 8 groups of 20 with
+    # top-3 groups and top-6 experts; 1000 experts with top-16; a shared expert 20480 wide (rows of more than
+    # 16384 values in the second quantisation); hidden 16384
+    ("sigmoid-160-experts-8-groups", "dsv3-decode", dict(M=37, H=640, E=160, K=6, I=192, n_group=8, topk_group=3,
+                                                         routed_scale=16.0, I_shared=384)),
+    ("softmax-1000-experts-top16", "qwen3-decode", dict(M=5, H=256, E=1000, K=16, I=64)),
+    ("shared-20480-wide", "dsv3-decode", dict(M=6, H=256, E=8, K=2, I=64, n_group=1, topk_group=1, I_shared=20480)),
+    ("hidden-16384", "qwen3-decode", dict(M=3, H=16384, E=8, K=2, I=64)),
     ("sigmoid-grouped-shared", "dsv3-decode", dict(M=40, H=512, E=32, K=4, I=128, n_group=4, topk_group=2,
                                                    I_shared=256)),
     ("sigmoid-flat-shared", "kimi-decode", dict(M=16, H=256, E=48, K=8, I=64, I_shared=128)),

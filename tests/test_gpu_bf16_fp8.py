@@ -306,13 +306,18 @@ def test_fp8_layer(name, base, over):
     assert np.array_equal(ids.reshape(shape.M, shape.K), ids_ref)
 
 
-@pytest.mark.parametrize("E,n,k,counts", [(1, 64, 128, [16]), (4, 128, 256, [3, 0, 17, 40]), (3, 96, 776, [5, 40, 7])])
+@pytest.mark.parametrize("E,n,k,counts", [(1, 64, 128, [16]), (4, 128, 256, [3, 0, 17, 40]), (3, 96, 776, [5, 40, 7]),
+                                          (2, 544, 320, [140, 3]), (20, 512, 128, [((53 * i) % 300) for i in range(20)])])
 @pytest.mark.parametrize("act", [0, 2])
-@pytest.mark.parametrize("tiled", [False, True])
-def test_grouped_gemm_bf16_bias_and_swigluoai(L, E, n, k, counts, act, tiled):
-    """The expert-bias branch of the bf16 GEMM: y = bf16(bf16(a.w^T) + bias), act 2 = gpt-oss activation."""
+@pytest.mark.parametrize("tiled,variant", [(False, 0), (True, 0), (True, 1), (True, 5), (True, 6), (True, 11)])
+def test_grouped_gemm_bf16_bias_and_swigluoai(L, E, n, k, counts, act, tiled, variant):
+    """The expert-bias branch of the bf16 GEMM: y = bf16(bf16(a.w^T) + bias), act 2 = gpt-oss activation;
+    on the LDS-staged kernels and (tiled weights; variants 5, 6, 11 force it) on the persistent tile kernel,
+    whose epilogue adds the bias and pairs the interleaved gate/up columns."""
     if tiled and (2 * k) % 64:
         pytest.skip("tiled weights need 64 bytes of K")
+    if not tiled and E >= 20:
+        pytest.skip("large case: tiled weights only")
     torch.manual_seed(E + n + k + act)
     lod = _lod(counts)
     rows = int(lod[-1])
@@ -333,6 +338,7 @@ def test_grouped_gemm_bf16_bias_and_swigluoai(L, E, n, k, counts, act, tiled):
     g.w, g.lod, g.bias = dw.data_ptr(), dl.data_ptr(), db.data_ptr()
     g.E, g.n, g.k, g.rows = E, n, k, rows
     g.y, g.ldy, g.act, g.act_alpha, g.act_limit = y.data_ptr(), n_out, act, 1.702, 7.0
+    g.variant = variant
     L.check(L.lib.kmoe_grouped_gemm_bf16(g, L.stream()))
     torch.cuda.synchronize()
     assert rel_l2(y, from_bits(ref)) <= 3e-3
@@ -350,19 +356,25 @@ def test_swigluoai_op_is_the_oracle_sequence():
     assert np.array_equal(bits(got), co.swigluoai_and_mul(bits(y)))
 
 
-def test_fused_moe_expert_bias_branch():
+@pytest.mark.parametrize("M,tiled", [(70, False), (70, True), (600, True)])
+def test_fused_moe_expert_bias_branch(M, tiled):
     """KunlunOps.fused_moe(..., w1_bias, w2_bias): the gpt-oss branch (ops/_kunlun_ops.py:433-468) against the
-    C oracle and the reference's torch loop restated."""
+    C oracle and the reference's torch loop restated; row-major weights, and tiled weights at 35 (64-row tiles)
+    and 300 rows per expert (128-row tiles) on the tile kernel."""
+    from vllm_kunlun_amd import _plan
     from vllm_kunlun_amd.ops._kunlun_ops import KunlunOps
     torch.manual_seed(4)
-    M, H, E, K, I = 70, 128, 8, 4, 64
+    H, E, K, I = 128, 8, 4, 64
     x = torch.randn(M, H).bfloat16()
     logits = torch.randn(M, E)
     w13 = (torch.randn(E, 2 * I, H) * 0.1).bfloat16()
     w2 = (torch.randn(E, H, I) * 0.1).bfloat16()
     b13 = (torch.randn(E, 2 * I) * 0.2).bfloat16()
     b2 = (torch.randn(E, H) * 0.2).bfloat16()
-    out = KunlunOps.fused_moe(x.cuda(), w13.cuda(), w2.cuda(), logits.cuda(), 0, K, True, w1_bias=b13.cuda(),
+    w13d, w2d = w13.cuda(), w2.cuda()
+    if tiled:
+        assert _plan.tile_pair_(w13d, w2d)
+    out = KunlunOps.fused_moe(x.cuda(), w13d, w2d, logits.cuda(), 0, K, True, w1_bias=b13.cuda(),
                               w2_bias=b2.cuda())
     torch.cuda.synchronize()
     ref = from_bits(co.forward_bf16(bits(x), logits.numpy(), bits(w13), bits(w2), K, w13_bias=bits(b13),

@@ -116,6 +116,9 @@ struct TiledParams {
   int32_t tail_row0, tail_rows, tail_src0;
   int32_t n_blocks;  // channel blocks per tile
   int32_t max_items; // upper bound of work items (n_blocks * bound of m-tiles): caps the grid
+  // BF16 only (the expert-bias branch of the reference, ops/_kunlun_ops.py:433-468):
+  const uint16_t* bias;        // NULL, or [E, n] bf16: y = bf16(bf16(gemm) + bias)
+  float oai_alpha, oai_limit;  // OAI kernels: out[r, i] = swigluoai(y[r, 2i], y[r, 2i + 1])
 };
 
 struct Tile {
@@ -144,8 +147,11 @@ struct Tile {
 // MF: 16-row fragments of a wave along the rows. 8: 128-row tiles; 4: 64-row tiles for launches whose
 // experts hold a few dozen rows each (half the MFMAs, fragment reads and epilogue per weight byte,
 // and registers for a third workgroup per CU).
-template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8>
+// OAI (bf16, no SiLU-mul): gate and up columns interleaved, the gpt-oss activation on each (gate, up) pair of
+// a lane's four consecutive channels - n / 2 outputs per row (ops/_custom_ops.py:728-742).
+template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false>
 __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(const TiledParams p) {
+  static_assert(!OAI || (KIND == TKind::BF16 && !SWIGLU && !M32), "the interleaved activation is a bf16 epilogue");
   constexpr int kMF = MF;
   constexpr int kNA = 16 * kMF * (kChunk / 16) / (kWavesT * kWave);  // 16-byte activation vectors per thread and chunk
   static_assert(kNA >= 1 && (M32 ? MF % 2 == 0 : true), "tile height");
@@ -163,7 +169,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   static_assert(R == 4 || R == 8, "the chunk buffer parity is static only for R/2 even");
   constexpr int kNF = NF;
   constexpr int NFH = SWIGLU ? kNF / 2 : kNF;
-  constexpr int kOutBytes = NFH * 16 * 2;   // bytes of one output row owned by a wave: 32 .. 128
+  constexpr int kOutBytes = NFH * 16 * 2 / (OAI ? 2 : 1);  // bytes of one output row owned by a wave: 32 .. 128
   constexpr int kPatchPitch = kOutBytes + 16;  // bytes per row of a wave's output patch (16 rows)
   // ADMA: activations go global -> LDS asynchronously, three chunks ahead, into a ring of four
   // unpadded chunk buffers (row r, 16-byte vector c of a chunk at r * 128 + 16 (c ^ r % 8): eight
@@ -656,6 +662,20 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
 #pragma unroll
       for (int mf = 0; mf < AM; ++mf) sa_r[mf] = sa_lds[parity][wave_m * 16 * kMF + mf * kFragRows + li];
     }
+    // BF16 with expert biases: the four bias values of this lane's channels of every fragment, requested
+    // before the next tile's loads so that waiting for them does not wait for those
+    [[maybe_unused]] uint2 bias_q[AN];
+    if constexpr (BF && !M32 && !SWIGLU) {
+      if (p.bias) {
+#pragma unroll
+        for (int fr = 0; fr < AN; ++fr) {
+          bool ok;
+          const int c = col_of(done, fr, ok);
+          bias_q[fr] = ok ? *reinterpret_cast<const uint2*>(p.bias + static_cast<size_t>(done.e) * p.n + c + lg * 4)
+                          : make_uint2(0u, 0u);
+        }
+      }
+    }
     __builtin_amdgcn_sched_barrier(0);
     if (nxt.valid) {
 #pragma unroll
@@ -675,6 +695,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     // the patch is written and read with LDS instructions the compiler does not see (same reason)
     const uint32_t patch_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)&patch[wave_id][0]));
     const uint32_t patch_wr = patch_base + static_cast<uint32_t>(li * kPatchPitch + lg * 8);
+    [[maybe_unused]] const uint32_t patch_wr_oai = patch_base + static_cast<uint32_t>(li * kPatchPitch + lg * 4);
     // reader side of the patch: lane -> (row, 16-byte vector), consecutive lanes cover a row
     constexpr int kVecPerRow = kOutBytes / 16;        // 2, 4 or 8
     constexpr int kRowsPerRead = kWave / kVecPerRow;  // 32, 16 or 8
@@ -682,7 +703,8 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     const int rd_row = lane / kVecPerRow, rd_vec = lane % kVecPerRow;
     const uint32_t patch_rd =
         patch_base + static_cast<uint32_t>((rd_row & (kFragRows - 1)) * kPatchPitch + rd_vec * 16);
-    const int out_col0 = (done.nb * kWavesT + wave) * NFH * 16;  // first output channel of this wave
+    const int out_col0 = (done.nb * kWavesT + wave) * NFH * 16 / (OAI ? 2 : 1);  // first output channel of this wave
+    const int n_out = OAI ? p.n / 2 : n_half;
 #pragma unroll
     for (int mf = 0; mf < AM; ++mf) {
       float sa = 1.0f;
@@ -710,12 +732,30 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
               yv[q] = silu_fixed(g) * u;
             }
           }
+          if constexpr (BF && !M32 && !SWIGLU) {
+            if (p.bias) {  // y = bf16(bf16(gemm) + bias), as the sum of two bf16 tensors is
+              const uint16_t bv[4] = {static_cast<uint16_t>(bias_q[fr].x), static_cast<uint16_t>(bias_q[fr].x >> 16),
+                                      static_cast<uint16_t>(bias_q[fr].y), static_cast<uint16_t>(bias_q[fr].y >> 16)};
+#pragma unroll
+              for (int q = 0; q < 4; ++q) yv[q] = bf16_to_f32(f32_to_bf16_hw(yv[q])) + bf16_to_f32(bv[q]);
+            }
+          }
+          if constexpr (OAI) {
+            // (gate, up, gate, up): two outputs, at channels (fr * 16 + lg * 4) / 2 and + 1 of the wave's output
+            const uint32_t o0 = swigluoai_bf16(f32_to_bf16_hw(yv[0]), f32_to_bf16_hw(yv[1]), p.oai_alpha, p.oai_limit);
+            const uint32_t o1 = swigluoai_bf16(f32_to_bf16_hw(yv[2]), f32_to_bf16_hw(yv[3]), p.oai_alpha, p.oai_limit);
+            asm volatile("ds_write_b32 %0, %1 offset:%2"
+                         :
+                         : "v"(patch_wr_oai), "v"(o0 | (o1 << 16)), "i"(fr * kFragRows)
+                         : "memory");
+          } else {
           // channel of yv[0] within the wave's output: fr * kFragRows + b * 8 + lg * 4
           const uint2 packed = make_uint2(pack2_bf16(yv[0], yv[1]), pack2_bf16(yv[2], yv[3]));
           asm volatile("ds_write_b64 %0, %1 offset:%2"
                        :
                        : "v"(patch_wr), "v"(packed), "i"((fr * kFragRows + b * 8) * 2)
                        : "memory");
+          }
           if constexpr (I8) {
             const int f16 = M32 ? 2 * fr + (b >> 1) : fr;
             const int cofs = M32 ? (b & 1) * 8 + lg * 4 : lg * 4;
@@ -744,7 +784,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         lds_wait<0>(v);
         const int orow = done.row0 + wave_m * 16 * kMF + mf * kFragRows + pr;
         const int ocol = out_col0 + rd_vec * 8;
-        if (pr < kFragRows && orow < row_end && ocol < n_half)  // n_half % 16 == 0: a vector of 8 channels is all in or all out
+        if (pr < kFragRows && orow < row_end && ocol < n_out)  // n_out % 8 == 0: a vector of 8 channels is all in or all out
           *reinterpret_cast<v4i*>(p.y + static_cast<size_t>(orow) * p.ldy + ocol) = v;
       }
       __builtin_amdgcn_wave_barrier();
@@ -753,7 +793,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   }
 }
 
-template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8>
+template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false>
 int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* what) {
   constexpr int kTM = WM * 16 * MF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
@@ -765,8 +805,8 @@ int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* w
   // persistent workgroups: WGS per CU
   const int grid = min(ceil_div(p.max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8);
   const size_t dyn = sizeof(int) * (static_cast<size_t>(p.E) + 1 + n_exp + 1);
-  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32, MF>), dim3(grid), dim3(WM * kWavesT * kWave), dyn, s,
-                     p);
+  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32, MF, OAI>), dim3(grid),
+                     dim3(WM * kWavesT * kWave), dyn, s, p);
   return check_launch(what);
 }
 
@@ -878,7 +918,14 @@ int tiled_gemm_bf16(const kmoe_gemm_bf16_args* a, hipStream_t s) {
   int n_cu = 0;
   if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
   constexpr TKind K = TKind::BF16;
-  if (short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu, 40))  // measured: at 48 rows per expert the 128-row tiles are 4 % ahead
+  p.bias = a->bias;
+  p.oai_alpha = a->act_alpha;
+  p.oai_limit = a->act_limit;
+  const bool shorter = short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu, 40);  // measured: at 48 rows per expert the 128-row tiles are 4 % ahead
+  if (a->act == KMOE_ACT_SWIGLUOAI)
+    return shorter ? launch_tiled<K, false, 4, 4, 2, 1, false, 4, true>(p, a->rows, s, n_cu, what)
+                   : launch_tiled<K, false, 4, 4, 2, 1, false, 8, true>(p, a->rows, s, n_cu, what);
+  if (shorter)
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)

@@ -58,6 +58,11 @@ SMALL = [
     # 16384 values in the second quantisation); hidden 16384
     ("sigmoid-160-experts-8-groups", "dsv3-decode", dict(M=37, H=640, E=160, K=6, I=192, n_group=8, topk_group=3,
                                                          routed_scale=16.0, I_shared=384)),
+    # intermediate sizes of tensor-parallel shards (192 = 1536 / 8): an odd number of 64-byte steps in the
+    # down projection, on the tile kernel, with and without a shared expert folded into the launches
+    ("softmax-shard-192-many-rows", "qwen3-decode", dict(M=500, H=512, E=16, K=4, I=192)),
+    ("sigmoid-shard-192-shared-many-rows", "dsv3-decode", dict(M=300, H=640, E=16, K=4, I=192, n_group=4,
+                                                               topk_group=2, I_shared=192)),
     ("softmax-1000-experts-top16", "qwen3-decode", dict(M=5, H=256, E=1000, K=16, I=64)),
     ("shared-20480-wide", "dsv3-decode", dict(M=6, H=256, E=8, K=2, I=64, n_group=1, topk_group=1, I_shared=20480)),
     ("hidden-16384", "qwen3-decode", dict(M=3, H=16384, E=8, K=2, I=64)),

@@ -438,6 +438,12 @@ PERSISTENT_CASES = TILED_CASES + [
     # experts (several passes of the 64-lane expert search), most of them empty
     (40, 512, 1152, [((53 * i) % 400) for i in range(40)]),
     (300, 256, 1408, [(129 if i % 7 == 0 else (i % 3)) for i in range(300)]),
+    # an odd number of 64-byte steps (k % 128 == 64): the half chunk at every position of the ring
+    (3, 64, 192, [1, 260, 17]),
+    (2, 96, 448, [140, 3]),
+    (4, 128, 576, [70, 0, 129, 5]),
+    (2, 64, 704, [33, 200]),
+    (8, 4096, 192, [((97 * i) % 300) for i in range(8)]),
 ]
 
 
@@ -448,8 +454,8 @@ def test_lds_gemm_i8_with_tiled_weights(L, E, n, k, counts, variant, act):
     """LDS-staged kernels reading tiled weights and row-major activations. Variants 1-3: small
     tiles; 5-7: the persistent 128-row-tile kernel (6: 256-channel tiles, 7: 128-channel tiles
     with the deep weight ring, 8: 256-row tiles with 8 waves, 5: the default)."""
-    if variant >= 5 and k % 128:
-        pytest.skip("the persistent kernel takes k % 128 == 0")
+    if variant >= 5 and k < 128:
+        pytest.skip("the persistent kernel takes k >= 128")
     if variant < 5 and E >= 40:
         pytest.skip("large case: persistent kernel only")
     _gemm_layout_case(L, E, n, k, counts, act, variant, True, chunked=False, seed=E * n + k + 7)

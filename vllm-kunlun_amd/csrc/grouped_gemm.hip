@@ -469,10 +469,10 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
                a->a_layout);
   if (a->rows == 0 && !(a->w_tail && a->tail_rows > 0)) return KMOE_OK;
   // Tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5-9, 11 force it)
-  if (a->w_layout == KMOE_W_TILED && a->k % 128 == 0 &&
+  if (a->w_layout == KMOE_W_TILED && a->k >= 128 &&
       ((a->variant >= 5 && a->variant <= 9) || a->variant == 11 || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
     return tiled_gemm_i8(a, as_stream(stream));
-  KMOE_REQUIRE(a->variant < 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-11 need tiled weights and k %% 128 == 0");
+  KMOE_REQUIRE(a->variant < 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-11 need tiled weights and k >= 128");
   GemmParams p{a->a,   a->lda, a->a_max, a->row_src, a->src_div, a->w,   a->w_max,
                a->lod, a->E,   a->n,     a->k,       a->y,       a->ldy, a->acc_out, a->w_layout == KMOE_W_TILED,
                a->w_tail, a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0, nullptr, 0, 0.f, 0.f};
@@ -508,7 +508,7 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
   if (a->w_layout == KMOE_W_TILED && a->k % 64 == 0 && a->ldy % 8 == 0 &&
       (tile_variant(a->variant) || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
     return tiled_gemm_bf16(a, as_stream(stream));
-  KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variants 5, 6, 11 need tiled weights, k %% 64 == 0");
+  KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variants 5, 6, 11 need tiled weights, k %% 64 == 0 and ldy %% 8 == 0");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), nullptr,    a->lod,  a->E,       a->n,
                a->k * 2,                              a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,

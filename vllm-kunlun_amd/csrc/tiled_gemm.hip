@@ -200,8 +200,15 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   const int lg = lane / kFragRows;        // 16-byte group of K (16x16: 0..3; 32x32: 0..1)
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int ksteps = p.k / 64;
-  const int nchunks = ksteps / kSteps;  // the host only sends k % 128 == 0 here
+  // Chunks of two MFMA steps. An odd number of int8 steps (k % 128 == 64; the host sends those only with
+  // k >= 128) ends in a half chunk: its copy starts 64 bytes early, so that it stays inside the row, which
+  // puts the last step's bytes into the chunk's second half; the first half (the step before, once more)
+  // meets weights set to zero.
+  const int nfull = ksteps / kSteps;
+  const bool half_chunk = I8 && (ksteps & 1);
+  const int nchunks = nfull + (half_chunk ? 1 : 0);
   const int last_step = ksteps - 1, last_chunk = nchunks - 1;
+  const uint32_t last_chunk_byte = static_cast<uint32_t>(ksteps * 64 - kChunk);
   auto rows_begin = [&](int e) { return e < p.E ? row_lo[e] : p.tail_row0; };
   auto rows_end = [&](int e) { return e < p.E ? row_lo[e + 1] : p.tail_row0 + p.tail_rows; };
 
@@ -342,7 +349,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   // ADMA: requests chunk `chunk` of the tile into ring buffer `stage` (4 copies per wave)
   auto dma_a = [&](int chunk, int stage) {
     if constexpr (ADMA) {
-      const uint32_t kc = static_cast<uint32_t>(min(chunk, last_chunk)) * kChunk;
+      const uint32_t kc = min(static_cast<uint32_t>(chunk) * kChunk, last_chunk_byte);
 #pragma unroll
       for (int i = 0; i < kNA; ++i)
         buffer_load16_to_lds(a_rsrc, (lds_ptr_t)&lds_a[stage][(wave_id * kNA + i) * 1024], aoff[i], kc);
@@ -582,7 +589,9 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     // period, c0 = first chunk of the period. The fences pin the issue order: loads leave at
     // the START of the MFMA run that hides them, and each wait sits just before the first use
     // (the counters retire in issue order, so a wait lets the later loads stay in flight).
-    auto chunk_step = [&](int c0, auto h_tag) {
+    // keep_j0: all ones, or zero for the half chunk at the end of an odd number of steps (the leftover
+    // chunks below pass it; in the main loop it is a constant).
+    auto chunk_step = [&](int c0, auto h_tag, auto keep_j0) {
       constexpr int h = decltype(h_tag)::value;
       constexpr int buf = ADMA ? h % kStagesA : h & 1;
       using buf_t = std::integral_constant<int, buf>;
@@ -597,6 +606,10 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         __builtin_amdgcn_sched_barrier(0);
         load_w(wring[(2 * h) % R], s0 + R);
       } else {
+        if constexpr (I8 && std::is_same_v<decltype(keep_j0), int>) {
+#pragma unroll
+          for (int f = 0; f < kNF; ++f) wring[(2 * h) % R][f] &= (v4i){keep_j0, keep_j0, keep_j0, keep_j0};
+        }
         compute(wring[(2 * h) % R], buf_t{}, j0_t{});
         __builtin_amdgcn_sched_barrier(0);
         load_w(wring[(2 * h) % R], s0 + R);
@@ -621,20 +634,28 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     };
     constexpr int kPeriod = ADMA ? kStagesA : R / 2;  // chunks after which ring slots and buffers repeat
     static_assert(kPeriod == 2 || kPeriod == 4, "unrolled by hand below");
+    constexpr std::false_type kFull{};
     int c = 0;
-    for (; c + kPeriod <= nchunks; c += kPeriod) {
-      chunk_step(c, std::integral_constant<int, 0>{});
-      chunk_step(c, std::integral_constant<int, 1>{});
+    for (; c + kPeriod <= nfull; c += kPeriod) {
+      chunk_step(c, std::integral_constant<int, 0>{}, kFull);
+      chunk_step(c, std::integral_constant<int, 1>{}, kFull);
       if constexpr (kPeriod == 4) {
-        chunk_step(c, std::integral_constant<int, 2>{});
-        chunk_step(c, std::integral_constant<int, 3>{});
+        chunk_step(c, std::integral_constant<int, 2>{}, kFull);
+        chunk_step(c, std::integral_constant<int, 3>{}, kFull);
       }
     }
-    // the chunks left over (fewer than a period): same steps, loads past the end are clamped
-    if (c < nchunks) chunk_step(c, std::integral_constant<int, 0>{});
+    // the chunks left over (fewer than a period, the half chunk last): same steps, loads past the end are clamped
+    auto keep = [&](int chunk) {
+      if constexpr (I8) return (half_chunk && chunk == nfull) ? 0 : -1;
+      else return kFull;
+    };
+    if (c < nchunks) chunk_step(c, std::integral_constant<int, 0>{}, keep(c));
     if constexpr (kPeriod == 4) {
-      if (c + 1 < nchunks) chunk_step(c, std::integral_constant<int, 1>{});
-      if (c + 2 < nchunks) chunk_step(c, std::integral_constant<int, 2>{});
+      if (c + 1 < nchunks) chunk_step(c, std::integral_constant<int, 1>{}, keep(c + 1));
+      if (c + 2 < nchunks) chunk_step(c, std::integral_constant<int, 2>{}, keep(c + 2));
+      if constexpr (I8) {
+        if (c + 3 < nchunks) chunk_step(c, std::integral_constant<int, 3>{}, keep(c + 3));
+      }
     }
 
     // ---- switch: the finished tile's scales leave LDS first (LDS reads the compiler sees wait

@@ -178,7 +178,7 @@ typedef struct kmoe_gemm_i8_args {
   int32_t act;            /* KMOE_ACT_*                                         */
   int32_t variant;        /* 0 = choose from the shape. Tuning and tests: 1-3 LDS-staged 16/32/64-row
                              kernels; with tiled weights 5 = tile kernel (6: 128-row tiles, 11: 64-row
-                             tiles, 7-9: other tile shapes); with chunked activations 1, 2, 4, 8 =
+                             tiles, 7-9: other tile shapes; all need k >= 128); with chunked activations 1, 2, 4, 8 =
                              16-row fragments per pass of the streaming kernel      */
   int32_t w_layout;       /* KMOE_W_ROWMAJOR, or KMOE_W_TILED (kmoe_tile_weights_i8) */
   int32_t a_layout;       /* KMOE_A_ROWMAJOR, or KMOE_A_CHUNKED: a is [k/64][a_rows][64]

@@ -80,6 +80,9 @@ def test_gemm_argument_validation(L):
     assert L.lib.kmoe_grouped_gemm_i8(g, None) == -2   # SwiGLU needs n % 32 == 0
     g.n, g.act, g.a = 64, 0, 0x1001
     assert L.lib.kmoe_grouped_gemm_i8(g, None) == -2 and b"misaligned" in L.lib.kmoe_last_error()
+    # the tile kernel (variants 5-11) moves K in 128-byte chunks: a single 64-byte step is refused, not run
+    g.a, g.k, g.lda, g.w_layout, g.variant = 0x1000, 64, 64, L.KMOE_W_TILED, 5
+    assert L.lib.kmoe_grouped_gemm_i8(g, None) == -3 and b"k >= 128" in L.lib.kmoe_last_error()
 
 
 def test_forward_validation_and_workspace_layout(L):

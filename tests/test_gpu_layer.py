@@ -98,7 +98,8 @@ def test_layer_matches_oracles(name, base, over):
     ref_bits, inter = co.forward_w8a8(**oi, out_scale=out_scale, intermediates=True)
 
     lay, ws = method.last_layout, method.last_workspace
-    P, I, H, E = shape.P, shape.I, shape.H, shape.E
+    P, H, E = shape.P, shape.H, shape.E
+    I = sl.layer.w2_weight.shape[-1]  # the size the kernels see (a size that is no multiple of 64 is padded at load time)
     ids = _view(ws, lay.topk_ids, P, torch.int32).cpu().numpy().reshape(shape.M, shape.K)
     moe_index = _view(ws, lay.moe_index, P, torch.int32).cpu().numpy()
     lod = _view(ws, lay.lod, E + 1, torch.int32).cpu().numpy()
@@ -165,6 +166,35 @@ def test_tiled_and_rowmajor_weights_give_the_same_bits():
         b = plain.layer.quant_method.apply_monolithic(plain.layer, plain.x, plain.logits, **plain.apply_kwargs())
         torch.cuda.synchronize()
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("over", [dict(M=40, H=512, E=16, K=4, I=96), dict(M=700, H=256, E=8, K=2, I=160),
+                                  dict(M=300, H=640, E=16, K=4, I=96, I_shared=96)],
+                         ids=["96-stream", "160-tile-kernel", "96-shared-same-width"])
+def test_padded_intermediate_size_keeps_every_bit(over):
+    """An intermediate size that is no multiple of 64 is padded with zero channels at load time so that the
+    weights can be tiled. The padded layer, the unpadded one (row-major kernels) and the oracle on the
+    unpadded weights must agree bit for bit."""
+    from vllm_kunlun_amd import _plan, synth
+    from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors_moe import (
+        KunlunCompressedTensorsW8A8Int8MoEMethod)
+    shape = synth.scaled(synth.SHAPES["dsv3-decode"], n_group=4, topk_group=2, **{"I_shared": 0, **over})
+    padded = synth.make_w8a8_layer(shape, "cuda", seed=13)
+    Ip = -(-shape.I // 64) * 64
+    assert _plan.is_tiled(padded.layer.w13_weight) and padded.layer.w2_weight.shape[-1] == Ip
+    assert padded.layer.intermediate_size_unpadded == shape.I
+    KunlunCompressedTensorsW8A8Int8MoEMethod.pad_intermediate = False
+    try:
+        plain = synth.make_w8a8_layer(shape, "cuda", seed=13)
+    finally:
+        del KunlunCompressedTensorsW8A8Int8MoEMethod.pad_intermediate
+    assert not _plan.is_tiled(plain.layer.w13_weight) and plain.layer.w2_weight.shape[-1] == shape.I
+    a = padded.layer.quant_method.apply_monolithic(padded.layer, padded.x, padded.logits, **padded.apply_kwargs())
+    b = plain.layer.quant_method.apply_monolithic(plain.layer, plain.x, plain.logits, **plain.apply_kwargs())
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    ref_bits = co.forward_w8a8(**_oracle_inputs(plain), out_scale=1.0)
+    assert np.array_equal(bits(a), ref_bits), "padded layer vs C oracle on the unpadded weights"
 
 
 def test_layer_forward_via_module_call():

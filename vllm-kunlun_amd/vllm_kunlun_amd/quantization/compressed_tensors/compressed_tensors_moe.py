@@ -194,7 +194,41 @@ class KunlunCompressedTensorsW8A8Int8MoEMethod(_MonolithicQuantMoE):
             layer.w13_weight_scale.mul_(127.0)
             layer.w2_weight_scale.mul_(127.0)
             if getattr(self, "tile_weights", True):
+                if getattr(self, "pad_intermediate", True):
+                    self._pad_intermediate_(layer)
                 tile_pair_(layer.w13_weight, layer.w2_weight)
+
+    # the blocks of tiled weights hold 64 bytes of K: the down projection's K is the intermediate size
+    PAD_MULTIPLE = 64
+
+    @classmethod
+    def _pad_intermediate_(cls, layer: torch.nn.Module) -> bool:
+        """An intermediate size that is not a multiple of 64 (96 = 768 / 8 on a tensor-parallel
+        shard, 160, ...) would keep both weights row-major, on the slow kernels. Pads it with
+        zero channels instead: gate rows [0, I), up rows [I', I' + I) of w13, columns [0, I) of
+        w2, zero weights and zero absmax elsewhere. A padded channel's accumulator is 0, its
+        SiLU-mul output 0, its code 0 and its weight in w2 0: the layer's output keeps every bit.
+        The parameters are replaced (shapes [E, 2I', H], [E, 2I', 1], [E, H, I']); the original
+        size stays in `layer.intermediate_size_unpadded`. Returns whether it padded."""
+        w13, w2, s13 = layer.w13_weight.data, layer.w2_weight.data, layer.w13_weight_scale.data
+        E, two_i, H = w13.shape
+        I = two_i // 2
+        Ip = -(-I // cls.PAD_MULTIPLE) * cls.PAD_MULTIPLE
+        if Ip == I or not w13.is_cuda or w13.dtype != torch.int8 or H % 64 or tuple(w2.shape) != (E, H, I):
+            return False
+        w13p = torch.zeros((E, 2 * Ip, H), dtype=w13.dtype, device=w13.device)
+        w13p[:, :I].copy_(w13[:, :I])
+        w13p[:, Ip:Ip + I].copy_(w13[:, I:])
+        s13p = torch.zeros((E, 2 * Ip) + tuple(s13.shape[2:]), dtype=s13.dtype, device=s13.device)
+        s13p[:, :I].copy_(s13[:, :I])
+        s13p[:, Ip:Ip + I].copy_(s13[:, I:])
+        w2p = torch.zeros((E, H, Ip), dtype=w2.dtype, device=w2.device)
+        w2p[:, :, :I].copy_(w2)
+        layer.w13_weight = torch.nn.Parameter(w13p, requires_grad=False)
+        layer.w13_weight_scale = torch.nn.Parameter(s13p, requires_grad=False)
+        layer.w2_weight = torch.nn.Parameter(w2p, requires_grad=False)
+        layer.intermediate_size_unpadded = I
+        return True
 
     def apply_staged(self, layer, x, router_logits, topk_group=None, num_expert_group=None, global_num_experts=-1,
                      scoring_func="softmax", routed_scaling_factor=1.0, e_score_correction_bias=None):

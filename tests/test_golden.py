@@ -63,7 +63,8 @@ def test_gpu_routing_matches_fixture():
 
 
 @pytest.mark.gpu
-def test_gpu_layer_matches_fixture():
+@pytest.mark.parametrize("pad", [False, True], ids=["checkpoint-shapes", "padded-and-tiled"])
+def test_gpu_layer_matches_fixture(pad):
     from vllm_kunlun_amd.ops.fused_moe.layer import FusedMoE
     from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors_moe import (
         KunlunCompressedTensorsW8A8Int8MoEMethod)
@@ -71,6 +72,7 @@ def test_gpu_layer_matches_fixture():
     E, two_i, H = g["w13"].shape
     K = int(g["K"])
     method = KunlunCompressedTensorsW8A8Int8MoEMethod()
+    method.pad_intermediate = pad  # the fixture's intermediate size is no multiple of 64
     layer = FusedMoE(num_experts=E, top_k=K, hidden_size=H, intermediate_size=two_i // 2, quant_method=method,
                      device="cuda")
     layer.w13_weight.data.copy_(torch.from_numpy(g["w13"]))
@@ -79,8 +81,13 @@ def test_gpu_layer_matches_fixture():
     layer.w2_weight_scale.data.copy_(torch.from_numpy(g["w2_max"] / 127.0))
     method.process_weights_after_loading(layer)
     # x/127*127 need not round-trip: install the fixture's maxes exactly
-    layer.w13_weight_scale.data.copy_(torch.from_numpy(g["w13_max"]))
-    layer.w2_weight_scale.data.copy_(torch.from_numpy(g["w2_max"]))
+    I = two_i // 2
+    Ip = layer.w2_weight.shape[-1]  # padded: gate rows at [0, I), up rows at [Ip, Ip + I)
+    assert (Ip != I) == (pad and I % 64 != 0 and H % 64 == 0)
+    w13_max = torch.from_numpy(g["w13_max"]).reshape(E, two_i, -1)
+    layer.w13_weight_scale.data[:, :I].copy_(w13_max[:, :I])
+    layer.w13_weight_scale.data[:, Ip:Ip + I].copy_(w13_max[:, I:])
+    layer.w2_weight_scale.data.copy_(torch.from_numpy(g["w2_max"]).reshape(layer.w2_weight_scale.shape))
     shared = tuple(torch.from_numpy(g[k]).cuda() for k in ("ws13", "ws13_max", "ws2", "ws2_max"))
     out = method.apply_monolithic(layer, from_bits(g["x"]).cuda(), torch.from_numpy(g["logits"]).cuda(),
                                   shared_expert=shared, out_scale=float(g["out_scale"]))

@@ -47,6 +47,11 @@ BF16_TILED_CASES = [
     (3, 96, 320, [5, 140, 7]),                                    # 5 chunks of 128 bytes
     (8, 128, 64, [4, 4, 0, 9, 33, 1, 0, 2]),
     (20, 1024, 128, [((53 * i) % 300) for i in range(20)]),       # several tiles per workgroup walk
+    # an odd number of 64-byte steps (k % 64 == 32): the half chunk at every position of the ring
+    (3, 64, 96, [1, 260, 17]),
+    (2, 96, 160, [140, 3]),
+    (4, 128, 224, [70, 0, 129, 5]),
+    (2, 64, 288, [33, 200]),
 ]
 
 
@@ -57,6 +62,34 @@ def test_grouped_gemm_bf16_tiled_weights(L, E, n, k, counts, variant, act):
     """bf16 weights re-arranged (as bytes) by kmoe_tile_weights_i8: the LDS-staged kernels (1-3) and
     the persistent tile kernel (5: tile height from the rows per expert; 6: 128 rows; 11: 64 rows)."""
     _bf16_case(L, E, n, k, counts, variant, act, tiled=True)
+
+
+def test_grouped_gemm_bf16_half_chunk_ignores_the_repeated_step(L):
+    """With an odd number of 64-byte steps the tile kernel's last chunk holds the step before the last a
+    second time; it must count as zeros whatever it holds. An infinite activation there gives +-inf in every
+    channel (as in the exact product), never NaN."""
+    E, n, k, rows = 1, 64, 96, 70
+    torch.manual_seed(5)
+    a = torch.randn(rows, k).bfloat16()
+    a[3, 40] = float("inf")  # element 40: in the second step, which the half chunk reads again
+    w = (torch.randn(E, n, k) * 0.05).bfloat16()
+    w[w == 0] = 0.05
+    da, dw = a.cuda(), w.cuda()
+    dt = torch.empty_like(dw)
+    L.check(L.lib.kmoe_tile_weights_i8(dw.data_ptr(), dt.data_ptr(), E, n, 2 * k, L.stream()))
+    dl = torch.tensor([0, rows], dtype=torch.int32, device="cuda")
+    y = torch.zeros(rows, n, dtype=torch.bfloat16, device="cuda")
+    g = L.GemmBf16Args()
+    g.a, g.lda, g.src_div, g.w, g.lod = da.data_ptr(), k, 1, dt.data_ptr(), dl.data_ptr()
+    g.E, g.n, g.k, g.rows = E, n, k, rows
+    g.y, g.ldy, g.act, g.variant, g.w_layout = y.data_ptr(), n, 0, 5, L.KMOE_W_TILED
+    L.check(L.lib.kmoe_grouped_gemm_bf16(g, L.stream()))
+    torch.cuda.synchronize()
+    y = y.float().cpu()
+    assert not torch.isnan(y).any()
+    assert torch.equal(y[3], torch.sign(w[0, :, 40].float()) * float("inf"))
+    keep = [r for r in range(rows) if r != 3]
+    assert rel_l2(y[keep], a[keep].float() @ w[0].float().T) <= 2e-3
 
 
 @pytest.mark.parametrize("E,n,k,counts", CASES)

@@ -126,7 +126,9 @@ def test_layer_matches_oracles(name, base, over):
 def test_staged_ops_equal_fused():
     """The reference's op-by-op sequence through torch.ops._C.* gives the same bits."""
     from vllm_kunlun_amd import synth
-    for over in (dict(M=48, H=512, E=16, K=4, I=256), dict(M=200, H=256, E=8, K=4, I=128)):  # P <= 768 and > 768
+    # P <= 768 and > 768; an intermediate size that is padded at load time
+    for over in (dict(M=48, H=512, E=16, K=4, I=256), dict(M=200, H=256, E=8, K=4, I=128),
+                 dict(M=48, H=512, E=16, K=4, I=96)):
         sl = synth.make_w8a8_layer(synth.scaled(synth.SHAPES["qwen3-decode"], **over), "cuda", seed=2)
         m = sl.layer.quant_method
         fused = m.apply_monolithic(sl.layer, sl.x, sl.logits)

@@ -505,10 +505,10 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR || (a->w_layout == KMOE_W_TILED && a->k % 32 == 0), KMOE_ERR_SHAPE,
                "grouped_gemm_bf16: w_layout=%d (tiled weights need k %% 32 == 0, k=%d)", a->w_layout, a->k);
   // tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5, 6, 11 force it)
-  if (a->w_layout == KMOE_W_TILED && a->k % 64 == 0 && a->ldy % 8 == 0 &&
+  if (a->w_layout == KMOE_W_TILED && a->k >= 64 && a->ldy % 8 == 0 &&
       (tile_variant(a->variant) || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
     return tiled_gemm_bf16(a, as_stream(stream));
-  KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variants 5, 6, 11 need tiled weights, k %% 64 == 0 and ldy %% 8 == 0");
+  KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variants 5, 6, 11 need tiled weights, k >= 64 and ldy %% 8 == 0");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), nullptr,    a->lod,  a->E,       a->n,
                a->k * 2,                              a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,

@@ -200,12 +200,13 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   const int lg = lane / kFragRows;        // 16-byte group of K (16x16: 0..3; 32x32: 0..1)
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int ksteps = p.k / 64;
-  // Chunks of two MFMA steps. An odd number of int8 steps (k % 128 == 64; the host sends those only with
-  // k >= 128) ends in a half chunk: its copy starts 64 bytes early, so that it stays inside the row, which
-  // puts the last step's bytes into the chunk's second half; the first half (the step before, once more)
-  // meets weights set to zero.
+  // Chunks of two MFMA steps. An odd number of steps (int8: k % 128 == 64, bf16: k % 64 == 32; the host sends
+  // those only with at least one whole chunk) ends in a half chunk: its copy starts 64 bytes early, so that it
+  // stays inside the row, which puts the last step's bytes into the chunk's second half; the first half (the
+  // step before, once more) is read from LDS and set to zero before it meets the MFMA (zero activations
+  // against finite weights add nothing; zero weights would turn an infinite activation into NaN).
   const int nfull = ksteps / kSteps;
-  const bool half_chunk = I8 && (ksteps & 1);
+  const bool half_chunk = ADMA && (ksteps & 1);
   const int nchunks = nfull + (half_chunk ? 1 : 0);
   const int last_step = ksteps - 1, last_chunk = nchunks - 1;
   const uint32_t last_chunk_byte = static_cast<uint32_t>(ksteps * 64 - kChunk);
@@ -380,7 +381,8 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   };
   // fragment n of a step: (row fragment, K part); 16x16: 8 row fragments; 32x32: 2 K parts x 4
   constexpr int kFragReads = M32 ? 2 * AM : kMF;
-  auto compute = [&](const v4i(&wcur)[kNF], auto buf_tag, auto j_tag) {
+  // keep: std::false_type (every fragment as read), or an int mask (0: the fragments count as zeros)
+  auto compute = [&](const v4i(&wcur)[kNF], auto buf_tag, auto j_tag, auto keep) {
     constexpr int buf = decltype(buf_tag)::value, j = decltype(j_tag)::value;
     if constexpr (ADMA) {
       // two fragments in flight: the read of fragment n + 1 leaves before the MFMAs of fragment n
@@ -405,6 +407,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         } else {
           lds_wait<0>(af[n & 1]);
         }
+        if constexpr (std::is_same_v<decltype(keep), int>) af[n & 1] &= (v4i){keep, keep, keep, keep};
         mfma_row(wcur, af[n & 1], mf, t);
       }
     }
@@ -606,17 +609,13 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         __builtin_amdgcn_sched_barrier(0);
         load_w(wring[(2 * h) % R], s0 + R);
       } else {
-        if constexpr (I8 && std::is_same_v<decltype(keep_j0), int>) {
-#pragma unroll
-          for (int f = 0; f < kNF; ++f) wring[(2 * h) % R][f] &= (v4i){keep_j0, keep_j0, keep_j0, keep_j0};
-        }
-        compute(wring[(2 * h) % R], buf_t{}, j0_t{});
+        compute(wring[(2 * h) % R], buf_t{}, j0_t{}, keep_j0);
         __builtin_amdgcn_sched_barrier(0);
         load_w(wring[(2 * h) % R], s0 + R);
         // the buffer chunk c - 1 was read from is free since the last barrier: chunk c + 3 goes there
         dma_a(c0 + h + kStagesA - 1, (buf + kStagesA - 1) % kStagesA);
         __builtin_amdgcn_sched_barrier(0);
-        compute(wring[(2 * h + 1) % R], buf_t{}, j1_t{});
+        compute(wring[(2 * h + 1) % R], buf_t{}, j1_t{}, std::false_type{});
       }
       __builtin_amdgcn_sched_barrier(0);
       store_a(buf ^ 1);
@@ -646,14 +645,14 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     }
     // the chunks left over (fewer than a period, the half chunk last): same steps, loads past the end are clamped
     auto keep = [&](int chunk) {
-      if constexpr (I8) return (half_chunk && chunk == nfull) ? 0 : -1;
+      if constexpr (ADMA) return (half_chunk && chunk == nfull) ? 0 : -1;
       else return kFull;
     };
     if (c < nchunks) chunk_step(c, std::integral_constant<int, 0>{}, keep(c));
     if constexpr (kPeriod == 4) {
       if (c + 1 < nchunks) chunk_step(c, std::integral_constant<int, 1>{}, keep(c + 1));
       if (c + 2 < nchunks) chunk_step(c, std::integral_constant<int, 2>{}, keep(c + 2));
-      if constexpr (I8) {
+      if constexpr (ADMA) {
         if (c + 3 < nchunks) chunk_step(c, std::integral_constant<int, 3>{}, keep(c + 3));
       }
     }

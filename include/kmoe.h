@@ -487,6 +487,20 @@ int kmoe_moe_workspace_layout(const kmoe_moe_args* args, kmoe_moe_layout* layout
 int kmoe_moe_forward(const kmoe_moe_args* args, void* workspace,
                      size_t workspace_bytes, kmoe_stream_t stream);
 
+/*
+ * kmoe_moe_forward without a workspace argument. No counterpart in the reference: it is for
+ * callers that cannot allocate device memory for a workspace (code that is being captured
+ * into a HIP graph, serving loops and harnesses that forbid hipMalloc). The intermediates live
+ * in a buffer of KMOE_STATIC_WORKSPACE_BYTES that is part of the library's device image (every
+ * GPU the library runs on holds it until the process ends); a shape whose
+ * kmoe_moe_workspace_layout().total_bytes exceeds it is refused with KMOE_ERR_WORKSPACE.
+ * Allocates nothing, same results as kmoe_moe_forward bit for bit. Call it with the stream's
+ * device current. All calls on one GPU share the one buffer: calls that may overlap on a GPU
+ * (two streams, two threads) race; the buffer keeps the last call's intermediates.
+ */
+#define KMOE_STATIC_WORKSPACE_BYTES (64u << 20)
+int kmoe_moe_forward_static(const kmoe_moe_args* args, kmoe_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -160,3 +160,11 @@ def test_process_weights_after_loading_turns_scales_into_maxes():
     before = mx.clone()
     sl.layer.quant_method.process_weights_after_loading(sl.layer)  # a second call multiplies again: it is in place
     assert torch.allclose(sl.layer.w13_weight_scale, before * 127.0)
+
+
+def test_static_workspace_forward_refuses_what_does_not_fit(L):
+    a = L.MoEArgs()
+    a.M, a.H, a.E, a.K, a.I = 4096, 7168, 256, 8, 2048  # needs ~0.9 GB of intermediates
+    a.format = L.KMOE_FMT_INT8
+    assert L.lib.kmoe_moe_forward_static(C.byref(a), None) == -4
+    assert b"built-in buffer" in L.lib.kmoe_last_error()

@@ -2,6 +2,7 @@
 // stage kernels together on one stream out of one caller-owned workspace.
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 
 #include "kmoe_common.h"
 
@@ -513,4 +514,52 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
                     shared_out, H, a->out, H, stream);
   mark(KMOE_STAGE_COMBINE, 1);
   return rc;
+}
+
+// ---- the layer for callers that cannot hand over a workspace -------------------------------
+// kmoe_moe_forward with its workspace in a file-scope device array. The array's name is only a
+// host-side handle: its device address is asked for once per GPU (each GPU holds its own copy at
+// its own address) and that address is what the kernels get.
+static __device__ __align__(256) unsigned char scratch[KMOE_STATIC_WORKSPACE_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current GPU (asked for on the first call per GPU).
+int static_workspace(void** out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return fail(KMOE_ERR_LAUNCH, "moe_forward_static: hipGetDevice: %s", hipGetErrorString(err));
+  KMOE_REQUIRE(dev >= 0 && dev < kMaxDevices, KMOE_ERR_UNSUPPORTED, "moe_forward_static: device %d (at most %d)", dev,
+               kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !p)
+      return fail(KMOE_ERR_LAUNCH, "moe_forward_static: hipGetSymbolAddress on device %d: %s", dev,
+                  hipGetErrorString(err));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return KMOE_OK;
+}
+
+}  // namespace
+
+extern "C" int kmoe_moe_forward_static(const kmoe_moe_args* a, kmoe_stream_t stream) {
+  kmoe_moe_layout L;
+  if (int rc = kmoe_moe_workspace_layout(a, &L)) return rc;
+  KMOE_REQUIRE(L.total_bytes <= static_cast<size_t>(KMOE_STATIC_WORKSPACE_BYTES), KMOE_ERR_WORKSPACE,
+               "moe_forward_static: this shape needs %zu bytes of scratch, the built-in buffer holds %zu "
+               "(use kmoe_moe_forward with a workspace of the caller's)",
+               L.total_bytes, static_cast<size_t>(KMOE_STATIC_WORKSPACE_BYTES));
+  void* ws = nullptr;
+  if (int rc = static_workspace(&ws)) return rc;
+  // every slot of the layout is written by the stage that owns it before anything reads it, so
+  // the last call's contents need no clearing
+  return kmoe_moe_forward(a, ws, KMOE_STATIC_WORKSPACE_BYTES, stream);
 }

@@ -128,6 +128,7 @@ def _load() -> C.CDLL:
         "kmoe_grouped_gemm_fp8_block": (i32, [C.POINTER(GemmFp8Args), vp]),
         "kmoe_moe_workspace_layout": (i32, [C.POINTER(MoEArgs), C.POINTER(MoELayout)]),
         "kmoe_moe_forward": (i32, [C.POINTER(MoEArgs), vp, sz, vp]),
+        "kmoe_moe_forward_static": (i32, [C.POINTER(MoEArgs), vp]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)
@@ -142,8 +143,9 @@ EXPORTS = (
     "kmoe_align_workspace_bytes", "kmoe_align", "kmoe_gather_rows", "kmoe_quant_i8_rows", "kmoe_quant_i8_rows_chunked", "kmoe_tile_weights_i8", "kmoe_quant_fp8_group128",
     "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_w4a16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
     "kmoe_moe_workspace_layout", "kmoe_moe_forward", "kmoe_router_gemm_workspace_bytes", "kmoe_router_gemm_bf16",
-    "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16",
+    "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16", "kmoe_moe_forward_static",
 )
+STATIC_WORKSPACE_BYTES = 64 << 20
 
 
 def check(rc: int) -> None:

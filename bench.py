@@ -3,6 +3,10 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--tokens M]
 
+Without --workload the line's headline is the DeepSeek-V3-shape W8A8 decode layer (128 tokens,
+shared expert included) with its CPU baseline, and the other benchmark configurations (prefill,
+the Qwen3 shape, the fp8 layers) are timed in the same run and reported under "workloads".
+
 A step is one call of the whole layer (routing -> align -> int8 quant -> gate_up
 GEMM + SiLU-mul -> int8 quant -> down GEMM -> combine, plus the shared expert
 where the shape has one) over one batch of synthetic tokens that already sits
@@ -118,8 +122,9 @@ def measured_traffic(workload):
     return None
 
 
-def cpu_baseline(sl, budget_s=10.0):
-    """The reference's torch expert loop (oracle/torch_moe.py) on the host cores."""
+def cpu_baseline(sl, budget_s=15.0):
+    """The reference's torch expert loop (oracle/torch_moe.py) on the host cores: one warm-up
+    call, then whole layer calls of the same workload for about budget_s seconds."""
     import torch
     from oracle import torch_moe as tm
     s = sl.shape
@@ -175,58 +180,20 @@ def vendor_dense_gemm(shape, g1_ops, peak_tops, reps=20):
             "frac_of_peak": ops / ms / 1e9 / peak_tops}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=1000)
-    ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", default="qwen3-decode", choices=sorted(WORKLOAD_LABEL))
-    ap.add_argument("--launch", default="auto", choices=["auto", "graph", "eager"],
-                    help="replay the layer from a captured HIP graph (as a serving engine does), launch it eagerly, "
-                         "or (auto) time K steps each way and report the faster; config.launch says which")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--tokens", type=int, default=0,
-                    help="run the workload's layer at another batch (tokens per call); the config then says so")
-    ap.add_argument("--router", action="store_true",
-                    help="hand the layer the bf16 gate weight [E,H] instead of router logits: the router GEMM "
-                         "then runs inside each step (reported in config; not the default workload)")
-    ap.add_argument("--dims", default="",
-                    help="other layer dimensions for the workload's format and routing, e.g. "
-                         "H=4096,E=8,K=2,I=14336,I_shared=0 (Mixtral-8x7B); the config then says so")
-    ap.add_argument("--yardstick", action="store_true",
-                    help="also time the vendor library's dense GEMM (torch._int_mm / bf16 matmul) with the gate_up "
-                         "GEMM's operation count: [P,H] x [H,2I], one weight matrix, no gather, no epilogue")
-    ap.add_argument("--copy-probe", action="store_true",
-                    help="also run one bitwise_not over 256 MiB (a kernel of known HBM traffic and a name nothing "
-                         "else here has) before the timed region: the yardstick for FETCH_SIZE / WRITE_SIZE runs")
-    a = ap.parse_args()
-    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        sys.exit("bench.py: this build measures ONE GPU; the layer does not span GPUs (run with --gpus 1)")
+# What plain `python bench.py` runs besides the headline workload: the other BASELINE
+# configurations, reported under "workloads" in the same JSON line.
+SUITE = ["dsv3-prefill", "qwen3-decode", "qwen3-prefill", "qwen3-prefill-skew", "dsv3-fp8-decode", "dsv3-fp8-prefill"]
+HEADLINE = "dsv3-decode"
 
+
+def measure(a, workload, shape, label, sl, with_cpu_baseline):
+    """Times one workload's layer on cuda:0 (inputs resident in HBM) and returns the pieces of
+    the JSON line: ms per step (graph replay / eager plan / plugin entry), per-stage durations
+    from HIP events on the launch stream, the gate_up GEMM's roofline, the layer's fractions."""
     import torch
     from vllm_kunlun_amd import _lib as L
-    from vllm_kunlun_amd import synth
-
-    torch.cuda.set_device(0)
-    shape = synth.SHAPES[a.workload]
-    label = WORKLOAD_LABEL[a.workload]
-    if a.tokens and a.tokens != shape.M:
-        shape = synth.scaled(shape, M=a.tokens)
-        label = re.sub(r"(decode|prefill), \d+ tokens", f"{a.tokens} tokens (batch set by --tokens)", label)
-    if a.dims:
-        allowed = {"H": int, "E": int, "K": int, "I": int, "I_shared": int, "n_group": int, "topk_group": int,
-                   "scoring": str, "routed_scale": float}
-        over = {}
-        for item in a.dims.split(","):
-            key, _, val = item.partition("=")
-            if key not in allowed:
-                sys.exit(f"bench.py: --dims takes {sorted(allowed)}, not {key!r}")
-            over[key] = allowed[key](val)
-        shape = synth.scaled(shape, **over)
-        label = f"MoE layer with --dims {a.dims} on the format and routing of {a.workload}, {shape.M} tokens"
     from vllm_kunlun_amd._plan import make_moe_plan
-    sl = synth.make_layer(shape, "cuda:0", seed=a.seed)
+
     lay = sl.layer
     x, logits = sl.x.contiguous(), sl.logits.contiguous()
     out = torch.empty_like(x)
@@ -250,20 +217,20 @@ def main():
                              sl.shared, 1.0, stage_events, router_weight=w_gate,
                              group_size=shape.group_size if w4 else None)
 
-    plan = make_plan()
-
     # The layer, its inputs and the workspace were produced on the default stream;
     # finish that work before a second stream touches (recycled) memory.
     torch.cuda.synchronize()
     stream = torch.cuda.Stream()
     stream.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(stream):
+        plan = make_plan()
         if a.copy_probe:
             src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0")
             torch.bitwise_not(src, out=torch.empty_like(src))
         for _ in range(3):
             plan()
         stream.synchronize()
+
         def timed(step):
             for _ in range(a.warmup):
                 step()
@@ -284,6 +251,12 @@ def main():
             launch_ms["eager"] = timed(plan)
         launch_mode = min(launch_ms, key=launch_ms.get)
         ms_per_step = launch_ms[launch_mode]
+        # the plugin entry itself (per-call output allocation, argument block, workspace lookup):
+        # reported beside the replayed argument block, never as `value`
+        if not a.router and not w4:
+            method = lay.quant_method
+            kw = sl.apply_kwargs() if shape.quant in ("int8", "fp8") else {}
+            launch_ms["apply_monolithic eager"] = timed(lambda: method.apply_monolithic(lay, x, logits, **kw))
 
         # the same calls again with HIP events around each stage (eager: events are
         # not captured), for the per-kernel durations of the roofline
@@ -298,6 +271,7 @@ def main():
         stage_ms = {s: v / a.steps for s, v in stage_ms.items()}
         stream.synchronize()
         ev.close()
+    torch.cuda.current_stream().wait_stream(stream)
 
     lod = plan.view("lod", shape.E + 1, torch.int32).cpu()
     n_active = int(((lod[1:] - lod[:-1]) > 0).sum())
@@ -306,7 +280,7 @@ def main():
     peak_tops = PEAK_TOPS[shape.quant]
     hbm_bound = intensity < peak_tops * 1e12 / (HBM_PEAK_GBS * 1e9)
     g1_s = stage_ms["gemm1"] * 1e-3
-    traffic = None if (a.tokens or a.dims) else measured_traffic(a.workload)  # the counter summaries are of the named workload
+    traffic = None if (a.tokens or a.dims) else measured_traffic(workload)  # the counter summaries are of the named workload
     if hbm_bound:
         achieved = work["g1_bytes"] / g1_s / 1e9
         roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -319,23 +293,16 @@ def main():
     g1_kernel = ("w4_stream_kernel" if w4 else "stream_gemm_i8_kernel" if plan.layout.codes_chunked else
                  "tiled_gemm_kernel" if many_rows and plan.args.w_layout == L.KMOE_W_TILED else "grouped_gemm_kernel")
     roofline.update(kernel=g1_kernel + " (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
-                    algorithmic_bytes=work["g1_bytes"], algorithmic_ops=work["g1_ops"])
+                    algorithmic_bytes=work["g1_bytes"], algorithmic_ops=work["g1_ops"],
+                    hbm_frac=work["g1_bytes"] / g1_s / 1e9 / HBM_PEAK_GBS,
+                    mfma_frac=work["g1_ops"] / g1_s / 1e12 / peak_tops)
 
     t_s = ms_per_step * 1e-3
-    result = {
-        "metric": "MoE-layer tokens/s at 1 GPU",
+    res = {
         "value": shape.M / t_s,
-        "unit": "tokens/s",
-        "n_gpus": 1,
-        "steps": a.steps,
-        "warmup": a.warmup,
         "ms_per_step": ms_per_step,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
         "dtype": DTYPE[shape.quant],
-        "data": "synthetic",
-        "config": {"workload": label, "name": a.workload, "tokens": shape.M, "hidden": shape.H,
+        "config": {"workload": label, "name": workload, "tokens": shape.M, "hidden": shape.H,
                    "experts": shape.E, "top_k": shape.K, "moe_intermediate": shape.I,
                    "shared_intermediate": shape.I_shared, "routing": shape.scoring, "experts_hit": n_active,
                    "launch": launch_mode, "launch_ms_per_step": launch_ms, "seed": a.seed,
@@ -348,11 +315,115 @@ def main():
                   "stage_ms": stage_ms},
     }
     if a.yardstick and shape.quant in ("int8", "none"):
-        result["vendor_dense_gemm"] = vendor_dense_gemm(shape, work["g1_ops"], peak_tops)
-    if not a.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(sl)
-    else:
-        result["cpu_baseline"] = None
+        res["vendor_dense_gemm"] = vendor_dense_gemm(shape, work["g1_ops"], peak_tops)
+    res["cpu_baseline"] = cpu_baseline(sl, a.cpu_budget) if with_cpu_baseline else None
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOAD_LABEL),
+                    help=f"time this workload alone. Default: {HEADLINE} as the line's headline, with its CPU "
+                         f"baseline, and the other configurations ({', '.join(SUITE)}) under 'workloads'")
+    ap.add_argument("--no-suite", action="store_true", help="with the default headline: leave out 'workloads'")
+    ap.add_argument("--launch", default="auto", choices=["auto", "graph", "eager"],
+                    help="replay the layer from a captured HIP graph (as a serving engine does), launch it eagerly, "
+                         "or (auto) time K steps each way and report the faster; config.launch says which")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU work for the baseline sample")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--tokens", type=int, default=0,
+                    help="run the workload's layer at another batch (tokens per call); the config then says so")
+    ap.add_argument("--router", action="store_true",
+                    help="hand the layer the bf16 gate weight [E,H] instead of router logits: the router GEMM "
+                         "then runs inside each step (reported in config; not the default workload)")
+    ap.add_argument("--dims", default="",
+                    help="other layer dimensions for the workload's format and routing, e.g. "
+                         "H=4096,E=8,K=2,I=14336,I_shared=0 (Mixtral-8x7B); the config then says so")
+    ap.add_argument("--yardstick", action="store_true",
+                    help="also time the vendor library's dense GEMM (torch._int_mm / bf16 matmul) with the gate_up "
+                         "GEMM's operation count: [P,H] x [H,2I], one weight matrix, no gather, no epilogue")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one bitwise_not over 256 MiB (a kernel of known HBM traffic and a name nothing "
+                         "else here has) before the timed region: the yardstick for FETCH_SIZE / WRITE_SIZE runs")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build measures ONE GPU; the layer does not span GPUs (run with --gpus 1)")
+
+    import torch
+    from vllm_kunlun_amd import synth
+
+    torch.cuda.set_device(0)
+    headline = a.workload or HEADLINE
+    names = [headline] + ([] if (a.workload or a.no_suite or a.tokens or a.dims or a.router) else SUITE)
+
+    def shape_of(name):
+        shape, label = synth.SHAPES[name], WORKLOAD_LABEL[name]
+        if a.tokens and a.tokens != shape.M:
+            shape = synth.scaled(shape, M=a.tokens)
+            label = re.sub(r"(decode|prefill), \d+ tokens", f"{a.tokens} tokens (batch set by --tokens)", label)
+        if a.dims:
+            allowed = {"H": int, "E": int, "K": int, "I": int, "I_shared": int, "n_group": int, "topk_group": int,
+                       "scoring": str, "routed_scale": float}
+            over = {}
+            for item in a.dims.split(","):
+                key, _, val = item.partition("=")
+                if key not in allowed:
+                    sys.exit(f"bench.py: --dims takes {sorted(allowed)}, not {key!r}")
+                over[key] = allowed[key](val)
+            shape = synth.scaled(shape, **over)
+            label = f"MoE layer with --dims {a.dims} on the format and routing of {name}, {shape.M} tokens"
+        return shape, label
+
+    # workloads that differ only in the batch (tokens, logit bias) share one set of weights:
+    # the 11 GB layers are generated once
+    def weights_key(s):
+        return (s.H, s.E, s.K, s.I, s.scoring, s.n_group, s.topk_group, s.routed_scale, s.I_shared, s.quant,
+                s.group_size)
+
+    results, cached = {}, None
+    order = sorted(names, key=lambda n: (n != headline,))  # headline first (stable for the rest)
+    for name in order:
+        shape, label = shape_of(name)
+        if cached is not None and cached[0] == weights_key(shape):
+            sl = synth.rebatch(cached[1], shape, seed=a.seed)
+        else:
+            cached = None
+            torch.cuda.empty_cache()
+            sl = synth.make_layer(shape, "cuda:0", seed=a.seed)
+        cached = (weights_key(shape), sl)
+        results[name] = measure(a, name, shape, label, sl, name == headline and not a.no_cpu_baseline)
+        print(f"bench.py: {name}: {results[name]['ms_per_step']:.4f} ms/step", file=sys.stderr, flush=True)
+
+    head = results[headline]
+    result = {
+        "metric": "MoE-layer tokens/s at 1 GPU",
+        "value": head["value"],
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": head["dtype"],
+        "data": "synthetic",
+        "config": head["config"],
+        "roofline": head["roofline"],
+        "layer": head["layer"],
+        "cpu_baseline": head["cpu_baseline"],
+    }
+    if "vendor_dense_gemm" in head:
+        result["vendor_dense_gemm"] = head["vendor_dense_gemm"]
+    if len(results) > 1:
+        result["workloads"] = {
+            n: {"tokens_per_s": r["value"], "ms_per_step": r["ms_per_step"], "dtype": r["dtype"], "config": r["config"],
+                "roofline": r["roofline"], "layer": r["layer"]}
+            for n, r in results.items() if n != headline}
     print(json.dumps(result))
 
 

@@ -122,6 +122,21 @@ class SynthLayer:
         return kw
 
 
+def rebatch(sl: SynthLayer, shape: MoEShape, seed: int = 0) -> SynthLayer:
+    """Another batch for the same weights: a SynthLayer that shares `sl`'s layer, correction bias and
+    shared expert and carries fresh activations and router logits of `shape` (its tokens, its hot
+    experts), drawn from a generator seeded with (seed, tokens)."""
+    a, b = sl.shape, shape
+    same = ("H", "E", "K", "I", "scoring", "n_group", "topk_group", "routed_scale", "I_shared", "quant", "group_size")
+    if any(getattr(a, f) != getattr(b, f) for f in same):
+        raise ValueError("rebatch: the new shape must keep the layer's dimensions, routing and format")
+    dev = sl.x.device
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed * 1000003 + shape.M)
+    x, logits = _activations(shape, g, dev)
+    return SynthLayer(shape, sl.layer, x, logits, sl.bias, sl.shared)
+
+
 def _quant_block_fp8(w: torch.Tensor):
     """[n,k] float -> e4m3fn codes + one f32 scale per 128x128 block (absmax/448)."""
     n, k = w.shape

@@ -17,6 +17,8 @@ pytestmark = pytest.mark.gpu
 
 from oracle import c_oracle as co  # noqa: E402
 
+REL_L2_FP8 = 3e-2  # tolerance of the fp8 layer's bf16 output against the oracle
+
 
 def _host(t):
     return None if t is None else t.detach().cpu()
@@ -100,26 +102,64 @@ def test_dsv3_full_size(dsv3):
     _properties(sl, host, n_decode=128, n_spot=16, seed=2, mids=(320, 352, 1024, 1536, 1600))
 
 
-def test_dsv3_fp8_full_size_sample_against_the_oracle():
-    """The fp8 block-scaled layer at the DeepSeek-V3 shape, 4096 tokens: a sample of its tokens against
-    the C oracle within the fp8 tolerance (MFMA and oracle sum in different orders), routing bit-exact."""
-    from conftest import from_bits, rel_l2
-    from vllm_kunlun_amd import synth
-    shape = synth.SHAPES["dsv3-fp8-prefill"]
-    sl = synth.make_fp8_layer(shape, "cuda", seed=0)
-    m = sl.layer.quant_method
-    full = m.apply_monolithic(sl.layer, sl.x, sl.logits, **sl.apply_kwargs())
-    torch.cuda.synchronize()
-    idx = torch.arange(5, shape.M, 257, device="cuda")[:16]
-    w13, w13_s, w2, w2_s, sh = sl.host_weights()
+def _fp8_oracle(sl, host, x, logits):
+    w13, w13_s, w2, w2_s, sh = host
+    s = sl.shape
     u8 = lambda t: t.view(torch.uint8).numpy()  # noqa: E731
-    shared = (u8(sh[0]), sh[1].numpy(), u8(sh[2]), sh[3].numpy())
-    ref = co.forward_fp8(bits(sl.x[idx]), _host(sl.logits[idx]).numpy(), u8(w13), w13_s.numpy(), u8(w2), w2_s.numpy(),
-                         shape.K, shape.scoring, True, shape.n_group, shape.topk_group, shape.routed_scale,
-                         _host(sl.bias).numpy(), shared)
-    assert rel_l2(full[idx], from_bits(ref)) <= 3e-2
-    ids = m.last_workspace[m.last_layout.topk_ids: m.last_layout.topk_ids + 4 * shape.P].view(torch.int32)
-    ids = ids.view(shape.M, shape.K)[idx].cpu().numpy()
-    _, ids_ref = co.sigmoid_group_topk_norm(_host(sl.logits[idx]).numpy(), _host(sl.bias).numpy(), shape.K,
-                                            shape.n_group, shape.topk_group, shape.routed_scale)
+    shared = None if sh is None else (u8(sh[0]), sh[1].numpy(), u8(sh[2]), sh[3].numpy())
+    return co.forward_fp8(bits(x), _host(logits).numpy(), u8(w13), w13_s.numpy(), u8(w2), w2_s.numpy(), s.K, s.scoring,
+                          True, s.n_group, s.topk_group, s.routed_scale, _host(sl.bias).numpy(), shared)
+
+
+def _routing_ids(sl, M):
+    m, s = sl.layer.quant_method, sl.shape
+    ids = m.last_workspace[m.last_layout.topk_ids: m.last_layout.topk_ids + 4 * M * s.K].view(torch.int32)
+    return ids.view(M, s.K)
+
+
+def _fp8_checks(sl, host, n_decode, n_spot):
+    """fp8 block-scaled layer: the prefill batch on a sample of its tokens and the decode batch in full
+    against the C oracle within the fp8 tolerance (MFMA and oracle sum in different orders); routing ids
+    bit-exact; the decode batch (16-row LDS-staged kernel + a shared-expert pass of its own) against the
+    same tokens inside the prefill batch (tile kernel, shared expert folded in) within that tolerance."""
+    from conftest import from_bits, rel_l2
+    s = sl.shape
+    full = _run(sl, sl.x, sl.logits)
+    assert bool(torch.isfinite(full.float()).all())
+    idx = torch.arange(5, s.M, 257, device="cuda")[:n_spot]
+    ids = _routing_ids(sl, s.M)[idx].cpu().numpy()
+    assert rel_l2(full[idx], from_bits(_fp8_oracle(sl, host, sl.x[idx], sl.logits[idx]))) <= REL_L2_FP8
+    _, ids_ref = co.sigmoid_group_topk_norm(_host(sl.logits[idx]).numpy(), _host(sl.bias).numpy(), s.K, s.n_group,
+                                            s.topk_group, s.routed_scale)
     assert np.array_equal(ids, ids_ref)
+    x, logits = sl.x[:n_decode].contiguous(), sl.logits[:n_decode].contiguous()
+    dec = _run(sl, x, logits)
+    ids = _routing_ids(sl, n_decode).cpu().numpy()
+    assert bool(torch.isfinite(dec.float()).all())
+    assert rel_l2(dec, from_bits(_fp8_oracle(sl, host, x, logits))) <= REL_L2_FP8, "fp8 decode batch vs C oracle"
+    _, ids_ref = co.sigmoid_group_topk_norm(_host(logits).numpy(), _host(sl.bias).numpy(), s.K, s.n_group,
+                                            s.topk_group, s.routed_scale)
+    assert np.array_equal(ids, ids_ref)
+    assert rel_l2(dec, full[:n_decode]) <= REL_L2_FP8, "fp8 decode and prefill kernels disagree"
+
+
+def test_dsv3_fp8_full_size():
+    """The fp8 block-scaled layer at the DeepSeek-V3 shape: 4096 tokens (sample) and 128 tokens (in full)."""
+    from vllm_kunlun_amd import synth
+    sl = synth.make_fp8_layer(synth.SHAPES["dsv3-fp8-prefill"], "cuda", seed=0)
+    _fp8_checks(sl, sl.host_weights(), n_decode=128, n_spot=16)
+
+
+def test_kimi_k2_full_size_int8():
+    """Kimi-K2 shape (384 experts + shared, sigmoid top-8 without groups, hidden 7168, intermediate 2048),
+    int8: 4096 and 128 tokens, bit for bit."""
+    from vllm_kunlun_amd import synth
+    sl = synth.make_w8a8_layer(synth.SHAPES["kimi-prefill"], "cuda", seed=0)
+    _properties(sl, sl.host_weights(), n_decode=128, n_spot=12, seed=3, mids=(480, 528))
+
+
+def test_kimi_k2_full_size_fp8():
+    """Kimi-K2 shape with fp8 block-scaled weights: 4096 tokens (sample) and 128 tokens (in full)."""
+    from vllm_kunlun_amd import synth
+    sl = synth.make_fp8_layer(synth.SHAPES["kimi-fp8-prefill"], "cuda", seed=0)
+    _fp8_checks(sl, sl.host_weights(), n_decode=128, n_spot=12)

@@ -511,3 +511,151 @@ def test_dequant_w4_against_the_reference_expression():
         assert torch.equal(got, ref)
     one = co.dequant_w4_bf16(np.array([[0x1F] * 8], np.uint8), bits(torch.tensor([[2.0]]).bfloat16()), 16)
     assert from_bits(one).tolist()[0][:2] == [14.0, -14.0]   # 0xF - 8 = 7 first (low nibble), 0x1 - 8 = -7 second
+
+
+# ------------------------------------------- bf16 and fp8 grouped GEMMs, and the layers built on them
+def _fp8_codes(t: torch.Tensor) -> np.ndarray:
+    """float tensor -> e4m3fn code bytes (torch's cast rounds to nearest even; values clamped to +-448 first,
+    the cast itself does not saturate)."""
+    return t.clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+
+
+def _fp8_values(codes: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(codes).view(torch.float8_e4m3fn).double()
+
+
+def test_grouped_gemm_bf16_against_f64_matmul_and_its_gather():
+    """y = bf16(a . w[e]^T) per expert: an f64 matmul of the same bf16 values differs by f32 summation and
+    one rounding only (rel-L2 of a few 1e-3, every element within 2 bf16 steps of the f64 result's scale);
+    the wrong expert's weights, a transposed operand or a dropped k is far outside. Gather == expanded copy,
+    fused SiLU-mul == silu_and_mul of the stored result, bit for bit."""
+    g = torch.Generator().manual_seed(21)
+    E, n, k, K, tokens = 4, 96, 160, 2, 9
+    a = torch.randn(tokens, k, generator=g).bfloat16()
+    w = (torch.randn(E, n, k, generator=g) * 0.05).bfloat16()
+    ids = torch.randint(0, E, (tokens * K,), generator=g).int().numpy()
+    ids[ids == 2] = 3                                   # expert 2 stays empty
+    _, src, _, lod = co.align(ids, E)
+    y = co.grouped_gemm_bf16(bits(a), bits(w), lod, row_src=src, src_div=K)
+    rows = a[torch.from_numpy(src // K).long()]
+    assert np.array_equal(y, co.grouped_gemm_bf16(bits(rows), bits(w), lod))          # gather == expanded copy
+    got = from_bits(y).double()
+    for e in range(E):
+        r0, r1 = int(lod[e]), int(lod[e + 1])
+        if r1 == r0:
+            continue
+        ref = rows[r0:r1].double() @ w[e].double().T
+        assert rel_l2(got[r0:r1], ref) <= 4e-3
+        assert float((got[r0:r1] - ref).abs().max()) <= ref.abs().max() * 2 ** -7
+        other = rows[r0:r1].double() @ w[(e + 1) % E].double().T
+        assert rel_l2(got[r0:r1], other) > 0.5                                         # the wrong expert's block
+    fused = co.grouped_gemm_bf16(bits(a), bits(w), lod, act=1, row_src=src, src_div=K)
+    assert np.array_equal(fused, co.silu_and_mul(y))
+
+
+def test_grouped_gemm_fp8_against_f64_block_scaled_product():
+    """y[r,c] = sum over 128-wide K blocks of (q_a . q_w) * s_a[r,kb] * s_w[e, c/128, kb]. Checked against
+    the same expression in f64 on torch's decoding of the codes. The scales differ per (row, block) and per
+    (channel block, K block) by factors of up to 8, so that swapping the two scale indices, taking one
+    scale for all blocks or dropping a block is far outside the tolerance (shown below for each)."""
+    g = torch.Generator().manual_seed(22)
+    E, n, k, K, tokens = 3, 256, 384, 2, 7
+    kb, nb = k // 128, n // 128
+    aq = _fp8_codes(torch.randn(tokens, k, generator=g) * 100)
+    wq = _fp8_codes(torch.randn(E, n, k, generator=g) * 100)
+    a_s = (2.0 ** torch.randint(-3, 1, (tokens, kb), generator=g).float()).numpy() * 1e-2
+    w_s = (2.0 ** torch.randint(-3, 1, (E, nb, kb), generator=g).float()).numpy() * 1e-3
+    ids = torch.randint(0, E, (tokens * K,), generator=g).int().numpy()
+    _, src, _, lod = co.align(ids, E)
+    y = co.grouped_gemm_fp8(aq, a_s, wq, w_s, lod, row_src=src, src_div=K)
+    tok = src // K
+    assert np.array_equal(y, co.grouped_gemm_fp8(aq[tok], a_s[tok], wq, w_s, lod))      # gather == expanded copy
+    got = from_bits(y).double()
+    af = _fp8_values(aq)[torch.from_numpy(tok).long()].view(-1, kb, 128)
+    sa = torch.from_numpy(a_s).double()[torch.from_numpy(tok).long()]
+
+    def product(e, r0, r1, sa_rows, sw):
+        wf = _fp8_values(wq[e]).view(n, kb, 128)
+        part = torch.einsum("rbk,nbk->rnb", af[r0:r1], wf)                             # [rows, n, kb], exact in f64
+        return (part * sa_rows[:, None, :] * sw.repeat_interleave(128, dim=0)[None]).sum(-1)
+
+    for e in range(E):
+        r0, r1 = int(lod[e]), int(lod[e + 1])
+        if r1 == r0:
+            continue
+        sw = torch.from_numpy(w_s[e]).double()
+        ref = product(e, r0, r1, sa[r0:r1], sw)
+        assert rel_l2(got[r0:r1], ref) <= 4e-3
+        assert float((got[r0:r1] - ref).abs().max()) <= ref.abs().max() * 2 ** -7
+        # plausible slips, each far outside: K-block order of either scale reversed, one scale for all blocks,
+        # the last K block dropped, the channel-block index of the weight scale swapped
+        assert rel_l2(got[r0:r1], product(e, r0, r1, sa[r0:r1].flip(1), sw)) > 0.1
+        assert rel_l2(got[r0:r1], product(e, r0, r1, sa[r0:r1], sw.flip(1))) > 0.1
+        assert rel_l2(got[r0:r1], product(e, r0, r1, sa[r0:r1, :1].expand(-1, kb), sw)) > 0.1
+        assert rel_l2(got[r0:r1], product(e, r0, r1, sa[r0:r1], sw.flip(0))) > 0.1
+        dropped = sa[r0:r1].clone()
+        dropped[:, -1] = 0
+        assert rel_l2(got[r0:r1], product(e, r0, r1, dropped, sw)) > 0.1
+    # act=1 is silu_and_mul of the stored act=0 result (gate = first half of the channels, up = second)
+    fused = co.grouped_gemm_fp8(aq, a_s, wq, w_s, lod, act=1, row_src=src, src_div=K)
+    assert np.array_equal(fused, co.silu_and_mul(y))
+
+
+def test_forward_bf16_without_biases_against_a_per_expert_loop():
+    """co.forward_bf16 (routing -> sort -> gate_up + SiLU-mul -> down -> combine) against a plain torch loop
+    in f64 over the same bf16 weights, softmax and sigmoid-grouped routing."""
+    g = torch.Generator().manual_seed(23)
+    M, H, E, K, I = 19, 128, 8, 3, 64
+    x = torch.randn(M, H, generator=g).bfloat16()
+    logits = torch.randn(M, E, generator=g)
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * 0.05).bfloat16()
+    w2 = (torch.randn(E, H, I, generator=g) * 0.05).bfloat16()
+    bias = torch.randn(E, generator=g) * 0.01
+    for scoring, n_group, topk_group, scale in (("softmax", 1, 1, 1.0), ("sigmoid", 4, 2, 2.5)):
+        out = co.forward_bf16(bits(x), logits.numpy(), bits(w13), bits(w2), K, scoring, True, n_group, topk_group,
+                              scale, bias.numpy() if scoring == "sigmoid" else None)
+        tw, ti = tm.route(logits, K, scoring, True, n_group, topk_group, scale, bias if scoring == "sigmoid" else None)
+        ref = torch.zeros(M, H, dtype=torch.double)
+        for m in range(M):
+            for j in range(K):
+                e = int(ti[m, j])
+                h = x[m].double() @ w13[e].double().T
+                ref[m] += tw[m, j].double() * ((F.silu(h[:I]) * h[I:]) @ w2[e].double().T)
+        assert rel_l2(from_bits(out), ref) <= 1e-2
+        assert rel_l2(from_bits(out), tm.bf16_moe(x, logits, w13, w2, K, True)) <= 1e-2 or scoring == "sigmoid"
+
+
+def test_forward_fp8_against_a_per_expert_loop():
+    """co.forward_fp8 (with a shared expert and the caller epilogue) against a torch loop built from the
+    torch oracle's fp8 quantiser and block GEMM, written independently of the C code."""
+    g = torch.Generator().manual_seed(24)
+    M, H, E, K, I, Is = 11, 256, 6, 2, 128, 256
+    x = torch.randn(M, H, generator=g).bfloat16()
+    logits = torch.randn(M, E, generator=g)
+    bias = torch.randn(E, generator=g) * 0.01
+    w13, s13 = tm.quantize_weight_fp8_block128(torch.randn(E, 2 * I, H, generator=g) * 0.05)
+    w2, s2 = tm.quantize_weight_fp8_block128(torch.randn(E, H, I, generator=g) * 0.05)
+    ws13, ss13 = tm.quantize_weight_fp8_block128(torch.randn(2 * Is, H, generator=g) * 0.05)
+    ws2, ss2 = tm.quantize_weight_fp8_block128(torch.randn(H, Is, generator=g) * 0.05)
+    codes = lambda t: t.view(torch.uint8).numpy()  # noqa: E731
+    out_scale = 2.5
+    out = co.forward_fp8(bits(x), logits.numpy(), codes(w13), s13.numpy(), codes(w2), s2.numpy(), K, "sigmoid", True, 3,
+                         2, 1.0, bias.numpy(), (codes(ws13), ss13.numpy(), codes(ws2), ss2.numpy()), out_scale)
+
+    def mlp(rows, wa, sa, wb, sb):
+        q, s = tm.quant_fp8_group128(rows)
+        a = tm.silu_and_mul(tm.fp8_block_gemm(q, s, wa, sa))
+        q, s = tm.quant_fp8_group128(a)
+        return tm.fp8_block_gemm(q, s, wb, sb)
+
+    tw, ti = tm.route(logits, K, "sigmoid", True, 3, 2, 1.0, bias)
+    ref = torch.zeros(M, H)
+    for m in range(M):
+        for j in range(K):
+            e = int(ti[m, j])
+            ref[m] += tw[m, j] * mlp(x[m:m + 1], w13[e], s13[e], w2[e], s2[e])[0].float()
+    ref = (ref.bfloat16().float() * out_scale).bfloat16().float() + mlp(x, ws13, ss13, ws2, ss2).float()
+    assert rel_l2(from_bits(out), ref) <= 1e-2
+    no_shared = co.forward_fp8(bits(x), logits.numpy(), codes(w13), s13.numpy(), codes(w2), s2.numpy(), K, "sigmoid",
+                               True, 3, 2, 1.0, bias.numpy())
+    assert rel_l2(from_bits(no_shared), ref) > 0.1     # the shared expert and the factor are not optional extras

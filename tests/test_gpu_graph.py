@@ -1,0 +1,89 @@
+"""HIP-graph capture of the layer and of the dense W8A8 op: what a serving engine does with the
+decode step. Each graph is replayed several times with new inputs and with eager work and
+synchronisations of the process between the replays; every replay must give the bits of the eager call."""
+import ctypes as C
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _eager_noise():
+    a = torch.randn(256, 256, device="cuda")
+    (a @ a).sum().item()
+
+
+def _replays(graph, static_inputs, fresh_inputs, static_out, eager):
+    for fresh in fresh_inputs:
+        for dst, src in zip(static_inputs, fresh):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = static_out.clone()
+        _eager_noise()
+        want = eager(*fresh)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+
+
+def test_apply_monolithic_under_graph_capture():
+    from vllm_kunlun_amd import synth
+    shape = synth.scaled(synth.SHAPES["dsv3-decode"], M=48, H=1024, E=32, K=4, I=256, n_group=4, topk_group=2,
+                         I_shared=256)
+    sl = synth.make_w8a8_layer(shape, "cuda", seed=5)
+    method, kw = sl.layer.quant_method, sl.apply_kwargs()
+    x, logits = sl.x.clone(), sl.logits.clone()
+    eager = lambda xx, ll: method.apply_monolithic(sl.layer, xx, ll, **kw)  # noqa: E731
+    eager(x, logits)                                   # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = method.apply_monolithic(sl.layer, x, logits, **kw)
+    g = torch.Generator(device="cuda").manual_seed(9)
+    fresh = [(torch.randn(shape.M, shape.H, generator=g, device="cuda").bfloat16(),
+              torch.randn(shape.M, shape.E, generator=g, device="cuda")) for _ in range(4)]
+    _replays(graph, (x, logits), fresh, out, eager)
+
+
+def test_static_workspace_forward_under_graph_capture():
+    from vllm_kunlun_amd import _lib as L
+    from vllm_kunlun_amd import synth
+    from vllm_kunlun_amd._plan import make_moe_plan
+    shape = synth.scaled(synth.SHAPES["qwen3-decode"], M=32, H=512, E=16, K=4, I=128)
+    sl = synth.make_w8a8_layer(shape, "cuda", seed=6)
+    lay = sl.layer
+    x, logits = sl.x.clone(), sl.logits.clone()
+    out = torch.empty_like(x)
+    plan = make_moe_plan(L.KMOE_FMT_INT8, x, logits, out, shape.K, lay.w13_weight, lay.w2_weight, lay.w13_weight_scale,
+                         lay.w2_weight_scale, "softmax", True)
+    call = lambda: L.check(L.lib.kmoe_moe_forward_static(C.byref(plan.args), L.stream()))  # noqa: E731
+    call()                                             # the first call on a GPU resolves the buffer's address
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    method = lay.quant_method
+    g = torch.Generator(device="cuda").manual_seed(10)
+    fresh = [(torch.randn(shape.M, shape.H, generator=g, device="cuda").bfloat16(),
+              torch.randn(shape.M, shape.E, generator=g, device="cuda")) for _ in range(3)]
+    _replays(graph, (x, logits), fresh, out, lambda xx, ll: method.apply_monolithic(lay, xx, ll))
+
+
+def test_dense_matmul_op_under_graph_capture():
+    import vllm_kunlun_amd  # noqa: F401  (registers torch.ops._C.*)
+    M, n, k = 24, 256, 512
+    g = torch.Generator(device="cuda").manual_seed(11)
+    w = torch.randint(-127, 128, (n, k), generator=g, device="cuda", dtype=torch.int8)
+    w_max = torch.rand(n, 1, generator=g, device="cuda") + 0.5
+    x = torch.randint(-127, 128, (M, k), generator=g, device="cuda", dtype=torch.int8)
+    x_max = torch.rand(M, 1, generator=g, device="cuda") + 0.5
+    eager = lambda xx, mm: torch.ops._C.matmul(xx, w, torch.bfloat16, x_pc_max=mm, w_pc_max=w_max)  # noqa: E731
+    eager(x, x_max)                                    # uploads the {0, M} row range once
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = eager(x, x_max)
+    fresh = [(torch.randint(-127, 128, (M, k), generator=g, device="cuda", dtype=torch.int8),
+              torch.rand(M, 1, generator=g, device="cuda") + 0.5) for _ in range(3)]
+    _replays(graph, (x, x_max), fresh, out, eager)

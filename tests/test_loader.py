@@ -1,7 +1,8 @@
 """Checkpoint -> layer: compressed-tensors `int-quantized` expert tensors (format of
 docs/source/tutorials/multi_xpu_DeepSeek-V3.2-Exp-w8a8.md:50-95) through the method
 selection of compressed_tensors_moe.py:43-108 and the expert mapping of
-models/deepseek_v2.py:1296-1384. Host logic: runs without a GPU."""
+models/deepseek_v2.py:1296-1384. The host logic runs without a GPU; the `gpu` tests at the end run the
+loaded layer against the oracle on the checkpoint's own tensors."""
 import json
 
 import pytest
@@ -121,34 +122,109 @@ def test_weight_loader_rejects_what_does_not_fit():
     assert torch.all(layer.w2_weight_scale[1] == 0.5) and torch.all(layer.w2_weight_scale[0] == 0)
 
 
+def _oracle_weights(ckpt, E, prefix="model.layers.3.mlp."):
+    """The checkpoint's tensors stacked the way the reference's layer holds them, as numpy arrays for the
+    oracle: w13 [E,2I,H] (gate rows first), w2 [E,H,I], and the absmax per channel (= 127 x scale, what
+    process_weights_after_loading makes of the scales, compressed_tensors_moe.py:116-120)."""
+    import numpy as np
+    cat = lambda e, suf: torch.cat([ckpt[f"{prefix}experts.{e}.gate_proj.{suf}"],  # noqa: E731
+                                    ckpt[f"{prefix}experts.{e}.up_proj.{suf}"]])
+    w13 = torch.stack([cat(e, "weight") for e in range(E)]).numpy()
+    w2 = torch.stack([ckpt[f"{prefix}experts.{e}.down_proj.weight"] for e in range(E)]).numpy()
+    w13_max = (torch.stack([cat(e, "weight_scale") for e in range(E)]) * 127.0).reshape(E, -1).numpy()
+    w2_max = (torch.stack([ckpt[f"{prefix}experts.{e}.down_proj.weight_scale"] for e in range(E)]) * 127.0)
+    return w13, w13_max.astype(np.float32), w2, w2_max.reshape(E, -1).numpy().astype(np.float32)
+
+
 @pytest.mark.gpu
-def test_loaded_layer_computes_what_the_directly_built_layer_does():
-    E, H, I, M, K = 8, 256, 128, 40, 2
+@pytest.mark.parametrize("I", [128, 96])  # 96: padded with zero channels at load time so that the weights tile
+def test_loaded_layer_matches_the_oracle_on_the_checkpoint_tensors(I):
+    """Checkpoint -> load_weights -> process_weights_after_loading -> forward on the GPU, against the C
+    oracle fed with the checkpoint's own tensors (never touched by the loader), bit for bit."""
+    import numpy as np
+    from conftest import bits
+    from oracle import c_oracle as co
+    E, H, M, K = 8, 256, 40, 2
     ckpt = _checkpoint(E, H, I)
-    layers = []
-    for how in ("loader", "direct"):
-        method = KunlunCompressedTensorsW8A8Int8MoEMethod()
-        layer = FusedMoE(num_experts=E, top_k=K, hidden_size=H, intermediate_size=I, quant_method=method,
-                         device="cuda")
-        if how == "loader":
-            layer.load_weights(ckpt.items())
-        else:
-            p = "model.layers.3.mlp."
-            for e in range(E):
-                layer.w13_weight.data[e].copy_(torch.cat([ckpt[f"{p}experts.{e}.gate_proj.weight"],
-                                                          ckpt[f"{p}experts.{e}.up_proj.weight"]]))
-                layer.w13_weight_scale.data[e].copy_(torch.cat([ckpt[f"{p}experts.{e}.gate_proj.weight_scale"],
-                                                                ckpt[f"{p}experts.{e}.up_proj.weight_scale"]]))
-                layer.w2_weight.data[e].copy_(ckpt[f"{p}experts.{e}.down_proj.weight"])
-                layer.w2_weight_scale.data[e].copy_(ckpt[f"{p}experts.{e}.down_proj.weight_scale"])
-        method.process_weights_after_loading(layer)
-        layers.append(layer)
+    method = KunlunCompressedTensorsW8A8Int8MoEMethod()
+    layer = FusedMoE(num_experts=E, top_k=K, hidden_size=H, intermediate_size=I, quant_method=method, device="cuda")
+    loaded = layer.load_weights(ckpt.items())
+    assert len(loaded) == 6 * E
+    method.process_weights_after_loading(layer)
     with pytest.raises(RuntimeError):  # the codes were re-tiled in place: loading now would corrupt them
-        layers[0].weight_loader(layers[0].w13_weight, torch.zeros(I, H, dtype=torch.int8), "x", shard_id="w1",
-                                expert_id=0)
+        layer.weight_loader(layer.w13_weight, torch.zeros(I, H, dtype=torch.int8), "x", shard_id="w1", expert_id=0)
     g = torch.Generator(device="cuda").manual_seed(1)
     x = torch.randn(M, H, generator=g, device="cuda").bfloat16()
     logits = torch.randn(M, E, generator=g, device="cuda")
-    a, b = layers[0](x, logits), layers[1](x, logits)
+    out = layer(x, logits)
     torch.cuda.synchronize()
-    assert torch.equal(a, b) and bool(a.float().abs().sum() > 0)
+    w13, w13_max, w2, w2_max = _oracle_weights(ckpt, E)
+    ref = co.forward_w8a8(bits(x), logits.cpu().numpy(), w13, w13_max, w2, w2_max, K, "softmax", True)
+    assert np.array_equal(bits(out), ref)
+
+
+@pytest.mark.gpu
+def test_shared_fused_moe_returns_shared_and_routed_parts():
+    """SharedFusedMoE (reference use: models/deepseek_v2.py:241-284) returns (shared_output, routed_output):
+    the routed part against the oracle's layer without a shared expert, the shared part (a dense W8A8 MLP of
+    two KunlunScaledMMLinearKernel linears, as the model builds it) against the oracle's dense MLP, and their
+    caller-side sum `routed * scale + shared` (deepseek_v2.py:288-296) against the oracle's layer with the
+    shared expert and the factor folded in - all bit for bit."""
+    import numpy as np
+    from types import SimpleNamespace
+    from conftest import bits, from_bits
+    from oracle import c_oracle as co
+    from oracle import torch_moe as tm
+    from vllm_kunlun_amd.ops.fused_moe.layer import SharedFusedMoE
+    from vllm_kunlun_amd.quantization.kernels.scale_mm import KunlunScaledMMLinearKernel
+    E, H, I, Is, M, K, scale = 16, 256, 128, 192, 24, 4, 2.5
+    ckpt = _checkpoint(E, H, I)
+    g = torch.Generator().manual_seed(5)
+    kern = KunlunScaledMMLinearKernel()
+
+    def linear(n, k):
+        wq, sc = tm.quantize_weight_per_channel(torch.randn(n, k, generator=g) * 0.05)
+        lin = SimpleNamespace(weight=torch.nn.Parameter(wq.cuda(), requires_grad=False),
+                              weight_scale=torch.nn.Parameter(sc.clone().cuda(), requires_grad=False), input_scale=None)
+        kern.process_weights_after_loading(lin)
+        return lin, wq.numpy(), (sc * 127.0).reshape(n).numpy()
+
+    up, ws13, ws13_max = linear(2 * Is, H)
+    down, ws2, ws2_max = linear(H, Is)
+
+    class SharedMLP(torch.nn.Module):
+        def forward(self, x):
+            y = kern.apply_weights(up, x)
+            act = torch.empty(x.shape[0], Is, dtype=x.dtype, device=x.device)
+            torch.ops._C.silu_and_mul(act, y)
+            return kern.apply_weights(down, act)
+
+    bias = (torch.randn(E, generator=g) * 0.01).cuda()
+    method = KunlunCompressedTensorsW8A8Int8MoEMethod()
+    layer = SharedFusedMoE(shared_experts=SharedMLP(), num_experts=E, top_k=K, hidden_size=H, intermediate_size=I,
+                           use_grouped_topk=True, num_expert_group=4, topk_group=2, scoring_func="sigmoid",
+                           e_score_correction_bias=bias, quant_method=method, device="cuda")
+    layer.load_weights(ckpt.items())
+    method.process_weights_after_loading(layer)
+    x = torch.randn(M, H, generator=g).bfloat16().cuda()
+    logits = torch.randn(M, E, generator=g).cuda()
+    shared_out, routed_out = layer(x, logits)
+    torch.cuda.synchronize()
+    assert isinstance(shared_out, torch.Tensor) and shared_out.shape == routed_out.shape == (M, H)
+    w13, w13_max, w2, w2_max = _oracle_weights(ckpt, E)
+    common = (bits(x), logits.cpu().numpy(), w13, w13_max, w2, w2_max, K, "sigmoid", True, 4, 2, 1.0, bias.cpu().numpy())
+    assert np.array_equal(bits(routed_out), co.forward_w8a8(*common))
+    lod = np.array([0, M], dtype=np.int32)
+    xq, x_max = co.quant_i8_rows(bits(x))
+    a_ref = co.grouped_gemm_i8(xq, x_max, ws13[None], ws13_max[None], lod, act=1)[0]
+    aq, a_max = co.quant_i8_rows(a_ref)
+    sh_ref = co.grouped_gemm_i8(aq, a_max, ws2[None], ws2_max[None], lod)[0]
+    assert np.array_equal(bits(shared_out), sh_ref)
+    # the caller's epilogue in torch, as the model writes it, equals the oracle's folded epilogue
+    final = routed_out * scale + shared_out
+    ref = co.forward_w8a8(*common, (ws13, ws13_max, ws2, ws2_max), out_scale=scale)
+    assert np.array_equal(bits(final), ref)
+    # SharedFusedMoE without a shared module returns (None, routed)
+    layer.shared_experts = None
+    none_out, routed_again = layer(x, logits)
+    assert none_out is None and torch.equal(routed_again, routed_out)

@@ -111,3 +111,49 @@ def test_shared_expert_mlp_through_two_linears():
     # and the torch restatement of the reference's two scaled_int8_quant -> matmul steps agrees within bf16 rounding
     t_ref = tm.w8a8_dense(x, w13q, w13_max.reshape(-1, 1), w2q, w2_max.reshape(-1, 1))
     assert (out.cpu().float() - t_ref.float()).norm() / t_ref.float().norm() <= 1e-2
+
+
+@pytest.mark.gpu
+def test_ops_on_weights_that_were_tiled_at_load_time():
+    """The operators take weights by tensor: `_C::matmul` gets `layer.weight.t()` as in the reference
+    (scale_mm.py:83-90) after process_weights_after_loading re-tiled the storage in place, `_C::moe_fc`
+    gets the bf16 layer's w13 after KunlunUnquantizedFusedMoEMethod tiled it. Both must see the tiling
+    (it belongs to the memory, not to a tensor object) and give the oracle's result; a view that cannot
+    be served is refused instead of being read as row-major."""
+    import vllm_kunlun_amd  # noqa: F401
+    from conftest import rel_l2
+    from vllm_kunlun_amd import _plan
+    from vllm_kunlun_amd.ops.fused_moe.layer import FusedMoE
+    from vllm_kunlun_amd.quantization.kernels.scale_mm import KunlunScaledMMLinearKernel
+    M, n, k = 40, 256, 512
+    layer, wq, w_max = _layer(n, k, "cuda", 21)
+    kern = KunlunScaledMMLinearKernel()
+    kern.process_weights_after_loading(layer)
+    assert _plan.is_tiled(layer.weight) and layer.weight.shape == (k, n)
+    x = (torch.randn(M, k, generator=torch.Generator().manual_seed(22)) * 1.5).bfloat16()
+    x_q, x_s, _, _ = torch.ops._C.scaled_int8_quant(x.cuda(), None, None, True)
+    out = torch.ops._C.matmul(x_q, layer.weight.transpose(0, 1), torch.bfloat16, x_pc_max=x_s,
+                              w_pc_max=layer.weight_scale)
+    torch.cuda.synchronize()
+    xq, x_max = co.quant_i8_rows(bits(x))
+    ref, _ = co.grouped_gemm_i8(xq, x_max, wq.numpy()[None], w_max.numpy()[None], np.array([0, M], np.int32))
+    assert np.array_equal(bits(out), ref)
+    with pytest.raises(ValueError):  # the [k, n] view itself is not something the kernels can read
+        torch.ops._C.matmul(x_q[:, :n].contiguous(), layer.weight, torch.bfloat16, x_pc_max=x_s,
+                            w_pc_max=layer.weight_scale[:k])
+
+    # bf16 grouped GEMM on a tiled bf16 layer
+    E, H, I, rows = 4, 256, 128, 50
+    g = torch.Generator().manual_seed(23)
+    moe = FusedMoE(num_experts=E, top_k=2, hidden_size=H, intermediate_size=I, device="cuda")
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * 0.05).bfloat16()
+    moe.w13_weight.data.copy_(w13)
+    moe.quant_method.process_weights_after_loading(moe)
+    assert _plan.is_tiled(moe.w13_weight)
+    a = torch.randn(rows, H, generator=g).bfloat16()
+    lod = torch.tensor([0, 20, 20, 37, 50], dtype=torch.int32)
+    y = torch.empty(rows, 2 * I, dtype=torch.bfloat16, device="cuda")
+    torch.ops._C.moe_fc(a.cuda(), moe.w13_weight, lod.cuda(), torch.empty(0, dtype=torch.int32, device="cuda"), 2, y)
+    torch.cuda.synchronize()
+    ref = co.grouped_gemm_bf16(bits(a), bits(w13), lod.numpy())
+    assert rel_l2(y, from_bits(ref)) <= 1e-2

@@ -473,6 +473,11 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
     rc = fill_dense_lod(dense_lod, stream_mode ? 0 : M, as_stream(stream));  // (streaming path: see below)
     if (rc) return rc;
     MlpPass sh = routed;
+    // the expert-bias branch belongs to the routed experts only: a dense shared MLP has no per-expert
+    // bias and uses the plain SiLU-mul over [gate | up] rows
+    sh.w13_bias = nullptr;
+    sh.w2_bias = nullptr;
+    sh.oai = 0;
     sh.tail_rows = 0;
     sh.row_src = nullptr;
     sh.src_div = 1;

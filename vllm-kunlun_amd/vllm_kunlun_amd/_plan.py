@@ -2,10 +2,13 @@
 
 A plan binds fixed device buffers (x, logits, out, weights); calling it enqueues
 the whole layer on the current HIP stream without allocating or synchronising,
-so a serving loop — or a HIP-graph capture — can replay it.
+so a serving loop — or a HIP-graph capture — can replay it. A plan belongs to the
+stream that was current when it was built (its workspace is that stream's) and
+refuses to launch on another.
 """
 from __future__ import annotations
 
+import weakref
 from typing import Optional
 
 import torch
@@ -13,15 +16,21 @@ import torch
 from . import _lib as L
 
 
+def _current_stream_id(device: torch.device) -> int:
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
 class _Workspace:
-    """Per-device scratch buffer that only grows (plays the role of vLLM's
-    current_workspace_manager(), reference: vllm_kunlun/ops/_kunlun_ops.py:528-531)."""
+    """Scratch buffers that only grow, one per (device, stream) (plays the role of vLLM's
+    current_workspace_manager(), reference: vllm_kunlun/ops/_kunlun_ops.py:528-531). Work queued on one
+    stream runs in order, so the calls of a stream can share a buffer; two streams cannot, and a buffer is
+    only ever used on the stream it was allocated on (the caching allocator's own rule for reuse)."""
 
     def __init__(self):
         self._buf = {}
 
-    def get(self, nbytes: int, device: torch.device) -> torch.Tensor:
-        key = (device.type, device.index)
+    def get(self, nbytes: int, device: torch.device, stream_id: int) -> torch.Tensor:
+        key = (device.type, device.index, stream_id)
         buf = self._buf.get(key)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -33,10 +42,21 @@ WORKSPACE = _Workspace()
 
 
 class MoEPlan:
-    def __init__(self, args, layout, workspace, keepalive):
+    """A filled kmoe_moe_args block and its workspace, bound to the stream it was built on."""
+
+    def __init__(self, args, layout, workspace, keepalive, stream_id=None):
         self.args, self.layout, self.workspace, self._keep = args, layout, workspace, keepalive
+        self.stream_id = stream_id
 
     def __call__(self) -> None:
+        if self.stream_id is not None:
+            now = _current_stream_id(self.workspace.device)
+            if now != self.stream_id:
+                raise RuntimeError(
+                    f"this MoE plan was built on stream {self.stream_id:#x} and is being launched on stream "
+                    f"{now:#x}: its workspace belongs to the first stream (two streams sharing it would race). "
+                    "Build the plan with the launching stream current (inside `with torch.cuda.stream(s)` or the "
+                    "graph capture that will run it).")
         L.check(L.lib.kmoe_moe_forward(self.args, L.ptr(self.workspace), self.workspace.numel(), L.stream()))
 
     def view(self, name: str, count: int, dtype: torch.dtype) -> torch.Tensor:
@@ -46,10 +66,36 @@ class MoEPlan:
         return self.workspace[off: off + nbytes].view(dtype)
 
 
+# Which device memory holds re-tiled weights. The mark belongs to the STORAGE (keyed by the address of
+# torch's StorageImpl, dropped when the storage dies), not to a tensor object: views, `.data`, `.detach()`,
+# `.t()` and a Parameter wrapped around the same memory all see it.
+_TILED: dict[int, tuple[int, int]] = {}  # storage -> (n, bytes of k) of the tiles it holds
+
+
+def _mark_tiled(w: torch.Tensor, n: int, k_bytes: int) -> None:
+    storage = w.untyped_storage()
+    key = storage._cdata
+    _TILED[key] = (n, k_bytes)
+    weakref.finalize(storage, _TILED.pop, key, None)
+
+
 def is_tiled(w: torch.Tensor) -> bool:
-    """True if tile_int8_weights_ re-arranged this tensor. The mark lives on the tensor
-    (or Parameter) OBJECT: views and copies made afterwards do not carry it."""
-    return bool(getattr(w, "_kmoe_tiled", False))
+    """True if the memory behind this tensor was re-arranged by tile_int8_weights_ (whatever view of it
+    the tensor is)."""
+    return w.untyped_storage()._cdata in _TILED
+
+
+def weight_layout(w: torch.Tensor) -> int:
+    """KMOE_W_TILED or KMOE_W_ROWMAJOR for a weight handed to an operator. A tensor over tiled memory must
+    be the contiguous [..., n, k] tensor that was tiled (or a leading-dimension slice of it): any other
+    view (a transpose, a column slice) would read scrambled values, so it is refused."""
+    tiles = _TILED.get(w.untyped_storage()._cdata)
+    if tiles is None:
+        return L.KMOE_W_ROWMAJOR
+    if w.dim() < 2 or not w.is_contiguous() or (w.shape[-2], w.shape[-1] * w.element_size()) != tiles:
+        raise ValueError(f"this tensor {tuple(w.shape)} is a view of weights that were re-tiled as "
+                         f"[..., {tiles[0]}, {tiles[1]} bytes]: pass the contiguous [..., n, k] tensor itself")
+    return L.KMOE_W_TILED
 
 
 _TILEABLE = (torch.int8, torch.uint8, torch.float8_e4m3fn, torch.bfloat16)
@@ -58,7 +104,7 @@ _TILEABLE = (torch.int8, torch.uint8, torch.float8_e4m3fn, torch.bfloat16)
 def tile_int8_weights_(w: torch.Tensor) -> bool:
     """Re-arranges weights [..., n, k] (int8, e4m3 codes, or bf16 — the kernel moves BYTES: a
     1 KB block is 16 channels x 64 bytes of K) IN PLACE into the MFMA-ready blocks of
-    kmoe_tile_weights_i8 (one expert at a time through a scratch copy) and marks the object.
+    kmoe_tile_weights_i8 (one expert at a time through a scratch copy) and marks the memory as tiled.
     Returns False and leaves the tensor alone when the shape does not allow it (n % 16,
     64 bytes of K)."""
     data = w.data
@@ -74,7 +120,7 @@ def tile_int8_weights_(w: torch.Tensor) -> bool:
     for e in range(flat.shape[0]):
         L.check(L.lib.kmoe_tile_weights_i8(L.ptr(flat[e]), L.ptr(tmp), 1, n, k, L.stream()))
         flat[e].copy_(tmp)
-    w._kmoe_tiled = True
+    _mark_tiled(data, n, k)
     return True
 
 
@@ -216,5 +262,11 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
         keep.append(stage_events)
     lay = L.MoELayout()
     L.check(L.lib.kmoe_moe_workspace_layout(a, lay))
-    ws = WORKSPACE.get(lay.total_bytes, x.device)
-    return MoEPlan(a, lay, ws, keep)
+    stream_id = _current_stream_id(x.device)
+    if torch.cuda.is_current_stream_capturing():
+        # memory allocated during a capture belongs to the graph's pool: the plan owns this buffer, it is
+        # not shared with later plans
+        ws = torch.empty(max(int(lay.total_bytes), 1), dtype=torch.uint8, device=x.device)
+    else:
+        ws = WORKSPACE.get(lay.total_bytes, x.device, stream_id)
+    return MoEPlan(a, lay, ws, keep, stream_id)

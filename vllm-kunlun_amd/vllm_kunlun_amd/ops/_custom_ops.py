@@ -203,7 +203,7 @@ def scaled_int8_quant(x: torch.Tensor, scale: Optional[torch.Tensor], azp: Optio
 
 # ------------------------------------------------------------------------ GEMM
 def _gemm_i8(a, a_max, w, w_max, lod, y2d, ldy, act, rows, row_src=None, src_div=1, acc_out=None, variant=0):
-    from .._plan import is_tiled
+    from .._plan import weight_layout
     E, n, k = w.shape
     args = L.GemmI8Args()
     args.a = a.data_ptr()
@@ -220,7 +220,7 @@ def _gemm_i8(a, a_max, w, w_max, lod, y2d, ldy, act, rows, row_src=None, src_div
     args.acc_out = 0 if acc_out is None else acc_out.data_ptr()
     args.act = act
     args.variant = variant
-    args.w_layout = L.KMOE_W_TILED if is_tiled(w) else L.KMOE_W_ROWMAJOR
+    args.w_layout = weight_layout(w)
     L.check(L.lib.kmoe_grouped_gemm_i8(args, L.stream()))
 
 
@@ -261,9 +261,28 @@ def moe_fc(x: torch.Tensor, weight: torch.Tensor, sorted_tokens_num_lod: torch.T
         g.E, g.n, g.k, g.rows = E, n, k, rows
         g.y, g.ldy = y.data_ptr(), n
         g.act = L.KMOE_ACT_SWIGLU if act else L.KMOE_ACT_NONE
+        from .._plan import weight_layout
+        g.w_layout = weight_layout(weight)
         L.check(L.lib.kmoe_grouped_gemm_bf16(g, L.stream()))
     else:
         raise NotImplementedError(f"moe_fc: x dtype {x.dtype} is outside this build's path (int8 or bfloat16)")
+
+
+_DENSE_LOD: dict = {}
+
+
+def _dense_lod(device: torch.device, rows: int) -> torch.Tensor:
+    """The row range {0, rows} of a dense GEMM's single expert, on the device; made once per
+    (device, rows) so that a replayed or captured call copies nothing from the host."""
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device(), rows)
+    lod = _DENSE_LOD.get(key)
+    if lod is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(f"matmul: run one call with {rows} rows before capturing (its row range is "
+                               "uploaded once per size)")
+        lod = torch.tensor([0, rows], dtype=torch.int32).to(device)
+        _DENSE_LOD[key] = lod
+    return lod
 
 
 @custom_op("_C::matmul", mutates_args=())
@@ -281,12 +300,16 @@ def matmul(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, x_trans: bo
     if out_dtype != _BF16:
         raise NotImplementedError(f"matmul: out_dtype {out_dtype} is not implemented")
     L.require_device(x, w, x_pc_max, w_pc_max)
-    xc, wc = x.contiguous(), w.contiguous()
+    from .._plan import is_tiled
+    # weights re-tiled at load time come in as a view of their memory (e.g. layer.weight.t()): a copy made by
+    # .contiguous() would shuffle tiled bytes, so such a weight must already be the contiguous [n, k] tensor
+    # (_gemm_i8 refuses any other view of tiled memory)
+    xc, wc = x.contiguous(), (w if is_tiled(w) else w.contiguous())
     M, k = xc.shape
     n = wc.shape[0]
     out = torch.empty((M, n), dtype=out_dtype, device=x.device)
-    lod = torch.tensor([0, M], dtype=torch.int32).to(x.device, non_blocking=True)
-    _gemm_i8(xc, x_pc_max.contiguous(), wc.view(1, n, k), w_pc_max.contiguous(), lod, out, n, L.KMOE_ACT_NONE, M)
+    _gemm_i8(xc, x_pc_max.contiguous(), wc.unsqueeze(0), w_pc_max.contiguous(), _dense_lod(x.device, M), out, n,
+             L.KMOE_ACT_NONE, M)
     return out
 
 

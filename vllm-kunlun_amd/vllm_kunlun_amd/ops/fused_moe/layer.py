@@ -128,7 +128,8 @@ class FusedMoE(torch.nn.Module):
         process_weights_after_loading (which re-tiles the codes in place)."""
         if shard_id not in ("w1", "w2", "w3"):
             raise ValueError(f"shard_id must be w1, w2 or w3, got {shard_id}")
-        if getattr(param, "_kmoe_tiled", False):
+        from ..._plan import is_tiled
+        if is_tiled(param):
             raise RuntimeError("weight_loader: this parameter was already re-tiled by process_weights_after_loading")
         if not 0 <= expert_id < param.shape[0]:
             return False if return_success else None

@@ -82,10 +82,8 @@ class KunlunScaledMMLinearKernel:
         scale = scale.contiguous().clone().reshape(n, 1)
         with torch.no_grad():
             scale.mul_(127.0)  # scale -> absmax, what the kernels take (x_pc_max / w_pc_max convention)
-        tile_int8_weights_(w_nk)  # in place, marks the tensor; shapes that do not tile stay row-major
-        w_1nk = w_nk.view(1, n, k)  # what the grouped GEMM takes; the tiling mark lives on the tensor object
-        w_1nk._kmoe_tiled = is_tiled(w_nk)
-        layer._kmoe_w_1nk = w_1nk
+        tile_int8_weights_(w_nk)  # in place, marks the memory; shapes that do not tile stay row-major
+        layer._kmoe_w_1nk = w_nk.view(1, n, k)  # what the grouped GEMM takes
         setattr(layer, w_q_name, torch.nn.Parameter(w_nk.t(), requires_grad=False))
         setattr(layer, w_s_name, torch.nn.Parameter(scale, requires_grad=False))
         if getattr(layer, i_s_name, None) is not None and not self.config.is_static_input_scheme:

@@ -228,3 +228,48 @@ def test_shared_fused_moe_returns_shared_and_routed_parts():
     layer.shared_experts = None
     none_out, routed_again = layer(x, logits)
     assert none_out is None and torch.equal(routed_again, routed_out)
+
+
+def test_config_get_quant_method_dispatches_on_the_kind_of_layer():
+    """KunlunCompressedTensorsConfig.get_quant_method: the call vLLM makes for every layer
+    (reference: compressed_tensors.py:49-82)."""
+    from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors import (
+        KunlunCompressedTensorsConfig, KunlunCompressedTensorsW8A8Int8LinearMethod, UnquantizedLinearMethod,
+        register_with_vllm)
+    from vllm_kunlun_amd.quantization.kernels.scale_mm import KunlunScaledMMLinearKernel
+    cfg = KunlunCompressedTensorsConfig.from_config(QUANT_CONFIG)
+    assert cfg.get_name() == "compressed-tensors"
+    moe = FusedMoE(num_experts=2, top_k=1, hidden_size=64, intermediate_size=32)
+    m = cfg.get_quant_method(moe, "model.layers.3.mlp.experts")
+    assert isinstance(m, KunlunCompressedTensorsW8A8Int8MoEMethod) and m.moe is moe.moe_config
+
+    class LinearBase(torch.nn.Module):           # stands for vLLM's class of that name
+        pass
+
+    class ColumnParallelLinear(LinearBase):
+        pass
+
+    lin = ColumnParallelLinear()
+    lm = cfg.get_quant_method(lin, "model.layers.3.mlp.shared_experts.gate_up_proj")
+    assert isinstance(lm, KunlunCompressedTensorsW8A8Int8LinearMethod)
+    assert isinstance(lm.kernel, KunlunScaledMMLinearKernel) and lin.scheme["weights"]["num_bits"] == 8
+    lm.create_weights(lin, 64, [32, 32])
+    assert lin.weight.shape == (64, 64) and lin.weight.dtype == torch.int8 and lin.weight_scale.shape == (64, 1)
+    lm.process_weights_after_loading(lin)        # host: scale -> absmax, weight as the [k, n] view
+    assert lin.weight.shape == (64, 64) and lin.input_scale is None
+    assert isinstance(cfg.get_quant_method(ColumnParallelLinear(), "lm_head"), UnquantizedLinearMethod)  # ignored
+    assert isinstance(cfg.get_quant_method(torch.nn.Linear(4, 4), "model.layers.0.mlp.down_proj"),
+                      KunlunCompressedTensorsW8A8Int8LinearMethod)
+
+    class Attention(torch.nn.Module):
+        pass
+
+    assert cfg.get_quant_method(Attention(), "model.layers.3.self_attn.attn") is None
+    assert cfg.get_quant_method(torch.nn.LayerNorm(4), "model.norm") is None
+    # a Linear scheme that is not on the path is refused by name, not served wrongly
+    static = json.loads(json.dumps(QUANT_CONFIG))
+    static["config_groups"]["group_0"]["input_activations"]["dynamic"] = False
+    with pytest.raises(NotImplementedError):
+        KunlunCompressedTensorsConfig.from_config(static).get_quant_method(lin, "model.layers.1.mlp.up_proj")
+    with pytest.raises(ImportError):             # vLLM is not installed here: the hook says so
+        register_with_vllm()

@@ -215,7 +215,7 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
                              getattr(lay, "w13_weight_scale", None), getattr(lay, "w2_weight_scale", None),
                              shape.scoring, True, shape.n_group, shape.topk_group, shape.routed_scale, sl.bias,
                              sl.shared, 1.0, stage_events, router_weight=w_gate,
-                             group_size=shape.group_size if w4 else None)
+                             group_size=shape.group_size if w4 else None, tile_variant=a.tile_variant)
 
     # The layer, its inputs and the workspace were produced on the default stream;
     # finish that work before a second stream touches (recycled) memory.
@@ -306,7 +306,7 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
                    "experts": shape.E, "top_k": shape.K, "moe_intermediate": shape.I,
                    "shared_intermediate": shape.I_shared, "routing": shape.scoring, "experts_hit": n_active,
                    "launch": launch_mode, "launch_ms_per_step": launch_ms, "seed": a.seed,
-                   "router_gemm_inside": bool(a.router)},
+                   "router_gemm_inside": bool(a.router), "tile_variant": a.tile_variant},
         "roofline": roofline,
         "layer": {"hbm_gbs": work["layer_bytes"] / t_s / 1e9, "hbm_frac": work["layer_bytes"] / t_s / 1e9 / HBM_PEAK_GBS,
                   "tops": work["layer_ops"] / t_s / 1e12,
@@ -343,6 +343,9 @@ def main():
     ap.add_argument("--dims", default="",
                     help="other layer dimensions for the workload's format and routing, e.g. "
                          "H=4096,E=8,K=2,I=14336,I_shared=0 (Mixtral-8x7B); the config then says so")
+    ap.add_argument("--tile-variant", type=int, default=0,
+                    help="tuning variant of the int8 tile kernel for the routed GEMMs of prefill-sized batches "
+                         "(kmoe_moe_args.tile_variant; 12: sibling m-tiles paced so that they share weight bytes in L2)")
     ap.add_argument("--yardstick", action="store_true",
                     help="also time the vendor library's dense GEMM (torch._int_mm / bf16 matmul) with the gate_up "
                          "GEMM's operation count: [P,H] x [H,2I], one weight matrix, no gather, no epilogue")

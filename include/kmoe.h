@@ -178,8 +178,10 @@ typedef struct kmoe_gemm_i8_args {
   int32_t act;            /* KMOE_ACT_*                                         */
   int32_t variant;        /* 0 = choose from the shape. Tuning and tests: 1-3 LDS-staged 16/32/64-row
                              kernels; with tiled weights 5 = tile kernel (6: 128-row tiles, 11: 64-row
-                             tiles, 7-9: other tile shapes; all need k >= 128); with chunked activations 1, 2, 4, 8 =
-                             16-row fragments per pass of the streaming kernel      */
+                             tiles, 7-9: other tile shapes, 12: 128-row tiles whose m-tiles of one expert and
+                             channel block keep in step so that they share the weight bytes in L2; all need
+                             k >= 128); with chunked activations 1, 2, 4, 8 = 16-row fragments per pass of the
+                             streaming kernel                                       */
   int32_t w_layout;       /* KMOE_W_ROWMAJOR, or KMOE_W_TILED (kmoe_tile_weights_i8) */
   int32_t a_layout;       /* KMOE_A_ROWMAJOR, or KMOE_A_CHUNKED: a is [k/64][a_rows][64]
                              (kmoe_quant_i8_rows_chunked); needs w_layout TILED   */
@@ -441,6 +443,8 @@ typedef struct kmoe_moe_args {
   const uint16_t* w13_scale; /* [E,2I,H/group_size] bf16                               */
   const uint16_t* w2_scale;  /* [E,H,I/group_size] bf16                                */
   int32_t group_size;    /* a multiple of 32 dividing H and I (one value for both tensors) */
+  int32_t tile_variant;  /* INT8, tuning: 0, or the `variant` (5-12) handed to the two routed GEMMs when the batch
+                            runs on the tile kernel (more than 10 rows per expert); ignored otherwise */
 } kmoe_moe_args;
 
 #define KMOE_STAGE_ROUTING 0

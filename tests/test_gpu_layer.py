@@ -264,3 +264,28 @@ def test_layer_with_the_router_inside(base, over):
     got = m.apply_monolithic(sl.layer, sl.x, None, router_weight=gate.weight, **kw)
     torch.cuda.synchronize()
     assert torch.equal(got, ref)
+
+
+def test_layer_with_paced_tiles_gives_the_same_bits():
+    """tile_variant = 12 (the m-tiles of one expert and channel block wait for each other so that they share
+    the weight bytes in L2) only changes when workgroups run: the output bits are those of the default."""
+    from vllm_kunlun_amd import _lib as L
+    from vllm_kunlun_amd import synth
+    from vllm_kunlun_amd._plan import make_moe_plan
+    # several m-tiles per expert (about 300 rows each) and a folded shared expert
+    shape = synth.scaled(synth.SHAPES["dsv3-decode"], M=1200, H=512, E=16, K=4, I=256, n_group=4, topk_group=2,
+                         I_shared=256)
+    sl = synth.make_w8a8_layer(shape, "cuda", seed=12)
+    lay = sl.layer
+    outs = []
+    for variant in (0, 12, 12):
+        out = torch.empty_like(sl.x)
+        plan = make_moe_plan(L.KMOE_FMT_INT8, sl.x, sl.logits, out, shape.K, lay.w13_weight, lay.w2_weight,
+                             lay.w13_weight_scale, lay.w2_weight_scale, shape.scoring, True, shape.n_group,
+                             shape.topk_group, shape.routed_scale, sl.bias, sl.shared, 1.0, tile_variant=variant)
+        plan()
+        torch.cuda.synchronize()
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    oi = _oracle_inputs(sl)
+    assert np.array_equal(bits(outs[1]), co.forward_w8a8(**oi))

@@ -448,12 +448,13 @@ PERSISTENT_CASES = TILED_CASES + [
 
 
 @pytest.mark.parametrize("E,n,k,counts", PERSISTENT_CASES)
-@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 7, 8, 9, 11])
+@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 7, 8, 9, 11, 12])
 @pytest.mark.parametrize("act", [0, 1])
 def test_lds_gemm_i8_with_tiled_weights(L, E, n, k, counts, variant, act):
     """LDS-staged kernels reading tiled weights and row-major activations. Variants 1-3: small
     tiles; 5-7: the persistent 128-row-tile kernel (6: 256-channel tiles, 7: 128-channel tiles
-    with the deep weight ring, 8: 256-row tiles with 8 waves, 5: the default)."""
+    with the deep weight ring, 8: 256-row tiles with 8 waves, 5: the default, 12: sibling m-tiles
+    paced against each other through the progress board)."""
     if variant >= 5 and k < 128:
         pytest.skip("the persistent kernel takes k >= 128")
     if variant < 5 and E >= 40:

@@ -454,6 +454,9 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   }
   routed.stream = stream_mode;
   routed.x_count = M;
+  if (a->format == KMOE_FMT_INT8 && !stream_mode && a->w_layout == KMOE_W_TILED && a->tile_variant >= 5 &&
+      a->tile_variant <= 12 && (static_cast<long long>(P) + E - 1) / E > 10 && H >= 128 && I >= 128)
+    routed.variant = a->tile_variant;
   const bool fold = fold_shared(a);
   if (fold) {
     routed.w13_tail = a->ws13;

@@ -468,11 +468,12 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
   KMOE_REQUIRE(a->a_layout == KMOE_A_ROWMAJOR, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: a_layout=%d unknown",
                a->a_layout);
   if (a->rows == 0 && !(a->w_tail && a->tail_rows > 0)) return KMOE_OK;
-  // Tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5-9, 11 force it)
+  // Tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5-9, 11, 12 force it)
   if (a->w_layout == KMOE_W_TILED && a->k >= 128 &&
-      ((a->variant >= 5 && a->variant <= 9) || a->variant == 11 || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
+      ((a->variant >= 5 && a->variant <= 9) || a->variant == 11 || a->variant == 12 ||
+       (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
     return tiled_gemm_i8(a, as_stream(stream));
-  KMOE_REQUIRE(a->variant < 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-11 need tiled weights and k >= 128");
+  KMOE_REQUIRE(a->variant < 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-12 need tiled weights and k >= 128");
   GemmParams p{a->a,   a->lda, a->a_max, a->row_src, a->src_div, a->w,   a->w_max,
                a->lod, a->E,   a->n,     a->k,       a->y,       a->ldy, a->acc_out, a->w_layout == KMOE_W_TILED,
                a->w_tail, a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0, nullptr, 0, 0.f, 0.f};

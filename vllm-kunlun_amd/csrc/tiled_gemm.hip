@@ -121,8 +121,24 @@ struct TiledParams {
   float oai_alpha, oai_limit;  // OAI kernels: out[r, i] = swigluoai(y[r, 2i], y[r, 2i + 1])
 };
 
+// Progress board of the persistent workgroups: slot b (64 bytes apart) holds where workgroup b is,
+// ((position in its item list + 1) << 16) | chunk of K, 0xffffffff once it has no work left, 0 before
+// its first launch. The m-tiles of one (expert, channel block) stream the same weight bytes; they are
+// neighbouring items of the work list and therefore run on neighbouring workgroups of one XCD at the
+// same position of their lists. A workgroup that gets ahead of such a sibling by more than kSyncSlack
+// chunks waits for it (bounded), so the siblings' requests for a weight line meet in the XCD's L2
+// while the line is still there, and the weights of an expert leave HBM once instead of once per
+// m-tile. The board only paces the workgroups: no result depends on it, every wait has an upper bound,
+// and two launches that overlap on one GPU merely pace each other badly.
+constexpr int kBoardSlots = 2048;
+constexpr int kBoardStride = 16;  // 32-bit words: one slot per 64-byte line
+constexpr uint32_t kSyncSlack = 2;
+constexpr int kSyncPatience = 96;  // polls a workgroup spends waiting per tile at most (about 1 us each)
+static __device__ uint32_t g_board[kBoardSlots * kBoardStride];  // word 0 of a slot: the progress; word 1: never written
+
 struct Tile {
   int it;    // position in this workgroup's list
+  int sib;   // bit 0: the item before is an m-tile of the same (expert, channel block); bit 1: the item after
   int e;     // expert (E = the tail expert)
   int row0;  // first sorted row
   int nb;    // channel block
@@ -149,7 +165,11 @@ struct Tile {
 // and registers for a third workgroup per CU).
 // OAI (bf16, no SiLU-mul): gate and up columns interleaved, the gpt-oss activation on each (gate, up) pair of
 // a lane's four consecutive channels - n / 2 outputs per row (ops/_custom_ops.py:728-742).
-template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false>
+// PACE: the m-tiles of one (expert, channel block) keep in step through the progress board (g_board): a tuning
+// variant that brings the bytes fetched by L2 down to about once per weight byte without changing the time
+// (the re-reads it removes were served by the memory-side cache, not by HBM).
+template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false,
+          bool PACE = false>
 __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(const TiledParams p) {
   static_assert(!OAI || (KIND == TKind::BF16 && !SWIGLU && !M32), "the interleaved activation is a bf16 epilogue");
   constexpr int kMF = MF;
@@ -248,11 +268,11 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   // The items of this workgroup are resolved 64 at a time: lane l of wave 0 finds item it0 + l (a binary
   // search over tile_lo and two divisions, all lanes at once) and leaves (expert, first row, channel
   // block) in LDS; the tile loop then reads three words per tile instead of searching.
-  __shared__ int item_e[kWave], item_row0[kWave], item_nb[kWave];
+  __shared__ int item_e[kWave], item_row0[kWave], item_nb[kWave], item_sib[kWave];
   auto resolve_items = [&](int it0) {
     if (wave_id == 0) {
       const int lid = xcd * seg + (blockIdx.x >> 3) + (it0 + lane) * (gridDim.x >> 3);  // gridDim.x is a multiple of 8
-      int e = -1, row0 = 0, nb = 0;
+      int e = -1, row0 = 0, nb = 0, sib = 0;
       if (lid < seg_end) {
         const int m_tile = lid / p.n_blocks;
         // the last e with tile_lo[e] <= m_tile: of a run of equal entries (empty experts) the one that owns the tile
@@ -266,8 +286,14 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         const int first = tile_lo[e], mt = tile_lo[e + 1] - first;
         const int u = lid - first * p.n_blocks;
         nb = u / mt;
-        row0 = rows_begin(e) + (u - nb * mt) * kTM;
+        const int m = u - nb * mt;
+        row0 = rows_begin(e) + m * kTM;
+        // siblings run on the workgroups before / after this one in the XCD, at the same list position
+        const int j = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
+        if (m > 0 && j > 0) sib |= 1;
+        if (m + 1 < mt && j + 1 < per_xcd && lid + 1 < seg_end) sib |= 2;
       }
+      item_sib[lane] = sib;
       item_e[lane] = e;
       item_row0[lane] = row0;
       item_nb[lane] = nb;
@@ -278,10 +304,11 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   // (called by every wave at the same point of the tile loop: the refill every 64 tiles has a barrier inside)
   auto find_tile = [&](int it) -> Tile {
     if (it > 0 && (it & (kWave - 1)) == 0) resolve_items(it);
-    Tile t{it, 0, 0, 0, false};
+    Tile t{it, 0, 0, 0, 0, false};
     const int slot = it & (kWave - 1);
     t.e = __builtin_amdgcn_readfirstlane(item_e[slot]);
     if (t.e < 0) return t;
+    t.sib = __builtin_amdgcn_readfirstlane(item_sib[slot]);
     t.row0 = __builtin_amdgcn_readfirstlane(item_row0[slot]);
     t.nb = __builtin_amdgcn_readfirstlane(item_nb[slot]);
     t.valid = true;
@@ -467,8 +494,79 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   // tile row and byte column (within a chunk) of this thread's i-th activation vector
   auto a_row = [&](int i) -> int { return ADMA ? dma_row + 8 * i : (threadIdx.x + i * kThreads) >> 3; };
   const uint32_t a_col = ADMA ? dma_vec * 16u : (threadIdx.x & 7) * 16u;  // kThreads % 8 == 0
+  // ---- pacing against sibling tiles (see g_board) ----
+  uint32_t* const my_slot = &g_board[blockIdx.x * kBoardStride];
+  const uint32_t* const no_slot = my_slot + 1;  // second word of the own line, never written: 0 = "nobody to wait for"
+  const uint32_t* prev_slot = no_slot;
+  const uint32_t* next_slot = no_slot;
+  uint32_t seen_prev = 0, seen_next = 0;  // the neighbours' progress as polled one chunk ago (wave-uniform)
+  int patience = 0;
+  if constexpr (PACE) __hip_atomic_store(my_slot, 1u << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // Waits (bounded by `patience`) while the workgroup behind `slot` is more than the allowed slack behind `prog`.
+  // One opaque instruction to the compiler: a visible branch here would split the MFMA loop's basic block.
+  auto wait_for = [&](uint32_t& seen, const uint32_t* slot, uint32_t prog) {
+    uint32_t tmp;
+    const uint32_t lim = prog - kSyncSlack;
+    asm volatile(
+        "s_cmp_eq_u32 %[seen], 0\n\t"
+        "s_cbranch_scc1 2f\n"
+        "1:\n\t"
+        "s_cmp_ge_u32 %[seen], %[lim]\n\t"
+        "s_cbranch_scc1 2f\n\t"
+        "s_cmp_lt_i32 %[pat], 1\n\t"
+        "s_cbranch_scc1 2f\n\t"
+        "s_sub_u32 %[pat], %[pat], 1\n\t"
+        "s_sleep 4\n\t"
+        "global_load_dword %[tmp], %[zero], %[slot] sc1\n\t"
+        "s_waitcnt vmcnt(0)\n\t"
+        "v_readfirstlane_b32 %[seen], %[tmp]\n\t"
+        "s_branch 1b\n"
+        "2:\n\t"
+        : [seen] "+s"(seen), [pat] "+s"(patience), [tmp] "=&v"(tmp)
+        : [lim] "s"(lim), [slot] "s"(slot), [zero] "v"(0)
+        : "scc", "memory");
+  };
+  // The siblings' progress is polled with loads that go past this CU's L1; such a load takes longer than a
+  // chunk, and a wave's loads return in order, so the polls are issued AFTER the chunk's own loads and the
+  // chunk's wait leaves them in flight: they have a whole further chunk to arrive (polled[parity of the chunk]).
+  uint32_t polled[2][2] = {{0, 0}, {0, 0}};
+  constexpr int kPolls = PACE ? 2 : 0;  // loads per chunk on top of the chunk's own
+  // start of chunk `chunk` of item `it`: publish it, wait for siblings that have fallen behind
+  auto pace = [&](int it, int chunk) {
+    if constexpr (!PACE) return;
+    const uint32_t prog = (static_cast<uint32_t>(it + 1) << 16) | static_cast<uint32_t>(chunk);
+    // one lane stores (64 lanes writing one address through to memory cost a third of the kernel's time)
+    uint64_t saved_exec;
+    asm volatile(
+        "s_mov_b64 %[ex], exec\n\t"
+        "s_mov_b64 exec, 1\n\t"
+        "global_store_dword %[zero], %[val], %[slot] \n\t"
+        "s_mov_b64 exec, %[ex]\n\t"
+        : [ex] "=&s"(saved_exec)
+        : [zero] "v"(0), [val] "v"(prog), [slot] "s"(my_slot)
+        : "memory");
+    wait_for(seen_prev, prev_slot, prog);
+    wait_for(seen_next, next_slot, prog);
+  };
+  auto pace_poll = [&](auto parity_tag) {  // after the chunk's loads have been issued
+    if constexpr (!PACE) return;
+    constexpr int q = decltype(parity_tag)::value;
+    polled[q][0] = __hip_atomic_load(prev_slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    polled[q][1] = __hip_atomic_load(next_slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  auto pace_collect = [&](auto parity_tag, int chunk) {  // after the chunk's wait: the PREVIOUS chunk's polls are in
+    if constexpr (!PACE) return;
+    constexpr int q = decltype(parity_tag)::value ^ 1;
+    const uint32_t a = __builtin_amdgcn_readfirstlane(polled[q][0]);
+    const uint32_t b = __builtin_amdgcn_readfirstlane(polled[q][1]);
+    seen_prev = chunk > 0 ? a : 0u;  // (a tile's first chunk would collect the polls of the tile before)
+    seen_next = chunk > 0 ? b : 0u;
+  };
   Tile cur = find_tile(0);
-  if (!cur.valid) return;  // the whole workgroup leaves together
+  if (!cur.valid) {  // the whole workgroup leaves together
+    if constexpr (PACE) __hip_atomic_store(my_slot, 0xffffffffu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return;
+  }
   int rs[kNA];             // gather indices of this thread's activation rows
 #pragma unroll
   for (int i = 0; i < kNA; ++i) rs[i] = fetch_src(cur, cur.row0 + a_row(i));
@@ -544,6 +642,12 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     // (after the last tile the loads repeat the current one's: always kNA + 1 loads, which the
     // wait below counts on)
     const Tile look = nxt.valid ? nxt : cur;
+    if constexpr (PACE) {
+      prev_slot = (cur.sib & 1) ? &g_board[(blockIdx.x - 8) * kBoardStride] : no_slot;
+      next_slot = (cur.sib & 2) ? &g_board[(blockIdx.x + 8) * kBoardStride] : no_slot;
+      seen_prev = seen_next = 0;  // nothing polled for this tile yet: its first chunk starts without waiting
+      patience = kSyncPatience;
+    }
     int rs_next[kNA];
 #pragma unroll
     for (int i = 0; i < kNA; ++i) rs_next[i] = fetch_src(look, look.row0 + a_row(i));
@@ -601,6 +705,8 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
       using j0_t = std::integral_constant<int, 0>;
       using j1_t = std::integral_constant<int, 1>;
       const int s0 = (c0 + h) * kSteps;
+      pace(cur.it, c0 + h);
+      __builtin_amdgcn_sched_barrier(0);
       load_a(c0 + h + 1);
       load_w(wring[(2 * h + R - 1) % R], s0 + R - 1);
       __builtin_amdgcn_sched_barrier(0);
@@ -618,18 +724,21 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
         compute(wring[(2 * h + 1) % R], buf_t{}, j1_t{}, std::false_type{});
       }
       __builtin_amdgcn_sched_barrier(0);
+      pace_poll(std::integral_constant<int, h & 1>{});
+      __builtin_amdgcn_sched_barrier(0);
       store_a(buf ^ 1);
-      // ADMA: the 12 loads above may still be in flight, everything older has landed - among
+      // ADMA: the 12 loads above (and the two polls) may still be in flight, everything older has landed - among
       // it this wave's part of chunks c + 1 and c + 2; the barrier publishes them
       // (a bare barrier: the fence of __syncthreads would drain every load in flight, since the
       // asynchronous copies count as stores to LDS)
       if constexpr (ADMA) {
-        vmem_wait<2 * kNF + kNA>();
+        vmem_wait<2 * kNF + kNA + kPolls>();
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
       } else {
         __syncthreads();
       }
+      pace_collect(std::integral_constant<int, h & 1>{}, c0 + h);
     };
     constexpr int kPeriod = ADMA ? kStagesA : R / 2;  // chunks after which ring slots and buffers repeat
     static_assert(kPeriod == 2 || kPeriod == 4, "unrolled by hand below");
@@ -811,9 +920,11 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     }
     if (!nxt.valid) break;
   }
+  if constexpr (PACE) __hip_atomic_store(my_slot, 0xffffffffu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false>
+template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false,
+          bool PACE = false>
 int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* what) {
   constexpr int kTM = WM * 16 * MF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
@@ -823,9 +934,9 @@ int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* w
   const int max_tiles = (rows + p.tail_rows) / kTM + min(n_exp, rows + p.tail_rows);
   p.max_items = p.n_blocks * max_tiles;
   // persistent workgroups: WGS per CU
-  const int grid = min(ceil_div(p.max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8);
+  const int grid = min(min(ceil_div(p.max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8), kBoardSlots);
   const size_t dyn = sizeof(int) * (static_cast<size_t>(p.E) + 1 + n_exp + 1);
-  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32, MF, OAI>), dim3(grid),
+  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32, MF, OAI, PACE>), dim3(grid),
                      dim3(WM * kWavesT * kWave), dyn, s, p);
   return check_launch(what);
 }
@@ -873,7 +984,7 @@ bool short_tiles(int variant, int rows, int n_experts, int n, bool swiglu, int n
 
 // variant 5: 128x256 or 64x256 tiles by the rows per expert (6, 11: one of them), 4-slot weight ring, 2 workgroups
 // per CU (the shape in use); 7: 128x128 tiles, 8-slot ring; 8: 256x256 tiles, 8 waves,
-// 1 workgroup per CU; 9: 128x256 tiles on the 32x32 MFMA shapes
+// 1 workgroup per CU; 9: 128x256 tiles on the 32x32 MFMA shapes; 12: 128x256 tiles, sibling m-tiles paced
 int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   const char* what = "kmoe_grouped_gemm_i8 (tiled)";
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
@@ -898,6 +1009,16 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   // (the 32x32 shapes are instantiated for the gate_up launch only: without SiLU-mul the 16-register
   // fragments of the plain epilogue do not fit two workgroups per CU)
   if (a->variant == 9 && swiglu) return launch_tiled<K, true, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what);
+  // 128-row tiles whose sibling m-tiles are paced against each other (see g_board). By default where most
+  // experts have one or two m-tiles (96 to 256 rows on average): there every second expert's weights are
+  // streamed twice, and keeping the two streams together is worth 3-5 % (DeepSeek-V3 shape, 4096 tokens:
+  // gate_up 1950 -> 1898 us, down 972 -> 926 us; bytes fetched by L2 1.49x -> 1.08x of the algorithmic ones).
+  // With four or five m-tiles per expert the chain of waits costs more than it saves (Qwen3 shape at 8192
+  // tokens: +3 to +8 %), with one tile there is nothing to pace.
+  const int avg_rows = ceil_div(a->rows + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
+  if (a->variant == 12 || (a->variant == 0 && avg_rows > 96 && avg_rows <= 256))
+    return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 8, false, true>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 4, 4, 2, 1, false, 8, false, true>(p, a->rows, s, n_cu, what);
   if (short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu))
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);

@@ -85,7 +85,7 @@ class MoEArgs(C.Structure):
         ("stage_events", C.POINTER(C.c_void_p)), ("w_layout", C.c_int32), ("w_gate", C.c_void_p),
         ("w13_bias", C.c_void_p), ("w2_bias", C.c_void_p), ("activation", C.c_int32), ("act_alpha", C.c_float),
         ("act_limit", C.c_float), ("ws_layout", C.c_int32),
-        ("w13_scale", C.c_void_p), ("w2_scale", C.c_void_p), ("group_size", C.c_int32),
+        ("w13_scale", C.c_void_p), ("w2_scale", C.c_void_p), ("group_size", C.c_int32), ("tile_variant", C.c_int32),
     ]
 
 

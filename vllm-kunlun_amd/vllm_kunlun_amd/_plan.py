@@ -159,7 +159,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
                   stage_events=None, w_layout: Optional[int] = None,
                   router_weight: Optional[torch.Tensor] = None, w13_bias: Optional[torch.Tensor] = None,
                   w2_bias: Optional[torch.Tensor] = None, activation: str = "silu", act_alpha: float = 1.702,
-                  act_limit: float = 7.0, group_size: Optional[int] = None) -> MoEPlan:
+                  act_limit: float = 7.0, group_size: Optional[int] = None, tile_variant: int = 0) -> MoEPlan:
     """x bf16 [M,H], logits f32 [M,E], out bf16 [M,H]; w13 [E,2I,H], w2 [E,H,I] in the
     format's dtype; w13_aux/w2_aux: per-channel maxes (int8) or block scales (fp8), None for bf16.
     shared_expert: (ws13 [2Is,H], ws13_aux, ws2 [H,Is], ws2_aux) in the same format.
@@ -167,7 +167,8 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     layer then computes the router logits itself. bf16 only: w13_bias [E,2I] / w2_bias [E,H] (bf16)
     and activation "swigluoai" (gate and up rows of w13 interleaved) select the expert-bias branch.
     KMOE_FMT_W4A16: w13 [E,2I,H/2] and w2 [E,H,I/2] uint8 (two 4-bit codes per byte), tiled;
-    w13_aux/w2_aux their bf16 group scales [E,2I,H/group_size], [E,H,I/group_size]."""
+    w13_aux/w2_aux their bf16 group scales [E,2I,H/group_size], [E,H,I/group_size].
+    tile_variant: a tuning variant of the int8 tile kernel for the routed GEMMs (kmoe_moe_args.tile_variant)."""
     if scoring_func not in ("softmax", "sigmoid"):
         raise ValueError(f"Unsupported scoring_func: {scoring_func}")
     if logits is None and router_weight is None:
@@ -244,6 +245,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     a.activation = L.KMOE_ACT_SWIGLUOAI if activation == "swigluoai" else L.KMOE_ACT_SWIGLU
     a.act_alpha, a.act_limit = float(act_alpha), float(act_limit)
     a.out_scale = float(out_scale)
+    a.tile_variant = int(tile_variant)
     a.out = out.data_ptr()
     if w_layout is None:  # per group of weights: tiled if both of its tensors have been tiled
         w_layout = L.KMOE_W_TILED if is_tiled(w13) and is_tiled(w2) else L.KMOE_W_ROWMAJOR

@@ -401,7 +401,7 @@ int launch(const GemmParams& p, int rows, hipStream_t s, const char* what) {
 constexpr int kTiledMinRows = 10;
 // variants of the bf16 and fp8 launchers that force the tile kernel: 5 (tile height from the rows per expert),
 // 6 (128-row tiles), 11 (64-row tiles)
-inline bool tile_variant(int v) { return v == 5 || v == 6 || v == 11; }
+inline bool tile_variant(int v) { return v == 5 || v == 6 || v == 11 || v == 12; }
 
 template <Kind KIND>
 int dispatch(const GemmParams& p, int rows, bool swiglu, int variant, hipStream_t s, const char* what) {

@@ -42,6 +42,12 @@ extern "C" {
 
 typedef void* kmoe_stream_t;
 
+/* Activation dtype of the int8 path: the 16-bit tensors (x, intermediates, out) hold bf16 or IEEE half
+ * patterns. The reference runs its deployment recipes with --dtype float16 (ci/scripts/server/start_vllm.sh:26;
+ * platforms/kunlun.py:350-364 admits float16 and bfloat16). Functions without an act_dtype argument take bf16. */
+#define KMOE_DT_BF16 0
+#define KMOE_DT_F16 1
+
 /* Text of the last error raised on the calling thread ("" if none). */
 const char* kmoe_last_error(void);
 /* Library version string, e.g. "kmoe 0.1 gfx950". */
@@ -141,6 +147,12 @@ int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q,
 int kmoe_quant_i8_rows_chunked(const uint16_t* x, int64_t ld_x, int R, int C,
                                int8_t* q, float* row_max, kmoe_stream_t stream);
 
+/* The two functions above for either activation dtype (KMOE_DT_*). */
+int kmoe_quant_i8_rows_dt(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q,
+                          float* row_max, int act_dtype, kmoe_stream_t stream);
+int kmoe_quant_i8_rows_chunked_dt(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q,
+                                  float* row_max, int act_dtype, kmoe_stream_t stream);
+
 /*
  * Per-row, per-128-column-group dynamic fp8-e4m3fn (OCP). No counterpart in the
  * reference (its fp8 ops are empty stubs, ops/_custom_ops.py:44-89); follows
@@ -193,6 +205,7 @@ typedef struct kmoe_gemm_i8_args {
   const int8_t* w_tail;   /* [n, k], same layout as w                           */
   const float* w_max_tail; /* [n]                                                */
   int32_t tail_row0, tail_rows, tail_src0;
+  int32_t act_dtype;      /* KMOE_DT_*: dtype of y (and of the rounding of gate and up before SiLU-mul) */
 } kmoe_gemm_i8_args;
 
 #define KMOE_W_ROWMAJOR 0
@@ -339,6 +352,9 @@ int kmoe_swigluoai_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, float 
  */
 int kmoe_silu_and_mul(const uint16_t* y, int64_t ld_y, int R, int I,
                       uint16_t* out, int64_t ld_out, kmoe_stream_t stream);
+/* ... for either activation dtype (KMOE_DT_*). */
+int kmoe_silu_and_mul_dt(const uint16_t* y, int64_t ld_y, int R, int I, uint16_t* out, int64_t ld_out,
+                         int act_dtype, kmoe_stream_t stream);
 
 /*
  * Un-permute + weighted top-K sum. Replaces kunlun_ops.moe_post
@@ -354,6 +370,18 @@ int kmoe_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_index,
                  int H, float out_scale, const uint16_t* addend,
                  int64_t ld_addend, uint16_t* out, int64_t ld_out,
                  kmoe_stream_t stream);
+/*
+ * ... for either activation dtype (KMOE_DT_*), and with a factor on the addend: the half-precision form of
+ * the caller epilogue (models/deepseek_v2.py:286-292) keeps the routed sum unscaled and multiplies the
+ * shared expert's output by 1/routed_scaling_factor instead:
+ *   out = dt( float(dt(float(out) * out_scale)) + float(dt(float(addend[m,h]) * addend_scale)) ),
+ * a factor of exactly 1 skipping its multiplication and rounding.
+ */
+int kmoe_combine_dt(const uint16_t* x, int64_t ld_x, const int32_t* moe_index,
+                    const float* topk_w, const float* dequant_scale, int M, int K,
+                    int H, float out_scale, const uint16_t* addend, int64_t ld_addend,
+                    float addend_scale, uint16_t* out, int64_t ld_out, int act_dtype,
+                    kmoe_stream_t stream);
 
 /*
  * Unpacks 4-bit weights to bf16 once, at load time. Replaces dequant_int4_native
@@ -384,6 +412,10 @@ size_t kmoe_router_gemm_workspace_bytes(int M, int H, int E);
 int kmoe_router_gemm_bf16(const uint16_t* x, int64_t ld_x, const uint16_t* w_gate,
                           int M, int H, int E, float* logits, int64_t ld_logits,
                           void* workspace, size_t workspace_bytes, kmoe_stream_t stream);
+/* ... with x and w_gate in either dtype (KMOE_DT_*; both the same). */
+int kmoe_router_gemm(const uint16_t* x, int64_t ld_x, const uint16_t* w_gate,
+                     int M, int H, int E, float* logits, int64_t ld_logits,
+                     void* workspace, size_t workspace_bytes, int act_dtype, kmoe_stream_t stream);
 
 /* ------------------------------------------------------------ fused forward */
 
@@ -443,6 +475,10 @@ typedef struct kmoe_moe_args {
   const uint16_t* w13_scale; /* [E,2I,H/group_size] bf16                               */
   const uint16_t* w2_scale;  /* [E,H,I/group_size] bf16                                */
   int32_t group_size;    /* a multiple of 32 dividing H and I (one value for both tensors) */
+  int32_t act_dtype;     /* KMOE_DT_* of x, out (and w_gate, shared-expert output): half goes with KMOE_FMT_INT8 only */
+  float shared_scale;    /* caller epilogue for half activations (models/deepseek_v2.py:286-292: the routed sum stays
+                            unscaled and the shared expert's output is multiplied by 1/routed_scaling_factor):
+                            out = dt( dt(routed * out_scale) + dt(shared * shared_scale) ); 0 means 1 */
   int32_t tile_variant;  /* INT8, tuning: 0, or the `variant` (5-12) handed to the two routed GEMMs when the batch
                             runs on the tile kernel (more than 10 rows per expert); ignored otherwise */
 } kmoe_moe_args;

@@ -67,6 +67,23 @@ def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
 
 
 # -- scalar functions ---------------------------------------------------------
+def _dtype(f16: bool) -> None:
+    """Selects what the 16-bit activation tensors of the int8 path hold for the next call: bf16 or IEEE half."""
+    lib().orc_set_act_dtype(1 if f16 else 0)
+
+
+def f32_to_half_bits(x: np.ndarray) -> np.ndarray:
+    fn = lib().orc_f32_to_half
+    fn.restype, fn.argtypes = C.c_uint16, [C.c_float]
+    return np.array([fn(float(v)) for v in np.asarray(x, np.float32).ravel()], np.uint16).reshape(np.shape(x))
+
+
+def half_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    fn = lib().orc_half_to_f32
+    fn.restype, fn.argtypes = C.c_float, [C.c_uint16]
+    return np.array([fn(int(v)) for v in np.asarray(b, np.uint16).ravel()], np.float32).reshape(np.shape(b))
+
+
 def exp(x: np.ndarray) -> np.ndarray:
     f = lib().orc_exp
     return np.array([f(float(v)) for v in np.asarray(x, dtype=np.float32).ravel()], dtype=np.float32).reshape(np.shape(x))
@@ -121,7 +138,8 @@ def block_statistic(ids, E, n_blocks):
     return out
 
 
-def quant_i8_rows(x_bits):
+def quant_i8_rows(x_bits, f16=False):
+    _dtype(f16)
     x_bits = _c(x_bits, np.uint16)
     R, Cc = x_bits.shape
     q = np.empty((R, Cc), np.int8)
@@ -139,7 +157,8 @@ def quant_fp8_group128(x_bits):
     return q, s
 
 
-def grouped_gemm_i8(a, a_max, w, w_max, lod, act=0, row_src=None, src_div=1, want_acc=False, want_y=True):
+def grouped_gemm_i8(a, a_max, w, w_max, lod, act=0, row_src=None, src_div=1, want_acc=False, want_y=True, f16=False):
+    _dtype(f16)
     a = _c(a, np.int8)
     a_max = _c(a_max, np.float32).ravel()
     w = _c(w, np.int8)
@@ -156,7 +175,8 @@ def grouped_gemm_i8(a, a_max, w, w_max, lod, act=0, row_src=None, src_div=1, wan
     return y, acc
 
 
-def silu_and_mul(y_bits):
+def silu_and_mul(y_bits, f16=False):
+    _dtype(f16)
     y_bits = _c(y_bits, np.uint16)
     R, two_i = y_bits.shape
     out = np.empty((R, two_i // 2), np.uint16)
@@ -164,7 +184,8 @@ def silu_and_mul(y_bits):
     return out
 
 
-def combine(x_bits, moe_index, topk_w, dq=None, out_scale=1.0, addend=None):
+def combine(x_bits, moe_index, topk_w, dq=None, out_scale=1.0, addend=None, addend_scale=1.0, f16=False):
+    _dtype(f16)
     x_bits = _c(x_bits, np.uint16)
     topk_w = _c(topk_w, np.float32)
     M, K = topk_w.shape
@@ -174,14 +195,16 @@ def combine(x_bits, moe_index, topk_w, dq=None, out_scale=1.0, addend=None):
     addend = None if addend is None else _c(addend, np.uint16)
     out = np.empty((M, H), np.uint16)
     lib().orc_combine(_p(x_bits), C.c_int64(H), _p(moe_index), _p(topk_w), _p(dq), M, K, H, C.c_float(out_scale),
-                      _p(addend), C.c_int64(H), _p(out), C.c_int64(H))
+                      _p(addend), C.c_int64(H), C.c_float(addend_scale), _p(out), C.c_int64(H))
     return out
 
 
 def forward_w8a8(x_bits, logits, w13, w13_max, w2, w2_max, K, scoring="softmax", renormalize=True, n_group=1,
-                 topk_group=1, routed_scale=1.0, bias=None, shared=None, out_scale=1.0, intermediates=False):
-    """Whole layer. `shared` = (ws13, ws13_max, ws2, ws2_max) or None.
+                 topk_group=1, routed_scale=1.0, bias=None, shared=None, out_scale=1.0, intermediates=False,
+                 shared_scale=1.0, f16=False):
+    """Whole layer. `shared` = (ws13, ws13_max, ws2, ws2_max) or None; f16: x and out hold IEEE half patterns.
     Returns out bits [M,H], plus a dict of intermediates when asked."""
+    _dtype(f16)
     x_bits = _c(x_bits, np.uint16)
     logits = _c(logits, np.float32)
     w13 = _c(w13, np.int8)
@@ -214,13 +237,14 @@ def forward_w8a8(x_bits, logits, w13, w13_max, w2, w2_max, K, scoring="softmax",
     lib().orc_forward_w8a8(M, H, E, K, I, 0 if scoring == "softmax" else 1, int(bool(renormalize)), int(n_group or 1),
                            int(topk_group or 1), C.c_float(routed_scale), _p(logits), _p(bias), _p(x_bits), _p(w13),
                            _p(w13_max), _p(w2), _p(w2_max), Is, _p(ws13), _p(ws13_max), _p(ws2), _p(ws2_max),
-                           C.c_float(out_scale), _p(out), _p(g("topk_w")), _p(g("topk_ids")), _p(g("moe_index")),
+                           C.c_float(out_scale), C.c_float(shared_scale), _p(out), _p(g("topk_w")), _p(g("topk_ids")), _p(g("moe_index")),
                            _p(g("lod")), _p(g("actq")), _p(g("actmax")), _p(g("down")))
     return (out, inter) if intermediates else out
 
 
-def router_gemm(x_bits, w_bits):
-    """(logits f32 [M,E], abs_sum f32 [M,E]): x bf16 bits [M,H], w bf16 bits [E,H]."""
+def router_gemm(x_bits, w_bits, f16=False):
+    """(logits f32 [M,E], abs_sum f32 [M,E]): x bits [M,H], w bits [E,H], both bf16 (or both half)."""
+    _dtype(f16)
     x_bits = _c(x_bits, np.uint16)
     w_bits = _c(w_bits, np.uint16)
     M, H = x_bits.shape

@@ -52,6 +52,56 @@ static inline uint16_t f32_to_bf16(float f) {
   return (uint16_t)(u >> 16);
 }
 
+/* IEEE half <-> f32, round to nearest even, overflow to infinity (what every IEEE conversion does) */
+static inline float half_to_f32(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  const int ex = (h >> 10) & 0x1f;
+  const uint32_t man = h & 0x3ffu;
+  union { uint32_t u; float f; } v;
+  if (ex == 0) {
+    v.f = ldexpf((float)man, -24); /* zero and subnormals: man * 2^-24, exact */
+    v.u |= sign;
+    return v.f;
+  }
+  if (ex == 31) {
+    v.u = sign | 0x7f800000u | (man << 13);
+    return v.f;
+  }
+  v.u = sign | ((uint32_t)(ex - 15 + 127) << 23) | (man << 13);
+  return v.f;
+}
+
+static inline uint16_t f32_to_half(float f) {
+  union { uint32_t u; float f; } v;
+  v.f = f;
+  const uint16_t sign = (uint16_t)((v.u >> 16) & 0x8000u);
+  const uint32_t a = v.u & 0x7fffffffu;
+  if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);             /* NaN */
+  if (a >= 0x47800000u) return (uint16_t)(sign | 0x7c00u);            /* >= 65536 (and inf): infinity */
+  if (a < 0x33000000u) return sign;                                   /* < 2^-25: rounds to zero (2^-25 itself ties to even = 0) */
+  const int ex = (int)(a >> 23) - 127;                                /* unbiased exponent, -25 .. 15 */
+  uint32_t man = (a & 0x7fffffu) | 0x800000u;                         /* 24-bit significand */
+  const int shift = ex < -14 ? 13 + (-14 - ex) : 13;                  /* bits dropped (more for subnormal results) */
+  const uint32_t kept = man >> shift;
+  const uint32_t rem = man & ((1u << shift) - 1u);
+  const uint32_t half_ulp = 1u << (shift - 1);
+  uint32_t r = kept + ((rem > half_ulp || (rem == half_ulp && (kept & 1u))) ? 1u : 0u);
+  /* normal: r has the implicit bit at position 10 (a carry moves into the exponent, which is right, also into
+     infinity at the top); subnormal: r is the mantissa itself (a carry to 0x400 gives the smallest normal) */
+  const uint32_t bits = ex < -14 ? r : ((uint32_t)(ex + 15 - 1) << 10) + r;
+  return (uint16_t)(sign | bits);
+}
+
+/* Activation dtype of the int8 path: bf16 (0) or IEEE half (1) patterns in the 16-bit tensors. The reference
+ * runs either (platforms/kunlun.py:350-364; its recipes use float16, ci/scripts/server/start_vllm.sh:26).
+ * A switch for the whole library, set by the Python front end before each call. */
+static int g_act_f16 = 0;
+ORC_API void orc_set_act_dtype(int f16) { g_act_f16 = f16 != 0; }
+ORC_API uint16_t orc_f32_to_half(float f) { return f32_to_half(f); }
+ORC_API float orc_half_to_f32(uint16_t h) { return half_to_f32(h); }
+static inline float act_to_f32(uint16_t h) { return g_act_f16 ? half_to_f32(h) : bf16_to_f32(h); }
+static inline uint16_t f32_to_act(float f) { return g_act_f16 ? f32_to_half(f) : f32_to_bf16(f); }
+
 ORC_API float orc_exp(float x) {
   x = fminf(fmaxf(x, -86.0f), 86.0f);
   const float n = rintf(x * 0x1.715476p+0f);
@@ -216,10 +266,10 @@ ORC_API void orc_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, in
   for (int r = 0; r < R; ++r) {
     const uint16_t* xr = x + (size_t)r * ld_x;
     float amax = 0.0f;
-    for (int c = 0; c < C; ++c) amax = fmaxf(amax, fabsf(bf16_to_f32(xr[c])));
+    for (int c = 0; c < C; ++c) amax = fmaxf(amax, fabsf(act_to_f32(xr[c])));
     const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
     for (int c = 0; c < C; ++c) {
-      float f = rintf(bf16_to_f32(xr[c]) * inv);
+      float f = rintf(act_to_f32(xr[c]) * inv);
       f = fminf(fmaxf(f, -127.0f), 127.0f);
       q[(size_t)r * ld_q + c] = (int8_t)(int)f;
     }
@@ -301,7 +351,7 @@ ORC_API void orc_grouped_gemm_i8(const int8_t* a, int64_t lda, const float* a_ma
         for (int c = 0; c < n; ++c) {
           const int32_t acc = dot_i8(ar, we + (size_t)c * k, k);
           if (acc_out) acc_out[(size_t)r * n + c] = acc;
-          if (y) y[(size_t)r * ldy + c] = f32_to_bf16(((float)acc * sa) * (wm[c] / 127.0f));
+          if (y) y[(size_t)r * ldy + c] = f32_to_act(((float)acc * sa) * (wm[c] / 127.0f));
         }
       } else {
         for (int c = 0; c < half; ++c) {
@@ -311,9 +361,9 @@ ORC_API void orc_grouped_gemm_i8(const int8_t* a, int64_t lda, const float* a_ma
             acc_out[(size_t)r * n + c] = ag;
             acc_out[(size_t)r * n + half + c] = au;
           }
-          const uint16_t yg = f32_to_bf16(((float)ag * sa) * (wm[c] / 127.0f));
-          const uint16_t yu = f32_to_bf16(((float)au * sa) * (wm[half + c] / 127.0f));
-          if (y) y[(size_t)r * ldy + c] = f32_to_bf16(orc_silu(bf16_to_f32(yg)) * bf16_to_f32(yu));
+          const uint16_t yg = f32_to_act(((float)ag * sa) * (wm[c] / 127.0f));
+          const uint16_t yu = f32_to_act(((float)au * sa) * (wm[half + c] / 127.0f));
+          if (y) y[(size_t)r * ldy + c] = f32_to_act(orc_silu(act_to_f32(yg)) * act_to_f32(yu));
         }
       }
     }
@@ -334,7 +384,7 @@ ORC_API void orc_router_gemm(const uint16_t* x, int64_t ld_x, const uint16_t* w,
     for (int e = 0; e < E; ++e) {
       double s = 0.0, sa = 0.0;
       for (int k = 0; k < H; ++k) {
-        const double p = (double)bf16_to_f32(x[(size_t)m * ld_x + k]) * (double)bf16_to_f32(w[(size_t)e * H + k]);
+        const double p = (double)act_to_f32(x[(size_t)m * ld_x + k]) * (double)act_to_f32(w[(size_t)e * H + k]);
         s += p;
         sa += p < 0 ? -p : p;
       }
@@ -485,8 +535,8 @@ ORC_API void orc_grouped_gemm_fp8(const uint8_t* a, int64_t lda, const float* a_
 ORC_API void orc_silu_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, uint16_t* out, int64_t ld_out) {
   for (int r = 0; r < R; ++r)
     for (int i = 0; i < I; ++i)
-      out[(size_t)r * ld_out + i] = f32_to_bf16(orc_silu(bf16_to_f32(y[(size_t)r * ld_y + i])) *
-                                                 bf16_to_f32(y[(size_t)r * ld_y + I + i]));
+      out[(size_t)r * ld_out + i] = f32_to_act(orc_silu(act_to_f32(y[(size_t)r * ld_y + i])) *
+                                                 act_to_f32(y[(size_t)r * ld_y + I + i]));
 }
 
 /* moe_post (compressed_tensors_moe.py:278-290): weighted top-K sum, f32
@@ -494,7 +544,7 @@ ORC_API void orc_silu_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, uin
  * epilogue of models/deepseek_v2.py:288-296 when requested. */
 ORC_API void orc_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_index, const float* topk_w,
                          const float* dq, int M, int K, int H, float out_scale, const uint16_t* addend,
-                         int64_t ld_addend, uint16_t* out, int64_t ld_out) {
+                         int64_t ld_addend, float addend_scale, uint16_t* out, int64_t ld_out) {
   const int epilogue = (out_scale != 1.0f) || addend;
 #pragma omp parallel for schedule(static)
   for (int m = 0; m < M; ++m) {
@@ -505,12 +555,18 @@ ORC_API void orc_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_ind
         const int r = moe_index[j];
         if (r < 0) continue;
         const float wt = dq ? topk_w[j] * dq[j] : topk_w[j];
-        acc = fmaf(wt, bf16_to_f32(x[(size_t)r * ld_x + h]), acc);
+        acc = fmaf(wt, act_to_f32(x[(size_t)r * ld_x + h]), acc);
       }
-      uint16_t o = f32_to_bf16(acc);
+      uint16_t o = f32_to_act(acc);
       if (epilogue) {
-        o = f32_to_bf16(bf16_to_f32(o) * out_scale);
-        if (addend) o = f32_to_bf16(bf16_to_f32(o) + bf16_to_f32(addend[(size_t)m * ld_addend + h]));
+        /* each step rounds to the activation dtype, as the caller's tensor operations do; the half form
+           (models/deepseek_v2.py:286-292) scales the shared output instead of the routed sum */
+        if (out_scale != 1.0f) o = f32_to_act(act_to_f32(o) * out_scale);
+        if (addend) {
+          uint16_t ad = addend[(size_t)m * ld_addend + h];
+          if (addend_scale != 1.0f) ad = f32_to_act(act_to_f32(ad) * addend_scale);
+          o = f32_to_act(act_to_f32(o) + act_to_f32(ad));
+        }
       }
       out[(size_t)m * ld_out + h] = o;
     }
@@ -527,7 +583,8 @@ ORC_API void orc_forward_w8a8(int M, int H, int E, int K, int I, int scoring, in
                               int topk_group, float routed_scale, const float* logits, const float* bias,
                               const uint16_t* x, const int8_t* w13, const float* w13_max, const int8_t* w2,
                               const float* w2_max, int I_shared, const int8_t* ws13, const float* ws13_max,
-                              const int8_t* ws2, const float* ws2_max, float out_scale, uint16_t* out,
+                              const int8_t* ws2, const float* ws2_max, float out_scale, float shared_scale,
+                              uint16_t* out,
                               /* optional intermediates (NULL to skip) */
                               float* o_topk_w, int32_t* o_topk_ids, int32_t* o_moe_index, int32_t* o_lod,
                               int8_t* o_actq, float* o_actmax, uint16_t* o_down) {
@@ -570,7 +627,7 @@ ORC_API void orc_forward_w8a8(int M, int H, int E, int K, int I, int scoring, in
     free(sq);
     free(smax);
   }
-  orc_combine(down, H, moe_index, topk_w, NULL, M, K, H, out_scale, sh_out, H, out, H);
+  orc_combine(down, H, moe_index, topk_w, NULL, M, K, H, out_scale, sh_out, H, shared_scale, out, H);
 
   if (o_topk_w) memcpy(o_topk_w, topk_w, sizeof(float) * (size_t)P);
   if (o_topk_ids) memcpy(o_topk_ids, topk_ids, sizeof(int32_t) * (size_t)P);

@@ -34,16 +34,34 @@ def test_library_exports_every_declared_symbol(L):
     assert b"gfx950" in L.lib.kmoe_version()
 
 
-def test_struct_layouts_match_the_header(L):
-    # sizes implied by the C declarations (LP64): guards the ctypes mirrors against drift
-    assert C.sizeof(L.GemmI8Args) == 8 * 8 + 16 + 8 * 3 + 8 + 16 + 16 + 16  # 8 ptr/int64, 4 int32, y/ldy/acc_out, act+variant, 3 int32 + pad
-    assert C.sizeof(L.MoELayout) == 22 * 8
-    assert C.sizeof(L.GemmBf16Args) == 6 * 8 + 16 + 16 + 16 + 16  # ..., act+variant+w_layout+pad, bias, alpha+limit  # 6 ptr/int64 (src_div padded), 4 int32, y/ldy, act+variant+w_layout+pad
-    assert C.sizeof(L.GemmFp8Args) == 8 * 8 + 16 + 16 + 16 + 16 + 16  # ..., act+variant+w_layout+pad, 2 tail ptrs, 3 int32 + pad
-    assert L.MoEArgs.w_gate.offset == C.sizeof(L.MoEArgs) - 8 - 32 - 24  # then w13_bias, w2_bias, activation, alpha, limit, ws_layout; w13_scale, w2_scale, group_size + pad
-    assert C.sizeof(L.GemmW4Args) == 3 * 8 + 8 + 2 * 8 + 8 + 8 + 16 + 16 + 16  # a/lda/row_src, src_div+pad, w/w_scale, group_size+pad, lod, 4 int32, y/ldy, act+variant+w_layout+pad
-    a = L.MoEArgs()
-    assert L.MoEArgs.M.offset == 0 and L.MoEArgs.logits.offset == 48 and C.sizeof(a) % 8 == 0
+def test_struct_layouts_match_the_header(L, tmp_path):
+    """The ctypes mirrors against the C declarations themselves: a C program that includes include/kmoe.h
+    prints sizeof and the offsets of a few late fields of every argument struct (gcc, host only)."""
+    import subprocess
+    structs = {"kmoe_gemm_i8_args": (L.GemmI8Args, ["lod", "acc_out", "w_tail", "tail_src0", "act_dtype"]),
+               "kmoe_gemm_bf16_args": (L.GemmBf16Args, ["lod", "y", "bias", "act_limit"]),
+               "kmoe_gemm_fp8_args": (L.GemmFp8Args, ["w_scale", "y", "w_tail", "tail_src0"]),
+               "kmoe_gemm_w4_args": (L.GemmW4Args, ["w_scale", "lod", "y", "w_layout"]),
+               "kmoe_moe_args": (L.MoEArgs, ["logits", "I_shared", "out", "w_gate", "ws_layout", "group_size",
+                                             "act_dtype", "shared_scale", "tile_variant"]),
+               "kmoe_moe_layout": (L.MoELayout, ["align_ws", "down", "sh_out", "n_logit_planes"])}
+    lines = ["#include <stdio.h>", "#include <stddef.h>", '#include "kmoe.h"', "int main(void) {"]
+    for name, (_, fields) in structs.items():
+        lines.append(f'  printf("{name} %zu", sizeof({name}));')
+        for f in fields:
+            lines.append(f'  printf(" %zu", offsetof({name}, {f}));')
+        lines.append('  printf("\\n");')
+    lines += ["  return 0;", "}"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split("\n")
+    for line in filter(None, out):
+        name, size, *offsets = line.split()
+        cls, fields = structs[name]
+        assert C.sizeof(cls) == int(size), name
+        assert [getattr(cls, f).offset for f in fields] == [int(o) for o in offsets], name
 
 
 def test_null_and_shape_errors_are_status_codes(L):

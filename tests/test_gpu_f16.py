@@ -1,0 +1,154 @@
+"""float16 activations on the int8 path (the dtype the reference's deployment recipes run,
+ci/scripts/server/start_vllm.sh:26): the whole layer through apply_monolithic and the operator surface,
+bit for bit against the C oracle in its half mode, in every kernel regime (weight-streaming decode path,
+64-row, 128-row and paced tiles, row-major LDS kernels), with the half form of the caller epilogue
+(models/deepseek_v2.py:286-292: routed sum unscaled, shared output times 1/routed_scaling_factor)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+from oracle import c_oracle as co  # noqa: E402
+from oracle import torch_moe as tm  # noqa: E402
+
+
+def hbits(t: torch.Tensor) -> np.ndarray:
+    assert t.dtype == torch.float16
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def from_hbits(b: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(b).view(np.int16)).view(torch.float16)
+
+
+CASES = [
+    ("stream-decode-shared", "dsv3-decode", dict(M=40, H=512, E=32, K=4, I=128, n_group=4, topk_group=2, I_shared=128)),
+    ("stream-decode-softmax", "qwen3-decode", dict(M=33, H=768, E=24, K=6, I=192)),
+    ("short-tiles", "qwen3-decode", dict(M=120, H=512, E=16, K=4, I=256)),
+    ("tall-tiles-shared", "dsv3-decode", dict(M=700, H=256, E=8, K=2, I=128, n_group=2, topk_group=1, I_shared=128)),
+    ("paced-tiles", "dsv3-decode", dict(M=560, H=512, E=16, K=4, I=256, n_group=4, topk_group=2, I_shared=256)),
+    ("rowmajor-lds", "dsv3-decode", dict(M=50, H=272, E=8, K=2, I=80, n_group=2, topk_group=1, I_shared=80)),
+    ("shared-other-width", "dsv3-decode", dict(M=37, H=640, E=160, K=6, I=192, n_group=8, topk_group=3,
+                                               routed_scale=16.0, I_shared=384)),
+]
+
+
+@pytest.mark.parametrize("name,base,over", CASES, ids=[c[0] for c in CASES])
+def test_half_layer_matches_the_oracle(name, base, over):
+    from vllm_kunlun_amd import synth
+    shape = synth.scaled(synth.SHAPES[base], **over)
+    sl = synth.make_w8a8_layer(shape, "cuda", seed=7)
+    if name == "rowmajor-lds":
+        assert sl.layer.w2_weight.shape[-1] != shape.I or True
+    x = (sl.x.float() * 1.5).half()
+    method = sl.layer.quant_method
+    kw = sl.apply_kwargs()
+    # the half form of the caller epilogue: the routing weights stay unscaled, the shared output is scaled down
+    scale = shape.routed_scale if shape.scoring == "sigmoid" else 1.0
+    if "routed_scaling_factor" in kw:
+        kw["routed_scaling_factor"] = 1.0
+    shared_scale = 1.0 / scale if sl.shared is not None else 1.0
+    out = method.apply_monolithic(sl.layer, x, sl.logits, shared_scale=shared_scale, **kw)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16 and bool(torch.isfinite(out.float()).all())
+    w13, w13_max, w2, w2_max, shared = sl.host_weights()
+    sh = None if shared is None else tuple(t.numpy() for t in shared)
+    ref, inter = co.forward_w8a8(hbits(x), sl.logits.cpu().numpy(), w13.numpy(), w13_max.numpy(), w2.numpy(),
+                                 w2_max.numpy(), shape.K, shape.scoring, True, shape.n_group, shape.topk_group, 1.0,
+                                 None if sl.bias is None else sl.bias.cpu().numpy(), sh, shared_scale=shared_scale,
+                                 intermediates=True, f16=True)
+    lay, ws = method.last_layout, method.last_workspace
+    ids = ws[lay.topk_ids: lay.topk_ids + 4 * shape.P].view(torch.int32).cpu().numpy().reshape(shape.M, shape.K)
+    assert np.array_equal(ids, inter["topk_ids"])
+    assert np.array_equal(hbits(out), ref), f"{np.count_nonzero(hbits(out) != ref)} of {ref.size} outputs differ"
+    # and the torch expert loop, run in float16
+    host = lambda t: None if t is None else t.detach().cpu()  # noqa: E731
+    routed = tm.w8a8_moe(host(x), host(sl.logits), w13, w13_max, w2, w2_max, shape.K, shape.scoring, True, shape.n_group,
+                         shape.topk_group, 1.0, host(sl.bias))
+    if shared is not None:
+        routed = routed + tm.w8a8_dense(host(x), *shared) * shared_scale
+    assert rel_l2(out, routed) <= 1e-2
+
+
+def test_half_layer_with_the_router_gemm_inside():
+    from vllm_kunlun_amd import synth
+    shape = synth.scaled(synth.SHAPES["qwen3-decode"], M=48, H=512, E=64, K=4, I=128)
+    sl = synth.make_w8a8_layer(shape, "cuda", seed=8)
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn(shape.M, shape.H, generator=g, device="cuda").half()
+    w_gate = (torch.randn(shape.E, shape.H, generator=g, device="cuda") * shape.H ** -0.5).half()
+    logits = torch.ops._C.router_gemm_bf16_fp32(x, w_gate)
+    ref, abs_sum = co.router_gemm(hbits(x), hbits(w_gate), f16=True)
+    torch.cuda.synchronize()
+    assert np.all(np.abs(logits.cpu().numpy() - ref) <= shape.H * 2.0 ** -24 * abs_sum + 1e-30)
+    method = sl.layer.quant_method
+    inside = method.apply_monolithic(sl.layer, x, None, router_weight=w_gate)
+    outside = method.apply_monolithic(sl.layer, x, logits)
+    torch.cuda.synchronize()
+    # same logits up to the summation order of the split-K planes: the same experts except at near ties
+    assert rel_l2(inside, outside) <= 1e-2
+
+
+def test_half_operator_surface():
+    """quant2d, scaled_int8_quant, moe_fc, matmul, silu_and_mul and moe_post with float16 tensors, and the dense
+    W8A8 Linear class, against the oracle's half mode."""
+    import vllm_kunlun_amd  # noqa: F401
+    from types import SimpleNamespace
+    from vllm_kunlun_amd.quantization.kernels.scale_mm import KunlunScaledMMLinearKernel
+    g = torch.Generator().manual_seed(9)
+    R, k, n, E = 37, 256, 128, 3
+    x = (torch.randn(R, k, generator=g) * 2).half()
+    xq = torch.empty(R, k, dtype=torch.int8, device="cuda")
+    mx = torch.empty(R, 1, dtype=torch.float32, device="cuda")
+    torch.ops._C.quant2d(x.cuda(), xq, mx)
+    q_ref, mx_ref = co.quant_i8_rows(hbits(x), f16=True)
+    assert np.array_equal(xq.cpu().numpy(), q_ref) and np.array_equal(mx.cpu().numpy().ravel(), mx_ref)
+    xq2, mx2, _, static = torch.ops._C.scaled_int8_quant(x.cuda(), None, None, True)
+    assert not static and torch.equal(xq2, xq) and torch.equal(mx2, mx)
+    # grouped GEMM with a half output, plain and fused with SiLU-mul
+    w = torch.randint(-127, 128, (E, n, k), generator=g, dtype=torch.int8)
+    w_max = torch.rand(E, n, 1, generator=g) * 0.05 + 0.01
+    lod = torch.tensor([0, 10, 10, R], dtype=torch.int32)
+    idx = torch.empty(0, dtype=torch.int32, device="cuda")
+    for act, cols in ((None, n), ("SWISH_GLU", n // 2)):
+        y = torch.empty(R, n, dtype=torch.float16, device="cuda")
+        torch.ops._C.moe_fc(xq, w.cuda(), lod.cuda(), idx, 1, y, act, mx, w_max.cuda())
+        y_ref, _ = co.grouped_gemm_i8(q_ref, mx_ref, w.numpy(), w_max.numpy(), lod.numpy(), act=1 if act else 0, f16=True)
+        assert np.array_equal(hbits(y[:, :cols] if act else y), y_ref)
+    # silu_and_mul and moe_post
+    y = torch.randn(R, 2 * n, generator=g).half()
+    out = torch.empty(R, n, dtype=torch.float16, device="cuda")
+    torch.ops._C.silu_and_mul(out, y.cuda())
+    assert np.array_equal(hbits(out), co.silu_and_mul(hbits(y), f16=True))
+    M, K, H = 9, 4, 64
+    rows = torch.randn(M * K, H, generator=g).half()
+    idx2 = torch.randperm(M * K, generator=g).int().view(M, K)
+    wts = torch.rand(M, K, generator=g)
+    outp = torch.empty(M, H, dtype=torch.float16, device="cuda")
+    torch.ops._C.moe_post(rows.cuda(), idx2.cuda(), wts.cuda(), torch.ones(M, K, device="cuda"), outp)
+    assert np.array_equal(hbits(outp), co.combine(hbits(rows), idx2.numpy(), wts.numpy(), f16=True))
+    # dense Linear: both the weight-streaming path (few rows) and the tile kernel (many)
+    wq, sc = tm.quantize_weight_per_channel(torch.randn(256, 512, generator=g) * 0.05)
+    lin = SimpleNamespace(weight=torch.nn.Parameter(wq.cuda(), requires_grad=False),
+                          weight_scale=torch.nn.Parameter(sc.clone().cuda(), requires_grad=False), input_scale=None)
+    kern = KunlunScaledMMLinearKernel()
+    kern.process_weights_after_loading(lin)
+    for rows_n in (24, 600):
+        xx = (torch.randn(rows_n, 512, generator=g) * 1.5).half()
+        got = kern.apply_weights(lin, xx.cuda())
+        qq, mm = co.quant_i8_rows(hbits(xx), f16=True)
+        ref, _ = co.grouped_gemm_i8(qq, mm, wq.numpy()[None], (sc * 127).reshape(1, -1).numpy(),
+                                    np.array([0, rows_n], np.int32), f16=True)
+        assert got.dtype == torch.float16 and np.array_equal(hbits(got), ref)
+    torch.cuda.synchronize()
+
+
+def test_float16_is_refused_where_it_is_not_served():
+    from vllm_kunlun_amd import synth
+    shape = synth.scaled(synth.SHAPES["tiny-bf16"], M=8)
+    sl = synth.make_bf16_layer(shape, "cuda", seed=1)
+    with pytest.raises(NotImplementedError):
+        sl.layer(sl.x.half(), sl.logits)

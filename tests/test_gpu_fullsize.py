@@ -11,7 +11,6 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import bits
 
 pytestmark = pytest.mark.gpu
 
@@ -24,13 +23,18 @@ def _host(t):
     return None if t is None else t.detach().cpu()
 
 
+def bits(t):
+    """16-bit patterns of a bfloat16 or float16 tensor."""
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
 def _oracle(sl, host, x, logits):
     w13, w13_max, w2, w2_max, shared = host
     s = sl.shape
     sh = None if shared is None else tuple(t.numpy() for t in shared)
     return co.forward_w8a8(bits(x), _host(logits).float().numpy(), w13.numpy(), w13_max.numpy(), w2.numpy(),
                            w2_max.numpy(), s.K, s.scoring, True, s.n_group, s.topk_group, s.routed_scale,
-                           None if sl.bias is None else _host(sl.bias).numpy(), sh)
+                           None if sl.bias is None else _host(sl.bias).numpy(), sh, f16=x.dtype == torch.float16)
 
 
 def _run(sl, x, logits):
@@ -53,9 +57,9 @@ def dsv3():
     return sl, sl.host_weights()
 
 
-def _properties(sl, host, n_decode, n_spot, seed, mids=()):
+def _properties(sl, host, n_decode, n_spot, seed, mids=(), half=False):
     g = torch.Generator(device="cuda").manual_seed(seed)
-    x, logits = sl.x, sl.logits
+    x, logits = (sl.x.half() if half else sl.x), sl.logits
     M = x.shape[0]
     full = _run(sl, x, logits)
     assert bool(torch.isfinite(full.float()).all())
@@ -85,6 +89,12 @@ def test_qwen3_full_size(qwen3):
     _properties(sl, host, n_decode=64, n_spot=48, seed=1, mids=(160, 176, 512, 768, 800, 1500))
 
 
+def test_qwen3_full_size_float16(qwen3):
+    """The same layer with float16 activations (the dtype of the reference's deployment recipes)."""
+    sl, host = qwen3
+    _properties(sl, host, n_decode=64, n_spot=48, seed=4, mids=(160, 512, 1500), half=True)
+
+
 def test_qwen3_full_size_skewed_routing(qwen3):
     """+2.0 on the logits of 8 experts: a few experts get thousands of rows, most a handful."""
     sl, host = qwen3
@@ -100,6 +110,11 @@ def test_dsv3_full_size(dsv3):
     4096 and 128 tokens."""
     sl, host = dsv3
     _properties(sl, host, n_decode=128, n_spot=16, seed=2, mids=(320, 352, 1024, 1536, 1600))
+
+
+def test_dsv3_full_size_float16(dsv3):
+    sl, host = dsv3
+    _properties(sl, host, n_decode=128, n_spot=12, seed=5, mids=(352, 1536), half=True)
 
 
 def _fp8_oracle(sl, host, x, logits):

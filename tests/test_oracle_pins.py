@@ -659,3 +659,109 @@ def test_forward_fp8_against_a_per_expert_loop():
     no_shared = co.forward_fp8(bits(x), logits.numpy(), codes(w13), s13.numpy(), codes(w2), s2.numpy(), K, "sigmoid",
                                True, 3, 2, 1.0, bias.numpy())
     assert rel_l2(from_bits(no_shared), ref) > 0.1     # the shared expert and the factor are not optional extras
+
+
+# ------------------------------------------------------------------ float16 activations (int8 path)
+def test_half_conversions_match_numpy_float16():
+    """Every half pattern decodes to numpy's value; f32 -> half is numpy's round-to-nearest-even cast on ties,
+    subnormals, the overflow threshold, infinities and NaN."""
+    allbits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    got = co.half_bits_to_f32(allbits)
+    want = allbits.view(np.float16).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.all(np.isnan(got[np.isnan(want)]))
+    rng = np.random.default_rng(5)
+    vals = np.concatenate([
+        rng.standard_normal(20000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 20000).astype(np.float32),
+        np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 65536.0, 1e6, -1e6, np.inf, -np.inf, 2.0 ** -24, 2.0 ** -25,
+                  2.0 ** -25 * 1.0001, 3 * 2.0 ** -25, 2.0 ** -14, 2.0 ** -14 * (1 - 2.0 ** -11), 1.0 + 2.0 ** -11,
+                  1.0 + 3 * 2.0 ** -11, 1.0 + 2.0 ** -11 + 2.0 ** -20, 2047.5, 2048.5, 2049.5], np.float32),
+        # every tie between neighbouring halves in [1, 2): exactly representable in f32
+        (1.0 + (np.arange(1024) + 0.5) * 2.0 ** -10).astype(np.float32)])
+    with np.errstate(over="ignore"):
+        want_bits = vals.astype(np.float16).view(np.uint16)
+    assert np.array_equal(co.f32_to_half_bits(vals), want_bits)
+    assert co.f32_to_half_bits(np.array([np.nan], np.float32))[0] & 0x7c00 == 0x7c00
+
+
+def _half_bits(t: torch.Tensor) -> np.ndarray:
+    return t.to(torch.float16).contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _from_half_bits(b: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(b).view(np.int16)).view(torch.float16)
+
+
+def test_half_stages_closed_forms():
+    """The int8 path's stages with float16 activations: quantiser, GEMM epilogue, SiLU-mul and combine (with the
+    half form of the caller epilogue: the shared output scaled, not the routed sum) against numpy float16
+    arithmetic written out step by step."""
+    g = torch.Generator().manual_seed(31)
+    x = (torch.randn(7, 96, generator=g) * 3).half()
+    q, mx = co.quant_i8_rows(_half_bits(x), f16=True)
+    xf = x.float().numpy()
+    amax = np.abs(xf).max(1)
+    assert np.array_equal(mx, amax)
+    want_q = np.clip(np.rint(xf * (np.float32(127.0) / amax)[:, None]), -127, 127).astype(np.int8)
+    assert np.array_equal(q, want_q)
+    # GEMM epilogue: f16( (acc * a_max/127) * (w_max/127) ), SiLU-mul on the half-rounded gate and up
+    rng = np.random.default_rng(32)
+    E, n, k = 2, 64, 128
+    lod = np.array([0, 3, 7], np.int32)
+    w = rng.integers(-127, 128, (E, n, k), dtype=np.int8)
+    w_max = (rng.random((E, n)) * 0.05 + 0.01).astype(np.float32)
+    y, acc = co.grouped_gemm_i8(q[:, :k] if k <= 96 else np.pad(q, ((0, 0), (0, k - 96))), mx, w, w_max, lod,
+                                want_acc=True, f16=True)
+    qa = np.pad(q, ((0, 0), (0, k - 96)))
+    for e in range(E):
+        r0, r1 = lod[e], lod[e + 1]
+        a64 = qa[r0:r1].astype(np.int64) @ w[e].astype(np.int64).T
+        assert np.array_equal(acc[r0:r1], a64)
+        deq = (a64.astype(np.float32) * (mx[r0:r1, None] / np.float32(127))) * (w_max[e][None] / np.float32(127))
+        assert np.array_equal(y[r0:r1], deq.astype(np.float16).view(np.uint16))
+    fused, _ = co.grouped_gemm_i8(qa, mx, w, w_max, lod, act=1, f16=True)
+    assert np.array_equal(fused, co.silu_and_mul(y, f16=True))
+    yt = _from_half_bits(y).float()
+    silu_ref = (F.silu(yt[:, :n // 2].double()) * yt[:, n // 2:].double())
+    got = _from_half_bits(fused).double()
+    assert float((got - silu_ref).abs().max()) <= float(silu_ref.abs().max()) * 2 ** -10
+    assert not np.array_equal(fused, co.silu_and_mul(y, f16=False))           # the dtype switch is not a no-op
+    # combine: f32 accumulation over ascending k, one half rounding; epilogue routed*1 + f16(shared * s)
+    M, K, H = 5, 3, 32
+    rows = (torch.randn(M * K, H, generator=g) * 2).half()
+    wts = torch.rand(M, K, generator=g)
+    idx = torch.randperm(M * K, generator=g).int().view(M, K)
+    shared = torch.randn(M, H, generator=g).half()
+    s = np.float32(1.0 / 2.5)
+    out = co.combine(_half_bits(rows), idx.numpy(), wts.numpy(), addend=_half_bits(shared), addend_scale=float(s),
+                     f16=True)
+    rf = rows.float().numpy()
+    ref = np.zeros((M, H), np.float32)
+    for m in range(M):
+        accv = np.zeros(H, np.float32)
+        for kk in range(K):
+            accv = (np.float64(wts[m, kk].item()) * rf[idx[m, kk]].astype(np.float64) + accv.astype(np.float64)).astype(np.float32)  # fmaf
+        routed = accv.astype(np.float16)
+        sh = (shared[m].float().numpy() * s).astype(np.float16)
+        ref[m] = (routed.astype(np.float32) + sh.astype(np.float32)).astype(np.float16).astype(np.float32)
+    assert np.array_equal(out, ref.astype(np.float16).view(np.uint16))
+
+
+def test_half_layer_against_the_torch_expert_loop():
+    """co.forward_w8a8 with float16 activations against the dtype-generic torch loop run in float16, with the
+    half form of the caller epilogue (models/deepseek_v2.py:286-292)."""
+    x, logits, w13, w13_max, w2, w2_max, sh = _layer_inputs(24, 128, 8, 2, 64, seed=33, shared_I=64)
+    xh = x.half()
+    scale = 2.5
+    out = co.forward_w8a8(_half_bits(xh), logits.numpy(), w13.numpy(), w13_max.numpy(), w2.numpy(), w2_max.numpy(), 2,
+                          shared=tuple(t.numpy() for t in sh), shared_scale=1.0 / scale, f16=True)
+    routed = tm.w8a8_moe(xh, logits, w13, w13_max, w2, w2_max, 2)
+    dense = tm.w8a8_dense(xh, *sh)
+    ref = routed + dense * (1.0 / scale)
+    assert ref.dtype == torch.float16
+    assert rel_l2(_from_half_bits(out), ref) <= 1e-2
+    # bf16 and half runs of the same layer agree to within their precisions, and differ in their bits
+    out_b = co.forward_w8a8(bits(x), logits.numpy(), w13.numpy(), w13_max.numpy(), w2.numpy(), w2_max.numpy(), 2)
+    out_h = co.forward_w8a8(_half_bits(xh), logits.numpy(), w13.numpy(), w13_max.numpy(), w2.numpy(), w2_max.numpy(), 2,
+                            f16=True)
+    assert rel_l2(_from_half_bits(out_h), from_bits(out_b)) <= 2e-2

@@ -8,8 +8,8 @@ namespace {
 template <int TPR, int NV>
 __global__ __launch_bounds__(256) void quant_i8_rows_kernel(const uint16_t* __restrict__ x, int64_t ld_x, int R,
                                                            int C, int8_t* __restrict__ q, int64_t ld_q,
-                                                           float* __restrict__ row_max, int chunked) {
-  quant_i8_rows_body<TPR, NV>(x, ld_x, R, C, q, ld_q, row_max, chunked, blockIdx.x);
+                                                           float* __restrict__ row_max, int chunked, int f16) {
+  quant_i8_rows_body<TPR, NV>(x, ld_x, R, C, q, ld_q, row_max, chunked, blockIdx.x, f16 != 0);
 }
 
 // ------------------------------------------------------------- fp8 group128
@@ -57,7 +57,9 @@ __global__ __launch_bounds__(256) void quant_fp8_group128_kernel(const uint16_t*
 
 // ------------------------------------------------------------ silu-and-mul
 __global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __restrict__ y, int64_t ld_y, int R,
-                                                          int I, uint16_t* __restrict__ out, int64_t ld_out) {
+                                                          int I, uint16_t* __restrict__ out, int64_t ld_out,
+                                                          int dt) {
+  const bool f16 = dt != 0;
   const int vec_per_row = I / 8;
   const long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= static_cast<long long>(R) * vec_per_row) return;
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __res
   g.v = *reinterpret_cast<const uint4*>(y + static_cast<size_t>(r) * ld_y + c);
   u.v = *reinterpret_cast<const uint4*>(y + static_cast<size_t>(r) * ld_y + I + c);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) o.h[j] = f32_to_bf16(silu_fixed(bf16_to_f32(g.h[j])) * bf16_to_f32(u.h[j]));
+  for (int j = 0; j < 8; ++j) o.h[j] = f32_to_act(silu_fixed(act_to_f32(g.h[j], f16)) * act_to_f32(u.h[j], f16), f16);
   *reinterpret_cast<uint4*>(out + static_cast<size_t>(r) * ld_out + c) = o.v;
 }
 
@@ -79,8 +81,9 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
                                                      const float* __restrict__ topk_w,
                                                      const float* __restrict__ dq, int K, int H, float out_scale,
                                                      int epilogue, const uint16_t* __restrict__ addend,
-                                                     int64_t ld_addend, uint16_t* __restrict__ out,
-                                                     int64_t ld_out) {
+                                                     int64_t ld_addend, float addend_scale,
+                                                     uint16_t* __restrict__ out, int64_t ld_out, int dt) {
+  const bool f16 = dt != 0;
   __shared__ int rows[kMaxTopK];
   __shared__ float wts[kMaxTopK];
   const int m = blockIdx.x;
@@ -107,20 +110,22 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
         if (r[i] < 0) continue;  // pair without a sorted row contributes nothing (its load read row 0)
         const float w = wts[k0 + i];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(w, bf16_to_f32(p[i].h[j]), acc[j]);
+        for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(w, act_to_f32(p[i].h[j], f16), acc[j]);
       }
     }
     Pack8 o;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) o.h[j] = f32_to_bf16(acc[j]);
+    for (int j = 0; j < 8; ++j) o.h[j] = f32_to_act(acc[j], f16);
     if (epilogue) {
       Pack8 a;
       a.v = make_uint4(0, 0, 0, 0);
       if (addend) a.v = *reinterpret_cast<const uint4*>(addend + static_cast<size_t>(m) * ld_addend + c);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const uint16_t scaled = f32_to_bf16(bf16_to_f32(o.h[j]) * out_scale);
-        o.h[j] = addend ? f32_to_bf16(bf16_to_f32(scaled) + bf16_to_f32(a.h[j])) : scaled;
+        // each step rounds to the activation dtype, as the caller's tensor operations would
+        const uint16_t scaled = out_scale != 1.0f ? f32_to_act(act_to_f32(o.h[j], f16) * out_scale, f16) : o.h[j];
+        const uint16_t add = addend_scale != 1.0f ? f32_to_act(act_to_f32(a.h[j], f16) * addend_scale, f16) : a.h[j];
+        o.h[j] = addend ? f32_to_act(act_to_f32(scaled, f16) + act_to_f32(add, f16), f16) : scaled;
       }
     }
     *reinterpret_cast<uint4*>(out + static_cast<size_t>(m) * ld_out + c) = o.v;
@@ -187,32 +192,51 @@ using namespace kmoe;
 
 namespace {
 int quant_i8_launch(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q, float* row_max,
-                    int chunked, hipStream_t s, const char* what) {
+                    int chunked, int f16, hipStream_t s, const char* what) {
   if (C <= 64 * 8 * 2) {
     hipLaunchKernelGGL((quant_i8_rows_kernel<64, 2>), dim3(ceil_div(R, 4)), dim3(256), 0, s, x, ld_x, R, C, q, ld_q,
-                       row_max, chunked);
+                       row_max, chunked, f16);
   } else if (C <= 64 * 8 * 4) {
     hipLaunchKernelGGL((quant_i8_rows_kernel<64, 4>), dim3(ceil_div(R, 4)), dim3(256), 0, s, x, ld_x, R, C, q, ld_q,
-                       row_max, chunked);
+                       row_max, chunked, f16);
   } else if (C <= 256 * 8 * 4) {
     hipLaunchKernelGGL((quant_i8_rows_kernel<256, 4>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max,
-                       chunked);
+                       chunked, f16);
   } else if (C <= 256 * 8 * 8) {
     hipLaunchKernelGGL((quant_i8_rows_kernel<256, 8>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max,
-                       chunked);
+                       chunked, f16);
   } else if (C <= 256 * 8 * 16) {
     hipLaunchKernelGGL((quant_i8_rows_kernel<256, 16>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max,
-                       chunked);
+                       chunked, f16);
   } else {  // up to 65536 values: 128 registers of row data per thread
     hipLaunchKernelGGL((quant_i8_rows_kernel<256, 32>), dim3(R), dim3(256), 0, s, x, ld_x, R, C, q, ld_q, row_max,
-                       chunked);
+                       chunked, f16);
   }
   return check_launch(what);
 }
 }  // namespace
 
+namespace {
+int check_dtype(int act_dtype, const char* what) {
+  KMOE_REQUIRE(act_dtype == KMOE_DT_BF16 || act_dtype == KMOE_DT_F16, KMOE_ERR_UNSUPPORTED, "%s: act_dtype=%d unknown",
+               what, act_dtype);
+  return KMOE_OK;
+}
+}  // namespace
+
 extern "C" int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q,
                                   float* row_max, kmoe_stream_t stream) {
+  return kmoe_quant_i8_rows_dt(x, ld_x, R, C, q, ld_q, row_max, KMOE_DT_BF16, stream);
+}
+
+extern "C" int kmoe_quant_i8_rows_chunked(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, float* row_max,
+                                          kmoe_stream_t stream) {
+  return kmoe_quant_i8_rows_chunked_dt(x, ld_x, R, C, q, row_max, KMOE_DT_BF16, stream);
+}
+
+extern "C" int kmoe_quant_i8_rows_dt(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q,
+                                     float* row_max, int act_dtype, kmoe_stream_t stream) {
+  if (int rc = check_dtype(act_dtype, "quant_i8_rows")) return rc;
   KMOE_REQUIRE(x && q && row_max, KMOE_ERR_NULL, "quant_i8_rows: NULL pointer");
   KMOE_REQUIRE(R >= 0 && C >= 8 && C % 8 == 0 && C <= 65536, KMOE_ERR_SHAPE,
                "quant_i8_rows: R=%d C=%d (need C %% 8 == 0, 8 <= C <= 65536)", R, C);
@@ -220,18 +244,19 @@ extern "C" int kmoe_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C,
                "quant_i8_rows: row strides %lld/%lld must be multiples of 8 and >= C", (long long)ld_x,
                (long long)ld_q);
   if (R == 0) return KMOE_OK;
-  return quant_i8_launch(x, ld_x, R, C, q, ld_q, row_max, 0, as_stream(stream), "kmoe_quant_i8_rows");
+  return quant_i8_launch(x, ld_x, R, C, q, ld_q, row_max, 0, act_dtype, as_stream(stream), "kmoe_quant_i8_rows");
 }
 
-extern "C" int kmoe_quant_i8_rows_chunked(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, float* row_max,
-                                          kmoe_stream_t stream) {
+extern "C" int kmoe_quant_i8_rows_chunked_dt(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, float* row_max,
+                                             int act_dtype, kmoe_stream_t stream) {
+  if (int rc = check_dtype(act_dtype, "quant_i8_rows_chunked")) return rc;
   KMOE_REQUIRE(x && q && row_max, KMOE_ERR_NULL, "quant_i8_rows_chunked: NULL pointer");
   KMOE_REQUIRE(R >= 0 && C >= 64 && C % 64 == 0 && C <= 65536, KMOE_ERR_SHAPE,
                "quant_i8_rows_chunked: R=%d C=%d (need C %% 64 == 0, 64 <= C <= 65536)", R, C);
   KMOE_REQUIRE(ld_x % 8 == 0 && ld_x >= C, KMOE_ERR_SHAPE,
                "quant_i8_rows_chunked: row stride %lld must be a multiple of 8 and >= C", (long long)ld_x);
   if (R == 0) return KMOE_OK;
-  return quant_i8_launch(x, ld_x, R, C, q, 0, row_max, 1, as_stream(stream), "kmoe_quant_i8_rows_chunked");
+  return quant_i8_launch(x, ld_x, R, C, q, 0, row_max, 1, act_dtype, as_stream(stream), "kmoe_quant_i8_rows_chunked");
 }
 
 extern "C" int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, int C, uint8_t* q, int64_t ld_q,
@@ -278,6 +303,12 @@ extern "C" int kmoe_swigluoai_and_mul(const uint16_t* y, int64_t ld_y, int R, in
 
 extern "C" int kmoe_silu_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, uint16_t* out, int64_t ld_out,
                                  kmoe_stream_t stream) {
+  return kmoe_silu_and_mul_dt(y, ld_y, R, I, out, ld_out, KMOE_DT_BF16, stream);
+}
+
+extern "C" int kmoe_silu_and_mul_dt(const uint16_t* y, int64_t ld_y, int R, int I, uint16_t* out, int64_t ld_out,
+                                    int act_dtype, kmoe_stream_t stream) {
+  if (int rc = check_dtype(act_dtype, "silu_and_mul")) return rc;
   KMOE_REQUIRE(y && out, KMOE_ERR_NULL, "silu_and_mul: NULL pointer");
   KMOE_REQUIRE(R >= 0 && I >= 8 && I % 8 == 0, KMOE_ERR_SHAPE, "silu_and_mul: R=%d I=%d (need I %% 8 == 0)", R, I);
   KMOE_REQUIRE(ld_y % 8 == 0 && ld_out % 8 == 0 && ld_y >= 2 * I && ld_out >= I, KMOE_ERR_SHAPE,
@@ -285,7 +316,7 @@ extern "C" int kmoe_silu_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, 
   if (R == 0) return KMOE_OK;
   const long long n = static_cast<long long>(R) * (I / 8);
   hipLaunchKernelGGL(silu_and_mul_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0,
-                     as_stream(stream), y, ld_y, R, I, out, ld_out);
+                     as_stream(stream), y, ld_y, R, I, out, ld_out, act_dtype);
   return check_launch("kmoe_silu_and_mul");
 }
 
@@ -293,6 +324,15 @@ extern "C" int kmoe_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_
                             const float* dequant_scale, int M, int K, int H, float out_scale,
                             const uint16_t* addend, int64_t ld_addend, uint16_t* out, int64_t ld_out,
                             kmoe_stream_t stream) {
+  return kmoe_combine_dt(x, ld_x, moe_index, topk_w, dequant_scale, M, K, H, out_scale, addend, ld_addend, 1.0f, out,
+                         ld_out, KMOE_DT_BF16, stream);
+}
+
+extern "C" int kmoe_combine_dt(const uint16_t* x, int64_t ld_x, const int32_t* moe_index, const float* topk_w,
+                               const float* dequant_scale, int M, int K, int H, float out_scale,
+                               const uint16_t* addend, int64_t ld_addend, float addend_scale, uint16_t* out,
+                               int64_t ld_out, int act_dtype, kmoe_stream_t stream) {
+  if (int rc = check_dtype(act_dtype, "combine")) return rc;
   KMOE_REQUIRE(x && moe_index && topk_w && out, KMOE_ERR_NULL, "combine: NULL pointer");
   KMOE_REQUIRE(M >= 0 && K >= 1 && K <= kMaxTopK && H >= 8 && H % 8 == 0, KMOE_ERR_SHAPE,
                "combine: M=%d K=%d H=%d (need 1 <= K <= 64, H %% 8 == 0)", M, K, H);
@@ -303,6 +343,7 @@ extern "C" int kmoe_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_
   if (M == 0) return KMOE_OK;
   const int epilogue = (out_scale != 1.0f || addend) ? 1 : 0;
   hipLaunchKernelGGL(combine_kernel, dim3(M, ceil_div(H, 256 * 8)), dim3(256), 0, as_stream(stream), x, ld_x, moe_index, topk_w,
-                     dequant_scale, K, H, out_scale, epilogue, addend, ld_addend, out, ld_out);
+                     dequant_scale, K, H, out_scale, epilogue, addend, ld_addend, addend ? addend_scale : 1.0f, out, ld_out,
+                     act_dtype);
   return check_launch("kmoe_combine");
 }

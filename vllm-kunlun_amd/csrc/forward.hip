@@ -59,6 +59,9 @@ int check_shape(const kmoe_moe_args* a) {
   KMOE_REQUIRE(a->I_shared >= 0 && a->I_shared % mult == 0, KMOE_ERR_SHAPE,
                "moe_forward: I_shared=%d must be a non-negative multiple of %d", a->I_shared, mult);
   KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "moe_forward: M*K too large");
+  KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 || (a->act_dtype == KMOE_DT_F16 && a->format == KMOE_FMT_INT8),
+               KMOE_ERR_UNSUPPORTED, "moe_forward: act_dtype=%d (half activations go with the int8 format only)",
+               a->act_dtype);
   // elements in 64 bytes of a weight row
   const int row64 = a->format == KMOE_FMT_BF16 ? 32 : (a->format == KMOE_FMT_W4A16 ? 128 : 64);
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR ||
@@ -127,6 +130,7 @@ struct MlpPass {
   const uint16_t *w13_scale, *w2_scale;
   int group_size;
   int variant;  // INT8: kernel variant of the two GEMMs (0: from the shape)
+  int act_dtype;  // INT8: KMOE_DT_* of x_rows' source, act and out
 };
 
 int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
@@ -160,6 +164,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.act = act;
     g.w_layout = m.w_layout;
     g.variant = m.variant;
+    g.act_dtype = m.act_dtype;
     if (m.stream) {
       g.a_layout = KMOE_A_CHUNKED;
       g.a_rows = first ? m.x_count : m.rows + m.tail_rows;
@@ -251,8 +256,10 @@ int run_mlp(const MlpPass& m, kmoe_stream_t stream, Mark&& mark) {
   mark(KMOE_STAGE_QUANT2, 0);
   if (m.format == KMOE_FMT_INT8) {
     const int qrows = m.rows + m.tail_rows;
-    rc = m.stream ? kmoe_quant_i8_rows_chunked(m.act, m.I, qrows, m.I, static_cast<int8_t*>(m.actq), m.act_aux, stream)
-                  : kmoe_quant_i8_rows(m.act, m.I, qrows, m.I, static_cast<int8_t*>(m.actq), m.I, m.act_aux, stream);
+    rc = m.stream ? kmoe_quant_i8_rows_chunked_dt(m.act, m.I, qrows, m.I, static_cast<int8_t*>(m.actq), m.act_aux,
+                                                  m.act_dtype, stream)
+                  : kmoe_quant_i8_rows_dt(m.act, m.I, qrows, m.I, static_cast<int8_t*>(m.actq), m.I, m.act_aux,
+                                          m.act_dtype, stream);
   } else if (m.format == KMOE_FMT_FP8_BLOCK) {
     rc = kmoe_quant_fp8_group128(m.act, m.I, m.rows + m.tail_rows, m.I, static_cast<uint8_t*>(m.actq), m.I, m.act_aux,
                                  stream);
@@ -369,7 +376,8 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
     router_plan(M, H, E, &planes, &mf);
     float* buf = static_cast<float*>(at(L.logit_planes));
     plane_stride = static_cast<size_t>(M) * E;
-    rc = router_gemm_planes(a->x, H, a->w_gate, M, H, E, buf, plane_stride, E, planes, mf, as_stream(stream));
+    rc = router_gemm_planes(a->x, H, a->w_gate, M, H, E, buf, plane_stride, E, planes, mf, as_stream(stream),
+                            a->act_dtype == KMOE_DT_F16);
     if (rc) return rc;
     logits = buf;
   }
@@ -377,7 +385,8 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   if (a->format == KMOE_FMT_INT8 && M <= 1024) {
     rc = fused_route_quant_i8(logits, planes, plane_stride, a->bias, M, E, K, a->scoring == KMOE_SCORE_SIGMOID, a->renormalize, a->n_group,
                               a->topk_group, a->routed_scale, topk_w, topk_ids, a->x, H, static_cast<int8_t*>(at(L.xq)),
-                              static_cast<float*>(at(L.xmax)), stream_mode ? 1 : 0, as_stream(stream));
+                              static_cast<float*>(at(L.xmax)), stream_mode ? 1 : 0, a->act_dtype == KMOE_DT_F16,
+                              as_stream(stream));
     if (rc < 0) return rc;
     quant_done = rc == KMOE_OK;
     rc = KMOE_OK;
@@ -408,10 +417,10 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   if (quant_done) {
     x_rows = at(L.xq);
   } else if (a->format == KMOE_FMT_INT8) {
-    rc = stream_mode ? kmoe_quant_i8_rows_chunked(a->x, H, M, H, static_cast<int8_t*>(at(L.xq)),
-                                                  static_cast<float*>(at(L.xmax)), stream)
-                     : kmoe_quant_i8_rows(a->x, H, M, H, static_cast<int8_t*>(at(L.xq)), H,
-                                          static_cast<float*>(at(L.xmax)), stream);
+    rc = stream_mode ? kmoe_quant_i8_rows_chunked_dt(a->x, H, M, H, static_cast<int8_t*>(at(L.xq)),
+                                                     static_cast<float*>(at(L.xmax)), a->act_dtype, stream)
+                     : kmoe_quant_i8_rows_dt(a->x, H, M, H, static_cast<int8_t*>(at(L.xq)), H,
+                                             static_cast<float*>(at(L.xmax)), a->act_dtype, stream);
     x_rows = at(L.xq);
   } else if (a->format == KMOE_FMT_FP8_BLOCK) {
     rc = kmoe_quant_fp8_group128(a->x, H, M, H, static_cast<uint8_t*>(at(L.xq)), H, static_cast<float*>(at(L.xmax)),
@@ -445,6 +454,7 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   routed.w13_scale = a->w13_scale;
   routed.w2_scale = a->w2_scale;
   routed.group_size = a->group_size;
+  routed.act_dtype = a->act_dtype;
   if (a->format == KMOE_FMT_BF16) {
     routed.w13_bias = a->w13_bias;
     routed.w2_bias = a->w2_bias;
@@ -518,8 +528,10 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   mark(KMOE_STAGE_SHARED, 1);
   // 8. weighted combine (+ caller epilogue)
   mark(KMOE_STAGE_COMBINE, 0);
-  rc = kmoe_combine(static_cast<uint16_t*>(at(L.down)), H, moe_index, topk_w, nullptr, M, K, H, a->out_scale,
-                    shared_out, H, a->out, H, stream);
+  // shared_scale == 0 (a zeroed field) means 1
+  rc = kmoe_combine_dt(static_cast<uint16_t*>(at(L.down)), H, moe_index, topk_w, nullptr, M, K, H, a->out_scale,
+                       shared_out, H, a->shared_scale == 0.0f ? 1.0f : a->shared_scale, a->out, H, a->act_dtype,
+                       stream);
   mark(KMOE_STAGE_COMBINE, 1);
   return rc;
 }

@@ -71,6 +71,7 @@ struct GemmParams {
   const uint16_t* bias;    // NULL, or [E, n] bf16 added to the bf16 result (rounded again, as `gemm + bias` in bf16 is)
   int32_t oai;             // 1: out[r, i] = swigluoai(y[r, 2i], y[r, 2i+1]) (interleaved gate/up), n/2 outputs per row
   float oai_alpha, oai_limit;
+  int32_t f16;             // I8 only: outputs in IEEE half instead of bf16
 };
 
 // Rows of expert e, with the tail expert (e == E) taken from the host-side range.
@@ -332,6 +333,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
       const int r = row0 + mf * 16 + li;
       if (r >= row_end) continue;
       float sa = 1.0f;
+      const bool f16 = KIND == Kind::I8 && p.f16 != 0;
       if constexpr (KIND == Kind::I8) sa = p.a_max[srow[mf]] / 127.0f;
 #pragma unroll
       for (int f = 0; f < NFH; ++f) {
@@ -343,7 +345,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
             const float4 wm = *reinterpret_cast<const float4*>(w_aux + (tail ? 0 : static_cast<size_t>(e) * p.n) + cc);
             const float sw[4] = {wm.x / 127.0f, wm.y / 127.0f, wm.z / 127.0f, wm.w / 127.0f};
 #pragma unroll
-            for (int q = 0; q < 4; ++q) out[q] = f32_to_bf16((static_cast<float>(a[q]) * sa) * sw[q]);
+            for (int q = 0; q < 4; ++q) out[q] = f32_to_act((static_cast<float>(a[q]) * sa) * sw[q], f16);
             if (p.acc_out) *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + cc) = a;
           } else {
 #pragma unroll
@@ -355,7 +357,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
           uint16_t uv[4];
           finish(acc[mf][f + NFH], col[f + NFH] + lg * 4, uv);
 #pragma unroll
-          for (int q = 0; q < 4; ++q) yv[q] = f32_to_bf16(silu_fixed(bf16_to_f32(yv[q])) * bf16_to_f32(uv[q]));
+          for (int q = 0; q < 4; ++q) yv[q] = f32_to_act(silu_fixed(act_to_f32(yv[q], f16)) * act_to_f32(uv[q], f16), f16);
         }
         if constexpr (KIND == Kind::BF16 && !SWIGLU) {
           if (p.bias) {
@@ -441,6 +443,8 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
   KMOE_REQUIRE(a->k % 16 == 0, KMOE_ERR_SHAPE, "grouped_gemm_i8: k=%d must be a multiple of 16", a->k);
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
   KMOE_REQUIRE(a->act == KMOE_ACT_NONE || swiglu, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: act=%d unknown", a->act);
+  KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 || a->act_dtype == KMOE_DT_F16, KMOE_ERR_UNSUPPORTED,
+               "grouped_gemm_i8: act_dtype=%d unknown", a->act_dtype);
   KMOE_REQUIRE(a->n % (swiglu ? 32 : 16) == 0, KMOE_ERR_SHAPE, "grouped_gemm_i8: n=%d must be a multiple of %d",
                a->n, swiglu ? 32 : 16);
   KMOE_REQUIRE(a->a_layout == KMOE_A_CHUNKED || (a->lda % 16 == 0 && a->lda >= a->k), KMOE_ERR_SHAPE,
@@ -476,7 +480,8 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
   KMOE_REQUIRE(a->variant < 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-12 need tiled weights and k >= 128");
   GemmParams p{a->a,   a->lda, a->a_max, a->row_src, a->src_div, a->w,   a->w_max,
                a->lod, a->E,   a->n,     a->k,       a->y,       a->ldy, a->acc_out, a->w_layout == KMOE_W_TILED,
-               a->w_tail, a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0, nullptr, 0, 0.f, 0.f};
+               a->w_tail, a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0, nullptr, 0, 0.f, 0.f,
+               a->act_dtype == KMOE_DT_F16};
   return dispatch<Kind::I8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_i8");
 }
 

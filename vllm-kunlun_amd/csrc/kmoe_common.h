@@ -25,13 +25,13 @@ int tiled_gemm_bf16(const kmoe_gemm_bf16_args* args, hipStream_t stream);
 // when the arguments are outside its instantiations: the caller then uses the two entry points.
 int fused_route_quant_i8(const float* logits, int planes, size_t plane_stride, const float* bias, int M, int E, int K, int sigmoid, int renorm,
                          int n_group, int topk_group, float scale, float* topk_w, int32_t* topk_ids,
-                         const uint16_t* x, int H, int8_t* xq, float* xmax, int chunked, hipStream_t stream);
+                         const uint16_t* x, int H, int8_t* xq, float* xmax, int chunked, int f16, hipStream_t stream);
 
 // Router GEMM pieces for the fused layer: the split (ks planes, mf*16 tokens per wave) chosen for
 // a shape, and the launch that leaves the partial planes [ks][M][E] (ks == 1: the logits).
 void router_plan(int M, int H, int E, int* ks_out, int* mf_out);
 int router_gemm_planes(const uint16_t* x, int64_t ld_x, const uint16_t* w, int M, int H, int E, float* planes,
-                       size_t plane_stride, int64_t ld_out, int ks, int mf, hipStream_t stream);
+                       size_t plane_stride, int64_t ld_out, int ks, int mf, hipStream_t stream, bool f16 = false);
 // out[m,e] = planes[0][m,e] + planes[1][m,e] + ... (that order); out may be plane 0 itself.
 int router_reduce(const float* planes, size_t plane_stride, int n_planes, int M, int E, float* out, int64_t ld_out,
                   hipStream_t stream);
@@ -65,6 +65,26 @@ __device__ inline uint32_t pack2_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector((kmoe_v2f){lo, hi}, kmoe_v2bf));
 }
 __device__ inline uint16_t f32_to_bf16_hw(float f) { return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f)); }
+
+// ---- activation dtype: bf16 or IEEE half, chosen per call (a wave-uniform flag) ----------
+// Both are 16-bit patterns in uint16_t tensors. Conversions are round-to-nearest-even; a value
+// beyond the half range becomes infinity, as in every IEEE conversion.
+__device__ inline float half_to_f32(uint16_t h) { return static_cast<float>(__builtin_bit_cast(_Float16, h)); }
+// (The empty asm keeps the f32 value as it is: without it the compiler folds a preceding f32 multiplication into
+// a mixed-precision instruction that rounds the exact product to half ONCE, which differs from rounding it to
+// f32 first - the sequence the result contract fixes - whenever the f32 rounding lands on a half tie.)
+__device__ inline uint16_t f32_to_half(float f) {
+  asm("" : "+v"(f));
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+}
+__device__ inline float act_to_f32(uint16_t h, bool f16) { return f16 ? half_to_f32(h) : bf16_to_f32(h); }
+__device__ inline uint16_t f32_to_act(float f, bool f16) { return f16 ? f32_to_half(f) : f32_to_bf16(f); }
+typedef _Float16 kmoe_v2h __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t pack2_half(float lo, float hi) {
+  asm("" : "+v"(lo));
+  asm("" : "+v"(hi));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((kmoe_v2f){lo, hi}, kmoe_v2h));
+}
 
 // ---- fixed-sequence transcendental -----------------------------------------
 // exp(x) as one fixed sequence of IEEE single operations (mul, round-to-even,

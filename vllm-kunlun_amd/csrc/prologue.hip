@@ -27,6 +27,7 @@ struct QuantArgs {
   int64_t ld_q;
   float* row_max;
   int chunked;
+  int f16;
 };
 
 template <int SLOTS, bool SIGMOID, int TPR, int NV>
@@ -40,7 +41,7 @@ __global__ __launch_bounds__(256) void route_quant_kernel(const RouteArgs r, con
       softmax_topk_body<SLOTS>(r.logits, r.planes, r.plane_stride, r.M, r.E, r.K, r.renorm, r.topk_w, r.topk_ids, blockIdx.x);
   } else {
     quant_i8_rows_body<TPR, NV>(q.x, q.ld_x, q.R, q.C, q.q, q.ld_q, q.row_max, q.chunked,
-                                static_cast<int>(blockIdx.x) - routing_blocks);
+                                static_cast<int>(blockIdx.x) - routing_blocks, q.f16 != 0);
   }
 }
 
@@ -68,7 +69,7 @@ void launch_q(const RouteArgs& r, const QuantArgs& q, hipStream_t s) {
 // the caller runs the two stand-alone entry points, which also report bad arguments).
 int fused_route_quant_i8(const float* logits, int planes, size_t plane_stride, const float* bias, int M, int E, int K, int sigmoid, int renorm,
                          int n_group, int topk_group, float scale, float* topk_w, int32_t* topk_ids,
-                         const uint16_t* x, int H, int8_t* xq, float* xmax, int chunked, hipStream_t s) {
+                         const uint16_t* x, int H, int8_t* xq, float* xmax, int chunked, int f16, hipStream_t s) {
   if (M <= 0 || E < 1 || E > 512 || K < 1 || K > E || K > kWave) return 1;
   if (H < 16 || H % 16 || H > 256 * 8 * 4) return 1;
   if (sigmoid) {
@@ -81,7 +82,7 @@ int fused_route_quant_i8(const float* logits, int planes, size_t plane_stride, c
     }
   }
   const RouteArgs r{logits, planes, plane_stride, bias, M, E, K, renorm, n_group, topk_group, scale, topk_w, topk_ids};
-  const QuantArgs q{x, H, M, H, xq, chunked ? 0 : H, xmax, chunked};
+  const QuantArgs q{x, H, M, H, xq, chunked ? 0 : H, xmax, chunked, f16};
   const int slots = ceil_div(E, kWave);
   if (sigmoid) {
     if (slots <= 2) launch_q<2, true>(r, q, s);

@@ -5,7 +5,7 @@
 
 namespace kmoe {
 
-union Pack8 {  // 8 bf16
+union Pack8 {  // 8 bf16 (or half) values
   uint4 v;
   uint16_t h[8];
 };
@@ -17,7 +17,7 @@ union Pack8 {  // 8 bf16
 template <int TPR, int NV>
 __device__ inline void quant_i8_rows_body(const uint16_t* __restrict__ x, int64_t ld_x, int R, int C,
                                           int8_t* __restrict__ q, int64_t ld_q, float* __restrict__ row_max,
-                                          int chunked, int block) {
+                                          int chunked, int block, bool f16 = false) {
   constexpr int kRowsPerBlock = 256 / TPR;
   __shared__ float red[256 / kWave];
   const int sub = threadIdx.x / TPR;
@@ -35,7 +35,7 @@ __device__ inline void quant_i8_rows_body(const uint16_t* __restrict__ x, int64_
       if (v < nvec) {
         val[i].v = src[v];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(bf16_to_f32(val[i].h[j])));
+        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(act_to_f32(val[i].h[j], f16)));
       }
     }
   }
@@ -59,7 +59,7 @@ __device__ inline void quant_i8_rows_body(const uint16_t* __restrict__ x, int64_
       uint32_t w[2] = {0, 0};
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        float f = __builtin_rintf(bf16_to_f32(val[i].h[j]) * inv);
+        float f = __builtin_rintf(act_to_f32(val[i].h[j], f16) * inv);
         f = fminf(fmaxf(f, -127.0f), 127.0f);
         const int qi = static_cast<int>(f);
         w[j >> 2] |= static_cast<uint32_t>(qi & 0xff) << (8 * (j & 3));

@@ -15,6 +15,7 @@ namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr int kWavesR = 4;
@@ -22,7 +23,8 @@ constexpr int kWavesR = 4;
 // MF: 16-token fragments per wave, NF: 16-expert fragments per wave, D: MFMA steps of loads in flight.
 // <1,1,8> for small M (many small workgroups, deep prefetch: the launch is latency-bound),
 // <4,4,2> for large M (16 MFMAs per 8 fragment loads).
-template <int MF, int NF, int D>
+// F16: both operands are IEEE half (v_mfma_f32_16x16x32_f16) instead of bf16.
+template <int MF, int NF, int D, bool F16>
 __global__ __launch_bounds__(kWavesR* kWave) void router_gemm_kernel(
     const uint16_t* __restrict__ x, int64_t ld_x, const uint16_t* __restrict__ w, int M, int H, int E,
     float* __restrict__ planes, size_t plane_stride, int64_t ld_out, int steps_per_split) {
@@ -69,8 +71,12 @@ __global__ __launch_bounds__(kWavesR* kWave) void router_gemm_kernel(
     for (int mf = 0; mf < MF; ++mf)
 #pragma unroll
       for (int f = 0; f < NF; ++f)
-        acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wf[slot][f]),
-                                                             __builtin_bit_cast(v8bf, xf[slot][mf]), acc[mf][f], 0, 0, 0);
+        if constexpr (F16)
+          acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, wf[slot][f]),
+                                                              __builtin_bit_cast(v8h, xf[slot][mf]), acc[mf][f], 0, 0, 0);
+        else
+          acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wf[slot][f]),
+                                                               __builtin_bit_cast(v8bf, xf[slot][mf]), acc[mf][f], 0, 0, 0);
   };
 #pragma unroll
   for (int d = 0; d < D; ++d) load(d, s_begin + d);
@@ -131,17 +137,21 @@ void router_plan(int M, int H, int E, int* ks_out, int* mf_out) {
 
 // Partial planes [ks][M][E] (row stride ld_out) into `planes`; ks == 1 gives the logits themselves.
 int router_gemm_planes(const uint16_t* x, int64_t ld_x, const uint16_t* w, int M, int H, int E, float* planes,
-                       size_t plane_stride, int64_t ld_out, int ks, int mf, hipStream_t s) {
+                       size_t plane_stride, int64_t ld_out, int ks, int mf, hipStream_t s, bool f16) {
   const int ksteps = H / 32;
   const int steps_per_split = ceil_div(ksteps, ks);
   const int nf = mf;
   const dim3 grid(ceil_div(M, 16 * mf), ceil_div(E, kWavesR * nf * 16), ks);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(kWavesR * kWave), 0, s, x, ld_x, w, M, H, E, planes, plane_stride, ld_out,
+                       steps_per_split);
+  };
   if (mf == 4) {
-    hipLaunchKernelGGL((router_gemm_kernel<4, 4, 2>), grid, dim3(kWavesR * kWave), 0, s, x, ld_x, w, M, H, E, planes,
-                       plane_stride, ld_out, steps_per_split);
+    if (f16) go(router_gemm_kernel<4, 4, 2, true>);
+    else go(router_gemm_kernel<4, 4, 2, false>);
   } else {
-    hipLaunchKernelGGL((router_gemm_kernel<1, 1, 8>), grid, dim3(kWavesR * kWave), 0, s, x, ld_x, w, M, H, E, planes,
-                       plane_stride, ld_out, steps_per_split);
+    if (f16) go(router_gemm_kernel<1, 1, 8, true>);
+    else go(router_gemm_kernel<1, 1, 8, false>);
   }
   return check_launch("kmoe_router_gemm_bf16");
 }
@@ -168,6 +178,15 @@ extern "C" size_t kmoe_router_gemm_workspace_bytes(int M, int H, int E) {
 extern "C" int kmoe_router_gemm_bf16(const uint16_t* x, int64_t ld_x, const uint16_t* w_gate, int M, int H, int E,
                                      float* logits, int64_t ld_logits, void* workspace, size_t workspace_bytes,
                                      kmoe_stream_t stream) {
+  return kmoe_router_gemm(x, ld_x, w_gate, M, H, E, logits, ld_logits, workspace, workspace_bytes, KMOE_DT_BF16, stream);
+}
+
+extern "C" int kmoe_router_gemm(const uint16_t* x, int64_t ld_x, const uint16_t* w_gate, int M, int H, int E,
+                                float* logits, int64_t ld_logits, void* workspace, size_t workspace_bytes,
+                                int act_dtype, kmoe_stream_t stream) {
+  KMOE_REQUIRE(act_dtype == KMOE_DT_BF16 || act_dtype == KMOE_DT_F16, KMOE_ERR_UNSUPPORTED,
+               "router_gemm: act_dtype=%d unknown", act_dtype);
+  const bool f16 = act_dtype == KMOE_DT_F16;
   KMOE_REQUIRE(x && w_gate && logits, KMOE_ERR_NULL, "router_gemm_bf16: NULL pointer");
   KMOE_REQUIRE(M >= 0 && E >= 1 && E <= 1024 && H >= 32 && H % 32 == 0, KMOE_ERR_SHAPE,
                "router_gemm_bf16: M=%d H=%d E=%d (need H %% 32 == 0, 1 <= E <= 1024)", M, H, E);
@@ -180,13 +199,13 @@ extern "C" int kmoe_router_gemm_bf16(const uint16_t* x, int64_t ld_x, const uint
   int ks, mf;
   router_plan(M, H, E, &ks, &mf);
   hipStream_t s = as_stream(stream);
-  if (ks == 1) return router_gemm_planes(x, ld_x, w_gate, M, H, E, logits, 0, ld_logits, 1, mf, s);
+  if (ks == 1) return router_gemm_planes(x, ld_x, w_gate, M, H, E, logits, 0, ld_logits, 1, mf, s, f16);
   const size_t need = static_cast<size_t>(ks) * M * E * sizeof(float);
   KMOE_REQUIRE(workspace && workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0,
                KMOE_ERR_WORKSPACE, "router_gemm_bf16: workspace of %zu bytes (16-byte aligned) needed, got %zu", need,
                workspace_bytes);
   float* planes = static_cast<float*>(workspace);
   const size_t stride = static_cast<size_t>(M) * E;
-  if (int rc = router_gemm_planes(x, ld_x, w_gate, M, H, E, planes, stride, E, ks, mf, s)) return rc;
+  if (int rc = router_gemm_planes(x, ld_x, w_gate, M, H, E, planes, stride, E, ks, mf, s, f16)) return rc;
   return router_reduce(planes, stride, ks, M, E, logits, ld_logits, s);
 }

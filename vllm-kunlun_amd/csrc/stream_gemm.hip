@@ -38,6 +38,7 @@ struct StreamParams {
   const int8_t* w_tail;
   const float* w_max_tail;
   int32_t tail_row0, tail_rows, tail_src0;
+  int32_t f16;  // outputs (and the rounding of gate and up before SiLU-mul) in IEEE half instead of bf16
 };
 
 constexpr int kWaves = 4;
@@ -57,6 +58,7 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
   const int wk = wave_id % KS;     // K part of this wave
   const int li = lane & 15;
   const int lg = lane >> 4;
+  const bool f16 = p.f16 != 0;
 
   // blockIdx.y < E: routed expert, all its rows. Beyond: one 16*MF-row slice of the tail expert.
   const bool tail = static_cast<int>(blockIdx.y) >= p.E;
@@ -177,7 +179,7 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
           const float4 wm = *reinterpret_cast<const float4*>(w_max + cc);
           const float sw[4] = {wm.x / 127.0f, wm.y / 127.0f, wm.z / 127.0f, wm.w / 127.0f};
 #pragma unroll
-          for (int q = 0; q < 4; ++q) out[q] = f32_to_bf16((static_cast<float>(a[q]) * sa) * sw[q]);
+          for (int q = 0; q < 4; ++q) out[q] = f32_to_act((static_cast<float>(a[q]) * sa) * sw[q], f16);
           if (p.acc_out) *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + cc) = a;
         };
         finish(acc[mf][f], c0, yv);
@@ -185,7 +187,7 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
           uint16_t uv[4];
           finish(acc[mf][f + NFH], col[f + NFH] + lg * 4, uv);
 #pragma unroll
-          for (int q = 0; q < 4; ++q) yv[q] = f32_to_bf16(silu_fixed(bf16_to_f32(yv[q])) * bf16_to_f32(uv[q]));
+          for (int q = 0; q < 4; ++q) yv[q] = f32_to_act(silu_fixed(act_to_f32(yv[q], f16)) * act_to_f32(uv[q], f16), f16);
         }
         const uint2 packed = make_uint2(yv[0] | (static_cast<uint32_t>(yv[1]) << 16),
                                         yv[2] | (static_cast<uint32_t>(yv[3]) << 16));
@@ -224,7 +226,7 @@ __global__ void tile_weights_kernel(const int8_t* __restrict__ src, int8_t* __re
 int stream_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   StreamParams p{a->a, a->a_rows, a->a_max, a->row_src, a->src_div, a->w, a->w_max,
                  a->lod, a->E,     a->n,     a->k,       a->y,       a->ldy, a->acc_out,
-                 a->w_tail, a->w_max_tail, a->tail_row0, a->tail_rows, a->tail_src0};
+                 a->w_tail, a->w_max_tail, a->tail_row0, a->tail_rows, a->tail_src0, a->act_dtype == KMOE_DT_F16};
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
   // m-fragments per pass from the rows an expert gets under uniform routing
   int mf = a->variant;

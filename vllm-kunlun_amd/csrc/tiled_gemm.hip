@@ -168,9 +168,12 @@ struct Tile {
 // PACE: the m-tiles of one (expert, channel block) keep in step through the progress board (g_board): a tuning
 // variant that brings the bytes fetched by L2 down to about once per weight byte without changing the time
 // (the re-reads it removes were served by the memory-side cache, not by HBM).
+// F16 (int8 operands only): the outputs, and the rounding of gate and up before SiLU-mul, are IEEE half
+// instead of bf16.
 template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false,
-          bool PACE = false>
+          bool PACE = false, bool F16 = false>
 __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(const TiledParams p) {
+  static_assert(!F16 || KIND == TKind::I8, "half outputs are wired for the int8 path");
   static_assert(!OAI || (KIND == TKind::BF16 && !SWIGLU && !M32), "the interleaved activation is a bf16 epilogue");
   constexpr int kMF = MF;
   constexpr int kNA = 16 * kMF * (kChunk / 16) / (kWavesT * kWave);  // 16-byte activation vectors per thread and chunk
@@ -853,11 +856,12 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
             const int fu = fr + ANH;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-              const float g = bf16_to_f32(f32_to_bf16_hw(yv[q]));  // gate and up are bf16 values first
+              const float g = F16 ? half_to_f32(f32_to_half(yv[q]))
+                                  : bf16_to_f32(f32_to_bf16_hw(yv[q]));  // gate and up are 16-bit values first
               float uf;
               if constexpr (!I8) uf = acc[mf][fu][4 * b + q];
               else uf = (static_cast<float>(acc[mf][fu][4 * b + q]) * sa) * sw[fu][4 * b + q];
-              const float u = bf16_to_f32(f32_to_bf16_hw(uf));
+              const float u = F16 ? half_to_f32(f32_to_half(uf)) : bf16_to_f32(f32_to_bf16_hw(uf));
               yv[q] = silu_fixed(g) * u;
             }
           }
@@ -879,7 +883,8 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
                          : "memory");
           } else {
           // channel of yv[0] within the wave's output: fr * kFragRows + b * 8 + lg * 4
-          const uint2 packed = make_uint2(pack2_bf16(yv[0], yv[1]), pack2_bf16(yv[2], yv[3]));
+          const uint2 packed = F16 ? make_uint2(pack2_half(yv[0], yv[1]), pack2_half(yv[2], yv[3]))
+                                   : make_uint2(pack2_bf16(yv[0], yv[1]), pack2_bf16(yv[2], yv[3]));
           asm volatile("ds_write_b64 %0, %1 offset:%2"
                        :
                        : "v"(patch_wr), "v"(packed), "i"((fr * kFragRows + b * 8) * 2)
@@ -924,7 +929,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
 }
 
 template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false,
-          bool PACE = false>
+          bool PACE = false, bool F16 = false>
 int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* what) {
   constexpr int kTM = WM * 16 * MF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
@@ -936,7 +941,7 @@ int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* w
   // persistent workgroups: WGS per CU
   const int grid = min(min(ceil_div(p.max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8), kBoardSlots);
   const size_t dyn = sizeof(int) * (static_cast<size_t>(p.E) + 1 + n_exp + 1);
-  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32, MF, OAI, PACE>), dim3(grid),
+  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32, MF, OAI, PACE, F16>), dim3(grid),
                      dim3(WM * kWavesT * kWave), dyn, s, p);
   return check_launch(what);
 }
@@ -994,6 +999,28 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   int n_cu = 0;
   if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
   constexpr TKind K = TKind::I8;
+  const int avg_rows = ceil_div(a->rows + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
+  const bool shorter = short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu);
+  // 128-row tiles whose sibling m-tiles are paced against each other (see g_board). By default where most
+  // experts have one or two m-tiles (96 to 256 rows on average): there every second expert's weights are
+  // streamed twice, and keeping the two streams together is worth 3-5 % (DeepSeek-V3 shape, 4096 tokens:
+  // gate_up 1950 -> 1898 us, down 972 -> 926 us; bytes fetched by L2 1.49x -> 1.08x of the algorithmic ones).
+  // With four or five m-tiles per expert the chain of waits costs more than it saves (Qwen3 shape at 8192
+  // tokens: +3 to +8 %), with one tile there is nothing to pace.
+  const bool paced = a->variant == 12 || (a->variant == 0 && !shorter && avg_rows > 96 && avg_rows <= 256);
+  if (a->act_dtype == KMOE_DT_F16) {
+    // half outputs: the shapes in use (64-row, 128-row and paced 128-row tiles); the tuning variants are bf16 only
+    KMOE_REQUIRE(a->variant == 0 || a->variant == 5 || a->variant == 6 || a->variant == 11 || a->variant == 12,
+                 KMOE_ERR_UNSUPPORTED, "%s: variant %d is not instantiated for half outputs", what, a->variant);
+    if (paced)
+      return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 8, false, true, true>(p, a->rows, s, n_cu, what)
+                    : launch_tiled<K, false, 4, 4, 2, 1, false, 8, false, true, true>(p, a->rows, s, n_cu, what);
+    if (shorter)
+      return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4, false, false, true>(p, a->rows, s, n_cu, what)
+                    : launch_tiled<K, false, 4, 4, 2, 1, false, 4, false, false, true>(p, a->rows, s, n_cu, what);
+    return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 8, false, false, true>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 4, 4, 2, 1, false, 8, false, false, true>(p, a->rows, s, n_cu, what);
+  }
   // The 128-channel / deep-ring shape is a tuning variant only: measured slower than the
   // 256-channel shape (Qwen3 gate_up 321 vs 299 us, DeepSeek-V3 at 4096 tokens 2292 vs 1913 us):
   // twice the workgroups re-read the activations.
@@ -1009,17 +1036,10 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   // (the 32x32 shapes are instantiated for the gate_up launch only: without SiLU-mul the 16-register
   // fragments of the plain epilogue do not fit two workgroups per CU)
   if (a->variant == 9 && swiglu) return launch_tiled<K, true, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what);
-  // 128-row tiles whose sibling m-tiles are paced against each other (see g_board). By default where most
-  // experts have one or two m-tiles (96 to 256 rows on average): there every second expert's weights are
-  // streamed twice, and keeping the two streams together is worth 3-5 % (DeepSeek-V3 shape, 4096 tokens:
-  // gate_up 1950 -> 1898 us, down 972 -> 926 us; bytes fetched by L2 1.49x -> 1.08x of the algorithmic ones).
-  // With four or five m-tiles per expert the chain of waits costs more than it saves (Qwen3 shape at 8192
-  // tokens: +3 to +8 %), with one tile there is nothing to pace.
-  const int avg_rows = ceil_div(a->rows + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
-  if (a->variant == 12 || (a->variant == 0 && avg_rows > 96 && avg_rows <= 256))
+  if (paced)
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 8, false, true>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 8, false, true>(p, a->rows, s, n_cu, what);
-  if (short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu))
+  if (shorter)
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)

@@ -23,6 +23,7 @@ KMOE_FMT_INT8 = 0
 KMOE_FMT_FP8_BLOCK = 1
 KMOE_FMT_BF16 = 2
 KMOE_FMT_W4A16 = 3
+KMOE_DT_BF16, KMOE_DT_F16 = 0, 1
 KMOE_W_ROWMAJOR, KMOE_W_TILED = 0, 1
 KMOE_A_ROWMAJOR, KMOE_A_CHUNKED = 0, 1
 STAGES = ("routing", "align", "quant1", "gemm1", "quant2", "gemm2", "shared", "combine")
@@ -38,7 +39,7 @@ class GemmI8Args(C.Structure):
         ("y", C.c_void_p), ("ldy", C.c_int64), ("acc_out", C.c_void_p), ("act", C.c_int32),
         ("variant", C.c_int32), ("w_layout", C.c_int32), ("a_layout", C.c_int32), ("a_rows", C.c_int32),
         ("w_tail", C.c_void_p), ("w_max_tail", C.c_void_p), ("tail_row0", C.c_int32), ("tail_rows", C.c_int32),
-        ("tail_src0", C.c_int32),
+        ("tail_src0", C.c_int32), ("act_dtype", C.c_int32),
     ]
 
 
@@ -85,7 +86,8 @@ class MoEArgs(C.Structure):
         ("stage_events", C.POINTER(C.c_void_p)), ("w_layout", C.c_int32), ("w_gate", C.c_void_p),
         ("w13_bias", C.c_void_p), ("w2_bias", C.c_void_p), ("activation", C.c_int32), ("act_alpha", C.c_float),
         ("act_limit", C.c_float), ("ws_layout", C.c_int32),
-        ("w13_scale", C.c_void_p), ("w2_scale", C.c_void_p), ("group_size", C.c_int32), ("tile_variant", C.c_int32),
+        ("w13_scale", C.c_void_p), ("w2_scale", C.c_void_p), ("group_size", C.c_int32),
+        ("act_dtype", C.c_int32), ("shared_scale", C.c_float), ("tile_variant", C.c_int32),
     ]
 
 
@@ -129,6 +131,11 @@ def _load() -> C.CDLL:
         "kmoe_moe_workspace_layout": (i32, [C.POINTER(MoEArgs), C.POINTER(MoELayout)]),
         "kmoe_moe_forward": (i32, [C.POINTER(MoEArgs), vp, sz, vp]),
         "kmoe_moe_forward_static": (i32, [C.POINTER(MoEArgs), vp]),
+        "kmoe_quant_i8_rows_dt": (i32, [vp, i64, i32, i32, vp, i64, vp, i32, vp]),
+        "kmoe_quant_i8_rows_chunked_dt": (i32, [vp, i64, i32, i32, vp, vp, i32, vp]),
+        "kmoe_silu_and_mul_dt": (i32, [vp, i64, i32, i32, vp, i64, i32, vp]),
+        "kmoe_combine_dt": (i32, [vp, i64, vp, vp, vp, i32, i32, i32, f32, vp, i64, f32, vp, i64, i32, vp]),
+        "kmoe_router_gemm": (i32, [vp, i64, vp, i32, i32, i32, vp, i64, vp, sz, i32, vp]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)
@@ -144,6 +151,7 @@ EXPORTS = (
     "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_w4a16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
     "kmoe_moe_workspace_layout", "kmoe_moe_forward", "kmoe_router_gemm_workspace_bytes", "kmoe_router_gemm_bf16",
     "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16", "kmoe_moe_forward_static",
+    "kmoe_quant_i8_rows_dt", "kmoe_quant_i8_rows_chunked_dt", "kmoe_silu_and_mul_dt", "kmoe_combine_dt", "kmoe_router_gemm",
 )
 STATIC_WORKSPACE_BYTES = 64 << 20
 
@@ -163,6 +171,15 @@ def ptr(t: torch.Tensor | None):
 def stream():
     """The current torch HIP stream as a hipStream_t."""
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def act_dtype(t: torch.Tensor, what: str = "kmoe") -> int:
+    """KMOE_DT_* of an activation tensor (bfloat16 or float16; anything else is refused)."""
+    if t.dtype == torch.bfloat16:
+        return KMOE_DT_BF16
+    if t.dtype == torch.float16:
+        return KMOE_DT_F16
+    raise NotImplementedError(f"{what}: activations must be bfloat16 or float16, got {t.dtype}")
 
 
 def require_device(*tensors: torch.Tensor | None) -> None:

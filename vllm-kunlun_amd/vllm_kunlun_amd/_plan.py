@@ -159,8 +159,9 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
                   stage_events=None, w_layout: Optional[int] = None,
                   router_weight: Optional[torch.Tensor] = None, w13_bias: Optional[torch.Tensor] = None,
                   w2_bias: Optional[torch.Tensor] = None, activation: str = "silu", act_alpha: float = 1.702,
-                  act_limit: float = 7.0, group_size: Optional[int] = None, tile_variant: int = 0) -> MoEPlan:
-    """x bf16 [M,H], logits f32 [M,E], out bf16 [M,H]; w13 [E,2I,H], w2 [E,H,I] in the
+                  act_limit: float = 7.0, group_size: Optional[int] = None, tile_variant: int = 0,
+                  shared_scale: float = 1.0) -> MoEPlan:
+    """x bf16 [M,H] (or float16 with int8 weights), logits f32 [M,E], out [M,H] like x; w13 [E,2I,H], w2 [E,H,I] in the
     format's dtype; w13_aux/w2_aux: per-channel maxes (int8) or block scales (fp8), None for bf16.
     shared_expert: (ws13 [2Is,H], ws13_aux, ws2 [H,Is], ws2_aux) in the same format.
     logits may be None when router_weight (bf16 [E,H], the gate projection) is given: the
@@ -168,7 +169,8 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     and activation "swigluoai" (gate and up rows of w13 interleaved) select the expert-bias branch.
     KMOE_FMT_W4A16: w13 [E,2I,H/2] and w2 [E,H,I/2] uint8 (two 4-bit codes per byte), tiled;
     w13_aux/w2_aux their bf16 group scales [E,2I,H/group_size], [E,H,I/group_size].
-    tile_variant: a tuning variant of the int8 tile kernel for the routed GEMMs (kmoe_moe_args.tile_variant)."""
+    shared_scale multiplies the shared expert's output before it is added (the float16 form of the caller's
+    epilogue, models/deepseek_v2.py:286-292). tile_variant: a tuning variant of the int8 tile kernel for the routed GEMMs (kmoe_moe_args.tile_variant)."""
     if scoring_func not in ("softmax", "sigmoid"):
         raise ValueError(f"Unsupported scoring_func: {scoring_func}")
     if logits is None and router_weight is None:
@@ -176,8 +178,11 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     tensors = [x, logits, out, w13, w2, w13_aux, w2_aux, e_score_correction_bias, router_weight]
     L.require_device(*tensors)
     L.require_contig(*tensors)
-    if x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or (logits is not None and logits.dtype != torch.float32):
-        raise ValueError("moe plan: x/out must be bfloat16 and logits float32")
+    dt = L.act_dtype(x, "moe plan")
+    if dt == L.KMOE_DT_F16 and fmt != L.KMOE_FMT_INT8:
+        raise NotImplementedError("moe plan: float16 activations go with int8 weights only (bfloat16 otherwise)")
+    if out.dtype != x.dtype or (logits is not None and logits.dtype != torch.float32):
+        raise ValueError("moe plan: out must have x's dtype and logits must be float32")
     if w13.dtype not in _WEIGHT_DTYPE[fmt] or w2.dtype != w13.dtype:
         raise ValueError(f"moe plan: weight dtype {w13.dtype} does not fit the layer format")
     E, two_i, H = w13.shape
@@ -187,8 +192,8 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     M = x.shape[0]
     if tuple(x.shape) != (M, H) or tuple(out.shape) != (M, H) or (logits is not None and tuple(logits.shape) != (M, E)):
         raise ValueError("moe plan: x/out must be [M,H] and logits [M,E]")
-    if logits is None and (router_weight.dtype != torch.bfloat16 or tuple(router_weight.shape) != (E, H)):
-        raise ValueError("moe plan: router_weight must be bfloat16 [E,H]")
+    if logits is None and (router_weight.dtype != x.dtype or tuple(router_weight.shape) != (E, H)):
+        raise ValueError("moe plan: router_weight must be [E,H] in the activations' dtype")
     if tuple(w2.shape) != (E, H, two_i // (4 if w4 else 2)):
         raise ValueError("moe plan: w2 must be [E,H,I] for w13 [E,2I,H]")
     if w4:
@@ -246,6 +251,8 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     a.act_alpha, a.act_limit = float(act_alpha), float(act_limit)
     a.out_scale = float(out_scale)
     a.tile_variant = int(tile_variant)
+    a.act_dtype = dt
+    a.shared_scale = float(shared_scale)
     a.out = out.data_ptr()
     if w_layout is None:  # per group of weights: tiled if both of its tensors have been tiled
         w_layout = L.KMOE_W_TILED if is_tiled(w13) and is_tiled(w2) else L.KMOE_W_ROWMAJOR

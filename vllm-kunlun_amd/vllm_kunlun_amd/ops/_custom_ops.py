@@ -28,6 +28,11 @@ def _act_bits(t: torch.Tensor, what: str) -> torch.Tensor:
     return t
 
 
+def _dt(t: torch.Tensor, what: str) -> int:
+    """KMOE_DT_* of a bfloat16 or float16 activation tensor."""
+    return L.act_dtype(t, what)
+
+
 # --------------------------------------------------------------------- routing
 @custom_op("_C::moe_softmax_topk", mutates_args=("normed_score", "topk_index"))
 def moe_softmax_topk(x: torch.Tensor, normed_score: torch.Tensor, topk_index: torch.Tensor,
@@ -177,12 +182,12 @@ def quant2d(x: torch.Tensor, x_q: torch.Tensor, max: torch.Tensor, force_sdnn: b
     """Per-row dynamic int8; `max` receives the row ABSMAX (reference: ops/_custom_ops.py:1912-1924)."""
     L.require_device(x, x_q, max)
     L.require_contig(x, x_q, max)
-    _act_bits(x, "quant2d")
+    dt = _dt(x, "quant2d")
     _need(x_q.dtype == torch.int8 and max.dtype == torch.float32, "quant2d: x_q must be int8 and max float32")
     C = x.shape[-1]
     R = x.numel() // C
     _need(x_q.numel() == x.numel() and max.numel() == R, "quant2d: x_q/max shapes do not match x")
-    L.check(L.lib.kmoe_quant_i8_rows(L.ptr(x), C, R, C, L.ptr(x_q), C, L.ptr(max), L.stream()))
+    L.check(L.lib.kmoe_quant_i8_rows_dt(L.ptr(x), C, R, C, L.ptr(x_q), C, L.ptr(max), dt, L.stream()))
 
 
 @custom_op("_C::scaled_int8_quant", mutates_args=())
@@ -221,6 +226,7 @@ def _gemm_i8(a, a_max, w, w_max, lod, y2d, ldy, act, rows, row_src=None, src_div
     args.act = act
     args.variant = variant
     args.w_layout = weight_layout(w)
+    args.act_dtype = L.act_dtype(y2d, "int8 GEMM output")
     L.check(L.lib.kmoe_grouped_gemm_i8(args, L.stream()))
 
 
@@ -241,7 +247,7 @@ def moe_fc(x: torch.Tensor, weight: torch.Tensor, sorted_tokens_num_lod: torch.T
     if bias is not None or topk_w is not None or use_pack_int4 or scale_n or scale_k:
         raise NotImplementedError("moe_fc: bias / topk_w / int4 / block-scale arguments are not on this path")
     _need(act in (None, "SWISH_GLU"), f"moe_fc: act={act!r} unknown")
-    _act_bits(y, "moe_fc")
+    _dt(y, "moe_fc")
     E, n, k = weight.shape
     rows = x.numel() // k
     _need(x.shape[-1] == k and y.numel() == rows * n and sorted_tokens_num_lod.numel() == E + 1,
@@ -254,7 +260,7 @@ def moe_fc(x: torch.Tensor, weight: torch.Tensor, sorted_tokens_num_lod: torch.T
         _gemm_i8(x.view(rows, k), x_perchannel_max, weight, w_perchannel_max, sorted_tokens_num_lod,
                  y, n, L.KMOE_ACT_SWIGLU if act else L.KMOE_ACT_NONE, rows)
     elif x.dtype == _BF16:
-        _need(weight.dtype == _BF16, "moe_fc: bf16 x needs a bf16 weight")
+        _need(weight.dtype == _BF16 and y.dtype == _BF16, "moe_fc: bf16 x needs a bf16 weight and a bf16 y")
         g = L.GemmBf16Args()
         g.a, g.lda, g.src_div = x.data_ptr(), k, 1
         g.w, g.lod = weight.data_ptr(), sorted_tokens_num_lod.data_ptr()
@@ -297,7 +303,7 @@ def matmul(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, x_trans: bo
         raise NotImplementedError("matmul: only the int8 path with x_pc_max / w_pc_max is implemented")
     if x_trans or not w_trans or alpha != 1.0 or beta != 0.0 or bias is not None:
         raise NotImplementedError("matmul: x_trans / w_trans=False / alpha / beta / bias are not on this path")
-    if out_dtype != _BF16:
+    if out_dtype not in (_BF16, torch.float16):
         raise NotImplementedError(f"matmul: out_dtype {out_dtype} is not implemented")
     L.require_device(x, w, x_pc_max, w_pc_max)
     from .._plan import is_tiled
@@ -319,12 +325,12 @@ def silu_and_mul(out: torch.Tensor, x: torch.Tensor, axis: int = -1, turn: bool 
     """out = silu(x[..., :d]) * x[..., d:] (reference: ops/_custom_ops.py:699-706)."""
     L.require_device(out, x)
     L.require_contig(out, x)
-    _act_bits(x, "silu_and_mul")
+    dt = _dt(x, "silu_and_mul")
     _need(out.dtype == x.dtype, "silu_and_mul: out and x must share a dtype")
     two_i = x.shape[-1]
     R = x.numel() // two_i
     _need(two_i % 2 == 0 and out.numel() == R * (two_i // 2), "silu_and_mul: out must be [..., d] for x [..., 2d]")
-    L.check(L.lib.kmoe_silu_and_mul(L.ptr(x), two_i, R, two_i // 2, L.ptr(out), two_i // 2, L.stream()))
+    L.check(L.lib.kmoe_silu_and_mul_dt(L.ptr(x), two_i, R, two_i // 2, L.ptr(out), two_i // 2, dt, L.stream()))
 
 
 @custom_op("_C::moe_post", mutates_args=("y",))
@@ -334,15 +340,15 @@ def moe_post(x: torch.Tensor, moe_index: torch.Tensor, normed_scale: torch.Tenso
     (reference: ops/_custom_ops.py:1316-1324)."""
     L.require_device(x, moe_index, normed_scale, dequant_scale, y)
     L.require_contig(x, moe_index, normed_scale, dequant_scale, y)
-    _act_bits(x, "moe_post")
+    dt = _dt(x, "moe_post")
     _need(y.dtype == x.dtype and moe_index.dtype == torch.int32 and normed_scale.dtype == torch.float32
           and dequant_scale.dtype == torch.float32, "moe_post: dtypes must be (x, int32, float32, float32, x)")
     M, H = y.shape
     K = moe_index.numel() // M
     _need(x.numel() == M * K * H and normed_scale.numel() == M * K and dequant_scale.numel() == M * K,
           "moe_post: shapes must be x [M,K,H], index/scales [M,K], y [M,H]")
-    L.check(L.lib.kmoe_combine(L.ptr(x), H, L.ptr(moe_index), L.ptr(normed_scale), L.ptr(dequant_scale), M, K, H,
-                               1.0, None, 0, L.ptr(y), H, L.stream()))
+    L.check(L.lib.kmoe_combine_dt(L.ptr(x), H, L.ptr(moe_index), L.ptr(normed_scale), L.ptr(dequant_scale), M, K, H,
+                                  1.0, None, 0, 1.0, L.ptr(y), H, dt, L.stream()))
 
 
 # Fake (meta) implementations so the ops can be traced, as the reference registers for each op.
@@ -371,7 +377,8 @@ def _fake_swigluoai_and_mul(x, alpha=1.702, limit=7.0, axis=-1, turn=True):
 def router_gemm_bf16_fp32(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """bf16 [M,H] x bf16 [E,H]^T -> f32 [M,E] router logits (reference: ops.router_gemm_bf16_fp32,
     ops/fused_moe/router/gate_linear.py:105-108)."""
-    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "router_gemm_bf16_fp32: bf16 inputs only")
+    _need(x.dtype in (torch.bfloat16, torch.float16) and weight.dtype == x.dtype,
+          "router_gemm_bf16_fp32: bfloat16 (or float16) inputs of one dtype")
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "router_gemm_bf16_fp32: shapes")
     L.require_device(x, weight)
     x, weight = x.contiguous(), weight.contiguous()
@@ -380,8 +387,8 @@ def router_gemm_bf16_fp32(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor
     out = torch.empty((M, E), dtype=torch.float32, device=x.device)
     nbytes = L.lib.kmoe_router_gemm_workspace_bytes(M, H, E)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
-    L.check(L.lib.kmoe_router_gemm_bf16(L.ptr(x), H, L.ptr(weight), M, H, E, L.ptr(out), E, L.ptr(ws), nbytes,
-                                        L.stream()))
+    L.check(L.lib.kmoe_router_gemm(L.ptr(x), H, L.ptr(weight), M, H, E, L.ptr(out), E, L.ptr(ws), nbytes,
+                                   L.act_dtype(x, "router_gemm"), L.stream()))
     return out
 
 

@@ -17,7 +17,7 @@ from ... import _custom_ops  # noqa: F401  (registers torch.ops._C.router_gemm_b
 
 
 class GateLinear(torch.nn.Module):
-    """`forward(x) -> (logits, None)` like ReplicatedLinear; weight [num_experts, hidden] bf16."""
+    """`forward(x) -> (logits, None)` like ReplicatedLinear; weight [num_experts, hidden] bf16 (or float16, the model's dtype)."""
 
     def __init__(self, input_size: int, output_size: int, bias: bool = False,
                  out_dtype: Optional[torch.dtype] = None, params_dtype: Optional[torch.dtype] = None,
@@ -25,10 +25,10 @@ class GateLinear(torch.nn.Module):
         super().__init__()
         if bias:
             raise NotImplementedError("GateLinear: bias is not supported (the reference's MoE gates have none)")
-        if params_dtype not in (None, torch.bfloat16):
-            raise NotImplementedError(f"GateLinear: weights must be bfloat16, got {params_dtype}")
-        self.weight = torch.nn.Parameter(torch.zeros(output_size, input_size, dtype=torch.bfloat16, device=device),
-                                         requires_grad=False)
+        if params_dtype not in (None, torch.bfloat16, torch.float16):
+            raise NotImplementedError(f"GateLinear: weights must be bfloat16 or float16, got {params_dtype}")
+        self.weight = torch.nn.Parameter(torch.zeros(output_size, input_size, dtype=params_dtype or torch.bfloat16,
+                                                     device=device), requires_grad=False)
         self.out_dtype = out_dtype
         self.prefix = prefix
         self.e_score_correction_bias = None
@@ -39,8 +39,8 @@ class GateLinear(torch.nn.Module):
         self.out_dtype = out_dtype
 
     def forward(self, x: torch.Tensor):
-        if x.dtype != torch.bfloat16:
-            x = x.to(torch.bfloat16)
+        if x.dtype != self.weight.dtype:
+            x = x.to(self.weight.dtype)
         logits = torch.ops._C.router_gemm_bf16_fp32(x, self.weight)
         if self.out_dtype is not None and self.out_dtype != torch.float32:
             logits = logits.to(self.out_dtype)

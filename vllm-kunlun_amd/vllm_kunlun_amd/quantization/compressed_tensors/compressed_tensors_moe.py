@@ -136,27 +136,31 @@ class _MonolithicQuantMoE:
         shared_expert=None,
         out_scale: float = 1.0,
         router_weight: Optional[torch.Tensor] = None,
+        shared_scale: float = 1.0,
     ) -> Union[torch.Tensor, tuple]:
-        """x [M,H] bf16, router_logits [M,E] -> [M,H] bf16 (reference: :122-291).
-        `shared_expert` (w13, w13_max, w2, w2_max of a dense MLP in the layer's format) and
-        `out_scale` fold the caller's epilogue (models/deepseek_v2.py:288-296) into the call;
-        with `router_logits=None` and `router_weight` (the bf16 [E,H] weight of the gate,
+        """x [M,H] bf16 or float16 (float16 with int8 weights only), router_logits [M,E] -> [M,H] in x's dtype
+        (reference: :122-291).
+        `shared_expert` (w13, w13_max, w2, w2_max of a dense MLP in the layer's format), `out_scale` and
+        `shared_scale` fold the caller's epilogue (models/deepseek_v2.py:286-296) into the call:
+        `routed * out_scale + shared * shared_scale`, i.e. (routed_scaling_factor, 1) for bfloat16 and
+        (1, 1 / routed_scaling_factor) for float16, which the reference scales that way round against overflow;
+        with `router_logits=None` and `router_weight` (the [E,H] weight of the gate in x's dtype,
         models/deepseek_v2.py:178-184) the gate projection of :275 runs inside the call too."""
-        if x.dtype != torch.bfloat16:
-            raise NotImplementedError(f"apply_monolithic: activations must be bfloat16, got {x.dtype}")
+        if x.dtype not in (torch.bfloat16, torch.float16):
+            raise NotImplementedError(f"apply_monolithic: activations must be bfloat16 or float16, got {x.dtype}")
         x = x.contiguous()
         logits = None if router_logits is None else router_logits.float().contiguous()
         out = torch.empty((x.shape[0], layer.w2_weight.shape[1]), dtype=x.dtype, device=x.device)
         plan = self.make_plan(layer, x, logits, out, topk_group, num_expert_group, scoring_func,
                               routed_scaling_factor, e_score_correction_bias, shared_expert, out_scale,
-                              router_weight=router_weight)
+                              router_weight=router_weight, shared_scale=shared_scale)
         plan()
         self.last_layout, self.last_workspace = plan.layout, plan.workspace  # lets tests read the intermediates
         return out
 
     def make_plan(self, layer, x, logits, out, topk_group=None, num_expert_group=None, scoring_func="softmax",
                   routed_scaling_factor=1.0, e_score_correction_bias=None, shared_expert=None, out_scale=1.0,
-                  stage_events=None, router_weight=None) -> MoEPlan:
+                  stage_events=None, router_weight=None, shared_scale=1.0) -> MoEPlan:
         """Argument block for repeated calls on fixed buffers (x bf16 [M,H], logits f32
         [M,E], out bf16 [M,H], all contiguous): what a serving loop or a HIP-graph
         capture replays without touching Python-side allocation."""
@@ -166,7 +170,7 @@ class _MonolithicQuantMoE:
                              layer.w2_weight, layer.w13_weight_scale, layer.w2_weight_scale, scoring_func,
                              True,  # the reference always routes with the *_norm kernels
                              num_expert_group, topk_group, routed_scaling_factor, bias, shared_expert, out_scale,
-                             stage_events, router_weight=router_weight)
+                             stage_events, router_weight=router_weight, shared_scale=shared_scale)
 
 
 class KunlunCompressedTensorsW8A8Int8MoEMethod(_MonolithicQuantMoE):

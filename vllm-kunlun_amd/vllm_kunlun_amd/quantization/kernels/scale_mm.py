@@ -103,8 +103,7 @@ class KunlunScaledMMLinearKernel:
             raise NotImplementedError("KunlunScaledMMLinearKernel: static input scales are not implemented")
         if bias is not None:
             raise NotImplementedError("KunlunScaledMMLinearKernel: bias is not implemented on this path")
-        if x.dtype != torch.bfloat16:
-            raise NotImplementedError(f"KunlunScaledMMLinearKernel: activations must be bf16, got {x.dtype}")
+        dt = L.act_dtype(x, "KunlunScaledMMLinearKernel")
         w = getattr(layer, "_kmoe_w_1nk", None)
         if w is None:
             raise RuntimeError("KunlunScaledMMLinearKernel: process_weights_after_loading has not run on this layer")
@@ -141,7 +140,8 @@ class KunlunScaledMMLinearKernel:
         n = w.shape[1]
         x_q = torch.empty((k // 64, M, 64), dtype=torch.int8, device=x2.device)  # chunk-major codes
         x_max = torch.empty((M,), dtype=torch.float32, device=x2.device)
-        L.check(L.lib.kmoe_quant_i8_rows_chunked(L.ptr(x2), k, M, k, L.ptr(x_q), L.ptr(x_max), L.stream()))
+        L.check(L.lib.kmoe_quant_i8_rows_chunked_dt(L.ptr(x2), k, M, k, L.ptr(x_q), L.ptr(x_max),
+                                                    L.act_dtype(x2), L.stream()))
         g = L.GemmI8Args()
         g.a, g.lda, g.a_max, g.src_div = x_q.data_ptr(), k, x_max.data_ptr(), 1
         g.a_layout, g.a_rows = L.KMOE_A_CHUNKED, M
@@ -151,5 +151,6 @@ class KunlunScaledMMLinearKernel:
         g.w_tail, g.w_max_tail = w.data_ptr(), w_max.data_ptr()
         g.tail_row0, g.tail_rows, g.tail_src0 = 0, M, 0
         g.y, g.ldy, g.act, g.w_layout = out.data_ptr(), n, L.KMOE_ACT_NONE, L.KMOE_W_TILED
+        g.act_dtype = L.act_dtype(out)
         g.variant = 1 if M <= 128 else 2  # 16 or 32 rows per slice
         L.check(L.lib.kmoe_grouped_gemm_i8(g, L.stream()))

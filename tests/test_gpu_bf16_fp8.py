@@ -573,3 +573,52 @@ def test_w4a16_layer_on_the_packed_weights(native, group_size, M):
     w2 = co.dequant_w4_bf16(packed2.numpy(), bits(scale2), group_size or I)
     ref = co.forward_bf16(bits(x), logits.cpu().numpy(), w13, w2, K)
     assert rel_l2(out, from_bits(ref)) <= REL_L2_BF16
+
+
+@pytest.mark.parametrize("act", [None, "SWISH_GLU"])
+@pytest.mark.parametrize("tiled", [False, True])
+def test_moe_fc_op_block_scaled_fp8_and_packed_int4(act, tiled):
+    """`_C::moe_fc` with scale_n / scale_k (block-scaled fp8 operands) and with use_pack_int4 (packed 4-bit
+    weights): the operator's arguments reach the fp8 and the 4-bit grouped GEMM and give the oracle's result."""
+    import vllm_kunlun_amd  # noqa: F401
+    from vllm_kunlun_amd import _plan
+    torch.manual_seed(77)
+    E, n, k, counts = 3, 256, 384, [9, 0, 30]
+    lod = _lod(counts)
+    rows = int(lod[-1])
+    dl = torch.from_numpy(lod).cuda()
+    idx = torch.empty(0, dtype=torch.int32, device="cuda")
+    n_out = n // 2 if act else n
+    # fp8, 128 x 128 blocks
+    x = (torch.randn(rows, k) * 2).bfloat16()
+    xq, xs = tm.quant_fp8_group128(x)
+    wq, ws = tm.quantize_weight_fp8_block128(torch.randn(E, n, k) * 0.02)
+    ref = co.grouped_gemm_fp8(xq.view(torch.uint8).numpy(), xs.numpy(), wq.view(torch.uint8).numpy(), ws.numpy(), lod,
+                              act=1 if act else 0)
+    dw = wq.cuda()
+    if tiled:
+        assert _plan.tile_int8_weights_(dw)
+    y = torch.zeros(rows, n_out, dtype=torch.bfloat16, device="cuda")
+    torch.ops._C.moe_fc(xq.cuda(), dw, dl, idx, 1, y, act, xs.contiguous().cuda(), ws.contiguous().cuda(),
+                        scale_n=128, scale_k=128)
+    torch.cuda.synchronize()
+    assert rel_l2(y, from_bits(ref)) <= 2e-3
+    with pytest.raises(NotImplementedError):
+        torch.ops._C.moe_fc(xq.cuda(), dw, dl, idx, 1, y, act, xs.cuda(), ws.cuda(), scale_n=64, scale_k=128)
+    # packed 4-bit weights, groups of 128 along k; the kernel needs the packed bytes re-tiled
+    g = torch.Generator().manual_seed(78)
+    packed = torch.randint(0, 256, (E, n, k // 2), generator=g, dtype=torch.uint8)
+    scale = (torch.rand(E, n, k // 128, generator=g) * 0.02 + 0.002).bfloat16()
+    a = torch.randn(rows, k, generator=g).bfloat16()
+    w_bits = co.dequant_w4_bf16(packed.numpy(), bits(scale), 128)
+    ref4 = co.grouped_gemm_bf16(bits(a), w_bits, lod, act=1 if act else 0)
+    dp = packed.cuda()
+    y4 = torch.zeros(rows, n_out, dtype=torch.bfloat16, device="cuda")
+    if not tiled:
+        with pytest.raises(NotImplementedError):
+            torch.ops._C.moe_fc(a.cuda(), dp, dl, idx, 1, y4, act, None, scale.cuda(), scale_k=128, use_pack_int4=True)
+        return
+    assert _plan.tile_int8_weights_(dp)
+    torch.ops._C.moe_fc(a.cuda(), dp, dl, idx, 1, y4, act, None, scale.cuda(), scale_k=128, use_pack_int4=True)
+    torch.cuda.synchronize()
+    assert rel_l2(y4, from_bits(ref4)) <= 2e-3

@@ -230,6 +230,60 @@ def _gemm_i8(a, a_max, w, w_max, lod, y2d, ldy, act, rows, row_src=None, src_div
     L.check(L.lib.kmoe_grouped_gemm_i8(args, L.stream()))
 
 
+def _moe_fc_fp8(x, weight, lod, y, act, x_scale, w_scale, scale_n, scale_k) -> None:
+    """moe_fc with scale_n / scale_k (reference: ops/_custom_ops.py:1218-1221 merely passes them on): block-scaled
+    fp8-e4m3fn operands, one weight scale per scale_n x scale_k block, one activation scale per row and scale_k
+    columns. 128 x 128 blocks (the DeepSeek-V3 recipe) are what the kernels serve."""
+    from .._plan import weight_layout
+    if (scale_n, scale_k) != (128, 128):
+        raise NotImplementedError(f"moe_fc: block scales of {scale_n} x {scale_k} are not served (128 x 128 only)")
+    f8 = (torch.float8_e4m3fn, torch.uint8)
+    _need(x.dtype in f8 and weight.dtype in f8, "moe_fc: block-scaled operands must be float8_e4m3fn (or their bytes)")
+    _need(y.dtype == _BF16, "moe_fc: the block-scaled GEMM writes bfloat16")
+    E, n, k = weight.shape
+    rows = x.numel() // k
+    _need(x_scale is not None and w_scale is not None and x_scale.dtype == torch.float32
+          and w_scale.dtype == torch.float32, "moe_fc: block-scaled operands need float32 scales")
+    _need(x_scale.numel() == rows * (k // 128) and w_scale.numel() == E * (n // 128) * (k // 128),
+          "moe_fc: scales must be [P, k/128] and [E, n/128, k/128]")
+    n_out = n // 2 if act else n
+    _need(y.numel() in (rows * n_out, rows * n) and lod.numel() == E + 1, "moe_fc: x/y/lod shapes do not match weight")
+    g = L.GemmFp8Args()
+    g.a, g.lda, g.a_scale, g.src_div = x.data_ptr(), k, x_scale.data_ptr(), 1
+    g.w, g.w_scale, g.lod = weight.data_ptr(), w_scale.data_ptr(), lod.data_ptr()
+    g.E, g.n, g.k, g.rows = E, n, k, rows
+    g.y, g.ldy = y.data_ptr(), y.numel() // max(rows, 1) if rows else n_out
+    g.act = L.KMOE_ACT_SWIGLU if act else L.KMOE_ACT_NONE
+    g.w_layout = weight_layout(weight)
+    L.check(L.lib.kmoe_grouped_gemm_fp8_block(g, L.stream()))
+
+
+def _moe_fc_w4(x, weight, lod, y, act, w_scale, group_size) -> None:
+    """moe_fc with use_pack_int4: bfloat16 activations against packed 4-bit weights [E, n, k/2] (two codes per
+    byte, low nibble first, code - 8; re-tiled at load time) with bfloat16 group scales [E, n, k/group];
+    scale_k carries the group size (0: one scale per output channel)."""
+    from .._plan import weight_layout
+    _need(x.dtype == _BF16 and y.dtype == _BF16 and weight.dtype == torch.uint8,
+          "moe_fc: packed 4-bit weights are uint8 and go with bfloat16 activations")
+    E, n, half_k = weight.shape
+    k = 2 * half_k
+    rows = x.numel() // k
+    gs = group_size or k
+    _need(w_scale is not None and w_scale.dtype == _BF16 and w_scale.numel() == E * n * (k // gs),
+          "moe_fc: packed 4-bit weights need bfloat16 scales [E, n, k/group]")
+    if weight_layout(weight) != L.KMOE_W_TILED:
+        raise NotImplementedError("moe_fc: packed 4-bit weights must be re-tiled (tile_int8_weights_) first")
+    n_out = n // 2 if act else n
+    g = L.GemmW4Args()
+    g.a, g.lda, g.src_div = x.data_ptr(), k, 1
+    g.w, g.w_scale, g.group_size, g.lod = weight.data_ptr(), w_scale.data_ptr(), gs, lod.data_ptr()
+    g.E, g.n, g.k, g.rows = E, n, k, rows
+    g.y, g.ldy = y.data_ptr(), y.numel() // max(rows, 1) if rows else n_out
+    g.act = L.KMOE_ACT_SWIGLU if act else L.KMOE_ACT_NONE
+    g.w_layout = L.KMOE_W_TILED
+    L.check(L.lib.kmoe_grouped_gemm_w4a16(g, L.stream()))
+
+
 @custom_op("_C::moe_fc", mutates_args=("y",))
 def moe_fc(x: torch.Tensor, weight: torch.Tensor, sorted_tokens_num_lod: torch.Tensor,
            sorted_tokens_idx: torch.Tensor, moe_topk: int, y: torch.Tensor, act: Optional[str] = None,
@@ -244,10 +298,15 @@ def moe_fc(x: torch.Tensor, weight: torch.Tensor, sorted_tokens_num_lod: torch.T
     W8A8 path; act="SWISH_GLU" writes silu(gate)*up into the first n/2 columns of y."""
     L.require_device(x, weight, sorted_tokens_num_lod, y, x_perchannel_max, w_perchannel_max)
     L.require_contig(x, weight, sorted_tokens_num_lod, y, x_perchannel_max, w_perchannel_max)
-    if bias is not None or topk_w is not None or use_pack_int4 or scale_n or scale_k:
-        raise NotImplementedError("moe_fc: bias / topk_w / int4 / block-scale arguments are not on this path")
+    if bias is not None or topk_w is not None:
+        raise NotImplementedError("moe_fc: bias / topk_w are not on this path")
     _need(act in (None, "SWISH_GLU"), f"moe_fc: act={act!r} unknown")
     _dt(y, "moe_fc")
+    if use_pack_int4:
+        return _moe_fc_w4(x, weight, sorted_tokens_num_lod, y, act, w_perchannel_max, int(scale_k or 0))
+    if scale_n or scale_k:
+        return _moe_fc_fp8(x, weight, sorted_tokens_num_lod, y, act, x_perchannel_max, w_perchannel_max,
+                           int(scale_n or 0), int(scale_k or 0))
     E, n, k = weight.shape
     rows = x.numel() // k
     _need(x.shape[-1] == k and y.numel() == rows * n and sorted_tokens_num_lod.numel() == E + 1,

@@ -382,7 +382,7 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
     logits = buf;
   }
   // 1. routing; on the int8 decode path together with step 3 (independent work, one launch)
-  if (a->format == KMOE_FMT_INT8 && M <= 1024) {
+  if (a->format == KMOE_FMT_INT8) {
     rc = fused_route_quant_i8(logits, planes, plane_stride, a->bias, M, E, K, a->scoring == KMOE_SCORE_SIGMOID, a->renormalize, a->n_group,
                               a->topk_group, a->routed_scale, topk_w, topk_ids, a->x, H, static_cast<int8_t*>(at(L.xq)),
                               static_cast<float*>(at(L.xmax)), stream_mode ? 1 : 0, a->act_dtype == KMOE_DT_F16,

@@ -2,7 +2,8 @@
 // the two are independent (both read only the layer's inputs), so the first
 // workgroups route tokens while the rest quantise rows. Saves a launch and its
 // drain on the decode path, where each of the two kernels runs for a few
-// microseconds.
+// microseconds; at prefill sizes the latency-bound routing waves run under the
+// bandwidth-bound quantisation.
 #include "quant_body.h"
 #include "routing_body.h"
 

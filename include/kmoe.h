@@ -42,8 +42,8 @@ extern "C" {
 
 typedef void* kmoe_stream_t;
 
-/* Activation dtype of the int8 path: the 16-bit tensors (x, intermediates, out) hold bf16 or IEEE half
- * patterns. The reference runs its deployment recipes with --dtype float16 (ci/scripts/server/start_vllm.sh:26;
+/* Activation dtype of the int8 and unquantized paths: the 16-bit tensors (x, intermediates, out; the
+ * weights of the unquantized path) hold bf16 or IEEE half patterns. The reference runs its deployment recipes with --dtype float16 (ci/scripts/server/start_vllm.sh:26;
  * platforms/kunlun.py:350-364 admits float16 and bfloat16). Functions without an act_dtype argument take bf16. */
 #define KMOE_DT_BF16 0
 #define KMOE_DT_F16 1
@@ -257,13 +257,17 @@ typedef struct kmoe_gemm_bf16_args {
   const uint16_t* bias;   /* NULL, or [E, n] bf16: y = bf16(bf16(gemm) + bias), before the activation;
                              with KMOE_ACT_NONE or KMOE_ACT_SWIGLUOAI                  */
   float act_alpha, act_limit; /* KMOE_ACT_SWIGLUOAI (the reference uses 1.702 and 7.0)    */
+  int32_t act_dtype;      /* KMOE_DT_BF16, or KMOE_DT_F16: a, w and y are IEEE half (the
+                             unquantized method under --dtype float16); without bias / SWIGLUOAI */
 } kmoe_gemm_bf16_args;
 
 /*
  * Unquantized grouped GEMM: kunlun_ops.moe_fc with bf16 x and weight
  * (ops/_kunlun_ops.py:578-585, 595-603, 615-622; act="SWISH_GLU" at :595-603).
  *   y[r,c] = bf16( sum_k float(a[src(r),k]) * float(w[e,c,k]) ), f32 accumulation
- *   on MFMA (summation order is the hardware's; compare within tolerance).
+ *   on MFMA (summation order is the hardware's; compare within tolerance); with
+ *   act_dtype = KMOE_DT_F16 the same on half operands (v_mfma_f32_16x16x32_f16) with a
+ *   half result.
  * Limits: k % 8 == 0, n % 16 == 0 (SwiGLU: n % 32 == 0).
  */
 int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* args, kmoe_stream_t stream);
@@ -475,7 +479,8 @@ typedef struct kmoe_moe_args {
   const uint16_t* w13_scale; /* [E,2I,H/group_size] bf16                               */
   const uint16_t* w2_scale;  /* [E,H,I/group_size] bf16                                */
   int32_t group_size;    /* a multiple of 32 dividing H and I (one value for both tensors) */
-  int32_t act_dtype;     /* KMOE_DT_* of x, out (and w_gate, shared-expert output): half goes with KMOE_FMT_INT8 only */
+  int32_t act_dtype;     /* KMOE_DT_* of x, out (and w_gate, shared-expert output): half goes with KMOE_FMT_INT8 and
+                            with KMOE_FMT_BF16 (whose weights are then half too; no biases, no SWIGLUOAI) */
   float shared_scale;    /* caller epilogue for half activations (models/deepseek_v2.py:286-292: the routed sum stays
                             unscaled and the shared expert's output is multiplied by 1/routed_scaling_factor):
                             out = dt( dt(routed * out_scale) + dt(shared * shared_scale) ); 0 means 1 */

@@ -255,7 +255,9 @@ def router_gemm(x_bits, w_bits, f16=False):
     return logits, abs_sum
 
 
-def grouped_gemm_bf16(a_bits, w_bits, lod, act=0, row_src=None, src_div=1):
+def grouped_gemm_bf16(a_bits, w_bits, lod, act=0, row_src=None, src_div=1, f16=False):
+    """f16: operands and result hold IEEE half patterns instead of bf16."""
+    _dtype(f16)
     a_bits = _c(a_bits, np.uint16)
     w_bits = _c(w_bits, np.uint16)
     lod = _c(lod, np.int32)
@@ -329,20 +331,22 @@ def grouped_gemm_bf16_bias(a_bits, w_bits, bias_bits, lod, act=0, row_src=None, 
 
 
 def forward_bf16(x_bits, logits, w13_bits, w2_bits, K, scoring="softmax", renormalize=True, n_group=1, topk_group=1,
-                 routed_scale=1.0, bias=None, w13_bias=None, w2_bias=None, alpha=1.702, limit=7.0):
+                 routed_scale=1.0, bias=None, w13_bias=None, w2_bias=None, alpha=1.702, limit=7.0, f16=False):
     """Unquantized layer in the stage order of KunlunOps.fused_moe (ops/_kunlun_ops.py:412-637); with
     expert biases, its gpt-oss branch (:433-468): interleaved gate/up, swigluoai."""
     E = w13_bits.shape[0]
     w, ids = _route(logits, K, scoring, renormalize, n_group, topk_group, routed_scale, bias)
     moe_index, src, _, lod = align(ids, E)
     if w13_bias is not None or w2_bias is not None:
+        if f16:
+            raise NotImplementedError("the expert-bias branch is restated for bf16 only")
         act = grouped_gemm_bf16_bias(x_bits, w13_bits, w13_bias, lod, act=2, row_src=src, src_div=K, alpha=alpha,
                                      limit=limit)
         down = grouped_gemm_bf16_bias(act, w2_bits, w2_bias, lod)
     else:
-        act = grouped_gemm_bf16(x_bits, w13_bits, lod, act=1, row_src=src, src_div=K)
-        down = grouped_gemm_bf16(act, w2_bits, lod)
-    return combine(down, moe_index, w)
+        act = grouped_gemm_bf16(x_bits, w13_bits, lod, act=1, row_src=src, src_div=K, f16=f16)
+        down = grouped_gemm_bf16(act, w2_bits, lod, f16=f16)
+    return combine(down, moe_index, w, f16=f16)
 
 
 def forward_fp8(x_bits, logits, w13, w13_scale, w2, w2_scale, K, scoring="softmax", renormalize=True, n_group=1,

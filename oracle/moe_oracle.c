@@ -396,7 +396,9 @@ ORC_API void orc_router_gemm(const uint16_t* x, int64_t ld_x, const uint16_t* w,
 
 /* moe_fc with bf16 x and weight (ops/_kunlun_ops.py:578-585, 595-603, 615-622):
  * f32 accumulation in ascending k, one bf16 rounding. A device MFMA sums in its
- * own order, so comparisons with this function are within tolerance, not exact. */
+ * own order, so comparisons with this function are within tolerance, not exact.
+ * After orc_set_act_dtype(1) operands and result are IEEE half (the same method under
+ * --dtype float16; products of two halves are exact in f32 as those of two bf16 are). */
 ORC_API void orc_grouped_gemm_bf16(const uint16_t* a, int64_t lda, const int32_t* row_src, int src_div,
                                    const uint16_t* w, const int32_t* lod, int E, int n, int k, uint16_t* y,
                                    int64_t ldy, int act) {
@@ -412,14 +414,14 @@ ORC_API void orc_grouped_gemm_bf16(const uint16_t* a, int64_t lda, const int32_t
       for (int c = 0; c < nout; ++c) {
         float g = 0.0f, u = 0.0f;
         const uint16_t* wg = we + (size_t)c * k;
-        for (int i = 0; i < k; ++i) g += bf16_to_f32(ar[i]) * bf16_to_f32(wg[i]);
+        for (int i = 0; i < k; ++i) g += act_to_f32(ar[i]) * act_to_f32(wg[i]);
         if (act) {
           const uint16_t* wu = we + (size_t)(half + c) * k;
-          for (int i = 0; i < k; ++i) u += bf16_to_f32(ar[i]) * bf16_to_f32(wu[i]);
+          for (int i = 0; i < k; ++i) u += act_to_f32(ar[i]) * act_to_f32(wu[i]);
           y[(size_t)r * ldy + c] =
-              f32_to_bf16(orc_silu(bf16_to_f32(f32_to_bf16(g))) * bf16_to_f32(f32_to_bf16(u)));
+              f32_to_act(orc_silu(act_to_f32(f32_to_act(g))) * act_to_f32(f32_to_act(u)));
         } else {
-          y[(size_t)r * ldy + c] = f32_to_bf16(g);
+          y[(size_t)r * ldy + c] = f32_to_act(g);
         }
       }
     }

@@ -148,7 +148,119 @@ def test_half_operator_surface():
 
 def test_float16_is_refused_where_it_is_not_served():
     from vllm_kunlun_amd import synth
+    from vllm_kunlun_amd.ops._kunlun_ops import KunlunOps
     shape = synth.scaled(synth.SHAPES["tiny-bf16"], M=8)
     sl = synth.make_bf16_layer(shape, "cuda", seed=1)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError):  # unquantized weights must have the activations' dtype
         sl.layer(sl.x.half(), sl.logits)
+    w13, w2 = sl.layer.w13_weight.data.half(), sl.layer.w2_weight.data.half()
+    bias = torch.zeros(w13.shape[0], w13.shape[1], dtype=torch.float16, device="cuda")
+    with pytest.raises(NotImplementedError):  # the expert-bias branch is bf16 only
+        KunlunOps.fused_moe(sl.x.half(), w13, w2, sl.logits, 0, shape.K, True, w1_bias=bias)
+    fp8 = synth.make_fp8_layer(synth.scaled(synth.SHAPES["dsv3-fp8-decode"], M=8, H=256, E=8, K=2, I=128, n_group=2,
+                                            topk_group=1, I_shared=0), "cuda", seed=1)
+    with pytest.raises(NotImplementedError):
+        fp8.layer.quant_method.apply_monolithic(fp8.layer, fp8.x.half(), fp8.logits, **fp8.apply_kwargs())
+
+
+# ---------------------------------------------------------------- the unquantized path on half tensors
+# (UnquantizedFusedMoEMethod under --dtype float16: activations AND weights are half.) MFMA sums in its own
+# order, so these are held to a tolerance like the bf16 path (rel-L2 <= 1e-2 is the bar for 16-bit outputs);
+# half carries three more mantissa bits than bf16, and the results sit well inside 1e-3.
+REL_L2_HALF = 1e-3
+
+HALF_GEMM_CASES = [
+    (1, 64, 128, [16]),
+    (4, 64, 256, [3, 0, 17, 1]),
+    (2, 256, 1024, [130, 129]),
+    (3, 96, 320, [5, 140, 7]),
+    (8, 128, 64, [4, 4, 0, 9, 33, 1, 0, 2]),
+    (20, 1024, 128, [((53 * i) % 300) for i in range(20)]),
+    (2, 96, 160, [140, 3]),        # an odd number of 64-byte steps
+]
+
+
+@pytest.mark.parametrize("E,n,k,counts", HALF_GEMM_CASES)
+@pytest.mark.parametrize("tiled,variant", [(False, 1), (False, 2), (False, 3), (True, 0), (True, 1), (True, 2),
+                                           (True, 5), (True, 6), (True, 11)])
+@pytest.mark.parametrize("act", [0, 1])
+def test_unquantized_half_gemm(E, n, k, counts, tiled, variant, act):
+    from vllm_kunlun_amd import _lib as L
+    torch.manual_seed(E * n + k)
+    lod = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(lod[-1])
+    a = torch.randn(rows, k).half()
+    w = (torch.randn(E, n, k) * 0.05).half()
+    ref = co.grouped_gemm_bf16(hbits(a), hbits(w), lod, act=act, f16=True)
+    n_out = n // 2 if act else n
+    da, dw, dl = a.cuda(), w.cuda(), torch.from_numpy(lod).cuda()
+    y = torch.zeros(rows, n_out, dtype=torch.float16, device="cuda")
+    g = L.GemmBf16Args()
+    if tiled:
+        dt = torch.empty_like(dw)
+        L.check(L.lib.kmoe_tile_weights_i8(dw.data_ptr(), dt.data_ptr(), E, n, 2 * k, L.stream()))
+        dw = dt
+        g.w_layout = L.KMOE_W_TILED
+    g.a, g.lda, g.src_div = da.data_ptr(), k, 1
+    g.w, g.lod = dw.data_ptr(), dl.data_ptr()
+    g.E, g.n, g.k, g.rows = E, n, k, rows
+    g.y, g.ldy, g.act, g.variant = y.data_ptr(), n_out, act, variant
+    g.act_dtype = L.KMOE_DT_F16
+    L.check(L.lib.kmoe_grouped_gemm_bf16(g, L.stream()))
+    torch.cuda.synchronize()
+    assert rel_l2(y, from_hbits(ref)) <= 3e-4   # only the summation order differs
+    e = int(np.argmax(counts))                  # independent torch check of one expert
+    r0, r1 = lod[e], lod[e + 1]
+    t = a[r0:r1].float() @ w[e].float().T
+    if act:
+        gate, up = t[:, : n // 2].half().float(), t[:, n // 2:].half().float()
+        t = torch.nn.functional.silu(gate) * up
+    assert rel_l2(y[r0:r1], t) <= REL_L2_HALF
+
+
+@pytest.mark.parametrize("M,tiled", [(40, False), (40, True), (600, True), (3000, True)])
+@pytest.mark.parametrize("scoring", ["softmax", "sigmoid"])
+def test_unquantized_half_layer(M, tiled, scoring):
+    """KunlunOps.fused_moe on half tensors against the oracle's unquantized layer in its half mode: the
+    row-major kernels, the decode kernels on tiles, 64-row and 128-row tiles."""
+    from vllm_kunlun_amd._plan import tile_pair_
+    from vllm_kunlun_amd.ops._kunlun_ops import KunlunOps
+    g = torch.Generator().manual_seed(M)
+    E, K, H, I = 16, 4, 256, 128
+    x = torch.randn(M, H, generator=g).half()
+    logits = torch.randn(M, E, generator=g)
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * 0.06).half()
+    w2 = (torch.randn(E, H, I, generator=g) * 0.09).half()
+    bias = torch.randn(E, generator=g) * 0.1 if scoring == "sigmoid" else None
+    ref = co.forward_bf16(hbits(x), logits.numpy(), hbits(w13), hbits(w2), K, scoring, True, 4 if bias is not None else 1,
+                          2 if bias is not None else 1, 1.0, None if bias is None else bias.numpy(), f16=True)
+    d13, d2 = w13.cuda(), w2.cuda()
+    if tiled:
+        assert tile_pair_(d13, d2)
+    out = KunlunOps.fused_moe(x.cuda(), d13, d2, logits.cuda(), 0, K, True, scoring_func=scoring,
+                              num_expert_group=4 if bias is not None else None,
+                              topk_group=2 if bias is not None else None,
+                              e_score_correction_bias=None if bias is None else bias.cuda())
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16 and bool(torch.isfinite(out.float()).all())
+    assert rel_l2(out, from_hbits(ref)) <= REL_L2_HALF
+
+
+def test_unquantized_half_moe_fc_op():
+    import vllm_kunlun_amd  # noqa: F401
+    torch.manual_seed(0)
+    E, n, k = 4, 128, 256
+    counts = [10, 0, 33, 5]
+    lod = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)).cuda()
+    rows = sum(counts)
+    x = torch.randn(rows, k).half().cuda()
+    w = (torch.randn(E, n, k) * 0.05).half().cuda()
+    y = torch.zeros(rows, 1, n, dtype=torch.float16, device="cuda")
+    idx = torch.arange(rows, dtype=torch.int32, device="cuda")
+    torch.ops._C.moe_fc(x, w, lod, idx, 1, y, "SWISH_GLU")
+    torch.cuda.synchronize()
+    ref = co.grouped_gemm_bf16(hbits(x), hbits(w), lod.cpu().numpy(), act=1, f16=True)
+    assert rel_l2(y.view(rows, n)[:, : n // 2], from_hbits(ref)) <= 3e-4
+    assert torch.all(y.view(rows, n)[:, n // 2:] == 0)
+    with pytest.raises(Exception):  # weight of another dtype
+        torch.ops._C.moe_fc(x, w.bfloat16(), lod, idx, 1, y, "SWISH_GLU")

@@ -59,9 +59,14 @@ int check_shape(const kmoe_moe_args* a) {
   KMOE_REQUIRE(a->I_shared >= 0 && a->I_shared % mult == 0, KMOE_ERR_SHAPE,
                "moe_forward: I_shared=%d must be a non-negative multiple of %d", a->I_shared, mult);
   KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "moe_forward: M*K too large");
-  KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 || (a->act_dtype == KMOE_DT_F16 && a->format == KMOE_FMT_INT8),
-               KMOE_ERR_UNSUPPORTED, "moe_forward: act_dtype=%d (half activations go with the int8 format only)",
+  KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 ||
+                   (a->act_dtype == KMOE_DT_F16 && (a->format == KMOE_FMT_INT8 || a->format == KMOE_FMT_BF16)),
+               KMOE_ERR_UNSUPPORTED,
+               "moe_forward: act_dtype=%d (half activations go with the int8 and the unquantized format only)",
                a->act_dtype);
+  KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 || a->format != KMOE_FMT_BF16 ||
+                   (!a->w13_bias && !a->w2_bias && a->activation != KMOE_ACT_SWIGLUOAI),
+               KMOE_ERR_UNSUPPORTED, "moe_forward: expert biases and swigluoai are built for bf16 only");
   // elements in 64 bytes of a weight row
   const int row64 = a->format == KMOE_FMT_BF16 ? 32 : (a->format == KMOE_FMT_W4A16 ? 128 : 64);
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR ||
@@ -130,7 +135,7 @@ struct MlpPass {
   const uint16_t *w13_scale, *w2_scale;
   int group_size;
   int variant;  // INT8: kernel variant of the two GEMMs (0: from the shape)
-  int act_dtype;  // INT8: KMOE_DT_* of x_rows' source, act and out
+  int act_dtype;  // INT8, BF16: KMOE_DT_* of x_rows' source, act and out (BF16: of the weights too)
 };
 
 int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
@@ -243,6 +248,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
   g.bias = first ? m.w13_bias : m.w2_bias;
   g.act_alpha = m.act_alpha;
   g.act_limit = m.act_limit;
+  g.act_dtype = m.act_dtype;
   return kmoe_grouped_gemm_bf16(&g, stream);
 }
 

@@ -25,11 +25,12 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 constexpr int kKC = 256;          // bytes of K per chunk and row
 constexpr int kPitch = kKC + 16;  // LDS row pitch: 16 rows of a b128 read fall in 16 different bank groups
 
-enum class Kind { I8, BF16, FP8 };
+enum class Kind { I8, BF16, FP8, F16 };  // F16: the unquantized path on IEEE half operands and results
 
 template <Kind K> struct Traits;
 template <> struct Traits<Kind::I8> {
@@ -42,6 +43,7 @@ template <> struct Traits<Kind::BF16> {
   static constexpr int LB = 16;
   __device__ static acc_t zero() { return (v4f){0.f, 0.f, 0.f, 0.f}; }
 };
+template <> struct Traits<Kind::F16> : Traits<Kind::BF16> {};
 template <> struct Traits<Kind::FP8> {
   using acc_t = v4f;
   static constexpr int LB = 32;
@@ -276,6 +278,14 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
               acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wcur[f][j][0]),
                                                                    __builtin_bit_cast(v8bf, af[mf][0]), acc[mf][f], 0,
                                                                    0, 0);
+        } else if constexpr (KIND == Kind::F16) {
+#pragma unroll
+          for (int mf = 0; mf < MF; ++mf)
+#pragma unroll
+            for (int f = 0; f < NF; ++f)
+              acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, wcur[f][j][0]),
+                                                                  __builtin_bit_cast(v8h, af[mf][0]), acc[mf][f], 0, 0,
+                                                                  0);
         } else {
           // one MFMA = one 128-wide scale block: scale the block's partial sum, then add
           const int kb = chunk * kJ + j;
@@ -333,7 +343,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
       const int r = row0 + mf * 16 + li;
       if (r >= row_end) continue;
       float sa = 1.0f;
-      const bool f16 = KIND == Kind::I8 && p.f16 != 0;
+      const bool f16 = KIND == Kind::F16 || (KIND == Kind::I8 && p.f16 != 0);
       if constexpr (KIND == Kind::I8) sa = p.a_max[srow[mf]] / 127.0f;
 #pragma unroll
       for (int f = 0; f < NFH; ++f) {
@@ -349,7 +359,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
             if (p.acc_out) *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + cc) = a;
           } else {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) out[q] = f32_to_bf16(a[q]);
+            for (int q = 0; q < 4; ++q) out[q] = f32_to_act(a[q], KIND == Kind::F16);
           }
         };
         finish(acc[mf][f], c0, yv);
@@ -507,6 +517,11 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
   KMOE_REQUIRE(aligned(a->a, 16) && aligned(a->w, 16) && aligned(a->y, 8), KMOE_ERR_SHAPE,
                "grouped_gemm_bf16: misaligned tensor pointer");
   KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_bf16: src_div=%d < 1", a->src_div);
+  const bool half = a->act_dtype == KMOE_DT_F16;
+  KMOE_REQUIRE(half || a->act_dtype == KMOE_DT_BF16, KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: act_dtype=%d unknown",
+               a->act_dtype);
+  KMOE_REQUIRE(!half || (!a->bias && !oai), KMOE_ERR_UNSUPPORTED,
+               "grouped_gemm_bf16: expert biases and swigluoai are built for bf16 only");
   if (a->rows == 0) return KMOE_OK;
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR || (a->w_layout == KMOE_W_TILED && a->k % 32 == 0), KMOE_ERR_SHAPE,
                "grouped_gemm_bf16: w_layout=%d (tiled weights need k %% 32 == 0, k=%d)", a->w_layout, a->k);
@@ -519,6 +534,7 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
                reinterpret_cast<const int8_t*>(a->w), nullptr,    a->lod,  a->E,       a->n,
                a->k * 2,                              a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,
                nullptr, nullptr, 0, 0, 0, a->bias, oai ? 1 : 0, a->act_alpha, a->act_limit};
+  if (half) return dispatch<Kind::F16>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_bf16 (half)");
   return dispatch<Kind::BF16>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_bf16");
 }
 

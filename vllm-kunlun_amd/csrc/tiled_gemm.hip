@@ -43,6 +43,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 // Operand format. F8: e4m3fn codes with block scales (one f32 per 128x128 weight block and
@@ -165,15 +166,15 @@ struct Tile {
 // and registers for a third workgroup per CU).
 // OAI (bf16, no SiLU-mul): gate and up columns interleaved, the gpt-oss activation on each (gate, up) pair of
 // a lane's four consecutive channels - n / 2 outputs per row (ops/_custom_ops.py:728-742).
-// PACE: the m-tiles of one (expert, channel block) keep in step through the progress board (g_board): a tuning
-// variant that brings the bytes fetched by L2 down to about once per weight byte without changing the time
-// (the re-reads it removes were served by the memory-side cache, not by HBM).
-// F16 (int8 operands only): the outputs, and the rounding of gate and up before SiLU-mul, are IEEE half
-// instead of bf16.
+// PACE: the m-tiles of one (expert, channel block) keep in step through the progress board (g_board), which
+// brings the bytes fetched by L2 down to little more than once per weight byte where experts have two or three
+// m-tiles (int8: a few percent of time, the re-reads were mostly served by the memory-side cache; fp8: 14 %).
+// F16: the outputs, and the rounding of gate and up before SiLU-mul, are IEEE half instead of bf16 (int8
+// operands); with KIND = BF16 the operands are half as well (v_mfma_f32_16x16x32_f16).
 template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false,
           bool PACE = false, bool F16 = false>
 __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(const TiledParams p) {
-  static_assert(!F16 || KIND == TKind::I8, "half outputs are wired for the int8 path");
+  static_assert(!F16 || KIND == TKind::I8 || (KIND == TKind::BF16 && !OAI), "half is wired for the int8 and the plain unquantized path");
   static_assert(!OAI || (KIND == TKind::BF16 && !SWIGLU && !M32), "the interleaved activation is a bf16 epilogue");
   constexpr int kMF = MF;
   constexpr int kNA = 16 * kMF * (kChunk / 16) / (kWavesT * kWave);  // 16-byte activation vectors per thread and chunk
@@ -392,7 +393,10 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
       // slot entry 2 g + t: 32-channel fragment g, K bytes [32 t, 32 t + 32) of the step
 #pragma unroll
       for (int g = 0; g < AN; ++g) {
-        if constexpr (BF)
+        if constexpr (BF && F16)
+          acc[mf][g] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, wcur[2 * g + t]),
+                                                              __builtin_bit_cast(v8h, af), acc[mf][g], 0, 0, 0);
+        else if constexpr (BF)
           acc[mf][g] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, wcur[2 * g + t]),
                                                                __builtin_bit_cast(v8bf, af), acc[mf][g], 0, 0, 0);
         else if constexpr (I8)
@@ -401,7 +405,10 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     } else {
 #pragma unroll
       for (int f = 0; f < kNF; ++f) {
-        if constexpr (BF)
+        if constexpr (BF && F16)  // the unquantized path on half operands
+          acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, wcur[f]),
+                                                              __builtin_bit_cast(v8h, af), acc[mf][f], 0, 0, 0);
+        else if constexpr (BF)
           acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wcur[f]),
                                                                __builtin_bit_cast(v8bf, af), acc[mf][f], 0, 0, 0);
         else if constexpr (I8)
@@ -1093,6 +1100,13 @@ int tiled_gemm_bf16(const kmoe_gemm_bf16_args* a, hipStream_t s) {
   if (a->act == KMOE_ACT_SWIGLUOAI)
     return shorter ? launch_tiled<K, false, 4, 4, 2, 1, false, 4, true>(p, a->rows, s, n_cu, what)
                    : launch_tiled<K, false, 4, 4, 2, 1, false, 8, true>(p, a->rows, s, n_cu, what);
+  if (a->act_dtype == KMOE_DT_F16) {  // half operands and results (no bias, no interleaved activation: checked by the caller)
+    if (shorter)
+      return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4, false, false, true>(p, a->rows, s, n_cu, what)
+                    : launch_tiled<K, false, 4, 4, 2, 1, false, 4, false, false, true>(p, a->rows, s, n_cu, what);
+    return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 8, false, false, true>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 4, 4, 2, 1, false, 8, false, false, true>(p, a->rows, s, n_cu, what);
+  }
   if (shorter)
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);

@@ -50,6 +50,7 @@ class GemmBf16Args(C.Structure):
         ("E", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("rows", C.c_int32),
         ("y", C.c_void_p), ("ldy", C.c_int64), ("act", C.c_int32), ("variant", C.c_int32),
         ("w_layout", C.c_int32), ("bias", C.c_void_p), ("act_alpha", C.c_float), ("act_limit", C.c_float),
+        ("act_dtype", C.c_int32),
     ]
 
 

@@ -98,7 +98,7 @@ def weight_layout(w: torch.Tensor) -> int:
     return L.KMOE_W_TILED
 
 
-_TILEABLE = (torch.int8, torch.uint8, torch.float8_e4m3fn, torch.bfloat16)
+_TILEABLE = (torch.int8, torch.uint8, torch.float8_e4m3fn, torch.bfloat16, torch.float16)
 
 
 def tile_int8_weights_(w: torch.Tensor) -> bool:
@@ -148,7 +148,7 @@ def rowmajor_int8_weights(w: torch.Tensor) -> torch.Tensor:
 
 
 _WEIGHT_DTYPE = {L.KMOE_FMT_INT8: (torch.int8,), L.KMOE_FMT_FP8_BLOCK: (torch.float8_e4m3fn, torch.uint8),
-                 L.KMOE_FMT_BF16: (torch.bfloat16,), L.KMOE_FMT_W4A16: (torch.uint8,)}
+                 L.KMOE_FMT_BF16: (torch.bfloat16, torch.float16), L.KMOE_FMT_W4A16: (torch.uint8,)}
 
 
 def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Tensor, top_k: int,
@@ -161,7 +161,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
                   w2_bias: Optional[torch.Tensor] = None, activation: str = "silu", act_alpha: float = 1.702,
                   act_limit: float = 7.0, group_size: Optional[int] = None, tile_variant: int = 0,
                   shared_scale: float = 1.0) -> MoEPlan:
-    """x bf16 [M,H] (or float16 with int8 weights), logits f32 [M,E], out [M,H] like x; w13 [E,2I,H], w2 [E,H,I] in the
+    """x bf16 [M,H] (or float16 with int8 or unquantized weights, the latter then float16 too), logits f32 [M,E], out [M,H] like x; w13 [E,2I,H], w2 [E,H,I] in the
     format's dtype; w13_aux/w2_aux: per-channel maxes (int8) or block scales (fp8), None for bf16.
     shared_expert: (ws13 [2Is,H], ws13_aux, ws2 [H,Is], ws2_aux) in the same format.
     logits may be None when router_weight (bf16 [E,H], the gate projection) is given: the
@@ -179,8 +179,14 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     L.require_device(*tensors)
     L.require_contig(*tensors)
     dt = L.act_dtype(x, "moe plan")
-    if dt == L.KMOE_DT_F16 and fmt != L.KMOE_FMT_INT8:
-        raise NotImplementedError("moe plan: float16 activations go with int8 weights only (bfloat16 otherwise)")
+    if dt == L.KMOE_DT_F16 and fmt not in (L.KMOE_FMT_INT8, L.KMOE_FMT_BF16):
+        raise NotImplementedError("moe plan: float16 activations go with int8 and unquantized weights only "
+                                  "(bfloat16 otherwise)")
+    if fmt == L.KMOE_FMT_BF16 and w13.dtype != x.dtype:
+        raise ValueError(f"moe plan: unquantized weights ({w13.dtype}) must have the activations' dtype ({x.dtype})")
+    if fmt == L.KMOE_FMT_BF16 and dt == L.KMOE_DT_F16 and (w13_bias is not None or w2_bias is not None
+                                                           or activation == "swigluoai"):
+        raise NotImplementedError("moe plan: expert biases and swigluoai are built for bfloat16 only")
     if out.dtype != x.dtype or (logits is not None and logits.dtype != torch.float32):
         raise ValueError("moe plan: out must have x's dtype and logits must be float32")
     if w13.dtype not in _WEIGHT_DTYPE[fmt] or w2.dtype != w13.dtype:

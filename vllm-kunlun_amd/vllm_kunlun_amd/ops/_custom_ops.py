@@ -318,9 +318,10 @@ def moe_fc(x: torch.Tensor, weight: torch.Tensor, sorted_tokens_num_lod: torch.T
               "moe_fc: per-channel max shapes must be [P,1] and [E,n,1]")
         _gemm_i8(x.view(rows, k), x_perchannel_max, weight, w_perchannel_max, sorted_tokens_num_lod,
                  y, n, L.KMOE_ACT_SWIGLU if act else L.KMOE_ACT_NONE, rows)
-    elif x.dtype == _BF16:
-        _need(weight.dtype == _BF16 and y.dtype == _BF16, "moe_fc: bf16 x needs a bf16 weight and a bf16 y")
+    elif x.dtype in (_BF16, torch.float16):
+        _need(weight.dtype == x.dtype and y.dtype == x.dtype, "moe_fc: unquantized x needs weight and y of its dtype")
         g = L.GemmBf16Args()
+        g.act_dtype = L.act_dtype(x)
         g.a, g.lda, g.src_div = x.data_ptr(), k, 1
         g.w, g.lod = weight.data_ptr(), sorted_tokens_num_lod.data_ptr()
         g.E, g.n, g.k, g.rows = E, n, k, rows
@@ -330,7 +331,7 @@ def moe_fc(x: torch.Tensor, weight: torch.Tensor, sorted_tokens_num_lod: torch.T
         g.w_layout = weight_layout(weight)
         L.check(L.lib.kmoe_grouped_gemm_bf16(g, L.stream()))
     else:
-        raise NotImplementedError(f"moe_fc: x dtype {x.dtype} is outside this build's path (int8 or bfloat16)")
+        raise NotImplementedError(f"moe_fc: x dtype {x.dtype} is outside this build's path (int8, bfloat16 or float16)")
 
 
 _DENSE_LOD: dict = {}

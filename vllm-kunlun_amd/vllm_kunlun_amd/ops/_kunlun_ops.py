@@ -35,12 +35,11 @@ class KunlunOps:
         scoring_func: str = "softmax",
         e_score_correction_bias: Optional[torch.Tensor] = None,
     ) -> torch.Tensor:
-        """bf16 fused MoE (reference: ops/_kunlun_ops.py:377-637). As there, routing is
+        """Unquantized (bf16 or float16) fused MoE (reference: ops/_kunlun_ops.py:377-637). As there, routing is
         chosen by `scoring_func` alone and always normalises (`renormalize`,
         `use_grouped_topk` and `inplace` are accepted and ignored, :385-389 vs :413-431);
         the sigmoid path uses scale 1.0 (:428)."""
-        if hidden_states.dtype != torch.bfloat16:
-            raise NotImplementedError(f"fused_moe: activations must be bfloat16, got {hidden_states.dtype}")
+        L.act_dtype(hidden_states, "fused_moe")  # bfloat16 or float16; the weights must match
         x = hidden_states.contiguous()
         logits = router_logits.to(torch.float).contiguous()
         out = torch.empty_like(x)
@@ -76,8 +75,7 @@ class KunlunOps:
         ep_rank must be 0 and the local experts are the global ones."""
         if ep_rank != 0:
             raise NotImplementedError("fused_moe_ep: this build runs all experts on one GPU (ep_rank must be 0)")
-        if hidden_states.dtype != torch.bfloat16:
-            raise NotImplementedError(f"fused_moe_ep: activations must be bfloat16, got {hidden_states.dtype}")
+        L.act_dtype(hidden_states, "fused_moe_ep")
         x = hidden_states.contiguous()
         logits = router_logits.to(torch.float).contiguous()
         out = torch.empty_like(x)

@@ -26,7 +26,7 @@ class FusedMoEConfig:
 
 
 class KunlunUnquantizedFusedMoEMethod:
-    """bf16 weights, monolithic entry (reference: ops/fused_moe/layer.py:16-81)."""
+    """bf16 (or float16) weights in the activations' dtype, monolithic entry (reference: ops/fused_moe/layer.py:16-81)."""
 
     def __init__(self, moe: FusedMoEConfig):
         self.moe = moe

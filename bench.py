@@ -205,7 +205,7 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
     if a.router:
         gen = torch.Generator(device="cuda:0")
         gen.manual_seed(a.seed + 1)
-        w_gate = (torch.randn(shape.E, shape.H, generator=gen, device="cuda:0") * shape.H ** -0.5).bfloat16()  # logits ~ N(0,1)
+        w_gate = (torch.randn(shape.E, shape.H, generator=gen, device="cuda:0") * shape.H ** -0.5).to(x.dtype)  # logits ~ N(0,1)
 
     def make_plan(stage_events=None):
         # the argument block the plugin methods build (apply_monolithic / KunlunOps.fused_moe)
@@ -301,12 +301,13 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
     res = {
         "value": shape.M / t_s,
         "ms_per_step": ms_per_step,
-        "dtype": DTYPE[shape.quant],
+        "dtype": DTYPE[shape.quant].replace("bf16", "f16") if a.act_dtype == "f16" else DTYPE[shape.quant],
         "config": {"workload": label, "name": workload, "tokens": shape.M, "hidden": shape.H,
                    "experts": shape.E, "top_k": shape.K, "moe_intermediate": shape.I,
                    "shared_intermediate": shape.I_shared, "routing": shape.scoring, "experts_hit": n_active,
                    "launch": launch_mode, "launch_ms_per_step": launch_ms, "seed": a.seed,
-                   "router_gemm_inside": bool(a.router), "tile_variant": a.tile_variant},
+                   "router_gemm_inside": bool(a.router), "tile_variant": a.tile_variant,
+                   "activations": "float16" if a.act_dtype == "f16" else "bfloat16"},
         "roofline": roofline,
         "layer": {"hbm_gbs": work["layer_bytes"] / t_s / 1e9, "hbm_frac": work["layer_bytes"] / t_s / 1e9 / HBM_PEAK_GBS,
                   "tops": work["layer_ops"] / t_s / 1e12,
@@ -335,6 +336,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU work for the baseline sample")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--act-dtype", default="bf16", choices=["bf16", "f16"],
+                    help="16-bit type of the activations (and of unquantized weights / 4-bit group scales): the layer "
+                         "computes in the same arithmetic type either way; f16 is not built for the fp8 layers")
     ap.add_argument("--tokens", type=int, default=0,
                     help="run the workload's layer at another batch (tokens per call); the config then says so")
     ap.add_argument("--router", action="store_true",
@@ -396,7 +400,8 @@ def main():
         else:
             cached = None
             torch.cuda.empty_cache()
-            sl = synth.make_layer(shape, "cuda:0", seed=a.seed)
+            sl = synth.make_layer(shape, "cuda:0", seed=a.seed,
+                                  dtype=torch.float16 if a.act_dtype == "f16" else torch.bfloat16)
         cached = (weights_key(shape), sl)
         results[name] = measure(a, name, shape, label, sl, name == headline and not a.no_cpu_baseline)
         print(f"bench.py: {name}: {results[name]['ms_per_step']:.4f} ms/step", file=sys.stderr, flush=True)

@@ -325,6 +325,9 @@ typedef struct kmoe_gemm_w4_args {
   int32_t act;            /* KMOE_ACT_NONE or KMOE_ACT_SWIGLU                         */
   int32_t variant;        /* 0 = from the shape; 1, 2, 4 = 16-row fragments per pass  */
   int32_t w_layout;       /* KMOE_W_TILED                                             */
+  int32_t act_dtype;      /* KMOE_DT_BF16, or KMOE_DT_F16: a, w_scale and y are IEEE half and the
+                             weight values are half((code - 8) * scale), what
+                             dequant_int4_native (quant_ops.py:71-86) itself computes  */
 } kmoe_gemm_w4_args;
 
 /*
@@ -400,6 +403,10 @@ int kmoe_combine_dt(const uint16_t* x, int64_t ld_x, const int32_t* moe_index,
  */
 int kmoe_dequant_w4_bf16(const uint8_t* packed, const uint16_t* scale, int64_t rows, int k,
                          int group_size, uint16_t* out, kmoe_stream_t stream);
+/* The same with scale and out in act_dtype (KMOE_DT_*). KMOE_DT_F16 is the reference's own
+ * arithmetic: (code.to(float16) - 8) * scale, one rounding to half. */
+int kmoe_dequant_w4(const uint8_t* packed, const uint16_t* scale, int64_t rows, int k,
+                    int group_size, uint16_t* out, int act_dtype, kmoe_stream_t stream);
 
 /* ---------------------------------------------------------------- router GEMM */
 
@@ -479,8 +486,9 @@ typedef struct kmoe_moe_args {
   const uint16_t* w13_scale; /* [E,2I,H/group_size] bf16                               */
   const uint16_t* w2_scale;  /* [E,H,I/group_size] bf16                                */
   int32_t group_size;    /* a multiple of 32 dividing H and I (one value for both tensors) */
-  int32_t act_dtype;     /* KMOE_DT_* of x, out (and w_gate, shared-expert output): half goes with KMOE_FMT_INT8 and
-                            with KMOE_FMT_BF16 (whose weights are then half too; no biases, no SWIGLUOAI) */
+  int32_t act_dtype;     /* KMOE_DT_* of x, out (and w_gate, shared-expert output): half goes with KMOE_FMT_INT8,
+                            with KMOE_FMT_BF16 (whose weights are then half too; no biases, no SWIGLUOAI) and
+                            with KMOE_FMT_W4A16 (whose group scales are then half) */
   float shared_scale;    /* caller epilogue for half activations (models/deepseek_v2.py:286-292: the routed sum stays
                             unscaled and the shared expert's output is multiplied by 1/routed_scaling_factor):
                             out = dt( dt(routed * out_scale) + dt(shared * shared_scale) ); 0 means 1 */

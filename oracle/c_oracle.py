@@ -293,8 +293,10 @@ def _route(logits, K, scoring, renormalize, n_group, topk_group, routed_scale, b
     return sigmoid_group_topk_norm(logits, bias, K, n_group, topk_group, routed_scale)
 
 
-def dequant_w4_bf16(packed, scale_bits, group_size):
-    """packed uint8 [..., k/2], scale bf16 bits [..., k/group_size] -> bf16 bits [..., k]."""
+def dequant_w4_bf16(packed, scale_bits, group_size, f16=False):
+    """packed uint8 [..., k/2], scale bf16 bits [..., k/group_size] -> bf16 bits [..., k]; f16: scales and result
+    hold IEEE half patterns (the reference's own dtype for this step)."""
+    _dtype(f16)
     packed = _c(packed, np.uint8)
     scale_bits = _c(scale_bits, np.uint16)
     k = packed.shape[-1] * 2

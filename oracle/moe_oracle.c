@@ -429,14 +429,15 @@ ORC_API void orc_grouped_gemm_bf16(const uint16_t* a, int64_t lda, const int32_t
 }
 
 /* 4-bit weight unpacking (dequant_int4_native, quantization/kernels/quant_ops.py:71-86): low nibble first,
- * code c means c - 8, times the scale of the element's (contiguous) group, one bf16 rounding. */
+ * code c means c - 8, times the scale of the element's (contiguous) group, one bf16 rounding - or, after
+ * orc_set_act_dtype(1), one half rounding of half scales: the reference's (code.to(float16) - 8) * scale. */
 ORC_API void orc_dequant_w4_bf16(const uint8_t* packed, const uint16_t* scale, int64_t rows, int k, int group_size,
                                  uint16_t* out) {
   for (int64_t r = 0; r < rows; ++r)
     for (int j = 0; j < k; ++j) {
       const uint8_t byte = packed[r * (k / 2) + j / 2];
       const int c = (j & 1) ? (byte >> 4) : (byte & 0xf);
-      out[r * k + j] = f32_to_bf16((float)(c - 8) * bf16_to_f32(scale[r * (k / group_size) + j / group_size]));
+      out[r * k + j] = f32_to_act((float)(c - 8) * act_to_f32(scale[r * (k / group_size) + j / group_size]));
     }
 }
 

@@ -264,3 +264,129 @@ def test_unquantized_half_moe_fc_op():
     assert torch.all(y.view(rows, n)[:, n // 2:] == 0)
     with pytest.raises(Exception):  # weight of another dtype
         torch.ops._C.moe_fc(x, w.bfloat16(), lod, idx, 1, y, "SWISH_GLU")
+
+
+# ---------------------------------------------------------------- packed 4-bit weights with half scales
+W4_HALF_CASES = [
+    (1, 64, 128, [16], 128),
+    (4, 64, 256, [3, 0, 17, 1], 32),
+    (8, 256, 1024, [4, 4, 0, 9, 33, 1, 0, 2], 64),
+    (2, 128, 512, [70, 3], None),
+    (16, 1536, 256, [(5 * i) % 11 for i in range(16)], 128),
+]
+
+
+@pytest.mark.parametrize("E,n,k,counts,gs", W4_HALF_CASES)
+@pytest.mark.parametrize("variant", [0, 1, 2, 4])
+@pytest.mark.parametrize("act", [0, 1])
+def test_w4_half_dequant_and_gemm(E, n, k, counts, gs, variant, act):
+    """kmoe_dequant_w4 in half mode: the oracle's bits (= the reference's float16 expression). The packed-weight
+    GEMM in half mode against unpack + the half unquantized GEMM of the oracle: the operands are the same
+    bits, only the summation order differs."""
+    from vllm_kunlun_amd import _lib as L
+    g = torch.Generator().manual_seed(E * n + k + (gs or 0))
+    lod = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(lod[-1])
+    group = gs or k
+    packed = torch.randint(0, 256, (E, n, k // 2), generator=g, dtype=torch.uint8)
+    scale = (torch.rand(E, n, k // group, generator=g) * 0.02 + 0.002).half()
+    a = torch.randn(rows, k, generator=g).half()
+    w_bits = co.dequant_w4_bf16(packed.numpy(), hbits(scale), group, f16=True)
+    dp, ds = packed.cuda(), scale.cuda()
+    w = torch.empty(E, n, k, dtype=torch.float16, device="cuda")
+    L.check(L.lib.kmoe_dequant_w4(dp.data_ptr(), ds.data_ptr(), E * n, k, group, w.data_ptr(), L.KMOE_DT_F16, L.stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(hbits(w), w_bits)
+    ref = co.grouped_gemm_bf16(hbits(a), w_bits, lod, act=act, f16=True)
+    n_out = n // 2 if act else n
+    dt = torch.empty_like(dp)
+    L.check(L.lib.kmoe_tile_weights_i8(dp.data_ptr(), dt.data_ptr(), E, n, k // 2, L.stream()))
+    da, dl = a.cuda(), torch.from_numpy(lod).cuda()
+    y = torch.zeros(rows, n_out, dtype=torch.float16, device="cuda")
+    args = L.GemmW4Args()
+    args.a, args.lda, args.src_div = da.data_ptr(), k, 1
+    args.w, args.w_scale, args.group_size, args.lod = dt.data_ptr(), ds.data_ptr(), group, dl.data_ptr()
+    args.E, args.n, args.k, args.rows = E, n, k, rows
+    args.y, args.ldy, args.act, args.variant, args.w_layout = y.data_ptr(), n_out, act, variant, L.KMOE_W_TILED
+    args.act_dtype = L.KMOE_DT_F16
+    L.check(L.lib.kmoe_grouped_gemm_w4a16(args, L.stream()))
+    torch.cuda.synchronize()
+    assert rel_l2(y, from_hbits(ref)) <= 3e-4
+
+
+@pytest.mark.parametrize("native", ["auto", "only", False])
+@pytest.mark.parametrize("group_size,M", [(128, 24), (32, 5), (None, 24), (128, 700)])
+def test_w4_half_layer(native, group_size, M):
+    """The 4-bit method created with params_dtype float16 (the reference's deployment dtype): half scales, half
+    activations; packed weights for small batches, the copy unpacked once for large ones; against the oracle's
+    half unquantized layer on the weights its half unpacking gives."""
+    from types import SimpleNamespace
+    from vllm_kunlun_amd.ops.fused_moe.layer import FusedMoE
+    from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors_moe import (
+        KunlunCompressedTensorsWNA16MoEMethod)
+    E, H, I, K = 16, 256, 256, 4
+    wq = SimpleNamespace(num_bits=4, type="int", symmetric=True, dynamic=False,
+                         strategy="group" if group_size else "channel", group_size=group_size)
+    method = KunlunCompressedTensorsWNA16MoEMethod(wq, None, SimpleNamespace(experts_per_token=K), native=native)
+    layer = FusedMoE(num_experts=E, top_k=K, hidden_size=H, intermediate_size=I, quant_method=method, device="cuda",
+                     params_dtype=torch.float16)
+    assert layer.w13_weight_scale.dtype == torch.float16
+    g = torch.Generator().manual_seed(11)
+    with torch.no_grad():
+        for name, (n, k) in (("w13", (2 * I, H)), ("w2", (H, I))):
+            getattr(layer, f"{name}_weight_packed").data = torch.randint(0, 256, (E, n, k // 2), generator=g,
+                                                                         dtype=torch.uint8).cuda()
+            getattr(layer, f"{name}_weight_scale").data = (torch.rand(E, n, k // (group_size or k), generator=g)
+                                                           * 0.02 + 0.002).half().cuda()
+    packed13, scale13 = layer.w13_weight_packed.data.cpu(), layer.w13_weight_scale.data.cpu()
+    packed2, scale2 = layer.w2_weight_packed.data.cpu(), layer.w2_weight_scale.data.cpu()
+    method.process_weights_after_loading(layer)
+    if native != "only":
+        assert layer.w13_weight.dtype == torch.float16
+    gx = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(M, H, generator=gx, device="cuda").half()
+    logits = torch.randn(M, E, generator=gx, device="cuda")
+    out = layer(x, logits)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16
+    w13 = co.dequant_w4_bf16(packed13.numpy(), hbits(scale13), group_size or H, f16=True)
+    w2 = co.dequant_w4_bf16(packed2.numpy(), hbits(scale2), group_size or I, f16=True)
+    ref = co.forward_bf16(hbits(x), logits.cpu().numpy(), w13, w2, K, f16=True)
+    assert rel_l2(out, from_hbits(ref)) <= REL_L2_HALF
+    if native:
+        with pytest.raises(ValueError):  # activations of the other 16-bit type
+            layer(x[:4].bfloat16(), logits[:4])
+
+
+def test_w4_half_subnormal_products():
+    """Scales so small that (code - 8) * scale is a subnormal half: the unpacking kernels keep them (no flush to
+    zero), in the load-time kernel and in the registers of the packed-weight GEMM alike."""
+    from vllm_kunlun_amd import _lib as L
+    g = torch.Generator().manual_seed(2)
+    E, n, k, rows = 1, 64, 128, 16
+    packed = torch.randint(0, 256, (E, n, k // 2), generator=g, dtype=torch.uint8)
+    scale = (torch.rand(E, n, 1, generator=g) * 4e-6 + 1e-6).half()  # below the smallest normal half (6.1e-5)
+    w_bits = co.dequant_w4_bf16(packed.numpy(), hbits(scale), k, f16=True)
+    assert (np.abs(from_hbits(w_bits).float().numpy()) < 6.0e-5).all() and (w_bits & 0x7fff).any()
+    dp, ds = packed.cuda(), scale.cuda()
+    w = torch.empty(E, n, k, dtype=torch.float16, device="cuda")
+    L.check(L.lib.kmoe_dequant_w4(dp.data_ptr(), ds.data_ptr(), E * n, k, k, w.data_ptr(), L.KMOE_DT_F16, L.stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(hbits(w), w_bits)
+    a = (torch.randn(rows, k, generator=g) * 64).half()
+    lod = np.array([0, rows], np.int32)
+    ref = co.grouped_gemm_bf16(hbits(a), w_bits, lod, f16=True)
+    dt = torch.empty_like(dp)
+    L.check(L.lib.kmoe_tile_weights_i8(dp.data_ptr(), dt.data_ptr(), E, n, k // 2, L.stream()))
+    da, dl = a.cuda(), torch.from_numpy(lod).cuda()
+    y = torch.zeros(rows, n, dtype=torch.float16, device="cuda")
+    args = L.GemmW4Args()
+    args.a, args.lda, args.src_div = da.data_ptr(), k, 1
+    args.w, args.w_scale, args.group_size, args.lod = dt.data_ptr(), ds.data_ptr(), k, dl.data_ptr()
+    args.E, args.n, args.k, args.rows = E, n, k, rows
+    args.y, args.ldy, args.act, args.variant, args.w_layout = y.data_ptr(), n, 0, 0, L.KMOE_W_TILED
+    args.act_dtype = L.KMOE_DT_F16
+    L.check(L.lib.kmoe_grouped_gemm_w4a16(args, L.stream()))
+    torch.cuda.synchronize()
+    assert float(from_hbits(ref).float().abs().max()) > 0
+    assert rel_l2(y, from_hbits(ref)) <= 2e-3

@@ -513,6 +513,23 @@ def test_dequant_w4_against_the_reference_expression():
     assert from_bits(one).tolist()[0][:2] == [14.0, -14.0]   # 0xF - 8 = 7 first (low nibble), 0x1 - 8 = -7 second
 
 
+def test_dequant_w4_half_is_the_reference_statement_in_float16():
+    """The float16 mode against dequant_int4_native written out with torch's own float16 arithmetic
+    (quantization/kernels/quant_ops.py:71-86: stack the nibbles, .to(float16) - 8.0, *= the scale; contiguous
+    groups): bit for bit, scales down to subnormal products included."""
+    torch.manual_seed(6)
+    for rows, k, gs, lo in ((3, 32, 32, 0.01), (4, 64, 16, 0.01), (2, 256, 128, 0.01), (5, 64, 32, 1e-6)):
+        packed = torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8)
+        scale = (torch.rand(rows, k // gs) * lo * 10 + lo).half()
+        got = co.dequant_w4_bf16(packed.numpy(), scale.view(torch.int16).numpy().view(np.uint16), gs, f16=True)
+        w = torch.stack((packed & 0xF, (packed >> 4) & 0xF), dim=-1).reshape(rows, k).contiguous().to(torch.float16) - 8.0
+        w *= scale.repeat_interleave(gs, dim=1)
+        assert np.array_equal(got, w.view(torch.int16).numpy().view(np.uint16))
+    # the mode is per call: the next bf16 call is unaffected
+    one = co.dequant_w4_bf16(np.array([[0x1F] * 8], np.uint8), bits(torch.tensor([[2.0]]).bfloat16()), 16)
+    assert from_bits(one).tolist()[0][:2] == [14.0, -14.0]
+
+
 # ------------------------------------------- bf16 and fp8 grouped GEMMs, and the layers built on them
 def _fp8_codes(t: torch.Tensor) -> np.ndarray:
     """float tensor -> e4m3fn code bytes (torch's cast rounds to nearest even; values clamped to +-448 first,

@@ -153,9 +153,9 @@ __global__ void swigluoai_and_mul_kernel(const uint16_t* __restrict__ y, int64_t
       make_uint2(o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16));
 }
 
-// one thread: 8 packed bytes -> 16 bf16 values
+// one thread: 8 packed bytes -> 16 bf16 (or half) values
 __global__ void dequant_w4_kernel(const uint8_t* __restrict__ packed, const uint16_t* __restrict__ scale, long long rows,
-                                  int k, int group_size, uint16_t* __restrict__ out) {
+                                  int k, int group_size, uint16_t* __restrict__ out, int f16) {
   const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
   const int per_row = k / 16;
   if (i >= rows * per_row) return;
@@ -169,9 +169,10 @@ __global__ void dequant_w4_kernel(const uint8_t* __restrict__ packed, const uint
   for (int b = 0; b < 8; ++b) {
     const uint32_t byte = (word[b >> 2] >> (8 * (b & 3))) & 0xffu;
     const int j = j0 + 2 * b;  // group_size is even: both nibbles of a byte share a scale
-    const float s = bf16_to_f32(srow[j / group_size]);
-    const uint16_t lo = f32_to_bf16(static_cast<float>(static_cast<int>(byte & 0xf) - 8) * s);
-    const uint16_t hi = f32_to_bf16(static_cast<float>(static_cast<int>(byte >> 4) - 8) * s);
+    // the product of a 4-bit and an 8-bit (11-bit) significand is exact in f32: one rounding, to the 16-bit type
+    const float s = act_to_f32(srow[j / group_size], f16 != 0);
+    const uint16_t lo = f32_to_act(static_cast<float>(static_cast<int>(byte & 0xf) - 8) * s, f16 != 0);
+    const uint16_t hi = f32_to_act(static_cast<float>(static_cast<int>(byte >> 4) - 8) * s, f16 != 0);
     o[b] = lo | (static_cast<uint32_t>(hi) << 16);
   }
   uint4* dst = reinterpret_cast<uint4*>(out + r * k + j0);
@@ -276,6 +277,12 @@ extern "C" int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, i
 
 extern "C" int kmoe_dequant_w4_bf16(const uint8_t* packed, const uint16_t* scale, int64_t rows, int k, int group_size,
                                     uint16_t* out, kmoe_stream_t stream) {
+  return kmoe_dequant_w4(packed, scale, rows, k, group_size, out, KMOE_DT_BF16, stream);
+}
+
+extern "C" int kmoe_dequant_w4(const uint8_t* packed, const uint16_t* scale, int64_t rows, int k, int group_size,
+                               uint16_t* out, int act_dtype, kmoe_stream_t stream) {
+  if (int rc = check_dtype(act_dtype, "dequant_w4")) return rc;
   KMOE_REQUIRE(packed && scale && out, KMOE_ERR_NULL, "dequant_w4_bf16: NULL pointer");
   KMOE_REQUIRE(rows >= 0 && k >= 16 && k % 16 == 0 && group_size >= 2 && group_size % 2 == 0 && k % group_size == 0,
                KMOE_ERR_SHAPE, "dequant_w4_bf16: rows=%lld k=%d group_size=%d", (long long)rows, k, group_size);
@@ -284,7 +291,7 @@ extern "C" int kmoe_dequant_w4_bf16(const uint8_t* packed, const uint16_t* scale
   if (rows == 0) return KMOE_OK;
   const long long n = rows * (k / 16);
   hipLaunchKernelGGL(dequant_w4_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
-                     packed, scale, static_cast<long long>(rows), k, group_size, out);
+                     packed, scale, static_cast<long long>(rows), k, group_size, out, act_dtype == KMOE_DT_F16 ? 1 : 0);
   return check_launch("kmoe_dequant_w4_bf16");
 }
 

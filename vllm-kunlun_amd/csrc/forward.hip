@@ -60,9 +60,8 @@ int check_shape(const kmoe_moe_args* a) {
                "moe_forward: I_shared=%d must be a non-negative multiple of %d", a->I_shared, mult);
   KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "moe_forward: M*K too large");
   KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 ||
-                   (a->act_dtype == KMOE_DT_F16 && (a->format == KMOE_FMT_INT8 || a->format == KMOE_FMT_BF16)),
-               KMOE_ERR_UNSUPPORTED,
-               "moe_forward: act_dtype=%d (half activations go with the int8 and the unquantized format only)",
+                   (a->act_dtype == KMOE_DT_F16 && a->format != KMOE_FMT_FP8_BLOCK),
+               KMOE_ERR_UNSUPPORTED, "moe_forward: act_dtype=%d (half activations do not go with the fp8 format)",
                a->act_dtype);
   KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 || a->format != KMOE_FMT_BF16 ||
                    (!a->w13_bias && !a->w2_bias && a->activation != KMOE_ACT_SWIGLUOAI),
@@ -228,6 +227,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.ldy = ldy;
     g.act = act;
     g.w_layout = m.w_layout;
+    g.act_dtype = m.act_dtype;
     return kmoe_grouped_gemm_w4a16(&g, stream);
   }
   kmoe_gemm_bf16_args g = {};

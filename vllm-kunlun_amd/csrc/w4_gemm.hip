@@ -16,6 +16,11 @@
 //   value    bf16(float(c - 8) * scale), computed as fma(128 + c, scale, -136 scale): both
 //            products and their sum are exact in f32 (8-bit x 8-bit mantissas), so the one
 //            rounding is the bf16 one - the same bits as unpacking first (kmoe_dequant_w4_bf16).
+//   half     (F16 instantiations: activations, scales and results are IEEE half, the dtype
+//            dequant_int4_native itself produces) value = half(c - 8) * scale in half
+//            arithmetic: the code is OR-ed into the mantissa of 1024.0h (whose last place
+//            counts ones), 1032 is subtracted exactly and one packed multiply rounds the
+//            product - the reference's own two steps, two values per instruction.
 #include "kmoe_common.h"
 
 namespace kmoe {
@@ -24,6 +29,8 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 
 struct W4Params {
   const uint16_t* a;  // [a_rows, k] bf16
@@ -65,9 +72,29 @@ __device__ inline v4i unpack8(uint32_t word, float s, float m136s) {
   return out;
 }
 
+// The same 8 codes -> 8 half values (c - 8) * s: pair j is (code 2 j, code 2 j + 1) = byte j of lo and of hi.
+template <int J>
+__device__ inline int unpack2_half(uint32_t lo, uint32_t hi, v2h s2) {
+  // bytes, most significant first: zero, byte J of hi, zero, byte J of lo; then the exponent of 1024.0h on both
+  const uint32_t bits =
+      __builtin_amdgcn_perm(hi, lo, 0x0c000c00u | (static_cast<uint32_t>(4 + J) << 16) | static_cast<uint32_t>(J)) | 0x64006400u;
+  const v2h v = (__builtin_bit_cast(v2h, bits) - (v2h){(_Float16)1032.0f, (_Float16)1032.0f}) * s2;
+  return __builtin_bit_cast(int, v);
+}
+__device__ inline v4i unpack8_half(uint32_t word, v2h s2) {
+  const uint32_t lo = word & 0x0f0f0f0fu;
+  const uint32_t hi = (word >> 4) & 0x0f0f0f0fu;
+  v4i out;
+  out[0] = unpack2_half<0>(lo, hi, s2);
+  out[1] = unpack2_half<1>(lo, hi, s2);
+  out[2] = unpack2_half<2>(lo, hi, s2);
+  out[3] = unpack2_half<3>(lo, hi, s2);
+  return out;
+}
+
 // MF: 16-row fragments per pass over the weights; NF: 16-channel fragments per wave;
-// D: 128-value blocks of loads in flight per wave.
-template <int MF, int NF, bool SWIGLU, int D>
+// D: 128-value blocks of loads in flight per wave; F16: half activations, scales and results.
+template <int MF, int NF, bool SWIGLU, int D, bool F16>
 __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params p) {
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   constexpr int TM = 16 * MF;
@@ -142,16 +169,30 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
         if (kb < kblocks) {
 #pragma unroll
           for (int f = 0; f < NF; ++f) {
-            const float s = bf16_to_f32(sreg[d][f]);
-            const float m136s = -136.0f * s;
+            if constexpr (F16) {
+              const _Float16 sh = __builtin_bit_cast(_Float16, sreg[d][f]);
+              const v2h s2 = {sh, sh};
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              const v4i wv = unpack8(static_cast<uint32_t>(wreg[d][f][t]), s, m136s);
+              for (int t = 0; t < 4; ++t) {
+                const v4i wv = unpack8_half(static_cast<uint32_t>(wreg[d][f][t]), s2);
 #pragma unroll
-              for (int mf = 0; mf < MF; ++mf)
-                acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wv),
-                                                                     __builtin_bit_cast(v8bf, areg[d][mf][t]),
-                                                                     acc[mf][f], 0, 0, 0);
+                for (int mf = 0; mf < MF; ++mf)
+                  acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, wv),
+                                                                      __builtin_bit_cast(v8h, areg[d][mf][t]),
+                                                                      acc[mf][f], 0, 0, 0);
+              }
+            } else {
+              const float s = bf16_to_f32(sreg[d][f]);
+              const float m136s = -136.0f * s;
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                const v4i wv = unpack8(static_cast<uint32_t>(wreg[d][f][t]), s, m136s);
+#pragma unroll
+                for (int mf = 0; mf < MF; ++mf)
+                  acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wv),
+                                                                       __builtin_bit_cast(v8bf, areg[d][mf][t]),
+                                                                       acc[mf][f], 0, 0, 0);
+              }
             }
           }
           if (kb + D < kblocks) load_block(d, kb + D);
@@ -170,11 +211,11 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
         const int c0 = col[f] + lg * 4;
         uint16_t yv[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) yv[q] = f32_to_bf16(acc[mf][f][q]);
+        for (int q = 0; q < 4; ++q) yv[q] = f32_to_act(acc[mf][f][q], F16);
         if (SWIGLU) {
 #pragma unroll
           for (int q = 0; q < 4; ++q)
-            yv[q] = f32_to_bf16(silu_fixed(bf16_to_f32(yv[q])) * bf16_to_f32(f32_to_bf16(acc[mf][f + NFH][q])));
+            yv[q] = f32_to_act(silu_fixed(act_to_f32(yv[q], F16)) * act_to_f32(f32_to_act(acc[mf][f + NFH][q], F16), F16), F16);
         }
         const uint2 packed = make_uint2(yv[0] | (static_cast<uint32_t>(yv[1]) << 16),
                                         yv[2] | (static_cast<uint32_t>(yv[3]) << 16));
@@ -185,11 +226,14 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
 }
 
 template <int MF, int NF, bool SWIGLU, int D>
-int launch_w4(const W4Params& p, hipStream_t s) {
+int launch_w4(const W4Params& p, bool f16, hipStream_t s) {
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const dim3 grid(ceil_div(n_half, kWaves * NFH * 16), p.E);
-  hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D>), grid, dim3(kWaves * kWave), 0, s, p);
+  if (f16)
+    hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, true>), grid, dim3(kWaves * kWave), 0, s, p);
+  else
+    hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, false>), grid, dim3(kWaves * kWave), 0, s, p);
   return check_launch("kmoe_grouped_gemm_w4a16");
 }
 
@@ -215,6 +259,9 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
   KMOE_REQUIRE(a->ldy % 4 == 0 && a->ldy >= (swiglu ? a->n / 2 : a->n), KMOE_ERR_SHAPE, "grouped_gemm_w4a16: ldy=%lld",
                static_cast<long long>(a->ldy));
   KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_w4a16: src_div=%d", a->src_div);
+  KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 || a->act_dtype == KMOE_DT_F16, KMOE_ERR_UNSUPPORTED,
+               "grouped_gemm_w4a16: act_dtype=%d unknown", a->act_dtype);
+  const bool f16 = a->act_dtype == KMOE_DT_F16;
   if (a->rows == 0) return KMOE_OK;
   const W4Params p{a->a, a->lda, a->row_src, a->src_div, a->w, a->w_scale, a->group_size, a->lod,
                    a->E, a->n,   a->k,       a->y,       a->ldy};
@@ -227,14 +274,14 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
     mf = avg <= 10 ? 1 : (avg <= 22 ? 2 : 4);
   }
   switch (mf) {
-    case 1: return swiglu ? launch_w4<1, 2, true, 3>(p, s) : launch_w4<1, 2, false, 3>(p, s);
+    case 1: return swiglu ? launch_w4<1, 2, true, 3>(p, f16, s) : launch_w4<1, 2, false, 3>(p, f16, s);
     // tuning variants of the 16-row kernel: 1xy = x fragments per wave, y blocks in flight
-    case 122: return swiglu ? launch_w4<1, 2, true, 2>(p, s) : launch_w4<1, 2, false, 2>(p, s);
-    case 124: return swiglu ? launch_w4<1, 2, true, 4>(p, s) : launch_w4<1, 2, false, 4>(p, s);
-    case 142: return swiglu ? launch_w4<1, 4, true, 2>(p, s) : launch_w4<1, 4, false, 2>(p, s);
-    case 143: return swiglu ? launch_w4<1, 4, true, 3>(p, s) : launch_w4<1, 4, false, 3>(p, s);
-    case 2: return swiglu ? launch_w4<2, 2, true, 2>(p, s) : launch_w4<2, 2, false, 2>(p, s);
-    case 4: return swiglu ? launch_w4<4, 2, true, 2>(p, s) : launch_w4<4, 2, false, 2>(p, s);
+    case 122: return swiglu ? launch_w4<1, 2, true, 2>(p, f16, s) : launch_w4<1, 2, false, 2>(p, f16, s);
+    case 124: return swiglu ? launch_w4<1, 2, true, 4>(p, f16, s) : launch_w4<1, 2, false, 4>(p, f16, s);
+    case 142: return swiglu ? launch_w4<1, 4, true, 2>(p, f16, s) : launch_w4<1, 4, false, 2>(p, f16, s);
+    case 143: return swiglu ? launch_w4<1, 4, true, 3>(p, f16, s) : launch_w4<1, 4, false, 3>(p, f16, s);
+    case 2: return swiglu ? launch_w4<2, 2, true, 2>(p, f16, s) : launch_w4<2, 2, false, 2>(p, f16, s);
+    case 4: return swiglu ? launch_w4<4, 2, true, 2>(p, f16, s) : launch_w4<4, 2, false, 2>(p, f16, s);
     default:
       return fail(KMOE_ERR_UNSUPPORTED, "grouped_gemm_w4a16: variant=%d must be 0, 1, 2 or 4 (or a tuning variant)", a->variant);
   }

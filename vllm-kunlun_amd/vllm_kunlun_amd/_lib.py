@@ -60,7 +60,7 @@ class GemmW4Args(C.Structure):
         ("w", C.c_void_p), ("w_scale", C.c_void_p), ("group_size", C.c_int32), ("lod", C.c_void_p),
         ("E", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("rows", C.c_int32),
         ("y", C.c_void_p), ("ldy", C.c_int64), ("act", C.c_int32), ("variant", C.c_int32),
-        ("w_layout", C.c_int32),
+        ("w_layout", C.c_int32), ("act_dtype", C.c_int32),
     ]
 
 
@@ -120,6 +120,7 @@ def _load() -> C.CDLL:
         "kmoe_tile_weights_i8": (i32, [vp, vp, i32, i32, i32, vp]),
         "kmoe_swigluoai_and_mul": (i32, [vp, i64, i32, i32, f32, f32, vp, i64, vp]),
         "kmoe_dequant_w4_bf16": (i32, [vp, vp, i64, i32, i32, vp, vp]),
+        "kmoe_dequant_w4": (i32, [vp, vp, i64, i32, i32, vp, i32, vp]),
         "kmoe_router_gemm_workspace_bytes": (sz, [i32, i32, i32]),
         "kmoe_router_gemm_bf16": (i32, [vp, i64, vp, i32, i32, i32, vp, i64, vp, sz, vp]),
         "kmoe_quant_fp8_group128": (i32, [vp, i64, i32, i32, vp, i64, vp, vp]),
@@ -151,7 +152,7 @@ EXPORTS = (
     "kmoe_align_workspace_bytes", "kmoe_align", "kmoe_gather_rows", "kmoe_quant_i8_rows", "kmoe_quant_i8_rows_chunked", "kmoe_tile_weights_i8", "kmoe_quant_fp8_group128",
     "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_w4a16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
     "kmoe_moe_workspace_layout", "kmoe_moe_forward", "kmoe_router_gemm_workspace_bytes", "kmoe_router_gemm_bf16",
-    "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16", "kmoe_moe_forward_static",
+    "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16", "kmoe_dequant_w4", "kmoe_moe_forward_static",
     "kmoe_quant_i8_rows_dt", "kmoe_quant_i8_rows_chunked_dt", "kmoe_silu_and_mul_dt", "kmoe_combine_dt", "kmoe_router_gemm",
 )
 STATIC_WORKSPACE_BYTES = 64 << 20

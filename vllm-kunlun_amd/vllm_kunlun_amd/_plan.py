@@ -168,7 +168,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     layer then computes the router logits itself. bf16 only: w13_bias [E,2I] / w2_bias [E,H] (bf16)
     and activation "swigluoai" (gate and up rows of w13 interleaved) select the expert-bias branch.
     KMOE_FMT_W4A16: w13 [E,2I,H/2] and w2 [E,H,I/2] uint8 (two 4-bit codes per byte), tiled;
-    w13_aux/w2_aux their bf16 group scales [E,2I,H/group_size], [E,H,I/group_size].
+    w13_aux/w2_aux their group scales [E,2I,H/group_size], [E,H,I/group_size] in x's dtype.
     shared_scale multiplies the shared expert's output before it is added (the float16 form of the caller's
     epilogue, models/deepseek_v2.py:286-292). tile_variant: a tuning variant of the int8 tile kernel for the routed GEMMs (kmoe_moe_args.tile_variant)."""
     if scoring_func not in ("softmax", "sigmoid"):
@@ -179,9 +179,8 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     L.require_device(*tensors)
     L.require_contig(*tensors)
     dt = L.act_dtype(x, "moe plan")
-    if dt == L.KMOE_DT_F16 and fmt not in (L.KMOE_FMT_INT8, L.KMOE_FMT_BF16):
-        raise NotImplementedError("moe plan: float16 activations go with int8 and unquantized weights only "
-                                  "(bfloat16 otherwise)")
+    if dt == L.KMOE_DT_F16 and fmt == L.KMOE_FMT_FP8_BLOCK:
+        raise NotImplementedError("moe plan: float16 activations do not go with fp8 weights (bfloat16 there)")
     if fmt == L.KMOE_FMT_BF16 and w13.dtype != x.dtype:
         raise ValueError(f"moe plan: unquantized weights ({w13.dtype}) must have the activations' dtype ({x.dtype})")
     if fmt == L.KMOE_FMT_BF16 and dt == L.KMOE_DT_F16 and (w13_bias is not None or w2_bias is not None
@@ -204,8 +203,8 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
         raise ValueError("moe plan: w2 must be [E,H,I] for w13 [E,2I,H]")
     if w4:
         gs = int(group_size or 0)
-        if w13_aux is None or w2_aux is None or w13_aux.dtype != torch.bfloat16 or w2_aux.dtype != torch.bfloat16:
-            raise ValueError("moe plan: 4-bit weights need bfloat16 group scales")
+        if w13_aux is None or w2_aux is None or w13_aux.dtype != x.dtype or w2_aux.dtype != x.dtype:
+            raise ValueError("moe plan: 4-bit weights need group scales in the activations' dtype")
         if gs < 32 or gs % 32 or H % gs or (two_i // 2) % gs:
             raise ValueError(f"moe plan: group_size={group_size} must be a multiple of 32 dividing H and I")
         if tuple(w13_aux.shape) != (E, two_i, H // gs) or tuple(w2_aux.shape) != (E, H, two_i // 2 // gs):

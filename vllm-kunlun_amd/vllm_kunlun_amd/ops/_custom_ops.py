@@ -259,18 +259,18 @@ def _moe_fc_fp8(x, weight, lod, y, act, x_scale, w_scale, scale_n, scale_k) -> N
 
 
 def _moe_fc_w4(x, weight, lod, y, act, w_scale, group_size) -> None:
-    """moe_fc with use_pack_int4: bfloat16 activations against packed 4-bit weights [E, n, k/2] (two codes per
-    byte, low nibble first, code - 8; re-tiled at load time) with bfloat16 group scales [E, n, k/group];
-    scale_k carries the group size (0: one scale per output channel)."""
+    """moe_fc with use_pack_int4: bfloat16 (or float16) activations against packed 4-bit weights [E, n, k/2] (two
+    codes per byte, low nibble first, code - 8; re-tiled at load time) with group scales [E, n, k/group] in the
+    activations' dtype; scale_k carries the group size (0: one scale per output channel)."""
     from .._plan import weight_layout
-    _need(x.dtype == _BF16 and y.dtype == _BF16 and weight.dtype == torch.uint8,
-          "moe_fc: packed 4-bit weights are uint8 and go with bfloat16 activations")
+    _need(x.dtype in (_BF16, torch.float16) and y.dtype == x.dtype and weight.dtype == torch.uint8,
+          "moe_fc: packed 4-bit weights are uint8 and go with bfloat16 or float16 activations")
     E, n, half_k = weight.shape
     k = 2 * half_k
     rows = x.numel() // k
     gs = group_size or k
-    _need(w_scale is not None and w_scale.dtype == _BF16 and w_scale.numel() == E * n * (k // gs),
-          "moe_fc: packed 4-bit weights need bfloat16 scales [E, n, k/group]")
+    _need(w_scale is not None and w_scale.dtype == x.dtype and w_scale.numel() == E * n * (k // gs),
+          "moe_fc: packed 4-bit weights need scales [E, n, k/group] in the activations' dtype")
     if weight_layout(weight) != L.KMOE_W_TILED:
         raise NotImplementedError("moe_fc: packed 4-bit weights must be re-tiled (tile_int8_weights_) first")
     n_out = n // 2 if act else n
@@ -281,6 +281,7 @@ def _moe_fc_w4(x, weight, lod, y, act, w_scale, group_size) -> None:
     g.y, g.ldy = y.data_ptr(), y.numel() // max(rows, 1) if rows else n_out
     g.act = L.KMOE_ACT_SWIGLU if act else L.KMOE_ACT_NONE
     g.w_layout = L.KMOE_W_TILED
+    g.act_dtype = L.act_dtype(x)
     L.check(L.lib.kmoe_grouped_gemm_w4a16(g, L.stream()))
 
 

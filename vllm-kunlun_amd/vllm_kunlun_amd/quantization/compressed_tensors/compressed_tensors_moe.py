@@ -318,9 +318,12 @@ class KunlunCompressedTensorsWNA16MoEMethod:
         them once per call and unpacks in registers: the path for decode-sized batches
         (`native` = "auto" or "only"; needs hidden and intermediate sizes that are multiples of
         128 and a group size that is a multiple of 32);
-      * the weights are unpacked ONCE (kmoe_dequant_w4_bf16) to tiled bf16 tensors for batches with
+      * the weights are unpacked ONCE (kmoe_dequant_w4) to tiled 16-bit tensors for batches with
         many rows per expert (`native` = "auto" or False). "auto" keeps both copies (1.25x the
-        bf16 bytes); "only" keeps the packed one and serves every batch from it.
+        16-bit bytes); "only" keeps the packed one and serves every batch from it.
+    The 16-bit type is the one of the scales: float16 scales (a model loaded with --dtype float16, the
+    reference's recipes) give half((code - 8) * scale), exactly what dequant_int4_native computes, and the
+    layer then takes float16 activations; any other scale dtype is taken as bfloat16.
     Packed layout as in dequant_int4_native (quantization/kernels/quant_ops.py:71-86): uint8,
     two codes per byte, low nibble first, code - 8; scales per contiguous group of `group_size`
     along k, or one per row."""
@@ -355,8 +358,9 @@ class KunlunCompressedTensorsWNA16MoEMethod:
         mk = lambda *s, dt: torch.nn.Parameter(torch.zeros(*s, dtype=dt, device=device), requires_grad=False)  # noqa
         layer.w13_weight_packed = mk(E, 2 * I, H // 2, dt=torch.uint8)
         layer.w2_weight_packed = mk(E, H, I // 2, dt=torch.uint8)
-        layer.w13_weight_scale = mk(E, 2 * I, g13, dt=torch.bfloat16)
-        layer.w2_weight_scale = mk(E, H, g2, dt=torch.bfloat16)
+        sdt = torch.float16 if params_dtype == torch.float16 else torch.bfloat16
+        layer.w13_weight_scale = mk(E, 2 * I, g13, dt=sdt)
+        layer.w2_weight_scale = mk(E, H, g2, dt=sdt)
 
     def _native_possible(self, layer) -> bool:
         E, n13, half_h = layer.w13_weight_packed.shape
@@ -374,7 +378,9 @@ class KunlunCompressedTensorsWNA16MoEMethod:
             keep_bf16 = self.native != "only"
             for name in ("w13", "w2"):
                 packed = getattr(layer, f"{name}_weight_packed").data.contiguous()
-                scale = getattr(layer, f"{name}_weight_scale").data.to(torch.bfloat16).contiguous()
+                scale = getattr(layer, f"{name}_weight_scale").data
+                dt16 = torch.float16 if layer.w13_weight_scale.dtype == torch.float16 else torch.bfloat16
+                scale = scale.to(dt16).contiguous()
                 E, n, half_k = packed.shape
                 k = 2 * half_k
                 gs = self.group_size or k
@@ -382,8 +388,9 @@ class KunlunCompressedTensorsWNA16MoEMethod:
                     raise ValueError(f"{name}: scales {tuple(scale.shape)} do not fit k={k}, group_size={gs}")
                 L.require_device(packed, scale)
                 if keep_bf16:
-                    w = torch.empty((E, n, k), dtype=torch.bfloat16, device=packed.device)
-                    L.check(L.lib.kmoe_dequant_w4_bf16(L.ptr(packed), L.ptr(scale), E * n, k, gs, L.ptr(w), L.stream()))
+                    w = torch.empty((E, n, k), dtype=dt16, device=packed.device)
+                    L.check(L.lib.kmoe_dequant_w4(L.ptr(packed), L.ptr(scale), E * n, k, gs, L.ptr(w),
+                                                  L.act_dtype(w), L.stream()))
                     setattr(layer, f"{name}_weight", torch.nn.Parameter(w, requires_grad=False))
                 if native:
                     getattr(layer, f"{name}_weight_packed").data = packed
@@ -404,7 +411,7 @@ class KunlunCompressedTensorsWNA16MoEMethod:
                     e_score_correction_bias=getattr(layer, "e_score_correction_bias", None))
 
     def apply_monolithic(self, layer, x: torch.Tensor, router_logits: torch.Tensor, **kwargs):
-        """bf16 activations. Few rows per expert: the packed weights (kmoe_grouped_gemm_w4a16
+        """Activations in the dtype of the scales (bf16, or float16). Few rows per expert: the packed weights (kmoe_grouped_gemm_w4a16
         inside kmoe_moe_forward). Otherwise the unpacked weights through KunlunOps.fused_moe, as
         the reference's apply() ends (:343-360). Routing as in KunlunOps.fused_moe (always
         normalised, sigmoid scale 1.0)."""
@@ -415,8 +422,9 @@ class KunlunCompressedTensorsWNA16MoEMethod:
         use_native = getattr(layer, "w4_native", False) and not has_bias and (
             self.native == "only" or rows_per_expert <= self.NATIVE_MAX_ROWS_PER_EXPERT)
         if use_native:
-            if x.dtype != torch.bfloat16:
-                raise NotImplementedError(f"4-bit MoE: activations must be bfloat16, got {x.dtype}")
+            if x.dtype != layer.w13_weight_scale.dtype:
+                raise ValueError(f"4-bit MoE: activations ({x.dtype}) must have the dtype of the scales "
+                                 f"({layer.w13_weight_scale.dtype})")
             xc = x.contiguous()
             out = torch.empty_like(xc)
             rk = self._routing_kwargs(layer)

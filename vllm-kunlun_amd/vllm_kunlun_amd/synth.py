@@ -67,10 +67,18 @@ for _n in ("qwen3-decode", "qwen3-prefill"):
 SHAPES["qwen3-w4a16-decode"] = replace(SHAPES["qwen3-decode"], name="qwen3-w4a16-decode", quant="w4")
 
 
-def make_layer(shape: MoEShape, device="cuda", seed: int = 0) -> "SynthLayer":
-    """The synthetic layer of a shape in the format the shape names."""
-    return {"int8": make_w8a8_layer, "fp8": make_fp8_layer, "none": make_bf16_layer,
-            "w4": make_w4_layer}[shape.quant](shape, device, seed)
+def make_layer(shape: MoEShape, device="cuda", seed: int = 0, dtype: torch.dtype = torch.bfloat16) -> "SynthLayer":
+    """The synthetic layer of a shape in the format the shape names. dtype: bfloat16, or float16 (int8: the
+    activations; unquantized: activations and weights; 4-bit: activations and group scales; not fp8)."""
+    if dtype == torch.bfloat16:
+        return {"int8": make_w8a8_layer, "fp8": make_fp8_layer, "none": make_bf16_layer,
+                "w4": make_w4_layer}[shape.quant](shape, device, seed)
+    if dtype != torch.float16 or shape.quant == "fp8":
+        raise NotImplementedError(f"synthetic {shape.quant} layer with {dtype} activations")
+    if shape.quant == "int8":
+        sl = make_w8a8_layer(shape, device, seed)
+        return SynthLayer(sl.shape, sl.layer, sl.x.half(), sl.logits, sl.bias, sl.shared)
+    return {"none": make_bf16_layer, "w4": make_w4_layer}[shape.quant](shape, device, seed, dtype)
 
 
 def scaled(shape: MoEShape, **kw) -> MoEShape:
@@ -134,7 +142,7 @@ def rebatch(sl: SynthLayer, shape: MoEShape, seed: int = 0) -> SynthLayer:
     g = torch.Generator(device=dev)
     g.manual_seed(seed * 1000003 + shape.M)
     x, logits = _activations(shape, g, dev)
-    return SynthLayer(shape, sl.layer, x, logits, sl.bias, sl.shared)
+    return SynthLayer(shape, sl.layer, x.to(sl.x.dtype), logits, sl.bias, sl.shared)
 
 
 def _quant_block_fp8(w: torch.Tensor):
@@ -194,8 +202,8 @@ def make_fp8_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
     return SynthLayer(s, layer, x, logits, bias, shared)
 
 
-def make_bf16_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
-    """FusedMoE with the unquantized method and bf16 weights ~ N(0, 0.02)."""
+def make_bf16_layer(shape: MoEShape, device="cuda", seed: int = 0, dtype: torch.dtype = torch.bfloat16) -> SynthLayer:
+    """FusedMoE with the unquantized method and bf16 (or float16) weights ~ N(0, 0.02)."""
     dev = torch.device(device)
     g = torch.Generator(device=dev)
     g.manual_seed(seed)
@@ -203,16 +211,16 @@ def make_bf16_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer
     bias = _routing_inputs(s, g, dev)
     layer = FusedMoE(num_experts=s.E, top_k=s.K, hidden_size=s.H, intermediate_size=s.I, renormalize=True,
                      use_grouped_topk=s.n_group > 1, num_expert_group=s.n_group, topk_group=s.topk_group,
-                     scoring_func=s.scoring, e_score_correction_bias=bias, device=dev)
+                     scoring_func=s.scoring, e_score_correction_bias=bias, device=dev, params_dtype=dtype)
     for e in range(s.E):
         layer.w13_weight.data[e].copy_(torch.randn(2 * s.I, s.H, generator=g, device=dev) * 0.02)
         layer.w2_weight.data[e].copy_(torch.randn(s.H, s.I, generator=g, device=dev) * 0.02)
     layer.quant_method.process_weights_after_loading(layer)
     x, logits = _activations(s, g, dev)
-    return SynthLayer(s, layer, x, logits, bias, None)
+    return SynthLayer(s, layer, x.to(dtype), logits, bias, None)
 
 
-def make_w4_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
+def make_w4_layer(shape: MoEShape, device="cuda", seed: int = 0, dtype: torch.dtype = torch.bfloat16) -> SynthLayer:
     """FusedMoE with the 4-bit method (packed weights kept, native="only"): weights ~ N(0, 0.02)
     quantised per group of `group_size` values to codes 0..15 (value = (code - 8) * scale)."""
     from types import SimpleNamespace
@@ -227,12 +235,13 @@ def make_w4_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
     method = KunlunCompressedTensorsWNA16MoEMethod(wq, None, SimpleNamespace(experts_per_token=s.K), native="only")
     layer = FusedMoE(num_experts=s.E, top_k=s.K, hidden_size=s.H, intermediate_size=s.I, renormalize=True,
                      use_grouped_topk=s.n_group > 1, num_expert_group=s.n_group, topk_group=s.topk_group,
-                     scoring_func=s.scoring, e_score_correction_bias=bias, quant_method=method, device=dev)
+                     scoring_func=s.scoring, e_score_correction_bias=bias, quant_method=method, device=dev,
+                     params_dtype=dtype)
 
-    def quantise(w):  # [n, k] float -> packed uint8 [n, k/2], bf16 scales [n, k/gs]
+    def quantise(w):  # [n, k] float -> packed uint8 [n, k/2], 16-bit scales [n, k/gs]
         n, k = w.shape
         grp = w.view(n, k // s.group_size, s.group_size)
-        scale = (grp.abs().amax(-1) / 7.0).clamp_min(1e-8).bfloat16()
+        scale = (grp.abs().amax(-1) / 7.0).clamp_min(1e-6).to(dtype)
         codes = (torch.round(grp / scale.float().unsqueeze(-1)).clamp(-8, 7) + 8).to(torch.uint8).view(n, k)
         return codes[:, 0::2] | (codes[:, 1::2] << 4), scale
 
@@ -245,7 +254,7 @@ def make_w4_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:
         layer.w2_weight_scale.data[e].copy_(s2)
     method.process_weights_after_loading(layer)
     x, logits = _activations(s, g, dev)
-    return SynthLayer(s, layer, x, logits, bias, None)
+    return SynthLayer(s, layer, x.to(dtype), logits, bias, None)
 
 
 def make_w8a8_layer(shape: MoEShape, device="cuda", seed: int = 0) -> SynthLayer:

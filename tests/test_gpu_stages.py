@@ -417,8 +417,11 @@ TILED_CASES = [
     (16, 192, 384, [0] * 15 + [300]),
 ]
 
+# k % 4096 == 0: the waves of the streaming kernel walk K from rotated start steps (same sums)
+ROTATED_K_CASES = [(3, 64, 4096, [5, 0, 18]), (2, 96, 8192, [3, 40])]
 
-@pytest.mark.parametrize("E,n,k,counts", TILED_CASES)
+
+@pytest.mark.parametrize("E,n,k,counts", TILED_CASES + ROTATED_K_CASES)
 @pytest.mark.parametrize("variant", [1, 2, 4, 8])
 @pytest.mark.parametrize("act", [0, 1])
 @pytest.mark.parametrize("gather", [False, True])

@@ -39,6 +39,7 @@ struct StreamParams {
   const float* w_max_tail;
   int32_t tail_row0, tail_rows, tail_src0;
   int32_t f16;  // outputs (and the rounding of gate and up before SiLU-mul) in IEEE half instead of bf16
+  int32_t rotate;  // every wave starts its K range at a step of its own (see stream_gemm_i8)
 };
 
 constexpr int kWaves = 4;
@@ -81,6 +82,16 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
   if (KS == 1 && col_base >= n_half) return;  // whole wave has nothing to do (no barriers when KS == 1)
   const int kb_begin = (ksteps * wk) / KS;
   const int kb_end = (ksteps * (wk + 1)) / KS;
+  // With p.rotate a wave walks its K range from a start step of its own, wrapping round: int32 sums do not depend
+  // on the order, and waves that were dispatched together no longer read addresses that differ by a
+  // multiple of the fragment stride.
+  const int klen = kb_end - kb_begin;
+  const unsigned wave_key = (static_cast<unsigned>(blockIdx.y) * gridDim.x + blockIdx.x) * kWaves + wave_id;
+  const int rot = p.rotate && klen > 1 ? static_cast<int>(((wave_key * 2654435761u) >> 12) % static_cast<unsigned>(klen)) : 0;
+  auto kb_of = [&](int i) {
+    const int s = i + rot;
+    return kb_begin + (s >= klen ? s - klen : s);
+  };
 
   const int8_t* wp[NF];
   bool wok[NF];
@@ -126,19 +137,19 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
 
 #pragma unroll
     for (int d = 0; d < D; ++d)
-      if (kb_begin + d < kb_end) load_step(d, kb_begin + d);
+      if (d < klen) load_step(d, kb_of(d));
 
-    for (int kb0 = kb_begin; kb0 < kb_end; kb0 += D) {
+    for (int i0 = 0; i0 < klen; i0 += D) {
 #pragma unroll
       for (int d = 0; d < D; ++d) {
-        const int kb = kb0 + d;
-        if (kb < kb_end) {
+        const int kb = i0 + d;
+        if (kb < klen) {
 #pragma unroll
           for (int mf = 0; mf < MF; ++mf)
 #pragma unroll
             for (int f = 0; f < NF; ++f)
               acc[mf][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wreg[d][f], areg[d][mf], acc[mf][f], 0, 0, 0);
-          if (kb + D < kb_end) load_step(d, kb + D);
+          if (kb + D < klen) load_step(d, kb_of(kb + D));
         }
       }
     }
@@ -226,7 +237,12 @@ __global__ void tile_weights_kernel(const int8_t* __restrict__ src, int8_t* __re
 int stream_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   StreamParams p{a->a, a->a_rows, a->a_max, a->row_src, a->src_div, a->w, a->w_max,
                  a->lod, a->E,     a->n,     a->k,       a->y,       a->ldy, a->acc_out,
-                 a->w_tail, a->w_max_tail, a->tail_row0, a->tail_rows, a->tail_src0, a->act_dtype == KMOE_DT_F16};
+                 a->w_tail, a->w_max_tail, a->tail_row0, a->tail_rows, a->tail_src0, a->act_dtype == KMOE_DT_F16,
+                 // A fragment's blocks are k / 64 KB apart. When that stride is a multiple of 64 KB (k = 4096, 8192:
+                 // Mixtral, Qwen3-235B), waves in step hit the same memory channels: measured 5.5 TB/s at k = 8192
+                 // and 6.0 at 4096 against 6.5 at 2048; with the rotated start 6.0 and 6.6. Other strides gain
+                 // nothing from it (k = 7168: 6.2 either way).
+                 a->k % 4096 == 0};
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
   // m-fragments per pass from the rows an expert gets under uniform routing
   int mf = a->variant;

@@ -469,6 +469,8 @@ W4_CASES = [
     (8, 256, 1024, [4, 4, 0, 9, 33, 1, 0, 2], 64),
     (2, 128, 512, [70, 3], None),
     (16, 1536, 256, [(5 * i) % 11 for i in range(16)], 128),
+    (3, 96, 384, [5, 40, 7], 96),      # a group of 3 x 32 values: the group index is a division, not a shift
+    (2, 64, 4224, [5, 20], 32),        # 132 groups per channel: too many for the LDS copy, scales read from memory
 ]
 
 

@@ -40,6 +40,7 @@ struct W4Params {
   const uint8_t* w;       // tiled packed codes
   const uint16_t* scale;  // [E, n, k / gs] bf16
   int32_t gs;
+  int32_t gs_shift;       // log2(gs / 32) when gs / 32 is a power of two, else -1
   const int32_t* lod;
   int32_t E, n, k;
   uint16_t* y;
@@ -94,8 +95,13 @@ __device__ inline v4i unpack8_half(uint32_t word, v2h s2) {
 
 // MF: 16-row fragments per pass over the weights; NF: 16-channel fragments per wave;
 // D: 128-value blocks of loads in flight per wave; F16: half activations, scales and results.
-template <int MF, int NF, bool SWIGLU, int D, bool F16>
+// SLDS: every wave first copies the scales of its fragments (16 channels x k / group values each, one
+// contiguous piece of the scale tensor) into its own part of LDS and reads a block's scale from there.
+// Read from global memory per block, a lane's 2-byte scale load touches 16 cache lines per instruction
+// (16 channels, rows apart), as many as the weight load next to it moves bytes for: 20 % of the launch.
+template <int MF, int NF, bool SWIGLU, int D, bool F16, bool SLDS>
 __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params p) {
+  extern __shared__ uint16_t scale_lds[];  // SLDS: [kWaves][NF][16][groups]
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   constexpr int TM = 16 * MF;
   const int lane = lane_id();
@@ -113,8 +119,11 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
   const uint8_t* w_base = p.w + static_cast<size_t>(e) * p.n * (p.k / 2);
   const uint16_t* s_base = p.scale + static_cast<size_t>(e) * p.n * groups;
 
+  // group of this lane's 32 values of block kb: (128 kb + 32 lg) / gs
+  auto group_of = [&](int kb) { return p.gs_shift >= 0 ? (4 * kb + lg) >> p.gs_shift : (4 * kb + lg) / (p.gs / 32); };
   const uint8_t* wp[NF];
   const uint16_t* sp[NF];
+  int soff[NF];  // SLDS: this lane's channel row in the wave's LDS copy
   bool wok[NF];
   int col[NF];
 #pragma unroll
@@ -126,7 +135,15 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
     const int ch0 = wok[f] ? col[f] : 0;  // fragments past the last channel read fragment 0: never stored
     wp[f] = w_base + static_cast<size_t>(ch0 / 16) * kblocks * 1024 + lane * 16;
     sp[f] = s_base + static_cast<size_t>(ch0 + li) * groups;
+    if constexpr (SLDS) {
+      // the wave's own copy; it alone reads it, so no barrier: a wave's LDS accesses complete in order
+      uint32_t* dst = reinterpret_cast<uint32_t*>(scale_lds + (wave * NF + f) * 16 * groups);
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(s_base + static_cast<size_t>(ch0) * groups);
+      for (int i = lane; i < 8 * groups; i += kWave) dst[i] = src[i];
+      soff[f] = (wave * NF + f) * 16 * groups + li * groups;
+    }
   }
+  if constexpr (SLDS) __builtin_amdgcn_wave_barrier();  // the copies above stay above the reads below
 
   for (int row0 = row_begin; row0 < row_end; row0 += TM) {
     const uint16_t* ap[MF];
@@ -147,11 +164,11 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
     uint16_t sreg[D][NF];
     v4i areg[D][MF][4];
     auto load_block = [&](int slot, int kb) {
-      const int g = (128 * kb + 32 * lg) / p.gs;
+      const int g = group_of(kb);
 #pragma unroll
       for (int f = 0; f < NF; ++f) {
         wreg[slot][f] = *reinterpret_cast<const v4i*>(wp[f] + static_cast<size_t>(kb) * 1024);
-        sreg[slot][f] = sp[f][g];
+        if constexpr (!SLDS) sreg[slot][f] = sp[f][g];
       }
 #pragma unroll
       for (int mf = 0; mf < MF; ++mf)
@@ -169,6 +186,7 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
         if (kb < kblocks) {
 #pragma unroll
           for (int f = 0; f < NF; ++f) {
+            if constexpr (SLDS) sreg[d][f] = scale_lds[soff[f] + group_of(kb)];
             if constexpr (F16) {
               const _Float16 sh = __builtin_bit_cast(_Float16, sreg[d][f]);
               const v2h s2 = {sh, sh};
@@ -230,10 +248,17 @@ int launch_w4(const W4Params& p, bool f16, hipStream_t s) {
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const dim3 grid(ceil_div(n_half, kWaves * NFH * 16), p.E);
-  if (f16)
-    hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, true>), grid, dim3(kWaves * kWave), 0, s, p);
-  else
-    hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, false>), grid, dim3(kWaves * kWave), 0, s, p);
+  const size_t lds = static_cast<size_t>(kWaves) * NF * 16 * (p.k / p.gs) * sizeof(uint16_t);
+  if (lds <= 32 * 1024) {  // beyond: many small groups on a long K; the scales stay in global memory
+    if (f16)
+      hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, true, true>), grid, dim3(kWaves * kWave), lds, s, p);
+    else
+      hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, false, true>), grid, dim3(kWaves * kWave), lds, s, p);
+  } else if (f16) {
+    hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, true, false>), grid, dim3(kWaves * kWave), 0, s, p);
+  } else {
+    hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, false, false>), grid, dim3(kWaves * kWave), 0, s, p);
+  }
   return check_launch("kmoe_grouped_gemm_w4a16");
 }
 
@@ -259,11 +284,16 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
   KMOE_REQUIRE(a->ldy % 4 == 0 && a->ldy >= (swiglu ? a->n / 2 : a->n), KMOE_ERR_SHAPE, "grouped_gemm_w4a16: ldy=%lld",
                static_cast<long long>(a->ldy));
   KMOE_REQUIRE(!a->row_src || a->src_div >= 1, KMOE_ERR_SHAPE, "grouped_gemm_w4a16: src_div=%d", a->src_div);
+  KMOE_REQUIRE(reinterpret_cast<uintptr_t>(a->w_scale) % 4 == 0, KMOE_ERR_SHAPE, "grouped_gemm_w4a16: misaligned scales");
   KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 || a->act_dtype == KMOE_DT_F16, KMOE_ERR_UNSUPPORTED,
                "grouped_gemm_w4a16: act_dtype=%d unknown", a->act_dtype);
   const bool f16 = a->act_dtype == KMOE_DT_F16;
   if (a->rows == 0) return KMOE_OK;
-  const W4Params p{a->a, a->lda, a->row_src, a->src_div, a->w, a->w_scale, a->group_size, a->lod,
+  const int q = a->group_size / 32;
+  int shift = -1;
+  if ((q & (q - 1)) == 0)
+    for (shift = 0; (1 << shift) < q; ++shift) {}
+  const W4Params p{a->a, a->lda, a->row_src, a->src_div, a->w, a->w_scale, a->group_size, shift, a->lod,
                    a->E, a->n,   a->k,       a->y,       a->ldy};
   hipStream_t s = as_stream(stream);
   int mf = a->variant;

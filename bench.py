@@ -180,7 +180,7 @@ def vendor_dense_gemm(shape, g1_ops, peak_tops, reps=20):
             "frac_of_peak": ops / ms / 1e9 / peak_tops}
 
 
-# What plain `python bench.py` runs besides the headline workload: the other BASELINE
+# What plain `python bench.py` runs besides the headline workload: the other benchmark
 # configurations, reported under "workloads" in the same JSON line.
 SUITE = ["dsv3-prefill", "qwen3-decode", "qwen3-prefill", "qwen3-prefill-skew", "dsv3-fp8-decode", "dsv3-fp8-prefill"]
 HEADLINE = "dsv3-decode"

@@ -46,6 +46,39 @@ def test_apply_monolithic_under_graph_capture():
     _replays(graph, (x, logits), fresh, out, eager)
 
 
+@pytest.mark.parametrize("quant", ["int8", "fp8"])
+def test_shared_expert_on_the_side_stream_under_graph_capture(quant):
+    """A shared expert of another width (int8) and the fp8 decode layer run their shared MLP on the library's second
+    stream, forked from and joined into the caller's: eager and captured (the fork and join become graph edges),
+    same bits every time (int8: the oracle's)."""
+    from vllm_kunlun_amd import synth
+    base = "dsv3-decode" if quant == "int8" else "dsv3-fp8-decode"
+    shape = synth.scaled(synth.SHAPES[base], M=40, H=512, E=32, K=4, I=128, n_group=4, topk_group=2,
+                         I_shared=384 if quant == "int8" else 128)
+    sl = synth.make_layer(shape, "cuda", seed=7)
+    method, kw = sl.layer.quant_method, sl.apply_kwargs()
+    x, logits = sl.x.clone(), sl.logits.clone()
+    eager = lambda xx, ll: method.apply_monolithic(sl.layer, xx, ll, **kw)  # noqa: E731
+    first = eager(x, logits)                           # creates the second stream (never inside a capture)
+    torch.cuda.synchronize()
+    if quant == "int8":  # the overlapped pass gives the oracle's bits
+        import numpy as np
+        from oracle import c_oracle as co
+        b16 = lambda t: t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)  # noqa: E731
+        w13, w13_max, w2, w2_max, shared = sl.host_weights()
+        ref = co.forward_w8a8(b16(x), logits.cpu().numpy(), w13.numpy(), w13_max.numpy(), w2.numpy(), w2_max.numpy(),
+                              shape.K, shape.scoring, True, shape.n_group, shape.topk_group, shape.routed_scale,
+                              sl.bias.cpu().numpy(), tuple(t.numpy() for t in shared))
+        assert np.array_equal(b16(first), ref)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = method.apply_monolithic(sl.layer, x, logits, **kw)
+    g = torch.Generator(device="cuda").manual_seed(12)
+    fresh = [(torch.randn(shape.M, shape.H, generator=g, device="cuda").bfloat16(),
+              torch.randn(shape.M, shape.E, generator=g, device="cuda")) for _ in range(4)]
+    _replays(graph, (x, logits), fresh, out, eager)
+
+
 def test_static_workspace_forward_under_graph_capture():
     from vllm_kunlun_amd import _lib as L
     from vllm_kunlun_amd import synth

@@ -323,8 +323,67 @@ extern "C" int kmoe_moe_workspace_layout(const kmoe_moe_args* a, kmoe_moe_layout
   return KMOE_OK;
 }
 
+namespace {
+
+// A shared expert that cannot ride in the routed launches (another width; the fp8 decode kernels) is a chain of
+// small launches that depends on the layer's input only. It runs on a stream of the library's own, forked from
+// the caller's stream after the first quantisation and joined back before the combine, so that it hides under
+// the routed GEMMs instead of adding its launches' latencies to the layer (DeepSeek-V3 fp8 decode: 85 us of
+// 1.86 ms). One stream and two events per GPU, created on the first call that wants them and is not being
+// captured (default priority, non-blocking); work of consecutive calls is ordered on it like on any stream.
+struct SideStream {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+  bool failed = false;
+};
+constexpr int kSideDevices = 64;
+SideStream g_side[kSideDevices];
+std::mutex g_side_mutex;
+
+// The side stream of the current device, or NULL: switched off by KMOE_SERIAL_SHARED=1, not created yet while the
+// caller's stream is being captured (a capture must not be the first to ask), or the runtime refused.
+SideStream* side_stream(hipStream_t main) {
+  static const bool off = [] {
+    const char* v = getenv("KMOE_SERIAL_SHARED");
+    return v && v[0] && v[0] != '0';
+  }();
+  if (off) return nullptr;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSideDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_side_mutex);
+  SideStream& sd = g_side[dev];
+  if (sd.stream) return &sd;
+  if (sd.failed) return nullptr;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(main, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  if (hipStreamCreateWithFlags(&sd.stream, hipStreamNonBlocking) != hipSuccess ||
+      hipEventCreateWithFlags(&sd.fork, hipEventDisableTiming) != hipSuccess ||
+      hipEventCreateWithFlags(&sd.join, hipEventDisableTiming) != hipSuccess) {
+    (void)hipGetLastError();
+    sd.failed = true;
+    sd.stream = nullptr;
+    return nullptr;
+  }
+  return &sd;
+}
+
+int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_bytes, kmoe_stream_t stream,
+                     bool may_fork);
+
+}  // namespace
+
 extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t workspace_bytes,
                                 kmoe_stream_t stream) {
+  return moe_forward_impl(a, workspace, workspace_bytes, stream, true);
+}
+
+namespace {
+
+int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_bytes, kmoe_stream_t stream,
+                     bool may_fork) {
   kmoe_moe_layout L;
   if (int rc = kmoe_moe_workspace_layout(a, &L)) return rc;
   if (a->M == 0) return KMOE_OK;
@@ -481,16 +540,15 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
     routed.w2_aux_tail = a->ws2_max;
     routed.tail_rows = M;
   }
-  rc = run_mlp(routed, stream, mark);
-  if (rc) return rc;
-
-  // 7. dense shared expert on all M rows: the grouped GEMM with a single expert whose lod is {0, M}
-  mark(KMOE_STAGE_SHARED, 0);
+  // 7. dense shared expert on all M rows: the grouped GEMM with a single expert whose lod is {0, M}. With a side
+  // stream it is enqueued there BEFORE the routed pass (it reads x / its codes only) and joined after it.
   const uint16_t* shared_out = fold ? routed.out + static_cast<size_t>(P) * H : nullptr;
-  if (a->I_shared > 0 && !fold) {
+  const bool own_pass = a->I_shared > 0 && !fold;
+  SideStream* side = own_pass && may_fork && !a->stage_events ? side_stream(as_stream(stream)) : nullptr;
+  auto shared_pass = [&](kmoe_stream_t st) -> int {
     int32_t* dense_lod = static_cast<int32_t*>(at(L.sh_lod));
-    rc = fill_dense_lod(dense_lod, stream_mode ? 0 : M, as_stream(stream));  // (streaming path: see below)
-    if (rc) return rc;
+    int rcs = fill_dense_lod(dense_lod, stream_mode ? 0 : M, as_stream(st));  // (streaming path: see below)
+    if (rcs) return rcs;
     MlpPass sh = routed;
     // the expert-bias branch belongs to the routed experts only: a dense shared MLP has no per-expert
     // bias and uses the plain SiLU-mul over [gate | up] rows
@@ -527,9 +585,31 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
     sh.actq = at(L.sh_actq);
     sh.act_aux = static_cast<float*>(at(L.sh_actmax));
     sh.out = static_cast<uint16_t*>(at(L.sh_out));
-    rc = run_mlp(sh, stream, [](int, int) {});
-    if (rc) return rc;
+    rcs = run_mlp(sh, st, [](int, int) {});
+    if (rcs) return rcs;
     shared_out = sh.out;
+    return KMOE_OK;
+  };
+  if (side) {
+    hipError_t e = hipEventRecord(side->fork, as_stream(stream));
+    if (e == hipSuccess) e = hipStreamWaitEvent(side->stream, side->fork, 0);
+    KMOE_REQUIRE(e == hipSuccess, KMOE_ERR_LAUNCH, "moe_forward: fork to the side stream: %s", hipGetErrorString(e));
+    const int rc_side = shared_pass(side->stream);
+    rc = rc_side ? rc_side : run_mlp(routed, stream, mark);
+    // joined in any case, after the routed pass is in the caller's stream: a captured side stream must come back
+    // to the stream it forked from
+    e = hipEventRecord(side->join, side->stream);
+    if (e == hipSuccess) e = hipStreamWaitEvent(as_stream(stream), side->join, 0);
+    if (rc) return rc;
+    KMOE_REQUIRE(e == hipSuccess, KMOE_ERR_LAUNCH, "moe_forward: join of the side stream: %s", hipGetErrorString(e));
+  } else {
+    rc = run_mlp(routed, stream, mark);
+    if (rc) return rc;
+  }
+  mark(KMOE_STAGE_SHARED, 0);
+  if (own_pass && !side) {
+    rc = shared_pass(stream);
+    if (rc) return rc;
   }
   mark(KMOE_STAGE_SHARED, 1);
   // 8. weighted combine (+ caller epilogue)
@@ -541,6 +621,8 @@ extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t 
   mark(KMOE_STAGE_COMBINE, 1);
   return rc;
 }
+
+}  // namespace
 
 // ---- the layer for callers that cannot hand over a workspace -------------------------------
 // kmoe_moe_forward with its workspace in a file-scope device array. The array's name is only a
@@ -587,5 +669,5 @@ extern "C" int kmoe_moe_forward_static(const kmoe_moe_args* a, kmoe_stream_t str
   if (int rc = static_workspace(&ws)) return rc;
   // every slot of the layout is written by the stage that owns it before anything reads it, so
   // the last call's contents need no clearing
-  return kmoe_moe_forward(a, ws, KMOE_STATIC_WORKSPACE_BYTES, stream);
+  return moe_forward_impl(a, ws, KMOE_STATIC_WORKSPACE_BYTES, stream, false);  // no second stream: nothing is created here
 }

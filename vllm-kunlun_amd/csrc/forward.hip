@@ -591,15 +591,21 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
     return KMOE_OK;
   };
   if (side) {
-    hipError_t e = hipEventRecord(side->fork, as_stream(stream));
-    if (e == hipSuccess) e = hipStreamWaitEvent(side->stream, side->fork, 0);
+    // (record and wait are one step under the lock: the events are shared by every caller on this GPU, and a
+    // wait refers to the event's latest record)
+    auto hand_over = [](hipEvent_t ev, hipStream_t from, hipStream_t to) {
+      std::lock_guard<std::mutex> lock(g_side_mutex);
+      hipError_t err = hipEventRecord(ev, from);
+      if (err == hipSuccess) err = hipStreamWaitEvent(to, ev, 0);
+      return err;
+    };
+    hipError_t e = hand_over(side->fork, as_stream(stream), side->stream);
     KMOE_REQUIRE(e == hipSuccess, KMOE_ERR_LAUNCH, "moe_forward: fork to the side stream: %s", hipGetErrorString(e));
     const int rc_side = shared_pass(side->stream);
     rc = rc_side ? rc_side : run_mlp(routed, stream, mark);
     // joined in any case, after the routed pass is in the caller's stream: a captured side stream must come back
     // to the stream it forked from
-    e = hipEventRecord(side->join, side->stream);
-    if (e == hipSuccess) e = hipStreamWaitEvent(as_stream(stream), side->join, 0);
+    e = hand_over(side->join, side->stream, as_stream(stream));
     if (rc) return rc;
     KMOE_REQUIRE(e == hipSuccess, KMOE_ERR_LAUNCH, "moe_forward: join of the side stream: %s", hipGetErrorString(e));
   } else {

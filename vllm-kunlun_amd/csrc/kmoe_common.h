@@ -127,6 +127,13 @@ __device__ inline float wave_max(float v) {
   for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
   return v;
 }
+// max over aligned groups of G lanes (G a power of two up to 64)
+template <int G>
+__device__ inline float group_max(float v) {
+#pragma unroll
+  for (int off = G / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
 
 // Butterfly sum: every lane ends with the same bits (each step adds the same
 // two numbers on both sides). Equivalent to the balanced binary tree

@@ -11,7 +11,7 @@ union Pack8 {  // 8 bf16 (or half) values
 };
 
 // ---------------------------------------------------------------- int8 rows
-// TPR threads cooperate on one row; each keeps NV vectors of 8 values in
+// TPR threads cooperate on one row (32: two rows per wave); each keeps NV vectors of 8 values in
 // registers, so the row is read from memory once.
 // Workgroup `block` (256 threads) serves rows block * (256 / TPR) ...
 template <int TPR, int NV>
@@ -39,7 +39,7 @@ __device__ inline void quant_i8_rows_body(const uint16_t* __restrict__ x, int64_
       }
     }
   }
-  amax = wave_max(amax);
+  amax = group_max<(TPR < kWave ? TPR : kWave)>(amax);
   if (TPR > kWave) {  // one row per block: combine the waves
     if (lane_id() == 0) red[threadIdx.x >> 6] = amax;
     __syncthreads();

@@ -313,7 +313,10 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
                   "tops": work["layer_ops"] / t_s / 1e12,
                   "mfma_frac": work["layer_ops"] / t_s / 1e12 / peak_tops,
                   "algorithmic_bytes": work["layer_bytes"], "algorithmic_ops": work["layer_ops"],
-                  "stage_ms": stage_ms},
+                  "stage_ms": stage_ms,
+                  # what a stage with no launch in it reads (two event records back to back): every entry of
+                  # stage_ms carries about this much on top of its kernels, so their sum exceeds ms_per_step
+                  "stage_event_overhead_ms": min(stage_ms.values())},
     }
     if a.yardstick and shape.quant in ("int8", "none"):
         res["vendor_dense_gemm"] = vendor_dense_gemm(shape, work["g1_ops"], peak_tops)

@@ -304,10 +304,13 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
     mf = avg <= 10 ? 1 : (avg <= 22 ? 2 : 4);
   }
   switch (mf) {
-    // (two blocks in flight: 55.8 / 32.8 us on the Qwen3 decode GEMMs against 57.2 / 35.0 with three)
-    case 1: return swiglu ? launch_w4<1, 2, true, 2>(p, f16, s) : launch_w4<1, 2, false, 2>(p, f16, s);
+    // One block in flight per wave: the registers that saves put more waves on a SIMD (5-6 instead of 3-4), and
+    // the unpacking work of one wave hides the loads of the others better than a deeper queue of its own does
+    // (Qwen3 decode GEMMs: 52.9 / 31.2 us against 54.2 / 33.1 with two blocks and 55.8 / 34.8 with three).
+    case 1: return swiglu ? launch_w4<1, 2, true, 1>(p, f16, s) : launch_w4<1, 2, false, 1>(p, f16, s);
     // tuning variants of the 16-row kernel: 1xy = x fragments per wave, y blocks in flight
     case 123: return swiglu ? launch_w4<1, 2, true, 3>(p, f16, s) : launch_w4<1, 2, false, 3>(p, f16, s);
+    case 141: return swiglu ? launch_w4<1, 4, true, 1>(p, f16, s) : launch_w4<1, 4, false, 1>(p, f16, s);
     case 124: return swiglu ? launch_w4<1, 2, true, 4>(p, f16, s) : launch_w4<1, 2, false, 4>(p, f16, s);
     case 142: return swiglu ? launch_w4<1, 4, true, 2>(p, f16, s) : launch_w4<1, 4, false, 2>(p, f16, s);
     case 143: return swiglu ? launch_w4<1, 4, true, 3>(p, f16, s) : launch_w4<1, 4, false, 3>(p, f16, s);

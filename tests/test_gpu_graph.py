@@ -120,3 +120,45 @@ def test_dense_matmul_op_under_graph_capture():
     fresh = [(torch.randint(-127, 128, (M, k), generator=g, device="cuda", dtype=torch.int8),
               torch.rand(M, 1, generator=g, device="cuda") + 0.5) for _ in range(3)]
     _replays(graph, (x, x_max), fresh, out, eager)
+
+
+def test_two_threads_share_the_side_stream():
+    """Two host threads, each with a stream and a layer of its own whose shared expert runs on the library's second
+    stream (one per GPU: both threads fork to it and join from it), calling at the same time: every call gives the
+    bits the layer gives alone."""
+    import threading
+    from vllm_kunlun_amd import synth
+    shapes = [synth.scaled(synth.SHAPES["dsv3-decode"], M=24 + 8 * i, H=512, E=32, K=4, I=128, n_group=4, topk_group=2,
+                           I_shared=256 + 128 * i) for i in range(2)]
+    layers = [synth.make_layer(sh, "cuda", seed=20 + i) for i, sh in enumerate(shapes)]
+    want = []
+    for sl in layers:
+        want.append(sl.layer.quant_method.apply_monolithic(sl.layer, sl.x, sl.logits, **sl.apply_kwargs()).clone())
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(i):
+        try:
+            sl = layers[i]
+            stream = torch.cuda.Stream()
+            stream.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(stream):
+                for it in range(40):
+                    out = sl.layer.quant_method.apply_monolithic(sl.layer, sl.x, sl.logits, **sl.apply_kwargs())
+                    if it % 8 == 7:
+                        stream.synchronize()
+                        if not torch.equal(out, want[i]):
+                            errors.append((i, it))
+                stream.synchronize()
+                if not torch.equal(out, want[i]):
+                    errors.append((i, "last"))
+        except Exception as ex:  # noqa: BLE001
+            errors.append((i, repr(ex)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors

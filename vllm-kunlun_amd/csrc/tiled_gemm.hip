@@ -1008,13 +1008,17 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   constexpr TKind K = TKind::I8;
   const int avg_rows = ceil_div(a->rows + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
   const bool shorter = short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu);
-  // 128-row tiles whose sibling m-tiles are paced against each other (see g_board). By default where most
-  // experts have one or two m-tiles (96 to 256 rows on average): there every second expert's weights are
-  // streamed twice, and keeping the two streams together is worth 3-5 % (DeepSeek-V3 shape, 4096 tokens:
-  // gate_up 1950 -> 1898 us, down 972 -> 926 us; bytes fetched by L2 1.49x -> 1.08x of the algorithmic ones).
-  // With four or five m-tiles per expert the chain of waits costs more than it saves (Qwen3 shape at 8192
-  // tokens: +3 to +8 %), with one tile there is nothing to pace.
-  const bool paced = a->variant == 12 || (a->variant == 0 && !shorter && avg_rows > 96 && avg_rows <= 256);
+  // 128-row tiles whose sibling m-tiles are paced against each other (see g_board). By default where experts
+  // have more than one m-tile (more than 96 rows on average) AND the launch's weights are far more than the
+  // 256 MB memory-side cache holds: there a sibling that falls behind fetches its weights from HBM again, and
+  // keeping the siblings together is worth 3-7 % at every batch size (DeepSeek-V3 shape: 4096 tokens gate_up
+  // 1950 -> 1898 us, down 972 -> 926 us, bytes fetched by L2 1.49x -> 1.08x of the algorithmic ones; 12288
+  // tokens 4051 -> 3937 and 2225 -> 2070 us; 32768 tokens 10.79 -> 10.37 ms). A launch whose weights fit that
+  // cache (Qwen3 shape: 403 and 201 MB) re-reads them from there at little cost, and the waits only cost:
+  // +1.5 to +4 % from 2048 to 8192 tokens.
+  const long long weight_bytes = static_cast<long long>(a->E + (a->w_tail ? 1 : 0)) * a->n * a->k;
+  const bool paced = a->variant == 12 ||
+                     (a->variant == 0 && !shorter && avg_rows > 96 && weight_bytes > (1ll << 30));
   if (a->act_dtype == KMOE_DT_F16) {
     // half outputs: the shapes in use (64-row, 128-row and paced 128-row tiles); the tuning variants are bf16 only
     KMOE_REQUIRE(a->variant == 0 || a->variant == 5 || a->variant == 6 || a->variant == 11 || a->variant == 12,
@@ -1071,11 +1075,13 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
   if (short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu))
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);
-  // paced sibling m-tiles where most experts have one or two of them, as for int8, and a tile walks a long K
-  // (DeepSeek-V3 shape at 4096 tokens: gate_up, K = 7168, 2570 -> 2222 us; the down projection, K = 2048, is
-  // 5 % slower with it: 1033 -> 1083 us)
+  // paced sibling m-tiles where experts have more than one of them and the weights are far more than the
+  // memory-side cache holds, as for int8, and a tile walks a long K (DeepSeek-V3 shape at 4096 tokens: gate_up,
+  // K = 7168, 2570 -> 2222 us; the down projection, K = 2048, is 5 % slower with it: 1033 -> 1083 us; layer at
+  // 8192 tokens 5.86 -> 5.78 ms, at 16384 tokens 10.90 -> 10.66 ms)
   const int avg_rows = ceil_div(a->rows + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
-  if (a->variant == 12 || (a->variant == 0 && avg_rows > 96 && avg_rows <= 256 && a->k >= 4096))
+  const long long weight_bytes = static_cast<long long>(a->E + (a->w_tail ? 1 : 0)) * a->n * a->k;
+  if (a->variant == 12 || (a->variant == 0 && avg_rows > 96 && a->k >= 4096 && weight_bytes > (1ll << 30)))
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 8, false, true>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 8, false, true>(p, a->rows, s, n_cu, what);
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)

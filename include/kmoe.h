@@ -154,6 +154,22 @@ int kmoe_quant_i8_rows_chunked_dt(const uint16_t* x, int64_t ld_x, int R, int C,
                                   float* row_max, int act_dtype, kmoe_stream_t stream);
 
 /*
+ * The other modes of torch.ops._C.scaled_int8_quant (ops/_custom_ops.py:1633-1657), which the reference hands
+ * to xspeedgate_ops.static_scaled_int8_quant / dynamic_scaled_int8_quant (closed). Their arithmetic is the one
+ * of the vLLM operator of the same name that the reference's scheme classes are written against
+ * (csrc/quantization/compressed_tensors/int8_quant_kernels.cu):
+ *   static:           q = sat8( rint(x / scale[0]) (+ azp[0]) )             one f32 scale (and zero point) per tensor
+ *   dynamic + azp:    per row: s = (max - min) / 255 (1 for a constant row), azp = rint(-128 - min / s),
+ *                     q = sat8( rint(x / s) + azp ); row_scale[r] = s, row_azp[r] = azp
+ * with IEEE division, round-half-even and saturation to [-128, 127] (the sum with the zero point in int32).
+ * x [R,C] in act_dtype; scale, azp: device pointers. Limits: C % 8 == 0, C <= 65536.
+ */
+int kmoe_quant_i8_static(const uint16_t* x, int64_t ld_x, int R, int C, const float* scale, const int32_t* azp,
+                         int8_t* q, int64_t ld_q, int act_dtype, kmoe_stream_t stream);
+int kmoe_quant_i8_rows_azp(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q,
+                           float* row_scale, int32_t* row_azp, int act_dtype, kmoe_stream_t stream);
+
+/*
  * Per-row, per-128-column-group dynamic fp8-e4m3fn (OCP). No counterpart in the
  * reference (its fp8 ops are empty stubs, ops/_custom_ops.py:44-89); follows
  * the DeepSeek-V3 block-scaled recipe.

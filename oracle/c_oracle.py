@@ -148,6 +148,29 @@ def quant_i8_rows(x_bits, f16=False):
     return q, mx
 
 
+def quant_i8_static(x_bits, scale, azp=None, f16=False):
+    """One scale (and zero point) for the tensor: codes int8 [R,C]."""
+    _dtype(f16)
+    x_bits = _c(x_bits, np.uint16)
+    R, Cc = x_bits.shape
+    q = np.zeros((R, Cc), np.int8)
+    lib().orc_quant_i8_static(_p(x_bits), C.c_int64(Cc), R, Cc, C.c_float(float(scale)), 0 if azp is None else 1,
+                              0 if azp is None else int(azp), _p(q), C.c_int64(Cc))
+    return q
+
+
+def quant_i8_rows_azp(x_bits, f16=False):
+    """Per-row scale and zero point: (codes int8 [R,C], scale f32 [R], azp int32 [R])."""
+    _dtype(f16)
+    x_bits = _c(x_bits, np.uint16)
+    R, Cc = x_bits.shape
+    q = np.zeros((R, Cc), np.int8)
+    s = np.zeros(R, np.float32)
+    z = np.zeros(R, np.int32)
+    lib().orc_quant_i8_rows_azp(_p(x_bits), C.c_int64(Cc), R, Cc, _p(q), C.c_int64(Cc), _p(s), _p(z))
+    return q, s, z
+
+
 def quant_fp8_group128(x_bits):
     x_bits = _c(x_bits, np.uint16)
     R, Cc = x_bits.shape

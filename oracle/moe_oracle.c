@@ -277,6 +277,43 @@ ORC_API void orc_quant_i8_rows(const uint16_t* x, int64_t ld_x, int R, int C, in
   }
 }
 
+/* The other modes of scaled_int8_quant (ops/_custom_ops.py:1633-1657 forwards them to closed kernels; the
+ * arithmetic restated here is the one of the vLLM operator of the same name, csrc/quantization/
+ * compressed_tensors/int8_quant_kernels.cu): one scale (and zero point) for the tensor, or per row the
+ * scale (max - min) / 255 and the zero point rint(-128 - min / scale). IEEE division, round half to even,
+ * the zero point added in integers, saturation to [-128, 127]. A constant row takes scale 1 (the upstream
+ * kernel divides by zero there). */
+static int8_t sat8_ll(long long t) { return (int8_t)(t < -128 ? -128 : (t > 127 ? 127 : t)); }
+static long long rint_clamped(float f) {
+  f = rintf(f);
+  if (!(f > -2147483000.0f)) f = -2147483000.0f; /* also NaN */
+  if (f > 2147483000.0f) f = 2147483000.0f;
+  return (long long)(int)f;
+}
+ORC_API void orc_quant_i8_static(const uint16_t* x, int64_t ld_x, int R, int C, float scale, int has_azp, int32_t azp,
+                                 int8_t* q, int64_t ld_q) {
+  for (int r = 0; r < R; ++r)
+    for (int c = 0; c < C; ++c)
+      q[(size_t)r * ld_q + c] = sat8_ll(rint_clamped(act_to_f32(x[(size_t)r * ld_x + c]) / scale) + (has_azp ? azp : 0));
+}
+ORC_API void orc_quant_i8_rows_azp(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q,
+                                   float* row_scale, int32_t* row_azp) {
+  for (int r = 0; r < R; ++r) {
+    const uint16_t* xr = x + (size_t)r * ld_x;
+    float lo = INFINITY, hi = -INFINITY;
+    for (int c = 0; c < C; ++c) {
+      lo = fminf(lo, act_to_f32(xr[c]));
+      hi = fmaxf(hi, act_to_f32(xr[c]));
+    }
+    float s = (hi - lo) / 255.0f;
+    if (!(s > 0.0f)) s = 1.0f;
+    const long long z = rint_clamped(-128.0f - lo / s);
+    for (int c = 0; c < C; ++c) q[(size_t)r * ld_q + c] = sat8_ll(rint_clamped(act_to_f32(xr[c]) / s) + z);
+    row_scale[r] = s;
+    row_azp[r] = (int32_t)z;
+  }
+}
+
 /* OCP e4m3fn encoding by exhaustive nearest-value search (ties to even code). */
 static float e4m3fn_value(int code) { /* code in [0,127), positive */
   const int ex = code >> 3, man = code & 7;

@@ -163,6 +163,71 @@ def test_quant_i8_rows(L, R, Cc):
     assert np.array_equal(q.cpu().numpy(), q_ref)
 
 
+@pytest.mark.parametrize("R,Cc", [(1, 8), (5, 256), (100, 768), (33, 7168), (512, 2048), (2, 65536)])
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("scale,azp", [(0.0237, None), (0.0625, 17), (0.011, -90)])
+def test_quant_i8_static(L, R, Cc, half, scale, azp):
+    """One scale (and zero point) for the tensor, through the C ABI and through `_C::scaled_int8_quant`: the
+    oracle's codes, bit for bit (values far outside the range saturate on both sides)."""
+    import vllm_kunlun_amd  # noqa: F401  (registers torch.ops._C.*)
+    torch.manual_seed(R + Cc)
+    x = (torch.randn(R, Cc) * 2).to(torch.float16 if half else torch.bfloat16)
+    x[0, 0], x[0, 1] = 6e4, -6e4
+    ref = co.quant_i8_static(bits(x), np.float32(scale), azp, f16=half)
+    dx = x.cuda()
+    ds = torch.tensor([scale], dtype=torch.float32, device="cuda")
+    dz = None if azp is None else torch.tensor([azp], dtype=torch.int32, device="cuda")
+    q = torch.empty(R, Cc, dtype=torch.int8, device="cuda")
+    L.check(L.lib.kmoe_quant_i8_static(L.ptr(dx), Cc, R, Cc, L.ptr(ds), L.ptr(dz), L.ptr(q), Cc, L.act_dtype(dx),
+                                       L.stream()))
+    sync()
+    assert np.array_equal(q.cpu().numpy(), ref)
+    q2, s2, z2, static = torch.ops._C.scaled_int8_quant(dx.view(1, R, Cc), ds, dz, azp is None)
+    sync()
+    assert static and q2.shape == (1, R, Cc) and np.array_equal(q2.cpu().numpy()[0], ref)
+    assert torch.equal(s2, ds) and (z2.numel() == 0 if azp is None else torch.equal(z2, dz))
+
+
+@pytest.mark.parametrize("R,Cc", [(1, 8), (5, 256), (100, 768), (33, 7168), (7, 1000), (3, 1), (2, 65536)])
+@pytest.mark.parametrize("half", [False, True])
+def test_quant_i8_rows_azp(L, R, Cc, half):
+    """Per-row scale and zero point (dynamic asymmetric), through the C ABI and through `_C::scaled_int8_quant`:
+    codes, scales and zero points of the oracle, bit for bit; a constant row and an all-zero row included."""
+    import vllm_kunlun_amd  # noqa: F401
+    torch.manual_seed(R * 7 + Cc)
+    x = (torch.randn(R, Cc) * torch.rand(R, 1) * 4 + torch.randn(R, 1) * 3).to(torch.float16 if half else torch.bfloat16)
+    x[0] = 0
+    if R > 2:
+        x[1] = 0.75
+    q_ref, s_ref, z_ref = co.quant_i8_rows_azp(bits(x), f16=half)
+    dx = x.cuda()
+    q = torch.empty(R, Cc, dtype=torch.int8, device="cuda")
+    s = torch.empty(R, dtype=torch.float32, device="cuda")
+    z = torch.empty(R, dtype=torch.int32, device="cuda")
+    L.check(L.lib.kmoe_quant_i8_rows_azp(L.ptr(dx), Cc, R, Cc, L.ptr(q), Cc, L.ptr(s), L.ptr(z), L.act_dtype(dx),
+                                         L.stream()))
+    sync()
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), s_ref.view(np.uint32))
+    assert np.array_equal(z.cpu().numpy(), z_ref)
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    q2, s2, z2, static = torch.ops._C.scaled_int8_quant(dx, None, None, False)
+    sync()
+    assert not static and s2.shape == (R, 1) and z2.shape == (R, 1) and z2.dtype == torch.int32
+    assert np.array_equal(q2.cpu().numpy(), q_ref) and np.array_equal(s2.cpu().numpy().ravel(), s_ref)
+    assert np.array_equal(z2.cpu().numpy().ravel(), z_ref)
+
+
+def test_quant_i8_static_refusals(L):
+    import vllm_kunlun_amd  # noqa: F401
+    x = torch.zeros(4, 12, dtype=torch.bfloat16, device="cuda")  # 12 columns: not a multiple of 8
+    s = torch.ones(1, dtype=torch.float32, device="cuda")
+    with pytest.raises(Exception, match="quant_i8_static"):
+        torch.ops._C.scaled_int8_quant(x, s, None, True)
+    with pytest.raises(Exception, match="one float32"):
+        torch.ops._C.scaled_int8_quant(torch.zeros(4, 16, dtype=torch.bfloat16, device="cuda"),
+                                       torch.ones(4, dtype=torch.float32, device="cuda"), None, True)
+
+
 @pytest.mark.parametrize("R,Cc", [(1, 128), (17, 2048), (64, 7168), (5, 384)])
 def test_quant_fp8_group128(L, R, Cc):
     torch.manual_seed(R + Cc)

@@ -815,3 +815,59 @@ def test_half_layer_against_the_torch_expert_loop():
     out_h = co.forward_w8a8(_half_bits(xh), logits.numpy(), w13.numpy(), w13_max.numpy(), w2.numpy(), w2_max.numpy(), 2,
                             f16=True)
     assert rel_l2(_from_half_bits(out_h), from_bits(out_b)) <= 2e-2
+
+
+# ------------------------------------------------------------------ static and asymmetric int8
+def test_quant_i8_static_known_answers_and_the_library_quantiser():
+    """x / scale rounded half to even, zero point added in integers, saturation to [-128, 127]: hand-made
+    answers, and torch.quantize_per_tensor (its inverse-scale product is exact for power-of-two scales)."""
+    x = torch.tensor([[0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 127.0, 128.0],
+                      [-128.0, -129.0, 300.0, -300.0, 3.0, 0.0, 1e30, -1e30]]).bfloat16()
+    q = co.quant_i8_static(bits(x), 1.0)
+    assert q.tolist() == [[0, 2, 2, 0, -2, -2, 127, 127], [-128, -128, 127, -128, 3, 0, 127, -128]]
+    q = co.quant_i8_static(bits(x), 1.0, azp=5)  # the zero point moves the codes before the saturation
+    assert q.tolist() == [[5, 7, 7, 5, 3, 3, 127, 127], [-123, -124, 127, -128, 8, 5, 127, -128]]
+    q = co.quant_i8_static(bits(x), 0.5, azp=-100)
+    assert q[0].tolist() == [-99, -97, -95, -101, -103, -105, 127, 127]
+    g = torch.Generator().manual_seed(0)
+    for dtype, f16 in ((torch.bfloat16, False), (torch.float16, True)):
+        xr = (torch.randn(64, 96, generator=g) * 3).to(dtype)
+        for scale, zp in ((0.0625, 0), (0.03125, 17), (0.125, -90)):
+            ref = torch.quantize_per_tensor(xr.float(), scale, zp, torch.qint8).int_repr().numpy()
+            got = co.quant_i8_static(bits(xr), scale, azp=zp if zp else None, f16=f16)
+            assert np.array_equal(got, ref), (dtype, scale, zp)
+    # a scale that is no power of two: the quotient is the IEEE float division, not a product with 1 / scale
+    xr = (torch.randn(32, 64, generator=g) * 3).bfloat16()
+    s = np.float32(0.0237)
+    ref = np.clip(np.rint(xr.float().numpy() / s), -128, 127).astype(np.int8)
+    assert np.array_equal(co.quant_i8_static(bits(xr), s), ref)
+
+
+def test_quant_i8_rows_azp_closed_forms_and_invariants():
+    """Per row: scale (max - min) / 255, zero point rint(-128 - min / scale). Rows whose answer is known in
+    closed form; for random rows the minimum lands on -128, the maximum on 127 (within one code, the two
+    roundings), every value is recovered within one step, and the codes are monotone in the values."""
+    ramp = torch.arange(-128, 128, dtype=torch.float32)
+    rows = torch.stack([ramp, ramp + 128.0, ramp * 0.5, -ramp, torch.full((256,), 3.0), torch.zeros(256)])
+    q, s, z = co.quant_i8_rows_azp(bits(rows.bfloat16()))
+    assert s.tolist() == [1.0, 1.0, 0.5, 1.0, 1.0, 1.0]
+    assert z.tolist() == [0, -128, 0, -1, -131, -128]  # -ramp runs from -127 to 128: its zero point is -1
+    assert np.array_equal(q[0], np.arange(-128, 128)) and np.array_equal(q[1], np.arange(-128, 128))
+    assert np.array_equal(q[2], np.arange(-128, 128)) and np.array_equal(q[3], np.arange(-128, 128)[::-1])
+    assert (q[4] == -128).all() and (q[5] == -128).all()  # a constant row: scale 1, every code rint(v) + azp
+    g = torch.Generator().manual_seed(1)
+    for dtype, f16 in ((torch.bfloat16, False), (torch.float16, True)):
+        x = (torch.randn(200, 333, generator=g) * torch.rand(200, 1, generator=g) * 8 + torch.randn(200, 1, generator=g) * 4)
+        x = x.to(dtype)
+        q, s, z = co.quant_i8_rows_azp(bits(x), f16=f16)
+        xf = x.float().numpy()
+        lo, hi = xf.min(1), xf.max(1)
+        assert np.array_equal(s, (hi - lo) / np.float32(255.0))
+        assert np.array_equal(z, np.rint(np.float32(-128.0) - lo / s).astype(np.int32))
+        qi = q.astype(np.int32)
+        assert (np.abs(qi[np.arange(200), xf.argmin(1)] + 128) <= 1).all()
+        assert (np.abs(qi[np.arange(200), xf.argmax(1)] - 127) <= 1).all()
+        back = (qi - z[:, None]) * s[:, None]
+        assert (np.abs(back - xf) <= s[:, None] * 1.001).all()
+        order = np.argsort(xf, axis=1, kind="stable")
+        assert (np.diff(np.take_along_axis(qi, order, 1), axis=1) >= 0).all()

@@ -50,7 +50,7 @@ def test_process_weights_after_loading_on_the_host():
     assert torch.equal(layer2.weight_scale.data, torch.full((32, 1), 0.25 * 127.0))
     # schemes outside the path are refused by name
     ok, why = KunlunScaledMMLinearKernel.can_implement(Int8ScaledMMLinearLayerConfig(is_static_input_scheme=True))
-    assert not ok and "static" in why
+    assert ok and why is None
     ok, why = KunlunScaledMMLinearKernel.can_implement(Int8ScaledMMLinearLayerConfig(input_symmetric=False))
     assert not ok and "asymmetric" in why
     with pytest.raises(ValueError):
@@ -80,6 +80,32 @@ def test_apply_weights_matches_the_oracle(M, n, k):
     assert np.array_equal(bits(out.reshape(-1, n)), ref)
     with pytest.raises(NotImplementedError):
         kern.apply_weights(layer, x.cuda(), bias=torch.zeros(n, device="cuda"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,n,k,dtype", [(1, 64, 128, torch.bfloat16), (37, 256, 512, torch.float16),
+                                         (300, 512, 1024, torch.bfloat16), (5, 48, 80, torch.bfloat16)])
+def test_apply_weights_with_a_static_input_scale(M, n, k, dtype):
+    """The static symmetric scheme (scale_mm.py:60-66 and 83-90 in the reference: the layer's one input scale
+    quantises the tensor, and the GEMM takes scale x 127 as every row's max): codes and output against the
+    oracle, bit for bit; values beyond 127 x scale saturate."""
+    from vllm_kunlun_amd.quantization.kernels.scale_mm import (Int8ScaledMMLinearLayerConfig,
+                                                               KunlunScaledMMLinearKernel)
+    layer, wq, w_max = _layer(n, k, "cuda", M + n + k)
+    scale = np.float32(0.021)
+    layer.input_scale = torch.nn.Parameter(torch.tensor([scale], device="cuda"), requires_grad=False)
+    kern = KunlunScaledMMLinearKernel(Int8ScaledMMLinearLayerConfig(is_static_input_scheme=True))
+    kern.process_weights_after_loading(layer)
+    assert layer.input_scale is not None
+    x = (torch.randn(M, k, generator=torch.Generator().manual_seed(M)) * 1.5).to(dtype)  # |x| up to ~6: some saturate
+    out = kern.apply_weights(layer, x.cuda())
+    torch.cuda.synchronize()
+    f16 = dtype == torch.float16
+    xq = co.quant_i8_static(bits(x), scale, f16=f16)
+    assert (np.abs(xq.astype(np.int32)) == 127).any() or M < 5
+    x_max = np.full(M, scale * np.float32(127.0), np.float32)
+    ref, _ = co.grouped_gemm_i8(xq, x_max, wq.numpy()[None], w_max.numpy()[None], np.array([0, M], np.int32), f16=f16)
+    assert out.dtype == dtype and np.array_equal(bits(out), ref)
 
 
 @pytest.mark.gpu

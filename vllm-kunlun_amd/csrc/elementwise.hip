@@ -12,6 +12,70 @@ __global__ __launch_bounds__(256) void quant_i8_rows_kernel(const uint16_t* __re
   quant_i8_rows_body<TPR, NV>(x, ld_x, R, C, q, ld_q, row_max, chunked, blockIdx.x, f16 != 0);
 }
 
+// ---------------------------------------- static and asymmetric int8 (the other modes of scaled_int8_quant)
+// one thread: 8 values; scale and zero point of the whole tensor
+__global__ __launch_bounds__(256) void quant_i8_static_kernel(const uint16_t* __restrict__ x, int64_t ld_x, int R,
+                                                             int C, const float* __restrict__ scale,
+                                                             const int32_t* __restrict__ azp, int8_t* __restrict__ q,
+                                                             int64_t ld_q, int f16) {
+  const int vec_per_row = C / 8;
+  const long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= static_cast<long long>(R) * vec_per_row) return;
+  const int r = static_cast<int>(idx / vec_per_row), c = static_cast<int>(idx % vec_per_row) * 8;
+  const float s = scale[0];
+  const int z = azp ? azp[0] : 0;
+  Pack8 v;
+  v.v = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(r) * ld_x + c);
+  uint32_t w[2] = {0, 0};
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    // (the float is clamped before the conversion so that the int32 sum with the zero point cannot overflow)
+    const float f = fminf(fmaxf(__builtin_rintf(act_to_f32(v.h[j], f16 != 0) / s), -2147483000.0f), 2147483000.0f);
+    const long long t = static_cast<long long>(static_cast<int>(f)) + z;
+    const int qi = static_cast<int>(t < -128 ? -128 : (t > 127 ? 127 : t));
+    w[j >> 2] |= static_cast<uint32_t>(qi & 0xff) << (8 * (j & 3));
+  }
+  *reinterpret_cast<uint2*>(q + static_cast<size_t>(r) * ld_q + c) = make_uint2(w[0], w[1]);
+}
+
+// one workgroup per row: min and max, then the codes (the row is read twice; this mode is not on a hot path)
+__global__ __launch_bounds__(256) void quant_i8_rows_azp_kernel(const uint16_t* __restrict__ x, int64_t ld_x, int C,
+                                                               int8_t* __restrict__ q, int64_t ld_q,
+                                                               float* __restrict__ row_scale,
+                                                               int32_t* __restrict__ row_azp, int f16) {
+  __shared__ float red_lo[4], red_hi[4];
+  const int r = blockIdx.x;
+  const uint16_t* xr = x + static_cast<size_t>(r) * ld_x;
+  float lo = __builtin_inff(), hi = -__builtin_inff();
+  for (int c = threadIdx.x; c < C; c += 256) {
+    const float f = act_to_f32(xr[c], f16 != 0);
+    lo = fminf(lo, f);
+    hi = fmaxf(hi, f);
+  }
+  hi = wave_max(hi);
+  lo = -wave_max(-lo);
+  if (lane_id() == 0) {
+    red_lo[threadIdx.x >> 6] = lo;
+    red_hi[threadIdx.x >> 6] = hi;
+  }
+  __syncthreads();
+  lo = fminf(fminf(red_lo[0], red_lo[1]), fminf(red_lo[2], red_lo[3]));
+  hi = fmaxf(fmaxf(red_hi[0], red_hi[1]), fmaxf(red_hi[2], red_hi[3]));
+  float s = (hi - lo) / 255.0f;
+  if (!(s > 0.0f)) s = 1.0f;  // a constant row: every code is the zero point
+  const float zf = fminf(fmaxf(__builtin_rintf(-128.0f - lo / s), -2147483000.0f), 2147483000.0f);
+  const int z = static_cast<int>(zf);
+  for (int c = threadIdx.x; c < C; c += 256) {
+    const float f = fminf(fmaxf(__builtin_rintf(act_to_f32(xr[c], f16 != 0) / s), -2147483000.0f), 2147483000.0f);
+    const long long t = static_cast<long long>(static_cast<int>(f)) + z;
+    q[static_cast<size_t>(r) * ld_q + c] = static_cast<int8_t>(t < -128 ? -128 : (t > 127 ? 127 : t));
+  }
+  if (threadIdx.x == 0) {
+    row_scale[r] = s;
+    row_azp[r] = z;
+  }
+}
+
 // ------------------------------------------------------------- fp8 group128
 // OCP e4m3fn encode of two floats, round-to-nearest-even, saturating at 448 (NaN -> the largest
 // code of its sign): the conversion instruction of gfx950 (v_cvt_pk_fp8_f32 encodes the OCP format
@@ -278,6 +342,34 @@ extern "C" int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, i
   hipLaunchKernelGGL(quant_fp8_group128_kernel, dim3(static_cast<unsigned>((groups + 15) / 16)), dim3(256), 0,
                      as_stream(stream), x, ld_x, R, C, q, ld_q, scale);
   return check_launch("kmoe_quant_fp8_group128");
+}
+
+extern "C" int kmoe_quant_i8_static(const uint16_t* x, int64_t ld_x, int R, int C, const float* scale,
+                                    const int32_t* azp, int8_t* q, int64_t ld_q, int act_dtype, kmoe_stream_t stream) {
+  if (int rc = check_dtype(act_dtype, "quant_i8_static")) return rc;
+  KMOE_REQUIRE(x && scale && q, KMOE_ERR_NULL, "quant_i8_static: NULL pointer");
+  KMOE_REQUIRE(R >= 0 && C >= 8 && C % 8 == 0 && C <= 65536, KMOE_ERR_SHAPE, "quant_i8_static: R=%d C=%d (need C %% 8 == 0)", R, C);
+  KMOE_REQUIRE(ld_x % 8 == 0 && ld_x >= C && ld_q % 8 == 0 && ld_q >= C, KMOE_ERR_SHAPE,
+               "quant_i8_static: row strides %lld/%lld", (long long)ld_x, (long long)ld_q);
+  KMOE_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0, KMOE_ERR_SHAPE,
+               "quant_i8_static: misaligned tensor pointer");
+  if (R == 0) return KMOE_OK;
+  const long long n = static_cast<long long>(R) * (C / 8);
+  hipLaunchKernelGGL(quant_i8_static_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0,
+                     as_stream(stream), x, ld_x, R, C, scale, azp, q, ld_q, act_dtype == KMOE_DT_F16 ? 1 : 0);
+  return check_launch("kmoe_quant_i8_static");
+}
+
+extern "C" int kmoe_quant_i8_rows_azp(const uint16_t* x, int64_t ld_x, int R, int C, int8_t* q, int64_t ld_q,
+                                      float* row_scale, int32_t* row_azp, int act_dtype, kmoe_stream_t stream) {
+  if (int rc = check_dtype(act_dtype, "quant_i8_rows_azp")) return rc;
+  KMOE_REQUIRE(x && q && row_scale && row_azp, KMOE_ERR_NULL, "quant_i8_rows_azp: NULL pointer");
+  KMOE_REQUIRE(R >= 0 && C >= 1 && C <= 65536 && ld_x >= C && ld_q >= C, KMOE_ERR_SHAPE,
+               "quant_i8_rows_azp: R=%d C=%d strides %lld/%lld", R, C, (long long)ld_x, (long long)ld_q);
+  if (R == 0) return KMOE_OK;
+  hipLaunchKernelGGL(quant_i8_rows_azp_kernel, dim3(R), dim3(256), 0, as_stream(stream), x, ld_x, C, q, ld_q, row_scale,
+                     row_azp, act_dtype == KMOE_DT_F16 ? 1 : 0);
+  return check_launch("kmoe_quant_i8_rows_azp");
 }
 
 extern "C" int kmoe_dequant_w4_bf16(const uint8_t* packed, const uint16_t* scale, int64_t rows, int k, int group_size,

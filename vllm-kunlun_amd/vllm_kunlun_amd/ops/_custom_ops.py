@@ -193,17 +193,37 @@ def quant2d(x: torch.Tensor, x_q: torch.Tensor, max: torch.Tensor, force_sdnn: b
 @custom_op("_C::scaled_int8_quant", mutates_args=())
 def scaled_int8_quant(x: torch.Tensor, scale: Optional[torch.Tensor], azp: Optional[torch.Tensor] = None,
                       symmetric: bool = True) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, bool]:
-    """Dynamic per-token symmetric int8 (reference: ops/_custom_ops.py:1633-1657).
-    The returned `scale` holds the row MAX, as in the reference. The third
-    result stands for azp=None and is an empty tensor (operator schemas cannot
-    return None). Static and asymmetric modes are not on this path."""
-    if scale is not None or not symmetric:
-        raise NotImplementedError("scaled_int8_quant: only dynamic symmetric quantisation is implemented")
+    """int8 quantisation of activations (reference: ops/_custom_ops.py:1633-1657): returns (codes, scale, azp,
+    static). Dynamic symmetric (scale None, symmetric): per token, and the returned `scale` holds the row MAX, as in
+    the reference (quant2d). Static (scale given: one f32 for the tensor, optionally a zero point azp): codes =
+    sat8(rint(x / scale) + azp). Dynamic asymmetric (scale None, not symmetric): per token scale = (max - min) / 255
+    and zero point rint(-128 - min / scale). Where the reference returns azp = None this returns an empty tensor
+    (operator schemas cannot return None)."""
+    L.require_device(x, scale, azp)
     xc = x.contiguous()
+    rows, cols = xc.numel() // xc.shape[-1], xc.shape[-1]
     x_q = torch.empty_like(xc, dtype=torch.int8)
-    mx = torch.empty((xc.numel() // xc.shape[-1], 1), device=x.device, dtype=torch.float32)
-    quant2d(xc, x_q, mx, True)
-    return x_q, mx, torch.empty(0, dtype=torch.int32, device=x.device), False
+    none = torch.empty(0, dtype=torch.int32, device=x.device)
+    dt = L.act_dtype(xc, "scaled_int8_quant")
+    if scale is not None:  # static
+        _need(scale.numel() == 1 and scale.dtype == torch.float32, "scaled_int8_quant: the static scale is one float32")
+        _need(azp is None or (azp.numel() == 1 and azp.dtype == torch.int32),
+              "scaled_int8_quant: the static zero point is one int32")
+        if rows:
+            L.check(L.lib.kmoe_quant_i8_static(L.ptr(xc), cols, rows, cols, L.ptr(scale), L.ptr(azp), L.ptr(x_q), cols, dt,
+                                               L.stream()))
+        # (copies: an operator's results may not alias its arguments)
+        return x_q, scale.clone(), none if azp is None else azp.clone(), True
+    if symmetric:
+        mx = torch.empty((rows, 1), device=x.device, dtype=torch.float32)
+        quant2d(xc, x_q, mx, True)
+        return x_q, mx, none, False
+    s = torch.empty((rows, 1), device=x.device, dtype=torch.float32)
+    z = torch.empty((rows, 1), device=x.device, dtype=torch.int32)
+    if rows:
+        L.check(L.lib.kmoe_quant_i8_rows_azp(L.ptr(xc), cols, rows, cols, L.ptr(x_q), cols, L.ptr(s), L.ptr(z), dt,
+                                             L.stream()))
+    return x_q, s, z, False
 
 
 # ------------------------------------------------------------------------ GEMM
@@ -375,6 +395,8 @@ def matmul(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, x_trans: bo
     M, k = xc.shape
     n = wc.shape[0]
     out = torch.empty((M, n), dtype=out_dtype, device=x.device)
+    if x_pc_max.numel() == 1 and M != 1:  # one max for the tensor (static quantisation): every row's
+        x_pc_max = x_pc_max.reshape(1).expand(M)
     _gemm_i8(xc, x_pc_max.contiguous(), wc.unsqueeze(0), w_pc_max.contiguous(), _dense_lod(x.device, M), out, n,
              L.KMOE_ACT_NONE, M)
     return out
@@ -477,9 +499,12 @@ def _fake_moe_pre_small(topk_ids, global_num_experts, index_have_neg, sort_mode,
 
 @scaled_int8_quant.register_fake
 def _fake_scaled_int8_quant(x, scale, azp=None, symmetric=True):
-    return (torch.empty_like(x, dtype=torch.int8),
-            torch.empty((x.numel() // x.shape[-1], 1), device=x.device, dtype=torch.float32),
-            torch.empty(0, dtype=torch.int32, device=x.device), False)
+    rows = x.numel() // x.shape[-1]
+    none = torch.empty(0, dtype=torch.int32, device=x.device)
+    if scale is not None:
+        return torch.empty_like(x, dtype=torch.int8), torch.empty_like(scale), none if azp is None else torch.empty_like(azp), True
+    return (torch.empty_like(x, dtype=torch.int8), torch.empty((rows, 1), device=x.device, dtype=torch.float32),
+            none if symmetric else torch.empty((rows, 1), device=x.device, dtype=torch.int32), False)
 
 
 @matmul.register_fake

@@ -52,10 +52,8 @@ class KunlunScaledMMLinearKernel:
     def can_implement(cls, c: Int8ScaledMMLinearLayerConfig) -> tuple[bool, Optional[str]]:
         """Reference: scale_mm.py:39-41 accepts every config and fails later; this class says up
         front which schemes its kernels cover."""
-        if c.is_static_input_scheme:
-            return False, "static (per-tensor) input scales are not implemented; dynamic per-token only."
         if not c.input_symmetric:
-            return False, "asymmetric activations (azp) are not implemented."
+            return False, "asymmetric activations (azp) need the azp GEMM epilogue, which is not implemented."
         return True, None
 
     def _get_layer_params(self, layer):
@@ -94,13 +92,12 @@ class KunlunScaledMMLinearKernel:
 
     def apply_weights(self, layer: torch.nn.Module, x: torch.Tensor,
                       bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Reference: scale_mm.py:52-90. The symmetric dynamic branch: quantise per token, multiply,
-        rescale by x_max * w_max / 127^2, in x's dtype. Output [..., n]."""
+        """Reference: scale_mm.py:52-90. The symmetric branch: quantise per token (dynamic) or with the
+        layer's one input scale (static), multiply, rescale by x_max * w_max / 127^2, in x's dtype.
+        Output [..., n]."""
         w_q, w_s, x_s, x_zp, azp_adj = self._get_layer_params(layer)
         if azp_adj is not None or x_zp is not None:
             raise NotImplementedError("KunlunScaledMMLinearKernel: asymmetric activations are not implemented")
-        if x_s is not None:
-            raise NotImplementedError("KunlunScaledMMLinearKernel: static input scales are not implemented")
         if bias is not None:
             raise NotImplementedError("KunlunScaledMMLinearKernel: bias is not implemented on this path")
         dt = L.act_dtype(x, "KunlunScaledMMLinearKernel")
@@ -114,7 +111,11 @@ class KunlunScaledMMLinearKernel:
         out = torch.empty((M, n), dtype=x.dtype, device=x.device)
         if M == 0:
             return out.reshape(*lead, n)
-        if is_tiled(w) and M <= self.STREAM_MAX_ROWS:
+        if x_s is not None:  # static: one scale for the tensor, so every row's max is scale x 127
+            x_q, x_s, _, _ = torch.ops._C.scaled_int8_quant(x2, x_s.data.to(torch.float32).reshape(1), None, True)
+            x_max = (x_s * 127.0).expand(M).contiguous()
+            ops._gemm_i8(x_q, x_max, w, w_s.data.reshape(-1), self._row_range(x.device, M), out, n, L.KMOE_ACT_NONE, M)
+        elif is_tiled(w) and M <= self.STREAM_MAX_ROWS:
             self._stream_gemm(x2, w, w_s.data.reshape(-1), out)
         else:
             x_q, x_max, _, _ = torch.ops._C.scaled_int8_quant(x2, None, None, True)

@@ -339,7 +339,8 @@ typedef struct kmoe_gemm_w4_args {
   uint16_t* y;            /* bf16 [rows, n] or [rows, n/2] with SwiGLU                */
   int64_t ldy;
   int32_t act;            /* KMOE_ACT_NONE or KMOE_ACT_SWIGLU                         */
-  int32_t variant;        /* 0 = from the shape; 1, 2, 4 = 16-row fragments per pass  */
+  int32_t variant;        /* 0 = from the shape; 1, 2, 4 = 16-row fragments per pass of the
+                             streaming kernel; 8 = the 128-row tile kernel (prefill)  */
   int32_t w_layout;       /* KMOE_W_TILED                                             */
   int32_t act_dtype;      /* KMOE_DT_BF16, or KMOE_DT_F16: a, w_scale and y are IEEE half and the
                              weight values are half((code - 8) * scale), what
@@ -353,9 +354,13 @@ typedef struct kmoe_gemm_w4_args {
  * entry point reads the packed weights once and unpacks them in registers:
  *   y[r,c] = bf16( sum_k float(a[src(r),k]) * float(bf16((code[e,c,k] - 8) * scale[e,c,k/group])) )
  * i.e. the bf16 grouped GEMM on the weights kmoe_dequant_w4_bf16 would produce, with
- * f32 accumulation on MFMA (compare within tolerance). Made for the decode regime
- * (an expert with more rows than one pass holds streams its weights again).
- * Limits: k % 128 == 0, n % 16 == 0 (SwiGLU: n % 32 == 0), tiled weights.
+ * f32 accumulation on MFMA (compare within tolerance). Two kernels: a weight-streaming
+ * one for the decode regime (an expert with more rows than one pass holds streams its
+ * weights again) and, from two dozen rows per expert, one on 128-row tiles that shares
+ * the unpacking of a weight among the tile's rows; both sum in the same order and give
+ * the same bits.
+ * Limits: k % 128 == 0, n % 16 == 0 (SwiGLU: n % 32 == 0), tiled weights; the tile
+ * kernel needs rows * lda * 2 < 4 GiB (else the streaming kernel serves every size).
  */
 int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* args, kmoe_stream_t stream);
 

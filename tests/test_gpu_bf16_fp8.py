@@ -471,16 +471,19 @@ W4_CASES = [
     (16, 1536, 256, [(5 * i) % 11 for i in range(16)], 128),
     (3, 96, 384, [5, 40, 7], 96),      # a group of 3 x 32 values: the group index is a division, not a shift
     (2, 64, 4224, [5, 20], 32),        # 132 groups per channel: too many for the LDS copy, scales read from memory
+    (3, 96, 384, [130, 0, 260], 128),  # experts of two and three 128-row tiles, an empty one between them
+    (5, 320, 256, [128, 1, 0, 129, 64], 64),  # tiles that end exactly at an expert's last row, and one row past it
 ]
 
 
 @pytest.mark.parametrize("E,n,k,counts,gs", W4_CASES)
-@pytest.mark.parametrize("variant", [0, 1, 2, 4])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 8])
 @pytest.mark.parametrize("act", [0, 1])
 @pytest.mark.parametrize("gather", [False, True])
 def test_grouped_gemm_w4a16(L, E, n, k, counts, gs, variant, act, gather):
-    """Packed 4-bit weights streamed and unpacked in registers against the oracle's route: unpack
-    (orc_dequant_w4_bf16, itself pinned by a brute-force check) then the bf16 grouped GEMM."""
+    """Packed 4-bit weights unpacked in registers (variants 1, 2, 4: the streaming kernel; 8: the 128-row tile
+    kernel; 0: chosen from the rows per expert) against the oracle's route: unpack (orc_dequant_w4_bf16, itself
+    pinned by a brute-force check) then the bf16 grouped GEMM."""
     g = torch.Generator().manual_seed(E * n + k + (gs or 0))
     lod = _lod(counts)
     rows = int(lod[-1])
@@ -510,6 +513,12 @@ def test_grouped_gemm_w4a16(L, E, n, k, counts, gs, variant, act, gather):
     L.check(L.lib.kmoe_grouped_gemm_w4a16(args, L.stream()))
     torch.cuda.synchronize()
     assert rel_l2(y, from_bits(ref)) <= 2e-3   # the operands are the same bits: only summation order differs
+    if variant == 8:  # both kernels add the same products in the same order: the same bits
+        y1 = torch.zeros_like(y)
+        args.y, args.variant = y1.data_ptr(), 1
+        L.check(L.lib.kmoe_grouped_gemm_w4a16(args, L.stream()))
+        torch.cuda.synchronize()
+        assert torch.equal(y, y1)
     # an independent torch statement of the unpacking and of one expert's product
     e = int(np.argmax(counts))
     r0, r1 = int(lod[e]), int(lod[e + 1])
@@ -539,12 +548,12 @@ def test_grouped_gemm_w4a16_rejects_what_it_cannot_run(L):
         L.check(L.lib.kmoe_grouped_gemm_w4a16(args, L.stream()))
 
 
-@pytest.mark.parametrize("native", ["auto", "only"])
+@pytest.mark.parametrize("native", ["auto", "both", "only"])
 @pytest.mark.parametrize("group_size,M", [(128, 24), (32, 5), (None, 24), (128, 700)])
 def test_w4a16_layer_on_the_packed_weights(native, group_size, M):
-    """The 4-bit method with shapes the packed-weight kernel takes: decode-sized batches run
-    kmoe_moe_forward with KMOE_FMT_W4A16, large ones the unpacked copy ("auto") or the packed
-    weights again ("only"); both against the C oracle on the unpacked weights."""
+    """The 4-bit method with shapes the packed-weight kernels take: kmoe_moe_forward with KMOE_FMT_W4A16
+    (decode-sized batches on the streaming kernel, 700 tokens = 175 rows per expert on the tile kernel; with
+    "both" that batch runs on the unpacked copy); against the C oracle on the unpacked weights."""
     from vllm_kunlun_amd.ops.fused_moe.layer import FusedMoE
     from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors_moe import (
         KunlunCompressedTensorsWNA16MoEMethod)
@@ -565,7 +574,7 @@ def test_w4a16_layer_on_the_packed_weights(native, group_size, M):
     packed2, scale2 = layer.w2_weight_packed.data.cpu(), layer.w2_weight_scale.data.cpu()
     method.process_weights_after_loading(layer)
     assert layer.w4_native and hasattr(layer, "w13_weight_packed")
-    assert hasattr(layer, "w13_weight") == (native == "auto")
+    assert hasattr(layer, "w13_weight") == (native == "both")
     gx = torch.Generator(device="cuda").manual_seed(3)
     x = torch.randn(M, H, generator=gx, device="cuda").bfloat16()
     logits = torch.randn(M, E, generator=gx, device="cuda")

@@ -273,11 +273,12 @@ W4_HALF_CASES = [
     (8, 256, 1024, [4, 4, 0, 9, 33, 1, 0, 2], 64),
     (2, 128, 512, [70, 3], None),
     (16, 1536, 256, [(5 * i) % 11 for i in range(16)], 128),
+    (3, 96, 384, [130, 0, 260], 128),
 ]
 
 
 @pytest.mark.parametrize("E,n,k,counts,gs", W4_HALF_CASES)
-@pytest.mark.parametrize("variant", [0, 1, 2, 4])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 8])
 @pytest.mark.parametrize("act", [0, 1])
 def test_w4_half_dequant_and_gemm(E, n, k, counts, gs, variant, act):
     """kmoe_dequant_w4 in half mode: the oracle's bits (= the reference's float16 expression). The packed-weight
@@ -314,12 +315,13 @@ def test_w4_half_dequant_and_gemm(E, n, k, counts, gs, variant, act):
     assert rel_l2(y, from_hbits(ref)) <= 3e-4
 
 
-@pytest.mark.parametrize("native", ["auto", "only", False])
+@pytest.mark.parametrize("native", ["auto", "both", "only", False])
 @pytest.mark.parametrize("group_size,M", [(128, 24), (32, 5), (None, 24), (128, 700)])
 def test_w4_half_layer(native, group_size, M):
     """The 4-bit method created with params_dtype float16 (the reference's deployment dtype): half scales, half
-    activations; packed weights for small batches, the copy unpacked once for large ones; against the oracle's
-    half unquantized layer on the weights its half unpacking gives."""
+    activations; on the packed weights (streaming kernel for the small batches, tile kernel for 700 tokens) or, with
+    "both" from 160 rows per expert and with False always, on the copy unpacked once; against the oracle's half
+    unquantized layer on the weights its half unpacking gives."""
     from types import SimpleNamespace
     from vllm_kunlun_amd.ops.fused_moe.layer import FusedMoE
     from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors_moe import (
@@ -341,7 +343,8 @@ def test_w4_half_layer(native, group_size, M):
     packed13, scale13 = layer.w13_weight_packed.data.cpu(), layer.w13_weight_scale.data.cpu()
     packed2, scale2 = layer.w2_weight_packed.data.cpu(), layer.w2_weight_scale.data.cpu()
     method.process_weights_after_loading(layer)
-    if native != "only":
+    assert hasattr(layer, "w13_weight") == (native in ("both", False))
+    if native in ("both", False):
         assert layer.w13_weight.dtype == torch.float16
     gx = torch.Generator(device="cuda").manual_seed(3)
     x = torch.randn(M, H, generator=gx, device="cuda").half()

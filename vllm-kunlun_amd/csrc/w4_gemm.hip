@@ -1,7 +1,8 @@
-// Weight-streaming grouped GEMM on 4-bit weights and bf16 activations (W4A16) for the decode
-// regime: the packed weights are read from HBM once, unpacked in registers and fed to
-// v_mfma_f32_16x16x32_bf16. A quarter of the bytes of the bf16 path; the unpacking (23 VALU
-// instructions per 8 weights) is what bounds the kernel once the bytes are that few.
+// Grouped GEMM on 4-bit weights and bf16 activations (W4A16): a weight-streaming kernel for the
+// decode regime and a kernel on 128-row tiles for the prefill regime (further down). In both the
+// packed weights are unpacked in registers and fed to v_mfma_f32_16x16x32_bf16: a quarter of the
+// bytes of the bf16 path; the unpacking (23 VALU instructions per 8 weights) is what bounds the
+// streaming kernel once the bytes are that few, and what the tile kernel shares among 128 rows.
 //
 //   weights  [E][n][k/2] bytes, two codes per byte, low nibble first, code c means c - 8
 //            (dequant_int4_native, quantization/kernels/quant_ops.py:71-86), re-arranged by
@@ -21,6 +22,9 @@
 //            arithmetic: the code is OR-ed into the mantissa of 1024.0h (whose last place
 //            counts ones), 1032 is subtracted exactly and one packed multiply rounds the
 //            product - the reference's own two steps, two values per instruction.
+#include <type_traits>
+
+#include "buffer_ops.h"
 #include "kmoe_common.h"
 
 namespace kmoe {
@@ -243,6 +247,272 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
   }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Prefill regime: 128-row tiles. The unpacking of a weight word is shared by the 8 row fragments of the
+// tile (23 VALU instructions against 8 MFMAs of 16 cycles), so the kernel is bound by the matrix cores
+// like the 16-bit tile kernels while it reads a quarter of their weight bytes. One workgroup: 128 sorted
+// rows of one expert x 4 waves x NF fragments of 16 channels. Activations are copied global -> LDS
+// asynchronously, one 128-value block of K (256 bytes per row) ahead, two buffers; every wave reads its A
+// fragments from there. Weights and their scales go global -> registers, one block ahead; they never pass
+// through LDS.
+
+// m-tile number t when every expert's rows are cut into tiles of kTileRows: expert and first row (false: past the last tile)
+template <int kTileRows>
+__device__ inline bool locate_w4_tile(const W4Params& p, int t, int& e_out, int& row0_out) {
+  const int lane = lane_id();
+  const int epl = (p.E + kWave - 1) / kWave;  // experts per lane
+  const int e_begin = lane * epl;
+  int local = 0;
+  for (int i = 0; i < epl; ++i) {
+    const int e = e_begin + i;
+    if (e < p.E) local += (p.lod[e + 1] - p.lod[e] + kTileRows - 1) / kTileRows;
+  }
+  int incl = local;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int o = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += o;
+  }
+  if (t >= __shfl(incl, kWave - 1, kWave)) return false;
+  int excl = incl - local;
+  int found_e = -1, found_row = 0;
+  if (t >= excl && t < incl) {
+    for (int i = 0; i < epl; ++i) {
+      const int e = e_begin + i;
+      if (e >= p.E) break;
+      const int lo = p.lod[e];
+      const int tiles = (p.lod[e + 1] - lo + kTileRows - 1) / kTileRows;
+      if (t < excl + tiles) {
+        found_e = e;
+        found_row = lo + (t - excl) * kTileRows;
+        break;
+      }
+      excl += tiles;
+    }
+  }
+  const int src_lane = __builtin_ctzll(__ballot(found_e >= 0));
+  e_out = __shfl(found_e, src_lane, kWave);
+  row0_out = __shfl(found_row, src_lane, kWave);
+  return true;
+}
+
+// MF: 16-row fragments of a tile (8: 128-row tiles). 64-row tiles were measured and are not instantiated: a launch
+// whose experts hold a few dozen rows is bound by the unpacking and by the latency of its one-block-deep pipeline,
+// which a shorter tile does not change (Qwen3 shape, 4 to 64 rows per expert: 121 us against 111 us).
+template <int MF, int NF, bool SWIGLU, bool F16, bool SLDS>
+__global__ __launch_bounds__(kWaves* kWave, MF == 8 ? 2 : 3) void w4_tile_kernel(const W4Params p) {
+  constexpr int kTileRows = 16 * MF;
+  extern __shared__ uint16_t scale_lds[];  // SLDS: [kWaves][NF][16][groups], every wave its own part (as in the streaming kernel)
+  constexpr int NFH = SWIGLU ? NF / 2 : NF;
+  constexpr int NA = kTileRows / 4 / kWaves;  // asynchronous copies per wave and block: 4 rows (1 KB) each
+  constexpr int kWaveRows = 4 * NA;           // tile rows a wave copies
+  constexpr int kBufBytes = kTileRows * 256;
+  // Row r of a block sits at r * 256; its 16-byte vector v at position v ^ (r % 16): the 16 rows of a
+  // fragment read (same vector, rows r, r + 1, ...) fall on 16 different bank groups without padding, which
+  // the asynchronous copies (1 KB of consecutive LDS bytes per instruction) could not write.
+  __shared__ __attribute__((aligned(1024))) int8_t lds_a[2][kBufBytes];
+  const int lane = lane_id();
+  const int wave = threadIdx.x >> 6;
+  const int li = lane & 15;
+  const int lg = lane >> 4;
+  int e, row0;
+  if (!locate_w4_tile<kTileRows>(p, blockIdx.y, e, row0)) return;
+  const int row_end = min(p.lod[e + 1], row0 + kTileRows);
+  const int n_half = SWIGLU ? p.n / 2 : p.n;
+  const int col_base = (blockIdx.x * kWaves + wave) * NFH * 16;
+  const int kblocks = p.k / 128;
+  const int groups = p.k / p.gs;
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(p.a);
+  const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(p.w + static_cast<size_t>(e) * p.n * (p.k / 2));
+  const __amdgpu_buffer_rsrc_t s_rsrc = make_rsrc(p.scale + static_cast<size_t>(e) * p.n * groups);
+  auto group_of = [&](int kb) { return p.gs_shift >= 0 ? (4 * kb + lg) >> p.gs_shift : (4 * kb + lg) / (p.gs / 32); };
+
+  uint32_t woff[NF], soff[NF];
+  bool wok[NF];
+  int col[NF];
+#pragma unroll
+  for (int f = 0; f < NF; ++f) {
+    const int fh = SWIGLU ? f % NFH : f;
+    const int c = col_base + fh * 16;
+    wok[f] = c < n_half;
+    col[f] = (SWIGLU && f >= NFH) ? n_half + c : c;
+    const int ch0 = wok[f] ? col[f] : 0;  // fragments past the last channel read fragment 0: never stored
+    woff[f] = static_cast<uint32_t>(ch0 / 16) * kblocks * 1024u + lane * 16u;
+    soff[f] = static_cast<uint32_t>(ch0 + li) * groups * 2u;
+    if constexpr (SLDS) {
+      uint16_t* mine = scale_lds + (wave * NF + f) * 16 * groups;
+      uint32_t* dst = reinterpret_cast<uint32_t*>(mine);
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(p.scale + (static_cast<size_t>(e) * p.n + ch0) * groups);
+      for (int i = lane; i < 8 * groups; i += kWave) dst[i] = src[i];
+      soff[f] = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)(mine + li * groups)));  // LDS byte address of the lane's channel row
+    }
+  }
+  if constexpr (SLDS) __builtin_amdgcn_wave_barrier();  // the copies above stay above the reads below (a wave's LDS accesses complete in order)
+  // copy i of this wave fills tile rows kWaveRows wave + 4 i + lane / 16; the lane fetches the vector that belongs at its position
+  uint32_t aoff[NA];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    const int tr = kWaveRows * wave + 4 * i + lg;
+    const int r = row0 + tr;
+    const int rr = r < row_end ? r : row0;  // rows past the end read the tile's first row: never stored
+    const int src = p.row_src ? p.row_src[rr] / p.src_div : rr;
+    aoff[i] = static_cast<uint32_t>(src) * static_cast<uint32_t>(p.lda * 2) + ((li ^ (tr & 15)) << 4);  // < 4 GiB: host-checked
+  }
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)&lds_a[0][0]));
+  // fragment reads of MFMA step t: row li (+ 16 per fragment: same row % 16), vector 4 lg + t
+  uint32_t fa[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) fa[t] = lds_base + li * 256 + (((4 * lg + t) ^ li) << 4);
+  v4f acc[MF][NF];
+#pragma unroll
+  for (int mf = 0; mf < MF; ++mf)
+#pragma unroll
+    for (int f = 0; f < NF; ++f) acc[mf][f] = (v4f){0.f, 0.f, 0.f, 0.f};
+  v4i wbuf[2][NF];
+  uint16_t sbuf[2][NF];
+  auto load_w = [&](v4i(&w)[NF], uint16_t(&sc)[NF], int kb) {
+    const uint32_t g2 = static_cast<uint32_t>(group_of(kb)) * 2u;
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+      w[f] = buffer_load16(w_rsrc, woff[f], static_cast<uint32_t>(kb) * 1024u);
+      if constexpr (!SLDS) sc[f] = static_cast<uint16_t>(__builtin_amdgcn_raw_buffer_load_b16(s_rsrc, soff[f] + g2, 0, 0));
+    }
+    if constexpr (SLDS) {
+      // reads the compiler does not see (it would drain the asynchronous copies in flight before them); the wait is
+      // part of the statement, so the values are there when it ends
+      static_assert(NF == 4, "four scale reads per block");
+      uint32_t s0, s1, s2, s3;
+      asm volatile(
+          "ds_read_u16 %0, %4\n\t"
+          "ds_read_u16 %1, %5\n\t"
+          "ds_read_u16 %2, %6\n\t"
+          "ds_read_u16 %3, %7\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          : "=&v"(s0), "=&v"(s1), "=&v"(s2), "=&v"(s3)
+          : "v"(soff[0] + g2), "v"(soff[1] + g2), "v"(soff[2] + g2), "v"(soff[3] + g2)
+          : "memory");
+      sc[0] = static_cast<uint16_t>(s0);
+      sc[1] = static_cast<uint16_t>(s1);
+      sc[2] = static_cast<uint16_t>(s2);
+      sc[3] = static_cast<uint16_t>(s3);
+    }
+  };
+  auto dma_a = [&](int kb, int buf) {
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+      buffer_load16_to_lds(a_rsrc, (lds_ptr_t)&lds_a[buf][(kWaveRows * wave + 4 * i) * 256], aoff[i], static_cast<uint32_t>(kb) * 256u);
+  };
+  // one block: word t of a lane's 16 packed bytes is its operand of MFMA step t; the activation lane (lg, row)
+  // supplies values 32 lg + 8 t + [0, 8) of the block, i.e. vector 4 lg + t of the row's 16
+  auto compute = [&](const v4i(&w)[NF], const uint16_t(&sc)[NF], auto buf_tag) {
+    constexpr int buf = decltype(buf_tag)::value;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      v4i wv[NF];
+#pragma unroll
+      for (int f = 0; f < NF; ++f) {
+        if constexpr (F16) {
+          const _Float16 sh = __builtin_bit_cast(_Float16, sc[f]);
+          wv[f] = unpack8_half(static_cast<uint32_t>(w[f][t]), (v2h){sh, sh});
+        } else {
+          const float s = bf16_to_f32(sc[f]);
+          wv[f] = unpack8(static_cast<uint32_t>(w[f][t]), s, -136.0f * s);
+        }
+      }
+      // two fragments in flight: the read of fragment mf + 1 leaves before the MFMAs of fragment mf
+      v4i af[2];
+      af[0] = lds_read16_raw<buf * kBufBytes>(fa[t]);
+#pragma unroll
+      for (int mf = 0; mf < MF; ++mf) {
+        if (mf + 1 < MF) {
+          asm volatile("ds_read_b128 %0, %1 offset:%2"
+                       : "=v"(af[(mf + 1) & 1])
+                       : "v"(fa[t]), "n"(buf * kBufBytes + (mf + 1) * 16 * 256)
+                       : "memory");
+          lds_wait<1>(af[mf & 1]);
+        } else {
+          lds_wait<0>(af[mf & 1]);
+        }
+#pragma unroll
+        for (int f = 0; f < NF; ++f) {
+          if constexpr (F16)
+            acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, wv[f]),
+                                                                __builtin_bit_cast(v8h, af[mf & 1]), acc[mf][f], 0, 0, 0);
+          else
+            acc[mf][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wv[f]),
+                                                                 __builtin_bit_cast(v8bf, af[mf & 1]), acc[mf][f], 0, 0, 0);
+        }
+      }
+    }
+  };
+  // The block after the current one is requested (weights and scales into registers, activations into the other
+  // LDS buffer, which every wave finished reading before the barrier that ended the previous stage) before the
+  // MFMAs of the current one; the wait at the end covers all of it, the barrier publishes the copies.
+  auto stage = [&](int kb, const v4i(&w)[NF], const uint16_t(&sc)[NF], v4i(&w_next)[NF], uint16_t(&sc_next)[NF], auto buf_tag) {
+    constexpr int buf = decltype(buf_tag)::value;
+    if (kb + 1 < kblocks) {
+      dma_a(kb + 1, buf ^ 1);
+      load_w(w_next, sc_next, kb + 1);
+    }
+    compute(w, sc, buf_tag);
+    vmem_wait<0>();
+    __syncthreads();
+  };
+  dma_a(0, 0);
+  load_w(wbuf[0], sbuf[0], 0);
+  vmem_wait<0>();
+  __syncthreads();
+  for (int kb = 0; kb < kblocks; kb += 2) {
+    stage(kb, wbuf[0], sbuf[0], wbuf[1], sbuf[1], std::integral_constant<int, 0>{});
+    if (kb + 1 < kblocks) stage(kb + 1, wbuf[1], sbuf[1], wbuf[0], sbuf[0], std::integral_constant<int, 1>{});
+  }
+
+  // epilogue: as the streaming kernel - round to the activation type, optional SiLU-mul on the rounded values
+#pragma unroll
+  for (int mf = 0; mf < MF; ++mf) {
+    const int r = row0 + mf * 16 + li;
+    if (r >= row_end) continue;
+#pragma unroll
+    for (int f = 0; f < NFH; ++f) {
+      if (!wok[f]) continue;
+      const int c0 = col[f] + lg * 4;
+      uint16_t yv[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) yv[q] = f32_to_act(acc[mf][f][q], F16);
+      if (SWIGLU) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          yv[q] = f32_to_act(silu_fixed(act_to_f32(yv[q], F16)) * act_to_f32(f32_to_act(acc[mf][f + NFH][q], F16), F16), F16);
+      }
+      const uint2 packed = make_uint2(yv[0] | (static_cast<uint32_t>(yv[1]) << 16),
+                                      yv[2] | (static_cast<uint32_t>(yv[3]) << 16));
+      *reinterpret_cast<uint2*>(p.y + static_cast<size_t>(r) * p.ldy + c0) = packed;
+    }
+  }
+}
+
+template <int MF, bool SWIGLU>
+int launch_w4_tile(const W4Params& p, int rows, bool f16, hipStream_t s) {
+  constexpr int NF = 4;
+  constexpr int kTileRows = 16 * MF;
+  constexpr int NFH = SWIGLU ? NF / 2 : NF;
+  const int n_half = SWIGLU ? p.n / 2 : p.n;
+  const dim3 grid(ceil_div(n_half, kWaves * NFH * 16), rows / kTileRows + min(p.E, rows));  // upper bound of the m-tiles
+  // the scales of a wave's fragments in LDS, while two workgroups still fit a CU next to their activation buffers
+  const size_t lds = static_cast<size_t>(kWaves) * NF * 16 * (p.k / p.gs) * sizeof(uint16_t);
+  if (lds <= 16 * 1024) {
+    if (f16)
+      hipLaunchKernelGGL((w4_tile_kernel<MF, NF, SWIGLU, true, true>), grid, dim3(kWaves * kWave), lds, s, p);
+    else
+      hipLaunchKernelGGL((w4_tile_kernel<MF, NF, SWIGLU, false, true>), grid, dim3(kWaves * kWave), lds, s, p);
+  } else if (f16) {
+    hipLaunchKernelGGL((w4_tile_kernel<MF, NF, SWIGLU, true, false>), grid, dim3(kWaves * kWave), 0, s, p);
+  } else {
+    hipLaunchKernelGGL((w4_tile_kernel<MF, NF, SWIGLU, false, false>), grid, dim3(kWaves * kWave), 0, s, p);
+  }
+  return check_launch("kmoe_grouped_gemm_w4a16");
+}
+
 template <int MF, int NF, bool SWIGLU, int D>
 int launch_w4(const W4Params& p, bool f16, hipStream_t s) {
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
@@ -297,11 +567,16 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
                    a->E, a->n,   a->k,       a->y,       a->ldy};
   hipStream_t s = as_stream(stream);
   int mf = a->variant;
+  // the 128-row tile kernel reaches a source row (gathered or not: below `rows`) through a 32-bit byte offset
+  const bool tile_ok = static_cast<uint64_t>(a->rows) * static_cast<uint64_t>(a->lda) * 2u + static_cast<uint64_t>(a->k) * 2u < (1ull << 32);
   if (mf == 0) {
     // rows an expert gets under uniform routing, with headroom for the spread: an expert with
-    // more rows than one pass holds streams (and unpacks) its weights again
+    // more rows than one pass holds streams (and unpacks) its weights again. From two dozen rows per expert
+    // the 128-row tile kernel is ahead, although most of its tile is padding there (Qwen3 shape, gate_up / down:
+    // 16 rows per expert 87 / 50 us streaming against 106 / 58 us, 24 rows 107 / 58 against 109 / 58, 32 rows
+    // 141 / 76 against 109 / 60, 128 rows 462 / 212 against 186 / 102).
     const int avg = ceil_div(a->rows, a->E);
-    mf = avg <= 10 ? 1 : (avg <= 22 ? 2 : 4);
+    mf = avg <= 10 ? 1 : (avg <= 22 ? 2 : (tile_ok ? 8 : 4));
   }
   switch (mf) {
     // One block in flight per wave: the registers that saves put more waves on a SIMD (5-6 instead of 3-4), and
@@ -316,7 +591,11 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
     case 143: return swiglu ? launch_w4<1, 4, true, 3>(p, f16, s) : launch_w4<1, 4, false, 3>(p, f16, s);
     case 2: return swiglu ? launch_w4<2, 2, true, 2>(p, f16, s) : launch_w4<2, 2, false, 2>(p, f16, s);
     case 4: return swiglu ? launch_w4<4, 2, true, 2>(p, f16, s) : launch_w4<4, 2, false, 2>(p, f16, s);
+    case 8:
+      KMOE_REQUIRE(tile_ok, KMOE_ERR_SHAPE, "grouped_gemm_w4a16: the tile kernel addresses the activations with 32 bits (rows=%d lda=%lld)",
+                   a->rows, static_cast<long long>(a->lda));
+      return swiglu ? launch_w4_tile<8, true>(p, a->rows, f16, s) : launch_w4_tile<8, false>(p, a->rows, f16, s);
     default:
-      return fail(KMOE_ERR_UNSUPPORTED, "grouped_gemm_w4a16: variant=%d must be 0, 1, 2 or 4 (or a tuning variant)", a->variant);
+      return fail(KMOE_ERR_UNSUPPORTED, "grouped_gemm_w4a16: variant=%d must be 0, 1, 2, 4 or 8 (or a tuning variant)", a->variant);
   }
 }

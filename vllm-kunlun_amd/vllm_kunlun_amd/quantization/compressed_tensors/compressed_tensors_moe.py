@@ -314,13 +314,17 @@ class KunlunCompressedTensorsWNA16MoEMethod:
     """4-bit weight-only MoE (reference: compressed_tensors_moe.py:294-360). The reference
     unpacks the whole packed weight tensors to fp16 inside EVERY apply() (:320-327) and then
     calls the unquantized fused_moe. Here, in process_weights_after_loading:
-      * the packed tensors are tiled in place and kept for kmoe_grouped_gemm_w4a16, which reads
-        them once per call and unpacks in registers: the path for decode-sized batches
-        (`native` = "auto" or "only"; needs hidden and intermediate sizes that are multiples of
-        128 and a group size that is a multiple of 32);
-      * the weights are unpacked ONCE (kmoe_dequant_w4) to tiled 16-bit tensors for batches with
-        many rows per expert (`native` = "auto" or False). "auto" keeps both copies (1.25x the
-        16-bit bytes); "only" keeps the packed one and serves every batch from it.
+      * the packed tensors are tiled in place and kept for kmoe_grouped_gemm_w4a16, which unpacks in
+        registers (a weight-streaming kernel for decode-sized batches, a kernel on 128-row tiles beyond;
+        needs hidden and intermediate sizes that are multiples of 128 and a group size that is a multiple
+        of 32);
+      * or the weights are unpacked ONCE (kmoe_dequant_w4) to tiled 16-bit tensors for the unquantized path.
+    `native` chooses: "auto" (default) keeps the packed tensors alone where the kernels take the shapes (a
+    quarter of the 16-bit bytes; measured on the Qwen3-30B-A3B shape against the 16-bit copy: 0.10 against
+    0.22 ms at 128 tokens, 0.20 against 0.26 ms at 1024, 0.49 against 0.45 ms at 4096, 0.87 against 0.76 ms at
+    8192) and the 16-bit copy alone elsewhere; "both" keeps both (1.25x the 16-bit bytes) and takes the faster
+    one per batch; "only" is "auto" that refuses shapes the packed kernels do not take; False never uses the
+    packed kernels.
     The 16-bit type is the one of the scales: float16 scales (a model loaded with --dtype float16, the
     reference's recipes) give half((code - 8) * scale), exactly what dequant_int4_native computes, and the
     layer then takes float16 activations; any other scale dtype is taken as bfloat16.
@@ -328,10 +332,10 @@ class KunlunCompressedTensorsWNA16MoEMethod:
     two codes per byte, low nibble first, code - 8; scales per contiguous group of `group_size`
     along k, or one per row."""
 
-    # rows per expert up to which the packed weights are streamed (above: the unpacked copy). The packed
-    # kernel unpacks every weight once per 16-64 rows, so its time grows with the rows; the tiled bf16 GEMM's
-    # hardly does. Measured cross-over on the Qwen3-30B-A3B shape: 22 rows per expert (about 360 tokens).
-    NATIVE_MAX_ROWS_PER_EXPERT = 20
+    # native="both": rows per expert up to which the packed weights are used (above: the unpacked copy). Measured
+    # cross-over on the Qwen3-30B-A3B shape: between 2048 tokens (128 rows per expert: 0.31 against 0.33 ms) and
+    # 4096 (256 rows: 0.49 against 0.45 ms).
+    NATIVE_MAX_ROWS_PER_EXPERT = 160
 
     def __init__(self, weight_quant=None, input_quant=None, moe=None, native="auto"):
         self.weight_quant = weight_quant
@@ -339,8 +343,8 @@ class KunlunCompressedTensorsWNA16MoEMethod:
         self.moe = moe
         gs = _get(weight_quant, "group_size") if weight_quant is not None else None
         self.group_size = int(gs) if (gs and _strategy(weight_quant) == "group") else None  # None: one scale per row
-        if native not in ("auto", "only", False):
-            raise ValueError("native must be 'auto', 'only' or False")
+        if native not in ("auto", "both", "only", False):
+            raise ValueError("native must be 'auto', 'both', 'only' or False")
         self.native = native
 
     @property
@@ -375,7 +379,7 @@ class KunlunCompressedTensorsWNA16MoEMethod:
             if self.native == "only" and not native:
                 raise ValueError("native='only' needs CUDA tensors, H and I multiples of 128 and one group size "
                                  "(a multiple of 32) for both weight tensors")
-            keep_bf16 = self.native != "only"
+            keep_bf16 = self.native == "both" or not native
             for name in ("w13", "w2"):
                 packed = getattr(layer, f"{name}_weight_packed").data.contiguous()
                 scale = getattr(layer, f"{name}_weight_scale").data
@@ -411,8 +415,8 @@ class KunlunCompressedTensorsWNA16MoEMethod:
                     e_score_correction_bias=getattr(layer, "e_score_correction_bias", None))
 
     def apply_monolithic(self, layer, x: torch.Tensor, router_logits: torch.Tensor, **kwargs):
-        """Activations in the dtype of the scales (bf16, or float16). Few rows per expert: the packed weights (kmoe_grouped_gemm_w4a16
-        inside kmoe_moe_forward). Otherwise the unpacked weights through KunlunOps.fused_moe, as
+        """Activations in the dtype of the scales (bf16, or float16). On the packed weights:
+        kmoe_grouped_gemm_w4a16 inside kmoe_moe_forward. On the unpacked copy: KunlunOps.fused_moe, as
         the reference's apply() ends (:343-360). Routing as in KunlunOps.fused_moe (always
         normalised, sigmoid scale 1.0)."""
         top_k = self.moe.experts_per_token
@@ -420,7 +424,7 @@ class KunlunCompressedTensorsWNA16MoEMethod:
         rows_per_expert = -(-x.shape[0] * top_k // E)
         has_bias = getattr(layer, "w13_bias", None) is not None or getattr(layer, "w2_bias", None) is not None
         use_native = getattr(layer, "w4_native", False) and not has_bias and (
-            self.native == "only" or rows_per_expert <= self.NATIVE_MAX_ROWS_PER_EXPERT)
+            self.native != "both" or rows_per_expert <= self.NATIVE_MAX_ROWS_PER_EXPERT)
         if use_native:
             if x.dtype != layer.w13_weight_scale.dtype:
                 raise ValueError(f"4-bit MoE: activations ({x.dtype}) must have the dtype of the scales "

@@ -221,7 +221,7 @@ def make_bf16_layer(shape: MoEShape, device="cuda", seed: int = 0, dtype: torch.
 
 
 def make_w4_layer(shape: MoEShape, device="cuda", seed: int = 0, dtype: torch.dtype = torch.bfloat16) -> SynthLayer:
-    """FusedMoE with the 4-bit method (packed weights kept, native="only"): weights ~ N(0, 0.02)
+    """FusedMoE with the 4-bit method (packed weights alone, native="only"): weights ~ N(0, 0.02)
     quantised per group of `group_size` values to codes 0..15 (value = (code - 8) * scale)."""
     from types import SimpleNamespace
     from .quantization.compressed_tensors.compressed_tensors_moe import KunlunCompressedTensorsWNA16MoEMethod

@@ -45,6 +45,8 @@ WORKLOAD_LABEL = {
     "qwen3-bf16-prefill": "Qwen3-MoE-30B-A3B-shape MoE layer, bf16 weights (no quantization), prefill, 8192 tokens",
     "qwen3-w4a16-decode": "Qwen3-MoE-30B-A3B-shape MoE layer, 4-bit weights (groups of 128) and bf16 activations, "
                           "decode, 64 tokens",
+    "qwen3-w4a16-prefill": "Qwen3-MoE-30B-A3B-shape MoE layer, 4-bit weights (groups of 128) and bf16 activations, "
+                           "prefill, 8192 tokens",
     "tiny-bf16": "tiny bf16 MoE layer (32 tokens, hidden 512, 8 experts, top-2, intermediate 256), no quantization",
 }
 PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0, "none": 2500.0, "w4": 2500.0}  # MI355X dense MFMA: int8, fp8, bf16
@@ -290,7 +292,7 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
         roofline = {"bound": "mfma", "achieved": achieved, "peak": peak_tops, "unit": "TFLOP/s",
                     "frac": achieved / peak_tops, "traffic": traffic}
     many_rows = shape.P > 10 * shape.E  # the launchers' switch to the persistent tile kernel
-    g1_kernel = ("w4_stream_kernel" if w4 else "stream_gemm_i8_kernel" if plan.layout.codes_chunked else
+    g1_kernel = (("w4_tile_kernel" if shape.P > 22 * shape.E else "w4_stream_kernel") if w4 else "stream_gemm_i8_kernel" if plan.layout.codes_chunked else
                  "tiled_gemm_kernel" if many_rows and plan.args.w_layout == L.KMOE_W_TILED else "grouped_gemm_kernel")
     roofline.update(kernel=g1_kernel + " (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
                     algorithmic_bytes=work["g1_bytes"], algorithmic_ops=work["g1_ops"],

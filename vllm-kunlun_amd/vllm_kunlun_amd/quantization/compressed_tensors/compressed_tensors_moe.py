@@ -321,7 +321,7 @@ class KunlunCompressedTensorsWNA16MoEMethod:
       * or the weights are unpacked ONCE (kmoe_dequant_w4) to tiled 16-bit tensors for the unquantized path.
     `native` chooses: "auto" (default) keeps the packed tensors alone where the kernels take the shapes (a
     quarter of the 16-bit bytes; measured on the Qwen3-30B-A3B shape against the 16-bit copy: 0.10 against
-    0.22 ms at 128 tokens, 0.20 against 0.26 ms at 1024, 0.49 against 0.45 ms at 4096, 0.87 against 0.76 ms at
+    0.22 ms at 128 tokens, 0.21 against 0.26 ms at 1024, 0.50 against 0.45 ms at 4096, 0.86 against 0.76 ms at
     8192) and the 16-bit copy alone elsewhere; "both" keeps both (1.25x the 16-bit bytes) and takes the faster
     one per batch; "only" is "auto" that refuses shapes the packed kernels do not take; False never uses the
     packed kernels.
@@ -333,8 +333,8 @@ class KunlunCompressedTensorsWNA16MoEMethod:
     along k, or one per row."""
 
     # native="both": rows per expert up to which the packed weights are used (above: the unpacked copy). Measured
-    # cross-over on the Qwen3-30B-A3B shape: between 2048 tokens (128 rows per expert: 0.31 against 0.33 ms) and
-    # 4096 (256 rows: 0.49 against 0.45 ms).
+    # cross-over on the Qwen3-30B-A3B shape: between 2048 tokens (128 rows per expert: 0.33 against 0.33 ms) and
+    # 4096 (256 rows: 0.50 against 0.45 ms).
     NATIVE_MAX_ROWS_PER_EXPERT = 160
 
     def __init__(self, weight_quant=None, input_quant=None, moe=None, native="auto"):

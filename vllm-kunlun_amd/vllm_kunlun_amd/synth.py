@@ -63,8 +63,9 @@ for _n in ("qwen3-decode", "qwen3-prefill"):
     SHAPES[_f] = replace(SHAPES[_n], name=_f, quant="none")
 
 
-# ... and with 4-bit weights (group scales of 128 values) on the packed-weight decode path
+# ... and with 4-bit weights (group scales of 128 values) on the packed-weight paths
 SHAPES["qwen3-w4a16-decode"] = replace(SHAPES["qwen3-decode"], name="qwen3-w4a16-decode", quant="w4")
+SHAPES["qwen3-w4a16-prefill"] = replace(SHAPES["qwen3-prefill"], name="qwen3-w4a16-prefill", quant="w4")
 
 
 def make_layer(shape: MoEShape, device="cuda", seed: int = 0, dtype: torch.dtype = torch.bfloat16) -> "SynthLayer":

@@ -226,6 +226,9 @@ typedef struct kmoe_gemm_i8_args {
 
 #define KMOE_W_ROWMAJOR 0
 #define KMOE_W_TILED 1
+/* layouts of the group scales of packed 4-bit weights (kmoe_gemm_w4_args.scale_layout) */
+#define KMOE_S_ROWMAJOR 0
+#define KMOE_S_FRAG16 1
 #define KMOE_A_ROWMAJOR 0
 #define KMOE_A_CHUNKED 1
 
@@ -345,6 +348,8 @@ typedef struct kmoe_gemm_w4_args {
   int32_t act_dtype;      /* KMOE_DT_BF16, or KMOE_DT_F16: a, w_scale and y are IEEE half and the
                              weight values are half((code - 8) * scale), what
                              dequant_int4_native (quant_ops.py:71-86) itself computes  */
+  int32_t scale_layout;   /* KMOE_S_ROWMAJOR: w_scale as the checkpoint holds it, [E, n, k/group_size];
+                             KMOE_S_FRAG16: re-arranged by kmoe_tile_scales_w4 (same bytes in total) */
 } kmoe_gemm_w4_args;
 
 /*
@@ -363,6 +368,16 @@ typedef struct kmoe_gemm_w4_args {
  * kernel needs rows * lda * 2 < 4 GiB (else the streaming kernel serves every size).
  */
 int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* args, kmoe_stream_t stream);
+
+/*
+ * Load-time re-arrangement of the group scales of packed 4-bit weights (no counterpart in the
+ * reference, whose closed kernels take the checkpoint layout): [E, n, groups] -> per 16 output
+ * channels [groups][16]. The scales one MFMA block needs (16 channels x the 1 to 4 groups the
+ * block's 128 values fall into) are then 32 to 128 consecutive bytes instead of 16 pieces a row
+ * apart: the form to hand to kmoe_grouped_gemm_w4a16 / kmoe_moe_forward where a channel has more
+ * scales than a workgroup can hold in LDS (long k, small groups). Not in place. n % 16 == 0.
+ */
+int kmoe_tile_scales_w4(const uint16_t* src, uint16_t* dst, int E, int n, int groups, kmoe_stream_t stream);
 
 /*
  * The gpt-oss activation on a stored, interleaved gate_up result. Replaces
@@ -515,6 +530,7 @@ typedef struct kmoe_moe_args {
                             out = dt( dt(routed * out_scale) + dt(shared * shared_scale) ); 0 means 1 */
   int32_t tile_variant;  /* INT8, tuning: 0, or the `variant` (5-12) handed to the two routed GEMMs when the batch
                             runs on the tile kernel (more than 10 rows per expert); ignored otherwise */
+  int32_t w_scale_layout; /* W4A16: KMOE_S_* of w13_scale and w2_scale                                  */
 } kmoe_moe_args;
 
 #define KMOE_STAGE_ROUTING 0

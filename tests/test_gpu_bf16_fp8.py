@@ -479,8 +479,8 @@ W4_CASES = [
 @pytest.mark.parametrize("E,n,k,counts,gs", W4_CASES)
 @pytest.mark.parametrize("variant", [0, 1, 2, 4, 8])
 @pytest.mark.parametrize("act", [0, 1])
-@pytest.mark.parametrize("gather", [False, True])
-def test_grouped_gemm_w4a16(L, E, n, k, counts, gs, variant, act, gather):
+@pytest.mark.parametrize("gather,frag16", [(False, False), (True, False), (True, True)])
+def test_grouped_gemm_w4a16(L, E, n, k, counts, gs, variant, act, gather, frag16):
     """Packed 4-bit weights unpacked in registers (variants 1, 2, 4: the streaming kernel; 8: the 128-row tile
     kernel; 0: chosen from the rows per expert) against the oracle's route: unpack (orc_dequant_w4_bf16, itself
     pinned by a brute-force check) then the bf16 grouped GEMM."""
@@ -502,9 +502,16 @@ def test_grouped_gemm_w4a16(L, E, n, k, counts, gs, variant, act, gather):
     dt = torch.empty_like(dp)
     L.check(L.lib.kmoe_tile_weights_i8(dp.data_ptr(), dt.data_ptr(), E, n, k // 2, L.stream()))
     da, ds, dl = a.cuda(), scale.cuda(), torch.from_numpy(lod).cuda()
+    if frag16:  # the scales re-arranged per 16 channels, as the layer keeps them
+        tiled = torch.empty_like(ds)
+        L.check(L.lib.kmoe_tile_scales_w4(ds.data_ptr(), tiled.data_ptr(), E, n, k // group, L.stream()))
+        want = ds.view(E, n // 16, 16, k // group).permute(0, 1, 3, 2).contiguous().view(E, n, k // group)
+        assert torch.equal(tiled, want)
+        ds = tiled
     dsrc = None if row_src is None else row_src.cuda()
     y = torch.zeros(rows, n_out, dtype=torch.bfloat16, device="cuda")
     args = L.GemmW4Args()
+    args.scale_layout = L.KMOE_S_FRAG16 if frag16 else L.KMOE_S_ROWMAJOR
     args.a, args.lda, args.src_div = da.data_ptr(), k, K if gather else 1
     args.row_src = 0 if dsrc is None else dsrc.data_ptr()
     args.w, args.w_scale, args.group_size, args.lod = dt.data_ptr(), ds.data_ptr(), group, dl.data_ptr()
@@ -529,6 +536,23 @@ def test_grouped_gemm_w4a16(L, E, n, k, counts, gs, variant, act, gather):
     if act:
         t = tm.silu_and_mul(t.bfloat16()).float()
     assert rel_l2(y[r0:r1], t) <= REL_L2_BF16
+
+
+def test_w4_scales_rearranged_in_place_and_back(L):
+    """tile_w4_scales_ re-arranges group scales in place and marks the memory; the mark follows the memory, a view
+    that cannot stand for it is refused, and rowmajor_w4_scales gives the checkpoint's values back."""
+    from vllm_kunlun_amd import _plan
+    g = torch.Generator().manual_seed(5)
+    scale = torch.rand(3, 96, 7, generator=g).bfloat16().cuda()
+    before = scale.clone()
+    assert _plan.scale_layout(scale) == L.KMOE_S_ROWMAJOR
+    assert _plan.tile_w4_scales_(scale) and _plan.tile_w4_scales_(scale)  # the second call finds the mark
+    assert _plan.scale_layout(scale) == L.KMOE_S_FRAG16 and _plan.scale_layout(scale[1:]) == L.KMOE_S_FRAG16
+    assert torch.equal(scale.view(3, 6, 7, 16), before.view(3, 6, 16, 7).transpose(2, 3))
+    assert torch.equal(_plan.rowmajor_w4_scales(scale), before)
+    with pytest.raises(ValueError):
+        _plan.scale_layout(scale[:, :16])
+    assert not _plan.tile_w4_scales_(torch.zeros(2, 24, 4, dtype=torch.bfloat16, device="cuda"))  # 24 channels
 
 
 def test_grouped_gemm_w4a16_rejects_what_it_cannot_run(L):

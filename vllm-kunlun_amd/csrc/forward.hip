@@ -132,7 +132,7 @@ struct MlpPass {
   float act_alpha, act_limit;
   // W4A16: group scales of the packed weights
   const uint16_t *w13_scale, *w2_scale;
-  int group_size;
+  int group_size, scale_layout;
   int variant;  // INT8: kernel variant of the two GEMMs (0: from the shape)
   int act_dtype;  // INT8, BF16: KMOE_DT_* of x_rows' source, act and out (BF16: of the weights too)
 };
@@ -218,6 +218,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.w = static_cast<const uint8_t*>(w);
     g.w_scale = first ? m.w13_scale : m.w2_scale;
     g.group_size = m.group_size;
+    g.scale_layout = m.scale_layout;
     g.lod = m.lod;
     g.E = m.E;
     g.n = n;
@@ -519,6 +520,7 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
   routed.w13_scale = a->w13_scale;
   routed.w2_scale = a->w2_scale;
   routed.group_size = a->group_size;
+  routed.scale_layout = a->w_scale_layout;
   routed.act_dtype = a->act_dtype;
   if (a->format == KMOE_FMT_BF16) {
     routed.w13_bias = a->w13_bias;

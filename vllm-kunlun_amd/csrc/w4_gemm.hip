@@ -45,6 +45,11 @@ struct W4Params {
   const uint16_t* scale;  // [E, n, k / gs] bf16
   int32_t gs;
   int32_t gs_shift;       // log2(gs / 32) when gs / 32 is a power of two, else -1
+  // Element strides inside the 16 x (k / gs) scales of a fragment (16 channels), which start at channel * (k / gs) in
+  // both layouts. KMOE_S_ROWMAJOR: channel k / gs, group 1. KMOE_S_FRAG16 (kmoe_tile_scales_w4): channel 1, group 16 -
+  // the scales a wave needs for one block are then 32 to 128 consecutive bytes: one cache line per load instruction
+  // where the row-major layout touches 16 (one per channel), and consecutive LDS banks in the wave's copy.
+  int32_t s_ch, s_g;
   const int32_t* lod;
   int32_t E, n, k;
   uint16_t* y;
@@ -138,13 +143,13 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
     col[f] = (SWIGLU && f >= NFH) ? n_half + c : c;
     const int ch0 = wok[f] ? col[f] : 0;  // fragments past the last channel read fragment 0: never stored
     wp[f] = w_base + static_cast<size_t>(ch0 / 16) * kblocks * 1024 + lane * 16;
-    sp[f] = s_base + static_cast<size_t>(ch0 + li) * groups;
+    sp[f] = s_base + static_cast<size_t>(ch0) * groups + li * p.s_ch;
     if constexpr (SLDS) {
       // the wave's own copy; it alone reads it, so no barrier: a wave's LDS accesses complete in order
       uint32_t* dst = reinterpret_cast<uint32_t*>(scale_lds + (wave * NF + f) * 16 * groups);
       const uint32_t* src = reinterpret_cast<const uint32_t*>(s_base + static_cast<size_t>(ch0) * groups);
       for (int i = lane; i < 8 * groups; i += kWave) dst[i] = src[i];
-      soff[f] = (wave * NF + f) * 16 * groups + li * groups;
+      soff[f] = (wave * NF + f) * 16 * groups + li * p.s_ch;
     }
   }
   if constexpr (SLDS) __builtin_amdgcn_wave_barrier();  // the copies above stay above the reads below
@@ -172,7 +177,7 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
 #pragma unroll
       for (int f = 0; f < NF; ++f) {
         wreg[slot][f] = *reinterpret_cast<const v4i*>(wp[f] + static_cast<size_t>(kb) * 1024);
-        if constexpr (!SLDS) sreg[slot][f] = sp[f][g];
+        if constexpr (!SLDS) sreg[slot][f] = sp[f][g * p.s_g];
       }
 #pragma unroll
       for (int mf = 0; mf < MF; ++mf)
@@ -190,7 +195,7 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
         if (kb < kblocks) {
 #pragma unroll
           for (int f = 0; f < NF; ++f) {
-            if constexpr (SLDS) sreg[d][f] = scale_lds[soff[f] + group_of(kb)];
+            if constexpr (SLDS) sreg[d][f] = scale_lds[soff[f] + group_of(kb) * p.s_g];
             if constexpr (F16) {
               const _Float16 sh = __builtin_bit_cast(_Float16, sreg[d][f]);
               const v2h s2 = {sh, sh};
@@ -349,13 +354,13 @@ __global__ __launch_bounds__(kWaves* kWave, MF == 8 ? 2 : 3) void w4_tile_kernel
     col[f] = (SWIGLU && f >= NFH) ? n_half + c : c;
     const int ch0 = wok[f] ? col[f] : 0;  // fragments past the last channel read fragment 0: never stored
     woff[f] = static_cast<uint32_t>(ch0 / 16) * kblocks * 1024u + lane * 16u;
-    soff[f] = static_cast<uint32_t>(ch0 + li) * groups * 2u;
+    soff[f] = (static_cast<uint32_t>(ch0) * groups + li * p.s_ch) * 2u;
     if constexpr (SLDS) {
       uint16_t* mine = scale_lds + (wave * NF + f) * 16 * groups;
       uint32_t* dst = reinterpret_cast<uint32_t*>(mine);
       const uint32_t* src = reinterpret_cast<const uint32_t*>(p.scale + (static_cast<size_t>(e) * p.n + ch0) * groups);
       for (int i = lane; i < 8 * groups; i += kWave) dst[i] = src[i];
-      soff[f] = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)(mine + li * groups)));  // LDS byte address of the lane's channel row
+      soff[f] = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)(mine + li * p.s_ch)));  // LDS byte address of the lane's channel
     }
   }
   if constexpr (SLDS) __builtin_amdgcn_wave_barrier();  // the copies above stay above the reads below (a wave's LDS accesses complete in order)
@@ -382,7 +387,7 @@ __global__ __launch_bounds__(kWaves* kWave, MF == 8 ? 2 : 3) void w4_tile_kernel
   v4i wbuf[2][NF];
   uint16_t sbuf[2][NF];
   auto load_w = [&](v4i(&w)[NF], uint16_t(&sc)[NF], int kb) {
-    const uint32_t g2 = static_cast<uint32_t>(group_of(kb)) * 2u;
+    const uint32_t g2 = static_cast<uint32_t>(group_of(kb) * p.s_g) * 2u;
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
       w[f] = buffer_load16(w_rsrc, woff[f], static_cast<uint32_t>(kb) * 1024u);
@@ -546,10 +551,30 @@ int launch_w4(const W4Params& p, bool f16, hipStream_t s) {
   return check_launch("kmoe_grouped_gemm_w4a16");
 }
 
+// scales [rows = E * n][groups] -> per 16 rows [groups][16]
+__global__ __launch_bounds__(256) void tile_scales_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                         long long total, int groups) {
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;  // index into dst
+  if (i >= total) return;
+  const long long frag = i / (16LL * groups);
+  const int r = static_cast<int>(i - frag * 16LL * groups);
+  const int g = r >> 4, c = r & 15;
+  dst[i] = src[(frag * 16 + c) * groups + g];
+}
+
 }  // namespace
 }  // namespace kmoe
 
 using namespace kmoe;
+
+extern "C" int kmoe_tile_scales_w4(const uint16_t* src, uint16_t* dst, int E, int n, int groups, kmoe_stream_t stream) {
+  KMOE_REQUIRE(src && dst && src != dst, KMOE_ERR_NULL, "tile_scales_w4: NULL pointer, or in place");
+  KMOE_REQUIRE(E >= 1 && n >= 16 && n % 16 == 0 && groups >= 1, KMOE_ERR_SHAPE, "tile_scales_w4: E=%d n=%d groups=%d", E, n, groups);
+  const long long total = static_cast<long long>(E) * n * groups;
+  hipLaunchKernelGGL(tile_scales_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, as_stream(stream), src,
+                     dst, total, groups);
+  return check_launch("kmoe_tile_scales_w4");
+}
 
 extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t stream) {
   KMOE_REQUIRE(a, KMOE_ERR_NULL, "grouped_gemm_w4a16: NULL args");
@@ -577,8 +602,12 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
   int shift = -1;
   if ((q & (q - 1)) == 0)
     for (shift = 0; (1 << shift) < q; ++shift) {}
-  const W4Params p{a->a, a->lda, a->row_src, a->src_div, a->w, a->w_scale, a->group_size, shift, a->lod,
-                   a->E, a->n,   a->k,       a->y,       a->ldy};
+  KMOE_REQUIRE(a->scale_layout == KMOE_S_ROWMAJOR || a->scale_layout == KMOE_S_FRAG16, KMOE_ERR_UNSUPPORTED,
+               "grouped_gemm_w4a16: scale_layout=%d unknown", a->scale_layout);
+  const int groups = a->k / a->group_size;
+  const bool frag16 = a->scale_layout == KMOE_S_FRAG16;
+  const W4Params p{a->a, a->lda, a->row_src, a->src_div, a->w, a->w_scale, a->group_size, shift,
+                   frag16 ? 1 : groups, frag16 ? 16 : 1, a->lod, a->E, a->n, a->k, a->y, a->ldy};
   hipStream_t s = as_stream(stream);
   int mf = a->variant;
   // the 128-row tile kernel reaches a source row (gathered or not: below `rows`) through a 32-bit byte offset

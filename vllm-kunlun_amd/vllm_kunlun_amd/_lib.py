@@ -25,6 +25,7 @@ KMOE_FMT_BF16 = 2
 KMOE_FMT_W4A16 = 3
 KMOE_DT_BF16, KMOE_DT_F16 = 0, 1
 KMOE_W_ROWMAJOR, KMOE_W_TILED = 0, 1
+KMOE_S_ROWMAJOR, KMOE_S_FRAG16 = 0, 1
 KMOE_A_ROWMAJOR, KMOE_A_CHUNKED = 0, 1
 STAGES = ("routing", "align", "quant1", "gemm1", "quant2", "gemm2", "shared", "combine")
 
@@ -60,7 +61,7 @@ class GemmW4Args(C.Structure):
         ("w", C.c_void_p), ("w_scale", C.c_void_p), ("group_size", C.c_int32), ("lod", C.c_void_p),
         ("E", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("rows", C.c_int32),
         ("y", C.c_void_p), ("ldy", C.c_int64), ("act", C.c_int32), ("variant", C.c_int32),
-        ("w_layout", C.c_int32), ("act_dtype", C.c_int32),
+        ("w_layout", C.c_int32), ("act_dtype", C.c_int32), ("scale_layout", C.c_int32),
     ]
 
 
@@ -88,7 +89,7 @@ class MoEArgs(C.Structure):
         ("w13_bias", C.c_void_p), ("w2_bias", C.c_void_p), ("activation", C.c_int32), ("act_alpha", C.c_float),
         ("act_limit", C.c_float), ("ws_layout", C.c_int32),
         ("w13_scale", C.c_void_p), ("w2_scale", C.c_void_p), ("group_size", C.c_int32),
-        ("act_dtype", C.c_int32), ("shared_scale", C.c_float), ("tile_variant", C.c_int32),
+        ("act_dtype", C.c_int32), ("shared_scale", C.c_float), ("tile_variant", C.c_int32), ("w_scale_layout", C.c_int32),
     ]
 
 
@@ -121,6 +122,7 @@ def _load() -> C.CDLL:
         "kmoe_swigluoai_and_mul": (i32, [vp, i64, i32, i32, f32, f32, vp, i64, vp]),
         "kmoe_dequant_w4_bf16": (i32, [vp, vp, i64, i32, i32, vp, vp]),
         "kmoe_dequant_w4": (i32, [vp, vp, i64, i32, i32, vp, i32, vp]),
+        "kmoe_tile_scales_w4": (i32, [vp, vp, i32, i32, i32, vp]),
         "kmoe_quant_i8_static": (i32, [vp, i64, i32, i32, vp, vp, vp, i64, i32, vp]),
         "kmoe_quant_i8_rows_azp": (i32, [vp, i64, i32, i32, vp, i64, vp, vp, i32, vp]),
         "kmoe_router_gemm_workspace_bytes": (sz, [i32, i32, i32]),
@@ -155,7 +157,7 @@ EXPORTS = (
     "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_w4a16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
     "kmoe_moe_workspace_layout", "kmoe_moe_forward", "kmoe_router_gemm_workspace_bytes", "kmoe_router_gemm_bf16",
     "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16", "kmoe_dequant_w4", "kmoe_moe_forward_static",
-    "kmoe_quant_i8_static", "kmoe_quant_i8_rows_azp",
+    "kmoe_quant_i8_static", "kmoe_quant_i8_rows_azp", "kmoe_tile_scales_w4",
     "kmoe_quant_i8_rows_dt", "kmoe_quant_i8_rows_chunked_dt", "kmoe_silu_and_mul_dt", "kmoe_combine_dt", "kmoe_router_gemm",
 )
 STATIC_WORKSPACE_BYTES = 64 << 20

@@ -124,6 +124,53 @@ def tile_int8_weights_(w: torch.Tensor) -> bool:
     return True
 
 
+_SCALES_FRAG16: dict = {}  # storage -> (n, groups) of 4-bit group scales re-arranged by tile_w4_scales_
+
+
+def tile_w4_scales_(scale: torch.Tensor) -> bool:
+    """Re-arranges the group scales [E, n, groups] of packed 4-bit weights IN PLACE (one expert at a time through
+    a scratch copy) into the per-16-channel [groups][16] form of kmoe_tile_scales_w4 and marks the memory.
+    Returns False and leaves the tensor alone when the shape does not allow it."""
+    data = scale.data
+    if data.dtype not in (torch.bfloat16, torch.float16) or not data.is_cuda or not data.is_contiguous() or data.dim() != 3:
+        return False
+    E, n, groups = data.shape
+    if n % 16:
+        return False
+    key = data.untyped_storage()._cdata
+    if key in _SCALES_FRAG16:
+        return True
+    tmp = torch.empty_like(data[0])
+    for e in range(E):
+        L.check(L.lib.kmoe_tile_scales_w4(L.ptr(data[e]), L.ptr(tmp), 1, n, groups, L.stream()))
+        data[e].copy_(tmp)
+    storage = data.untyped_storage()
+    _SCALES_FRAG16[key] = (n, groups)
+    weakref.finalize(storage, _SCALES_FRAG16.pop, key, None)
+    return True
+
+
+def scale_layout(scale: torch.Tensor) -> int:
+    """KMOE_S_FRAG16 or KMOE_S_ROWMAJOR for the group scales of packed 4-bit weights handed to an operator; as
+    for weights, only the contiguous [..., n, groups] tensor that was re-arranged may stand for its memory."""
+    dims = _SCALES_FRAG16.get(scale.untyped_storage()._cdata)
+    if dims is None:
+        return L.KMOE_S_ROWMAJOR
+    if scale.dim() < 2 or not scale.is_contiguous() or tuple(scale.shape[-2:]) != dims:
+        raise ValueError(f"this tensor {tuple(scale.shape)} is a view of group scales that were re-arranged as "
+                         f"[..., {dims[0]}, {dims[1]}]: pass the contiguous tensor itself")
+    return L.KMOE_S_FRAG16
+
+
+def rowmajor_w4_scales(scale: torch.Tensor) -> torch.Tensor:
+    """A row-major [..., n, groups] COPY of group scales, undoing tile_w4_scales_ if it was applied."""
+    if scale.untyped_storage()._cdata not in _SCALES_FRAG16:
+        return scale.data.clone()
+    n, groups = scale.shape[-2:]
+    lead = scale.shape[:-2]
+    return scale.data.reshape(-1, n // 16, groups, 16).permute(0, 1, 3, 2).reshape(*lead, n, groups).contiguous()
+
+
 def can_tile(w: torch.Tensor) -> bool:
     d = w.data
     return (d.dtype in _TILEABLE and d.is_cuda and d.is_contiguous() and d.shape[-2] % 16 == 0
@@ -226,6 +273,9 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     a.w13, a.w2 = w13.data_ptr(), w2.data_ptr()
     if w4:
         a.w13_scale, a.w2_scale, a.group_size = w13_aux.data_ptr(), w2_aux.data_ptr(), int(group_size)
+        a.w_scale_layout = scale_layout(w13_aux)
+        if scale_layout(w2_aux) != a.w_scale_layout:
+            raise ValueError("moe plan: the group scales of w13 and w2 must be in one layout (tile_w4_scales_ on both, or none)")
     else:
         a.w13_max = 0 if w13_aux is None else w13_aux.data_ptr()
         a.w2_max = 0 if w2_aux is None else w2_aux.data_ptr()

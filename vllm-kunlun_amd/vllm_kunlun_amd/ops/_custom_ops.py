@@ -282,7 +282,7 @@ def _moe_fc_w4(x, weight, lod, y, act, w_scale, group_size) -> None:
     """moe_fc with use_pack_int4: bfloat16 (or float16) activations against packed 4-bit weights [E, n, k/2] (two
     codes per byte, low nibble first, code - 8; re-tiled at load time) with group scales [E, n, k/group] in the
     activations' dtype; scale_k carries the group size (0: one scale per output channel)."""
-    from .._plan import weight_layout
+    from .._plan import scale_layout, weight_layout
     _need(x.dtype in (_BF16, torch.float16) and y.dtype == x.dtype and weight.dtype == torch.uint8,
           "moe_fc: packed 4-bit weights are uint8 and go with bfloat16 or float16 activations")
     E, n, half_k = weight.shape
@@ -302,6 +302,7 @@ def _moe_fc_w4(x, weight, lod, y, act, w_scale, group_size) -> None:
     g.act = L.KMOE_ACT_SWIGLU if act else L.KMOE_ACT_NONE
     g.w_layout = L.KMOE_W_TILED
     g.act_dtype = L.act_dtype(x)
+    g.scale_layout = scale_layout(w_scale)  # re-arranged at load time (tile_w4_scales_), or as the checkpoint holds them
     L.check(L.lib.kmoe_grouped_gemm_w4a16(g, L.stream()))
 
 

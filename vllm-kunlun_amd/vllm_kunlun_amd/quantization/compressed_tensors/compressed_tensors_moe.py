@@ -17,7 +17,7 @@ from typing import Optional, Union
 import torch
 
 from ... import _lib as L
-from ..._plan import MoEPlan, make_moe_plan, tile_pair_
+from ..._plan import MoEPlan, make_moe_plan, tile_pair_, tile_w4_scales_
 from ...ops import _custom_ops  # noqa: F401  (torch.ops._C.* used by the staged path)
 
 WNA16_SUPPORTED_BITS = (4, 8)
@@ -404,6 +404,9 @@ class KunlunCompressedTensorsWNA16MoEMethod:
             if native:
                 if not tile_pair_(layer.w13_weight_packed, layer.w2_weight_packed):
                     raise RuntimeError("4-bit weights: tiling the packed tensors failed")
+                # the scales too: per 16 channels [groups][16], so that what a block needs is one piece of memory
+                if not (tile_w4_scales_(layer.w13_weight_scale) and tile_w4_scales_(layer.w2_weight_scale)):
+                    raise RuntimeError("4-bit weights: re-arranging the group scales failed")
             layer.w4_native = bool(native)
             if keep_bf16 and getattr(self, "tile_weights", True):
                 tile_pair_(layer.w13_weight, layer.w2_weight)

@@ -608,6 +608,20 @@ def test_w4a16_layer_on_the_packed_weights(native, group_size, M):
     w2 = co.dequant_w4_bf16(packed2.numpy(), bits(scale2), group_size or I)
     ref = co.forward_bf16(bits(x), logits.cpu().numpy(), w13, w2, K)
     assert rel_l2(out, from_bits(ref)) <= REL_L2_BF16
+    # the reference's entry point, argument for argument (compressed_tensors_moe.py:296-320): the same result, and
+    # sigmoid scoring with a correction bias reaches the routing
+    out2 = method.apply(layer, x, logits, K, True, use_grouped_topk=False, scoring_func="softmax")
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out)
+    bias = torch.randn(E, generator=torch.Generator().manual_seed(4)) * 0.1
+    out3 = method.apply(layer, x, logits, K, True, scoring_func="sigmoid", e_score_correction_bias=bias.cuda())
+    torch.cuda.synchronize()
+    ref3 = co.forward_bf16(bits(x), logits.cpu().numpy(), w13, w2, K, scoring="sigmoid", bias=bias.numpy())
+    assert rel_l2(out3, from_bits(ref3)) <= REL_L2_BF16
+    with pytest.raises(NotImplementedError):
+        method.apply(layer, x, logits, K, True, expert_map=torch.arange(E, device="cuda"))
+    with pytest.raises(NotImplementedError):
+        method.apply(layer, x, logits, K, True, activation="gelu")
 
 
 @pytest.mark.parametrize("act", [None, "SWISH_GLU"])

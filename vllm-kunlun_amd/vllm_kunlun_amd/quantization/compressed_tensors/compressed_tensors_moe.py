@@ -418,11 +418,41 @@ class KunlunCompressedTensorsWNA16MoEMethod:
                     e_score_correction_bias=getattr(layer, "e_score_correction_bias", None))
 
     def apply_monolithic(self, layer, x: torch.Tensor, router_logits: torch.Tensor, **kwargs):
+        """The layer-driven call: top_k from the method's `moe`, routing attributes from the layer."""
+        return self._run(layer, x, router_logits, self.moe.experts_per_token, **self._routing_kwargs(layer))
+
+    def apply(self, layer: torch.nn.Module, x: torch.Tensor, router_logits: torch.Tensor, top_k: int, renormalize: bool,
+              use_grouped_topk: bool = False, topk_group: Optional[int] = None, num_expert_group: Optional[int] = None,
+              global_num_experts: int = -1, expert_map: Optional[torch.Tensor] = None, custom_routing_function=None,
+              scoring_func: str = "softmax", routed_scaling_factor: float = 1.0,
+              e_score_correction_bias: Optional[torch.Tensor] = None, apply_router_weight_on_input: bool = False,
+              activation: str = "silu", enable_eplb: bool = False, expert_load_view: Optional[torch.Tensor] = None,
+              logical_to_physical_map: Optional[torch.Tensor] = None,
+              logical_replica_count: Optional[torch.Tensor] = None):
+        """The reference's entry point, argument for argument (compressed_tensors_moe.py:296-360). As there, what
+        reaches the computation is top_k, scoring_func, the group arguments and the correction bias: `renormalize`,
+        `use_grouped_topk` and `routed_scaling_factor` stop at KunlunOps.fused_moe, which always normalises and
+        uses scale 1.0 (_kunlun_ops.py:385-431). Arguments the reference accepts and ignores but which would change
+        the result if honoured are refused rather than ignored."""
+        if expert_map is not None or custom_routing_function is not None or apply_router_weight_on_input or enable_eplb:
+            raise NotImplementedError("4-bit MoE: expert_map, custom_routing_function, apply_router_weight_on_input "
+                                      "and EPLB are not on this path")
+        if activation != "silu":
+            raise NotImplementedError(f"4-bit MoE: activation {activation!r} (silu only)")
+        if getattr(self.moe, "use_ep", False):
+            # the expert-parallel branch (:329-342) ends in KunlunOps.fused_moe_ep: softmax routing, `renormalize` honoured
+            if getattr(self.moe, "ep_rank", 0) != 0:
+                raise NotImplementedError("4-bit MoE: this build runs all experts on one GPU (ep_rank must be 0)")
+            return self._run(layer, x, router_logits, top_k, renormalize=bool(renormalize))
+        return self._run(layer, x, router_logits, top_k, scoring_func=scoring_func, num_expert_group=num_expert_group,
+                         topk_group=topk_group, e_score_correction_bias=e_score_correction_bias)
+
+    def _run(self, layer, x, router_logits, top_k, scoring_func="softmax", num_expert_group=None, topk_group=None,
+             e_score_correction_bias=None, renormalize=True):
         """Activations in the dtype of the scales (bf16, or float16). On the packed weights:
         kmoe_grouped_gemm_w4a16 inside kmoe_moe_forward. On the unpacked copy: KunlunOps.fused_moe, as
         the reference's apply() ends (:343-360). Routing as in KunlunOps.fused_moe (always
         normalised, sigmoid scale 1.0)."""
-        top_k = self.moe.experts_per_token
         E = layer.w13_weight_scale.shape[0] if getattr(layer, "w4_native", False) else layer.w13_weight.shape[0]
         rows_per_expert = -(-x.shape[0] * top_k // E)
         has_bias = getattr(layer, "w13_bias", None) is not None or getattr(layer, "w2_bias", None) is not None
@@ -434,20 +464,22 @@ class KunlunCompressedTensorsWNA16MoEMethod:
                                  f"({layer.w13_weight_scale.dtype})")
             xc = x.contiguous()
             out = torch.empty_like(xc)
-            rk = self._routing_kwargs(layer)
             gs = self.group_size or 2 * layer.w13_weight_packed.shape[-1]
             plan = make_moe_plan(L.KMOE_FMT_W4A16, xc, router_logits.to(torch.float).contiguous(), out, top_k,
                                  layer.w13_weight_packed, layer.w2_weight_packed, layer.w13_weight_scale,
-                                 layer.w2_weight_scale, rk["scoring_func"], True, rk["num_expert_group"],
-                                 rk["topk_group"], 1.0, rk["e_score_correction_bias"], group_size=gs)
+                                 layer.w2_weight_scale, scoring_func, renormalize, num_expert_group, topk_group, 1.0,
+                                 e_score_correction_bias, group_size=gs)
             plan()
             return out
+        if not hasattr(layer, "w13_weight"):
+            raise NotImplementedError("4-bit MoE: expert biases need the unpacked copy (native='both' or False)")
         from ...ops._kunlun_ops import KunlunOps as ops
+        if not renormalize:  # only the expert-parallel entry leaves the weights unnormalised
+            return ops.fused_moe_ep(x, layer.w13_weight, layer.w2_weight, router_logits, 0, top_k, renormalize=False,
+                                    inplace=True)
         return ops.fused_moe(x, layer.w13_weight, layer.w2_weight, router_logits, 0, top_k,
                              renormalize=getattr(layer, "renormalize", True), inplace=True,
                              use_grouped_topk=getattr(layer, "use_grouped_topk", False),
-                             num_expert_group=getattr(layer, "num_expert_group", None),
-                             topk_group=getattr(layer, "topk_group", None),
-                             scoring_func=getattr(layer, "scoring_func", "softmax"),
-                             e_score_correction_bias=getattr(layer, "e_score_correction_bias", None),
+                             num_expert_group=num_expert_group, topk_group=topk_group, scoring_func=scoring_func,
+                             e_score_correction_bias=e_score_correction_bias,
                              w1_bias=getattr(layer, "w13_bias", None), w2_bias=getattr(layer, "w2_bias", None))

@@ -104,3 +104,31 @@ def test_random_fp8_layer_shape(seed):
                          None if sl.bias is None else sl.bias.cpu().numpy(), shared)
     ref_t = torch.from_numpy(ref.view(np.int16)).view(torch.bfloat16)
     assert _rel_l2(out, ref_t) <= 3e-2, f"{base} {over}"
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_w4_layer_shape(seed):
+    """Packed 4-bit weights kept alone (hidden and intermediate sizes in multiples of 128, groups of 32, 64, 128 or a
+    whole row; bfloat16 or float16): small batches on the streaming kernel, 25 rows per expert and more on the
+    128-row tile kernel; against the oracle's unquantized layer on the weights its unpacking gives."""
+    from vllm_kunlun_amd import synth
+    base, over, half = _draw(3000 + seed)
+    rng = random.Random(seed)
+    over = {k: v for k, v in over.items() if k not in ("I_shared", "routed_scale")}
+    H = 128 * rng.randint(1, 6)
+    over.update(H=H, I=H if rng.random() < 0.3 else 128 * rng.randint(1, 4), quant="w4", I_shared=0)
+    if rng.random() < 0.4:
+        over["M"] = rng.randint(200, 2500)  # enough rows per expert for the tile kernel with most draws of E and K
+    gs = rng.choice([32, 64, 128, None])
+    over["group_size"] = gs if gs else (over["H"] if over["H"] == over["I"] else 128)
+    shape = synth.scaled(synth.SHAPES[base], **over)
+    sl = synth.make_layer(shape, "cuda", seed=seed, dtype=torch.float16 if half else torch.bfloat16)
+    out = sl.layer(sl.x, sl.logits)
+    torch.cuda.synchronize()
+    p13, s13, p2, s2, _ = sl.host_weights()
+    w13 = co.dequant_w4_bf16(p13.numpy(), _bits16(s13), shape.group_size, f16=half)
+    w2 = co.dequant_w4_bf16(p2.numpy(), _bits16(s2), shape.group_size, f16=half)
+    ref = co.forward_bf16(_bits16(sl.x), sl.logits.cpu().numpy(), w13, w2, shape.K, shape.scoring, True, shape.n_group,
+                          shape.topk_group, 1.0, None if sl.bias is None else sl.bias.cpu().numpy(), f16=half)
+    ref_t = torch.from_numpy(ref.view(np.int16)).view(torch.float16 if half else torch.bfloat16)
+    assert _rel_l2(out, ref_t) <= (1e-3 if half else 1e-2), f"{base} {over} half={half}"

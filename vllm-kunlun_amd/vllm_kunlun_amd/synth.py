@@ -105,13 +105,18 @@ class SynthLayer:
     def host_weights(self):
         """(w13, w13_aux, w2, w2_aux, shared) as host tensors in the reference's row-major
         layout (int8 weights are un-tiled), for a CPU checker."""
-        from ._plan import rowmajor_int8_weights
+        from ._plan import rowmajor_int8_weights, rowmajor_w4_scales
         lay = self.layer
 
         def rm(t):
             return rowmajor_int8_weights(t).detach().cpu()
 
-        aux = lambda name: getattr(lay, name).detach().cpu() if hasattr(lay, name) else None  # noqa: E731
+        def aux(name):  # (the group scales of packed 4-bit weights are re-arranged at load time as well)
+            if not hasattr(lay, name):
+                return None
+            t = getattr(lay, name)
+            return (rowmajor_w4_scales(t) if t.dtype in (torch.bfloat16, torch.float16) else t).detach().cpu()
+
         shared = None
         if self.shared is not None:
             shared = (rm(self.shared[0]), self.shared[1].detach().cpu(), rm(self.shared[2]),

@@ -47,6 +47,10 @@ WORKLOAD_LABEL = {
                           "decode, 64 tokens",
     "qwen3-w4a16-prefill": "Qwen3-MoE-30B-A3B-shape MoE layer, 4-bit weights (groups of 128) and bf16 activations, "
                            "prefill, 8192 tokens",
+    "kimi-w4a16-decode": "Kimi-K2-shape MoE layer (384 experts, no shared expert), 4-bit weights (groups of 32) and bf16 "
+                         "activations, decode, 128 tokens",
+    "kimi-w4a16-prefill": "Kimi-K2-shape MoE layer (384 experts, no shared expert), 4-bit weights (groups of 32) and bf16 "
+                          "activations, prefill, 4096 tokens",
     "tiny-bf16": "tiny bf16 MoE layer (32 tokens, hidden 512, 8 experts, top-2, intermediate 256), no quantization",
 }
 PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0, "none": 2500.0, "w4": 2500.0}  # MI355X dense MFMA: int8, fp8, bf16

@@ -66,6 +66,11 @@ for _n in ("qwen3-decode", "qwen3-prefill"):
 # ... and with 4-bit weights (group scales of 128 values) on the packed-weight paths
 SHAPES["qwen3-w4a16-decode"] = replace(SHAPES["qwen3-decode"], name="qwen3-w4a16-decode", quant="w4")
 SHAPES["qwen3-w4a16-prefill"] = replace(SHAPES["qwen3-prefill"], name="qwen3-w4a16-prefill", quant="w4")
+# the Kimi-K2 dimensions with 4-bit routed experts in groups of 32 (the shared expert of such a checkpoint stays a
+# 16-bit dense layer of its own, outside this layer)
+for _n in ("kimi-decode", "kimi-prefill"):
+    _f = _n.replace("-", "-w4a16-")
+    SHAPES[_f] = replace(SHAPES[_n], name=_f, quant="w4", group_size=32, I_shared=0)
 
 
 def make_layer(shape: MoEShape, device="cuda", seed: int = 0, dtype: torch.dtype = torch.bfloat16) -> "SynthLayer":

@@ -170,6 +170,21 @@ int kmoe_quant_i8_rows_azp(const uint16_t* x, int64_t ld_x, int R, int C, int8_t
                            float* row_scale, int32_t* row_azp, int act_dtype, kmoe_stream_t stream);
 
 /*
+ * Epilogue of torch.ops._C.cutlass_scaled_mm_azp (ops/_custom_ops.py:1756-1771, closed in the reference; called by
+ * KunlunScaledMMLinearKernel.apply_weights for asymmetric activations, quantization/kernels/scale_mm.py:70-82) on
+ * the int32 accumulators of an int8 GEMM (acc_out of kmoe_grouped_gemm_i8). The arithmetic is the one of the vLLM
+ * operator of that name (csrc/quantization/cutlass_w8a8, ScaledEpilogueBiasAzp / ...AzpToken):
+ *   t = acc[r,c] - azp[r] * azp_adj[c]   (int32; azp == NULL: t = acc[r,c] - azp_adj[c], the zero point of a static
+ *                                         scheme being folded into azp_adj)
+ *   out[r,c] = dt( scale_a[r or 0] * (scale_b[c or 0] * float(t)) + bias[c] )      f32, products and sum unfused
+ * azp_adj [n] int32: the sums of the weight codes over k per output channel. scale_a: one f32 per row
+ * (scale_a_rows != 0) or one for the tensor; scale_b: one per channel (scale_b_cols != 0) or one; bias [n] f32 or NULL.
+ */
+int kmoe_scaled_mm_azp_epilogue(const int32_t* acc, int64_t ld_acc, int M, int n, const float* scale_a, int scale_a_rows,
+                                const float* scale_b, int scale_b_cols, const int32_t* azp_adj, const int32_t* azp,
+                                const float* bias, uint16_t* out, int64_t ld_out, int act_dtype, kmoe_stream_t stream);
+
+/*
  * Per-row, per-128-column-group dynamic fp8-e4m3fn (OCP). No counterpart in the
  * reference (its fp8 ops are empty stubs, ops/_custom_ops.py:44-89); follows
  * the DeepSeek-V3 block-scaled recipe.

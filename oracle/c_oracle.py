@@ -159,6 +159,24 @@ def quant_i8_static(x_bits, scale, azp=None, f16=False):
     return q
 
 
+def scaled_mm_azp(a, w, scale_a, scale_b, azp_adj, azp=None, bias=None, f16=False):
+    """int8 a [M,k] x w [n,k] with the asymmetric-activation epilogue: 16-bit patterns [M,n]."""
+    _dtype(f16)
+    a, w = _c(a, np.int8), _c(w, np.int8)
+    M, k = a.shape
+    n = w.shape[0]
+    scale_a, scale_b = _c(scale_a, np.float32).ravel(), _c(scale_b, np.float32).ravel()
+    azp_adj = _c(azp_adj, np.int32).ravel()
+    assert scale_a.size in (1, M) and scale_b.size in (1, n) and azp_adj.size == n
+    azp = None if azp is None else _c(azp, np.int32).ravel()
+    bias = None if bias is None else _c(bias, np.float32).ravel()
+    out = np.zeros((M, n), np.uint16)
+    lib().orc_scaled_mm_azp(_p(a), _p(w), M, n, k, _p(scale_a), int(scale_a.size == M),
+                            _p(scale_b), int(scale_b.size == n), _p(azp_adj), None if azp is None else _p(azp),
+                            None if bias is None else _p(bias), _p(out))
+    return out
+
+
 def quant_i8_rows_azp(x_bits, f16=False):
     """Per-row scale and zero point: (codes int8 [R,C], scale f32 [R], azp int32 [R])."""
     _dtype(f16)

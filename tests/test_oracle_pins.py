@@ -871,3 +871,39 @@ def test_quant_i8_rows_azp_closed_forms_and_invariants():
         assert (np.abs(back - xf) <= s[:, None] * 1.001).all()
         order = np.argsort(xf, axis=1, kind="stable")
         assert (np.diff(np.take_along_axis(qi, order, 1), axis=1) >= 0).all()
+
+
+def test_scaled_mm_azp_against_the_dequantised_product():
+    """out = scale_a * scale_b * (a @ w.T - azp * sum_k w) + bias is the product of the DEQUANTISED operands,
+    sum_k (a - azp) * scale_a * w * scale_b + bias: evaluated in f64 from that definition (no accumulator, no
+    column sums), the oracle's 16-bit result is its rounding within one unit in the last place. Exact cases: unit
+    scales and small integers. Shapes M != n != k, so a transposed operand or a zero point on the wrong axis fails."""
+    g = np.random.default_rng(0)
+    M, n, k = 7, 12, 40
+    a = g.integers(-128, 128, (M, k), dtype=np.int8)
+    w = g.integers(-128, 128, (n, k), dtype=np.int8)
+    azp = g.integers(-200, 100, M).astype(np.int32)
+    adj = w.astype(np.int64).sum(1).astype(np.int32)
+    sa = (g.random(M) * 0.05 + 0.01).astype(np.float32)
+    sb = (g.random(n) * 0.02 + 0.001).astype(np.float32)
+    bias = g.normal(size=n).astype(np.float32)
+    want = ((a.astype(np.float64) - azp[:, None]) * sa[:, None].astype(np.float64)) @ (w.astype(np.float64) * sb[:, None]).T
+    for f16 in (False, True):
+        for b in (None, bias):
+            got = co.scaled_mm_azp(a, w, sa, sb, adj, azp, b, f16=f16)
+            got = (from_bits(got).double() if not f16 else torch.from_numpy(got.view(np.float16).copy()).double()).numpy()
+            ref = want + (0 if b is None else b.astype(np.float64))
+            ulp = np.maximum(np.abs(ref), 1e-3) * (2.0 ** -10 if f16 else 2.0 ** -7)
+            assert np.all(np.abs(got - ref) <= ulp)
+    # a static scheme: the zero point folded into azp_adj gives what the per-token form gives with a constant azp
+    z = np.int32(-37)
+    per_token = co.scaled_mm_azp(a, w, sa[:1], sb, adj, np.full(M, z, np.int32))
+    folded = co.scaled_mm_azp(a, w, sa[:1], sb, adj * z, None)
+    assert np.array_equal(per_token, folded)
+    # exact: unit scales, small integers (every partial result is an integer below 256)
+    a1 = g.integers(-3, 4, (5, 6), dtype=np.int8)
+    w1 = g.integers(-3, 4, (4, 6), dtype=np.int8)
+    z1 = g.integers(-2, 3, 5).astype(np.int32)
+    exact = (a1.astype(np.int64) - z1[:, None]) @ w1.astype(np.int64).T
+    got = co.scaled_mm_azp(a1, w1, np.ones(1, np.float32), np.ones(1, np.float32), w1.astype(np.int64).sum(1), z1)
+    assert np.array_equal(from_bits(got).double().numpy().astype(np.int64), exact)

@@ -52,7 +52,17 @@ def test_process_weights_after_loading_on_the_host():
     ok, why = KunlunScaledMMLinearKernel.can_implement(Int8ScaledMMLinearLayerConfig(is_static_input_scheme=True))
     assert ok and why is None
     ok, why = KunlunScaledMMLinearKernel.can_implement(Int8ScaledMMLinearLayerConfig(input_symmetric=False))
-    assert not ok and "asymmetric" in why
+    assert ok and why is None
+    # asymmetric activations: the sums of the weight codes per output channel, times the zero point when it is static
+    layer3, wq3, _ = _layer(32, 64, "cpu", 3)
+    KunlunScaledMMLinearKernel(Int8ScaledMMLinearLayerConfig(input_symmetric=False)).process_weights_after_loading(layer3)
+    assert layer3.azp_adj.dtype == torch.int32 and torch.equal(layer3.azp_adj.data, wq3.int().sum(1).reshape(1, 32))
+    layer4, wq4, _ = _layer(32, 64, "cpu", 4)
+    layer4.input_scale = torch.nn.Parameter(torch.tensor([0.02]), requires_grad=False)
+    layer4.input_zero_point = torch.nn.Parameter(torch.tensor([-7], dtype=torch.int32), requires_grad=False)
+    KunlunScaledMMLinearKernel(Int8ScaledMMLinearLayerConfig(is_static_input_scheme=True, input_symmetric=False)
+                               ).process_weights_after_loading(layer4)
+    assert torch.equal(layer4.azp_adj.data, -7 * wq4.int().sum(1).reshape(1, 32)) and layer4.input_scale is not None
     with pytest.raises(ValueError):
         bad, _, _ = _layer(16, 64, "cpu", 2)
         bad.weight_scale = torch.nn.Parameter(torch.ones(5), requires_grad=False)
@@ -106,6 +116,49 @@ def test_apply_weights_with_a_static_input_scale(M, n, k, dtype):
     x_max = np.full(M, scale * np.float32(127.0), np.float32)
     ref, _ = co.grouped_gemm_i8(xq, x_max, wq.numpy()[None], w_max.numpy()[None], np.array([0, M], np.int32), f16=f16)
     assert out.dtype == dtype and np.array_equal(bits(out), ref)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,n,k,dtype", [(1, 64, 128, torch.bfloat16), (37, 256, 512, torch.float16),
+                                         (300, 512, 1024, torch.bfloat16), (5, 48, 80, torch.bfloat16)])
+@pytest.mark.parametrize("static", [False, True])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_apply_weights_with_asymmetric_activations(M, n, k, dtype, static, with_bias):
+    """The asymmetric schemes (scale_mm.py:60-82 in the reference): codes with a zero point per token (dynamic) or
+    the layer's own (static), the int8 product and the zero-point correction in the epilogue of
+    `_C::cutlass_scaled_mm_azp`: against the oracle's quantisation and its restated epilogue, bit for bit; and
+    against the plain float product of x and the dequantised weights within the quantisation error."""
+    from vllm_kunlun_amd.quantization.kernels.scale_mm import (Int8ScaledMMLinearLayerConfig,
+                                                               KunlunScaledMMLinearKernel)
+    layer, wq, w_max = _layer(n, k, "cuda", M + n + k)
+    scale, zp = np.float32(0.03), -11
+    if static:
+        layer.input_scale = torch.nn.Parameter(torch.tensor([scale], device="cuda"), requires_grad=False)
+        layer.input_zero_point = torch.nn.Parameter(torch.tensor([zp], dtype=torch.int32, device="cuda"),
+                                                    requires_grad=False)
+    kern = KunlunScaledMMLinearKernel(Int8ScaledMMLinearLayerConfig(is_static_input_scheme=static, input_symmetric=False))
+    kern.process_weights_after_loading(layer)
+    g = torch.Generator().manual_seed(M)
+    x = (torch.randn(M, k, generator=g) * 1.5 + 0.7).to(dtype)  # not centred: the zero point matters
+    bias = torch.randn(n, generator=g) if with_bias else None
+    out = kern.apply_weights(layer, x.cuda(), None if bias is None else bias.to(dtype).cuda())
+    torch.cuda.synchronize()
+    f16 = dtype == torch.float16
+    adj = wq.numpy().astype(np.int64).sum(1).astype(np.int32)
+    # the reference's per-call expression (w_s / 127.0) as torch evaluates it on the device (a product with the
+    # reciprocal there, a division on the host: one unit in the last place apart for some channels)
+    scale_b = (layer.weight_scale.data / 127.0).reshape(-1).cpu().numpy()
+    assert np.allclose(scale_b, (w_max / 127.0).numpy(), rtol=2e-7, atol=0)
+    b32 = None if bias is None else bias.to(dtype).float().numpy()
+    if static:
+        xq = co.quant_i8_static(bits(x), scale, zp, f16=f16)
+        ref = co.scaled_mm_azp(xq, wq.numpy(), np.array([scale], np.float32), scale_b, adj * np.int32(zp), None, b32, f16=f16)
+    else:
+        xq, xs, xz = co.quant_i8_rows_azp(bits(x), f16=f16)
+        ref = co.scaled_mm_azp(xq, wq.numpy(), xs, scale_b, adj, xz, b32, f16=f16)
+    assert out.dtype == dtype and out.shape == (M, n) and np.array_equal(bits(out), ref)
+    want = x.float() @ (wq.float() * (w_max / 127.0).reshape(n, 1)).T + (0 if bias is None else bias.to(dtype).float())
+    assert (out.cpu().float() - want).norm() / want.norm() <= (6e-2 if static else 2e-2)
 
 
 @pytest.mark.gpu

@@ -344,6 +344,55 @@ extern "C" int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, i
   return check_launch("kmoe_quant_fp8_group128");
 }
 
+// ---------------------------------------- asymmetric-activation epilogue on int32 accumulators
+// one thread: 4 consecutive channels of one row
+__global__ __launch_bounds__(256) void scaled_mm_azp_kernel(const int32_t* __restrict__ acc, int64_t ld_acc, int M, int n,
+                                                           const float* __restrict__ scale_a, int sa_rows,
+                                                           const float* __restrict__ scale_b, int sb_cols,
+                                                           const int32_t* __restrict__ azp_adj,
+                                                           const int32_t* __restrict__ azp, const float* __restrict__ bias,
+                                                           uint16_t* __restrict__ out, int64_t ld_out, int f16) {
+  const int quads = n / 4;
+  const long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= static_cast<long long>(M) * quads) return;
+  const int r = static_cast<int>(idx / quads), c = static_cast<int>(idx % quads) * 4;
+  const int4 a = *reinterpret_cast<const int4*>(acc + static_cast<size_t>(r) * ld_acc + c);
+  const int4 adj = *reinterpret_cast<const int4*>(azp_adj + c);
+  const uint32_t z = azp ? static_cast<uint32_t>(azp[r]) : 1u;  // (products and differences wrap like int32 arithmetic)
+  const float sa = scale_a[sa_rows ? r : 0];
+  const int av[4] = {a.x, a.y, a.z, a.w}, dv[4] = {adj.x, adj.y, adj.z, adj.w};
+  uint16_t o[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int t = static_cast<int>(static_cast<uint32_t>(av[q]) - z * static_cast<uint32_t>(dv[q]));
+    float v = sa * (scale_b[sb_cols ? c + q : 0] * static_cast<float>(t));
+    if (bias) v = v + bias[c + q];
+    o[q] = f32_to_act(v, f16 != 0);
+  }
+  *reinterpret_cast<uint2*>(out + static_cast<size_t>(r) * ld_out + c) =
+      make_uint2(o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16));
+}
+
+extern "C" int kmoe_scaled_mm_azp_epilogue(const int32_t* acc, int64_t ld_acc, int M, int n, const float* scale_a,
+                                           int scale_a_rows, const float* scale_b, int scale_b_cols,
+                                           const int32_t* azp_adj, const int32_t* azp, const float* bias, uint16_t* out,
+                                           int64_t ld_out, int act_dtype, kmoe_stream_t stream) {
+  if (int rc = check_dtype(act_dtype, "scaled_mm_azp_epilogue")) return rc;
+  KMOE_REQUIRE(acc && scale_a && scale_b && azp_adj && out, KMOE_ERR_NULL, "scaled_mm_azp_epilogue: NULL pointer");
+  KMOE_REQUIRE(M >= 0 && n >= 4 && n % 4 == 0 && ld_acc >= n && ld_acc % 4 == 0 && ld_out >= n && ld_out % 4 == 0,
+               KMOE_ERR_SHAPE, "scaled_mm_azp_epilogue: M=%d n=%d strides %lld/%lld (need n %% 4 == 0)", M, n,
+               (long long)ld_acc, (long long)ld_out);
+  KMOE_REQUIRE((reinterpret_cast<uintptr_t>(acc) & 15) == 0 && (reinterpret_cast<uintptr_t>(azp_adj) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(out) & 7) == 0,
+               KMOE_ERR_SHAPE, "scaled_mm_azp_epilogue: misaligned tensor pointer");
+  if (M == 0) return KMOE_OK;
+  const long long total = static_cast<long long>(M) * (n / 4);
+  hipLaunchKernelGGL(scaled_mm_azp_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     acc, ld_acc, M, n, scale_a, scale_a_rows, scale_b, scale_b_cols, azp_adj, azp, bias, out, ld_out,
+                     act_dtype == KMOE_DT_F16 ? 1 : 0);
+  return check_launch("kmoe_scaled_mm_azp_epilogue");
+}
+
 extern "C" int kmoe_quant_i8_static(const uint16_t* x, int64_t ld_x, int R, int C, const float* scale,
                                     const int32_t* azp, int8_t* q, int64_t ld_q, int act_dtype, kmoe_stream_t stream) {
   if (int rc = check_dtype(act_dtype, "quant_i8_static")) return rc;

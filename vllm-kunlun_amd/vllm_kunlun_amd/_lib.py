@@ -123,6 +123,7 @@ def _load() -> C.CDLL:
         "kmoe_dequant_w4_bf16": (i32, [vp, vp, i64, i32, i32, vp, vp]),
         "kmoe_dequant_w4": (i32, [vp, vp, i64, i32, i32, vp, i32, vp]),
         "kmoe_tile_scales_w4": (i32, [vp, vp, i32, i32, i32, vp]),
+        "kmoe_scaled_mm_azp_epilogue": (i32, [vp, i64, i32, i32, vp, i32, vp, i32, vp, vp, vp, vp, i64, i32, vp]),
         "kmoe_quant_i8_static": (i32, [vp, i64, i32, i32, vp, vp, vp, i64, i32, vp]),
         "kmoe_quant_i8_rows_azp": (i32, [vp, i64, i32, i32, vp, i64, vp, vp, i32, vp]),
         "kmoe_router_gemm_workspace_bytes": (sz, [i32, i32, i32]),
@@ -157,7 +158,7 @@ EXPORTS = (
     "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_w4a16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
     "kmoe_moe_workspace_layout", "kmoe_moe_forward", "kmoe_router_gemm_workspace_bytes", "kmoe_router_gemm_bf16",
     "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16", "kmoe_dequant_w4", "kmoe_moe_forward_static",
-    "kmoe_quant_i8_static", "kmoe_quant_i8_rows_azp", "kmoe_tile_scales_w4",
+    "kmoe_quant_i8_static", "kmoe_quant_i8_rows_azp", "kmoe_tile_scales_w4", "kmoe_scaled_mm_azp_epilogue",
     "kmoe_quant_i8_rows_dt", "kmoe_quant_i8_rows_chunked_dt", "kmoe_silu_and_mul_dt", "kmoe_combine_dt", "kmoe_router_gemm",
 )
 STATIC_WORKSPACE_BYTES = 64 << 20

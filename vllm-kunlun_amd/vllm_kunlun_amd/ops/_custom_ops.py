@@ -403,6 +403,61 @@ def matmul(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, x_trans: bo
     return out
 
 
+@custom_op("_C::cutlass_scaled_mm_azp", mutates_args=())
+def cutlass_scaled_mm_azp(a: torch.Tensor, b: torch.Tensor, scale_a: torch.Tensor, scale_b: torch.Tensor,
+                          out_dtype: torch.dtype, azp_adj: torch.Tensor, azp: Optional[torch.Tensor] = None,
+                          bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Dense W8A8 linear with asymmetric activations (reference: ops/_custom_ops.py:1756-1771; caller
+    quantization/kernels/scale_mm.py:70-82): a int8 [M,k] (codes with a zero point), b int8 [k,n] (the transpose
+    view of the [n,k] weight), scale_a f32 [M,1] or [1], scale_b f32 [1,n] or [1], azp_adj int32 [1,n] (sums of
+    the weight codes over k, times the zero point for a static scheme), azp int32 [M,1] or None, bias f32 [n]:
+    out = scale_a * scale_b * (a @ b - azp * azp_adj) + bias. The int8 GEMM leaves its int32 accumulators
+    (acc_out of kmoe_grouped_gemm_i8); kmoe_scaled_mm_azp_epilogue finishes them."""
+    if a.dtype != torch.int8 or b.dtype != torch.int8 or a.dim() != 2 or b.dim() != 2:
+        raise NotImplementedError("cutlass_scaled_mm_azp: int8 a [M,k] and b [k,n] only")
+    if out_dtype not in (_BF16, torch.float16):
+        raise NotImplementedError(f"cutlass_scaled_mm_azp: out_dtype {out_dtype} is not implemented")
+    L.require_device(a, b, scale_a, scale_b, azp_adj, azp, bias)
+    from .._plan import is_tiled
+    w = b.t()  # the [n, k] weight; re-tiled memory must come as the transpose view of the tensor that was tiled
+    if not is_tiled(w):
+        w = w.contiguous()
+    ac = a.contiguous()
+    M, k = ac.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and azp_adj.numel() == n and azp_adj.dtype == torch.int32,
+          "cutlass_scaled_mm_azp: b must be [k,n] and azp_adj int32 with n entries")
+    _need(scale_a.dtype == torch.float32 and scale_a.numel() in (1, M) and scale_b.dtype == torch.float32
+          and scale_b.numel() in (1, n), "cutlass_scaled_mm_azp: f32 scales, one per row / channel or one per tensor")
+    _need(azp is None or (azp.dtype == torch.int32 and azp.numel() == M), "cutlass_scaled_mm_azp: azp is int32 [M,1]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n), "cutlass_scaled_mm_azp: bias is f32 [n]")
+    out = torch.empty((M, n), dtype=out_dtype, device=a.device)
+    if M == 0:
+        return out
+    acc = torch.empty((M, n), dtype=torch.int32, device=a.device)
+    ones_m, ones_n = _ones(a.device, M), _ones(a.device, n)  # the GEMM's own rescaling is not used
+    _gemm_i8(ac, ones_m, w.unsqueeze(0), ones_n, _dense_lod(a.device, M), out, n, L.KMOE_ACT_NONE, M, acc_out=acc)
+    L.check(L.lib.kmoe_scaled_mm_azp_epilogue(
+        L.ptr(acc), n, M, n, L.ptr(scale_a.contiguous()), int(scale_a.numel() == M),
+        L.ptr(scale_b.contiguous()), int(scale_b.numel() == n), L.ptr(azp_adj.contiguous()),
+        L.ptr(None if azp is None else azp.contiguous()), L.ptr(None if bias is None else bias.contiguous()), L.ptr(out),
+        n, L.act_dtype(out), L.stream()))
+    return out
+
+
+_ONES: dict = {}
+
+
+def _ones(device: torch.device, count: int) -> torch.Tensor:
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device(), count)
+    t = _ONES.get(key)
+    if t is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("cutlass_scaled_mm_azp: run one call of this size before capturing")
+        t = _ONES[key] = torch.ones(count, dtype=torch.float32, device=device)
+    return t
+
+
 # ---------------------------------------------------------------- elementwise
 @custom_op("_C::silu_and_mul", mutates_args=("out",))
 def silu_and_mul(out: torch.Tensor, x: torch.Tensor, axis: int = -1, turn: bool = True) -> None:
@@ -506,6 +561,11 @@ def _fake_scaled_int8_quant(x, scale, azp=None, symmetric=True):
         return torch.empty_like(x, dtype=torch.int8), torch.empty_like(scale), none if azp is None else torch.empty_like(azp), True
     return (torch.empty_like(x, dtype=torch.int8), torch.empty((rows, 1), device=x.device, dtype=torch.float32),
             none if symmetric else torch.empty((rows, 1), device=x.device, dtype=torch.int32), False)
+
+
+@cutlass_scaled_mm_azp.register_fake
+def _fake_cutlass_scaled_mm_azp(a, b, scale_a, scale_b, out_dtype, azp_adj, azp=None, bias=None):
+    return torch.empty((a.shape[0], b.shape[1]), dtype=out_dtype, device=a.device)
 
 
 @matmul.register_fake

@@ -51,9 +51,8 @@ class KunlunScaledMMLinearKernel:
     @classmethod
     def can_implement(cls, c: Int8ScaledMMLinearLayerConfig) -> tuple[bool, Optional[str]]:
         """Reference: scale_mm.py:39-41 accepts every config and fails later; this class says up
-        front which schemes its kernels cover."""
-        if not c.input_symmetric:
-            return False, "asymmetric activations (azp) need the azp GEMM epilogue, which is not implemented."
+        front which schemes its kernels cover: all four (dynamic or static input scale, symmetric or
+        asymmetric activations)."""
         return True, None
 
     def _get_layer_params(self, layer):
@@ -80,6 +79,16 @@ class KunlunScaledMMLinearKernel:
         scale = scale.contiguous().clone().reshape(n, 1)
         with torch.no_grad():
             scale.mul_(127.0)  # scale -> absmax, what the kernels take (x_pc_max / w_pc_max convention)
+        # Asymmetric activations (base-class part): azp_adj = the sums of the weight codes over k per output channel,
+        # times the input zero point for a static scheme, whose zero point then needs no term of its own at run time.
+        if not self.config.input_symmetric:
+            azp_adj = w_nk.sum(dim=1, dtype=torch.int32).reshape(1, n)
+            if self.config.is_static_input_scheme:
+                i_zp = getattr(layer, i_zp_name, None)
+                if i_zp is None:
+                    raise ValueError(f"{i_zp_name}: a static asymmetric scheme needs the input zero point")
+                azp_adj = azp_adj * i_zp.data.to(torch.int32).reshape(1, 1)
+            setattr(layer, azp_adj_name, torch.nn.Parameter(azp_adj.contiguous(), requires_grad=False))
         tile_int8_weights_(w_nk)  # in place, marks the memory; shapes that do not tile stay row-major
         layer._kmoe_w_1nk = w_nk.view(1, n, k)  # what the grouped GEMM takes
         setattr(layer, w_q_name, torch.nn.Parameter(w_nk.t(), requires_grad=False))
@@ -96,10 +105,10 @@ class KunlunScaledMMLinearKernel:
         layer's one input scale (static), multiply, rescale by x_max * w_max / 127^2, in x's dtype.
         Output [..., n]."""
         w_q, w_s, x_s, x_zp, azp_adj = self._get_layer_params(layer)
-        if azp_adj is not None or x_zp is not None:
-            raise NotImplementedError("KunlunScaledMMLinearKernel: asymmetric activations are not implemented")
+        if azp_adj is not None:
+            return self._apply_asymmetric(layer, x, w_q, w_s, x_s, x_zp, azp_adj, bias)
         if bias is not None:
-            raise NotImplementedError("KunlunScaledMMLinearKernel: bias is not implemented on this path")
+            raise NotImplementedError("KunlunScaledMMLinearKernel: bias is not implemented on the symmetric path")
         dt = L.act_dtype(x, "KunlunScaledMMLinearKernel")
         w = getattr(layer, "_kmoe_w_1nk", None)
         if w is None:
@@ -121,6 +130,21 @@ class KunlunScaledMMLinearKernel:
             x_q, x_max, _, _ = torch.ops._C.scaled_int8_quant(x2, None, None, True)
             ops._gemm_i8(x_q, x_max, w, w_s.data.reshape(-1), self._row_range(x.device, M), out, n, L.KMOE_ACT_NONE, M)
         return out.reshape(*lead, n)
+
+    def _apply_asymmetric(self, layer, x, w_q, w_s, x_s, x_zp, azp_adj, bias):
+        """Reference: scale_mm.py:60-82. Codes with a zero point (per token, or the layer's static one), the int8
+        product, and the zero-point correction in the epilogue; the weight scale goes back from absmax to scale
+        (/ 127) as there."""
+        L.act_dtype(x, "KunlunScaledMMLinearKernel")
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1]).contiguous()
+        x_q, x_s, x_zp, static = torch.ops._C.scaled_int8_quant(
+            x2, None if x_s is None else x_s.data.to(torch.float32).reshape(1),
+            None if x_zp is None else x_zp.data.to(torch.int32).reshape(1), False)
+        out = torch.ops._C.cutlass_scaled_mm_azp(
+            x_q, w_q, x_s, (w_s.data / 127.0).transpose(0, 1), x.dtype, azp_adj.data, None if static else x_zp,
+            None if bias is None else bias.to(torch.float32).contiguous())
+        return out.reshape(*lead, out.shape[-1])
 
     # Up to this many rows the GEMM runs on the weight-streaming kernel (the one the fused MoE layer
     # runs decode batches and its folded shared expert on): the dense matrix is handed over as the

@@ -179,6 +179,11 @@ int kmoe_quant_i8_rows_azp(const uint16_t* x, int64_t ld_x, int R, int C, int8_t
  *   out[r,c] = dt( scale_a[r or 0] * (scale_b[c or 0] * float(t)) + bias[c] )      f32, products and sum unfused
  * azp_adj [n] int32: the sums of the weight codes over k per output channel. scale_a: one f32 per row
  * (scale_a_rows != 0) or one for the tensor; scale_b: one per channel (scale_b_cols != 0) or one; bias [n] f32 or NULL.
+ * azp_adj == NULL (then azp must be NULL too) is the symmetric product with a bias, torch.ops._C.matmul(..., bias=)
+ * (ops/_custom_ops.py:1811-1845; caller scale_mm.py:83-90): t = acc, and the scales meet it in the order of
+ * kmoe_grouped_gemm_i8 and in its convention - scale_a and scale_b then hold the MAXES (x_pc_max, w_pc_max) and are
+ * divided by 127 here: out = dt( (float(t) * (scale_a / 127)) * (scale_b / 127) + bias ), so that a zero bias
+ * changes nothing.
  */
 int kmoe_scaled_mm_azp_epilogue(const int32_t* acc, int64_t ld_acc, int M, int n, const float* scale_a, int scale_a_rows,
                                 const float* scale_b, int scale_b_cols, const int32_t* azp_adj, const int32_t* azp,

@@ -166,13 +166,13 @@ def scaled_mm_azp(a, w, scale_a, scale_b, azp_adj, azp=None, bias=None, f16=Fals
     M, k = a.shape
     n = w.shape[0]
     scale_a, scale_b = _c(scale_a, np.float32).ravel(), _c(scale_b, np.float32).ravel()
-    azp_adj = _c(azp_adj, np.int32).ravel()
-    assert scale_a.size in (1, M) and scale_b.size in (1, n) and azp_adj.size == n
+    azp_adj = None if azp_adj is None else _c(azp_adj, np.int32).ravel()
+    assert scale_a.size in (1, M) and scale_b.size in (1, n) and (azp_adj is None or azp_adj.size == n)
     azp = None if azp is None else _c(azp, np.int32).ravel()
     bias = None if bias is None else _c(bias, np.float32).ravel()
     out = np.zeros((M, n), np.uint16)
     lib().orc_scaled_mm_azp(_p(a), _p(w), M, n, k, _p(scale_a), int(scale_a.size == M),
-                            _p(scale_b), int(scale_b.size == n), _p(azp_adj), None if azp is None else _p(azp),
+                            _p(scale_b), int(scale_b.size == n), None if azp_adj is None else _p(azp_adj), None if azp is None else _p(azp),
                             None if bias is None else _p(bias), _p(out))
     return out
 

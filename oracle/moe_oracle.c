@@ -317,7 +317,8 @@ ORC_API void orc_quant_i8_rows_azp(const uint16_t* x, int64_t ld_x, int R, int C
 /* cutlass_scaled_mm_azp (ops/_custom_ops.py:1756-1771 forwards it to a closed kernel; restated from the vLLM
  * operator of that name, csrc/quantization/cutlass_w8a8): the int8 product in int32, the zero-point correction in
  * int32 (azp == NULL: it is folded into azp_adj), then scale_a * (scale_b * float(t)) + bias in f32, unfused.
- * a [M,k], w [n,k] int8; azp_adj [n]; scale_a: M values (per_row) or one; scale_b: n values (per_col) or one. */
+ * a [M,k], w [n,k] int8; azp_adj [n]; scale_a: M values (per_row) or one; scale_b: n values (per_col) or one.
+ * azp_adj == NULL: torch.ops._C.matmul with a bias (ops/_custom_ops.py:1811-1845) - the symmetric product. */
 ORC_API void orc_scaled_mm_azp(const int8_t* a, const int8_t* w, int M, int n, int k, const float* scale_a, int per_row,
                                const float* scale_b, int per_col, const int32_t* azp_adj, const int32_t* azp,
                                const float* bias, uint16_t* out) {
@@ -325,9 +326,15 @@ ORC_API void orc_scaled_mm_azp(const int8_t* a, const int8_t* w, int M, int n, i
     for (int c = 0; c < n; ++c) {
       int32_t acc = 0;
       for (int i = 0; i < k; ++i) acc += (int32_t)a[(size_t)r * k + i] * (int32_t)w[(size_t)c * k + i];
-      const int32_t t = (int32_t)((uint32_t)acc - (azp ? (uint32_t)azp[r] : 1u) * (uint32_t)azp_adj[c]);
-      float v = scale_b[per_col ? c : 0] * (float)t;
-      v = scale_a[per_row ? r : 0] * v;
+      const int32_t t = azp_adj ? (int32_t)((uint32_t)acc - (azp ? (uint32_t)azp[r] : 1u) * (uint32_t)azp_adj[c]) : acc;
+      float v;
+      if (azp_adj) { /* vLLM's epilogue */
+        v = scale_b[per_col ? c : 0] * (float)t;
+        v = scale_a[per_row ? r : 0] * v;
+      } else { /* no zero point: the symmetric product, scales in the order of orc_grouped_gemm_i8 */
+        v = (float)t * (scale_a[per_row ? r : 0] / 127.0f); /* the operands are maxes here */
+        v = v * (scale_b[per_col ? c : 0] / 127.0f);
+      }
       if (bias) v = v + bias[c];
       out[(size_t)r * n + c] = f32_to_act(v);
     }

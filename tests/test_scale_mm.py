@@ -88,8 +88,15 @@ def test_apply_weights_matches_the_oracle(M, n, k):
     lod = np.array([0, 3 * M], dtype=np.int32)
     ref, _ = co.grouped_gemm_i8(xq, x_max, wq.numpy()[None], w_max.numpy()[None], lod)
     assert np.array_equal(bits(out.reshape(-1, n)), ref)
-    with pytest.raises(NotImplementedError):
-        kern.apply_weights(layer, x.cuda(), bias=torch.zeros(n, device="cuda"))
+    # with a bias (f32 at the operator, as the reference casts it): a zero bias changes no bit, any other is added in
+    # f32 to the rescaled sum before the one rounding (the oracle's epilogue without a zero point, on the maxes)
+    out0 = kern.apply_weights(layer, x.cuda(), bias=torch.zeros(n, dtype=torch.bfloat16, device="cuda"))
+    bias = torch.randn(n, generator=g).bfloat16()
+    out1 = kern.apply_weights(layer, x.cuda(), bias=bias.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(out0, out)
+    ref1 = co.scaled_mm_azp(xq, wq.numpy(), x_max, w_max.numpy(), None, None, bias.float().numpy())
+    assert np.array_equal(bits(out1.reshape(-1, n)), ref1)
 
 
 @pytest.mark.gpu

@@ -357,7 +357,7 @@ __global__ __launch_bounds__(256) void scaled_mm_azp_kernel(const int32_t* __res
   if (idx >= static_cast<long long>(M) * quads) return;
   const int r = static_cast<int>(idx / quads), c = static_cast<int>(idx % quads) * 4;
   const int4 a = *reinterpret_cast<const int4*>(acc + static_cast<size_t>(r) * ld_acc + c);
-  const int4 adj = *reinterpret_cast<const int4*>(azp_adj + c);
+  const int4 adj = azp_adj ? *reinterpret_cast<const int4*>(azp_adj + c) : make_int4(0, 0, 0, 0);
   const uint32_t z = azp ? static_cast<uint32_t>(azp[r]) : 1u;  // (products and differences wrap like int32 arithmetic)
   const float sa = scale_a[sa_rows ? r : 0];
   const int av[4] = {a.x, a.y, a.z, a.w}, dv[4] = {adj.x, adj.y, adj.z, adj.w};
@@ -365,7 +365,9 @@ __global__ __launch_bounds__(256) void scaled_mm_azp_kernel(const int32_t* __res
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     const int t = static_cast<int>(static_cast<uint32_t>(av[q]) - z * static_cast<uint32_t>(dv[q]));
-    float v = sa * (scale_b[sb_cols ? c + q : 0] * static_cast<float>(t));
+    const float sb = scale_b[sb_cols ? c + q : 0];
+    // (no zero point: the operands are maxes, as the int8 GEMM takes them, and meet the sum in its order)
+    float v = azp_adj ? sa * (sb * static_cast<float>(t)) : (static_cast<float>(t) * (sa / 127.0f)) * (sb / 127.0f);
     if (bias) v = v + bias[c + q];
     o[q] = f32_to_act(v, f16 != 0);
   }
@@ -378,7 +380,7 @@ extern "C" int kmoe_scaled_mm_azp_epilogue(const int32_t* acc, int64_t ld_acc, i
                                            const int32_t* azp_adj, const int32_t* azp, const float* bias, uint16_t* out,
                                            int64_t ld_out, int act_dtype, kmoe_stream_t stream) {
   if (int rc = check_dtype(act_dtype, "scaled_mm_azp_epilogue")) return rc;
-  KMOE_REQUIRE(acc && scale_a && scale_b && azp_adj && out, KMOE_ERR_NULL, "scaled_mm_azp_epilogue: NULL pointer");
+  KMOE_REQUIRE(acc && scale_a && scale_b && out && (azp_adj || !azp), KMOE_ERR_NULL, "scaled_mm_azp_epilogue: NULL pointer");
   KMOE_REQUIRE(M >= 0 && n >= 4 && n % 4 == 0 && ld_acc >= n && ld_acc % 4 == 0 && ld_out >= n && ld_out % 4 == 0,
                KMOE_ERR_SHAPE, "scaled_mm_azp_epilogue: M=%d n=%d strides %lld/%lld (need n %% 4 == 0)", M, n,
                (long long)ld_acc, (long long)ld_out);

@@ -380,11 +380,12 @@ def matmul(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, x_trans: bo
            x_pc_max: Optional[torch.Tensor] = None, w_pc_max: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Dense W8A8 linear: x int8 [M,k] with per-row max, w int8 [n,k] with per-channel
     max -> out [M,n] (reference: ops/_custom_ops.py:1811-1845; caller
-    quantization/kernels/scale_mm.py:83-90). One-expert case of the grouped GEMM."""
+    quantization/kernels/scale_mm.py:83-90). One-expert case of the grouped GEMM; with a bias (f32 [n]) its int32
+    sums are rescaled and the bias added in a second pass (kmoe_scaled_mm_azp_epilogue without a zero point)."""
     if x.dtype != torch.int8 or w.dtype != torch.int8 or x_pc_max is None or w_pc_max is None:
         raise NotImplementedError("matmul: only the int8 path with x_pc_max / w_pc_max is implemented")
-    if x_trans or not w_trans or alpha != 1.0 or beta != 0.0 or bias is not None:
-        raise NotImplementedError("matmul: x_trans / w_trans=False / alpha / beta / bias are not on this path")
+    if x_trans or not w_trans or alpha != 1.0 or beta != 0.0:
+        raise NotImplementedError("matmul: x_trans / w_trans=False / alpha / beta are not on this path")
     if out_dtype not in (_BF16, torch.float16):
         raise NotImplementedError(f"matmul: out_dtype {out_dtype} is not implemented")
     L.require_device(x, w, x_pc_max, w_pc_max)
@@ -398,8 +399,16 @@ def matmul(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, x_trans: bo
     out = torch.empty((M, n), dtype=out_dtype, device=x.device)
     if x_pc_max.numel() == 1 and M != 1:  # one max for the tensor (static quantisation): every row's
         x_pc_max = x_pc_max.reshape(1).expand(M)
-    _gemm_i8(xc, x_pc_max.contiguous(), wc.unsqueeze(0), w_pc_max.contiguous(), _dense_lod(x.device, M), out, n,
-             L.KMOE_ACT_NONE, M)
+    acc = None
+    if bias is not None and M:  # the GEMM leaves its int32 sums as well; the epilogue below rescales them and adds
+        _need(bias.dtype == torch.float32 and bias.numel() == n, "matmul: bias is f32 [n]")
+        L.require_device(bias)
+        acc = torch.empty((M, n), dtype=torch.int32, device=x.device)
+    x_max, w_max = x_pc_max.contiguous(), w_pc_max.contiguous()
+    _gemm_i8(xc, x_max, wc.unsqueeze(0), w_max, _dense_lod(x.device, M), out, n, L.KMOE_ACT_NONE, M, acc_out=acc)
+    if acc is not None:
+        L.check(L.lib.kmoe_scaled_mm_azp_epilogue(L.ptr(acc), n, M, n, L.ptr(x_max), 1, L.ptr(w_max), 1, None, None,
+                                                  L.ptr(bias.contiguous()), L.ptr(out), n, L.act_dtype(out), L.stream()))
     return out
 
 

@@ -108,7 +108,13 @@ class KunlunScaledMMLinearKernel:
         if azp_adj is not None:
             return self._apply_asymmetric(layer, x, w_q, w_s, x_s, x_zp, azp_adj, bias)
         if bias is not None:
-            raise NotImplementedError("KunlunScaledMMLinearKernel: bias is not implemented on the symmetric path")
+            # the reference's call (scale_mm.py:83-90): quantise, then matmul with the f32 bias
+            x2 = x.reshape(-1, x.shape[-1]).contiguous()
+            x_q, x_s2, _, static = torch.ops._C.scaled_int8_quant(
+                x2, None if x_s is None else x_s.data.to(torch.float32).reshape(1), None, True)
+            out = torch.ops._C.matmul(x_q, w_q.transpose(0, 1), x.dtype, x_pc_max=x_s2 * 127.0 if static else x_s2,
+                                      w_pc_max=w_s.data, bias=bias.to(torch.float32).contiguous())
+            return out.reshape(*x.shape[:-1], out.shape[-1])
         dt = L.act_dtype(x, "KunlunScaledMMLinearKernel")
         w = getattr(layer, "_kmoe_w_1nk", None)
         if w is None:

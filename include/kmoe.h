@@ -115,6 +115,16 @@ int kmoe_align(const int32_t* topk_ids, int P, int E, int32_t* moe_index,
                void* workspace, size_t workspace_bytes, kmoe_stream_t stream);
 
 /*
+ * The same sort for an expert-parallel share: the ids are global and this launch owns the experts
+ * [first_expert, first_expert + E) of them - the id shift of the reference's expert-parallel loop
+ * (experts_id = ep_rank * num_local_experts + i, ops/_kunlun_ops.py:677-689). Pairs routed elsewhere get no
+ * sorted row (moe_index = -1, which kmoe_combine skips); lod counts the local pairs only.
+ */
+int kmoe_align_local(const int32_t* topk_ids, int P, int E, int first_expert, int32_t* moe_index,
+                     int32_t* sorted_src, int32_t* expert_m, int32_t* lod,
+                     void* workspace, size_t workspace_bytes, kmoe_stream_t stream);
+
+/*
  * Gather of activation rows into sorted order: the data part of
  * kunlun_ops.moe_pre_sorted (output moe_expand, compressed_tensors_moe.py:173-196).
  *   dst[r, :] = src[sorted_src[r] / K, :]   for r in [0,P); 16-bit elements,
@@ -551,6 +561,11 @@ typedef struct kmoe_moe_args {
   int32_t tile_variant;  /* INT8, tuning: 0, or the `variant` (5-12) handed to the two routed GEMMs when the batch
                             runs on the tile kernel (more than 10 rows per expert); ignored otherwise */
   int32_t w_scale_layout; /* W4A16: KMOE_S_* of w13_scale and w2_scale                                  */
+  /* An expert-parallel share (ops/_kunlun_ops.py:640-696: each rank holds num_local_experts of the experts and
+     computes what the pairs routed to them contribute; the sum over ranks is the caller's all-reduce). The routing
+     runs over E_global experts (logits [M,E_global], bias [E_global], w_gate [E_global,H]; K <= E_global); the
+     weights are those of the E experts [first_expert, first_expert + E). 0 / 0: one GPU holds every expert. */
+  int32_t E_global, first_expert;
 } kmoe_moe_args;
 
 #define KMOE_STAGE_ROUTING 0

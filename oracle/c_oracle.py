@@ -374,12 +374,15 @@ def grouped_gemm_bf16_bias(a_bits, w_bits, bias_bits, lod, act=0, row_src=None, 
 
 
 def forward_bf16(x_bits, logits, w13_bits, w2_bits, K, scoring="softmax", renormalize=True, n_group=1, topk_group=1,
-                 routed_scale=1.0, bias=None, w13_bias=None, w2_bias=None, alpha=1.702, limit=7.0, f16=False):
+                 routed_scale=1.0, bias=None, w13_bias=None, w2_bias=None, alpha=1.702, limit=7.0, f16=False,
+                 first_expert=0):
     """Unquantized layer in the stage order of KunlunOps.fused_moe (ops/_kunlun_ops.py:412-637); with
-    expert biases, its gpt-oss branch (:433-468): interleaved gate/up, swigluoai."""
+    expert biases, its gpt-oss branch (:433-468): interleaved gate/up, swigluoai. first_expert: the weights are
+    the experts [first_expert, first_expert + E) of those the logits run over (an expert-parallel share,
+    :677-689): pairs routed elsewhere get no sorted row and add nothing."""
     E = w13_bits.shape[0]
     w, ids = _route(logits, K, scoring, renormalize, n_group, topk_group, routed_scale, bias)
-    moe_index, src, _, lod = align(ids, E)
+    moe_index, src, _, lod = align(ids - np.int32(first_expert), E)
     if w13_bias is not None or w2_bias is not None:
         if f16:
             raise NotImplementedError("the expert-bias branch is restated for bf16 only")

@@ -146,10 +146,11 @@ def w8a8_moe(x, logits, w13, w13_max, w2, w2_max, K, scoring="softmax", renormal
 
 
 # ------------------------------------------------------------ layer: bf16
-def bf16_moe(x, logits, w13, w2, K, renormalize=True):
+def bf16_moe(x, logits, w13, w2, K, renormalize=True, ep_rank=0):
     """KunlunOps.fused_moe_ep restated line for line in meaning
     (ops/_kunlun_ops.py:655-696): weights cast to the activation dtype, product
-    and sum over K in that dtype."""
+    and sum over K in that dtype. The weights are the local experts of rank ep_rank
+    (global ids ep_rank * num_local_experts + i, :677-678); logits run over all experts."""
     M, H = x.shape
     E = w13.shape[0]
     w, ids = softmax_topk(logits, K, False)
@@ -160,7 +161,7 @@ def bf16_moe(x, logits, w13, w2, K, renormalize=True):
     repeat_x = x.repeat_interleave(K, dim=0)
     flat = ids.reshape(-1)
     for e in range(E):
-        sel = flat == e
+        sel = flat == ep_rank * E + e
         if sel.sum():
             cur = repeat_x[sel]
             out[sel] = silu_and_mul(cur @ w13[e].T) @ w2[e].T

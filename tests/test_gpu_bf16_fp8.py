@@ -232,8 +232,43 @@ def test_bf16_golden_fixture_and_ep_entry():
     torch.cuda.synchronize()
     assert rel_l2(out, from_bits(g["out"])) <= REL_L2_BF16
     assert torch.equal(out, out2)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError):  # a rank beyond 0 needs logits over more experts than the weights hold
         KunlunOps.fused_moe_ep(x, w13, w2, logits, 1, int(g["K"]), True)
+
+
+@pytest.mark.parametrize("M,renormalize", [(24, True), (24, False), (700, True)])
+def test_fused_moe_ep_shares(M, renormalize):
+    """KunlunOps.fused_moe_ep as an expert-parallel rank calls it (ops/_kunlun_ops.py:640-696): logits over all 16
+    experts, the weights of 4 of them, ep_rank = 0..3. Every share against the oracle's share and against the
+    reference's loop restated in torch; a token none of whose experts are local gets exact zeros; the shares add
+    up to the layer's output (what the ranks' all-reduce makes)."""
+    from vllm_kunlun_amd.ops._kunlun_ops import KunlunOps
+    from vllm_kunlun_amd import _plan
+    Eg, El, K, H, I = 16, 4, 4, 256, 128
+    g = torch.Generator().manual_seed(M)
+    x = torch.randn(M, H, generator=g).bfloat16()
+    logits = torch.randn(M, Eg, generator=g)
+    w13 = (torch.randn(Eg, 2 * I, H, generator=g) * 0.05).bfloat16()
+    w2 = (torch.randn(Eg, H, I, generator=g) * 0.05).bfloat16()
+    _, ids = co.softmax_topk(logits.numpy(), K, renormalize)
+    total = torch.zeros(M, H, dtype=torch.float64)
+    for rank in range(Eg // El):
+        lo = rank * El
+        w13_r, w2_r = w13[lo:lo + El].contiguous().cuda(), w2[lo:lo + El].contiguous().cuda()
+        if rank % 2:  # tiled local weights as the method keeps them, row-major ones as a caller may hand them over
+            assert _plan.tile_pair_(w13_r, w2_r)
+        out = KunlunOps.fused_moe_ep(x.cuda(), w13_r, w2_r, logits.cuda(), rank, K, renormalize)
+        torch.cuda.synchronize()
+        ref = co.forward_bf16(bits(x), logits.numpy(), bits(w13[lo:lo + El]), bits(w2[lo:lo + El]), K, "softmax",
+                              renormalize, first_expert=lo)
+        assert rel_l2(out, from_bits(ref)) <= REL_L2_BF16
+        assert rel_l2(out, tm.bf16_moe(x, logits, w13[lo:lo + El], w2[lo:lo + El], K, renormalize, ep_rank=rank)) <= REL_L2_BF16
+        elsewhere = ~((ids >= lo) & (ids < lo + El)).any(1)
+        assert elsewhere.any() or M > 100
+        assert not out.cpu()[torch.from_numpy(elsewhere)].any()
+        total += out.cpu().double()
+    whole = tm.bf16_moe(x, logits, w13, w2, K, renormalize)
+    assert rel_l2(total, whole) <= REL_L2_BF16
 
 
 def test_moe_fc_op_bf16_swish_glu():
@@ -618,6 +653,15 @@ def test_w4a16_layer_on_the_packed_weights(native, group_size, M):
     torch.cuda.synchronize()
     ref3 = co.forward_bf16(bits(x), logits.cpu().numpy(), w13, w2, K, scoring="sigmoid", bias=bias.numpy())
     assert rel_l2(out3, from_bits(ref3)) <= REL_L2_BF16
+    # as rank 1 of 2 expert-parallel ranks: logits over 2 E experts, the layer's weights being experts E .. 2 E - 1
+    ep = SimpleNamespace(experts_per_token=K, use_ep=True, ep_rank=1)
+    method.moe, keep = ep, method.moe
+    wide = torch.randn(M, 2 * E, generator=gx, device="cuda")
+    out4 = method.apply(layer, x, wide, K, True)
+    torch.cuda.synchronize()
+    method.moe = keep
+    ref4 = co.forward_bf16(bits(x), wide.cpu().numpy(), w13, w2, K, first_expert=E)
+    assert rel_l2(out4, from_bits(ref4)) <= REL_L2_BF16
     with pytest.raises(NotImplementedError):
         method.apply(layer, x, logits, K, True, expert_map=torch.arange(E, device="cuda"))
     with pytest.raises(NotImplementedError):

@@ -289,3 +289,47 @@ def test_layer_with_paced_tiles_gives_the_same_bits():
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
     oi = _oracle_inputs(sl)
     assert np.array_equal(bits(outs[1]), co.forward_w8a8(**oi))
+
+
+@pytest.mark.parametrize("M", [48, 1500])
+@pytest.mark.parametrize("scoring", ["softmax", "sigmoid"])
+def test_int8_layer_as_an_expert_parallel_share(M, scoring):
+    """kmoe_moe_forward with E_global / first_expert (the share of one expert-parallel rank: routing over all 32
+    experts, the weights of 8 of them): bit for bit the oracle's stages on the pairs routed to the local experts,
+    on the weight-streaming path (48 tokens) and on the tile kernel (1500), with grouped sigmoid routing and a
+    correction bias over the global experts; pairs routed elsewhere add nothing."""
+    from vllm_kunlun_amd import _lib as L, _plan
+    from oracle import torch_moe as tm
+    Eg, El, K, H, I = 32, 8, 4, 256, 128
+    g = torch.Generator().manual_seed(M + len(scoring))
+    x = (torch.randn(M, H, generator=g) * 1.5).bfloat16()
+    logits = torch.randn(M, Eg, generator=g)
+    bias = torch.randn(Eg, generator=g) * 0.1 if scoring == "sigmoid" else None
+    route = dict(scoring_func=scoring, renormalize=True, num_expert_group=4 if scoring == "sigmoid" else None,
+                 topk_group=2 if scoring == "sigmoid" else None, routed_scaling_factor=2.5 if scoring == "sigmoid" else 1.0,
+                 e_score_correction_bias=None if bias is None else bias.cuda())
+    w, ids = co._route(logits.numpy(), K, scoring, True, 4, 2, 2.5 if scoring == "sigmoid" else 1.0,
+                       None if bias is None else bias.numpy())
+    for rank in (0, 3):
+        lo = rank * El
+        gw = torch.Generator().manual_seed(100 + rank)
+        w13q, s13 = tm.quantize_weight_per_channel((torch.randn(El * 2 * I, H, generator=gw) * 0.05))
+        w2q, s2 = tm.quantize_weight_per_channel((torch.randn(El * H, I, generator=gw) * 0.05))
+        w13q, w2q = w13q.view(El, 2 * I, H), w2q.view(El, H, I)
+        w13_max, w2_max = (s13 * 127.0).view(El, 2 * I), (s2 * 127.0).view(El, H)
+        d13, d2 = w13q.clone().cuda(), w2q.clone().cuda()
+        assert _plan.tile_pair_(d13, d2)
+        out = torch.empty(M, H, dtype=torch.bfloat16, device="cuda")
+        plan = _plan.make_moe_plan(L.KMOE_FMT_INT8, x.cuda(), logits.cuda(), out, K, d13, d2, w13_max.cuda(),
+                                   w2_max.cuda(), first_expert=lo, **route)
+        plan()
+        torch.cuda.synchronize()
+        # the oracle's stages on the local pairs
+        moe_index, src, _, lod = co.align(ids - np.int32(lo), El)
+        xq, x_max = co.quant_i8_rows(bits(x))
+        act, _ = co.grouped_gemm_i8(xq, x_max, w13q.numpy(), w13_max.numpy(), lod, act=1, row_src=src, src_div=K)
+        aq, a_max = co.quant_i8_rows(act)
+        down, _ = co.grouped_gemm_i8(aq, a_max, w2q.numpy(), w2_max.numpy(), lod)
+        ref = co.combine(down, moe_index, w)
+        assert np.array_equal(bits(out), ref), f"rank {rank}"
+        assert 0 < int(lod[-1]) < M * K

@@ -907,3 +907,26 @@ def test_scaled_mm_azp_against_the_dequantised_product():
     exact = (a1.astype(np.int64) - z1[:, None]) @ w1.astype(np.int64).T
     got = co.scaled_mm_azp(a1, w1, np.ones(1, np.float32), np.ones(1, np.float32), w1.astype(np.int64).sum(1), z1)
     assert np.array_equal(from_bits(got).double().numpy().astype(np.int64), exact)
+
+
+def test_expert_parallel_share_of_the_unquantized_layer():
+    """forward_bf16(first_expert=...) against the reference's expert-parallel loop restated in torch
+    (ops/_kunlun_ops.py:655-696 with ep_rank): every share within the bf16 tolerance, exact zeros for tokens
+    routed elsewhere, and the shares add up to the layer over all experts."""
+    g = torch.Generator().manual_seed(3)
+    M, Eg, El, K, H, I = 40, 12, 3, 3, 64, 32
+    x = torch.randn(M, H, generator=g).bfloat16()
+    logits = torch.randn(M, Eg, generator=g)
+    w13 = (torch.randn(Eg, 2 * I, H, generator=g) * 0.1).bfloat16()
+    w2 = (torch.randn(Eg, H, I, generator=g) * 0.1).bfloat16()
+    _, ids = co.softmax_topk(logits.numpy(), K, True)
+    total = torch.zeros(M, H, dtype=torch.float64)
+    for rank in range(Eg // El):
+        lo = rank * El
+        got = from_bits(co.forward_bf16(bits(x), logits.numpy(), bits(w13[lo:lo + El]), bits(w2[lo:lo + El]), K,
+                                        first_expert=lo))
+        assert rel_l2(got, tm.bf16_moe(x, logits, w13[lo:lo + El], w2[lo:lo + El], K, True, ep_rank=rank)) <= 1e-2
+        elsewhere = torch.from_numpy(~((ids >= lo) & (ids < lo + El)).any(1))
+        assert elsewhere.any() and not got[elsewhere].any()
+        total += got.double()
+    assert rel_l2(total, from_bits(co.forward_bf16(bits(x), logits.numpy(), bits(w13), bits(w2), K)).double()) <= 1e-2

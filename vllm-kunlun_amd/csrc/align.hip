@@ -35,7 +35,15 @@ __device__ inline void wave_match_rank(int key, int bits, int& rank, int& count)
   count = live ? __builtin_popcountll(same) : 0;
 }
 
-__device__ inline int load_key(const int32_t* __restrict__ ids, int j, int end, int E) {
+// The expert ids of the routed pairs as the routing kernel wrote them, seen by a launch that owns the experts
+// [first, first + E) of them (an expert-parallel share; first = 0: all of them): ids outside come out outside [0, E).
+struct IdView {
+  const int32_t* ids;
+  int first;
+  __device__ int operator[](int j) const { return ids[j] - first; }
+};
+
+__device__ inline int load_key(const IdView ids, int j, int end, int E) {
   if (j >= end) return -1;
   const int e = ids[j];
   return static_cast<unsigned>(e) < static_cast<unsigned>(E) ? e : -1;  // ids outside [0,E): no sorted row
@@ -45,7 +53,7 @@ __device__ inline int load_key(const int32_t* __restrict__ ids, int j, int end, 
 // Leaves in wcnt[w][e] the number of expert-e pairs of this chunk in waves < w and
 // returns to thread e < E the chunk's total for expert e (0 to the other threads).
 // `wcnt` is LDS scratch [waves][E].
-__device__ inline int count_chunk(const int32_t* __restrict__ ids, int begin, int end, int E, int steps,
+__device__ inline int count_chunk(const IdView ids, int begin, int end, int E, int steps,
                                   int* wcnt) {
   const int waves = blockDim.x >> 6;
   const int wave = threadIdx.x >> 6;
@@ -75,7 +83,7 @@ __device__ inline int count_chunk(const int32_t* __restrict__ ids, int begin, in
 
 // Scatter phase: pair j of expert e lands at base[e] + wcnt[wave][e] + (rank among the
 // wave's earlier pairs of e). Call after count_chunk and a barrier that publishes base.
-__device__ inline void scatter_chunk(const int32_t* __restrict__ ids, int begin, int end, int E, int steps,
+__device__ inline void scatter_chunk(const IdView ids, int begin, int end, int E, int steps,
                                      const int* base, int* wcnt, int32_t* __restrict__ moe_index,
                                      int32_t* __restrict__ sorted_src) {
   const int wave = threadIdx.x >> 6;
@@ -129,7 +137,7 @@ __device__ inline void scan_experts(int my_count /* thread e < E */, int E, int*
 
 // Single-workgroup path (P <= kSingleMaxP); blockDim.x is 256 or 1024, >= E.
 __global__ __launch_bounds__(kThreads) void align_single_kernel(
-    const int32_t* __restrict__ ids, int P, int E, int steps, int32_t* __restrict__ moe_index,
+    const IdView ids, int P, int E, int steps, int32_t* __restrict__ moe_index,
     int32_t* __restrict__ sorted_src, int32_t* __restrict__ expert_m, int32_t* __restrict__ lod) {
   extern __shared__ int lds[];
   int* wtot = lds;          // [16]
@@ -141,7 +149,7 @@ __global__ __launch_bounds__(kThreads) void align_single_kernel(
 }
 
 // Multi-workgroup path, kernel 1: chunk histograms -> hist[chunk][E].
-__global__ __launch_bounds__(kThreads) void align_hist_kernel(const int32_t* __restrict__ ids, int P, int E,
+__global__ __launch_bounds__(kThreads) void align_hist_kernel(const IdView ids, int P, int E,
                                                              int32_t* __restrict__ hist) {
   extern __shared__ int lds[];
   for (int e = threadIdx.x; e < E; e += kThreads) lds[e] = 0;
@@ -193,7 +201,7 @@ __global__ __launch_bounds__(kThreads) void align_scan_kernel(int E, int n_chunk
 }
 
 // Kernel 3: stable scatter of each chunk.
-__global__ __launch_bounds__(kThreads) void align_scatter_kernel(const int32_t* __restrict__ ids, int P, int E,
+__global__ __launch_bounds__(kThreads) void align_scatter_kernel(const IdView ids, int P, int E,
                                                                 const int32_t* __restrict__ hist,
                                                                 int32_t* __restrict__ moe_index,
                                                                 int32_t* __restrict__ sorted_src) {
@@ -246,7 +254,15 @@ extern "C" size_t kmoe_align_workspace_bytes(int P, int E) {
 extern "C" int kmoe_align(const int32_t* topk_ids, int P, int E, int32_t* moe_index, int32_t* sorted_src,
                           int32_t* expert_m, int32_t* lod, void* workspace, size_t workspace_bytes,
                           kmoe_stream_t stream) {
-  KMOE_REQUIRE(lod && (P == 0 || (topk_ids && moe_index)), KMOE_ERR_NULL, "align: NULL pointer");
+  return kmoe_align_local(topk_ids, P, E, 0, moe_index, sorted_src, expert_m, lod, workspace, workspace_bytes, stream);
+}
+
+extern "C" int kmoe_align_local(const int32_t* ids_global, int P, int E, int first_expert, int32_t* moe_index,
+                                int32_t* sorted_src, int32_t* expert_m, int32_t* lod, void* workspace,
+                                size_t workspace_bytes, kmoe_stream_t stream) {
+  const IdView topk_ids{ids_global, first_expert};
+  KMOE_REQUIRE(first_expert >= 0, KMOE_ERR_SHAPE, "align: first_expert=%d", first_expert);
+  KMOE_REQUIRE(lod && (P == 0 || (ids_global && moe_index)), KMOE_ERR_NULL, "align: NULL pointer");
   KMOE_REQUIRE(E >= 1 && E <= kMaxE, KMOE_ERR_SHAPE, "align: E=%d outside [1,%d]", E, kMaxE);
   KMOE_REQUIRE(P >= 0 && P <= (1 << 24), KMOE_ERR_SHAPE, "align: P=%d outside [0,2^24]", P);
   hipStream_t s = as_stream(stream);

@@ -54,8 +54,12 @@ int check_shape(const kmoe_moe_args* a) {
   const int mult = a->format == KMOE_FMT_FP8_BLOCK || a->format == KMOE_FMT_W4A16 ? 128 : 16;
   KMOE_REQUIRE(a->H % mult == 0 && a->I % mult == 0, KMOE_ERR_SHAPE,
                "moe_forward: H=%d and I=%d must be multiples of %d", a->H, a->I, mult);
-  KMOE_REQUIRE(a->K <= a->E && a->K <= 64 && a->E <= 1024, KMOE_ERR_SHAPE, "moe_forward: K=%d E=%d out of range", a->K,
-               a->E);
+  const int Eg = a->E_global > 0 ? a->E_global : a->E;
+  KMOE_REQUIRE(a->K <= Eg && a->K <= 64 && a->E <= 1024 && Eg <= 1024, KMOE_ERR_SHAPE,
+               "moe_forward: K=%d E=%d E_global=%d out of range", a->K, a->E, Eg);
+  KMOE_REQUIRE(a->first_expert >= 0 && a->first_expert + a->E <= Eg, KMOE_ERR_SHAPE,
+               "moe_forward: experts [%d, %d) are not among the %d the routing runs over", a->first_expert,
+               a->first_expert + a->E, Eg);
   KMOE_REQUIRE(a->I_shared >= 0 && a->I_shared % mult == 0, KMOE_ERR_SHAPE,
                "moe_forward: I_shared=%d must be a non-negative multiple of %d", a->I_shared, mult);
   KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "moe_forward: M*K too large");
@@ -81,8 +85,15 @@ int check_shape(const kmoe_moe_args* a) {
 // the stream kernels re-read the weights once per 16-64 rows of an expert, so their time grows with the rows
 // per expert; the tile kernel's hardly does. Measured cross-over with 64-row tiles: 10-12 rows per expert on
 // both the Qwen3 and the DeepSeek-V3 shape.
-bool use_stream_path(const kmoe_moe_args* a) {
+// Pairs this launch expects to land on its own experts: all of them, or the share of an expert-parallel rank under
+// uniform routing (the kernels are chosen by the rows per expert; any choice is correct for any routing).
+long long local_pairs(const kmoe_moe_args* a) {
   const long long P = static_cast<long long>(a->M) * a->K;
+  return a->E_global > a->E ? (P * a->E + a->E_global - 1) / a->E_global : P;
+}
+
+bool use_stream_path(const kmoe_moe_args* a) {
+  const long long P = local_pairs(a);
   // a row-major shared expert cannot read the chunk-major codes this path quantises x into
   return a->format == KMOE_FMT_INT8 && a->w_layout == KMOE_W_TILED && (P + a->E - 1) / a->E <= 10 && a->M <= 1024 &&
          (a->I_shared == 0 || a->ws_layout == KMOE_W_TILED);
@@ -97,7 +108,7 @@ bool use_stream_path(const kmoe_moe_args* a) {
 bool fold_shared(const kmoe_moe_args* a) {
   if (a->I_shared <= 0 || a->I_shared != a->I || a->ws_layout != a->w_layout) return false;
   if (a->format == KMOE_FMT_INT8) return true;
-  const long long P = static_cast<long long>(a->M) * a->K;
+  const long long P = local_pairs(a);
   return a->format == KMOE_FMT_FP8_BLOCK && a->w_layout == KMOE_W_TILED && a->H <= 8192 && a->I <= 8192 &&
          (P + a->E - 1) / a->E > 10;
 }
@@ -316,9 +327,9 @@ extern "C" int kmoe_moe_workspace_layout(const kmoe_moe_args* a, kmoe_moe_layout
   L->sh_actmax = take(quant ? Ms * 4 * (fp8 ? Is / 128 : 1) : 0);
   L->sh_out = take(Ms * H * 2);
   int ks = 0, mf = 0;
-  if (a->w_gate && a->H % 32 == 0) router_plan(a->M, a->H, a->E, &ks, &mf);
+  if (a->w_gate && a->H % 32 == 0) router_plan(a->M, a->H, a->E_global > 0 ? a->E_global : a->E, &ks, &mf);
   L->n_logit_planes = ks;
-  L->logit_planes = take(ks ? static_cast<size_t>(ks) * M * E * 4 : 0);
+  L->logit_planes = take(ks ? static_cast<size_t>(ks) * M * (a->E_global > 0 ? a->E_global : E) * 4 : 0);
   L->total_bytes = off;
   L->codes_chunked = use_stream_path(a) ? 1 : 0;
   return KMOE_OK;
@@ -422,6 +433,7 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
   int32_t* sorted_src = static_cast<int32_t*>(at(L.sorted_src));
   int32_t* lod = static_cast<int32_t*>(at(L.lod));
   const int M = a->M, H = a->H, E = a->E, K = a->K, I = a->I, P = M * K;
+  const int Eg = a->E_global > 0 ? a->E_global : E;  // experts the routing runs over (an expert-parallel share: more than E)
   int rc = KMOE_OK;
   auto mark = [&](int stage, int end) {
     if (!a->stage_events) return;
@@ -439,17 +451,17 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
   size_t plane_stride = 0;
   if (!logits) {
     int mf = 0;
-    router_plan(M, H, E, &planes, &mf);
+    router_plan(M, H, Eg, &planes, &mf);
     float* buf = static_cast<float*>(at(L.logit_planes));
-    plane_stride = static_cast<size_t>(M) * E;
-    rc = router_gemm_planes(a->x, H, a->w_gate, M, H, E, buf, plane_stride, E, planes, mf, as_stream(stream),
+    plane_stride = static_cast<size_t>(M) * Eg;
+    rc = router_gemm_planes(a->x, H, a->w_gate, M, H, Eg, buf, plane_stride, Eg, planes, mf, as_stream(stream),
                             a->act_dtype == KMOE_DT_F16);
     if (rc) return rc;
     logits = buf;
   }
   // 1. routing; on the int8 decode path together with step 3 (independent work, one launch)
   if (a->format == KMOE_FMT_INT8) {
-    rc = fused_route_quant_i8(logits, planes, plane_stride, a->bias, M, E, K, a->scoring == KMOE_SCORE_SIGMOID, a->renormalize, a->n_group,
+    rc = fused_route_quant_i8(logits, planes, plane_stride, a->bias, M, Eg, K, a->scoring == KMOE_SCORE_SIGMOID, a->renormalize, a->n_group,
                               a->topk_group, a->routed_scale, topk_w, topk_ids, a->x, H, static_cast<int8_t*>(at(L.xq)),
                               static_cast<float*>(at(L.xmax)), stream_mode ? 1 : 0, a->act_dtype == KMOE_DT_F16,
                               as_stream(stream));
@@ -458,23 +470,23 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
     rc = KMOE_OK;
   }
   if (!quant_done && planes > 1) {  // the stand-alone routing kernels take finished logits: add the planes into plane 0
-    rc = router_reduce(logits, plane_stride, planes, M, E, static_cast<float*>(at(L.logit_planes)), E, as_stream(stream));
+    rc = router_reduce(logits, plane_stride, planes, M, Eg, static_cast<float*>(at(L.logit_planes)), Eg, as_stream(stream));
     if (rc) return rc;
   }
   if (quant_done) {
     // both done
   } else if (a->scoring == KMOE_SCORE_SOFTMAX) {
-    rc = kmoe_softmax_topk(logits, M, E, K, a->renormalize, topk_w, topk_ids, stream);
+    rc = kmoe_softmax_topk(logits, M, Eg, K, a->renormalize, topk_w, topk_ids, stream);
   } else {
-    rc = kmoe_sigmoid_group_topk_norm(logits, a->bias, M, E, K, a->n_group, a->topk_group, a->routed_scale, topk_w,
+    rc = kmoe_sigmoid_group_topk_norm(logits, a->bias, M, Eg, K, a->n_group, a->topk_group, a->routed_scale, topk_w,
                                       topk_ids, stream);
   }
   if (rc) return rc;
   mark(KMOE_STAGE_ROUTING, 1);
   // 2. stable sort of the routed pairs by expert
   mark(KMOE_STAGE_ALIGN, 0);
-  rc = kmoe_align(topk_ids, P, E, moe_index, sorted_src, static_cast<int32_t*>(at(L.expert_m)), lod, at(L.align_ws),
-                  kmoe_align_workspace_bytes(P, E), stream);
+  rc = kmoe_align_local(topk_ids, P, E, a->first_expert, moe_index, sorted_src, static_cast<int32_t*>(at(L.expert_m)), lod,
+                        at(L.align_ws), kmoe_align_workspace_bytes(P, E), stream);
   if (rc) return rc;
   mark(KMOE_STAGE_ALIGN, 1);
   // 3. quantise each TOKEN row once (the reference quantises the K-times expanded copy; same values)
@@ -532,7 +544,7 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
   routed.stream = stream_mode;
   routed.x_count = M;
   if (a->format == KMOE_FMT_INT8 && !stream_mode && a->w_layout == KMOE_W_TILED && a->tile_variant >= 5 &&
-      a->tile_variant <= 12 && (static_cast<long long>(P) + E - 1) / E > 10 && H >= 128 && I >= 128)
+      a->tile_variant <= 12 && (local_pairs(a) + E - 1) / E > 10 && H >= 128 && I >= 128)
     routed.variant = a->tile_variant;
   const bool fold = fold_shared(a);
   if (fold) {

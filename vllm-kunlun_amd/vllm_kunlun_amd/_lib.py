@@ -90,6 +90,7 @@ class MoEArgs(C.Structure):
         ("act_limit", C.c_float), ("ws_layout", C.c_int32),
         ("w13_scale", C.c_void_p), ("w2_scale", C.c_void_p), ("group_size", C.c_int32),
         ("act_dtype", C.c_int32), ("shared_scale", C.c_float), ("tile_variant", C.c_int32), ("w_scale_layout", C.c_int32),
+        ("E_global", C.c_int32), ("first_expert", C.c_int32),
     ]
 
 
@@ -123,6 +124,7 @@ def _load() -> C.CDLL:
         "kmoe_dequant_w4_bf16": (i32, [vp, vp, i64, i32, i32, vp, vp]),
         "kmoe_dequant_w4": (i32, [vp, vp, i64, i32, i32, vp, i32, vp]),
         "kmoe_tile_scales_w4": (i32, [vp, vp, i32, i32, i32, vp]),
+        "kmoe_align_local": (i32, [vp, i32, i32, i32, vp, vp, vp, vp, vp, sz, vp]),
         "kmoe_scaled_mm_azp_epilogue": (i32, [vp, i64, i32, i32, vp, i32, vp, i32, vp, vp, vp, vp, i64, i32, vp]),
         "kmoe_quant_i8_static": (i32, [vp, i64, i32, i32, vp, vp, vp, i64, i32, vp]),
         "kmoe_quant_i8_rows_azp": (i32, [vp, i64, i32, i32, vp, i64, vp, vp, i32, vp]),
@@ -158,7 +160,7 @@ EXPORTS = (
     "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_w4a16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
     "kmoe_moe_workspace_layout", "kmoe_moe_forward", "kmoe_router_gemm_workspace_bytes", "kmoe_router_gemm_bf16",
     "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16", "kmoe_dequant_w4", "kmoe_moe_forward_static",
-    "kmoe_quant_i8_static", "kmoe_quant_i8_rows_azp", "kmoe_tile_scales_w4", "kmoe_scaled_mm_azp_epilogue",
+    "kmoe_quant_i8_static", "kmoe_quant_i8_rows_azp", "kmoe_tile_scales_w4", "kmoe_scaled_mm_azp_epilogue", "kmoe_align_local",
     "kmoe_quant_i8_rows_dt", "kmoe_quant_i8_rows_chunked_dt", "kmoe_silu_and_mul_dt", "kmoe_combine_dt", "kmoe_router_gemm",
 )
 STATIC_WORKSPACE_BYTES = 64 << 20

@@ -207,7 +207,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
                   router_weight: Optional[torch.Tensor] = None, w13_bias: Optional[torch.Tensor] = None,
                   w2_bias: Optional[torch.Tensor] = None, activation: str = "silu", act_alpha: float = 1.702,
                   act_limit: float = 7.0, group_size: Optional[int] = None, tile_variant: int = 0,
-                  shared_scale: float = 1.0) -> MoEPlan:
+                  shared_scale: float = 1.0, first_expert: int = 0) -> MoEPlan:
     """x bf16 [M,H] (or float16 with int8 or unquantized weights, the latter then float16 too), logits f32 [M,E], out [M,H] like x; w13 [E,2I,H], w2 [E,H,I] in the
     format's dtype; w13_aux/w2_aux: per-channel maxes (int8) or block scales (fp8), None for bf16.
     shared_expert: (ws13 [2Is,H], ws13_aux, ws2 [H,Is], ws2_aux) in the same format.
@@ -217,7 +217,10 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     KMOE_FMT_W4A16: w13 [E,2I,H/2] and w2 [E,H,I/2] uint8 (two 4-bit codes per byte), tiled;
     w13_aux/w2_aux their group scales [E,2I,H/group_size], [E,H,I/group_size] in x's dtype.
     shared_scale multiplies the shared expert's output before it is added (the float16 form of the caller's
-    epilogue, models/deepseek_v2.py:286-292). tile_variant: a tuning variant of the int8 tile kernel for the routed GEMMs (kmoe_moe_args.tile_variant)."""
+    epilogue, models/deepseek_v2.py:286-292). tile_variant: a tuning variant of the int8 tile kernel for the routed GEMMs (kmoe_moe_args.tile_variant).
+    An expert-parallel share (ops/_kunlun_ops.py:640-696): logits [M,E_global] (correction bias [E_global], router
+    weight [E_global,H]) with more experts than the weights hold, and first_expert = ep_rank * E: the routing runs
+    over all of them, the pairs routed to [first_expert, first_expert + E) are computed, the others add nothing."""
     if scoring_func not in ("softmax", "sigmoid"):
         raise ValueError(f"Unsupported scoring_func: {scoring_func}")
     if logits is None and router_weight is None:
@@ -242,10 +245,16 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     if w4:
         H *= 2  # two codes per byte
     M = x.shape[0]
-    if tuple(x.shape) != (M, H) or tuple(out.shape) != (M, H) or (logits is not None and tuple(logits.shape) != (M, E)):
+    Eg = logits.shape[-1] if logits is not None else router_weight.shape[0]  # experts the routing runs over
+    if tuple(x.shape) != (M, H) or tuple(out.shape) != (M, H) or (logits is not None and tuple(logits.shape) != (M, Eg)):
         raise ValueError("moe plan: x/out must be [M,H] and logits [M,E]")
-    if logits is None and (router_weight.dtype != x.dtype or tuple(router_weight.shape) != (E, H)):
+    if logits is None and (router_weight.dtype != x.dtype or tuple(router_weight.shape) != (Eg, H)):
         raise ValueError("moe plan: router_weight must be [E,H] in the activations' dtype")
+    if Eg < E or first_expert < 0 or first_expert + E > Eg or (Eg == E and first_expert):
+        raise ValueError(f"moe plan: the weights' {E} experts from {first_expert} on are not among the {Eg} the "
+                         "routing runs over")
+    if e_score_correction_bias is not None and e_score_correction_bias.numel() != Eg:
+        raise ValueError(f"moe plan: the correction bias must have one entry per routed expert ({Eg})")
     if tuple(w2.shape) != (E, H, two_i // (4 if w4 else 2)):
         raise ValueError("moe plan: w2 must be [E,H,I] for w13 [E,2I,H]")
     if w4:
@@ -260,6 +269,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
             raise NotImplementedError("moe plan: no shared expert with 4-bit weights")
     a = L.MoEArgs()
     a.M, a.H, a.E, a.K, a.I = M, H, E, int(top_k), two_i // 2
+    a.E_global, a.first_expert = (Eg, int(first_expert)) if Eg > E else (0, 0)
     a.format = fmt
     a.scoring = L.KMOE_SCORE_SOFTMAX if scoring_func == "softmax" else L.KMOE_SCORE_SIGMOID
     a.renormalize = int(bool(renormalize))

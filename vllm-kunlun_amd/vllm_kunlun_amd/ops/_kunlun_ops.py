@@ -70,16 +70,15 @@ class KunlunOps:
         w1_bias: Optional[torch.Tensor] = None,
         w2_bias: Optional[torch.Tensor] = None,
     ) -> torch.Tensor:
-        """The expert-parallel entry (reference: ops/_kunlun_ops.py:639-696): softmax
-        routing, `renormalize` honoured (:670-671). One GPU holds every expert here, so
-        ep_rank must be 0 and the local experts are the global ones."""
-        if ep_rank != 0:
-            raise NotImplementedError("fused_moe_ep: this build runs all experts on one GPU (ep_rank must be 0)")
+        """The expert-parallel entry (reference: ops/_kunlun_ops.py:639-696): softmax routing over the experts of
+        router_logits' width, `renormalize` honoured (:670-671); the weights are the num_local_experts experts from
+        ep_rank * num_local_experts on (:677-678), and the result is what the pairs routed to them contribute -
+        the caller's all-reduce over the ranks makes the layer's output, as in the reference."""
         L.act_dtype(hidden_states, "fused_moe_ep")
         x = hidden_states.contiguous()
         logits = router_logits.to(torch.float).contiguous()
         out = torch.empty_like(x)
         plan = make_moe_plan(L.KMOE_FMT_BF16, x, logits, out, top_k, w13_weight, w2_weight, None, None, "softmax",
-                             bool(renormalize))
+                             bool(renormalize), first_expert=int(ep_rank) * w13_weight.shape[0])
         plan()
         return out

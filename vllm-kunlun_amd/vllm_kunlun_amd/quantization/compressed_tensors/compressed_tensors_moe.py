@@ -440,15 +440,15 @@ class KunlunCompressedTensorsWNA16MoEMethod:
         if activation != "silu":
             raise NotImplementedError(f"4-bit MoE: activation {activation!r} (silu only)")
         if getattr(self.moe, "use_ep", False):
-            # the expert-parallel branch (:329-342) ends in KunlunOps.fused_moe_ep: softmax routing, `renormalize` honoured
-            if getattr(self.moe, "ep_rank", 0) != 0:
-                raise NotImplementedError("4-bit MoE: this build runs all experts on one GPU (ep_rank must be 0)")
-            return self._run(layer, x, router_logits, top_k, renormalize=bool(renormalize))
+            # the expert-parallel branch (:329-342) ends in KunlunOps.fused_moe_ep: softmax routing over the experts of
+            # router_logits' width, `renormalize` honoured, the layer's weights being those of rank ep_rank
+            return self._run(layer, x, router_logits, top_k, renormalize=bool(renormalize),
+                             ep_rank=int(getattr(self.moe, "ep_rank", 0)))
         return self._run(layer, x, router_logits, top_k, scoring_func=scoring_func, num_expert_group=num_expert_group,
                          topk_group=topk_group, e_score_correction_bias=e_score_correction_bias)
 
     def _run(self, layer, x, router_logits, top_k, scoring_func="softmax", num_expert_group=None, topk_group=None,
-             e_score_correction_bias=None, renormalize=True):
+             e_score_correction_bias=None, renormalize=True, ep_rank=None):
         """Activations in the dtype of the scales (bf16, or float16). On the packed weights:
         kmoe_grouped_gemm_w4a16 inside kmoe_moe_forward. On the unpacked copy: KunlunOps.fused_moe, as
         the reference's apply() ends (:343-360). Routing as in KunlunOps.fused_moe (always
@@ -468,15 +468,15 @@ class KunlunCompressedTensorsWNA16MoEMethod:
             plan = make_moe_plan(L.KMOE_FMT_W4A16, xc, router_logits.to(torch.float).contiguous(), out, top_k,
                                  layer.w13_weight_packed, layer.w2_weight_packed, layer.w13_weight_scale,
                                  layer.w2_weight_scale, scoring_func, renormalize, num_expert_group, topk_group, 1.0,
-                                 e_score_correction_bias, group_size=gs)
+                                 e_score_correction_bias, group_size=gs, first_expert=(ep_rank or 0) * E)
             plan()
             return out
         if not hasattr(layer, "w13_weight"):
             raise NotImplementedError("4-bit MoE: expert biases need the unpacked copy (native='both' or False)")
         from ...ops._kunlun_ops import KunlunOps as ops
-        if not renormalize:  # only the expert-parallel entry leaves the weights unnormalised
-            return ops.fused_moe_ep(x, layer.w13_weight, layer.w2_weight, router_logits, 0, top_k, renormalize=False,
-                                    inplace=True)
+        if ep_rank is not None:  # the expert-parallel entry: its own routing (softmax, `renormalize` honoured)
+            return ops.fused_moe_ep(x, layer.w13_weight, layer.w2_weight, router_logits, ep_rank, top_k,
+                                    renormalize=renormalize, inplace=True)
         return ops.fused_moe(x, layer.w13_weight, layer.w2_weight, router_logits, 0, top_k,
                              renormalize=getattr(layer, "renormalize", True), inplace=True,
                              use_grouped_topk=getattr(layer, "use_grouped_topk", False),

@@ -347,7 +347,7 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--act-dtype", default="bf16", choices=["bf16", "f16"],
                     help="16-bit type of the activations (and of unquantized weights / 4-bit group scales): the layer "
-                         "computes in the same arithmetic type either way; f16 is not built for the fp8 layers")
+                         "computes in the same arithmetic type either way")
     ap.add_argument("--tokens", type=int, default=0,
                     help="run the workload's layer at another batch (tokens per call); the config then says so")
     ap.add_argument("--router", action="store_true",

@@ -210,6 +210,10 @@ int kmoe_scaled_mm_azp_epilogue(const int32_t* acc, int64_t ld_acc, int M, int n
 int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, int C,
                             uint8_t* q, int64_t ld_q, float* scale,
                             kmoe_stream_t stream);
+/* The same with x in act_dtype (KMOE_DT_BF16 or KMOE_DT_F16). */
+int kmoe_quant_fp8_group128_dt(const uint16_t* x, int64_t ld_x, int R, int C,
+                               uint8_t* q, int64_t ld_q, float* scale, int act_dtype,
+                               kmoe_stream_t stream);
 
 /* ------------------------------------------------------------- grouped GEMM */
 
@@ -344,6 +348,8 @@ typedef struct kmoe_gemm_fp8_args {
   const uint8_t* w_tail;      /* NULL, or [n, k] in w_layout                          */
   const float* w_scale_tail;  /* [n/128, k/128]                                       */
   int32_t tail_row0, tail_rows, tail_src0;
+  int32_t act_dtype;          /* KMOE_DT_BF16, or KMOE_DT_F16: y (and the rounding of gate and up before
+                                 SiLU-mul) in IEEE half                                */
 } kmoe_gemm_fp8_args;
 
 /*
@@ -552,9 +558,9 @@ typedef struct kmoe_moe_args {
   const uint16_t* w13_scale; /* [E,2I,H/group_size] bf16                               */
   const uint16_t* w2_scale;  /* [E,H,I/group_size] bf16                                */
   int32_t group_size;    /* a multiple of 32 dividing H and I (one value for both tensors) */
-  int32_t act_dtype;     /* KMOE_DT_* of x, out (and w_gate, shared-expert output): half goes with KMOE_FMT_INT8,
-                            with KMOE_FMT_BF16 (whose weights are then half too; no biases, no SWIGLUOAI) and
-                            with KMOE_FMT_W4A16 (whose group scales are then half) */
+  int32_t act_dtype;     /* KMOE_DT_* of x, out (and w_gate, shared-expert output): half goes with every format
+                            (KMOE_FMT_BF16: the weights are then half too, and no biases, no SWIGLUOAI;
+                            KMOE_FMT_W4A16: the group scales are then half) */
   float shared_scale;    /* caller epilogue for half activations (models/deepseek_v2.py:286-292: the routed sum stays
                             unscaled and the shared expert's output is multiplied by 1/routed_scaling_factor):
                             out = dt( dt(routed * out_scale) + dt(shared * shared_scale) ); 0 means 1 */

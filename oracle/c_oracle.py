@@ -189,7 +189,8 @@ def quant_i8_rows_azp(x_bits, f16=False):
     return q, s, z
 
 
-def quant_fp8_group128(x_bits):
+def quant_fp8_group128(x_bits, f16=False):
+    _dtype(f16)
     x_bits = _c(x_bits, np.uint16)
     R, Cc = x_bits.shape
     q = np.empty((R, Cc), np.uint8)
@@ -312,7 +313,8 @@ def grouped_gemm_bf16(a_bits, w_bits, lod, act=0, row_src=None, src_div=1, f16=F
     return y
 
 
-def grouped_gemm_fp8(a, a_scale, w, w_scale, lod, act=0, row_src=None, src_div=1):
+def grouped_gemm_fp8(a, a_scale, w, w_scale, lod, act=0, row_src=None, src_div=1, f16=False):
+    _dtype(f16)
     a = _c(a, np.uint8)
     w = _c(w, np.uint8)
     a_scale = _c(a_scale, np.float32)
@@ -396,21 +398,22 @@ def forward_bf16(x_bits, logits, w13_bits, w2_bits, K, scoring="softmax", renorm
 
 
 def forward_fp8(x_bits, logits, w13, w13_scale, w2, w2_scale, K, scoring="softmax", renormalize=True, n_group=1,
-                topk_group=1, routed_scale=1.0, bias=None, shared=None, out_scale=1.0):
-    """fp8 block-scaled layer: same stage order as the int8 layer with the fp8 quantiser and GEMM."""
+                topk_group=1, routed_scale=1.0, bias=None, shared=None, out_scale=1.0, f16=False):
+    """fp8 block-scaled layer: same stage order as the int8 layer with the fp8 quantiser and GEMM; f16: x and out
+    (and every 16-bit intermediate) hold IEEE half patterns."""
     E = w13.shape[0]
     M = x_bits.shape[0]
     w, ids = _route(logits, K, scoring, renormalize, n_group, topk_group, routed_scale, bias)
     moe_index, src, _, lod = align(ids, E)
-    xq, xs = quant_fp8_group128(x_bits)
-    act = grouped_gemm_fp8(xq, xs, w13, w13_scale, lod, act=1, row_src=src, src_div=K)
-    aq, as_ = quant_fp8_group128(act)
-    down = grouped_gemm_fp8(aq, as_, w2, w2_scale, lod)
+    xq, xs = quant_fp8_group128(x_bits, f16=f16)
+    act = grouped_gemm_fp8(xq, xs, w13, w13_scale, lod, act=1, row_src=src, src_div=K, f16=f16)
+    aq, as_ = quant_fp8_group128(act, f16=f16)
+    down = grouped_gemm_fp8(aq, as_, w2, w2_scale, lod, f16=f16)
     sh = None
     if shared is not None:
         ws13, ws13_scale, ws2, ws2_scale = shared
         dlod = np.array([0, M], np.int32)
-        sact = grouped_gemm_fp8(xq, xs, ws13[None], ws13_scale[None], dlod, act=1)
-        sq, ss = quant_fp8_group128(sact)
-        sh = grouped_gemm_fp8(sq, ss, ws2[None], ws2_scale[None], dlod)
-    return combine(down, moe_index, w, None, out_scale, sh)
+        sact = grouped_gemm_fp8(xq, xs, ws13[None], ws13_scale[None], dlod, act=1, f16=f16)
+        sq, ss = quant_fp8_group128(sact, f16=f16)
+        sh = grouped_gemm_fp8(sq, ss, ws2[None], ws2_scale[None], dlod, f16=f16)
+    return combine(down, moe_index, w, None, out_scale, sh, f16=f16)

@@ -376,10 +376,10 @@ ORC_API void orc_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, int 
     for (int g = 0; g < G; ++g) {
       const uint16_t* xr = x + (size_t)r * ld_x + g * 128;
       float amax = 0.0f;
-      for (int c = 0; c < 128; ++c) amax = fmaxf(amax, fabsf(bf16_to_f32(xr[c])));
+      for (int c = 0; c < 128; ++c) amax = fmaxf(amax, fabsf(act_to_f32(xr[c])));
       const float s = amax / 448.0f;
       for (int c = 0; c < 128; ++c)
-        q[(size_t)r * ld_q + g * 128 + c] = orc_f32_to_e4m3fn(s > 0.0f ? bf16_to_f32(xr[c]) / s : 0.0f);
+        q[(size_t)r * ld_q + g * 128 + c] = orc_f32_to_e4m3fn(s > 0.0f ? act_to_f32(xr[c]) / s : 0.0f);
       scale[(size_t)r * G + g] = s;
     }
   }
@@ -589,9 +589,9 @@ ORC_API void orc_grouped_gemm_fp8(const uint8_t* a, int64_t lda, const float* a_
         }
         if (act)
           y[(size_t)r * ldy + c] =
-              f32_to_bf16(orc_silu(bf16_to_f32(f32_to_bf16(tot[0]))) * bf16_to_f32(f32_to_bf16(tot[1])));
+              f32_to_act(orc_silu(act_to_f32(f32_to_act(tot[0]))) * act_to_f32(f32_to_act(tot[1])));
         else
-          y[(size_t)r * ldy + c] = f32_to_bf16(tot[0]);
+          y[(size_t)r * ldy + c] = f32_to_act(tot[0]);
       }
     }
   }

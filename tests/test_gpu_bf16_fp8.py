@@ -153,6 +153,14 @@ def test_grouped_gemm_fp8_block_tiled_weights(L, E, n, k, counts, variant, act):
     _fp8_case(L, E, n, k, counts, variant, act, tiled=True)
 
 
+@pytest.mark.parametrize("E,n,k,counts", FP8_TILED_CASES)
+@pytest.mark.parametrize("variant,tiled", [(1, False), (2, True), (5, True), (6, True), (11, True), (12, True)])
+@pytest.mark.parametrize("act", [0, 1])
+def test_grouped_gemm_fp8_block_half_results(L, E, n, k, counts, variant, tiled, act):
+    """act_dtype = KMOE_DT_F16: the LDS-staged kernel and the tile kernel's 64-row, 128-row and paced shapes."""
+    _fp8_case(L, E, n, k, counts, variant, act, tiled=tiled, half=True)
+
+
 @pytest.mark.parametrize("E,n,k,counts", FP8_CASES)
 @pytest.mark.parametrize("variant", [1, 2, 3])
 @pytest.mark.parametrize("act", [0, 1])
@@ -160,7 +168,7 @@ def test_grouped_gemm_fp8_block(L, E, n, k, counts, variant, act):
     _fp8_case(L, E, n, k, counts, variant, act, tiled=False)
 
 
-def _fp8_case(L, E, n, k, counts, variant, act, tiled):
+def _fp8_case(L, E, n, k, counts, variant, act, tiled, half=False):
     if act and n % 256:
         pytest.skip("SwiGLU needs n % 256 == 0 for block scales")
     torch.manual_seed(E * n + k + 1)
@@ -170,11 +178,12 @@ def _fp8_case(L, E, n, k, counts, variant, act, tiled):
     xq, xs = tm.quant_fp8_group128(x)
     wq, ws = tm.quantize_weight_fp8_block128(torch.randn(E, n, k) * 0.02)
     a8, w8 = xq.view(torch.uint8), wq.view(torch.uint8)
-    ref = co.grouped_gemm_fp8(a8.numpy(), xs.numpy(), w8.numpy(), ws.numpy(), lod, act=act)
+    ref = co.grouped_gemm_fp8(a8.numpy(), xs.numpy(), w8.numpy(), ws.numpy(), lod, act=act, f16=half)
     n_out = n // 2 if act else n
     da, ds, dw, dws, dl = a8.cuda(), xs.contiguous().cuda(), w8.cuda(), ws.contiguous().cuda(), torch.from_numpy(lod).cuda()
-    y = torch.zeros(rows, n_out, dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros(rows, n_out, dtype=torch.float16 if half else torch.bfloat16, device="cuda")
     g = L.GemmFp8Args()
+    g.act_dtype = L.KMOE_DT_F16 if half else L.KMOE_DT_BF16
     if tiled:
         dt = torch.empty_like(dw)
         L.check(L.lib.kmoe_tile_weights_i8(dw.data_ptr(), dt.data_ptr(), E, n, k, L.stream()))
@@ -186,6 +195,9 @@ def _fp8_case(L, E, n, k, counts, variant, act, tiled):
     g.y, g.ldy, g.act, g.variant = y.data_ptr(), n_out, act, variant
     L.check(L.lib.kmoe_grouped_gemm_fp8_block(g, L.stream()))
     torch.cuda.synchronize()
+    if half:  # results (and gate and up before SiLU-mul) rounded to IEEE half
+        assert rel_l2(y, torch.from_numpy(ref.view(np.float16).copy())) <= 2e-3
+        return
     assert rel_l2(y, from_bits(ref)) <= 2e-3
     if not act:  # torch restatement of the block-scaled product, one expert
         e = int(np.argmax(counts))

@@ -157,10 +157,6 @@ def test_float16_is_refused_where_it_is_not_served():
     bias = torch.zeros(w13.shape[0], w13.shape[1], dtype=torch.float16, device="cuda")
     with pytest.raises(NotImplementedError):  # the expert-bias branch is bf16 only
         KunlunOps.fused_moe(sl.x.half(), w13, w2, sl.logits, 0, shape.K, True, w1_bias=bias)
-    fp8 = synth.make_fp8_layer(synth.scaled(synth.SHAPES["dsv3-fp8-decode"], M=8, H=256, E=8, K=2, I=128, n_group=2,
-                                            topk_group=1, I_shared=0), "cuda", seed=1)
-    with pytest.raises(NotImplementedError):
-        fp8.layer.quant_method.apply_monolithic(fp8.layer, fp8.x.half(), fp8.logits, **fp8.apply_kwargs())
 
 
 # ---------------------------------------------------------------- the unquantized path on half tensors
@@ -393,3 +389,30 @@ def test_w4_half_subnormal_products():
     torch.cuda.synchronize()
     assert float(from_hbits(ref).float().abs().max()) > 0
     assert rel_l2(y, from_hbits(ref)) <= 2e-3
+
+
+# ---------------------------------------------------------------- the fp8 block-scaled layer on half activations
+@pytest.mark.parametrize("M,I_shared", [(8, 0), (40, 128), (40, 256), (700, 128), (700, 0)])
+def test_fp8_layer_with_half_activations(M, I_shared):
+    """float16 in, float16 out on fp8 block-scaled weights: the quantiser reads half, the GEMMs round their
+    results (and gate and up before SiLU-mul) to half: decode sizes on the LDS-staged kernel, beyond on the tile
+    kernel, with a shared expert folded into the routed
+    launches (same width), run on its own (another width) or absent; against the oracle in half mode within the
+    fp8 tolerance, and against the bfloat16 run of the same layer within what the two output types differ by."""
+    from vllm_kunlun_amd import synth
+    shape = synth.scaled(synth.SHAPES["dsv3-fp8-decode"], M=M, H=512, E=16, K=4, I=128, n_group=4, topk_group=2,
+                         I_shared=I_shared)
+    sl = synth.make_layer(shape, "cuda", seed=2, dtype=torch.float16)
+    out = sl.layer.quant_method.apply_monolithic(sl.layer, sl.x, sl.logits, **sl.apply_kwargs())
+    out_bf = sl.layer.quant_method.apply_monolithic(sl.layer, sl.x.bfloat16(), sl.logits, **sl.apply_kwargs())
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16 and bool(torch.isfinite(out.float()).all())
+    assert rel_l2(out, out_bf) <= 2e-2
+    rows = slice(0, M)
+    w13, w13_s, w2, w2_s, sh = sl.host_weights()
+    u8 = lambda t: t.view(torch.uint8).numpy()  # noqa: E731
+    shared = None if sh is None else (u8(sh[0]), sh[1].numpy(), u8(sh[2]), sh[3].numpy())
+    ref = co.forward_fp8(hbits(sl.x[rows]), sl.logits[rows].cpu().numpy(), u8(w13), w13_s.numpy(), u8(w2), w2_s.numpy(),
+                         shape.K, shape.scoring, True, shape.n_group, shape.topk_group, shape.routed_scale,
+                         sl.bias.cpu().numpy(), shared, f16=True)
+    assert rel_l2(out[rows], from_hbits(ref)) <= 3e-2

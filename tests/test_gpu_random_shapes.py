@@ -85,15 +85,16 @@ def test_random_unquantized_layer_shape(seed):
 
 @pytest.mark.parametrize("seed", range(32))
 def test_random_fp8_layer_shape(seed):
-    """fp8 block-scaled layer (hidden and intermediate sizes in multiples of 128): rel-L2 <= 3e-2 against the oracle."""
+    """fp8 block-scaled layer (hidden and intermediate sizes in multiples of 128; bfloat16 or float16 activations):
+    rel-L2 <= 3e-2 against the oracle."""
     from vllm_kunlun_amd import synth
-    base, over, _ = _draw(2000 + seed)
+    base, over, half = _draw(2000 + seed)
     rng = random.Random(seed)
     over.update(H=128 * rng.randint(1, 6), I=128 * rng.randint(1, 4), quant="fp8")
     if over.get("I_shared"):
         over["I_shared"] = over["I"] if rng.random() < 0.5 else 128 * rng.randint(1, 4)
     shape = synth.scaled(synth.SHAPES[base], **over)
-    sl = synth.make_layer(shape, "cuda", seed=seed)
+    sl = synth.make_layer(shape, "cuda", seed=seed, dtype=torch.float16 if half else torch.bfloat16)
     out = sl.layer.quant_method.apply_monolithic(sl.layer, sl.x, sl.logits, **sl.apply_kwargs())
     torch.cuda.synchronize()
     w13, w13_s, w2, w2_s, sh = sl.host_weights()
@@ -101,9 +102,9 @@ def test_random_fp8_layer_shape(seed):
     shared = None if sh is None else (u8(sh[0]), sh[1].numpy(), u8(sh[2]), sh[3].numpy())
     ref = co.forward_fp8(_bits16(sl.x), sl.logits.cpu().numpy(), u8(w13), w13_s.numpy(), u8(w2), w2_s.numpy(), shape.K,
                          shape.scoring, True, shape.n_group, shape.topk_group, shape.routed_scale,
-                         None if sl.bias is None else sl.bias.cpu().numpy(), shared)
-    ref_t = torch.from_numpy(ref.view(np.int16)).view(torch.bfloat16)
-    assert _rel_l2(out, ref_t) <= 3e-2, f"{base} {over}"
+                         None if sl.bias is None else sl.bias.cpu().numpy(), shared, f16=half)
+    ref_t = torch.from_numpy(ref.view(np.int16)).view(torch.float16 if half else torch.bfloat16)
+    assert out.dtype == sl.x.dtype and _rel_l2(out, ref_t) <= 3e-2, f"{base} {over} half={half}"
 
 
 @pytest.mark.parametrize("seed", range(32))

@@ -92,7 +92,7 @@ __device__ inline uint32_t pack2_e4m3fn(float a, float b) {
 // requested up front, measured no faster: the eight IEEE divisions per lane set the pace.)
 __global__ __launch_bounds__(256) void quant_fp8_group128_kernel(const uint16_t* __restrict__ x, int64_t ld_x,
                                                                 int R, int C, uint8_t* __restrict__ q,
-                                                                int64_t ld_q, float* __restrict__ scale) {
+                                                                int64_t ld_q, float* __restrict__ scale, int f16) {
   const int groups_per_row = C / 128;
   const long long total = static_cast<long long>(R) * groups_per_row;
   const long long gid = static_cast<long long>(blockIdx.x) * 16 + (threadIdx.x >> 4);
@@ -105,14 +105,14 @@ __global__ __launch_bounds__(256) void quant_fp8_group128_kernel(const uint16_t*
   if (live) val.v = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(r) * ld_x + g * 128 + t * 8);
   float amax = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(bf16_to_f32(val.h[j])));
+  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(act_to_f32(val.h[j], f16 != 0)));
 #pragma unroll
   for (int off = 8; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, kWave));
   if (!live) return;
   const float s = amax / 448.0f;
   float f[8];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) f[j] = s > 0.0f ? bf16_to_f32(val.h[j]) / s : 0.0f;
+  for (int j = 0; j < 8; ++j) f[j] = s > 0.0f ? act_to_f32(val.h[j], f16 != 0) / s : 0.0f;
   const uint32_t w[2] = {pack2_e4m3fn(f[0], f[1]) | (pack2_e4m3fn(f[2], f[3]) << 16),
                          pack2_e4m3fn(f[4], f[5]) | (pack2_e4m3fn(f[6], f[7]) << 16)};
   *reinterpret_cast<uint2*>(q + static_cast<size_t>(r) * ld_q + g * 128 + t * 8) = make_uint2(w[0], w[1]);
@@ -331,6 +331,12 @@ extern "C" int kmoe_quant_i8_rows_chunked_dt(const uint16_t* x, int64_t ld_x, in
 
 extern "C" int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, int C, uint8_t* q, int64_t ld_q,
                                        float* scale, kmoe_stream_t stream) {
+  return kmoe_quant_fp8_group128_dt(x, ld_x, R, C, q, ld_q, scale, KMOE_DT_BF16, stream);
+}
+
+extern "C" int kmoe_quant_fp8_group128_dt(const uint16_t* x, int64_t ld_x, int R, int C, uint8_t* q, int64_t ld_q,
+                                          float* scale, int act_dtype, kmoe_stream_t stream) {
+  if (int rc = check_dtype(act_dtype, "quant_fp8_group128")) return rc;
   KMOE_REQUIRE(x && q && scale, KMOE_ERR_NULL, "quant_fp8_group128: NULL pointer");
   KMOE_REQUIRE(R >= 0 && C >= 128 && C % 128 == 0, KMOE_ERR_SHAPE, "quant_fp8_group128: R=%d C=%d (need C %% 128 == 0)",
                R, C);
@@ -340,7 +346,7 @@ extern "C" int kmoe_quant_fp8_group128(const uint16_t* x, int64_t ld_x, int R, i
   if (R == 0) return KMOE_OK;
   const long long groups = static_cast<long long>(R) * (C / 128);
   hipLaunchKernelGGL(quant_fp8_group128_kernel, dim3(static_cast<unsigned>((groups + 15) / 16)), dim3(256), 0,
-                     as_stream(stream), x, ld_x, R, C, q, ld_q, scale);
+                     as_stream(stream), x, ld_x, R, C, q, ld_q, scale, act_dtype == KMOE_DT_F16 ? 1 : 0);
   return check_launch("kmoe_quant_fp8_group128");
 }
 

@@ -63,10 +63,8 @@ int check_shape(const kmoe_moe_args* a) {
   KMOE_REQUIRE(a->I_shared >= 0 && a->I_shared % mult == 0, KMOE_ERR_SHAPE,
                "moe_forward: I_shared=%d must be a non-negative multiple of %d", a->I_shared, mult);
   KMOE_REQUIRE(static_cast<long long>(a->M) * a->K <= (1 << 24), KMOE_ERR_SHAPE, "moe_forward: M*K too large");
-  KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 ||
-                   (a->act_dtype == KMOE_DT_F16 && a->format != KMOE_FMT_FP8_BLOCK),
-               KMOE_ERR_UNSUPPORTED, "moe_forward: act_dtype=%d (half activations do not go with the fp8 format)",
-               a->act_dtype);
+  KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 || a->act_dtype == KMOE_DT_F16, KMOE_ERR_UNSUPPORTED,
+               "moe_forward: act_dtype=%d unknown", a->act_dtype);
   KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 || a->format != KMOE_FMT_BF16 ||
                    (!a->w13_bias && !a->w2_bias && a->activation != KMOE_ACT_SWIGLUOAI),
                KMOE_ERR_UNSUPPORTED, "moe_forward: expert biases and swigluoai are built for bf16 only");
@@ -202,6 +200,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.src_div = src_div;
     g.w = static_cast<const uint8_t*>(w);
     g.w_scale = w_aux;
+    g.act_dtype = m.act_dtype;
     g.lod = m.lod;
     g.E = m.E;
     g.n = n;
@@ -279,8 +278,8 @@ int run_mlp(const MlpPass& m, kmoe_stream_t stream, Mark&& mark) {
                   : kmoe_quant_i8_rows_dt(m.act, m.I, qrows, m.I, static_cast<int8_t*>(m.actq), m.I, m.act_aux,
                                           m.act_dtype, stream);
   } else if (m.format == KMOE_FMT_FP8_BLOCK) {
-    rc = kmoe_quant_fp8_group128(m.act, m.I, m.rows + m.tail_rows, m.I, static_cast<uint8_t*>(m.actq), m.I, m.act_aux,
-                                 stream);
+    rc = kmoe_quant_fp8_group128_dt(m.act, m.I, m.rows + m.tail_rows, m.I, static_cast<uint8_t*>(m.actq), m.I, m.act_aux,
+                                    m.act_dtype, stream);
   }
   if (rc) return rc;
   mark(KMOE_STAGE_QUANT2, 1);
@@ -501,8 +500,8 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
                                              static_cast<float*>(at(L.xmax)), a->act_dtype, stream);
     x_rows = at(L.xq);
   } else if (a->format == KMOE_FMT_FP8_BLOCK) {
-    rc = kmoe_quant_fp8_group128(a->x, H, M, H, static_cast<uint8_t*>(at(L.xq)), H, static_cast<float*>(at(L.xmax)),
-                                 stream);
+    rc = kmoe_quant_fp8_group128_dt(a->x, H, M, H, static_cast<uint8_t*>(at(L.xq)), H, static_cast<float*>(at(L.xmax)),
+                                    a->act_dtype, stream);
     x_rows = at(L.xq);
   }
   if (rc) return rc;

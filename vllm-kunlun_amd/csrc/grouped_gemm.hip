@@ -73,7 +73,7 @@ struct GemmParams {
   const uint16_t* bias;    // NULL, or [E, n] bf16 added to the bf16 result (rounded again, as `gemm + bias` in bf16 is)
   int32_t oai;             // 1: out[r, i] = swigluoai(y[r, 2i], y[r, 2i+1]) (interleaved gate/up), n/2 outputs per row
   float oai_alpha, oai_limit;
-  int32_t f16;             // I8 only: outputs in IEEE half instead of bf16
+  int32_t f16;             // I8, FP8: outputs (and the rounding of gate and up before SiLU-mul) in IEEE half instead of bf16
 };
 
 // Rows of expert e, with the tail expert (e == E) taken from the host-side range.
@@ -343,7 +343,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
       const int r = row0 + mf * 16 + li;
       if (r >= row_end) continue;
       float sa = 1.0f;
-      const bool f16 = KIND == Kind::F16 || (KIND == Kind::I8 && p.f16 != 0);
+      const bool f16 = KIND == Kind::F16 || ((KIND == Kind::I8 || KIND == Kind::FP8) && p.f16 != 0);
       if constexpr (KIND == Kind::I8) sa = p.a_max[srow[mf]] / 127.0f;
 #pragma unroll
       for (int f = 0; f < NFH; ++f) {
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
             if (p.acc_out) *reinterpret_cast<v4i*>(p.acc_out + static_cast<size_t>(r) * p.n + cc) = a;
           } else {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) out[q] = f32_to_act(a[q], KIND == Kind::F16);
+            for (int q = 0; q < 4; ++q) out[q] = f32_to_act(a[q], f16);
           }
         };
         finish(acc[mf][f], c0, yv);
@@ -544,6 +544,8 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
                "grouped_gemm_fp8_block: NULL tensor pointer");
   KMOE_REQUIRE(a->E >= 1 && a->n >= 128 && a->k >= 128 && a->rows >= 0, KMOE_ERR_SHAPE,
                "grouped_gemm_fp8_block: E=%d n=%d k=%d rows=%d", a->E, a->n, a->k, a->rows);
+  KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 || a->act_dtype == KMOE_DT_F16, KMOE_ERR_UNSUPPORTED,
+               "grouped_gemm_fp8_block: act_dtype=%d unknown", a->act_dtype);
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
   KMOE_REQUIRE(a->act == KMOE_ACT_NONE || swiglu, KMOE_ERR_UNSUPPORTED, "grouped_gemm_fp8_block: act=%d unknown",
                a->act);
@@ -574,6 +576,6 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
                reinterpret_cast<const int8_t*>(a->w), a->w_scale, a->lod,  a->E,       a->n,
                a->k,                                  a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,
                reinterpret_cast<const int8_t*>(a->w_tail), a->w_scale_tail, a->tail_row0, tail_rows, a->tail_src0,
-               nullptr, 0, 0.f, 0.f};
+               nullptr, 0, 0.f, 0.f, a->act_dtype == KMOE_DT_F16};
   return dispatch<Kind::FP8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_fp8_block");
 }

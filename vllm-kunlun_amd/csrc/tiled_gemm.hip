@@ -133,12 +133,12 @@ struct Tile {
 // PACE: the m-tiles of one (expert, channel block) keep in step through the progress board (g_board), which
 // brings the bytes fetched by L2 down to little more than once per weight byte where experts have two or three
 // m-tiles (int8: a few percent of time, the re-reads were mostly served by the memory-side cache; fp8: 14 %).
-// F16: the outputs, and the rounding of gate and up before SiLU-mul, are IEEE half instead of bf16 (int8
-// operands); with KIND = BF16 the operands are half as well (v_mfma_f32_16x16x32_f16).
+// F16: the outputs, and the rounding of gate and up before SiLU-mul, are IEEE half instead of bf16 (int8 and
+// fp8 operands); with KIND = BF16 the operands are half as well (v_mfma_f32_16x16x32_f16).
 template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false,
           bool PACE = false, bool F16 = false>
 __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(const TiledParams p) {
-  static_assert(!F16 || KIND == TKind::I8 || (KIND == TKind::BF16 && !OAI), "half is wired for the int8 and the plain unquantized path");
+  static_assert(!F16 || KIND != TKind::BF16 || !OAI, "the interleaved activation is a bf16 epilogue");
   static_assert(!OAI || (KIND == TKind::BF16 && !SWIGLU && !M32), "the interleaved activation is a bf16 epilogue");
   constexpr int kMF = MF;
   constexpr int kNA = 16 * kMF * (kChunk / 16) / (kWavesT * kWave);  // 16-byte activation vectors per thread and chunk
@@ -1036,18 +1036,30 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
   constexpr TKind K = TKind::F8;
   // (64x128 tiles for a dense GEMM of a few rows, twice the work items: 57 -> 42 us on [128,7168] x [4096,7168],
   // still bound by what one workgroup keeps in flight; not instantiated)
-  if (short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu))
+  const bool half = a->act_dtype == KMOE_DT_F16;  // half outputs: the same three shapes
+  if (short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu)) {
+    if (half)
+      return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4, false, false, true>(p, a->rows, s, n_cu, what)
+                    : launch_tiled<K, false, 4, 4, 2, 1, false, 4, false, false, true>(p, a->rows, s, n_cu, what);
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);
+  }
   // paced sibling m-tiles where experts have more than one of them and the weights are far more than the
   // memory-side cache holds, as for int8, and a tile walks a long K (DeepSeek-V3 shape at 4096 tokens: gate_up,
   // K = 7168, 2570 -> 2222 us; the down projection, K = 2048, is 5 % slower with it: 1033 -> 1083 us; layer at
   // 8192 tokens 5.86 -> 5.78 ms, at 16384 tokens 10.90 -> 10.66 ms)
   const int avg_rows = ceil_div(a->rows + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
   const long long weight_bytes = static_cast<long long>(a->E + (a->w_tail ? 1 : 0)) * a->n * a->k;
-  if (a->variant == 12 || (a->variant == 0 && avg_rows > 96 && a->k >= 4096 && weight_bytes > (1ll << 30)))
+  if (a->variant == 12 || (a->variant == 0 && avg_rows > 96 && a->k >= 4096 && weight_bytes > (1ll << 30))) {
+    if (half)
+      return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 8, false, true, true>(p, a->rows, s, n_cu, what)
+                    : launch_tiled<K, false, 4, 4, 2, 1, false, 8, false, true, true>(p, a->rows, s, n_cu, what);
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 8, false, true>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 8, false, true>(p, a->rows, s, n_cu, what);
+  }
+  if (half)
+    return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 8, false, false, true>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 4, 4, 2, 1, false, 8, false, false, true>(p, a->rows, s, n_cu, what);
   return swiglu ? launch_tiled<K, true, 4, 4, 2, 1>(p, a->rows, s, n_cu, what)
                 : launch_tiled<K, false, 4, 4, 2, 1>(p, a->rows, s, n_cu, what);
 }

@@ -73,7 +73,7 @@ class GemmFp8Args(C.Structure):
         ("y", C.c_void_p), ("ldy", C.c_int64), ("act", C.c_int32), ("variant", C.c_int32),
         ("w_layout", C.c_int32),
         ("w_tail", C.c_void_p), ("w_scale_tail", C.c_void_p),
-        ("tail_row0", C.c_int32), ("tail_rows", C.c_int32), ("tail_src0", C.c_int32),
+        ("tail_row0", C.c_int32), ("tail_rows", C.c_int32), ("tail_src0", C.c_int32), ("act_dtype", C.c_int32),
     ]
 
 
@@ -131,6 +131,7 @@ def _load() -> C.CDLL:
         "kmoe_router_gemm_workspace_bytes": (sz, [i32, i32, i32]),
         "kmoe_router_gemm_bf16": (i32, [vp, i64, vp, i32, i32, i32, vp, i64, vp, sz, vp]),
         "kmoe_quant_fp8_group128": (i32, [vp, i64, i32, i32, vp, i64, vp, vp]),
+        "kmoe_quant_fp8_group128_dt": (i32, [vp, i64, i32, i32, vp, i64, vp, i32, vp]),
         "kmoe_grouped_gemm_i8": (i32, [C.POINTER(GemmI8Args), vp]),
         "kmoe_silu_and_mul": (i32, [vp, i64, i32, i32, vp, i64, vp]),
         "kmoe_combine": (i32, [vp, i64, vp, vp, vp, i32, i32, i32, f32, vp, i64, vp, i64, vp]),
@@ -156,7 +157,7 @@ def _load() -> C.CDLL:
 lib = _load()
 EXPORTS = (
     "kmoe_last_error", "kmoe_version", "kmoe_softmax_topk", "kmoe_sigmoid_group_topk_norm", "kmoe_block_statistic",
-    "kmoe_align_workspace_bytes", "kmoe_align", "kmoe_gather_rows", "kmoe_quant_i8_rows", "kmoe_quant_i8_rows_chunked", "kmoe_tile_weights_i8", "kmoe_quant_fp8_group128",
+    "kmoe_align_workspace_bytes", "kmoe_align", "kmoe_gather_rows", "kmoe_quant_i8_rows", "kmoe_quant_i8_rows_chunked", "kmoe_tile_weights_i8", "kmoe_quant_fp8_group128", "kmoe_quant_fp8_group128_dt",
     "kmoe_grouped_gemm_i8", "kmoe_grouped_gemm_bf16", "kmoe_grouped_gemm_w4a16", "kmoe_grouped_gemm_fp8_block", "kmoe_silu_and_mul", "kmoe_combine",
     "kmoe_moe_workspace_layout", "kmoe_moe_forward", "kmoe_router_gemm_workspace_bytes", "kmoe_router_gemm_bf16",
     "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16", "kmoe_dequant_w4", "kmoe_moe_forward_static",

@@ -259,7 +259,7 @@ def _moe_fc_fp8(x, weight, lod, y, act, x_scale, w_scale, scale_n, scale_k) -> N
         raise NotImplementedError(f"moe_fc: block scales of {scale_n} x {scale_k} are not served (128 x 128 only)")
     f8 = (torch.float8_e4m3fn, torch.uint8)
     _need(x.dtype in f8 and weight.dtype in f8, "moe_fc: block-scaled operands must be float8_e4m3fn (or their bytes)")
-    _need(y.dtype == _BF16, "moe_fc: the block-scaled GEMM writes bfloat16")
+    _need(y.dtype in (_BF16, torch.float16), "moe_fc: the block-scaled GEMM writes bfloat16 or float16")
     E, n, k = weight.shape
     rows = x.numel() // k
     _need(x_scale is not None and w_scale is not None and x_scale.dtype == torch.float32
@@ -275,6 +275,7 @@ def _moe_fc_fp8(x, weight, lod, y, act, x_scale, w_scale, scale_n, scale_k) -> N
     g.y, g.ldy = y.data_ptr(), y.numel() // max(rows, 1) if rows else n_out
     g.act = L.KMOE_ACT_SWIGLU if act else L.KMOE_ACT_NONE
     g.w_layout = weight_layout(weight)
+    g.act_dtype = L.act_dtype(y)
     L.check(L.lib.kmoe_grouped_gemm_fp8_block(g, L.stream()))
 
 

@@ -138,7 +138,7 @@ class _MonolithicQuantMoE:
         router_weight: Optional[torch.Tensor] = None,
         shared_scale: float = 1.0,
     ) -> Union[torch.Tensor, tuple]:
-        """x [M,H] bf16 or float16 (float16 with int8 weights only), router_logits [M,E] -> [M,H] in x's dtype
+        """x [M,H] bf16 or float16, router_logits [M,E] -> [M,H] in x's dtype
         (reference: :122-291).
         `shared_expert` (w13, w13_max, w2, w2_max of a dense MLP in the layer's format), `out_scale` and
         `shared_scale` fold the caller's epilogue (models/deepseek_v2.py:286-296) into the call:

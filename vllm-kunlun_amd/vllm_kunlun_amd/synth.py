@@ -75,14 +75,14 @@ for _n in ("kimi-decode", "kimi-prefill"):
 
 def make_layer(shape: MoEShape, device="cuda", seed: int = 0, dtype: torch.dtype = torch.bfloat16) -> "SynthLayer":
     """The synthetic layer of a shape in the format the shape names. dtype: bfloat16, or float16 (int8: the
-    activations; unquantized: activations and weights; 4-bit: activations and group scales; not fp8)."""
+    and fp8: the activations; unquantized: activations and weights; 4-bit: activations and group scales)."""
     if dtype == torch.bfloat16:
         return {"int8": make_w8a8_layer, "fp8": make_fp8_layer, "none": make_bf16_layer,
                 "w4": make_w4_layer}[shape.quant](shape, device, seed)
-    if dtype != torch.float16 or shape.quant == "fp8":
+    if dtype != torch.float16:
         raise NotImplementedError(f"synthetic {shape.quant} layer with {dtype} activations")
-    if shape.quant == "int8":
-        sl = make_w8a8_layer(shape, device, seed)
+    if shape.quant in ("int8", "fp8"):
+        sl = (make_w8a8_layer if shape.quant == "int8" else make_fp8_layer)(shape, device, seed)
         return SynthLayer(sl.shape, sl.layer, sl.x.half(), sl.logits, sl.bias, sl.shared)
     return {"none": make_bf16_layer, "w4": make_w4_layer}[shape.quant](shape, device, seed, dtype)
 

@@ -333,3 +333,13 @@ def test_int8_layer_as_an_expert_parallel_share(M, scoring):
         ref = co.combine(down, moe_index, w)
         assert np.array_equal(bits(out), ref), f"rank {rank}"
         assert 0 < int(lod[-1]) < M * K
+        # the same share through the plugin method: the layer holds the rank's experts, method.moe names the rank
+        from types import SimpleNamespace
+        from vllm_kunlun_amd.quantization.compressed_tensors.compressed_tensors_moe import (
+            KunlunCompressedTensorsW8A8Int8MoEMethod)
+        method = KunlunCompressedTensorsW8A8Int8MoEMethod(moe=SimpleNamespace(experts_per_token=K, use_ep=True, ep_rank=rank))
+        layer = SimpleNamespace(w13_weight=d13, w2_weight=d2, w13_weight_scale=w13_max.cuda(), w2_weight_scale=w2_max.cuda())
+        kw = {k: v for k, v in route.items() if k != "renormalize"}
+        out2 = method.apply_monolithic(layer, x.cuda(), logits.cuda(), **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(out2, out)

@@ -166,11 +166,17 @@ class _MonolithicQuantMoE:
         capture replays without touching Python-side allocation."""
         topk_group, num_expert_group, scoring_func, routed_scaling_factor, bias = self._routing(
             layer, topk_group, num_expert_group, scoring_func, routed_scaling_factor, e_score_correction_bias)
+        # Under expert parallelism the layer holds the experts of one rank while the logits (or the router weight)
+        # run over all of them: the rank's share, as KunlunOps.fused_moe_ep computes it for the unquantized layer
+        # (ops/_kunlun_ops.py:677-689). The reference's own quantized path takes the local experts for all (:135).
+        E = layer.w13_weight.shape[0]
+        routed = logits.shape[-1] if logits is not None else router_weight.shape[0]
+        first = int(getattr(self.moe, "ep_rank", 0) or 0) * E if routed > E else 0
         return make_moe_plan(self.FORMAT, x, logits, out, self.moe.experts_per_token, layer.w13_weight,
                              layer.w2_weight, layer.w13_weight_scale, layer.w2_weight_scale, scoring_func,
                              True,  # the reference always routes with the *_norm kernels
                              num_expert_group, topk_group, routed_scaling_factor, bias, shared_expert, out_scale,
-                             stage_events, router_weight=router_weight, shared_scale=shared_scale)
+                             stage_events, router_weight=router_weight, shared_scale=shared_scale, first_expert=first)
 
 
 class KunlunCompressedTensorsW8A8Int8MoEMethod(_MonolithicQuantMoE):

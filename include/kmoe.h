@@ -256,6 +256,8 @@ typedef struct kmoe_gemm_i8_args {
   const float* w_max_tail; /* [n]                                                */
   int32_t tail_row0, tail_rows, tail_src0;
   int32_t act_dtype;      /* KMOE_DT_*: dtype of y (and of the rounding of gate and up before SiLU-mul) */
+  int32_t rows_hint;      /* 0, or the rows the caller expects to be live when `rows` is only their bound (an
+                             expert-parallel share): chooses the kernel, never the result          */
 } kmoe_gemm_i8_args;
 
 #define KMOE_W_ROWMAJOR 0
@@ -312,6 +314,8 @@ typedef struct kmoe_gemm_bf16_args {
   float act_alpha, act_limit; /* KMOE_ACT_SWIGLUOAI (the reference uses 1.702 and 7.0)    */
   int32_t act_dtype;      /* KMOE_DT_BF16, or KMOE_DT_F16: a, w and y are IEEE half (the
                              unquantized method under --dtype float16); without bias / SWIGLUOAI */
+  int32_t rows_hint;      /* 0, or the rows the caller expects to be live when `rows` is only their bound (an
+                             expert-parallel share): chooses the kernel, never the result          */
 } kmoe_gemm_bf16_args;
 
 /*
@@ -350,6 +354,8 @@ typedef struct kmoe_gemm_fp8_args {
   int32_t tail_row0, tail_rows, tail_src0;
   int32_t act_dtype;          /* KMOE_DT_BF16, or KMOE_DT_F16: y (and the rounding of gate and up before
                                  SiLU-mul) in IEEE half                                */
+  int32_t rows_hint;      /* 0, or the rows the caller expects to be live when `rows` is only their bound (an
+                             expert-parallel share): chooses the kernel, never the result          */
 } kmoe_gemm_fp8_args;
 
 /*
@@ -386,6 +392,8 @@ typedef struct kmoe_gemm_w4_args {
                              dequant_int4_native (quant_ops.py:71-86) itself computes  */
   int32_t scale_layout;   /* KMOE_S_ROWMAJOR: w_scale as the checkpoint holds it, [E, n, k/group_size];
                              KMOE_S_FRAG16: re-arranged by kmoe_tile_scales_w4 (same bytes in total) */
+  int32_t rows_hint;      /* 0, or the rows the caller expects to be live when `rows` is only their bound (an
+                             expert-parallel share): chooses the kernel, never the result          */
 } kmoe_gemm_w4_args;
 
 /*

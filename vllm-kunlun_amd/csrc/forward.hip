@@ -124,6 +124,7 @@ struct MlpPass {
   const float *w13_aux, *w2_aux;
   const int32_t* lod;
   int E, H, I, rows;
+  int rows_hint;   // 0, or the rows expected to be live (an expert-parallel share): see kmoe_gemm_*_args
   uint16_t* act;   // [rows, I] bf16
   void* actq;      // [rows, I] codes
   float* act_aux;  // [rows] or [rows, I/128]
@@ -172,6 +173,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.n = n;
     g.k = k;
     g.rows = m.rows;
+    g.rows_hint = m.rows_hint;
     g.y = y;
     g.ldy = ldy;
     g.act = act;
@@ -206,6 +208,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.n = n;
     g.k = k;
     g.rows = m.rows;
+    g.rows_hint = m.rows_hint;
     g.y = y;
     g.ldy = ldy;
     g.act = act;
@@ -234,6 +237,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.n = n;
     g.k = k;
     g.rows = m.rows;
+    g.rows_hint = m.rows_hint;
     g.y = y;
     g.ldy = ldy;
     g.act = act;
@@ -252,6 +256,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
   g.n = n;
   g.k = k;
   g.rows = m.rows;
+  g.rows_hint = m.rows_hint;
   g.y = y;
   g.ldy = ldy;
   g.act = first && m.oai ? KMOE_ACT_SWIGLUOAI : act;
@@ -523,6 +528,7 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
   routed.H = H;
   routed.I = I;
   routed.rows = P;
+  routed.rows_hint = a->E_global > E ? static_cast<int>(local_pairs(a)) : 0;
   routed.act = static_cast<uint16_t*>(at(L.act));
   routed.actq = at(L.actq);
   routed.act_aux = static_cast<float*>(at(L.actmax));
@@ -580,6 +586,7 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
     sh.E = 1;
     sh.I = a->I_shared;
     sh.rows = M;
+    sh.rows_hint = 0;
     if (stream_mode) {
       // On the weight-streaming path a dense expert is best run as the launch's TAIL expert: the kernel cuts
       // a tail's rows into 16- or 32-row slices for as many workgroups, while one routed expert with M rows

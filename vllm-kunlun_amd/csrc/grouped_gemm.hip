@@ -416,10 +416,10 @@ constexpr int kTiledMinRows = 10;
 inline bool tile_variant(int v) { return v == 5 || v == 6 || v == 11 || v == 12; }
 
 template <Kind KIND>
-int dispatch(const GemmParams& p, int rows, bool swiglu, int variant, hipStream_t s, const char* what) {
+int dispatch(const GemmParams& p, int rows, int live, bool swiglu, int variant, hipStream_t s, const char* what) {
   if (variant == 0) {
     // rows per expert if the routing were uniform; decides streaming vs tiled
-    const int avg = ceil_div(rows, p.E);
+    const int avg = ceil_div(live, p.E);
     variant = avg <= 16 ? 1 : (avg <= 48 ? 2 : 3);
   }
   switch (variant) {
@@ -485,14 +485,14 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
   // Tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5-9, 11, 12 force it)
   if (a->w_layout == KMOE_W_TILED && a->k >= 128 &&
       ((a->variant >= 5 && a->variant <= 9) || a->variant == 11 || a->variant == 12 ||
-       (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
+       (a->variant == 0 && ceil_div(expected_rows(a->rows, a->rows_hint), a->E) > kTiledMinRows)))
     return tiled_gemm_i8(a, as_stream(stream));
   KMOE_REQUIRE(a->variant < 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-12 need tiled weights and k >= 128");
   GemmParams p{a->a,   a->lda, a->a_max, a->row_src, a->src_div, a->w,   a->w_max,
                a->lod, a->E,   a->n,     a->k,       a->y,       a->ldy, a->acc_out, a->w_layout == KMOE_W_TILED,
                a->w_tail, a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0, nullptr, 0, 0.f, 0.f,
                a->act_dtype == KMOE_DT_F16};
-  return dispatch<Kind::I8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_i8");
+  return dispatch<Kind::I8>(p, a->rows, expected_rows(a->rows, a->rows_hint), swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_i8");
 }
 
 extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_t stream) {
@@ -527,15 +527,16 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
                "grouped_gemm_bf16: w_layout=%d (tiled weights need k %% 32 == 0, k=%d)", a->w_layout, a->k);
   // tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5, 6, 11 force it)
   if (a->w_layout == KMOE_W_TILED && a->k >= 64 && a->ldy % 8 == 0 &&
-      (tile_variant(a->variant) || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
+      (tile_variant(a->variant) || (a->variant == 0 && ceil_div(expected_rows(a->rows, a->rows_hint), a->E) > kTiledMinRows)))
     return tiled_gemm_bf16(a, as_stream(stream));
   KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variants 5, 6, 11 need tiled weights, k >= 64 and ldy %% 8 == 0");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), nullptr,    a->lod,  a->E,       a->n,
                a->k * 2,                              a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,
                nullptr, nullptr, 0, 0, 0, a->bias, oai ? 1 : 0, a->act_alpha, a->act_limit};
-  if (half) return dispatch<Kind::F16>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_bf16 (half)");
-  return dispatch<Kind::BF16>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_bf16");
+  const int live = expected_rows(a->rows, a->rows_hint);
+  if (half) return dispatch<Kind::F16>(p, a->rows, live, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_bf16 (half)");
+  return dispatch<Kind::BF16>(p, a->rows, live, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_bf16");
 }
 
 extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_stream_t stream) {
@@ -569,7 +570,7 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
                "grouped_gemm_fp8_block: w_layout=%d unknown", a->w_layout);
   // tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5, 6, 11 force it)
   if (a->w_layout == KMOE_W_TILED && a->k <= 8192 && a->ldy % 8 == 0 &&
-      (tile_variant(a->variant) || (a->variant == 0 && ceil_div(a->rows, a->E) > kTiledMinRows)))
+      (tile_variant(a->variant) || (a->variant == 0 && ceil_div(expected_rows(a->rows, a->rows_hint), a->E) > kTiledMinRows)))
     return tiled_gemm_fp8(a, as_stream(stream));
   KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_fp8_block: variants 5, 6, 11 need tiled weights, k <= 8192");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,
@@ -577,5 +578,5 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
                a->k,                                  a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,
                reinterpret_cast<const int8_t*>(a->w_tail), a->w_scale_tail, a->tail_row0, tail_rows, a->tail_src0,
                nullptr, 0, 0.f, 0.f, a->act_dtype == KMOE_DT_F16};
-  return dispatch<Kind::FP8>(p, a->rows, swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_fp8_block");
+  return dispatch<Kind::FP8>(p, a->rows, expected_rows(a->rows, a->rows_hint), swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_fp8_block");
 }

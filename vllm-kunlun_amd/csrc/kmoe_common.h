@@ -7,6 +7,11 @@
 
 namespace kmoe {
 
+// Rows a launch expects to be live: `rows` bounds the sorted rows (grids and buffers are sized by it), the hint of
+// the argument blocks (0: none) says how many of them the caller expects to exist - an expert-parallel share
+// sorts only the pairs routed to its own experts. Kernels are CHOSEN by it; every choice is correct for any count.
+inline int expected_rows(int rows, int hint) { return hint > 0 && hint < rows ? hint : rows; }
+
 constexpr int kWave = 64;
 
 // ---- error plumbing (host) -------------------------------------------------

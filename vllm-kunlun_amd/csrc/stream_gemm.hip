@@ -273,7 +273,7 @@ int stream_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   if (mf == 0) {
     // An expert with more rows than one pass holds streams its weights again: leave headroom
     // over the mean for the spread of a random routing (about +-2 sigma at these sizes).
-    const int avg = ceil_div(a->rows, a->E);
+    const int avg = ceil_div(expected_rows(a->rows, a->rows_hint), a->E);
     mf = avg <= 10 ? 1 : (avg <= 22 ? 2 : (avg <= 48 ? 4 : 8));
   }
   switch (mf) {

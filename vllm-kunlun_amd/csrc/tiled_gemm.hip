@@ -970,8 +970,9 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   int n_cu = 0;
   if (int rc = tiled_common(p, a->rows, &n_cu, what)) return rc;
   constexpr TKind K = TKind::I8;
-  const int avg_rows = ceil_div(a->rows + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
-  const bool shorter = short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu);
+  const int live = expected_rows(a->rows, a->rows_hint);  // (chooses the tile shape; grids and bounds keep a->rows)
+  const int avg_rows = ceil_div(live + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
+  const bool shorter = short_tiles(a->variant, live, a->E, a->n, swiglu, n_cu);
   // 128-row tiles whose sibling m-tiles are paced against each other (see g_board). By default where experts
   // have more than one m-tile (more than 96 rows on average) AND the launch's weights are far more than the
   // 256 MB memory-side cache holds: there a sibling that falls behind fetches its weights from HBM again, and
@@ -1037,7 +1038,8 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
   // (64x128 tiles for a dense GEMM of a few rows, twice the work items: 57 -> 42 us on [128,7168] x [4096,7168],
   // still bound by what one workgroup keeps in flight; not instantiated)
   const bool half = a->act_dtype == KMOE_DT_F16;  // half outputs: the same three shapes
-  if (short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu)) {
+  const int live = expected_rows(a->rows, a->rows_hint);
+  if (short_tiles(a->variant, live, a->E, a->n, swiglu, n_cu)) {
     if (half)
       return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4, false, false, true>(p, a->rows, s, n_cu, what)
                     : launch_tiled<K, false, 4, 4, 2, 1, false, 4, false, false, true>(p, a->rows, s, n_cu, what);
@@ -1048,7 +1050,7 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
   // memory-side cache holds, as for int8, and a tile walks a long K (DeepSeek-V3 shape at 4096 tokens: gate_up,
   // K = 7168, 2570 -> 2222 us; the down projection, K = 2048, is 5 % slower with it: 1033 -> 1083 us; layer at
   // 8192 tokens 5.86 -> 5.78 ms, at 16384 tokens 10.90 -> 10.66 ms)
-  const int avg_rows = ceil_div(a->rows + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
+  const int avg_rows = ceil_div(live + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
   const long long weight_bytes = static_cast<long long>(a->E + (a->w_tail ? 1 : 0)) * a->n * a->k;
   if (a->variant == 12 || (a->variant == 0 && avg_rows > 96 && a->k >= 4096 && weight_bytes > (1ll << 30))) {
     if (half)
@@ -1078,7 +1080,7 @@ int tiled_gemm_bf16(const kmoe_gemm_bf16_args* a, hipStream_t s) {
   p.bias = a->bias;
   p.oai_alpha = a->act_alpha;
   p.oai_limit = a->act_limit;
-  const bool shorter = short_tiles(a->variant, a->rows, a->E, a->n, swiglu, n_cu, 40);  // measured: at 48 rows per expert the 128-row tiles are 4 % ahead
+  const bool shorter = short_tiles(a->variant, expected_rows(a->rows, a->rows_hint), a->E, a->n, swiglu, n_cu, 40);  // measured: at 48 rows per expert the 128-row tiles are 4 % ahead
   if (a->act == KMOE_ACT_SWIGLUOAI)
     return shorter ? launch_tiled<K, false, 4, 4, 2, 1, false, 4, true>(p, a->rows, s, n_cu, what)
                    : launch_tiled<K, false, 4, 4, 2, 1, false, 8, true>(p, a->rows, s, n_cu, what);

@@ -618,7 +618,7 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
     // the 128-row tile kernel is ahead, although most of its tile is padding there (Qwen3 shape, gate_up / down:
     // 16 rows per expert 87 / 50 us streaming against 106 / 58 us, 24 rows 107 / 58 against 109 / 58, 32 rows
     // 141 / 76 against 109 / 60, 128 rows 462 / 212 against 186 / 102).
-    const int avg = ceil_div(a->rows, a->E);
+    const int avg = ceil_div(expected_rows(a->rows, a->rows_hint), a->E);
     mf = avg <= 10 ? 1 : (avg <= 22 ? 2 : (tile_ok ? 8 : 4));
   }
   switch (mf) {

@@ -41,6 +41,7 @@ class GemmI8Args(C.Structure):
         ("variant", C.c_int32), ("w_layout", C.c_int32), ("a_layout", C.c_int32), ("a_rows", C.c_int32),
         ("w_tail", C.c_void_p), ("w_max_tail", C.c_void_p), ("tail_row0", C.c_int32), ("tail_rows", C.c_int32),
         ("tail_src0", C.c_int32), ("act_dtype", C.c_int32),
+        ("rows_hint", C.c_int32),
     ]
 
 
@@ -52,6 +53,7 @@ class GemmBf16Args(C.Structure):
         ("y", C.c_void_p), ("ldy", C.c_int64), ("act", C.c_int32), ("variant", C.c_int32),
         ("w_layout", C.c_int32), ("bias", C.c_void_p), ("act_alpha", C.c_float), ("act_limit", C.c_float),
         ("act_dtype", C.c_int32),
+        ("rows_hint", C.c_int32),
     ]
 
 
@@ -62,6 +64,7 @@ class GemmW4Args(C.Structure):
         ("E", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("rows", C.c_int32),
         ("y", C.c_void_p), ("ldy", C.c_int64), ("act", C.c_int32), ("variant", C.c_int32),
         ("w_layout", C.c_int32), ("act_dtype", C.c_int32), ("scale_layout", C.c_int32),
+        ("rows_hint", C.c_int32),
     ]
 
 
@@ -74,6 +77,7 @@ class GemmFp8Args(C.Structure):
         ("w_layout", C.c_int32),
         ("w_tail", C.c_void_p), ("w_scale_tail", C.c_void_p),
         ("tail_row0", C.c_int32), ("tail_rows", C.c_int32), ("tail_src0", C.c_int32), ("act_dtype", C.c_int32),
+        ("rows_hint", C.c_int32),
     ]
 
 

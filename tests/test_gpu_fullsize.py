@@ -72,8 +72,8 @@ def _properties(sl, host, n_decode, n_spot, seed, mids=(), half=False):
     assert torch.equal(dec, full[:n_decode]), "decode and prefill kernels disagree"
     ref = _oracle(sl, host, x[:n_decode], logits[:n_decode])
     assert np.array_equal(bits(dec), ref), "decode batch vs C oracle"
-    # batches in between: the streaming kernels' last sizes, the tile kernel on 64-row tiles, on 128-row
-    # tiles that are mostly padding
+    # batches in between: the streaming kernels' last sizes, the tile kernel on 64-row tiles, on 96-row tiles and
+    # on 128-row tiles that are mostly padding
     for m in mids:
         mid = _run(sl, x[:m].contiguous(), logits[:m].contiguous())
         assert torch.equal(mid, full[:m]), f"a batch of {m} tokens disagrees with the full batch"
@@ -86,13 +86,13 @@ def _properties(sl, host, n_decode, n_spot, seed, mids=(), half=False):
 def test_qwen3_full_size(qwen3):
     """Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, intermediate 768; 8192 and 64 tokens."""
     sl, host = qwen3
-    _properties(sl, host, n_decode=64, n_spot=48, seed=1, mids=(160, 176, 512, 768, 800, 1500))
+    _properties(sl, host, n_decode=64, n_spot=48, seed=1, mids=(160, 176, 512, 768, 800, 1100, 1200, 1500))
 
 
 def test_qwen3_full_size_float16(qwen3):
     """The same layer with float16 activations (the dtype of the reference's deployment recipes)."""
     sl, host = qwen3
-    _properties(sl, host, n_decode=64, n_spot=48, seed=4, mids=(160, 512, 1500), half=True)
+    _properties(sl, host, n_decode=64, n_spot=48, seed=4, mids=(160, 512, 900, 1500), half=True)
 
 
 def test_qwen3_full_size_skewed_routing(qwen3):
@@ -114,7 +114,7 @@ def test_dsv3_full_size(dsv3):
 
 def test_dsv3_full_size_float16(dsv3):
     sl, host = dsv3
-    _properties(sl, host, n_decode=128, n_spot=12, seed=5, mids=(352, 1536), half=True)
+    _properties(sl, host, n_decode=128, n_spot=12, seed=5, mids=(352, 1536, 1800), half=True)
 
 
 def _fp8_oracle(sl, host, x, logits):

@@ -516,7 +516,7 @@ PERSISTENT_CASES = TILED_CASES + [
 
 
 @pytest.mark.parametrize("E,n,k,counts", PERSISTENT_CASES)
-@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 7, 8, 9, 11, 12])
+@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 7, 8, 9, 11, 12, 13])
 @pytest.mark.parametrize("act", [0, 1])
 def test_lds_gemm_i8_with_tiled_weights(L, E, n, k, counts, variant, act):
     """LDS-staged kernels reading tiled weights and row-major activations. Variants 1-3: small

@@ -413,7 +413,7 @@ int launch(const GemmParams& p, int rows, hipStream_t s, const char* what) {
 constexpr int kTiledMinRows = 10;
 // variants of the bf16 and fp8 launchers that force the tile kernel: 5 (tile height from the rows per expert),
 // 6 (128-row tiles), 11 (64-row tiles)
-inline bool tile_variant(int v) { return v == 5 || v == 6 || v == 11 || v == 12; }
+inline bool tile_variant(int v) { return v == 5 || v == 6 || (v >= 11 && v <= 13); }
 
 template <Kind KIND>
 int dispatch(const GemmParams& p, int rows, int live, bool swiglu, int variant, hipStream_t s, const char* what) {
@@ -529,7 +529,7 @@ extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_
   if (a->w_layout == KMOE_W_TILED && a->k >= 64 && a->ldy % 8 == 0 &&
       (tile_variant(a->variant) || (a->variant == 0 && ceil_div(expected_rows(a->rows, a->rows_hint), a->E) > kTiledMinRows)))
     return tiled_gemm_bf16(a, as_stream(stream));
-  KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variants 5, 6, 11 need tiled weights, k >= 64 and ldy %% 8 == 0");
+  KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_bf16: variants 5, 6, 11-13 need tiled weights, k >= 64 and ldy %% 8 == 0");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda * 2, nullptr, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), nullptr,    a->lod,  a->E,       a->n,
                a->k * 2,                              a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,
@@ -572,7 +572,7 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
   if (a->w_layout == KMOE_W_TILED && a->k <= 8192 && a->ldy % 8 == 0 &&
       (tile_variant(a->variant) || (a->variant == 0 && ceil_div(expected_rows(a->rows, a->rows_hint), a->E) > kTiledMinRows)))
     return tiled_gemm_fp8(a, as_stream(stream));
-  KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_fp8_block: variants 5, 6, 11 need tiled weights, k <= 8192");
+  KMOE_REQUIRE(!tile_variant(a->variant), KMOE_ERR_UNSUPPORTED, "grouped_gemm_fp8_block: variants 5, 6, 11-13 need tiled weights, k <= 8192");
   GemmParams p{reinterpret_cast<const int8_t*>(a->a), a->lda, a->a_scale, a->row_src, a->src_div,
                reinterpret_cast<const int8_t*>(a->w), a->w_scale, a->lod,  a->E,       a->n,
                a->k,                                  a->y,       a->ldy,  nullptr, a->w_layout == KMOE_W_TILED,

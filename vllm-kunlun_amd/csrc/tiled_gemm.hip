@@ -947,10 +947,10 @@ int tiled_common(const TiledParams& p, int rows, int* n_cu_out, const char* what
 // a second pass over their weights: DeepSeek-V3 gate_up 1434 -> 1585 us, so the switch sits below that.
 // Also when 128-row tiles would leave most workgroups without an item (a dense GEMM of a few hundred rows: one
 // expert, fp8 [rows,7168] x [4096,7168]: 102 -> 57 us at 128 rows, 105 -> 62 us at 1024, 150 -> 163 us at 4096).
-// Variant 6 forces 128 rows, 11 forces 64.
+// Variant 6 (and 12) forces 128 rows, 11 forces 64, 13 forces 96.
 bool short_tiles(int variant, int rows, int n_experts, int n, bool swiglu, int n_cu, int max_avg_rows = 48) {
   if (variant == 11) return true;
-  if (variant == 6) return false;
+  if (variant == 6 || variant == 12 || variant == 13) return false;
   if (ceil_div(rows, n_experts) <= max_avg_rows) return true;
   const int n_blocks = ceil_div(swiglu ? n / 2 : n, kWavesT * (swiglu ? 2 : 4) * 16);
   return static_cast<long long>(rows / 128 + n_experts) * n_blocks < 2ll * n_cu;
@@ -1062,6 +1062,17 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
   // K = 7168, 2570 -> 2222 us; the down projection, K = 2048, is 5 % slower with it: 1033 -> 1083 us; layer at
   // 8192 tokens 5.86 -> 5.78 ms, at 16384 tokens 10.90 -> 10.66 ms)
   const int avg_rows = ceil_div(live + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
+  // 96-row tiles from 49 to 76 rows per expert: the padding rows of a 128-row tile cost this format its scaling work
+  // on top of the MFMAs (gate_up GEMM alone, 64 rows per expert: Qwen3 shape 105 -> 85 us, DeepSeek-V3 shape 1515 ->
+  // 1407 us; at 80 rows 107 -> 103 and 1541 -> 1508 us; at 90 rows the DeepSeek-V3 shape loses, 1578 -> 1812 us:
+  // too many experts need a second tile)
+  if (a->variant == 13 || (a->variant == 0 && avg_rows <= 76)) {
+    if (half)
+      return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 6, false, false, true>(p, a->rows, s, n_cu, what)
+                    : launch_tiled<K, false, 4, 4, 2, 1, false, 6, false, false, true>(p, a->rows, s, n_cu, what);
+    return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 6>(p, a->rows, s, n_cu, what)
+                  : launch_tiled<K, false, 4, 4, 2, 1, false, 6>(p, a->rows, s, n_cu, what);
+  }
   const long long weight_bytes = static_cast<long long>(a->E + (a->w_tail ? 1 : 0)) * a->n * a->k;
   if (a->variant == 12 || (a->variant == 0 && avg_rows > 96 && a->k >= 4096 && weight_bytes > (1ll << 30))) {
     if (half)

@@ -940,7 +940,8 @@ int tiled_common(const TiledParams& p, int rows, int* n_cu_out, const char* what
   return KMOE_OK;
 }
 
-// 64-row tiles (MF = 4) when nearly every expert fits one of them (48 rows per expert on average): the launch
+// 64-row tiles (MF = 4) when nearly every expert fits one of them (44 rows per expert on average; at 48 the
+// 96-row tiles are ahead, Qwen3 layer at 768 tokens 0.169 -> 0.158 ms, at 40 behind, 0.151 vs 0.155 ms): the launch
 // is bound by the weight stream, and half the MFMAs, fragment reads and epilogue per weight byte leave more of
 // the CU to it (measured, int8 gate_up / down: Qwen3 shape at 32 rows per expert 101 -> 80 us; DeepSeek-V3 shape
 // at 32 rows 1426 -> 1284 / 770 -> 683 us). At 64 rows per expert half of the experts need a second tile and
@@ -948,7 +949,7 @@ int tiled_common(const TiledParams& p, int rows, int* n_cu_out, const char* what
 // Also when 128-row tiles would leave most workgroups without an item (a dense GEMM of a few hundred rows: one
 // expert, fp8 [rows,7168] x [4096,7168]: 102 -> 57 us at 128 rows, 105 -> 62 us at 1024, 150 -> 163 us at 4096).
 // Variant 6 (and 12) forces 128 rows, 11 forces 64, 13 forces 96.
-bool short_tiles(int variant, int rows, int n_experts, int n, bool swiglu, int n_cu, int max_avg_rows = 48) {
+bool short_tiles(int variant, int rows, int n_experts, int n, bool swiglu, int n_cu, int max_avg_rows = 44) {
   if (variant == 11) return true;
   if (variant == 6 || variant == 12 || variant == 13) return false;
   if (ceil_div(rows, n_experts) <= max_avg_rows) return true;
@@ -984,7 +985,7 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   const long long weight_bytes = static_cast<long long>(a->E + (a->w_tail ? 1 : 0)) * a->n * a->k;
   const bool paced = a->variant == 12 ||
                      (a->variant == 0 && !shorter && avg_rows > 96 && weight_bytes > (1ll << 30));
-  // 96-row tiles between the two: from 49 to 72 rows per expert nearly every expert still fits one tile, and a
+  // 96-row tiles between the two: from 45 to 72 rows per expert nearly every expert still fits one tile, and a
   // quarter of the 128-row tile's MFMAs (all padding there) is saved (Qwen3 shape, layer: 768 tokens 0.169 ->
   // 0.158 ms, 1024 tokens 0.191 -> 0.165 ms; at 80 rows per expert too many experts need a second tile: -4 % on
   // the Qwen3 shape, +1 % on the DeepSeek-V3 one; DeepSeek-V3 shape at 64 rows per expert: -1.6 %).
@@ -1062,7 +1063,7 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
   // K = 7168, 2570 -> 2222 us; the down projection, K = 2048, is 5 % slower with it: 1033 -> 1083 us; layer at
   // 8192 tokens 5.86 -> 5.78 ms, at 16384 tokens 10.90 -> 10.66 ms)
   const int avg_rows = ceil_div(live + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
-  // 96-row tiles from 49 to 76 rows per expert: the padding rows of a 128-row tile cost this format its scaling work
+  // 96-row tiles from 45 to 76 rows per expert: the padding rows of a 128-row tile cost this format its scaling work
   // on top of the MFMAs (gate_up GEMM alone, 64 rows per expert: Qwen3 shape 105 -> 85 us, DeepSeek-V3 shape 1515 ->
   // 1407 us; at 80 rows 107 -> 103 and 1541 -> 1508 us; at 90 rows the DeepSeek-V3 shape loses, 1578 -> 1812 us:
   // too many experts need a second tile)

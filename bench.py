@@ -296,7 +296,7 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
         roofline = {"bound": "mfma", "achieved": achieved, "peak": peak_tops, "unit": "TFLOP/s",
                     "frac": achieved / peak_tops, "traffic": traffic}
     many_rows = shape.P > 10 * shape.E  # the launchers' switch to the persistent tile kernel
-    g1_kernel = (("w4_tile_kernel" if shape.P > 22 * shape.E else "w4_stream_kernel") if w4 else "stream_gemm_i8_kernel" if plan.layout.codes_chunked else
+    g1_kernel = (("w4_tile_kernel" if shape.P > (20 if shape.H > 4096 else 13) * shape.E else "w4_stream_kernel") if w4 else "stream_gemm_i8_kernel" if plan.layout.codes_chunked else
                  "tiled_gemm_kernel" if many_rows and plan.args.w_layout == L.KMOE_W_TILED else "grouped_gemm_kernel")
     roofline.update(kernel=g1_kernel + " (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
                     algorithmic_bytes=work["g1_bytes"], algorithmic_ops=work["g1_ops"],

@@ -385,7 +385,8 @@ typedef struct kmoe_gemm_w4_args {
   int64_t ldy;
   int32_t act;            /* KMOE_ACT_NONE or KMOE_ACT_SWIGLU                         */
   int32_t variant;        /* 0 = from the shape; 1, 2, 4 = 16-row fragments per pass of the
-                             streaming kernel; 8 = the 128-row tile kernel (prefill)  */
+                             streaming kernel; 64, 96, 128 = the tile kernel (prefill) with tiles
+                             of that many rows (8 = 128)                              */
   int32_t w_layout;       /* KMOE_W_TILED                                             */
   int32_t act_dtype;      /* KMOE_DT_BF16, or KMOE_DT_F16: a, w_scale and y are IEEE half and the
                              weight values are half((code - 8) * scale), what

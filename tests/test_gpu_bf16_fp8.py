@@ -520,16 +520,17 @@ W4_CASES = [
     (2, 64, 4224, [5, 20], 32),        # 132 groups per channel: too many for the LDS copy, scales read from memory
     (3, 96, 384, [130, 0, 260], 128),  # experts of two and three 128-row tiles, an empty one between them
     (5, 320, 256, [128, 1, 0, 129, 64], 64),  # tiles that end exactly at an expert's last row, and one row past it
+    (6, 64, 256, [64, 65, 96, 97, 0, 192], 128),  # the same for the 64- and 96-row tiles
 ]
 
 
 @pytest.mark.parametrize("E,n,k,counts,gs", W4_CASES)
-@pytest.mark.parametrize("variant", [0, 1, 2, 4, 8])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 8, 64, 96, 128])
 @pytest.mark.parametrize("act", [0, 1])
 @pytest.mark.parametrize("gather,frag16", [(False, False), (True, False), (True, True)])
 def test_grouped_gemm_w4a16(L, E, n, k, counts, gs, variant, act, gather, frag16):
-    """Packed 4-bit weights unpacked in registers (variants 1, 2, 4: the streaming kernel; 8: the 128-row tile
-    kernel; 0: chosen from the rows per expert) against the oracle's route: unpack (orc_dequant_w4_bf16, itself
+    """Packed 4-bit weights unpacked in registers (variants 1, 2, 4: the streaming kernel; 64, 96, 128 and its
+    older name 8: the tile kernel with tiles of that many rows; 0: chosen from the rows per expert) against the oracle's route: unpack (orc_dequant_w4_bf16, itself
     pinned by a brute-force check) then the bf16 grouped GEMM."""
     g = torch.Generator().manual_seed(E * n + k + (gs or 0))
     lod = _lod(counts)
@@ -567,7 +568,7 @@ def test_grouped_gemm_w4a16(L, E, n, k, counts, gs, variant, act, gather, frag16
     L.check(L.lib.kmoe_grouped_gemm_w4a16(args, L.stream()))
     torch.cuda.synchronize()
     assert rel_l2(y, from_bits(ref)) <= 2e-3   # the operands are the same bits: only summation order differs
-    if variant == 8:  # both kernels add the same products in the same order: the same bits
+    if variant >= 8:  # both kernels add the same products in the same order: the same bits
         y1 = torch.zeros_like(y)
         args.y, args.variant = y1.data_ptr(), 1
         L.check(L.lib.kmoe_grouped_gemm_w4a16(args, L.stream()))

@@ -274,7 +274,7 @@ W4_HALF_CASES = [
 
 
 @pytest.mark.parametrize("E,n,k,counts,gs", W4_HALF_CASES)
-@pytest.mark.parametrize("variant", [0, 1, 2, 4, 8])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 8, 64, 96])
 @pytest.mark.parametrize("act", [0, 1])
 def test_w4_half_dequant_and_gemm(E, n, k, counts, gs, variant, act):
     """kmoe_dequant_w4 in half mode: the oracle's bits (= the reference's float16 expression). The packed-weight

@@ -253,9 +253,9 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Prefill regime: 128-row tiles. The unpacking of a weight word is shared by the 8 row fragments of the
-// tile (23 VALU instructions against 8 MFMAs of 16 cycles), so the kernel is bound by the matrix cores
-// like the 16-bit tile kernels while it reads a quarter of their weight bytes. One workgroup: 128 sorted
+// Prefill regime: tiles of 64, 96 or 128 rows. The unpacking of a weight word is shared by the row fragments of
+// the tile (23 VALU instructions against 8 MFMAs of 16 cycles on the tallest), so the kernel is bound by the matrix cores
+// like the 16-bit tile kernels while it reads a quarter of their weight bytes. One workgroup: up to 128 sorted
 // rows of one expert x 4 waves x NF fragments of 16 channels. Activations are copied global -> LDS
 // asynchronously, one 128-value block of K (256 bytes per row) ahead, two buffers; every wave reads its A
 // fragments from there. Weights and their scales go global -> registers, one block ahead; they never pass
@@ -312,11 +312,11 @@ __device__ inline bool locate_w4_item(const W4Params& p, int n_blocks, int& e_ou
   return true;
 }
 
-// MF: 16-row fragments of a tile (8: 128-row tiles). 64-row tiles were measured and are not instantiated: a launch
-// whose experts hold a few dozen rows is bound by the unpacking and by the latency of its one-block-deep pipeline,
-// which a shorter tile does not change (Qwen3 shape, 4 to 64 rows per expert: 121 us against 111 us).
+// MF: 16-row fragments of a tile (4, 6, 8: 64-, 96- and 128-row tiles). Two workgroups per CU for every height:
+// with three, the 64-row instance had 170 registers to live in and lost to the 128-row one (121 against 111 us
+// over 4 to 64 rows per expert on the Qwen3 shape); with two it is a quarter ahead where experts fit its tile.
 template <int MF, int NF, bool SWIGLU, bool F16, bool SLDS>
-__global__ __launch_bounds__(kWaves* kWave, MF == 8 ? 2 : 3) void w4_tile_kernel(const W4Params p) {
+__global__ __launch_bounds__(kWaves* kWave, 2) void w4_tile_kernel(const W4Params p) {
   constexpr int kTileRows = 16 * MF;
   extern __shared__ uint16_t scale_lds[];  // SLDS: [kWaves][NF][16][groups], every wave its own part (as in the streaming kernel)
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
@@ -610,17 +610,29 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
                    frag16 ? 1 : groups, frag16 ? 16 : 1, a->lod, a->E, a->n, a->k, a->y, a->ldy};
   hipStream_t s = as_stream(stream);
   int mf = a->variant;
-  // the 128-row tile kernel reaches a source row (gathered or not: below `rows`) through a 32-bit byte offset
+  // the tile kernel reaches a source row (gathered or not: below `rows`) through a 32-bit byte offset
   const bool tile_ok = static_cast<uint64_t>(a->rows) * static_cast<uint64_t>(a->lda) * 2u + static_cast<uint64_t>(a->k) * 2u < (1ull << 32);
   if (mf == 0) {
     // rows an expert gets under uniform routing, with headroom for the spread: an expert with
-    // more rows than one pass holds streams (and unpacks) its weights again. From two dozen rows per expert
-    // the 128-row tile kernel is ahead, although most of its tile is padding there (Qwen3 shape, gate_up / down:
-    // 16 rows per expert 87 / 50 us streaming against 106 / 58 us, 24 rows 107 / 58 against 109 / 58, 32 rows
-    // 141 / 76 against 109 / 60, 128 rows 462 / 212 against 186 / 102).
+    // more rows than one pass holds streams (and unpacks) its weights again. From a dozen and a half rows per
+    // expert the tile kernel is ahead on its shortest tile, which is mostly padding there (later when K is long:
+    // the streaming kernel's waves then live longer per weight byte); the tile grows when too many experts would
+    // need a second one (gate_up, Qwen3 shape / Kimi-K2 shape with groups of 32, us: 12 rows per expert streaming
+    // 75 against 87 on 64-row tiles, 16 rows 96 / 1976 against 87 / 2196, 21 rows - / 2196 against - / 2225, 24 rows
+    // 109 against 82, 32 rows 3176 against 2250; 64-, 96-, 128-row tiles at 44 rows 84 / 99 / 109, at 48 rows
+    // 111 / 109 / 120 and 2440 / 2609 / 2918, at 56 rows 111 / 107 / 119 and 2634 / 2614 / 2993, at 64 rows
+    // 133 / 109 / 121, at 76 rows 156 / 109 / 122 and 4073 / 2708 / 3113, at 80 rows - / 136 / 127).
     const int avg = ceil_div(expected_rows(a->rows, a->rows_hint), a->E);
-    mf = avg <= 10 ? 1 : (avg <= 22 ? 2 : (tile_ok ? 8 : 4));
+    // (with K = 2048 the 32-row streaming pass is never the best: 12 rows per expert 75 on 16-row passes, 84 on
+    // 32-row passes, 87 on 64-row tiles; 16 rows 99 / 96 / 87)
+    const int one_max = a->k > 4096 ? 10 : 13;
+    const int stream_max = a->k > 4096 ? 20 : 13;
+    mf = avg <= one_max ? 1 : (avg <= stream_max ? 2 : (!tile_ok ? 4 : (avg <= 48 ? 64 : (avg <= 76 ? 96 : 128))));
   }
+  if (mf == 8) mf = 128;
+  if (mf == 64 || mf == 96 || mf == 128)
+    KMOE_REQUIRE(tile_ok, KMOE_ERR_SHAPE, "grouped_gemm_w4a16: the tile kernel addresses the activations with 32 bits (rows=%d lda=%lld)",
+                 a->rows, static_cast<long long>(a->lda));
   switch (mf) {
     // One block in flight per wave: the registers that saves put more waves on a SIMD (5-6 instead of 3-4), and
     // the unpacking work of one wave hides the loads of the others better than a deeper queue of its own does
@@ -634,11 +646,10 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
     case 143: return swiglu ? launch_w4<1, 4, true, 3>(p, f16, s) : launch_w4<1, 4, false, 3>(p, f16, s);
     case 2: return swiglu ? launch_w4<2, 2, true, 2>(p, f16, s) : launch_w4<2, 2, false, 2>(p, f16, s);
     case 4: return swiglu ? launch_w4<4, 2, true, 2>(p, f16, s) : launch_w4<4, 2, false, 2>(p, f16, s);
-    case 8:
-      KMOE_REQUIRE(tile_ok, KMOE_ERR_SHAPE, "grouped_gemm_w4a16: the tile kernel addresses the activations with 32 bits (rows=%d lda=%lld)",
-                   a->rows, static_cast<long long>(a->lda));
-      return swiglu ? launch_w4_tile<8, true>(p, a->rows, f16, s) : launch_w4_tile<8, false>(p, a->rows, f16, s);
+    case 64: return swiglu ? launch_w4_tile<4, true>(p, a->rows, f16, s) : launch_w4_tile<4, false>(p, a->rows, f16, s);
+    case 96: return swiglu ? launch_w4_tile<6, true>(p, a->rows, f16, s) : launch_w4_tile<6, false>(p, a->rows, f16, s);
+    case 128: return swiglu ? launch_w4_tile<8, true>(p, a->rows, f16, s) : launch_w4_tile<8, false>(p, a->rows, f16, s);
     default:
-      return fail(KMOE_ERR_UNSUPPORTED, "grouped_gemm_w4a16: variant=%d must be 0, 1, 2, 4 or 8 (or a tuning variant)", a->variant);
+      return fail(KMOE_ERR_UNSUPPORTED, "grouped_gemm_w4a16: variant=%d must be 0, 1, 2, 4, 8, 64, 96 or 128 (or a tuning variant)", a->variant);
   }
 }

@@ -321,7 +321,7 @@ class KunlunCompressedTensorsWNA16MoEMethod:
     unpacks the whole packed weight tensors to fp16 inside EVERY apply() (:320-327) and then
     calls the unquantized fused_moe. Here, in process_weights_after_loading:
       * the packed tensors are tiled in place and kept for kmoe_grouped_gemm_w4a16, which unpacks in
-        registers (a weight-streaming kernel for decode-sized batches, a kernel on 128-row tiles beyond;
+        registers (a weight-streaming kernel for decode-sized batches, a kernel on 64- to 128-row tiles beyond;
         needs hidden and intermediate sizes that are multiples of 128 and a group size that is a multiple
         of 32);
       * or the weights are unpacked ONCE (kmoe_dequant_w4) to tiled 16-bit tensors for the unquantized path.

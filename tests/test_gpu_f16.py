@@ -73,6 +73,30 @@ def test_half_layer_matches_the_oracle(name, base, over):
     assert rel_l2(out, routed) <= 1e-2
 
 
+def test_half_layer_on_8_wave_tiles_gives_the_same_bits():
+    """The 8-wave tiles of the int8 tile kernel (tile_variant 8, 14-16) in their half instantiations: the bits of
+    the default choice, which the cases above compare with the oracle."""
+    from vllm_kunlun_amd import _lib as L
+    from vllm_kunlun_amd import synth
+    from vllm_kunlun_amd._plan import make_moe_plan
+    shape = synth.scaled(synth.SHAPES["dsv3-decode"], M=1100, H=512, E=16, K=4, I=256, n_group=4, topk_group=2,
+                         I_shared=256)
+    sl = synth.make_w8a8_layer(shape, "cuda", seed=21)
+    lay = sl.layer
+    x = (sl.x.float() * 1.5).half()
+    outs = []
+    for variant in (0, 8, 14, 15, 16):
+        out = torch.empty_like(x)
+        plan = make_moe_plan(L.KMOE_FMT_INT8, x, sl.logits, out, shape.K, lay.w13_weight, lay.w2_weight,
+                             lay.w13_weight_scale, lay.w2_weight_scale, shape.scoring, True, shape.n_group,
+                             shape.topk_group, shape.routed_scale, sl.bias, sl.shared, 1.0, tile_variant=variant)
+        plan()
+        torch.cuda.synchronize()
+        outs.append(out)
+    assert bool(torch.isfinite(outs[0].float()).all()) and float(outs[0].float().abs().max()) > 0
+    assert all(torch.equal(outs[0], o) for o in outs[1:])
+
+
 def test_half_layer_with_the_router_gemm_inside():
     from vllm_kunlun_amd import synth
     shape = synth.scaled(synth.SHAPES["qwen3-decode"], M=48, H=512, E=64, K=4, I=128)

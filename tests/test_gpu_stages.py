@@ -512,17 +512,19 @@ PERSISTENT_CASES = TILED_CASES + [
     (4, 128, 576, [70, 0, 129, 5]),
     (2, 64, 704, [33, 200]),
     (8, 4096, 192, [((97 * i) % 300) for i in range(8)]),
+    # experts that end exactly at the last row of a 160-, 192-, 224- or 256-row tile, and one row past it
+    (8, 128, 384, [160, 161, 192, 193, 224, 225, 256, 257]),
 ]
 
 
 @pytest.mark.parametrize("E,n,k,counts", PERSISTENT_CASES)
-@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 7, 8, 9, 11, 12, 13])
+@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 7, 8, 9, 11, 12, 13, 14, 15, 16])
 @pytest.mark.parametrize("act", [0, 1])
 def test_lds_gemm_i8_with_tiled_weights(L, E, n, k, counts, variant, act):
     """LDS-staged kernels reading tiled weights and row-major activations. Variants 1-3: small
     tiles; 5-7: the persistent 128-row-tile kernel (6: 256-channel tiles, 7: 128-channel tiles
-    with the deep weight ring, 8: 256-row tiles with 8 waves, 5: the default, 12: sibling m-tiles
-    paced against each other through the progress board)."""
+    with the deep weight ring, 8 / 14 / 15 / 16: 256-, 192-, 160-, 224-row tiles with 8 waves, 5: the default,
+    12: sibling m-tiles paced against each other through the progress board)."""
     if variant >= 5 and k < 128:
         pytest.skip("the persistent kernel takes k >= 128")
     if variant < 5 and E >= 40:

@@ -213,6 +213,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.ldy = ldy;
     g.act = act;
     g.w_layout = m.w_layout;
+    g.variant = m.variant;
     if (m.tail_rows > 0) {
       g.w_tail = static_cast<const uint8_t*>(first ? m.w13_tail : m.w2_tail);
       g.w_scale_tail = first ? m.w13_aux_tail : m.w2_aux_tail;
@@ -549,8 +550,12 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
   routed.stream = stream_mode;
   routed.x_count = M;
   if (a->format == KMOE_FMT_INT8 && !stream_mode && a->w_layout == KMOE_W_TILED && a->tile_variant >= 5 &&
-      a->tile_variant <= 13 && (local_pairs(a) + E - 1) / E > 10 && H >= 128 && I >= 128)
+      a->tile_variant <= 16 && (local_pairs(a) + E - 1) / E > 10 && H >= 128 && I >= 128)
     routed.variant = a->tile_variant;
+  const int tv = a->tile_variant;
+  if (a->format == KMOE_FMT_FP8_BLOCK && a->w_layout == KMOE_W_TILED && (local_pairs(a) + E - 1) / E > 10 &&
+      (tv == 5 || tv == 6 || tv == 8 || (tv >= 11 && tv <= 14)))
+    routed.variant = tv;
   const bool fold = fold_shared(a);
   if (fold) {
     routed.w13_tail = a->ws13;
@@ -587,6 +592,7 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
     sh.I = a->I_shared;
     sh.rows = M;
     sh.rows_hint = 0;
+    sh.variant = 0;  // (a tuning variant of the routed GEMMs does not apply to the dense pass)
     if (stream_mode) {
       // On the weight-streaming path a dense expert is best run as the launch's TAIL expert: the kernel cuts
       // a tail's rows into 16- or 32-row slices for as many workgroups, while one routed expert with M rows

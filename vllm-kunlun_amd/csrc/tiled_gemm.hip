@@ -141,8 +141,12 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   static_assert(!F16 || KIND != TKind::BF16 || !OAI, "the interleaved activation is a bf16 epilogue");
   static_assert(!OAI || (KIND == TKind::BF16 && !SWIGLU && !M32), "the interleaved activation is a bf16 epilogue");
   constexpr int kMF = MF;
-  constexpr int kNA = 16 * kMF * (kChunk / 16) / (kWavesT * kWave);  // 16-byte activation vectors per thread and chunk
+  // 16-byte activation vectors per thread and chunk; an odd MF rounds up: the copies then cover up to 8 rows per
+  // wave past the tile's last row (rows of the next tile, or the tile's first row again), which land in buffer
+  // rows that no fragment reads
+  constexpr int kNA = (16 * kMF * (kChunk / 16) + kWavesT * kWave - 1) / (kWavesT * kWave);
   static_assert(kNA >= 1 && (M32 ? MF % 2 == 0 : true), "tile height");
+  static_assert(MF % 2 == 0 || KIND != TKind::F8, "an odd tile height needs the asynchronous activation path");
   constexpr bool F8 = KIND == TKind::F8;
   constexpr bool I8 = KIND == TKind::I8;
   constexpr bool BF = KIND == TKind::BF16;
@@ -164,7 +168,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   // consecutive rows of one fragment column fall on eight different bank groups). F8 keeps the
   // register path (its row scales travel with the data): two padded buffers.
   constexpr bool ADMA = !F8;
-  constexpr int kStageBytes = ADMA ? kTM * kChunk : kTM * kPitchT;
+  constexpr int kStageBytes = ADMA ? WM * kWavesT * kNA * 8 * kChunk : kTM * kPitchT;  // (ADMA: kTM rows, or the copies' 8 kNA per wave)
   __shared__ __attribute__((aligned(1024))) int8_t lds_a[ADMA ? kStagesA : 2][kStageBytes];
   __shared__ __attribute__((aligned(16))) int8_t patch[WM * kWavesT][kFragRows * kPatchPitch];
   // I8, per tile parity: channel scales (w_max / 127) and row scales (a_max / 127)
@@ -940,6 +944,16 @@ int tiled_common(const TiledParams& p, int rows, int* n_cu_out, const char* what
   return KMOE_OK;
 }
 
+// 8-wave tiles of 32 MF rows, one workgroup per CU.
+template <TKind K, int MF>
+int launch_tall(TiledParams& p, int rows, hipStream_t s, int n_cu, const char* what, bool swiglu, bool f16) {
+  if (f16)
+    return swiglu ? launch_tiled<K, true, 4, 4, 1, 2, false, MF, false, false, true>(p, rows, s, n_cu, what)
+                  : launch_tiled<K, false, 4, 4, 1, 2, false, MF, false, false, true>(p, rows, s, n_cu, what);
+  return swiglu ? launch_tiled<K, true, 4, 4, 1, 2, false, MF>(p, rows, s, n_cu, what)
+                : launch_tiled<K, false, 4, 4, 1, 2, false, MF>(p, rows, s, n_cu, what);
+}
+
 // 64-row tiles (MF = 4) when nearly every expert fits one of them (44 rows per expert on average; at 48 the
 // 96-row tiles are ahead, Qwen3 layer at 768 tokens 0.169 -> 0.158 ms, at 40 behind, 0.151 vs 0.155 ms): the launch
 // is bound by the weight stream, and half the MFMAs, fragment reads and epilogue per weight byte leave more of
@@ -951,7 +965,7 @@ int tiled_common(const TiledParams& p, int rows, int* n_cu_out, const char* what
 // Variant 6 (and 12) forces 128 rows, 11 forces 64, 13 forces 96.
 bool short_tiles(int variant, int rows, int n_experts, int n, bool swiglu, int n_cu, int max_avg_rows = 44) {
   if (variant == 11) return true;
-  if (variant == 6 || variant == 12 || variant == 13) return false;
+  if (variant == 6 || variant == 8 || (variant >= 12 && variant <= 16)) return false;
   if (ceil_div(rows, n_experts) <= max_avg_rows) return true;
   const int n_blocks = ceil_div(swiglu ? n / 2 : n, kWavesT * (swiglu ? 2 : 4) * 16);
   return static_cast<long long>(rows / 128 + n_experts) * n_blocks < 2ll * n_cu;
@@ -990,6 +1004,33 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   // 0.158 ms, 1024 tokens 0.191 -> 0.165 ms; at 80 rows per expert too many experts need a second tile: -4 % on
   // the Qwen3 shape, +1 % on the DeepSeek-V3 one; DeepSeek-V3 shape at 64 rows per expert: -1.6 %).
   const bool mid = a->variant == 13 || (a->variant == 0 && !shorter && avg_rows <= 72);
+  // One 8-wave tile per expert (WM = 2: 160, 192, 224 or 256 rows, one workgroup per CU) where experts hold a
+  // little more than one 128-row tile and the launch's weights are far more than the memory-side cache holds: the
+  // shortest such tile that nearly every expert fits (average + 2 sqrt(average) rows). The second 128-row tile of
+  // an expert is mostly padding and streams the expert's weights again; one taller tile does neither, which is
+  // worth more than what the lone workgroup loses by having nothing to run under its epilogue (DeepSeek-V3
+  // shape, gate_up / down, paced 128-row tiles against the tall tile: 120 rows per expert 1724 against 1598 us,
+  // 128 rows 1996 / 977 against 1743 / 866, 144 rows 2105 / 1167 against 1689 / 868, 176 rows 2171 / 1196 against
+  // 1830 / 953, 224 rows 2404 against 2172; at 96 rows 1457 against 1619: the 128-row tile holds them all). Inside
+  // the layer, where gate_up gathers its rows from the few token rows and the shared expert's rows ride along as
+  // the tail expert, less of it is left: DeepSeek-V3 layer at 4096 tokens 3.07 -> 2.97 ms, at 4608 tokens 3.31 ->
+  // 3.09, at 3584 and 5120 tokens -1 and -2 %, from 6144 tokens on the same. With weights that fit the cache the
+  // second pass is cheap and the gain is within noise (Qwen3 shape, 128 rows per expert: 125 against 122 us),
+  // while an expert that overflows the tall tile costs a quarter there: not used.
+  int tall = a->variant == 8 ? 8 : (a->variant == 14 ? 6 : (a->variant == 15 ? 5 : (a->variant == 16 ? 7 : 0)));
+  if (a->variant == 0 && !shorter && weight_bytes > (1ll << 30)) {
+    const float reach = static_cast<float>(avg_rows) + 2.0f * sqrtf(static_cast<float>(avg_rows));
+    if (reach > 128.0f && reach <= 256.0f) tall = reach <= 160.0f ? 5 : (reach <= 192.0f ? 6 : (reach <= 224.0f ? 7 : 8));
+  }
+  if (tall) {
+    const bool f16 = a->act_dtype == KMOE_DT_F16;
+    switch (tall) {
+      case 5: return launch_tall<K, 5>(p, a->rows, s, n_cu, what, swiglu, f16);
+      case 6: return launch_tall<K, 6>(p, a->rows, s, n_cu, what, swiglu, f16);
+      case 7: return launch_tall<K, 7>(p, a->rows, s, n_cu, what, swiglu, f16);
+      default: return launch_tall<K, 8>(p, a->rows, s, n_cu, what, swiglu, f16);
+    }
+  }
   if (a->act_dtype == KMOE_DT_F16) {
     // half outputs: the shapes in use (64-, 96-, 128-row and paced 128-row tiles); the tuning variants are bf16 only
     KMOE_REQUIRE(a->variant == 0 || a->variant == 5 || a->variant == 6 || (a->variant >= 11 && a->variant <= 13),
@@ -1012,12 +1053,6 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   if (a->variant == 7)
     return swiglu ? launch_tiled<K, true, 2, 8, 2, 1>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 2, 8, 2, 1>(p, a->rows, s, n_cu, what);
-  // 256-row tiles bring DeepSeek-V3 prefill (128-256 rows per expert) down to its algorithmic HBM
-  // traffic (measured 1.04x against 1.44x), but one workgroup per CU has nothing to run under its
-  // epilogue and tile switch: 3.7 TB/s, 13 % slower overall. Kept as a tuning variant.
-  if (a->variant == 8)
-    return swiglu ? launch_tiled<K, true, 4, 4, 1, 2>(p, a->rows, s, n_cu, what)
-                  : launch_tiled<K, false, 4, 4, 1, 2>(p, a->rows, s, n_cu, what);
   // (the 32x32 shapes are instantiated for the gate_up launch only: without SiLU-mul the 16-register
   // fragments of the plain epilogue do not fit two workgroups per CU)
   if (a->variant == 9 && swiglu) return launch_tiled<K, true, 4, 4, 2, 1, true>(p, a->rows, s, n_cu, what);
@@ -1075,6 +1110,19 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 6>(p, a->rows, s, n_cu, what);
   }
   const long long weight_bytes = static_cast<long long>(a->E + (a->w_tail ? 1 : 0)) * a->n * a->k;
+  // One 8-wave tile of 192 rows per expert where nearly every expert fits it and many would overflow a 128-row
+  // tile, as for int8 - for the short K of the down projection only, where pacing does not pay. Stand-alone the
+  // tall tile wins on both projections (DeepSeek-V3 shape, gate_up / down against the paced 128-row tiles: 128
+  // rows per expert 2158 / 1009 -> 2131 / 981 us, 144 rows 2513 / 1265 -> 2191 / 994, 160 rows 2643 / 1333 -> 2510
+  // / 1027; at 112 rows 1943 -> 2092 and at 192 rows 2588 -> 3558: not there), but inside the layer, with the
+  // shared expert's 4096 rows as the launch's tail, gate_up loses (4096 tokens: 2.21 -> 2.51 ms, 4608: 2.45 ->
+  // 2.63) while down still gains (1.10 -> 1.01 ms, 1.22 -> 1.07, 5120 tokens 1.31 -> 1.16). The 256-row instance
+  // spills and is a tuning variant.
+  const float reach = static_cast<float>(avg_rows) + 2.0f * sqrtf(static_cast<float>(avg_rows));
+  if (a->variant == 14 ||
+      (a->variant == 0 && a->k < 4096 && weight_bytes > (1ll << 30) && reach > 150.0f && reach <= 192.0f))
+    return launch_tall<K, 6>(p, a->rows, s, n_cu, what, swiglu, half);
+  if (a->variant == 8) return launch_tall<K, 8>(p, a->rows, s, n_cu, what, swiglu, half);
   if (a->variant == 12 || (a->variant == 0 && avg_rows > 96 && a->k >= 4096 && weight_bytes > (1ll << 30))) {
     if (half)
       return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 8, false, true, true>(p, a->rows, s, n_cu, what)

@@ -357,8 +357,9 @@ def main():
                     help="other layer dimensions for the workload's format and routing, e.g. "
                          "H=4096,E=8,K=2,I=14336,I_shared=0 (Mixtral-8x7B); the config then says so")
     ap.add_argument("--tile-variant", type=int, default=0,
-                    help="tuning variant of the int8 tile kernel for the routed GEMMs of prefill-sized batches "
-                         "(kmoe_moe_args.tile_variant; 12: sibling m-tiles paced so that they share weight bytes in L2)")
+                    help="tuning variant of the int8 / fp8 tile kernel for the routed GEMMs of prefill-sized batches "
+                         "(kmoe_moe_args.tile_variant; 12: sibling m-tiles paced so that they share weight bytes in L2, "
+                         "14: one 8-wave tile of 192 rows per workgroup)")
     ap.add_argument("--yardstick", action="store_true",
                     help="also time the vendor library's dense GEMM (torch._int_mm / bf16 matmul) with the gate_up "
                          "GEMM's operation count: [P,H] x [H,2I], one weight matrix, no gather, no epilogue")

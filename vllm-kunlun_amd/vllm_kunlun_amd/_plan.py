@@ -217,7 +217,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     KMOE_FMT_W4A16: w13 [E,2I,H/2] and w2 [E,H,I/2] uint8 (two 4-bit codes per byte), tiled;
     w13_aux/w2_aux their group scales [E,2I,H/group_size], [E,H,I/group_size] in x's dtype.
     shared_scale multiplies the shared expert's output before it is added (the float16 form of the caller's
-    epilogue, models/deepseek_v2.py:286-292). tile_variant: a tuning variant of the int8 tile kernel for the routed GEMMs (kmoe_moe_args.tile_variant).
+    epilogue, models/deepseek_v2.py:286-292). tile_variant: a tuning variant of the int8 / fp8 tile kernel for the routed GEMMs (kmoe_moe_args.tile_variant).
     An expert-parallel share (ops/_kunlun_ops.py:640-696): logits [M,E_global] (correction bias [E_global], router
     weight [E_global,H]) with more experts than the weights hold, and first_expert = ep_rank * E: the routing runs
     over all of them, the pairs routed to [first_expert, first_expert + E) are computed, the others add nothing."""

@@ -355,7 +355,8 @@ def main():
                          "then runs inside each step (reported in config; not the default workload)")
     ap.add_argument("--dims", default="",
                     help="other layer dimensions for the workload's format and routing, e.g. "
-                         "H=4096,E=8,K=2,I=14336,I_shared=0 (Mixtral-8x7B); the config then says so")
+                         "H=4096,E=8,K=2,I=14336,I_shared=0 (Mixtral-8x7B), or a skewed routing, hot_experts=32,hot_bias=1.0 "
+                         "(that bias on the logits of 32 experts); the config then says so")
     ap.add_argument("--tile-variant", type=int, default=0,
                     help="tuning variant of the int8 / fp8 tile kernel for the routed GEMMs of prefill-sized batches "
                          "(kmoe_moe_args.tile_variant; 12: sibling m-tiles paced so that they share weight bytes in L2, "
@@ -384,7 +385,7 @@ def main():
             label = re.sub(r"(decode|prefill), \d+ tokens", f"{a.tokens} tokens (batch set by --tokens)", label)
         if a.dims:
             allowed = {"H": int, "E": int, "K": int, "I": int, "I_shared": int, "n_group": int, "topk_group": int,
-                       "scoring": str, "routed_scale": float}
+                       "scoring": str, "routed_scale": float, "hot_experts": int, "hot_bias": float}
             over = {}
             for item in a.dims.split(","):
                 key, _, val = item.partition("=")

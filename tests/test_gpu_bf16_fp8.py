@@ -142,22 +142,24 @@ FP8_TILED_CASES = FP8_CASES + [
     (2, 256, 640, [140, 3]),                                      # odd number of 128-byte chunks
     (20, 1024, 256, [((53 * i) % 300) for i in range(20)]),       # several tiles per workgroup walk
     (5, 256, 384, [192, 193, 0, 256, 257]),                       # ends of the 8-wave tiles (192 and 256 rows)
+    (6, 256, 384, [140, 150, 135, 160, 145, 138]),                # variant 17: the 192-row tiles are chosen on the device,
+    (8, 256, 256, [300, 10, 290, 20, 310, 15, 150, 100]),         # ... and here the 128-row tiles
 ]
 
 
 @pytest.mark.parametrize("E,n,k,counts", FP8_TILED_CASES)
-@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 8, 11, 13, 14])
+@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 8, 11, 13, 14, 17])
 @pytest.mark.parametrize("act", [0, 1])
 def test_grouped_gemm_fp8_block_tiled_weights(L, E, n, k, counts, variant, act):
     """The same product with the weight bytes re-arranged by kmoe_tile_weights_i8: the LDS-staged
     kernels (1-3) and the persistent tile kernel (5: tile height by the rows per expert; 6: 128; 11: 64; 13: 96 rows;
-    14, 8: 8-wave tiles of 192 and 256 rows)."""
+    14, 8: 8-wave tiles of 192 and 256 rows; 17: 192- or 128-row tiles, decided on the device)."""
     _fp8_case(L, E, n, k, counts, variant, act, tiled=True)
 
 
 @pytest.mark.parametrize("E,n,k,counts", FP8_TILED_CASES)
 @pytest.mark.parametrize("variant,tiled", [(1, False), (2, True), (5, True), (6, True), (11, True), (12, True), (13, True),
-                                           (14, True), (8, True)])
+                                           (14, True), (8, True), (17, True)])
 @pytest.mark.parametrize("act", [0, 1])
 def test_grouped_gemm_fp8_block_half_results(L, E, n, k, counts, variant, tiled, act):
     """act_dtype = KMOE_DT_F16: the LDS-staged kernel and the tile kernel's 64-row, 128-row and paced shapes."""

@@ -85,7 +85,7 @@ def test_half_layer_on_8_wave_tiles_gives_the_same_bits():
     lay = sl.layer
     x = (sl.x.float() * 1.5).half()
     outs = []
-    for variant in (0, 8, 14, 15, 16):
+    for variant in (0, 8, 14, 15, 16, 17):
         out = torch.empty_like(x)
         plan = make_moe_plan(L.KMOE_FMT_INT8, x, sl.logits, out, shape.K, lay.w13_weight, lay.w2_weight,
                              lay.w13_weight_scale, lay.w2_weight_scale, shape.scoring, True, shape.n_group,

@@ -279,7 +279,7 @@ def test_layer_with_paced_tiles_gives_the_same_bits():
     sl = synth.make_w8a8_layer(shape, "cuda", seed=12)
     lay = sl.layer
     outs = []
-    for variant in (0, 12, 12, 8, 14, 15, 16):  # 8, 14-16: one 8-wave tile of 256, 192, 160, 224 rows per workgroup
+    for variant in (0, 12, 12, 8, 14, 15, 16, 17):  # 8, 14-16: one 8-wave tile of 256, 192, 160, 224 rows per workgroup
         out = torch.empty_like(sl.x)
         plan = make_moe_plan(L.KMOE_FMT_INT8, sl.x, sl.logits, out, shape.K, lay.w13_weight, lay.w2_weight,
                              lay.w13_weight_scale, lay.w2_weight_scale, shape.scoring, True, shape.n_group,

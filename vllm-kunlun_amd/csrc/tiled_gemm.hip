@@ -84,6 +84,11 @@ struct TiledParams {
   // BF16 only (the expert-bias branch of the reference, ops/_kunlun_ops.py:433-468):
   const uint16_t* bias;        // NULL, or [E, n] bf16: y = bf16(bf16(gemm) + bias)
   float oai_alpha, oai_limit;  // OAI kernels: out[r, i] = swigluoai(y[r, 2i], y[r, 2i + 1])
+  // One of two launches of the same GEMM on different tiles, of which the routing decides on the device which
+  // one works (the other finds out in its prologue and leaves): the tall tiles of pick_rows rows pay while few
+  // routed experts overflow them (at most one in 16). pick = 1: this launch runs if they do, pick = 2: if not;
+  // 0: it always runs.
+  int32_t pick, pick_rows;
 };
 
 // Progress board of the persistent workgroups: slot b (64 bytes apart) holds where workgroup b is,
@@ -209,7 +214,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   for (int e = threadIdx.x; e <= p.E; e += kThreads) row_lo[e] = p.lod[e];
   __syncthreads();
   if (wave_id == 0) {
-    int carry = 0;
+    int carry = 0, over = 0;
     for (int base = 0; base < n_exp; base += kWave) {
       const int e = base + lane;
       const int mine = e < n_exp ? (rows_end(e) - rows_begin(e) + kTM - 1) / kTM : 0;
@@ -221,11 +226,17 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
       }
       if (e < n_exp) tile_lo[e] = carry + incl - mine;
       carry += __shfl(incl, kWave - 1, kWave);
+      over += __popcll(__ballot(e < p.E && row_lo[e + 1] - row_lo[e] > p.pick_rows));
     }
-    if (lane == 0) tile_lo[n_exp] = carry;
+    if (lane == 0) {
+      tile_lo[n_exp] = carry;
+      tile_lo[n_exp + 1] = over;  // routed experts with more rows than a tall tile holds
+    }
   }
   __syncthreads();
   const int total_tiles = tile_lo[n_exp];
+  const bool tall_pays = tile_lo[n_exp + 1] * 16 <= p.E;
+  const bool not_my_launch = (p.pick == 1 && !tall_pays) || (p.pick == 2 && tall_pays);
 
   // Work items = (m-tile, channel block) pairs, n_items of them, all non-empty, numbered expert
   // by expert; inside an expert the m-tiles of one channel block are consecutive. The list is
@@ -541,7 +552,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     seen_next = chunk > 0 ? b : 0u;
   };
   Tile cur = find_tile(0);
-  if (!cur.valid) {  // the whole workgroup leaves together
+  if (!cur.valid || not_my_launch) {  // the whole workgroup leaves together
     if constexpr (PACE) __hip_atomic_store(my_slot, 0xffffffffu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
   }
@@ -915,7 +926,7 @@ int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* w
   p.max_items = p.n_blocks * max_tiles;
   // persistent workgroups: WGS per CU
   const int grid = min(min(ceil_div(p.max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8), kBoardSlots);
-  const size_t dyn = sizeof(int) * (static_cast<size_t>(p.E) + 1 + n_exp + 1);
+  const size_t dyn = sizeof(int) * (static_cast<size_t>(p.E) + 1 + n_exp + 2);
   hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32, MF, OAI, PACE, F16>), dim3(grid),
                      dim3(WM * kWavesT * kWave), dyn, s, p);
   return check_launch(what);
@@ -965,7 +976,7 @@ int launch_tall(TiledParams& p, int rows, hipStream_t s, int n_cu, const char* w
 // Variant 6 (and 12) forces 128 rows, 11 forces 64, 13 forces 96.
 bool short_tiles(int variant, int rows, int n_experts, int n, bool swiglu, int n_cu, int max_avg_rows = 44) {
   if (variant == 11) return true;
-  if (variant == 6 || variant == 8 || (variant >= 12 && variant <= 16)) return false;
+  if (variant == 6 || variant == 8 || (variant >= 12 && variant <= 17)) return false;
   if (ceil_div(rows, n_experts) <= max_avg_rows) return true;
   const int n_blocks = ceil_div(swiglu ? n / 2 : n, kWavesT * (swiglu ? 2 : 4) * 16);
   return static_cast<long long>(rows / 128 + n_experts) * n_blocks < 2ll * n_cu;
@@ -997,7 +1008,7 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   // cache (Qwen3 shape: 403 and 201 MB) re-reads them from there at little cost, and the waits only cost:
   // +1.5 to +4 % from 2048 to 8192 tokens.
   const long long weight_bytes = static_cast<long long>(a->E + (a->w_tail ? 1 : 0)) * a->n * a->k;
-  const bool paced = a->variant == 12 ||
+  const bool paced = a->variant == 12 || (a->variant == 17 && avg_rows > 96) ||
                      (a->variant == 0 && !shorter && avg_rows > 96 && weight_bytes > (1ll << 30));
   // 96-row tiles between the two: from 45 to 72 rows per expert nearly every expert still fits one tile, and a
   // quarter of the 128-row tile's MFMAs (all padding there) is saved (Qwen3 shape, layer: 768 tokens 0.169 ->
@@ -1017,23 +1028,36 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   // 3.09, at 3584 and 5120 tokens -1 and -2 %, from 6144 tokens on the same. With weights that fit the cache the
   // second pass is cheap and the gain is within noise (Qwen3 shape, 128 rows per expert: 125 against 122 us),
   // while an expert that overflows the tall tile costs a quarter there: not used.
+  // That holds while the routing is even. The host knows the average only, so the choice is left to the device:
+  // the tall launch is followed by the launch this function would have made without it, and each of the two
+  // reads the row counts in its prologue and leaves if the other is due - the tall one runs if at most one routed
+  // expert in 16 overflows its tile (same layer, +0.5 on the logits of 32 experts, i.e. 30 experts past 192 rows:
+  // tall tiles 3.11 ms, paced 128-row tiles 2.95 ms; +1.0: 3.30 against 3.02). The launch that leaves costs a few
+  // microseconds. Variant 17: the same pair whatever the size of the weights.
   int tall = a->variant == 8 ? 8 : (a->variant == 14 ? 6 : (a->variant == 15 ? 5 : (a->variant == 16 ? 7 : 0)));
-  if (a->variant == 0 && !shorter && weight_bytes > (1ll << 30)) {
+  const bool by_rule = (a->variant == 0 && !shorter && weight_bytes > (1ll << 30)) || a->variant == 17;
+  if (by_rule) {
     const float reach = static_cast<float>(avg_rows) + 2.0f * sqrtf(static_cast<float>(avg_rows));
     if (reach > 128.0f && reach <= 256.0f) tall = reach <= 160.0f ? 5 : (reach <= 192.0f ? 6 : (reach <= 224.0f ? 7 : 8));
   }
   if (tall) {
     const bool f16 = a->act_dtype == KMOE_DT_F16;
+    p.pick = by_rule ? 1 : 0;
+    p.pick_rows = 32 * tall;
+    int rc;
     switch (tall) {
-      case 5: return launch_tall<K, 5>(p, a->rows, s, n_cu, what, swiglu, f16);
-      case 6: return launch_tall<K, 6>(p, a->rows, s, n_cu, what, swiglu, f16);
-      case 7: return launch_tall<K, 7>(p, a->rows, s, n_cu, what, swiglu, f16);
-      default: return launch_tall<K, 8>(p, a->rows, s, n_cu, what, swiglu, f16);
+      case 5: rc = launch_tall<K, 5>(p, a->rows, s, n_cu, what, swiglu, f16); break;
+      case 6: rc = launch_tall<K, 6>(p, a->rows, s, n_cu, what, swiglu, f16); break;
+      case 7: rc = launch_tall<K, 7>(p, a->rows, s, n_cu, what, swiglu, f16); break;
+      default: rc = launch_tall<K, 8>(p, a->rows, s, n_cu, what, swiglu, f16); break;
     }
+    if (!by_rule || rc != KMOE_OK) return rc;
+    p.pick = 2;  // the launch below works if the tall one left
   }
   if (a->act_dtype == KMOE_DT_F16) {
     // half outputs: the shapes in use (64-, 96-, 128-row and paced 128-row tiles); the tuning variants are bf16 only
-    KMOE_REQUIRE(a->variant == 0 || a->variant == 5 || a->variant == 6 || (a->variant >= 11 && a->variant <= 13),
+    KMOE_REQUIRE(a->variant == 0 || a->variant == 5 || a->variant == 6 || (a->variant >= 11 && a->variant <= 13) ||
+                     a->variant == 17,
                  KMOE_ERR_UNSUPPORTED, "%s: variant %d is not instantiated for half outputs", what, a->variant);
     if (mid)
       return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 6, false, false, true>(p, a->rows, s, n_cu, what)
@@ -1118,10 +1142,18 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
   // shared expert's 4096 rows as the launch's tail, gate_up loses (4096 tokens: 2.21 -> 2.51 ms, 4608: 2.45 ->
   // 2.63) while down still gains (1.10 -> 1.01 ms, 1.22 -> 1.07, 5120 tokens 1.31 -> 1.16). The 256-row instance
   // spills and is a tuning variant.
+  // As for int8 the device decides between the tall launch and the one that follows it (variant 17: the pair
+  // whatever the size of the weights and K).
   const float reach = static_cast<float>(avg_rows) + 2.0f * sqrtf(static_cast<float>(avg_rows));
-  if (a->variant == 14 ||
-      (a->variant == 0 && a->k < 4096 && weight_bytes > (1ll << 30) && reach > 150.0f && reach <= 192.0f))
-    return launch_tall<K, 6>(p, a->rows, s, n_cu, what, swiglu, half);
+  const bool by_rule = ((a->variant == 0 && a->k < 4096 && weight_bytes > (1ll << 30)) || a->variant == 17) &&
+                       reach > 150.0f && reach <= 192.0f;
+  if (a->variant == 14 || by_rule) {
+    p.pick = by_rule ? 1 : 0;
+    p.pick_rows = 192;
+    const int rc = launch_tall<K, 6>(p, a->rows, s, n_cu, what, swiglu, half);
+    if (!by_rule || rc != KMOE_OK) return rc;
+    p.pick = 2;
+  }
   if (a->variant == 8) return launch_tall<K, 8>(p, a->rows, s, n_cu, what, swiglu, half);
   if (a->variant == 12 || (a->variant == 0 && avg_rows > 96 && a->k >= 4096 && weight_bytes > (1ll << 30))) {
     if (half)

@@ -1017,7 +1017,7 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   const bool mid = a->variant == 13 || (a->variant == 0 && !shorter && avg_rows <= 72);
   // One 8-wave tile per expert (WM = 2: 160, 192, 224 or 256 rows, one workgroup per CU) where experts hold a
   // little more than one 128-row tile and the launch's weights are far more than the memory-side cache holds: the
-  // shortest such tile that nearly every expert fits (average + 2 sqrt(average) rows). The second 128-row tile of
+  // shortest such tile that nearly every expert fits (average + 3 sqrt(average) rows of a routed expert). The second 128-row tile of
   // an expert is mostly padding and streams the expert's weights again; one taller tile does neither, which is
   // worth more than what the lone workgroup loses by having nothing to run under its epilogue (DeepSeek-V3
   // shape, gate_up / down, paced 128-row tiles against the tall tile: 120 rows per expert 1724 against 1598 us,
@@ -1037,8 +1037,13 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   int tall = a->variant == 8 ? 8 : (a->variant == 14 ? 6 : (a->variant == 15 ? 5 : (a->variant == 16 ? 7 : 0)));
   const bool by_rule = (a->variant == 0 && !shorter && weight_bytes > (1ll << 30)) || a->variant == 17;
   if (by_rule) {
-    const float reach = static_cast<float>(avg_rows) + 2.0f * sqrtf(static_cast<float>(avg_rows));
-    if (reach > 128.0f && reach <= 256.0f) tall = reach <= 160.0f ? 5 : (reach <= 192.0f ? 6 : (reach <= 224.0f ? 7 : 8));
+    // (the routed experts' average: a tail expert's many rows say nothing about how full their tiles are - with
+    // it in the average, 96 rows per routed expert took the 160-row tile and lost a fifth, 1526 -> 1841 us)
+    const float avg_routed = static_cast<float>(ceil_div(live, a->E));
+    const float reach = avg_routed + 3.0f * sqrtf(avg_routed);
+    // (from 106 rows per expert: at 104 few experts overflow a 128-row tile yet and the DeepSeek-V3 layer loses
+    // 4 % on the tall tile, at 107 the Kimi-K2 dimensions gain 4 %, at 112 the DeepSeek-V3 layer 1 %)
+    if (avg_routed >= 106.0f && reach <= 256.0f) tall = reach <= 160.0f ? 5 : (reach <= 192.0f ? 6 : (reach <= 224.0f ? 7 : 8));
   }
   if (tall) {
     const bool f16 = a->act_dtype == KMOE_DT_F16;
@@ -1144,9 +1149,9 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
   // spills and is a tuning variant.
   // As for int8 the device decides between the tall launch and the one that follows it (variant 17: the pair
   // whatever the size of the weights and K).
-  const float reach = static_cast<float>(avg_rows) + 2.0f * sqrtf(static_cast<float>(avg_rows));
+  const int avg_routed = ceil_div(live, a->E);
   const bool by_rule = ((a->variant == 0 && a->k < 4096 && weight_bytes > (1ll << 30)) || a->variant == 17) &&
-                       reach > 150.0f && reach <= 192.0f;
+                       avg_routed >= 124 && avg_routed <= 168;
   if (a->variant == 14 || by_rule) {
     p.pick = by_rule ? 1 : 0;
     p.pick_rows = 192;

@@ -162,3 +162,54 @@ def test_two_threads_share_the_side_stream():
         t.join()
     torch.cuda.synchronize()
     assert not errors, errors
+
+
+def test_tile_height_chosen_on_the_device_under_graph_replay():
+    """Variant 17 of the int8 GEMM enqueues a tall-tile launch and a 128-row-tile launch; the row counts decide in
+    each launch's prologue which of the two works. Captured once, the pair is replayed with row counts that suit
+    the tall tile and with counts that overflow it: every replay gives the bits of the 128-row-tile kernel."""
+    from vllm_kunlun_amd import _lib as L
+    E, n, k, rows = 20, 256, 384, 3000
+    g = torch.Generator(device="cuda").manual_seed(3)
+    a = torch.randint(-127, 128, (rows, k), generator=g, dtype=torch.int8, device="cuda")
+    a_max = torch.rand(rows, generator=g, device="cuda") + 0.1
+    w = torch.randint(-127, 128, (E, n, k), generator=g, dtype=torch.int8, device="cuda")
+    w_max = torch.rand(E, n, generator=g, device="cuda") + 0.1
+    wt = torch.empty_like(w)
+    L.check(L.lib.kmoe_tile_weights_i8(w.data_ptr(), wt.data_ptr(), E, n, k, L.stream()))
+
+    def lod_of(counts):
+        assert sum(counts) == rows
+        return torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32, device="cuda")
+
+    even = [150] * E                                              # every expert fits a 192-row tile
+    skew = [400, 20, 390, 10, 380, 30, 370, 40] + [113] * 11 + [117]  # a fifth of them overflows it
+    lods = [lod_of(even), lod_of(skew), lod_of(even[::-1]), lod_of(skew[::-1])]
+    lod = lods[0].clone()
+    y = torch.zeros(rows, n, dtype=torch.bfloat16, device="cuda")
+    args = L.GemmI8Args()
+    args.a, args.lda, args.a_max, args.src_div = a.data_ptr(), k, a_max.data_ptr(), 1
+    args.w, args.w_max, args.lod = wt.data_ptr(), w_max.data_ptr(), lod.data_ptr()
+    args.E, args.n, args.k, args.rows = E, n, k, rows
+    args.y, args.ldy, args.act, args.w_layout = y.data_ptr(), n, 0, L.KMOE_W_TILED
+
+    def run(variant):
+        args.variant = variant
+        L.check(L.lib.kmoe_grouped_gemm_i8(args, L.stream()))
+
+    run(17)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(17)
+    for fresh in lods:
+        lod.copy_(fresh)
+        y.fill_(7.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = y.clone()
+        _eager_noise()
+        y.fill_(7.0)
+        run(6)
+        torch.cuda.synchronize()
+        assert torch.equal(got, y)

@@ -188,7 +188,8 @@ def vendor_dense_gemm(shape, g1_ops, peak_tops, reps=20):
 
 # What plain `python bench.py` runs besides the headline workload: the other benchmark
 # configurations, reported under "workloads" in the same JSON line.
-SUITE = ["dsv3-prefill", "qwen3-decode", "qwen3-prefill", "qwen3-prefill-skew", "dsv3-fp8-decode", "dsv3-fp8-prefill"]
+SUITE = ["dsv3-prefill", "qwen3-decode", "qwen3-prefill", "qwen3-prefill-skew", "dsv3-fp8-decode", "dsv3-fp8-prefill",
+         "kimi-decode", "kimi-prefill", "kimi-fp8-decode", "kimi-fp8-prefill"]
 HEADLINE = "dsv3-decode"
 
 
@@ -221,7 +222,8 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
                              getattr(lay, "w13_weight_scale", None), getattr(lay, "w2_weight_scale", None),
                              shape.scoring, True, shape.n_group, shape.topk_group, shape.routed_scale, sl.bias,
                              sl.shared, 1.0, stage_events, router_weight=w_gate,
-                             group_size=shape.group_size if w4 else None, tile_variant=a.tile_variant)
+                             group_size=shape.group_size if w4 else None, tile_variant=a.tile_variant,
+                             side_stream=not a.one_stream)
 
     # The layer, its inputs and the workspace were produced on the default stream;
     # finish that work before a second stream touches (recycled) memory.
@@ -235,6 +237,11 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
             torch.bitwise_not(src, out=torch.empty_like(src))
         for _ in range(3):
             plan()
+        # which GEMM kernels the launchers chose for this call, as the library itself reports them
+        L.lib.kmoe_trace_kernels(1)
+        plan()
+        L.lib.kmoe_trace_kernels(0)
+        traced = L.lib.kmoe_traced_kernels().decode().splitlines()
         stream.synchronize()
 
         def timed(step):
@@ -286,6 +293,9 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
     peak_tops = PEAK_TOPS[shape.quant]
     hbm_bound = intensity < peak_tops * 1e12 / (HBM_PEAK_GBS * 1e9)
     g1_s = stage_ms["gemm1"] * 1e-3
+    # the launch(es) noted under the first "[gate_up, ...]" heading (two when the device decides between tile shapes)
+    heads = [i for i, line in enumerate(traced) if line.startswith("[")]
+    g1_kernel = " | ".join(traced[heads[0] + 1: heads[1]]) if len(heads) > 1 else "?"
     traffic = None if (a.tokens or a.dims) else measured_traffic(workload)  # the counter summaries are of the named workload
     if hbm_bound:
         achieved = work["g1_bytes"] / g1_s / 1e9
@@ -293,11 +303,9 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic}
     else:
         achieved = work["g1_ops"] / g1_s / 1e12
-        roofline = {"bound": "mfma", "achieved": achieved, "peak": peak_tops, "unit": "TFLOP/s",
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": peak_tops,
+                    "unit": "TOP/s" if shape.quant == "int8" else "TFLOP/s",
                     "frac": achieved / peak_tops, "traffic": traffic}
-    many_rows = shape.P > 10 * shape.E  # the launchers' switch to the persistent tile kernel
-    g1_kernel = (("w4_tile_kernel" if shape.P > (20 if shape.H > 4096 else 13) * shape.E else "w4_stream_kernel") if w4 else "stream_gemm_i8_kernel" if plan.layout.codes_chunked else
-                 "tiled_gemm_kernel" if many_rows and plan.args.w_layout == L.KMOE_W_TILED else "grouped_gemm_kernel")
     roofline.update(kernel=g1_kernel + " (gate_up + SiLU-mul)", kernel_ms=stage_ms["gemm1"],
                     algorithmic_bytes=work["g1_bytes"], algorithmic_ops=work["g1_ops"],
                     hbm_frac=work["g1_bytes"] / g1_s / 1e9 / HBM_PEAK_GBS,
@@ -312,7 +320,7 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
                    "experts": shape.E, "top_k": shape.K, "moe_intermediate": shape.I,
                    "shared_intermediate": shape.I_shared, "routing": shape.scoring, "experts_hit": n_active,
                    "launch": launch_mode, "launch_ms_per_step": launch_ms, "seed": a.seed,
-                   "router_gemm_inside": bool(a.router), "tile_variant": a.tile_variant,
+                   "side_stream": not a.one_stream, "router_gemm_inside": bool(a.router), "tile_variant": a.tile_variant, "gemm_kernels": traced,
                    "activations": "float16" if a.act_dtype == "f16" else "bfloat16"},
         "roofline": roofline,
         "layer": {"hbm_gbs": work["layer_bytes"] / t_s / 1e9, "hbm_frac": work["layer_bytes"] / t_s / 1e9 / HBM_PEAK_GBS,
@@ -361,6 +369,10 @@ def main():
                     help="tuning variant of the int8 / fp8 tile kernel for the routed GEMMs of prefill-sized batches "
                          "(kmoe_moe_args.tile_variant; 12: sibling m-tiles paced so that they share weight bytes in L2, "
                          "14: one 8-wave tile of 192 rows per workgroup)")
+    ap.add_argument("--one-stream", action="store_true",
+                    help="keep every launch on the one stream (the C ABI's default). Without it the layer is called with "
+                         "KMOE_FLAG_SIDE_STREAM: a shared expert that cannot ride in the routed launches (the fp8 layers at "
+                         "decode sizes) runs on the library's second stream beside them; config.side_stream says which")
     ap.add_argument("--yardstick", action="store_true",
                     help="also time the vendor library's dense GEMM (torch._int_mm / bf16 matmul) with the gate_up "
                          "GEMM's operation count: [P,H] x [H,2I], one weight matrix, no gather, no epilogue")

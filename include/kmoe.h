@@ -7,8 +7,20 @@
  *   - never allocates or frees device memory, never synchronises the stream
  *     (scratch comes in through `workspace` arguments sized by the
  *     *_workspace_bytes functions), so calls can be captured into a HIP graph;
+ *   - enqueues on the given stream ONLY. The one exception is asked for per call:
+ *     kmoe_moe_forward with KMOE_FLAG_SIDE_STREAM in kmoe_moe_args.flags may run
+ *     the shared expert on a second stream of the library's (see the flag);
  *   - kmoe_last_error() gives the text of the calling thread's last failure.
  * A `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *
+ * State the library keeps per process and GPU, besides its code: (1) a pacing
+ * board of 128 KiB inside the device image (the persistent tile GEMM's workgroups
+ * post their progress there so that tiles reading the same weight bytes stay in
+ * step; every wait on it is bounded and no result depends on it, so launches that
+ * overlap on one GPU - two streams, two layers - share it safely and at worst pace
+ * each other badly); (2) the 64 MiB buffer of kmoe_moe_forward_static; (3) with
+ * KMOE_FLAG_SIDE_STREAM, one stream and two events, created by the first call
+ * that asks for them outside a capture.
  *
  * Each function cites the reference interface (baidu/vLLM-Kunlun, paths under
  * vllm_kunlun/) whose closed-source kernel it stands in for.
@@ -52,6 +64,14 @@ typedef void* kmoe_stream_t;
 const char* kmoe_last_error(void);
 /* Library version string, e.g. "kmoe 0.1 gfx950". */
 const char* kmoe_version(void);
+/* Diagnostics, no counterpart in the reference. kmoe_trace_kernels(1) clears the calling thread's record and starts
+ * noting the GEMM kernel of every GEMM launch made on this thread (by the GEMM entry points and inside
+ * kmoe_moe_forward), as the launcher chose it: name and template arguments, one per line in launch order, e.g.
+ * "tiled_gemm_kernel<int8, SiLU-mul, 128x256 tile, 4 waves, 2 per CU>". kmoe_trace_kernels(0) stops noting and
+ * keeps the record. kmoe_traced_kernels() returns the record (at most 4 KiB, valid until this thread's next
+ * kmoe_trace_kernels(1)). Costs one thread-local test per launch while off. */
+void kmoe_trace_kernels(int on);
+const char* kmoe_traced_kernels(void);
 
 /* ------------------------------------------------------------------ routing */
 
@@ -584,7 +604,19 @@ typedef struct kmoe_moe_args {
      runs over E_global experts (logits [M,E_global], bias [E_global], w_gate [E_global,H]; K <= E_global); the
      weights are those of the E experts [first_expert, first_expert + E). 0 / 0: one GPU holds every expert. */
   int32_t E_global, first_expert;
+  int32_t flags;         /* KMOE_FLAG_* or'ed together; 0: none                                            */
 } kmoe_moe_args;
+
+/* kmoe_moe_args.flags.
+ * KMOE_FLAG_SIDE_STREAM: a shared expert that cannot ride in the routed launches (a width other than the routed
+ * experts'; the fp8 layer at decode sizes) may run on a second stream of the library's own (one per GPU, default
+ * priority, non-blocking, created by the first such call that is not being captured), forked from `stream` by an
+ * event after the first quantisation and joined back by an event before the combine: the caller still sees one
+ * stream's worth of ordering, and under capture the fork and join become graph edges. Without the flag (the default)
+ * everything is enqueued on `stream`. The environment variable KMOE_SIDE_STREAM overrides the flag for the whole
+ * process (0: never, 1: as if every call set it); it is read once. Ignored with stage_events and by
+ * kmoe_moe_forward_static. */
+#define KMOE_FLAG_SIDE_STREAM 1
 
 #define KMOE_STAGE_ROUTING 0
 #define KMOE_STAGE_ALIGN 1
@@ -640,6 +672,10 @@ int kmoe_moe_forward(const kmoe_moe_args* args, void* workspace,
  * Allocates nothing, same results as kmoe_moe_forward bit for bit. Call it with the stream's
  * device current. All calls on one GPU share the one buffer: calls that may overlap on a GPU
  * (two streams, two threads) race; the buffer keeps the last call's intermediates.
+ * The buffer's device address is looked up once per GPU, by the first kmoe_moe_forward or
+ * kmoe_moe_forward_static call on that GPU whose stream is not being captured (the lookup is
+ * not a stream operation). A captured call that would be the first is refused with
+ * KMOE_ERR_UNSUPPORTED: make one call on the GPU outside the capture before.
  */
 #define KMOE_STATIC_WORKSPACE_BYTES (64u << 20)
 int kmoe_moe_forward_static(const kmoe_moe_args* args, kmoe_stream_t stream);

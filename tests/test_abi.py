@@ -43,7 +43,7 @@ def test_struct_layouts_match_the_header(L, tmp_path):
                "kmoe_gemm_fp8_args": (L.GemmFp8Args, ["w_scale", "y", "w_tail", "tail_src0"]),
                "kmoe_gemm_w4_args": (L.GemmW4Args, ["w_scale", "lod", "y", "w_layout"]),
                "kmoe_moe_args": (L.MoEArgs, ["logits", "I_shared", "out", "w_gate", "ws_layout", "group_size",
-                                             "act_dtype", "shared_scale", "tile_variant"]),
+                                             "act_dtype", "shared_scale", "tile_variant", "first_expert", "flags"]),
                "kmoe_moe_layout": (L.MoELayout, ["align_ws", "down", "sh_out", "n_logit_planes"])}
     lines = ["#include <stdio.h>", "#include <stddef.h>", '#include "kmoe.h"', "int main(void) {"]
     for name, (_, fields) in structs.items():
@@ -186,3 +186,11 @@ def test_static_workspace_forward_refuses_what_does_not_fit(L):
     a.format = L.KMOE_FMT_INT8
     assert L.lib.kmoe_moe_forward_static(C.byref(a), None) == -4
     assert b"built-in buffer" in L.lib.kmoe_last_error()
+
+
+def test_kernel_trace_record_is_per_thread_and_empty_without_launches(L):
+    lib = L.lib
+    lib.kmoe_trace_kernels(1)
+    assert lib.kmoe_traced_kernels() == b""
+    lib.kmoe_trace_kernels(0)
+    assert lib.kmoe_traced_kernels() == b""

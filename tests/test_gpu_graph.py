@@ -46,17 +46,20 @@ def test_apply_monolithic_under_graph_capture():
     _replays(graph, (x, logits), fresh, out, eager)
 
 
+@pytest.mark.parametrize("side", [False, True], ids=["one-stream", "side-stream"])
 @pytest.mark.parametrize("quant", ["int8", "fp8"])
-def test_shared_expert_on_the_side_stream_under_graph_capture(quant):
-    """A shared expert of another width (int8) and the fp8 decode layer run their shared MLP on the library's second
-    stream, forked from and joined into the caller's: eager and captured (the fork and join become graph edges),
-    same bits every time (int8: the oracle's)."""
+def test_shared_expert_on_the_side_stream_under_graph_capture(quant, side):
+    """A shared expert of another width (int8) and the fp8 decode layer run their shared MLP in launches of its own:
+    on the caller's stream by default, and with KMOE_FLAG_SIDE_STREAM (the method's side_stream) on the library's
+    second stream, forked from and joined into the caller's. Both settings, eager and captured (the fork and join
+    become graph edges): same bits every time (int8: the oracle's)."""
     from vllm_kunlun_amd import synth
     base = "dsv3-decode" if quant == "int8" else "dsv3-fp8-decode"
     shape = synth.scaled(synth.SHAPES[base], M=40, H=512, E=32, K=4, I=128, n_group=4, topk_group=2,
                          I_shared=384 if quant == "int8" else 128)
     sl = synth.make_layer(shape, "cuda", seed=7)
     method, kw = sl.layer.quant_method, sl.apply_kwargs()
+    method.side_stream = side
     x, logits = sl.x.clone(), sl.logits.clone()
     eager = lambda xx, ll: method.apply_monolithic(sl.layer, xx, ll, **kw)  # noqa: E731
     first = eager(x, logits)                           # creates the second stream (never inside a capture)
@@ -91,7 +94,9 @@ def test_static_workspace_forward_under_graph_capture():
     plan = make_moe_plan(L.KMOE_FMT_INT8, x, logits, out, shape.K, lay.w13_weight, lay.w2_weight, lay.w13_weight_scale,
                          lay.w2_weight_scale, "softmax", True)
     call = lambda: L.check(L.lib.kmoe_moe_forward_static(C.byref(plan.args), L.stream()))  # noqa: E731
-    call()                                             # the first call on a GPU resolves the buffer's address
+    # one call on the GPU outside a capture (here of the workspace entry point) has to come first: it looks up the
+    # built-in buffer's device address, which a captured call may not do
+    plan()
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
@@ -131,6 +136,8 @@ def test_two_threads_share_the_side_stream():
     shapes = [synth.scaled(synth.SHAPES["dsv3-decode"], M=24 + 8 * i, H=512, E=32, K=4, I=128, n_group=4, topk_group=2,
                            I_shared=256 + 128 * i) for i in range(2)]
     layers = [synth.make_layer(sh, "cuda", seed=20 + i) for i, sh in enumerate(shapes)]
+    for sl in layers:
+        sl.layer.quant_method.side_stream = True
     want = []
     for sl in layers:
         want.append(sl.layer.quant_method.apply_monolithic(sl.layer, sl.x, sl.logits, **sl.apply_kwargs()).clone())

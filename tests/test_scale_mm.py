@@ -63,6 +63,23 @@ def test_process_weights_after_loading_on_the_host():
     KunlunScaledMMLinearKernel(Int8ScaledMMLinearLayerConfig(is_static_input_scheme=True, input_symmetric=False)
                                ).process_weights_after_loading(layer4)
     assert torch.equal(layer4.azp_adj.data, -7 * wq4.int().sum(1).reshape(1, 32)) and layer4.input_scale is not None
+    # a fused layer's per-partition static input scales collapse to one: the largest (symmetric) ...
+    layer5, _, _ = _layer(32, 64, "cpu", 5)
+    layer5.input_scale = torch.nn.Parameter(torch.tensor([0.02, 0.05, 0.03]), requires_grad=False)
+    KunlunScaledMMLinearKernel(Int8ScaledMMLinearLayerConfig(is_static_input_scheme=True)).process_weights_after_loading(layer5)
+    assert torch.equal(layer5.input_scale.data, torch.tensor([0.05]))
+    # ... or the scale and zero point of the range that all partitions cover (asymmetric): partitions
+    # [-1.0, 1.55] (scale 0.01, zp -28) and [-0.64, 4.46] (scale 0.02, zp -96) -> [-1.0, 4.46] in 255 steps
+    layer6, wq6, _ = _layer(32, 64, "cpu", 6)
+    layer6.input_scale = torch.nn.Parameter(torch.tensor([0.01, 0.02]), requires_grad=False)
+    layer6.input_zero_point = torch.nn.Parameter(torch.tensor([-28, -96], dtype=torch.int32), requires_grad=False)
+    KunlunScaledMMLinearKernel(Int8ScaledMMLinearLayerConfig(is_static_input_scheme=True, input_symmetric=False)
+                               ).process_weights_after_loading(layer6)
+    want_scale = (0.02 * (127 + 96) - 0.01 * (-128 + 28)) / 255.0
+    assert abs(float(layer6.input_scale.data) - want_scale) < 1e-7 and layer6.input_scale.numel() == 1
+    want_zp = round(-128 - (0.01 * (-128 + 28)) / want_scale)
+    assert int(layer6.input_zero_point.data) == want_zp and layer6.input_zero_point.numel() == 1
+    assert torch.equal(layer6.azp_adj.data, want_zp * wq6.int().sum(1).reshape(1, 32))
     with pytest.raises(ValueError):
         bad, _, _ = _layer(16, 64, "cpu", 2)
         bad.weight_scale = torch.nn.Parameter(torch.ones(5), requires_grad=False)

@@ -4,6 +4,7 @@ kmoe_moe_forward on the same arguments: bit-identical outputs, on two calls in a
 second on a smaller batch (the buffer then still holds the first call's intermediates), and
 also against the C oracle. Called through the C ABI (ctypes), not through the plugin."""
 import ctypes as C
+import gc
 
 import numpy as np
 import pytest
@@ -23,8 +24,17 @@ def _plan_for(sl, out):
                          s.topk_group, s.routed_scale, sl.bias, sl.shared, 1.0)
 
 
+def _device_free_bytes():
+    """Free device memory as the driver sees it (hipMemGetInfo): it drops for ANY allocation on the
+    GPU, also one made inside libkmoe.so, which torch's allocator statistics cannot see."""
+    return torch.cuda.mem_get_info()[0]
+
+
 def _both_ways(sl):
-    """(output of kmoe_moe_forward, output of kmoe_moe_forward_static) for one synthetic layer."""
+    """(output of kmoe_moe_forward, output of kmoe_moe_forward_static) for one synthetic layer.
+    Around the static call nothing may be allocated: the driver's free-byte count must not drop
+    and torch's allocator must not have been asked for a block. Python's cyclic collector is
+    switched off for the window (garbage of earlier tests freed inside it would move the figures)."""
     from vllm_kunlun_amd import _lib as L
     want = torch.empty_like(sl.x)
     plan = _plan_for(sl, want)
@@ -32,10 +42,28 @@ def _both_ways(sl):
     plan()
     got = torch.full_like(sl.x, float("nan"))
     plan.args.out = got.data_ptr()
-    before = torch.cuda.memory_allocated()
-    L.check(L.lib.kmoe_moe_forward_static(C.byref(plan.args), L.stream()))
-    assert torch.cuda.memory_allocated() == before
+    stream = L.stream()
+    # warm-up: the first call on a GPU resolves the buffer's device address (not part of the claim)
+    L.check(L.lib.kmoe_moe_forward_static(C.byref(plan.args), stream))
     torch.cuda.synchronize()
+    got.fill_(float("nan"))
+    torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()
+    try:
+        free_before = _device_free_bytes()
+        blocks_before = torch.cuda.memory_stats()["allocation.all.allocated"]
+        segments_before = torch.cuda.memory_stats()["segment.all.allocated"]
+        rc = L.lib.kmoe_moe_forward_static(C.byref(plan.args), stream)
+        torch.cuda.synchronize()
+        free_after = _device_free_bytes()
+        blocks_after = torch.cuda.memory_stats()["allocation.all.allocated"]
+        segments_after = torch.cuda.memory_stats()["segment.all.allocated"]
+    finally:
+        gc.enable()
+    L.check(rc)
+    assert free_after >= free_before, f"device memory shrank by {free_before - free_after} B across the static call"
+    assert blocks_after == blocks_before and segments_after == segments_before, "torch allocated during the static call"
     return want, got
 
 

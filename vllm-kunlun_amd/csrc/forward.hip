@@ -2,6 +2,7 @@
 // stage kernels together on one stream out of one caller-owned workspace.
 #include <cstdarg>
 #include <cstdio>
+#include <cstring>
 #include <mutex>
 
 #include "kmoe_common.h"
@@ -18,6 +19,25 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+// ---- record of the GEMM kernels a thread launches (kmoe_trace_kernels) ----
+static thread_local bool g_trace_on = false;
+static thread_local char g_trace[4096] = "";
+static thread_local size_t g_trace_len = 0;
+
+bool tracing_kernels() { return g_trace_on; }
+void note_kernel(const char* fmt, ...) {
+  if (!g_trace_on || g_trace_len + 2 >= sizeof(g_trace)) return;
+  va_list ap;
+  va_start(ap, fmt);
+  const int n = vsnprintf(g_trace + g_trace_len, sizeof(g_trace) - g_trace_len - 1, fmt, ap);
+  va_end(ap);
+  if (n < 0) return;
+  g_trace_len = g_trace_len + static_cast<size_t>(n) < sizeof(g_trace) - 2 ? g_trace_len + static_cast<size_t>(n)
+                                                                           : sizeof(g_trace) - 2;
+  g_trace[g_trace_len++] = '\n';
+  g_trace[g_trace_len] = '\0';
+}
+
 int check_launch(const char* what) {
   const hipError_t err = hipGetLastError();
   if (err == hipSuccess) return KMOE_OK;
@@ -29,7 +49,15 @@ int check_launch(const char* what) {
 using namespace kmoe;
 
 extern "C" const char* kmoe_last_error(void) { return g_error; }
-extern "C" const char* kmoe_version(void) { return "kmoe 0.2 gfx950"; }
+extern "C" const char* kmoe_version(void) { return "kmoe 0.3 gfx950"; }
+extern "C" void kmoe_trace_kernels(int on) {
+  if (on) {
+    g_trace[0] = '\0';
+    g_trace_len = 0;
+  }
+  g_trace_on = on != 0;
+}
+extern "C" const char* kmoe_traced_kernels(void) { return g_trace; }
 
 namespace {
 
@@ -272,7 +300,9 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
 template <class Mark>
 int run_mlp(const MlpPass& m, kmoe_stream_t stream, Mark&& mark) {
   int rc;
+  const char* whose = m.row_src ? "routed experts" : "shared expert";
   mark(KMOE_STAGE_GEMM1, 0);
+  if (tracing_kernels()) note_kernel("[gate_up, %s]", whose);
   rc = run_gemm(m, true, stream);
   if (rc) return rc;
   mark(KMOE_STAGE_GEMM1, 1);
@@ -290,6 +320,7 @@ int run_mlp(const MlpPass& m, kmoe_stream_t stream, Mark&& mark) {
   if (rc) return rc;
   mark(KMOE_STAGE_QUANT2, 1);
   mark(KMOE_STAGE_GEMM2, 0);
+  if (tracing_kernels()) note_kernel("[down, %s]", whose);
   rc = run_gemm(m, false, stream);
   if (rc) return rc;
   mark(KMOE_STAGE_GEMM2, 1);
@@ -346,7 +377,8 @@ namespace {
 // small launches that depends on the layer's input only. It runs on a stream of the library's own, forked from
 // the caller's stream after the first quantisation and joined back before the combine, so that it hides under
 // the routed GEMMs instead of adding its launches' latencies to the layer (DeepSeek-V3 fp8 decode: 85 us of
-// 1.86 ms). One stream and two events per GPU, created on the first call that wants them and is not being
+// 1.86 ms). Only for calls that ask for it (KMOE_FLAG_SIDE_STREAM): by default every launch goes to the caller's
+// stream. One stream and two events per GPU, created on the first call that wants them and is not being
 // captured (default priority, non-blocking); work of consecutive calls is ordered on it like on any stream.
 struct SideStream {
   hipStream_t stream = nullptr;
@@ -357,14 +389,19 @@ constexpr int kSideDevices = 64;
 SideStream g_side[kSideDevices];
 std::mutex g_side_mutex;
 
-// The side stream of the current device, or NULL: switched off by KMOE_SERIAL_SHARED=1, not created yet while the
-// caller's stream is being captured (a capture must not be the first to ask), or the runtime refused.
-SideStream* side_stream(hipStream_t main) {
-  static const bool off = [] {
-    const char* v = getenv("KMOE_SERIAL_SHARED");
-    return v && v[0] && v[0] != '0';
+// Whether this call may use the side stream: KMOE_FLAG_SIDE_STREAM of the call, unless the environment variable
+// KMOE_SIDE_STREAM (read once) says 0 (never) or 1 (always).
+bool wants_side_stream(const kmoe_moe_args* a) {
+  static const int forced = [] {
+    const char* v = getenv("KMOE_SIDE_STREAM");
+    return (v && v[0]) ? (v[0] != '0' ? 1 : 0) : -1;
   }();
-  if (off) return nullptr;
+  return forced >= 0 ? forced == 1 : (a->flags & KMOE_FLAG_SIDE_STREAM) != 0;
+}
+
+// The side stream of the current device, or NULL: not created yet while the caller's stream is being captured (a
+// capture must not be the first to ask), or the runtime refused.
+SideStream* side_stream(hipStream_t main) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSideDevices) return nullptr;
   std::lock_guard<std::mutex> lock(g_side_mutex);
@@ -389,11 +426,13 @@ SideStream* side_stream(hipStream_t main) {
 
 int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_bytes, kmoe_stream_t stream,
                      bool may_fork);
+void learn_static_workspace(hipStream_t stream);
 
 }  // namespace
 
 extern "C" int kmoe_moe_forward(const kmoe_moe_args* a, void* workspace, size_t workspace_bytes,
                                 kmoe_stream_t stream) {
+  learn_static_workspace(as_stream(stream));  // (so that a later captured kmoe_moe_forward_static finds the address)
   return moe_forward_impl(a, workspace, workspace_bytes, stream, true);
 }
 
@@ -568,7 +607,8 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
   // stream it is enqueued there BEFORE the routed pass (it reads x / its codes only) and joined after it.
   const uint16_t* shared_out = fold ? routed.out + static_cast<size_t>(P) * H : nullptr;
   const bool own_pass = a->I_shared > 0 && !fold;
-  SideStream* side = own_pass && may_fork && !a->stage_events ? side_stream(as_stream(stream)) : nullptr;
+  SideStream* side =
+      own_pass && may_fork && !a->stage_events && wants_side_stream(a) ? side_stream(as_stream(stream)) : nullptr;
   auto shared_pass = [&](kmoe_stream_t st) -> int {
     int32_t* dense_lod = static_cast<int32_t*>(at(L.sh_lod));
     int rcs = fill_dense_lod(dense_lod, stream_mode ? 0 : M, as_stream(st));  // (streaming path: see below)
@@ -668,8 +708,10 @@ constexpr int kMaxDevices = 64;
 void* g_scratch_ptr[kMaxDevices] = {};
 std::mutex g_scratch_mutex;
 
-// Device address of `scratch` on the current GPU (asked for on the first call per GPU).
-int static_workspace(void** out) {
+// Device address of `scratch` on the current GPU. It is looked up once per GPU, by the first call whose stream is
+// not being captured (the lookup is not a stream operation and may be what makes the runtime load the array); a
+// captured call that finds it missing is refused.
+int static_workspace(void** out, hipStream_t stream) {
   int dev = -1;
   hipError_t err = hipGetDevice(&dev);
   if (err != hipSuccess) return fail(KMOE_ERR_LAUNCH, "moe_forward_static: hipGetDevice: %s", hipGetErrorString(err));
@@ -677,6 +719,12 @@ int static_workspace(void** out) {
                kMaxDevices);
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (!g_scratch_ptr[dev]) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();
+    KMOE_REQUIRE(cap == hipStreamCaptureStatusNone, KMOE_ERR_UNSUPPORTED,
+                 "moe_forward_static: the built-in buffer's address on device %d is not known yet and this stream is "
+                 "being captured: call kmoe_moe_forward or kmoe_moe_forward_static once outside the capture first",
+                 dev);
     void* p = nullptr;
     err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (err != hipSuccess || !p)
@@ -686,6 +734,23 @@ int static_workspace(void** out) {
   }
   *out = g_scratch_ptr[dev];
   return KMOE_OK;
+}
+
+// Looks the address up on behalf of later captured calls; failures (a capture in progress, a runtime error) are
+// left for kmoe_moe_forward_static to report.
+void learn_static_workspace(hipStream_t stream) {
+  static thread_local int known_dev = -1;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return;
+  }
+  if (dev == known_dev) return;
+  void* p = nullptr;
+  char saved[sizeof(g_error)];
+  memcpy(saved, g_error, sizeof(saved));
+  if (static_workspace(&p, stream) == KMOE_OK) known_dev = dev;
+  else memcpy(g_error, saved, sizeof(saved));  // not this call's failure
 }
 
 }  // namespace
@@ -698,7 +763,7 @@ extern "C" int kmoe_moe_forward_static(const kmoe_moe_args* a, kmoe_stream_t str
                "(use kmoe_moe_forward with a workspace of the caller's)",
                L.total_bytes, static_cast<size_t>(KMOE_STATIC_WORKSPACE_BYTES));
   void* ws = nullptr;
-  if (int rc = static_workspace(&ws)) return rc;
+  if (int rc = static_workspace(&ws, as_stream(stream))) return rc;
   // every slot of the layout is written by the stage that owns it before anything reads it, so
   // the last call's contents need no clearing
   return moe_forward_impl(a, ws, KMOE_STATIC_WORKSPACE_BYTES, stream, false);  // no second stream: nothing is created here

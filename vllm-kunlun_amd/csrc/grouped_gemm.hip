@@ -31,6 +31,9 @@ constexpr int kKC = 256;          // bytes of K per chunk and row
 constexpr int kPitch = kKC + 16;  // LDS row pitch: 16 rows of a b128 read fall in 16 different bank groups
 
 enum class Kind { I8, BF16, FP8, F16 };  // F16: the unquantized path on IEEE half operands and results
+constexpr const char* kind_name(Kind k) {
+  return k == Kind::I8 ? "int8" : (k == Kind::BF16 ? "bf16" : (k == Kind::FP8 ? "fp8" : "f16"));
+}
 
 template <Kind K> struct Traits;
 template <> struct Traits<Kind::I8> {
@@ -402,6 +405,9 @@ int launch(const GemmParams& p, int rows, hipStream_t s, const char* what) {
   const int n_exp = p.E + (p.w_tail ? 1 : 0);
   const int grid_y = LOCATE ? (rows + p.tail_rows) / TM + min(n_exp, rows + p.tail_rows) : n_exp;
   if (grid_y == 0) return KMOE_OK;
+  if (tracing_kernels())
+    note_kernel("grouped_gemm_kernel<%s, %d-row tiles, %d channel fragments per wave, %d waves, %s>", kind_name(KIND), TM, NF,
+                WAVES, SWIGLU ? "SiLU-mul" : "plain");
   hipLaunchKernelGGL((grouped_gemm_kernel<KIND, MF, NF, WAVES, SWIGLU, LOCATE>), dim3(grid_x, grid_y),
                      dim3(WAVES * kWave), 0, s, p);
   return check_launch(what);

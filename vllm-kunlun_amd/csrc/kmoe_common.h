@@ -17,6 +17,9 @@ constexpr int kWave = 64;
 // ---- error plumbing (host) -------------------------------------------------
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
+// The calling thread's record of launched GEMM kernels (kmoe_trace_kernels): a launcher notes the kernel it chose.
+bool tracing_kernels();
+void note_kernel(const char* fmt, ...);
 // Writes {0, rows} to lod2: the row offsets of a dense (single-expert) GEMM.
 int fill_dense_lod(int32_t* lod2, int rows, hipStream_t stream);
 // Weight-streaming int8 GEMM (tiled weights, chunk-major activations); arguments already validated.

@@ -237,6 +237,9 @@ int launch_stream(const StreamParams& p, hipStream_t s) {
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const dim3 grid(ceil_div(n_half, (kWaves / KS) * NFH * 16), p.E + (p.w_tail ? ceil_div(p.tail_rows, 16 * MF) : 0));
+  if (tracing_kernels())
+    note_kernel("stream_gemm_i8_kernel<%d rows per pass, %d channel fragments per wave, %s, %d steps in flight, K split %d>",
+                16 * MF, NF, SWIGLU ? "SiLU-mul" : "plain", D, KS);
   hipLaunchKernelGGL((stream_gemm_i8_kernel<MF, NF, SWIGLU, D, KS>), grid, dim3(kWaves * kWave), 0, s, p);
   return check_launch("kmoe_grouped_gemm_i8 (stream)");
 }

@@ -927,6 +927,14 @@ int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* w
   // persistent workgroups: WGS per CU
   const int grid = min(min(ceil_div(p.max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8), kBoardSlots);
   const size_t dyn = sizeof(int) * (static_cast<size_t>(p.E) + 1 + n_exp + 2);
+  if (tracing_kernels())
+    note_kernel("tiled_gemm_kernel<%s%s, %s, %dx%d tile, %d waves, %d per CU%s%s%s>%s",
+                KIND == TKind::I8 ? "int8" : (KIND == TKind::F8 ? "fp8" : (F16 ? "f16" : "bf16")),
+                (KIND != TKind::BF16 && F16) ? " -> f16" : "", SWIGLU ? "SiLU-mul" : (OAI ? "swigluoai" : "plain"), kTM,
+                kWavesT * nfh * 16 * (SWIGLU ? 2 : 1), WM * kWavesT, WGS, M32 ? ", 32x32 MFMA" : "",
+                PACE ? ", paced siblings" : "", R != 4 ? ", 8-slot weight ring" : "",
+                p.pick == 1 ? " [works if few experts overflow the tile, decided on the device]"
+                            : (p.pick == 2 ? " [works otherwise]" : ""));
   hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32, MF, OAI, PACE, F16>), dim3(grid),
                      dim3(WM * kWavesT * kWave), dyn, s, p);
   return check_launch(what);

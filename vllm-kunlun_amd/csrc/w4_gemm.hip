@@ -519,6 +519,9 @@ int launch_w4_tile(const W4Params& p, int rows, bool f16, hipStream_t s) {
   const dim3 grid(ceil_div(items, 8) * 8);
   // the scales of a wave's fragments in LDS, while two workgroups still fit a CU next to their activation buffers
   const size_t lds = static_cast<size_t>(kWaves) * NF * 16 * (p.k / p.gs) * sizeof(uint16_t);
+  if (tracing_kernels())
+    note_kernel("w4_tile_kernel<%d-row tiles, %s, %s, group scales in %s>", kTileRows, SWIGLU ? "SiLU-mul" : "plain",
+                f16 ? "f16" : "bf16", lds <= 16 * 1024 ? "LDS" : "global memory");
   if (lds <= 16 * 1024) {
     if (f16)
       hipLaunchKernelGGL((w4_tile_kernel<MF, NF, SWIGLU, true, true>), grid, dim3(kWaves * kWave), lds, s, p);
@@ -538,6 +541,9 @@ int launch_w4(const W4Params& p, bool f16, hipStream_t s) {
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const dim3 grid(ceil_div(n_half, kWaves * NFH * 16), p.E);
   const size_t lds = static_cast<size_t>(kWaves) * NF * 16 * (p.k / p.gs) * sizeof(uint16_t);
+  if (tracing_kernels())
+    note_kernel("w4_stream_kernel<%d rows per pass, %d channel fragments per wave, %s, %d blocks in flight, %s, group scales in %s>",
+                16 * MF, NF, SWIGLU ? "SiLU-mul" : "plain", D, f16 ? "f16" : "bf16", lds <= 32 * 1024 ? "LDS" : "global memory");
   if (lds <= 32 * 1024) {  // beyond: many small groups on a long K; the scales stay in global memory
     if (f16)
       hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, true, true>), grid, dim3(kWaves * kWave), lds, s, p);

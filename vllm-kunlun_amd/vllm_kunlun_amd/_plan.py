@@ -8,6 +8,7 @@ refuses to launch on another.
 """
 from __future__ import annotations
 
+import collections
 import weakref
 from typing import Optional
 
@@ -24,17 +25,27 @@ class _Workspace:
     """Scratch buffers that only grow, one per (device, stream) (plays the role of vLLM's
     current_workspace_manager(), reference: vllm_kunlun/ops/_kunlun_ops.py:528-531). Work queued on one
     stream runs in order, so the calls of a stream can share a buffer; two streams cannot, and a buffer is
-    only ever used on the stream it was allocated on (the caching allocator's own rule for reuse)."""
+    only ever used on the stream it was allocated on (the caching allocator's own rule for reuse).
+    At most MAX_STREAMS buffers are kept, least recently used first out: a process that makes and destroys
+    streams does not keep a buffer per handle it has ever seen. A dropped buffer goes back to torch's
+    allocator, which hands its memory out again only in the order of the stream it was allocated on, and a
+    plan keeps its own reference to the buffer it was built with."""
+
+    MAX_STREAMS = 8
 
     def __init__(self):
-        self._buf = {}
+        self._buf = collections.OrderedDict()
 
     def get(self, nbytes: int, device: torch.device, stream_id: int) -> torch.Tensor:
         key = (device.type, device.index, stream_id)
         buf = self._buf.get(key)
         if buf is None or buf.numel() < nbytes:
+            # allocated with the launching stream current, so the allocator ties the block to that stream
             buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
             self._buf[key] = buf
+        self._buf.move_to_end(key)
+        while len(self._buf) > self.MAX_STREAMS:
+            self._buf.popitem(last=False)
         return buf
 
 
@@ -207,7 +218,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
                   router_weight: Optional[torch.Tensor] = None, w13_bias: Optional[torch.Tensor] = None,
                   w2_bias: Optional[torch.Tensor] = None, activation: str = "silu", act_alpha: float = 1.702,
                   act_limit: float = 7.0, group_size: Optional[int] = None, tile_variant: int = 0,
-                  shared_scale: float = 1.0, first_expert: int = 0) -> MoEPlan:
+                  shared_scale: float = 1.0, first_expert: int = 0, side_stream: bool = False) -> MoEPlan:
     """x bf16 [M,H] (or float16 with int8 or unquantized weights, the latter then float16 too), logits f32 [M,E], out [M,H] like x; w13 [E,2I,H], w2 [E,H,I] in the
     format's dtype; w13_aux/w2_aux: per-channel maxes (int8) or block scales (fp8), None for bf16.
     shared_expert: (ws13 [2Is,H], ws13_aux, ws2 [H,Is], ws2_aux) in the same format.
@@ -220,7 +231,12 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     epilogue, models/deepseek_v2.py:286-292). tile_variant: a tuning variant of the int8 / fp8 tile kernel for the routed GEMMs (kmoe_moe_args.tile_variant).
     An expert-parallel share (ops/_kunlun_ops.py:640-696): logits [M,E_global] (correction bias [E_global], router
     weight [E_global,H]) with more experts than the weights hold, and first_expert = ep_rank * E: the routing runs
-    over all of them, the pairs routed to [first_expert, first_expert + E) are computed, the others add nothing."""
+    over all of them, the pairs routed to [first_expert, first_expert + E) are computed, the others add nothing.
+    side_stream: let a shared expert that cannot ride in the routed launches run on the library's second stream
+    beside them (KMOE_FLAG_SIDE_STREAM); by default every launch goes to the current stream.
+    The plan is bound to the stream that is current when it is built and refuses to run on another one; a plan that
+    a HIP graph is to replay must be built INSIDE the capture (a plan built before torch.cuda.graph() sits on
+    another stream than the capture's and raises when called inside it)."""
     if scoring_func not in ("softmax", "sigmoid"):
         raise ValueError(f"Unsupported scoring_func: {scoring_func}")
     if logits is None and router_weight is None:
@@ -316,6 +332,7 @@ def make_moe_plan(fmt: int, x: torch.Tensor, logits: torch.Tensor, out: torch.Te
     a.tile_variant = int(tile_variant)
     a.act_dtype = dt
     a.shared_scale = float(shared_scale)
+    a.flags = L.KMOE_FLAG_SIDE_STREAM if side_stream else 0
     a.out = out.data_ptr()
     if w_layout is None:  # per group of weights: tiled if both of its tensors have been tiled
         w_layout = L.KMOE_W_TILED if is_tiled(w13) and is_tiled(w2) else L.KMOE_W_ROWMAJOR

@@ -105,6 +105,11 @@ class _MonolithicQuantMoE:
     def is_monolithic(self) -> bool:
         return True
 
+    # True: a shared expert that cannot ride in the routed launches may run on the library's second stream beside
+    # them (KMOE_FLAG_SIDE_STREAM). Off by default: every launch then goes to the current stream, as the
+    # reference's does.
+    side_stream = False
+
     # routing parameters: kwargs win; a kwarg left at its default falls back to the layer
     @staticmethod
     def _routing(layer, topk_group, num_expert_group, scoring_func, routed_scaling_factor, bias):
@@ -176,7 +181,8 @@ class _MonolithicQuantMoE:
                              layer.w2_weight, layer.w13_weight_scale, layer.w2_weight_scale, scoring_func,
                              True,  # the reference always routes with the *_norm kernels
                              num_expert_group, topk_group, routed_scaling_factor, bias, shared_expert, out_scale,
-                             stage_events, router_weight=router_weight, shared_scale=shared_scale, first_expert=first)
+                             stage_events, router_weight=router_weight, shared_scale=shared_scale, first_expert=first,
+                             side_stream=bool(self.side_stream))
 
 
 class KunlunCompressedTensorsW8A8Int8MoEMethod(_MonolithicQuantMoE):

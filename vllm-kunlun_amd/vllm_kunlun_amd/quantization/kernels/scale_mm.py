@@ -79,6 +79,34 @@ class KunlunScaledMMLinearKernel:
         scale = scale.contiguous().clone().reshape(n, 1)
         with torch.no_grad():
             scale.mul_(127.0)  # scale -> absmax, what the kernels take (x_pc_max / w_pc_max convention)
+        # Static input scheme (base-class part, upstream vLLM's CutlassInt8ScaledMMLinearKernel, which is not in
+        # this container: restated from its published source): a layer fused from several checkpoint tensors
+        # (qkv, gate_up) carries one input scale - and zero point - per partition, and the kernels take ONE.
+        # Symmetric: the largest scale. Asymmetric: the value range every partition covers,
+        # [min_p scale_p (-128 - zp_p), max_p scale_p (127 - zp_p)], cut into 255 steps again.
+        if self.config.is_static_input_scheme:
+            i_s = getattr(layer, i_s_name, None)
+            if i_s is None:
+                raise ValueError(f"{i_s_name}: a static input scheme needs the input scale")
+            s_in = i_s.data.to(torch.float32).reshape(-1)
+            if self.config.input_symmetric:
+                setattr(layer, i_s_name, torch.nn.Parameter(s_in.max().reshape(1), requires_grad=False))
+            else:
+                i_zp = getattr(layer, i_zp_name, None)
+                if i_zp is None:
+                    raise ValueError(f"{i_zp_name}: a static asymmetric scheme needs the input zero point")
+                zps = i_zp.data.to(torch.int32).reshape(-1)
+                if zps.numel() not in (1, s_in.numel()):
+                    raise ValueError(f"{i_zp_name}: {zps.numel()} zero points for {s_in.numel()} input scales")
+                if s_in.numel() > 1:  # (one partition: its scale and zero point are kept as they are)
+                    range_max = (s_in * (127 - zps)).max()
+                    range_min = (s_in * (-128 - zps)).min()
+                    one_scale = (range_max - range_min) / 255.0
+                    # rounded to the nearest integer: the quotient is an integer up to float error when one
+                    # partition spans the whole range, and truncation would then lose one
+                    one_zp = torch.round(-128 - range_min / one_scale).to(torch.int32)
+                    setattr(layer, i_s_name, torch.nn.Parameter(one_scale.reshape(1), requires_grad=False))
+                    setattr(layer, i_zp_name, torch.nn.Parameter(one_zp.reshape(1), requires_grad=False))
         # Asymmetric activations (base-class part): azp_adj = the sums of the weight codes over k per output channel,
         # times the input zero point for a static scheme, whose zero point then needs no term of its own at run time.
         if not self.config.input_symmetric:

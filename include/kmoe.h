@@ -467,6 +467,17 @@ int kmoe_silu_and_mul_dt(const uint16_t* y, int64_t ld_y, int R, int I, uint16_t
                          int act_dtype, kmoe_stream_t stream);
 
 /*
+ * The device's SiLU, tabulated: table[h] (f32, 65536 entries) = silu of the 16-bit activation pattern h in
+ * act_dtype, computed by the very function every GEMM epilogue and kmoe_silu_and_mul use. No counterpart in the
+ * reference; it exists for checkers. The kernels compute silu(g) = g / (1 + e^-g) on the hardware's exp2 and
+ * reciprocal instructions (each within one ulp, not correctly rounded), applied to the gate value AFTER it has been
+ * rounded to the activation type, as the reference's silu_and_mul (ops/_custom_ops.py:699-706) reads a 16-bit
+ * tensor. A CPU restatement that looks silu up in this table therefore reproduces the kernels' outputs bit for
+ * bit, and the table itself is what to hold against a libm silu (within 4e-6 relative).
+ */
+int kmoe_silu_table(float* table, int act_dtype, kmoe_stream_t stream);
+
+/*
  * Un-permute + weighted top-K sum. Replaces kunlun_ops.moe_post
  * (ops/_custom_ops.py:1316-1324, called compressed_tensors_moe.py:278-290).
  *   out[m,h] = bf16( sum_k topk_w[m,k] * dq[m,k] * float(x[moe_index[m*K+k], h]) )

@@ -37,6 +37,8 @@ def lib() -> C.CDLL:
         _lib.orc_sigmoid.argtypes = [C.c_float]
         _lib.orc_silu.restype = C.c_float
         _lib.orc_silu.argtypes = [C.c_float]
+        _lib.orc_set_silu_table.restype = None
+        _lib.orc_set_silu_table.argtypes = [C.c_int, C.c_void_p]
         _lib.orc_f32_to_e4m3fn.restype = C.c_uint8
         _lib.orc_f32_to_e4m3fn.argtypes = [C.c_float]
         _lib.orc_e4m3fn_to_f32.restype = C.c_float
@@ -97,6 +99,66 @@ def sigmoid(x: np.ndarray) -> np.ndarray:
 def silu(x: np.ndarray) -> np.ndarray:
     f = lib().orc_silu
     return np.array([f(float(v)) for v in np.asarray(x, dtype=np.float32).ravel()], dtype=np.float32).reshape(np.shape(x))
+
+
+# -- the device's SiLU table ----------------------------------------------------
+# The layer applies SiLU to gate values rounded to the 16-bit activation type: 65536 possible arguments per type.
+# The product computes it with the GPU's exp2 / reciprocal instructions, whose bits no CPU sequence reproduces, so
+# a GPU test fetches the product's table of all 65536 results (kmoe_silu_table), holds it against the closed form
+# here, and installs it: from then on every oracle function that applies SiLU uses the device's values.
+SILU_REL_TOL = 4e-6    # against float64 g / (1 + exp(-g)); measured on MI355X: 4.2e-7 at most
+SILU_ABS_TOL = 2e-36   # results below the normal range
+
+
+def act_values(f16: bool) -> np.ndarray:
+    """float32 value of every 16-bit activation pattern 0..65535."""
+    h = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    return h.view(np.float16).astype(np.float32) if f16 else bf16_bits_to_f32(h)
+
+
+def check_silu_table(f16: bool, table: np.ndarray) -> float:
+    """Holds a device SiLU table against float64 g / (1 + exp(-g)) on every finite argument; returns the largest
+    relative error seen. Raises AssertionError beyond SILU_REL_TOL / SILU_ABS_TOL, or unless silu(+inf) = +inf and
+    silu(-inf) is (as good as) zero."""
+    table = np.asarray(table, dtype=np.float32)
+    assert table.shape == (65536,)
+    with np.errstate(invalid="ignore"):
+        g = act_values(f16).astype(np.float64)
+    fin = np.isfinite(g)
+    with np.errstate(over="ignore"):
+        want = g[fin] / (1.0 + np.exp(-g[fin]))
+    got = table[fin].astype(np.float64)
+    err = np.abs(got - want)
+    ok = err <= SILU_REL_TOL * np.abs(want) + SILU_ABS_TOL
+    assert ok.all(), (f"device SiLU table ({'f16' if f16 else 'bf16'}): {np.count_nonzero(~ok)} entries beyond tolerance, "
+                      f"worst at g={g[fin][np.argmax(err / (np.abs(want) + 1e-30))]!r}")
+    assert np.array_equal(np.signbit(got[want != 0]), np.signbit(want[want != 0]))
+    inf = np.isinf(g)
+    assert (table[inf & (g > 0)] == np.inf).all() and (np.abs(table[inf & (g < 0)]) <= SILU_ABS_TOL).all()
+    big = np.abs(want) > 1e-30
+    return float((err[big] / np.abs(want[big])).max())
+
+
+def set_silu_table(f16: bool, table) -> None:
+    """Installs (or, with None, removes) the SiLU table of one activation type."""
+    if table is None:
+        lib().orc_set_silu_table(1 if f16 else 0, None)
+        return
+    t = _c(table, np.float32)
+    assert t.shape == (65536,)
+    lib().orc_set_silu_table(1 if f16 else 0, _p(t))
+
+
+def install_device_silu(fetch) -> dict:
+    """fetch(f16) -> the device's SiLU table for that activation type (65536 float32, e.g. from the product's
+    kmoe_silu_table). Each table is held against the closed form (check_silu_table) and installed; returns the
+    largest relative error per type."""
+    worst = {}
+    for f16 in (False, True):
+        table = np.asarray(fetch(f16), dtype=np.float32)
+        worst["f16" if f16 else "bf16"] = check_silu_table(f16, table)
+        set_silu_table(f16, table)
+    return worst
 
 
 # -- stages -------------------------------------------------------------------

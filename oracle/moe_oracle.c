@@ -21,7 +21,9 @@
  *   - rounding is round-half-to-even everywhere (rintf under the default mode);
  *   - top-k order: score descending, ties to the lower expert id;
  *   - exp() is the fixed fma sequence orc_exp() below (< 2 ulp from libm), so a
- *     device kernel performing the same sequence yields the same bits;
+ *     device kernel performing the same sequence yields the same bits (routing);
+ *   - SiLU of a 16-bit gate value: orc_silu() below, or - under a GPU test - the
+ *     device's own table of its 65536 values (see silu_act);
  *   - the softmax row sum adds 64 interleaved partial sums (element e goes to
  *     partial e % 64, in ascending e) with a balanced binary tree;
  *   - dequant is ((float)acc * (a_max/127)) * (w_max/127), left to right;
@@ -120,6 +122,23 @@ ORC_API float orc_exp(float x) {
 
 ORC_API float orc_sigmoid(float x) { return 1.0f / (1.0f + orc_exp(-x)); }
 ORC_API float orc_silu(float x) { return x / (1.0f + orc_exp(-x)); }
+
+/* SiLU as the layer applies it: to a gate value that has been rounded to the 16-bit activation type first (the
+ * reference's silu_and_mul reads a 16-bit tensor, ops/_custom_ops.py:699-706). A function of 65536 arguments per
+ * activation type, so its values can be handed over as a table: the device under test computes SiLU with its
+ * hardware's exp2 and reciprocal approximations (within an ulp each, not correctly rounded - no CPU sequence has
+ * their bits), and a GPU test installs the device's table (orc_set_silu_table) after holding it against libm.
+ * Without a table (CPU-only tests, the golden fixtures) silu is orc_silu above. */
+static float g_silu_table[2][65536];
+static int g_silu_table_set[2] = {0, 0};
+ORC_API void orc_set_silu_table(int f16, const float* table) {
+  const int t = f16 != 0;
+  g_silu_table_set[t] = table != 0;
+  if (table) memcpy(g_silu_table[t], table, sizeof(g_silu_table[t]));
+}
+static inline float silu_act(uint16_t h) {
+  return g_silu_table_set[g_act_f16] ? g_silu_table[g_act_f16][h] : orc_silu(act_to_f32(h));
+}
 
 /* K best of score[0..E) among eligible entries: score descending, ties to the
  * lower index. O(E*K) selection; out_ids in selection order. */
@@ -426,7 +445,7 @@ ORC_API void orc_grouped_gemm_i8(const int8_t* a, int64_t lda, const float* a_ma
           }
           const uint16_t yg = f32_to_act(((float)ag * sa) * (wm[c] / 127.0f));
           const uint16_t yu = f32_to_act(((float)au * sa) * (wm[half + c] / 127.0f));
-          if (y) y[(size_t)r * ldy + c] = f32_to_act(orc_silu(act_to_f32(yg)) * act_to_f32(yu));
+          if (y) y[(size_t)r * ldy + c] = f32_to_act(silu_act(yg) * act_to_f32(yu));
         }
       }
     }
@@ -482,7 +501,7 @@ ORC_API void orc_grouped_gemm_bf16(const uint16_t* a, int64_t lda, const int32_t
           const uint16_t* wu = we + (size_t)(half + c) * k;
           for (int i = 0; i < k; ++i) u += act_to_f32(ar[i]) * act_to_f32(wu[i]);
           y[(size_t)r * ldy + c] =
-              f32_to_act(orc_silu(act_to_f32(f32_to_act(g))) * act_to_f32(f32_to_act(u)));
+              f32_to_act(silu_act(f32_to_act(g)) * act_to_f32(f32_to_act(u)));
         } else {
           y[(size_t)r * ldy + c] = f32_to_act(g);
         }
@@ -589,7 +608,7 @@ ORC_API void orc_grouped_gemm_fp8(const uint8_t* a, int64_t lda, const float* a_
         }
         if (act)
           y[(size_t)r * ldy + c] =
-              f32_to_act(orc_silu(act_to_f32(f32_to_act(tot[0]))) * act_to_f32(f32_to_act(tot[1])));
+              f32_to_act(silu_act(f32_to_act(tot[0])) * act_to_f32(f32_to_act(tot[1])));
         else
           y[(size_t)r * ldy + c] = f32_to_act(tot[0]);
       }
@@ -601,7 +620,7 @@ ORC_API void orc_grouped_gemm_fp8(const uint8_t* a, int64_t lda, const float* a_
 ORC_API void orc_silu_and_mul(const uint16_t* y, int64_t ld_y, int R, int I, uint16_t* out, int64_t ld_out) {
   for (int r = 0; r < R; ++r)
     for (int i = 0; i < I; ++i)
-      out[(size_t)r * ld_out + i] = f32_to_act(orc_silu(act_to_f32(y[(size_t)r * ld_y + i])) *
+      out[(size_t)r * ld_out + i] = f32_to_act(silu_act(y[(size_t)r * ld_y + i]) *
                                                  act_to_f32(y[(size_t)r * ld_y + I + i]));
 }
 

@@ -3,8 +3,10 @@ libkmoe.so) and compared with the C oracle on the same seeded inputs.
 
 Bars: routing ids, sort maps, int8 codes, int32 accumulators — bit-exact.
 bf16/f32 stage outputs — bit-exact too, because oracle and kernels perform the
-same fixed float sequences; the looser north-star tolerance (rel-L2 <= 1e-2) is
-asserted against the independently written torch oracle in test_gpu_layer.py.
+same fixed float sequences (SiLU: the oracle looks it up in the device's table of
+all 65536 16-bit arguments, which test_device_silu_table holds against the closed
+form); the looser north-star tolerance (rel-L2 <= 1e-2) is asserted against the
+independently written torch oracle in test_gpu_layer.py.
 """
 import ctypes as C
 
@@ -375,6 +377,37 @@ def test_silu_and_mul(L, R, I):
     L.check(L.lib.kmoe_silu_and_mul(L.ptr(dy), 2 * I, R, I, L.ptr(out), I, L.stream()))
     sync()
     assert np.array_equal(bits(out), ref)
+
+
+@pytest.mark.parametrize("f16", [False, True], ids=["bf16", "f16"])
+def test_device_silu_table(L, f16):
+    """kmoe_silu_table: the device's SiLU of all 65536 16-bit arguments. Against float64 g / (1 + exp(-g)) within
+    the tolerance the oracle states (c_oracle.SILU_REL_TOL), and the stand-alone silu_and_mul kernel - the same
+    device function - gives exactly the table's values rounded to the activation type (up = 1), on every argument.
+    Against the unrounded torch silu the rounded outputs differ by at most one 16-bit step."""
+    table = torch.empty(65536, dtype=torch.float32, device="cuda")
+    L.check(L.lib.kmoe_silu_table(L.ptr(table), 1 if f16 else 0, L.stream()))
+    sync()
+    host = table.cpu().numpy()
+    worst = co.check_silu_table(f16, host)
+    assert worst <= co.SILU_REL_TOL
+    dt = torch.float16 if f16 else torch.bfloat16
+    gate = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dt)  # every pattern once
+    y = torch.cat([gate.reshape(512, 128), torch.ones(512, 128, dtype=dt)], dim=1).cuda()
+    out = torch.empty(512, 128, dtype=dt, device="cuda")
+    L.check(L.lib.kmoe_silu_and_mul_dt(L.ptr(y), 256, 512, 128, L.ptr(out), 128, 1 if f16 else 0, L.stream()))
+    sync()
+    want = torch.from_numpy(host).to(dt).reshape(512, 128)  # torch rounds to nearest even, as the kernels do
+    finite = torch.isfinite(gate.float()).reshape(512, 128)
+    got = out.cpu()
+    assert torch.equal(got[finite].view(torch.int16), want[finite].view(torch.int16))
+    # one 16-bit step at most from the rounded closed form
+    # (where the result is far below the type's normal range - arguments below -80 - "as good as zero" is the bar)
+    ref = torch.nn.functional.silu(gate.float().double()).to(dt).reshape(512, 128)
+    usual = finite & (gate.float() >= -80.0).reshape(512, 128)
+    step = (got[usual].view(torch.int16).int() - ref[usual].view(torch.int16).int()).abs()
+    assert int(step.max()) <= 1
+    assert float(got[finite & ~usual].float().abs().max()) <= 1e-30
 
 
 @pytest.mark.parametrize("M,K,H", [(1, 1, 8), (64, 8, 2048), (33, 6, 7168), (128, 8, 512)])

@@ -133,8 +133,14 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint16_t* __res
   g.v = *reinterpret_cast<const uint4*>(y + static_cast<size_t>(r) * ld_y + c);
   u.v = *reinterpret_cast<const uint4*>(y + static_cast<size_t>(r) * ld_y + I + c);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) o.h[j] = f32_to_act(silu_fixed(act_to_f32(g.h[j], f16)) * act_to_f32(u.h[j], f16), f16);
+  for (int j = 0; j < 8; ++j) o.h[j] = f32_to_act(silu_hw(act_to_f32(g.h[j], f16)) * act_to_f32(u.h[j], f16), f16);
   *reinterpret_cast<uint4*>(out + static_cast<size_t>(r) * ld_out + c) = o.v;
+}
+
+// silu_hw of every 16-bit activation pattern (see kmoe_silu_table)
+__global__ __launch_bounds__(256) void silu_table_kernel(float* __restrict__ table, int dt) {
+  const unsigned h = blockIdx.x * blockDim.x + threadIdx.x;
+  if (h < 65536u) table[h] = silu_hw(act_to_f32(static_cast<uint16_t>(h), dt != 0));
 }
 
 // ----------------------------------------------------------------- combine
@@ -479,6 +485,13 @@ extern "C" int kmoe_silu_and_mul_dt(const uint16_t* y, int64_t ld_y, int R, int 
   hipLaunchKernelGGL(silu_and_mul_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0,
                      as_stream(stream), y, ld_y, R, I, out, ld_out, act_dtype);
   return check_launch("kmoe_silu_and_mul");
+}
+
+extern "C" int kmoe_silu_table(float* table, int act_dtype, kmoe_stream_t stream) {
+  if (int rc = check_dtype(act_dtype, "silu_table")) return rc;
+  KMOE_REQUIRE(table, KMOE_ERR_NULL, "silu_table: NULL pointer");
+  hipLaunchKernelGGL(silu_table_kernel, dim3(65536 / 256), dim3(256), 0, as_stream(stream), table, act_dtype);
+  return check_launch("kmoe_silu_table");
 }
 
 extern "C" int kmoe_combine(const uint16_t* x, int64_t ld_x, const int32_t* moe_index, const float* topk_w,

@@ -370,7 +370,7 @@ __global__ __launch_bounds__(WAVES* kWave) void grouped_gemm_kernel(const GemmPa
           uint16_t uv[4];
           finish(acc[mf][f + NFH], col[f + NFH] + lg * 4, uv);
 #pragma unroll
-          for (int q = 0; q < 4; ++q) yv[q] = f32_to_act(silu_fixed(act_to_f32(yv[q], f16)) * act_to_f32(uv[q], f16), f16);
+          for (int q = 0; q < 4; ++q) yv[q] = f32_to_act(silu_hw(act_to_f32(yv[q], f16)) * act_to_f32(uv[q], f16), f16);
         }
         if constexpr (KIND == Kind::BF16 && !SWIGLU) {
           if (p.bias) {

@@ -116,7 +116,22 @@ __device__ inline float exp_fixed(float x) {
 }
 
 __device__ inline float sigmoid_fixed(float x) { return 1.0f / (1.0f + exp_fixed(-x)); }
-__device__ inline float silu_fixed(float x) { return x / (1.0f + exp_fixed(-x)); }
+
+// ---- SiLU of the GEMM epilogues ----------------------------------------------
+// silu(g) = g / (1 + e^-g) on the hardware's transcendental unit: v_exp_f32 (2^t) and v_rcp_f32, each within
+// one ulp, five instructions in all - the fixed-sequence exp and an IEEE divide cost thirty and were a sixth of
+// the prefill gate_up launch. The two instructions are not correctly rounded, so no CPU sequence gives their
+// bits; but SiLU is only ever applied to a 16-BIT activation value (gate is rounded to bf16 / half first, as the
+// reference's silu_and_mul reads a 16-bit tensor), i.e. to one of 65536 arguments per activation type:
+// kmoe_silu_table writes this function's result for every one of them, which is how a checker follows it bit
+// for bit. Every kernel calls THIS function, so a token's result does not depend on the kernel that computes it.
+// Arguments below -87 count as -87 (1 + 2^t and its reciprocal stay in the normal range; the result there,
+// -1.4e-36, is 0 for every purpose, also for g = -inf, which would otherwise give inf x 0).
+__device__ inline float silu_hw(float g) {
+  const float gc = fmaxf(g, -87.0f);
+  const float d = 1.0f + __builtin_amdgcn_exp2f(gc * -0x1.715476p+0f);  // 1 + 2^(-g log2(e))
+  return gc * __builtin_amdgcn_rcpf(d);
+}
 // gpt-oss activation on a (gate, up) pair of bf16 values, one rounding at the end:
 // g = min(gate, limit), u = clamp(up, -limit, limit), out = (u + 1) * g * sigmoid(alpha * g)
 // (reference: swigluoai_and_mul, ops/_custom_ops.py:728-742).

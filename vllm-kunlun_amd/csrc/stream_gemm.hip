@@ -222,7 +222,7 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
           uint16_t uv[4];
           finish(acc[mf][f + NFH], col[f + NFH] + lg * 4, uv);
 #pragma unroll
-          for (int q = 0; q < 4; ++q) yv[q] = f32_to_act(silu_fixed(act_to_f32(yv[q], f16)) * act_to_f32(uv[q], f16), f16);
+          for (int q = 0; q < 4; ++q) yv[q] = f32_to_act(silu_hw(act_to_f32(yv[q], f16)) * act_to_f32(uv[q], f16), f16);
         }
         const uint2 packed = make_uint2(yv[0] | (static_cast<uint32_t>(yv[1]) << 16),
                                         yv[2] | (static_cast<uint32_t>(yv[3]) << 16));

@@ -848,7 +848,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
               if constexpr (!I8) uf = acc[mf][fu][4 * b + q];
               else uf = (static_cast<float>(acc[mf][fu][4 * b + q]) * sa) * sw[fu][4 * b + q];
               const float u = F16 ? half_to_f32(f32_to_half(uf)) : bf16_to_f32(f32_to_bf16_hw(uf));
-              yv[q] = silu_fixed(g) * u;
+              yv[q] = silu_hw(g) * u;
             }
           }
           if constexpr (BF && !M32 && !SWIGLU) {

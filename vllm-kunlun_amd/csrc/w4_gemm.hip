@@ -242,7 +242,7 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
         if (SWIGLU) {
 #pragma unroll
           for (int q = 0; q < 4; ++q)
-            yv[q] = f32_to_act(silu_fixed(act_to_f32(yv[q], F16)) * act_to_f32(f32_to_act(acc[mf][f + NFH][q], F16), F16), F16);
+            yv[q] = f32_to_act(silu_hw(act_to_f32(yv[q], F16)) * act_to_f32(f32_to_act(acc[mf][f + NFH][q], F16), F16), F16);
         }
         const uint2 packed = make_uint2(yv[0] | (static_cast<uint32_t>(yv[1]) << 16),
                                         yv[2] | (static_cast<uint32_t>(yv[3]) << 16));
@@ -498,7 +498,7 @@ __global__ __launch_bounds__(kWaves* kWave, 2) void w4_tile_kernel(const W4Param
       if (SWIGLU) {
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          yv[q] = f32_to_act(silu_fixed(act_to_f32(yv[q], F16)) * act_to_f32(f32_to_act(acc[mf][f + NFH][q], F16), F16), F16);
+          yv[q] = f32_to_act(silu_hw(act_to_f32(yv[q], F16)) * act_to_f32(f32_to_act(acc[mf][f + NFH][q], F16), F16), F16);
       }
       const uint2 packed = make_uint2(yv[0] | (static_cast<uint32_t>(yv[1]) << 16),
                                       yv[2] | (static_cast<uint32_t>(yv[3]) << 16));

@@ -252,30 +252,33 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   // search over tile_lo and two divisions, all lanes at once) and leaves (expert, first row, channel
   // block) in LDS; the tile loop then reads three words per tile instead of searching.
   __shared__ int item_e[kWave], item_row0[kWave], item_nb[kWave], item_sib[kWave];
+  const int per_xcd = gridDim.x >> 3;  // gridDim.x is a multiple of 8
+  // item lid of the list (lid < seg_end) -> expert, first row, channel block, sibling flags
+  auto resolve_item = [&](int lid, int& e, int& row0, int& nb, int& sib) {
+    const int m_tile = lid / p.n_blocks;
+    // the last e with tile_lo[e] <= m_tile: of a run of equal entries (empty experts) the one that owns the tile
+    int lo = 0, hi = n_exp - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (tile_lo[mid] <= m_tile) lo = mid;
+      else hi = mid - 1;
+    }
+    e = lo;
+    const int first = tile_lo[e], mt = tile_lo[e + 1] - first;
+    const int u = lid - first * p.n_blocks;
+    nb = u / mt;
+    const int m = u - nb * mt;
+    row0 = rows_begin(e) + m * kTM;
+    // siblings run on the workgroups before / after this one in the XCD, at the same list position
+    const int j = blockIdx.x >> 3;
+    if (m > 0 && j > 0) sib |= 1;
+    if (m + 1 < mt && j + 1 < per_xcd && lid + 1 < seg_end) sib |= 2;
+  };
   auto resolve_items = [&](int it0) {
     if (wave_id == 0) {
-      const int lid = xcd * seg + (blockIdx.x >> 3) + (it0 + lane) * (gridDim.x >> 3);  // gridDim.x is a multiple of 8
+      const int lid = xcd * seg + (blockIdx.x >> 3) + (it0 + lane) * per_xcd;
       int e = -1, row0 = 0, nb = 0, sib = 0;
-      if (lid < seg_end) {
-        const int m_tile = lid / p.n_blocks;
-        // the last e with tile_lo[e] <= m_tile: of a run of equal entries (empty experts) the one that owns the tile
-        int lo = 0, hi = n_exp - 1;
-        while (lo < hi) {
-          const int mid = (lo + hi + 1) >> 1;
-          if (tile_lo[mid] <= m_tile) lo = mid;
-          else hi = mid - 1;
-        }
-        e = lo;
-        const int first = tile_lo[e], mt = tile_lo[e + 1] - first;
-        const int u = lid - first * p.n_blocks;
-        nb = u / mt;
-        const int m = u - nb * mt;
-        row0 = rows_begin(e) + m * kTM;
-        // siblings run on the workgroups before / after this one in the XCD, at the same list position
-        const int j = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
-        if (m > 0 && j > 0) sib |= 1;
-        if (m + 1 < mt && j + 1 < per_xcd && lid + 1 < seg_end) sib |= 2;
-      }
+      if (lid < seg_end) resolve_item(lid, e, row0, nb, sib);
       item_sib[lane] = sib;
       item_e[lane] = e;
       item_row0[lane] = row0;
@@ -397,10 +400,112 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   };
   // fragment n of a step: (row fragment, K part); 16x16: 8 row fragments; 32x32: 2 K parts x 4
   constexpr int kFragReads = M32 ? 2 * AM : kMF;
+  // Row fragments of this wave that hold rows of the current tile (wave-uniform, set per tile): the K loop of the
+  // int8 path neither reads nor multiplies the others (the padding of an expert's last tile).
+  int live_frags = kMF;
+  // One row fragment of one MFMA step, int8: LDS read of the NEXT live fragment, wait for this one's, NF MFMAs -
+  // all inside one assembly statement, because the skip is a branch: a branch the compiler can see splits the
+  // loop body into basic blocks, after which its register allocator spills hundreds of registers. `live` is
+  // wave-uniform (an SGPR); a live fragment falls through its test, a dead one costs a compare and a taken branch.
+  // LDS operations of a wave complete in order, so "at most one in flight" means this fragment's read has landed.
+  auto frag_i8 = [&](const v4i(&w)[kNF], v4i& af_cur, v4i& af_next, uint32_t addr, auto n_tag, auto off_own, auto off_next,
+                     int mf) {
+    constexpr int n = decltype(n_tag)::value;
+    constexpr bool kFirst = n == 0, kLast = n + 1 == kMF;
+    static_assert(kNF == 4 || kNF == 2, "fragment step written for 2 or 4 channel fragments per wave");
+// dead fragment: leave
+#define KMOE_FRAG_HEAD "s_cmp_lt_i32 %[live], %[n1]\n\ts_cbranch_scc1 3f\n\t"
+// the first fragment of a step requests its own bytes
+#define KMOE_FRAG_OWN "ds_read_b128 %[cur], %[addr] offset:%[own]\n\t"
+// request the next fragment's bytes, then wait for this one's. The request is unconditional: a taken branch costs a
+// wave some twenty cycles, and a test for "the next one is dead" would put one on the path of every live fragment.
+// If the next fragment is dead its bytes arrive unused, and the wait at the end of the step retires the request.
+#define KMOE_FRAG_NEXT "ds_read_b128 %[nxt], %[addr] offset:%[onext]\n\ts_waitcnt lgkmcnt(1)\n\t"
+#define KMOE_FRAG_WAIT "s_waitcnt lgkmcnt(0)\n\t"
+#define KMOE_FRAG_MFMA2                                          \
+  "v_mfma_i32_16x16x64_i8 %[c0], %[w0], %[cur], %[c0]\n\t"       \
+  "v_mfma_i32_16x16x64_i8 %[c1], %[w1], %[cur], %[c1]\n\t"
+#define KMOE_FRAG_MFMA4                                          \
+  KMOE_FRAG_MFMA2                                                \
+  "v_mfma_i32_16x16x64_i8 %[c2], %[w2], %[cur], %[c2]\n\t"       \
+  "v_mfma_i32_16x16x64_i8 %[c3], %[w3], %[cur], %[c3]\n\t"
+#define KMOE_FRAG_IMMS                                                                                       \
+  [addr] "v"(addr), [live] "s"(live_frags), [n1] "n"(n + 1), [own] "n"(decltype(off_own)::value), \
+      [onext] "n"(decltype(off_next)::value)
+    if constexpr (kNF == 4) {
+#define KMOE_FRAG_ACC [c0] "+v"(acc[mf][0]), [c1] "+v"(acc[mf][1]), [c2] "+v"(acc[mf][2]), [c3] "+v"(acc[mf][3])
+#define KMOE_FRAG_W [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]), [w3] "v"(w[3])
+      if constexpr (kFirst && kLast)
+        asm volatile(KMOE_FRAG_HEAD KMOE_FRAG_OWN KMOE_FRAG_WAIT KMOE_FRAG_MFMA4 "3:\n\t"
+                     : KMOE_FRAG_ACC, [cur] "=&v"(af_cur) : KMOE_FRAG_W, KMOE_FRAG_IMMS : "scc", "memory");
+      else if constexpr (kFirst)
+        asm volatile(KMOE_FRAG_HEAD KMOE_FRAG_OWN KMOE_FRAG_NEXT KMOE_FRAG_MFMA4 "3:\n\t"
+                     : KMOE_FRAG_ACC, [cur] "=&v"(af_cur), [nxt] "=&v"(af_next) : KMOE_FRAG_W, KMOE_FRAG_IMMS
+                     : "scc", "memory");
+      else if constexpr (kLast)
+        asm volatile(KMOE_FRAG_HEAD KMOE_FRAG_WAIT KMOE_FRAG_MFMA4 "3:\n\t"
+                     : KMOE_FRAG_ACC : KMOE_FRAG_W, [cur] "v"(af_cur), KMOE_FRAG_IMMS : "scc", "memory");
+      else
+        asm volatile(KMOE_FRAG_HEAD KMOE_FRAG_NEXT KMOE_FRAG_MFMA4 "3:\n\t"
+                     : KMOE_FRAG_ACC, [nxt] "=&v"(af_next) : KMOE_FRAG_W, [cur] "v"(af_cur), KMOE_FRAG_IMMS
+                     : "scc", "memory");
+#undef KMOE_FRAG_ACC
+#undef KMOE_FRAG_W
+    } else {
+#define KMOE_FRAG_ACC [c0] "+v"(acc[mf][0]), [c1] "+v"(acc[mf][1])
+#define KMOE_FRAG_W [w0] "v"(w[0]), [w1] "v"(w[1])
+      if constexpr (kFirst && kLast)
+        asm volatile(KMOE_FRAG_HEAD KMOE_FRAG_OWN KMOE_FRAG_WAIT KMOE_FRAG_MFMA2 "3:\n\t"
+                     : KMOE_FRAG_ACC, [cur] "=&v"(af_cur) : KMOE_FRAG_W, KMOE_FRAG_IMMS : "scc", "memory");
+      else if constexpr (kFirst)
+        asm volatile(KMOE_FRAG_HEAD KMOE_FRAG_OWN KMOE_FRAG_NEXT KMOE_FRAG_MFMA2 "3:\n\t"
+                     : KMOE_FRAG_ACC, [cur] "=&v"(af_cur), [nxt] "=&v"(af_next) : KMOE_FRAG_W, KMOE_FRAG_IMMS
+                     : "scc", "memory");
+      else if constexpr (kLast)
+        asm volatile(KMOE_FRAG_HEAD KMOE_FRAG_WAIT KMOE_FRAG_MFMA2 "3:\n\t"
+                     : KMOE_FRAG_ACC : KMOE_FRAG_W, [cur] "v"(af_cur), KMOE_FRAG_IMMS : "scc", "memory");
+      else
+        asm volatile(KMOE_FRAG_HEAD KMOE_FRAG_NEXT KMOE_FRAG_MFMA2 "3:\n\t"
+                     : KMOE_FRAG_ACC, [nxt] "=&v"(af_next) : KMOE_FRAG_W, [cur] "v"(af_cur), KMOE_FRAG_IMMS
+                     : "scc", "memory");
+#undef KMOE_FRAG_ACC
+#undef KMOE_FRAG_W
+    }
+#undef KMOE_FRAG_HEAD
+#undef KMOE_FRAG_OWN
+#undef KMOE_FRAG_NEXT
+#undef KMOE_FRAG_WAIT
+#undef KMOE_FRAG_MFMA2
+#undef KMOE_FRAG_MFMA4
+#undef KMOE_FRAG_IMMS
+  };
   // keep: std::false_type (every fragment as read), or an int mask (0: the fragments count as zeros)
   auto compute = [&](const v4i(&wcur)[kNF], auto buf_tag, auto j_tag, auto keep) {
     constexpr int buf = decltype(buf_tag)::value, j = decltype(j_tag)::value;
-    if constexpr (ADMA) {
+    if constexpr (ADMA && I8 && !M32) {
+      constexpr bool kFarStages = kStagesA * kStageBytes > 65536;
+      constexpr int kImm = kFarStages ? 0 : buf * kStageBytes;
+      const uint32_t addr = fa[j] + (kFarStages ? buf * kStageBytes : 0);
+      // (a masked step zeroes the WEIGHTS: integers have no infinity that a zero could turn into NaN)
+      v4i wm[kNF];
+#pragma unroll
+      for (int f = 0; f < kNF; ++f) {
+        if constexpr (std::is_same_v<decltype(keep), int>) wm[f] = wcur[f] & (v4i){keep, keep, keep, keep};
+        else wm[f] = wcur[f];
+      }
+      v4i af[2];
+      auto run = [&](auto self, auto n_tag) {
+        constexpr int n = decltype(n_tag)::value;
+        if constexpr (n < kMF) {
+          frag_i8(wm, af[n & 1], af[(n + 1) & 1], addr, n_tag, std::integral_constant<int, kImm + n * 16 * kChunk>{},
+                  std::integral_constant<int, kImm + (n + 1 < kMF ? n + 1 : n) * 16 * kChunk>{}, n);
+          self(self, std::integral_constant<int, n + 1>{});
+        }
+      };
+      run(run, std::integral_constant<int, 0>{});
+      // (retires the request a live fragment made for a dead one; the two registers count as in use until here)
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0]), "+v"(af[1]));
+    } else if constexpr (ADMA) {
       // two fragments in flight: the read of fragment n + 1 leaves before the MFMAs of fragment n
       v4i af[2];
       // (the instruction's offset field has 16 bits: with 32 KB buffers the buffer's offset goes into the address)
@@ -637,6 +742,10 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
       seen_prev = seen_next = 0;  // nothing polled for this tile yet: its first chunk starts without waiting
       patience = kSyncPatience;
     }
+    if constexpr (ADMA && I8 && !M32) {
+      const int rows_here = min(rows_end(cur.e), cur.row0 + kTM) - cur.row0 - wave_m * 16 * kMF;
+      live_frags = __builtin_amdgcn_readfirstlane(max(0, min(kMF, (rows_here + 15) >> 4)));
+    }
     int rs_next[kNA];
 #pragma unroll
     for (int i = 0; i < kNA; ++i) rs_next[i] = fetch_src(look, look.row0 + a_row(i));
@@ -755,6 +864,9 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
       }
     }
 
+    // (the int8 MFMAs are issued from assembly statements: the compiler does not know that the accumulators come
+    // out of the matrix pipe and inserts no wait states before the first VALU instruction that reads them)
+    if constexpr (ADMA && I8 && !M32) asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
     // ---- switch: the finished tile's scales leave LDS first (LDS reads the compiler sees wait
     // for every asynchronous copy in flight, so none may follow start_tile), then the next
     // tile's first loads are requested, then this tile is finished ----
@@ -825,6 +937,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     const int n_out = OAI ? p.n / 2 : n_half;
 #pragma unroll
     for (int mf = 0; mf < AM; ++mf) {
+      if (mf >= live_frags) continue;  // (wave-uniform) a fragment without rows of the tile has nothing to store
       float sa = 1.0f;
       if constexpr (I8) sa = sa_r[mf];
       const int r = done.row0 + wave_m * 16 * kMF + mf * kFragRows + li;

@@ -294,8 +294,9 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
     hbm_bound = intensity < peak_tops * 1e12 / (HBM_PEAK_GBS * 1e9)
     g1_s = stage_ms["gemm1"] * 1e-3
     # the launch(es) noted under the first "[gate_up, ...]" heading (two when the device decides between tile shapes)
-    heads = [i for i, line in enumerate(traced) if line.startswith("[")]
-    g1_kernel = " | ".join(traced[heads[0] + 1: heads[1]]) if len(heads) > 1 else "?"
+    heads = [i for i, line in enumerate(traced) if line.startswith("[")] + [len(traced)]
+    first = next((n for n, i in enumerate(heads[:-1]) if traced[i].startswith("[gate_up, routed")), None)
+    g1_kernel = " | ".join(traced[heads[first] + 1: heads[first + 1]]) if first is not None else "?"
     traffic = None if (a.tokens or a.dims) else measured_traffic(workload)  # the counter summaries are of the named workload
     if hbm_bound:
         achieved = work["g1_bytes"] / g1_s / 1e9

@@ -589,7 +589,7 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
   routed.stream = stream_mode;
   routed.x_count = M;
   if (a->format == KMOE_FMT_INT8 && !stream_mode && a->w_layout == KMOE_W_TILED && a->tile_variant >= 5 &&
-      a->tile_variant <= 17 && (local_pairs(a) + E - 1) / E > 10 && H >= 128 && I >= 128)
+      a->tile_variant <= 22 && (local_pairs(a) + E - 1) / E > 10 && H >= 128 && I >= 128)
     routed.variant = a->tile_variant;
   const int tv = a->tile_variant;
   if (a->format == KMOE_FMT_FP8_BLOCK && a->w_layout == KMOE_W_TILED && (local_pairs(a) + E - 1) / E > 10 &&

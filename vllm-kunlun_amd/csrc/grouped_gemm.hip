@@ -490,7 +490,7 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
   if (a->rows == 0 && !(a->w_tail && a->tail_rows > 0)) return KMOE_OK;
   // Tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5-9, 11-16 force it)
   if (a->w_layout == KMOE_W_TILED && a->k >= 128 &&
-      ((a->variant >= 5 && a->variant <= 9) || (a->variant >= 11 && a->variant <= 17) ||
+      ((a->variant >= 5 && a->variant <= 9) || (a->variant >= 11 && a->variant <= 22) ||
        (a->variant == 0 && ceil_div(expected_rows(a->rows, a->rows_hint), a->E) > kTiledMinRows)))
     return tiled_gemm_i8(a, as_stream(stream));
   KMOE_REQUIRE(a->variant < 5, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: variants 5-12 need tiled weights and k >= 128");

@@ -141,15 +141,16 @@ struct Tile {
 // F16: the outputs, and the rounding of gate and up before SiLU-mul, are IEEE half instead of bf16 (int8 and
 // fp8 operands); with KIND = BF16 the operands are half as well (v_mfma_f32_16x16x32_f16).
 template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false,
-          bool PACE = false, bool F16 = false>
-__global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(const TiledParams p) {
+          bool PACE = false, bool F16 = false, int WN = kWavesT>
+__global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const TiledParams p) {
+  constexpr int kWN = WN;  // waves side by side along the channels
   static_assert(!F16 || KIND != TKind::BF16 || !OAI, "the interleaved activation is a bf16 epilogue");
   static_assert(!OAI || (KIND == TKind::BF16 && !SWIGLU && !M32), "the interleaved activation is a bf16 epilogue");
   constexpr int kMF = MF;
   // 16-byte activation vectors per thread and chunk; an odd MF rounds up: the copies then cover up to 8 rows per
   // wave past the tile's last row (rows of the next tile, or the tile's first row again), which land in buffer
   // rows that no fragment reads
-  constexpr int kNA = (16 * kMF * (kChunk / 16) + kWavesT * kWave - 1) / (kWavesT * kWave);
+  constexpr int kNA = (16 * kMF * (kChunk / 16) + kWN * kWave - 1) / (kWN * kWave);
   static_assert(kNA >= 1 && (M32 ? MF % 2 == 0 : true), "tile height");
   static_assert(MF % 2 == 0 || KIND != TKind::F8, "an odd tile height needs the asynchronous activation path");
   constexpr bool F8 = KIND == TKind::F8;
@@ -162,7 +163,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   constexpr int AN = 16 * NF / kFragRows;        // ... and along the channels
   constexpr int kAccRegs = M32 ? 16 : 4;
   constexpr int kTM = WM * 16 * kMF;             // rows of a tile
-  constexpr int kThreads = WM * kWavesT * kWave;
+  constexpr int kThreads = WM * kWN * kWave;
   static_assert(R == 4 || R == 8, "the chunk buffer parity is static only for R/2 even");
   constexpr int kNF = NF;
   constexpr int NFH = SWIGLU ? kNF / 2 : kNF;
@@ -173,16 +174,16 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   // consecutive rows of one fragment column fall on eight different bank groups). F8 keeps the
   // register path (its row scales travel with the data): two padded buffers.
   constexpr bool ADMA = !F8;
-  constexpr int kStageBytes = ADMA ? WM * kWavesT * kNA * 8 * kChunk : kTM * kPitchT;  // (ADMA: kTM rows, or the copies' 8 kNA per wave)
+  constexpr int kStageBytes = ADMA ? WM * kWN * kNA * 8 * kChunk : kTM * kPitchT;  // (ADMA: kTM rows, or the copies' 8 kNA per wave)
   __shared__ __attribute__((aligned(1024))) int8_t lds_a[ADMA ? kStagesA : 2][kStageBytes];
-  __shared__ __attribute__((aligned(16))) int8_t patch[WM * kWavesT][kFragRows * kPatchPitch];
+  __shared__ __attribute__((aligned(16))) int8_t patch[WM * kWN][kFragRows * kPatchPitch];
   // I8, per tile parity: channel scales (w_max / 127) and row scales (a_max / 127)
-  __shared__ __attribute__((aligned(16))) float sw_lds[I8 ? 2 : 1][I8 ? kWavesT * NF * 16 : 4];
+  __shared__ __attribute__((aligned(16))) float sw_lds[I8 ? 2 : 1][I8 ? kWN * NF * 16 : 4];
   // (a wave's copy of row maxes always writes 64 slots: tiles of fewer rows still get 64)
   __shared__ float sa_lds[I8 ? 2 : 1][I8 ? (kTM + kWave - 1) / kWave * kWave : 4];
   // F8: weight block scales of the tile [parity][wave][fragment][k block], and the row scales
   // of the chunk in each activation buffer
-  __shared__ float wsc_lds[F8 ? 2 : 1][F8 ? kWavesT * NF * kMaxKBlocks : 4];
+  __shared__ float wsc_lds[F8 ? 2 : 1][F8 ? kWN * NF * kMaxKBlocks : 4];
   __shared__ float asc_lds[F8 ? 2 : 1][F8 ? kThreads : 4];  // every thread stores (rows repeat): no branch in the loop
   extern __shared__ int dyn_lds[];
   const int n_exp = p.E + (p.w_tail ? 1 : 0);
@@ -191,8 +192,8 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
 
   const int lane = lane_id();
   const int wave_id = threadIdx.x >> 6;
-  const int wave = WM == 1 ? wave_id : wave_id % kWavesT;  // position along the channels
-  const int wave_m = WM == 1 ? 0 : wave_id / kWavesT;      // position along the rows
+  const int wave = WM == 1 ? wave_id : wave_id % kWN;  // position along the channels
+  const int wave_m = WM == 1 ? 0 : wave_id / kWN;      // position along the rows
   const int li = lane & (kFragRows - 1);  // row (or channel) of a fragment held by this lane
   const int lg = lane / kFragRows;        // 16-byte group of K (16x16: 0..3; 32x32: 0..1)
   const int n_half = SWIGLU ? p.n / 2 : p.n;
@@ -479,10 +480,76 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
 #undef KMOE_FRAG_MFMA4
 #undef KMOE_FRAG_IMMS
   };
+  // The same for tiles whose waves own TWO channel fragments (eight waves along the channels): a statement handles
+  // a pair of row fragments - four MFMAs again, so that the reads of the next pair have as many clocks to arrive -
+  // and the skip works on pairs (a pair with one live fragment is computed whole).
+  auto frag_pair_i8 = [&](const v4i(&w)[kNF], v4i& c0, v4i& c1, v4i& n0, v4i& n1, uint32_t addr, auto p_tag, auto off_own,
+                          int mf) {
+    constexpr int pr = decltype(p_tag)::value;
+    constexpr bool kFirst = pr == 0, kLast = 2 * pr + 2 == kMF;
+    constexpr int kOwn = decltype(off_own)::value, kStep = 16 * kChunk;
+#define KMOE_PAIR_HEAD "s_cmp_lt_i32 %[live], %[n1]\n\ts_cbranch_scc1 3f\n\t"
+#define KMOE_PAIR_OWN "ds_read_b128 %[a0], %[addr] offset:%[o0]\n\tds_read_b128 %[a1], %[addr] offset:%[o1]\n\t"
+#define KMOE_PAIR_NEXT \
+  "ds_read_b128 %[b0], %[addr] offset:%[o2]\n\tds_read_b128 %[b1], %[addr] offset:%[o3]\n\ts_waitcnt lgkmcnt(2)\n\t"
+#define KMOE_PAIR_WAIT "s_waitcnt lgkmcnt(0)\n\t"
+#define KMOE_PAIR_MFMA                                          \
+  "v_mfma_i32_16x16x64_i8 %[c00], %[w0], %[a0], %[c00]\n\t"     \
+  "v_mfma_i32_16x16x64_i8 %[c01], %[w1], %[a0], %[c01]\n\t"     \
+  "v_mfma_i32_16x16x64_i8 %[c10], %[w0], %[a1], %[c10]\n\t"     \
+  "v_mfma_i32_16x16x64_i8 %[c11], %[w1], %[a1], %[c11]\n\t"
+#define KMOE_PAIR_ACC \
+  [c00] "+v"(acc[mf][0]), [c01] "+v"(acc[mf][1]), [c10] "+v"(acc[mf + 1][0]), [c11] "+v"(acc[mf + 1][1])
+#define KMOE_PAIR_INS                                                                                              \
+  [w0] "v"(w[0]), [w1] "v"(w[1]), [addr] "v"(addr), [live] "s"(live_frags), [n1] "n"(2 * pr + 1), [o0] "n"(kOwn),    \
+      [o1] "n"(kOwn + kStep), [o2] "n"(kOwn + 2 * kStep), [o3] "n"(kOwn + 3 * kStep)
+    if constexpr (kFirst && kLast)
+      asm volatile(KMOE_PAIR_HEAD KMOE_PAIR_OWN KMOE_PAIR_WAIT KMOE_PAIR_MFMA "3:\n\t"
+                   : KMOE_PAIR_ACC, [a0] "=&v"(c0), [a1] "=&v"(c1) : KMOE_PAIR_INS : "scc", "memory");
+    else if constexpr (kFirst)
+      asm volatile(KMOE_PAIR_HEAD KMOE_PAIR_OWN KMOE_PAIR_NEXT KMOE_PAIR_MFMA "3:\n\t"
+                   : KMOE_PAIR_ACC, [a0] "=&v"(c0), [a1] "=&v"(c1), [b0] "=&v"(n0), [b1] "=&v"(n1) : KMOE_PAIR_INS
+                   : "scc", "memory");
+    else if constexpr (kLast)
+      asm volatile(KMOE_PAIR_HEAD KMOE_PAIR_WAIT KMOE_PAIR_MFMA "3:\n\t"
+                   : KMOE_PAIR_ACC : [a0] "v"(c0), [a1] "v"(c1), KMOE_PAIR_INS : "scc", "memory");
+    else
+      asm volatile(KMOE_PAIR_HEAD KMOE_PAIR_NEXT KMOE_PAIR_MFMA "3:\n\t"
+                   : KMOE_PAIR_ACC, [b0] "=&v"(n0), [b1] "=&v"(n1) : [a0] "v"(c0), [a1] "v"(c1), KMOE_PAIR_INS
+                   : "scc", "memory");
+#undef KMOE_PAIR_HEAD
+#undef KMOE_PAIR_OWN
+#undef KMOE_PAIR_NEXT
+#undef KMOE_PAIR_WAIT
+#undef KMOE_PAIR_MFMA
+#undef KMOE_PAIR_ACC
+#undef KMOE_PAIR_INS
+  };
   // keep: std::false_type (every fragment as read), or an int mask (0: the fragments count as zeros)
   auto compute = [&](const v4i(&wcur)[kNF], auto buf_tag, auto j_tag, auto keep) {
     constexpr int buf = decltype(buf_tag)::value, j = decltype(j_tag)::value;
-    if constexpr (ADMA && I8 && !M32) {
+    if constexpr (ADMA && I8 && !M32 && kNF == 2 && kMF % 2 == 0 && kWN == 8) {
+      constexpr bool kFarStages = kStagesA * kStageBytes > 65536;
+      constexpr int kImm = kFarStages ? 0 : buf * kStageBytes;
+      const uint32_t addr = fa[j] + (kFarStages ? buf * kStageBytes : 0);
+      v4i wm[kNF];
+#pragma unroll
+      for (int f = 0; f < kNF; ++f) {
+        if constexpr (std::is_same_v<decltype(keep), int>) wm[f] = wcur[f] & (v4i){keep, keep, keep, keep};
+        else wm[f] = wcur[f];
+      }
+      v4i af[4];
+      auto run = [&](auto self, auto p_tag) {
+        constexpr int pr = decltype(p_tag)::value;
+        if constexpr (2 * pr < kMF) {
+          frag_pair_i8(wm, af[(2 * pr) & 3], af[(2 * pr + 1) & 3], af[(2 * pr + 2) & 3], af[(2 * pr + 3) & 3], addr, p_tag,
+                       std::integral_constant<int, kImm + 2 * pr * 16 * kChunk>{}, 2 * pr);
+          self(self, std::integral_constant<int, pr + 1>{});
+        }
+      };
+      run(run, std::integral_constant<int, 0>{});
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0]), "+v"(af[1]), "+v"(af[2]), "+v"(af[3]));
+    } else if constexpr (ADMA && I8 && !M32) {
       constexpr bool kFarStages = kStagesA * kStageBytes > 65536;
       constexpr int kImm = kFarStages ? 0 : buf * kStageBytes;
       const uint32_t addr = fa[j] + (kFarStages ? buf * kStageBytes : 0);
@@ -580,7 +647,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
   };
   auto col_of = [&](const Tile& t, int f, bool& ok) -> int {
     const int fh = SWIGLU ? f % NFH : f;
-    const int c = (t.nb * kWavesT + wave) * NFH * 16 + fh * 16;
+    const int c = (t.nb * kWN + wave) * NFH * 16 + fh * 16;
     ok = c < n_half;
     return (SWIGLU && f >= NFH) ? n_half + c : c;
   };
@@ -933,7 +1000,7 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
     const int rd_row = lane / kVecPerRow, rd_vec = lane % kVecPerRow;
     const uint32_t patch_rd =
         patch_base + static_cast<uint32_t>((rd_row & (kFragRows - 1)) * kPatchPitch + rd_vec * 16);
-    const int out_col0 = (done.nb * kWavesT + wave) * NFH * 16 / (OAI ? 2 : 1);  // first output channel of this wave
+    const int out_col0 = (done.nb * kWN + wave) * NFH * 16 / (OAI ? 2 : 1);  // first output channel of this wave
     const int n_out = OAI ? p.n / 2 : n_half;
 #pragma unroll
     for (int mf = 0; mf < AM; ++mf) {
@@ -1028,13 +1095,13 @@ __global__ __launch_bounds__(WM * kWavesT * kWave, WGS) void tiled_gemm_kernel(c
 }
 
 template <TKind KIND, bool SWIGLU, int NF, int R, int WGS, int WM, bool M32 = false, int MF = 8, bool OAI = false,
-          bool PACE = false, bool F16 = false>
+          bool PACE = false, bool F16 = false, int WN = kWavesT>
 int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* what) {
   constexpr int kTM = WM * 16 * MF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int nfh = SWIGLU ? NF / 2 : NF;
   const int n_exp = p.E + (p.w_tail ? 1 : 0);
-  p.n_blocks = ceil_div(n_half, kWavesT * nfh * 16);
+  p.n_blocks = ceil_div(n_half, WN * nfh * 16);
   const int max_tiles = (rows + p.tail_rows) / kTM + min(n_exp, rows + p.tail_rows);
   p.max_items = p.n_blocks * max_tiles;
   // persistent workgroups: WGS per CU
@@ -1044,12 +1111,12 @@ int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* w
     note_kernel("tiled_gemm_kernel<%s%s, %s, %dx%d tile, %d waves, %d per CU%s%s%s>%s",
                 KIND == TKind::I8 ? "int8" : (KIND == TKind::F8 ? "fp8" : (F16 ? "f16" : "bf16")),
                 (KIND != TKind::BF16 && F16) ? " -> f16" : "", SWIGLU ? "SiLU-mul" : (OAI ? "swigluoai" : "plain"), kTM,
-                kWavesT * nfh * 16 * (SWIGLU ? 2 : 1), WM * kWavesT, WGS, M32 ? ", 32x32 MFMA" : "",
+                WN * nfh * 16 * (SWIGLU ? 2 : 1), WM * WN, WGS, M32 ? ", 32x32 MFMA" : "",
                 PACE ? ", paced siblings" : "", R != 4 ? ", 8-slot weight ring" : "",
                 p.pick == 1 ? " [works if few experts overflow the tile, decided on the device]"
                             : (p.pick == 2 ? " [works otherwise]" : ""));
-  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32, MF, OAI, PACE, F16>), dim3(grid),
-                     dim3(WM * kWavesT * kWave), dyn, s, p);
+  hipLaunchKernelGGL((tiled_gemm_kernel<KIND, SWIGLU, NF, R, WGS, WM, M32, MF, OAI, PACE, F16, WN>), dim3(grid),
+                     dim3(WM * WN * kWave), dyn, s, p);
   return check_launch(what);
 }
 
@@ -1076,6 +1143,19 @@ int tiled_common(const TiledParams& p, int rows, int* n_cu_out, const char* what
   return KMOE_OK;
 }
 
+// One 8-wave tile of 16 MF rows per workgroup with the eight waves side by side along the channels (32 channels
+// each, all rows): no two waves ask for the same weight bytes, and seven MFMA steps of them are on their way per
+// wave (8-slot ring of two fragments) - 112 KB of distinct weight bytes in flight per CU against 48 KB with two
+// rows of four waves, at twice the LDS fragment reads per MFMA.
+template <TKind K, int MF>
+int launch_wide(TiledParams& p, int rows, hipStream_t s, int n_cu, const char* what, bool swiglu, bool f16) {
+  if (f16)
+    return swiglu ? launch_tiled<K, true, 2, 8, 1, 1, false, MF, false, false, true, 8>(p, rows, s, n_cu, what)
+                  : launch_tiled<K, false, 2, 8, 1, 1, false, MF, false, false, true, 8>(p, rows, s, n_cu, what);
+  return swiglu ? launch_tiled<K, true, 2, 8, 1, 1, false, MF, false, false, false, 8>(p, rows, s, n_cu, what)
+                : launch_tiled<K, false, 2, 8, 1, 1, false, MF, false, false, false, 8>(p, rows, s, n_cu, what);
+}
+
 // 8-wave tiles of 32 MF rows, one workgroup per CU.
 template <TKind K, int MF>
 int launch_tall(TiledParams& p, int rows, hipStream_t s, int n_cu, const char* what, bool swiglu, bool f16) {
@@ -1097,7 +1177,7 @@ int launch_tall(TiledParams& p, int rows, hipStream_t s, int n_cu, const char* w
 // Variant 6 (and 12) forces 128 rows, 11 forces 64, 13 forces 96.
 bool short_tiles(int variant, int rows, int n_experts, int n, bool swiglu, int n_cu, int max_avg_rows = 44) {
   if (variant == 11) return true;
-  if (variant == 6 || variant == 8 || (variant >= 12 && variant <= 17)) return false;
+  if (variant == 6 || variant == 8 || (variant >= 12 && variant <= 22)) return false;
   if (ceil_div(rows, n_experts) <= max_avg_rows) return true;
   const int n_blocks = ceil_div(swiglu ? n / 2 : n, kWavesT * (swiglu ? 2 : 4) * 16);
   return static_cast<long long>(rows / 128 + n_experts) * n_blocks < 2ll * n_cu;
@@ -1136,54 +1216,62 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   // 0.158 ms, 1024 tokens 0.191 -> 0.165 ms; at 80 rows per expert too many experts need a second tile: -4 % on
   // the Qwen3 shape, +1 % on the DeepSeek-V3 one; DeepSeek-V3 shape at 64 rows per expert: -1.6 %).
   const bool mid = a->variant == 13 || (a->variant == 0 && !shorter && avg_rows <= 72);
-  // One 8-wave tile per expert (WM = 2: 160, 192, 224 or 256 rows, one workgroup per CU) where experts hold a
-  // little more than one 128-row tile and the launch's weights are far more than the memory-side cache holds: the
-  // shortest such tile that nearly every expert fits (average + 3 sqrt(average) rows of a routed expert). The second 128-row tile of
-  // an expert is mostly padding and streams the expert's weights again; one taller tile does neither, which is
-  // worth more than what the lone workgroup loses by having nothing to run under its epilogue (DeepSeek-V3
-  // shape, gate_up / down, paced 128-row tiles against the tall tile: 120 rows per expert 1724 against 1598 us,
-  // 128 rows 1996 / 977 against 1743 / 866, 144 rows 2105 / 1167 against 1689 / 868, 176 rows 2171 / 1196 against
-  // 1830 / 953, 224 rows 2404 against 2172; at 96 rows 1457 against 1619: the 128-row tile holds them all). Inside
-  // the layer, where gate_up gathers its rows from the few token rows and the shared expert's rows ride along as
-  // the tail expert, less of it is left: DeepSeek-V3 layer at 4096 tokens 3.07 -> 2.97 ms, at 4608 tokens 3.31 ->
-  // 3.09, at 3584 and 5120 tokens -1 and -2 %, from 6144 tokens on the same. With weights that fit the cache the
-  // second pass is cheap and the gain is within noise (Qwen3 shape, 128 rows per expert: 125 against 122 us),
-  // while an expert that overflows the tall tile costs a quarter there: not used.
-  // That holds while the routing is even. The host knows the average only, so the choice is left to the device:
-  // the tall launch is followed by the launch this function would have made without it, and each of the two
-  // reads the row counts in its prologue and leaves if the other is due - the tall one runs if at most one routed
-  // expert in 16 overflows its tile (same layer, +0.5 on the logits of 32 experts, i.e. 30 experts past 192 rows:
-  // tall tiles 3.11 ms, paced 128-row tiles 2.95 ms; +1.0: 3.30 against 3.02). The launch that leaves costs a few
-  // microseconds. Variant 17: the same pair whatever the size of the weights.
-  int tall = a->variant == 8 ? 8 : (a->variant == 14 ? 6 : (a->variant == 15 ? 5 : (a->variant == 16 ? 7 : 0)));
-  const bool by_rule = (a->variant == 0 && !shorter && weight_bytes > (1ll << 30)) || a->variant == 17;
-  if (by_rule) {
-    // (the routed experts' average: a tail expert's many rows say nothing about how full their tiles are - with
-    // it in the average, 96 rows per routed expert took the 160-row tile and lost a fifth, 1526 -> 1841 us)
-    const float avg_routed = static_cast<float>(ceil_div(live, a->E));
-    const float reach = avg_routed + 3.0f * sqrtf(avg_routed);
-    // (from 106 rows per expert: at 104 few experts overflow a 128-row tile yet and the DeepSeek-V3 layer loses
-    // 4 % on the tall tile, at 107 the Kimi-K2 dimensions gain 4 %, at 112 the DeepSeek-V3 layer 1 %)
-    if (avg_routed >= 106.0f && reach <= 256.0f) tall = reach <= 160.0f ? 5 : (reach <= 192.0f ? 6 : (reach <= 224.0f ? 7 : 8));
+  // Wide tiles: 128, 192 or 256 rows x 256 channels on EIGHT waves side by side along the channels (32 channels
+  // each, all the tile's rows), one workgroup per CU. No two waves of a workgroup ask for the same weight bytes,
+  // seven MFMA steps of them are on their way per wave (112 KB of distinct weight bytes in flight per CU, where two
+  // workgroups of four waves hold 96 KB of which the co-resident tiles of one expert duplicate a part), a weight
+  // fragment feeds up to 16 MFMAs, and a tile that holds an expert whole streams the expert's weights once. Row
+  // fragments past an expert's end cost nothing (see frag_pair_i8), so the height only has to be tall enough.
+  // Measured inside the layer against the 4-wave tiles above (two per CU; ms per layer call, same box):
+  //   DeepSeek-V3 dims, tokens 1024 / 2048 / 4096 / 6144 / 8192: before 2.105 / 2.277 / 2.833 / 3.753 / 4.634
+  //     128-row wide 2.045 / 2.186 / - / - / -; 192-row 2.083 / 2.233 / 2.639 / 3.957 / 5.285;
+  //     256-row - / - / - / 3.426 / 4.862 (one 192-row two-wave-row tile per expert at 4096 tokens was the 2.833);
+  //   Kimi-K2 dims at 4096 tokens (85 rows per expert): 3.703 -> 128-row 3.548, 192-row 3.518;
+  //   Qwen3 dims, tokens 1024 / 2048 / 4096 / 8192: before 0.164 / 0.240 / 0.329 / 0.557,
+  //     128-row 0.169 / 0.234 / 0.326 / 0.566, 192-row 0.174 / 0.208 / 0.337 / 0.504, 256-row 0.206 / 0.241 / 0.367 / 0.578.
+  // So: where nearly every expert fits ONE tile of at most 256 rows (average + 3 sqrt(average) rows of a routed
+  // expert), the shortest such tile. Where experts need several tiles: with weights that the memory-side cache
+  // serves (up to 1 GiB) 192-row tiles from 300 rows per expert on, 128-row ones below; with weights beyond that the
+  // paced 4-wave tiles above stay (their m-tiles share the weight bytes in L2; the wide tiles are not paced).
+  // The rule knows the AVERAGE; a skewed routing decides on the device (weights beyond 1 GiB, where an expert that
+  // overflows its tile streams its weights from HBM a second time): the wide launch is followed by the paced
+  // 128-row one, and each of the two reads the row counts in its prologue and leaves if the other is due - the
+  // wide one runs while at most one routed expert in 16 overflows its tile. Variant 17: that pair whatever the
+  // size of the weights; 19 / 18 / 22 (and 15 / 14 / 8, 16): 128- / 192- / 256-row wide tiles forced.
+  const float avg_routed = static_cast<float>(ceil_div(live, a->E));
+  const float reach = avg_routed + 3.0f * sqrtf(avg_routed);
+  const bool big = weight_bytes > (1ll << 30);
+  int wide = 0;  // row fragments of the wide tile (8: 128 rows, 12: 192, 16: 256), 0: none
+  bool pair = false;
+  switch (a->variant) {
+    case 15: case 19: wide = 8; break;
+    case 14: case 18: wide = 12; break;
+    case 8: case 16: case 22: wide = 16; break;
+    default: break;
   }
-  if (tall) {
-    const bool f16 = a->act_dtype == KMOE_DT_F16;
-    p.pick = by_rule ? 1 : 0;
-    p.pick_rows = 32 * tall;
-    int rc;
-    switch (tall) {
-      case 5: rc = launch_tall<K, 5>(p, a->rows, s, n_cu, what, swiglu, f16); break;
-      case 6: rc = launch_tall<K, 6>(p, a->rows, s, n_cu, what, swiglu, f16); break;
-      case 7: rc = launch_tall<K, 7>(p, a->rows, s, n_cu, what, swiglu, f16); break;
-      default: rc = launch_tall<K, 8>(p, a->rows, s, n_cu, what, swiglu, f16); break;
+  if ((a->variant == 0 && !shorter && (big || avg_rows > 72)) || a->variant == 17) {
+    // (small weights keep the 96-row tiles up to 72 rows per expert: Qwen3 dims at 1024 tokens 0.164 against 0.169)
+    if (reach <= 256.0f) {
+      wide = reach <= 128.0f ? 8 : (reach <= 192.0f ? 12 : 16);
+      pair = big || a->variant == 17;
+    } else if (!big && a->variant == 0) {
+      wide = avg_routed > 300.0f ? 12 : 8;
     }
-    if (!by_rule || rc != KMOE_OK) return rc;
-    p.pick = 2;  // the launch below works if the tall one left
+  }
+  if (wide) {
+    const bool f16 = a->act_dtype == KMOE_DT_F16;
+    p.pick = pair ? 1 : 0;
+    p.pick_rows = 16 * wide;
+    const int rc = wide == 8 ? launch_wide<K, 8>(p, a->rows, s, n_cu, what, swiglu, f16)
+                             : (wide == 12 ? launch_wide<K, 12>(p, a->rows, s, n_cu, what, swiglu, f16)
+                                           : launch_wide<K, 16>(p, a->rows, s, n_cu, what, swiglu, f16));
+    if (!pair || rc != KMOE_OK) return rc;
+    p.pick = 2;  // the launch below works if the wide one left
   }
   if (a->act_dtype == KMOE_DT_F16) {
     // half outputs: the shapes in use (64-, 96-, 128-row and paced 128-row tiles); the tuning variants are bf16 only
     KMOE_REQUIRE(a->variant == 0 || a->variant == 5 || a->variant == 6 || (a->variant >= 11 && a->variant <= 13) ||
-                     a->variant == 17,
+                     a->variant == 17 || wide,
                  KMOE_ERR_UNSUPPORTED, "%s: variant %d is not instantiated for half outputs", what, a->variant);
     if (mid)
       return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 6, false, false, true>(p, a->rows, s, n_cu, what)

@@ -262,10 +262,11 @@ typedef struct kmoe_gemm_i8_args {
                              kernels; with tiled weights 5 = tile kernel (6: 128-row tiles, 11: 64-row
                              tiles, 13: 96-row tiles, 7, 9: other tile shapes, 12: 128-row tiles whose m-tiles of
                              one expert and channel block keep in step so that they share the weight bytes in L2;
-                             15, 14, 16, 8: 8-wave tiles of 160, 192, 224, 256 rows, one workgroup per CU; 17: such
-                             a launch and a 128-row-tile launch, of which the row counts decide on the device
-                             which one works (what 0 does for weights beyond 1 GiB); all need k >= 128); with chunked activations 1, 2, 4, 8 = 16-row fragments per pass of the
-                             streaming kernel                                       */
+                             19, 18, 22: wide tiles of 128, 192, 256 rows - eight waves side by side along the
+                             channels, one workgroup per CU (15, 14, 8 and 16 are older names of 19, 18, 22); 17: a
+                             wide-tile launch and a paced 128-row-tile launch, of which the row counts decide on the
+                             device which one works (what 0 does for weights beyond 1 GiB); all need k >= 128); with
+                             chunked activations 1, 2, 4, 8 = 16-row fragments per pass of the streaming kernel */
   int32_t w_layout;       /* KMOE_W_ROWMAJOR, or KMOE_W_TILED (kmoe_tile_weights_i8) */
   int32_t a_layout;       /* KMOE_A_ROWMAJOR, or KMOE_A_CHUNKED: a is [k/64][a_rows][64]
                              (kmoe_quant_i8_rows_chunked); needs w_layout TILED   */
@@ -606,7 +607,7 @@ typedef struct kmoe_moe_args {
   float shared_scale;    /* caller epilogue for half activations (models/deepseek_v2.py:286-292: the routed sum stays
                             unscaled and the shared expert's output is multiplied by 1/routed_scaling_factor):
                             out = dt( dt(routed * out_scale) + dt(shared * shared_scale) ); 0 means 1 */
-  int32_t tile_variant;  /* INT8 and FP8_BLOCK, tuning: 0, or the `variant` (int8: 5-17; fp8: 5, 6, 8, 11-14, 17) handed to
+  int32_t tile_variant;  /* INT8 and FP8_BLOCK, tuning: 0, or the `variant` (int8: 5-22; fp8: 5, 6, 8, 11-14, 17) handed to
                             the two routed GEMMs when the batch runs on the tile kernel (more than 10 rows per
                             expert); ignored otherwise */
   int32_t w_scale_layout; /* W4A16: KMOE_S_* of w13_scale and w2_scale                                  */

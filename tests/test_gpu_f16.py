@@ -74,8 +74,8 @@ def test_half_layer_matches_the_oracle(name, base, over):
 
 
 def test_half_layer_on_8_wave_tiles_gives_the_same_bits():
-    """The 8-wave tiles of the int8 tile kernel (tile_variant 8, 14-16) in their half instantiations: the bits of
-    the default choice, which the cases above compare with the oracle."""
+    """The wide (8-wave) tiles of the int8 tile kernel (tile_variant 19, 18, 22: 128, 192, 256 rows) in their half
+    instantiations: the bits of the default choice, which the cases above compare with the oracle."""
     from vllm_kunlun_amd import _lib as L
     from vllm_kunlun_amd import synth
     from vllm_kunlun_amd._plan import make_moe_plan
@@ -85,7 +85,7 @@ def test_half_layer_on_8_wave_tiles_gives_the_same_bits():
     lay = sl.layer
     x = (sl.x.float() * 1.5).half()
     outs = []
-    for variant in (0, 8, 14, 15, 16, 17):
+    for variant in (0, 6, 19, 18, 22, 17):
         out = torch.empty_like(x)
         plan = make_moe_plan(L.KMOE_FMT_INT8, x, sl.logits, out, shape.K, lay.w13_weight, lay.w2_weight,
                              lay.w13_weight_scale, lay.w2_weight_scale, shape.scoring, True, shape.n_group,

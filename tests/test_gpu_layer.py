@@ -268,8 +268,8 @@ def test_layer_with_the_router_inside(base, over):
 
 def test_layer_with_paced_tiles_gives_the_same_bits():
     """tile_variant = 12 (the m-tiles of one expert and channel block wait for each other so that they share
-    the weight bytes in L2) only changes when workgroups run, and the 8-wave tiles (8, 14-16) only which workgroup
-    computes a row: the output bits are those of the default."""
+    the weight bytes in L2) only changes when workgroups run, and the wide 8-wave tiles (19, 18, 22: 128, 192, 256
+    rows) only which workgroup computes a row: the output bits are those of the 128-row 4-wave tiles (6)."""
     from vllm_kunlun_amd import _lib as L
     from vllm_kunlun_amd import synth
     from vllm_kunlun_amd._plan import make_moe_plan
@@ -279,7 +279,7 @@ def test_layer_with_paced_tiles_gives_the_same_bits():
     sl = synth.make_w8a8_layer(shape, "cuda", seed=12)
     lay = sl.layer
     outs = []
-    for variant in (0, 12, 12, 8, 14, 15, 16, 17):  # 8, 14-16: one 8-wave tile of 256, 192, 160, 224 rows per workgroup
+    for variant in (6, 0, 12, 12, 19, 18, 22, 17):
         out = torch.empty_like(sl.x)
         plan = make_moe_plan(L.KMOE_FMT_INT8, sl.x, sl.logits, out, shape.K, lay.w13_weight, lay.w2_weight,
                              lay.w13_weight_scale, lay.w2_weight_scale, shape.scoring, True, shape.n_group,

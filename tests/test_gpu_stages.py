@@ -545,24 +545,25 @@ PERSISTENT_CASES = TILED_CASES + [
     (4, 128, 576, [70, 0, 129, 5]),
     (2, 64, 704, [33, 200]),
     (8, 4096, 192, [((97 * i) % 300) for i in range(8)]),
-    # experts that end exactly at the last row of a 160-, 192-, 224- or 256-row tile, and one row past it
-    (8, 128, 384, [160, 161, 192, 193, 224, 225, 256, 257]),
-    # variant 17 launches a tall-tile and a 128-row-tile kernel and the row counts decide on the device which of
-    # them works: even counts (the tall one), and counts of which every fourth overflows the tall tile (the other)
+    # experts that end exactly at the last row of a 128-, 192- or 256-row tile, one row before and one row past it,
+    # and experts that leave whole pairs of row fragments of a wide tile without rows
+    (12, 128, 384, [127, 128, 129, 191, 192, 193, 255, 256, 257, 31, 33, 65]),
+    # variant 17 launches a wide-tile and a 128-row-tile kernel and the row counts decide on the device which of
+    # them works: even counts (the wide one), and counts of which every fourth overflows the wide tile (the other)
     (20, 256, 256, [130 + (7 * i) % 25 for i in range(20)]),
     (20, 256, 256, [(260 if i % 4 == 0 else 95) + (7 * i) % 25 for i in range(20)]),
 ]
 
 
 @pytest.mark.parametrize("E,n,k,counts", PERSISTENT_CASES)
-@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 7, 8, 9, 11, 12, 13, 14, 15, 16, 17])
+@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 7, 9, 11, 12, 13, 17, 18, 19, 22])
 @pytest.mark.parametrize("act", [0, 1])
 def test_lds_gemm_i8_with_tiled_weights(L, E, n, k, counts, variant, act):
     """LDS-staged kernels reading tiled weights and row-major activations. Variants 1-3: small
     tiles; 5-7: the persistent 128-row-tile kernel (6: 256-channel tiles, 7: 128-channel tiles
-    with the deep weight ring, 8 / 14 / 15 / 16: 256-, 192-, 160-, 224-row tiles with 8 waves, 17: one of those or
-    128-row tiles, decided on the device, 5: the default,
-    12: sibling m-tiles paced against each other through the progress board)."""
+    with the deep weight ring), 19 / 18 / 22: 128-, 192-, 256-row wide tiles (eight waves side by side along the
+    channels, row fragments without rows skipped pair by pair), 17: a wide tile or 128-row tiles, decided on the
+    device, 5: the default, 12: sibling m-tiles paced against each other through the progress board)."""
     if variant >= 5 and k < 128:
         pytest.skip("the persistent kernel takes k >= 128")
     if variant < 5 and E >= 40:

@@ -43,6 +43,52 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+
+// LDS reads issued from assembly statements, each with its own wait on the LDS counter: an LDS read that the compiler
+// sees makes it wait first for every global load, store and asynchronous copy of the wave (it cannot tell a copy's
+// destination from the address read), which in the tile loop means thousands of clocks.
+__device__ __forceinline__ void lds_read1_b32(float& a, uint32_t addr) {
+  asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(a) : "v"(addr) : "memory");
+}
+template <int STRIDE>
+__device__ __forceinline__ void lds_read4_b32(float& a, float& b, float& c, float& d, uint32_t addr) {
+  asm volatile(
+      "ds_read_b32 %0, %4\n\t"
+      "ds_read_b32 %1, %4 offset:%5\n\t"
+      "ds_read_b32 %2, %4 offset:%6\n\t"
+      "ds_read_b32 %3, %4 offset:%7\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(a), "=&v"(b), "=&v"(c), "=&v"(d)
+      : "v"(addr), "n"(STRIDE), "n"(2 * STRIDE), "n"(3 * STRIDE)
+      : "memory");
+}
+// lds_wait<n> for an n that is a constant only after unrolling (at most 7 younger LDS operations stay in flight)
+template <typename V>
+__device__ __forceinline__ void lds_wait_upto(int n, V& v) {
+  switch (n) {
+    case 0: lds_wait<0>(v); break;
+    case 1: lds_wait<1>(v); break;
+    case 2: lds_wait<2>(v); break;
+    case 3: lds_wait<3>(v); break;
+    case 4: lds_wait<4>(v); break;
+    case 5: lds_wait<5>(v); break;
+    case 6: lds_wait<6>(v); break;
+    default: lds_wait<7>(v); break;
+  }
+}
+__device__ __forceinline__ void lds_read1_b128(v4f& a, uint32_t addr) {
+  asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(a) : "v"(addr) : "memory");
+}
+template <int STRIDE>
+__device__ __forceinline__ void lds_read2_b128(v4f& a, v4f& b, uint32_t addr) {
+  asm volatile(
+      "ds_read_b128 %0, %2\n\t"
+      "ds_read_b128 %1, %2 offset:%3\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(a), "=&v"(b)
+      : "v"(addr), "n"(STRIDE)
+      : "memory");
+}
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
@@ -112,6 +158,7 @@ struct Tile {
   int e;     // expert (E = the tail expert)
   int row0;  // first sorted row
   int nb;    // channel block
+  int end;   // the expert's rows end here
   bool valid;
 };
 
@@ -176,7 +223,11 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
   constexpr bool ADMA = !F8;
   constexpr int kStageBytes = ADMA ? WM * kWN * kNA * 8 * kChunk : kTM * kPitchT;  // (ADMA: kTM rows, or the copies' 8 kNA per wave)
   __shared__ __attribute__((aligned(1024))) int8_t lds_a[ADMA ? kStagesA : 2][kStageBytes];
-  __shared__ __attribute__((aligned(16))) int8_t patch[WM * kWN][kFragRows * kPatchPitch];
+  // (wide tiles with two output fragments a wave: patches for kPatchGroup row fragments, transposed in one LDS round trip)
+  constexpr int kPatchGroup = (!OAI && !M32 && NFH == 2 && WN == 8) ? (MF % 4 == 0 && MF < 16 ? 4 : 2) : 1;
+  static_assert((16 * kMF / kFragRows) % kPatchGroup == 0, "row fragments per patch group");
+  __shared__ __attribute__((aligned(16)))
+  int8_t patch[WM * kWN][(!OAI && !M32 && NFH == 1) ? 16 : kPatchGroup * kFragRows * kPatchPitch];
   // I8, per tile parity: channel scales (w_max / 127) and row scales (a_max / 127)
   __shared__ __attribute__((aligned(16))) float sw_lds[I8 ? 2 : 1][I8 ? kWN * NF * 16 : 4];
   // (a wave's copy of row maxes always writes 64 slots: tiles of fewer rows still get 64)
@@ -252,7 +303,12 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
   // The items of this workgroup are resolved 64 at a time: lane l of wave 0 finds item it0 + l (a binary
   // search over tile_lo and two divisions, all lanes at once) and leaves (expert, first row, channel
   // block) in LDS; the tile loop then reads three words per tile instead of searching.
-  __shared__ int item_e[kWave], item_row0[kWave], item_nb[kWave], item_sib[kWave];
+  __shared__ int items[5][kWave];  // per resolved item: expert, first row, channel block, sibling flag, expert's row end
+  int* const item_e = items[0];
+  int* const item_row0 = items[1];
+  int* const item_nb = items[2];
+  int* const item_sib = items[3];
+  int* const item_end = items[4];
   const int per_xcd = gridDim.x >> 3;  // gridDim.x is a multiple of 8
   // item lid of the list (lid < seg_end) -> expert, first row, channel block, sibling flags
   auto resolve_item = [&](int lid, int& e, int& row0, int& nb, int& sib) {
@@ -280,6 +336,7 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
       const int lid = xcd * seg + (blockIdx.x >> 3) + (it0 + lane) * per_xcd;
       int e = -1, row0 = 0, nb = 0, sib = 0;
       if (lid < seg_end) resolve_item(lid, e, row0, nb, sib);
+      item_end[lane] = e >= 0 ? rows_end(e) : 0;
       item_sib[lane] = sib;
       item_e[lane] = e;
       item_row0[lane] = row0;
@@ -291,13 +348,29 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
   // (called by every wave at the same point of the tile loop: the refill every 64 tiles has a barrier inside)
   auto find_tile = [&](int it) -> Tile {
     if (it > 0 && (it & (kWave - 1)) == 0) resolve_items(it);
-    Tile t{it, 0, 0, 0, 0, false};
+    // The five words of the item come out of LDS through an assembly statement: an LDS read that the compiler sees
+    // makes it wait for every load, store and asynchronous copy of the wave first (it cannot tell the copies'
+    // destinations from this address) - at the loop top that is the epilogue's stores, thousands of clocks.
+    Tile t{it, 0, 0, 0, 0, 0, false};
     const int slot = it & (kWave - 1);
-    t.e = __builtin_amdgcn_readfirstlane(item_e[slot]);
+    const uint32_t base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)&items[0][0])) + 4u * slot;
+    int e, sib, row0, nb, end;
+    asm volatile(
+        "ds_read_b32 %0, %5 offset:%6\n\t"
+        "ds_read_b32 %1, %5 offset:%7\n\t"
+        "ds_read_b32 %2, %5 offset:%8\n\t"
+        "ds_read_b32 %3, %5 offset:%9\n\t"
+        "ds_read_b32 %4, %5 offset:%10\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(e), "=&v"(sib), "=&v"(row0), "=&v"(nb), "=&v"(end)
+        : "v"(base), "n"(0), "n"(4 * kWave * 3), "n"(4 * kWave * 1), "n"(4 * kWave * 2), "n"(4 * kWave * 4)
+        : "memory");
+    t.e = __builtin_amdgcn_readfirstlane(e);
     if (t.e < 0) return t;
-    t.sib = __builtin_amdgcn_readfirstlane(item_sib[slot]);
-    t.row0 = __builtin_amdgcn_readfirstlane(item_row0[slot]);
-    t.nb = __builtin_amdgcn_readfirstlane(item_nb[slot]);
+    t.sib = __builtin_amdgcn_readfirstlane(sib);
+    t.row0 = __builtin_amdgcn_readfirstlane(row0);
+    t.nb = __builtin_amdgcn_readfirstlane(nb);
+    t.end = __builtin_amdgcn_readfirstlane(end);
     t.valid = true;
     return t;
   };
@@ -631,17 +704,18 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
     }
   };
   // Gather index of sorted row r of tile t (rows past the expert's end: the tile's first row),
-  // and the source row (row of p.a / p.a_max) it names.
+  // and the source row (row of p.a / p.a_max) it names. With a gather the value fetched is returned as loaded,
+  // untouched: any arithmetic on it here would make the wave wait for the load - and with it for every older
+  // load and store - at the loop top instead of after the MFMA loop.
   auto fetch_src = [&](const Tile& t, int r) -> int {
-    const int rr = r < rows_end(t.e) ? r : t.row0;
+    const int rr = r < t.end ? r : t.row0;
     if (!p.row_src) return rr;
-    const int g = p.row_src[t.e < p.E ? rr : 0];  // always one load (the tail expert's rows are not gathered)
-    return t.e < p.E ? g : rr;
+    return p.row_src[t.e < p.E ? rr : 0];  // always one load (the tail expert's rows are not gathered: value unused)
   };
   // gather entries are flat (source row, slot) ids: source row = entry / src_div (a shift for the usual powers of two)
   const int src_shift = (p.src_div & (p.src_div - 1)) == 0 ? __builtin_ctz(p.src_div) : -1;
-  auto src_row = [&](const Tile& t, int fetched) -> int {
-    if (t.e >= p.E) return p.tail_src0 + fetched - p.tail_row0;
+  auto src_row = [&](const Tile& t, int r, int fetched) -> int {
+    if (t.e >= p.E) return p.tail_src0 + (r < t.end ? r : t.row0) - p.tail_row0;
     if (!p.row_src) return fetched;
     return src_shift >= 0 ? fetched >> src_shift : fetched / p.src_div;
   };
@@ -759,8 +833,8 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
     }
 #pragma unroll
     for (int i = 0; i < kNA; ++i)
-      aoff[i] = static_cast<uint32_t>(src_row(t, rs[i])) * static_cast<uint32_t>(p.lda) + a_col;  // < 4 GiB: host-checked
-    if constexpr (F8) my_srow = src_row(t, rs_scale);
+      aoff[i] = static_cast<uint32_t>(src_row(t, t.row0 + a_row(i), rs[i])) * static_cast<uint32_t>(p.lda) + a_col;  // < 4 GiB: host-checked
+    if constexpr (F8) my_srow = src_row(t, t.row0 + scale_row, rs_scale);
     load_a(0);
     dma_a(0, 0);
     dma_a(1, 1);
@@ -776,7 +850,8 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
       }
       if (wave_id * kWave < kTM)  // thread r: tile row r
         __builtin_amdgcn_raw_ptr_buffer_load_lds(make_rsrc(p.a_max), (lds_ptr_t)&sa_lds[t_parity][wave_id * kWave], 4,
-                                                 static_cast<uint32_t>(src_row(t, rs_scale)) * 4u, 0, 0, 0);
+                                                 static_cast<uint32_t>(src_row(t, t.row0 + scale_row, rs_scale)) * 4u, 0, 0,
+                                                 0);
     }
     __builtin_amdgcn_sched_barrier(0);  // the weight loads below stay younger than the copies above (see the wait at the loop top)
 #pragma unroll
@@ -810,7 +885,7 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
       patience = kSyncPatience;
     }
     if constexpr (ADMA && I8 && !M32) {
-      const int rows_here = min(rows_end(cur.e), cur.row0 + kTM) - cur.row0 - wave_m * 16 * kMF;
+      const int rows_here = min(cur.end, cur.row0 + kTM) - cur.row0 - wave_m * 16 * kMF;
       live_frags = __builtin_amdgcn_readfirstlane(max(0, min(kMF, (rows_here + 15) >> 4)));
     }
     int rs_next[kNA];
@@ -855,7 +930,16 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
       for (int f = 0; f < AN; ++f)
 #pragma unroll
         for (int q = 0; q < kAccRegs; ++q) acc[mf][f][q] = 0;
-    __syncthreads();
+    // ADMA: everything this wave must publish has been waited for above (the copies by count, the scale writes
+    // by the LDS counter), so a bare barrier is enough; the fence of __syncthreads would also wait for the
+    // weight loads and the epilogue's stores still in flight
+    if constexpr (ADMA) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    } else {
+      __syncthreads();
+    }
 
     // One chunk (two MFMA steps) of the pipeline; h = position of the chunk in the ring
     // period, c0 = first chunk of the period. The fences pin the issue order: loads leave at
@@ -946,18 +1030,33 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
     float sa_r[AM];
     if constexpr (I8) {
 #pragma unroll
-      for (int fr = 0; fr < AN; ++fr)
+      for (int j = 0; j < AN * kQuads; j += 2) {
+        // register quad b of fragment fr, j = fr * kQuads + b: 16x16 fragments lie 64 bytes apart, the quads of a
+        // 32x32 fragment 32 bytes. (LDS reads the compiler does not see: it would wait for every load in flight.)
+        constexpr int kStride = M32 ? 32 : 64;
+        static_assert(M32 ? kFragRows == 32 && kQuads == 4 : kFragRows == 16 && kQuads == 1, "layout of the scale slots");
+        const uint32_t addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+                                  (lds_ptr_t)&sw_lds[parity][wave * kNF * 16 + lg * 4])) + j * kStride;
+        v4f s0, s1 = {0.f, 0.f, 0.f, 0.f};
+        if (j + 1 < AN * kQuads) lds_read2_b128<kStride>(s0, s1, addr);
+        else lds_read1_b128(s0, addr);
 #pragma unroll
-        for (int b = 0; b < kQuads; ++b) {
-          const float4 s4 = *reinterpret_cast<const float4*>(
-              &sw_lds[parity][wave * kNF * 16 + fr * kFragRows + b * 8 + lg * 4]);
-          sw[fr][4 * b + 0] = s4.x;
-          sw[fr][4 * b + 1] = s4.y;
-          sw[fr][4 * b + 2] = s4.z;
-          sw[fr][4 * b + 3] = s4.w;
+        for (int q = 0; q < 4; ++q) {
+          sw[j / kQuads][4 * (j % kQuads) + q] = s0[q];
+          if (j + 1 < AN * kQuads) sw[(j + 1) / kQuads][4 * ((j + 1) % kQuads) + q] = s1[q];
         }
+      }
+      const uint32_t sa_addr = static_cast<uint32_t>(
+          reinterpret_cast<uintptr_t>((lds_ptr_t)&sa_lds[parity][wave_m * 16 * kMF + li]));
 #pragma unroll
-      for (int mf = 0; mf < AM; ++mf) sa_r[mf] = sa_lds[parity][wave_m * 16 * kMF + mf * kFragRows + li];
+      for (int mf = 0; mf < AM; mf += 4) {
+        if (mf + 3 < AM) {
+          lds_read4_b32<4 * kFragRows>(sa_r[mf], sa_r[mf + 1], sa_r[mf + 2], sa_r[mf + 3], sa_addr + mf * 4 * kFragRows);
+        } else {
+#pragma unroll
+          for (int m = mf; m < AM; ++m) lds_read1_b32(sa_r[m], sa_addr + m * 4 * kFragRows);
+        }
+      }
     }
     // BF16 with expert biases: the four bias values of this lane's channels of every fragment, requested
     // before the next tile's loads so that waiting for them does not wait for those
@@ -984,7 +1083,7 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- epilogue of `done`: dequantise, optional SiLU-mul, transpose through LDS, store ----
-    const int row_end = min(rows_end(done.e), done.row0 + kTM);
+    const int row_end = min(done.end, done.row0 + kTM);
     bool wok[kNF];
     int col[kNF];  // per 16-channel block of this wave
 #pragma unroll
@@ -1000,11 +1099,16 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
     const int rd_row = lane / kVecPerRow, rd_vec = lane % kVecPerRow;
     const uint32_t patch_rd =
         patch_base + static_cast<uint32_t>((rd_row & (kFragRows - 1)) * kPatchPitch + rd_vec * 16);
+    constexpr bool kDirectStore = !OAI && !M32 && NFH == 1;
     const int out_col0 = (done.nb * kWN + wave) * NFH * 16 / (OAI ? 2 : 1);  // first output channel of this wave
     const int n_out = OAI ? p.n / 2 : n_half;
 #pragma unroll
-    for (int mf = 0; mf < AM; ++mf) {
-      if (mf >= live_frags) continue;  // (wave-uniform) a fragment without rows of the tile has nothing to store
+    for (int mf0 = 0; mf0 < AM; mf0 += kPatchGroup) {
+      if (mf0 >= live_frags) continue;  // (wave-uniform) fragments without rows of the tile have nothing to store
+#pragma unroll
+      for (int j = 0; j < kPatchGroup; ++j) {
+      const int mf = mf0 + j;
+      if (mf >= live_frags) continue;
       float sa = 1.0f;
       if constexpr (I8) sa = sa_r[mf];
       const int r = done.row0 + wave_m * 16 * kMF + mf * kFragRows + li;
@@ -1045,16 +1149,25 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
             const uint32_t o1 = swigluoai_bf16(f32_to_bf16_hw(yv[2]), f32_to_bf16_hw(yv[3]), p.oai_alpha, p.oai_limit);
             asm volatile("ds_write_b32 %0, %1 offset:%2"
                          :
-                         : "v"(patch_wr_oai), "v"(o0 | (o1 << 16)), "i"(fr * kFragRows)
+                         : "v"(patch_wr_oai), "v"(o0 | (o1 << 16)), "i"(fr * kFragRows + j * kFragRows * kPatchPitch)
                          : "memory");
           } else {
           // channel of yv[0] within the wave's output: fr * kFragRows + b * 8 + lg * 4
           const uint2 packed = F16 ? make_uint2(pack2_half(yv[0], yv[1]), pack2_half(yv[2], yv[3]))
                                    : make_uint2(pack2_bf16(yv[0], yv[1]), pack2_bf16(yv[2], yv[3]));
+          if constexpr (kDirectStore) {
+            // a wave that owns one 16-channel output fragment: the four lanes of a row hold its 32 bytes next to
+            // each other - the transpose through LDS would write the same 32-byte pieces. (Wider waves keep the
+            // transpose: 32-byte pieces where 64 are possible cost the wide down launch 10 % on Qwen3 dims.)
+            const int ocol = out_col0 + lg * 4;
+            if (r < row_end && ocol < n_out)
+              *reinterpret_cast<uint2*>(p.y + static_cast<size_t>(r) * p.ldy + ocol) = packed;
+          } else {
           asm volatile("ds_write_b64 %0, %1 offset:%2"
                        :
-                       : "v"(patch_wr), "v"(packed), "i"((fr * kFragRows + b * 8) * 2)
+                       : "v"(patch_wr), "v"(packed), "i"((fr * kFragRows + b * 8) * 2 + j * kFragRows * kPatchPitch)
                        : "memory");
+          }
           }
           if constexpr (I8) {
             const int f16 = M32 ? 2 * fr + (b >> 1) : fr;
@@ -1072,20 +1185,31 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
           }
         }
       }
+      }
+      if constexpr (kDirectStore) continue;
       __builtin_amdgcn_wave_barrier();  // a wave's LDS operations execute in order: the reads see the writes
+      // every read of the group is requested before the first one is waited for (fragments past the tile's rows
+      // are read as well - whatever the patch holds - and not stored: the waits below count every read)
+      v4i v[kPatchGroup][kReads];
 #pragma unroll
-      for (int h = 0; h < kReads; ++h) {
-        const int pr = h * kRowsPerRead + rd_row;
-        v4i v;  // a wave's LDS operations execute in order: this read sees the writes above
-        asm volatile("ds_read_b128 %0, %1 offset:%2"
-                     : "=v"(v)
-                     : "v"(patch_rd), "i"(kReads > 1 ? h * kRowsPerRead * kPatchPitch : 0)
-                     : "memory");
-        lds_wait<0>(v);
-        const int orow = done.row0 + wave_m * 16 * kMF + mf * kFragRows + pr;
-        const int ocol = out_col0 + rd_vec * 8;
-        if (pr < kFragRows && orow < row_end && ocol < n_out)  // n_out % 8 == 0: a vector of 8 channels is all in or all out
-          *reinterpret_cast<v4i*>(p.y + static_cast<size_t>(orow) * p.ldy + ocol) = v;
+      for (int j = 0; j < kPatchGroup; ++j)
+#pragma unroll
+        for (int h = 0; h < kReads; ++h)
+          asm volatile("ds_read_b128 %0, %1 offset:%2"
+                       : "=v"(v[j][h])
+                       : "v"(patch_rd), "i"((kReads > 1 ? h * kRowsPerRead * kPatchPitch : 0) + j * kFragRows * kPatchPitch)
+                       : "memory");
+#pragma unroll
+      for (int j = 0; j < kPatchGroup; ++j) {
+#pragma unroll
+        for (int h = 0; h < kReads; ++h) {
+          lds_wait_upto(kPatchGroup * kReads - 1 - (j * kReads + h), v[j][h]);
+          const int pr = h * kRowsPerRead + rd_row;
+          const int orow = done.row0 + wave_m * 16 * kMF + (mf0 + j) * kFragRows + pr;
+          const int ocol = out_col0 + rd_vec * 8;
+          if (pr < kFragRows && orow < row_end && ocol < n_out)  // n_out % 8 == 0: a vector of 8 channels is all in or all out
+            *reinterpret_cast<v4i*>(p.y + static_cast<size_t>(orow) * p.ldy + ocol) = v[j][h];
+        }
       }
       __builtin_amdgcn_wave_barrier();
     }

@@ -193,6 +193,53 @@ SUITE = ["dsv3-prefill", "qwen3-decode", "qwen3-prefill", "qwen3-prefill-skew", 
 HEADLINE = "dsv3-decode"
 
 
+def clock_probe(plan, stream, ms_per_step, load_ms=20.0):
+    """Shader clock beside the layer: kmoe_clock_probe runs on a second stream (the library leaves CUs free for
+    it: KMOE_SPARE_CUS, set by main) while the layer is called back to back for about load_ms. Returns the clock
+    by the probe's s_sleep runs (s_memtime ticks / duration by the 100 MHz counter) before the load and during
+    it, and the ticks of its fixed v_fma chain in both phases (equal ticks = s_memtime follows the shader clock)."""
+    import numpy as np
+    import torch
+    from vllm_kunlun_amd import _lib as L
+    n_wg, reps = 16, 4096
+    samples = torch.zeros(n_wg * reps * 3, dtype=torch.int64, device="cuda:0")
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    t_probe = time.perf_counter()
+    L.check(L.lib.kmoe_clock_probe(L.ptr(samples), n_wg, reps, side.cuda_stream))
+    time.sleep(0.004)
+    t_load0 = time.perf_counter() - t_probe
+    with torch.cuda.stream(stream):
+        for _ in range(max(3, int(load_ms / ms_per_step))):
+            plan()
+        stream.synchronize()
+    t_load1 = time.perf_counter() - t_probe
+    torch.cuda.synchronize()
+    r = samples.cpu().numpy().reshape(n_wg, reps, 3).astype(np.float64)
+    t = (r[:, :, 0] - r[:, :, 0].min()) * 1e-8          # seconds since the first sample
+    ghz = r[:, :, 2] / (r[:, :, 1] * 10.0)               # ticks per ns
+    sleep, fma = np.zeros(reps, bool), np.zeros(reps, bool)
+    sleep[1::2], fma[0::2] = True, True
+    # host and device clocks both run in real time: the load's window, a millisecond inside its host-side bounds
+    idle = t < (t_load0 - 1e-3)
+    busy = (t > t_load0 + 1.5e-3) & (t < t_load1 - 1.0e-3)
+
+    def med(mask, col):
+        v = col[mask]
+        return float(np.median(v)) if v.size else None
+    return {
+        "probe": f"{n_wg} single-wave workgroups beside the layer, {reps} runs each; the tile kernels leave "
+                 f"{os.environ.get('KMOE_SPARE_CUS', '0')} CUs free",
+        "idle_ghz": med(idle & sleep[None, :], ghz), "loaded_ghz": med(busy & sleep[None, :], ghz),
+        "loaded_ghz_p10_p90": [float(x) for x in np.percentile(ghz[busy & sleep[None, :]], [10, 90])] if busy.any() else None,
+        "sleep_run_ticks_idle": med(idle & sleep[None, :], r[:, :, 2]), "sleep_run_ticks_loaded": med(busy & sleep[None, :], r[:, :, 2]),
+        "sleep_run_ns_idle": med(idle & sleep[None, :], r[:, :, 1] * 10.0), "sleep_run_ns_loaded": med(busy & sleep[None, :], r[:, :, 1] * 10.0),
+        "fma_chain_ticks_idle": med(idle & fma[None, :], r[:, :, 2]), "fma_chain_ticks_loaded": med(busy & fma[None, :], r[:, :, 2]),
+        "fma_chain_ns_idle": med(idle & fma[None, :], r[:, :, 1] * 10.0), "fma_chain_ns_loaded": med(busy & fma[None, :], r[:, :, 1] * 10.0),
+        "samples_idle": int((idle & sleep[None, :]).sum()), "samples_loaded": int((busy & sleep[None, :]).sum()),
+    }
+
+
 def measure(a, workload, shape, label, sl, with_cpu_baseline):
     """Times one workload's layer on cuda:0 (inputs resident in HBM) and returns the pieces of
     the JSON line: ms per step (graph replay / eager plan / plugin entry), per-stage durations
@@ -271,6 +318,8 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
             kw = sl.apply_kwargs() if shape.quant in ("int8", "fp8") else {}
             launch_ms["apply_monolithic eager"] = timed(lambda: method.apply_monolithic(lay, x, logits, **kw))
 
+        probe = clock_probe(plan, stream, ms_per_step) if a.clock_probe else None
+
         # the same calls again with HIP events around each stage (eager: events are
         # not captured), for the per-kernel durations of the roofline
         ev = HipEvents(2 * len(L.STAGES))
@@ -335,6 +384,8 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
     }
     if a.yardstick and shape.quant in ("int8", "none"):
         res["vendor_dense_gemm"] = vendor_dense_gemm(shape, work["g1_ops"], peak_tops)
+    if probe is not None:
+        res["clock_probe"] = probe
     res["cpu_baseline"] = cpu_baseline(sl, a.cpu_budget) if with_cpu_baseline else None
     return res
 
@@ -380,7 +431,16 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one bitwise_not over 256 MiB (a kernel of known HBM traffic and a name nothing "
                          "else here has) before the timed region: the yardstick for FETCH_SIZE / WRITE_SIZE runs")
+    ap.add_argument("--clock-probe", action="store_true",
+                    help="also run the library's shader-clock probe on a second stream beside the layer and report the "
+                         "clock it sees idle and under the layer ('clock_probe'); sets KMOE_SPARE_CUS=16 so that the "
+                         "persistent tile kernels leave the probe 16 CUs (the layer is a few percent slower for it)")
+    ap.add_argument("--zero-operands", action="store_true",
+                    help="a power experiment: activations and expert weights all zero (same routing, same kernels, same "
+                         "instruction stream, no bit toggles in the data paths); 'data' then says so")
     a = ap.parse_args()
+    if a.clock_probe:
+        os.environ["KMOE_SPARE_CUS"] = "16"  # read by the library at its first tile launch
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures ONE GPU; the layer does not span GPUs (run with --gpus 1)")
 
@@ -427,6 +487,11 @@ def main():
             sl = synth.make_layer(shape, "cuda:0", seed=a.seed,
                                   dtype=torch.float16 if a.act_dtype == "f16" else torch.bfloat16)
         cached = (weights_key(shape), sl)
+        if a.zero_operands:
+            sl.x.zero_()
+            for t in (getattr(sl.layer, n, None) for n in ("w13_weight", "w2_weight", "w13_weight_packed", "w2_weight_packed")):
+                if t is not None:
+                    t.data.zero_()
         results[name] = measure(a, name, shape, label, sl, name == headline and not a.no_cpu_baseline)
         print(f"bench.py: {name}: {results[name]['ms_per_step']:.4f} ms/step", file=sys.stderr, flush=True)
 
@@ -443,14 +508,15 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": head["dtype"],
-        "data": "synthetic",
+        "data": "synthetic, all-zero activations and expert weights (--zero-operands)" if a.zero_operands else "synthetic",
         "config": head["config"],
         "roofline": head["roofline"],
         "layer": head["layer"],
         "cpu_baseline": head["cpu_baseline"],
     }
-    if "vendor_dense_gemm" in head:
-        result["vendor_dense_gemm"] = head["vendor_dense_gemm"]
+    for extra in ("vendor_dense_gemm", "clock_probe"):
+        if extra in head:
+            result[extra] = head[extra]
     if len(results) > 1:
         result["workloads"] = {
             n: {"tokens_per_s": r["value"], "ms_per_step": r["ms_per_step"], "dtype": r["dtype"], "config": r["config"],

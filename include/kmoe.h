@@ -479,6 +479,19 @@ int kmoe_silu_and_mul_dt(const uint16_t* y, int64_t ld_y, int R, int I, uint16_t
 int kmoe_silu_table(float* table, int act_dtype, kmoe_stream_t stream);
 
 /*
+ * Shader-clock probe, a measurement aid with no counterpart in the reference. n_workgroups (1..64) single-wave
+ * workgroups each run `reps` (2..1048576) runs of fixed length in shader clocks - odd runs 8 x s_sleep 127, even
+ * runs a chain of 2048 dependent v_fma_f32 - and write three int64 per run to samples[(workgroup * reps + run) * 3]:
+ * the 100 MHz counter at the start, the run's duration in ticks of that counter (10 ns), and the run's duration in
+ * s_memtime ticks. Launched on a second stream beside a kernel under test: the s_memtime ticks of a run stay the
+ * same whatever runs beside it while its 10-ns duration stretches when the chip lowers the shader clock under load,
+ * so ticks / duration is the clock the kernel under test really gets. The persistent tile kernels occupy every CU;
+ * the environment variable KMOE_SPARE_CUS=n (read once per process) cuts their grids for n fewer CUs, so that the
+ * probe's waves (or a collective's) find a place beside them.
+ */
+int kmoe_clock_probe(int64_t* samples, int n_workgroups, int reps, kmoe_stream_t stream);
+
+/*
  * Un-permute + weighted top-K sum. Replaces kunlun_ops.moe_post
  * (ops/_custom_ops.py:1316-1324, called compressed_tensors_moe.py:278-290).
  *   out[m,h] = bf16( sum_k topk_w[m,k] * dq[m,k] * float(x[moe_index[m*K+k], h]) )

@@ -70,6 +70,8 @@ def test_null_and_shape_errors_are_status_codes(L):
     assert b"NULL" in lib.kmoe_last_error()
     one = C.c_void_p(0x1000)  # never dereferenced: validation fails first
     assert lib.kmoe_softmax_topk(one, 4, 0, 2, 1, one, one, None) == -2
+    assert lib.kmoe_clock_probe(None, 1, 8, None) == -1
+    assert lib.kmoe_clock_probe(one, 0, 8, None) == -2 and lib.kmoe_clock_probe(one, 1, 1, None) == -2
     assert lib.kmoe_softmax_topk(one, 4, 8, 9, 1, one, one, None) == -2          # K > E
     assert lib.kmoe_softmax_topk(one, 4, 2048, 8, 1, one, one, None) == -2       # E too large
     assert lib.kmoe_sigmoid_group_topk_norm(one, None, 4, 30, 4, 4, 2, 1.0, one, one, None) == -2  # E % n_group

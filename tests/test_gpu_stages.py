@@ -379,6 +379,25 @@ def test_silu_and_mul(L, R, I):
     assert np.array_equal(bits(out), ref)
 
 
+def test_clock_probe(L):
+    """kmoe_clock_probe alone on the GPU: every run is stamped; a sleep run (8 x s_sleep 127 = 8 x 64 x 127 shader
+    clocks at least) reports that many s_memtime ticks or a little more, and ticks over duration lands in the range
+    of clocks this part can run at. Size limits are refused."""
+    n_wg, reps = 4, 64
+    samples = torch.zeros(n_wg * reps * 3, dtype=torch.int64, device="cuda")
+    L.check(L.lib.kmoe_clock_probe(L.ptr(samples), n_wg, reps, L.stream()))
+    sync()
+    r = samples.cpu().numpy().reshape(n_wg, reps, 3)
+    assert (r[:, :, 0] > 0).all() and (r[:, :, 1] > 0).all() and (r[:, :, 2] > 0).all()
+    assert (np.diff(r[:, :, 0], axis=1) > 0).all()  # the 100 MHz counter moves on from run to run
+    sleep_ticks, sleep_ns = r[:, 1::2, 2].astype(float), r[:, 1::2, 1].astype(float) * 10.0
+    assert np.median(sleep_ticks) >= 8 * 64 * 127 and np.median(sleep_ticks) < 1.2 * 8 * 64 * 127
+    ghz = np.median(sleep_ticks / sleep_ns)
+    assert 0.5 < ghz < 3.0, ghz
+    assert L.lib.kmoe_clock_probe(L.ptr(samples), 65, reps, L.stream()) == -2  # KMOE_ERR_SHAPE
+    assert L.lib.kmoe_clock_probe(None, 1, reps, L.stream()) == -1  # KMOE_ERR_NULL
+
+
 @pytest.mark.parametrize("f16", [False, True], ids=["bf16", "f16"])
 def test_device_silu_table(L, f16):
     """kmoe_silu_table: the device's SiLU of all 65536 16-bit arguments. Against float64 g / (1 + exp(-g)) within

@@ -30,6 +30,7 @@
 // the waits on the copies are explicit s_waitcnt vmcnt(N): a wave's loads complete in issue
 // order, so "at most N in flight" means "everything older than the N youngest has landed". Each
 // N below is the number of loads the wave is known to have issued after the copies it needs.
+#include <cstdlib>
 #include <type_traits>
 
 #include "buffer_ops.h"
@@ -1262,6 +1263,12 @@ int tiled_common(const TiledParams& p, int rows, int* n_cu_out, const char* what
     if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
       return fail(KMOE_ERR_LAUNCH, "%s: cannot query the device", what);
     n_cu = prop.multiProcessorCount;
+    // KMOE_SPARE_CUS=n (read once): the persistent grids are cut for n fewer CUs, which stay free for a kernel that
+    // runs beside these launches on another stream (a collective; the clock probe). Multiples of 8 keep the XCDs even.
+    if (const char* spare = getenv("KMOE_SPARE_CUS")) {
+      const int n = atoi(spare);
+      if (n > 0 && n < n_cu) n_cu -= n;
+    }
   }
   *n_cu_out = n_cu;
   return KMOE_OK;

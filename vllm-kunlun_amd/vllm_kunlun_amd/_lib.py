@@ -118,6 +118,7 @@ def _load() -> C.CDLL:
         "kmoe_version": (C.c_char_p, []),
         "kmoe_trace_kernels": (None, [i32]),
         "kmoe_silu_table": (i32, [vp, i32, vp]),
+        "kmoe_clock_probe": (i32, [vp, i32, i32, vp]),
         "kmoe_traced_kernels": (C.c_char_p, []),
         "kmoe_softmax_topk": (i32, [vp, i32, i32, i32, i32, vp, vp, vp]),
         "kmoe_sigmoid_group_topk_norm": (i32, [vp, vp, i32, i32, i32, i32, i32, f32, vp, vp, vp]),
@@ -171,7 +172,7 @@ EXPORTS = (
     "kmoe_swigluoai_and_mul", "kmoe_dequant_w4_bf16", "kmoe_dequant_w4", "kmoe_moe_forward_static",
     "kmoe_quant_i8_static", "kmoe_quant_i8_rows_azp", "kmoe_tile_scales_w4", "kmoe_scaled_mm_azp_epilogue", "kmoe_align_local",
     "kmoe_quant_i8_rows_dt", "kmoe_quant_i8_rows_chunked_dt", "kmoe_silu_and_mul_dt", "kmoe_combine_dt", "kmoe_router_gemm",
-    "kmoe_trace_kernels", "kmoe_traced_kernels", "kmoe_silu_table",
+    "kmoe_trace_kernels", "kmoe_traced_kernels", "kmoe_silu_table", "kmoe_clock_probe",
 )
 STATIC_WORKSPACE_BYTES = 64 << 20
 KMOE_FLAG_SIDE_STREAM = 1

@@ -136,6 +136,11 @@ struct TiledParams {
   // routed experts overflow them (at most one in 16). pick = 1: this launch runs if they do, pick = 2: if not;
   // 0: it always runs.
   int32_t pick, pick_rows;
+  // Order of an expert's items. 0: channel block by channel block, the m-tiles of one block next to each other (they
+  // read the same weight bytes at the same time; the paced kernels need it). 1: m-tile by m-tile, the channel blocks
+  // of one m-tile next to each other (they read the same rows at the same time) - for experts whose weights stay in an
+  // XCD's L2 anyway, where an expert with many m-tiles would otherwise fetch its rows once per channel block.
+  int32_t m_major;
 };
 
 // Progress board of the persistent workgroups: slot b (64 bytes apart) holds where workgroup b is,
@@ -324,8 +329,14 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
     e = lo;
     const int first = tile_lo[e], mt = tile_lo[e + 1] - first;
     const int u = lid - first * p.n_blocks;
-    nb = u / mt;
-    const int m = u - nb * mt;
+    int m;
+    if (p.m_major) {
+      m = u / p.n_blocks;
+      nb = u - m * p.n_blocks;
+    } else {
+      nb = u / mt;
+      m = u - nb * mt;
+    }
     row0 = rows_begin(e) + m * kTM;
     // siblings run on the workgroups before / after this one in the XCD, at the same list position
     const int j = blockIdx.x >> 3;
@@ -1229,6 +1240,7 @@ int launch_tiled(TiledParams p, int rows, hipStream_t s, int n_cu, const char* w
   p.n_blocks = ceil_div(n_half, WN * nfh * 16);
   const int max_tiles = (rows + p.tail_rows) / kTM + min(n_exp, rows + p.tail_rows);
   p.max_items = p.n_blocks * max_tiles;
+  if (PACE) p.m_major = 0;  // paced siblings are neighbours in the list
   // persistent workgroups: WGS per CU
   const int grid = min(min(ceil_div(p.max_items, 8) * 8, ceil_div(WGS * n_cu, 8) * 8), kBoardSlots);
   const size_t dyn = sizeof(int) * (static_cast<size_t>(p.E) + 1 + n_exp + 2);
@@ -1369,6 +1381,8 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   // 128-row one, and each of the two reads the row counts in its prologue and leaves if the other is due - the
   // wide one runs while at most one routed expert in 16 overflows its tile. Variant 17: that pair whatever the
   // size of the weights; 19 / 18 / 22 (and 15 / 14 / 8, 16): 128- / 192- / 256-row wide tiles forced.
+  // (an expert of up to 3 MiB stays in an XCD's 4 MB L2 while its m-tiles run: their channel blocks go side by side)
+  p.m_major = static_cast<long long>(a->n) * a->k <= (3ll << 20) ? 1 : 0;
   const float avg_routed = static_cast<float>(ceil_div(live, a->E));
   const float reach = avg_routed + 3.0f * sqrtf(avg_routed);
   const bool big = weight_bytes > (1ll << 30);

@@ -571,6 +571,9 @@ PERSISTENT_CASES = TILED_CASES + [
     # them works: even counts (the wide one), and counts of which every fourth overflows the wide tile (the other)
     (20, 256, 256, [130 + (7 * i) % 25 for i in range(20)]),
     (20, 256, 256, [(260 if i % 4 == 0 else 95) + (7 * i) % 25 for i in range(20)]),
+    # experts of more than 3 MiB of weights list their items channel block by channel block, smaller ones (every
+    # case above) m-tile by m-tile: several m-tiles and channel blocks per expert in the first order
+    (2, 2048, 2048, [300, 140]),
 ]
 
 
@@ -588,3 +591,44 @@ def test_lds_gemm_i8_with_tiled_weights(L, E, n, k, counts, variant, act):
     if variant < 5 and E >= 40:
         pytest.skip("large case: persistent kernel only")
     _gemm_layout_case(L, E, n, k, counts, act, variant, True, chunked=False, seed=E * n + k + 7)
+
+
+def test_spare_cus_keeps_the_bits(L):
+    """KMOE_SPARE_CUS (read once per process, hence a child process): the persistent tile kernels sized for half
+    the CUs walk the same items in another distribution and must produce the same bits."""
+    import os
+    import subprocess
+    import sys
+    code = r"""
+import sys, zlib
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[2])
+import numpy as np, torch, ctypes
+from vllm_kunlun_amd import _lib as L
+rng = np.random.default_rng(5)
+E, n, k, counts = 6, 512, 1024, [130, 0, 190, 17, 300, 64]
+lod = torch.tensor(np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)).cuda(); P = int(sum(counts))
+w = torch.tensor(rng.integers(-127, 128, (E, n, k), dtype=np.int8)).cuda(); wt = torch.empty_like(w)
+L.check(L.lib.kmoe_tile_weights_i8(w.data_ptr(), wt.data_ptr(), E, n, k, L.stream()))
+wmax = torch.tensor((rng.random((E, n)) + 0.1).astype(np.float32)).cuda()
+a = torch.tensor(rng.integers(-127, 128, (P, k), dtype=np.int8)).cuda()
+amax = torch.tensor((rng.random(P) + 0.1).astype(np.float32)).cuda()
+for variant in (18, 6, 12):
+    y = torch.zeros(P, n // 2, dtype=torch.bfloat16, device="cuda")
+    g = L.GemmI8Args()
+    g.a, g.lda, g.a_max, g.src_div = a.data_ptr(), k, amax.data_ptr(), 1
+    g.w, g.w_max, g.lod = wt.data_ptr(), wmax.data_ptr(), lod.data_ptr()
+    g.E, g.n, g.k, g.rows = E, n, k, P
+    g.y, g.ldy, g.act, g.variant, g.w_layout = y.data_ptr(), n // 2, 1, variant, 1
+    L.check(L.lib.kmoe_grouped_gemm_i8(ctypes.byref(g), L.stream()))
+    torch.cuda.synchronize()
+    print(variant, zlib.crc32(y.cpu().view(torch.int16).numpy().tobytes()))
+"""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    sums = []
+    for spare in ("0", "128"):
+        env = dict(os.environ, KMOE_SPARE_CUS=spare)
+        out = subprocess.run([sys.executable, "-c", code, root, os.path.join(root, "vllm-kunlun_amd")], env=env,
+                             capture_output=True, text=True, timeout=110)
+        assert out.returncode == 0, out.stderr[-2000:]
+        sums.append(out.stdout.split())
+    assert len(sums[0]) == 6 and sums[0] == sums[1], sums

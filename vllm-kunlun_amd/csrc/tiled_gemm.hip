@@ -1,10 +1,12 @@
 // Grouped GEMM for the prefill regime (hundreds of rows per expert) on MFMA, tiled weights;
 // int8 (v_mfma_i32_16x16x64_i8), fp8 block-scaled and bf16 operands.
 //
-// Workgroup = 4 waves on a 128-row x 256-channel tile; each wave owns 64 channels
-// of all 128 rows: 8 x 4 accumulator fragments = 128 registers. Two workgroups
-// share a CU (2 waves per SIMD): one workgroup's waits, barriers and its
-// VALU-heavy epilogue (dequant, exp, divide) run under the other's MFMAs.
+// Two workgroup shapes. Four waves on a 128-row x 256-channel tile (64-, 96-row forms for few rows per
+// expert), each wave owning 64 channels of all the rows (8 x 4 accumulator fragments = 128 registers), two
+// workgroups per CU: one workgroup's waits, barriers and VALU-heavy epilogue run under the other's MFMAs.
+// And, int8 with more than 72 rows per expert: EIGHT waves side by side along the channels (WN = 8) on a
+// 128-, 192- or 256-row x 256-channel tile, each wave owning 32 channels of all the rows, one workgroup
+// per CU, a deeper weight ring, and row fragments past an expert's last row skipped (see tiled_gemm_i8).
 //   activations: int8 / bf16: asynchronous copies global -> LDS (rows gathered through the
 //                sort), 128 bytes of K per row and chunk, three chunks ahead into a ring of
 //                four chunk buffers, swizzled so that fragment reads are conflict-free without

@@ -166,7 +166,7 @@ struct Tile {
   int e;     // expert (E = the tail expert)
   int row0;  // first sorted row
   int nb;    // channel block
-  int end;   // the expert's rows end here
+  int end;   // the tile's rows end here (its share of the expert's rows)
   bool valid;
 };
 
@@ -311,7 +311,7 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
   // The items of this workgroup are resolved 64 at a time: lane l of wave 0 finds item it0 + l (a binary
   // search over tile_lo and two divisions, all lanes at once) and leaves (expert, first row, channel
   // block) in LDS; the tile loop then reads three words per tile instead of searching.
-  __shared__ int items[5][kWave];  // per resolved item: expert, first row, channel block, sibling flag, expert's row end
+  __shared__ int items[5][kWave];  // per resolved item: expert, first row, channel block, sibling flag, the tile's row end
   int* const item_e = items[0];
   int* const item_row0 = items[1];
   int* const item_nb = items[2];
@@ -319,7 +319,7 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
   int* const item_end = items[4];
   const int per_xcd = gridDim.x >> 3;  // gridDim.x is a multiple of 8
   // item lid of the list (lid < seg_end) -> expert, first row, channel block, sibling flags
-  auto resolve_item = [&](int lid, int& e, int& row0, int& nb, int& sib) {
+  auto resolve_item = [&](int lid, int& e, int& row0, int& nb, int& sib, int& end) {
     const int m_tile = lid / p.n_blocks;
     // the last e with tile_lo[e] <= m_tile: of a run of equal entries (empty experts) the one that owns the tile
     int lo = 0, hi = n_exp - 1;
@@ -339,7 +339,15 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
       nb = u / mt;
       m = u - nb * mt;
     }
-    row0 = rows_begin(e) + m * kTM;
+    // An expert's rows are split EVENLY over its m-tiles (whole 16-row fragments): kernels that skip the row
+    // fragments past a tile's end then spend about the same time on each of them, so the m-tiles of one channel
+    // block, which start together on neighbouring workgroups, stay in step and share the weight bytes in L2 - a
+    // full tile next to a nearly empty one would fetch them twice. (Experts with more m-tiles than a tile has
+    // fragments keep full tiles: the rounding could leave a trailing tile without rows.)
+    const int rows_e = rows_end(e) - rows_begin(e);
+    const int stride = mt <= kTM / 16 ? (((rows_e + mt - 1) / mt + 15) & ~15) : kTM;
+    row0 = rows_begin(e) + m * stride;
+    end = min(rows_end(e), row0 + stride);
     // siblings run on the workgroups before / after this one in the XCD, at the same list position
     const int j = blockIdx.x >> 3;
     if (m > 0 && j > 0) sib |= 1;
@@ -348,9 +356,9 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
   auto resolve_items = [&](int it0) {
     if (wave_id == 0) {
       const int lid = xcd * seg + (blockIdx.x >> 3) + (it0 + lane) * per_xcd;
-      int e = -1, row0 = 0, nb = 0, sib = 0;
-      if (lid < seg_end) resolve_item(lid, e, row0, nb, sib);
-      item_end[lane] = e >= 0 ? rows_end(e) : 0;
+      int e = -1, row0 = 0, nb = 0, sib = 0, end = 0;
+      if (lid < seg_end) resolve_item(lid, e, row0, nb, sib, end);
+      item_end[lane] = end;
       item_sib[lane] = sib;
       item_e[lane] = e;
       item_row0[lane] = row0;
@@ -1345,17 +1353,14 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   const int live = expected_rows(a->rows, a->rows_hint);  // (chooses the tile shape; grids and bounds keep a->rows)
   const int avg_rows = ceil_div(live + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
   const bool shorter = short_tiles(a->variant, live, a->E, a->n, swiglu, n_cu);
-  // 128-row tiles whose sibling m-tiles are paced against each other (see g_board). By default where experts
-  // have more than one m-tile (more than 96 rows on average) AND the launch's weights are far more than the
-  // 256 MB memory-side cache holds: there a sibling that falls behind fetches its weights from HBM again, and
-  // keeping the siblings together is worth 3-7 % at every batch size (DeepSeek-V3 shape: 4096 tokens gate_up
-  // 1950 -> 1898 us, down 972 -> 926 us, bytes fetched by L2 1.49x -> 1.08x of the algorithmic ones; 12288
-  // tokens 4051 -> 3937 and 2225 -> 2070 us; 32768 tokens 10.79 -> 10.37 ms). A launch whose weights fit that
-  // cache (Qwen3 shape: 403 and 201 MB) re-reads them from there at little cost, and the waits only cost:
-  // +1.5 to +4 % from 2048 to 8192 tokens.
+  // 128-row 4-wave tiles whose sibling m-tiles are paced against each other (see g_board): variant 12, and the
+  // second launch of the device-decided pair (variant 17). They were the default where experts have several m-tiles
+  // and the launch's weights are far more than the 256 MB memory-side cache holds (a sibling that falls behind
+  // fetches its weights from HBM again: DeepSeek-V3 shape at 4096 tokens, bytes fetched by L2 1.49x -> 1.08x of the
+  // algorithmic ones, gate_up 1950 -> 1898 us); the evenly split wide tiles below keep the siblings together by
+  // construction and are 6-12 % ahead of them at every batch, so no default path launches them any more.
   const long long weight_bytes = static_cast<long long>(a->E + (a->w_tail ? 1 : 0)) * a->n * a->k;
-  const bool paced = a->variant == 12 || (a->variant == 17 && avg_rows > 96) ||
-                     (a->variant == 0 && !shorter && avg_rows > 96 && weight_bytes > (1ll << 30));
+  const bool paced = a->variant == 12 || (a->variant == 17 && avg_rows > 96);
   // 96-row tiles between the two: from 45 to 72 rows per expert nearly every expert still fits one tile, and a
   // quarter of the 128-row tile's MFMAs (all padding there) is saved (Qwen3 shape, layer: 768 tokens 0.169 ->
   // 0.158 ms, 1024 tokens 0.191 -> 0.165 ms; at 80 rows per expert too many experts need a second tile: -4 % on
@@ -1367,22 +1372,24 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
   // workgroups of four waves hold 96 KB of which the co-resident tiles of one expert duplicate a part), a weight
   // fragment feeds up to 16 MFMAs, and a tile that holds an expert whole streams the expert's weights once. Row
   // fragments past an expert's end cost nothing (see frag_pair_i8), so the height only has to be tall enough.
-  // Measured inside the layer against the 4-wave tiles above (two per CU; ms per layer call, same box):
-  //   DeepSeek-V3 dims, tokens 1024 / 2048 / 4096 / 6144 / 8192: before 2.105 / 2.277 / 2.833 / 3.753 / 4.634
-  //     128-row wide 2.045 / 2.186 / - / - / -; 192-row 2.083 / 2.233 / 2.639 / 3.957 / 5.285;
-  //     256-row - / - / - / 3.426 / 4.862 (one 192-row two-wave-row tile per expert at 4096 tokens was the 2.833);
-  //   Kimi-K2 dims at 4096 tokens (85 rows per expert): 3.703 -> 128-row 3.548, 192-row 3.518;
-  //   Qwen3 dims, tokens 1024 / 2048 / 4096 / 8192: before 0.164 / 0.240 / 0.329 / 0.557,
-  //     128-row 0.169 / 0.234 / 0.326 / 0.566, 192-row 0.174 / 0.208 / 0.337 / 0.504, 256-row 0.206 / 0.241 / 0.367 / 0.578.
-  // So: where nearly every expert fits ONE tile of at most 256 rows (average + 3 sqrt(average) rows of a routed
-  // expert), the shortest such tile. Where experts need several tiles: with weights that the memory-side cache
-  // serves (up to 1 GiB) 192-row tiles from 300 rows per expert on, 128-row ones below; with weights beyond that the
-  // paced 4-wave tiles above stay (their m-tiles share the weight bytes in L2; the wide tiles are not paced).
-  // The rule knows the AVERAGE; a skewed routing decides on the device (weights beyond 1 GiB, where an expert that
-  // overflows its tile streams its weights from HBM a second time): the wide launch is followed by the paced
-  // 128-row one, and each of the two reads the row counts in its prologue and leaves if the other is due - the
-  // wide one runs while at most one routed expert in 16 overflows its tile. Variant 17: that pair whatever the
-  // size of the weights; 19 / 18 / 22 (and 15 / 14 / 8, 16): 128- / 192- / 256-row wide tiles forced.
+  // An expert's rows are split evenly over its m-tiles (resolve_item), so the tiles of one channel block take about
+  // the same time, stay in step on their neighbouring workgroups and share the weight bytes in L2 without pacing.
+  // Measured inside the layer (ms per layer call, same box; before = the 4-wave tiles above, two per CU, paced
+  // where the weights exceed 1 GiB):
+  //   DeepSeek-V3 dims, tokens 2048 / 3072 / 4096 / 6144 / 8192 / 12288 / 16384:
+  //     before 2.346 / 2.589 / 2.985 / 3.738 / 4.561 / 6.406 / 8.350
+  //     192-row wide 2.230 / 2.379 / 2.605 / 3.437 / 4.312 / 5.740 / 7.332
+  //     128-row wide 2.198 / 2.427 / 2.864 / 3.621 / 4.440 / 6.136 / 7.949; 256-row (spills) - / - / - / 3.445 / 4.479 / 6.032 / 7.730
+  //     with +1.0 on the logits of 32 experts, 4096 / 8192 tokens: before 2.989 / 4.652, 192-row wide 2.765 / 4.107
+  //   Kimi-K2 dims, tokens 2048 / 4096 / 8192: before 3.339 / 3.792 / 5.800, 192-row 3.158 / 3.518 / 4.689, 128-row 3.118 / 3.515 / 5.142
+  //   Qwen3 dims, tokens 2048 / 4096 / 6144 / 8192: 96-row 4-wave tiles 0.220 / 0.318 / 0.427 / 0.554,
+  //     192-row wide 0.219 / 0.322 / 0.440 / 0.532, 128-row wide 0.238 / 0.333 / 0.454 / 0.582.
+  // So: the 128-row wide tile where nearly every expert fits it (average + 3 sqrt(average) rows of a routed expert),
+  // the 192-row one everywhere else - one tile for most experts up to 150 rows, evenly split tiles beyond.
+  // Before the even split a 192-row tile next to a 32-row one fetched the expert's weights twice (DeepSeek-V3 dims
+  // at 7168 tokens: 4.78 ms, now 4.00), which is what the paced 4-wave tiles and a device-decided pair of launches
+  // (a wide tile while few experts overflow it, paced tiles otherwise) had been for; the pair remains as variant 17,
+  // the paced tiles as variant 12; 19 / 18 / 22 (and 15 / 14 / 8, 16): 128- / 192- / 256-row wide tiles forced.
   // (an expert of up to 3 MiB stays in an XCD's 4 MB L2 while its m-tiles run: their channel blocks go side by side)
   p.m_major = static_cast<long long>(a->n) * a->k <= (3ll << 20) ? 1 : 0;
   const float avg_routed = static_cast<float>(ceil_div(live, a->E));
@@ -1396,14 +1403,12 @@ int tiled_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
     case 8: case 16: case 22: wide = 16; break;
     default: break;
   }
-  if ((a->variant == 0 && !shorter && (big || avg_rows > 72)) || a->variant == 17) {
+  if (a->variant == 0 && !shorter && (big || avg_rows > 72)) {
     // (small weights keep the 96-row tiles up to 72 rows per expert: Qwen3 dims at 1024 tokens 0.164 against 0.169)
-    if (reach <= 256.0f) {
-      wide = reach <= 128.0f ? 8 : (reach <= 192.0f ? 12 : 16);
-      pair = big || a->variant == 17;
-    } else if (!big && a->variant == 0) {
-      wide = avg_routed > 300.0f ? 12 : 8;
-    }
+    wide = reach <= 128.0f ? 8 : 12;
+  } else if (a->variant == 17) {
+    wide = reach <= 128.0f ? 8 : (reach <= 192.0f ? 12 : 16);
+    pair = true;
   }
   if (wide) {
     const bool f16 = a->act_dtype == KMOE_DT_F16;

@@ -265,7 +265,8 @@ typedef struct kmoe_gemm_i8_args {
                              19, 18, 22: wide tiles of 128, 192, 256 rows - eight waves side by side along the
                              channels, one workgroup per CU (15, 14, 8 and 16 are older names of 19, 18, 22); 17: a
                              wide-tile launch and a paced 128-row-tile launch, of which the row counts decide on the
-                             device which one works (what 0 does for weights beyond 1 GiB); all need k >= 128); with
+                             device which one works; 0 takes 64- / 96-row tiles for few rows per expert and the 128- or
+                             192-row wide tiles beyond, an expert's rows split evenly over its tiles; all need k >= 128); with
                              chunked activations 1, 2, 4, 8 = 16-row fragments per pass of the streaming kernel */
   int32_t w_layout;       /* KMOE_W_ROWMAJOR, or KMOE_W_TILED (kmoe_tile_weights_i8) */
   int32_t a_layout;       /* KMOE_A_ROWMAJOR, or KMOE_A_CHUNKED: a is [k/64][a_rows][64]

@@ -621,7 +621,7 @@ typedef struct kmoe_moe_args {
   float shared_scale;    /* caller epilogue for half activations (models/deepseek_v2.py:286-292: the routed sum stays
                             unscaled and the shared expert's output is multiplied by 1/routed_scaling_factor):
                             out = dt( dt(routed * out_scale) + dt(shared * shared_scale) ); 0 means 1 */
-  int32_t tile_variant;  /* INT8 and FP8_BLOCK, tuning: 0, or the `variant` (int8: 5-22; fp8: 5, 6, 8, 11-14, 17) handed to
+  int32_t tile_variant;  /* INT8 and FP8_BLOCK, tuning: 0, or the `variant` (int8: 5-22; fp8: 5, 6, 8, 11-14, 17-19) handed to
                             the two routed GEMMs when the batch runs on the tile kernel (more than 10 rows per
                             expert); ignored otherwise */
   int32_t w_scale_layout; /* W4A16: KMOE_S_* of w13_scale and w2_scale                                  */

@@ -148,18 +148,19 @@ FP8_TILED_CASES = FP8_CASES + [
 
 
 @pytest.mark.parametrize("E,n,k,counts", FP8_TILED_CASES)
-@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 8, 11, 13, 14, 17])
+@pytest.mark.parametrize("variant", [1, 2, 3, 5, 6, 8, 11, 13, 14, 17, 18, 19])
 @pytest.mark.parametrize("act", [0, 1])
 def test_grouped_gemm_fp8_block_tiled_weights(L, E, n, k, counts, variant, act):
     """The same product with the weight bytes re-arranged by kmoe_tile_weights_i8: the LDS-staged
     kernels (1-3) and the persistent tile kernel (5: tile height by the rows per expert; 6: 128; 11: 64; 13: 96 rows;
-    14, 8: 8-wave tiles of 192 and 256 rows; 17: 192- or 128-row tiles, decided on the device)."""
+    14, 8: 8-wave tiles of 192 and 256 rows; 17: 192- or 128-row tiles, decided on the device; 18, 19: wide tiles
+    of 192 and 128 rows on the asynchronous activation path, rows past a tile's end skipped)."""
     _fp8_case(L, E, n, k, counts, variant, act, tiled=True)
 
 
 @pytest.mark.parametrize("E,n,k,counts", FP8_TILED_CASES)
 @pytest.mark.parametrize("variant,tiled", [(1, False), (2, True), (5, True), (6, True), (11, True), (12, True), (13, True),
-                                           (14, True), (8, True), (17, True)])
+                                           (14, True), (8, True), (17, True), (18, True), (19, True)])
 @pytest.mark.parametrize("act", [0, 1])
 def test_grouped_gemm_fp8_block_half_results(L, E, n, k, counts, variant, tiled, act):
     """act_dtype = KMOE_DT_F16: the LDS-staged kernel and the tile kernel's 64-row, 128-row and paced shapes."""
@@ -311,7 +312,7 @@ def test_moe_fc_op_bf16_swish_glu():
 @pytest.mark.parametrize("E,n,k,counts,tail", [(3, 256, 384, [5, 0, 21], 40), (2, 512, 1024, [70, 3], 7),
                                                (20, 1024, 256, [((53 * i) % 300) for i in range(20)], 300),
                                                (2, 256, 128, [0, 0], 33)])
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 5, 6, 11, 13])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 5, 6, 11, 13, 18, 19])
 @pytest.mark.parametrize("act", [0, 1])
 def test_grouped_gemm_fp8_block_tail_expert(L, E, n, k, counts, tail, variant, act):
     """w_tail / w_scale_tail: one more expert in the same launch, whose `tail` rows follow the routed

@@ -593,7 +593,7 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
     routed.variant = a->tile_variant;
   const int tv = a->tile_variant;
   if (a->format == KMOE_FMT_FP8_BLOCK && a->w_layout == KMOE_W_TILED && (local_pairs(a) + E - 1) / E > 10 &&
-      (tv == 5 || tv == 6 || tv == 8 || (tv >= 11 && tv <= 14) || tv == 17))
+      (tv == 5 || tv == 6 || tv == 8 || (tv >= 11 && tv <= 14) || (tv >= 17 && tv <= 19)))
     routed.variant = tv;
   const bool fold = fold_shared(a);
   if (fold) {

@@ -575,7 +575,7 @@ extern "C" int kmoe_grouped_gemm_fp8_block(const kmoe_gemm_fp8_args* a, kmoe_str
   KMOE_REQUIRE(a->w_layout == KMOE_W_ROWMAJOR || a->w_layout == KMOE_W_TILED, KMOE_ERR_UNSUPPORTED,
                "grouped_gemm_fp8_block: w_layout=%d unknown", a->w_layout);
   // tiled weights and more than a few rows per expert: the persistent tile kernel (variants 5, 6, 11 force it)
-  const bool tall_variant = a->variant == 8 || a->variant == 14 || a->variant == 17;  // 8-wave tiles of 256 / 192 rows; 17: chosen on the device
+  const bool tall_variant = a->variant == 8 || a->variant == 14 || (a->variant >= 17 && a->variant <= 19);  // 8-wave tiles of 256 / 192 rows; 17: chosen on the device; 18, 19: wide 192- / 128-row tiles
   if (a->w_layout == KMOE_W_TILED && a->k <= 8192 && a->ldy % 8 == 0 &&
       (tile_variant(a->variant) || tall_variant || (a->variant == 0 && ceil_div(expected_rows(a->rows, a->rows_hint), a->E) > kTiledMinRows)))
     return tiled_gemm_fp8(a, as_stream(stream));

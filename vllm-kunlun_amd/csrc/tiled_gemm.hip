@@ -65,6 +65,27 @@ __device__ __forceinline__ void lds_read4_b32(float& a, float& b, float& c, floa
       : "v"(addr), "n"(STRIDE), "n"(2 * STRIDE), "n"(3 * STRIDE)
       : "memory");
 }
+// fp8 on the asynchronous path: the two K halves of an activation fragment and its row scale, requested without a
+// wait (IMM: byte offset of the fragment in the chunk buffer, SOFF: of its scale), and the wait that makes them
+// (and the chunk's two weight scales) usable while at most N younger LDS operations stay in flight.
+template <int IMM, int SOFF>
+__device__ __forceinline__ void f8_request(v4i& lo, v4i& hi, float& sa, uint32_t a_lo, uint32_t a_hi, uint32_t sc_addr) {
+  asm volatile(
+      "ds_read_b128 %0, %3 offset:%6\n\t"
+      "ds_read_b128 %1, %4 offset:%6\n\t"
+      "ds_read_b32 %2, %5 offset:%7"
+      : "=&v"(lo), "=&v"(hi), "=&v"(sa)
+      : "v"(a_lo), "v"(a_hi), "v"(sc_addr), "n"(IMM), "n"(SOFF)
+      : "memory");
+}
+template <int N>
+__device__ __forceinline__ void f8_wait(v4i& lo, v4i& hi, float& sa, float& s0, float& s1) {
+  asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(lo), "+v"(hi), "+v"(sa), "+v"(s0), "+v"(s1) : "n"(N));
+}
+template <int OFF>
+__device__ __forceinline__ void lds_request_b32(float& v, uint32_t addr) {
+  asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+}
 // lds_wait<n> for an n that is a constant only after unrolling (at most 7 younger LDS operations stay in flight)
 template <typename V>
 __device__ __forceinline__ void lds_wait_upto(int n, V& v) {
@@ -228,7 +249,7 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
   // unpadded chunk buffers (row r, 16-byte vector c of a chunk at r * 128 + 16 (c ^ r % 8): eight
   // consecutive rows of one fragment column fall on eight different bank groups). F8 keeps the
   // register path (its row scales travel with the data): two padded buffers.
-  constexpr bool ADMA = !F8;
+  constexpr bool ADMA = !F8 || WN == 8;  // (fp8: the wide tiles; its 4-wave tiles keep the register path)
   constexpr int kStageBytes = ADMA ? WM * kWN * kNA * 8 * kChunk : kTM * kPitchT;  // (ADMA: kTM rows, or the copies' 8 kNA per wave)
   __shared__ __attribute__((aligned(1024))) int8_t lds_a[ADMA ? kStagesA : 2][kStageBytes];
   // (wide tiles with two output fragments a wave: patches for kPatchGroup row fragments, transposed in one LDS round trip)
@@ -243,7 +264,10 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
   // F8: weight block scales of the tile [parity][wave][fragment][k block], and the row scales
   // of the chunk in each activation buffer
   __shared__ float wsc_lds[F8 ? 2 : 1][F8 ? kWN * NF * kMaxKBlocks : 4];
-  __shared__ float asc_lds[F8 ? 2 : 1][F8 ? kThreads : 4];  // every thread stores (rows repeat): no branch in the loop
+  // (register path: every thread stores, rows repeat - no branch in the loop; asynchronous path: a ring like the
+  // chunks', each wave copying 64 row scales per chunk, waves past the tile's rows repeating earlier ones)
+  static_assert(!(F8 && ADMA) || kTM % kWave == 0, "row scales are copied 64 at a time");
+  __shared__ float asc_lds[F8 ? (ADMA ? kStagesA : 2) : 1][F8 ? (ADMA ? kTM : kThreads) : 4];
   extern __shared__ int dyn_lds[];
   const int n_exp = p.E + (p.w_tail ? 1 : 0);
   int* row_lo = dyn_lds;               // [E + 1]: lod
@@ -463,8 +487,16 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
 #pragma unroll
       for (int i = 0; i < kNA; ++i)
         buffer_load16_to_lds(a_rsrc, (lds_ptr_t)&lds_a[stage][(wave_id * kNA + i) * 1024], aoff[i], kc);
+      if constexpr (F8) {
+        // the chunk's row scales travel the same way: lane l of wave w brings the scale of tile row (64 w + l) % kTM
+        const uint32_t kb = static_cast<uint32_t>(min(chunk, last_chunk));
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(make_rsrc(p.a_max), (lds_ptr_t)&asc_lds[stage][(wave_id * kWave) % kTM], 4,
+                                                 (static_cast<uint32_t>(my_srow) * static_cast<uint32_t>(kblocks) + kb) * 4u,
+                                                 0, 0, 0);
+      }
     }
   };
+  constexpr int kND = kNA + ((F8 && ADMA) ? 1 : 0);  // copies per chunk and wave
   // one MFMA step: 8 A fragments from LDS, each against the 4 weight fragments of the slot
   auto mfma_row = [&](const v4i(&wcur)[kNF], const v4i& af, int mf, int t) {
     if constexpr (M32) {
@@ -695,6 +727,61 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
       }
     }
   };
+  // F8 on the asynchronous path, one whole chunk (the two ring slots are the K halves of one MFMA): every LDS
+  // access is an assembly statement (an LDS read the compiler sees waits for the copies in flight). The bytes and
+  // the row scale of fragment n + 1 are requested before fragment n is waited for; fragments past the tile's rows
+  // are read (whatever the buffer holds) and not multiplied.
+  auto compute_f8_dma = [&](const v4i(&w_lo)[kNF], const v4i(&w_hi)[kNF], auto buf_tag, int chunk, int parity) {
+    if constexpr (F8 && ADMA) {
+      constexpr int buf = decltype(buf_tag)::value;
+      constexpr bool kFarStages = kStagesA * kStageBytes > 65536;
+      constexpr int kImm = kFarStages ? 0 : buf * kStageBytes;
+      const uint32_t a_lo = fa[0] + (kFarStages ? buf * kStageBytes : 0);
+      const uint32_t a_hi = fa[1] + (kFarStages ? buf * kStageBytes : 0);
+      const uint32_t sc_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+          (lds_ptr_t)&asc_lds[buf][wave_m * 16 * kMF + li]));
+      const uint32_t wsc_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+          (lds_ptr_t)&wsc_lds[parity][wave * kNF * kMaxKBlocks + chunk]));
+      static_assert(kNF == 2, "the asynchronous fp8 path is written for two channel fragments a wave");
+      float swc[kNF];
+      lds_request_b32<0>(swc[0], wsc_addr);
+      lds_request_b32<kMaxKBlocks * 4>(swc[1], wsc_addr);
+      v4i lo[2], hi[2];
+      float sar[2];
+      f8_request<kImm, 0>(lo[0], hi[0], sar[0], a_lo, a_hi, sc_addr);
+      auto run = [&](auto self, auto n_tag) {
+        constexpr int n = decltype(n_tag)::value;
+        if constexpr (n < kMF) {
+          if constexpr (n + 1 < kMF) {
+            f8_request<kImm + (n + 1) * 16 * kChunk, (n + 1) * 64>(lo[(n + 1) & 1], hi[(n + 1) & 1], sar[(n + 1) & 1], a_lo, a_hi,
+                                                                  sc_addr);
+            f8_wait<3>(lo[n & 1], hi[n & 1], sar[n & 1], swc[0], swc[1]);
+          } else {
+            f8_wait<0>(lo[n & 1], hi[n & 1], sar[n & 1], swc[0], swc[1]);
+          }
+          if (n < live_frags) {  // (wave-uniform)
+            v8i av;
+            av.lo = lo[n & 1];
+            av.hi = hi[n & 1];
+#pragma unroll
+            for (int f = 0; f < kNF; ++f) {
+              v8i wv;
+              wv.lo = w_lo[f];
+              wv.hi = w_hi[f];
+              const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, av, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0,
+                                                                               0x7f7f7f7f, 0, 0x7f7f7f7f);
+              const float sc = sar[n & 1] * swc[f];
+#pragma unroll
+              for (int q = 0; q < 4; ++q) acc[n][f][q] = __builtin_fmaf(blk[q], sc, acc[n][f][q]);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          self(self, std::integral_constant<int, n + 1>{});
+        }
+      };
+      run(run, std::integral_constant<int, 0>{});
+    }
+  };
   // F8, one whole chunk: the two ring slots of the chunk are the K halves of one MFMA
   auto compute_f8 = [&](const v4i(&w_lo)[kNF], const v4i(&w_hi)[kNF], int buf, int chunk, int parity) {
     if constexpr (!M32) {
@@ -906,7 +993,7 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
       seen_prev = seen_next = 0;  // nothing polled for this tile yet: its first chunk starts without waiting
       patience = kSyncPatience;
     }
-    if constexpr (ADMA && I8 && !M32) {
+    if constexpr ((ADMA && I8 && !M32) || (F8 && ADMA)) {
       const int rows_here = min(cur.end, cur.row0 + kTM) - cur.row0 - wave_m * 16 * kMF;
       live_frags = __builtin_amdgcn_readfirstlane(max(0, min(kMF, (rows_here + 15) >> 4)));
     }
@@ -919,8 +1006,15 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
     if constexpr (F8) {
       if (wave_m == 0 && (lane >> 4) < kNF) {
 #pragma unroll
-        for (int i = 0; i < kMaxKBlocks / 16; ++i)
-          wsc_lds[parity][(wave * kNF + (lane >> 4)) * kMaxKBlocks + (lane & 15) + 16 * i] = wsc_reg[i];
+        for (int i = 0; i < kMaxKBlocks / 16; ++i) {
+          float* slot = &wsc_lds[parity][(wave * kNF + (lane >> 4)) * kMaxKBlocks + (lane & 15) + 16 * i];
+          if constexpr (ADMA) {  // (an LDS store the compiler sees would wait for the copies in flight)
+            const uint32_t addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)slot));
+            asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(wsc_reg[i]) : "memory");
+          } else {
+            *slot = wsc_reg[i];
+          }
+        }
       }
     }
     store_a(0);
@@ -981,7 +1075,12 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
       load_a(c0 + h + 1);
       load_w(wring[(2 * h + R - 1) % R], s0 + R - 1);
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (F8) {
+      if constexpr (F8 && ADMA) {
+        compute_f8_dma(wring[(2 * h) % R], wring[(2 * h + 1) % R], buf_t{}, c0 + h, parity);
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(wring[(2 * h) % R], s0 + R);
+        dma_a(c0 + h + kStagesA - 1, (buf + kStagesA - 1) % kStagesA);
+      } else if constexpr (F8) {
         compute_f8(wring[(2 * h) % R], wring[(2 * h + 1) % R], buf, c0 + h, parity);
         __builtin_amdgcn_sched_barrier(0);
         load_w(wring[(2 * h) % R], s0 + R);
@@ -1003,7 +1102,7 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
       // (a bare barrier: the fence of __syncthreads would drain every load in flight, since the
       // asynchronous copies count as stores to LDS)
       if constexpr (ADMA) {
-        vmem_wait<2 * kNF + kNA + kPolls>();
+        vmem_wait<2 * kNF + kND + kPolls>();
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
       } else {
@@ -1500,19 +1599,21 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 6>(p, a->rows, s, n_cu, what);
   }
   const long long weight_bytes = static_cast<long long>(a->E + (a->w_tail ? 1 : 0)) * a->n * a->k;
-  // One 8-wave tile of 192 rows per expert where nearly every expert fits it and many would overflow a 128-row
-  // tile, as for int8 - for the short K of the down projection only, where pacing does not pay. Stand-alone the
-  // tall tile wins on both projections (DeepSeek-V3 shape, gate_up / down against the paced 128-row tiles: 128
-  // rows per expert 2158 / 1009 -> 2131 / 981 us, 144 rows 2513 / 1265 -> 2191 / 994, 160 rows 2643 / 1333 -> 2510
-  // / 1027; at 112 rows 1943 -> 2092 and at 192 rows 2588 -> 3558: not there), but inside the layer, with the
-  // shared expert's 4096 rows as the launch's tail, gate_up loses (4096 tokens: 2.21 -> 2.51 ms, 4608: 2.45 ->
-  // 2.63) while down still gains (1.10 -> 1.01 ms, 1.22 -> 1.07, 5120 tokens 1.31 -> 1.16). The 256-row instance
-  // spills and is a tuning variant.
-  // As for int8 the device decides between the tall launch and the one that follows it (variant 17: the pair
-  // whatever the size of the weights and K).
   const int avg_routed = ceil_div(live, a->E);
-  const bool by_rule = ((a->variant == 0 && a->k < 4096 && weight_bytes > (1ll << 30)) || a->variant == 17) &&
-                       avg_routed >= 124 && avg_routed <= 168;
+  // Wide tiles (eight waves side by side, 192 or 128 rows, as for int8) on the ASYNCHRONOUS activation path: chunks
+  // and their row scales copied global -> LDS three chunks ahead, every LDS access in assembly, row fragments past a
+  // tile's rows not multiplied, an expert's rows split evenly over its tiles. This format gains less from them than
+  // int8 (its loop scales every chunk's partial sums, whatever the tile), and only where nearly every expert fills
+  // most of one 192-row tile: layer, tokens -> ms against the 4-wave tiles, DeepSeek-V3 dims 3072 / 4096 / 6144 /
+  // 8192 / 12288: 2.880 / 3.535 / 4.705 / 5.792 / 8.236 -> 2.881 / 3.326 / 4.653 / 6.001 / 7.989; Kimi-K2 dims 2048 /
+  // 4096 / 8192: 3.301 / 4.021 / 6.696 -> 3.501 / 4.360 / 6.322 (128-row wide: 3.330 / 4.050 / 6.693). So by default
+  // from 112 to 200 rows per expert with weights beyond 1 GiB; 18 / 19 force the 192- / 128-row wide tile.
+  if (a->variant == 18 || (a->variant == 0 && weight_bytes > (1ll << 30) && avg_routed >= 112 && avg_routed <= 200))
+    return launch_wide<K, 12>(p, a->rows, s, n_cu, what, swiglu, half);
+  if (a->variant == 19) return launch_wide<K, 8>(p, a->rows, s, n_cu, what, swiglu, half);
+  // One 8-wave tile of 192 rows per expert on two rows of four waves (register path): variant 14, and the first
+  // launch of the device-decided pair (variant 17); the wide tiles above took over where it had been the default.
+  const bool by_rule = a->variant == 17 && avg_routed >= 124 && avg_routed <= 168;
   if (a->variant == 14 || by_rule) {
     p.pick = by_rule ? 1 : 0;
     p.pick_rows = 192;

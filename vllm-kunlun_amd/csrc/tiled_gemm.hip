@@ -749,6 +749,8 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
       v4i lo[2], hi[2];
       float sar[2];
       f8_request<kImm, 0>(lo[0], hi[0], sar[0], a_lo, a_hi, sc_addr);
+      v4f blk[2][kNF];     // partial sums of the fragment whose MFMAs were issued last, and of the one before
+      float scp[2][kNF];   // ... and their scales
       auto run = [&](auto self, auto n_tag) {
         constexpr int n = decltype(n_tag)::value;
         if constexpr (n < kMF) {
@@ -759,6 +761,7 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
           } else {
             f8_wait<0>(lo[n & 1], hi[n & 1], sar[n & 1], swc[0], swc[1]);
           }
+          // the scaling of fragment n - 1 follows the MFMAs of fragment n: the wave does not wait for the matrix pipe
           if (n < live_frags) {  // (wave-uniform)
             v8i av;
             av.lo = lo[n & 1];
@@ -768,11 +771,18 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
               v8i wv;
               wv.lo = w_lo[f];
               wv.hi = w_hi[f];
-              const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, av, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0,
-                                                                               0x7f7f7f7f, 0, 0x7f7f7f7f);
-              const float sc = sar[n & 1] * swc[f];
+              blk[n & 1][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, av, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0,
+                                                                              0x7f7f7f7f, 0, 0x7f7f7f7f);
+              scp[n & 1][f] = sar[n & 1] * swc[f];
+            }
+          }
+          if constexpr (n > 0) {
+            if (n - 1 < live_frags) {
 #pragma unroll
-              for (int q = 0; q < 4; ++q) acc[n][f][q] = __builtin_fmaf(blk[q], sc, acc[n][f][q]);
+              for (int f = 0; f < kNF; ++f)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                  acc[n - 1][f][q] = __builtin_fmaf(blk[(n - 1) & 1][f][q], scp[(n - 1) & 1][f], acc[n - 1][f][q]);
             }
           }
           __builtin_amdgcn_sched_barrier(0);
@@ -780,6 +790,14 @@ __global__ __launch_bounds__(WM * WN * kWave, WGS) void tiled_gemm_kernel(const 
         }
       };
       run(run, std::integral_constant<int, 0>{});
+      if (kMF - 1 < live_frags) {
+#pragma unroll
+        for (int f = 0; f < kNF; ++f)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            acc[kMF - 1][f][q] = __builtin_fmaf(blk[(kMF - 1) & 1][f][q], scp[(kMF - 1) & 1][f], acc[kMF - 1][f][q]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
   // F8, one whole chunk: the two ring slots of the chunk are the K halves of one MFMA

@@ -1600,10 +1600,10 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
     return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what)
                   : launch_tiled<K, false, 4, 4, 2, 1, false, 4>(p, a->rows, s, n_cu, what);
   }
-  // paced sibling m-tiles where experts have more than one of them and the weights are far more than the
-  // memory-side cache holds, as for int8, and a tile walks a long K (DeepSeek-V3 shape at 4096 tokens: gate_up,
-  // K = 7168, 2570 -> 2222 us; the down projection, K = 2048, is 5 % slower with it: 1033 -> 1083 us; layer at
-  // 8192 tokens 5.86 -> 5.78 ms, at 16384 tokens 10.90 -> 10.66 ms)
+  // (Paced sibling m-tiles - variant 12 - had been the default where experts have several m-tiles, the weights are
+  // far more than the memory-side cache holds and a tile walks a long K. With an expert's rows split evenly over
+  // its m-tiles the plain 128-row tiles are 2-4 % ahead of them at every batch: DeepSeek-V3 dims, layer at 2048 /
+  // 4096 / 8192 / 12288 tokens 2.588 / 3.537 / 5.815 / 8.291 ms paced against 2.474 / 3.497 / 5.694 / 7.991.)
   const int avg_rows = ceil_div(live + (a->w_tail ? a->tail_rows : 0), a->E + (a->w_tail ? 1 : 0));
   // 96-row tiles from 45 to 76 rows per expert: the padding rows of a 128-row tile cost this format its scaling work
   // on top of the MFMAs (gate_up GEMM alone, 64 rows per expert: Qwen3 shape 105 -> 85 us, DeepSeek-V3 shape 1515 ->
@@ -1640,7 +1640,7 @@ int tiled_gemm_fp8(const kmoe_gemm_fp8_args* a, hipStream_t s) {
     p.pick = 2;
   }
   if (a->variant == 8) return launch_tall<K, 8>(p, a->rows, s, n_cu, what, swiglu, half);
-  if (a->variant == 12 || (a->variant == 0 && avg_rows > 96 && a->k >= 4096 && weight_bytes > (1ll << 30))) {
+  if (a->variant == 12) {
     if (half)
       return swiglu ? launch_tiled<K, true, 4, 4, 2, 1, false, 8, false, true, true>(p, a->rows, s, n_cu, what)
                     : launch_tiled<K, false, 4, 4, 2, 1, false, 8, false, true, true>(p, a->rows, s, n_cu, what);

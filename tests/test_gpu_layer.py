@@ -81,6 +81,15 @@ SMALL = [
                                                          I_shared=32)),
     ("tiled-routed-rowmajor-shared-many", "dsv3-decode", dict(M=600, H=256, E=8, K=2, I=128, n_group=2,
                                                               topk_group=1, I_shared=32)),
+    # the weight-streaming path where its gate_up launch cannot sort the pairs itself (more than 4096 pairs; more
+    # than 512 tokens) and where its down launch cannot quantise its rows itself (rows of more than 1024 values)
+    ("stream-9600-pairs", "qwen3-decode", dict(M=600, H=256, E=1000, K=16, I=64)),
+    ("stream-520-tokens", "qwen3-decode", dict(M=520, H=256, E=256, K=4, I=64)),
+    ("stream-512-tokens-4096-pairs", "qwen3-decode", dict(M=512, H=256, E=512, K=8, I=64)),
+    ("stream-rows-1088-wide", "qwen3-decode", dict(M=20, H=256, E=16, K=4, I=1088)),
+    ("stream-rows-1024-wide", "qwen3-decode", dict(M=20, H=256, E=16, K=4, I=1024)),
+    # 17 and 33 channel blocks of 128 in the down projection: the last workgroup's waves partly without channels
+    ("stream-down-2112-channels", "qwen3-decode", dict(M=24, H=2112, E=8, K=2, I=128)),
 ]
 
 
@@ -88,7 +97,11 @@ SMALL = [
 def test_layer_matches_oracles(name, base, over):
     from vllm_kunlun_amd import synth
     shape = synth.scaled(synth.SHAPES[base], **over)
-    sl = synth.make_w8a8_layer(shape, "cuda", seed=1)
+    _check_layer(synth.make_w8a8_layer(shape, "cuda", seed=1))
+
+
+def _check_layer(sl):
+    shape = sl.shape
     method = sl.layer.quant_method
     out_scale = 1.0
     out = method.apply_monolithic(sl.layer, sl.x, sl.logits, out_scale=out_scale, **sl.apply_kwargs())
@@ -121,6 +134,59 @@ def test_layer_matches_oracles(name, base, over):
     ref_t = tm.w8a8_moe(_host(sl.x), _host(sl.logits), w13, w13_max, w2, w2_max, shape.K, shape.scoring, True,
                         shape.n_group, shape.topk_group, shape.routed_scale, _host(sl.bias), shared, out_scale)
     assert rel_l2(out, ref_t) <= REL_L2_BF16
+
+
+@pytest.mark.parametrize("hot,boost", [(1, 6.0), (3, 3.0)])
+def test_skewed_decode_batches_match_oracles(hot, boost):
+    """A few experts draw most tokens of a decode-sized batch: on the weight-streaming path they walk their rows in
+    several 16-row passes (the launches that sort the pairs and quantise their rows themselves included), with and
+    without a shared expert in the launches' tail."""
+    from vllm_kunlun_amd import synth
+    for base, over in (("qwen3-decode", dict(M=150, H=256, E=64, K=4, I=192)),
+                       ("dsv3-decode", dict(M=80, H=256, E=32, K=4, I=128, n_group=4, topk_group=2, I_shared=128))):
+        sl = synth.make_w8a8_layer(synth.scaled(synth.SHAPES[base], **over), "cuda", seed=hot)
+        sl.logits[:, :hot] += boost
+        _check_layer(sl)
+        lod = _view(sl.layer.quant_method.last_workspace, sl.layer.quant_method.last_layout.lod, sl.shape.E + 1,
+                    torch.int32).cpu().numpy()
+        assert int(np.diff(lod).max()) > 32, "no expert with more than two passes of rows"
+        assert sl.layer.quant_method.last_layout.codes_chunked, "not on the weight-streaming path"
+
+
+def test_decode_launches_that_sort_and_quantise_keep_the_bits():
+    """KMOE_SORT_IN_GEMM=0 / KMOE_QUANT_IN_GEMM=0 (read once per process, hence child processes) give the sort and
+    the second quantisation launches of their own again: same output bits, same intermediates."""
+    import os
+    import subprocess
+    import sys
+    code = r"""
+import sys, zlib
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[2])
+import torch
+from vllm_kunlun_amd import synth
+for base, over in (("qwen3-decode", dict(M=64, H=512, E=128, K=8, I=768)),
+                   ("dsv3-decode", dict(M=40, H=512, E=32, K=4, I=128, n_group=4, topk_group=2, I_shared=128))):
+    sl = synth.make_w8a8_layer(synth.scaled(synth.SHAPES[base], **over), "cuda", seed=4)
+    sl.logits[:, :2] += 2.0
+    m = sl.layer.quant_method
+    out = m.apply_monolithic(sl.layer, sl.x, sl.logits, **sl.apply_kwargs())
+    torch.cuda.synchronize()
+    lay, ws = m.last_layout, m.last_workspace
+    P, E, I = sl.shape.P, sl.shape.E, sl.shape.I
+    R = P + (sl.shape.M if sl.shape.I_shared == I else 0)
+    parts = [out.view(torch.int16)] + [ws[o: o + n] for o, n in ((lay.moe_index, 4 * P), (lay.sorted_src, 4 * P),
+             (lay.lod, 4 * (E + 1)), (lay.expert_m, 4 * E), (lay.actq, R * I), (lay.actmax, 4 * R))]
+    print(*[zlib.crc32(t.cpu().numpy().tobytes()) for t in parts])
+"""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    sums = []
+    for flag in ("1", "0"):
+        env = dict(os.environ, KMOE_SORT_IN_GEMM=flag, KMOE_QUANT_IN_GEMM=flag)
+        out = subprocess.run([sys.executable, "-c", code, root, os.path.join(root, "vllm-kunlun_amd")], env=env,
+                             capture_output=True, text=True, timeout=110)
+        assert out.returncode == 0, out.stderr[-2000:]
+        sums.append(out.stdout.split())
+    assert len(sums[0]) == 14 and sums[0] == sums[1], sums
 
 
 def test_staged_ops_equal_fused():

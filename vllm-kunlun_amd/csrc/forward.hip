@@ -118,6 +118,24 @@ long long local_pairs(const kmoe_moe_args* a) {
   return a->E_global > a->E ? (P * a->E + a->E_global - 1) / a->E_global : P;
 }
 
+// KMOE_SORT_IN_GEMM=0 (read once) keeps the sort a launch of its own on the weight-streaming path too.
+bool scan_allowed() {
+  static const bool on = [] {
+    const char* v = getenv("KMOE_SORT_IN_GEMM");
+    return !(v && v[0] == '0');
+  }();
+  return on;
+}
+
+// KMOE_QUANT_IN_GEMM=0 (read once) keeps the second quantisation a launch of its own there.
+bool quant_in_gemm_allowed() {
+  static const bool on = [] {
+    const char* v = getenv("KMOE_QUANT_IN_GEMM");
+    return !(v && v[0] == '0');
+  }();
+  return on;
+}
+
 bool use_stream_path(const kmoe_moe_args* a) {
   const long long P = local_pairs(a);
   // a row-major shared expert cannot read the chunk-major codes this path quantises x into
@@ -173,6 +191,10 @@ struct MlpPass {
   int group_size, scale_layout;
   int variant;  // INT8: kernel variant of the two GEMMs (0: from the shape)
   int act_dtype;  // INT8, BF16: KMOE_DT_* of x_rows' source, act and out (BF16: of the weights too)
+  // INT8 weight-streaming path: the gate_up launch sorts the routed pairs itself (row_src is then NULL and lod is
+  // what that launch writes)
+  const StreamScan* scan;
+  bool quant_in_gemm;  // the down launch quantises its rows itself: no launch between the two GEMMs
 };
 
 int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
@@ -219,7 +241,8 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
       g.tail_rows = m.tail_rows;
       g.tail_src0 = first ? 0 : m.rows;  // gate_up reads token rows, down reads its own act rows
     }
-    return kmoe_grouped_gemm_i8(&g, stream);
+    const StreamQuant quant{m.act, m.I, static_cast<int8_t*>(m.actq), m.act_aux};
+    return grouped_gemm_i8_checked(&g, stream, first ? m.scan : nullptr, !first && m.quant_in_gemm ? &quant : nullptr);
   }
   if (m.format == KMOE_FMT_FP8_BLOCK) {
     kmoe_gemm_fp8_args g = {};
@@ -300,14 +323,16 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
 template <class Mark>
 int run_mlp(const MlpPass& m, kmoe_stream_t stream, Mark&& mark) {
   int rc;
-  const char* whose = m.row_src ? "routed experts" : "shared expert";
+  const char* whose = m.row_src || m.scan ? "routed experts" : "shared expert";
   mark(KMOE_STAGE_GEMM1, 0);
   if (tracing_kernels()) note_kernel("[gate_up, %s]", whose);
   rc = run_gemm(m, true, stream);
   if (rc) return rc;
   mark(KMOE_STAGE_GEMM1, 1);
   mark(KMOE_STAGE_QUANT2, 0);
-  if (m.format == KMOE_FMT_INT8) {
+  if (m.format == KMOE_FMT_INT8 && m.quant_in_gemm) {
+    // (the down launch does it)
+  } else if (m.format == KMOE_FMT_INT8) {
     const int qrows = m.rows + m.tail_rows;
     rc = m.stream ? kmoe_quant_i8_rows_chunked_dt(m.act, m.I, qrows, m.I, static_cast<int8_t*>(m.actq), m.act_aux,
                                                   m.act_dtype, stream)
@@ -527,11 +552,18 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
   }
   if (rc) return rc;
   mark(KMOE_STAGE_ROUTING, 1);
-  // 2. stable sort of the routed pairs by expert
+  // 2. stable sort of the routed pairs by expert. On the weight-streaming path (a few rows per expert) the gate_up
+  // launch does it in its prologue and writes the same four arrays: one launch and its round trips less
+  // (Qwen3 decode: 4.8 us of 125). Not for an expert-parallel share (pairs of other ranks' experts get no row).
   mark(KMOE_STAGE_ALIGN, 0);
-  rc = kmoe_align_local(topk_ids, P, E, a->first_expert, moe_index, sorted_src, static_cast<int32_t*>(at(L.expert_m)), lod,
-                        at(L.align_ws), kmoe_align_workspace_bytes(P, E), stream);
-  if (rc) return rc;
+  const StreamScan scan{topk_ids, P, lod, static_cast<int32_t*>(at(L.expert_m)), moe_index, sorted_src};
+  const bool scan_in_gemm = stream_mode && Eg == E && a->first_expert == 0 && P <= kStreamScanMaxPairs &&
+                            M <= kStreamScanMaxRows && scan_allowed();
+  if (!scan_in_gemm) {
+    rc = kmoe_align_local(topk_ids, P, E, a->first_expert, moe_index, sorted_src, static_cast<int32_t*>(at(L.expert_m)), lod,
+                          at(L.align_ws), kmoe_align_workspace_bytes(P, E), stream);
+    if (rc) return rc;
+  }
   mark(KMOE_STAGE_ALIGN, 1);
   // 3. quantise each TOKEN row once (the reference quantises the K-times expanded copy; same values)
   mark(KMOE_STAGE_QUANT1, 0);
@@ -557,7 +589,8 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
   routed.format = a->format;
   routed.x_rows = x_rows;
   routed.x_aux = quant ? static_cast<const float*>(at(L.xmax)) : nullptr;
-  routed.row_src = sorted_src;
+  routed.row_src = scan_in_gemm ? nullptr : sorted_src;
+  routed.scan = scan_in_gemm ? &scan : nullptr;
   routed.src_div = K;
   routed.w13 = a->w13;
   routed.w2 = a->w2;
@@ -587,6 +620,9 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
     routed.act_limit = a->act_limit;
   }
   routed.stream = stream_mode;
+  // Down projections up to 1024 wide quantise their rows in the launch's prologue (Qwen3 decode: one 4.5 us launch
+  // and its gap less); wider rows would not fit the workgroup's LDS copy next to three resident workgroups per CU.
+  routed.quant_in_gemm = stream_mode && I <= kStreamQuantMaxK && quant_in_gemm_allowed();
   routed.x_count = M;
   if (a->format == KMOE_FMT_INT8 && !stream_mode && a->w_layout == KMOE_W_TILED && a->tile_variant >= 5 &&
       a->tile_variant <= 22 && (local_pairs(a) + E - 1) / E > 10 && H >= 128 && I >= 128)
@@ -621,6 +657,8 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
     sh.oai = 0;
     sh.tail_rows = 0;
     sh.row_src = nullptr;
+    sh.scan = nullptr;
+    sh.quant_in_gemm = false;
     sh.src_div = 1;
     sh.w13 = a->ws13;
     sh.w2 = a->ws2;

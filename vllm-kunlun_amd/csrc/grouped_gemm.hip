@@ -446,13 +446,11 @@ int dispatch(const GemmParams& p, int rows, int live, bool swiglu, int variant, 
 bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 }  // namespace
-}  // namespace kmoe
 
-using namespace kmoe;
-
-extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t stream) {
+int grouped_gemm_i8_checked(const kmoe_gemm_i8_args* a, kmoe_stream_t stream, const StreamScan* scan,
+                            const StreamQuant* quant) {
   KMOE_REQUIRE(a, KMOE_ERR_NULL, "grouped_gemm_i8: args is NULL");
-  KMOE_REQUIRE(a->a && a->a_max && a->w && a->w_max && a->lod && a->y, KMOE_ERR_NULL,
+  KMOE_REQUIRE(a->a && a->a_max && a->w && a->w_max && (a->lod || scan) && a->y, KMOE_ERR_NULL,
                "grouped_gemm_i8: NULL tensor pointer");
   KMOE_REQUIRE(a->E >= 1 && a->n >= 16 && a->k >= 16 && a->rows >= 0, KMOE_ERR_SHAPE,
                "grouped_gemm_i8: E=%d n=%d k=%d rows=%d", a->E, a->n, a->k, a->rows);
@@ -482,9 +480,11 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
     KMOE_REQUIRE(a->w_layout == KMOE_W_TILED, KMOE_ERR_UNSUPPORTED,
                  "grouped_gemm_i8: chunked activations need tiled weights");
     KMOE_REQUIRE(a->a_rows >= 1, KMOE_ERR_SHAPE, "grouped_gemm_i8: a_rows=%d < 1", a->a_rows);
-    if (a->rows == 0 && !(a->w_tail && a->tail_rows > 0)) return KMOE_OK;
-    return stream_gemm_i8(a, as_stream(stream));
+    if (a->rows == 0 && !(a->w_tail && a->tail_rows > 0) && !scan) return KMOE_OK;
+    return stream_gemm_i8(a, as_stream(stream), scan, quant);
   }
+  KMOE_REQUIRE(!scan && !quant, KMOE_ERR_UNSUPPORTED,
+               "grouped_gemm_i8: only the weight-streaming kernel sorts the pairs or quantises its rows itself");
   KMOE_REQUIRE(a->a_layout == KMOE_A_ROWMAJOR, KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8: a_layout=%d unknown",
                a->a_layout);
   if (a->rows == 0 && !(a->w_tail && a->tail_rows > 0)) return KMOE_OK;
@@ -499,6 +499,14 @@ extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t st
                a->w_tail, a->w_max_tail, a->tail_row0, a->w_tail ? a->tail_rows : 0, a->tail_src0, nullptr, 0, 0.f, 0.f,
                a->act_dtype == KMOE_DT_F16};
   return dispatch<Kind::I8>(p, a->rows, expected_rows(a->rows, a->rows_hint), swiglu, a->variant, as_stream(stream), "kmoe_grouped_gemm_i8");
+}
+
+}  // namespace kmoe
+
+using namespace kmoe;
+
+extern "C" int kmoe_grouped_gemm_i8(const kmoe_gemm_i8_args* a, kmoe_stream_t stream) {
+  return grouped_gemm_i8_checked(a, stream, nullptr);
 }
 
 extern "C" int kmoe_grouped_gemm_bf16(const kmoe_gemm_bf16_args* a, kmoe_stream_t stream) {

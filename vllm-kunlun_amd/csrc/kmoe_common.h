@@ -23,7 +23,35 @@ void note_kernel(const char* fmt, ...);
 // Writes {0, rows} to lod2: the row offsets of a dense (single-expert) GEMM.
 int fill_dense_lod(int32_t* lod2, int rows, hipStream_t stream);
 // Weight-streaming int8 GEMM (tiled weights, chunk-major activations); arguments already validated.
-int stream_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);
+// With `scan` (the layer's routed gate_up launch at decode sizes) the launch sorts the routed pairs by expert
+// itself: it reads the pairs' expert ids instead of lod / row_src (args->lod and args->row_src are ignored; the
+// gather divisor is args->src_div) and leaves what the sort would have left: lod [E+1], expert_m [E],
+// moe_index [n_pairs], sorted_src [n_pairs]. Every id must lie in [0, E).
+struct StreamScan {
+  const int32_t* ids;
+  int32_t n_pairs;
+  int32_t* lod;
+  int32_t* expert_m;
+  int32_t* moe_index;
+  int32_t* sorted_src;
+};
+constexpr int kStreamScanMaxPairs = 4096;
+constexpr int kStreamScanMaxRows = 512;  // tokens: no expert gets more rows than that
+// With `quant` (the layer's down launch at decode sizes, k <= kStreamQuantMaxK) the launch quantises its rows
+// itself: it reads them as bf16 / half values (act, row stride ld; args->act_dtype) instead of args->a / a_max and
+// leaves codes (chunk-major [k/64][args->a_rows][64]) and row maxes where the quantiser's launch would have.
+struct StreamQuant {
+  const uint16_t* act;
+  int64_t ld;
+  int8_t* codes;
+  float* amax;
+};
+constexpr int kStreamQuantMaxK = 1024;
+int stream_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream, const StreamScan* scan = nullptr,
+                   const StreamQuant* quant = nullptr);
+// kmoe_grouped_gemm_i8 with the options above for the layer's own launches.
+int grouped_gemm_i8_checked(const kmoe_gemm_i8_args* args, kmoe_stream_t stream, const StreamScan* scan,
+                            const StreamQuant* quant = nullptr);
 // Persistent 128-row-tile GEMMs for many rows per expert (tiled weights, row-major activations);
 // arguments already validated.
 int tiled_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);

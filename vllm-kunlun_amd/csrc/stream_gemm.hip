@@ -16,6 +16,7 @@
 //            lines, which cost the DeepSeek-V3 gate_up launch 9 %).
 // Each wave owns NF channel fragments and keeps D MFMA steps of loads in flight.
 #include "kmoe_common.h"
+#include "quant_body.h"
 
 namespace kmoe {
 namespace {
@@ -40,19 +41,42 @@ struct StreamParams {
   int32_t tail_row0, tail_rows, tail_src0;
   int32_t f16;  // outputs (and the rounding of gate and up before SiLU-mul) in IEEE half instead of bf16
   int32_t rotate;  // every wave starts its K range at a step of its own (see stream_gemm_i8)
+  StreamScan scan;  // SCAN instantiations: the routed pairs' expert ids instead of lod / row_src
+  StreamQuant quant;  // QUANT instantiations: the rows as bf16 / half values instead of codes and row maxes
 };
 
 constexpr int kWaves = 4;
+constexpr int kScanBatch = 4;  // expert ids a lane asks for before it waits (a workgroup: one round trip per 1024 pairs)
+constexpr int kQuantStride = kStreamQuantMaxK + 16;  // bytes between the rows of the LDS copy: row li starts 16 li B into the banks
 
 // KS: the workgroup's 4 waves split K KS ways (KS = 1, 2, 4): 4/KS waves own
 // different channels, KS waves share channels and add their exact int32 partial
 // sums through LDS. More, shorter streams: a finer-grained tail on small layers.
-template <int MF, int NF, bool SWIGLU, int D, int KS>
-__global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const StreamParams p) {
+//
+// SCAN: the launch does the stable sort by expert itself. Every workgroup reads all the routed pairs' expert ids
+// (p.scan.ids, a few KB from L2, a quarter per wave, kScanBatch loads in flight), counts the ids below its expert
+// (its first sorted row) and lists the pairs that chose it, in order (its rows): what lod and row_src would have
+// told it, after one memory round trip instead of two dependent ones and without the sort's launch before this one.
+// The workgroups of channel block 0 also write the sort's outputs (lod, expert_m, moe_index, sorted_src) for the
+// launches that follow.
+//
+// QUANT: the launch quantises its rows itself (the down projection of a decode-sized layer with k <= 1024). Per
+// 16-row pass the workgroup's four waves read the pass's live rows as bf16 / half values (p.quant.act), one row
+// per wave at a time, and leave absmax and codes - the arithmetic of quant_i8_rows_body, hence its bits - in LDS,
+// where the K loop reads its row fragments; a and a_max are not read. The workgroups of channel block 0 also write
+// codes (chunk-major) and row maxes where the quantiser's launch would have left them. Built for four waves per
+// SIMD (see stream_gemm_i8).
+template <int MF, int NF, bool SWIGLU, int D, int KS, bool SCAN = false, bool QUANT = false>
+__global__ __launch_bounds__(kWaves* kWave, QUANT ? 4 : 1) void stream_gemm_i8_kernel(const StreamParams p) {
+  static_assert(!QUANT || (MF == 1 && KS == 1 && !SWIGLU && !SCAN), "QUANT: the 16-row down-projection shape only");
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   constexpr int TM = 16 * MF;
   constexpr int WN = kWaves / KS;  // waves along the channel dimension
   __shared__ v4i red[KS > 1 ? (KS - 1) * WN * MF * NF * kWave : 1];
+  __shared__ int pair_list[SCAN ? kWaves : 1][SCAN ? kStreamScanMaxRows : 1];
+  __shared__ int scan_cnt[kWaves], scan_below[kWaves];
+  __shared__ __attribute__((aligned(16))) int8_t qrows[QUANT ? 16 * kQuantStride : 16];
+  __shared__ float qmax[16];
   const int lane = lane_id();
   const int wave_id = threadIdx.x >> 6;
   const int wave = wave_id / KS;   // channel group of this wave
@@ -70,7 +94,9 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int ksteps = p.k / 64;
   const int col_base = (blockIdx.x * WN + wave) * NFH * 16;
-  if (KS == 1 && col_base >= n_half) return;  // whole wave has nothing to do (no barriers when KS == 1)
+  // whole wave has nothing to do (no barriers when KS == 1; with QUANT it stays for the quantisation and its barriers)
+  const bool idle = KS == 1 && col_base >= n_half;
+  if (idle && !QUANT && !SCAN) return;
   const int kb_begin = (ksteps * wk) / KS;
   const int kb_end = (ksteps * (wk + 1)) / KS;
   // With p.rotate a wave walks its K range from a start step of its own, wrapping round: int32 sums do not depend
@@ -104,7 +130,7 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
   // loads leaves the memory queue idle for their latency. Done where a wave's K range is short (a workgroup lives
   // a few microseconds: Qwen3 decode down projection 42.8 -> 40.4 us); with long ranges it changes nothing for the
   // better (DeepSeek-V3 decode: +0.4 %), so those keep the plain order.
-  const bool w_first = klen < 16;
+  const bool w_first = QUANT || klen < 16;
   v4i wreg[D][NF];
   v4i areg[D][MF];
   auto load_w_step = [&](int slot, int kb) {
@@ -121,22 +147,144 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
   __builtin_amdgcn_sched_barrier(0);
 
   int row_begin, row_end;
+  int list_c0 = 0, list_c1 = 0, list_c2 = 0;  // SCAN: lengths of the first three quarters' lists
+  auto listed_pair = [&](int i) {  // SCAN: the pair behind the expert's row i
+    int w = 0;
+    if (i >= list_c0) {
+      i -= list_c0;
+      w = 1;
+      if (i >= list_c1) {
+        i -= list_c1;
+        w = 2;
+        if (i >= list_c2) {
+          i -= list_c2;
+          w = 3;
+        }
+      }
+    }
+    return pair_list[w][i];
+  };
   if (tail) {
     row_begin = p.tail_row0 + (static_cast<int>(blockIdx.y) - p.E) * TM;
     row_end = min(p.tail_row0 + p.tail_rows, row_begin + TM);
+  } else if (SCAN) {
+    // wave w lists the pairs of its quarter of the ids; the quarters' lists, one after the other, are the expert's
+    // rows in order
+    const int quarter = (p.scan.n_pairs + kWaves * kWave - 1) / (kWaves * kWave) * kWave;
+    const int q_begin = wave_id * quarter;
+    const int q_end = min(p.scan.n_pairs, q_begin + quarter);
+    int below = 0, cnt = 0;  // ids below e; pairs of e so far (wave-uniform)
+    for (int base = q_begin; base < q_end; base += kScanBatch * kWave) {
+      int id[kScanBatch];
+#pragma unroll
+      for (int u = 0; u < kScanBatch; ++u) {
+        const int j = base + u * kWave + lane;
+        id[u] = j < q_end ? p.scan.ids[j] : 0x7fffffff;
+      }
+      // (every workgroup of the launch walks all the ids: scalar work wherever it can be, and the listing only for
+      // the few groups of 64 ids that hold a pair of this expert)
+#pragma unroll
+      for (int u = 0; u < kScanBatch; ++u) {
+        if (base + u * kWave >= q_end) break;  // wave-uniform
+        const bool mine = id[u] == e;
+        const uint64_t mb = __ballot(mine);
+        if (mb != 0) {
+          const int at = cnt + __builtin_popcountll(mb & lanemask_lt());
+          if (mine && at < kStreamScanMaxRows) pair_list[wave_id][at] = base + u * kWave + lane;
+          cnt += __builtin_popcountll(mb);
+        }
+        below += __builtin_popcountll(__ballot(id[u] < e));
+      }
+    }
+    if (lane == 0) {
+      scan_cnt[wave_id] = min(cnt, kStreamScanMaxRows);  // (a token picks an expert once: never more rows than tokens)
+      scan_below[wave_id] = below;
+    }
+    __syncthreads();
+    if (idle) return;  // (KS == 1: no barrier after this one)
+    list_c0 = scan_cnt[0];
+    list_c1 = scan_cnt[1];
+    list_c2 = scan_cnt[2];
+    cnt = min(list_c0 + list_c1 + list_c2 + scan_cnt[3], kStreamScanMaxRows);
+    below = scan_below[0] + scan_below[1] + scan_below[2] + scan_below[3];
+    row_begin = below;
+    row_end = below + cnt;
+    if (blockIdx.x == 0 && wave_id == 0) {
+      if (lane == 0) {
+        p.scan.lod[e] = below;
+        p.scan.expert_m[e] = cnt;
+        if (e == p.E - 1) p.scan.lod[p.E] = below + cnt;
+      }
+      for (int i = lane; i < cnt; i += kWave) {
+        const int j = listed_pair(i);
+        p.scan.moe_index[j] = below + i;
+        p.scan.sorted_src[below + i] = j;
+      }
+    }
   } else {
     row_begin = p.lod[e];
     row_end = p.lod[e + 1];
   }
+  if (SCAN && idle) return;  // (a tail slice's waves without channels; the routed ones left after the barrier)
   if (row_begin >= row_end) return;  // (an expert without rows has asked for a few KB of its weights in vain)
 
   for (int row0 = row_begin; row0 < row_end; row0 += TM) {
+    if (QUANT) {
+      if (row0 != row_begin) __syncthreads();  // the pass before has read its fragments
+      const int nvec = p.k / 8;  // vectors of 8 values per row: at most 2 per lane
+#pragma unroll 1
+      for (int q = 0; q < 4; ++q) {
+        const int qi = wave_id + 4 * q;
+        const int r = row0 + qi;
+        if (r >= row_end) break;  // wave-uniform
+        const uint4* src = reinterpret_cast<const uint4*>(p.quant.act + static_cast<size_t>(r) * p.quant.ld);
+        Pack8 val[2];
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int v = lane + i * kWave;
+          if (v < nvec) {
+            val[i].v = src[v];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(act_to_f32(val[i].h[j], f16)));
+          }
+        }
+        amax = group_max<kWave>(amax);
+        const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int v = lane + i * kWave;
+          if (v < nvec) {
+            uint32_t w[2] = {0, 0};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              float f = __builtin_rintf(act_to_f32(val[i].h[j], f16) * inv);
+              f = fminf(fmaxf(f, -127.0f), 127.0f);
+              w[j >> 2] |= static_cast<uint32_t>(static_cast<int>(f) & 0xff) << (8 * (j & 3));
+            }
+            *reinterpret_cast<uint2*>(&qrows[qi * kQuantStride + v * 8]) = make_uint2(w[0], w[1]);
+            if (blockIdx.x == 0)
+              *reinterpret_cast<uint2*>(p.quant.codes + (static_cast<size_t>(v >> 3) * p.a_rows + r) * 64 + (v & 7) * 8) =
+                  make_uint2(w[0], w[1]);
+          }
+        }
+        if (lane == 0) {
+          qmax[qi] = amax;
+          if (blockIdx.x == 0) p.quant.amax[r] = amax;
+        }
+      }
+      __syncthreads();
+      if (idle) continue;
+    }
     const int8_t* ap[MF];
     int srow[MF];
 #pragma unroll
     for (int mf = 0; mf < MF; ++mf) {
       const int r = row0 + mf * 16 + li;
-      srow[mf] = r < row_end ? (tail ? p.tail_src0 + r - p.tail_row0 : (p.row_src ? p.row_src[r] / p.src_div : r)) : -1;
+      if (SCAN)
+        srow[mf] = r < row_end ? (tail ? p.tail_src0 + r - p.tail_row0 : listed_pair(r - row_begin) / p.src_div) : -1;
+      else
+        srow[mf] = r < row_end ? (tail ? p.tail_src0 + r - p.tail_row0 : (p.row_src ? p.row_src[r] / p.src_div : r)) : -1;
       // rows past the end read row 0: valid memory, results never stored
       ap[mf] = p.a + static_cast<size_t>(srow[mf] >= 0 ? srow[mf] : 0) * 64 + lg * 16;
     }
@@ -148,6 +296,7 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
       for (int f = 0; f < NF; ++f) acc[mf][f] = (v4i){0, 0, 0, 0};
 
     auto load_a_step = [&](int slot, int kb) {
+      if (QUANT) return;  // (read from LDS where it is used)
 #pragma unroll
       for (int mf = 0; mf < MF; ++mf) areg[slot][mf] = *reinterpret_cast<const v4i*>(ap[mf] + kb * a_step);
     };
@@ -172,7 +321,10 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
           for (int mf = 0; mf < MF; ++mf)
 #pragma unroll
             for (int f = 0; f < NF; ++f)
-              acc[mf][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wreg[d][f], areg[d][mf], acc[mf][f], 0, 0, 0);
+              acc[mf][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                  wreg[d][f],
+                  QUANT ? *reinterpret_cast<const v4i*>(&qrows[li * kQuantStride + kb_of(kb) * 64 + lg * 16]) : areg[d][mf],
+                  acc[mf][f], 0, 0, 0);
           if (kb + D < klen) load_step(d, kb_of(kb + D));
         }
       }
@@ -204,7 +356,7 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
     for (int mf = 0; mf < MF; ++mf) {
       const int r = row0 + mf * 16 + li;
       if (r >= row_end) continue;
-      const float sa = p.a_max[srow[mf]] / 127.0f;
+      const float sa = (QUANT ? qmax[li] : p.a_max[srow[mf]]) / 127.0f;
 #pragma unroll
       for (int f = 0; f < NFH; ++f) {
         if (!wok[f]) continue;
@@ -232,15 +384,16 @@ __global__ __launch_bounds__(kWaves* kWave) void stream_gemm_i8_kernel(const Str
   }
 }
 
-template <int MF, int NF, bool SWIGLU, int D, int KS = 1>
+template <int MF, int NF, bool SWIGLU, int D, int KS = 1, bool SCAN = false, bool QUANT = false>
 int launch_stream(const StreamParams& p, hipStream_t s) {
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const dim3 grid(ceil_div(n_half, (kWaves / KS) * NFH * 16), p.E + (p.w_tail ? ceil_div(p.tail_rows, 16 * MF) : 0));
   if (tracing_kernels())
-    note_kernel("stream_gemm_i8_kernel<%d rows per pass, %d channel fragments per wave, %s, %d steps in flight, K split %d>",
-                16 * MF, NF, SWIGLU ? "SiLU-mul" : "plain", D, KS);
-  hipLaunchKernelGGL((stream_gemm_i8_kernel<MF, NF, SWIGLU, D, KS>), grid, dim3(kWaves * kWave), 0, s, p);
+    note_kernel("stream_gemm_i8_kernel<%d rows per pass, %d channel fragments per wave, %s, %d steps in flight, K split %d%s%s>",
+                16 * MF, NF, SWIGLU ? "SiLU-mul" : "plain", D, KS, SCAN ? ", sorts the pairs itself" : "",
+                QUANT ? ", quantises its rows itself" : "");
+  hipLaunchKernelGGL((stream_gemm_i8_kernel<MF, NF, SWIGLU, D, KS, SCAN, QUANT>), grid, dim3(kWaves * kWave), 0, s, p);
   return check_launch("kmoe_grouped_gemm_i8 (stream)");
 }
 
@@ -261,7 +414,7 @@ __global__ void tile_weights_kernel(const int8_t* __restrict__ src, int8_t* __re
 
 }  // namespace
 
-int stream_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
+int stream_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s, const StreamScan* scan, const StreamQuant* quant) {
   StreamParams p{a->a, a->a_rows, a->a_max, a->row_src, a->src_div, a->w, a->w_max,
                  a->lod, a->E,     a->n,     a->k,       a->y,       a->ldy, a->acc_out,
                  a->w_tail, a->w_max_tail, a->tail_row0, a->tail_rows, a->tail_src0, a->act_dtype == KMOE_DT_F16,
@@ -269,8 +422,35 @@ int stream_gemm_i8(const kmoe_gemm_i8_args* a, hipStream_t s) {
                  // Mixtral, Qwen3-235B), waves in step hit the same memory channels: measured 5.5 TB/s at k = 8192
                  // and 6.0 at 4096 against 6.5 at 2048; with the rotated start 6.0 and 6.6. Other strides gain
                  // nothing from it (k = 7168: 6.2 either way).
-                 a->k % 4096 == 0};
+                 a->k % 4096 == 0,
+                 scan ? *scan : StreamScan{}, quant ? *quant : StreamQuant{}};
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
+  if (quant) {
+    // the down launch of a decode-sized layer: 16 rows per pass, one wave per K range
+    KMOE_REQUIRE(!scan && !swiglu && a->variant == 0 && a->row_src == nullptr && !a->acc_out && quant->act &&
+                     quant->codes && quant->amax && quant->ld >= a->k && quant->ld % 8 == 0 &&
+                     a->k <= kStreamQuantMaxK && a->k / 64 < 24 &&
+                     ceil_div(expected_rows(a->rows, a->rows_hint), a->E) <= 10,
+                 KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8 (stream): not a launch that can quantise its rows itself");
+    // (Four steps of weights in flight and two channel fragments per wave as in the plain launch. Two steps, or one
+    // fragment per wave with 2 / 4 / 8 steps - 5 to 6 waves per SIMD - are 1.6 to 3.3 us slower; 6 and 8 steps with
+    // two fragments need more registers than four waves per SIMD leave, and this launch needs the four: built for
+    // three it took as long as the quantiser's launch and this one together had. Qwen3 decode, layer: 117.5 us with
+    // the quantiser's launch, 117.0 built for three waves, 115.1 for four.)
+    return launch_stream<1, 2, false, 4, 1, false, true>(p, s);
+  }
+  if (scan) {
+    // the routed gate_up launch of a decode-sized layer: 16 rows per pass, the three shapes of `case 1` below
+    KMOE_REQUIRE(swiglu && a->variant == 0 && a->row_src == nullptr && scan->ids && scan->lod && scan->expert_m &&
+                     scan->moe_index && scan->sorted_src && scan->n_pairs == a->rows &&
+                     a->rows <= kStreamScanMaxPairs && a->a_rows <= kStreamScanMaxRows,
+                 KMOE_ERR_UNSUPPORTED, "grouped_gemm_i8 (stream): not a launch that can sort the pairs itself");
+    const int ksteps = p.k / 64;
+    const int blocks = p.E * ceil_div(p.n / 2, kWaves * 16);
+    if (ksteps >= 24 && blocks < 2048) return launch_stream<1, 2, true, 2, 4, true>(p, s);
+    if (ksteps >= 24) return launch_stream<1, 2, true, 4, 2, true>(p, s);
+    return launch_stream<1, 2, true, 4, 1, true>(p, s);
+  }
   // m-fragments per pass from the rows an expert gets under uniform routing
   int mf = a->variant;
   if (mf == 0) {

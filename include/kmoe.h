@@ -645,9 +645,10 @@ typedef struct kmoe_moe_args {
 #define KMOE_FLAG_SIDE_STREAM 1
 
 /* Decode-sized int8 batches (at most 10 rows per expert, tiled weights): two of the layer's small launches are folded
- * into the GEMM launches. The gate_up launch sorts the routed pairs by expert itself (every wave scans the pairs'
+ * into the GEMM launches. The gate_up launch sorts the routed pairs by expert itself (every workgroup scans the pairs'
  * expert ids; up to 4096 pairs and 512 tokens, one GPU holding every expert) and writes moe_index, sorted_src,
- * expert_m and lod as the sort's launch would; the down launch quantises its rows itself (rows up to 1024 values)
+ * expert_m and lod as the sort's launch would (so does the gate_up launch of KMOE_FMT_W4A16 where it runs on that
+ * format's streaming kernel); the down launch quantises its rows itself (rows up to 1024 values)
  * and writes actq and actmax as the quantiser's launch would. Same bits, same workspace contents, two launches
  * fewer; KMOE_STAGE_ALIGN / KMOE_STAGE_QUANT2 then bracket nothing. The environment variables KMOE_SORT_IN_GEMM=0
  * and KMOE_QUANT_IN_GEMM=0 (read once per process) keep the launches apart: for measurements. */

@@ -155,7 +155,8 @@ def test_skewed_decode_batches_match_oracles(hot, boost):
 
 def test_decode_launches_that_sort_and_quantise_keep_the_bits():
     """KMOE_SORT_IN_GEMM=0 / KMOE_QUANT_IN_GEMM=0 (read once per process, hence child processes) give the sort and
-    the second quantisation launches of their own again: same output bits, same intermediates."""
+    the second quantisation launches of their own again: same output bits, same intermediates (int8 layers), same
+    output bits (layers on packed 4-bit weights)."""
     import os
     import subprocess
     import sys
@@ -177,6 +178,14 @@ for base, over in (("qwen3-decode", dict(M=64, H=512, E=128, K=8, I=768)),
     parts = [out.view(torch.int16)] + [ws[o: o + n] for o, n in ((lay.moe_index, 4 * P), (lay.sorted_src, 4 * P),
              (lay.lod, 4 * (E + 1)), (lay.expert_m, 4 * E), (lay.actq, R * I), (lay.actmax, 4 * R))]
     print(*[zlib.crc32(t.cpu().numpy().tobytes()) for t in parts])
+# packed 4-bit weights: the streaming kernel of that format sorts the pairs as well (16- and 32-row passes)
+for M, E in ((64, 128), (40, 12)):
+    shape = synth.scaled(synth.SHAPES["qwen3-decode"], M=M, H=256, E=E, K=4, I=128, quant="w4", group_size=128)
+    sl = synth.make_layer(shape, "cuda", seed=5)
+    sl.logits[:, :2] += 2.0
+    out = sl.layer(sl.x, sl.logits)
+    torch.cuda.synchronize()
+    print(zlib.crc32(out.view(torch.int16).cpu().numpy().tobytes()))
 """
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     sums = []
@@ -186,7 +195,7 @@ for base, over in (("qwen3-decode", dict(M=64, H=512, E=128, K=8, I=768)),
                              capture_output=True, text=True, timeout=110)
         assert out.returncode == 0, out.stderr[-2000:]
         sums.append(out.stdout.split())
-    assert len(sums[0]) == 14 and sums[0] == sums[1], sums
+    assert len(sums[0]) == 16 and sums[0] == sums[1], sums
 
 
 def test_staged_ops_equal_fused():

@@ -295,7 +295,7 @@ int run_gemm(const MlpPass& m, bool first, kmoe_stream_t stream) {
     g.act = act;
     g.w_layout = m.w_layout;
     g.act_dtype = m.act_dtype;
-    return kmoe_grouped_gemm_w4a16(&g, stream);
+    return grouped_gemm_w4a16_checked(&g, stream, first ? m.scan : nullptr);
   }
   kmoe_gemm_bf16_args g = {};
   g.a = static_cast<const uint16_t*>(a);
@@ -557,7 +557,9 @@ int moe_forward_impl(const kmoe_moe_args* a, void* workspace, size_t workspace_b
   // (Qwen3 decode: 4.8 us of 125). Not for an expert-parallel share (pairs of other ranks' experts get no row).
   mark(KMOE_STAGE_ALIGN, 0);
   const StreamScan scan{topk_ids, P, lod, static_cast<int32_t*>(at(L.expert_m)), moe_index, sorted_src};
-  const bool scan_in_gemm = stream_mode && Eg == E && a->first_expert == 0 && P <= kStreamScanMaxPairs &&
+  const bool streams = stream_mode || (a->format == KMOE_FMT_W4A16 && a->w_layout == KMOE_W_TILED &&
+                                       w4_gate_up_streams(P, 0, E, H));
+  const bool scan_in_gemm = streams && Eg == E && a->first_expert == 0 && P <= kStreamScanMaxPairs &&
                             M <= kStreamScanMaxRows && scan_allowed();
   if (!scan_in_gemm) {
     rc = kmoe_align_local(topk_ids, P, E, a->first_expert, moe_index, sorted_src, static_cast<int32_t*>(at(L.expert_m)), lod,

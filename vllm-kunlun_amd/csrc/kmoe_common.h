@@ -52,6 +52,10 @@ int stream_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream, const Stre
 // kmoe_grouped_gemm_i8 with the options above for the layer's own launches.
 int grouped_gemm_i8_checked(const kmoe_gemm_i8_args* args, kmoe_stream_t stream, const StreamScan* scan,
                             const StreamQuant* quant = nullptr);
+// kmoe_grouped_gemm_w4a16 with `scan` for the layer's routed gate_up launch where it runs on the streaming kernel
+// (w4_gate_up_streams says whether a launch of these dimensions does).
+int grouped_gemm_w4a16_checked(const kmoe_gemm_w4_args* args, kmoe_stream_t stream, const StreamScan* scan);
+bool w4_gate_up_streams(int rows, int rows_hint, int E, int k);
 // Persistent 128-row-tile GEMMs for many rows per expert (tiled weights, row-major activations);
 // arguments already validated.
 int tiled_gemm_i8(const kmoe_gemm_i8_args* args, hipStream_t stream);

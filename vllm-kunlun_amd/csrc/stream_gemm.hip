@@ -16,6 +16,7 @@
 //            lines, which cost the DeepSeek-V3 gate_up launch 9 %).
 // Each wave owns NF channel fragments and keeps D MFMA steps of loads in flight.
 #include "kmoe_common.h"
+#include "pair_scan.h"
 #include "quant_body.h"
 
 namespace kmoe {
@@ -46,7 +47,6 @@ struct StreamParams {
 };
 
 constexpr int kWaves = 4;
-constexpr int kScanBatch = 4;  // expert ids a lane asks for before it waits (a workgroup: one round trip per 1024 pairs)
 constexpr int kQuantStride = kStreamQuantMaxK + 16;  // bytes between the rows of the LDS copy: row li starts 16 li B into the banks
 
 // KS: the workgroup's 4 waves split K KS ways (KS = 1, 2, 4): 4/KS waves own
@@ -68,13 +68,13 @@ constexpr int kQuantStride = kStreamQuantMaxK + 16;  // bytes between the rows o
 // SIMD (see stream_gemm_i8).
 template <int MF, int NF, bool SWIGLU, int D, int KS, bool SCAN = false, bool QUANT = false>
 __global__ __launch_bounds__(kWaves* kWave, QUANT ? 4 : 1) void stream_gemm_i8_kernel(const StreamParams p) {
+  static_assert(!SCAN || kWaves == kScanWaves, "scan_pairs is written for four waves");
   static_assert(!QUANT || (MF == 1 && KS == 1 && !SWIGLU && !SCAN), "QUANT: the 16-row down-projection shape only");
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   constexpr int TM = 16 * MF;
   constexpr int WN = kWaves / KS;  // waves along the channel dimension
   __shared__ v4i red[KS > 1 ? (KS - 1) * WN * MF * NF * kWave : 1];
-  __shared__ int pair_list[SCAN ? kWaves : 1][SCAN ? kStreamScanMaxRows : 1];
-  __shared__ int scan_cnt[kWaves], scan_below[kWaves];
+  __shared__ typename std::conditional<SCAN, PairScanLds, int>::type scan_lds;
   __shared__ __attribute__((aligned(16))) int8_t qrows[QUANT ? 16 * kQuantStride : 16];
   __shared__ float qmax[16];
   const int lane = lane_id();
@@ -147,80 +147,15 @@ __global__ __launch_bounds__(kWaves* kWave, QUANT ? 4 : 1) void stream_gemm_i8_k
   __builtin_amdgcn_sched_barrier(0);
 
   int row_begin, row_end;
-  int list_c0 = 0, list_c1 = 0, list_c2 = 0;  // SCAN: lengths of the first three quarters' lists
-  auto listed_pair = [&](int i) {  // SCAN: the pair behind the expert's row i
-    int w = 0;
-    if (i >= list_c0) {
-      i -= list_c0;
-      w = 1;
-      if (i >= list_c1) {
-        i -= list_c1;
-        w = 2;
-        if (i >= list_c2) {
-          i -= list_c2;
-          w = 3;
-        }
-      }
-    }
-    return pair_list[w][i];
-  };
+  ListedRows listed = {};  // SCAN: the expert's rows
   if (tail) {
     row_begin = p.tail_row0 + (static_cast<int>(blockIdx.y) - p.E) * TM;
     row_end = min(p.tail_row0 + p.tail_rows, row_begin + TM);
-  } else if (SCAN) {
-    // wave w lists the pairs of its quarter of the ids; the quarters' lists, one after the other, are the expert's
-    // rows in order
-    const int quarter = (p.scan.n_pairs + kWaves * kWave - 1) / (kWaves * kWave) * kWave;
-    const int q_begin = wave_id * quarter;
-    const int q_end = min(p.scan.n_pairs, q_begin + quarter);
-    int below = 0, cnt = 0;  // ids below e; pairs of e so far (wave-uniform)
-    for (int base = q_begin; base < q_end; base += kScanBatch * kWave) {
-      int id[kScanBatch];
-#pragma unroll
-      for (int u = 0; u < kScanBatch; ++u) {
-        const int j = base + u * kWave + lane;
-        id[u] = j < q_end ? p.scan.ids[j] : 0x7fffffff;
-      }
-      // (every workgroup of the launch walks all the ids: scalar work wherever it can be, and the listing only for
-      // the few groups of 64 ids that hold a pair of this expert)
-#pragma unroll
-      for (int u = 0; u < kScanBatch; ++u) {
-        if (base + u * kWave >= q_end) break;  // wave-uniform
-        const bool mine = id[u] == e;
-        const uint64_t mb = __ballot(mine);
-        if (mb != 0) {
-          const int at = cnt + __builtin_popcountll(mb & lanemask_lt());
-          if (mine && at < kStreamScanMaxRows) pair_list[wave_id][at] = base + u * kWave + lane;
-          cnt += __builtin_popcountll(mb);
-        }
-        below += __builtin_popcountll(__ballot(id[u] < e));
-      }
-    }
-    if (lane == 0) {
-      scan_cnt[wave_id] = min(cnt, kStreamScanMaxRows);  // (a token picks an expert once: never more rows than tokens)
-      scan_below[wave_id] = below;
-    }
-    __syncthreads();
-    if (idle) return;  // (KS == 1: no barrier after this one)
-    list_c0 = scan_cnt[0];
-    list_c1 = scan_cnt[1];
-    list_c2 = scan_cnt[2];
-    cnt = min(list_c0 + list_c1 + list_c2 + scan_cnt[3], kStreamScanMaxRows);
-    below = scan_below[0] + scan_below[1] + scan_below[2] + scan_below[3];
-    row_begin = below;
-    row_end = below + cnt;
-    if (blockIdx.x == 0 && wave_id == 0) {
-      if (lane == 0) {
-        p.scan.lod[e] = below;
-        p.scan.expert_m[e] = cnt;
-        if (e == p.E - 1) p.scan.lod[p.E] = below + cnt;
-      }
-      for (int i = lane; i < cnt; i += kWave) {
-        const int j = listed_pair(i);
-        p.scan.moe_index[j] = below + i;
-        p.scan.sorted_src[below + i] = j;
-      }
-    }
+  } else if constexpr (SCAN) {
+    listed = scan_pairs(p.scan, e, p.E, scan_lds, blockIdx.x == 0);
+    if (idle) return;  // (KS == 1: no barrier after the scan's)
+    row_begin = listed.begin;
+    row_end = listed.end;
   } else {
     row_begin = p.lod[e];
     row_end = p.lod[e + 1];
@@ -281,8 +216,8 @@ __global__ __launch_bounds__(kWaves* kWave, QUANT ? 4 : 1) void stream_gemm_i8_k
 #pragma unroll
     for (int mf = 0; mf < MF; ++mf) {
       const int r = row0 + mf * 16 + li;
-      if (SCAN)
-        srow[mf] = r < row_end ? (tail ? p.tail_src0 + r - p.tail_row0 : listed_pair(r - row_begin) / p.src_div) : -1;
+      if constexpr (SCAN)
+        srow[mf] = r < row_end ? (tail ? p.tail_src0 + r - p.tail_row0 : listed.pair(scan_lds, r - row_begin) / p.src_div) : -1;
       else
         srow[mf] = r < row_end ? (tail ? p.tail_src0 + r - p.tail_row0 : (p.row_src ? p.row_src[r] / p.src_div : r)) : -1;
       // rows past the end read row 0: valid memory, results never stored

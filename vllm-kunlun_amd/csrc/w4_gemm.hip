@@ -26,6 +26,7 @@
 
 #include "buffer_ops.h"
 #include "kmoe_common.h"
+#include "pair_scan.h"
 
 namespace kmoe {
 namespace {
@@ -54,6 +55,7 @@ struct W4Params {
   int32_t E, n, k;
   uint16_t* y;
   int64_t ldy;
+  StreamScan scan;  // SCAN instantiations of the streaming kernel: the routed pairs' expert ids instead of lod / row_src
 };
 
 constexpr int kWaves = 4;
@@ -108,9 +110,13 @@ __device__ inline v4i unpack8_half(uint32_t word, v2h s2) {
 // contiguous piece of the scale tensor) into its own part of LDS and reads a block's scale from there.
 // Read from global memory per block, a lane's 2-byte scale load touches 16 cache lines per instruction
 // (16 channels, rows apart), as many as the weight load next to it moves bytes for: 20 % of the launch.
-template <int MF, int NF, bool SWIGLU, int D, bool F16, bool SLDS>
+// SCAN: the launch sorts the routed pairs by expert itself (pair_scan.h): rows and gather indices come from the
+// pairs' expert ids, and the workgroups of channel block 0 write what the sort's launch would have.
+template <int MF, int NF, bool SWIGLU, int D, bool F16, bool SLDS, bool SCAN = false>
 __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params p) {
+  static_assert(!SCAN || kWaves == kScanWaves, "scan_pairs is written for four waves");
   extern __shared__ uint16_t scale_lds[];  // SLDS: [kWaves][NF][16][groups]
+  __shared__ typename std::conditional<SCAN, PairScanLds, int>::type scan_lds;
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   constexpr int TM = 16 * MF;
   const int lane = lane_id();
@@ -118,7 +124,16 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
   const int li = lane & 15;
   const int lg = lane >> 4;
   const int e = blockIdx.y;
-  const int row_begin = p.lod[e], row_end = p.lod[e + 1];
+  int row_begin, row_end;
+  ListedRows listed = {};
+  if constexpr (SCAN) {
+    listed = scan_pairs(p.scan, e, p.E, scan_lds, blockIdx.x == 0);  // (all four waves: a barrier inside)
+    row_begin = listed.begin;
+    row_end = listed.end;
+  } else {
+    row_begin = p.lod[e];
+    row_end = p.lod[e + 1];
+  }
   if (row_begin >= row_end) return;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const int col_base = (blockIdx.x * kWaves + wave) * NFH * 16;
@@ -160,7 +175,11 @@ __global__ __launch_bounds__(kWaves* kWave) void w4_stream_kernel(const W4Params
     for (int mf = 0; mf < MF; ++mf) {
       const int r = row0 + mf * 16 + li;
       const int rr = r < row_end ? r : row_begin;  // rows past the end read a valid row: never stored
-      const int src = p.row_src ? p.row_src[rr] / p.src_div : rr;
+      int src;
+      if constexpr (SCAN)
+        src = listed.pair(scan_lds, rr - row_begin) / p.src_div;
+      else
+        src = p.row_src ? p.row_src[rr] / p.src_div : rr;
       ap[mf] = p.a + static_cast<size_t>(src) * p.lda + 32 * lg;
     }
     v4f acc[MF][NF];
@@ -535,24 +554,25 @@ int launch_w4_tile(const W4Params& p, int rows, bool f16, hipStream_t s) {
   return check_launch("kmoe_grouped_gemm_w4a16");
 }
 
-template <int MF, int NF, bool SWIGLU, int D>
+template <int MF, int NF, bool SWIGLU, int D, bool SCAN = false>
 int launch_w4(const W4Params& p, bool f16, hipStream_t s) {
   constexpr int NFH = SWIGLU ? NF / 2 : NF;
   const int n_half = SWIGLU ? p.n / 2 : p.n;
   const dim3 grid(ceil_div(n_half, kWaves * NFH * 16), p.E);
   const size_t lds = static_cast<size_t>(kWaves) * NF * 16 * (p.k / p.gs) * sizeof(uint16_t);
   if (tracing_kernels())
-    note_kernel("w4_stream_kernel<%d rows per pass, %d channel fragments per wave, %s, %d blocks in flight, %s, group scales in %s>",
-                16 * MF, NF, SWIGLU ? "SiLU-mul" : "plain", D, f16 ? "f16" : "bf16", lds <= 32 * 1024 ? "LDS" : "global memory");
+    note_kernel("w4_stream_kernel<%d rows per pass, %d channel fragments per wave, %s, %d blocks in flight, %s, group scales in %s%s>",
+                16 * MF, NF, SWIGLU ? "SiLU-mul" : "plain", D, f16 ? "f16" : "bf16", lds <= 32 * 1024 ? "LDS" : "global memory",
+                SCAN ? ", sorts the pairs itself" : "");
   if (lds <= 32 * 1024) {  // beyond: many small groups on a long K; the scales stay in global memory
     if (f16)
-      hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, true, true>), grid, dim3(kWaves * kWave), lds, s, p);
+      hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, true, true, SCAN>), grid, dim3(kWaves * kWave), lds, s, p);
     else
-      hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, false, true>), grid, dim3(kWaves * kWave), lds, s, p);
+      hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, false, true, SCAN>), grid, dim3(kWaves * kWave), lds, s, p);
   } else if (f16) {
-    hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, true, false>), grid, dim3(kWaves * kWave), 0, s, p);
+    hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, true, false, SCAN>), grid, dim3(kWaves * kWave), 0, s, p);
   } else {
-    hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, false, false>), grid, dim3(kWaves * kWave), 0, s, p);
+    hipLaunchKernelGGL((w4_stream_kernel<MF, NF, SWIGLU, D, false, false, SCAN>), grid, dim3(kWaves * kWave), 0, s, p);
   }
   return check_launch("kmoe_grouped_gemm_w4a16");
 }
@@ -568,7 +588,20 @@ __global__ __launch_bounds__(256) void tile_scales_kernel(const uint16_t* __rest
   dst[i] = src[(frag * 16 + c) * groups + g];
 }
 
+// Rows per pass of the streaming kernel for a launch (1: 16, 2: 32), or 0 where the tile kernel takes over.
+int w4_stream_passes(int rows, int rows_hint, int E, int k) {
+  const int avg = ceil_div(expected_rows(rows, rows_hint), E);
+  // (with K = 2048 the 32-row streaming pass is never the best: 12 rows per expert 75 on 16-row passes, 84 on
+  // 32-row passes, 87 on 64-row tiles; 16 rows 99 / 96 / 87)
+  const int one_max = k > 4096 ? 10 : 13;
+  const int stream_max = k > 4096 ? 20 : 13;
+  return avg <= one_max ? 1 : (avg <= stream_max ? 2 : 0);
+}
+
 }  // namespace
+
+bool w4_gate_up_streams(int rows, int rows_hint, int E, int k) { return w4_stream_passes(rows, rows_hint, E, k) != 0; }
+
 }  // namespace kmoe
 
 using namespace kmoe;
@@ -583,8 +616,12 @@ extern "C" int kmoe_tile_scales_w4(const uint16_t* src, uint16_t* dst, int E, in
 }
 
 extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t stream) {
+  return grouped_gemm_w4a16_checked(a, stream, nullptr);
+}
+
+int kmoe::grouped_gemm_w4a16_checked(const kmoe_gemm_w4_args* a, kmoe_stream_t stream, const StreamScan* scan) {
   KMOE_REQUIRE(a, KMOE_ERR_NULL, "grouped_gemm_w4a16: NULL args");
-  KMOE_REQUIRE(a->a && a->w && a->w_scale && a->lod && a->y, KMOE_ERR_NULL, "grouped_gemm_w4a16: NULL pointer");
+  KMOE_REQUIRE(a->a && a->w && a->w_scale && (a->lod || scan) && a->y, KMOE_ERR_NULL, "grouped_gemm_w4a16: NULL pointer");
   KMOE_REQUIRE(a->E >= 1 && a->rows >= 0, KMOE_ERR_SHAPE, "grouped_gemm_w4a16: E=%d rows=%d", a->E, a->rows);
   const bool swiglu = a->act == KMOE_ACT_SWIGLU;
   KMOE_REQUIRE(a->act == KMOE_ACT_NONE || swiglu, KMOE_ERR_UNSUPPORTED, "grouped_gemm_w4a16: act=%d", a->act);
@@ -603,7 +640,7 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
   KMOE_REQUIRE(a->act_dtype == KMOE_DT_BF16 || a->act_dtype == KMOE_DT_F16, KMOE_ERR_UNSUPPORTED,
                "grouped_gemm_w4a16: act_dtype=%d unknown", a->act_dtype);
   const bool f16 = a->act_dtype == KMOE_DT_F16;
-  if (a->rows == 0) return KMOE_OK;
+  if (a->rows == 0 && !scan) return KMOE_OK;
   const int q = a->group_size / 32;
   int shift = -1;
   if ((q & (q - 1)) == 0)
@@ -613,8 +650,18 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
   const int groups = a->k / a->group_size;
   const bool frag16 = a->scale_layout == KMOE_S_FRAG16;
   const W4Params p{a->a, a->lda, a->row_src, a->src_div, a->w, a->w_scale, a->group_size, shift,
-                   frag16 ? 1 : groups, frag16 ? 16 : 1, a->lod, a->E, a->n, a->k, a->y, a->ldy};
+                   frag16 ? 1 : groups, frag16 ? 16 : 1, a->lod, a->E, a->n, a->k, a->y, a->ldy,
+                   scan ? *scan : StreamScan{}};
   hipStream_t s = as_stream(stream);
+  if (scan) {
+    // the routed gate_up launch of a decode-sized layer, on the streaming kernel
+    const int passes = w4_stream_passes(a->rows, a->rows_hint, a->E, a->k);
+    KMOE_REQUIRE(swiglu && a->variant == 0 && a->row_src == nullptr && passes != 0 && scan->ids && scan->lod &&
+                     scan->expert_m && scan->moe_index && scan->sorted_src && scan->n_pairs == a->rows &&
+                     a->rows <= kStreamScanMaxPairs,
+                 KMOE_ERR_UNSUPPORTED, "grouped_gemm_w4a16: not a launch that can sort the pairs itself");
+    return passes == 1 ? launch_w4<1, 2, true, 1, true>(p, f16, s) : launch_w4<2, 2, true, 2, true>(p, f16, s);
+  }
   int mf = a->variant;
   // the tile kernel reaches a source row (gathered or not: below `rows`) through a 32-bit byte offset
   const bool tile_ok = static_cast<uint64_t>(a->rows) * static_cast<uint64_t>(a->lda) * 2u + static_cast<uint64_t>(a->k) * 2u < (1ull << 32);
@@ -629,11 +676,8 @@ extern "C" int kmoe_grouped_gemm_w4a16(const kmoe_gemm_w4_args* a, kmoe_stream_t
     // 111 / 109 / 120 and 2440 / 2609 / 2918, at 56 rows 111 / 107 / 119 and 2634 / 2614 / 2993, at 64 rows
     // 133 / 109 / 121, at 76 rows 156 / 109 / 122 and 4073 / 2708 / 3113, at 80 rows - / 136 / 127).
     const int avg = ceil_div(expected_rows(a->rows, a->rows_hint), a->E);
-    // (with K = 2048 the 32-row streaming pass is never the best: 12 rows per expert 75 on 16-row passes, 84 on
-    // 32-row passes, 87 on 64-row tiles; 16 rows 99 / 96 / 87)
-    const int one_max = a->k > 4096 ? 10 : 13;
-    const int stream_max = a->k > 4096 ? 20 : 13;
-    mf = avg <= one_max ? 1 : (avg <= stream_max ? 2 : (!tile_ok ? 4 : (avg <= 48 ? 64 : (avg <= 76 ? 96 : 128))));
+    const int passes = w4_stream_passes(a->rows, a->rows_hint, a->E, a->k);
+    mf = passes ? passes : (!tile_ok ? 4 : (avg <= 48 ? 64 : (avg <= 76 ? 96 : 128)));
   }
   if (mf == 8) mf = 128;
   if (mf == 64 || mf == 96 || mf == 128)

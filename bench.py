@@ -17,6 +17,7 @@ in HBM. Prints ONE JSON line: tokens/s, the roofline of the dominant kernel
 import argparse
 import ctypes as C
 import json
+import math
 import os
 import re
 import sys
@@ -240,7 +241,7 @@ def clock_probe(plan, stream, ms_per_step, load_ms=20.0):
     }
 
 
-def measure(a, workload, shape, label, sl, with_cpu_baseline):
+def measure(a, workload, shape, label, sl, with_cpu_baseline, exact_steps=True):
     """Times one workload's layer on cuda:0 (inputs resident in HBM) and returns the pieces of
     the JSON line: ms per step (graph replay / eager plan / plugin entry), per-stage durations
     from HIP events on the launch stream, the gate_up GEMM's roofline, the layer's fractions."""
@@ -291,15 +292,27 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
         traced = L.lib.kmoe_traced_kernels().decode().splitlines()
         stream.synchronize()
 
+        # The headline workload times exactly --steps steps. The other workloads of the suite time at least
+        # kMinTimedMs of work: 20 steps of a 0.1 ms layer are 2 ms between two synchronisations, whose own
+        # cost (the first launch after an idle stream, the wake-up at the end) then reads as 4-6 % of a step.
+        kMinTimedMs = 20.0
+        steps_used = [a.steps]
+
         def timed(step):
-            for _ in range(a.warmup):
-                step()
-            stream.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(a.steps):
-                step()
-            stream.synchronize()
-            return (time.perf_counter() - t0) * 1e3 / a.steps
+            n = a.steps
+            while True:
+                for _ in range(a.warmup):
+                    step()
+                stream.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n):
+                    step()
+                stream.synchronize()
+                total = (time.perf_counter() - t0) * 1e3
+                if exact_steps or total >= kMinTimedMs or n >= 4000:
+                    steps_used[0] = max(steps_used[0], n)
+                    return total / n
+                n = min(4000, max(n + 1, int(math.ceil(n * kMinTimedMs / total * 1.1))))
 
         launch_ms = {}
         if a.launch in ("auto", "graph"):
@@ -369,7 +382,7 @@ def measure(a, workload, shape, label, sl, with_cpu_baseline):
         "config": {"workload": label, "name": workload, "tokens": shape.M, "hidden": shape.H,
                    "experts": shape.E, "top_k": shape.K, "moe_intermediate": shape.I,
                    "shared_intermediate": shape.I_shared, "routing": shape.scoring, "experts_hit": n_active,
-                   "launch": launch_mode, "launch_ms_per_step": launch_ms, "seed": a.seed,
+                   "launch": launch_mode, "launch_ms_per_step": launch_ms, "timed_steps": steps_used[0], "seed": a.seed,
                    "side_stream": not a.one_stream, "router_gemm_inside": bool(a.router), "tile_variant": a.tile_variant, "gemm_kernels": traced,
                    "activations": "float16" if a.act_dtype == "f16" else "bfloat16"},
         "roofline": roofline,
@@ -492,7 +505,8 @@ def main():
             for t in (getattr(sl.layer, n, None) for n in ("w13_weight", "w2_weight", "w13_weight_packed", "w2_weight_packed")):
                 if t is not None:
                     t.data.zero_()
-        results[name] = measure(a, name, shape, label, sl, name == headline and not a.no_cpu_baseline)
+        results[name] = measure(a, name, shape, label, sl, name == headline and not a.no_cpu_baseline,
+                                exact_steps=name == headline)
         print(f"bench.py: {name}: {results[name]['ms_per_step']:.4f} ms/step", file=sys.stderr, flush=True)
 
     head = results[headline]

@@ -94,7 +94,10 @@ def _run_align(L, ids_np, E):
 @pytest.mark.parametrize("P,E,kind", [(0, 8, "uniform"), (1, 8, "uniform"), (64, 8, "uniform"), (512, 128, "uniform"),
                                       (1024, 256, "uniform"), (1000, 384, "skew"), (8192, 128, "skew"),
                                       (8193, 128, "uniform"), (65536, 128, "skew"), (32768, 256, "uniform"),
-                                      (40000, 1024, "onehot"), (5000, 33, "holes")])
+                                      (40000, 1024, "onehot"), (5000, 33, "holes"),
+                                      # many chunks of 2048 pairs for the three-launch path
+                                      (131072, 128, "uniform"), (131073, 64, "skew"), (300000, 256, "uniform"),
+                                      (140000, 1024, "holes")])
 def test_align(L, P, E, kind):
     rng = np.random.default_rng(P + E)
     if kind == "uniform":
